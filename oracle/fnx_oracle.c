@@ -1,0 +1,624 @@
+/* CPU oracle: see fnx_oracle.h. TEST INFRASTRUCTURE ONLY - never linked into the device library.
+ * Build: gcc -O2 -ffp-contract=off -fopenmp -fPIC -shared (oracle/Makefile). -ffp-contract=off matters: every fused
+ * multiply-add below is written as fmaf() on purpose, everything else must stay an unfused multiply and add. */
+#include "fnx_oracle.h"
+
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#include "iq3s_grid.h"
+
+#define IQ3S_BLOCK 110
+#define Q8_1_BLOCK 36
+
+int fnx_o_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
+
+/* ---------------------------------------------------------------- half <-> float (tensor_convert.hpp:23-50) */
+float fnx_o_h2f(uint16_t h) {
+    const uint32_t sign = (h >> 15) & 1u, ex = (h >> 10) & 31u, man = h & 1023u;
+    float f;
+    if (ex == 0) f = ldexpf((float) man, -24);
+    else if (ex == 31) f = man ? NAN : INFINITY;
+    else f = ldexpf((float) (man + 1024u), (int) ex - 25);
+    return sign ? -f : f;
+}
+
+uint16_t fnx_o_f2h(float x) { /* round to nearest even */
+    uint32_t b;
+    memcpy(&b, &x, 4);
+    const uint32_t sign = (b >> 16) & 0x8000u, ex = (b >> 23) & 0xFFu, man = b & 0x7FFFFFu;
+    if (ex == 0xFF) return (uint16_t) (sign | 0x7C00u | (man ? 0x200u : 0u));
+    const int ne = (int) ex - 127 + 15;
+    if (ne >= 31) return (uint16_t) (sign | 0x7C00u);
+    if (ne <= 0) {
+        if (ne < -10) return (uint16_t) sign;
+        const uint32_t mm = (man | 0x800000u) >> (1 - ne);
+        uint32_t r = mm >> 13;
+        const uint32_t rem = mm & 0x1FFFu;
+        if (rem > 0x1000u || (rem == 0x1000u && (r & 1u))) ++r;
+        return (uint16_t) (sign | r);
+    }
+    uint32_t r = ((uint32_t) ne << 10) | (man >> 13);
+    const uint32_t rem = man & 0x1FFFu;
+    if (rem > 0x1000u || (rem == 0x1000u && (r & 1u))) ++r;
+    return (uint16_t) (sign | r);
+}
+
+static float bf16_to_f32(uint16_t b) {
+    const uint32_t u = (uint32_t) b << 16;
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+/* ---------------------------------------------------------------- dp4a (p100_compat.h:18-22) */
+int fnx_o_dp4a(int a, int b, int c) {
+    return c + (int) (signed char) a * (int) (signed char) b + (int) (signed char) (a >> 8) * (int) (signed char) (b >> 8) +
+           (int) (signed char) (a >> 16) * (int) (signed char) (b >> 16) + (a >> 24) * (b >> 24);
+}
+
+/* ---------------------------------------------------------------- IQ3_S decode (tensor_convert.hpp:295-322) */
+void fnx_o_iq3s_dequant(const uint8_t* src, size_t n, float* y) {
+    for (size_t b = 0; b < n / 256; ++b) {
+        const uint8_t* p = src + b * IQ3S_BLOCK;
+        uint16_t dh;
+        memcpy(&dh, p, 2);
+        const float d = fnx_o_h2f(dh);
+        const uint8_t *qs = p + 2, *qh = p + 66, *signs = p + 74, *scales = p + 106;
+        float* o = y + b * 256;
+        for (int ib = 0; ib < 8; ++ib) { /* sub-block ib: qs[8 ib..], qh[ib], signs[4 ib..], nibble ib & 1 of scales[ib / 2] */
+            const int s4 = (scales[ib / 2] >> (4 * (ib & 1))) & 0xF;
+            const float db = d * (float) (1 + 2 * s4);
+            for (int l = 0; l < 4; ++l) {
+                const uint32_t g1 = fnx_o_iq3s_grid[qs[8 * ib + 2 * l] | ((qh[ib] << (8 - 2 * l)) & 256)];
+                const uint32_t g2 = fnx_o_iq3s_grid[qs[8 * ib + 2 * l + 1] | ((qh[ib] << (7 - 2 * l)) & 256)];
+                const uint8_t sg = signs[4 * ib + l];
+                for (int j = 0; j < 4; ++j) {
+                    o[32 * ib + 8 * l + j] = db * (float) ((g1 >> (8 * j)) & 255) * ((sg >> j) & 1 ? -1.f : 1.f);
+                    o[32 * ib + 8 * l + 4 + j] = db * (float) ((g2 >> (8 * j)) & 255) * ((sg >> (j + 4)) & 1 ? -1.f : 1.f);
+                }
+            }
+        }
+    }
+}
+
+/* ---------------------------------------------------------------- IQ3_S encoder (this build's own; parity unpinned)
+ * Per 32-weight sub-block: try five candidate scales amax / c, c in {15, 13.5, 12, 10.5, 9}; for each, every 4-group
+ * takes the nearest codebook entry (squared error on magnitudes, ties to the lower index); keep the scale with the
+ * least error. Block scale d = max sub-block scale / 31 (stored as half); sub-block code s = round((scale/d - 1)/2)
+ * clamped to 0..15; the groups are then re-coded against the final d (1 + 2 s). Signs are the weights' own. */
+static int nearest_grid(const float a[4]) { /* a: magnitudes in codebook units */
+    int best = 0;
+    float be = INFINITY;
+    for (int g = 0; g < 512; ++g) {
+        const uint32_t v = fnx_o_iq3s_grid[g];
+        float e = 0.f;
+        for (int j = 0; j < 4; ++j) {
+            const float df = a[j] - (float) ((v >> (8 * j)) & 255);
+            e = e + df * df;
+        }
+        if (e < be) {
+            be = e;
+            best = g;
+        }
+    }
+    return best;
+}
+static float group_err(const float a[4], int g) {
+    const uint32_t v = fnx_o_iq3s_grid[g];
+    float e = 0.f;
+    for (int j = 0; j < 4; ++j) {
+        const float df = a[j] - (float) ((v >> (8 * j)) & 255);
+        e = e + df * df;
+    }
+    return e;
+}
+void fnx_o_iq3s_quantize(const float* w, size_t n, uint8_t* dst) {
+    static const float cand[5] = {15.0f, 13.5f, 12.0f, 10.5f, 9.0f};
+    for (size_t b = 0; b < n / 256; ++b) {
+        const float* x = w + b * 256;
+        uint8_t* p = dst + b * IQ3S_BLOCK;
+        memset(p, 0, IQ3S_BLOCK);
+        float sc[8], smax = 0.f;
+        for (int ib = 0; ib < 8; ++ib) {
+            float amax = 0.f;
+            for (int j = 0; j < 32; ++j) amax = fmaxf(amax, fabsf(x[32 * ib + j]));
+            sc[ib] = 0.f;
+            if (amax > 0.f) {
+                float beste = INFINITY;
+                for (int c = 0; c < 5; ++c) {
+                    const float s = amax / cand[c];
+                    float err = 0.f;
+                    for (int g = 0; g < 8; ++g) {
+                        float a[4];
+                        for (int j = 0; j < 4; ++j) a[j] = fabsf(x[32 * ib + 4 * g + j]) / s;
+                        err = err + group_err(a, nearest_grid(a));
+                    }
+                    err = err * s * s;
+                    if (err < beste) {
+                        beste = err;
+                        sc[ib] = s;
+                    }
+                }
+            }
+            smax = fmaxf(smax, sc[ib]);
+        }
+        const uint16_t dh = fnx_o_f2h(smax / 31.0f);
+        memcpy(p, &dh, 2);
+        const float d = fnx_o_h2f(dh);
+        uint8_t *qs = p + 2, *qh = p + 66, *signs = p + 74, *scales = p + 106;
+        for (int ib = 0; ib < 8; ++ib) {
+            int s4 = 0;
+            if (d > 0.f) {
+                s4 = (int) roundf((sc[ib] / d - 1.0f) * 0.5f);
+                s4 = s4 < 0 ? 0 : s4 > 15 ? 15 : s4;
+            }
+            scales[ib / 2] |= (uint8_t) (s4 << (4 * (ib & 1)));
+            const float db = d * (float) (1 + 2 * s4);
+            for (int g = 0; g < 8; ++g) {
+                float a[4];
+                uint8_t sg = 0;
+                for (int j = 0; j < 4; ++j) {
+                    const float v = x[32 * ib + 4 * g + j];
+                    a[j] = db > 0.f ? fabsf(v) / db : 0.f;
+                    if (v < 0.f) sg |= (uint8_t) (1u << j);
+                }
+                const int gi = nearest_grid(a);
+                qs[8 * ib + g] = (uint8_t) (gi & 255);
+                qh[ib] |= (uint8_t) ((gi >> 8) << g);
+                signs[4 * ib + g / 2] |= (uint8_t) (sg << (4 * (g & 1)));
+            }
+        }
+    }
+}
+
+/* ---------------------------------------------------------------- q8_1 (kernels.cu:131-145)
+ * one warp per 32 values: amax and the sum by xor-butterfly over the 32 lanes (16, 8, 4, 2, 1) */
+static float butterfly_sum(float* v, int n) { /* v[l] += v[l ^ o] for o = n/2 .. 1; every lane ends with the same value */
+    float t[64];
+    for (int o = n / 2; o; o >>= 1) {
+        for (int l = 0; l < n; ++l) t[l] = v[l] + v[l ^ o];
+        memcpy(v, t, (size_t) n * sizeof(float));
+    }
+    return v[0];
+}
+static void q8_1_block(const float* xi, uint8_t* blk) {
+    float amax = 0.f, lanes[32];
+    for (int j = 0; j < 32; ++j) {
+        amax = fmaxf(amax, fabsf(xi[j]));
+        lanes[j] = xi[j];
+    }
+    const float sum = butterfly_sum(lanes, 32);
+    const float d = amax / 127.0f;
+    const uint16_t dh = fnx_o_f2h(d), sh = fnx_o_f2h(sum);
+    memcpy(blk, &dh, 2);
+    memcpy(blk + 2, &sh, 2);
+    for (int j = 0; j < 32; ++j) blk[4 + j] = (uint8_t) (int8_t) (amax == 0.0f ? 0 : (int) roundf(xi[j] / d));
+}
+void fnx_o_quantize_q8_1(const float* x, uint8_t* q, int n, int rows) {
+    for (int r = 0; r < rows; ++r)
+        for (int b = 0; b < n / 32; ++b) q8_1_block(x + (size_t) r * n + 32 * b, q + ((size_t) r * (n / 32) + b) * Q8_1_BLOCK);
+}
+
+/* ---------------------------------------------------------------- the integer dot (iq3s_x.cuh:4-41) */
+static int ld32(const uint8_t* p) { /* get_int_b2 / get_int_b4: a little-endian 32-bit load */
+    uint32_t v;
+    memcpy(&v, p, 4);
+    return (int) v;
+}
+static int vcmpne4_zero(uint32_t a) { /* __vcmpne4(a, 0): 0xff in every byte of a that is not zero */
+    uint32_t r = 0;
+    for (int k = 0; k < 4; ++k)
+        if ((a >> (8 * k)) & 0xFFu) r |= 0xFFu << (8 * k);
+    return (int) r;
+}
+static int vsub4(uint32_t a, uint32_t b) { /* __vsub4: per-byte a - b, wrapping */
+    uint32_t r = 0;
+    for (int k = 0; k < 4; ++k) r |= (((a >> (8 * k)) - (b >> (8 * k))) & 0xFFu) << (8 * k);
+    return (int) r;
+}
+float fnx_o_vec_dot_iq3s_q8_1(const uint8_t* blk, const uint8_t* q8, int iqs) {
+    const uint8_t *bqs = blk + 2, *bqh = blk + 66, *bsigns = blk + 74, *bscales = blk + 106;
+    const uint8_t* qs = bqs + 4 * iqs; /* the two ints at iqs, iqs + 1 */
+    const int qh = bqh[iqs / 2];
+    const uint8_t* sp = bsigns + 4 * (iqs / 2);
+    const uint8_t* yb = q8 + (size_t) (iqs / 2) * Q8_1_BLOCK;
+    int sumi = 0;
+    for (int l0 = 0; l0 < 8; l0 += 2) {
+        const uint32_t gx = fnx_o_iq3s_grid[qs[l0] | ((qh << (8 - l0)) & 0x100)];
+        const uint32_t gy = fnx_o_iq3s_grid[qs[l0 + 1] | ((qh << (7 - l0)) & 0x100)];
+        const uint32_t sb = sp[l0 / 2];
+        const int signs0 = vcmpne4_zero(((sb & 0x03u) << 7) | ((sb & 0x0Cu) << 21));
+        const int signs1 = vcmpne4_zero(((sb & 0x30u) << 3) | ((sb & 0xC0u) << 17));
+        const int grid_l = vsub4(gx ^ (uint32_t) signs0, (uint32_t) signs0);
+        const int grid_h = vsub4(gy ^ (uint32_t) signs1, (uint32_t) signs1);
+        const int u0 = ld32(yb + 4 + 4 * l0), u1 = ld32(yb + 4 + 4 * (l0 + 1));
+        sumi = fnx_o_dp4a(grid_l, u0, sumi);
+        sumi = fnx_o_dp4a(grid_h, u1, sumi);
+    }
+    sumi *= 1 + 2 * ((bscales[iqs / 4] >> ((iqs << 1) & 0x04)) & 0x0F);
+    uint16_t dw, dx;
+    memcpy(&dw, blk, 2);
+    memcpy(&dx, yb, 2);
+    const float d = fnx_o_h2f(dw) * fnx_o_h2f(dx);
+    return d * (float) sumi;
+}
+
+/* lanes per row as moe_g picks them (moe.cuh:664-670): 8 lanes a super-block, doubled up to 32 */
+static int lanes_per_row(int ncols) {
+    const int lanes = ncols / 256 * 8;
+    int G = 8;
+    while (G < lanes && G < 32) G *= 2;
+    return G;
+}
+/* one weight row against one q8_1 row: lane gl takes super-blocks gl / 8, + G / 8, ... with its sub-block 2 (gl % 8);
+ * the lanes' sums then meet in a butterfly (kernels.cu:209-228) */
+static float row_dot(const uint8_t* wr, int ncols, const uint8_t* yq) {
+    const int G = lanes_per_row(ncols), bpi = G / 8, bpr = ncols / 256;
+    float tmp[32];
+    for (int gl = 0; gl < G; ++gl) {
+        float t = 0.f;
+        for (int kbx = gl / 8; kbx < bpr; kbx += bpi)
+            t += fnx_o_vec_dot_iq3s_q8_1(wr + (size_t) kbx * IQ3S_BLOCK, yq + (size_t) kbx * 8 * Q8_1_BLOCK, 2 * (gl % 8));
+        tmp[gl] = t;
+    }
+    return butterfly_sum(tmp, G);
+}
+void fnx_o_mmvq_iq3s(const uint8_t* wbase, size_t w_stride, const uint8_t* const* ep, int nrows, int ncols,
+                     const fnx_o_job* jobs, int njobs, const uint8_t* y, float* out, int out_stride, int threads) {
+    const size_t row_bytes = (size_t) (ncols / 256) * IQ3S_BLOCK, y_row = (size_t) (ncols / 32) * Q8_1_BLOCK;
+    const long total = (long) njobs * nrows;
+    (void) threads;
+#pragma omp parallel for schedule(static) num_threads(threads > 0 ? threads : 1)
+    for (long q = 0; q < total; ++q) {
+        const int ji = (int) (q / nrows), r = (int) (q % nrows);
+        const fnx_o_job* jb = jobs + ji;
+        const uint8_t* we = ep ? ep[jb->w] : wbase + (size_t) jb->w * w_stride;
+        for (int j = 0; j < jb->n; ++j)
+            out[(size_t) jb->out[j] * out_stride + r] = row_dot(we + (size_t) r * row_bytes, ncols, y + (size_t) jb->y[j] * y_row);
+    }
+}
+
+void fnx_o_gemv_exact(const uint8_t* w, int nrows, int ncols, const float* x, int T, double* out) {
+    const size_t row_bytes = (size_t) (ncols / 256) * IQ3S_BLOCK;
+    float* wf = (float*) malloc((size_t) ncols * sizeof(float));
+    for (int r = 0; r < nrows; ++r) {
+        fnx_o_iq3s_dequant(w + (size_t) r * row_bytes, (size_t) ncols, wf);
+        for (int t = 0; t < T; ++t) {
+            double s = 0.0;
+            for (int i = 0; i < ncols; ++i) s += (double) wf[i] * (double) x[(size_t) t * ncols + i];
+            out[(size_t) t * nrows + r] = s;
+        }
+    }
+    free(wf);
+}
+
+/* ---------------------------------------------------------------- f32 / bf16 mat-vec in the fixed 64-lane order */
+static float dot64(const float* w, const uint16_t* wb, const float* x, int n) {
+    float lane[64];
+    const int chunks = n / 4;
+    for (int l = 0; l < 64; ++l) {
+        float a = 0.f;
+        for (int c = l; c < chunks; c += 64)
+            for (int k = 0; k < 4; ++k) {
+                const float wv = w ? w[4 * c + k] : bf16_to_f32(wb[4 * c + k]);
+                a = fmaf(wv, x[4 * c + k], a);
+            }
+        lane[l] = a;
+    }
+    return butterfly_sum(lane, 64);
+}
+void fnx_o_gemv_f32(const float* W, const float* x, float* y, int rows, int n, int T) {
+#pragma omp parallel for schedule(static)
+    for (int r = 0; r < rows; ++r)
+        for (int t = 0; t < T; ++t) y[(size_t) t * rows + r] = dot64(W + (size_t) r * n, NULL, x + (size_t) t * n, n);
+}
+void fnx_o_gemv_bf16(const uint16_t* W, const float* x, float* y, int rows, int n, int T) {
+#pragma omp parallel for schedule(static)
+    for (int r = 0; r < rows; ++r)
+        for (int t = 0; t < T; ++t) y[(size_t) t * rows + r] = dot64(NULL, W + (size_t) r * n, x + (size_t) t * n, n);
+}
+
+/* ---------------------------------------------------------------- routing */
+void fnx_o_topk_logits(const float* logits, int stride, int T, int nexp, int topk, int* topi, float* topw) {
+    unsigned char* taken = (unsigned char*) malloc((size_t) nexp);
+    for (int t = 0; t < T; ++t) {
+        const float* v = logits + (size_t) t * stride;
+        memset(taken, 0, (size_t) nexp);
+        float top0 = 0.f, z = 0.f, e[64];
+        for (int k = 0; k < topk; ++k) {
+            float bv = -INFINITY;
+            int bi = nexp;
+            for (int i = 0; i < nexp; ++i) /* ascending index with a strict compare: the lower index wins a tie */
+                if (!taken[i] && v[i] > bv) {
+                    bv = v[i];
+                    bi = i;
+                }
+            if (bi < nexp) taken[bi] = 1;
+            if (k == 0) top0 = bv;
+            e[k] = expf(bv - top0);
+            z += e[k];
+            topi[t * topk + k] = bi;
+        }
+        for (int k = 0; k < topk; ++k) topw[t * topk + k] = e[k] / z;
+    }
+    free(taken);
+}
+void fnx_o_topk_softmax(const float* logits, int stride, int T, int nexp, int topk, int* topi, float* topw) {
+    float* p = (float*) malloc((size_t) nexp * sizeof(float));
+    for (int t = 0; t < T; ++t) {
+        const float* l = logits + (size_t) t * stride;
+        float m = -INFINITY, z = 0.f;
+        for (int i = 0; i < nexp; ++i) m = fmaxf(m, l[i]);
+        for (int i = 0; i < nexp; ++i) {
+            p[i] = expf(l[i] - m);
+            z += p[i];
+        }
+        for (int i = 0; i < nexp; ++i) p[i] = p[i] / z;
+        float sel = 0.f;
+        for (int k = 0; k < topk; ++k) {
+            float bv = p[0];
+            int bi = 0;
+            for (int i = 1; i < nexp; ++i)
+                if (p[i] > bv) {
+                    bv = p[i];
+                    bi = i;
+                }
+            topi[t * topk + k] = bi;
+            topw[t * topk + k] = bv;
+            p[bi] = -1.0f;
+        }
+        for (int k = 0; k < topk; ++k) sel += topw[t * topk + k];
+        for (int k = 0; k < topk; ++k) topw[t * topk + k] /= sel;
+    }
+    free(p);
+}
+int fnx_o_jobs(const int* topi, int T, int topk, fnx_o_job* gu, fnx_o_job* dn) {
+    int nj = 0;
+    for (int t = 0; t < T; ++t)
+        for (int k = 0; k < topk; ++k) {
+            const int e = topi[t * topk + k], pair = t * topk + k;
+            int j = 0;
+            while (j < nj && gu[j].w != e) ++j;
+            if (j == nj) {
+                gu[j].w = e;
+                gu[j].n = 0;
+                dn[j].w = e;
+                dn[j].n = 0;
+                ++nj;
+            }
+            gu[j].y[gu[j].n] = t;
+            gu[j].out[gu[j].n] = pair;
+            ++gu[j].n;
+            dn[j].y[dn[j].n] = pair;
+            dn[j].out[dn[j].n] = pair;
+            ++dn[j].n;
+        }
+    return nj;
+}
+
+/* ---------------------------------------------------------------- swiglu, combine (kernels.cu:67-68, 400-419) */
+static float sigm(float x) { return 1.0f / (1.0f + expf(-x)); }
+static float silu(float x) { return x / (1.0f + expf(-x)); }
+void fnx_o_swiglu_q8_1(const float* g, const float* u, uint8_t* q, int n, int rows) {
+    float h[32];
+    for (int r = 0; r < rows; ++r)
+        for (int b = 0; b < n / 32; ++b) {
+            for (int j = 0; j < 32; ++j) {
+                const size_t i = (size_t) r * n + 32 * b + j;
+                h[j] = silu(g[i]) * u[i];
+            }
+            q8_1_block(h, q + ((size_t) r * (n / 32) + b) * Q8_1_BLOCK);
+        }
+}
+void fnx_o_swiglu_stacked_q8_1(const float* gu, uint8_t* hq, int ffs, int rows) {
+    float h[32];
+    for (int r = 0; r < rows; ++r) {
+        const float* g = gu + (size_t) r * 2 * ffs;
+        for (int b = 0; b < ffs / 32; ++b) {
+            for (int j = 0; j < 32; ++j) h[j] = silu(g[32 * b + j]) * g[ffs + 32 * b + j];
+            q8_1_block(h, hq + ((size_t) r * (ffs / 32) + b) * Q8_1_BLOCK);
+        }
+    }
+}
+void fnx_o_moe_combine(const float* part, const float* topw, const float* sh, const float* sh_logit, int sh_logit_stride,
+                       float* out, int T, int n, int topk) {
+    for (int t = 0; t < T; ++t) {
+        const float gate = sigm(sh_logit[(size_t) t * sh_logit_stride]);
+        for (int i = 0; i < n; ++i) {
+            float s = 0.f;
+            for (int k = 0; k < topk; ++k) s = fmaf(topw[t * topk + k], part[((size_t) t * topk + k) * n + i], s);
+            out[(size_t) t * n + i] = s + gate * sh[(size_t) t * n + i];
+        }
+    }
+}
+
+/* ---------------------------------------------------------------- argmax (kernels.cu:1045-1083) */
+static uint32_t fkey(float v) {
+    uint32_t u;
+    memcpy(&u, &v, 4);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+static float fkey_inv(uint32_t k) {
+    const uint32_t u = (k & 0x80000000u) ? (k & 0x7fffffffu) : ~k;
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+unsigned fnx_o_argmax(const float* logits, int rows, int T, int v0, float* best_v, int* best_i) {
+    unsigned err = 0;
+    for (int t = 0; t < T; ++t) {
+        const float* r = logits + (size_t) t * rows;
+        uint64_t best = 0;
+        for (int i = 0; i < rows; ++i) {
+            if (!isfinite(r[i])) err |= 16u;
+            const uint64_t k = (uint64_t) fkey(r[i]) << 32 | (uint32_t) ~(uint32_t) i;
+            if (k > best) best = k;
+        }
+        best_v[t] = fkey_inv((uint32_t) (best >> 32));
+        best_i[t] = (int) ~(uint32_t) best + v0;
+    }
+    return err;
+}
+
+/* ---------------------------------------------------------------- prompt lookup, acceptance */
+#define LOOKUP_MIN 3       /* session.cpp:18 */
+#define IMAGE_TOK (1 << 30) /* engine.hpp:84 */
+int fnx_o_lookup_drafts(const int* ctx, int n_ctx, int key_n, int lk, int d1, int* out, int* match) {
+    int nr = 0;
+    if (match) *match = -1;
+    if (lk == 0 || n_ctx <= key_n) return 0;
+    const long n0 = (long) n_ctx - key_n;
+    for (long s = n0; s-- > 0;)
+        if (memcmp(ctx + s, ctx + n0, (size_t) key_n * sizeof(int)) == 0) {
+            if (s + key_n < n_ctx && (d1 < 0 || ctx[s + key_n] == d1)) {
+                int m = key_n;
+                while (m < lk && (long) (m - key_n) < s && ctx[s - 1 - (m - key_n)] == ctx[n0 - 1 - (m - key_n)]) ++m;
+                int k = m > LOOKUP_MIN ? m : LOOKUP_MIN;
+                if (k > lk) k = lk;
+                long end = s + key_n + k;
+                if (end > n_ctx) end = n_ctx;
+                for (long i = s + key_n; i < end; ++i) out[nr++] = ctx[i];
+                if (match) *match = (int) s;
+            }
+            break;
+        }
+    for (int i = 0; i < nr; ++i)
+        if (out[i] >= IMAGE_TOK) {
+            nr = i;
+            break;
+        }
+    return nr;
+}
+int fnx_o_lookup_fixed(const int* ctx, int n_ctx, int key_n, int lk, int d1, int* out) {
+    int nr = 0;
+    if (lk == 0 || n_ctx <= key_n) return 0;
+    const long n0 = (long) n_ctx - key_n;
+    for (long st = n0; st-- > 0;)
+        if (memcmp(ctx + st, ctx + n0, (size_t) key_n * sizeof(int)) == 0) {
+            if (st + key_n < n_ctx && ctx[st + key_n] == d1) {
+                long end = st + key_n + lk;
+                if (end > n_ctx) end = n_ctx;
+                for (long i = st + key_n; i < end; ++i) out[nr++] = ctx[i];
+            }
+            break;
+        }
+    return nr;
+}
+int fnx_o_accept_greedy(const int* rows, const int* o, int R) {
+    int n = 1;
+    while (n < R && rows[n] == o[n - 1]) ++n;
+    return n;
+}
+
+/* ---------------------------------------------------------------- prefill jobs (prefill.cu:320-377)
+ * jobs are arrays of ints {w, n, y[pf_job], out[pf_job]} */
+int fnx_o_pf_jobs(const int* topi, int C, int topk, int nexp, int pf_job, int* jobs_gu, int* jobs_dn, int* cnt) {
+    const int P = C * topk, js = 2 + 2 * pf_job;
+    int* jbase = (int*) malloc((size_t) nexp * sizeof(int));
+    int* fill = (int*) calloc((size_t) nexp, sizeof(int));
+    memset(cnt, 0, (size_t) nexp * sizeof(int));
+    for (int p = 0; p < P; ++p) ++cnt[topi[p]];
+    int nj = 0;
+    for (int e = 0; e < nexp; ++e) {
+        jbase[e] = nj;
+        nj += (cnt[e] + pf_job - 1) / pf_job;
+    }
+    for (int p = 0; p < P; ++p) { /* ascending pair index: a pair always lands in the same job and slot */
+        const int e = topi[p], s = fill[e]++, j = jbase[e] + s / pf_job, k = s % pf_job;
+        int *g = jobs_gu + (size_t) j * js, *d = jobs_dn + (size_t) j * js;
+        g[2 + k] = p / topk;
+        g[2 + pf_job + k] = p;
+        d[2 + k] = p;
+        d[2 + pf_job + k] = p;
+        if (k == 0) {
+            const int left = cnt[e] - (s / pf_job) * pf_job;
+            g[0] = d[0] = e;
+            g[1] = d[1] = left < pf_job ? left : pf_job;
+        }
+    }
+    free(jbase);
+    free(fill);
+    return nj;
+}
+
+/* ---------------------------------------------------------------- one MoE verify layer */
+void fnx_o_moe_verify_layer(const fnx_o_moe_layer* L, const float* x, int T, float* out, float* logits_out, int* topi_out,
+                            float* topw_out, int* njobs_out, int threads) {
+    const int n = L->n, ff = L->ff, nexp = L->nexp, topk = L->topk, P = T * topk;
+    const size_t gu_stride = (size_t) 2 * ff * (n / 256) * IQ3S_BLOCK, dn_stride = (size_t) n * (ff / 256) * IQ3S_BLOCK;
+    if (threads <= 0) threads = 1;
+#ifdef _OPENMP
+    const int prev = omp_get_max_threads();
+    omp_set_num_threads(threads);
+#endif
+    uint8_t* xq = (uint8_t*) malloc((size_t) T * (n / 32) * Q8_1_BLOCK);
+    float* logits = (float*) malloc((size_t) T * (nexp + 1) * sizeof(float));
+    float* lt = (float*) malloc((size_t) T * (nexp + 1) * sizeof(float));
+    int* topi = (int*) malloc((size_t) P * sizeof(int));
+    float* topw = (float*) malloc((size_t) P * sizeof(float));
+    fnx_o_job* jgu = (fnx_o_job*) calloc((size_t) P + 1, sizeof(fnx_o_job));
+    fnx_o_job* jdn = (fnx_o_job*) calloc((size_t) P + 1, sizeof(fnx_o_job));
+    float* gu = (float*) malloc((size_t) (P + T) * 2 * ff * sizeof(float));
+    uint8_t* hq = (uint8_t*) malloc((size_t) (P + T) * (ff / 32) * Q8_1_BLOCK);
+    float* part = (float*) malloc((size_t) (P + T) * n * sizeof(float));
+
+    fnx_o_quantize_q8_1(x, xq, n, T);
+    fnx_o_gemv_f32(L->router, x, lt, nexp + 1, n, T); /* lt[t][row] with stride nexp + 1 */
+    memcpy(logits, lt, (size_t) T * (nexp + 1) * sizeof(float));
+    fnx_o_topk_logits(logits, nexp + 1, T, nexp, topk, topi, topw);
+    const int nj = fnx_o_jobs(topi, T, topk, jgu, jdn);
+    /* routed experts */
+    fnx_o_mmvq_iq3s(L->gu, gu_stride, NULL, 2 * ff, n, jgu, nj, xq, gu, 2 * ff, threads);
+    /* shared expert: one job of all T rows, outputs at rows P + t (kernels.hpp:277-282) */
+    fnx_o_job sh;
+    sh.w = 0;
+    sh.n = T;
+    for (int t = 0; t < T; ++t) {
+        sh.y[t] = t;
+        sh.out[t] = P + t;
+    }
+    fnx_o_mmvq_iq3s(L->sh_gu, 0, NULL, 2 * ff, n, &sh, 1, xq, gu, 2 * ff, threads);
+    fnx_o_swiglu_stacked_q8_1(gu, hq, ff, P + T);
+    fnx_o_mmvq_iq3s(L->down, dn_stride, NULL, n, ff, jdn, nj, hq, part, n, threads);
+    for (int t = 0; t < T; ++t) sh.y[t] = P + t;
+    fnx_o_mmvq_iq3s(L->sh_down, 0, NULL, n, ff, &sh, 1, hq, part, n, threads);
+    fnx_o_moe_combine(part, topw, part + (size_t) P * n, logits + nexp, nexp + 1, out, T, n, topk);
+
+    if (logits_out) memcpy(logits_out, logits, (size_t) T * (nexp + 1) * sizeof(float));
+    if (topi_out) memcpy(topi_out, topi, (size_t) P * sizeof(int));
+    if (topw_out) memcpy(topw_out, topw, (size_t) P * sizeof(float));
+    if (njobs_out) *njobs_out = nj;
+    free(xq);
+    free(logits);
+    free(lt);
+    free(topi);
+    free(topw);
+    free(jgu);
+    free(jdn);
+    free(gu);
+    free(hq);
+    free(part);
+#ifdef _OPENMP
+    omp_set_num_threads(prev);
+#endif
+}
+
+/* ---------------------------------------------------------------- selftest.cu:29-40 */
+void fnx_o_rng_init(fnx_o_rng* r, unsigned long long seed) { r->s = seed * 2685821657736338717ull + 1442695040888963407ull; }
+unsigned fnx_o_rng_next(fnx_o_rng* r) {
+    r->s ^= r->s >> 12;
+    r->s ^= r->s << 25;
+    r->s ^= r->s >> 27;
+    return (unsigned) ((r->s * 2685821657736338717ull) >> 32);
+}

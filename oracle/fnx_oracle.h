@@ -1,0 +1,126 @@
+/* CPU oracle for the speculative-decode verify path.
+ *
+ * TEST INFRASTRUCTURE ONLY. This is a plain-C restatement of the reference engine's arithmetic for the path
+ * (IQ3_S x q8_1 expert mat-vec, router top-k, SwiGLU, combine, argmax, prompt-lookup drafting, greedy acceptance).
+ * Only the test-suite, the smoke check and the benchmark's CPU-baseline leg may link or call it. The device library
+ * never does: it has no CPU fallback and fails loudly when its HIP code object is missing.
+ *
+ * Every function cites the reference lines it follows (paths relative to the reference's root).
+ *
+ * Parity status of each function (what pins it is in tests/test_oracle_*.py):
+ *   pinned:   h2f/f2h, iq3s_dequant (reference's own tensor_convert.hpp compiled as oracle/_ref + closed forms),
+ *             dp4a (selftest.cu's generator), vec_dot/mmvq (vs dequant in f64), q8_1 (closed forms, round trip),
+ *             route/topk (two in-tree definitions agree; brute-force sort), jobs (two in-tree builders' invariants),
+ *             argmax (brute force + tie/NaN cases), lookup (second in-tree implementation + brute force), accept
+ *             (speculative == greedy invariant), swiglu/combine (f64 closed forms).
+ *   parity unpinned: fnx_o_iq3s_quantize_row (the encoder). ggml's quantize_row_iq3_s is not in the reference tree
+ *             (third_party/ggml holds only a commit hash) and nothing in the reference calls or tests it. The encoder
+ *             here is this build's own; parity of the path is defined from the quantised bytes onward.
+ *   parity unpinned: ggml's CPU kernel ggml_vec_dot_iq3_s_q8_K (256-wide Q8_K activations). Not in the tree, never
+ *             called by the reference. The oracle follows the reference's own arithmetic (q8_1, 32-wide blocks).
+ */
+#ifndef FNX_ORACLE_H
+#define FNX_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FNX_O_MAXT 16
+
+/* engine/src/kernels.hpp:18-23 */
+typedef struct {
+    int w;
+    int n;
+    int y[FNX_O_MAXT];
+    int out[FNX_O_MAXT];
+} fnx_o_job;
+
+/* half <-> float, engine/src/tensor_convert.hpp:23-50 */
+float fnx_o_h2f(uint16_t h);
+uint16_t fnx_o_f2h(float x);
+
+/* p100_compat.h:18-22 (the scalar definition of the 4-way signed byte dot) */
+int fnx_o_dp4a(int a, int b, int c);
+
+/* IQ3_S: 110-byte blocks of 256 weights. tensor_convert.hpp:295-322 */
+void fnx_o_iq3s_dequant(const uint8_t* src, size_t n, float* y);
+/* this build's own encoder (parity unpinned, see header) */
+void fnx_o_iq3s_quantize(const float* w, size_t n, uint8_t* dst);
+
+/* q8_1 activation rows: 36-byte blocks {half d; half sum; int8 qs[32]}. kernels.cu:131-145 */
+void fnx_o_quantize_q8_1(const float* x, uint8_t* q, int n, int rows);
+
+/* one lane's share of a super-block: iq3s_x.cuh:4-41. blk: the 110-byte block; q8: the super-block's 8 q8_1 blocks */
+float fnx_o_vec_dot_iq3s_q8_1(const uint8_t* blk, const uint8_t* q8, int iqs);
+
+/* out[job.out[j]][r] = W[job.w][r] . y[job.y[j]]   (kernels.cu:192-229, moe.cuh:519-548: lane order and butterfly) */
+void fnx_o_mmvq_iq3s(const uint8_t* wbase, size_t w_stride, const uint8_t* const* ep, int nrows, int ncols,
+                     const fnx_o_job* jobs, int njobs, const uint8_t* y, float* out, int out_stride, int threads);
+
+/* exact variant: dequantised weights x f32 activations summed in double */
+void fnx_o_gemv_exact(const uint8_t* w, int nrows, int ncols, const float* x, int T, double* out);
+
+/* y[t][r] = W[r] . x[t], f32 or bf16 weights. Semantics of kernels.cu:239-287 (k_gemv_f32); the summation order is
+ * this build's fixed one, shared bit for bit with the device kernel: 64 lanes, lane l takes float4 chunks l, l+64, ...
+ * in order with fmaf on x,y,z,w, then an xor-butterfly 32,16,8,4,2,1 of plain adds. */
+void fnx_o_gemv_f32(const float* W, const float* x, float* y, int rows, int n, int T);
+void fnx_o_gemv_bf16(const uint16_t* W, const float* x, float* y, int rows, int n, int T);
+
+/* top-k by logit, ties to the lower index, w_k = exp(l_k - l_0) / sum (pick order). moe.cuh:382-411 */
+void fnx_o_topk_logits(const float* logits, int stride, int T, int nexp, int topk, int* topi, float* topw);
+/* softmax over all experts, top-k of the probabilities, renormalised. kernels.cu:338-378 */
+void fnx_o_topk_softmax(const float* logits, int stride, int T, int nexp, int topk, int* topi, float* topw);
+/* distinct experts in first-pick order. kernels.cu:381-398. returns the job count */
+int fnx_o_jobs(const int* topi, int T, int topk, fnx_o_job* gu, fnx_o_job* dn);
+
+/* h = silu(g) * u -> q8_1, rows of n. kernels.cu:400-410 */
+void fnx_o_swiglu_q8_1(const float* g, const float* u, uint8_t* q, int n, int rows);
+/* rows of [gate (ffs) | up (ffs)] -> q8_1 rows of ffs. moe.cuh:597-608, kernels.cu:2475-2490 */
+void fnx_o_swiglu_stacked_q8_1(const float* gu, uint8_t* hq, int ffs, int rows);
+/* out[t] = sum_k topw[t][k] part[t*topk+k] (fmaf, k ascending) + sigmoid(sh_logit[t]) sh[t]. kernels.cu:412-419 */
+void fnx_o_moe_combine(const float* part, const float* topw, const float* sh, const float* sh_logit, int sh_logit_stride,
+                       float* out, int T, int n, int topk);
+
+/* greatest value, lowest index on ties; returns the error word (bit 16: NaN or inf). kernels.cu:1045-1083 */
+unsigned fnx_o_argmax(const float* logits, int rows, int T, int v0, float* best_v, int* best_i);
+
+/* session.cpp:428-447 with the key length as a parameter (3 = the reference's LOOKUP_N). returns the draft count */
+int fnx_o_lookup_drafts(const int* ctx, int n_ctx, int key_n, int lk, int d1, int* out, int* match);
+/* tools/fnx_run.cpp:1046-1059: the fixed-length form */
+int fnx_o_lookup_fixed(const int* ctx, int n_ctx, int key_n, int lk, int d1, int* out);
+/* session.cpp:573 */
+int fnx_o_accept_greedy(const int* rows, const int* o, int R);
+
+/* prefill routing: top-k per row, histogram, jobs of <= pf_job rows per expert, pairs in ascending order.
+ * prefill.cu:288-377. jobs: arrays of {w, n, y[pf_job], out[pf_job]} ints. returns the job count */
+int fnx_o_pf_jobs(const int* topi, int C, int topk, int nexp, int pf_job, int* jobs_gu, int* jobs_dn, int* cnt);
+
+/* one MoE verify layer (engine.cu:1569-1757 without the cards/streaming): router -> top-k -> jobs -> gate|up ->
+ * swiglu q8_1 -> down -> shared expert -> combine. Weights IQ3_S; experts at base + e*stride. */
+typedef struct {
+    int n, ff, nexp, topk;           /* hidden, expert width, experts, picks */
+    const float* router;             /* [nexp + 1][n] f32: the router's rows, then the shared expert's gate */
+    const uint8_t* gu;               /* [nexp][2 ff][n] IQ3_S */
+    const uint8_t* down;             /* [nexp][n][ff] IQ3_S */
+    const uint8_t* sh_gu;            /* [2 ff][n] IQ3_S */
+    const uint8_t* sh_down;          /* [n][ff] IQ3_S */
+} fnx_o_moe_layer;
+/* out [T][n]; optional outputs (may be null): logits [T][nexp+1], topi/topw [T][topk], njobs */
+void fnx_o_moe_verify_layer(const fnx_o_moe_layer* L, const float* x, int T, float* out, float* logits, int* topi,
+                            float* topw, int* njobs, int threads);
+
+/* xorshift generator of the reference's self-test (selftest.cu:29-40) */
+typedef struct { unsigned long long s; } fnx_o_rng;
+void fnx_o_rng_init(fnx_o_rng* r, unsigned long long seed);
+unsigned fnx_o_rng_next(fnx_o_rng* r);
+
+int fnx_o_threads(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
