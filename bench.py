@@ -1,0 +1,166 @@
+#!/usr/bin/env python3
+"""Benchmark of the MoE verify step (BASELINE config 2) on one MI355X.
+
+A step = one MoE layer of a verify window: T = 16 rows, hidden 2048, 512 IQ3_S experts (gate|up 2048 -> 2 x 512, down
+512 -> 2048), top-10, one shared expert, f32 router of 513 rows. Inputs are resident in HBM before the timed region.
+Steps cycle through LAYERS distinct weight sets (about 11 GB) and fresh activations so that a step's ~190 MB working set
+is cold with respect to the 256 MB Infinity Cache.
+
+Prints ONE JSON line: whole-step throughput, the roofline of the dominant kernel (the routed gate|up mat-vec, timed on
+its own with events on the launch stream) and the CPU baseline (the oracle on the host's cores, bounded sample).
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+N, FF, NEXP, TOPK, T = 2048, 512, 512, 10, 16
+HBM_PEAK = 8.0e12
+IQ3S_BLOCK = 110
+GU_BYTES = 2 * FF * (N // 256) * IQ3S_BLOCK      # 901,120 per expert
+DN_BYTES = N * (FF // 256) * IQ3S_BLOCK          # 450,560 per expert
+ROUTER_BYTES = (NEXP + 1) * N * 4                # 4,202,496
+XIO_BYTES = 2 * T * N * 4                        # x in + out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--layers", type=int, default=16, help="distinct weight sets cycled through")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0: skip)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    import fnx_gpu
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = fnx_gpu.Dev()
+    pkg, lib, t = dev.pkg, dev.lib, torch
+    g = torch.Generator(device="cuda")
+    g.manual_seed(1234)
+
+    def rand_iq3s(nblocks):
+        b = torch.randint(0, 256, (nblocks, IQ3S_BLOCK), dtype=torch.uint8, device="cuda", generator=g)
+        d = (torch.rand(nblocks, device="cuda", generator=g) * 3e-4 + 1e-5).to(torch.float16)
+        b[:, 0:2] = d.view(torch.uint8).reshape(nblocks, 2)
+        return b.reshape(-1)
+
+    layers = []
+    for _ in range(args.layers):
+        router = (torch.randn((NEXP + 1, N), device="cuda", generator=g) * 0.02).contiguous()
+        gu = rand_iq3s(NEXP * 2 * FF * N // 256)
+        down = rand_iq3s(NEXP * N * FF // 256)
+        sh_gu = rand_iq3s(2 * FF * N // 256)
+        sh_down = rand_iq3s(N * FF // 256)
+        L = pkg.MoeLayer(N, FF, NEXP, TOPK, router.data_ptr(), 0, pkg.dw(gu, N, 2 * FF), GU_BYTES, pkg.dw(down, FF, N), DN_BYTES,
+                         pkg.dw(sh_gu, N, 2 * FF), pkg.dw(sh_down, FF, N))
+        layers.append((L, router, gu, down, sh_gu, sh_down))
+    NX = 64
+    xs = torch.randn((NX, T, N), device="cuda", generator=g)
+    outs = torch.zeros((NX, T, N), device="cuda")
+    P = T * TOPK
+    ws_t = dict(xq=dev.zeros(T * (N // 32) * 36, t.uint8), logits=dev.zeros((T, NEXP + 1), t.float32), topi=dev.zeros((T, TOPK), t.int32),
+                topw=dev.zeros((T, TOPK), t.float32), jobs_gu=dev.zeros((P + 1) * 136, t.uint8), jobs_dn=dev.zeros((P + 1) * 136, t.uint8),
+                njobs=dev.zeros(2, t.int32), gu=dev.zeros((P + T, 2 * FF), t.float32), part=dev.zeros((P + T, N), t.float32))
+    ws = pkg.MoeWs(*(ws_t[k].data_ptr() for k in ("xq", "logits", "topi", "topw", "jobs_gu", "jobs_dn", "njobs", "gu", "part")))
+    st = dev.st()
+
+    def step(i):
+        L = layers[i % args.layers][0]
+        x = xs[i % NX]
+        dev.ok(lib.fnx_moe_verify_layer(C.byref(L), x.data_ptr(), T, outs[i % NX].data_ptr(), C.byref(ws), st))
+
+    # ---- whole steps
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(args.warmup + i)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+
+    # ---- distinct experts per step (for the algorithmic bytes), from the routing the steps produced
+    njobs = []
+    for i in range(min(args.steps, 64)):
+        step(args.warmup + i)
+        torch.cuda.synchronize()
+        njobs.append(int(ws_t["njobs"][0].item()))
+    u_mean = float(np.mean(njobs))
+    step_bytes = u_mean * (GU_BYTES + DN_BYTES) + (GU_BYTES + DN_BYTES) + ROUTER_BYTES + XIO_BYTES
+
+    # ---- the dominant kernel on its own: routed gate|up over the step's jobs, events on the launch stream
+    xq_bytes = T * (N // 32) * 36
+    evs = []
+    reps = max(50, min(args.steps, 200))
+    for i in range(reps + 10):
+        L, x = layers[i % args.layers][0], xs[i % NX]
+        # routing for this (layer, x), then only the gate|up launch between the events
+        dev.ok(lib.fnx_quantize_q8_1(x.data_ptr(), ws.xq, N, T, st))
+        dev.ok(lib.fnx_router_route(L.router, 0, x.data_ptr(), ws.logits, T, N, NEXP, TOPK, ws.topi, ws.topw, ws.jobs_gu, ws.jobs_dn, ws.njobs, st))
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        dev.ok(lib.fnx_moe_gate_up(C.byref(L.gu), L.gu_stride, ws.jobs_gu, ws.njobs, P, ws.xq, ws.gu, st))
+        e1.record()
+        evs.append((e0, e1, i))
+    torch.cuda.synchronize()
+    k_ms = float(np.mean([a.elapsed_time(b) for a, b, i in evs[10:]]))
+    # algorithmic bytes of one launch: the distinct experts' gate|up blocks, the window's q8_1 rows, the f32 outputs
+    k_bytes = u_mean * GU_BYTES + xq_bytes + P * 2 * FF * 4
+    achieved = k_bytes / (k_ms * 1e-3)
+
+    # ---- CPU baseline: the oracle on the host's cores, same workload (layer set 0), bounded sample
+    cpu = None
+    if args.cpu_seconds > 0:
+        import oracle_lib
+        oracle = oracle_lib.Oracle()
+        threads = min(os.cpu_count() or 1, 16)
+        L, router, gu, down, sh_gu, sh_down = layers[0]
+        h = [a.cpu().numpy() for a in (router, gu, down, sh_gu, sh_down)]
+        xh = xs[0].cpu().numpy()
+        r = oracle.moe_verify_layer(N, FF, NEXP, TOPK, *h, xh, threads=threads)   # warm-up, and a last parity check
+        dev.ok(lib.fnx_moe_verify_layer(C.byref(L), xs[0].data_ptr(), T, outs[0].data_ptr(), C.byref(ws), st))
+        torch.cuda.synchronize()
+        err = float(np.linalg.norm(outs[0].cpu().numpy() - r["out"]) / np.linalg.norm(r["out"]))
+        same = bool(np.array_equal(ws_t["topi"].cpu().numpy(), r["topi"]))
+        c0 = time.perf_counter()
+        n_cpu = 0
+        while time.perf_counter() - c0 < args.cpu_seconds or n_cpu < 2:
+            oracle.moe_verify_layer(N, FF, NEXP, TOPK, *h, xh, threads=threads)
+            n_cpu += 1
+        cdt = time.perf_counter() - c0
+        cpu = {"value": n_cpu / cdt, "unit": "layer-steps/s", "cores": threads, "kind": "port",
+               "sample": f"{n_cpu} layer-steps of the same workload (weight set 0, T=16) on the oracle (q8_1 x IQ3_S restated from the reference, not ggml's Q8_K kernel)",
+               "parity_rel_l2": err, "routing_identical": same}
+
+    line = {
+        "metric": "MoE verify steps/sec at T=16 + IQ3_S expert GEMV achieved HBM GB/s (% peak)",
+        "value": args.steps / dt,
+        "unit": "layer-steps/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8 x IQ3_S (i32 dot, f32 accumulate)", "data": "synthetic",
+        "config": {"workload": "config 2: one MoE verify layer, T=16, hidden 2048, 512 IQ3_S experts top-10, SwiGLU ff 512, shared expert, f32 router",
+                   "weight_sets": args.layers, "distinct_experts_per_step": u_mean, "step_algorithmic_bytes": step_bytes,
+                   "step_hbm_frac": step_bytes / (ms_per_step * 1e-3) / HBM_PEAK},
+        "roofline": {"bound": "hbm", "kernel": "k_iq3s_jobs<64> (routed gate|up)", "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK, "traffic": None, "kernel_ms": k_ms, "algorithmic_bytes": k_bytes},
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

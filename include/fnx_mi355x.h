@@ -1,0 +1,155 @@
+/* fnx_mi355x.h - C ABI of the MI355X (gfx950) verify-path library.
+ *
+ * Every entry point replaces one operator of the reference engine's launch-wrapper API
+ * (engine/src/kernels.hpp, namespace fnx) or one host function of its session loop (engine/src/session.cpp), cited
+ * per declaration. Conventions kept from the reference:
+ *   - activations are device float rows, one row per token or per routed pair t*topk+k; the shared expert's rows sit
+ *     at T*topk+t (kernels.hpp:1-2, 277-282);
+ *   - quantised weights are raw ggml blocks, row-major over output rows, expert e at p + e*stride or ep[e]
+ *     (model.hpp:84-94);
+ *   - work lists are device arrays of fnx_job with a device-resident count; the grid is sized without reading it;
+ *   - `st` is a hipStream_t; every device call is asynchronous on it, allocates nothing and never synchronises, so a
+ *     caller may capture a whole window into a graph (engine_common.cu:993-1007);
+ *   - the caller owns every buffer.
+ * Differences: functions return an int status (0 = ok) instead of throwing, the message is in fnx_last_error()
+ * (thread-local); the reference's compile-time model constants (N, NEXP, TOPK) are run-time arguments.
+ * Data faults go to a device error word as in the reference (bit 16: a non-finite logit seen by argmax).
+ */
+#ifndef FNX_MI355X_H
+#define FNX_MI355X_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FNX_MAXT 16        /* rows per verify window (model.hpp:43) */
+#define FNX_PF_JOB 64      /* rows per prefill job (kernels.hpp:27-30) */
+#define FNX_T_IQ3_S 21u    /* ggml type id (gguf.hpp:22-27) */
+#define FNX_IQ3S_BLOCK 110 /* bytes per 256 weights */
+#define FNX_Q8_1_BLOCK 36  /* bytes per 32 activations: half d, half sum, int8 qs[32] */
+#define FNX_ERR_NONFINITE 16u /* error-word bit (engine_impl.hpp:211-218) */
+
+/* kernels.hpp:18-23 */
+typedef struct fnx_job {
+    int w;             /* matrix index: an expert, or 0 */
+    int n;             /* rows of the job */
+    int y[FNX_MAXT];   /* activation rows (q8_1) */
+    int out[FNX_MAXT]; /* output rows */
+} fnx_job;
+
+/* kernels.hpp:32-37 */
+typedef struct fnx_bigjob {
+    int w;
+    int n;
+    int y[FNX_PF_JOB];
+    int out[FNX_PF_JOB];
+} fnx_bigjob;
+
+/* model.hpp:84-94 (DW) without the split-Q8_0 twin, which this path does not use */
+typedef struct fnx_dw {
+    const void* p;          /* raw ggml blocks, row-major over output rows */
+    uint32_t type;          /* FNX_T_IQ3_S */
+    int n_in, n_out;        /* columns, rows */
+    size_t row_bytes;       /* n_in / 256 * 110 */
+    const void* const* ep;  /* optional device table: expert e's matrix; null: expert e at p + e * stride */
+} fnx_dw;
+
+/* message of the calling thread's last failed call ("" if none) */
+const char* fnx_last_error(void);
+/* library build id, and whether a usable GPU is present (no device work is started) */
+const char* fnx_version(void);
+
+/* kernels.hpp:41  quantize_q8_1: f32 rows of n -> q8_1 blocks, ggml's rounding (kernels.cu:131-145) */
+int fnx_quantize_q8_1(const float* x, void* q, int n, int rows, void* st);
+
+/* kernels.hpp:49  mmvq: out[job.out[j]][r] = W[job.w][r] . y[job.y[j]] for every job in jobs[0..*njobs)
+ * (njobs null: njobs_max jobs). y: q8_1 rows of W->n_in. */
+int fnx_mmvq(const fnx_dw* W, size_t w_stride, const fnx_job* jobs, const int* njobs, int njobs_max, const void* y,
+             float* out, int out_stride, void* st);
+
+/* kernels.hpp:54-55  gemv_f32 / gemv_bf16: y[t][r] = W[r] . x[t], W [rows][n], T <= 16, n % 256 == 0 */
+int fnx_gemv_f32(const float* W, const float* x, float* y, int rows, int n, int T, void* st);
+int fnx_gemv_bf16(const uint16_t* W, const float* x, float* y, int rows, int n, int T, void* st);
+
+/* kernels.hpp:79  route: logits [T][nexp] -> top-k (softmax, renormalised; ties to the lower index), the gate|up
+ * jobs (rows = tokens, outputs = pairs t*topk+k) and the down jobs (rows = outputs = pairs); njobs[0] = njobs[1] =
+ * the count. logits_stride: floats between rows (nexp, or nexp + 1 when the rows carry the shared gate's logit) */
+int fnx_route(const float* logits, int logits_stride, int T, int nexp, int topk, int* topi, float* topw, fnx_job* jobs_gu,
+              fnx_job* jobs_dn, int* njobs, void* st);
+
+/* kernels.hpp:294  router_route: logits rows of nexp + 1 = W [nexp + 1][n] . x (the router's rows, then the shared
+ * expert's gate), top-k per token by logit, weights the selected softmax renormalised, jobs as route. W: f32
+ * (w_bf16 = 0) or bf16 bits (w_bf16 = 1). njobs[0] = the count; njobs[1] is left at zero as in the reference. */
+int fnx_router_route(const void* W, int w_bf16, const float* x, float* logits, int T, int n, int nexp, int topk, int* topi,
+                     float* topw, fnx_job* jobs_gu, fnx_job* jobs_dn, int* njobs, void* st);
+
+/* kernels.hpp:81   swiglu_q8_1: h[r] = silu(g[r]) * u[r] -> q8_1, rows of n */
+int fnx_swiglu_q8_1(const float* g, const float* u, void* q, int n, int rows, void* st);
+/* kernels.hpp:349  swiglu_stacked_q8_1: T rows of [gate (ffs) | up (ffs)] -> q8_1 rows of ffs */
+int fnx_swiglu_stacked_q8_1(const float* gu, void* hq, int ffs, int T, void* st);
+
+/* kernels.hpp:319  moe_gate_up: gu rows of 2*ffs = A->n_out: [gate | up]; expert stride sa; xq: q8_1 rows of A->n_in */
+int fnx_moe_gate_up(const fnx_dw* A, size_t sa, const fnx_job* jobs, const int* njobs, int njobs_max, const void* xq, float* gu,
+                    void* st);
+/* kernels.hpp:343  moe_down: part rows of A->n_out from silu(gate) * up of the gu rows (rows of 2 * A->n_in).
+ * Like the reference (moe.cuh:592-594) the q8_1 rows of h live in one library-owned device buffer, so one MoE may be
+ * in flight per device; njobs_max (the window's pairs) <= 176. */
+int fnx_moe_down(const fnx_dw* A, size_t sa, const fnx_job* jobs, const int* njobs, int njobs_max, const float* gu, float* part,
+                 void* st);
+/* kernels.hpp:83   moe_combine: out[t] = sum_k topw[t][k] * part[t*topk + k] + sigmoid(sh_logit[t * stride]) * sh[t] */
+int fnx_moe_combine(const float* part, const float* topw, const float* sh, const float* sh_logit, int sh_logit_stride, float* out,
+                    int T, int n, int topk, void* st);
+
+/* kernels.hpp:433  argmax: best[t] = (value, index + v0), the lowest index on ties. keys: 16 words, zeroed once (left
+ * at zero). err bit 16: a logit was NaN or inf */
+int fnx_argmax(const float* logits, int rows, int T, int v0, float* best_v, int* best_i, unsigned long long* keys, unsigned* err,
+               void* st);
+
+/* session.hpp:55-58  lookup_drafts (host memory): the tokens after the latest earlier place of ctx's last key_n
+ * tokens, if the first of them is d1 (d1 < 0: whatever it is), as many as the match is long, 3 to lk. key_n = 3 is
+ * the reference's LOOKUP_N; 2 and 4 are this build's parameterisation. Returns the draft count (<= lk) or -1 on a
+ * bad argument; *match (may be null) = the run's start or -1. */
+int fnx_lookup_drafts(const int* ctx, int n_ctx, int key_n, int lk, int d1, int* out, int* match);
+/* the same on device memory, asynchronous: ctx, d1, out (lk ints), n_out, match are device pointers */
+int fnx_lookup_drafts_dev(const int* ctx, int n_ctx, int key_n, int lk, const int* d1, int* out, int* n_out, int* match, void* st);
+
+/* session.cpp:573  greedy acceptance: n = 1; while (n < R && rows[n] == o[n-1]) ++n  (host memory) */
+int fnx_accept_greedy(const int* rows, const int* o, int R);
+/* the same on device memory, asynchronous: n_accept[0] = n */
+int fnx_accept_greedy_dev(const int* rows, const int* o, int R, int* n_accept, void* st);
+
+/* ---- the whole MoE half of a verify window (engine.cu:1569-1757 Engine::ffn_half without cards and streaming):
+ * quantize -> router_route -> gate|up (routed + shared) -> swiglu q8_1 -> down (routed + shared) -> combine.
+ * Same results as the calls above made one by one. */
+typedef struct fnx_moe_layer {
+    int n, ff, nexp, topk;   /* hidden, expert width, experts, picks per token */
+    const void* router;      /* [nexp + 1][n]: the router's rows, then the shared expert's gate */
+    int router_bf16;         /* 0: f32, 1: bf16 bits */
+    fnx_dw gu;               /* routed gate|up: n_out = 2 ff, n_in = n */
+    size_t gu_stride;        /* bytes between experts */
+    fnx_dw down;             /* routed down: n_out = n, n_in = ff */
+    size_t down_stride;
+    fnx_dw sh_gu;            /* shared expert gate|up */
+    fnx_dw sh_down;          /* shared expert down */
+} fnx_moe_layer;
+/* caller-owned scratch for one window; sizes from fnx_moe_ws_bytes */
+typedef struct fnx_moe_ws {
+    void* xq;        /* q8_1 rows of x: T * n/32 * 36 bytes */
+    float* logits;   /* [T][nexp + 1] */
+    int* topi;       /* [T][topk] */
+    float* topw;     /* [T][topk] */
+    fnx_job* jobs_gu;/* [T * topk + 1] (the last one is the shared expert's) */
+    fnx_job* jobs_dn;/* [T * topk + 1] */
+    int* njobs;      /* [2], zeroed once */
+    float* gu;       /* [T * topk + T][2 ff] */
+    float* part;     /* [T * topk + T][n] */
+} fnx_moe_ws;
+int fnx_moe_verify_layer(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,105 @@
+"""Python-side plumbing for the MI355X verify-path library: loads libfnx_mi355x.so and exposes its C ABI.
+
+The product is the C ABI (include/fnx_mi355x.h); this module only carries device pointers of torch tensors across
+ctypes for the tests and the benchmark. There is no fallback: if the shared library is missing, import of `lib()`
+raises, and every compute call needs a GPU.
+"""
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libfnx_mi355x.so")
+
+MAXT = 16
+PF_JOB = 64
+T_IQ3_S = 21
+IQ3S_BLOCK = 110
+Q8_1_BLOCK = 36
+
+
+class Job(C.Structure):
+    _fields_ = [("w", C.c_int), ("n", C.c_int), ("y", C.c_int * MAXT), ("out", C.c_int * MAXT)]
+
+
+class BigJob(C.Structure):
+    _fields_ = [("w", C.c_int), ("n", C.c_int), ("y", C.c_int * PF_JOB), ("out", C.c_int * PF_JOB)]
+
+
+class DW(C.Structure):
+    _fields_ = [("p", C.c_void_p), ("type", C.c_uint32), ("n_in", C.c_int), ("n_out", C.c_int), ("row_bytes", C.c_size_t),
+                ("ep", C.c_void_p)]
+
+
+class MoeLayer(C.Structure):
+    _fields_ = [("n", C.c_int), ("ff", C.c_int), ("nexp", C.c_int), ("topk", C.c_int), ("router", C.c_void_p),
+                ("router_bf16", C.c_int), ("gu", DW), ("gu_stride", C.c_size_t), ("down", DW), ("down_stride", C.c_size_t),
+                ("sh_gu", DW), ("sh_down", DW)]
+
+
+class MoeWs(C.Structure):
+    _fields_ = [("xq", C.c_void_p), ("logits", C.c_void_p), ("topi", C.c_void_p), ("topw", C.c_void_p), ("jobs_gu", C.c_void_p),
+                ("jobs_dn", C.c_void_p), ("njobs", C.c_void_p), ("gu", C.c_void_p), ("part", C.c_void_p)]
+
+
+EXPORTS = {
+    # name: (restype, argtypes)
+    "fnx_last_error": (C.c_char_p, []),
+    "fnx_version": (C.c_char_p, []),
+    "fnx_quantize_q8_1": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
+    "fnx_mmvq": (C.c_int, [C.POINTER(DW), C.c_size_t, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]),
+    "fnx_gemv_f32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]),
+    "fnx_gemv_bf16": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]),
+    "fnx_route": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                            C.c_void_p]),
+    "fnx_router_route": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p,
+                                   C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "fnx_swiglu_q8_1": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
+    "fnx_swiglu_stacked_q8_1": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
+    "fnx_moe_gate_up": (C.c_int, [C.POINTER(DW), C.c_size_t, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "fnx_moe_down": (C.c_int, [C.POINTER(DW), C.c_size_t, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "fnx_moe_combine": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_int,
+                                  C.c_void_p]),
+    "fnx_argmax": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "fnx_lookup_drafts": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]),
+    "fnx_lookup_drafts_dev": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                        C.c_void_p]),
+    "fnx_accept_greedy": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int]),
+    "fnx_accept_greedy_dev": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
+    "fnx_moe_verify_layer": (C.c_int, [C.POINTER(MoeLayer), C.c_void_p, C.c_int, C.c_void_p, C.POINTER(MoeWs), C.c_void_p]),
+}
+
+_lib = None
+
+
+class FnxError(RuntimeError):
+    pass
+
+
+def lib():
+    """The loaded C-ABI library. Raises if it was not built (run qwen3.8-flash-next-2x-p100_amd/build.py)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise FnxError("libfnx_mi355x.so is not built: run __graft_entry__.build() or build.py (no CPU path exists)")
+        l = C.CDLL(LIB_PATH)
+        for name, (res, args) in EXPORTS.items():
+            fn = getattr(l, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = l
+    return _lib
+
+
+def check(status):
+    if status != 0:
+        raise FnxError(lib().fnx_last_error().decode())
+
+
+def dw(tensor_or_ptr, n_in, n_out, ep=None):
+    p = tensor_or_ptr if isinstance(tensor_or_ptr, int) or tensor_or_ptr is None else tensor_or_ptr.data_ptr()
+    return DW(p, T_IQ3_S, n_in, n_out, n_in // 256 * IQ3S_BLOCK, ep)
+
+
+def stream_ptr():
+    import torch
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)

@@ -1,0 +1,68 @@
+// Device-side helpers shared by the gfx950 kernels: wave64 reductions, half conversion, the signed IQ3_S lookup table.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "iq3s_grid.h"
+
+namespace fnx {
+
+constexpr int WAVE = 64;
+
+// ---- the signed codebook: entry (sign nibble << 9 | 9-bit code) = the group's four weights as signed bytes.
+// A lane turns 4 weights into one v_dot4_i32_i8 operand with a single LDS read: 8192 entries, 32 KiB.
+struct SignedGrid {
+    uint32_t v[8192];
+    constexpr SignedGrid() : v() {
+        for (int s = 0; s < 16; ++s)
+            for (int g = 0; g < 512; ++g) {
+                const uint32_t m = fnx_iq3s_grid_host[g];
+                uint32_t r = 0;
+                for (int j = 0; j < 4; ++j) {
+                    int b = (int) ((m >> (8 * j)) & 255u);
+                    if ((s >> j) & 1) b = -b;
+                    r |= ((uint32_t) b & 255u) << (8 * j);
+                }
+                v[s * 512 + g] = r;
+            }
+    }
+};
+constexpr int SGRID_WORDS = 8192;
+
+__device__ __forceinline__ float half_bits_to_float(uint32_t h) {
+    return __half2float(__ushort_as_half((unsigned short) h));
+}
+__device__ __forceinline__ unsigned short float_to_half_bits(float f) { return __half_as_ushort(__float2half_rn(f)); }
+
+// xor-butterfly over `width` lanes (a power of two <= 64): every lane of a group ends with the group's sum.
+// The order of the adds is part of the results' definition for the f32 mat-vec (the CPU oracle follows it).
+template <int width>
+__device__ __forceinline__ float group_sum(float v) {
+#pragma unroll
+    for (int o = width / 2; o; o >>= 1) v += __shfl_xor(v, o, WAVE);
+    return v;
+}
+template <int width>
+__device__ __forceinline__ float group_max(float v) {
+#pragma unroll
+    for (int o = width / 2; o; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, WAVE));
+    return v;
+}
+
+__device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
+__device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x)); }
+
+// little-endian loads from addresses that are only 2-byte aligned (IQ3_S blocks are 110 bytes)
+__device__ __forceinline__ uint32_t load_u32_a2(const uint8_t* p) {
+    uint32_t v;
+    __builtin_memcpy(&v, __builtin_assume_aligned(p, 2), 4);
+    return v;
+}
+__device__ __forceinline__ uint32_t load_u16(const uint8_t* p) {
+    unsigned short v;
+    __builtin_memcpy(&v, __builtin_assume_aligned(p, 2), 2);
+    return v;
+}
+
+}  // namespace fnx

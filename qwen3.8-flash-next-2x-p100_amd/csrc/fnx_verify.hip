@@ -1,0 +1,702 @@
+// MI355X (gfx950) kernels and C ABI of the speculative-decode verify path: q8_1 activation quantisation, f32/bf16
+// router mat-vec, top-k routing and job lists, IQ3_S x q8_1 expert mat-vec (gate|up, down, generic jobs), SwiGLU,
+// combine, argmax, prompt-lookup drafting and greedy acceptance. Each entry point names the reference operator it
+// replaces in include/fnx_mi355x.h.
+//
+// There is no CPU path in this library: every compute entry point launches HIP kernels and reports a HIP error
+// through its status when no device can run them.
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+
+#include "../../include/fnx_mi355x.h"
+#include "fnx_device.h"
+
+namespace fnx {
+
+// ================================================================ error plumbing
+static thread_local std::string t_err;
+static int fail(const std::string& m) {
+    t_err = m;
+    return 1;
+}
+static int launch_status(const char* what) {
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(std::string(what) + ": " + hipGetErrorString(e));
+    return 0;
+}
+static int env_int(const char* name, int dflt, int lo, int hi) {
+    const char* s = std::getenv(name);
+    if (!s || !*s) return dflt;
+    char* end = nullptr;
+    const long v = std::strtol(s, &end, 10);
+    if (*end || v < lo || v > hi) {
+        std::fprintf(stderr, "fnx: %s=%s ignored (want %d..%d)\n", name, s, lo, hi);
+        return dflt;
+    }
+    return (int) v;
+}
+
+// ================================================================ device globals
+__device__ const SignedGrid g_sgrid{};
+// h = silu(gate) * up of every pair of the window as q8_1 rows, made once for moe_down (one MoE in flight per device,
+// as the reference's g_moe_hq, moe.cuh:592-594)
+constexpr int HQ_ROWS = FNX_MAXT * 10 + FNX_MAXT, HQ_MAX_FF = 1024;
+__device__ uint8_t g_moe_hq[HQ_ROWS * (HQ_MAX_FF / 32) * FNX_Q8_1_BLOCK];
+
+// ================================================================ q8_1 quantisation (kernels.cu:131-145)
+// one 32-lane half-wave per block of 32 values
+__device__ __forceinline__ void q8_1_store(float xi, uint8_t* blk, int lane32) {
+    const float amax = group_max<32>(fabsf(xi)), sum = group_sum<32>(xi);
+    const float d = amax / 127.0f;
+    const int8_t qv = amax == 0.0f ? (int8_t) 0 : (int8_t) roundf(xi / d);
+    reinterpret_cast<int8_t*>(blk + 4)[lane32] = qv;
+    if (lane32 == 0) {
+        reinterpret_cast<unsigned short*>(blk)[0] = float_to_half_bits(d);
+        reinterpret_cast<unsigned short*>(blk)[1] = float_to_half_bits(sum);
+    }
+}
+__global__ void __launch_bounds__(256) k_quantize_q8_1(const float* __restrict__ x, uint8_t* __restrict__ q, int n) {
+    const int row = blockIdx.y, b = blockIdx.x * 8 + (threadIdx.x >> 5), lane = threadIdx.x & 31;
+    if (b >= n / 32) return;
+    const float xi = x[(size_t) row * n + b * 32 + lane];
+    q8_1_store(xi, q + ((size_t) row * (n / 32) + b) * FNX_Q8_1_BLOCK, lane);
+}
+// h = silu(g) * u -> q8_1 (kernels.cu:400-410, moe.cuh:597-608). q null: the library's own pair buffer
+__global__ void __launch_bounds__(256) k_swiglu_q8_1(const float* __restrict__ g, const float* __restrict__ u, size_t row_stride,
+                                                    uint8_t* __restrict__ q, int n) {
+    const int row = blockIdx.y, b = blockIdx.x * 8 + (threadIdx.x >> 5), lane = threadIdx.x & 31;
+    if (b >= n / 32) return;
+    const size_t i = (size_t) row * row_stride + b * 32 + lane;
+    const float xi = silu_f(g[i]) * u[i];
+    uint8_t* dst = q ? q : g_moe_hq;
+    q8_1_store(xi, dst + ((size_t) row * (n / 32) + b) * FNX_Q8_1_BLOCK, lane);
+}
+
+// ================================================================ f32 / bf16 mat-vec (router; kernels.cu:239-287)
+// A wave per weight row, the window's rows of x staged 256 columns at a time in LDS. Summation order (shared with
+// the CPU oracle, so routing picks are bit-exact): lane l takes float4 chunks l, l + 64, ... in order, fmaf over
+// x, y, z, w; then the xor-butterfly 32..1.
+constexpr int GV_WAVES = 8;
+template <bool BF>
+__global__ void __launch_bounds__(GV_WAVES * 64) k_gemv_rows(const void* __restrict__ Wv, const float* __restrict__ x, float* __restrict__ y,
+                                                            int rows, int n, int T) {
+    __shared__ float4 xs[FNX_MAXT][64];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int row = blockIdx.x * GV_WAVES + wave;
+    const bool live = row < rows;
+    float acc[FNX_MAXT];
+#pragma unroll
+    for (int t = 0; t < FNX_MAXT; ++t) acc[t] = 0.f;
+    for (int c0 = 0; c0 < n / 4; c0 += 64) {
+        __syncthreads();
+        for (int q = threadIdx.x; q < T * 64; q += GV_WAVES * 64) {
+            const int t = q >> 6, l = q & 63;
+            xs[t][l] = reinterpret_cast<const float4*>(x + (size_t) t * n)[c0 + l];
+        }
+        __syncthreads();
+        if (live) {
+            float4 w;
+            if constexpr (BF) {
+                const uint2 u = reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(Wv) + (size_t) row * n)[c0 + lane];
+                w = make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u), __uint_as_float(u.y << 16),
+                                __uint_as_float(u.y & 0xffff0000u));
+            } else {
+                w = reinterpret_cast<const float4*>(reinterpret_cast<const float*>(Wv) + (size_t) row * n)[c0 + lane];
+            }
+#pragma unroll
+            for (int t = 0; t < FNX_MAXT; ++t)
+                if (t < T) {
+                    const float4 b = xs[t][lane];
+                    float a = acc[t];
+                    a = fmaf(w.x, b.x, a);
+                    a = fmaf(w.y, b.y, a);
+                    a = fmaf(w.z, b.z, a);
+                    a = fmaf(w.w, b.w, a);
+                    acc[t] = a;
+                }
+        }
+    }
+    if (!live) return;
+#pragma unroll
+    for (int t = 0; t < FNX_MAXT; ++t)
+        if (t < T) {
+            const float v = group_sum<64>(acc[t]);
+            if (lane == 0) y[(size_t) t * rows + row] = v;
+        }
+}
+
+// ================================================================ top-k and jobs (moe.cuh:382-462, kernels.cu:381-398)
+// One block; wave t ranks token t's logits: topk rounds of a wave arg-max, greater value first, lower index on a tie.
+// Weights exp(l_k - l_0) / sum in pick order. Jobs: one per distinct expert, numbered by first pick, a job's pairs in
+// ascending order (the order k_jobs gives).
+constexpr int TK_MAXE = 1024, TK_THREADS = 1024;
+__global__ void __launch_bounds__(TK_THREADS) k_topk_jobs(const float* __restrict__ logits, int stride, int T, int nexp, int topk,
+                                                         int* __restrict__ topi, float* __restrict__ topw, fnx_job* __restrict__ gu,
+                                                         fnx_job* __restrict__ dn, int* __restrict__ njobs, int both_counts,
+                                                         int shared_job) {
+    __shared__ int ex[FNX_MAXT * 64];
+    __shared__ int jobof[TK_MAXE];
+    __shared__ unsigned char isfirst[FNX_MAXT * 64];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, P = T * topk;
+    if (wave < T) {
+        const int t = wave;
+        float v[TK_MAXE / 64];
+#pragma unroll
+        for (int i = 0; i < TK_MAXE / 64; ++i) {
+            const int e = lane + 64 * i;
+            v[i] = e < nexp ? logits[(size_t) t * stride + e] : -INFINITY;
+        }
+        unsigned taken = 0;
+        float top0 = 0.f, z = 0.f, wk = 0.f;
+        for (int k = 0; k < topk; ++k) {
+            float bv = -INFINITY;
+            int bi = nexp;
+#pragma unroll
+            for (int i = 0; i < TK_MAXE / 64; ++i)
+                if (!((taken >> i) & 1u) && v[i] > bv) {
+                    bv = v[i];
+                    bi = lane + 64 * i;
+                }
+#pragma unroll
+            for (int o = 32; o; o >>= 1) {
+                const float ov = __shfl_xor(bv, o, 64);
+                const int oi = __shfl_xor(bi, o, 64);
+                if (ov > bv || (ov == bv && oi < bi)) {
+                    bv = ov;
+                    bi = oi;
+                }
+            }
+            if (bi < nexp && (bi & 63) == lane) taken |= 1u << (bi >> 6);
+            if (k == 0) top0 = bv;
+            const float ek = expf(bv - top0);
+            z += ek;
+            if (lane == k) {
+                wk = ek;
+                const int pick = bi < nexp ? bi : nexp - 1;   // fewer than topk finite logits: stay inside the tables
+                topi[t * topk + k] = pick;
+                ex[t * topk + k] = pick;
+            }
+        }
+        if (lane < topk) topw[t * topk + lane] = wk / z;
+    }
+    __syncthreads();
+    if (!gu) return;
+    const int p = threadIdx.x;
+    int slot = 0, e = -1;
+    if (p < P) {
+        e = ex[p];
+        for (int q = 0; q < p; ++q) slot += ex[q] == e;
+        isfirst[p] = slot == 0;
+    }
+    __syncthreads();
+    if (p < P && slot == 0) {
+        int j = 0, cnt = 0;
+        for (int q = 0; q < p; ++q) j += isfirst[q];
+        for (int q = 0; q < P; ++q) cnt += ex[q] == e;
+        jobof[e] = j;
+        gu[j].w = dn[j].w = e;
+        gu[j].n = dn[j].n = cnt;
+    }
+    __syncthreads();
+    if (p < P) {
+        const int j = jobof[e];
+        gu[j].y[slot] = p / topk;
+        gu[j].out[slot] = p;
+        dn[j].y[slot] = p;
+        dn[j].out[slot] = p;
+    }
+    if (p == P) {
+        int nj = 0;
+        for (int q = 0; q < P; ++q) nj += isfirst[q];
+        njobs[0] = nj;
+        if (both_counts) njobs[1] = nj;
+    }
+    // the shared expert's job at index P: every row of the window, outputs at rows P + t (kernels.hpp:277-282)
+    if (shared_job && p < T) {
+        gu[P].y[p] = p;
+        gu[P].out[p] = P + p;
+        dn[P].y[p] = P + p;
+        dn[P].out[p] = P + p;
+        if (p == 0) {
+            gu[P].w = dn[P].w = 0;
+            gu[P].n = dn[P].n = T;
+        }
+    }
+}
+
+// ================================================================ IQ3_S x q8_1 jobs: the expert mat-vec
+// (k_mmvq kernels.cu:192-229, k_moe_gu moe.cuh:572-585, k_moe_down moe.cuh:613-658, vec_dot iq3s_x.cuh:4-41)
+//
+// Work is cut in units of 64 sub-blocks of 32 weights = 880 contiguous bytes: one row of 2048 columns, 4 rows of
+// 512, 8 rows of 256. Lane l of a wave owns sub-block l of the unit: it reads its 8 code bytes, its sign dword, its
+// high-bit byte and scale nibble straight from the raw ggml block, builds eight 13-bit indexes (sign nibble | high
+// bit | code) into the signed codebook in LDS and feeds each looked-up dword to v_dot4_i32_i8 against the token's
+// int8 activations, which stay in registers for the whole job (a lane's sub-block column never changes).
+// The waves of the grid split the units of all jobs evenly and walk them in order: consecutive rows, one expert
+// after the other, so every wave streams contiguous memory.
+struct RowsArgs {
+    const uint8_t* wbase;
+    size_t w_stride;
+    const uint8_t* const* ep;
+    size_t row_bytes;
+    int nrows, ncols;
+    const fnx_job* jobs;
+    const int* njobs;
+    int njobs_max;
+    const uint8_t* y;   // q8_1 rows; null: the library's pair buffer
+    float* out;
+    int out_stride;
+};
+
+struct RawSub {   // one lane's share of a unit as read from memory
+    uint32_t q0, q1, sg, hs, d;   // codes 0..3, 4..7, sign nibbles, high bits (low byte) | scales byte << 8, d bits
+};
+__device__ __forceinline__ RawSub load_sub(const uint8_t* blk, int ib) {
+    RawSub r;
+    r.d = load_u16(blk);
+    r.q0 = load_u32_a2(blk + 2 + 8 * ib);
+    r.q1 = load_u32_a2(blk + 6 + 8 * ib);
+    r.sg = load_u32_a2(blk + 74 + 4 * ib);
+    r.hs = (uint32_t) blk[66 + ib] | ((uint32_t) blk[106 + (ib >> 1)] << 8);
+    return r;
+}
+
+// SBR: sub-blocks per weight row (ncols / 32), a power of two <= 64. NT: tokens of the job held in registers.
+template <int SBR, int NT>
+__device__ __forceinline__ void job_units(const uint32_t* __restrict__ tab, const uint8_t* __restrict__ we, size_t row_bytes, int nrows,
+                                          int ua, int ub, const fnx_job* __restrict__ jb, int t0, const uint8_t* __restrict__ y,
+                                          float* __restrict__ out, int out_stride) {
+    constexpr int RW = 64 / SBR;   // rows per unit
+    const int lane = threadIdx.x & 63, g = lane / SBR, kb = lane % SBR, sb = kb >> 3, ib = kb & 7;
+    int xs[NT][8];
+    float dx[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        const uint8_t* yb = y + ((size_t) jb->y[t0 + t] * SBR + kb) * FNX_Q8_1_BLOCK;
+        dx[t] = half_bits_to_float(*reinterpret_cast<const unsigned short*>(yb));
+#pragma unroll
+        for (int j = 0; j < 8; ++j) xs[t][j] = reinterpret_cast<const int*>(yb + 4)[j];
+    }
+    const size_t lane_off = (size_t) g * row_bytes + (size_t) sb * FNX_IQ3S_BLOCK;
+    const uint8_t* p = we + (size_t) ua * RW * row_bytes + lane_off;
+    const size_t step = (size_t) RW * row_bytes;
+    bool live = ua * RW + g < nrows;
+    RawSub cur = live ? load_sub(p, ib) : RawSub{};
+    for (int u = ua; u < ub; ++u) {
+        const bool live_next = u + 1 < ub && (u + 1) * RW + g < nrows;
+        RawSub nxt = cur;
+        if (live_next) nxt = load_sub(p + step, ib);
+        int sum[NT];
+#pragma unroll
+        for (int t = 0; t < NT; ++t) sum[t] = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const uint32_t code = (((j < 4 ? cur.q0 : cur.q1) >> (8 * (j & 3))) & 0xFFu) | (((cur.hs >> j) & 1u) << 8) |
+                                  (((cur.sg >> (4 * j)) & 0xFu) << 9);
+            const int w4 = (int) tab[code];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) sum[t] = __builtin_amdgcn_sdot4(w4, xs[t][j], sum[t], false);
+        }
+        const int sc = 1 + 2 * (int) ((cur.hs >> (8 + 4 * (ib & 1))) & 0xFu);
+        const float dw = half_bits_to_float(cur.d);
+        const int row = u * RW + g;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            // one sub-block's term exactly as the reference forms it: (d_w * d_x) * (float) (sumi * (1 + 2 s))
+            float v = (dw * dx[t]) * (float) __mul24(sum[t], sc);
+            if (!live) v = 0.f;
+            v = group_sum<SBR>(v);
+            if (kb == 0 && live) out[(size_t) jb->out[t0 + t] * out_stride + row] = v;
+        }
+        cur = nxt;
+        live = live_next;
+        p += step;
+    }
+}
+
+template <int SBR>
+__device__ __forceinline__ void job_range(const uint32_t* tab, const uint8_t* we, const RowsArgs& a, int ua, int ub, const fnx_job* jb,
+                                          const uint8_t* y) {
+    const int n = jb->n;
+    for (int t0 = 0; t0 < n;) {
+        const int nt = n - t0;
+        if (nt >= 4) {
+            job_units<SBR, 4>(tab, we, a.row_bytes, a.nrows, ua, ub, jb, t0, y, a.out, a.out_stride);
+            t0 += 4;
+        } else if (nt == 3) {
+            job_units<SBR, 3>(tab, we, a.row_bytes, a.nrows, ua, ub, jb, t0, y, a.out, a.out_stride);
+            t0 += 3;
+        } else if (nt == 2) {
+            job_units<SBR, 2>(tab, we, a.row_bytes, a.nrows, ua, ub, jb, t0, y, a.out, a.out_stride);
+            t0 += 2;
+        } else {
+            job_units<SBR, 1>(tab, we, a.row_bytes, a.nrows, ua, ub, jb, t0, y, a.out, a.out_stride);
+            t0 += 1;
+        }
+    }
+}
+
+template <int SBR>
+__global__ void __launch_bounds__(1024) k_iq3s_jobs(const RowsArgs a) {
+    __shared__ uint32_t tab[SGRID_WORDS];
+    for (int i = threadIdx.x; i < SGRID_WORDS; i += blockDim.x) tab[i] = g_sgrid.v[i];
+    __syncthreads();
+    constexpr int RW = 64 / SBR;
+    const int nj = a.njobs ? min(*a.njobs, a.njobs_max) : a.njobs_max;
+    const int upj = (a.nrows + RW - 1) / RW;   // units per job
+    const long total = (long) nj * upj;
+    const int wpb = blockDim.x >> 6;
+    const long gw = (long) blockIdx.x * wpb + (threadIdx.x >> 6), nw = (long) gridDim.x * wpb;
+    long u = total * gw / nw;
+    const long u1 = total * (gw + 1) / nw;
+    const uint8_t* y = a.y ? a.y : g_moe_hq;
+    while (u < u1) {
+        const int ji = (int) (u / upj), ul = (int) (u % upj);
+        const int ue = (int) min((long) upj, ul + (u1 - u));
+        const fnx_job* jb = a.jobs + ji;
+        const uint8_t* we = a.ep ? a.ep[jb->w] : a.wbase + (size_t) jb->w * a.w_stride;
+        job_range<SBR>(tab, we, a, ul, ue, jb, y);
+        u += ue - ul;
+    }
+}
+
+// any other row length (a multiple of 256): a wave per (row, job), sub-blocks dealt round-robin to the lanes, the
+// codebook read from global memory. Not a tuned path.
+__global__ void __launch_bounds__(256) k_iq3s_jobs_any(const RowsArgs a) {
+    const int ji = blockIdx.y;
+    if (ji >= (a.njobs ? min(*a.njobs, a.njobs_max) : a.njobs_max)) return;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (row >= a.nrows) return;
+    const fnx_job* jb = a.jobs + ji;
+    const uint8_t* we = (a.ep ? a.ep[jb->w] : a.wbase + (size_t) jb->w * a.w_stride) + (size_t) row * a.row_bytes;
+    const uint8_t* y = a.y ? a.y : g_moe_hq;
+    const int sbr = a.ncols / 32;
+    for (int t = 0; t < jb->n; ++t) {
+        float acc = 0.f;
+        for (int kb = lane; kb < sbr; kb += 64) {
+            const int ib = kb & 7;
+            const RawSub r = load_sub(we + (size_t) (kb >> 3) * FNX_IQ3S_BLOCK, ib);
+            const uint8_t* yb = y + ((size_t) jb->y[t] * sbr + kb) * FNX_Q8_1_BLOCK;
+            int sum = 0;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const uint32_t code = (((j < 4 ? r.q0 : r.q1) >> (8 * (j & 3))) & 0xFFu) | (((r.hs >> j) & 1u) << 8) |
+                                      (((r.sg >> (4 * j)) & 0xFu) << 9);
+                sum = __builtin_amdgcn_sdot4((int) g_sgrid.v[code], reinterpret_cast<const int*>(yb + 4)[j], sum, false);
+            }
+            const int sc = 1 + 2 * (int) ((r.hs >> (8 + 4 * (ib & 1))) & 0xFu);
+            acc += (half_bits_to_float(r.d) * half_bits_to_float(*reinterpret_cast<const unsigned short*>(yb))) * (float) (sum * sc);
+        }
+        acc = group_sum<64>(acc);
+        if (lane == 0) a.out[(size_t) jb->out[t] * a.out_stride + row] = acc;
+    }
+}
+
+// ================================================================ combine (kernels.cu:412-419)
+__global__ void __launch_bounds__(256) k_combine(const float* __restrict__ part, const float* __restrict__ topw, const float* __restrict__ sh,
+                                                const float* __restrict__ sh_logit, int sh_logit_stride, float* __restrict__ out, int n,
+                                                int topk) {
+    const int t = blockIdx.y, i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float s = 0.f;
+    for (int k = 0; k < topk; ++k) s = fmaf(topw[t * topk + k], part[((size_t) t * topk + k) * n + i], s);
+    out[(size_t) t * n + i] = s + sigmoid_f(sh_logit[(size_t) t * sh_logit_stride]) * sh[(size_t) t * n + i];
+}
+
+// ================================================================ argmax (kernels.cu:1045-1083)
+__device__ __forceinline__ unsigned fkey(float v) {
+    const unsigned u = __float_as_uint(v);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float fkey_inv(unsigned k) { return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k); }
+constexpr int AM_THREADS = 256, AM_PER_BLOCK = 4096;
+// keys[t] = max over the row of (fkey(value) << 32 | ~index): the greatest value, the lower index on a tie
+__global__ void __launch_bounds__(AM_THREADS) k_argmax(const float* __restrict__ logits, int rows, unsigned long long* __restrict__ keys,
+                                                      unsigned* __restrict__ err) {
+    const int t = blockIdx.y, i0 = blockIdx.x * AM_PER_BLOCK, i1 = min(rows, i0 + AM_PER_BLOCK);
+    const float* r = logits + (size_t) t * rows;
+    unsigned long long best = 0;
+    bool bad = false;
+    for (int i = i0 + threadIdx.x; i < i1; i += AM_THREADS) {
+        const float v = r[i];
+        bad = bad || !isfinite(v);
+        const unsigned long long k = (unsigned long long) fkey(v) << 32 | (unsigned) ~i;
+        best = k > best ? k : best;
+    }
+    if (bad) atomicOr(err, FNX_ERR_NONFINITE);
+#pragma unroll
+    for (int o = 32; o; o >>= 1) {
+        const unsigned long long ok = __shfl_xor(best, o, 64);
+        best = ok > best ? ok : best;
+    }
+    if ((threadIdx.x & 63) == 0) atomicMax(&keys[t], best);
+}
+// decodes the keys into (value, index + v0) and leaves them at zero for the next argmax
+__global__ void k_argmax_fin(unsigned long long* keys, int T, int v0, float* bv, int* bi) {
+    const int t = threadIdx.x;
+    if (t >= T) return;
+    const unsigned long long k = keys[t];
+    bv[t] = fkey_inv((unsigned) (k >> 32));
+    bi[t] = (int) ~(unsigned) k + v0;
+    keys[t] = 0ull;
+}
+
+// ================================================================ prompt lookup and acceptance on the device
+// (session.cpp:428-447, 573). One block: every thread tests its share of start positions for the key, the block keeps
+// the greatest matching start, thread 0 walks the short backward match and copies the drafts.
+constexpr int LK_THREADS = 1024, LOOKUP_MIN = 3, IMAGE_TOK = 1 << 30;
+__global__ void __launch_bounds__(LK_THREADS) k_lookup(const int* __restrict__ ctx, int n_ctx, int key_n, int lk, const int* __restrict__ d1p,
+                                                      int* __restrict__ out, int* __restrict__ n_out, int* __restrict__ match) {
+    __shared__ int best;
+    if (threadIdx.x == 0) best = -1;
+    __syncthreads();
+    const int n0 = n_ctx - key_n;
+    if (lk > 0 && n0 > 0) {
+        int key[4];
+        for (int j = 0; j < key_n; ++j) key[j] = ctx[n0 + j];
+        int mine = -1;
+        for (int s = threadIdx.x; s < n0; s += LK_THREADS) {
+            bool eq = true;
+            for (int j = 0; j < key_n; ++j) eq = eq && ctx[s + j] == key[j];
+            if (eq) mine = s;   // ascending s: the last one kept is this thread's greatest
+        }
+#pragma unroll
+        for (int o = 32; o; o >>= 1) mine = max(mine, __shfl_xor(mine, o, 64));
+        if ((threadIdx.x & 63) == 0 && mine >= 0) atomicMax(&best, mine);
+    }
+    __syncthreads();
+    if (threadIdx.x != 0) return;
+    int nr = 0, m_at = -1;
+    const int s = best, d1 = *d1p;
+    if (s >= 0 && s + key_n < n_ctx && (d1 < 0 || ctx[s + key_n] == d1)) {
+        int m = key_n;
+        while (m < lk && (m - key_n) < s && ctx[s - 1 - (m - key_n)] == ctx[n0 - 1 - (m - key_n)]) ++m;
+        const int k = min(lk, max(LOOKUP_MIN, m)), end = min(n_ctx, s + key_n + k);
+        for (int i = s + key_n; i < end; ++i) {
+            const int tok = ctx[i];
+            if (tok >= IMAGE_TOK) break;   // an image cell is never a draft, nor anything after it
+            out[nr++] = tok;
+        }
+        m_at = s;
+    }
+    *n_out = nr;
+    if (match) *match = m_at;
+}
+__global__ void k_accept(const int* __restrict__ rows, const int* __restrict__ o, int R, int* __restrict__ n_accept) {
+    const int i = threadIdx.x;   // one wave; lane i tests draft i + 1 against row i's pick
+    const bool ok = i + 1 < R && rows[i + 1] == o[i];
+    const unsigned long long b = __ballot(ok);
+    if (i == 0) n_accept[0] = 1 + __builtin_ctzll(~b);
+}
+
+// ================================================================ launchers
+static int rows_launch(const fnx_dw* W, size_t w_stride, const fnx_job* jobs, const int* njobs, int njobs_max, const void* y, float* out,
+                       int out_stride, void* st, const char* who) {
+    if (!W || !jobs || !out) return fail(std::string(who) + ": null argument");
+    if (W->type != FNX_T_IQ3_S) return fail(std::string(who) + ": expert type " + std::to_string(W->type) + " not handled (IQ3_S only)");
+    if (W->n_in <= 0 || W->n_in % 256 || W->n_out <= 0) return fail(std::string(who) + ": shape does not fit IQ3_S super-blocks");
+    if (W->row_bytes != (size_t) (W->n_in / 256) * FNX_IQ3S_BLOCK) return fail(std::string(who) + ": row_bytes does not match n_in");
+    if (njobs_max <= 0) return fail(std::string(who) + ": njobs_max must be positive");
+    if (!W->p && !W->ep) return fail(std::string(who) + ": no weights");
+    RowsArgs a{(const uint8_t*) W->p, w_stride, (const uint8_t* const*) W->ep, W->row_bytes, W->n_out, W->n_in,
+               jobs, njobs, njobs_max, (const uint8_t*) y, out, out_stride};
+    hipStream_t s = (hipStream_t) st;
+    static const int blocks = env_int("FNX_ROWS_BLOCKS", 1024, 1, 65536), threads = env_int("FNX_ROWS_THREADS", 512, 64, 1024) / 64 * 64;
+    // no more waves than units: a wave with an empty range only loads the table
+    const long units = (long) njobs_max * ((W->n_out * (long) (W->n_in / 32) + 63) / 64);
+    const int grid = (int) std::max(1L, std::min((long) blocks, (units + threads / 64 - 1) / (threads / 64)));
+    switch (W->n_in) {
+        case 2048: k_iq3s_jobs<64><<<grid, threads, 0, s>>>(a); break;
+        case 1024: k_iq3s_jobs<32><<<grid, threads, 0, s>>>(a); break;
+        case 512: k_iq3s_jobs<16><<<grid, threads, 0, s>>>(a); break;
+        case 256: k_iq3s_jobs<8><<<grid, threads, 0, s>>>(a); break;
+        default: k_iq3s_jobs_any<<<dim3((W->n_out + 3) / 4, njobs_max), 256, 0, s>>>(a); break;
+    }
+    return launch_status(who);
+}
+
+}  // namespace fnx
+
+using namespace fnx;
+
+// ================================================================ C ABI
+extern "C" {
+
+const char* fnx_last_error(void) { return t_err.c_str(); }
+const char* fnx_version(void) { return "fnx-mi355x gfx950 verify path 0.1"; }
+
+int fnx_quantize_q8_1(const float* x, void* q, int n, int rows, void* st) {
+    if (!x || !q) return fail("quantize_q8_1: null argument");
+    if (n <= 0 || n % 32 || rows <= 0) return fail("quantize_q8_1: rows of whole 32-value blocks");
+    k_quantize_q8_1<<<dim3((n / 32 + 7) / 8, rows), 256, 0, (hipStream_t) st>>>(x, (uint8_t*) q, n);
+    return launch_status("quantize_q8_1");
+}
+
+int fnx_mmvq(const fnx_dw* W, size_t w_stride, const fnx_job* jobs, const int* njobs, int njobs_max, const void* y, float* out,
+             int out_stride, void* st) {
+    if (!y) return fail("mmvq: null activations");
+    return rows_launch(W, w_stride, jobs, njobs, njobs_max, y, out, out_stride, st, "mmvq");
+}
+
+static int gemv_any(const void* W, bool bf, const float* x, float* y, int rows, int n, int T, void* st, const char* who) {
+    if (!W || !x || !y) return fail(std::string(who) + ": null argument");
+    if (rows <= 0 || n <= 0 || n % 256) return fail(std::string(who) + ": n must be a positive multiple of 256");
+    if (T < 1 || T > FNX_MAXT) return fail(std::string(who) + ": T out of range");
+    const int grid = (rows + GV_WAVES - 1) / GV_WAVES;
+    if (bf) k_gemv_rows<true><<<grid, GV_WAVES * 64, 0, (hipStream_t) st>>>(W, x, y, rows, n, T);
+    else k_gemv_rows<false><<<grid, GV_WAVES * 64, 0, (hipStream_t) st>>>(W, x, y, rows, n, T);
+    return launch_status(who);
+}
+int fnx_gemv_f32(const float* W, const float* x, float* y, int rows, int n, int T, void* st) {
+    return gemv_any(W, false, x, y, rows, n, T, st, "gemv_f32");
+}
+int fnx_gemv_bf16(const uint16_t* W, const float* x, float* y, int rows, int n, int T, void* st) {
+    return gemv_any(W, true, x, y, rows, n, T, st, "gemv_bf16");
+}
+
+static int topk_check(int T, int nexp, int topk, const char* who) {
+    if (T < 1 || T > FNX_MAXT) return fail(std::string(who) + ": T out of range");
+    if (nexp < 1 || nexp > TK_MAXE) return fail(std::string(who) + ": 1..1024 experts");
+    if (topk < 1 || topk > 64 || topk > nexp) return fail(std::string(who) + ": topk out of range");
+    if (T * topk > TK_THREADS - 1) return fail(std::string(who) + ": too many pairs");
+    return 0;
+}
+int fnx_route(const float* logits, int logits_stride, int T, int nexp, int topk, int* topi, float* topw, fnx_job* jobs_gu, fnx_job* jobs_dn,
+              int* njobs, void* st) {
+    if (!logits || !topi || !topw || !jobs_gu || !jobs_dn || !njobs) return fail("route: null argument");
+    if (topk_check(T, nexp, topk, "route")) return 1;
+    if (logits_stride < nexp) return fail("route: logits_stride smaller than nexp");
+    k_topk_jobs<<<1, TK_THREADS, 0, (hipStream_t) st>>>(logits, logits_stride, T, nexp, topk, topi, topw, jobs_gu, jobs_dn, njobs, 1, 0);
+    return launch_status("route");
+}
+int fnx_router_route(const void* W, int w_bf16, const float* x, float* logits, int T, int n, int nexp, int topk, int* topi, float* topw,
+                     fnx_job* jobs_gu, fnx_job* jobs_dn, int* njobs, void* st) {
+    if (!W || !x || !logits || !topi || !topw || !jobs_gu || !jobs_dn || !njobs) return fail("router_route: null argument");
+    if (topk_check(T, nexp, topk, "router_route")) return 1;
+    if (gemv_any(W, w_bf16 != 0, x, logits, nexp + 1, n, T, st, "router_route")) return 1;
+    k_topk_jobs<<<1, TK_THREADS, 0, (hipStream_t) st>>>(logits, nexp + 1, T, nexp, topk, topi, topw, jobs_gu, jobs_dn, njobs, 0, 0);
+    return launch_status("router_route");
+}
+
+int fnx_swiglu_q8_1(const float* g, const float* u, void* q, int n, int rows, void* st) {
+    if (!g || !u || !q) return fail("swiglu_q8_1: null argument");
+    if (n <= 0 || n % 32 || rows <= 0) return fail("swiglu_q8_1: rows of whole 32-value blocks");
+    k_swiglu_q8_1<<<dim3((n / 32 + 7) / 8, rows), 256, 0, (hipStream_t) st>>>(g, u, (size_t) n, (uint8_t*) q, n);
+    return launch_status("swiglu_q8_1");
+}
+int fnx_swiglu_stacked_q8_1(const float* gu, void* hq, int ffs, int T, void* st) {
+    if (!gu || !hq) return fail("swiglu_stacked_q8_1: null argument");
+    if (ffs <= 0 || ffs % 32 || T <= 0) return fail("swiglu_stacked_q8_1: rows of whole 32-value blocks");
+    k_swiglu_q8_1<<<dim3((ffs / 32 + 7) / 8, T), 256, 0, (hipStream_t) st>>>(gu, gu + ffs, (size_t) 2 * ffs, (uint8_t*) hq, ffs);
+    return launch_status("swiglu_stacked_q8_1");
+}
+
+int fnx_moe_gate_up(const fnx_dw* A, size_t sa, const fnx_job* jobs, const int* njobs, int njobs_max, const void* xq, float* gu, void* st) {
+    if (!xq) return fail("moe_gate_up: null activations");
+    if (A && (A->n_out & 1)) return fail("moe_gate_up: rows are [gate | up], an even count");
+    return rows_launch(A, sa, jobs, njobs, njobs_max, xq, gu, A ? A->n_out : 0, st, "moe_gate_up");
+}
+int fnx_moe_down(const fnx_dw* A, size_t sa, const fnx_job* jobs, const int* njobs, int njobs_max, const float* gu, float* part, void* st) {
+    if (!A || !gu) return fail("moe_down: null argument");
+    const int ffs = A->n_in;
+    if (ffs <= 0 || ffs % 32 || ffs > HQ_MAX_FF) return fail("moe_down: expert width does not fit the pair buffer");
+    if (njobs_max < 1 || njobs_max > HQ_ROWS) return fail("moe_down: more pairs than the pair buffer holds");
+    // every pair's h once (moe.cuh:597-608), then the rows against it
+    k_swiglu_q8_1<<<dim3((ffs / 32 + 7) / 8, njobs_max), 256, 0, (hipStream_t) st>>>(gu, gu + ffs, (size_t) 2 * ffs, nullptr, ffs);
+    if (launch_status("moe_down")) return 1;
+    return rows_launch(A, sa, jobs, njobs, njobs_max, nullptr, part, A->n_out, st, "moe_down");
+}
+int fnx_moe_combine(const float* part, const float* topw, const float* sh, const float* sh_logit, int sh_logit_stride, float* out, int T, int n,
+                    int topk, void* st) {
+    if (!part || !topw || !sh || !sh_logit || !out) return fail("moe_combine: null argument");
+    if (T < 1 || n < 1 || topk < 1) return fail("moe_combine: bad shape");
+    k_combine<<<dim3((n + 255) / 256, T), 256, 0, (hipStream_t) st>>>(part, topw, sh, sh_logit, sh_logit_stride, out, n, topk);
+    return launch_status("moe_combine");
+}
+
+int fnx_argmax(const float* logits, int rows, int T, int v0, float* best_v, int* best_i, unsigned long long* keys, unsigned* err, void* st) {
+    if (!logits || !best_v || !best_i || !keys || !err) return fail("argmax: null argument");
+    if (rows < 1 || T < 1 || T > FNX_MAXT) return fail("argmax: bad shape");
+    k_argmax<<<dim3((rows + AM_PER_BLOCK - 1) / AM_PER_BLOCK, T), AM_THREADS, 0, (hipStream_t) st>>>(logits, rows, keys, err);
+    k_argmax_fin<<<1, 64, 0, (hipStream_t) st>>>(keys, T, v0, best_v, best_i);
+    return launch_status("argmax");
+}
+
+int fnx_lookup_drafts(const int* ctx, int n_ctx, int key_n, int lk, int d1, int* out, int* match) {
+    if (match) *match = -1;
+    if (!ctx || !out || n_ctx < 0 || lk < 0 || key_n < 1 || key_n > 4) {
+        fail("lookup_drafts: bad argument");
+        return -1;
+    }
+    if (lk == 0 || n_ctx <= key_n) return 0;
+    const int n0 = n_ctx - key_n;
+    int nr = 0;
+    for (int s = n0; s-- > 0;) {
+        if (std::memcmp(ctx + s, ctx + n0, (size_t) key_n * sizeof(int)) != 0) continue;
+        // only the latest earlier place is examined (session.cpp:442)
+        if (s + key_n < n_ctx && (d1 < 0 || ctx[s + key_n] == d1)) {
+            int m = key_n;
+            while (m < lk && (m - key_n) < s && ctx[s - 1 - (m - key_n)] == ctx[n0 - 1 - (m - key_n)]) ++m;
+            const int k = std::min(lk, std::max(LOOKUP_MIN, m)), end = std::min(n_ctx, s + key_n + k);
+            for (int i = s + key_n; i < end && ctx[i] < IMAGE_TOK; ++i) out[nr++] = ctx[i];
+            if (match) *match = s;
+        }
+        break;
+    }
+    return nr;
+}
+int fnx_lookup_drafts_dev(const int* ctx, int n_ctx, int key_n, int lk, const int* d1, int* out, int* n_out, int* match, void* st) {
+    if (!ctx || !d1 || !out || !n_out) return fail("lookup_drafts_dev: null argument");
+    if (n_ctx < 0 || lk < 0 || key_n < 1 || key_n > 4) return fail("lookup_drafts_dev: bad argument");
+    k_lookup<<<1, LK_THREADS, 0, (hipStream_t) st>>>(ctx, n_ctx, key_n, lk, d1, out, n_out, match);
+    return launch_status("lookup_drafts_dev");
+}
+
+int fnx_accept_greedy(const int* rows, const int* o, int R) {
+    if (!rows || !o || R < 1) {
+        fail("accept_greedy: bad argument");
+        return -1;
+    }
+    int n = 1;
+    while (n < R && rows[n] == o[n - 1]) ++n;
+    return n;
+}
+int fnx_accept_greedy_dev(const int* rows, const int* o, int R, int* n_accept, void* st) {
+    if (!rows || !o || !n_accept) return fail("accept_greedy_dev: null argument");
+    if (R < 1 || R > 64) return fail("accept_greedy_dev: 1..64 rows");
+    k_accept<<<1, 64, 0, (hipStream_t) st>>>(rows, o, R, n_accept);
+    return launch_status("accept_greedy_dev");
+}
+
+int fnx_moe_verify_layer(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st) {
+    if (!L || !x || !out || !ws) return fail("moe_verify_layer: null argument");
+    if (!ws->xq || !ws->logits || !ws->topi || !ws->topw || !ws->jobs_gu || !ws->jobs_dn || !ws->njobs || !ws->gu || !ws->part)
+        return fail("moe_verify_layer: incomplete workspace");
+    if (topk_check(T, L->nexp, L->topk, "moe_verify_layer")) return 1;
+    const int P = T * L->topk, n = L->n, ff = L->ff;
+    if (P + T > HQ_ROWS) return fail("moe_verify_layer: more pairs than the pair buffer holds");
+    if (L->gu.n_in != n || L->gu.n_out != 2 * ff || L->down.n_in != ff || L->down.n_out != n || L->sh_gu.n_in != n ||
+        L->sh_gu.n_out != 2 * ff || L->sh_down.n_in != ff || L->sh_down.n_out != n)
+        return fail("moe_verify_layer: weight shapes do not match n / ff");
+    hipStream_t s = (hipStream_t) st;
+    if (fnx_quantize_q8_1(x, ws->xq, n, T, st)) return 1;
+    if (gemv_any(L->router, L->router_bf16 != 0, x, ws->logits, L->nexp + 1, n, T, st, "moe_verify_layer router")) return 1;
+    k_topk_jobs<<<1, TK_THREADS, 0, s>>>(ws->logits, L->nexp + 1, T, L->nexp, L->topk, ws->topi, ws->topw, ws->jobs_gu, ws->jobs_dn, ws->njobs,
+                                         0, 1);
+    if (launch_status("moe_verify_layer topk")) return 1;
+    if (rows_launch(&L->gu, L->gu_stride, ws->jobs_gu, ws->njobs, P, ws->xq, ws->gu, 2 * ff, st, "moe_verify_layer gate|up")) return 1;
+    if (rows_launch(&L->sh_gu, 0, ws->jobs_gu + P, nullptr, 1, ws->xq, ws->gu, 2 * ff, st, "moe_verify_layer shared gate|up")) return 1;
+    k_swiglu_q8_1<<<dim3((ff / 32 + 7) / 8, P + T), 256, 0, s>>>(ws->gu, ws->gu + ff, (size_t) 2 * ff, nullptr, ff);
+    if (launch_status("moe_verify_layer swiglu")) return 1;
+    if (rows_launch(&L->down, L->down_stride, ws->jobs_dn, ws->njobs, P, nullptr, ws->part, n, st, "moe_verify_layer down")) return 1;
+    if (rows_launch(&L->sh_down, 0, ws->jobs_dn + P, nullptr, 1, nullptr, ws->part, n, st, "moe_verify_layer shared down")) return 1;
+    return fnx_moe_combine(ws->part, ws->topw, ws->part + (size_t) P * n, ws->logits + L->nexp, L->nexp + 1, out, T, n, L->topk, st);
+}
+
+}  // extern "C"

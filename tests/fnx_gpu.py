@@ -1,0 +1,199 @@
+"""Test-side helpers: import the package (its directory name is not a Python identifier) and move numpy data
+through the C ABI on torch device buffers."""
+import ctypes as C
+import importlib.util
+import os
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PKG_DIR = os.path.join(ROOT, "qwen3.8-flash-next-2x-p100_amd")
+
+
+def package():
+    name = "fnx_mi355x_pkg"
+    if name in sys.modules:
+        return sys.modules[name]
+    spec = importlib.util.spec_from_file_location(name, os.path.join(PKG_DIR, "__init__.py"), submodule_search_locations=[PKG_DIR])
+    mod = importlib.util.module_from_spec(spec)
+    sys.modules[name] = mod
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def random_iq3s(rng, nblocks, dmax=3e-4):
+    """valid IQ3_S blocks with uniformly random codes, signs and scales (any byte pattern is a valid block)"""
+    b = rng.integers(0, 256, size=(nblocks, 110), dtype=np.uint8)
+    d = (rng.random(nblocks) * dmax + 1e-5).astype(np.float16)
+    b[:, 0:2] = d.view(np.uint8).reshape(nblocks, 2)
+    return b.reshape(-1)
+
+
+JOB_DTYPE = np.dtype([("w", "<i4"), ("n", "<i4"), ("y", "<i4", (16,)), ("out", "<i4", (16,))])
+
+
+class Dev:
+    """numpy in, numpy out, through device memory and the C ABI on the current torch stream"""
+
+    def __init__(self):
+        import torch
+        self.torch = torch
+        self.pkg = package()
+        self.lib = self.pkg.lib()
+        self.dev = torch.device("cuda:0")
+
+    def up(self, a):
+        t = self.torch.from_numpy(np.ascontiguousarray(a))
+        return t.to(self.dev)
+
+    def zeros(self, shape, dtype):
+        return self.torch.zeros(shape, dtype=dtype, device=self.dev)
+
+    def st(self):
+        return self.pkg.stream_ptr()
+
+    def ok(self, status):
+        self.pkg.check(status)
+
+    def sync(self):
+        self.torch.cuda.synchronize()
+
+    # ---- operators
+    def quantize_q8_1(self, x):
+        t = self.torch
+        rows, n = x.shape
+        dx = self.up(x.astype(np.float32))
+        q = self.zeros(rows * (n // 32) * 36, t.uint8)
+        self.ok(self.lib.fnx_quantize_q8_1(dx.data_ptr(), q.data_ptr(), n, rows, self.st()))
+        self.sync()
+        return q.cpu().numpy()
+
+    def gemv(self, W, x, bf16=False):
+        t = self.torch
+        rows, n = W.shape
+        T = x.shape[0]
+        dW, dx = self.up(W), self.up(x.astype(np.float32))
+        y = self.zeros((T, rows), t.float32)
+        fn = self.lib.fnx_gemv_bf16 if bf16 else self.lib.fnx_gemv_f32
+        self.ok(fn(dW.data_ptr(), dx.data_ptr(), y.data_ptr(), rows, n, T, self.st()))
+        self.sync()
+        return y.cpu().numpy()
+
+    def mmvq(self, w, w_stride, nrows, ncols, jobs, yq, out_rows, njobs_dev=True):
+        t = self.torch
+        dw_, dj, dy = self.up(w), self.up(jobs.view(np.uint8).reshape(-1)), self.up(yq)
+        out = self.zeros((out_rows, nrows), t.float32)
+        W = self.pkg.dw(dw_, ncols, nrows)
+        nj = self.up(np.array([len(jobs)], dtype=np.int32))
+        self.ok(self.lib.fnx_mmvq(C.byref(W), w_stride, dj.data_ptr(), nj.data_ptr() if njobs_dev else None, len(jobs), dy.data_ptr(),
+                                  out.data_ptr(), nrows, self.st()))
+        self.sync()
+        return out.cpu().numpy()
+
+    def gemv_iq3s(self, w, nrows, ncols, x):
+        T = x.shape[0]
+        yq = self.quantize_q8_1(x)
+        jobs = np.zeros((T + 15) // 16, dtype=JOB_DTYPE)
+        for j in range(len(jobs)):
+            nt = min(16, T - 16 * j)
+            jobs["n"][j] = nt
+            jobs["y"][j, :nt] = np.arange(16 * j, 16 * j + nt)
+            jobs["out"][j, :nt] = np.arange(16 * j, 16 * j + nt)
+        return self.mmvq(w, 0, nrows, ncols, jobs, yq, T)
+
+    def route(self, logits, nexp, topk, fused_W=None, x=None, bf16=False):
+        t = self.torch
+        T = logits.shape[0] if logits is not None else x.shape[0]
+        P = T * topk
+        topi = self.zeros((T, topk), t.int32)
+        topw = self.zeros((T, topk), t.float32)
+        gu = self.zeros((P + 1) * 136, t.uint8)
+        dn = self.zeros((P + 1) * 136, t.uint8)
+        nj = self.zeros(2, t.int32)
+        if fused_W is None:
+            dl = self.up(logits.astype(np.float32))
+            self.ok(self.lib.fnx_route(dl.data_ptr(), logits.shape[1], T, nexp, topk, topi.data_ptr(), topw.data_ptr(), gu.data_ptr(),
+                                       dn.data_ptr(), nj.data_ptr(), self.st()))
+            lg = None
+        else:
+            dW, dx = self.up(fused_W), self.up(x.astype(np.float32))
+            dl = self.zeros((T, nexp + 1), t.float32)
+            self.ok(self.lib.fnx_router_route(dW.data_ptr(), int(bf16), dx.data_ptr(), dl.data_ptr(), T, x.shape[1], nexp, topk,
+                                              topi.data_ptr(), topw.data_ptr(), gu.data_ptr(), dn.data_ptr(), nj.data_ptr(), self.st()))
+            lg = dl
+        self.sync()
+        njh = nj.cpu().numpy()
+        n = int(njh[0])
+        return dict(topi=topi.cpu().numpy(), topw=topw.cpu().numpy(), njobs=njh,
+                    gu=gu.cpu().numpy()[:n * 136].view(JOB_DTYPE), dn=dn.cpu().numpy()[:n * 136].view(JOB_DTYPE),
+                    logits=None if lg is None else lg.cpu().numpy())
+
+    def argmax(self, logits, v0=0):
+        t = self.torch
+        T, rows = logits.shape
+        dl = self.up(logits.astype(np.float32))
+        bv, bi = self.zeros(T, t.float32), self.zeros(T, t.int32)
+        keys, err = self.zeros(16, t.int64), self.zeros(1, t.int32)
+        self.ok(self.lib.fnx_argmax(dl.data_ptr(), rows, T, v0, bv.data_ptr(), bi.data_ptr(), keys.data_ptr(), err.data_ptr(), self.st()))
+        self.sync()
+        assert int(keys.abs().sum().item()) == 0, "argmax leaves its keys at zero"
+        return bv.cpu().numpy(), bi.cpu().numpy(), int(err.item())
+
+    def lookup(self, ctx, lk, d1, key_n=3):
+        t = self.torch
+        dc = self.up(np.asarray(ctx, dtype=np.int32)) if len(ctx) else self.zeros(1, t.int32)
+        dd = self.up(np.array([d1], dtype=np.int32))
+        out, n_out, match = self.zeros(max(lk, 1), t.int32), self.zeros(1, t.int32), self.zeros(1, t.int32)
+        self.ok(self.lib.fnx_lookup_drafts_dev(dc.data_ptr(), len(ctx), key_n, lk, dd.data_ptr(), out.data_ptr(), n_out.data_ptr(),
+                                               match.data_ptr(), self.st()))
+        self.sync()
+        n = int(n_out.item())
+        return out.cpu().numpy()[:n], int(match.item())
+
+    def accept(self, rows, o):
+        t = self.torch
+        dr, do = self.up(np.asarray(rows, dtype=np.int32)), self.up(np.asarray(o, dtype=np.int32))
+        n = self.zeros(1, t.int32)
+        self.ok(self.lib.fnx_accept_greedy_dev(dr.data_ptr(), do.data_ptr(), len(rows), n.data_ptr(), self.st()))
+        self.sync()
+        return int(n.item())
+
+
+class MoeLayerDev:
+    """One MoE layer's weights on the device plus a workspace, for fnx_moe_verify_layer and the per-op calls."""
+
+    def __init__(self, dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, T=16):
+        t = dev.torch
+        self.dev, self.n, self.ff, self.nexp, self.topk = dev, n, ff, nexp, topk
+        pkg = dev.pkg
+        self.router = dev.up(router.astype(np.float32))
+        self.gu, self.down, self.sh_gu, self.sh_down = dev.up(gu), dev.up(down), dev.up(sh_gu), dev.up(sh_down)
+        self.gu_stride = 2 * ff * (n // 256) * 110
+        self.down_stride = n * (ff // 256) * 110
+        self.L = pkg.MoeLayer(n, ff, nexp, topk, self.router.data_ptr(), 0, pkg.dw(self.gu, n, 2 * ff), self.gu_stride,
+                              pkg.dw(self.down, ff, n), self.down_stride, pkg.dw(self.sh_gu, n, 2 * ff), pkg.dw(self.sh_down, ff, n))
+        P = T * topk
+        self.P = P
+        self.xq = dev.zeros(T * (n // 32) * 36, t.uint8)
+        self.logits = dev.zeros((T, nexp + 1), t.float32)
+        self.topi = dev.zeros((T, topk), t.int32)
+        self.topw = dev.zeros((T, topk), t.float32)
+        self.jobs_gu = dev.zeros((P + 1) * 136, t.uint8)
+        self.jobs_dn = dev.zeros((P + 1) * 136, t.uint8)
+        self.njobs = dev.zeros(2, t.int32)
+        self.gu_out = dev.zeros((P + T, 2 * ff), t.float32)
+        self.part = dev.zeros((P + T, n), t.float32)
+        self.ws = pkg.MoeWs(self.xq.data_ptr(), self.logits.data_ptr(), self.topi.data_ptr(), self.topw.data_ptr(), self.jobs_gu.data_ptr(),
+                            self.jobs_dn.data_ptr(), self.njobs.data_ptr(), self.gu_out.data_ptr(), self.part.data_ptr())
+
+    def run(self, x):
+        dev = self.dev
+        T = x.shape[0]
+        dx = dev.up(x.astype(np.float32))
+        out = dev.zeros((T, self.n), dev.torch.float32)
+        dev.ok(dev.lib.fnx_moe_verify_layer(C.byref(self.L), dx.data_ptr(), T, out.data_ptr(), C.byref(self.ws), dev.st()))
+        dev.sync()
+        return dict(out=out.cpu().numpy(), logits=self.logits.cpu().numpy()[:T], topi=self.topi.cpu().numpy()[:T],
+                    topw=self.topw.cpu().numpy()[:T], njobs=int(self.njobs.cpu().numpy()[0]),
+                    gu=self.gu_out.cpu().numpy(), part=self.part.cpu().numpy())

@@ -1,0 +1,109 @@
+"""Parity of the MoE verify layer (BASELINE config 2) with the CPU oracle: op by op and as one call."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import fnx_gpu
+from fnx_gpu import random_iq3s
+
+pytestmark = pytest.mark.gpu
+
+
+def rel_l2(a, b):
+    return float(np.linalg.norm(a.astype(np.float64) - b.astype(np.float64)) / max(np.linalg.norm(b.astype(np.float64)), 1e-30))
+
+
+@pytest.fixture(scope="module")
+def dev():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    return fnx_gpu.Dev()
+
+
+def make_layer(rng, n, ff, nexp, scale=1.0):
+    router = (rng.standard_normal((nexp + 1, n)) * 0.02 * scale).astype(np.float32)
+    gu = random_iq3s(rng, nexp * 2 * ff * n // 256)
+    down = random_iq3s(rng, nexp * n * ff // 256)
+    sh_gu = random_iq3s(rng, 2 * ff * n // 256)
+    sh_down = random_iq3s(rng, n * ff // 256)
+    return router, gu, down, sh_gu, sh_down
+
+
+def check_layer(dev, oracle, n, ff, nexp, topk, T, seed):
+    print(f"case moe layer n={n} ff={ff} nexp={nexp} topk={topk} T={T} seed={seed}", flush=True)
+    rng = np.random.default_rng(seed)
+    router, gu, down, sh_gu, sh_down = make_layer(rng, n, ff, nexp)
+    x = rng.standard_normal((T, n)).astype(np.float32)
+    want = oracle.moe_verify_layer(n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, x)
+    layer = fnx_gpu.MoeLayerDev(dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down)
+    got = layer.run(x)
+    assert np.array_equal(got["logits"].view(np.uint32), want["logits"].view(np.uint32)), "router logits bit-exact"
+    assert np.array_equal(got["topi"], want["topi"]), "routing picks bit-exact"
+    assert got["njobs"] == want["njobs"]
+    assert np.allclose(got["topw"], want["topw"], rtol=2e-6, atol=0)
+    err = rel_l2(got["out"], want["out"])
+    assert err <= 1e-3, err
+    return got, want, layer, x
+
+
+def test_moe_verify_layer_config2(dev, oracle):
+    # hidden 2048, 512 experts, top-10, SwiGLU experts 2048 -> 512 -> 2048, one shared expert, T = 16
+    got, want, layer, x = check_layer(dev, oracle, 2048, 512, 512, 10, 16, 900)
+    assert rel_l2(got["out"], want["out"]) <= 2e-4
+    # a second window on the same layer and workspace, fewer rows
+    rng = np.random.default_rng(901)
+    x2 = rng.standard_normal((5, 2048)).astype(np.float32)
+    router = layer.router.cpu().numpy()
+    want2 = oracle.moe_verify_layer(2048, 512, 512, 10, router, layer.gu.cpu().numpy(), layer.down.cpu().numpy(),
+                                    layer.sh_gu.cpu().numpy(), layer.sh_down.cpu().numpy(), x2)
+    got2 = layer.run(x2)
+    assert np.array_equal(got2["topi"], want2["topi"]) and got2["njobs"] == want2["njobs"]
+    assert rel_l2(got2["out"], want2["out"]) <= 1e-3
+
+
+@pytest.mark.parametrize("n,ff,nexp,topk,T", [(2048, 512, 64, 10, 1), (1024, 256, 32, 4, 16), (2048, 1024, 16, 2, 3), (512, 512, 16, 8, 7)])
+def test_moe_verify_layer_shapes(dev, oracle, n, ff, nexp, topk, T):
+    check_layer(dev, oracle, n, ff, nexp, topk, T, 910 + T)
+
+
+def test_moe_ops_one_by_one_equal_the_fused_call(dev, oracle):
+    # the reference's call sequence (engine.cu:1569-1757): quantize, router_route, gate|up, down, shared expert, combine
+    n, ff, nexp, topk, T = 2048, 512, 64, 10, 16
+    got, want, layer, x = check_layer(dev, oracle, n, ff, nexp, topk, T, 920)
+    t, lib, pkg = dev.torch, dev.lib, dev.pkg
+    P = T * topk
+    dx = dev.up(x)
+    xq = dev.zeros(T * (n // 32) * 36, t.uint8)
+    logits, topi, topw = dev.zeros((T, nexp + 1), t.float32), dev.zeros((T, topk), t.int32), dev.zeros((T, topk), t.float32)
+    jgu, jdn, nj = dev.zeros(P * 136, t.uint8), dev.zeros(P * 136, t.uint8), dev.zeros(2, t.int32)
+    gu, part, out = dev.zeros((P + T, 2 * ff), t.float32), dev.zeros((P + T, n), t.float32), dev.zeros((T, n), t.float32)
+    st = dev.st()
+    dev.ok(lib.fnx_quantize_q8_1(dx.data_ptr(), xq.data_ptr(), n, T, st))
+    dev.ok(lib.fnx_router_route(layer.router.data_ptr(), 0, dx.data_ptr(), logits.data_ptr(), T, n, nexp, topk, topi.data_ptr(),
+                                topw.data_ptr(), jgu.data_ptr(), jdn.data_ptr(), nj.data_ptr(), st))
+    dev.ok(lib.fnx_moe_gate_up(C.byref(layer.L.gu), layer.gu_stride, jgu.data_ptr(), nj.data_ptr(), P, xq.data_ptr(), gu.data_ptr(), st))
+    dev.ok(lib.fnx_moe_down(C.byref(layer.L.down), layer.down_stride, jdn.data_ptr(), nj.data_ptr(), P, gu.data_ptr(), part.data_ptr(), st))
+    # the shared expert as the reference runs it: a dense gate|up over all rows, swiglu to q8_1, a dense down
+    sh_job = np.zeros(1, dtype=fnx_gpu.JOB_DTYPE)
+    sh_job["n"] = T
+    sh_job["y"][0, :T] = np.arange(T)
+    sh_job["out"][0, :T] = np.arange(T)
+    dj = dev.up(sh_job.view(np.uint8).reshape(-1))
+    sh_gu, sh_hq, sh_part = dev.zeros((T, 2 * ff), t.float32), dev.zeros(T * (ff // 32) * 36, t.uint8), dev.zeros((T, n), t.float32)
+    dev.ok(lib.fnx_mmvq(C.byref(layer.L.sh_gu), 0, dj.data_ptr(), None, 1, xq.data_ptr(), sh_gu.data_ptr(), 2 * ff, st))
+    dev.ok(lib.fnx_swiglu_stacked_q8_1(sh_gu.data_ptr(), sh_hq.data_ptr(), ff, T, st))
+    dev.ok(lib.fnx_mmvq(C.byref(layer.L.sh_down), 0, dj.data_ptr(), None, 1, sh_hq.data_ptr(), sh_part.data_ptr(), n, st))
+    dev.ok(lib.fnx_moe_combine(part.data_ptr(), topw.data_ptr(), sh_part.data_ptr(), logits[:, nexp:].contiguous().data_ptr(), 1,
+                               out.data_ptr(), T, n, topk, st))
+    dev.sync()
+    assert np.array_equal(out.cpu().numpy().view(np.uint32), got["out"].view(np.uint32)), "the fused call is the same arithmetic"
+    # intermediate checks against the oracle's definitions
+    hq_want = oracle.swiglu_stacked_q8_1(sh_gu.cpu().numpy(), ff)
+    # q8_1 bytes of h: the device's expf may differ from libm's in the last bit, which can move a code by one
+    a, b = sh_hq.cpu().numpy().reshape(-1, 36), hq_want.reshape(-1, 36)
+    assert np.array_equal(a[:, :2], b[:, :2]) or np.mean(a[:, :2] != b[:, :2]) < 0.01
+    codes = a[:, 4:].view(np.int8).astype(np.int32) - b[:, 4:].view(np.int8).astype(np.int32)
+    assert np.abs(codes).max() <= 1 and np.mean(codes != 0) < 1e-3
+    comb = oracle.moe_combine(part.cpu().numpy()[:P], topw.cpu().numpy(), sh_part.cpu().numpy(), logits.cpu().numpy()[:, nexp])
+    assert rel_l2(out.cpu().numpy(), comb) <= 1e-6
