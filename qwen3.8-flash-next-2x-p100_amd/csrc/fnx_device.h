@@ -53,6 +53,17 @@ __device__ __forceinline__ float group_max(float v) {
 __device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
 __device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x)); }
 
+// A value every lane of the wave holds alike, moved to a scalar register: what is computed from it (addresses, loop
+// bounds) then runs on the scalar unit. Loads from memory the kernel may also write are vector loads even at a uniform
+// address, so job fields and table entries pass through here.
+__device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ const uint8_t* uniform_ptr(const uint8_t* p) {
+    const uint64_t u = (uint64_t) (uintptr_t) p;
+    const uint32_t lo = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) u);
+    const uint32_t hi = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) (u >> 32));
+    return (const uint8_t*) (uintptr_t) ((uint64_t) hi << 32 | lo);
+}
+
 // little-endian loads from addresses that are only 2-byte aligned (IQ3_S blocks are 110 bytes)
 __device__ __forceinline__ uint32_t load_u32_a2(const uint8_t* p) {
     uint32_t v;

@@ -254,105 +254,156 @@ struct RowsArgs {
     int out_stride;
 };
 
-struct RawSub {   // one lane's share of a unit as read from memory
-    uint32_t q0, q1, sg, hs, d;   // codes 0..3, 4..7, sign nibbles, high bits (low byte) | scales byte << 8, d bits
+// global-memory byte pointer (address space 1): loads through it are global_load, never flat_load
+typedef const __attribute__((address_space(1))) uint8_t* gbytes;
+__device__ __forceinline__ gbytes as_global(const uint8_t* p) { return (gbytes) (uintptr_t) p; }
+
+struct RawSub {   // one lane's share of a unit as read from memory; nothing is combined until it is used
+    uint32_t q0, q1, sg, qh, sc, d;   // codes 0..3, 4..7, sign nibbles, high bits, scales byte, d bits
 };
-__device__ __forceinline__ RawSub load_sub(const uint8_t* blk, int ib) {
+struct LaneOffs {   // byte offsets of a lane's fields inside a unit
+    uint32_t d, qs, qh, sg, sc;
+};
+__device__ __forceinline__ RawSub load_sub(gbytes unit, const LaneOffs& o) {   // unit: wave-uniform; o: per lane
+    typedef __attribute__((address_space(1), aligned(2))) const uint32_t gu32;
+    typedef __attribute__((address_space(1), aligned(2))) const unsigned short gu16;
+    // the empty asm keeps each 32-bit offset's zero-extension next to its load, where instruction selection can fold
+    // it into the SGPR-base addressing form (hoisted out of the loop it becomes a 64-bit add per load)
+    uint32_t od = o.d, oq = o.qs, os = o.sg, oh = o.qh, oc = o.sc;
+    asm volatile("" : "+v"(od), "+v"(oq), "+v"(os), "+v"(oh), "+v"(oc));
     RawSub r;
-    r.d = load_u16(blk);
-    r.q0 = load_u32_a2(blk + 2 + 8 * ib);
-    r.q1 = load_u32_a2(blk + 6 + 8 * ib);
-    r.sg = load_u32_a2(blk + 74 + 4 * ib);
-    r.hs = (uint32_t) blk[66 + ib] | ((uint32_t) blk[106 + (ib >> 1)] << 8);
+    r.d = *(gu16*) (unit + od);
+    r.q0 = *(gu32*) (unit + oq);
+    r.q1 = *(gu32*) (unit + oq + 4);
+    r.sg = *(gu32*) (unit + os);
+    r.qh = unit[oh];
+    r.sc = unit[oc];
     return r;
 }
 
+// byte address into the signed codebook of group j of a sub-block: (sign nibble << 9 | high bit << 8 | code) * 4.
+// Five VALU ops: byte select with shift (SDWA), two shifts, two and-or; the empty asm keeps the two and-or apart.
+__device__ __forceinline__ uint32_t code_addr(const RawSub& r, int j) {
+    uint32_t a = (((j < 4 ? r.q0 : r.q1) >> (8 * (j & 3))) & 0xFFu) << 2;
+    const uint32_t sg = 4 * j <= 11 ? r.sg << (11 - 4 * j) : r.sg >> (4 * j - 11);
+    a = (sg & 0x7800u) | a;
+    asm volatile("" : "+v"(a));
+    const uint32_t qh = r.qh << (10 - j);
+    return (qh & 0x400u) | a;
+}
+
+// sum over groups of `width` lanes with DPP moves (no LDS traffic). The lane with the highest index of each group
+// ends with the group's sum (for width <= 16 every lane does).
+template <int width>
+__device__ __forceinline__ float dpp_group_sum(float v) {
+#define FNX_DPP_ADD(ctrl, rmask)                                                                                          \
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, rmask, 0xF, false))
+    if constexpr (width >= 2) FNX_DPP_ADD(0xB1, 0xF);    // quad_perm [1,0,3,2]
+    if constexpr (width >= 4) FNX_DPP_ADD(0x4E, 0xF);    // quad_perm [2,3,0,1]
+    if constexpr (width >= 8) FNX_DPP_ADD(0x141, 0xF);   // row_half_mirror
+    if constexpr (width >= 16) FNX_DPP_ADD(0x140, 0xF);  // row_mirror
+    if constexpr (width >= 32) FNX_DPP_ADD(0x142, 0xA);  // row_bcast15 into rows 1 and 3
+    if constexpr (width >= 64) FNX_DPP_ADD(0x143, 0xC);  // row_bcast31 into rows 2 and 3
+#undef FNX_DPP_ADD
+    return v;
+}
+
 // SBR: sub-blocks per weight row (ncols / 32), a power of two <= 64. NT: tokens of the job held in registers.
-template <int SBR, int NT>
-__device__ __forceinline__ void job_units(const uint32_t* __restrict__ tab, const uint8_t* __restrict__ we, size_t row_bytes, int nrows,
-                                          int ua, int ub, const fnx_job* __restrict__ jb, int t0, const uint8_t* __restrict__ y,
+// R: units in flight per wave: the loads of the next R units are issued before the current R are decoded.
+template <int SBR, int NT, int R>
+__device__ __forceinline__ void job_units(const uint32_t* __restrict__ tab, const uint8_t* __restrict__ we, size_t row_bytes, int ua,
+                                          int ub, const fnx_job* __restrict__ jb, int t0, const uint8_t* __restrict__ y,
                                           float* __restrict__ out, int out_stride) {
     constexpr int RW = 64 / SBR;   // rows per unit
     const int lane = threadIdx.x & 63, g = lane / SBR, kb = lane % SBR, sb = kb >> 3, ib = kb & 7;
     int xs[NT][8];
     float dx[NT];
+    float* orow[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-        const uint8_t* yb = y + ((size_t) jb->y[t0 + t] * SBR + kb) * FNX_Q8_1_BLOCK;
+        const uint8_t* yb = y + ((size_t) uniform(jb->y[t0 + t]) * SBR + kb) * FNX_Q8_1_BLOCK;
         dx[t] = half_bits_to_float(*reinterpret_cast<const unsigned short*>(yb));
 #pragma unroll
         for (int j = 0; j < 8; ++j) xs[t][j] = reinterpret_cast<const int*>(yb + 4)[j];
+        orow[t] = out + (size_t) uniform(jb->out[t0 + t]) * out_stride + g;
     }
-    const size_t lane_off = (size_t) g * row_bytes + (size_t) sb * FNX_IQ3S_BLOCK;
-    const uint8_t* p = we + (size_t) ua * RW * row_bytes + lane_off;
+    LaneOffs o;
+    o.d = (uint32_t) (g * row_bytes) + sb * FNX_IQ3S_BLOCK;
+    o.qs = o.d + 2 + 8 * ib;
+    o.qh = o.d + 66 + ib;
+    o.sg = o.d + 74 + 4 * ib;
+    o.sc = o.d + 106 + (ib >> 1);
     const size_t step = (size_t) RW * row_bytes;
-    bool live = ua * RW + g < nrows;
-    RawSub cur = live ? load_sub(p, ib) : RawSub{};
-    for (int u = ua; u < ub; ++u) {
-        const bool live_next = u + 1 < ub && (u + 1) * RW + g < nrows;
-        RawSub nxt = cur;
-        if (live_next) nxt = load_sub(p + step, ib);
-        int sum[NT];
+    const int last = ub - 1;
+    // a unit's address as a scalar pair, the lane's field offsets as 32-bit registers: global_load with an SGPR base
+    auto unit_at = [&](int ui) { return as_global(uniform_ptr(we + (size_t) min(ui, last) * step)); };
+    const int sc_shift = 4 * (ib & 1);
+    RawSub cur[R];
 #pragma unroll
-        for (int t = 0; t < NT; ++t) sum[t] = 0;
+    for (int r = 0; r < R; ++r) cur[r] = load_sub(unit_at(ua + r), o);
+    for (int u = ua; u < ub; u += R) {
+        RawSub nxt[R];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const uint32_t code = (((j < 4 ? cur.q0 : cur.q1) >> (8 * (j & 3))) & 0xFFu) | (((cur.hs >> j) & 1u) << 8) |
-                                  (((cur.sg >> (4 * j)) & 0xFu) << 9);
-            const int w4 = (int) tab[code];
+        for (int r = 0; r < R; ++r) nxt[r] = load_sub(unit_at(u + R + r), o);   // past the end: the last unit again
 #pragma unroll
-            for (int t = 0; t < NT; ++t) sum[t] = __builtin_amdgcn_sdot4(w4, xs[t][j], sum[t], false);
+        for (int r = 0; r < R; ++r) {
+            int w4[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) w4[j] = *reinterpret_cast<const int*>(reinterpret_cast<const uint8_t*>(tab) + code_addr(cur[r], j));
+            const int sc = 1 + 2 * (int) ((cur[r].sc >> sc_shift) & 0xFu);
+            const float dw = half_bits_to_float(cur[r].d);
+            const bool store = kb == SBR - 1 && u + r < ub;
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                int sum = 0;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) sum = __builtin_amdgcn_sdot4(w4[j], xs[t][j], sum, false);
+                // one sub-block's term exactly as the reference forms it: (d_w * d_x) * (float) (sumi * (1 + 2 s))
+                const float v = dpp_group_sum<SBR>((dw * dx[t]) * (float) __mul24(sum, sc));
+                if (store) orow[t][(size_t) (u + r) * RW] = v;
+            }
         }
-        const int sc = 1 + 2 * (int) ((cur.hs >> (8 + 4 * (ib & 1))) & 0xFu);
-        const float dw = half_bits_to_float(cur.d);
-        const int row = u * RW + g;
 #pragma unroll
-        for (int t = 0; t < NT; ++t) {
-            // one sub-block's term exactly as the reference forms it: (d_w * d_x) * (float) (sumi * (1 + 2 s))
-            float v = (dw * dx[t]) * (float) __mul24(sum[t], sc);
-            if (!live) v = 0.f;
-            v = group_sum<SBR>(v);
-            if (kb == 0 && live) out[(size_t) jb->out[t0 + t] * out_stride + row] = v;
-        }
-        cur = nxt;
-        live = live_next;
-        p += step;
+        for (int r = 0; r < R; ++r) cur[r] = nxt[r];
     }
 }
 
-template <int SBR>
+// WIDE: jobs of many rows go four tokens at a time (fewer units in flight to stay within the registers); the narrow
+// variant takes one or two tokens a pass, which is what a verify window's routed jobs have (1.15 rows on average)
+template <int SBR, bool WIDE>
 __device__ __forceinline__ void job_range(const uint32_t* tab, const uint8_t* we, const RowsArgs& a, int ua, int ub, const fnx_job* jb,
                                           const uint8_t* y) {
-    const int n = jb->n;
+    const int n = uniform(jb->n);
     for (int t0 = 0; t0 < n;) {
         const int nt = n - t0;
-        if (nt >= 4) {
-            job_units<SBR, 4>(tab, we, a.row_bytes, a.nrows, ua, ub, jb, t0, y, a.out, a.out_stride);
+        if (WIDE && nt >= 4) {
+            job_units<SBR, 4, 2>(tab, we, a.row_bytes, ua, ub, jb, t0, y, a.out, a.out_stride);
             t0 += 4;
-        } else if (nt == 3) {
-            job_units<SBR, 3>(tab, we, a.row_bytes, a.nrows, ua, ub, jb, t0, y, a.out, a.out_stride);
+        } else if (WIDE && nt == 3) {
+            job_units<SBR, 3, 2>(tab, we, a.row_bytes, ua, ub, jb, t0, y, a.out, a.out_stride);
             t0 += 3;
-        } else if (nt == 2) {
-            job_units<SBR, 2>(tab, we, a.row_bytes, a.nrows, ua, ub, jb, t0, y, a.out, a.out_stride);
+        } else if (nt >= 2) {
+            job_units<SBR, 2, 4>(tab, we, a.row_bytes, ua, ub, jb, t0, y, a.out, a.out_stride);
             t0 += 2;
         } else {
-            job_units<SBR, 1>(tab, we, a.row_bytes, a.nrows, ua, ub, jb, t0, y, a.out, a.out_stride);
+            job_units<SBR, 1, 4>(tab, we, a.row_bytes, ua, ub, jb, t0, y, a.out, a.out_stride);
             t0 += 1;
         }
     }
 }
 
-template <int SBR>
-__global__ void __launch_bounds__(1024) k_iq3s_jobs(const RowsArgs a) {
+// requires nrows % (64 / SBR) == 0 (checked by the launcher): every unit is whole
+template <int SBR, bool WIDE>
+__global__ void __launch_bounds__(512) k_iq3s_jobs(const RowsArgs a) {
     __shared__ uint32_t tab[SGRID_WORDS];
     for (int i = threadIdx.x; i < SGRID_WORDS; i += blockDim.x) tab[i] = g_sgrid.v[i];
     __syncthreads();
     constexpr int RW = 64 / SBR;
-    const int nj = a.njobs ? min(*a.njobs, a.njobs_max) : a.njobs_max;
-    const int upj = (a.nrows + RW - 1) / RW;   // units per job
+    const int nj = a.njobs ? min(uniform(*a.njobs), a.njobs_max) : a.njobs_max;
+    const int upj = a.nrows / RW;   // units per job
     const long total = (long) nj * upj;
     const int wpb = blockDim.x >> 6;
-    const long gw = (long) blockIdx.x * wpb + (threadIdx.x >> 6), nw = (long) gridDim.x * wpb;
+    const long gw = (long) blockIdx.x * wpb + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), nw = (long) gridDim.x * wpb;
     long u = total * gw / nw;
     const long u1 = total * (gw + 1) / nw;
     const uint8_t* y = a.y ? a.y : g_moe_hq;
@@ -360,8 +411,9 @@ __global__ void __launch_bounds__(1024) k_iq3s_jobs(const RowsArgs a) {
         const int ji = (int) (u / upj), ul = (int) (u % upj);
         const int ue = (int) min((long) upj, ul + (u1 - u));
         const fnx_job* jb = a.jobs + ji;
-        const uint8_t* we = a.ep ? a.ep[jb->w] : a.wbase + (size_t) jb->w * a.w_stride;
-        job_range<SBR>(tab, we, a, ul, ue, jb, y);
+        const int w = uniform(jb->w);
+        const uint8_t* we = a.ep ? uniform_ptr(a.ep[w]) : a.wbase + (size_t) w * a.w_stride;
+        job_range<SBR, WIDE>(tab, we, a, ul, ue, jb, y);
         u += ue - ul;
     }
 }
@@ -381,16 +433,20 @@ __global__ void __launch_bounds__(256) k_iq3s_jobs_any(const RowsArgs a) {
         float acc = 0.f;
         for (int kb = lane; kb < sbr; kb += 64) {
             const int ib = kb & 7;
-            const RawSub r = load_sub(we + (size_t) (kb >> 3) * FNX_IQ3S_BLOCK, ib);
+            LaneOffs o;
+            o.d = (uint32_t) (kb >> 3) * FNX_IQ3S_BLOCK;
+            o.qs = o.d + 2 + 8 * ib;
+            o.qh = o.d + 66 + ib;
+            o.sg = o.d + 74 + 4 * ib;
+            o.sc = o.d + 106 + (ib >> 1);
+            const RawSub r = load_sub(as_global(we), o);
             const uint8_t* yb = y + ((size_t) jb->y[t] * sbr + kb) * FNX_Q8_1_BLOCK;
             int sum = 0;
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                const uint32_t code = (((j < 4 ? r.q0 : r.q1) >> (8 * (j & 3))) & 0xFFu) | (((r.hs >> j) & 1u) << 8) |
-                                      (((r.sg >> (4 * j)) & 0xFu) << 9);
-                sum = __builtin_amdgcn_sdot4((int) g_sgrid.v[code], reinterpret_cast<const int*>(yb + 4)[j], sum, false);
+                sum = __builtin_amdgcn_sdot4((int) g_sgrid.v[code_addr(r, j) >> 2], reinterpret_cast<const int*>(yb + 4)[j], sum, false);
             }
-            const int sc = 1 + 2 * (int) ((r.hs >> (8 + 4 * (ib & 1))) & 0xFu);
+            const int sc = 1 + 2 * (int) ((r.sc >> (4 * (ib & 1))) & 0xFu);
             acc += (half_bits_to_float(r.d) * half_bits_to_float(*reinterpret_cast<const unsigned short*>(yb))) * (float) (sum * sc);
         }
         acc = group_sum<64>(acc);
@@ -496,8 +552,9 @@ __global__ void k_accept(const int* __restrict__ rows, const int* __restrict__ o
 }
 
 // ================================================================ launchers
+// wide: the jobs are expected to hold many rows each (a dense matrix over the whole window) rather than one or two
 static int rows_launch(const fnx_dw* W, size_t w_stride, const fnx_job* jobs, const int* njobs, int njobs_max, const void* y, float* out,
-                       int out_stride, void* st, const char* who) {
+                       int out_stride, void* st, const char* who, bool wide = false) {
     if (!W || !jobs || !out) return fail(std::string(who) + ": null argument");
     if (W->type != FNX_T_IQ3_S) return fail(std::string(who) + ": expert type " + std::to_string(W->type) + " not handled (IQ3_S only)");
     if (W->n_in <= 0 || W->n_in % 256 || W->n_out <= 0) return fail(std::string(who) + ": shape does not fit IQ3_S super-blocks");
@@ -507,16 +564,23 @@ static int rows_launch(const fnx_dw* W, size_t w_stride, const fnx_job* jobs, co
     RowsArgs a{(const uint8_t*) W->p, w_stride, (const uint8_t* const*) W->ep, W->row_bytes, W->n_out, W->n_in,
                jobs, njobs, njobs_max, (const uint8_t*) y, out, out_stride};
     hipStream_t s = (hipStream_t) st;
-    static const int blocks = env_int("FNX_ROWS_BLOCKS", 1024, 1, 65536), threads = env_int("FNX_ROWS_THREADS", 512, 64, 1024) / 64 * 64;
+    static const int blocks = env_int("FNX_ROWS_BLOCKS", 1024, 1, 65536), threads = env_int("FNX_ROWS_THREADS", 512, 64, 512) / 64 * 64;
     // no more waves than units: a wave with an empty range only loads the table
     const long units = (long) njobs_max * ((W->n_out * (long) (W->n_in / 32) + 63) / 64);
     const int grid = (int) std::max(1L, std::min((long) blocks, (units + threads / 64 - 1) / (threads / 64)));
-    switch (W->n_in) {
-        case 2048: k_iq3s_jobs<64><<<grid, threads, 0, s>>>(a); break;
-        case 1024: k_iq3s_jobs<32><<<grid, threads, 0, s>>>(a); break;
-        case 512: k_iq3s_jobs<16><<<grid, threads, 0, s>>>(a); break;
-        case 256: k_iq3s_jobs<8><<<grid, threads, 0, s>>>(a); break;
-        default: k_iq3s_jobs_any<<<dim3((W->n_out + 3) / 4, njobs_max), 256, 0, s>>>(a); break;
+    const int sbr = W->n_in / 32;
+    const bool whole_units = sbr <= 64 && 64 % sbr == 0 && W->n_out % (64 / sbr) == 0;
+    if (!whole_units) k_iq3s_jobs_any<<<dim3((W->n_out + 3) / 4, njobs_max), 256, 0, s>>>(a);
+    else if (wide) {
+        if (sbr == 64) k_iq3s_jobs<64, true><<<grid, threads, 0, s>>>(a);
+        else if (sbr == 32) k_iq3s_jobs<32, true><<<grid, threads, 0, s>>>(a);
+        else if (sbr == 16) k_iq3s_jobs<16, true><<<grid, threads, 0, s>>>(a);
+        else k_iq3s_jobs<8, true><<<grid, threads, 0, s>>>(a);
+    } else {
+        if (sbr == 64) k_iq3s_jobs<64, false><<<grid, threads, 0, s>>>(a);
+        else if (sbr == 32) k_iq3s_jobs<32, false><<<grid, threads, 0, s>>>(a);
+        else if (sbr == 16) k_iq3s_jobs<16, false><<<grid, threads, 0, s>>>(a);
+        else k_iq3s_jobs<8, false><<<grid, threads, 0, s>>>(a);
     }
     return launch_status(who);
 }
@@ -541,7 +605,7 @@ int fnx_quantize_q8_1(const float* x, void* q, int n, int rows, void* st) {
 int fnx_mmvq(const fnx_dw* W, size_t w_stride, const fnx_job* jobs, const int* njobs, int njobs_max, const void* y, float* out,
              int out_stride, void* st) {
     if (!y) return fail("mmvq: null activations");
-    return rows_launch(W, w_stride, jobs, njobs, njobs_max, y, out, out_stride, st, "mmvq");
+    return rows_launch(W, w_stride, jobs, njobs, njobs_max, y, out, out_stride, st, "mmvq", njobs_max <= 8);
 }
 
 static int gemv_any(const void* W, bool bf, const float* x, float* y, int rows, int n, int T, void* st, const char* who) {
@@ -691,11 +755,11 @@ int fnx_moe_verify_layer(const fnx_moe_layer* L, const float* x, int T, float* o
                                          0, 1);
     if (launch_status("moe_verify_layer topk")) return 1;
     if (rows_launch(&L->gu, L->gu_stride, ws->jobs_gu, ws->njobs, P, ws->xq, ws->gu, 2 * ff, st, "moe_verify_layer gate|up")) return 1;
-    if (rows_launch(&L->sh_gu, 0, ws->jobs_gu + P, nullptr, 1, ws->xq, ws->gu, 2 * ff, st, "moe_verify_layer shared gate|up")) return 1;
+    if (rows_launch(&L->sh_gu, 0, ws->jobs_gu + P, nullptr, 1, ws->xq, ws->gu, 2 * ff, st, "moe_verify_layer shared gate|up", true)) return 1;
     k_swiglu_q8_1<<<dim3((ff / 32 + 7) / 8, P + T), 256, 0, s>>>(ws->gu, ws->gu + ff, (size_t) 2 * ff, nullptr, ff);
     if (launch_status("moe_verify_layer swiglu")) return 1;
     if (rows_launch(&L->down, L->down_stride, ws->jobs_dn, ws->njobs, P, nullptr, ws->part, n, st, "moe_verify_layer down")) return 1;
-    if (rows_launch(&L->sh_down, 0, ws->jobs_dn + P, nullptr, 1, nullptr, ws->part, n, st, "moe_verify_layer shared down")) return 1;
+    if (rows_launch(&L->sh_down, 0, ws->jobs_dn + P, nullptr, 1, nullptr, ws->part, n, st, "moe_verify_layer shared down", true)) return 1;
     return fnx_moe_combine(ws->part, ws->topw, ws->part + (size_t) P * n, ws->logits + L->nexp, L->nexp + 1, out, T, n, L->topk, st);
 }
 
