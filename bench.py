@@ -35,6 +35,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--layers", type=int, default=16, help="distinct weight sets cycled through")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0: skip)")
+    ap.add_argument("--raw-layout", action="store_true", help="leave the weights as raw ggml blocks (skip the load-time re-laying)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
@@ -62,9 +63,15 @@ def main():
         down = rand_iq3s(NEXP * N * FF // 256)
         sh_gu = rand_iq3s(2 * FF * N // 256)
         sh_down = rand_iq3s(N * FF // 256)
-        L = pkg.MoeLayer(N, FF, NEXP, TOPK, router.data_ptr(), 0, pkg.dw(gu, N, 2 * FF), GU_BYTES, pkg.dw(down, FF, N), DN_BYTES,
-                         pkg.dw(sh_gu, N, 2 * FF), pkg.dw(sh_down, FF, N))
-        layers.append((L, router, gu, down, sh_gu, sh_down))
+        # the CPU leg reads raw ggml blocks: keep weight set 0's before the load-time re-laying (fnx_iq3s_repack, in place)
+        raw = [a.cpu().numpy() for a in (gu, down, sh_gu, sh_down)] if not layers and args.cpu_seconds > 0 else None
+        if not args.raw_layout:
+            for w in (gu, down, sh_gu, sh_down):
+                dev.ok(lib.fnx_iq3s_repack(w.data_ptr(), w.data_ptr(), w.numel() // IQ3S_BLOCK * 256, dev.st()))
+        pk = not args.raw_layout
+        L = pkg.MoeLayer(N, FF, NEXP, TOPK, router.data_ptr(), 0, pkg.dw(gu, N, 2 * FF, packed=pk), GU_BYTES, pkg.dw(down, FF, N, packed=pk),
+                         DN_BYTES, pkg.dw(sh_gu, N, 2 * FF, packed=pk), pkg.dw(sh_down, FF, N, packed=pk))
+        layers.append((L, router, gu, down, sh_gu, sh_down, raw))
     NX = 64
     xs = torch.randn((NX, T, N), device="cuda", generator=g)
     outs = torch.zeros((NX, T, N), device="cuda")
@@ -111,7 +118,7 @@ def main():
         dev.ok(lib.fnx_router_route(L.router, 0, x.data_ptr(), ws.logits, T, N, NEXP, TOPK, ws.topi, ws.topw, ws.jobs_gu, ws.jobs_dn, ws.njobs, st))
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
-        dev.ok(lib.fnx_moe_gate_up(C.byref(L.gu), L.gu_stride, ws.jobs_gu, ws.njobs, P, ws.xq, ws.gu, st))
+        dev.ok(lib.fnx_moe_gate_up(C.byref(L.gu), L.gu_stride, ws.jobs_gu, ws.njobs, P, ws.xq, ws.gu, TOPK, st))
         e1.record()
         evs.append((e0, e1, i))
     torch.cuda.synchronize()
@@ -126,8 +133,8 @@ def main():
         import oracle_lib
         oracle = oracle_lib.Oracle()
         threads = min(os.cpu_count() or 1, 16)
-        L, router, gu, down, sh_gu, sh_down = layers[0]
-        h = [a.cpu().numpy() for a in (router, gu, down, sh_gu, sh_down)]
+        L, router = layers[0][0], layers[0][1]
+        h = [router.cpu().numpy()] + layers[0][6]
         xh = xs[0].cpu().numpy()
         r = oracle.moe_verify_layer(N, FF, NEXP, TOPK, *h, xh, threads=threads)   # warm-up, and a last parity check
         dev.ok(lib.fnx_moe_verify_layer(C.byref(L), xs[0].data_ptr(), T, outs[0].data_ptr(), C.byref(ws), st))
@@ -153,9 +160,9 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int8 x IQ3_S (i32 dot, f32 accumulate)", "data": "synthetic",
         "config": {"workload": "config 2: one MoE verify layer, T=16, hidden 2048, 512 IQ3_S experts top-10, SwiGLU ff 512, shared expert, f32 router",
-                   "weight_sets": args.layers, "distinct_experts_per_step": u_mean, "step_algorithmic_bytes": step_bytes,
+                   "weight_layout": "raw ggml blocks" if args.raw_layout else "unit64 (re-laid once at load, same bytes)", "weight_sets": args.layers, "distinct_experts_per_step": u_mean, "step_algorithmic_bytes": step_bytes,
                    "step_hbm_frac": step_bytes / (ms_per_step * 1e-3) / HBM_PEAK},
-        "roofline": {"bound": "hbm", "kernel": "k_iq3s_jobs<64> (routed gate|up)", "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+        "roofline": {"bound": "hbm", "kernel": "k_iq3s_jobs<64, narrow, " + ("raw" if args.raw_layout else "unit64") + "> (routed gate|up)", "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK, "traffic": None, "kernel_ms": k_ms, "algorithmic_bytes": k_bytes},
         "cpu_baseline": cpu,
     }

@@ -28,6 +28,7 @@ extern "C" {
 #define FNX_MAXT 16        /* rows per verify window (model.hpp:43) */
 #define FNX_PF_JOB 64      /* rows per prefill job (kernels.hpp:27-30) */
 #define FNX_T_IQ3_S 21u    /* ggml type id (gguf.hpp:22-27) */
+#define FNX_T_IQ3S_UNIT64 1021u /* this library's load-time re-laying of IQ3_S (fnx_iq3s_repack); not a ggml type */
 #define FNX_IQ3S_BLOCK 110 /* bytes per 256 weights */
 #define FNX_Q8_1_BLOCK 36  /* bytes per 32 activations: half d, half sum, int8 qs[32] */
 #define FNX_ERR_NONFINITE 16u /* error-word bit (engine_impl.hpp:211-218) */
@@ -51,7 +52,7 @@ typedef struct fnx_bigjob {
 /* model.hpp:84-94 (DW) without the split-Q8_0 twin, which this path does not use */
 typedef struct fnx_dw {
     const void* p;          /* raw ggml blocks, row-major over output rows */
-    uint32_t type;          /* FNX_T_IQ3_S */
+    uint32_t type;          /* FNX_T_IQ3_S (raw ggml blocks) or FNX_T_IQ3S_UNIT64 (after fnx_iq3s_repack) */
     int n_in, n_out;        /* columns, rows */
     size_t row_bytes;       /* n_in / 256 * 110 */
     const void* const* ep;  /* optional device table: expert e's matrix; null: expert e at p + e * stride */
@@ -61,6 +62,14 @@ typedef struct fnx_dw {
 const char* fnx_last_error(void);
 /* library build id, and whether a usable GPU is present (no device work is started) */
 const char* fnx_version(void);
+
+/* Load-time re-laying of IQ3_S weights, the counterpart of the reference's own load-time layouts (the split Q8_0
+ * twin, model.hpp:78-82; tensor_convert.hpp): raw ggml block_iq3_s -> "unit64", the same 110 bytes per 256 weights
+ * with each 32-weight sub-block's codes, high bits and signs merged into eight 13-bit codebook indexes. A tensor of
+ * n_weights (a multiple of 2048) in memory order; dst may equal src. Afterwards describe the tensor with
+ * fnx_dw.type = FNX_T_IQ3S_UNIT64: every operator below takes both types and gives the same results; the re-laid
+ * type is the fast path. Rows must have 256, 512, 1024 or 2048 columns and expert strides must be multiples of 880. */
+int fnx_iq3s_repack(const void* src, void* dst, size_t n_weights, void* st);
 
 /* kernels.hpp:41  quantize_q8_1: f32 rows of n -> q8_1 blocks, ggml's rounding (kernels.cu:131-145) */
 int fnx_quantize_q8_1(const float* x, void* q, int n, int rows, void* st);
@@ -91,9 +100,11 @@ int fnx_swiglu_q8_1(const float* g, const float* u, void* q, int n, int rows, vo
 /* kernels.hpp:349  swiglu_stacked_q8_1: T rows of [gate (ffs) | up (ffs)] -> q8_1 rows of ffs */
 int fnx_swiglu_stacked_q8_1(const float* gu, void* hq, int ffs, int T, void* st);
 
-/* kernels.hpp:319  moe_gate_up: gu rows of 2*ffs = A->n_out: [gate | up]; expert stride sa; xq: q8_1 rows of A->n_in */
+/* kernels.hpp:319  moe_gate_up: gu rows of 2*ffs = A->n_out: [gate | up]; expert stride sa; xq: q8_1 rows of A->n_in,
+ * one per row of the window: njobs_max / topk of them (njobs_max is the window's pairs, as in the reference, whose
+ * launcher takes T = njobs_max / TOPK, kernels.cu:2449); the jobs' y index them */
 int fnx_moe_gate_up(const fnx_dw* A, size_t sa, const fnx_job* jobs, const int* njobs, int njobs_max, const void* xq, float* gu,
-                    void* st);
+                    int topk, void* st);
 /* kernels.hpp:343  moe_down: part rows of A->n_out from silu(gate) * up of the gu rows (rows of 2 * A->n_in).
  * Like the reference (moe.cuh:592-594) the q8_1 rows of h live in one library-owned device buffer, so one MoE may be
  * in flight per device; njobs_max (the window's pairs) <= 176. */

@@ -8,11 +8,12 @@ import ctypes as C
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libfnx_mi355x.so")
+LIB_PATH = os.environ.get("FNX_LIB_PATH") or os.path.join(HERE, "libfnx_mi355x.so")
 
 MAXT = 16
 PF_JOB = 64
 T_IQ3_S = 21
+T_IQ3S_UNIT64 = 1021
 IQ3S_BLOCK = 110
 Q8_1_BLOCK = 36
 
@@ -45,6 +46,7 @@ EXPORTS = {
     # name: (restype, argtypes)
     "fnx_last_error": (C.c_char_p, []),
     "fnx_version": (C.c_char_p, []),
+    "fnx_iq3s_repack": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "fnx_quantize_q8_1": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
     "fnx_mmvq": (C.c_int, [C.POINTER(DW), C.c_size_t, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]),
     "fnx_gemv_f32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]),
@@ -55,7 +57,7 @@ EXPORTS = {
                                    C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "fnx_swiglu_q8_1": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
     "fnx_swiglu_stacked_q8_1": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
-    "fnx_moe_gate_up": (C.c_int, [C.POINTER(DW), C.c_size_t, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "fnx_moe_gate_up": (C.c_int, [C.POINTER(DW), C.c_size_t, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]),
     "fnx_moe_down": (C.c_int, [C.POINTER(DW), C.c_size_t, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
     "fnx_moe_combine": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_int,
                                   C.c_void_p]),
@@ -95,9 +97,9 @@ def check(status):
         raise FnxError(lib().fnx_last_error().decode())
 
 
-def dw(tensor_or_ptr, n_in, n_out, ep=None):
+def dw(tensor_or_ptr, n_in, n_out, ep=None, packed=False):
     p = tensor_or_ptr if isinstance(tensor_or_ptr, int) or tensor_or_ptr is None else tensor_or_ptr.data_ptr()
-    return DW(p, T_IQ3_S, n_in, n_out, n_in // 256 * IQ3S_BLOCK, ep)
+    return DW(p, T_IQ3S_UNIT64 if packed else T_IQ3_S, n_in, n_out, n_in // 256 * IQ3S_BLOCK, ep)
 
 
 def stream_ptr():

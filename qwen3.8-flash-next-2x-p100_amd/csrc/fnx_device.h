@@ -64,6 +64,10 @@ __device__ __forceinline__ const uint8_t* uniform_ptr(const uint8_t* p) {
     return (const uint8_t*) (uintptr_t) ((uint64_t) hi << 32 | lo);
 }
 
+// global-memory byte pointer (address space 1): loads through it are global_load, never flat_load
+typedef const __attribute__((address_space(1))) uint8_t* gbytes;
+__device__ __forceinline__ gbytes as_global(const uint8_t* p) { return (gbytes) (uintptr_t) p; }
+
 // little-endian loads from addresses that are only 2-byte aligned (IQ3_S blocks are 110 bytes)
 __device__ __forceinline__ uint32_t load_u32_a2(const uint8_t* p) {
     uint32_t v;

@@ -252,11 +252,8 @@ struct RowsArgs {
     const uint8_t* y;   // q8_1 rows; null: the library's pair buffer
     float* out;
     int out_stride;
+    int y_rows;         // how many activation rows y holds when that is known to be at most a window's (else 0)
 };
-
-// global-memory byte pointer (address space 1): loads through it are global_load, never flat_load
-typedef const __attribute__((address_space(1))) uint8_t* gbytes;
-__device__ __forceinline__ gbytes as_global(const uint8_t* p) { return (gbytes) (uintptr_t) p; }
 
 struct RawSub {   // one lane's share of a unit as read from memory; nothing is combined until it is used
     uint32_t q0, q1, sg, qh, sc, d;   // codes 0..3, 4..7, sign nibbles, high bits, scales byte, d bits
@@ -392,14 +389,20 @@ __device__ __forceinline__ void job_range(const uint32_t* tab, const uint8_t* we
     }
 }
 
-// requires nrows % (64 / SBR) == 0 (checked by the launcher): every unit is whole
-template <int SBR, bool WIDE>
+}  // namespace fnx
+#include "k_iq3s_packed.h"
+namespace fnx {
+
+// requires nrows % (64 / SBR) == 0 (checked by the launcher): every unit is whole. PACKED: the unit64 layout.
+// The waves of the grid split the units of all jobs evenly and walk them in order (consecutive rows, one expert after
+// the other), so a wave streams one contiguous range of memory and changes job at most once or twice.
+template <int SBR, bool WIDE, bool PACKED>
 __global__ void __launch_bounds__(512) k_iq3s_jobs(const RowsArgs a) {
     __shared__ uint32_t tab[SGRID_WORDS];
     for (int i = threadIdx.x; i < SGRID_WORDS; i += blockDim.x) tab[i] = g_sgrid.v[i];
-    __syncthreads();
     constexpr int RW = 64 / SBR;
     const int nj = a.njobs ? min(uniform(*a.njobs), a.njobs_max) : a.njobs_max;
+    __syncthreads();
     const int upj = a.nrows / RW;   // units per job
     const long total = (long) nj * upj;
     const int wpb = blockDim.x >> 6;
@@ -413,7 +416,8 @@ __global__ void __launch_bounds__(512) k_iq3s_jobs(const RowsArgs a) {
         const fnx_job* jb = a.jobs + ji;
         const int w = uniform(jb->w);
         const uint8_t* we = a.ep ? uniform_ptr(a.ep[w]) : a.wbase + (size_t) w * a.w_stride;
-        job_range<SBR, WIDE>(tab, we, a, ul, ue, jb, y);
+        if constexpr (PACKED) packed_range<SBR, WIDE>(tab, we, ul, ue, jb, y, a.out, a.out_stride);
+        else job_range<SBR, WIDE>(tab, we, a, ul, ue, jb, y);
         u += ue - ul;
     }
 }
@@ -552,36 +556,55 @@ __global__ void k_accept(const int* __restrict__ rows, const int* __restrict__ o
 }
 
 // ================================================================ launchers
+static int cu_count() {
+    static int cus[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (!cus[dev]) {
+        int n = 0;
+        cus[dev] = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0 ? n : 256;
+    }
+    return cus[dev];
+}
 // wide: the jobs are expected to hold many rows each (a dense matrix over the whole window) rather than one or two
 static int rows_launch(const fnx_dw* W, size_t w_stride, const fnx_job* jobs, const int* njobs, int njobs_max, const void* y, float* out,
-                       int out_stride, void* st, const char* who, bool wide = false) {
+                       int out_stride, void* st, const char* who, bool wide = false, int y_rows = 0) {
     if (!W || !jobs || !out) return fail(std::string(who) + ": null argument");
-    if (W->type != FNX_T_IQ3_S) return fail(std::string(who) + ": expert type " + std::to_string(W->type) + " not handled (IQ3_S only)");
+    if (W->type != FNX_T_IQ3_S && W->type != FNX_T_IQ3S_UNIT64)
+        return fail(std::string(who) + ": expert type " + std::to_string(W->type) + " not handled (IQ3_S only)");
     if (W->n_in <= 0 || W->n_in % 256 || W->n_out <= 0) return fail(std::string(who) + ": shape does not fit IQ3_S super-blocks");
     if (W->row_bytes != (size_t) (W->n_in / 256) * FNX_IQ3S_BLOCK) return fail(std::string(who) + ": row_bytes does not match n_in");
     if (njobs_max <= 0) return fail(std::string(who) + ": njobs_max must be positive");
     if (!W->p && !W->ep) return fail(std::string(who) + ": no weights");
     RowsArgs a{(const uint8_t*) W->p, w_stride, (const uint8_t* const*) W->ep, W->row_bytes, W->n_out, W->n_in,
-               jobs, njobs, njobs_max, (const uint8_t*) y, out, out_stride};
+               jobs, njobs, njobs_max, (const uint8_t*) y, out, out_stride, y_rows};
     hipStream_t s = (hipStream_t) st;
-    static const int blocks = env_int("FNX_ROWS_BLOCKS", 1024, 1, 65536), threads = env_int("FNX_ROWS_THREADS", 512, 64, 512) / 64 * 64;
-    // no more waves than units: a wave with an empty range only loads the table
+    // two blocks of 8 waves per CU by default: every block copies the 32 KiB codebook into LDS once
+    static const int blocks = env_int("FNX_ROWS_BLOCKS", 0, 0, 65536), threads = env_int("FNX_ROWS_THREADS", 512, 64, 512) / 64 * 64;
+    // no more waves than groups of four units: a wave with an empty range only fills the LDS
     const long units = (long) njobs_max * ((W->n_out * (long) (W->n_in / 32) + 63) / 64);
-    const int grid = (int) std::max(1L, std::min((long) blocks, (units + threads / 64 - 1) / (threads / 64)));
+    const long want = (units / 4 + threads / 64 - 1) / (threads / 64);
+    const int grid = (int) std::max(1L, std::min((long) (blocks ? blocks : 2 * cu_count()), want));
     const int sbr = W->n_in / 32;
     const bool whole_units = sbr <= 64 && 64 % sbr == 0 && W->n_out % (64 / sbr) == 0;
+    const bool packed = W->type == FNX_T_IQ3S_UNIT64;
+    if (packed && !whole_units) return fail(std::string(who) + ": the unit64 layout needs rows of 256, 512, 1024 or 2048 columns in whole units");
+    if (packed && (w_stride % UNIT_BYTES)) return fail(std::string(who) + ": the unit64 layout needs expert strides in whole units");
+#define FNX_ROWS(SBR_, WIDE_, PACKED_) k_iq3s_jobs<SBR_, WIDE_, PACKED_><<<grid, threads, 0, s>>>(a)
+#define FNX_ROWS_SBR(WIDE_, PACKED_)                                                                     \
+    do {                                                                                                 \
+        if (sbr == 64) FNX_ROWS(64, WIDE_, PACKED_);                                                     \
+        else if (sbr == 32) FNX_ROWS(32, WIDE_, PACKED_);                                                \
+        else if (sbr == 16) FNX_ROWS(16, WIDE_, PACKED_);                                                \
+        else FNX_ROWS(8, WIDE_, PACKED_);                                                                \
+    } while (0)
     if (!whole_units) k_iq3s_jobs_any<<<dim3((W->n_out + 3) / 4, njobs_max), 256, 0, s>>>(a);
-    else if (wide) {
-        if (sbr == 64) k_iq3s_jobs<64, true><<<grid, threads, 0, s>>>(a);
-        else if (sbr == 32) k_iq3s_jobs<32, true><<<grid, threads, 0, s>>>(a);
-        else if (sbr == 16) k_iq3s_jobs<16, true><<<grid, threads, 0, s>>>(a);
-        else k_iq3s_jobs<8, true><<<grid, threads, 0, s>>>(a);
-    } else {
-        if (sbr == 64) k_iq3s_jobs<64, false><<<grid, threads, 0, s>>>(a);
-        else if (sbr == 32) k_iq3s_jobs<32, false><<<grid, threads, 0, s>>>(a);
-        else if (sbr == 16) k_iq3s_jobs<16, false><<<grid, threads, 0, s>>>(a);
-        else k_iq3s_jobs<8, false><<<grid, threads, 0, s>>>(a);
-    }
+    else if (packed && wide) FNX_ROWS_SBR(true, true);
+    else if (packed) FNX_ROWS_SBR(false, true);
+    else if (wide) FNX_ROWS_SBR(true, false);
+    else FNX_ROWS_SBR(false, false);
+#undef FNX_ROWS_SBR
+#undef FNX_ROWS
     return launch_status(who);
 }
 
@@ -594,6 +617,14 @@ extern "C" {
 
 const char* fnx_last_error(void) { return t_err.c_str(); }
 const char* fnx_version(void) { return "fnx-mi355x gfx950 verify path 0.1"; }
+
+int fnx_iq3s_repack(const void* src, void* dst, size_t n_weights, void* st) {
+    if (!src || !dst) return fail("iq3s_repack: null argument");
+    if (n_weights == 0 || n_weights % 2048) return fail("iq3s_repack: whole units of 2048 weights");
+    const long units = (long) (n_weights / 2048);
+    k_iq3s_repack<<<(unsigned) ((units + 3) / 4), 256, 0, (hipStream_t) st>>>((const uint8_t*) src, (uint8_t*) dst, units);
+    return launch_status("iq3s_repack");
+}
 
 int fnx_quantize_q8_1(const float* x, void* q, int n, int rows, void* st) {
     if (!x || !q) return fail("quantize_q8_1: null argument");
@@ -661,10 +692,13 @@ int fnx_swiglu_stacked_q8_1(const float* gu, void* hq, int ffs, int T, void* st)
     return launch_status("swiglu_stacked_q8_1");
 }
 
-int fnx_moe_gate_up(const fnx_dw* A, size_t sa, const fnx_job* jobs, const int* njobs, int njobs_max, const void* xq, float* gu, void* st) {
+int fnx_moe_gate_up(const fnx_dw* A, size_t sa, const fnx_job* jobs, const int* njobs, int njobs_max, const void* xq, float* gu, int topk,
+                    void* st) {
     if (!xq) return fail("moe_gate_up: null activations");
     if (A && (A->n_out & 1)) return fail("moe_gate_up: rows are [gate | up], an even count");
-    return rows_launch(A, sa, jobs, njobs, njobs_max, xq, gu, A ? A->n_out : 0, st, "moe_gate_up");
+    if (topk < 1 || njobs_max % topk) return fail("moe_gate_up: njobs_max is the window's pairs, a multiple of topk");
+    // the window's rows: njobs_max / topk of them (kernels.cu:2449, T = njobs_max / TOPK); xq holds that many
+    return rows_launch(A, sa, jobs, njobs, njobs_max, xq, gu, A ? A->n_out : 0, st, "moe_gate_up", false, njobs_max / topk);
 }
 int fnx_moe_down(const fnx_dw* A, size_t sa, const fnx_job* jobs, const int* njobs, int njobs_max, const float* gu, float* part, void* st) {
     if (!A || !gu) return fail("moe_down: null argument");
@@ -754,8 +788,8 @@ int fnx_moe_verify_layer(const fnx_moe_layer* L, const float* x, int T, float* o
     k_topk_jobs<<<1, TK_THREADS, 0, s>>>(ws->logits, L->nexp + 1, T, L->nexp, L->topk, ws->topi, ws->topw, ws->jobs_gu, ws->jobs_dn, ws->njobs,
                                          0, 1);
     if (launch_status("moe_verify_layer topk")) return 1;
-    if (rows_launch(&L->gu, L->gu_stride, ws->jobs_gu, ws->njobs, P, ws->xq, ws->gu, 2 * ff, st, "moe_verify_layer gate|up")) return 1;
-    if (rows_launch(&L->sh_gu, 0, ws->jobs_gu + P, nullptr, 1, ws->xq, ws->gu, 2 * ff, st, "moe_verify_layer shared gate|up", true)) return 1;
+    if (rows_launch(&L->gu, L->gu_stride, ws->jobs_gu, ws->njobs, P, ws->xq, ws->gu, 2 * ff, st, "moe_verify_layer gate|up", false, T)) return 1;
+    if (rows_launch(&L->sh_gu, 0, ws->jobs_gu + P, nullptr, 1, ws->xq, ws->gu, 2 * ff, st, "moe_verify_layer shared gate|up", true, T)) return 1;
     k_swiglu_q8_1<<<dim3((ff / 32 + 7) / 8, P + T), 256, 0, s>>>(ws->gu, ws->gu + ff, (size_t) 2 * ff, nullptr, ff);
     if (launch_status("moe_verify_layer swiglu")) return 1;
     if (rows_launch(&L->down, L->down_stride, ws->jobs_dn, ws->njobs, P, nullptr, ws->part, n, st, "moe_verify_layer down")) return 1;

@@ -30,6 +30,35 @@ def random_iq3s(rng, nblocks, dmax=3e-4):
     return b.reshape(-1)
 
 
+def pack_unit64(raw):
+    """numpy restatement of the unit64 layout (written from the layout's description, independent of the kernel):
+    per 64 sub-blocks (880 bytes): each sub-block's eight 13-bit indexes (sign nibble << 9 | high bit << 8 | code) as
+    a 104-bit little-endian string split over plane A (bytes 0..7 of every sub-block, 512 bytes), plane B (bytes 8..11,
+    256 bytes) and plane C (byte 12, 64 bytes); then the 32 scale bytes in order, then the 8 d halves."""
+    raw = np.ascontiguousarray(raw, dtype=np.uint8).reshape(-1, 8, 110)      # units of 8 super-blocks
+    nu = raw.shape[0]
+    qs = raw[:, :, 2:66].reshape(nu, 8, 8, 8).astype(np.uint64)               # [unit][sb][ib][group]
+    qh = raw[:, :, 66:74].reshape(nu, 8, 8, 1).astype(np.uint64)
+    sg = raw[:, :, 74:106].reshape(nu, 8, 8, 4).astype(np.uint64)             # 4 sign bytes per sub-block
+    g = np.arange(8, dtype=np.uint64)
+    hb = (qh >> g) & np.uint64(1)
+    nib = (np.repeat(sg, 2, axis=3) >> ((g & np.uint64(1)) * np.uint64(4))) & np.uint64(0xF)
+    idx = qs | (hb << np.uint64(8)) | (nib << np.uint64(9))                    # [unit][sb][ib][8] 13-bit
+    idx = idx.reshape(nu, 64, 8)
+    out = np.zeros((nu, 880), dtype=np.uint8)
+    bits = np.zeros((nu, 64, 104), dtype=np.uint8)
+    for j in range(8):
+        for b in range(13):
+            bits[:, :, 13 * j + b] = (idx[:, :, j] >> np.uint64(b)) & np.uint64(1)
+    chunks = np.packbits(bits.reshape(nu, 64, 13, 8), axis=3, bitorder="little").reshape(nu, 64, 13)
+    out[:, 0:512] = chunks[:, :, 0:8].reshape(nu, 512)
+    out[:, 512:768] = chunks[:, :, 8:12].reshape(nu, 256)
+    out[:, 768:832] = chunks[:, :, 12]
+    out[:, 832:864] = raw[:, :, 106:110].reshape(nu, 32)
+    out[:, 864:880] = raw[:, :, 0:2].reshape(nu, 16)
+    return out.reshape(-1)
+
+
 JOB_DTYPE = np.dtype([("w", "<i4"), ("n", "<i4"), ("y", "<i4", (16,)), ("out", "<i4", (16,))])
 
 
@@ -80,18 +109,29 @@ class Dev:
         self.sync()
         return y.cpu().numpy()
 
-    def mmvq(self, w, w_stride, nrows, ncols, jobs, yq, out_rows, njobs_dev=True):
+    def repack(self, w, in_place=True):
+        """raw IQ3_S blocks (numpy) -> unit64 bytes (numpy), through the device"""
+        t = self.torch
+        src = self.up(w)
+        dst = src if in_place else self.zeros(src.numel(), t.uint8)
+        self.ok(self.lib.fnx_iq3s_repack(src.data_ptr(), dst.data_ptr(), w.size // 110 * 256, self.st()))
+        self.sync()
+        return dst.cpu().numpy()
+
+    def mmvq(self, w, w_stride, nrows, ncols, jobs, yq, out_rows, njobs_dev=True, packed=False):
         t = self.torch
         dw_, dj, dy = self.up(w), self.up(jobs.view(np.uint8).reshape(-1)), self.up(yq)
+        if packed:
+            self.ok(self.lib.fnx_iq3s_repack(dw_.data_ptr(), dw_.data_ptr(), w.size // 110 * 256, self.st()))
         out = self.zeros((out_rows, nrows), t.float32)
-        W = self.pkg.dw(dw_, ncols, nrows)
+        W = self.pkg.dw(dw_, ncols, nrows, packed=packed)
         nj = self.up(np.array([len(jobs)], dtype=np.int32))
         self.ok(self.lib.fnx_mmvq(C.byref(W), w_stride, dj.data_ptr(), nj.data_ptr() if njobs_dev else None, len(jobs), dy.data_ptr(),
                                   out.data_ptr(), nrows, self.st()))
         self.sync()
         return out.cpu().numpy()
 
-    def gemv_iq3s(self, w, nrows, ncols, x):
+    def gemv_iq3s(self, w, nrows, ncols, x, packed=False):
         T = x.shape[0]
         yq = self.quantize_q8_1(x)
         jobs = np.zeros((T + 15) // 16, dtype=JOB_DTYPE)
@@ -100,7 +140,7 @@ class Dev:
             jobs["n"][j] = nt
             jobs["y"][j, :nt] = np.arange(16 * j, 16 * j + nt)
             jobs["out"][j, :nt] = np.arange(16 * j, 16 * j + nt)
-        return self.mmvq(w, 0, nrows, ncols, jobs, yq, T)
+        return self.mmvq(w, 0, nrows, ncols, jobs, yq, T, packed=packed)
 
     def route(self, logits, nexp, topk, fused_W=None, x=None, bf16=False):
         t = self.torch
@@ -163,7 +203,7 @@ class Dev:
 class MoeLayerDev:
     """One MoE layer's weights on the device plus a workspace, for fnx_moe_verify_layer and the per-op calls."""
 
-    def __init__(self, dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, T=16):
+    def __init__(self, dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, T=16, packed=False):
         t = dev.torch
         self.dev, self.n, self.ff, self.nexp, self.topk = dev, n, ff, nexp, topk
         pkg = dev.pkg
@@ -171,8 +211,12 @@ class MoeLayerDev:
         self.gu, self.down, self.sh_gu, self.sh_down = dev.up(gu), dev.up(down), dev.up(sh_gu), dev.up(sh_down)
         self.gu_stride = 2 * ff * (n // 256) * 110
         self.down_stride = n * (ff // 256) * 110
-        self.L = pkg.MoeLayer(n, ff, nexp, topk, self.router.data_ptr(), 0, pkg.dw(self.gu, n, 2 * ff), self.gu_stride,
-                              pkg.dw(self.down, ff, n), self.down_stride, pkg.dw(self.sh_gu, n, 2 * ff), pkg.dw(self.sh_down, ff, n))
+        if packed:   # the load-time re-laying, in place
+            for w in (self.gu, self.down, self.sh_gu, self.sh_down):
+                dev.ok(dev.lib.fnx_iq3s_repack(w.data_ptr(), w.data_ptr(), w.numel() // 110 * 256, dev.st()))
+        self.L = pkg.MoeLayer(n, ff, nexp, topk, self.router.data_ptr(), 0, pkg.dw(self.gu, n, 2 * ff, packed=packed), self.gu_stride,
+                              pkg.dw(self.down, ff, n, packed=packed), self.down_stride, pkg.dw(self.sh_gu, n, 2 * ff, packed=packed),
+                              pkg.dw(self.sh_down, ff, n, packed=packed))
         P = T * topk
         self.P = P
         self.xq = dev.zeros(T * (n // 32) * 36, t.uint8)

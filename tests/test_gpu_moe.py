@@ -30,13 +30,14 @@ def make_layer(rng, n, ff, nexp, scale=1.0):
     return router, gu, down, sh_gu, sh_down
 
 
-def check_layer(dev, oracle, n, ff, nexp, topk, T, seed):
-    print(f"case moe layer n={n} ff={ff} nexp={nexp} topk={topk} T={T} seed={seed}", flush=True)
+def check_layer(dev, oracle, n, ff, nexp, topk, T, seed, packed=False):
+    print(f"case moe layer n={n} ff={ff} nexp={nexp} topk={topk} T={T} seed={seed} packed={packed}", flush=True)
     rng = np.random.default_rng(seed)
     router, gu, down, sh_gu, sh_down = make_layer(rng, n, ff, nexp)
     x = rng.standard_normal((T, n)).astype(np.float32)
     want = oracle.moe_verify_layer(n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, x)
-    layer = fnx_gpu.MoeLayerDev(dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down)
+    layer = fnx_gpu.MoeLayerDev(dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, packed=packed)
+    layer.raw = (gu, down, sh_gu, sh_down)
     got = layer.run(x)
     assert np.array_equal(got["logits"].view(np.uint32), want["logits"].view(np.uint32)), "router logits bit-exact"
     assert np.array_equal(got["topi"], want["topi"]), "routing picks bit-exact"
@@ -47,24 +48,25 @@ def check_layer(dev, oracle, n, ff, nexp, topk, T, seed):
     return got, want, layer, x
 
 
-def test_moe_verify_layer_config2(dev, oracle):
+@pytest.mark.parametrize("packed", [False, True])
+def test_moe_verify_layer_config2(dev, oracle, packed):
     # hidden 2048, 512 experts, top-10, SwiGLU experts 2048 -> 512 -> 2048, one shared expert, T = 16
-    got, want, layer, x = check_layer(dev, oracle, 2048, 512, 512, 10, 16, 900)
+    got, want, layer, x = check_layer(dev, oracle, 2048, 512, 512, 10, 16, 900, packed)
     assert rel_l2(got["out"], want["out"]) <= 2e-4
     # a second window on the same layer and workspace, fewer rows
     rng = np.random.default_rng(901)
     x2 = rng.standard_normal((5, 2048)).astype(np.float32)
     router = layer.router.cpu().numpy()
-    want2 = oracle.moe_verify_layer(2048, 512, 512, 10, router, layer.gu.cpu().numpy(), layer.down.cpu().numpy(),
-                                    layer.sh_gu.cpu().numpy(), layer.sh_down.cpu().numpy(), x2)
+    want2 = oracle.moe_verify_layer(2048, 512, 512, 10, router, *layer.raw, x2)
     got2 = layer.run(x2)
     assert np.array_equal(got2["topi"], want2["topi"]) and got2["njobs"] == want2["njobs"]
     assert rel_l2(got2["out"], want2["out"]) <= 1e-3
 
 
+@pytest.mark.parametrize("packed", [False, True])
 @pytest.mark.parametrize("n,ff,nexp,topk,T", [(2048, 512, 64, 10, 1), (1024, 256, 32, 4, 16), (2048, 1024, 16, 2, 3), (512, 512, 16, 8, 7)])
-def test_moe_verify_layer_shapes(dev, oracle, n, ff, nexp, topk, T):
-    check_layer(dev, oracle, n, ff, nexp, topk, T, 910 + T)
+def test_moe_verify_layer_shapes(dev, oracle, n, ff, nexp, topk, T, packed):
+    check_layer(dev, oracle, n, ff, nexp, topk, T, 910 + T, packed)
 
 
 def test_moe_ops_one_by_one_equal_the_fused_call(dev, oracle):
@@ -82,7 +84,7 @@ def test_moe_ops_one_by_one_equal_the_fused_call(dev, oracle):
     dev.ok(lib.fnx_quantize_q8_1(dx.data_ptr(), xq.data_ptr(), n, T, st))
     dev.ok(lib.fnx_router_route(layer.router.data_ptr(), 0, dx.data_ptr(), logits.data_ptr(), T, n, nexp, topk, topi.data_ptr(),
                                 topw.data_ptr(), jgu.data_ptr(), jdn.data_ptr(), nj.data_ptr(), st))
-    dev.ok(lib.fnx_moe_gate_up(C.byref(layer.L.gu), layer.gu_stride, jgu.data_ptr(), nj.data_ptr(), P, xq.data_ptr(), gu.data_ptr(), st))
+    dev.ok(lib.fnx_moe_gate_up(C.byref(layer.L.gu), layer.gu_stride, jgu.data_ptr(), nj.data_ptr(), P, xq.data_ptr(), gu.data_ptr(), topk, st))
     dev.ok(lib.fnx_moe_down(C.byref(layer.L.down), layer.down_stride, jdn.data_ptr(), nj.data_ptr(), P, gu.data_ptr(), part.data_ptr(), st))
     # the shared expert as the reference runs it: a dense gate|up over all rows, swiglu to q8_1, a dense down
     sh_job = np.zeros(1, dtype=fnx_gpu.JOB_DTYPE)

@@ -97,20 +97,33 @@ def test_router_route_fused_bit_exact(dev, oracle):
 
 
 # ---------------------------------------------------------------- IQ3_S x q8_1
-@pytest.mark.parametrize("nrows,ncols,T", [(4096, 2048, 1), (4096, 2048, 16), (2048, 512, 16), (1024, 2048, 3), (30, 512, 2),
-                                           (17, 256, 5), (64, 1024, 7), (12, 4096, 2), (9, 768, 3)])
-def test_gemv_iq3s(dev, oracle, nrows, ncols, T):
-    print(f"case gemv_iq3s nrows={nrows} ncols={ncols} T={T}", flush=True)
+def test_repack_unit64_bytes(dev):
+    # the device's load-time re-laying against a numpy restatement of the layout, out of place and in place
+    rng = np.random.default_rng(390)
+    raw = random_iq3s(rng, 8 * 37)
+    want = fnx_gpu.pack_unit64(raw)
+    assert np.array_equal(dev.repack(raw, in_place=False), want)
+    assert np.array_equal(dev.repack(raw, in_place=True), want)
+
+
+@pytest.mark.parametrize("packed", [False, True])
+@pytest.mark.parametrize("nrows,ncols,T", [(4096, 2048, 1), (4096, 2048, 16), (2048, 512, 16), (1024, 2048, 3), (32, 512, 2),
+                                           (16, 256, 5), (64, 1024, 7), (12, 4096, 2), (9, 768, 3), (30, 512, 2), (17, 256, 5)])
+def test_gemv_iq3s(dev, oracle, nrows, ncols, T, packed):
+    print(f"case gemv_iq3s nrows={nrows} ncols={ncols} T={T} packed={packed}", flush=True)
+    if packed and (ncols not in (256, 512, 1024, 2048) or (nrows * ncols) % 2048):
+        pytest.skip("the unit64 layout takes whole units only (the raw layout covers this shape)")
     rng = np.random.default_rng(400 + nrows + ncols + T)
     w = random_iq3s(rng, nrows * ncols // 256)
     x = rng.standard_normal((T, ncols)).astype(np.float32)
-    got = dev.gemv_iq3s(w, nrows, ncols, x)
+    got = dev.gemv_iq3s(w, nrows, ncols, x, packed=packed)
     want = oracle.gemv_iq3s(w, nrows, ncols, x)
     assert rel_l2(got, want) <= REL_L2
     assert rel_l2(got, want) <= 1e-5, "in practice only the order of a few float adds differs"
 
 
-def test_gemv_iq3s_encoded_gaussian_weights(dev, oracle):
+@pytest.mark.parametrize("packed", [False, True])
+def test_gemv_iq3s_encoded_gaussian_weights(dev, oracle, packed):
     # BASELINE config 1 in small: N(0, 0.02) weights through the encoder, N(0, 1) activations, against the q8_1 oracle
     # and within the int8 path's band of the exact f64 product
     rng = np.random.default_rng(410)
@@ -118,12 +131,13 @@ def test_gemv_iq3s_encoded_gaussian_weights(dev, oracle):
     w = oracle.iq3s_quantize((rng.standard_normal(nrows * ncols) * 0.02).astype(np.float32))
     for T in (1, 16):
         x = rng.standard_normal((T, ncols)).astype(np.float32)
-        got = dev.gemv_iq3s(w, nrows, ncols, x)
+        got = dev.gemv_iq3s(w, nrows, ncols, x, packed=packed)
         assert rel_l2(got, oracle.gemv_iq3s(w, nrows, ncols, x)) <= 1e-5
         assert rel_l2(got, oracle.gemv_exact(w, nrows, ncols, x)) < 3e-2
 
 
-def test_mmvq_jobs_pick_experts_and_rows(dev, oracle):
+@pytest.mark.parametrize("packed", [False, True])
+def test_mmvq_jobs_pick_experts_and_rows(dev, oracle, packed):
     # several experts, jobs with scattered activation and output rows, count read from device memory
     rng = np.random.default_rng(420)
     nexp, nrows, ncols, nrows_y = 6, 96, 2048, 9
@@ -139,11 +153,11 @@ def test_mmvq_jobs_pick_experts_and_rows(dev, oracle):
         jobs["y"][j, :len(ys)] = ys
         jobs["out"][j, :len(ys)] = np.arange(at, at + len(ys))
         at += len(ys)
-    got = dev.mmvq(w, stride, nrows, ncols, jobs, yq, at)
+    got = dev.mmvq(w, stride, nrows, ncols, jobs, yq, at, packed=packed)
     want = oracle.mmvq(w, stride, nrows, ncols, jobs, yq, at)
     assert rel_l2(got, want) <= 1e-5
     # with the device count null the host count is used
-    assert np.array_equal(dev.mmvq(w, stride, nrows, ncols, jobs, yq, at, njobs_dev=False), got)
+    assert np.array_equal(dev.mmvq(w, stride, nrows, ncols, jobs, yq, at, njobs_dev=False, packed=packed), got)
 
 
 # ---------------------------------------------------------------- head, drafting, acceptance
