@@ -88,29 +88,22 @@ __device__ __forceinline__ int reduce4_unit_of_row(int row) { return ((row & 1) 
 
 // SBR: sub-blocks per weight row (ncols / 32): 64, 32, 16 or 8. NT: tokens of the job kept in registers.
 // Units go four at a time; the loads of the next four are issued before the current four are decoded.
-template <int SBR, int NT>
-__device__ __forceinline__ void packed_units(const uint32_t* __restrict__ tab, const uint8_t* __restrict__ we, int ua, int ub,
-                                             const fnx_job* __restrict__ jb, int t0, const uint8_t* __restrict__ y, float* __restrict__ out,
-                                             int out_stride) {
+// prep(xs, dx, orow): fills the NT tokens' int8 activations of this lane's sub-block column (8 dwords each), their
+// scales and their output rows; it runs after the first weight loads are issued, so its own latency hides behind them.
+template <int SBR, int NT, class Prep>
+__device__ __forceinline__ void packed_units(const uint32_t* __restrict__ tab, const uint8_t* __restrict__ we, int ua, int ub, Prep prep) {
     constexpr int R = 4, RW = 64 / SBR;   // units in flight, rows per unit
     const int lane = threadIdx.x & 63, g = lane / SBR, kb = lane % SBR;
     const PackedOffs o = packed_offs(lane);
     const int sc_shift = 4 * (lane & 1), last = ub - 1;
     auto unit_at = [&](int ui) { return as_global(uniform_ptr(we + (size_t) min(ui, last) * UNIT_BYTES)); };
-    PackedSub cur[R];   // the first weights are on their way before the job's activations are fetched
+    PackedSub cur[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) cur[r] = load_packed(unit_at(ua + r), o);
     int xs[NT][8];
     float dx[NT];
     float* orow[NT];
-#pragma unroll
-    for (int t = 0; t < NT; ++t) {
-        const uint8_t* yb = y + ((size_t) uniform(jb->y[t0 + t]) * SBR + kb) * FNX_Q8_1_BLOCK;
-        dx[t] = half_bits_to_float(*reinterpret_cast<const unsigned short*>(yb));
-#pragma unroll
-        for (int j = 0; j < 8; ++j) xs[t][j] = reinterpret_cast<const int*>(yb + 4)[j];
-        orow[t] = out + (size_t) uniform(jb->out[t0 + t]) * out_stride;
-    }
+    prep(xs, dx, orow);
     for (int u = ua; u < ub; u += R) {
         PackedSub nxt[R];
 #pragma unroll
@@ -156,6 +149,27 @@ __device__ __forceinline__ void packed_units(const uint32_t* __restrict__ tab, c
     }
 }
 
+// tokens from a job list and q8_1 rows in memory (the operator entry points)
+template <int SBR, int NT>
+struct JobPrep {
+    const fnx_job* jb;
+    int t0;
+    const uint8_t* y;
+    float* out;
+    int out_stride;
+    __device__ __forceinline__ void operator()(int (&xs)[NT][8], float (&dx)[NT], float* (&orow)[NT]) const {
+        const int kb = (threadIdx.x & 63) % SBR;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            const uint8_t* yb = y + ((size_t) uniform(jb->y[t0 + t]) * SBR + kb) * FNX_Q8_1_BLOCK;
+            dx[t] = half_bits_to_float(*reinterpret_cast<const unsigned short*>(yb));
+#pragma unroll
+            for (int j = 0; j < 8; ++j) xs[t][j] = reinterpret_cast<const int*>(yb + 4)[j];
+            orow[t] = out + (size_t) uniform(jb->out[t0 + t]) * out_stride;
+        }
+    }
+};
+
 template <int SBR, bool WIDE>
 __device__ __forceinline__ void packed_range(const uint32_t* tab, const uint8_t* we, int ua, int ub, const fnx_job* jb, const uint8_t* y,
                                              float* out, int out_stride) {
@@ -163,16 +177,16 @@ __device__ __forceinline__ void packed_range(const uint32_t* tab, const uint8_t*
     for (int t0 = 0; t0 < n;) {
         const int nt = n - t0;
         if (WIDE && nt >= 4) {
-            packed_units<SBR, 4>(tab, we, ua, ub, jb, t0, y, out, out_stride);
+            packed_units<SBR, 4>(tab, we, ua, ub, JobPrep<SBR, 4>{jb, t0, y, out, out_stride});
             t0 += 4;
         } else if (WIDE && nt == 3) {
-            packed_units<SBR, 3>(tab, we, ua, ub, jb, t0, y, out, out_stride);
+            packed_units<SBR, 3>(tab, we, ua, ub, JobPrep<SBR, 3>{jb, t0, y, out, out_stride});
             t0 += 3;
         } else if (nt >= 2) {
-            packed_units<SBR, 2>(tab, we, ua, ub, jb, t0, y, out, out_stride);
+            packed_units<SBR, 2>(tab, we, ua, ub, JobPrep<SBR, 2>{jb, t0, y, out, out_stride});
             t0 += 2;
         } else {
-            packed_units<SBR, 1>(tab, we, ua, ub, jb, t0, y, out, out_stride);
+            packed_units<SBR, 1>(tab, we, ua, ub, JobPrep<SBR, 1>{jb, t0, y, out, out_stride});
             t0 += 1;
         }
     }
