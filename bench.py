@@ -35,7 +35,6 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--layers", type=int, default=16, help="distinct weight sets cycled through")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0: skip)")
-    ap.add_argument("--unfused", action="store_true", help="run the layer operator by operator instead of as one persistent kernel")
     ap.add_argument("--raw-layout", action="store_true", help="leave the weights as raw ggml blocks (skip the load-time re-laying)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -79,10 +78,8 @@ def main():
     P = T * TOPK
     ws_t = dict(xq=dev.zeros(T * (N // 32) * 36, t.uint8), logits=dev.zeros((T, NEXP + 1), t.float32), topi=dev.zeros((T, TOPK), t.int32),
                 topw=dev.zeros((T, TOPK), t.float32), jobs_gu=dev.zeros((P + 1) * 136, t.uint8), jobs_dn=dev.zeros((P + 1) * 136, t.uint8),
-                njobs=dev.zeros(2, t.int32), gu=dev.zeros((P + T, 2 * FF), t.float32), part=dev.zeros((P + T, N), t.float32),
-                sync=dev.zeros(4, t.int32))
-    ws = pkg.MoeWs(*(ws_t[k].data_ptr() for k in ("xq", "logits", "topi", "topw", "jobs_gu", "jobs_dn", "njobs", "gu", "part")),
-                   None if args.unfused else ws_t["sync"].data_ptr())
+                njobs=dev.zeros(2, t.int32), gu=dev.zeros((P + T, 2 * FF), t.float32), part=dev.zeros((P + T, N), t.float32))
+    ws = pkg.MoeWs(*(ws_t[k].data_ptr() for k in ("xq", "logits", "topi", "topw", "jobs_gu", "jobs_dn", "njobs", "gu", "part")))
     st = dev.st()
 
     def step(i):

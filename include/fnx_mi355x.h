@@ -134,7 +134,10 @@ int fnx_accept_greedy_dev(const int* rows, const int* o, int R, int* n_accept, v
 
 /* ---- the whole MoE half of a verify window (engine.cu:1569-1757 Engine::ffn_half without cards and streaming):
  * quantize -> router_route -> gate|up (routed + shared) -> swiglu q8_1 -> down (routed + shared) -> combine.
- * Same results as the calls above made one by one. */
+ * Same results as the calls above made one by one (up to the order of a few float additions). With unit64 weights,
+ * n = 2048 and ff of 256, 512 or 1024 the window runs in five launches: [router logits | q8_1 rows], [top-k, jobs],
+ * [gate|up routed + shared], [SwiGLU + down routed + shared], [combine]; other shapes run operator by operator.
+ * Like moe_down, one MoE may be in flight per device. */
 typedef struct fnx_moe_layer {
     int n, ff, nexp, topk;   /* hidden, expert width, experts, picks per token */
     const void* router;      /* [nexp + 1][n]: the router's rows, then the shared expert's gate */
@@ -157,18 +160,8 @@ typedef struct fnx_moe_ws {
     int* njobs;      /* [2], zeroed once */
     float* gu;       /* [T * topk + T][2 ff] */
     float* part;     /* [T * topk + T][n] */
-    unsigned* sync;  /* [4], zeroed once (left at zero), or null. With it, unit64 weights, n = 2048 and ff 256/512/1024 the
-                        whole layer runs as one persistent kernel whose phases meet at grid barriers; sync[2] is that
-                        kernel's error word (bit 4: a barrier timed out, as the reference's hc barrier, engine_impl.hpp:211-218).
-                        The kernel needs the device to itself for its few tens of microseconds: work of other streams delays it */
 } fnx_moe_ws;
 int fnx_moe_verify_layer(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st);
-/* Profiling aid (the reference's FNX_RR_TIMES stamps, moe.cuh:247-255, kernels.cu:2405-2444): the persistent kernel's
- * last launch on the current device as 8 ticks of the 100 MHz wall clock taken by its first block: start, logits
- * and q8_1 rows done, past the barrier, routing done, gate|up done, past the barrier, down done, past the barrier.
- * Synchronises the device. */
-int fnx_layer_stamps(unsigned long long* out8);
-
 #ifdef __cplusplus
 }
 #endif

@@ -39,7 +39,7 @@ class MoeLayer(C.Structure):
 
 class MoeWs(C.Structure):
     _fields_ = [("xq", C.c_void_p), ("logits", C.c_void_p), ("topi", C.c_void_p), ("topw", C.c_void_p), ("jobs_gu", C.c_void_p),
-                ("jobs_dn", C.c_void_p), ("njobs", C.c_void_p), ("gu", C.c_void_p), ("part", C.c_void_p), ("sync", C.c_void_p)]
+                ("jobs_dn", C.c_void_p), ("njobs", C.c_void_p), ("gu", C.c_void_p), ("part", C.c_void_p)]
 
 
 EXPORTS = {
@@ -67,7 +67,6 @@ EXPORTS = {
                                         C.c_void_p]),
     "fnx_accept_greedy": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int]),
     "fnx_accept_greedy_dev": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
-    "fnx_layer_stamps": (C.c_int, [C.c_void_p]),
     "fnx_moe_verify_layer": (C.c_int, [C.POINTER(MoeLayer), C.c_void_p, C.c_int, C.c_void_p, C.POINTER(MoeWs), C.c_void_p]),
 }
 

@@ -613,48 +613,32 @@ static int rows_launch(const fnx_dw* W, size_t w_stride, const fnx_job* jobs, co
     return launch_status(who);
 }
 
-// the persistent kernel's grid: as many blocks as are resident at once (asked of the runtime, once per device)
-template <int SBR_D>
-static int layer_grid() {
-    static int grids[64] = {};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
-    if (!grids[dev]) {
-        int per_cu = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_moe_layer<SBR_D>, FL_THREADS, 0) != hipSuccess || per_cu < 1) return 0;
-        static const int cap = env_int("FNX_LAYER_BLOCKS_PER_CU", 2, 1, 8);
-        grids[dev] = std::min(per_cu, cap) * cu_count();
-    }
-    return grids[dev];
-}
-static bool layer_fused_ok(const fnx_moe_layer* L, int T, const fnx_moe_ws* ws) {
-    static const int off = env_int("FNX_LAYER_FUSED", 1, 0, 1);
+static bool layer_fused_ok(const fnx_moe_layer* L, int T) {
+    static const int on = env_int("FNX_LAYER_FUSED", 1, 0, 1);
     const auto packed = [](const fnx_dw& w) { return w.type == FNX_T_IQ3S_UNIT64; };
-    return off && ws->sync && L->n == FL_N && (L->ff == 256 || L->ff == 512 || L->ff == 1024) && L->nexp <= 1024 && T * L->topk <= FL_MAXP &&
+    return on && L->n == FL_N && (L->ff == 256 || L->ff == 512 || L->ff == 1024) && L->nexp <= 1024 && T * L->topk <= FL_MAXP &&
            packed(L->gu) && packed(L->down) && packed(L->sh_gu) && packed(L->sh_down) && L->gu_stride % UNIT_BYTES == 0 &&
            L->down_stride % UNIT_BYTES == 0 && L->sh_gu.p && L->sh_down.p;
 }
+// the window's MoE half in five launches (k_moe_layer.h)
 static int layer_fused(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st) {
-    LayerArgs a{L->ff, L->nexp, L->topk, T, x, L->router, L->router_bf16,
-                (const uint8_t*) L->gu.p, L->gu_stride, (const uint8_t* const*) L->gu.ep,
-                (const uint8_t*) L->down.p, L->down_stride, (const uint8_t* const*) L->down.ep,
-                (const uint8_t*) L->sh_gu.p, (const uint8_t*) L->sh_down.p,
-                (uint8_t*) ws->xq, ws->logits, ws->topi, ws->topw, ws->jobs_gu, ws->jobs_dn, ws->njobs, ws->gu, ws->part, out, ws->sync};
     hipStream_t s = (hipStream_t) st;
-    int grid = 0;
-    switch (L->ff) {
-        case 256:
-            if ((grid = layer_grid<8>()) > 0) k_moe_layer<8><<<grid, FL_THREADS, 0, s>>>(a);
-            break;
-        case 512:
-            if ((grid = layer_grid<16>()) > 0) k_moe_layer<16><<<grid, FL_THREADS, 0, s>>>(a);
-            break;
-        default:
-            if ((grid = layer_grid<32>()) > 0) k_moe_layer<32><<<grid, FL_THREADS, 0, s>>>(a);
-            break;
-    }
-    if (grid <= 0) return fail("moe_verify_layer: the runtime reports no resident block for the fused kernel");
-    return launch_status("moe_verify_layer (fused)");
+    const int n = L->n, ff = L->ff, P = T * L->topk, LS = L->nexp + 1;
+    const int rblocks = (LS + RQ_ROWS - 1) / RQ_ROWS, qblocks = (T * 64 + 2 * FL_WAVES - 1) / (2 * FL_WAVES);
+    k_router_quant<<<rblocks + qblocks, FL_THREADS, 0, s>>>(RouterArgs{L->nexp, T, x, L->router, L->router_bf16, ws->logits, (uint8_t*) ws->xq});
+    k_route_plan<<<T, RT_THREADS, 0, s>>>(RouteArgs{L->nexp, L->topk, T, ws->logits, ws->topi, ws->topw, ws->jobs_gu, ws->jobs_dn, ws->njobs});
+    static const int per_cu = env_int("FNX_LAYER_BLOCKS_PER_CU", 2, 1, 8);
+    const int grid = per_cu * cu_count();
+    const PassArgs gu{2 * ff, (const uint8_t*) L->gu.p, L->gu_stride, (const uint8_t* const*) L->gu.ep, (const uint8_t*) L->sh_gu.p,
+                      (const uint8_t*) ws->xq, nullptr, ff, ws->gu};
+    k_moe_passes<64, false><<<grid, FL_THREADS, 0, s>>>(gu);
+    const PassArgs dn{n, (const uint8_t*) L->down.p, L->down_stride, (const uint8_t* const*) L->down.ep, (const uint8_t*) L->sh_down.p,
+                      nullptr, ws->gu, ff, ws->part};
+    if (ff == 256) k_moe_passes<8, true><<<grid, FL_THREADS, 0, s>>>(dn);
+    else if (ff == 512) k_moe_passes<16, true><<<grid, FL_THREADS, 0, s>>>(dn);
+    else k_moe_passes<32, true><<<grid, FL_THREADS, 0, s>>>(dn);
+    if (launch_status("moe_verify_layer")) return 1;
+    return fnx_moe_combine(ws->part, ws->topw, ws->part + (size_t) P * n, ws->logits + L->nexp, LS, out, T, n, L->topk, st);
 }
 
 }  // namespace fnx
@@ -821,13 +805,6 @@ int fnx_accept_greedy_dev(const int* rows, const int* o, int R, int* n_accept, v
     return launch_status("accept_greedy_dev");
 }
 
-int fnx_layer_stamps(unsigned long long* out8) {
-    if (!out8) return fail("layer_stamps: null argument");
-    const hipError_t e = hipMemcpyFromSymbol(out8, HIP_SYMBOL(g_layer_stamps), 8 * sizeof(unsigned long long));
-    if (e != hipSuccess) return fail(std::string("layer_stamps: ") + hipGetErrorString(e));
-    return 0;
-}
-
 int fnx_moe_verify_layer(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st) {
     if (!L || !x || !out || !ws) return fail("moe_verify_layer: null argument");
     if (!ws->xq || !ws->logits || !ws->topi || !ws->topw || !ws->jobs_gu || !ws->jobs_dn || !ws->njobs || !ws->gu || !ws->part)
@@ -838,7 +815,7 @@ int fnx_moe_verify_layer(const fnx_moe_layer* L, const float* x, int T, float* o
     if (L->gu.n_in != n || L->gu.n_out != 2 * ff || L->down.n_in != ff || L->down.n_out != n || L->sh_gu.n_in != n ||
         L->sh_gu.n_out != 2 * ff || L->sh_down.n_in != ff || L->sh_down.n_out != n)
         return fail("moe_verify_layer: weight shapes do not match n / ff");
-    if (layer_fused_ok(L, T, ws)) return layer_fused(L, x, T, out, ws, st);
+    if (layer_fused_ok(L, T)) return layer_fused(L, x, T, out, ws, st);
     hipStream_t s = (hipStream_t) st;
     if (fnx_quantize_q8_1(x, ws->xq, n, T, st)) return 1;
     if (gemv_any(L->router, L->router_bf16 != 0, x, ws->logits, L->nexp + 1, n, T, st, "moe_verify_layer router")) return 1;

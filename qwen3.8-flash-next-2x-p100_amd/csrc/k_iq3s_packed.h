@@ -90,16 +90,21 @@ __device__ __forceinline__ int reduce4_unit_of_row(int row) { return ((row & 1) 
 // Units go four at a time; the loads of the next four are issued before the current four are decoded.
 // prep(xs, dx, orow): fills the NT tokens' int8 activations of this lane's sub-block column (8 dwords each), their
 // scales and their output rows; it runs after the first weight loads are issued, so its own latency hides behind them.
+// issues the loads of units ua .. ua + 3 of an expert's matrix (past ub - 1: the last unit again)
+__device__ __forceinline__ void packed_first(const uint8_t* __restrict__ we, int ua, int ub, PackedSub (&cur)[4]) {
+    const PackedOffs o = packed_offs(threadIdx.x & 63);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) cur[r] = load_packed(as_global(uniform_ptr(we + (size_t) min(ua + r, ub - 1) * UNIT_BYTES)), o);
+}
+// cur: the first four units, loads already issued by packed_first (so the caller can put other latencies behind them)
 template <int SBR, int NT, class Prep>
-__device__ __forceinline__ void packed_units(const uint32_t* __restrict__ tab, const uint8_t* __restrict__ we, int ua, int ub, Prep prep) {
+__device__ __forceinline__ void packed_units(const uint32_t* __restrict__ tab, const uint8_t* __restrict__ we, int ua, int ub,
+                                             PackedSub (&cur)[4], Prep prep) {
     constexpr int R = 4, RW = 64 / SBR;   // units in flight, rows per unit
     const int lane = threadIdx.x & 63, g = lane / SBR, kb = lane % SBR;
     const PackedOffs o = packed_offs(lane);
     const int sc_shift = 4 * (lane & 1), last = ub - 1;
     auto unit_at = [&](int ui) { return as_global(uniform_ptr(we + (size_t) min(ui, last) * UNIT_BYTES)); };
-    PackedSub cur[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) cur[r] = load_packed(unit_at(ua + r), o);
     int xs[NT][8];
     float dx[NT];
     float* orow[NT];
@@ -174,19 +179,21 @@ template <int SBR, bool WIDE>
 __device__ __forceinline__ void packed_range(const uint32_t* tab, const uint8_t* we, int ua, int ub, const fnx_job* jb, const uint8_t* y,
                                              float* out, int out_stride) {
     const int n = uniform(jb->n);
+    PackedSub cur[4];
     for (int t0 = 0; t0 < n;) {
         const int nt = n - t0;
+        packed_first(we, ua, ub, cur);
         if (WIDE && nt >= 4) {
-            packed_units<SBR, 4>(tab, we, ua, ub, JobPrep<SBR, 4>{jb, t0, y, out, out_stride});
+            packed_units<SBR, 4>(tab, we, ua, ub, cur, JobPrep<SBR, 4>{jb, t0, y, out, out_stride});
             t0 += 4;
         } else if (WIDE && nt == 3) {
-            packed_units<SBR, 3>(tab, we, ua, ub, JobPrep<SBR, 3>{jb, t0, y, out, out_stride});
+            packed_units<SBR, 3>(tab, we, ua, ub, cur, JobPrep<SBR, 3>{jb, t0, y, out, out_stride});
             t0 += 3;
         } else if (nt >= 2) {
-            packed_units<SBR, 2>(tab, we, ua, ub, JobPrep<SBR, 2>{jb, t0, y, out, out_stride});
+            packed_units<SBR, 2>(tab, we, ua, ub, cur, JobPrep<SBR, 2>{jb, t0, y, out, out_stride});
             t0 += 2;
         } else {
-            packed_units<SBR, 1>(tab, we, ua, ub, JobPrep<SBR, 1>{jb, t0, y, out, out_stride});
+            packed_units<SBR, 1>(tab, we, ua, ub, cur, JobPrep<SBR, 1>{jb, t0, y, out, out_stride});
             t0 += 1;
         }
     }

@@ -1,12 +1,14 @@
-// The MoE half of a verify window as ONE persistent kernel (the work of Engine::ffn_half, engine.cu:1569-1757 of the
-// reference, on one GPU): router logits and q8_1 rows -> top-k and jobs -> routed + shared gate|up -> SwiGLU to q8_1
-// -> routed + shared down -> combine. The grid is sized to be resident at once (two blocks of 8 waves per CU) and its
-// phases meet at grid barriers, so the window pays one launch instead of nine and none of the ~4 us fixed cost each
-// small kernel has on this GPU.
+// The MoE half of a verify window (the work of Engine::ffn_half, engine.cu:1569-1757 of the reference, on one GPU) in
+// five launches: [router logits | q8_1 rows of x] -> [top-k, jobs, plan] -> [gate|up, routed and shared] ->
+// [SwiGLU to q8_1 on the fly + down, routed and shared] -> [combine].
 //
 // Arithmetic is the operators': the router sums in the fixed 64-lane order, top-k by (value, lower index), the q8_1
 // rounding, the IQ3_S sub-block terms, the combine's fmaf chain. Only the order in which a row's 64 (or 16) lane
 // sums are added differs from the one-operator-per-launch path.
+//
+// (A single persistent kernel with grid barriers between these phases was measured and dropped: on MI355X a barrier
+// of 512 blocks costs ~8.5 us in device-scope atomics alone and ~31 us with the release/acquire cache maintenance the
+// exchange of results between XCDs needs, against ~4 us for a kernel boundary.)
 #pragma once
 
 #include "k_iq3s_packed.h"
@@ -16,35 +18,7 @@ namespace fnx {
 constexpr int FL_THREADS = 512, FL_WAVES = FL_THREADS / 64;
 constexpr int FL_MAXP = FNX_MAXT * 10;    // routed pairs of a window (T * topk), at most
 constexpr int FL_MAXJ = FL_MAXP + 1;      // their jobs, and the shared expert's
-constexpr int FL_N = 2048;                // hidden size this kernel is built for (gate|up rows of 64 sub-blocks)
-constexpr unsigned FL_SPIN_LIMIT = 1u << 22;
-constexpr unsigned FL_ERR_BARRIER = 4u;   // error-word bit: a grid barrier timed out (engine_impl.hpp:211-218)
-
-struct LayerArgs {
-    int ff, nexp, topk, T;
-    const float* x;
-    const void* router;
-    int router_bf16;
-    const uint8_t* gu;
-    size_t gu_stride;
-    const uint8_t* const* gu_ep;
-    const uint8_t* dn;
-    size_t dn_stride;
-    const uint8_t* const* dn_ep;
-    const uint8_t* sh_gu;
-    const uint8_t* sh_dn;
-    uint8_t* xq;
-    float* logits;
-    int* topi;
-    float* topw;
-    fnx_job* jobs_gu;
-    fnx_job* jobs_dn;
-    int* njobs;
-    float* gu_out;
-    float* part;
-    float* out;
-    unsigned* sync;   // [0] barrier arrivals, [1] exits, [2] error word; all zero at launch, left at zero
-};
+constexpr int FL_N = 2048;                // hidden size these kernels are built for (gate|up rows of 64 sub-blocks)
 
 // what the routing block hands to every other block: the jobs in compact form and the list of passes.
 // A pass = (job, first token, 1 or 2 tokens) over all the job's units; the passes' units are what the waves split
@@ -60,49 +34,6 @@ struct LayerPlan {
 };
 // one MoE in flight per device (as g_moe_hq)
 __device__ LayerPlan g_layer_plan;
-
-struct LayerLds {
-    // phase 1 (router blocks): [tab | a] together hold half of the window's x (float4 [16][4][64] = 64 KiB)
-    uint32_t tab[SGRID_WORDS];
-    __attribute__((aligned(16))) uint8_t a[FNX_MAXT * 64 * FNX_Q8_1_BLOCK];   // from phase 3 on: the window's q8_1 rows
-    LayerPlan plan;
-    int ex[FL_MAXP];
-    int jobof[1024];
-    int last;
-    uint8_t isfirst[FL_MAXP];
-};
-
-// Phase stamps of the last launch, taken by block 0 (the counterpart of the reference's FNX_RR_TIMES stamps inside its
-// router launch, moe.cuh:247-255): wall_clock64() ticks at [start, logits/q8 done, routed and plan in LDS, gate|up done,
-// after barrier, down done, after barrier, end].
-__device__ unsigned long long g_layer_stamps[8];
-__device__ __forceinline__ void layer_stamp(int i) {
-    if (blockIdx.x == 0 && threadIdx.x == 0) g_layer_stamps[i] = wall_clock64();
-}
-
-// every block of the grid arrives; nobody leaves before all have. Bounded: after FL_SPIN_LIMIT polls the block goes on
-// and the error word says so (the results are then wrong, but every wave still reaches the end of the kernel).
-__device__ __forceinline__ void spin_until(unsigned* word, unsigned target, unsigned* err) {
-    unsigned spins = 0;
-    while (__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
-        __builtin_amdgcn_s_sleep(1);
-        if (++spins > FL_SPIN_LIMIT) {
-            atomicOr(err, FL_ERR_BARRIER);
-            break;
-        }
-    }
-}
-__device__ __forceinline__ void grid_sync(unsigned* sync, unsigned nblocks, unsigned& epoch) {
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        ++epoch;
-        __threadfence();
-        atomicAdd(&sync[0], 1u);
-        spin_until(&sync[0], epoch * nblocks, &sync[2]);
-        __threadfence();
-    }
-    __syncthreads();
-}
 
 // wave-wide max / min with DPP moves; every lane gets the result
 __device__ __forceinline__ float wave_max(float v) {
@@ -166,271 +97,296 @@ __device__ __forceinline__ void wave_topk(const float* __restrict__ row, int nex
     if (lane < topk) topw[lane] = wk / z;
 }
 
-// routing by one block: top-k per row of the window, the job lists the operator API returns, the plan for the grid
-__device__ __forceinline__ void route_block(const LayerArgs& a, LayerLds& L) {
+// ---------------------------------------------------------------- launch 2: top-k, jobs, plan
+// A block per row of the window: its first wave ranks the row's logits. The block that finishes last (a counter, as
+// k_router_route's last block, moe.cuh:324-330) builds the job lists and the plan from all rows' picks, without any
+// serial loop: a token picks an expert at most once, so a pair's slot in its job is the number of earlier tokens in the
+// expert's token mask, and a job's number is the rank of its first pair among the first pairs.
+struct RouteArgs {
+    int nexp, topk, T;
+    const float* logits;
+    int* topi;
+    float* topw;
+    fnx_job* jobs_gu;
+    fnx_job* jobs_dn;
+    int* njobs;   // [0] the job count, [1] the block counter (left at zero)
+};
+constexpr int RT_THREADS = 256;
+struct RouteLds {
+    LayerPlan plan;
+    int ex[FL_MAXP];
+    unsigned mask[1024];      // per expert: the window rows that picked it
+    int first[1024];          // per expert: its first pair
+    int jobof[1024];
+    int pass0[FL_MAXJ + 3];   // per job: its first pass
+    int wcnt[RT_THREADS / 64];
+    int last;
+};
+__global__ void __launch_bounds__(RT_THREADS) k_route_plan(const RouteArgs a) {
+    __shared__ RouteLds L;
     const int tid = threadIdx.x, wave = uniform(tid >> 6), lane = tid & 63;
-    const int T = a.T, P = T * a.topk, LS = a.nexp + 1;
-    LayerPlan& pl = L.plan;
-    for (int t = wave; t < T; t += FL_WAVES) {
-        if (a.nexp <= 512) wave_topk<8>(a.logits + (size_t) t * LS, a.nexp, a.topk, lane, L.ex + t * a.topk, a.topi + t * a.topk, a.topw + t * a.topk);
-        else wave_topk<16>(a.logits + (size_t) t * LS, a.nexp, a.topk, lane, L.ex + t * a.topk, a.topi + t * a.topk, a.topw + t * a.topk);
+    const int T = a.T, topk = a.topk, P = T * topk, LS = a.nexp + 1, t = blockIdx.x;
+    if (wave == 0) {
+        if (a.nexp <= 512) wave_topk<8>(a.logits + (size_t) t * LS, a.nexp, topk, lane, L.ex, a.topi + t * topk, a.topw + t * topk);
+        else wave_topk<16>(a.logits + (size_t) t * LS, a.nexp, topk, lane, L.ex, a.topi + t * topk, a.topw + t * topk);
     }
     __syncthreads();
-    // jobs: one per distinct expert, numbered by first pick, a job's pairs ascending (kernels.cu:381-398)
-    const int p = tid;
-    int slot = 0, e = -1;
-    if (p < P) {
-        e = L.ex[p];
-        for (int q = 0; q < p; ++q) slot += L.ex[q] == e;
-        L.isfirst[p] = slot == 0;
-        pl.pair_tok[p] = (uint8_t) (p / a.topk);
-    }
-    if (p < T) pl.pair_tok[P + p] = (uint8_t) p;
-    __syncthreads();
-    if (p < P && slot == 0) {
-        int j = 0, cnt = 0;
-        for (int q = 0; q < P; ++q) {
-            j += q < p && L.isfirst[q];
-            cnt += L.ex[q] == e;
+    if (tid == 0) {
+        __threadfence();
+        L.last = atomicAdd((unsigned*) &a.njobs[1], 1u) == (unsigned) T - 1;
+        if (L.last) {
+            __threadfence();
+            a.njobs[1] = 0;
         }
-        L.jobof[e] = j;
-        pl.job_w[j] = e;
-        pl.job_n[j] = (uint8_t) cnt;
-        a.jobs_gu[j].w = a.jobs_dn[j].w = e;
-        a.jobs_gu[j].n = a.jobs_dn[j].n = cnt;
     }
-    if (p == P) {
-        int nj = 0;
-        for (int q = 0; q < P; ++q) nj += L.isfirst[q];
+    __syncthreads();
+    if (!L.last) return;
+    LayerPlan& pl = L.plan;
+    for (int e = tid; e < a.nexp; e += RT_THREADS) {
+        L.mask[e] = 0u;
+        L.first[e] = P;
+    }
+    __syncthreads();
+    // every row's picks (this block's own included) from memory
+    for (int p = tid; p < P; p += RT_THREADS) {
+        const int e = __hip_atomic_load(&a.topi[p], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        L.ex[p] = e;
+        atomicOr(&L.mask[e], 1u << (p / topk));
+        atomicMin(&L.first[e], p);
+        pl.pair_tok[p] = (uint8_t) (p / topk);
+    }
+    if (tid < T) pl.pair_tok[P + tid] = (uint8_t) tid;
+    __syncthreads();
+    // job numbers: the rank of an expert's first pair among all first pairs (ballots over the pairs in order)
+    int base = 0;
+    for (int p0 = 0; p0 < P; p0 += RT_THREADS) {
+        const int p = p0 + tid;
+        const bool isfirst = p < P && L.first[L.ex[p]] == p;
+        const unsigned long long b = __ballot(isfirst);
+        if (lane == 0) L.wcnt[wave] = __popcll(b);
+        __syncthreads();
+        int before = base, total = 0;
+        for (int w = 0; w < RT_THREADS / 64; ++w) {
+            before += w < wave ? L.wcnt[w] : 0;
+            total += L.wcnt[w];
+        }
+        if (isfirst) {
+            const int e = L.ex[p], j = before + __popcll(b & ((1ull << lane) - 1ull)), cnt = __popc(L.mask[e]);
+            L.jobof[e] = j;
+            pl.job_w[j] = e;
+            pl.job_n[j] = (uint8_t) cnt;
+            a.jobs_gu[j].w = a.jobs_dn[j].w = e;
+            a.jobs_gu[j].n = a.jobs_dn[j].n = cnt;
+        }
+        base += total;
+        __syncthreads();
+    }
+    const int nj = base;
+    if (tid == 0) {
         pl.nj = nj;
         pl.job_w[nj] = -1;   // the shared expert's job: every row of the window, pairs P + t
         pl.job_n[nj] = (uint8_t) T;
         a.njobs[0] = nj;
     }
-    __syncthreads();
-    if (p < P) {
-        const int j = L.jobof[e];
+    // a pair's slot in its job: the earlier rows in its expert's mask (pairs of a job ascend with the row)
+    for (int p = tid; p < P; p += RT_THREADS) {
+        const int e = L.ex[p], j = L.jobof[e], row = p / topk, slot = __popc(L.mask[e] & ((1u << row) - 1u));
         pl.job_pairs[j][slot] = (uint8_t) p;
-        a.jobs_gu[j].y[slot] = p / a.topk;
+        a.jobs_gu[j].y[slot] = row;
         a.jobs_gu[j].out[slot] = p;
         a.jobs_dn[j].y[slot] = p;
         a.jobs_dn[j].out[slot] = p;
     }
-    if (p < T) {   // the shared expert's job, at index P of the lists the API returns (kernels.hpp:277-282)
-        pl.job_pairs[pl.nj][p] = (uint8_t) (P + p);
-        a.jobs_gu[P].y[p] = p;
-        a.jobs_gu[P].out[p] = P + p;
-        a.jobs_dn[P].y[p] = P + p;
-        a.jobs_dn[P].out[p] = P + p;
-        if (p == 0) {
+    if (tid < T) {   // the shared expert's job, at index P of the lists the API returns (kernels.hpp:277-282)
+        pl.job_pairs[nj][tid] = (uint8_t) (P + tid);
+        a.jobs_gu[P].y[tid] = tid;
+        a.jobs_gu[P].out[tid] = P + tid;
+        a.jobs_dn[P].y[tid] = P + tid;
+        a.jobs_dn[P].out[tid] = P + tid;
+        if (tid == 0) {
             a.jobs_gu[P].w = a.jobs_dn[P].w = 0;
             a.jobs_gu[P].n = a.jobs_dn[P].n = T;
         }
     }
-    // passes: job j's rows two at a time
-    if (p == 0) {
-        int np = 0;
-        for (int j = 0; j <= pl.nj; ++j)
-            for (int t0 = 0; t0 < pl.job_n[j]; t0 += 2) {
-                pl.pass_job[np] = (uint8_t) j;
-                pl.pass_t0[np] = (uint8_t) t0;
-                ++np;
-            }
-        pl.npass = np;
+    __syncthreads();
+    // passes: job j's rows two at a time; job j's first pass = the passes of the jobs before it
+    for (int j = tid; j <= nj; j += RT_THREADS) {
+        int at = 0;
+        for (int i = 0; i < j; ++i) at += (pl.job_n[i] + 1) >> 1;
+        L.pass0[j] = at;
+        if (j == nj) pl.npass = at + ((pl.job_n[j] + 1) >> 1);
     }
     __syncthreads();
-    for (int i = tid; i < (int) (sizeof(LayerPlan) / 4); i += FL_THREADS) reinterpret_cast<int*>(&g_layer_plan)[i] = reinterpret_cast<const int*>(&pl)[i];
+    for (int j = tid; j <= nj; j += RT_THREADS)
+        for (int t0 = 0, k = 0; t0 < pl.job_n[j]; t0 += 2, ++k) {
+            pl.pass_job[L.pass0[j] + k] = (uint8_t) j;
+            pl.pass_t0[L.pass0[j] + k] = (uint8_t) t0;
+        }
+    __syncthreads();
+    for (int i = tid; i < (int) (sizeof(LayerPlan) / 4); i += RT_THREADS) reinterpret_cast<int*>(&g_layer_plan)[i] = reinterpret_cast<const int*>(&pl)[i];
 }
 
-// SBR_D: sub-blocks per row of the down matrices (ff / 32): 8, 16 or 32
-template <int SBR_D>
-__global__ void __launch_bounds__(FL_THREADS, 4) k_moe_layer(const LayerArgs a) {   // 4 waves per SIMD: two blocks per CU
-    __shared__ LayerLds L;
+// ---------------------------------------------------------------- launch 1: router logits | q8_1 rows of x
+// Blocks [0, rblocks): a wave per router row with the row in registers; the window's x comes through LDS in two halves
+// of 1024 columns, the second half's loads in flight while the first is used: about one memory round trip in all.
+// Sums in the fixed order of k_gemv_rows (and of the CPU oracle): lane l takes float4 chunks l, l + 64, ... in order,
+// fmaf over x, y, z, w; then the xor-butterfly. Blocks after them: 16 q8_1 blocks of x each.
+struct RouterArgs {
+    int nexp, T;
+    const float* x;
+    const void* router;
+    int router_bf16;
+    float* logits;
+    uint8_t* xq;
+};
+constexpr int RQ_ROWS = 4;   // router rows per block: two waves per row, each with half of the window's rows
+__global__ void __launch_bounds__(FL_THREADS) k_router_quant(const RouterArgs a) {
+    __shared__ float4 xt[FNX_MAXT][4][64];   // [token][chunk][lane]: half of x
     const int tid = threadIdx.x, wave = uniform(tid >> 6), lane = tid & 63;
-    const unsigned nblocks = gridDim.x;
-    unsigned epoch = 0;
-    const int T = a.T, n = FL_N, ff = a.ff, P = T * a.topk, LS = a.nexp + 1;
-    layer_stamp(0);
-
-    // ------------------------------------------------------------ phase 1: router logits | q8_1 rows of x
-    {
-        const int rblocks = (LS + FL_WAVES - 1) / FL_WAVES, qblocks = (T * 64 + 2 * FL_WAVES - 1) / (2 * FL_WAVES);
-        for (int b = blockIdx.x; b < rblocks + qblocks; b += nblocks) {
-            if (b < rblocks) {
-                // A wave per router row with the row in registers; the window's x comes through LDS in two halves of
-                // 1024 columns, the second half's loads in flight while the first is used: about one memory round trip
-                // in all. Sums in the fixed order of k_gemv_rows (and of the CPU oracle): lane l takes float4 chunks
-                // l, l + 64, ... in order, fmaf over x, y, z, w; then the xor-butterfly.
-                float4(*xt)[4][64] = reinterpret_cast<float4(*)[4][64]>(L.tab);   // [token][chunk][lane], over tab and a
-                static_assert(sizeof(float4) * FNX_MAXT * 4 * 64 <= sizeof(L.tab) + sizeof(L.a), "half of x fits the stage");
-                const int row = b * FL_WAVES + wave;
-                const bool live = row < LS;
-                float4 w[8];
-#pragma unroll
-                for (int c = 0; c < 8; ++c) {
-                    if (!live) w[c] = make_float4(0.f, 0.f, 0.f, 0.f);
-                    else if (a.router_bf16) {
-                        const uint2 u = reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(a.router) + (size_t) row * n)[c * 64 + lane];
-                        w[c] = make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u), __uint_as_float(u.y << 16),
-                                           __uint_as_float(u.y & 0xffff0000u));
-                    } else w[c] = reinterpret_cast<const float4*>(reinterpret_cast<const float*>(a.router) + (size_t) row * n)[c * 64 + lane];
-                }
-                // thread -> 8 float4 of a half: token q / 32 ... : item i = tid + k * 512 over [token][chunk][lane]
-                auto load_half = [&](int h, float4(&xr)[8]) {
-#pragma unroll
-                    for (int k = 0; k < 8; ++k) {
-                        const int i = tid + k * FL_THREADS, t = i >> 8, c = (i >> 6) & 3, l = i & 63;
-                        xr[k] = t < T ? reinterpret_cast<const float4*>(a.x + (size_t) t * n)[(4 * h + c) * 64 + l] : make_float4(0.f, 0.f, 0.f, 0.f);
-                    }
-                };
-                float acc[FNX_MAXT];
-#pragma unroll
-                for (int t = 0; t < FNX_MAXT; ++t) acc[t] = 0.f;
-                float4 xr[8];
-                load_half(0, xr);
-                __syncthreads();   // a previous pass of this loop may still be reading the stage
-                for (int h = 0; h < 2; ++h) {
-#pragma unroll
-                    for (int k = 0; k < 8; ++k) {
-                        const int i = tid + k * FL_THREADS;
-                        xt[i >> 8][(i >> 6) & 3][i & 63] = xr[k];
-                    }
-                    __syncthreads();
-                    if (h == 0) load_half(1, xr);
-#pragma unroll
-                    for (int c = 0; c < 4; ++c)
-#pragma unroll
-                        for (int t = 0; t < FNX_MAXT; ++t)
-                            if (t < T) {
-                                const float4 bx = xt[t][c][lane];
-                                const float4 wc = w[4 * h + c];
-                                float s = acc[t];
-                                s = fmaf(wc.x, bx.x, s);
-                                s = fmaf(wc.y, bx.y, s);
-                                s = fmaf(wc.z, bx.z, s);
-                                s = fmaf(wc.w, bx.w, s);
-                                acc[t] = s;
-                            }
-                    __syncthreads();
-                }
-#pragma unroll
-                for (int t = 0; t < FNX_MAXT; ++t)
-                    if (t < T) {
-                        const float v = group_sum<64>(acc[t]);
-                        if (live && lane == 0) a.logits[(size_t) t * LS + row] = v;
-                    }
-            } else {
-                const int qb = (b - rblocks) * 2 * FL_WAVES + wave * 2 + (lane >> 5);
-                if (qb < T * 64) {
-                    const int t = qb >> 6, blk = qb & 63;
-                    const float xi = a.x[(size_t) t * n + blk * 32 + (lane & 31)];
-                    q8_1_store(xi, a.xq + (size_t) qb * FNX_Q8_1_BLOCK, lane & 31);
-                }
-            }
+    const int T = a.T, n = FL_N, LS = a.nexp + 1;
+    const int rblocks = (LS + RQ_ROWS - 1) / RQ_ROWS, b = blockIdx.x;
+    if (b >= rblocks) {
+        const int qb = (b - rblocks) * 2 * FL_WAVES + wave * 2 + (lane >> 5);
+        if (qb < T * 64) {
+            const int t = qb >> 6, blk = qb & 63;
+            const float xi = a.x[(size_t) t * n + blk * 32 + (lane & 31)];
+            q8_1_store(xi, a.xq + (size_t) qb * FNX_Q8_1_BLOCK, lane & 31);
         }
+        return;
     }
-    layer_stamp(1);
-
-    // ------------------------------------------------------------ the block that arrives last routes for everybody;
-    // the others wait for its word, having filled their codebook meanwhile
-    __syncthreads();
-    if (tid == 0) {
-        __threadfence();
-        L.last = atomicAdd(&a.sync[0], 1u) == nblocks - 1;
-        if (L.last) __threadfence();
-        ++epoch;
+    const int row = b * RQ_ROWS + (wave >> 1), tb = (wave & 1) * (FNX_MAXT / 2);   // this wave: tokens tb .. tb + 7
+    const bool live = row < LS;
+    float4 w[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        if (!live) w[c] = make_float4(0.f, 0.f, 0.f, 0.f);
+        else if (a.router_bf16) {
+            const uint2 u = reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(a.router) + (size_t) row * n)[c * 64 + lane];
+            w[c] = make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u), __uint_as_float(u.y << 16),
+                               __uint_as_float(u.y & 0xffff0000u));
+        } else w[c] = reinterpret_cast<const float4*>(reinterpret_cast<const float*>(a.router) + (size_t) row * n)[c * 64 + lane];
     }
-    for (int i = tid; i < SGRID_WORDS; i += FL_THREADS) L.tab[i] = g_sgrid.v[i];
-    __syncthreads();
-    if (L.last) {
-        route_block(a, L);
-        __syncthreads();
-        if (tid == 0) {
-            __threadfence();
-            __hip_atomic_store(&a.sync[3], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    auto load_half = [&](int h, float4(&xr)[8]) {   // item i = tid + 512 k of [token][chunk][lane]
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const int i = tid + k * FL_THREADS, t = i >> 8, c = (i >> 6) & 3, l = i & 63;
+            xr[k] = t < T ? reinterpret_cast<const float4*>(a.x + (size_t) t * n)[(4 * h + c) * 64 + l] : make_float4(0.f, 0.f, 0.f, 0.f);
         }
-    } else {
-        if (tid == 0) {
-            spin_until(&a.sync[3], 1u, &a.sync[2]);
-            __threadfence();
+    };
+    float acc[FNX_MAXT / 2];
+#pragma unroll
+    for (int t = 0; t < FNX_MAXT / 2; ++t) acc[t] = 0.f;
+    float4 xr[8];
+    load_half(0, xr);
+    for (int h = 0; h < 2; ++h) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const int i = tid + k * FL_THREADS;
+            xt[i >> 8][(i >> 6) & 3][i & 63] = xr[k];
         }
         __syncthreads();
-        for (int i = tid; i < (int) (sizeof(LayerPlan) / 4); i += FL_THREADS) reinterpret_cast<int*>(&L.plan)[i] = reinterpret_cast<const int*>(&g_layer_plan)[i];
+        if (h == 0) load_half(1, xr);
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+#pragma unroll
+            for (int t = 0; t < FNX_MAXT / 2; ++t)
+                if (tb + t < T) {
+                    const float4 bx = xt[tb + t][c][lane];
+                    const float4 wc = w[4 * h + c];
+                    float s = acc[t];
+                    s = fmaf(wc.x, bx.x, s);
+                    s = fmaf(wc.y, bx.y, s);
+                    s = fmaf(wc.z, bx.z, s);
+                    s = fmaf(wc.w, bx.w, s);
+                    acc[t] = s;
+                }
+        __syncthreads();
     }
-    for (int i = tid; i < T * 64 * FNX_Q8_1_BLOCK / 4; i += FL_THREADS) reinterpret_cast<int*>(L.a)[i] = reinterpret_cast<const int*>(a.xq)[i];
-    __syncthreads();
-    layer_stamp(2);
-    const LayerPlan& pl = L.plan;
-    const int npass = pl.npass;
-    const long gw = (long) blockIdx.x * FL_WAVES + wave, nw = (long) nblocks * FL_WAVES;
+#pragma unroll
+    for (int t = 0; t < FNX_MAXT / 2; ++t)
+        if (tb + t < T) {
+            const float v = group_sum<64>(acc[t]);
+            if (live && lane == 0) a.logits[(size_t) (tb + t) * LS + row] = v;
+        }
+}
 
-    // ------------------------------------------------------------ phase 3: gate|up, routed and shared
-    {
-        const int upj = 2 * ff;   // a unit is a row of 2048 columns
-        const long total = (long) npass * upj;
-        long u = total * gw / nw;
-        const long u1 = total * (gw + 1) / nw;
-        while (u < u1) {
-            const int pi = (int) (u / upj), ul = (int) (u % upj);
-            const int ue = (int) min((long) upj, ul + (u1 - u));
-            const int ji = uniform((int) pl.pass_job[pi]), t0 = uniform((int) pl.pass_t0[pi]);
-            const int w = uniform(pl.job_w[ji]), nt = uniform((int) pl.job_n[ji]) - t0;
-            const uint8_t* we = w < 0 ? a.sh_gu : a.gu_ep ? uniform_ptr(a.gu_ep[w]) : a.gu + (size_t) w * a.gu_stride;
-            const uint8_t* pairs = pl.job_pairs[ji] + t0;
+// ---------------------------------------------------------------- launches 3 and 4: the passes of the plan
+// DOWN = false: gate|up (rows of 2048 columns; activations: the window's q8_1 rows).
+// DOWN = true: down (rows of 32 SBR columns). A wave makes the q8_1 form of h = silu(gate) * up for its pass's pairs
+// itself (k_moe_down without PRE, moe.cuh:630-641): the 64 / SBR lanes that share a sub-block column split its 32 values.
+struct PassArgs {
+    int rows;                 // rows of every matrix
+    const uint8_t* w;         // routed experts: expert e at w + e * stride, or ep[e]
+    size_t stride;
+    const uint8_t* const* ep;
+    const uint8_t* w_shared;
+    const uint8_t* xq;        // gate|up: the window's q8_1 rows
+    const float* gu;          // down: the gate|up outputs [pair][2 ff]
+    int ff;
+    float* out;               // [pair][rows]
+};
+template <int SBR, bool DOWN>
+__global__ void __launch_bounds__(FL_THREADS) k_moe_passes(const PassArgs a) {
+    __shared__ uint32_t tab[SGRID_WORDS];
+    __shared__ LayerPlan pl;
+    const int tid = threadIdx.x, wave = uniform(tid >> 6), lane = tid & 63;
+    for (int i = tid; i < (int) (sizeof(LayerPlan) / 4); i += FL_THREADS) reinterpret_cast<int*>(&pl)[i] = reinterpret_cast<const int*>(&g_layer_plan)[i];
+    __syncthreads();
+    constexpr int RW = 64 / SBR;
+    const int upj = a.rows / RW;
+    const long total = (long) pl.npass * upj;
+    const long gw = (long) blockIdx.x * FL_WAVES + wave, nw = (long) gridDim.x * FL_WAVES;
+    long u = total * gw / nw;
+    const long u1 = total * (gw + 1) / nw;
+    struct Seg {
+        int ul, ue, ji, t0, nt;
+        const uint8_t* we;
+    };
+    auto seg_at = [&](long uu) {
+        Seg s;
+        const int pi = (int) (uu / upj);
+        s.ul = (int) (uu % upj);
+        s.ue = (int) min((long) upj, s.ul + (u1 - uu));
+        s.ji = uniform((int) pl.pass_job[pi]);
+        s.t0 = uniform((int) pl.pass_t0[pi]);
+        const int w = uniform(pl.job_w[s.ji]);
+        s.nt = uniform((int) pl.job_n[s.ji]) - s.t0;
+        s.we = w < 0 ? a.w_shared : a.ep ? uniform_ptr(a.ep[w]) : a.w + (size_t) w * a.stride;
+        return s;
+    };
+    // the first weights are on their way while the codebook is copied into LDS
+    PackedSub cur[4];
+    Seg s{};
+    if (u < u1) {
+        s = seg_at(u);
+        packed_first(s.we, s.ul, s.ue, cur);
+    }
+    for (int i = tid; i < SGRID_WORDS; i += FL_THREADS) tab[i] = g_sgrid.v[i];
+    __syncthreads();
+    const int g = lane / SBR, kb = lane % SBR;
+    while (u < u1) {
+        const uint8_t* pairs = pl.job_pairs[s.ji] + s.t0;
+        auto prep_for = [&](auto nt_tag) {
+            constexpr int NT = decltype(nt_tag)::value;
             const uint8_t* pair_tok = pl.pair_tok;
-            const uint8_t* xq = L.a;
-            auto prep_for = [&](auto nt_tag) {
-                constexpr int NT = decltype(nt_tag)::value;
-                return [=](int(&xs)[NT][8], float(&dx)[NT], float*(&orow)[NT]) {
+            return [=](int(&xs)[NT][8], float(&dx)[NT], float*(&orow)[NT]) {
 #pragma unroll
-                    for (int t = 0; t < NT; ++t) {
-                        const int pair = uniform((int) pairs[t]), tok = uniform((int) pair_tok[pair]);
-                        const uint8_t* yb = xq + (tok * 64 + lane) * FNX_Q8_1_BLOCK;
+                for (int t = 0; t < NT; ++t) {
+                    const int pair = uniform((int) pairs[t]);
+                    if constexpr (!DOWN) {
+                        const int tok = uniform((int) pair_tok[pair]);
+                        const uint8_t* yb = a.xq + ((size_t) tok * SBR + kb) * FNX_Q8_1_BLOCK;
                         dx[t] = half_bits_to_float(*reinterpret_cast<const unsigned short*>(yb));
 #pragma unroll
                         for (int j = 0; j < 8; ++j) xs[t][j] = reinterpret_cast<const int*>(yb + 4)[j];
-                        orow[t] = a.gu_out + (size_t) pair * 2 * ff;
-                    }
-                };
-            };
-            if (nt >= 2) packed_units<64, 2>(L.tab, we, ul, ue, prep_for(std::integral_constant<int, 2>{}));
-            else packed_units<64, 1>(L.tab, we, ul, ue, prep_for(std::integral_constant<int, 1>{}));
-            u += ue - ul;
-        }
-    }
-    layer_stamp(3);
-    grid_sync(a.sync, nblocks, epoch);
-    layer_stamp(4);
-
-    // ------------------------------------------------------------ phase 5: down, routed and shared. A wave makes the
-    // q8_1 form of h = silu(gate) * up for its pass's pairs itself (k_moe_down without PRE, moe.cuh:630-641): the
-    // 64 / SBR_D lanes that share a sub-block column split its 32 values.
-    {
-        constexpr int RW = 64 / SBR_D, VPL = 32 / RW;   // rows per unit; h values a lane makes
-        const int upj = n / RW;
-        const long total = (long) npass * upj;
-        long u = total * gw / nw;
-        const long u1 = total * (gw + 1) / nw;
-        const int g = lane / SBR_D, kb = lane % SBR_D;
-        while (u < u1) {
-            const int pi = (int) (u / upj), ul = (int) (u % upj);
-            const int ue = (int) min((long) upj, ul + (u1 - u));
-            const int ji = uniform((int) pl.pass_job[pi]), t0 = uniform((int) pl.pass_t0[pi]);
-            const int w = uniform(pl.job_w[ji]), nt = uniform((int) pl.job_n[ji]) - t0;
-            const uint8_t* we = w < 0 ? a.sh_dn : a.dn_ep ? uniform_ptr(a.dn_ep[w]) : a.dn + (size_t) w * a.dn_stride;
-            const uint8_t* pairs = pl.job_pairs[ji] + t0;
-            auto prep_for = [&](auto nt_tag) {
-                constexpr int NT = decltype(nt_tag)::value;
-                return [=](int(&xs)[NT][8], float(&dx)[NT], float*(&orow)[NT]) {
-#pragma unroll
-                    for (int t = 0; t < NT; ++t) {
-                        const int pair = uniform((int) pairs[t]);
-                        const float* gp = a.gu_out + (size_t) pair * 2 * ff + kb * 32 + g * VPL;
+                    } else {
+                        constexpr int VPL = 32 / RW;   // h values a lane makes
+                        const float* gp = a.gu + (size_t) pair * 2 * a.ff + kb * 32 + g * VPL;
                         float h[VPL];
                         float amax = 0.f;
 #pragma unroll
                         for (int j = 0; j < VPL; j += 4) {
-                            const float4 gv = *reinterpret_cast<const float4*>(gp + j), uv = *reinterpret_cast<const float4*>(gp + ff + j);
+                            const float4 gv = *reinterpret_cast<const float4*>(gp + j), uv = *reinterpret_cast<const float4*>(gp + a.ff + j);
                             h[j] = silu_f(gv.x) * uv.x;
                             h[j + 1] = silu_f(gv.y) * uv.y;
                             h[j + 2] = silu_f(gv.z) * uv.z;
@@ -439,7 +395,7 @@ __global__ void __launch_bounds__(FL_THREADS, 4) k_moe_layer(const LayerArgs a) 
 #pragma unroll
                         for (int j = 0; j < VPL; ++j) amax = fmaxf(amax, fabsf(h[j]));
 #pragma unroll
-                        for (int o = SBR_D; o < 64; o <<= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+                        for (int o = SBR; o < 64; o <<= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
                         const float d = amax / 127.0f;
                         int pk[VPL / 4];
 #pragma unroll
@@ -455,38 +411,19 @@ __global__ void __launch_bounds__(FL_THREADS, 4) k_moe_layer(const LayerArgs a) 
 #pragma unroll
                         for (int gg = 0; gg < RW; ++gg)
 #pragma unroll
-                            for (int k = 0; k < VPL / 4; ++k) xs[t][gg * (VPL / 4) + k] = __shfl(pk[k], kb + SBR_D * gg, 64);
+                            for (int k = 0; k < VPL / 4; ++k) xs[t][gg * (VPL / 4) + k] = __shfl(pk[k], kb + SBR * gg, 64);
                         dx[t] = half_bits_to_float(float_to_half_bits(d));
-                        orow[t] = a.part + (size_t) pair * n;
                     }
-                };
+                    orow[t] = a.out + (size_t) pair * a.rows;
+                }
             };
-            if (nt >= 2) packed_units<SBR_D, 2>(L.tab, we, ul, ue, prep_for(std::integral_constant<int, 2>{}));
-            else packed_units<SBR_D, 1>(L.tab, we, ul, ue, prep_for(std::integral_constant<int, 1>{}));
-            u += ue - ul;
-        }
-    }
-    layer_stamp(5);
-    grid_sync(a.sync, nblocks, epoch);
-    layer_stamp(6);
-
-    // ------------------------------------------------------------ phase 6: combine (kernels.cu:412-419)
-    for (long i = (long) blockIdx.x * FL_THREADS + tid; i < (long) T * n; i += (long) nblocks * FL_THREADS) {
-        const int t = (int) (i / n), c = (int) (i % n);
-        float s = 0.f;
-        for (int k = 0; k < a.topk; ++k) s = fmaf(a.topw[t * a.topk + k], a.part[((size_t) t * a.topk + k) * n + c], s);
-        a.out[i] = s + sigmoid_f(a.logits[(size_t) t * LS + a.nexp]) * a.part[((size_t) P + t) * n + c];
-    }
-    layer_stamp(7);
-
-    // the last block out leaves the barrier words at zero for the next launch
-    __syncthreads();
-    if (tid == 0) {
-        if (atomicAdd(&a.sync[1], 1u) == nblocks - 1) {
-            a.sync[0] = 0u;
-            a.sync[1] = 0u;
-            a.sync[3] = 0u;
-            __threadfence();
+        };
+        if (s.nt >= 2) packed_units<SBR, 2>(tab, s.we, s.ul, s.ue, cur, prep_for(std::integral_constant<int, 2>{}));
+        else packed_units<SBR, 1>(tab, s.we, s.ul, s.ue, cur, prep_for(std::integral_constant<int, 1>{}));
+        u += s.ue - s.ul;
+        if (u < u1) {
+            s = seg_at(u);
+            packed_first(s.we, s.ul, s.ue, cur);
         }
     }
 }

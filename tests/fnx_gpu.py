@@ -203,7 +203,7 @@ class Dev:
 class MoeLayerDev:
     """One MoE layer's weights on the device plus a workspace, for fnx_moe_verify_layer and the per-op calls."""
 
-    def __init__(self, dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, T=16, packed=False, fused=True):
+    def __init__(self, dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, T=16, packed=False):
         t = dev.torch
         self.dev, self.n, self.ff, self.nexp, self.topk = dev, n, ff, nexp, topk
         pkg = dev.pkg
@@ -228,10 +228,8 @@ class MoeLayerDev:
         self.njobs = dev.zeros(2, t.int32)
         self.gu_out = dev.zeros((P + T, 2 * ff), t.float32)
         self.part = dev.zeros((P + T, n), t.float32)
-        self.sync = dev.zeros(4, t.int32)   # the persistent kernel's barrier words; without them the layer runs operator by operator
         self.ws = pkg.MoeWs(self.xq.data_ptr(), self.logits.data_ptr(), self.topi.data_ptr(), self.topw.data_ptr(), self.jobs_gu.data_ptr(),
-                            self.jobs_dn.data_ptr(), self.njobs.data_ptr(), self.gu_out.data_ptr(), self.part.data_ptr(),
-                            self.sync.data_ptr() if fused else None)
+                            self.jobs_dn.data_ptr(), self.njobs.data_ptr(), self.gu_out.data_ptr(), self.part.data_ptr())
 
     def run(self, x):
         dev = self.dev
@@ -240,7 +238,6 @@ class MoeLayerDev:
         out = dev.zeros((T, self.n), dev.torch.float32)
         dev.ok(dev.lib.fnx_moe_verify_layer(C.byref(self.L), dx.data_ptr(), T, out.data_ptr(), C.byref(self.ws), dev.st()))
         dev.sync()
-        assert self.sync.cpu().numpy().tolist() == [0, 0, 0, 0], "barrier words left at zero, no barrier timed out"
         return dict(out=out.cpu().numpy(), logits=self.logits.cpu().numpy()[:T], topi=self.topi.cpu().numpy()[:T],
                     topw=self.topw.cpu().numpy()[:T], njobs=int(self.njobs.cpu().numpy()[0]),
                     gu=self.gu_out.cpu().numpy(), part=self.part.cpu().numpy(),
