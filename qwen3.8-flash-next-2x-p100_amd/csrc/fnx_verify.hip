@@ -631,12 +631,12 @@ static int layer_fused(const fnx_moe_layer* L, const float* x, int T, float* out
     const int grid = per_cu * cu_count();
     const PassArgs gu{2 * ff, (const uint8_t*) L->gu.p, L->gu_stride, (const uint8_t* const*) L->gu.ep, (const uint8_t*) L->sh_gu.p,
                       (const uint8_t*) ws->xq, nullptr, ff, ws->gu};
-    k_moe_passes<64, false><<<grid, FL_THREADS, 0, s>>>(gu);
+    k_moe_gate_up_passes<<<grid, FL_THREADS, 0, s>>>(gu);
     const PassArgs dn{n, (const uint8_t*) L->down.p, L->down_stride, (const uint8_t* const*) L->down.ep, (const uint8_t*) L->sh_down.p,
                       nullptr, ws->gu, ff, ws->part};
-    if (ff == 256) k_moe_passes<8, true><<<grid, FL_THREADS, 0, s>>>(dn);
-    else if (ff == 512) k_moe_passes<16, true><<<grid, FL_THREADS, 0, s>>>(dn);
-    else k_moe_passes<32, true><<<grid, FL_THREADS, 0, s>>>(dn);
+    if (ff == 256) k_moe_down_passes<8><<<grid, FL_THREADS, 0, s>>>(dn);
+    else if (ff == 512) k_moe_down_passes<16><<<grid, FL_THREADS, 0, s>>>(dn);
+    else k_moe_down_passes<32><<<grid, FL_THREADS, 0, s>>>(dn);
     if (launch_status("moe_verify_layer")) return 1;
     return fnx_moe_combine(ws->part, ws->topw, ws->part + (size_t) P * n, ws->logits + L->nexp, LS, out, T, n, L->topk, st);
 }

@@ -311,9 +311,6 @@ __global__ void __launch_bounds__(FL_THREADS) k_router_quant(const RouterArgs a)
 }
 
 // ---------------------------------------------------------------- launches 3 and 4: the passes of the plan
-// DOWN = false: gate|up (rows of 2048 columns; activations: the window's q8_1 rows).
-// DOWN = true: down (rows of 32 SBR columns). A wave makes the q8_1 form of h = silu(gate) * up for its pass's pairs
-// itself (k_moe_down without PRE, moe.cuh:630-641): the 64 / SBR lanes that share a sub-block column split its 32 values.
 struct PassArgs {
     int rows;                 // rows of every matrix
     const uint8_t* w;         // routed experts: expert e at w + e * stride, or ep[e]
@@ -325,45 +322,51 @@ struct PassArgs {
     int ff;
     float* out;               // [pair][rows]
 };
-template <int SBR, bool DOWN>
-__global__ void __launch_bounds__(FL_THREADS) k_moe_passes(const PassArgs a) {
+struct PassSeg {   // a stretch of one pass's units
+    int ul, ue, ji, t0, nt;
+    const uint8_t* we;
+};
+__device__ __forceinline__ PassSeg pass_seg(const LayerPlan& pl, const PassArgs& a, long uu, long u1, int upj) {
+    PassSeg s;
+    const int pi = (int) (uu / upj);
+    s.ul = (int) (uu % upj);
+    s.ue = (int) min((long) upj, s.ul + (u1 - uu));
+    s.ji = uniform((int) pl.pass_job[pi]);
+    s.t0 = uniform((int) pl.pass_t0[pi]);
+    const int w = uniform(pl.job_w[s.ji]);
+    s.nt = uniform((int) pl.job_n[s.ji]) - s.t0;
+    s.we = w < 0 ? a.w_shared : a.ep ? uniform_ptr(a.ep[w]) : a.w + (size_t) w * a.stride;
+    return s;
+}
+
+// gate|up: rows of 2048 columns; activations: the window's q8_1 rows. The waves of the grid split the passes' units
+// evenly and walk them in order.
+__global__ void __launch_bounds__(FL_THREADS) k_moe_gate_up_passes(const PassArgs a) {
+    constexpr int SBR = 64;
     __shared__ uint32_t tab[SGRID_WORDS];
     __shared__ LayerPlan pl;
     const int tid = threadIdx.x, wave = uniform(tid >> 6), lane = tid & 63;
+    // the codebook's loads go out first and land in registers; they are stored to LDS once the first weights have been
+    // asked for, so that the latencies overlap
+    uint32_t treg[SGRID_WORDS / FL_THREADS];
+#pragma unroll
+    for (int i = 0; i < SGRID_WORDS / FL_THREADS; ++i) treg[i] = g_sgrid.v[tid + i * FL_THREADS];
     for (int i = tid; i < (int) (sizeof(LayerPlan) / 4); i += FL_THREADS) reinterpret_cast<int*>(&pl)[i] = reinterpret_cast<const int*>(&g_layer_plan)[i];
     __syncthreads();
-    constexpr int RW = 64 / SBR;
-    const int upj = a.rows / RW;
+    const int upj = a.rows;
     const long total = (long) pl.npass * upj;
     const long gw = (long) blockIdx.x * FL_WAVES + wave, nw = (long) gridDim.x * FL_WAVES;
     long u = total * gw / nw;
     const long u1 = total * (gw + 1) / nw;
-    struct Seg {
-        int ul, ue, ji, t0, nt;
-        const uint8_t* we;
-    };
-    auto seg_at = [&](long uu) {
-        Seg s;
-        const int pi = (int) (uu / upj);
-        s.ul = (int) (uu % upj);
-        s.ue = (int) min((long) upj, s.ul + (u1 - uu));
-        s.ji = uniform((int) pl.pass_job[pi]);
-        s.t0 = uniform((int) pl.pass_t0[pi]);
-        const int w = uniform(pl.job_w[s.ji]);
-        s.nt = uniform((int) pl.job_n[s.ji]) - s.t0;
-        s.we = w < 0 ? a.w_shared : a.ep ? uniform_ptr(a.ep[w]) : a.w + (size_t) w * a.stride;
-        return s;
-    };
-    // the first weights are on their way while the codebook is copied into LDS
     PackedSub cur[4];
-    Seg s{};
+    PassSeg s{};
     if (u < u1) {
-        s = seg_at(u);
+        s = pass_seg(pl, a, u, u1, upj);
         packed_first(s.we, s.ul, s.ue, cur);
     }
-    for (int i = tid; i < SGRID_WORDS; i += FL_THREADS) tab[i] = g_sgrid.v[i];
+#pragma unroll
+    for (int i = 0; i < SGRID_WORDS / FL_THREADS; ++i) tab[tid + i * FL_THREADS] = treg[i];
     __syncthreads();
-    const int g = lane / SBR, kb = lane % SBR;
     while (u < u1) {
         const uint8_t* pairs = pl.job_pairs[s.ji] + s.t0;
         auto prep_for = [&](auto nt_tag) {
@@ -372,48 +375,11 @@ __global__ void __launch_bounds__(FL_THREADS) k_moe_passes(const PassArgs a) {
             return [=](int(&xs)[NT][8], float(&dx)[NT], float*(&orow)[NT]) {
 #pragma unroll
                 for (int t = 0; t < NT; ++t) {
-                    const int pair = uniform((int) pairs[t]);
-                    if constexpr (!DOWN) {
-                        const int tok = uniform((int) pair_tok[pair]);
-                        const uint8_t* yb = a.xq + ((size_t) tok * SBR + kb) * FNX_Q8_1_BLOCK;
-                        dx[t] = half_bits_to_float(*reinterpret_cast<const unsigned short*>(yb));
+                    const int pair = uniform((int) pairs[t]), tok = uniform((int) pair_tok[pair]);
+                    const uint8_t* yb = a.xq + ((size_t) tok * SBR + lane) * FNX_Q8_1_BLOCK;
+                    dx[t] = half_bits_to_float(*reinterpret_cast<const unsigned short*>(yb));
 #pragma unroll
-                        for (int j = 0; j < 8; ++j) xs[t][j] = reinterpret_cast<const int*>(yb + 4)[j];
-                    } else {
-                        constexpr int VPL = 32 / RW;   // h values a lane makes
-                        const float* gp = a.gu + (size_t) pair * 2 * a.ff + kb * 32 + g * VPL;
-                        float h[VPL];
-                        float amax = 0.f;
-#pragma unroll
-                        for (int j = 0; j < VPL; j += 4) {
-                            const float4 gv = *reinterpret_cast<const float4*>(gp + j), uv = *reinterpret_cast<const float4*>(gp + a.ff + j);
-                            h[j] = silu_f(gv.x) * uv.x;
-                            h[j + 1] = silu_f(gv.y) * uv.y;
-                            h[j + 2] = silu_f(gv.z) * uv.z;
-                            h[j + 3] = silu_f(gv.w) * uv.w;
-                        }
-#pragma unroll
-                        for (int j = 0; j < VPL; ++j) amax = fmaxf(amax, fabsf(h[j]));
-#pragma unroll
-                        for (int o = SBR; o < 64; o <<= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
-                        const float d = amax / 127.0f;
-                        int pk[VPL / 4];
-#pragma unroll
-                        for (int j = 0; j < VPL; j += 4) {
-                            uint32_t v = 0;
-#pragma unroll
-                            for (int k = 0; k < 4; ++k) {
-                                const int q = amax == 0.0f ? 0 : (int) (int8_t) roundf(h[j + k] / d);
-                                v |= ((uint32_t) q & 0xFFu) << (8 * k);
-                            }
-                            pk[j / 4] = (int) v;
-                        }
-#pragma unroll
-                        for (int gg = 0; gg < RW; ++gg)
-#pragma unroll
-                            for (int k = 0; k < VPL / 4; ++k) xs[t][gg * (VPL / 4) + k] = __shfl(pk[k], kb + SBR * gg, 64);
-                        dx[t] = half_bits_to_float(float_to_half_bits(d));
-                    }
+                    for (int j = 0; j < 8; ++j) xs[t][j] = reinterpret_cast<const int*>(yb + 4)[j];
                     orow[t] = a.out + (size_t) pair * a.rows;
                 }
             };
@@ -422,7 +388,91 @@ __global__ void __launch_bounds__(FL_THREADS) k_moe_passes(const PassArgs a) {
         else packed_units<SBR, 1>(tab, s.we, s.ul, s.ue, cur, prep_for(std::integral_constant<int, 1>{}));
         u += s.ue - s.ul;
         if (u < u1) {
-            s = seg_at(u);
+            s = pass_seg(pl, a, u, u1, upj);
+            packed_first(s.we, s.ul, s.ue, cur);
+        }
+    }
+}
+
+// down: rows of 32 SBR columns, split over the waves like gate|up. A wave makes the q8_1 form of h = silu(gate) * up
+// for its pass's pairs itself (k_moe_down without PRE, moe.cuh:630-641): the 64 / SBR lanes that share a sub-block
+// column split its 32 values. (Making h once per block in LDS for the block's 8 waves was measured slower: 30 us
+// against 25 us, the block-wide barriers cost more than the repeated SwiGLU.)
+template <int SBR>
+__global__ void __launch_bounds__(FL_THREADS) k_moe_down_passes(const PassArgs a) {
+    constexpr int RW = 64 / SBR, VPL = 32 / RW;   // rows per unit; h values a lane makes
+    __shared__ uint32_t tab[SGRID_WORDS];
+    __shared__ LayerPlan pl;
+    const int tid = threadIdx.x, wave = uniform(tid >> 6), lane = tid & 63;
+    uint32_t treg[SGRID_WORDS / FL_THREADS];
+#pragma unroll
+    for (int i = 0; i < SGRID_WORDS / FL_THREADS; ++i) treg[i] = g_sgrid.v[tid + i * FL_THREADS];
+    for (int i = tid; i < (int) (sizeof(LayerPlan) / 4); i += FL_THREADS) reinterpret_cast<int*>(&pl)[i] = reinterpret_cast<const int*>(&g_layer_plan)[i];
+    __syncthreads();
+    const int upj = a.rows / RW, ff = a.ff;
+    const long total = (long) pl.npass * upj;
+    const long gw = (long) blockIdx.x * FL_WAVES + wave, nw = (long) gridDim.x * FL_WAVES;
+    long u = total * gw / nw;
+    const long u1 = total * (gw + 1) / nw;
+    PackedSub cur[4];
+    PassSeg s{};
+    if (u < u1) {
+        s = pass_seg(pl, a, u, u1, upj);
+        packed_first(s.we, s.ul, s.ue, cur);
+    }
+#pragma unroll
+    for (int i = 0; i < SGRID_WORDS / FL_THREADS; ++i) tab[tid + i * FL_THREADS] = treg[i];
+    __syncthreads();
+    const int g = lane / SBR, kb = lane % SBR;
+    while (u < u1) {
+        const uint8_t* pairs = pl.job_pairs[s.ji] + s.t0;
+        auto prep_for = [&](auto nt_tag) {
+            constexpr int NT = decltype(nt_tag)::value;
+            return [=](int(&xs)[NT][8], float(&dx)[NT], float*(&orow)[NT]) {
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    const int pair = uniform((int) pairs[t]);
+                    const float* gp = a.gu + (size_t) pair * 2 * ff + kb * 32 + g * VPL;
+                    float h[VPL];
+                    float amax = 0.f;
+#pragma unroll
+                    for (int j = 0; j < VPL; j += 4) {
+                        const float4 gv = *reinterpret_cast<const float4*>(gp + j), uv = *reinterpret_cast<const float4*>(gp + ff + j);
+                        h[j] = silu_f(gv.x) * uv.x;
+                        h[j + 1] = silu_f(gv.y) * uv.y;
+                        h[j + 2] = silu_f(gv.z) * uv.z;
+                        h[j + 3] = silu_f(gv.w) * uv.w;
+                    }
+#pragma unroll
+                    for (int j = 0; j < VPL; ++j) amax = fmaxf(amax, fabsf(h[j]));
+#pragma unroll
+                    for (int o = SBR; o < 64; o <<= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+                    const float d = amax / 127.0f;
+                    int pk[VPL / 4];
+#pragma unroll
+                    for (int j = 0; j < VPL; j += 4) {
+                        uint32_t v = 0;
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) {
+                            const int q = amax == 0.0f ? 0 : (int) (int8_t) roundf(h[j + k] / d);
+                            v |= ((uint32_t) q & 0xFFu) << (8 * k);
+                        }
+                        pk[j / 4] = (int) v;
+                    }
+#pragma unroll
+                    for (int gg = 0; gg < RW; ++gg)
+#pragma unroll
+                        for (int k = 0; k < VPL / 4; ++k) xs[t][gg * (VPL / 4) + k] = __shfl(pk[k], kb + SBR * gg, 64);
+                    dx[t] = half_bits_to_float(float_to_half_bits(d));
+                    orow[t] = a.out + (size_t) pair * a.rows;
+                }
+            };
+        };
+        if (s.nt >= 2) packed_units<SBR, 2>(tab, s.we, s.ul, s.ue, cur, prep_for(std::integral_constant<int, 2>{}));
+        else packed_units<SBR, 1>(tab, s.we, s.ul, s.ue, cur, prep_for(std::integral_constant<int, 1>{}));
+        u += s.ue - s.ul;
+        if (u < u1) {
+            s = pass_seg(pl, a, u, u1, upj);
             packed_first(s.we, s.ul, s.ue, cur);
         }
     }
