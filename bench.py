@@ -21,6 +21,9 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 N, FF, NEXP, TOPK, T = 2048, 512, 512, 10, 16
 HBM_PEAK = 8.0e12
+# HBM bytes of one gate|up launch from the FETCH_SIZE / WRITE_SIZE counter runs (profiles/moe_gate_up_hbm_traffic.md),
+# as a ratio to the launch's algorithmic bytes at the profiled routing (139.2 distinct experts): 136.8 MB / 127.1 MB
+GATE_UP_TRAFFIC_RATIO = 1.076
 IQ3S_BLOCK = 110
 GU_BYTES = 2 * FF * (N // 256) * IQ3S_BLOCK      # 901,120 per expert
 DN_BYTES = N * (FF // 256) * IQ3S_BLOCK          # 450,560 per expert
@@ -35,6 +38,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--layers", type=int, default=16, help="distinct weight sets cycled through")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0: skip)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain device copy of 256 MiB, the known-size kernel that scales the FETCH_SIZE / WRITE_SIZE counters")
     ap.add_argument("--raw-layout", action="store_true", help="leave the weights as raw ggml blocks (skip the load-time re-laying)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -87,6 +92,13 @@ def main():
         x = xs[i % NX]
         dev.ok(lib.fnx_moe_verify_layer(C.byref(L), x.data_ptr(), T, outs[i % NX].data_ptr(), C.byref(ws), st))
 
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").random_()
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)
+        torch.cuda.synchronize()
+
     # ---- whole steps
     for i in range(args.warmup):
         step(i)
@@ -107,24 +119,42 @@ def main():
     u_mean = float(np.mean(njobs))
     step_bytes = u_mean * (GU_BYTES + DN_BYTES) + (GU_BYTES + DN_BYTES) + ROUTER_BYTES + XIO_BYTES
 
-    # ---- the dominant kernel on its own: routed gate|up over the step's jobs, events on the launch stream
-    xq_bytes = T * (N // 32) * 36
-    evs = []
+    # ---- the dominant kernel: the window's gate|up launch (routed experts + the shared expert), timed with events the
+    # library records on the launch stream around each of the window's five launches (fnx_layer_profile)
+    names = ["router+q8_1", "topk/jobs/plan", "gate|up", "down", "combine"]
+    per_launch = np.zeros(5)
     reps = max(50, min(args.steps, 200))
-    for i in range(reps + 10):
-        L, x = layers[i % args.layers][0], xs[i % NX]
-        # routing for this (layer, x), then only the gate|up launch between the events
-        dev.ok(lib.fnx_quantize_q8_1(x.data_ptr(), ws.xq, N, T, st))
-        dev.ok(lib.fnx_router_route(L.router, 0, x.data_ptr(), ws.logits, T, N, NEXP, TOPK, ws.topi, ws.topw, ws.jobs_gu, ws.jobs_dn, ws.njobs, st))
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        dev.ok(lib.fnx_moe_gate_up(C.byref(L.gu), L.gu_stride, ws.jobs_gu, ws.njobs, P, ws.xq, ws.gu, TOPK, st))
-        e1.record()
-        evs.append((e0, e1, i))
-    torch.cuda.synchronize()
-    k_ms = float(np.mean([a.elapsed_time(b) for a, b, i in evs[10:]]))
-    # algorithmic bytes of one launch: the distinct experts' gate|up blocks, the window's q8_1 rows, the f32 outputs
-    k_bytes = u_mean * GU_BYTES + xq_bytes + P * 2 * FF * 4
+    ms5 = np.zeros(5, dtype=np.float32)
+    fused = not args.raw_layout
+    if fused:
+        dev.ok(lib.fnx_layer_profile(1))
+        for i in range(reps + 10):
+            step(args.warmup + i)
+            dev.ok(lib.fnx_layer_profile_read(ms5.ctypes.data))
+            if i >= 10:
+                per_launch += ms5
+        dev.ok(lib.fnx_layer_profile(0))
+        per_launch /= reps
+        k_ms = float(per_launch[2])
+        kernel_name = "k_moe_gate_up_passes (unit64)"
+        # algorithmic bytes of one launch: the distinct experts' and the shared expert's gate|up blocks, the window's
+        # q8_1 rows, the f32 outputs
+        k_bytes = (u_mean + 1) * GU_BYTES + T * (N // 32) * 36 + (P + T) * 2 * FF * 4
+    else:
+        evs = []
+        for i in range(reps + 10):
+            L, x = layers[i % args.layers][0], xs[i % NX]
+            dev.ok(lib.fnx_quantize_q8_1(x.data_ptr(), ws.xq, N, T, st))
+            dev.ok(lib.fnx_router_route(L.router, 0, x.data_ptr(), ws.logits, T, N, NEXP, TOPK, ws.topi, ws.topw, ws.jobs_gu, ws.jobs_dn, ws.njobs, st))
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            dev.ok(lib.fnx_moe_gate_up(C.byref(L.gu), L.gu_stride, ws.jobs_gu, ws.njobs, P, ws.xq, ws.gu, TOPK, st))
+            e1.record()
+            evs.append((e0, e1))
+        torch.cuda.synchronize()
+        k_ms = float(np.mean([a.elapsed_time(b) for a, b in evs[10:]]))
+        kernel_name = "k_iq3s_jobs<64, narrow, raw> (routed gate|up)"
+        k_bytes = u_mean * GU_BYTES + T * (N // 32) * 36 + P * 2 * FF * 4
     achieved = k_bytes / (k_ms * 1e-3)
 
     # ---- CPU baseline: the oracle on the host's cores, same workload (layer set 0), bounded sample
@@ -162,8 +192,9 @@ def main():
         "config": {"workload": "config 2: one MoE verify layer, T=16, hidden 2048, 512 IQ3_S experts top-10, SwiGLU ff 512, shared expert, f32 router",
                    "weight_layout": "raw ggml blocks" if args.raw_layout else "unit64 (re-laid once at load, same bytes)", "weight_sets": args.layers, "distinct_experts_per_step": u_mean, "step_algorithmic_bytes": step_bytes,
                    "step_hbm_frac": step_bytes / (ms_per_step * 1e-3) / HBM_PEAK},
-        "roofline": {"bound": "hbm", "kernel": "k_iq3s_jobs<64, narrow, " + ("raw" if args.raw_layout else "unit64") + "> (routed gate|up)", "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK, "traffic": None, "kernel_ms": k_ms, "algorithmic_bytes": k_bytes},
+        "roofline": {"bound": "hbm", "kernel": kernel_name, "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK, "traffic": k_bytes * GATE_UP_TRAFFIC_RATIO if fused else None, "kernel_ms": k_ms, "algorithmic_bytes": k_bytes,
+                     "window_launch_us": {n_: round(float(v) * 1e3, 2) for n_, v in zip(names, per_launch)}},
         "cpu_baseline": cpu,
     }
     print(json.dumps(line))

@@ -162,6 +162,13 @@ typedef struct fnx_moe_ws {
     float* part;     /* [T * topk + T][n] */
 } fnx_moe_ws;
 int fnx_moe_verify_layer(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st);
+/* Profiling aid, the counterpart of the reference's FNX_PROF stamps in its window graph (engine.cu:1382-1530):
+ * fnx_layer_profile(1) makes the five-launch window record events on its stream around each launch (not to be
+ * used under graph capture), fnx_layer_profile(0) stops that; fnx_layer_profile_read waits for the last recorded
+ * window and returns its five launches' durations in milliseconds: router + q8_1 rows, top-k/jobs/plan, gate|up,
+ * down, combine. One profiled window at a time per process. */
+int fnx_layer_profile(int on);
+int fnx_layer_profile_read(float* ms5);
 #ifdef __cplusplus
 }
 #endif

@@ -67,6 +67,8 @@ EXPORTS = {
                                         C.c_void_p]),
     "fnx_accept_greedy": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int]),
     "fnx_accept_greedy_dev": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
+    "fnx_layer_profile": (C.c_int, [C.c_int]),
+    "fnx_layer_profile_read": (C.c_int, [C.c_void_p]),
     "fnx_moe_verify_layer": (C.c_int, [C.POINTER(MoeLayer), C.c_void_p, C.c_int, C.c_void_p, C.POINTER(MoeWs), C.c_void_p]),
 }
 

@@ -620,25 +620,39 @@ static bool layer_fused_ok(const fnx_moe_layer* L, int T) {
            packed(L->gu) && packed(L->down) && packed(L->sh_gu) && packed(L->sh_down) && L->gu_stride % UNIT_BYTES == 0 &&
            L->down_stride % UNIT_BYTES == 0 && L->sh_gu.p && L->sh_down.p;
 }
+// per-launch timing of the window (fnx_layer_profile): events recorded on the launch stream around each of the five
+// launches; the counterpart of the reference's FNX_PROF stamps in its window graph (engine.cu:1382-1530)
+static bool g_prof_on = false;
+static hipEvent_t g_prof_ev[6] = {};
+static void prof_mark(int i, hipStream_t s) {
+    if (g_prof_on) (void) hipEventRecord(g_prof_ev[i], s);
+}
 // the window's MoE half in five launches (k_moe_layer.h)
 static int layer_fused(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st) {
     hipStream_t s = (hipStream_t) st;
     const int n = L->n, ff = L->ff, P = T * L->topk, LS = L->nexp + 1;
     const int rblocks = (LS + RQ_ROWS - 1) / RQ_ROWS, qblocks = (T * 64 + 2 * FL_WAVES - 1) / (2 * FL_WAVES);
+    prof_mark(0, s);
     k_router_quant<<<rblocks + qblocks, FL_THREADS, 0, s>>>(RouterArgs{L->nexp, T, x, L->router, L->router_bf16, ws->logits, (uint8_t*) ws->xq});
+    prof_mark(1, s);
     k_route_plan<<<T, RT_THREADS, 0, s>>>(RouteArgs{L->nexp, L->topk, T, ws->logits, ws->topi, ws->topw, ws->jobs_gu, ws->jobs_dn, ws->njobs});
+    prof_mark(2, s);
     static const int per_cu = env_int("FNX_LAYER_BLOCKS_PER_CU", 2, 1, 8);
     const int grid = per_cu * cu_count();
     const PassArgs gu{2 * ff, (const uint8_t*) L->gu.p, L->gu_stride, (const uint8_t* const*) L->gu.ep, (const uint8_t*) L->sh_gu.p,
                       (const uint8_t*) ws->xq, nullptr, ff, ws->gu};
     k_moe_gate_up_passes<<<grid, FL_THREADS, 0, s>>>(gu);
+    prof_mark(3, s);
     const PassArgs dn{n, (const uint8_t*) L->down.p, L->down_stride, (const uint8_t* const*) L->down.ep, (const uint8_t*) L->sh_down.p,
                       nullptr, ws->gu, ff, ws->part};
     if (ff == 256) k_moe_down_passes<8><<<grid, FL_THREADS, 0, s>>>(dn);
     else if (ff == 512) k_moe_down_passes<16><<<grid, FL_THREADS, 0, s>>>(dn);
     else k_moe_down_passes<32><<<grid, FL_THREADS, 0, s>>>(dn);
+    prof_mark(4, s);
     if (launch_status("moe_verify_layer")) return 1;
-    return fnx_moe_combine(ws->part, ws->topw, ws->part + (size_t) P * n, ws->logits + L->nexp, LS, out, T, n, L->topk, st);
+    const int rc = fnx_moe_combine(ws->part, ws->topw, ws->part + (size_t) P * n, ws->logits + L->nexp, LS, out, T, n, L->topk, st);
+    prof_mark(5, s);
+    return rc;
 }
 
 }  // namespace fnx
@@ -803,6 +817,22 @@ int fnx_accept_greedy_dev(const int* rows, const int* o, int R, int* n_accept, v
     if (R < 1 || R > 64) return fail("accept_greedy_dev: 1..64 rows");
     k_accept<<<1, 64, 0, (hipStream_t) st>>>(rows, o, R, n_accept);
     return launch_status("accept_greedy_dev");
+}
+
+int fnx_layer_profile(int on) {
+    if (on && !g_prof_ev[0])
+        for (hipEvent_t& e : g_prof_ev)
+            if (hipEventCreate(&e) != hipSuccess) return fail("layer_profile: hipEventCreate failed");
+    g_prof_on = on != 0;
+    return 0;
+}
+int fnx_layer_profile_read(float* ms5) {
+    if (!ms5) return fail("layer_profile_read: null argument");
+    if (!g_prof_ev[0]) return fail("layer_profile_read: profiling was never switched on");
+    if (hipEventSynchronize(g_prof_ev[5]) != hipSuccess) return fail("layer_profile_read: no window was recorded");
+    for (int i = 0; i < 5; ++i)
+        if (hipEventElapsedTime(&ms5[i], g_prof_ev[i], g_prof_ev[i + 1]) != hipSuccess) return fail("layer_profile_read: no window was recorded");
+    return 0;
 }
 
 int fnx_moe_verify_layer(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st) {

@@ -1,0 +1,92 @@
+// C++ host-side mirror of the reference's operator API for the verify path (engine/src/kernels.hpp, namespace fnx):
+// the same function names and argument meaning, throwing std::runtime_error on failure as the reference's launch
+// wrappers do (ck_launch, kernels.cu:52-55), implemented over the C ABI of libfnx_mi355x.so.
+//
+// The reference fixes the model shape at compile time (N, NEXP, TOPK in model.hpp:38-43); here the same names are
+// template-free constants of a Shape the caller sets once (defaults: the benchmark's hidden 2048, 512 experts, top-10).
+#pragma once
+
+#include <cstddef>
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "../../include/fnx_mi355x.h"
+
+namespace fnx {
+
+constexpr int MAXT = FNX_MAXT;
+using Job = fnx_job;        // kernels.hpp:18-23
+using BigJob = fnx_bigjob;  // kernels.hpp:32-37
+using DW = fnx_dw;          // model.hpp:84-94
+
+struct Shape {
+    int N = 2048, NEXP = 512, TOPK = 10;
+};
+inline Shape& shape() {
+    static Shape s;
+    return s;
+}
+
+inline void ck(int status) {
+    if (status != 0) throw std::runtime_error(fnx_last_error());
+}
+
+constexpr size_t q8_1_bytes(int n) { return (size_t) (n / 32) * 36; }   // kernels.hpp:39
+
+// kernels.hpp:41
+inline void quantize_q8_1(const float* x, void* q, int n, int rows, void* st) { ck(fnx_quantize_q8_1(x, q, n, rows, st)); }
+// kernels.hpp:49
+inline void mmvq(const DW& W, size_t w_stride, const Job* jobs, const int* njobs, int njobs_max, const void* y, float* out, int out_stride,
+                 void* st) {
+    ck(fnx_mmvq(&W, w_stride, jobs, njobs, njobs_max, y, out, out_stride, st));
+}
+// kernels.hpp:54-55
+inline void gemv_f32(const float* W, const float* x, float* y, int rows, int n, int T, void* st) { ck(fnx_gemv_f32(W, x, y, rows, n, T, st)); }
+inline void gemv_bf16(const uint16_t* W, const float* x, float* y, int rows, int n, int T, void* st) { ck(fnx_gemv_bf16(W, x, y, rows, n, T, st)); }
+// kernels.hpp:79 (logits rows of NEXP)
+inline void route(const float* logits, int T, int* topi, float* topw, Job* jobs_gu, Job* jobs_down, int* njobs, void* st) {
+    ck(fnx_route(logits, shape().NEXP, T, shape().NEXP, shape().TOPK, topi, topw, jobs_gu, jobs_down, njobs, st));
+}
+// kernels.hpp:81, 349
+inline void swiglu_q8_1(const float* g, const float* u, void* q, int n, int rows, void* st) { ck(fnx_swiglu_q8_1(g, u, q, n, rows, st)); }
+inline void swiglu_stacked_q8_1(const float* gu, void* hq, int ffs, int T, void* st) { ck(fnx_swiglu_stacked_q8_1(gu, hq, ffs, T, st)); }
+// kernels.hpp:83
+inline void moe_combine(const float* part, const float* topw, const float* sh, const float* sh_logit, float* out, int T, void* st) {
+    ck(fnx_moe_combine(part, topw, sh, sh_logit, 1, out, T, shape().N, shape().TOPK, st));
+}
+// kernels.hpp:294 (the streaming, cache and fold arguments of the reference have no counterpart on one GPU)
+inline void router_route(const void* W, bool w_bf16, const float* x, float* logits, int T, int* topi, float* topw, Job* jobs_gu, Job* jobs_dn,
+                         int* njobs, void* st) {
+    ck(fnx_router_route(W, w_bf16 ? 1 : 0, x, logits, T, shape().N, shape().NEXP, shape().TOPK, topi, topw, jobs_gu, jobs_dn, njobs, st));
+}
+// kernels.hpp:319, 343
+inline void moe_gate_up(const DW& A, size_t sa, const Job* jobs, const int* njobs, int njobs_max, const void* xq, float* gu, void* st) {
+    ck(fnx_moe_gate_up(&A, sa, jobs, njobs, njobs_max, xq, gu, shape().TOPK, st));
+}
+inline void moe_down(const DW& A, size_t sa, const Job* jobs, const int* njobs, int njobs_max, const float* gu, float* part, void* st) {
+    ck(fnx_moe_down(&A, sa, jobs, njobs, njobs_max, gu, part, st));
+}
+// kernels.hpp:433
+inline void argmax(const float* logits, int rows, int T, int v0, float* best_v, int* best_i, unsigned long long* keys, unsigned* err, void* st) {
+    ck(fnx_argmax(logits, rows, T, v0, best_v, best_i, keys, err, st));
+}
+// session.hpp:55-58
+inline std::vector<int> lookup_drafts(const std::vector<int>& ctx, int lk, int d1, int* match = nullptr) {
+    std::vector<int> r((size_t) (lk > 0 ? lk : 0));
+    const int n = fnx_lookup_drafts(ctx.data(), (int) ctx.size(), 3, lk, d1, r.data(), match);
+    if (n < 0) throw std::runtime_error(fnx_last_error());
+    r.resize((size_t) n);
+    return r;
+}
+// session.cpp:573
+inline int accept_greedy(const std::vector<int>& rows, const std::vector<int>& o) {
+    const int n = fnx_accept_greedy(rows.data(), o.data(), (int) rows.size());
+    if (n < 0) throw std::runtime_error(fnx_last_error());
+    return n;
+}
+// load-time re-laying of an IQ3_S tensor (no counterpart in the reference's API; its own load-time layouts are model.hpp:78-82)
+inline void iq3s_repack(const void* src, void* dst, size_t n_weights, void* st) { ck(fnx_iq3s_repack(src, dst, n_weights, st)); }
+
+}  // namespace fnx
