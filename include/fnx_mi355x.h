@@ -169,6 +169,44 @@ int fnx_moe_verify_layer(const fnx_moe_layer* L, const float* x, int T, float* o
  * down, combine. One profiled window at a time per process. */
 int fnx_layer_profile(int on);
 int fnx_layer_profile_read(float* ms5);
+
+/* ---- the prompt path's MoE over a chunk of C rows (prefill.cu:1990-2083) */
+/* prefill.cu:288-377  k_pf_top10 / k_pf_count / k_pf_jobbase / k_pf_fill in one call: top-k and weights per row,
+ * cnt [nexp] pairs per expert, jbase [nexp] each expert's first job, jobs of up to FNX_PF_JOB rows per expert with
+ * the pairs in ascending order (gate|up: y = row, out = pair; down: y = out = pair), njobs[0] = the job count.
+ * njobs_cap = capacity of the job arrays; C * topk / FNX_PF_JOB + nexp is always enough. */
+int fnx_pf_route(const float* logits, int logits_stride, int C, int nexp, int topk, int* topi, float* topw, int* cnt, int* jbase,
+                 fnx_bigjob* jobs_gu, fnx_bigjob* jobs_dn, int njobs_cap, int* njobs, void* st);
+/* kernels.hpp (p100_f32_f16): f32 -> f16, round to nearest even */
+int fnx_f32_f16(const float* x, size_t n, uint16_t* out, void* st);
+/* kernels.hpp:328  moe_gate_up_mma: gu[jobs.out][2 ffs] = W_e[2 ffs][n] . xh[jobs.y] with f16 weights (each the f32
+ * value rounded once), f16 activations, fp32 accumulation, on the matrix cores. xh rows of A->n_in halves. */
+int fnx_moe_gate_up_mma(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const int* njobs, int njobs_cap, const uint16_t* xh, float* gu,
+                        void* st);
+/* kernels.hpp:329  swiglu_h16: h16[p][ffs] = f16(silu(gate) * up) of the P stacked rows [gate | up] */
+int fnx_swiglu_h16(const float* gu, int ffs, int P, uint16_t* h16, void* st);
+/* kernels.hpp:330  moe_down_mma: part[jobs.out][n] = W_e[n][ffs] . h16[jobs.y] */
+int fnx_moe_down_mma(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const int* njobs, int njobs_cap, const uint16_t* h16, float* part,
+                     void* st);
+/* caller-owned scratch for one chunk; P = C * topk, J = P / FNX_PF_JOB + nexp, S = ceil(C / FNX_PF_JOB) */
+typedef struct fnx_pf_ws {
+    float* logits;        /* [C][nexp + 1] */
+    int* topi;            /* [C][topk] */
+    float* topw;          /* [C][topk] */
+    int* cnt;             /* [nexp] */
+    int* jbase;           /* [nexp] */
+    fnx_bigjob* jobs_gu;  /* [J + S]: the routed jobs, then (at J) the shared expert's */
+    fnx_bigjob* jobs_dn;  /* [J + S] */
+    int* njobs;           /* [2]: routed jobs, shared jobs */
+    uint16_t* xh;         /* [C][n] f16 */
+    float* gu;            /* [P + C][2 ff] */
+    uint16_t* h16;        /* [P + C][ff] */
+    float* part;          /* [P + C][n] */
+} fnx_pf_ws;
+/* the MoE half of a prompt chunk on one GPU (prefill.cu:1990-2083: router -> top-k -> jobs -> gate|up -> swiglu ->
+ * down -> shared expert -> weighted sum); the shared expert (IQ3_S) runs as jobs over all rows through the same
+ * kernels. out [C][n]. */
+int fnx_moe_prefill_layer(const fnx_moe_layer* L, const float* x, int C, float* out, const fnx_pf_ws* ws, void* st);
 #ifdef __cplusplus
 }
 #endif

@@ -54,6 +54,30 @@ uint16_t fnx_o_f2h(float x) { /* round to nearest even */
     return (uint16_t) (sign | r);
 }
 
+/* IEEE round-to-nearest-even for every input, subnormal results included: what the device conversions (__float2half,
+ * kernels.cu:131-145, moe_mma.cuh:500-507, moe_mma_iq.cuh) do. The host routine above (tensor_convert.hpp:31-49) drops
+ * the bits it shifts out before it rounds a subnormal result, so the two differ on a few subnormal inputs. */
+uint16_t fnx_o_f2h_rn(float x) {
+    uint32_t b;
+    memcpy(&b, &x, 4);
+    const uint32_t sign = (b >> 16) & 0x8000u, ex = (b >> 23) & 0xFFu, man = b & 0x7FFFFFu;
+    if (ex == 0xFF) return (uint16_t) (sign | 0x7C00u | (man ? 0x200u : 0u));
+    const int ne = (int) ex - 127 + 15;
+    if (ne >= 31) return (uint16_t) (sign | 0x7C00u);
+    if (ne <= 0) {
+        if (ne < -10) return (uint16_t) sign;
+        const int shift = 14 - ne; /* 14..24 */
+        const uint32_t full = man | 0x800000u, half = 1u << (shift - 1), rem = full & ((1u << shift) - 1u);
+        uint32_t r = full >> shift;
+        if (rem > half || (rem == half && (r & 1u))) ++r;
+        return (uint16_t) (sign | r);
+    }
+    uint32_t r = ((uint32_t) ne << 10) | (man >> 13);
+    const uint32_t rem = man & 0x1FFFu;
+    if (rem > 0x1000u || (rem == 0x1000u && (r & 1u))) ++r;
+    return (uint16_t) (sign | r);
+}
+
 static float bf16_to_f32(uint16_t b) {
     const uint32_t u = (uint32_t) b << 16;
     float f;
@@ -200,7 +224,7 @@ static void q8_1_block(const float* xi, uint8_t* blk) {
     }
     const float sum = butterfly_sum(lanes, 32);
     const float d = amax / 127.0f;
-    const uint16_t dh = fnx_o_f2h(d), sh = fnx_o_f2h(sum);
+    const uint16_t dh = fnx_o_f2h_rn(d), sh = fnx_o_f2h_rn(sum);
     memcpy(blk, &dh, 2);
     memcpy(blk + 2, &sh, 2);
     for (int j = 0; j < 32; ++j) blk[4 + j] = (uint8_t) (int8_t) (amax == 0.0f ? 0 : (int) roundf(xi[j] / d));
@@ -609,6 +633,111 @@ void fnx_o_moe_verify_layer(const fnx_o_moe_layer* L, const float* x, int T, flo
     free(gu);
     free(hq);
     free(part);
+#ifdef _OPENMP
+    omp_set_num_threads(prev);
+#endif
+}
+
+/* ---------------------------------------------------------------- prompt path: f16 tiles (moe_mma_iq.cuh:108-152) */
+void fnx_o_iq3s_dequant_f16(const uint8_t* src, size_t n, uint16_t* y) {
+    float f[256];
+    for (size_t b = 0; b < n / 256; ++b) {
+        fnx_o_iq3s_dequant(src + b * IQ3S_BLOCK, 256, f); /* d * (1 + 2 s) * grid * sign: exact in f32 */
+        for (int i = 0; i < 256; ++i) y[b * 256 + i] = fnx_o_f2h_rn(f[i]);
+    }
+}
+void fnx_o_f32_f16(const float* x, size_t n, uint16_t* y) {
+    for (size_t i = 0; i < n; ++i) y[i] = fnx_o_f2h_rn(x[i]);
+}
+void fnx_o_moe_mma(const uint8_t* wbase, size_t w_stride, int nrows, int ncols, const int* jobs, int njobs, int pf_job,
+                   const uint16_t* x, int ldx, float* out, int threads) {
+    const int js = 2 + 2 * pf_job;
+    const size_t row_bytes = (size_t) (ncols / 256) * IQ3S_BLOCK;
+    if (threads <= 0) threads = 1;
+#pragma omp parallel num_threads(threads)
+    {
+        uint16_t* wh = (uint16_t*) malloc((size_t) ncols * sizeof(uint16_t));
+        float* wf = (float*) malloc((size_t) ncols * sizeof(float));
+        float* xf = (float*) malloc((size_t) pf_job * ncols * sizeof(float));
+        for (int ji = 0; ji < njobs; ++ji) {
+            const int* jb = jobs + (size_t) ji * js;
+            const uint8_t* we = wbase + (size_t) jb[0] * w_stride;
+            const int n = jb[1];
+            for (int j = 0; j < n; ++j)
+                for (int k = 0; k < ncols; ++k) xf[(size_t) j * ncols + k] = fnx_o_h2f(x[(size_t) jb[2 + j] * ldx + k]);
+#pragma omp for schedule(static)
+            for (int row = 0; row < nrows; ++row) {
+                fnx_o_iq3s_dequant_f16(we + (size_t) row * row_bytes, (size_t) ncols, wh);
+                for (int k = 0; k < ncols; ++k) wf[k] = fnx_o_h2f(wh[k]);
+                for (int j = 0; j < n; ++j) {
+                    double s = 0.0;
+                    const float* xr = xf + (size_t) j * ncols;
+                    for (int k = 0; k < ncols; ++k) s += (double) wf[k] * (double) xr[k];
+                    out[(size_t) jb[2 + pf_job + j] * nrows + row] = (float) s;
+                }
+            }
+        }
+        free(wh);
+        free(wf);
+        free(xf);
+    }
+}
+void fnx_o_swiglu_h16(const float* gu, int ffs, int P, uint16_t* h) {
+    for (int r = 0; r < P; ++r)
+        for (int i = 0; i < ffs; ++i) h[(size_t) r * ffs + i] = fnx_o_f2h_rn(silu(gu[(size_t) r * 2 * ffs + i]) * gu[(size_t) r * 2 * ffs + ffs + i]);
+}
+void fnx_o_moe_prefill_layer(const fnx_o_moe_layer* L, const float* x, int C, int pf_job, float* out, float* logits_out, int* topi_out,
+                             float* topw_out, int* njobs_out, int threads) {
+    const int n = L->n, ff = L->ff, nexp = L->nexp, topk = L->topk, P = C * topk, js = 2 + 2 * pf_job;
+    const size_t gu_stride = (size_t) 2 * ff * (n / 256) * IQ3S_BLOCK, dn_stride = (size_t) n * (ff / 256) * IQ3S_BLOCK;
+    const int maxjobs = P / pf_job + nexp + 1, shjobs = (C + pf_job - 1) / pf_job;
+    float* logits = (float*) malloc((size_t) C * (nexp + 1) * sizeof(float));
+    int* topi = (int*) malloc((size_t) P * sizeof(int));
+    float* topw = (float*) malloc((size_t) P * sizeof(float));
+    int* cnt = (int*) malloc((size_t) nexp * sizeof(int));
+    int* jgu = (int*) calloc((size_t) maxjobs * js, sizeof(int));
+    int* jdn = (int*) calloc((size_t) maxjobs * js, sizeof(int));
+    int* jsh = (int*) calloc((size_t) shjobs * js, sizeof(int));
+    uint16_t* xh = (uint16_t*) malloc((size_t) C * n * sizeof(uint16_t));
+    float* gu = (float*) malloc((size_t) (P + C) * 2 * ff * sizeof(float));
+    uint16_t* h16 = (uint16_t*) malloc((size_t) (P + C) * ff * sizeof(uint16_t));
+    float* part = (float*) malloc((size_t) (P + C) * n * sizeof(float));
+    if (threads <= 0) threads = 1;
+#ifdef _OPENMP
+    const int prev = omp_get_max_threads();
+    omp_set_num_threads(threads);
+#endif
+    for (int t0 = 0; t0 < C; t0 += 16) { /* the same sums whatever the grouping: each (row, token) sum stands alone */
+        const int T = C - t0 < 16 ? C - t0 : 16;
+        fnx_o_gemv_f32(L->router, x + (size_t) t0 * n, logits + (size_t) t0 * (nexp + 1), nexp + 1, n, T);
+    }
+    fnx_o_topk_logits(logits, nexp + 1, C, nexp, topk, topi, topw);
+    const int nj = fnx_o_pf_jobs(topi, C, topk, nexp, pf_job, jgu, jdn, cnt);
+    fnx_o_f32_f16(x, (size_t) C * n, xh);
+    fnx_o_moe_mma(L->gu, gu_stride, 2 * ff, n, jgu, nj, pf_job, xh, n, gu, threads);
+    for (int j = 0; j < shjobs; ++j) { /* the shared expert: every row, outputs at rows P + t */
+        int* jb = jsh + (size_t) j * js;
+        jb[0] = 0;
+        jb[1] = C - j * pf_job < pf_job ? C - j * pf_job : pf_job;
+        for (int i = 0; i < jb[1]; ++i) {
+            jb[2 + i] = j * pf_job + i;
+            jb[2 + pf_job + i] = P + j * pf_job + i;
+        }
+    }
+    fnx_o_moe_mma(L->sh_gu, 0, 2 * ff, n, jsh, shjobs, pf_job, xh, n, gu, threads);
+    fnx_o_swiglu_h16(gu, ff, P + C, h16);
+    fnx_o_moe_mma(L->down, dn_stride, n, ff, jdn, nj, pf_job, h16, ff, part, threads);
+    for (int j = 0; j < shjobs; ++j) {
+        int* jb = jsh + (size_t) j * js;
+        for (int i = 0; i < jb[1]; ++i) jb[2 + i] = P + j * pf_job + i;
+    }
+    fnx_o_moe_mma(L->sh_down, 0, n, ff, jsh, shjobs, pf_job, h16, ff, part, threads);
+    fnx_o_moe_combine(part, topw, part + (size_t) P * n, logits + nexp, nexp + 1, out, C, n, topk);
+    if (logits_out) memcpy(logits_out, logits, (size_t) C * (nexp + 1) * sizeof(float));
+    if (topi_out) memcpy(topi_out, topi, (size_t) P * sizeof(int));
+    if (topw_out) memcpy(topw_out, topw, (size_t) P * sizeof(float));
+    if (njobs_out) *njobs_out = nj;
+    free(logits); free(topi); free(topw); free(cnt); free(jgu); free(jdn); free(jsh); free(xh); free(gu); free(h16); free(part);
 #ifdef _OPENMP
     omp_set_num_threads(prev);
 #endif

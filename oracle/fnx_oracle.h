@@ -42,6 +42,8 @@ typedef struct {
 /* half <-> float, engine/src/tensor_convert.hpp:23-50 */
 float fnx_o_h2f(uint16_t h);
 uint16_t fnx_o_f2h(float x);
+/* IEEE round to nearest even, subnormal results included (the device's __float2half) */
+uint16_t fnx_o_f2h_rn(float x);
 
 /* p100_compat.h:18-22 (the scalar definition of the 4-way signed byte dot) */
 int fnx_o_dp4a(int a, int b, int c);
@@ -112,6 +114,22 @@ typedef struct {
 /* out [T][n]; optional outputs (may be null): logits [T][nexp+1], topi/topw [T][topk], njobs */
 void fnx_o_moe_verify_layer(const fnx_o_moe_layer* L, const float* x, int T, float* out, float* logits, int* topi,
                             float* topw, int* njobs, int threads);
+
+/* ---- the prompt path's routed experts on the matrix cores (moe_mma.cuh:1-11, 300-498; moe_mma_iq.cuh:108-152):
+ * each weight is the f32 product d * (1 + 2 s) * grid * sign rounded once to f16, activations are f16, products are
+ * accumulated in fp32 (the order is the hardware's; this restatement sums in double and rounds once) */
+void fnx_o_iq3s_dequant_f16(const uint8_t* src, size_t n, uint16_t* y);
+void fnx_o_f32_f16(const float* x, size_t n, uint16_t* y);
+/* jobs: {w, n, y[pf_job], out[pf_job]} ints; out[jobs.out[j] * nrows + row] = sum_k W_e[row][k] * x[jobs.y[j] * ldx + k] */
+void fnx_o_moe_mma(const uint8_t* wbase, size_t w_stride, int nrows, int ncols, const int* jobs, int njobs, int pf_job,
+                   const uint16_t* x, int ldx, float* out, int threads);
+/* h = silu(gate) * up of stacked rows [gate (ffs) | up (ffs)], rounded to f16 (moe_mma.cuh:500-507) */
+void fnx_o_swiglu_h16(const float* gu, int ffs, int P, uint16_t* h);
+/* one MoE layer over a prompt chunk of C rows (prefill.cu:1990-2083 on one card, IQ3_S shared expert run as jobs of
+ * all rows): router -> top-k -> BigJobs -> gate|up -> swiglu f16 -> down -> shared expert -> combine.
+ * optional outputs may be null: topi/topw [C][topk], njobs */
+void fnx_o_moe_prefill_layer(const fnx_o_moe_layer* L, const float* x, int C, int pf_job, float* out, float* logits, int* topi,
+                             float* topw, int* njobs, int threads);
 
 /* xorshift generator of the reference's self-test (selftest.cu:29-40) */
 typedef struct { unsigned long long s; } fnx_o_rng;

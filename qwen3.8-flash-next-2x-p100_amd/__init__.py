@@ -42,6 +42,10 @@ class MoeWs(C.Structure):
                 ("jobs_dn", C.c_void_p), ("njobs", C.c_void_p), ("gu", C.c_void_p), ("part", C.c_void_p)]
 
 
+class PfWs(C.Structure):
+    _fields_ = [(k, C.c_void_p) for k in ("logits", "topi", "topw", "cnt", "jbase", "jobs_gu", "jobs_dn", "njobs", "xh", "gu", "h16", "part")]
+
+
 EXPORTS = {
     # name: (restype, argtypes)
     "fnx_last_error": (C.c_char_p, []),
@@ -70,6 +74,13 @@ EXPORTS = {
     "fnx_layer_profile": (C.c_int, [C.c_int]),
     "fnx_layer_profile_read": (C.c_int, [C.c_void_p]),
     "fnx_moe_verify_layer": (C.c_int, [C.POINTER(MoeLayer), C.c_void_p, C.c_int, C.c_void_p, C.POINTER(MoeWs), C.c_void_p]),
+    "fnx_pf_route": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                               C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
+    "fnx_f32_f16": (C.c_int, [C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p]),
+    "fnx_moe_gate_up_mma": (C.c_int, [C.POINTER(DW), C.c_size_t, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "fnx_swiglu_h16": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p]),
+    "fnx_moe_down_mma": (C.c_int, [C.POINTER(DW), C.c_size_t, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "fnx_moe_prefill_layer": (C.c_int, [C.POINTER(MoeLayer), C.c_void_p, C.c_int, C.c_void_p, C.POINTER(PfWs), C.c_void_p]),
 }
 
 _lib = None

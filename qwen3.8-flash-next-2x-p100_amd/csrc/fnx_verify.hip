@@ -88,6 +88,10 @@ template <bool BF>
 __global__ void __launch_bounds__(GV_WAVES * 64) k_gemv_rows(const void* __restrict__ Wv, const float* __restrict__ x, float* __restrict__ y,
                                                             int rows, int n, int T) {
     __shared__ float4 xs[FNX_MAXT][64];
+    // blockIdx.y: a group of FNX_MAXT activation rows (each (row, token) sum stands alone, so the grouping is free)
+    x += (size_t) blockIdx.y * FNX_MAXT * n;
+    y += (size_t) blockIdx.y * FNX_MAXT * rows;
+    T = min(FNX_MAXT, T - (int) blockIdx.y * FNX_MAXT);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int row = blockIdx.x * GV_WAVES + wave;
     const bool live = row < rows;
@@ -425,6 +429,7 @@ __global__ void __launch_bounds__(512) k_iq3s_jobs(const RowsArgs a) {
 
 }  // namespace fnx
 #include "k_moe_layer.h"
+#include "k_prefill.h"
 namespace fnx {
 
 // any other row length (a multiple of 256): a wave per (row, job), sub-blocks dealt round-robin to the lanes, the
@@ -689,8 +694,8 @@ int fnx_mmvq(const fnx_dw* W, size_t w_stride, const fnx_job* jobs, const int* n
 static int gemv_any(const void* W, bool bf, const float* x, float* y, int rows, int n, int T, void* st, const char* who) {
     if (!W || !x || !y) return fail(std::string(who) + ": null argument");
     if (rows <= 0 || n <= 0 || n % 256) return fail(std::string(who) + ": n must be a positive multiple of 256");
-    if (T < 1 || T > FNX_MAXT) return fail(std::string(who) + ": T out of range");
-    const int grid = (rows + GV_WAVES - 1) / GV_WAVES;
+    if (T < 1 || T > 65535 * FNX_MAXT) return fail(std::string(who) + ": T out of range");
+    const dim3 grid((rows + GV_WAVES - 1) / GV_WAVES, (T + FNX_MAXT - 1) / FNX_MAXT);
     if (bf) k_gemv_rows<true><<<grid, GV_WAVES * 64, 0, (hipStream_t) st>>>(W, x, y, rows, n, T);
     else k_gemv_rows<false><<<grid, GV_WAVES * 64, 0, (hipStream_t) st>>>(W, x, y, rows, n, T);
     return launch_status(who);
@@ -859,6 +864,84 @@ int fnx_moe_verify_layer(const fnx_moe_layer* L, const float* x, int T, float* o
     if (rows_launch(&L->down, L->down_stride, ws->jobs_dn, ws->njobs, P, nullptr, ws->part, n, st, "moe_verify_layer down")) return 1;
     if (rows_launch(&L->sh_down, 0, ws->jobs_dn + P, nullptr, 1, nullptr, ws->part, n, st, "moe_verify_layer shared down", true)) return 1;
     return fnx_moe_combine(ws->part, ws->topw, ws->part + (size_t) P * n, ws->logits + L->nexp, L->nexp + 1, out, T, n, L->topk, st);
+}
+
+// ---------------------------------------------------------------- the prompt path
+int fnx_pf_route(const float* logits, int logits_stride, int C, int nexp, int topk, int* topi, float* topw, int* cnt, int* jbase,
+                 fnx_bigjob* jobs_gu, fnx_bigjob* jobs_dn, int njobs_cap, int* njobs, void* st) {
+    if (!logits || !topi || !topw || !cnt || !jbase || !jobs_gu || !jobs_dn || !njobs) return fail("pf_route: null argument");
+    if (C < 1 || nexp < 1 || nexp > TK_MAXE || topk < 1 || topk > 64 || topk > nexp) return fail("pf_route: bad shape");
+    if (logits_stride < nexp) return fail("pf_route: logits_stride smaller than nexp");
+    if ((long) C * topk > (1l << 30)) return fail("pf_route: too many pairs");
+    if (njobs_cap < 1) return fail("pf_route: no room for jobs");
+    hipStream_t s = (hipStream_t) st;
+    const int P = C * topk;
+    k_pf_topk<<<(C + PF_TOPK_WAVES - 1) / PF_TOPK_WAVES, PF_TOPK_WAVES * 64, 0, s>>>(logits, logits_stride, C, nexp, topk, topi, topw);
+    k_pf_jobbase<<<1, PF_BASE_THREADS, 0, s>>>(topi, P, nexp, cnt, jbase, njobs);
+    k_pf_fill<<<nexp, PF_FILL_THREADS, 0, s>>>(topi, P, topk, cnt, jbase, jobs_gu, jobs_dn, njobs_cap);
+    return launch_status("pf_route");
+}
+int fnx_f32_f16(const float* x, size_t n, uint16_t* out, void* st) {
+    if (!x || !out) return fail("f32_f16: null argument");
+    if (n == 0) return 0;
+    k_f32_f16<<<(unsigned) std::min<size_t>((n + 255) / 256, 8192), 256, 0, (hipStream_t) st>>>(x, n, out);
+    return launch_status("f32_f16");
+}
+int fnx_swiglu_h16(const float* gu, int ffs, int P, uint16_t* h16, void* st) {
+    if (!gu || !h16) return fail("swiglu_h16: null argument");
+    if (ffs < 1 || P < 1) return fail("swiglu_h16: bad shape");
+    const size_t total = (size_t) P * ffs;
+    k_swiglu_h16<<<(unsigned) std::min<size_t>((total + 255) / 256, 8192), 256, 0, (hipStream_t) st>>>(gu, ffs, total, h16);
+    return launch_status("swiglu_h16");
+}
+static int mma_launch(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const int* njobs, int njobs_cap, const uint16_t* x, float* out,
+                      void* st, const char* who) {
+    if (!A || !jobs || !njobs || !x || !out) return fail(std::string(who) + ": null argument");
+    if (!A->p && !A->ep) return fail(std::string(who) + ": no weights");
+    if (A->type != FNX_T_IQ3_S && A->type != FNX_T_IQ3S_UNIT64) return fail(std::string(who) + ": IQ3_S weights only");
+    if (A->n_in < 256 || A->n_in % 256 || A->n_out < 32 || A->n_out % 32) return fail(std::string(who) + ": columns in 256s, rows in 32s");
+    if (A->type == FNX_T_IQ3S_UNIT64 && ((size_t) A->n_out * A->n_in) % 2048) return fail(std::string(who) + ": whole units of 2048 weights");
+    if (njobs_cap < 1) return fail(std::string(who) + ": no jobs");
+    MmaArgs a{(const uint8_t*) A->p, sa, A->ep, A->n_out, A->n_in, jobs, njobs, njobs_cap, x, A->n_in, out};
+    static const int per_cu = env_int("FNX_MMA_BLOCKS_PER_CU", 2, 1, 8);
+    const long tasks = (long) njobs_cap * (A->n_out / 32);
+    const int grid = (int) std::max(1l, std::min<long>((long) per_cu * cu_count(), (tasks + MM_WAVES - 1) / MM_WAVES));
+    if (A->type == FNX_T_IQ3S_UNIT64) k_moe_mma<true, 2><<<grid, MM_THREADS, 0, (hipStream_t) st>>>(a);
+    else k_moe_mma<false, 2><<<grid, MM_THREADS, 0, (hipStream_t) st>>>(a);
+    return launch_status(who);
+}
+int fnx_moe_gate_up_mma(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const int* njobs, int njobs_cap, const uint16_t* xh, float* gu,
+                        void* st) {
+    return mma_launch(A, sa, jobs, njobs, njobs_cap, xh, gu, st, "moe_gate_up_mma");
+}
+int fnx_moe_down_mma(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const int* njobs, int njobs_cap, const uint16_t* h16, float* part,
+                     void* st) {
+    return mma_launch(A, sa, jobs, njobs, njobs_cap, h16, part, st, "moe_down_mma");
+}
+int fnx_moe_prefill_layer(const fnx_moe_layer* L, const float* x, int C, float* out, const fnx_pf_ws* ws, void* st) {
+    if (!L || !x || !out || !ws) return fail("moe_prefill_layer: null argument");
+    if (!ws->logits || !ws->topi || !ws->topw || !ws->cnt || !ws->jbase || !ws->jobs_gu || !ws->jobs_dn || !ws->njobs || !ws->xh || !ws->gu ||
+        !ws->h16 || !ws->part)
+        return fail("moe_prefill_layer: incomplete workspace");
+    const int n = L->n, ff = L->ff, nexp = L->nexp, topk = L->topk;
+    if (C < 1 || C > 65536) return fail("moe_prefill_layer: 1..65536 rows a chunk");
+    if (L->gu.n_in != n || L->gu.n_out != 2 * ff || L->down.n_in != ff || L->down.n_out != n || L->sh_gu.n_in != n ||
+        L->sh_gu.n_out != 2 * ff || L->sh_down.n_in != ff || L->sh_down.n_out != n)
+        return fail("moe_prefill_layer: weight shapes do not match n / ff");
+    const int P = C * topk, J = P / FNX_PF_JOB + nexp, S = (C + FNX_PF_JOB - 1) / FNX_PF_JOB;
+    hipStream_t s = (hipStream_t) st;
+    if (gemv_any(L->router, L->router_bf16 != 0, x, ws->logits, nexp + 1, n, C, st, "moe_prefill_layer router")) return 1;
+    if (fnx_pf_route(ws->logits, nexp + 1, C, nexp, topk, ws->topi, ws->topw, ws->cnt, ws->jbase, ws->jobs_gu, ws->jobs_dn, J, ws->njobs, st))
+        return 1;
+    k_pf_shared_jobs<<<(C + 255) / 256, 256, 0, s>>>(C, P, ws->jobs_gu + J, ws->jobs_dn + J, ws->njobs + 1);
+    if (launch_status("moe_prefill_layer shared jobs")) return 1;
+    if (fnx_f32_f16(x, (size_t) C * n, ws->xh, st)) return 1;
+    if (fnx_moe_gate_up_mma(&L->gu, L->gu_stride, ws->jobs_gu, ws->njobs, J, ws->xh, ws->gu, st)) return 1;
+    if (fnx_moe_gate_up_mma(&L->sh_gu, 0, ws->jobs_gu + J, ws->njobs + 1, S, ws->xh, ws->gu, st)) return 1;
+    if (fnx_swiglu_h16(ws->gu, ff, P + C, ws->h16, st)) return 1;
+    if (fnx_moe_down_mma(&L->down, L->down_stride, ws->jobs_dn, ws->njobs, J, ws->h16, ws->part, st)) return 1;
+    if (fnx_moe_down_mma(&L->sh_down, 0, ws->jobs_dn + J, ws->njobs + 1, S, ws->h16, ws->part, st)) return 1;
+    return fnx_moe_combine(ws->part, ws->topw, ws->part + (size_t) P * n, ws->logits + nexp, nexp + 1, out, C, n, topk, st);
 }
 
 }  // extern "C"

@@ -1,0 +1,272 @@
+// The prompt path's MoE: routing into jobs of up to FNX_PF_JOB rows per expert, and the routed experts on the matrix
+// cores with f16 weights and activations and fp32 accumulation (the numerics of the reference's moe_mma.cuh:1-11).
+//
+// Matrix-core kernel, CDNA4 form. A wave owns 16 (or 32) weight rows of one job and walks K; v_mfma_f32_16x16x32_f16
+// wants from lane l the operand row l % 16 and eight consecutive k "slots" of group l / 16. Which k a slot means is
+// free as long as both operands agree, so group g is given the sub-blocks sb = 4 q + g: a lane then decodes one whole
+// IQ3_S sub-block (32 weights, exactly what a lane of the mat-vec kernels decodes) straight into the A operands of four
+// MFMAs, and the B operand of MFMA i is the 16 contiguous bytes x[token][32 sb + 8 i ..]. The dequantised weights
+// never pass through LDS; LDS holds only the signed codebook as f16 (8192 entries of 4 halves, 64 KiB).
+// A weight becomes f16 as (grid * (1 + 2 s)) * d: the first product is an integer below 2048, exact in f16, so the
+// second rounds once - the same value as the reference's f32 product rounded to f16 (moe_mma_iq.cuh:136-149).
+#pragma once
+
+#include "k_moe_layer.h"
+
+namespace fnx {
+
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+// ---------------------------------------------------------------- routing (prefill.cu:288-377)
+// a wave per row: top-k of its logits, the weights
+constexpr int PF_TOPK_WAVES = 4;
+__global__ void __launch_bounds__(PF_TOPK_WAVES * 64) k_pf_topk(const float* __restrict__ logits, int ls, int C, int nexp, int topk,
+                                                               int* __restrict__ topi, float* __restrict__ topw) {
+    __shared__ int ex[PF_TOPK_WAVES][64];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, t = blockIdx.x * PF_TOPK_WAVES + wave;
+    if (t >= C) return;
+    if (nexp <= 512) wave_topk<8>(logits + (size_t) t * ls, nexp, topk, lane, ex[wave], topi + (size_t) t * topk, topw + (size_t) t * topk);
+    else wave_topk<16>(logits + (size_t) t * ls, nexp, topk, lane, ex[wave], topi + (size_t) t * topk, topw + (size_t) t * topk);
+}
+// one block: the experts' pair counts, each expert's first job (ceil(count / FNX_PF_JOB) jobs each), the job count
+constexpr int PF_BASE_THREADS = 1024;
+__global__ void __launch_bounds__(PF_BASE_THREADS) k_pf_jobbase(const int* __restrict__ topi, int P, int nexp, int* __restrict__ cnt,
+                                                               int* __restrict__ jbase, int* __restrict__ njobs) {
+    __shared__ int c[PF_BASE_THREADS], s[PF_BASE_THREADS];
+    const int e = threadIdx.x;
+    c[e] = 0;
+    __syncthreads();
+    for (int p = e; p < P; p += PF_BASE_THREADS) atomicAdd(&c[topi[p]], 1);
+    __syncthreads();
+    const int nj = e < nexp ? (c[e] + FNX_PF_JOB - 1) / FNX_PF_JOB : 0;
+    s[e] = nj;
+    __syncthreads();
+    for (int o = 1; o < PF_BASE_THREADS; o <<= 1) {
+        const int a = e >= o ? s[e - o] : 0;
+        __syncthreads();
+        s[e] += a;
+        __syncthreads();
+    }
+    if (e < nexp) {
+        cnt[e] = c[e];
+        jbase[e] = s[e] - nj;
+    }
+    if (e == PF_BASE_THREADS - 1) njobs[0] = s[e];
+}
+// a block per expert: its pairs in ascending order into the slots of its jobs (a pair always lands in the same job and
+// slot, prefill.cu:340-343); ballot prefix sums over the pairs
+constexpr int PF_FILL_THREADS = 256;
+__global__ void __launch_bounds__(PF_FILL_THREADS) k_pf_fill(const int* __restrict__ topi, int P, int topk, const int* __restrict__ cnt,
+                                                            const int* __restrict__ jbase, fnx_bigjob* __restrict__ gu,
+                                                            fnx_bigjob* __restrict__ dn, int cap) {
+    const int e = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int ce = cnt[e], jb = jbase[e];
+    if (ce == 0) return;
+    __shared__ int wsum[PF_FILL_THREADS / 64];
+    int base = 0;
+    for (int p0 = 0; p0 < P; p0 += PF_FILL_THREADS) {
+        const int p = p0 + tid;
+        const bool mine = p < P && topi[p] == e;
+        const unsigned long long m = __ballot(mine);
+        if (lane == 0) wsum[wave] = __popcll(m);
+        __syncthreads();
+        int before = 0, total = 0;
+#pragma unroll
+        for (int w = 0; w < PF_FILL_THREADS / 64; ++w) {
+            before += w < wave ? wsum[w] : 0;
+            total += wsum[w];
+        }
+        if (mine) {
+            const int s = base + before + __popcll(m & ((1ull << lane) - 1ull)), j = jb + s / FNX_PF_JOB, k = s % FNX_PF_JOB;
+            if (j < cap) {
+                gu[j].y[k] = p / topk;
+                gu[j].out[k] = p;
+                dn[j].y[k] = p;
+                dn[j].out[k] = p;
+                if (k == 0) {
+                    gu[j].w = dn[j].w = e;
+                    gu[j].n = dn[j].n = min(FNX_PF_JOB, ce - (s / FNX_PF_JOB) * FNX_PF_JOB);
+                }
+            }
+        }
+        base += total;
+        __syncthreads();
+    }
+}
+// the shared expert as jobs over every row: gate|up reads row t, writes row P + t; down reads and writes row P + t
+__global__ void k_pf_shared_jobs(int C, int P, fnx_bigjob* __restrict__ gu, fnx_bigjob* __restrict__ dn, int* __restrict__ nsh) {
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t == 0) *nsh = (C + FNX_PF_JOB - 1) / FNX_PF_JOB;
+    if (t >= C) return;
+    const int j = t / FNX_PF_JOB, k = t % FNX_PF_JOB;
+    gu[j].y[k] = t;
+    gu[j].out[k] = P + t;
+    dn[j].y[k] = P + t;
+    dn[j].out[k] = P + t;
+    if (k == 0) {
+        gu[j].w = dn[j].w = 0;
+        gu[j].n = dn[j].n = min(FNX_PF_JOB, C - j * FNX_PF_JOB);
+    }
+}
+
+// ---------------------------------------------------------------- element-wise
+__global__ void k_f32_f16(const float* __restrict__ x, size_t n, uint16_t* __restrict__ y) {
+    for (size_t i = blockIdx.x * (size_t) blockDim.x + threadIdx.x; i < n; i += (size_t) gridDim.x * blockDim.x) y[i] = float_to_half_bits(x[i]);
+}
+// moe_mma.cuh:500-507
+__global__ void k_swiglu_h16(const float* __restrict__ gu, int ffs, size_t total, uint16_t* __restrict__ h) {
+    for (size_t e = blockIdx.x * (size_t) blockDim.x + threadIdx.x; e < total; e += (size_t) gridDim.x * blockDim.x) {
+        const size_t r = e / ffs, i = e % ffs;
+        const float g = gu[r * 2 * ffs + i];
+        h[e] = float_to_half_bits(silu_f(g) * gu[r * 2 * ffs + ffs + i]);
+    }
+}
+
+// ---------------------------------------------------------------- the routed experts on the matrix cores
+struct MmaArgs {
+    const uint8_t* w;       // the experts' matrices: expert e at w + e * stride, or ep[e]
+    size_t stride;
+    const void* const* ep;
+    int nrows, ncols;
+    const fnx_bigjob* jobs;
+    const int* njobs;
+    int cap;
+    const uint16_t* x;      // f16 activation rows of ldx values
+    int ldx;
+    float* out;             // rows of nrows
+};
+constexpr int MM_THREADS = 512, MM_WAVES = MM_THREADS / 64, MM_TT = FNX_PF_JOB / 16;
+
+struct SubFields {   // one sub-block as loaded: four words of codes, the scale nibble, d's bits
+    uint32_t q0, q1, q2, q3, sc, d;
+};
+template <bool PACKED>
+__device__ __forceinline__ SubFields sub_load(const uint8_t* __restrict__ we, int row, int sb, int ks) {
+    SubFields r;
+    if constexpr (PACKED) {
+        const uint32_t L = (uint32_t) row * ks + sb, l = L & 63u;
+        const uint8_t* u = we + (size_t) (L >> 6) * UNIT_BYTES;
+        const uint2 a = *reinterpret_cast<const uint2*>(u + 8 * l);
+        r.q0 = a.x;
+        r.q1 = a.y;
+        r.q2 = *reinterpret_cast<const uint32_t*>(u + UNIT_B_AT + 4 * l);
+        r.q3 = u[UNIT_C_AT + l];
+        r.sc = (u[UNIT_SCALES_AT + (l >> 1)] >> (4 * (l & 1))) & 0xFu;
+        r.d = *reinterpret_cast<const unsigned short*>(u + UNIT_D_AT + 2 * (l >> 3));
+    } else {
+        const int ib = sb & 7;
+        const uint8_t* b = we + ((size_t) row * (ks >> 3) + (sb >> 3)) * 110;
+        r.q0 = load_u32_a2(b + 2 + 8 * ib);
+        r.q1 = load_u32_a2(b + 6 + 8 * ib);
+        r.q2 = load_u32_a2(b + 74 + 4 * ib);
+        r.q3 = b[66 + ib];
+        r.sc = (b[106 + (ib >> 1)] >> (4 * (ib & 1))) & 0xFu;
+        r.d = load_u16(b);
+    }
+    return r;
+}
+// LDS byte offset of group j's entry in the f16 codebook (entries of 8 bytes)
+template <bool PACKED>
+__device__ __forceinline__ uint32_t sub_entry(const SubFields& f, int j) {
+    if constexpr (PACKED) {
+        const uint32_t q[4] = {f.q0, f.q1, f.q2, f.q3};
+        const int bit = 13 * j, w = bit >> 5, s = bit & 31;
+        uint32_t v;
+        if (s + 13 <= 32) v = s >= 3 ? q[w] >> (s - 3) : q[w] << (3 - s);
+        else v = __builtin_amdgcn_alignbit(q[w + 1], q[w], s - 3);
+        return v & 0xFFF8u;
+    } else {
+        const uint32_t code = ((j < 4 ? f.q0 >> (8 * j) : f.q1 >> (8 * (j - 4))) & 0xFFu) | (((f.q3 >> j) & 1u) << 8);
+        return (((f.q2 >> (4 * j)) & 0xFu) << 12) | (code << 3);
+    }
+}
+__device__ __forceinline__ v2h as_v2h(uint32_t u) { return __builtin_bit_cast(v2h, u); }
+
+// RG: groups of 16 weight rows per wave. A task = (job, RG * 16 rows); consecutive waves take the same job's next rows.
+template <bool PACKED, int RG>
+__global__ void __launch_bounds__(MM_THREADS) k_moe_mma(const MmaArgs a) {
+    __shared__ uint2 tab[SGRID_WORDS];
+    for (int i = threadIdx.x; i < SGRID_WORDS; i += MM_THREADS) {
+        const uint32_t g = g_sgrid.v[i];
+        v2h lo, hi;
+        lo.x = (_Float16) (int) (int8_t) (g & 0xFFu);
+        lo.y = (_Float16) (int) (int8_t) ((g >> 8) & 0xFFu);
+        hi.x = (_Float16) (int) (int8_t) ((g >> 16) & 0xFFu);
+        hi.y = (_Float16) (int) (int8_t) (g >> 24);
+        tab[i] = make_uint2(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi));
+    }
+    __syncthreads();
+    const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
+    const int nj = min(a.cap, uniform(*a.njobs));
+    const int ks = a.ncols >> 5, groups = a.nrows / (16 * RG), steps = ks >> 2;
+    const int nwaves = gridDim.x * MM_WAVES;
+    for (int task = uniform(blockIdx.x * MM_WAVES + (threadIdx.x >> 6)); task < nj * groups; task += nwaves) {
+        const int ji = task / groups, row0 = (task - ji * groups) * 16 * RG;
+        const fnx_bigjob* jb = a.jobs + ji;
+        const int n = min(FNX_PF_JOB, uniform(jb->n)), e = uniform(jb->w), nt = (n + 15) >> 4;
+        if (n < 1) continue;
+        const uint8_t* we = a.ep ? (const uint8_t*) a.ep[e] : a.w + (size_t) e * a.stride;
+        const uint16_t* xr[MM_TT];
+#pragma unroll
+        for (int tt = 0; tt < MM_TT; ++tt) xr[tt] = a.x + (size_t) jb->y[min(tt * 16 + r, n - 1)] * a.ldx + 32 * g;
+        v4f acc[RG][MM_TT];
+#pragma unroll
+        for (int q = 0; q < RG; ++q)
+#pragma unroll
+            for (int tt = 0; tt < MM_TT; ++tt) acc[q][tt] = v4f{0.f, 0.f, 0.f, 0.f};
+        SubFields cur[RG];
+#pragma unroll
+        for (int q = 0; q < RG; ++q) cur[q] = sub_load<PACKED>(we, row0 + 16 * q + r, g, ks);
+        for (int st = 0; st < steps; ++st) {
+            SubFields nxt[RG];
+            const int sbn = 4 * min(st + 1, steps - 1) + g;   // past the end: the last step's again
+#pragma unroll
+            for (int q = 0; q < RG; ++q) nxt[q] = sub_load<PACKED>(we, row0 + 16 * q + r, sbn, ks);
+            // this lane's sub-block of each row group as 32 f16 weights: the A operands of four MFMAs
+            v8h A[RG][4];
+#pragma unroll
+            for (int q = 0; q < RG; ++q) {
+                const _Float16 sc = (_Float16) (int) (1 + 2 * cur[q].sc), d = __builtin_bit_cast(_Float16, (unsigned short) cur[q].d);
+                const v2h s2 = {sc, sc}, d2 = {d, d};
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const uint2 en = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint8_t*>(tab) + sub_entry<PACKED>(cur[q], j));
+                    const v2h lo = (as_v2h(en.x) * s2) * d2, hi = (as_v2h(en.y) * s2) * d2;
+                    A[q][j >> 1][4 * (j & 1) + 0] = lo.x;
+                    A[q][j >> 1][4 * (j & 1) + 1] = lo.y;
+                    A[q][j >> 1][4 * (j & 1) + 2] = hi.x;
+                    A[q][j >> 1][4 * (j & 1) + 3] = hi.y;
+                }
+            }
+#pragma unroll
+            for (int tt = 0; tt < MM_TT; ++tt)
+                if (tt < nt) {
+                    const uint4* xp = reinterpret_cast<const uint4*>(xr[tt] + 128 * st);
+                    uint4 B[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) B[i] = xp[i];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+#pragma unroll
+                        for (int q = 0; q < RG; ++q)
+                            acc[q][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[q][i], __builtin_bit_cast(v8h, B[i]), acc[q][tt], 0, 0, 0);
+                }
+#pragma unroll
+            for (int q = 0; q < RG; ++q) cur[q] = nxt[q];
+        }
+        // lane: token r of each tile, weight rows 4 g .. 4 g + 3 of each group
+#pragma unroll
+        for (int tt = 0; tt < MM_TT; ++tt) {
+            const int tok = tt * 16 + r;
+            if (tt < nt && tok < n) {
+                float* o = a.out + (size_t) jb->out[tok] * a.nrows + row0 + 4 * g;
+#pragma unroll
+                for (int q = 0; q < RG; ++q) *reinterpret_cast<float4*>(o + 16 * q) = make_float4(acc[q][tt].x, acc[q][tt].y, acc[q][tt].z, acc[q][tt].w);
+            }
+        }
+    }
+}
+
+}  // namespace fnx

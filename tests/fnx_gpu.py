@@ -200,6 +200,94 @@ class Dev:
         return int(n.item())
 
 
+    # ---- the prompt path
+    def pf_route(self, logits, nexp, topk):
+        t = self.torch
+        Cn = logits.shape[0]
+        P, cap = Cn * topk, Cn * topk // 64 + nexp
+        dl = self.up(logits.astype(np.float32))
+        topi, topw = self.zeros((Cn, topk), t.int32), self.zeros((Cn, topk), t.float32)
+        cnt, jbase, nj = self.zeros(nexp, t.int32), self.zeros(nexp, t.int32), self.zeros(2, t.int32)
+        gu, dn = self.zeros((cap, 130), t.int32), self.zeros((cap, 130), t.int32)
+        self.ok(self.lib.fnx_pf_route(dl.data_ptr(), logits.shape[1], Cn, nexp, topk, topi.data_ptr(), topw.data_ptr(), cnt.data_ptr(),
+                                      jbase.data_ptr(), gu.data_ptr(), dn.data_ptr(), cap, nj.data_ptr(), self.st()))
+        self.sync()
+        n = int(nj.cpu().numpy()[0])
+        return dict(topi=topi.cpu().numpy(), topw=topw.cpu().numpy(), cnt=cnt.cpu().numpy(), jbase=jbase.cpu().numpy(), njobs=n,
+                    gu=gu.cpu().numpy()[:n], dn=dn.cpu().numpy()[:n])
+
+    def f32_f16(self, x):
+        dx = self.up(x.astype(np.float32))
+        out = self.zeros(x.shape, self.torch.float16)
+        self.ok(self.lib.fnx_f32_f16(dx.data_ptr(), x.size, out.data_ptr(), self.st()))
+        self.sync()
+        return out.cpu().numpy()
+
+    def swiglu_h16(self, gu, ffs):
+        dg = self.up(gu.astype(np.float32))
+        out = self.zeros((gu.shape[0], ffs), self.torch.float16)
+        self.ok(self.lib.fnx_swiglu_h16(dg.data_ptr(), ffs, gu.shape[0], out.data_ptr(), self.st()))
+        self.sync()
+        return out.cpu().numpy()
+
+    def moe_mma(self, w, w_stride, nrows, ncols, jobs, x16, out_rows, packed=False, down=False, cap=None):
+        """jobs: int32 [njobs][130]; the job count is read from device memory, the arrays hold `cap` jobs"""
+        t = self.torch
+        cap = cap or len(jobs)
+        jpad = np.zeros((cap, 130), dtype=np.int32)
+        jpad[:len(jobs)] = jobs
+        dw_, dj, dx = self.up(w), self.up(jpad), self.up(np.ascontiguousarray(x16, dtype=np.float16))
+        if packed:
+            self.ok(self.lib.fnx_iq3s_repack(dw_.data_ptr(), dw_.data_ptr(), w.size // 110 * 256, self.st()))
+        out = self.zeros((out_rows, nrows), t.float32)
+        W = self.pkg.dw(dw_, ncols, nrows, packed=packed)
+        nj = self.up(np.array([len(jobs)], dtype=np.int32))
+        fn = self.lib.fnx_moe_down_mma if down else self.lib.fnx_moe_gate_up_mma
+        self.ok(fn(C.byref(W), w_stride, dj.data_ptr(), nj.data_ptr(), cap, dx.data_ptr(), out.data_ptr(), self.st()))
+        self.sync()
+        return out.cpu().numpy()
+
+
+class PfLayerDev:
+    """One MoE layer's weights plus a chunk workspace, for fnx_moe_prefill_layer."""
+
+    def __init__(self, dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, C_rows, packed=True):
+        t = dev.torch
+        pkg = dev.pkg
+        self.dev, self.n, self.ff, self.nexp, self.topk, self.C = dev, n, ff, nexp, topk, C_rows
+        self.router = dev.up(router.astype(np.float32))
+        self.gu, self.down, self.sh_gu, self.sh_down = dev.up(gu), dev.up(down), dev.up(sh_gu), dev.up(sh_down)
+        self.gu_stride = 2 * ff * (n // 256) * 110
+        self.down_stride = n * (ff // 256) * 110
+        if packed:
+            for w in (self.gu, self.down, self.sh_gu, self.sh_down):
+                dev.ok(dev.lib.fnx_iq3s_repack(w.data_ptr(), w.data_ptr(), w.numel() // 110 * 256, dev.st()))
+        self.L = pkg.MoeLayer(n, ff, nexp, topk, self.router.data_ptr(), 0, pkg.dw(self.gu, n, 2 * ff, packed=packed), self.gu_stride,
+                              pkg.dw(self.down, ff, n, packed=packed), self.down_stride, pkg.dw(self.sh_gu, n, 2 * ff, packed=packed),
+                              pkg.dw(self.sh_down, ff, n, packed=packed))
+        P = C_rows * topk
+        J, S = P // 64 + nexp, (C_rows + 63) // 64
+        self.P, self.J = P, J
+        self.bufs = dict(logits=dev.zeros((C_rows, nexp + 1), t.float32), topi=dev.zeros((C_rows, topk), t.int32),
+                         topw=dev.zeros((C_rows, topk), t.float32), cnt=dev.zeros(nexp, t.int32), jbase=dev.zeros(nexp, t.int32),
+                         jobs_gu=dev.zeros((J + S, 130), t.int32), jobs_dn=dev.zeros((J + S, 130), t.int32), njobs=dev.zeros(2, t.int32),
+                         xh=dev.zeros((C_rows, n), t.float16), gu=dev.zeros((P + C_rows, 2 * ff), t.float32),
+                         h16=dev.zeros((P + C_rows, ff), t.float16), part=dev.zeros((P + C_rows, n), t.float32))
+        self.ws = pkg.PfWs(*[self.bufs[k].data_ptr() for k in ("logits", "topi", "topw", "cnt", "jbase", "jobs_gu", "jobs_dn", "njobs", "xh",
+                                                               "gu", "h16", "part")])
+
+    def run(self, x):
+        dev = self.dev
+        Cn = x.shape[0]
+        dx = dev.up(x.astype(np.float32))
+        out = dev.zeros((Cn, self.n), dev.torch.float32)
+        dev.ok(dev.lib.fnx_moe_prefill_layer(C.byref(self.L), dx.data_ptr(), Cn, out.data_ptr(), C.byref(self.ws), dev.st()))
+        dev.sync()
+        r = {k: v.cpu().numpy() for k, v in self.bufs.items()}
+        r["out"] = out.cpu().numpy()
+        return r
+
+
 class MoeLayerDev:
     """One MoE layer's weights on the device plus a workspace, for fnx_moe_verify_layer and the per-op calls."""
 

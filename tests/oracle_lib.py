@@ -40,6 +40,7 @@ def load():
     sig = {
         "fnx_o_h2f": (f, [C.c_uint16]),
         "fnx_o_f2h": (C.c_uint16, [f]),
+        "fnx_o_f2h_rn": (C.c_uint16, [f]),
         "fnx_o_dp4a": (i, [i, i, i]),
         "fnx_o_iq3s_dequant": (None, [vp, sz, vp]),
         "fnx_o_iq3s_quantize": (None, [vp, sz, vp]),
@@ -61,6 +62,11 @@ def load():
         "fnx_o_accept_greedy": (i, [vp, vp, i]),
         "fnx_o_pf_jobs": (i, [vp, i, i, i, i, vp, vp, vp]),
         "fnx_o_moe_verify_layer": (None, [vp, vp, i, vp, vp, vp, vp, vp, i]),
+        "fnx_o_iq3s_dequant_f16": (None, [vp, sz, vp]),
+        "fnx_o_f32_f16": (None, [vp, sz, vp]),
+        "fnx_o_moe_mma": (None, [vp, sz, i, i, vp, i, i, vp, i, vp, i]),
+        "fnx_o_swiglu_h16": (None, [vp, i, i, vp]),
+        "fnx_o_moe_prefill_layer": (None, [vp, vp, i, i, vp, vp, vp, vp, vp, i]),
         "fnx_o_rng_init": (None, [vp, C.c_ulonglong]),
         "fnx_o_rng_next": (C.c_uint, [vp]),
         "fnx_o_threads": (i, []),
@@ -254,6 +260,48 @@ class Oracle:
         cnt = np.zeros(nexp, dtype=np.int32)
         nj = self.lib.fnx_o_pf_jobs(ptr(topi), Cn, topk, nexp, pf_job, ptr(gu), ptr(dn), ptr(cnt))
         return gu[:nj], dn[:nj], cnt
+
+    # ---- the prompt path
+    def iq3s_dequant_f16(self, blocks):
+        blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
+        n = blocks.size // IQ3S_BLOCK * 256
+        out = np.empty(n, dtype=np.float16)
+        self.lib.fnx_o_iq3s_dequant_f16(ptr(blocks), n, ptr(out))
+        return out
+
+    def f32_f16(self, x):
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        out = np.empty(x.shape, dtype=np.float16)
+        self.lib.fnx_o_f32_f16(ptr(x), x.size, ptr(out))
+        return out
+
+    def moe_mma(self, w, w_stride, nrows, ncols, jobs, pf_job, x16, out_rows, out=None, threads=8):
+        """jobs: int32 [njobs][2 + 2 pf_job]; x16: float16 [rows][ldx]"""
+        jobs = np.ascontiguousarray(jobs, dtype=np.int32)
+        x16 = np.ascontiguousarray(x16, dtype=np.float16)
+        if out is None:
+            out = np.zeros((out_rows, nrows), dtype=np.float32)
+        self.lib.fnx_o_moe_mma(ptr(w), w_stride, nrows, ncols, ptr(jobs), len(jobs), pf_job, ptr(x16), x16.shape[1], ptr(out), threads)
+        return out
+
+    def swiglu_h16(self, gu, ffs):
+        gu = np.ascontiguousarray(gu, dtype=np.float32)
+        out = np.empty((gu.shape[0], ffs), dtype=np.float16)
+        self.lib.fnx_o_swiglu_h16(ptr(gu), ffs, gu.shape[0], ptr(out))
+        return out
+
+    def moe_prefill_layer(self, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, x, pf_job=64, threads=8):
+        router = np.ascontiguousarray(router, dtype=np.float32)
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        Cn = x.shape[0]
+        L = MoeLayer(n, ff, nexp, topk, ptr(router), ptr(gu), ptr(down), ptr(sh_gu), ptr(sh_down))
+        out = np.zeros((Cn, n), dtype=np.float32)
+        logits = np.zeros((Cn, nexp + 1), dtype=np.float32)
+        topi = np.zeros((Cn, topk), dtype=np.int32)
+        topw = np.zeros((Cn, topk), dtype=np.float32)
+        nj = C.c_int(0)
+        self.lib.fnx_o_moe_prefill_layer(C.byref(L), ptr(x), Cn, pf_job, ptr(out), ptr(logits), ptr(topi), ptr(topw), C.byref(nj), threads)
+        return dict(out=out, logits=logits, topi=topi, topw=topw, njobs=nj.value)
 
     # ---- the layer
     def moe_verify_layer(self, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, x, threads=8):

@@ -43,7 +43,7 @@ def test_bad_arguments_are_refused_with_a_message():
     assert b"32" in lib.fnx_last_error()
     assert lib.fnx_quantize_q8_1(None, buf, 32, 1, None) != 0
     assert lib.fnx_gemv_f32(buf, buf, buf, 4, 100, 1, None) != 0
-    assert lib.fnx_gemv_f32(buf, buf, buf, 4, 256, 17, None) != 0 and b"T out of range" in lib.fnx_last_error()
+    assert lib.fnx_gemv_f32(buf, buf, buf, 4, 256, 0, None) != 0 and b"T out of range" in lib.fnx_last_error()
     bad = pkg.DW(buf, 8, 2048, 16, 880, None)               # Q8_0 experts are not handled
     assert lib.fnx_moe_gate_up(C.byref(bad), 0, buf, None, 10, buf, buf, 10, None) != 0
     assert b"IQ3_S" in lib.fnx_last_error()

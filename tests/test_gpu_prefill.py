@@ -1,0 +1,146 @@
+"""Parity of the prompt path (prefill routing, matrix-core expert products, the chunk layer) with the CPU oracle,
+through the C ABI.
+
+Bar: bit-exact for picks, counts, job bases and job lists (integers), and for f32 -> f16 conversion; relative L2 <= 1e-3
+for the matrix-core products (f16 operands identical to the oracle's, only the fp32 summation order differs: ~1e-6
+measured); SwiGLU f16 codes within one step in a small share of places (device expf).
+"""
+import numpy as np
+import pytest
+
+import fnx_gpu
+from fnx_gpu import random_iq3s
+
+pytestmark = pytest.mark.gpu
+
+REL_L2 = 1e-3
+PF = 64
+
+
+def rel_l2(a, b):
+    return float(np.linalg.norm(a.astype(np.float64) - b.astype(np.float64)) / max(np.linalg.norm(b.astype(np.float64)), 1e-30))
+
+
+@pytest.fixture(scope="module")
+def dev():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    return fnx_gpu.Dev()
+
+
+def zipf_logits(rng, Cn, nexp, s=1.1, scale=3.0):
+    """router logits whose picks follow a Zipf popularity over a random permutation of the experts"""
+    pop = 1.0 / np.arange(1, nexp + 1) ** s
+    bias = np.log(pop / pop.sum())[rng.permutation(nexp)]
+    lg = rng.standard_normal((Cn, nexp + 1)).astype(np.float32) * scale
+    lg[:, :nexp] += bias.astype(np.float32) * 2
+    return lg
+
+
+@pytest.mark.parametrize("Cn,nexp,topk,zipf", [(512, 512, 10, True), (512, 512, 10, False), (70, 8, 2, False), (1, 64, 4, False),
+                                              (300, 1000, 8, True)])
+def test_pf_route_bit_exact(dev, oracle, Cn, nexp, topk, zipf):
+    print(f"case pf_route C={Cn} nexp={nexp} topk={topk} zipf={zipf}", flush=True)
+    rng = np.random.default_rng(700 + Cn + nexp)
+    logits = zipf_logits(rng, Cn, nexp) if zipf else rng.standard_normal((Cn, nexp + 1)).astype(np.float32)
+    if Cn > 2:
+        logits[2, :topk + 3] = logits[2].max() + 1.0   # a run of ties: the lower indexes win
+    r = dev.pf_route(logits, nexp, topk)
+    topi, topw = oracle.topk_logits(logits, nexp, topk)
+    assert np.array_equal(r["topi"], topi)
+    assert np.allclose(r["topw"], topw, rtol=2e-6, atol=0)
+    gu, dn, cnt = oracle.pf_jobs(topi, nexp, PF)
+    assert np.array_equal(r["cnt"], cnt)
+    assert r["njobs"] == len(gu)
+    assert np.array_equal(r["jbase"], np.concatenate([[0], np.cumsum((cnt + PF - 1) // PF)[:-1]]))
+    for got, want in ((r["gu"], gu), (r["dn"], dn)):
+        assert np.array_equal(got[:, :2], want[:, :2])
+        for g, w in zip(got, want):
+            n = w[1]
+            assert np.array_equal(g[2:2 + n], w[2:2 + n]) and np.array_equal(g[2 + PF:2 + PF + n], w[2 + PF:2 + PF + n])
+
+
+def test_f32_f16_bit_exact(dev, oracle):
+    rng = np.random.default_rng(710)
+    x = (rng.standard_normal((33, 257)) * 10.0 ** rng.integers(-8, 4, (33, 257))).astype(np.float32)
+    assert np.array_equal(dev.f32_f16(x).view(np.uint16), oracle.f32_f16(x).view(np.uint16))
+
+
+def test_swiglu_h16(dev, oracle):
+    rng = np.random.default_rng(711)
+    gu = (rng.standard_normal((50, 1024)) * 3).astype(np.float32)
+    got, want = dev.swiglu_h16(gu, 512).view(np.uint16).astype(np.int32), oracle.swiglu_h16(gu, 512).view(np.uint16).astype(np.int32)
+    diff = np.abs(got - want)
+    assert diff.max() <= 1 and np.count_nonzero(diff) <= 1e-3 * diff.size
+
+
+def make_jobs(rng, nexp, rows_avail, sizes):
+    jobs = np.zeros((len(sizes), 2 + 2 * PF), dtype=np.int32)
+    at = 0
+    for j, n in enumerate(sizes):
+        jobs[j, 0], jobs[j, 1] = rng.integers(0, nexp), n
+        jobs[j, 2:2 + n] = rng.choice(rows_avail, size=n, replace=False)
+        jobs[j, 2 + PF:2 + PF + n] = np.arange(at, at + n)
+        at += n
+    return jobs, at
+
+
+@pytest.mark.parametrize("packed", [False, True])
+@pytest.mark.parametrize("nrows,ncols,down", [(1024, 2048, False), (2048, 512, True), (64, 256, False), (512, 1024, True)])
+def test_moe_mma_matches_oracle(dev, oracle, nrows, ncols, down, packed):
+    print(f"case moe_mma nrows={nrows} ncols={ncols} down={down} packed={packed}", flush=True)
+    if packed and (nrows * ncols) % 2048:
+        pytest.skip("unit64 takes whole units of 2048 weights")
+    rng = np.random.default_rng(720 + nrows + ncols)
+    nexp = 3
+    stride = nrows * ncols // 256 * 110
+    w = random_iq3s(rng, nexp * nrows * ncols // 256, dmax=2e-2)
+    x16 = rng.standard_normal((200, ncols)).astype(np.float16)
+    jobs, total = make_jobs(rng, nexp, 200, [64, 1, 17, 16, 33, 48, 5])
+    want = oracle.moe_mma(w, stride, nrows, ncols, jobs, PF, x16, total)
+    # the arrays hold more jobs than the count says: the rest must not run (their entries are zero: n = 0)
+    got = dev.moe_mma(w, stride, nrows, ncols, jobs, x16, total, packed=packed, down=down, cap=len(jobs) + 5)
+    assert rel_l2(got, want) <= REL_L2
+    assert rel_l2(got, want) <= 1e-5, "f16 operands are the oracle's: only the summation order may differ"
+
+
+def test_moe_mma_weights_equal_the_oracles_f16(dev, oracle):
+    # x = unit vectors: the product returns single weights, so every dequantised f16 value is checked bit for bit,
+    # subnormal ones included (tiny d)
+    rng = np.random.default_rng(730)
+    nrows, ncols = 32, 256
+    for dmax in (2e-2, 3e-6):
+        w = random_iq3s(rng, nrows * ncols // 256, dmax=dmax)
+        want = oracle.iq3s_dequant_f16(w).reshape(nrows, ncols)
+        x16 = np.eye(ncols, dtype=np.float16)
+        jobs = np.zeros((4, 2 + 2 * PF), dtype=np.int32)
+        for j in range(4):
+            jobs[j, 1] = 64
+            jobs[j, 2:2 + 64] = np.arange(64 * j, 64 * j + 64)
+            jobs[j, 2 + PF:] = np.arange(64 * j, 64 * j + 64)
+        for packed in (False, True):
+            got = dev.moe_mma(w, 0, nrows, ncols, jobs, x16, ncols, packed=packed)
+            assert np.array_equal(got.T.astype(np.float16).view(np.uint16), want.view(np.uint16))
+            assert np.array_equal(got.T, want.astype(np.float32))
+
+
+@pytest.mark.parametrize("n,ff,nexp,topk,Cn", [(2048, 512, 32, 4, 100), (2048, 512, 512, 10, 64), (256, 256, 8, 2, 70)])
+def test_prefill_layer_matches_oracle(dev, oracle, n, ff, nexp, topk, Cn):
+    print(f"case prefill_layer n={n} ff={ff} nexp={nexp} topk={topk} C={Cn}", flush=True)
+    rng = np.random.default_rng(740 + nexp + Cn)   # d small enough that h = silu(g) u stays inside f16's range
+    nb = lambda rows, cols: rows * cols // 256
+    gu = random_iq3s(rng, nexp * nb(2 * ff, n), dmax=1e-3)
+    down = random_iq3s(rng, nexp * nb(n, ff), dmax=1e-3)
+    sh_gu, sh_down = random_iq3s(rng, nb(2 * ff, n), dmax=1e-3), random_iq3s(rng, nb(n, ff), dmax=1e-3)
+    router = (rng.standard_normal((nexp + 1, n)) * 0.05).astype(np.float32)
+    x = rng.standard_normal((Cn, n)).astype(np.float32)
+    want = oracle.moe_prefill_layer(n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, x)
+    packed = (2 * ff * n) % 2048 == 0 and (n * ff) % 2048 == 0
+    L = fnx_gpu.PfLayerDev(dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, Cn, packed=packed)
+    for rep in range(2):   # a second chunk through the same workspace
+        r = L.run(x)
+        assert np.array_equal(r["logits"].view(np.uint32), want["logits"].view(np.uint32))
+        assert np.array_equal(r["topi"], want["topi"])
+        assert int(r["njobs"][0]) == want["njobs"] and int(r["njobs"][1]) == (Cn + PF - 1) // PF
+        assert np.all(np.isfinite(want["out"]))
+        assert rel_l2(r["out"], want["out"]) <= REL_L2
