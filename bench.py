@@ -41,10 +41,14 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain device copy of 256 MiB, the known-size kernel that scales the FETCH_SIZE / WRITE_SIZE counters")
     ap.add_argument("--raw-layout", action="store_true", help="leave the weights as raw ggml blocks (skip the load-time re-laying)")
+    ap.add_argument("--workload", choices=["verify", "prefill"], default="verify",
+                    help="verify: BASELINE config 2 (the headline metric, the default); prefill: config 5, one MoE layer over prompt chunks of 512 rows")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
         sys.exit(2)
+    if args.workload == "prefill":
+        return prefill_main(args)
 
     import numpy as np
     import torch
@@ -195,6 +199,137 @@ def main():
         "roofline": {"bound": "hbm", "kernel": kernel_name, "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK, "traffic": k_bytes * GATE_UP_TRAFFIC_RATIO if fused else None, "kernel_ms": k_ms, "algorithmic_bytes": k_bytes,
                      "window_launch_us": {n_: round(float(v) * 1e3, 2) for n_, v in zip(names, per_launch)}},
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(line))
+
+
+def prefill_main(args):
+    """BASELINE config 5: one MoE layer over prompt chunks of 512 rows (5,120 routed pairs), expert popularity Zipf(1.1)
+    imposed through a constant input feature and a bias column of the router. A step = one chunk."""
+    import numpy as np
+    import torch
+    import fnx_gpu
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = fnx_gpu.Dev()
+    pkg, lib, t = dev.pkg, dev.lib, torch
+    g = torch.Generator(device="cuda")
+    g.manual_seed(4321)
+    CH, PF = 512, 64
+    steps, warmup = min(args.steps, 76), min(args.warmup, 8)
+    nsets = min(args.layers, 4)
+
+    def rand_iq3s(nblocks):
+        b = torch.randint(0, 256, (nblocks, IQ3S_BLOCK), dtype=torch.uint8, device="cuda", generator=g)
+        d = (torch.rand(nblocks, device="cuda", generator=g) * 3e-4 + 1e-5).to(torch.float16)
+        b[:, 0:2] = d.view(torch.uint8).reshape(nblocks, 2)
+        return b.reshape(-1)
+
+    pop = 1.0 / np.arange(1, NEXP + 1) ** 1.1
+    layers = []
+    for _ in range(nsets):
+        router = torch.randn((NEXP + 1, N), device="cuda", generator=g) * 0.02
+        bias = np.zeros(NEXP + 1, dtype=np.float32)
+        bias[:NEXP] = np.log(pop / pop.sum())[np.random.default_rng(len(layers)).permutation(NEXP)]
+        router[:, 0] = torch.from_numpy(bias).cuda()
+        router = router.contiguous()
+        ws_ = [rand_iq3s(NEXP * 2 * FF * N // 256), rand_iq3s(NEXP * N * FF // 256), rand_iq3s(2 * FF * N // 256), rand_iq3s(N * FF // 256)]
+        raw = [a.cpu().numpy() for a in ws_] if not layers and args.cpu_seconds > 0 else None
+        for w in ws_:
+            dev.ok(lib.fnx_iq3s_repack(w.data_ptr(), w.data_ptr(), w.numel() // IQ3S_BLOCK * 256, dev.st()))
+        gu, down, sh_gu, sh_down = ws_
+        L = pkg.MoeLayer(N, FF, NEXP, TOPK, router.data_ptr(), 0, pkg.dw(gu, N, 2 * FF, packed=True), GU_BYTES, pkg.dw(down, FF, N, packed=True),
+                         DN_BYTES, pkg.dw(sh_gu, N, 2 * FF, packed=True), pkg.dw(sh_down, FF, N, packed=True))
+        layers.append((L, router, ws_, raw))
+    NX = 8
+    xs = torch.randn((NX, CH, N), device="cuda", generator=g)
+    xs[:, :, 0] = 1.0   # the constant feature the router's bias column multiplies
+    outs = torch.zeros((NX, CH, N), device="cuda")
+    P = CH * TOPK
+    J, S = P // PF + NEXP, (CH + PF - 1) // PF
+    b = dict(logits=dev.zeros((CH, NEXP + 1), t.float32), topi=dev.zeros((CH, TOPK), t.int32), topw=dev.zeros((CH, TOPK), t.float32),
+             cnt=dev.zeros(NEXP, t.int32), jbase=dev.zeros(NEXP, t.int32), jobs_gu=dev.zeros((J + S, 130), t.int32),
+             jobs_dn=dev.zeros((J + S, 130), t.int32), njobs=dev.zeros(2, t.int32), xh=dev.zeros((CH, N), t.float16),
+             gu=dev.zeros((P + CH, 2 * FF), t.float32), h16=dev.zeros((P + CH, FF), t.float16), part=dev.zeros((P + CH, N), t.float32))
+    order = ("logits", "topi", "topw", "cnt", "jbase", "jobs_gu", "jobs_dn", "njobs", "xh", "gu", "h16", "part")
+    ws = pkg.PfWs(*[b[k].data_ptr() for k in order])
+    st = dev.st()
+
+    def step(i):
+        dev.ok(lib.fnx_moe_prefill_layer(C.byref(layers[i % nsets][0]), xs[i % NX].data_ptr(), CH, outs[i % NX].data_ptr(), C.byref(ws), st))
+
+    for i in range(warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step(warmup + i)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    # routing statistics of the chunks
+    active, jobs = [], []
+    for i in range(min(steps, 16)):
+        step(warmup + i)
+        torch.cuda.synchronize()
+        active.append(int((b["cnt"] > 0).sum().item()))
+        jobs.append(int(b["njobs"][0].item()))
+    u_mean, j_mean = float(np.mean(active)), float(np.mean(jobs))
+    # the two matrix-core launches on their own, with events on the launch stream (torch's current stream)
+    reps = 20
+    evs = []
+    for i in range(reps + 3):
+        L = layers[i % nsets][0]
+        step(i)   # routes chunk i: the jobs and xh in the workspace are this chunk's
+        e = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
+        e[0].record()
+        dev.ok(lib.fnx_moe_gate_up_mma(C.byref(L.gu), L.gu_stride, ws.jobs_gu, ws.njobs, J, ws.xh, ws.gu, st))
+        e[1].record()
+        dev.ok(lib.fnx_swiglu_h16(ws.gu, FF, P + CH, ws.h16, st))
+        e[2].record()
+        dev.ok(lib.fnx_moe_down_mma(C.byref(L.down), L.down_stride, ws.jobs_dn, ws.njobs, J, ws.h16, ws.part, st))
+        e[3].record()
+        evs.append(e)
+    torch.cuda.synchronize()
+    gu_ms = float(np.mean([e[0].elapsed_time(e[1]) for e in evs[3:]]))
+    sw_ms = float(np.mean([e[1].elapsed_time(e[2]) for e in evs[3:]]))
+    dn_ms = float(np.mean([e[2].elapsed_time(e[3]) for e in evs[3:]]))
+    gu_bytes = u_mean * GU_BYTES + CH * N * 2 + P * 2 * FF * 4
+    dn_bytes = u_mean * DN_BYTES + P * FF * 2 + P * N * 4
+    gu_flops, dn_flops = 2.0 * P * 2 * FF * N, 2.0 * P * N * FF
+    step_bytes = (u_mean + 1) * (GU_BYTES + DN_BYTES) + ROUTER_BYTES + 2 * CH * N * 4
+    step_flops = 2.0 * (P + CH) * 3 * FF * N + 2.0 * CH * (NEXP + 1) * N
+    MFMA_F16 = 2.5e15
+    cpu = None
+    if args.cpu_seconds > 0:
+        import oracle_lib
+        oracle = oracle_lib.Oracle()
+        threads = min(os.cpu_count() or 1, 16)
+        CS = 64   # rows of the CPU sample
+        h = [layers[0][1].cpu().numpy()] + layers[0][3]
+        xc = xs[0, :CS].cpu().numpy()
+        c0 = time.perf_counter()
+        r = oracle.moe_prefill_layer(N, FF, NEXP, TOPK, *h, xc, threads=threads)
+        cdt = time.perf_counter() - c0
+        step(0)
+        torch.cuda.synchronize()
+        # the chunk's first CS rows are routed alone by the oracle: compare the rows' outputs (a row's result does not depend on its chunk)
+        err = float(np.linalg.norm(outs[0, :CS].cpu().numpy() - r["out"]) / np.linalg.norm(r["out"]))
+        cpu = {"value": CS / cdt, "unit": "tokens/s per layer", "cores": threads, "kind": "port",
+               "sample": f"one pass of the oracle's prefill layer over the first {CS} rows of chunk 0 (f16 operands, f64 accumulation)",
+               "parity_rel_l2": err}
+    line = {
+        "metric": "prefill MoE tokens/sec per layer (chunks of 512 rows) + grouped IQ3_S expert GEMM achieved GB/s and MFMA utilisation",
+        "value": CH * steps / dt, "unit": "tokens/s per layer", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": dt / steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16 x f16 (IQ3_S dequantised once to f16), f32 accumulate", "data": "synthetic",
+        "config": {"workload": "config 5: one MoE layer over prompt chunks of 512 rows, 5,120 routed pairs, 512 IQ3_S experts top-10 with Zipf(1.1) popularity, shared expert",
+                   "weight_sets": nsets, "active_experts_per_chunk": u_mean, "jobs_per_chunk": j_mean, "step_algorithmic_bytes": step_bytes,
+                   "step_flops": step_flops, "step_hbm_frac": step_bytes / (dt / steps) / HBM_PEAK, "step_mfma_frac": step_flops / (dt / steps) / MFMA_F16},
+        "roofline": {"bound": "hbm", "kernel": "k_moe_mma_block (routed gate|up, unit64)", "achieved": gu_bytes / (gu_ms * 1e-3) / 1e9, "peak": HBM_PEAK / 1e9,
+                     "unit": "GB/s", "frac": gu_bytes / (gu_ms * 1e-3) / HBM_PEAK, "traffic": None, "kernel_ms": gu_ms, "algorithmic_bytes": gu_bytes,
+                     "mfma_tflops": gu_flops / (gu_ms * 1e-3) / 1e12, "mfma_frac": gu_flops / (gu_ms * 1e-3) / MFMA_F16,
+                     "down": {"kernel_ms": dn_ms, "achieved": dn_bytes / (dn_ms * 1e-3) / 1e9, "mfma_tflops": dn_flops / (dn_ms * 1e-3) / 1e12},
+                     "swiglu_ms": sw_ms},
         "cpu_baseline": cpu,
     }
     print(json.dumps(line))

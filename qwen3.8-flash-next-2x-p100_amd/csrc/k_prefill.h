@@ -142,28 +142,35 @@ constexpr int MM_THREADS = 512, MM_WAVES = MM_THREADS / 64, MM_TT = FNX_PF_JOB /
 struct SubFields {   // one sub-block as loaded: four words of codes, the scale nibble, d's bits
     uint32_t q0, q1, q2, q3, sc, d;
 };
+// loads through address-space-1 pointers: global_load, which (unlike flat_load) does not tie up the LDS counter that
+// the codebook reads wait on
 template <bool PACKED>
 __device__ __forceinline__ SubFields sub_load(const uint8_t* __restrict__ we, int row, int sb, int ks) {
+    typedef __attribute__((address_space(1))) const v2u g64;
+    typedef __attribute__((address_space(1))) const uint32_t g32;
+    typedef __attribute__((address_space(1))) const unsigned short g16;
     SubFields r;
     if constexpr (PACKED) {
         const uint32_t L = (uint32_t) row * ks + sb, l = L & 63u;
-        const uint8_t* u = we + (size_t) (L >> 6) * UNIT_BYTES;
-        const uint2 a = *reinterpret_cast<const uint2*>(u + 8 * l);
+        const gbytes u = as_global(we + (size_t) (L >> 6) * UNIT_BYTES);
+        const v2u a = *(g64*) (u + 8 * l);
         r.q0 = a.x;
         r.q1 = a.y;
-        r.q2 = *reinterpret_cast<const uint32_t*>(u + UNIT_B_AT + 4 * l);
+        r.q2 = *(g32*) (u + UNIT_B_AT + 4 * l);
         r.q3 = u[UNIT_C_AT + l];
-        r.sc = (u[UNIT_SCALES_AT + (l >> 1)] >> (4 * (l & 1))) & 0xFu;
-        r.d = *reinterpret_cast<const unsigned short*>(u + UNIT_D_AT + 2 * (l >> 3));
+        r.sc = u[UNIT_SCALES_AT + (l >> 1)] >> (4 * (l & 1));
+        r.d = *(g16*) (u + UNIT_D_AT + 2 * (l >> 3));
     } else {
         const int ib = sb & 7;
-        const uint8_t* b = we + ((size_t) row * (ks >> 3) + (sb >> 3)) * 110;
-        r.q0 = load_u32_a2(b + 2 + 8 * ib);
-        r.q1 = load_u32_a2(b + 6 + 8 * ib);
-        r.q2 = load_u32_a2(b + 74 + 4 * ib);
+        const gbytes b = as_global(we + ((size_t) row * (ks >> 3) + (sb >> 3)) * 110);
+        const g16* q = (g16*) (b + 2 + 8 * ib);
+        r.q0 = q[0] | (uint32_t) q[1] << 16;
+        r.q1 = q[2] | (uint32_t) q[3] << 16;
+        const g16* sg = (g16*) (b + 74 + 4 * ib);
+        r.q2 = sg[0] | (uint32_t) sg[1] << 16;
         r.q3 = b[66 + ib];
-        r.sc = (b[106 + (ib >> 1)] >> (4 * (ib & 1))) & 0xFu;
-        r.d = load_u16(b);
+        r.sc = b[106 + (ib >> 1)] >> (4 * (ib & 1));
+        r.d = *(g16*) b;
     }
     return r;
 }
@@ -184,9 +191,15 @@ __device__ __forceinline__ uint32_t sub_entry(const SubFields& f, int j) {
 }
 __device__ __forceinline__ v2h as_v2h(uint32_t u) { return __builtin_bit_cast(v2h, u); }
 
-// RG: groups of 16 weight rows per wave. A task = (job, RG * 16 rows); consecutive waves take the same job's next rows.
+// A task = (job, RG * 16 weight rows, MM_TP token tiles of 16): uniform pieces, so a static split over the waves
+// balances; consecutive waves take the same job's next rows and share its activation rows in the caches.
+// Order of a k-step's loads matters because loads return in order: first this step's activation operands (from L2,
+// consumed after the decode), then the weights of two steps ahead (from HBM) - a wait for the former never waits for
+// the latter.
+constexpr int MM_TP = 2;
 template <bool PACKED, int RG>
-__global__ void __launch_bounds__(MM_THREADS) k_moe_mma(const MmaArgs a) {
+__global__ void __launch_bounds__(MM_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4))) k_moe_mma(const MmaArgs a) {
+    typedef __attribute__((address_space(1))) const v4u gx4;
     __shared__ uint2 tab[SGRID_WORDS];
     for (int i = threadIdx.x; i < SGRID_WORDS; i += MM_THREADS) {
         const uint32_t g = g_sgrid.v[i];
@@ -201,26 +214,37 @@ __global__ void __launch_bounds__(MM_THREADS) k_moe_mma(const MmaArgs a) {
     const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
     const int nj = min(a.cap, uniform(*a.njobs));
     const int ks = a.ncols >> 5, groups = a.nrows / (16 * RG), steps = ks >> 2;
-    const int nwaves = gridDim.x * MM_WAVES;
-    for (int task = uniform(blockIdx.x * MM_WAVES + (threadIdx.x >> 6)); task < nj * groups; task += nwaves) {
-        const int ji = task / groups, row0 = (task - ji * groups) * 16 * RG;
+    constexpr int HALVES = MM_TT / MM_TP;
+    const int nwaves = gridDim.x * MM_WAVES, per_job = groups * HALVES;
+    for (int task = uniform(blockIdx.x * MM_WAVES + (threadIdx.x >> 6)); task < nj * per_job; task += nwaves) {
+        const int ji = task / per_job, rem = task - ji * per_job, t0 = (rem / groups) * MM_TP, row0 = (rem % groups) * 16 * RG;
         const fnx_bigjob* jb = a.jobs + ji;
         const int n = min(FNX_PF_JOB, uniform(jb->n)), e = uniform(jb->w), nt = (n + 15) >> 4;
-        if (n < 1) continue;
+        if (t0 >= nt) continue;
+        const int ntile = min(MM_TP, nt - t0);
         const uint8_t* we = a.ep ? (const uint8_t*) a.ep[e] : a.w + (size_t) e * a.stride;
-        const uint16_t* xr[MM_TT];
+        const uint16_t* xr[MM_TP];
 #pragma unroll
-        for (int tt = 0; tt < MM_TT; ++tt) xr[tt] = a.x + (size_t) jb->y[min(tt * 16 + r, n - 1)] * a.ldx + 32 * g;
-        v4f acc[RG][MM_TT];
+        for (int tt = 0; tt < MM_TP; ++tt) xr[tt] = a.x + (size_t) jb->y[min((t0 + tt) * 16 + r, n - 1)] * a.ldx + 32 * g;
+        v4f acc[RG][MM_TP];
 #pragma unroll
         for (int q = 0; q < RG; ++q)
 #pragma unroll
-            for (int tt = 0; tt < MM_TT; ++tt) acc[q][tt] = v4f{0.f, 0.f, 0.f, 0.f};
-        SubFields cur[RG];
+            for (int tt = 0; tt < MM_TP; ++tt) acc[q][tt] = v4f{0.f, 0.f, 0.f, 0.f};
+        SubFields w0[RG], w1[RG];
 #pragma unroll
-        for (int q = 0; q < RG; ++q) cur[q] = sub_load<PACKED>(we, row0 + 16 * q + r, g, ks);
-        for (int st = 0; st < steps; ++st) {
-            SubFields nxt[RG];
+        for (int q = 0; q < RG; ++q) w0[q] = sub_load<PACKED>(we, row0 + 16 * q + r, g, ks);
+        // one k-step: cur holds its weights' fields; nxt receives the next step's (no register copies between steps: a
+        // copy of a loaded register would wait for the load)
+        auto step = [&](SubFields (&cur)[RG], SubFields (&nxt)[RG], int st) {
+            v4u B[MM_TP][4];
+#pragma unroll
+            for (int tt = 0; tt < MM_TP; ++tt)
+                if (tt < ntile) {
+                    const gx4* xp = (gx4*) (uintptr_t) (xr[tt] + 128 * st);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) B[tt][i] = xp[i];
+                }
             const int sbn = 4 * min(st + 1, steps - 1) + g;   // past the end: the last step's again
 #pragma unroll
             for (int q = 0; q < RG; ++q) nxt[q] = sub_load<PACKED>(we, row0 + 16 * q + r, sbn, ks);
@@ -228,7 +252,7 @@ __global__ void __launch_bounds__(MM_THREADS) k_moe_mma(const MmaArgs a) {
             v8h A[RG][4];
 #pragma unroll
             for (int q = 0; q < RG; ++q) {
-                const _Float16 sc = (_Float16) (int) (1 + 2 * cur[q].sc), d = __builtin_bit_cast(_Float16, (unsigned short) cur[q].d);
+                const _Float16 sc = (_Float16) (int) (1 + 2 * (cur[q].sc & 0xFu)), d = __builtin_bit_cast(_Float16, (unsigned short) cur[q].d);
                 const v2h s2 = {sc, sc}, d2 = {d, d};
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
@@ -241,29 +265,202 @@ __global__ void __launch_bounds__(MM_THREADS) k_moe_mma(const MmaArgs a) {
                 }
             }
 #pragma unroll
-            for (int tt = 0; tt < MM_TT; ++tt)
-                if (tt < nt) {
-                    const uint4* xp = reinterpret_cast<const uint4*>(xr[tt] + 128 * st);
-                    uint4 B[4];
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) B[i] = xp[i];
+            for (int tt = 0; tt < MM_TP; ++tt)
+                if (tt < ntile) {
 #pragma unroll
                     for (int i = 0; i < 4; ++i)
 #pragma unroll
                         for (int q = 0; q < RG; ++q)
-                            acc[q][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[q][i], __builtin_bit_cast(v8h, B[i]), acc[q][tt], 0, 0, 0);
+                            acc[q][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[q][i], __builtin_bit_cast(v8h, B[tt][i]), acc[q][tt], 0, 0, 0);
                 }
-#pragma unroll
-            for (int q = 0; q < RG; ++q) cur[q] = nxt[q];
+        };
+        for (int st = 0; st < steps; st += 2) {   // steps = ncols / 128, even for whole 256-column blocks
+            step(w0, w1, st);
+            step(w1, w0, st + 1);
         }
         // lane: token r of each tile, weight rows 4 g .. 4 g + 3 of each group
 #pragma unroll
-        for (int tt = 0; tt < MM_TT; ++tt) {
-            const int tok = tt * 16 + r;
-            if (tt < nt && tok < n) {
+        for (int tt = 0; tt < MM_TP; ++tt) {
+            const int tok = (t0 + tt) * 16 + r;
+            if (tt < ntile && tok < n) {
                 float* o = a.out + (size_t) jb->out[tok] * a.nrows + row0 + 4 * g;
 #pragma unroll
                 for (int q = 0; q < RG; ++q) *reinterpret_cast<float4*>(o + 16 * q) = make_float4(acc[q][tt].x, acc[q][tt].y, acc[q][tt].z, acc[q][tt].w);
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------- the same products, block form (unit64 weights, ncols % 512 == 0)
+// What limits the wave form above on MI355X is the vector-memory front end: every wave gathers its own activation
+// operands from 16 rows and its weights 32 bytes per row at a time, so each cache line is fetched four times and the
+// L1 sees a thousand lane accesses per k-step. Here a block of 8 waves takes one (job, 32 tokens, 256 weight rows):
+//   * the step's activation tile (32 tokens x 128 k, 8 KiB) is loaded once per block, one 16-byte load per thread,
+//     into LDS (rows padded to 272 bytes: conflict-free 16-byte operand reads), double-buffered: one barrier a step;
+//   * a lane owns four consecutive sub-blocks of its row per super-step of 512 k (sub-block 16 S + 4 g + p at step p),
+//     so its weight loads are whole 32/16/4/2-byte runs of the planes: 6 loads per row group and super-step, each
+//     line of a plane touched once; the next super-step's loads are issued a super-step ahead.
+constexpr int MB_RG = 2, MB_ROWS = MM_WAVES * 16 * MB_RG, MB_TOK = 16 * MM_TP, MB_XLD = 272;   // bytes per LDS activation row
+struct SuperFields {   // a lane's four sub-blocks of one row as loaded
+    v4u a0, a1, b;
+    uint32_t c, sc, d;
+};
+__device__ __forceinline__ SuperFields super_load(const uint8_t* __restrict__ we, int row, int sb0, int ks) {
+    typedef __attribute__((address_space(1))) const v4u g128;
+    typedef __attribute__((address_space(1))) const uint32_t g32;
+    typedef __attribute__((address_space(1))) const unsigned short g16;
+    const uint32_t L = (uint32_t) row * ks + sb0, l = L & 63u;   // l: a multiple of 4
+    const gbytes u = as_global(we + (size_t) (L >> 6) * UNIT_BYTES);
+    SuperFields r;
+    r.a0 = *(g128*) (u + 8 * l);
+    r.a1 = *(g128*) (u + 8 * l + 16);
+    r.b = *(g128*) (u + UNIT_B_AT + 4 * l);
+    r.c = *(g32*) (u + UNIT_C_AT + l);
+    r.sc = *(g16*) (u + UNIT_SCALES_AT + (l >> 1));
+    r.d = *(g16*) (u + UNIT_D_AT + 2 * (l >> 3));
+    return r;
+}
+template <int P>
+__device__ __forceinline__ SubFields super_sub(const SuperFields& f) {
+    SubFields s;
+    s.q0 = P < 2 ? f.a0[2 * (P & 1)] : f.a1[2 * (P & 1)];
+    s.q1 = P < 2 ? f.a0[2 * (P & 1) + 1] : f.a1[2 * (P & 1) + 1];
+    s.q2 = f.b[P];
+    s.q3 = (f.c >> (8 * P)) & 0xFFu;
+    s.sc = (f.sc >> (4 * P)) & 0xFu;
+    s.d = f.d;
+    return s;
+}
+constexpr int MB_XROW = 4 * MB_XLD + 16;   // a token's four step pieces of a super-step (+16: the 16 tokens of a tile fall on different banks)
+struct MmaLds {
+    uint2 tab[SGRID_WORDS];
+    uint8_t xt[2][MB_TOK * MB_XROW];   // [buffer][token][step p][lane group g][64 bytes], step rows padded to 272 bytes
+};
+__global__ void __launch_bounds__(MM_THREADS) k_moe_mma_block(const MmaArgs a) {
+    typedef __attribute__((address_space(1))) const v4u gx4;
+    __shared__ MmaLds L;
+    for (int i = threadIdx.x; i < SGRID_WORDS; i += MM_THREADS) {
+        const uint32_t g = g_sgrid.v[i];
+        v2h lo, hi;
+        lo.x = (_Float16) (int) (int8_t) (g & 0xFFu);
+        lo.y = (_Float16) (int) (int8_t) ((g >> 8) & 0xFFu);
+        hi.x = (_Float16) (int) (int8_t) ((g >> 16) & 0xFFu);
+        hi.y = (_Float16) (int) (int8_t) (g >> 24);
+        L.tab[i] = make_uint2(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi));
+    }
+    const int tid = threadIdx.x, lane = tid & 63, wave = uniform(tid >> 6), r = lane & 15, g = lane >> 4;
+    const int nj = min(a.cap, uniform(*a.njobs));
+    const int ks = a.ncols >> 5, nsuper = ks >> 4, rblocks = (a.nrows + MB_ROWS - 1) / MB_ROWS;
+    constexpr int HALVES = MM_TT / MM_TP;
+    const int per_job = rblocks * HALVES;
+    // this thread's share of a super-step's activation tile (32 tokens x 512 k): token xtok, 64 contiguous bytes
+    // (sub-block xsb of the 16); in LDS the sub-block 4 g + p goes to step p, lane group g
+    const int xtok = tid >> 4, xsb = tid & 15;
+    const int xdst = xtok * MB_XROW + (xsb & 3) * MB_XLD + (xsb >> 2) * 64;
+    for (int task = blockIdx.x; task < nj * per_job; task += gridDim.x) {
+        const int ji = task / per_job, rem = task - ji * per_job, t0 = (rem / rblocks) * MM_TP, row0 = (rem % rblocks) * MB_ROWS + wave * 16 * MB_RG;
+        const fnx_bigjob* jb = a.jobs + ji;
+        const int n = min(FNX_PF_JOB, uniform(jb->n)), e = uniform(jb->w), nt = (n + 15) >> 4;
+        if (n < 1 || t0 >= nt) continue;   // the same for every thread of the block
+        const int ntile = min(MM_TP, nt - t0);
+        const bool rows_live = row0 < a.nrows;   // per wave
+        const uint8_t* we = a.ep ? (const uint8_t*) a.ep[e] : a.w + (size_t) e * a.stride;
+        const uint16_t* xrow = a.x + (size_t) jb->y[min(t0 * 16 + xtok, n - 1)] * a.ldx + 32 * xsb;
+        struct XShare {
+            v4u v[4];
+        };
+        auto x_load = [&](int S) {
+            XShare t;
+            const gx4* p = (gx4*) (uintptr_t) (xrow + 512 * S);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) t.v[i] = p[i];
+            return t;
+        };
+        auto x_store = [&](const XShare& t, int buf) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) *reinterpret_cast<v4u*>(&L.xt[buf][xdst + 16 * i]) = t.v[i];
+        };
+        v4f acc[MB_RG][MM_TP];
+#pragma unroll
+        for (int q = 0; q < MB_RG; ++q)
+#pragma unroll
+            for (int tt = 0; tt < MM_TP; ++tt) acc[q][tt] = v4f{0.f, 0.f, 0.f, 0.f};
+        int rowq[MB_RG];
+#pragma unroll
+        for (int q = 0; q < MB_RG; ++q) rowq[q] = min(row0 + 16 * q + r, a.nrows - 1);
+        const XShare x0 = x_load(0);
+        SuperFields w0[MB_RG], w1[MB_RG];
+#pragma unroll
+        for (int q = 0; q < MB_RG; ++q) w0[q] = super_load(we, rowq[q], 4 * g, ks);
+        __syncthreads();   // the previous task's last reads of the tile buffers; the table on the first pass
+        x_store(x0, 0);
+        __syncthreads();
+        auto step = [&](const SubFields (&cur)[MB_RG], int buf, int p) {
+            v4u B[MM_TP][4];
+#pragma unroll
+            for (int tt = 0; tt < MM_TP; ++tt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) B[tt][i] = *reinterpret_cast<const v4u*>(&L.xt[buf][(tt * 16 + r) * MB_XROW + p * MB_XLD + 64 * g + 16 * i]);
+#pragma unroll
+            for (int q = 0; q < MB_RG; ++q) {
+                v8h A[4];
+                const _Float16 sc = (_Float16) (int) (1 + 2 * cur[q].sc), d = __builtin_bit_cast(_Float16, (unsigned short) cur[q].d);
+                const v2h s2 = {sc, sc}, d2 = {d, d};
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const uint2 en = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint8_t*>(L.tab) + sub_entry<true>(cur[q], j));
+                    const v2h lo = (as_v2h(en.x) * s2) * d2, hi = (as_v2h(en.y) * s2) * d2;
+                    A[j >> 1][4 * (j & 1) + 0] = lo.x;
+                    A[j >> 1][4 * (j & 1) + 1] = lo.y;
+                    A[j >> 1][4 * (j & 1) + 2] = hi.x;
+                    A[j >> 1][4 * (j & 1) + 3] = hi.y;
+                }
+#pragma unroll
+                for (int tt = 0; tt < MM_TP; ++tt)
+                    if (tt < ntile) {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                            acc[q][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[i], __builtin_bit_cast(v8h, B[tt][i]), acc[q][tt], 0, 0, 0);
+                    }
+            }
+        };
+        auto super = [&](SuperFields (&cur)[MB_RG], SuperFields (&nxt)[MB_RG], int S) {
+            const int buf = S & 1, Sn = min(S + 1, nsuper - 1);   // past the end: the last super-step's again
+            const XShare xn = x_load(Sn);
+#pragma unroll
+            for (int q = 0; q < MB_RG; ++q) nxt[q] = super_load(we, rowq[q], 16 * Sn + 4 * g, ks);
+            if (rows_live) {
+                SubFields c[MB_RG];
+#pragma unroll
+                for (int q = 0; q < MB_RG; ++q) c[q] = super_sub<0>(cur[q]);
+                step(c, buf, 0);
+#pragma unroll
+                for (int q = 0; q < MB_RG; ++q) c[q] = super_sub<1>(cur[q]);
+                step(c, buf, 1);
+#pragma unroll
+                for (int q = 0; q < MB_RG; ++q) c[q] = super_sub<2>(cur[q]);
+                step(c, buf, 2);
+#pragma unroll
+                for (int q = 0; q < MB_RG; ++q) c[q] = super_sub<3>(cur[q]);
+                step(c, buf, 3);
+            }
+            x_store(xn, buf ^ 1);
+            __syncthreads();
+        };
+        for (int S = 0; S < nsuper; S += 2) {
+            super(w0, w1, S);
+            if (S + 1 < nsuper) super(w1, w0, S + 1);
+        }
+        if (rows_live) {
+#pragma unroll
+            for (int tt = 0; tt < MM_TP; ++tt) {
+                const int tok = (t0 + tt) * 16 + r;
+                if (tt < ntile && tok < n) {
+                    float* o = a.out + (size_t) jb->out[tok] * a.nrows + row0 + 4 * g;
+#pragma unroll
+                    for (int q = 0; q < MB_RG; ++q)
+                        if (row0 + 16 * q < a.nrows) *reinterpret_cast<float4*>(o + 16 * q) = make_float4(acc[q][tt].x, acc[q][tt].y, acc[q][tt].z, acc[q][tt].w);
+                }
             }
         }
     }
