@@ -207,6 +207,79 @@ typedef struct fnx_pf_ws {
  * down -> shared expert -> weighted sum); the shared expert (IQ3_S) runs as jobs over all rows through the same
  * kernels. out [C][n]. */
 int fnx_moe_prefill_layer(const fnx_moe_layer* L, const float* x, int C, float* out, const fnx_pf_ws* ws, void* st);
+
+/* ---- the rest of a verify step around the MoE half: norms, dense projections, attention, the draft layer
+ * (BASELINE config 4: a reduced decoder of attention + MoE layers and the MTP draft layer). Head width 256, the first
+ * 64 dims rotated (model.hpp:41). */
+/* kernels.hpp:406  rms_norm_rows: y[r] = x[r] / sqrt(mean(x[r]^2) + eps) * w */
+int fnx_rms_norm_rows(const float* x, const float* w, float* y, int rows, int n, float eps, void* st);
+/* y = a + b over n floats (the residual adds between the halves of a layer) */
+int fnx_add_rows(const float* a, const float* b, float* y, size_t n, void* st);
+/* rows tokens[t] of an f16 table [vocab][n] as f32 (the window's input rows) */
+int fnx_embed_rows(const uint16_t* emb, const int* tokens, int T, int vocab, int n, float* y, void* st);
+/* model.hpp:78-82  Q8S: dense Q8_0 in the split layout: int8 values [n_out][n_in], f16 scale bits [n_out][n_in / 32] */
+typedef struct fnx_q8s {
+    const int8_t* q;
+    const uint16_t* d;
+    int n_out, n_in;
+} fnx_q8s;
+/* dense.cuh:79-214 (q8s_gemv): out[t * out_stride + r] = W[r] . y[t] for T <= 16 q8_1 rows */
+int fnx_q8s_gemv(const fnx_q8s* W, const void* yq, float* out, int out_stride, int T, void* st);
+/* rope.hpp:22-39  the rotary's constants (scaled = 0: plain frequencies base^(-2 i / 64), mscale 1) */
+typedef struct fnx_rope {
+    float base;
+    int scaled;
+    float c_low, c_high, inv_scale, mscale;
+} fnx_rope;
+/* kernels.hpp:259  attn_prep_append: q heads (qg [T][nq][q | gate], 2 x 256 each) and k heads RMS-normed with their
+ * weights and rotated at positions *pos0 + t, in place; k and v appended to the f16 cache [max_ctx][nkv][256]. */
+int fnx_attn_prep_append(float* qg, float* k, const float* v, const float* q_norm, const float* k_norm, uint16_t* kc, uint16_t* vc, int nq,
+                         int nkv, int T, const int* pos0, int max_ctx, float eps, const fnx_rope* rope, void* st);
+/* kernels.hpp:238  attn: row t attends positions [0, *pos0 + t]; out [T][nq][256] = softmax(q k / 16) v * sigmoid(gate).
+ * scratch: fnx_attn_scratch_floats(nq, T) floats (the splits' partial sums) */
+size_t fnx_attn_scratch_floats(int nq, int T);
+int fnx_attn(const float* qg, const uint16_t* kc, const uint16_t* vc, float* out, int nq, int nkv, const int* pos0, int T, float* scratch,
+             void* st);
+/* one decoder layer of the reduced model: x += wo . attn(norm(x)); x += moe(norm(x)) */
+typedef struct fnx_dec_layer {
+    const float *attn_norm, *q_norm, *k_norm, *ffn_norm;   /* [n], [256], [256], [n] */
+    fnx_q8s wq, wk, wv, wo;                                 /* [nq * 512][n], [nkv * 256][n], [nkv * 256][n], [n][nq * 256] */
+    fnx_moe_layer moe;
+    uint16_t *kc, *vc;                                      /* this layer's cache: [max_ctx][nkv][256] f16 each */
+} fnx_dec_layer;
+typedef struct fnx_decoder {
+    int n, nq, nkv, nlayers, vocab, max_ctx;
+    float eps;
+    fnx_rope rope;
+    const fnx_dec_layer* layers;   /* host array of nlayers */
+    const float* out_norm;         /* [n] */
+    fnx_q8s head;                  /* [vocab][n] */
+    const uint16_t* emb;           /* [vocab][n] f16 */
+} fnx_decoder;
+/* caller-owned scratch for windows of up to 16 rows */
+typedef struct fnx_dec_ws {
+    float *x, *xn, *qg, *k, *v, *att, *o;   /* [T][n], [T][n], [T][nq*512], [T][nkv*256] x2, [T][nq*256], [T][n] */
+    float* attn_scratch;                    /* fnx_attn_scratch_floats(nq, T) */
+    void* xq;                               /* q8_1 rows of max(n, nq * 256) values */
+    float *hidden, *logits, *best_v;        /* [T][n] (the rows before the output norm), [T][vocab], [T] */
+    int* best_i;                            /* [T] */
+    unsigned long long* keys;               /* [16], zero */
+    unsigned* err;                          /* [1] */
+    fnx_moe_ws moe;
+} fnx_dec_ws;
+/* engine.cu (Engine::enqueue, reduced): the window's rows through every layer, the output norm, the head and argmax:
+ * ws->hidden, ws->logits, ws->best_i. tokens: device, T ids; their K/V go to positions *pos0 + t. */
+int fnx_decoder_verify(const fnx_decoder* D, const int* tokens, int T, const int* pos0, const fnx_dec_ws* ws, void* st);
+/* engine.cu:2095-2133 (mtp_enqueue, without hyper-connection streams): R = fc_hid(rms(src)) + fc_emb(rms(emb[tokens])),
+ * one decoder layer (its own cache), the output norm, the head, argmax. src: [T][n] hidden rows (the verify's, or the
+ * draft layer's own for a chain). ws->hidden receives the layer's output rows. */
+typedef struct fnx_mtp {
+    const float *norm_emb, *norm_hid, *out_norm;   /* [n] each */
+    fnx_q8s fc_emb, fc_hid, head;                  /* [n][n], [n][n], [vocab][n] */
+    fnx_dec_layer layer;
+} fnx_mtp;
+int fnx_mtp_draft(const fnx_decoder* D, const fnx_mtp* M, const float* src, const int* tokens, int T, const int* pos0, const fnx_dec_ws* ws,
+                  void* st);
 #ifdef __cplusplus
 }
 #endif

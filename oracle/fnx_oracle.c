@@ -743,6 +743,178 @@ void fnx_o_moe_prefill_layer(const fnx_o_moe_layer* L, const float* x, int C, in
 #endif
 }
 
+/* ---------------------------------------------------------------- around the MoE half */
+void fnx_o_rms_norm_rows(const float* x, const float* w, float* y, int rows, int n, float eps) {
+    for (int r = 0; r < rows; ++r) {
+        double s = 0.0;
+        for (int i = 0; i < n; ++i) s += (double) x[(size_t) r * n + i] * x[(size_t) r * n + i];
+        const float sc = (float) (1.0 / sqrt(s / n + (double) eps));
+        for (int i = 0; i < n; ++i) y[(size_t) r * n + i] = x[(size_t) r * n + i] * sc * w[i];
+    }
+}
+void fnx_o_quantize_q8_0_split(const float* w, int rows, int cols, int8_t* q, uint16_t* d) {
+    const int nb = cols / 32;
+    for (int r = 0; r < rows; ++r)
+        for (int b = 0; b < nb; ++b) {
+            const float* x = w + (size_t) r * cols + 32 * b;
+            float amax = 0.f;
+            for (int j = 0; j < 32; ++j) amax = fmaxf(amax, fabsf(x[j]));
+            const float dd = amax / 127.0f, id = dd != 0.f ? 1.0f / dd : 0.f;
+            d[(size_t) r * nb + b] = fnx_o_f2h_rn(dd);
+            for (int j = 0; j < 32; ++j) q[(size_t) r * cols + 32 * b + j] = (int8_t) roundf(x[j] * id);
+        }
+}
+void fnx_o_q8s_gemv(const int8_t* q, const uint16_t* d, int rows, int cols, const uint8_t* yq, float* out, int out_stride, int T) {
+    const int nb = cols / 32;
+#pragma omp parallel for schedule(static)
+    for (int r = 0; r < rows; ++r)
+        for (int t = 0; t < T; ++t) {
+            float lane[64];
+            for (int l = 0; l < 64; ++l) {
+                float a = 0.f;
+                for (int c = 16 * l; c < cols; c += 1024) {
+                    const uint8_t* blk = yq + ((size_t) t * nb + (c >> 5)) * Q8_1_BLOCK;
+                    uint16_t dxh;
+                    memcpy(&dxh, blk, 2);
+                    const int8_t* xs = (const int8_t*) blk + 4 + (c & 16);
+                    int s = 0;
+                    for (int j = 0; j < 16; ++j) s += (int) q[(size_t) r * cols + c + j] * (int) xs[j];
+                    a = fmaf(fnx_o_h2f(d[(size_t) r * nb + (c >> 5)]) * fnx_o_h2f(dxh), (float) s, a);
+                }
+                lane[l] = a;
+            }
+            out[(size_t) t * out_stride + r] = butterfly_sum(lane, 64);
+        }
+}
+static float rope_unit_freq(const fnx_o_rope* r, int pair, int nrot) { /* rope.hpp:33-39 */
+    const float fe = powf(r->base, -2.0f * (float) pair / (float) nrot);
+    if (!r->scaled) return fe;
+    const float y = ((float) pair - r->c_low) / fmaxf(0.001f, r->c_high - r->c_low);
+    const float ramp = 1.0f - fminf(1.0f, fmaxf(0.0f, y));
+    return fe * (ramp + (1.0f - ramp) * r->inv_scale);
+}
+static void norm_rope(float* x, const float* w, int pos, int hd, int nrot, float eps, const fnx_o_rope* r) { /* kernels.cu:513-530 */
+    double ms = 0.0;
+    for (int i = 0; i < hd; ++i) ms += (double) x[i] * x[i];
+    const float sc = (float) (1.0 / sqrt(ms / hd + (double) eps));
+    for (int i = 0; i < hd; ++i) x[i] = x[i] * sc * w[i];
+    for (int i = 0; i < nrot / 2; ++i) {
+        const float theta = (float) pos * rope_unit_freq(r, i, nrot);
+        const float sn = sinf(theta) * r->mscale, cs = cosf(theta) * r->mscale;
+        const float x0 = x[i], x1 = x[i + nrot / 2];
+        x[i] = x0 * cs - x1 * sn;
+        x[i + nrot / 2] = x0 * sn + x1 * cs;
+    }
+}
+void fnx_o_attn_prep_append(float* qg, float* k, const float* v, const float* qn, const float* kn, uint16_t* kc, uint16_t* vc, int nq,
+                            int nkv, int hd, int nrot, int T, int pos0, float eps, const fnx_o_rope* rope) {
+    for (int t = 0; t < T; ++t) {
+        for (int h = 0; h < nq; ++h) norm_rope(qg + ((size_t) t * nq + h) * 2 * hd, qn, pos0 + t, hd, nrot, eps, rope);
+        for (int h = 0; h < nkv; ++h) {
+            float* kr = k + ((size_t) t * nkv + h) * hd;
+            norm_rope(kr, kn, pos0 + t, hd, nrot, eps, rope);
+            for (int i = 0; i < hd; ++i) {
+                kc[((size_t) (pos0 + t) * nkv + h) * hd + i] = fnx_o_f2h_rn(kr[i]);
+                vc[((size_t) (pos0 + t) * nkv + h) * hd + i] = fnx_o_f2h_rn(v[((size_t) t * nkv + h) * hd + i]);
+            }
+        }
+    }
+}
+void fnx_o_attn(const float* qg, const uint16_t* kc, const uint16_t* vc, float* out, int nq, int nkv, int hd, int T, int pos0) {
+    const int qpk = nq / nkv;
+#pragma omp parallel for schedule(dynamic) collapse(2)
+    for (int t = 0; t < T; ++t)
+        for (int h = 0; h < nq; ++h) {
+            const int ctx = pos0 + t + 1, kvh = h / qpk;
+            const float* q = qg + ((size_t) t * nq + h) * 2 * hd;
+            double* sc = (double*) malloc((size_t) ctx * sizeof(double));
+            double* acc = (double*) calloc((size_t) hd, sizeof(double));
+            double mx = -INFINITY, z = 0.0;
+            for (int p = 0; p < ctx; ++p) {
+                const uint16_t* kr = kc + ((size_t) p * nkv + kvh) * hd;
+                double s = 0.0;
+                for (int i = 0; i < hd; ++i) s += (double) q[i] * (double) fnx_o_h2f(kr[i]);
+                sc[p] = s / sqrt((double) hd);
+                if (sc[p] > mx) mx = sc[p];
+            }
+            for (int p = 0; p < ctx; ++p) {
+                const double w = exp(sc[p] - mx);
+                const uint16_t* vr = vc + ((size_t) p * nkv + kvh) * hd;
+                z += w;
+                for (int i = 0; i < hd; ++i) acc[i] += w * (double) fnx_o_h2f(vr[i]);
+            }
+            for (int i = 0; i < hd; ++i)
+                out[((size_t) t * nq + h) * hd + i] = (float) (acc[i] / z * (1.0 / (1.0 + exp(-(double) q[hd + i]))));
+            free(sc);
+            free(acc);
+        }
+}
+static void embed_rows(const uint16_t* emb, const int* tokens, int T, int n, float* y) {
+    for (int t = 0; t < T; ++t)
+        for (int i = 0; i < n; ++i) y[(size_t) t * n + i] = fnx_o_h2f(emb[(size_t) tokens[t] * n + i]);
+}
+static void dense_q8s(const fnx_o_q8s* W, const float* x, int T, float* out) { /* quantize_q8_1 then q8s_gemv (engine.cu dense()) */
+    uint8_t* xq = (uint8_t*) malloc((size_t) T * (W->n_in / 32) * Q8_1_BLOCK);
+    fnx_o_quantize_q8_1(x, xq, W->n_in, T);
+    fnx_o_q8s_gemv(W->q, W->d, W->n_out, W->n_in, xq, out, W->n_out, T);
+    free(xq);
+}
+static void dec_layer(const fnx_o_decoder* D, const fnx_o_dec_layer* L, float* x, int T, int pos0, int threads) {
+    const int n = D->n, nq = D->nq, nkv = D->nkv, hd = 256, nrot = 64;
+    float* xn = (float*) malloc((size_t) T * n * sizeof(float));
+    float* qg = (float*) malloc((size_t) T * nq * 2 * hd * sizeof(float));
+    float* k = (float*) malloc((size_t) T * nkv * hd * sizeof(float));
+    float* v = (float*) malloc((size_t) T * nkv * hd * sizeof(float));
+    float* att = (float*) malloc((size_t) T * nq * hd * sizeof(float));
+    float* o = (float*) malloc((size_t) T * n * sizeof(float));
+    fnx_o_rms_norm_rows(x, L->attn_norm, xn, T, n, D->eps);
+    dense_q8s(&L->wq, xn, T, qg);
+    dense_q8s(&L->wk, xn, T, k);
+    dense_q8s(&L->wv, xn, T, v);
+    fnx_o_attn_prep_append(qg, k, v, L->q_norm, L->k_norm, L->kc, L->vc, nq, nkv, hd, nrot, T, pos0, D->eps, &D->rope);
+    fnx_o_attn(qg, L->kc, L->vc, att, nq, nkv, hd, T, pos0);
+    dense_q8s(&L->wo, att, T, o);
+    for (size_t i = 0; i < (size_t) T * n; ++i) x[i] += o[i];
+    fnx_o_rms_norm_rows(x, L->ffn_norm, xn, T, n, D->eps);
+    fnx_o_moe_verify_layer(&L->moe, xn, T, o, NULL, NULL, NULL, NULL, threads);
+    for (size_t i = 0; i < (size_t) T * n; ++i) x[i] += o[i];
+    free(xn); free(qg); free(k); free(v); free(att); free(o);
+}
+static void dec_head(const fnx_o_decoder* D, const float* norm, const fnx_o_q8s* head, const float* x, int T, float* logits_out, int* best) {
+    float* xn = (float*) malloc((size_t) T * D->n * sizeof(float));
+    float* logits = logits_out ? logits_out : (float*) malloc((size_t) T * D->vocab * sizeof(float));
+    float* bv = (float*) malloc((size_t) T * sizeof(float));
+    fnx_o_rms_norm_rows(x, norm, xn, T, D->n, D->eps);
+    dense_q8s(head, xn, T, logits);
+    fnx_o_argmax(logits, D->vocab, T, 0, bv, best);
+    free(xn);
+    free(bv);
+    if (!logits_out) free(logits);
+}
+void fnx_o_decoder_verify(const fnx_o_decoder* D, const int* tokens, int T, int pos0, float* hidden, float* logits, int* best, int threads) {
+    embed_rows(D->emb, tokens, T, D->n, hidden);
+    for (int l = 0; l < D->nlayers; ++l) dec_layer(D, &D->layers[l], hidden, T, pos0, threads);
+    dec_head(D, D->out_norm, &D->head, hidden, T, logits, best);
+}
+void fnx_o_mtp_draft(const fnx_o_decoder* D, const fnx_o_mtp* M, const float* src, const int* tokens, int T, int pos0, float* hidden,
+                     float* logits, int* best, int threads) {
+    const int n = D->n;
+    float* xn = (float*) malloc((size_t) T * n * sizeof(float));
+    float* e = (float*) malloc((size_t) T * n * sizeof(float));
+    float* e2 = (float*) malloc((size_t) T * n * sizeof(float));
+    float* x = (float*) malloc((size_t) T * n * sizeof(float));
+    fnx_o_rms_norm_rows(src, M->norm_hid, xn, T, n, D->eps);
+    dense_q8s(&M->fc_hid, xn, T, x);
+    embed_rows(D->emb, tokens, T, n, e);
+    fnx_o_rms_norm_rows(e, M->norm_emb, xn, T, n, D->eps);
+    dense_q8s(&M->fc_emb, xn, T, e2);
+    for (size_t i = 0; i < (size_t) T * n; ++i) x[i] += e2[i];
+    dec_layer(D, &M->layer, x, T, pos0, threads);
+    memcpy(hidden, x, (size_t) T * n * sizeof(float));
+    dec_head(D, M->out_norm, &M->head, x, T, logits, best);
+    free(xn); free(e); free(e2); free(x);
+}
+
 /* ---------------------------------------------------------------- selftest.cu:29-40 */
 void fnx_o_rng_init(fnx_o_rng* r, unsigned long long seed) { r->s = seed * 2685821657736338717ull + 1442695040888963407ull; }
 unsigned fnx_o_rng_next(fnx_o_rng* r) {

@@ -131,6 +131,58 @@ void fnx_o_swiglu_h16(const float* gu, int ffs, int P, uint16_t* h);
 void fnx_o_moe_prefill_layer(const fnx_o_moe_layer* L, const float* x, int C, int pf_job, float* out, float* logits, int* topi,
                              float* topw, int* njobs, int threads);
 
+/* ---- around the MoE half (BASELINE config 4): norms, dense Q8_0 projections, attention, the draft layer */
+/* kernels.cu:2818-2826; the mean of squares summed in double */
+void fnx_o_rms_norm_rows(const float* x, const float* w, float* y, int rows, int n, float eps);
+/* ggml's Q8_0 in the reference's split layout (model.hpp:78-82): d = max|x| / 127 as f16, q = round(x / d) */
+void fnx_o_quantize_q8_0_split(const float* w, int rows, int cols, int8_t* q, uint16_t* d);
+/* dense.cuh:79-214: out[t * out_stride + r] = sum over 32-blocks of (d_w d_x) * (float) dot; 64 lanes, lane l takes the
+ * 16-column pieces l, l + 64, ... with fmaf, then the xor-butterfly (this build's fixed order, shared with the device) */
+void fnx_o_q8s_gemv(const int8_t* q, const uint16_t* d, int rows, int cols, const uint8_t* yq, float* out, int out_stride, int T);
+typedef struct {
+    float base;
+    int scaled;
+    float c_low, c_high, inv_scale, mscale;
+} fnx_o_rope;
+/* kernels.cu:513-537, 1878-1910: q and k heads RMS-normed (weights qn, kn) and NEOX-rotated on the first nrot dims at
+ * positions pos0 + t, in place; k and v rounded to f16 into the cache rows [pos][nkv][hd] */
+void fnx_o_attn_prep_append(float* qg, float* k, const float* v, const float* qn, const float* kn, uint16_t* kc, uint16_t* vc, int nq,
+                            int nkv, int hd, int nrot, int T, int pos0, float eps, const fnx_o_rope* rope);
+/* kernels.cu:541-643, 786-803 as textbook attention in double: row t over positions [0, pos0 + t], scores q.k / sqrt(hd),
+ * out = softmax . v * sigmoid(gate); qg [T][nq][q | gate] */
+void fnx_o_attn(const float* qg, const uint16_t* kc, const uint16_t* vc, float* out, int nq, int nkv, int hd, int T, int pos0);
+typedef struct {
+    const int8_t* q;
+    const uint16_t* d;
+    int n_out, n_in;
+} fnx_o_q8s;
+typedef struct {
+    const float *attn_norm, *q_norm, *k_norm, *ffn_norm;
+    fnx_o_q8s wq, wk, wv, wo;
+    fnx_o_moe_layer moe;
+    uint16_t *kc, *vc;
+} fnx_o_dec_layer;
+typedef struct {
+    int n, nq, nkv, nlayers, vocab, max_ctx;
+    float eps;
+    fnx_o_rope rope;
+    const fnx_o_dec_layer* layers;
+    const float* out_norm;
+    fnx_o_q8s head;
+    const uint16_t* emb;
+} fnx_o_decoder;
+typedef struct {
+    const float *norm_emb, *norm_hid, *out_norm;
+    fnx_o_q8s fc_emb, fc_hid, head;
+    fnx_o_dec_layer layer;
+} fnx_o_mtp;
+/* the reduced decoder's window (engine.cu Engine::enqueue without streams, cards, GDN layers): hidden [T][n], logits
+ * [T][vocab] (may be null), best [T] = argmax rows */
+void fnx_o_decoder_verify(const fnx_o_decoder* D, const int* tokens, int T, int pos0, float* hidden, float* logits, int* best, int threads);
+/* engine.cu:2095-2133 without streams: R = fc_hid(rms(src)) + fc_emb(rms(emb[tokens])), one layer, norm, head, argmax */
+void fnx_o_mtp_draft(const fnx_o_decoder* D, const fnx_o_mtp* M, const float* src, const int* tokens, int T, int pos0, float* hidden,
+                     float* logits, int* best, int threads);
+
 /* xorshift generator of the reference's self-test (selftest.cu:29-40) */
 typedef struct { unsigned long long s; } fnx_o_rng;
 void fnx_o_rng_init(fnx_o_rng* r, unsigned long long seed);

@@ -46,6 +46,35 @@ class PfWs(C.Structure):
     _fields_ = [(k, C.c_void_p) for k in ("logits", "topi", "topw", "cnt", "jbase", "jobs_gu", "jobs_dn", "njobs", "xh", "gu", "h16", "part")]
 
 
+class Q8S(C.Structure):
+    _fields_ = [("q", C.c_void_p), ("d", C.c_void_p), ("n_out", C.c_int), ("n_in", C.c_int)]
+
+
+class Rope(C.Structure):
+    _fields_ = [("base", C.c_float), ("scaled", C.c_int), ("c_low", C.c_float), ("c_high", C.c_float), ("inv_scale", C.c_float),
+                ("mscale", C.c_float)]
+
+
+class DecLayer(C.Structure):
+    _fields_ = [("attn_norm", C.c_void_p), ("q_norm", C.c_void_p), ("k_norm", C.c_void_p), ("ffn_norm", C.c_void_p), ("wq", Q8S), ("wk", Q8S),
+                ("wv", Q8S), ("wo", Q8S), ("moe", MoeLayer), ("kc", C.c_void_p), ("vc", C.c_void_p)]
+
+
+class Decoder(C.Structure):
+    _fields_ = [("n", C.c_int), ("nq", C.c_int), ("nkv", C.c_int), ("nlayers", C.c_int), ("vocab", C.c_int), ("max_ctx", C.c_int),
+                ("eps", C.c_float), ("rope", Rope), ("layers", C.c_void_p), ("out_norm", C.c_void_p), ("head", Q8S), ("emb", C.c_void_p)]
+
+
+class DecWs(C.Structure):
+    _fields_ = [(k, C.c_void_p) for k in ("x", "xn", "qg", "k", "v", "att", "o", "attn_scratch", "xq", "hidden", "logits", "best_v", "best_i",
+                                          "keys", "err")] + [("moe", MoeWs)]
+
+
+class Mtp(C.Structure):
+    _fields_ = [("norm_emb", C.c_void_p), ("norm_hid", C.c_void_p), ("out_norm", C.c_void_p), ("fc_emb", Q8S), ("fc_hid", Q8S), ("head", Q8S),
+                ("layer", DecLayer)]
+
+
 EXPORTS = {
     # name: (restype, argtypes)
     "fnx_last_error": (C.c_char_p, []),
@@ -80,6 +109,16 @@ EXPORTS = {
     "fnx_moe_gate_up_mma": (C.c_int, [C.POINTER(DW), C.c_size_t, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
     "fnx_swiglu_h16": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p]),
     "fnx_moe_down_mma": (C.c_int, [C.POINTER(DW), C.c_size_t, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "fnx_rms_norm_rows": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_float, C.c_void_p]),
+    "fnx_add_rows": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "fnx_embed_rows": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]),
+    "fnx_q8s_gemv": (C.c_int, [C.POINTER(Q8S), C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
+    "fnx_attn_prep_append": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int,
+                                       C.c_int, C.c_void_p, C.c_int, C.c_float, C.POINTER(Rope), C.c_void_p]),
+    "fnx_attn_scratch_floats": (C.c_size_t, [C.c_int, C.c_int]),
+    "fnx_attn": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
+    "fnx_decoder_verify": (C.c_int, [C.POINTER(Decoder), C.c_void_p, C.c_int, C.c_void_p, C.POINTER(DecWs), C.c_void_p]),
+    "fnx_mtp_draft": (C.c_int, [C.POINTER(Decoder), C.POINTER(Mtp), C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.POINTER(DecWs), C.c_void_p]),
     "fnx_moe_prefill_layer": (C.c_int, [C.POINTER(MoeLayer), C.c_void_p, C.c_int, C.c_void_p, C.POINTER(PfWs), C.c_void_p]),
 }
 

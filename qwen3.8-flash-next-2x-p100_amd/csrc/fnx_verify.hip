@@ -9,6 +9,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <cmath>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -430,6 +431,7 @@ __global__ void __launch_bounds__(512) k_iq3s_jobs(const RowsArgs a) {
 }  // namespace fnx
 #include "k_moe_layer.h"
 #include "k_prefill.h"
+#include "k_decoder.h"
 namespace fnx {
 
 // any other row length (a multiple of 256): a wave per (row, job), sub-blocks dealt round-robin to the lanes, the
@@ -949,6 +951,141 @@ int fnx_moe_prefill_layer(const fnx_moe_layer* L, const float* x, int C, float* 
     if (fnx_moe_down_mma(&L->down, L->down_stride, ws->jobs_dn, ws->njobs, J, ws->h16, ws->part, st)) return 1;
     if (fnx_moe_down_mma(&L->sh_down, 0, ws->jobs_dn + J, ws->njobs + 1, S, ws->h16, ws->part, st)) return 1;
     return fnx_moe_combine(ws->part, ws->topw, ws->part + (size_t) P * n, ws->logits + nexp, nexp + 1, out, C, n, topk, st);
+}
+
+// ---------------------------------------------------------------- around the MoE half: norms, dense projections, attention
+int fnx_rms_norm_rows(const float* x, const float* w, float* y, int rows, int n, float eps, void* st) {
+    if (!x || !w || !y) return fail("rms_norm_rows: null argument");
+    if (rows < 1 || n < 1) return fail("rms_norm_rows: bad shape");
+    k_rms_norm_rows<<<rows, 256, 0, (hipStream_t) st>>>(x, w, y, n, eps);
+    return launch_status("rms_norm_rows");
+}
+int fnx_add_rows(const float* a, const float* b, float* y, size_t n, void* st) {
+    if (!a || !b || !y) return fail("add_rows: null argument");
+    if (n == 0) return 0;
+    k_add_rows<<<(unsigned) std::min<size_t>((n + 255) / 256, 4096), 256, 0, (hipStream_t) st>>>(a, b, y, n);
+    return launch_status("add_rows");
+}
+int fnx_embed_rows(const uint16_t* emb, const int* tokens, int T, int vocab, int n, float* y, void* st) {
+    if (!emb || !tokens || !y) return fail("embed_rows: null argument");
+    if (T < 1 || vocab < 1 || n < 1) return fail("embed_rows: bad shape");
+    k_embed_rows<<<T, 256, 0, (hipStream_t) st>>>(emb, tokens, vocab, n, y);
+    return launch_status("embed_rows");
+}
+int fnx_q8s_gemv(const fnx_q8s* W, const void* yq, float* out, int out_stride, int T, void* st) {
+    if (!W || !W->q || !W->d || !yq || !out) return fail("q8s_gemv: null argument");
+    if (W->n_out < 1 || W->n_in < 32 || W->n_in % 32) return fail("q8s_gemv: columns in whole 32-value blocks");
+    if (W->n_in % 16 || ((uintptr_t) W->q & 15)) return fail("q8s_gemv: rows of 16-byte pieces");
+    if (T < 1 || T > FNX_MAXT) return fail("q8s_gemv: T out of range");
+    if (out_stride < W->n_out) return fail("q8s_gemv: out_stride smaller than the rows");
+    const size_t lds = (size_t) T * W->n_in + (size_t) T * (W->n_in / 32) * 4;
+    if (lds > 150 * 1024) return fail("q8s_gemv: the window's activations do not fit LDS");
+    static bool attr_set[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64 && !attr_set[dev]) {
+        if (hipFuncSetAttribute((const void*) k_q8s_gemv, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024) != hipSuccess)
+            return fail("q8s_gemv: cannot raise the dynamic LDS limit");
+        attr_set[dev] = true;
+    }
+    const Q8sArgs a{W->q, W->d, W->n_out, W->n_in, (const uint8_t*) yq, out, out_stride, T};
+    const int groups = (W->n_out + Q8S_R - 1) / Q8S_R;
+    const int grid = std::max(1, std::min(2 * cu_count(), (groups + Q8S_WAVES - 1) / Q8S_WAVES));
+    k_q8s_gemv<<<grid, Q8S_WAVES * 64, lds, (hipStream_t) st>>>(a);
+    return launch_status("q8s_gemv");
+}
+int fnx_attn_prep_append(float* qg, float* k, const float* v, const float* q_norm, const float* k_norm, uint16_t* kc, uint16_t* vc, int nq,
+                         int nkv, int T, const int* pos0, int max_ctx, float eps, const fnx_rope* rope, void* st) {
+    if (!qg || !k || !v || !q_norm || !k_norm || !kc || !vc || !pos0 || !rope) return fail("attn_prep_append: null argument");
+    if (nq < 1 || nkv < 1 || nq % nkv || T < 1 || T > FNX_MAXT || max_ctx < 1) return fail("attn_prep_append: bad shape");
+    RopeDev r;
+    for (int pair = 0; pair < AT_NROT / 2; ++pair) {   // rope.hpp:33-39
+        const float fe = powf(rope->base, -2.0f * (float) pair / (float) AT_NROT);
+        float f = fe;
+        if (rope->scaled) {
+            const float y = ((float) pair - rope->c_low) / fmaxf(0.001f, rope->c_high - rope->c_low);
+            const float ramp = 1.0f - fminf(1.0f, fmaxf(0.0f, y));
+            f = fe * (ramp + (1.0f - ramp) * rope->inv_scale);
+        }
+        r.freq[pair] = f;
+    }
+    r.mscale = rope->mscale;
+    k_attn_prep_append<<<dim3(nq + 2 * nkv, T), AT_HD, 0, (hipStream_t) st>>>(qg, k, v, q_norm, k_norm, kc, vc, nq, nkv, pos0, max_ctx, eps, r);
+    return launch_status("attn_prep_append");
+}
+size_t fnx_attn_scratch_floats(int nq, int T) { return (size_t) T * nq * AT_SPLITS * (AT_HD + 2); }
+int fnx_attn(const float* qg, const uint16_t* kc, const uint16_t* vc, float* out, int nq, int nkv, const int* pos0, int T, float* scratch,
+             void* st) {
+    if (!qg || !kc || !vc || !out || !pos0 || !scratch) return fail("attn: null argument");
+    if (nq < 1 || nkv < 1 || nq % nkv || nq / nkv > AT_MAXQ || T < 1 || T > FNX_MAXT) return fail("attn: bad shape");
+    float* acc = scratch;
+    AttPart* mz = reinterpret_cast<AttPart*>(scratch + (size_t) T * nq * AT_SPLITS * AT_HD);
+    k_attn_part<<<dim3(AT_SPLITS, T, nkv), AT_HD, 0, (hipStream_t) st>>>(qg, kc, vc, acc, mz, nq, nkv, pos0);
+    k_attn_combine<<<dim3(nq, T), AT_HD, 0, (hipStream_t) st>>>(qg, acc, mz, out, nq);
+    return launch_status("attn");
+}
+static int dec_ws_check(const fnx_dec_ws* ws, const char* who) {
+    if (!ws->x || !ws->xn || !ws->qg || !ws->k || !ws->v || !ws->att || !ws->o || !ws->attn_scratch || !ws->xq || !ws->hidden || !ws->logits ||
+        !ws->best_v || !ws->best_i || !ws->keys || !ws->err)
+        return fail(std::string(who) + ": incomplete workspace");
+    return 0;
+}
+// x (ws->x) through one layer, in place
+static int dec_layer(const fnx_decoder* D, const fnx_dec_layer* L, int T, const int* pos0, const fnx_dec_ws* ws, void* st) {
+    const int n = D->n, nq = D->nq, nkv = D->nkv;
+    if (fnx_rms_norm_rows(ws->x, L->attn_norm, ws->xn, T, n, D->eps, st)) return 1;
+    if (fnx_quantize_q8_1(ws->xn, ws->xq, n, T, st)) return 1;
+    if (fnx_q8s_gemv(&L->wq, ws->xq, ws->qg, nq * 2 * AT_HD, T, st)) return 1;
+    if (fnx_q8s_gemv(&L->wk, ws->xq, ws->k, nkv * AT_HD, T, st)) return 1;
+    if (fnx_q8s_gemv(&L->wv, ws->xq, ws->v, nkv * AT_HD, T, st)) return 1;
+    if (fnx_attn_prep_append(ws->qg, ws->k, ws->v, L->q_norm, L->k_norm, L->kc, L->vc, nq, nkv, T, pos0, D->max_ctx, D->eps, &D->rope, st)) return 1;
+    if (fnx_attn(ws->qg, L->kc, L->vc, ws->att, nq, nkv, pos0, T, ws->attn_scratch, st)) return 1;
+    if (fnx_quantize_q8_1(ws->att, ws->xq, nq * AT_HD, T, st)) return 1;
+    if (fnx_q8s_gemv(&L->wo, ws->xq, ws->o, n, T, st)) return 1;
+    if (fnx_add_rows(ws->x, ws->o, ws->x, (size_t) T * n, st)) return 1;
+    if (fnx_rms_norm_rows(ws->x, L->ffn_norm, ws->xn, T, n, D->eps, st)) return 1;
+    if (fnx_moe_verify_layer(&L->moe, ws->xn, T, ws->o, &ws->moe, st)) return 1;
+    return fnx_add_rows(ws->x, ws->o, ws->x, (size_t) T * n, st);
+}
+static int dec_shape_check(const fnx_decoder* D, int T, const char* who) {
+    if (D->n < 256 || D->n % 256 || D->nq < 1 || D->nkv < 1 || D->nq % D->nkv || D->nq / D->nkv > AT_MAXQ || D->vocab < 1 || D->max_ctx < 1)
+        return fail(std::string(who) + ": bad model shape");
+    if (T < 1 || T > FNX_MAXT) return fail(std::string(who) + ": T out of range");
+    return 0;
+}
+static int dec_head(const fnx_decoder* D, const float* norm, const fnx_q8s* head, int T, const fnx_dec_ws* ws, void* st) {
+    if (fnx_rms_norm_rows(ws->x, norm, ws->xn, T, D->n, D->eps, st)) return 1;
+    if (fnx_quantize_q8_1(ws->xn, ws->xq, D->n, T, st)) return 1;
+    if (fnx_q8s_gemv(head, ws->xq, ws->logits, D->vocab, T, st)) return 1;
+    return fnx_argmax(ws->logits, D->vocab, T, 0, ws->best_v, ws->best_i, ws->keys, ws->err, st);
+}
+int fnx_decoder_verify(const fnx_decoder* D, const int* tokens, int T, const int* pos0, const fnx_dec_ws* ws, void* st) {
+    if (!D || !tokens || !pos0 || !ws || !D->layers || !D->out_norm || !D->emb) return fail("decoder_verify: null argument");
+    if (dec_shape_check(D, T, "decoder_verify") || dec_ws_check(ws, "decoder_verify")) return 1;
+    if (fnx_embed_rows(D->emb, tokens, T, D->vocab, D->n, ws->x, st)) return 1;
+    for (int l = 0; l < D->nlayers; ++l)
+        if (dec_layer(D, &D->layers[l], T, pos0, ws, st)) return 1;
+    if (hipMemcpyAsync(ws->hidden, ws->x, (size_t) T * D->n * sizeof(float), hipMemcpyDeviceToDevice, (hipStream_t) st) != hipSuccess)
+        return fail("decoder_verify: copy of the hidden rows failed");
+    return dec_head(D, D->out_norm, &D->head, T, ws, st);
+}
+int fnx_mtp_draft(const fnx_decoder* D, const fnx_mtp* M, const float* src, const int* tokens, int T, const int* pos0, const fnx_dec_ws* ws,
+                  void* st) {
+    if (!D || !M || !src || !tokens || !pos0 || !ws || !M->norm_emb || !M->norm_hid || !M->out_norm || !D->emb) return fail("mtp_draft: null argument");
+    if (dec_shape_check(D, T, "mtp_draft") || dec_ws_check(ws, "mtp_draft")) return 1;
+    const int n = D->n;
+    // R = fc_hid(rms(src)) + fc_emb(rms(emb))
+    if (fnx_rms_norm_rows(src, M->norm_hid, ws->xn, T, n, D->eps, st)) return 1;
+    if (fnx_quantize_q8_1(ws->xn, ws->xq, n, T, st)) return 1;
+    if (fnx_q8s_gemv(&M->fc_hid, ws->xq, ws->x, n, T, st)) return 1;
+    if (fnx_embed_rows(D->emb, tokens, T, D->vocab, n, ws->o, st)) return 1;
+    if (fnx_rms_norm_rows(ws->o, M->norm_emb, ws->xn, T, n, D->eps, st)) return 1;
+    if (fnx_quantize_q8_1(ws->xn, ws->xq, n, T, st)) return 1;
+    if (fnx_q8s_gemv(&M->fc_emb, ws->xq, ws->o, n, T, st)) return 1;
+    if (fnx_add_rows(ws->x, ws->o, ws->x, (size_t) T * n, st)) return 1;
+    if (dec_layer(D, &M->layer, T, pos0, ws, st)) return 1;
+    if (hipMemcpyAsync(ws->hidden, ws->x, (size_t) T * n * sizeof(float), hipMemcpyDeviceToDevice, (hipStream_t) st) != hipSuccess)
+        return fail("mtp_draft: copy of the hidden rows failed");
+    return dec_head(D, M->out_norm, &M->head, T, ws, st);
 }
 
 }  // extern "C"

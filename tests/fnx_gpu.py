@@ -248,6 +248,130 @@ class Dev:
         return out.cpu().numpy()
 
 
+    # ---- around the MoE half
+    def rms_norm_rows(self, x, w, eps):
+        dx, dw_ = self.up(x.astype(np.float32)), self.up(w.astype(np.float32))
+        y = self.zeros(x.shape, self.torch.float32)
+        self.ok(self.lib.fnx_rms_norm_rows(dx.data_ptr(), dw_.data_ptr(), y.data_ptr(), x.shape[0], x.shape[1], eps, self.st()))
+        self.sync()
+        return y.cpu().numpy()
+
+    def q8s_gemv(self, q, d, yq, T):
+        rows, cols = q.shape
+        dq, dd, dy = self.up(q), self.up(d), self.up(yq)
+        out = self.zeros((T, rows), self.torch.float32)
+        W = self.pkg.Q8S(dq.data_ptr(), dd.data_ptr(), rows, cols)
+        self.ok(self.lib.fnx_q8s_gemv(C.byref(W), dy.data_ptr(), out.data_ptr(), rows, T, self.st()))
+        self.sync()
+        return out.cpu().numpy()
+
+    def attn_prep_append(self, qg, k, v, qn, kn, kc, vc, nq, nkv, pos0, eps, rope):
+        t = self.torch
+        T = qg.shape[0]
+        dq, dk, dv = self.up(qg.astype(np.float32)), self.up(k.astype(np.float32)), self.up(v.astype(np.float32))
+        dqn, dkn, dkc, dvc = self.up(qn), self.up(kn), self.up(kc), self.up(vc)
+        dp = self.up(np.array([pos0], dtype=np.int32))
+        r = self.pkg.Rope(*rope)
+        self.ok(self.lib.fnx_attn_prep_append(dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dqn.data_ptr(), dkn.data_ptr(), dkc.data_ptr(),
+                                              dvc.data_ptr(), nq, nkv, T, dp.data_ptr(), kc.shape[0], eps, C.byref(r), self.st()))
+        self.sync()
+        return dq.cpu().numpy(), dk.cpu().numpy(), dkc.cpu().numpy(), dvc.cpu().numpy()
+
+    def attn(self, qg, kc, vc, nq, nkv, pos0):
+        t = self.torch
+        T = qg.shape[0]
+        dq, dkc, dvc = self.up(qg.astype(np.float32)), self.up(kc), self.up(vc)
+        dp = self.up(np.array([pos0], dtype=np.int32))
+        out = self.zeros((T, nq, 256), t.float32)
+        scratch = self.zeros(self.lib.fnx_attn_scratch_floats(nq, T), t.float32)
+        self.ok(self.lib.fnx_attn(dq.data_ptr(), dkc.data_ptr(), dvc.data_ptr(), out.data_ptr(), nq, nkv, dp.data_ptr(), T, scratch.data_ptr(),
+                                  self.st()))
+        self.sync()
+        return out.cpu().numpy()
+
+
+class DecoderDev:
+    """tiny_decoder.TinyDecoder on the device: weights, caches, workspace; verify / draft through the C ABI"""
+
+    def __init__(self, dev, model, packed=True):
+        t = dev.torch
+        pkg = dev.pkg
+        c = model.cfg
+        self.dev, self.m, self.c = dev, model, c
+        self.keep = []
+        n, nq, nkv, ff, nexp, topk = c["n"], c["nq"], c["nkv"], c["ff"], c["nexp"], c["topk"]
+
+        def up(a):
+            d = dev.up(a)
+            self.keep.append(d)
+            return d
+
+        def q8s(tq, rows, cols):
+            return pkg.Q8S(up(tq[0]).data_ptr(), up(tq[1]).data_ptr(), rows, cols)
+
+        def lay(L):
+            ws = [up(L[k]) for k in ("gu", "down", "sh_gu", "sh_down")]
+            if packed:
+                for w in ws:
+                    dev.ok(dev.lib.fnx_iq3s_repack(w.data_ptr(), w.data_ptr(), w.numel() // 110 * 256, dev.st()))
+            moe = pkg.MoeLayer(n, ff, nexp, topk, up(L["router"]).data_ptr(), 0, pkg.dw(ws[0], n, 2 * ff, packed=packed),
+                               2 * ff * (n // 256) * 110, pkg.dw(ws[1], ff, n, packed=packed), n * (ff // 256) * 110,
+                               pkg.dw(ws[2], n, 2 * ff, packed=packed), pkg.dw(ws[3], ff, n, packed=packed))
+            kc, vc = dev.zeros((c["max_ctx"], nkv, 256), t.float16), dev.zeros((c["max_ctx"], nkv, 256), t.float16)
+            self.keep.extend([kc, vc])
+            return pkg.DecLayer(up(L["attn_norm"]).data_ptr(), up(L["q_norm"]).data_ptr(), up(L["k_norm"]).data_ptr(), up(L["ffn_norm"]).data_ptr(),
+                                q8s(L["wq"], nq * 512, n), q8s(L["wk"], nkv * 256, n), q8s(L["wv"], nkv * 256, n), q8s(L["wo"], n, nq * 256), moe,
+                                kc.data_ptr(), vc.data_ptr()), (kc, vc)
+
+        self.layer_arr = (pkg.DecLayer * c["nlayers"])()
+        self.caches = []
+        for i, L in enumerate(model.layers):
+            self.layer_arr[i], kv = lay(L)
+            self.caches.append(kv)
+        self.D = pkg.Decoder(n, nq, nkv, c["nlayers"], c["vocab"], c["max_ctx"], c["eps"], pkg.Rope(*model.rope),
+                             C.cast(self.layer_arr, C.c_void_p), up(model.out_norm).data_ptr(), q8s(model.head, c["vocab"], n),
+                             up(model.emb).data_ptr())
+        ml, self.mtp_cache = lay(model.mtp["layer"])
+        self.M = pkg.Mtp(up(model.mtp["norm_emb"]).data_ptr(), up(model.mtp["norm_hid"]).data_ptr(), up(model.mtp["out_norm"]).data_ptr(),
+                         q8s(model.mtp["fc_emb"], n, n), q8s(model.mtp["fc_hid"], n, n), q8s(model.mtp["head"], c["vocab"], n), ml)
+        T, P = 16, 16 * topk
+        z = dev.zeros
+        self.b = dict(x=z((T, n), t.float32), xn=z((T, n), t.float32), qg=z((T, nq * 512), t.float32), k=z((T, nkv * 256), t.float32),
+                      v=z((T, nkv * 256), t.float32), att=z((T, nq * 256), t.float32), o=z((T, n), t.float32),
+                      attn_scratch=z(dev.lib.fnx_attn_scratch_floats(nq, T), t.float32), xq=z(T * (max(n, nq * 256) // 32) * 36, t.uint8),
+                      hidden=z((T, n), t.float32), logits=z((T, c["vocab"]), t.float32), best_v=z(T, t.float32), best_i=z(T, t.int32),
+                      keys=z(16, t.int64), err=z(1, t.int32))
+        self.mb = dict(xq=z(T * (n // 32) * 36, t.uint8), logits=z((T, nexp + 1), t.float32), topi=z((T, topk), t.int32),
+                       topw=z((T, topk), t.float32), jobs_gu=z((P + 1) * 136, t.uint8), jobs_dn=z((P + 1) * 136, t.uint8), njobs=z(2, t.int32),
+                       gu=z((P + T, 2 * ff), t.float32), part=z((P + T, n), t.float32))
+        moe_ws = pkg.MoeWs(*(self.mb[k].data_ptr() for k in ("xq", "logits", "topi", "topw", "jobs_gu", "jobs_dn", "njobs", "gu", "part")))
+        self.ws = pkg.DecWs(*[self.b[k].data_ptr() for k in ("x", "xn", "qg", "k", "v", "att", "o", "attn_scratch", "xq", "hidden", "logits",
+                                                             "best_v", "best_i", "keys", "err")], moe_ws)
+        self.pos = dev.zeros(1, t.int32)
+
+    def _result(self, T):
+        return dict(hidden=self.b["hidden"].cpu().numpy()[:T], logits=self.b["logits"].cpu().numpy()[:T], best=self.b["best_i"].cpu().numpy()[:T],
+                    err=int(self.b["err"].item()))
+
+    def verify(self, tokens, pos0):
+        dev = self.dev
+        tok = dev.up(np.asarray(tokens, dtype=np.int32))
+        self.pos.fill_(pos0)
+        dev.ok(dev.lib.fnx_decoder_verify(C.byref(self.D), tok.data_ptr(), len(tokens), self.pos.data_ptr(), C.byref(self.ws), dev.st()))
+        dev.sync()
+        return self._result(len(tokens))
+
+    def draft(self, src, tokens, pos0):
+        dev = self.dev
+        tok = dev.up(np.asarray(tokens, dtype=np.int32))
+        dsrc = dev.up(np.ascontiguousarray(src, dtype=np.float32))
+        self.pos.fill_(pos0)
+        dev.ok(dev.lib.fnx_mtp_draft(C.byref(self.D), C.byref(self.M), dsrc.data_ptr(), tok.data_ptr(), len(tokens), self.pos.data_ptr(),
+                                     C.byref(self.ws), dev.st()))
+        dev.sync()
+        return self._result(len(tokens))
+
+
 class PfLayerDev:
     """One MoE layer's weights plus a chunk workspace, for fnx_moe_prefill_layer."""
 

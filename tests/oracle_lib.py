@@ -67,6 +67,11 @@ def load():
         "fnx_o_moe_mma": (None, [vp, sz, i, i, vp, i, i, vp, i, vp, i]),
         "fnx_o_swiglu_h16": (None, [vp, i, i, vp]),
         "fnx_o_moe_prefill_layer": (None, [vp, vp, i, i, vp, vp, vp, vp, vp, i]),
+        "fnx_o_rms_norm_rows": (None, [vp, vp, vp, i, i, f]),
+        "fnx_o_quantize_q8_0_split": (None, [vp, i, i, vp, vp]),
+        "fnx_o_q8s_gemv": (None, [vp, vp, i, i, vp, vp, i, i]),
+        "fnx_o_attn_prep_append": (None, [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, f, vp]),
+        "fnx_o_attn": (None, [vp, vp, vp, vp, i, i, i, i, i]),
         "fnx_o_rng_init": (None, [vp, C.c_ulonglong]),
         "fnx_o_rng_next": (C.c_uint, [vp]),
         "fnx_o_threads": (i, []),

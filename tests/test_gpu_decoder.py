@@ -1,0 +1,158 @@
+"""Parity of the norm / dense / attention operators, the reduced decoder's verify window, the draft layer and whole
+speculative rounds (BASELINE config 4 at test sizes) with the CPU oracle, through the C ABI.
+
+Bar: bit-exact for the dense Q8_0 mat-vec (the summation order is shared with the oracle), for argmax picks, drafts,
+accepted lengths and emitted tokens; relative L2 <= 1e-3 for float rows (norms and attention sum in another order and
+use the device's rsqrt / exp / sincos)."""
+import numpy as np
+import pytest
+
+import fnx_gpu
+import oracle_lib as ol
+import tiny_decoder as td
+
+pytestmark = pytest.mark.gpu
+REL_L2 = 1e-3
+ROPE = (1e7, 0, 0.0, 0.0, 1.0, 1.0)
+YARN = (1e4, 1, 4.0, 20.0, 0.25, float(1.0 + 0.1 * np.log(4.0)))
+
+
+def rel_l2(a, b):
+    return float(np.linalg.norm(a.astype(np.float64) - b.astype(np.float64)) / max(np.linalg.norm(b.astype(np.float64)), 1e-30))
+
+
+@pytest.fixture(scope="module")
+def dev():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    return fnx_gpu.Dev()
+
+
+def test_rms_norm_rows(dev, oracle):
+    rng = np.random.default_rng(801)
+    x, w = rng.standard_normal((16, 2048)).astype(np.float32) * 3, rng.standard_normal(2048).astype(np.float32)
+    want = np.zeros_like(x)
+    oracle.lib.fnx_o_rms_norm_rows(ol.ptr(x), ol.ptr(w), ol.ptr(want), 16, 2048, 1e-6)
+    err = float(np.abs(dev.rms_norm_rows(x, w, 1e-6) - want).max())
+    assert err <= 3e-6 * float(np.abs(want).max()), err
+
+
+@pytest.mark.parametrize("rows,cols,T", [(37, 1024, 3), (1000, 2048, 16), (2048, 4096, 16), (513, 256, 5), (8192, 2048, 1)])
+def test_q8s_gemv_bit_exact(dev, oracle, rows, cols, T):
+    print(f"case q8s_gemv rows={rows} cols={cols} T={T}", flush=True)
+    rng = np.random.default_rng(810 + rows)
+    w = (rng.standard_normal((rows, cols)) * 0.05).astype(np.float32)
+    q, d = np.zeros((rows, cols), dtype=np.int8), np.zeros((rows, cols // 32), dtype=np.uint16)
+    oracle.lib.fnx_o_quantize_q8_0_split(ol.ptr(w), rows, cols, ol.ptr(q), ol.ptr(d))
+    x = rng.standard_normal((T, cols)).astype(np.float32)
+    yq = oracle.quantize_q8_1(x)
+    want = np.zeros((T, rows), dtype=np.float32)
+    oracle.lib.fnx_o_q8s_gemv(ol.ptr(q), ol.ptr(d), rows, cols, ol.ptr(yq), ol.ptr(want), rows, T)
+    got = dev.q8s_gemv(q, d, yq, T)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert rel_l2(got, x.astype(np.float64) @ w.astype(np.float64).T) < 2e-2   # and it is the product it claims to be
+
+
+@pytest.mark.parametrize("rope", [ROPE, YARN])
+@pytest.mark.parametrize("nq,nkv,T,pos0", [(4, 2, 3, 5), (16, 2, 16, 32000), (8, 1, 1, 0)])
+def test_attn_prep_append(dev, oracle, nq, nkv, T, pos0, rope):
+    print(f"case attn_prep nq={nq} nkv={nkv} T={T} pos0={pos0} scaled={rope[1]}", flush=True)
+    rng = np.random.default_rng(820 + nq + T)
+    qg = rng.standard_normal((T, nq, 512)).astype(np.float32)
+    k, v = rng.standard_normal((T, nkv, 256)).astype(np.float32), rng.standard_normal((T, nkv, 256)).astype(np.float32)
+    qn, kn = (1 + 0.1 * rng.standard_normal(256)).astype(np.float32), (1 + 0.1 * rng.standard_normal(256)).astype(np.float32)
+    ctx = pos0 + T + 2
+    kc0 = rng.integers(0, 1000, (ctx, nkv, 256)).astype(np.uint16)
+    vc0 = rng.integers(0, 1000, (ctx, nkv, 256)).astype(np.uint16)
+    kc, vc, q2, k2 = kc0.copy(), vc0.copy(), qg.copy(), k.copy()
+    import ctypes as C
+    r = td.RopeO(*rope)
+    oracle.lib.fnx_o_attn_prep_append(ol.ptr(q2), ol.ptr(k2), ol.ptr(v), ol.ptr(qn), ol.ptr(kn), ol.ptr(kc), ol.ptr(vc), nq, nkv, 256, 64, T, pos0,
+                                      1e-6, C.cast(C.pointer(r), C.c_void_p))
+    gq, gk, gkc, gvc = dev.attn_prep_append(qg, k, v, qn, kn, kc0, vc0, nq, nkv, pos0, 1e-6, rope)
+    # the angles are the same floats on both sides (the frequencies come from the host); sin, cos and rsqrt differ in the last bits
+    dq, dk = float(np.abs(gq.reshape(q2.shape) - q2).max()), float(np.abs(gk.reshape(k2.shape) - k2).max())
+    assert dq <= 2e-5 and dk <= 2e-5, (dq, dk)
+    assert np.array_equal(gvc, vc), "v is only rounded to f16"
+    dkc = float(np.abs(gkc.view(np.float16).astype(np.float32) - kc.view(np.float16).astype(np.float32)).max())
+    assert dkc <= 4e-3, dkc   # one f16 step at magnitude 4
+    assert np.array_equal(gkc[:pos0], kc0[:pos0]) and np.array_equal(gkc[pos0 + T:], kc0[pos0 + T:]), "only the window's rows are written"
+
+
+@pytest.mark.parametrize("nq,nkv,T,pos0", [(4, 2, 3, 37), (16, 2, 16, 3000), (16, 2, 16, 0), (8, 1, 5, 511), (2, 2, 1, 64)])
+def test_attn_matches_oracle(dev, oracle, nq, nkv, T, pos0):
+    print(f"case attn nq={nq} nkv={nkv} T={T} pos0={pos0}", flush=True)
+    rng = np.random.default_rng(830 + nq + pos0)
+    qg = rng.standard_normal((T, nq, 512)).astype(np.float32)
+    kc = rng.standard_normal((pos0 + T, nkv, 256)).astype(np.float16)
+    vc = rng.standard_normal((pos0 + T, nkv, 256)).astype(np.float16)
+    want = np.zeros((T, nq, 256), dtype=np.float32)
+    oracle.lib.fnx_o_attn(ol.ptr(qg), ol.ptr(kc), ol.ptr(vc), ol.ptr(want), nq, nkv, 256, T, pos0)
+    got = dev.attn(qg, kc, vc, nq, nkv, pos0)
+    assert rel_l2(got, want) <= REL_L2
+    assert rel_l2(got, want) <= 1e-5
+
+
+@pytest.fixture(scope="module")
+def model(oracle):
+    return td.TinyDecoder(oracle, seed=11)
+
+
+def test_decoder_verify_and_draft(dev, oracle, model):
+    o, d = td.OracleSession(model), fnx_gpu.DecoderDev(dev, model)
+    pos = 0
+    for toks in ([3, 1, 4, 1, 5, 9, 2, 6, 5, 3, 5, 8, 9, 7, 9, 3], [2, 7, 18], [281]):
+        print(f"case decoder_verify T={len(toks)} pos={pos}", flush=True)
+        a, b = o.verify(toks, pos), d.verify(toks, pos)
+        assert b["err"] == 0
+        assert np.array_equal(a["best"], b["best"])
+        assert rel_l2(b["hidden"], a["hidden"]) <= REL_L2 and rel_l2(b["logits"], a["logits"]) <= REL_L2
+        nxt = toks[1:] + [int(a["best"][-1])]
+        da, db = o.draft(a["hidden"], nxt, pos), d.draft(a["hidden"], nxt, pos)
+        assert np.array_equal(da["best"], db["best"])
+        assert rel_l2(db["hidden"], da["hidden"]) <= REL_L2 and rel_l2(db["logits"], da["logits"]) <= REL_L2
+        pos += len(toks)
+    for (ka, va), (kb, vb) in zip(o.caches + [o.mtp_cache], d.caches + [d.mtp_cache]):
+        kb, vb = kb.cpu().numpy().view(np.uint16), vb.cpu().numpy().view(np.uint16)
+        assert rel_l2(kb.view(np.float16)[:pos], ka.view(np.float16)[:pos]) <= REL_L2
+        assert rel_l2(vb.view(np.float16)[:pos], va.view(np.float16)[:pos]) <= REL_L2
+
+
+def test_speculative_rounds_emit_the_greedy_tokens(dev, oracle, model):
+    # a prompt with repeats (so prompt lookup fires) decoded three ways: device speculative, oracle speculative, device plain greedy
+    rng = np.random.default_rng(12)
+    base = [int(t) for t in rng.integers(0, 1000, 12)]
+    prompt = base + base[:7] + [int(t) for t in rng.integers(0, 1000, 3)] + base[2:6]
+
+    def lookup_dev(ctx, lk, d1):
+        return dev.lookup(np.asarray(ctx, dtype=np.int32), lk, d1)
+
+    def lookup_cpu(ctx, lk, d1):
+        return oracle.lookup_drafts(np.asarray(ctx, dtype=np.int32), lk, d1)
+
+    out_d, rounds_d = td.spec_generate(fnx_gpu.DecoderDev(dev, model), lookup_dev, lambda r, o: dev.accept(r, o), prompt, 40)
+    out_o, rounds_o = td.spec_generate(td.OracleSession(model), lookup_cpu, lambda r, o: oracle.accept_greedy(r, o), prompt, 40)
+    out_g, rounds_g = td.spec_generate(fnx_gpu.DecoderDev(dev, model), lookup_dev, lambda r, o: dev.accept(r, o), prompt, 40, speculate=False)
+    print("rounds", rounds_d, flush=True)
+    assert out_d == out_o, "device and oracle emit the same tokens"
+    assert rounds_d == rounds_o, "and take the same drafts and accepted lengths every round"
+    assert out_d == out_g, "speculation does not change the greedy output (fnx_run.cpp:1198-1238)"
+    # drafts from outside: the true continuation with 30% of the tokens corrupted, up to 15 a round. Several rows stand
+    # per round, rejected rows' cache cells are overwritten by the next window, and the output is still the greedy one
+    crng = np.random.default_rng(13)
+
+    def forced(m, d1):
+        k = int(crng.integers(1, 16))
+        return [t if crng.random() > 0.3 else int(crng.integers(0, 1000)) for t in out_g[m:m + k]]
+
+    crng_o = np.random.default_rng(13)
+
+    def forced_o(m, d1):
+        k = int(crng_o.integers(1, 16))
+        return [t if crng_o.random() > 0.3 else int(crng_o.integers(0, 1000)) for t in out_g[m:m + k]]
+
+    out_f, rounds_f = td.spec_generate(fnx_gpu.DecoderDev(dev, model), lookup_dev, lambda r, o: dev.accept(r, o), prompt, 40, forced=forced)
+    out_fo, rounds_fo = td.spec_generate(td.OracleSession(model), lookup_cpu, lambda r, o: oracle.accept_greedy(r, o), prompt, 40, forced=forced_o)
+    print("forced rounds", rounds_f, flush=True)
+    assert out_f == out_g and out_fo == out_g and rounds_f == rounds_fo
+    assert len(rounds_f) < len(rounds_g) and max(u for _, u in rounds_f) > 2

@@ -1,0 +1,188 @@
+"""A reduced decoder with random weights (BASELINE config 4's shape at test sizes), held as numpy arrays, and its two
+renderings: the oracle's C structs (host pointers) and the device library's C structs (device pointers)."""
+import ctypes as C
+
+import numpy as np
+
+import oracle_lib as ol
+from fnx_gpu import random_iq3s
+
+HD = 256
+
+
+class Q8sO(C.Structure):
+    _fields_ = [("q", C.c_void_p), ("d", C.c_void_p), ("n_out", C.c_int), ("n_in", C.c_int)]
+
+
+class RopeO(C.Structure):
+    _fields_ = [("base", C.c_float), ("scaled", C.c_int), ("c_low", C.c_float), ("c_high", C.c_float), ("inv_scale", C.c_float),
+                ("mscale", C.c_float)]
+
+
+class DecLayerO(C.Structure):
+    _fields_ = [("attn_norm", C.c_void_p), ("q_norm", C.c_void_p), ("k_norm", C.c_void_p), ("ffn_norm", C.c_void_p), ("wq", Q8sO), ("wk", Q8sO),
+                ("wv", Q8sO), ("wo", Q8sO), ("moe", ol.MoeLayer), ("kc", C.c_void_p), ("vc", C.c_void_p)]
+
+
+class DecoderO(C.Structure):
+    _fields_ = [("n", C.c_int), ("nq", C.c_int), ("nkv", C.c_int), ("nlayers", C.c_int), ("vocab", C.c_int), ("max_ctx", C.c_int),
+                ("eps", C.c_float), ("rope", RopeO), ("layers", C.c_void_p), ("out_norm", C.c_void_p), ("head", Q8sO), ("emb", C.c_void_p)]
+
+
+class MtpO(C.Structure):
+    _fields_ = [("norm_emb", C.c_void_p), ("norm_hid", C.c_void_p), ("out_norm", C.c_void_p), ("fc_emb", Q8sO), ("fc_hid", Q8sO), ("head", Q8sO),
+                ("layer", DecLayerO)]
+
+
+def _q8s(rng, oracle, rows, cols, scale):
+    w = (rng.standard_normal((rows, cols)) * scale).astype(np.float32)
+    q = np.zeros((rows, cols), dtype=np.int8)
+    d = np.zeros((rows, cols // 32), dtype=np.uint16)
+    oracle.lib.fnx_o_quantize_q8_0_split(ol.ptr(w), rows, cols, ol.ptr(q), ol.ptr(d))
+    return q, d
+
+
+class TinyDecoder:
+    def __init__(self, oracle, seed=1, n=256, nq=4, nkv=2, nlayers=2, vocab=1000, max_ctx=128, nexp=8, topk=2, ff=256, rope_scaled=False):
+        rng = np.random.default_rng(seed)
+        self.oracle = oracle
+        self.cfg = dict(n=n, nq=nq, nkv=nkv, nlayers=nlayers, vocab=vocab, max_ctx=max_ctx, nexp=nexp, topk=topk, ff=ff, eps=1e-6)
+        self.rope = (1e7, 0, 0.0, 0.0, 1.0, 1.0) if not rope_scaled else (1e4, 1, 4.0, 20.0, 0.25, 1.0 + 0.1 * np.log(4.0))
+        nb = lambda rows, cols: rows * cols // 256
+        sw = 1.0 / np.sqrt(n)
+
+        def layer():
+            L = dict(attn_norm=(1 + 0.1 * rng.standard_normal(n)).astype(np.float32), q_norm=(1 + 0.1 * rng.standard_normal(HD)).astype(np.float32),
+                     k_norm=(1 + 0.1 * rng.standard_normal(HD)).astype(np.float32), ffn_norm=(1 + 0.1 * rng.standard_normal(n)).astype(np.float32),
+                     wq=_q8s(rng, oracle, nq * 2 * HD, n, sw), wk=_q8s(rng, oracle, nkv * HD, n, sw), wv=_q8s(rng, oracle, nkv * HD, n, sw),
+                     wo=_q8s(rng, oracle, n, nq * HD, 1.0 / np.sqrt(nq * HD)),
+                     router=(rng.standard_normal((nexp + 1, n)) * 0.05).astype(np.float32),
+                     gu=random_iq3s(rng, nexp * nb(2 * ff, n), dmax=4e-4), down=random_iq3s(rng, nexp * nb(n, ff), dmax=4e-4),
+                     sh_gu=random_iq3s(rng, nb(2 * ff, n), dmax=4e-4), sh_down=random_iq3s(rng, nb(n, ff), dmax=4e-4))
+            return L
+
+        self.layers = [layer() for _ in range(nlayers)]
+        self.out_norm = (1 + 0.1 * rng.standard_normal(n)).astype(np.float32)
+        self.head = _q8s(rng, oracle, vocab, n, sw)
+        self.emb = rng.standard_normal((vocab, n)).astype(np.float16)
+        self.mtp = dict(norm_emb=(1 + 0.1 * rng.standard_normal(n)).astype(np.float32), norm_hid=(1 + 0.1 * rng.standard_normal(n)).astype(np.float32),
+                        out_norm=(1 + 0.1 * rng.standard_normal(n)).astype(np.float32), fc_emb=_q8s(rng, oracle, n, n, sw),
+                        fc_hid=_q8s(rng, oracle, n, n, sw), head=_q8s(rng, oracle, vocab, n, sw), layer=layer())
+
+    # ---- the oracle's rendering: host arrays; the caches are numpy arrays kept here
+    def oracle_structs(self):
+        c = self.cfg
+        keep = []
+
+        def q8s(t, rows, cols):
+            return Q8sO(ol.ptr(t[0]), ol.ptr(t[1]), rows, cols)
+
+        def lay(L):
+            kc = np.zeros((c["max_ctx"], c["nkv"], HD), dtype=np.uint16)
+            vc = np.zeros_like(kc)
+            keep.extend([kc, vc])
+            moe = ol.MoeLayer(c["n"], c["ff"], c["nexp"], c["topk"], ol.ptr(L["router"]), ol.ptr(L["gu"]), ol.ptr(L["down"]), ol.ptr(L["sh_gu"]),
+                              ol.ptr(L["sh_down"]))
+            return DecLayerO(ol.ptr(L["attn_norm"]), ol.ptr(L["q_norm"]), ol.ptr(L["k_norm"]), ol.ptr(L["ffn_norm"]),
+                             q8s(L["wq"], c["nq"] * 2 * HD, c["n"]), q8s(L["wk"], c["nkv"] * HD, c["n"]), q8s(L["wv"], c["nkv"] * HD, c["n"]),
+                             q8s(L["wo"], c["n"], c["nq"] * HD), moe, ol.ptr(kc), ol.ptr(vc)), (kc, vc)
+
+        arr = (DecLayerO * c["nlayers"])()
+        caches = []
+        for i, L in enumerate(self.layers):
+            arr[i], kv = lay(L)
+            caches.append(kv)
+        D = DecoderO(c["n"], c["nq"], c["nkv"], c["nlayers"], c["vocab"], c["max_ctx"], c["eps"], RopeO(*self.rope), C.cast(arr, C.c_void_p),
+                     ol.ptr(self.out_norm), q8s(self.head, c["vocab"], c["n"]), ol.ptr(self.emb))
+        ml, mkv = lay(self.mtp["layer"])
+        M = MtpO(ol.ptr(self.mtp["norm_emb"]), ol.ptr(self.mtp["norm_hid"]), ol.ptr(self.mtp["out_norm"]), q8s(self.mtp["fc_emb"], c["n"], c["n"]),
+                 q8s(self.mtp["fc_hid"], c["n"], c["n"]), q8s(self.mtp["head"], c["vocab"], c["n"]), ml)
+        keep.extend([arr, D, M])
+        return D, M, caches, mkv, keep
+
+
+class OracleSession:
+    """verify / draft on the CPU oracle, with the caches kept between calls"""
+
+    def __init__(self, model):
+        self.m = model
+        self.D, self.M, self.caches, self.mtp_cache, self._keep = model.oracle_structs()
+        lib = model.oracle.lib
+        lib.fnx_o_decoder_verify.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]
+        lib.fnx_o_decoder_verify.restype = None
+        lib.fnx_o_mtp_draft.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]
+        lib.fnx_o_mtp_draft.restype = None
+
+    def verify(self, tokens, pos0):
+        c = self.m.cfg
+        tok = np.ascontiguousarray(tokens, dtype=np.int32)
+        T = len(tok)
+        hidden = np.zeros((T, c["n"]), dtype=np.float32)
+        logits = np.zeros((T, c["vocab"]), dtype=np.float32)
+        best = np.zeros(T, dtype=np.int32)
+        self.m.oracle.lib.fnx_o_decoder_verify(C.byref(self.D), ol.ptr(tok), T, pos0, ol.ptr(hidden), ol.ptr(logits), ol.ptr(best), 8)
+        return dict(hidden=hidden, logits=logits, best=best)
+
+    def draft(self, src, tokens, pos0):
+        c = self.m.cfg
+        tok = np.ascontiguousarray(tokens, dtype=np.int32)
+        src = np.ascontiguousarray(src, dtype=np.float32)
+        T = len(tok)
+        hidden = np.zeros((T, c["n"]), dtype=np.float32)
+        logits = np.zeros((T, c["vocab"]), dtype=np.float32)
+        best = np.zeros(T, dtype=np.int32)
+        self.m.oracle.lib.fnx_o_mtp_draft(C.byref(self.D), C.byref(self.M), ol.ptr(src), ol.ptr(tok), T, pos0, ol.ptr(hidden), ol.ptr(logits),
+                                          ol.ptr(best), 8)
+        return dict(hidden=hidden, logits=logits, best=best)
+
+
+def spec_generate(sess, lookup, accept, prompt, max_new, K=4, lk=15, speculate=True, forced=None):
+    """The greedy decode round of session.cpp:530-679 over a session with verify(tokens, pos0) / draft(src, tokens, pos0):
+    verify [x] + drafts -> accept -> commit -> draft d1 from the kept rows -> prompt lookup, else an MTP chain of K.
+    The prompt is read first (windows of up to 16 rows; the draft layer reads the same rows shifted by one, as the
+    reference's prompt pass keeps its cells current). Returns the emitted tokens and per-round statistics."""
+    ctx = list(prompt)
+    pos = 0
+    hidden_last = None
+    # read the prompt: rows 0 .. len-2 (the last token is the first window's row)
+    body = ctx[:-1]
+    for i in range(0, len(body), 16):
+        w = body[i:i + 16]
+        r = sess.verify(w, pos)
+        nxt = ctx[i + 1:i + 1 + len(w)]
+        sess.draft(r["hidden"], nxt, pos)
+        pos += len(w)
+    x, drafts, out, rounds = ctx[-1], [], [], []
+    while len(out) < max_new:
+        rows = [x] + drafts[:15]
+        p = pos
+        r = sess.verify(rows, p)
+        o = [int(t) for t in r["best"]]
+        n = accept(rows, o)
+        used = min(n, max_new - len(out))
+        out.extend(o[:used])
+        pos += used
+        ctx.extend(o[:used])
+        x = o[used - 1]
+        rounds.append((len(rows) - 1, used))
+        if len(out) >= max_new:
+            break
+        d = sess.draft(r["hidden"][:used], o[:used], p)
+        d1 = int(d["best"][used - 1])
+        if not speculate:
+            drafts = []
+            continue
+        if forced is not None:
+            drafts = [int(t) for t in forced(len(out), d1)]
+            continue
+        drafts, _ = lookup(ctx, lk, d1)
+        drafts = [int(t) for t in drafts]
+        if drafts:
+            continue
+        drafts = [d1]
+        src = d["hidden"][used - 1:used]
+        for j in range(1, K):
+            d = sess.draft(src, [drafts[-1]], p + used - 1 + j)
+            drafts.append(int(d["best"][0]))
+            src = d["hidden"][:1]
+    return out, rounds
