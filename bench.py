@@ -41,14 +41,22 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain device copy of 256 MiB, the known-size kernel that scales the FETCH_SIZE / WRITE_SIZE counters")
     ap.add_argument("--raw-layout", action="store_true", help="leave the weights as raw ggml blocks (skip the load-time re-laying)")
-    ap.add_argument("--workload", choices=["verify", "prefill"], default="verify",
-                    help="verify: BASELINE config 2 (the headline metric, the default); prefill: config 5, one MoE layer over prompt chunks of 512 rows")
+    ap.add_argument("--workload", choices=["verify", "prefill", "decoder", "head", "gemv"], default="verify",
+                    help="verify: BASELINE config 2 (the headline metric, the default); prefill: config 5, one MoE layer over prompt chunks of 512 "
+                         "rows; decoder: config 4, a verify step of the reduced decoder plus the draft layer; head: config 3, argmax + prompt "
+                         "lookup + acceptance; gemv: config 1, one IQ3_S matrix over T = 1 and 16 rows")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
         sys.exit(2)
     if args.workload == "prefill":
         return prefill_main(args)
+    if args.workload == "decoder":
+        return decoder_main(args)
+    if args.workload == "head":
+        return head_main(args)
+    if args.workload == "gemv":
+        return gemv_main(args)
 
     import numpy as np
     import torch
@@ -201,6 +209,268 @@ def main():
                      "window_launch_us": {n_: round(float(v) * 1e3, 2) for n_, v in zip(names, per_launch)}},
         "cpu_baseline": cpu,
     }
+    print(json.dumps(line))
+
+
+def _rand_iq3s(torch, g, nblocks):
+    b = torch.randint(0, 256, (nblocks, IQ3S_BLOCK), dtype=torch.uint8, device="cuda", generator=g)
+    d = (torch.rand(nblocks, device="cuda", generator=g) * 3e-4 + 1e-5).to(torch.float16)
+    b[:, 0:2] = d.view(torch.uint8).reshape(nblocks, 2)
+    return b.reshape(-1)
+
+
+def gemv_main(args):
+    """BASELINE config 1: one 4096 x 2048 IQ3_S matrix (3,604,480 bytes) over T = 1 and T = 16 q8_1 rows, cycling through
+    1,024 distinct matrices (3.7 GB) so that every launch reads its weights from HBM."""
+    import numpy as np
+    import torch
+    import fnx_gpu
+    dev = fnx_gpu.Dev()
+    pkg, lib = dev.pkg, dev.lib
+    g = torch.Generator(device="cuda")
+    g.manual_seed(11)
+    ROWS, COLS, NM = 4096, 2048, 1024
+    mbytes = ROWS * COLS // 256 * IQ3S_BLOCK
+    w = _rand_iq3s(torch, g, NM * ROWS * COLS // 256)
+    dev.ok(lib.fnx_iq3s_repack(w.data_ptr(), w.data_ptr(), w.numel() // IQ3S_BLOCK * 256, dev.st()))
+    st = dev.st()
+    res = {}
+    for T in (1, 16):
+        x = torch.randn((T, COLS), device="cuda", generator=g)
+        xq = torch.zeros(T * (COLS // 32) * 36, dtype=torch.uint8, device="cuda")
+        dev.ok(lib.fnx_quantize_q8_1(x.data_ptr(), xq.data_ptr(), COLS, T, st))
+        jobs = np.zeros(1, dtype=fnx_gpu.JOB_DTYPE)
+        jobs["n"][0] = T
+        jobs["y"][0, :T] = np.arange(T)
+        jobs["out"][0, :T] = np.arange(T)
+        dj = dev.up(jobs.view(np.uint8).reshape(-1))
+        out = torch.zeros((T, ROWS), device="cuda")
+        Ws = [pkg.dw(w.data_ptr() + i * mbytes, COLS, ROWS, packed=True) for i in range(NM)]
+        steps = max(args.steps, 512)
+        for i in range(64):
+            dev.ok(lib.fnx_mmvq(C.byref(Ws[i % NM]), 0, dj.data_ptr(), None, 1, xq.data_ptr(), out.data_ptr(), ROWS, st))
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for i in range(steps):
+            dev.ok(lib.fnx_mmvq(C.byref(Ws[(64 + i) % NM]), 0, dj.data_ptr(), None, 1, xq.data_ptr(), out.data_ptr(), ROWS, st))
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) / steps * 1e3
+        nbytes = mbytes + T * (COLS // 32) * 36 + T * ROWS * 4
+        res[T] = {"us_per_launch": us, "algorithmic_bytes": nbytes, "GBps": nbytes / (us * 1e-6) / 1e9, "hbm_frac": nbytes / (us * 1e-6) / HBM_PEAK}
+    line = {"metric": "IQ3_S GEMV achieved HBM GB/s (config 1: 4096 x 2048, T = 1 and 16)", "value": res[16]["GBps"], "unit": "GB/s", "n_gpus": 1,
+            "steps": max(args.steps, 512), "warmup": 64, "ms_per_step": res[16]["us_per_launch"] / 1e3, "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "int8 x IQ3_S (i32 dot, f32 accumulate)", "data": "synthetic",
+            "config": {"workload": "config 1: one IQ3_S 4096 x 2048 mat-vec, 1,024 distinct matrices cycled", "T1": res[1], "T16": res[16]},
+            "roofline": {"bound": "hbm", "kernel": "k_iq3s_jobs (unit64, one job)", "achieved": res[16]["GBps"], "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                         "frac": res[16]["hbm_frac"], "traffic": None, "note": "back-to-back launches of 3.6 MB each: dominated by the launch, not by HBM"},
+            "cpu_baseline": None}
+    print(json.dumps(line))
+
+
+def head_main(args):
+    """BASELINE config 3: argmax over 16 x 151,936 f32 logits (forced to the draft on 70% of the rows), prompt lookup
+    over a 38,862-token context with 200 copied spans, greedy acceptance; device forms, one stream."""
+    import numpy as np
+    import torch
+    import fnx_gpu
+    import oracle_lib
+    dev = fnx_gpu.Dev()
+    lib = dev.lib
+    oracle = oracle_lib.Oracle()
+    rng = np.random.default_rng(3)
+    V, NCTX, R = 151936, 38862, 16
+    ctx = rng.integers(0, V, NCTX).astype(np.int32)
+    for _ in range(200):
+        ln, src, dst = int(rng.integers(8, 65)), int(rng.integers(0, NCTX - 200)), int(rng.integers(200, NCTX - 64))
+        ctx[dst:dst + ln] = ctx[src:src + ln]
+    # the context ends inside a copied span, so the lookup finds a run
+    ctx[-12:] = ctx[1000:1012]
+    g = torch.Generator(device="cuda")
+    g.manual_seed(5)
+    NL = 8
+    logits = [torch.randn((R, V), device="cuda", generator=g) for _ in range(NL)]
+    d1 = int(ctx[1012])
+    drafts, match = oracle.lookup_drafts(ctx, 15, d1)
+    rows = np.concatenate([[int(ctx[-1])], drafts]).astype(np.int32)[:R]
+    keep = rng.random(R) < 0.7
+    for lg in logits:   # row j's argmax is the next row's token on 70% of the rows
+        for j in range(len(rows) - 1):
+            if keep[j]:
+                lg[j, int(rows[j + 1])] = lg[j].max() + 1.0
+    t = torch
+    dctx, dd1 = dev.up(ctx), dev.up(np.array([d1], dtype=np.int32))
+    dout, dn, dm = dev.zeros(15, t.int32), dev.zeros(1, t.int32), dev.zeros(1, t.int32)
+    drows = dev.up(np.pad(rows, (0, R - len(rows))))
+    bv, bi, keys, err, nacc = dev.zeros(R, t.float32), dev.zeros(R, t.int32), dev.zeros(16, t.int64), dev.zeros(1, t.int32), dev.zeros(1, t.int32)
+    st = dev.st()
+
+    def timed(fn, n):
+        for i in range(20):
+            fn(i)
+        e0, e1 = t.cuda.Event(enable_timing=True), t.cuda.Event(enable_timing=True)
+        t.cuda.synchronize()
+        e0.record()
+        for i in range(n):
+            fn(i)
+        e1.record()
+        t.cuda.synchronize()
+        return e0.elapsed_time(e1) / n * 1e3
+
+    n = max(args.steps, 200)
+    us_arg = timed(lambda i: dev.ok(lib.fnx_argmax(logits[i % NL].data_ptr(), V, R, 0, bv.data_ptr(), bi.data_ptr(), keys.data_ptr(), err.data_ptr(), st)), n)
+    us_lk = timed(lambda i: dev.ok(lib.fnx_lookup_drafts_dev(dctx.data_ptr(), NCTX, 3, 15, dd1.data_ptr(), dout.data_ptr(), dn.data_ptr(), dm.data_ptr(), st)), n)
+    us_acc = timed(lambda i: dev.ok(lib.fnx_accept_greedy_dev(drows.data_ptr(), bi.data_ptr(), len(rows), nacc.data_ptr(), st)), n)
+
+    def all3(i):
+        dev.ok(lib.fnx_argmax(logits[i % NL].data_ptr(), V, R, 0, bv.data_ptr(), bi.data_ptr(), keys.data_ptr(), err.data_ptr(), st))
+        dev.ok(lib.fnx_accept_greedy_dev(drows.data_ptr(), bi.data_ptr(), len(rows), nacc.data_ptr(), st))
+        dev.ok(lib.fnx_lookup_drafts_dev(dctx.data_ptr(), NCTX, 3, 15, dd1.data_ptr(), dout.data_ptr(), dn.data_ptr(), dm.data_ptr(), st))
+    us_all = timed(all3, n)
+    # parity on this exact input
+    all3(0)
+    t.cuda.synchronize()
+    o = bi.cpu().numpy()
+    _, want_i, _ = oracle.argmax(logits[0].cpu().numpy())
+    same = bool(np.array_equal(o, want_i)) and int(nacc.item()) == oracle.accept_greedy(rows, o[:len(rows)]) and \
+        list(dout.cpu().numpy()[:int(dn.item())]) == list(drafts) and int(dm.item()) == match
+    c0 = time.perf_counter()
+    reps = 0
+    while time.perf_counter() - c0 < min(args.cpu_seconds, 5.0) or reps < 2:
+        oracle.argmax(logits[0].cpu().numpy()) if reps == 0 else None
+        oracle.lookup_drafts(ctx, 15, d1)
+        oracle.accept_greedy(rows, o[:len(rows)])
+        reps += 1
+    cpu_us = (time.perf_counter() - c0) / reps * 1e6
+    arg_bytes = R * V * 4
+    line = {"metric": "verify head: argmax + acceptance + prompt lookup per round (config 3)", "value": 1e6 / us_all, "unit": "rounds/s", "n_gpus": 1,
+            "steps": n, "warmup": 20, "ms_per_step": us_all / 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32 compare / int32",
+            "data": "synthetic",
+            "config": {"workload": "config 3: logits 16 x 151,936 f32, context 38,862 int32 with 200 copied spans, key 3, up to 15 drafts",
+                       "argmax_us": us_arg, "lookup_us": us_lk, "accept_us": us_acc, "drafts": int(len(drafts)), "accepted": int(nacc.item()),
+                       "identical_to_oracle": same},
+            "roofline": {"bound": "hbm", "kernel": "k_argmax", "achieved": arg_bytes / (us_arg * 1e-6) / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                         "frac": arg_bytes / (us_arg * 1e-6) / HBM_PEAK, "traffic": None, "algorithmic_bytes": arg_bytes,
+                         "note": "two launches of about 4 us fixed cost each; the scan itself is 1.2 us at peak"},
+            "cpu_baseline": {"value": 1e6 / cpu_us, "unit": "rounds/s", "cores": 1, "kind": "port",
+                             "sample": f"{reps} rounds of lookup + acceptance on the oracle (the argmax scan once)"}}
+    print(json.dumps(line))
+
+
+def decoder_main(args):
+    """BASELINE config 4: a verify step of the reduced decoder (4 layers of GQA attention, 16 q / 2 kv heads of 256, f16
+    cache at 32,768 positions, and the config-2 MoE block) over 1 + 15 rows, the output head over 151,936 tokens, greedy
+    acceptance, then the draft layer over the same rows. Random weights; a step's weights are cold (two model copies
+    alternate is too large for the head, so the ~3.7 GB a step reads already exceeds the 256 MB cache many times)."""
+    import numpy as np
+    import torch
+    import fnx_gpu
+    dev = fnx_gpu.Dev()
+    pkg, lib, t = dev.pkg, dev.lib, torch
+    g = torch.Generator(device="cuda")
+    g.manual_seed(44)
+    NQ, NKV, HD, NL, V, CTX, R = 16, 2, 256, 4, 151936, 32768, 16
+    keep = []
+
+    def q8s(rows, cols):
+        q = torch.randint(-127, 128, (rows, cols), dtype=torch.int8, device="cuda", generator=g)
+        d = (torch.rand((rows, cols // 32), device="cuda", generator=g) * (2.0 / 127 / np.sqrt(cols)) + 1e-6).to(torch.float16)
+        keep.extend([q, d])
+        return pkg.Q8S(q.data_ptr(), d.data_ptr(), rows, cols)
+
+    def vec(n):
+        v = 1 + 0.1 * torch.randn(n, device="cuda", generator=g)
+        keep.append(v)
+        return v.data_ptr()
+
+    def layer():
+        ws = [_rand_iq3s(t, g, NEXP * 2 * FF * N // 256), _rand_iq3s(t, g, NEXP * N * FF // 256), _rand_iq3s(t, g, 2 * FF * N // 256),
+              _rand_iq3s(t, g, N * FF // 256)]
+        for w in ws:
+            dev.ok(lib.fnx_iq3s_repack(w.data_ptr(), w.data_ptr(), w.numel() // IQ3S_BLOCK * 256, dev.st()))
+        router = (torch.randn((NEXP + 1, N), device="cuda", generator=g) * 0.02).contiguous()
+        kc = (torch.randn((CTX, NKV, HD), device="cuda", generator=g)).to(torch.float16)
+        vc = (torch.randn((CTX, NKV, HD), device="cuda", generator=g)).to(torch.float16)
+        keep.extend(ws + [router, kc, vc])
+        moe = pkg.MoeLayer(N, FF, NEXP, TOPK, router.data_ptr(), 0, pkg.dw(ws[0], N, 2 * FF, packed=True), GU_BYTES, pkg.dw(ws[1], FF, N, packed=True),
+                           DN_BYTES, pkg.dw(ws[2], N, 2 * FF, packed=True), pkg.dw(ws[3], FF, N, packed=True))
+        return pkg.DecLayer(vec(N), vec(HD), vec(HD), vec(N), q8s(NQ * 2 * HD, N), q8s(NKV * HD, N), q8s(NKV * HD, N), q8s(N, NQ * HD), moe,
+                            kc.data_ptr(), vc.data_ptr())
+
+    arr = (pkg.DecLayer * NL)()
+    for i in range(NL):
+        arr[i] = layer()
+    emb = torch.randn((V, N), device="cuda", generator=g).to(torch.float16)
+    D = pkg.Decoder(N, NQ, NKV, NL, V, CTX, 1e-6, pkg.Rope(1e7, 0, 0.0, 0.0, 1.0, 1.0), C.cast(arr, C.c_void_p), vec(N), q8s(V, N), emb.data_ptr())
+    M = pkg.Mtp(vec(N), vec(N), vec(N), q8s(N, N), q8s(N, N), q8s(V, N), layer())
+    P = R * TOPK
+    z = dev.zeros
+    b = dict(x=z((R, N), t.float32), xn=z((R, N), t.float32), qg=z((R, NQ * 512), t.float32), k=z((R, NKV * 256), t.float32),
+             v=z((R, NKV * 256), t.float32), att=z((R, NQ * 256), t.float32), o=z((R, N), t.float32),
+             attn_scratch=z(lib.fnx_attn_scratch_floats(NQ, R, CTX), t.float32), xq=z(R * (NQ * 256 // 32) * 36, t.uint8), hidden=z((R, N), t.float32),
+             logits=z((R, V), t.float32), best_v=z(R, t.float32), best_i=z(R, t.int32), keys=z(16, t.int64), err=z(1, t.int32))
+    mb = dict(xq=z(R * (N // 32) * 36, t.uint8), logits=z((R, NEXP + 1), t.float32), topi=z((R, TOPK), t.int32), topw=z((R, TOPK), t.float32),
+              jobs_gu=z((P + 1) * 136, t.uint8), jobs_dn=z((P + 1) * 136, t.uint8), njobs=z(2, t.int32), gu=z((P + R, 2 * FF), t.float32),
+              part=z((P + R, N), t.float32))
+    moe_ws = pkg.MoeWs(*(mb[k].data_ptr() for k in ("xq", "logits", "topi", "topw", "jobs_gu", "jobs_dn", "njobs", "gu", "part")))
+    ws = pkg.DecWs(*[b[k].data_ptr() for k in ("x", "xn", "qg", "k", "v", "att", "o", "attn_scratch", "xq", "hidden", "logits", "best_v", "best_i",
+                                                 "keys", "err")], moe_ws)
+    pos = torch.full((1,), CTX - R, dtype=torch.int32, device="cuda")
+    toks = torch.randint(0, V, (8, R), dtype=torch.int32, device="cuda", generator=g)
+    nacc = z(1, t.int32)
+    st = dev.st()
+
+    def step(i):
+        tk = toks[i % 8]
+        dev.ok(lib.fnx_decoder_verify(C.byref(D), tk.data_ptr(), R, pos.data_ptr(), C.byref(ws), st))
+        dev.ok(lib.fnx_accept_greedy_dev(tk.data_ptr(), ws.best_i, R, nacc.data_ptr(), st))
+        dev.ok(lib.fnx_mtp_draft(C.byref(D), C.byref(M), ws.hidden, tk.data_ptr(), R, pos.data_ptr(), C.byref(ws), st))
+
+    steps, warmup = min(args.steps, 50), min(args.warmup, 5)
+    for i in range(warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step(warmup + i)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    # the attention on its own (the K/V scan of one layer): events on the launch stream
+    evs = []
+    L0 = arr[0]
+    for i in range(23):
+        e0, e1 = t.cuda.Event(enable_timing=True), t.cuda.Event(enable_timing=True)
+        e0.record()
+        dev.ok(lib.fnx_attn(ws.qg, arr[i % NL].kc, arr[i % NL].vc, ws.att, NQ, NKV, pos.data_ptr(), R, CTX, ws.attn_scratch, st))
+        e1.record()
+        evs.append((e0, e1))
+    hv = []
+    for i in range(13):
+        e0, e1 = t.cuda.Event(enable_timing=True), t.cuda.Event(enable_timing=True)
+        e0.record()
+        dev.ok(lib.fnx_q8s_gemv(C.byref(D.head if i % 2 else M.head), ws.xq, ws.logits, V, R, st))
+        e1.record()
+        hv.append((e0, e1))
+    torch.cuda.synchronize()
+    attn_ms = float(np.mean([a.elapsed_time(c) for a, c in evs[3:]]))
+    head_ms = float(np.mean([a.elapsed_time(c) for a, c in hv[3:]]))
+    kv_bytes = 2 * CTX * NKV * HD * 2
+    head_bytes = V * N + V * (N // 32) * 2
+    dense_bytes = (NQ * 2 * HD * N + 2 * NKV * HD * N + N * NQ * HD) * 34 // 32
+    moe_bytes = 139.2 * (GU_BYTES + DN_BYTES) + (GU_BYTES + DN_BYTES) + ROUTER_BYTES
+    step_bytes = (NL + 1) * (kv_bytes + dense_bytes + moe_bytes) + 2 * head_bytes + 2 * N * N * 34 // 32
+    line = {"metric": "verify steps/sec of the reduced decoder + draft layer (config 4)", "value": steps / dt, "unit": "steps/s", "n_gpus": 1,
+            "steps": steps, "warmup": warmup, "ms_per_step": dt / steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "int8 dot (IQ3_S, Q8_0) + f32 attention on an f16 cache", "data": "synthetic",
+            "config": {"workload": "config 4: 4 layers (GQA 16q/2kv x 256 at 32,768 positions + MoE as config 2) + head 151,936 + acceptance + draft layer, 16 rows",
+                       "step_algorithmic_bytes": step_bytes, "step_hbm_frac": step_bytes / (dt / steps) / HBM_PEAK,
+                       "attention_ms_per_layer": attn_ms, "attention_GBps": kv_bytes / (attn_ms * 1e-3) / 1e9, "head_ms": head_ms,
+                       "head_GBps": head_bytes / (head_ms * 1e-3) / 1e9},
+            "roofline": {"bound": "hbm", "kernel": "k_q8s_gemv (output head 151,936 x 2048)", "achieved": head_bytes / (head_ms * 1e-3) / 1e9,
+                         "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": head_bytes / (head_ms * 1e-3) / HBM_PEAK, "traffic": None, "kernel_ms": head_ms,
+                         "algorithmic_bytes": head_bytes},
+            "cpu_baseline": None}
     print(json.dumps(line))
 
 

@@ -232,20 +232,23 @@ typedef struct fnx_rope {
     float c_low, c_high, inv_scale, mscale;
 } fnx_rope;
 /* kernels.hpp:259  attn_prep_append: q heads (qg [T][nq][q | gate], 2 x 256 each) and k heads RMS-normed with their
- * weights and rotated at positions *pos0 + t, in place; k and v appended to the f16 cache [max_ctx][nkv][256]. */
+ * weights and rotated at positions *pos0 + t, in place; k and v appended to the f16 caches of max_ctx positions (a
+ * multiple of 4): K is [position][nkv][256]; V is this library's own layout [position / 4][nkv][256][position % 4]
+ * (four positions of a dimension together, the matrix-core attention's operand). */
 int fnx_attn_prep_append(float* qg, float* k, const float* v, const float* q_norm, const float* k_norm, uint16_t* kc, uint16_t* vc, int nq,
                          int nkv, int T, const int* pos0, int max_ctx, float eps, const fnx_rope* rope, void* st);
 /* kernels.hpp:238  attn: row t attends positions [0, *pos0 + t]; out [T][nq][256] = softmax(q k / 16) v * sigmoid(gate).
- * scratch: fnx_attn_scratch_floats(nq, T) floats (the splits' partial sums) */
-size_t fnx_attn_scratch_floats(int nq, int T);
-int fnx_attn(const float* qg, const uint16_t* kc, const uint16_t* vc, float* out, int nq, int nkv, const int* pos0, int T, float* scratch,
-             void* st);
+ * On the matrix cores: q and the probabilities enter as two f16 terms each (hi + lo), the cache is f16, sums are fp32. max_ctx: the caches' capacity (the grid
+ * covers it; *pos0 + T <= max_ctx). scratch: fnx_attn_scratch_floats(nq, T, max_ctx) floats (the splits' partial sums) */
+size_t fnx_attn_scratch_floats(int nq, int T, int max_ctx);
+int fnx_attn(const float* qg, const uint16_t* kc, const uint16_t* vc, float* out, int nq, int nkv, const int* pos0, int T, int max_ctx,
+             float* scratch, void* st);
 /* one decoder layer of the reduced model: x += wo . attn(norm(x)); x += moe(norm(x)) */
 typedef struct fnx_dec_layer {
     const float *attn_norm, *q_norm, *k_norm, *ffn_norm;   /* [n], [256], [256], [n] */
     fnx_q8s wq, wk, wv, wo;                                 /* [nq * 512][n], [nkv * 256][n], [nkv * 256][n], [n][nq * 256] */
     fnx_moe_layer moe;
-    uint16_t *kc, *vc;                                      /* this layer's cache: [max_ctx][nkv][256] f16 each */
+    uint16_t *kc, *vc;                                      /* this layer's caches, max_ctx x nkv x 256 f16 each (layouts: attn_prep_append) */
 } fnx_dec_layer;
 typedef struct fnx_decoder {
     int n, nq, nkv, nlayers, vocab, max_ctx;
@@ -259,7 +262,7 @@ typedef struct fnx_decoder {
 /* caller-owned scratch for windows of up to 16 rows */
 typedef struct fnx_dec_ws {
     float *x, *xn, *qg, *k, *v, *att, *o;   /* [T][n], [T][n], [T][nq*512], [T][nkv*256] x2, [T][nq*256], [T][n] */
-    float* attn_scratch;                    /* fnx_attn_scratch_floats(nq, T) */
+    float* attn_scratch;                    /* fnx_attn_scratch_floats(nq, T, max_ctx) */
     void* xq;                               /* q8_1 rows of max(n, nq * 256) values */
     float *hidden, *logits, *best_v;        /* [T][n] (the rows before the output norm), [T][vocab], [T] */
     int* best_i;                            /* [T] */

@@ -115,8 +115,9 @@ EXPORTS = {
     "fnx_q8s_gemv": (C.c_int, [C.POINTER(Q8S), C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
     "fnx_attn_prep_append": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int,
                                        C.c_int, C.c_void_p, C.c_int, C.c_float, C.POINTER(Rope), C.c_void_p]),
-    "fnx_attn_scratch_floats": (C.c_size_t, [C.c_int, C.c_int]),
-    "fnx_attn": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
+    "fnx_attn_scratch_floats": (C.c_size_t, [C.c_int, C.c_int, C.c_int]),
+    "fnx_attn": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p,
+                           C.c_void_p]),
     "fnx_decoder_verify": (C.c_int, [C.POINTER(Decoder), C.c_void_p, C.c_int, C.c_void_p, C.POINTER(DecWs), C.c_void_p]),
     "fnx_mtp_draft": (C.c_int, [C.POINTER(Decoder), C.POINTER(Mtp), C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.POINTER(DecWs), C.c_void_p]),
     "fnx_moe_prefill_layer": (C.c_int, [C.POINTER(MoeLayer), C.c_void_p, C.c_int, C.c_void_p, C.POINTER(PfWs), C.c_void_p]),

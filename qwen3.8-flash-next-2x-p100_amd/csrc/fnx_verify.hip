@@ -996,7 +996,7 @@ int fnx_q8s_gemv(const fnx_q8s* W, const void* yq, float* out, int out_stride, i
 int fnx_attn_prep_append(float* qg, float* k, const float* v, const float* q_norm, const float* k_norm, uint16_t* kc, uint16_t* vc, int nq,
                          int nkv, int T, const int* pos0, int max_ctx, float eps, const fnx_rope* rope, void* st) {
     if (!qg || !k || !v || !q_norm || !k_norm || !kc || !vc || !pos0 || !rope) return fail("attn_prep_append: null argument");
-    if (nq < 1 || nkv < 1 || nq % nkv || T < 1 || T > FNX_MAXT || max_ctx < 1) return fail("attn_prep_append: bad shape");
+    if (nq < 1 || nkv < 1 || nq % nkv || T < 1 || T > FNX_MAXT || max_ctx < 4 || max_ctx % 4) return fail("attn_prep_append: bad shape (the cache holds a multiple of 4 positions)");
     RopeDev r;
     for (int pair = 0; pair < AT_NROT / 2; ++pair) {   // rope.hpp:33-39
         const float fe = powf(rope->base, -2.0f * (float) pair / (float) AT_NROT);
@@ -1012,15 +1012,19 @@ int fnx_attn_prep_append(float* qg, float* k, const float* v, const float* q_nor
     k_attn_prep_append<<<dim3(nq + 2 * nkv, T), AT_HD, 0, (hipStream_t) st>>>(qg, k, v, q_norm, k_norm, kc, vc, nq, nkv, pos0, max_ctx, eps, r);
     return launch_status("attn_prep_append");
 }
-size_t fnx_attn_scratch_floats(int nq, int T) { return (size_t) T * nq * AT_SPLITS * (AT_HD + 2); }
-int fnx_attn(const float* qg, const uint16_t* kc, const uint16_t* vc, float* out, int nq, int nkv, const int* pos0, int T, float* scratch,
-             void* st) {
+// splits for a context of up to max_ctx positions
+static int attn_splits(int max_ctx) { return (max_ctx + AT_SPLIT - 1) / AT_SPLIT; }
+size_t fnx_attn_scratch_floats(int nq, int T, int max_ctx) { return (size_t) T * nq * attn_splits(max_ctx) * (AT_HD + 2); }
+int fnx_attn(const float* qg, const uint16_t* kc, const uint16_t* vc, float* out, int nq, int nkv, const int* pos0, int T, int max_ctx,
+             float* scratch, void* st) {
     if (!qg || !kc || !vc || !out || !pos0 || !scratch) return fail("attn: null argument");
-    if (nq < 1 || nkv < 1 || nq % nkv || nq / nkv > AT_MAXQ || T < 1 || T > FNX_MAXT) return fail("attn: bad shape");
+    if (nq < 1 || nkv < 1 || nq % nkv || nq / nkv > AT_MAXQ || T < 1 || T > FNX_MAXT || max_ctx < 1) return fail("attn: bad shape");
+    // the grid covers the cache's capacity (the position is on the device): splits past the context write empty parts
+    const int nsplit = attn_splits(max_ctx), waves = (T * (nq / nkv) + 15) / 16;
     float* acc = scratch;
-    AttPart* mz = reinterpret_cast<AttPart*>(scratch + (size_t) T * nq * AT_SPLITS * AT_HD);
-    k_attn_part<<<dim3(AT_SPLITS, T, nkv), AT_HD, 0, (hipStream_t) st>>>(qg, kc, vc, acc, mz, nq, nkv, pos0);
-    k_attn_combine<<<dim3(nq, T), AT_HD, 0, (hipStream_t) st>>>(qg, acc, mz, out, nq);
+    AttPart* mz = reinterpret_cast<AttPart*>(scratch + (size_t) T * nq * nsplit * AT_HD);
+    k_attn_part<<<dim3(nsplit, nkv), 64 * waves, 0, (hipStream_t) st>>>(qg, kc, vc, acc, mz, nq, nkv, T, nsplit, pos0);
+    k_attn_combine<<<dim3(nq, T), AT_HD, 0, (hipStream_t) st>>>(qg, acc, mz, out, nq, nsplit);
     return launch_status("attn");
 }
 static int dec_ws_check(const fnx_dec_ws* ws, const char* who) {
@@ -1038,7 +1042,7 @@ static int dec_layer(const fnx_decoder* D, const fnx_dec_layer* L, int T, const 
     if (fnx_q8s_gemv(&L->wk, ws->xq, ws->k, nkv * AT_HD, T, st)) return 1;
     if (fnx_q8s_gemv(&L->wv, ws->xq, ws->v, nkv * AT_HD, T, st)) return 1;
     if (fnx_attn_prep_append(ws->qg, ws->k, ws->v, L->q_norm, L->k_norm, L->kc, L->vc, nq, nkv, T, pos0, D->max_ctx, D->eps, &D->rope, st)) return 1;
-    if (fnx_attn(ws->qg, L->kc, L->vc, ws->att, nq, nkv, pos0, T, ws->attn_scratch, st)) return 1;
+    if (fnx_attn(ws->qg, L->kc, L->vc, ws->att, nq, nkv, pos0, T, D->max_ctx, ws->attn_scratch, st)) return 1;
     if (fnx_quantize_q8_1(ws->att, ws->xq, nq * AT_HD, T, st)) return 1;
     if (fnx_q8s_gemv(&L->wo, ws->xq, ws->o, n, T, st)) return 1;
     if (fnx_add_rows(ws->x, ws->o, ws->x, (size_t) T * n, st)) return 1;

@@ -110,7 +110,8 @@ struct RopeDev {
     float mscale;
 };
 // block (head h, row t), AT_HD threads: q heads normed and rotated in place; k heads normed, rotated and appended; v heads
-// appended. The cache is [position][kv head][AT_HD] f16.
+// appended. The K cache is [position][kv head][AT_HD] f16; the V cache keeps four positions of a dimension together,
+// [position / 4][kv head][AT_HD][position % 4], which is what the matrix-core attention's V operand loads.
 __global__ void __launch_bounds__(AT_HD) k_attn_prep_append(float* __restrict__ qg, float* __restrict__ k, const float* __restrict__ v,
                                                            const float* __restrict__ qn, const float* __restrict__ kn,
                                                            uint16_t* __restrict__ kc, uint16_t* __restrict__ vc, int nq, int nkv,
@@ -148,85 +149,169 @@ __global__ void __launch_bounds__(AT_HD) k_attn_prep_append(float* __restrict__ 
         x = v[((size_t) t * nkv + kh) * AT_HD + i];
     }
     if (p < 0 || p >= max_ctx) return;
-    (is_k ? kc : vc)[((size_t) p * nkv + kh) * AT_HD + i] = float_to_half_bits(x);
+    if (is_k) kc[((size_t) p * nkv + kh) * AT_HD + i] = float_to_half_bits(x);
+    else vc[(((size_t) (p >> 2) * nkv + kh) * AT_HD + i) * 4 + (p & 3)] = float_to_half_bits(x);   // vcache_at(p, nkv, kh, i)
 }
 
-// ---------------------------------------------------------------- attention: split-K decode (kernels.cu:541-643, 786-803)
-// block (split s, row t, kv head): positions [s * len, (s + 1) * len) of [0, pos0 + t] in chunks of 32, for the q heads
-// of that kv head, online softmax; each head's running max, sum and AT_HD accumulators go to scratch, the combine
-// weighs the splits, divides and applies sigmoid(gate).
-constexpr int AT_SPLITS = 16, AT_CH = 32, AT_MAXQ = 8;   // q heads per kv head held by a block
+// ---------------------------------------------------------------- attention: split-K decode on the matrix cores
+// (kernels.cu:541-643, 786-803 give the arithmetic: scores q.k / 16 over positions [0, pos0 + t], online softmax in
+// splits, the splits merged by their maxima, the result times sigmoid(gate).)
+//
+// A window's rows times a kv head's q heads are up to 128 query vectors against the same K/V rows: a dense contraction,
+// so it runs on v_mfma_f32_16x16x32_f16. A block takes (split of AT_SPLIT positions, kv head); wave j of it takes the
+// 16 queries 16 j .. 16 j + 15 (query = row * heads-per-kv + head). Per chunk of 32 positions:
+//   S^T = K Q^T  : A = K rows (lane: position l % 16, the 64 dims of lane group l / 16, 16 bytes a step from the cache),
+//                  B = Q^T (held in registers for the whole split, scaled by 1/16, as two f16 terms hi + lo);
+//                  the accumulator leaves lane (group pg, query q) with positions 4 pg .. 4 pg + 3 of both 16-position
+//                  tiles: the softmax of query q needs only in-lane work and two cross-group shuffles;
+//   O^T += V^T P^T: those eight positions are exactly lane group pg's contraction slots, so P goes from the accumulator
+//                  registers straight into the B operand, and V^T's A operand is two 8-byte loads because the V cache
+//                  keeps four positions of a dimension together ([position / 4][kv head][dim][position % 4]).
+// Nothing passes through LDS. Each (query, split) leaves its maximum, sum and 256 accumulators; k_attn_combine merges.
+constexpr int AT_SPLIT = 512, AT_CH = 32, AT_MAXQ = 8;
 struct AttPart {
     float m, z;
 };
-__global__ void __launch_bounds__(AT_HD) k_attn_part(const float* __restrict__ qg, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
-                                                    float* __restrict__ acc_out, AttPart* __restrict__ mz_out, int nq, int nkv,
-                                                    const int* __restrict__ pos0p) {
-    const int s = blockIdx.x, t = blockIdx.y, kvh = blockIdx.z, i = threadIdx.x;
-    const int qpk = nq / nkv, h0 = kvh * qpk, ctx = *pos0p + t + 1;
-    const int len = ((ctx + AT_SPLITS - 1) / AT_SPLITS + AT_CH - 1) / AT_CH * AT_CH;
-    const int p0 = s * len, p1 = min(ctx, p0 + len);
-    __shared__ float q[AT_MAXQ][AT_HD];
-    __shared__ float kk[AT_CH][AT_HD + 1];
-    __shared__ float e[AT_MAXQ][AT_CH];
-    __shared__ float scale[AT_MAXQ];
-    for (int k = i; k < qpk * AT_HD; k += AT_HD) q[k / AT_HD][k % AT_HD] = qg[((size_t) t * nq + h0 + k / AT_HD) * 2 * AT_HD + k % AT_HD];
-    // thread (head hh, position pp) of a chunk's scores; thread i also owns dimension i of the accumulators
-    const int hh = i >> 5, pp = i & 31;
-    float m = -INFINITY, z = 0.f;
-    float acc[AT_MAXQ];
+typedef _Float16 at_v8h __attribute__((ext_vector_type(8)));
+typedef _Float16 at_v4h __attribute__((ext_vector_type(4)));
+typedef float at_v4f __attribute__((ext_vector_type(4)));
+typedef unsigned at_v4u __attribute__((ext_vector_type(4)));
+typedef unsigned at_v2u __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ size_t vcache_at(int pos, int nkv, int kvh, int d) {   // the V cache's element index
+    return (((size_t) (pos >> 2) * nkv + kvh) * AT_HD + d) * 4 + (pos & 3);
+}
+
+__global__ void __launch_bounds__(512) k_attn_part(const float* __restrict__ qg, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
+                                                  float* __restrict__ acc_out, AttPart* __restrict__ mz_out, int nq, int nkv, int T,
+                                                  int nsplit, const int* __restrict__ pos0p) {
+    typedef __attribute__((address_space(1))) const at_v4u g128;
+    typedef __attribute__((address_space(1))) const at_v2u g64;
+    const int s = blockIdx.x, kvh = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int qpk = nq / nkv, nquery = T * qpk, pos0 = *pos0p;
+    const int ql = lane & 15, pg = lane >> 4;
+    const int qi = wave * 16 + ql;                      // this lane's query (as B column / accumulator column)
+    const bool qlive = qi < nquery;
+    const int qt = qlive ? qi / qpk : 0, qh = kvh * qpk + (qlive ? qi % qpk : 0);
+    const int ctx_q = qlive ? pos0 + qt + 1 : 0;        // positions [0, ctx_q) are this query's
+    const int ctx_max = pos0 + T;                       // the window's last row sees this many
+    const int p0 = s * AT_SPLIT, p1 = min(ctx_max, p0 + AT_SPLIT);
+    // Q^T operands: step ks holds dims 64 pg + 8 ks .. + 7 of query ql, times 1/16 (exact), as two f16 terms hi + lo:
+    // the cache is f16 already, so with q (and below the probabilities) split this way the products carry fp32's
+    // precision, as the reference's f32 arithmetic on the f16 cache does
+    at_v8h Q[8], Ql[8];
+    {
+        const float* qr = qg + ((size_t) qt * nq + qh) * 2 * AT_HD + 64 * pg;
+        const float sc = qlive ? 0.0625f : 0.f;
 #pragma unroll
-    for (int k = 0; k < AT_MAXQ; ++k) acc[k] = 0.f;
-    __syncthreads();
-    for (int c0 = p0; c0 < p1; c0 += AT_CH) {
-        const int np = min(AT_CH, p1 - c0);
-        float vr[AT_CH];
+        for (int ks = 0; ks < 8; ++ks) {
+            const float4 a = *reinterpret_cast<const float4*>(qr + 8 * ks), b = *reinterpret_cast<const float4*>(qr + 8 * ks + 4);
+            const float v[8] = {a.x * sc, a.y * sc, a.z * sc, a.w * sc, b.x * sc, b.y * sc, b.z * sc, b.w * sc};
 #pragma unroll
-        for (int j = 0; j < AT_CH; ++j) {
-            const size_t r = ((size_t) (c0 + min(j, np - 1)) * nkv + kvh) * AT_HD + i;
-            kk[j][i] = j < np ? half_bits_to_float(kc[r]) : 0.f;
-            vr[j] = j < np ? half_bits_to_float(vc[r]) : 0.f;
-        }
-        __syncthreads();
-        if (hh < qpk) {
-            float sacc = 0.f;
-#pragma unroll 8
-            for (int d = 0; d < AT_HD; ++d) sacc = fmaf(q[hh][d], kk[pp][d], sacc);
-            const float sv = pp < np ? sacc * rsqrtf((float) AT_HD) : -INFINITY;
-            const float mn = fmaxf(m, group_max<32>(sv));
-            const float w = sv == -INFINITY ? 0.f : expf(sv - mn);
-            const float sc = m == -INFINITY ? 0.f : expf(m - mn);
-            z = z * sc + group_sum<32>(w);
-            m = mn;
-            e[hh][pp] = w;
-            if (pp == 0) scale[hh] = sc;
-        }
-        __syncthreads();
-#pragma unroll
-        for (int k = 0; k < AT_MAXQ; ++k)
-            if (k < qpk) {
-                float av = acc[k] * scale[k];
-#pragma unroll
-                for (int j = 0; j < AT_CH; ++j) av = fmaf(e[k][j], vr[j], av);
-                acc[k] = av;
+            for (int j = 0; j < 8; ++j) {
+                const _Float16 hi = (_Float16) v[j];
+                Q[ks][j] = hi;
+                Ql[ks][j] = (_Float16) (v[j] - (float) hi);
             }
-        __syncthreads();
+        }
     }
+    at_v4f O[16];
 #pragma unroll
-    for (int k = 0; k < AT_MAXQ; ++k)
-        if (k < qpk) acc_out[(((size_t) t * nq + h0 + k) * AT_SPLITS + s) * AT_HD + i] = acc[k];
-    if (hh < qpk && pp == 0) mz_out[((size_t) t * nq + h0 + hh) * AT_SPLITS + s] = AttPart{m, z};
+    for (int dt = 0; dt < 16; ++dt) O[dt] = at_v4f{0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, z = 0.f;
+    const gbytes kbase = as_global(reinterpret_cast<const uint8_t*>(kc));
+    const gbytes vbase = as_global(reinterpret_cast<const uint8_t*>(vc));
+    for (int c0 = p0; c0 < p1; c0 += AT_CH) {
+        // K rows of the two position tiles (as A: position c0 + 16 tile + ql, dims 64 pg ..): clamped inside the window's rows
+        at_v4f S[2];
+#pragma unroll
+        for (int tile = 0; tile < 2; ++tile) {
+            const int pos = min(c0 + 16 * tile + ql, ctx_max - 1);
+            const gbytes kr = kbase + (((size_t) pos * nkv + kvh) * AT_HD + 64 * pg) * 2;
+            at_v4u kreg[8];
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks) kreg[ks] = *(g128*) (kr + 16 * ks);
+            at_v4f acc = at_v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks) {
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(at_v8h, kreg[ks]), Ql[ks], acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(at_v8h, kreg[ks]), Q[ks], acc, 0, 0, 0);
+            }
+            S[tile] = acc;
+        }
+        // V^T operands for the 16 dim tiles: positions c0 + 4 pg .. + 3 and c0 + 16 + 4 pg .. + 3, dim 16 dt + ql
+        // (clamped to the window's rows; the probabilities of positions past a query's own are zero)
+        const int vb0 = min(c0 + 4 * pg, (ctx_max - 1) & ~3) >> 2, vb1 = min(c0 + 16 + 4 * pg, (ctx_max - 1) & ~3) >> 2;
+        const gbytes v0 = vbase + (((size_t) vb0 * nkv + kvh) * AT_HD + ql) * 8, v1 = vbase + (((size_t) vb1 * nkv + kvh) * AT_HD + ql) * 8;
+        // this lane: query ql, positions c0 + 4 pg + r (tile 0) and c0 + 16 + 4 pg + r (tile 1)
+        float sv[8];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+            const int pos = c0 + 16 * (r >> 2) + 4 * pg + (r & 3);
+            sv[r] = pos < ctx_q && pos < p1 ? S[r >> 2][r & 3] : -INFINITY;
+            mx = fmaxf(mx, sv[r]);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float mn = fmaxf(m, mx);
+        const float sc = m == -INFINITY ? 0.f : __expf(m - mn);
+        float pw[8], ps = 0.f;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+            pw[r] = sv[r] == -INFINITY ? 0.f : __expf(sv[r] - mn);
+            ps += pw[r];
+        }
+        ps += __shfl_xor(ps, 16, 64);
+        ps += __shfl_xor(ps, 32, 64);
+        z = z * sc + ps;
+        m = mn;
+        at_v8h P, Pl;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+            const _Float16 hi = (_Float16) pw[r];
+            P[r] = hi;
+            Pl[r] = (_Float16) (pw[r] - (float) hi);
+        }
+        // positions past the window's rows were never written: whatever their cells hold must not reach the products
+        const bool tail = c0 + AT_CH > ctx_max;
+        unsigned keep0[2] = {~0u, ~0u}, keep1[2] = {~0u, ~0u};
+        if (tail) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (c0 + 4 * pg + j >= ctx_max) keep0[j >> 1] &= (j & 1) ? 0x0000FFFFu : 0xFFFF0000u;
+                if (c0 + 16 + 4 * pg + j >= ctx_max) keep1[j >> 1] &= (j & 1) ? 0x0000FFFFu : 0xFFFF0000u;
+            }
+        }
+#pragma unroll
+        for (int dt = 0; dt < 16; ++dt) {
+            const at_v2u a0 = *(g64*) (v0 + 128 * dt), a1 = *(g64*) (v1 + 128 * dt);
+            const at_v4u a = at_v4u{a0.x & keep0[0], a0.y & keep0[1], a1.x & keep1[0], a1.y & keep1[1]};
+            at_v4f o = O[dt];
+            o.x *= sc;
+            o.y *= sc;
+            o.z *= sc;
+            o.w *= sc;
+            o = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(at_v8h, a), Pl, o, 0, 0, 0);
+            O[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(at_v8h, a), P, o, 0, 0, 0);
+        }
+    }
+    if (!qlive) return;
+    // accumulator lane (dim group pg, query ql): dims 16 dt + 4 pg + r
+    const size_t slot = ((size_t) qt * nq + qh) * nsplit + s;
+#pragma unroll
+    for (int dt = 0; dt < 16; ++dt)
+        *reinterpret_cast<float4*>(acc_out + slot * AT_HD + 16 * dt + 4 * pg) = make_float4(O[dt].x, O[dt].y, O[dt].z, O[dt].w);
+    if (pg == 0) mz_out[slot] = AttPart{m, z};
 }
 __global__ void __launch_bounds__(AT_HD) k_attn_combine(const float* __restrict__ qg, const float* __restrict__ acc_in,
-                                                       const AttPart* __restrict__ mz_in, float* __restrict__ out, int nq) {
+                                                       const AttPart* __restrict__ mz_in, float* __restrict__ out, int nq, int nsplit) {
     const int h = blockIdx.x, t = blockIdx.y, i = threadIdx.x;
-    const size_t base = ((size_t) t * nq + h) * AT_SPLITS;
+    const size_t base = ((size_t) t * nq + h) * nsplit;
     float mx = -INFINITY;
-#pragma unroll
-    for (int s = 0; s < AT_SPLITS; ++s) mx = fmaxf(mx, mz_in[base + s].m);
+    for (int s = 0; s < nsplit; ++s) mx = fmaxf(mx, mz_in[base + s].m);
     float z = 0.f, acc = 0.f;
-#pragma unroll
-    for (int s = 0; s < AT_SPLITS; ++s) {
+    for (int s = 0; s < nsplit; ++s) {
         const AttPart p = mz_in[base + s];
         if (p.m == -INFINITY) continue;
         const float w = expf(p.m - mx);

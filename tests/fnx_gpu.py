@@ -62,6 +62,23 @@ def pack_unit64(raw):
 JOB_DTYPE = np.dtype([("w", "<i4"), ("n", "<i4"), ("y", "<i4", (16,)), ("out", "<i4", (16,))])
 
 
+def v_blocked(vc):
+    """[pos][nkv][256] -> the library's V cache layout [pos / 4][nkv][256][pos % 4] (pos a multiple of 4)"""
+    p, nkv, hd = vc.shape
+    return np.ascontiguousarray(vc.reshape(p // 4, 4, nkv, hd).transpose(0, 2, 3, 1))
+
+
+def v_rows(vb):
+    """the inverse of v_blocked"""
+    b, nkv, hd, _ = vb.shape
+    return np.ascontiguousarray(vb.transpose(0, 3, 1, 2)).reshape(b * 4, nkv, hd)
+
+
+def pad4(a):
+    extra = (-a.shape[0]) % 4
+    return a if not extra else np.concatenate([a, np.zeros((extra,) + a.shape[1:], dtype=a.dtype)])
+
+
 class Dev:
     """numpy in, numpy out, through device memory and the C ABI on the current torch stream"""
 
@@ -269,23 +286,27 @@ class Dev:
         t = self.torch
         T = qg.shape[0]
         dq, dk, dv = self.up(qg.astype(np.float32)), self.up(k.astype(np.float32)), self.up(v.astype(np.float32))
-        dqn, dkn, dkc, dvc = self.up(qn), self.up(kn), self.up(kc), self.up(vc)
+        rows = kc.shape[0]
+        kc, vc = pad4(kc), pad4(vc)
+        dqn, dkn, dkc, dvc = self.up(qn), self.up(kn), self.up(kc), self.up(v_blocked(vc))
         dp = self.up(np.array([pos0], dtype=np.int32))
         r = self.pkg.Rope(*rope)
         self.ok(self.lib.fnx_attn_prep_append(dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dqn.data_ptr(), dkn.data_ptr(), dkc.data_ptr(),
                                               dvc.data_ptr(), nq, nkv, T, dp.data_ptr(), kc.shape[0], eps, C.byref(r), self.st()))
         self.sync()
-        return dq.cpu().numpy(), dk.cpu().numpy(), dkc.cpu().numpy(), dvc.cpu().numpy()
+        return dq.cpu().numpy(), dk.cpu().numpy(), dkc.cpu().numpy()[:rows], v_rows(dvc.cpu().numpy())[:rows]
 
     def attn(self, qg, kc, vc, nq, nkv, pos0):
         t = self.torch
         T = qg.shape[0]
-        dq, dkc, dvc = self.up(qg.astype(np.float32)), self.up(kc), self.up(vc)
+        kc, vc = pad4(kc), pad4(vc)
+        max_ctx = kc.shape[0]
+        dq, dkc, dvc = self.up(qg.astype(np.float32)), self.up(kc), self.up(v_blocked(vc))
         dp = self.up(np.array([pos0], dtype=np.int32))
         out = self.zeros((T, nq, 256), t.float32)
-        scratch = self.zeros(self.lib.fnx_attn_scratch_floats(nq, T), t.float32)
-        self.ok(self.lib.fnx_attn(dq.data_ptr(), dkc.data_ptr(), dvc.data_ptr(), out.data_ptr(), nq, nkv, dp.data_ptr(), T, scratch.data_ptr(),
-                                  self.st()))
+        scratch = self.zeros(self.lib.fnx_attn_scratch_floats(nq, T, max_ctx), t.float32)
+        self.ok(self.lib.fnx_attn(dq.data_ptr(), dkc.data_ptr(), dvc.data_ptr(), out.data_ptr(), nq, nkv, dp.data_ptr(), T, max_ctx,
+                                  scratch.data_ptr(), self.st()))
         self.sync()
         return out.cpu().numpy()
 
@@ -338,7 +359,7 @@ class DecoderDev:
         z = dev.zeros
         self.b = dict(x=z((T, n), t.float32), xn=z((T, n), t.float32), qg=z((T, nq * 512), t.float32), k=z((T, nkv * 256), t.float32),
                       v=z((T, nkv * 256), t.float32), att=z((T, nq * 256), t.float32), o=z((T, n), t.float32),
-                      attn_scratch=z(dev.lib.fnx_attn_scratch_floats(nq, T), t.float32), xq=z(T * (max(n, nq * 256) // 32) * 36, t.uint8),
+                      attn_scratch=z(dev.lib.fnx_attn_scratch_floats(nq, T, c["max_ctx"]), t.float32), xq=z(T * (max(n, nq * 256) // 32) * 36, t.uint8),
                       hidden=z((T, n), t.float32), logits=z((T, c["vocab"]), t.float32), best_v=z(T, t.float32), best_i=z(T, t.int32),
                       keys=z(16, t.int64), err=z(1, t.int32))
         self.mb = dict(xq=z(T * (n // 32) * 36, t.uint8), logits=z((T, nexp + 1), t.float32), topi=z((T, topk), t.int32),
@@ -348,6 +369,15 @@ class DecoderDev:
         self.ws = pkg.DecWs(*[self.b[k].data_ptr() for k in ("x", "xn", "qg", "k", "v", "att", "o", "attn_scratch", "xq", "hidden", "logits",
                                                              "best_v", "best_i", "keys", "err")], moe_ws)
         self.pos = dev.zeros(1, t.int32)
+
+    def caches_numpy(self):
+        """every layer's (K, V) as [pos][nkv][256] uint16 arrays, the draft layer's last"""
+        out = []
+        for kc, vc in self.caches + [self.mtp_cache]:
+            k = kc.cpu().numpy().view(np.uint16)
+            v = vc.cpu().numpy().view(np.uint16).reshape(self.c["max_ctx"] // 4, self.c["nkv"], 256, 4)
+            out.append((k, v_rows(v)))
+        return out
 
     def _result(self, T):
         return dict(hidden=self.b["hidden"].cpu().numpy()[:T], logits=self.b["logits"].cpu().numpy()[:T], best=self.b["best_i"].cpu().numpy()[:T],
