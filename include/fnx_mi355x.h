@@ -223,7 +223,8 @@ typedef struct fnx_q8s {
     const uint16_t* d;
     int n_out, n_in;
 } fnx_q8s;
-/* dense.cuh:79-214 (q8s_gemv): out[t * out_stride + r] = W[r] . y[t] for T <= 16 q8_1 rows */
+/* dense.cuh:79-214 (q8s_gemv): out[t * out_stride + r] = W[r] . y[t] for T <= 16 q8_1 rows; n_in a multiple of 256. The
+ * 32-column blocks are folded in ascending order, acc = fmaf(d_w * d_x, (float) dot, acc) */
 int fnx_q8s_gemv(const fnx_q8s* W, const void* yq, float* out, int out_stride, int T, void* st);
 /* rope.hpp:22-39  the rotary's constants (scaled = 0: plain frequencies base^(-2 i / 64), mscale 1) */
 typedef struct fnx_rope {

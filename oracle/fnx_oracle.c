@@ -769,21 +769,17 @@ void fnx_o_q8s_gemv(const int8_t* q, const uint16_t* d, int rows, int cols, cons
 #pragma omp parallel for schedule(static)
     for (int r = 0; r < rows; ++r)
         for (int t = 0; t < T; ++t) {
-            float lane[64];
-            for (int l = 0; l < 64; ++l) {
-                float a = 0.f;
-                for (int c = 16 * l; c < cols; c += 1024) {
-                    const uint8_t* blk = yq + ((size_t) t * nb + (c >> 5)) * Q8_1_BLOCK;
-                    uint16_t dxh;
-                    memcpy(&dxh, blk, 2);
-                    const int8_t* xs = (const int8_t*) blk + 4 + (c & 16);
-                    int s = 0;
-                    for (int j = 0; j < 16; ++j) s += (int) q[(size_t) r * cols + c + j] * (int) xs[j];
-                    a = fmaf(fnx_o_h2f(d[(size_t) r * nb + (c >> 5)]) * fnx_o_h2f(dxh), (float) s, a);
-                }
-                lane[l] = a;
+            float a = 0.f;
+            for (int b = 0; b < nb; ++b) { /* ascending blocks, one fmaf each: the order is part of the definition */
+                const uint8_t* blk = yq + ((size_t) t * nb + b) * Q8_1_BLOCK;
+                uint16_t dxh;
+                memcpy(&dxh, blk, 2);
+                const int8_t* xs = (const int8_t*) blk + 4;
+                int s = 0;
+                for (int j = 0; j < 32; ++j) s += (int) q[(size_t) r * cols + 32 * b + j] * (int) xs[j];
+                a = fmaf(fnx_o_h2f(d[(size_t) r * nb + b]) * fnx_o_h2f(dxh), (float) s, a);
             }
-            out[(size_t) t * out_stride + r] = butterfly_sum(lane, 64);
+            out[(size_t) t * out_stride + r] = a;
         }
 }
 static float rope_unit_freq(const fnx_o_rope* r, int pair, int nrot) { /* rope.hpp:33-39 */

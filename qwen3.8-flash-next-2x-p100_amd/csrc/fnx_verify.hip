@@ -975,10 +975,10 @@ int fnx_embed_rows(const uint16_t* emb, const int* tokens, int T, int vocab, int
 int fnx_q8s_gemv(const fnx_q8s* W, const void* yq, float* out, int out_stride, int T, void* st) {
     if (!W || !W->q || !W->d || !yq || !out) return fail("q8s_gemv: null argument");
     if (W->n_out < 1 || W->n_in < 32 || W->n_in % 32) return fail("q8s_gemv: columns in whole 32-value blocks");
-    if (W->n_in % 16 || ((uintptr_t) W->q & 15)) return fail("q8s_gemv: rows of 16-byte pieces");
+    if (W->n_in % 256 || ((uintptr_t) W->q & 15) || ((uintptr_t) W->d & 15)) return fail("q8s_gemv: columns in 256s, 16-byte aligned rows");
     if (T < 1 || T > FNX_MAXT) return fail("q8s_gemv: T out of range");
     if (out_stride < W->n_out) return fail("q8s_gemv: out_stride smaller than the rows");
-    const size_t lds = (size_t) T * W->n_in + (size_t) T * (W->n_in / 32) * 4;
+    const size_t lds = (size_t) FNX_MAXT * (W->n_in + Q8S_XPAD) + (size_t) FNX_MAXT * (W->n_in / 32 + 2) * 4;
     if (lds > 150 * 1024) return fail("q8s_gemv: the window's activations do not fit LDS");
     static bool attr_set[64] = {};
     int dev = 0;
@@ -988,8 +988,9 @@ int fnx_q8s_gemv(const fnx_q8s* W, const void* yq, float* out, int out_stride, i
         attr_set[dev] = true;
     }
     const Q8sArgs a{W->q, W->d, W->n_out, W->n_in, (const uint8_t*) yq, out, out_stride, T};
-    const int groups = (W->n_out + Q8S_R - 1) / Q8S_R;
-    const int grid = std::max(1, std::min(2 * cu_count(), (groups + Q8S_WAVES - 1) / Q8S_WAVES));
+    const int tiles = (W->n_out + 15) / 16;
+    static const int per_cu = env_int("FNX_Q8S_BLOCKS_PER_CU", 2, 1, 8);
+    const int grid = std::max(1, std::min(per_cu * cu_count(), (tiles + Q8S_WAVES - 1) / Q8S_WAVES));
     k_q8s_gemv<<<grid, Q8S_WAVES * 64, lds, (hipStream_t) st>>>(a);
     return launch_status("q8s_gemv");
 }

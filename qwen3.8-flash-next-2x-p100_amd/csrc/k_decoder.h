@@ -7,6 +7,7 @@
 namespace fnx {
 
 constexpr int AT_HD = 256, AT_NROT = 64;   // head width and rotated dims (model.hpp:41 of the reference)
+typedef unsigned at_v4u_t __attribute__((ext_vector_type(4)));
 
 // ---------------------------------------------------------------- RMS norm (kernels.cu:2818-2826)
 // y[r] = x[r] / sqrt(mean(x[r]^2) + eps) * w, a block per row
@@ -32,10 +33,16 @@ __global__ void k_embed_rows(const uint16_t* __restrict__ emb, const int* __rest
 }
 
 // ---------------------------------------------------------------- dense Q8_0, split layout (dense.cuh:79-214)
-// int8 values [rows][cols], f16 scales [rows][cols / 32]; activations q8_1. A wave takes Q8S_R rows at a time; lane l takes
-// the 16-column pieces l, l + 64, ... of each row (one 16-byte load), acc = fmaf(d_w * d_x, (float) dot, acc) in that
-// order, then the xor-butterfly: this order is part of the result's definition (the CPU oracle follows it).
-constexpr int Q8S_R = 4, Q8S_WAVES = 4;
+// int8 values [rows][cols], f16 scales [rows][cols / 32]; activations q8_1 (up to 16 rows). The result is defined as
+//   out[t][r] = fold over the 32-column blocks b in ascending order of acc = fmaf(d_w[r][b] * d_x[t][b], (float) dot_b, acc)
+// (dot_b the exact integer dot product of the block): the reference's term (dense.cuh:196-200) in one fixed order, which
+// the CPU oracle follows bit for bit.
+// On the matrix cores: a wave owns 16 weight rows; v_mfma_i32_16x16x32_i8 wants 8 bytes of k from each of 4 lane groups.
+// A lane loads 16 contiguous bytes of its row per 64 columns (group g: bytes 16 g ..), so groups 0-1 hold block 2 j and
+// groups 2-3 block 2 j + 1; each block's dot product is two MFMAs (the lanes' low and high 8 bytes) whose B operand is
+// zero in the other block's groups. The 16 x 16 integer sums then take their scales in 12 VALU ops, against 44 for
+// the same block on the vector ALU, and no cross-lane reduction is left.
+constexpr int Q8S_WAVES = 4, Q8S_XPAD = 16;
 struct Q8sArgs {
     const int8_t* q;
     const uint16_t* d;
@@ -44,61 +51,81 @@ struct Q8sArgs {
     float* out;
     int out_stride, T;
 };
+typedef int q8s_v4i __attribute__((ext_vector_type(4)));
 __global__ void __launch_bounds__(Q8S_WAVES * 64) k_q8s_gemv(const Q8sArgs a) {
-    extern __shared__ __align__(16) uint8_t q8s_lds[];   // [T][cols] int8, then [T][cols / 32] f32 scales
-    const int nb = a.cols >> 5, T = a.T;
+    typedef __attribute__((address_space(1))) const at_v4u_t g128;
+    extern __shared__ __align__(16) uint8_t q8s_lds[];   // [16][cols + pad] int8, then [16][nb + 2] f32 scales
+    const int nb = a.cols >> 5, T = a.T, xld = a.cols + Q8S_XPAD, dld = nb + 2;
     int8_t* xs = reinterpret_cast<int8_t*>(q8s_lds);
-    float* xd = reinterpret_cast<float*>(q8s_lds + (size_t) T * a.cols);
-    for (int i = threadIdx.x; i < T * nb; i += blockDim.x) {
-        const uint8_t* blk = a.yq + (size_t) i * 36;   // row t = i / nb, block i % nb: rows are contiguous
-        xd[i] = half_bits_to_float(load_u16(blk));
-        const uint32_t* src = reinterpret_cast<const uint32_t*>(blk + 4);
-        uint32_t* dst = reinterpret_cast<uint32_t*>(xs + (size_t) i * 32);
+    float* xd = reinterpret_cast<float*>(q8s_lds + (size_t) FNX_MAXT * xld);
+    for (int i = threadIdx.x; i < FNX_MAXT * nb; i += blockDim.x) {
+        const int t = i / nb, b = i - t * nb;
+        uint32_t* dst = reinterpret_cast<uint32_t*>(xs + (size_t) t * xld + 32 * b);
+        if (t < T) {
+            const uint8_t* blk = a.yq + (size_t) i * 36;
+            xd[t * dld + b] = half_bits_to_float(load_u16(blk));
+            const uint32_t* src = reinterpret_cast<const uint32_t*>(blk + 4);
 #pragma unroll
-        for (int k = 0; k < 8; ++k) dst[k] = src[k];
+            for (int k = 0; k < 8; ++k) dst[k] = src[k];
+        } else {   // rows past the window: zeros, so their lanes' products stay finite
+            xd[t * dld + b] = 0.f;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) dst[k] = 0u;
+        }
     }
     __syncthreads();
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int groups = (a.rows + Q8S_R - 1) / Q8S_R;
-    for (int grp = blockIdx.x * Q8S_WAVES + wave; grp < groups; grp += gridDim.x * Q8S_WAVES) {
-        const int row0 = grp * Q8S_R;
-        float acc[Q8S_R][FNX_MAXT];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r16 = lane & 15, g = lane >> 4;
+    const int tiles = (a.rows + 15) / 16, nd = a.cols >> 6;   // double steps of 64 columns
+    const bool lo_groups = g < 2;
+    for (int tile = blockIdx.x * Q8S_WAVES + wave; tile < tiles; tile += gridDim.x * Q8S_WAVES) {
+        const int row0 = tile * 16;
+        const gbytes wrow = as_global(reinterpret_cast<const uint8_t*>(a.q) + (size_t) min(row0 + r16, a.rows - 1) * a.cols + 16 * g);
+        // the scales of the accumulator's rows 4 g .. 4 g + 3
+        const uint16_t* drow[4];
 #pragma unroll
-        for (int r = 0; r < Q8S_R; ++r)
+        for (int r = 0; r < 4; ++r) drow[r] = a.d + (size_t) min(row0 + 4 * g + r, a.rows - 1) * nb;
+        float acc[4] = {0.f, 0.f, 0.f, 0.f};
+        at_v4u_t wn = *(g128*) wrow;
+        // the rows' scales eight blocks (four double steps) at a time, fetched four double steps ahead
+        at_v4u_t dn[4];
 #pragma unroll
-            for (int t = 0; t < FNX_MAXT; ++t) acc[r][t] = 0.f;
-        for (int c = lane * 16; c < a.cols; c += 1024) {
-            int4 w[Q8S_R];
-            float dw[Q8S_R];
+        for (int r = 0; r < 4; ++r) dn[r] = *(g128*) as_global(reinterpret_cast<const uint8_t*>(drow[r]));
+        for (int j4 = 0; j4 < nd; j4 += 4) {
+            at_v4u_t dc[4];
 #pragma unroll
-            for (int r = 0; r < Q8S_R; ++r) {
-                const int row = min(row0 + r, a.rows - 1);
-                w[r] = *reinterpret_cast<const int4*>(a.q + (size_t) row * a.cols + c);
-                dw[r] = half_bits_to_float(a.d[(size_t) row * nb + (c >> 5)]);
+            for (int r = 0; r < 4; ++r) {
+                dc[r] = dn[r];
+                dn[r] = *(g128*) as_global(reinterpret_cast<const uint8_t*>(drow[r] + 2 * min(j4 + 4, nd - 4)));
             }
 #pragma unroll
-            for (int t = 0; t < FNX_MAXT; ++t)
-                if (t < T) {
-                    const int4 x = *reinterpret_cast<const int4*>(xs + (size_t) t * a.cols + c);
-                    const float da = xd[t * nb + (c >> 5)];
+            for (int u = 0; u < 4; ++u) {
+                const int j = j4 + u;
+                const at_v4u_t w = wn;
+                wn = *(g128*) (wrow + 64 * min(j + 1, nd - 1));   // past the end: the last piece again
+                const at_v4u_t x = *reinterpret_cast<const at_v4u_t*>(xs + (size_t) r16 * xld + 64 * j + 16 * g);
+                const float2 dx = *reinterpret_cast<const float2*>(xd + r16 * dld + 2 * j);
+                const long wl = (long) w.x | (long) w.y << 32, wh = (long) w.z | (long) w.w << 32;
+                const long xl = (long) x.x | (long) x.y << 32, xh = (long) x.z | (long) x.w << 32;
+                const long xl0 = lo_groups ? xl : 0, xh0 = lo_groups ? xh : 0, xl1 = lo_groups ? 0 : xl, xh1 = lo_groups ? 0 : xh;
+                q8s_v4i s0 = __builtin_amdgcn_mfma_i32_16x16x32_i8(wl, xl0, q8s_v4i{0, 0, 0, 0}, 0, 0, 0);
+                s0 = __builtin_amdgcn_mfma_i32_16x16x32_i8(wh, xh0, s0, 0, 0, 0);
+                q8s_v4i s1 = __builtin_amdgcn_mfma_i32_16x16x32_i8(wl, xl1, q8s_v4i{0, 0, 0, 0}, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_i32_16x16x32_i8(wh, xh1, s1, 0, 0, 0);
 #pragma unroll
-                    for (int r = 0; r < Q8S_R; ++r) {
-                        int s = __builtin_amdgcn_sdot4(w[r].x, x.x, 0, false);
-                        s = __builtin_amdgcn_sdot4(w[r].y, x.y, s, false);
-                        s = __builtin_amdgcn_sdot4(w[r].z, x.z, s, false);
-                        s = __builtin_amdgcn_sdot4(w[r].w, x.w, s, false);
-                        acc[r][t] = fmaf(dw[r] * da, (float) s, acc[r][t]);
-                    }
+                for (int r = 0; r < 4; ++r) {
+                    const uint32_t dd = dc[r][u];   // blocks 2 j and 2 j + 1
+                    acc[r] = fmaf(half_bits_to_float(dd & 0xFFFFu) * dx.x, (float) s0[r], acc[r]);
+                    acc[r] = fmaf(half_bits_to_float(dd >> 16) * dx.y, (float) s1[r], acc[r]);
                 }
+            }
         }
+        // accumulator lane (g, token r16): rows row0 + 4 g + r
+        if (r16 < T) {
+            float* o = a.out + (size_t) r16 * a.out_stride + row0 + 4 * g;
 #pragma unroll
-        for (int r = 0; r < Q8S_R; ++r)
-#pragma unroll
-            for (int t = 0; t < FNX_MAXT; ++t)
-                if (t < T) {
-                    const float v = group_sum<64>(acc[r][t]);
-                    if (lane == 0 && row0 + r < a.rows) a.out[(size_t) t * a.out_stride + row0 + r] = v;
-                }
+            for (int r = 0; r < 4; ++r)
+                if (row0 + 4 * g + r < a.rows) o[r] = acc[r];
+        }
     }
 }
 
