@@ -224,8 +224,12 @@ typedef struct fnx_q8s {
     int n_out, n_in;
 } fnx_q8s;
 /* dense.cuh:79-214 (q8s_gemv): out[t * out_stride + r] = W[r] . y[t] for T <= 16 q8_1 rows; n_in a multiple of 256. The
- * 32-column blocks are folded in ascending order, acc = fmaf(d_w * d_x, (float) dot, acc) */
+ * result is (s0 + s1) + (s2 + s3), s_q the q-th quarter of the columns, its 32-column blocks folded in ascending order with
+ * acc = fmaf(d_w * d_x, (float) dot, acc) */
 int fnx_q8s_gemv(const fnx_q8s* W, const void* yq, float* out, int out_stride, int T, void* st);
+/* kernels.hpp:414-418 (q8s_gemv_segs): n (1..3) matrices of the same columns over the same rows in one launch, each
+ * output as q8s_gemv of that matrix alone gives it; all but the last matrix hold a multiple of 16 rows */
+int fnx_q8s_gemv_segs(const fnx_q8s* const* W, float* const* out, const int* out_stride, int n, const void* yq, int T, void* st);
 /* rope.hpp:22-39  the rotary's constants (scaled = 0: plain frequencies base^(-2 i / 64), mscale 1) */
 typedef struct fnx_rope {
     float base;

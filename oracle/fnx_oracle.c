@@ -765,21 +765,21 @@ void fnx_o_quantize_q8_0_split(const float* w, int rows, int cols, int8_t* q, ui
         }
 }
 void fnx_o_q8s_gemv(const int8_t* q, const uint16_t* d, int rows, int cols, const uint8_t* yq, float* out, int out_stride, int T) {
-    const int nb = cols / 32;
+    const int nb = cols / 32, qb = nb / 4 > 0 ? nb / 4 : nb; /* blocks per quarter (fewer than 4 blocks: one part) */
 #pragma omp parallel for schedule(static)
     for (int r = 0; r < rows; ++r)
         for (int t = 0; t < T; ++t) {
-            float a = 0.f;
-            for (int b = 0; b < nb; ++b) { /* ascending blocks, one fmaf each: the order is part of the definition */
+            float part[4] = {0.f, 0.f, 0.f, 0.f};
+            for (int b = 0; b < nb; ++b) { /* each quarter: ascending blocks, one fmaf each; the order is part of the definition */
                 const uint8_t* blk = yq + ((size_t) t * nb + b) * Q8_1_BLOCK;
                 uint16_t dxh;
                 memcpy(&dxh, blk, 2);
                 const int8_t* xs = (const int8_t*) blk + 4;
                 int s = 0;
                 for (int j = 0; j < 32; ++j) s += (int) q[(size_t) r * cols + 32 * b + j] * (int) xs[j];
-                a = fmaf(fnx_o_h2f(d[(size_t) r * nb + b]) * fnx_o_h2f(dxh), (float) s, a);
+                part[b / qb] = fmaf(fnx_o_h2f(d[(size_t) r * nb + b]) * fnx_o_h2f(dxh), (float) s, part[b / qb]);
             }
-            out[(size_t) t * out_stride + r] = a;
+            out[(size_t) t * out_stride + r] = (part[0] + part[1]) + (part[2] + part[3]);
         }
 }
 static float rope_unit_freq(const fnx_o_rope* r, int pair, int nrot) { /* rope.hpp:33-39 */

@@ -136,9 +136,9 @@ void fnx_o_moe_prefill_layer(const fnx_o_moe_layer* L, const float* x, int C, in
 void fnx_o_rms_norm_rows(const float* x, const float* w, float* y, int rows, int n, float eps);
 /* ggml's Q8_0 in the reference's split layout (model.hpp:78-82): d = max|x| / 127 as f16, q = round(x / d) */
 void fnx_o_quantize_q8_0_split(const float* w, int rows, int cols, int8_t* q, uint16_t* d);
-/* dense.cuh:79-214: out[t * out_stride + r] = the 32-column blocks in ascending order folded with
- * acc = fmaf(d_w * d_x, (float) dot, acc) (the reference's term, dense.cuh:196-200, in this build's fixed order, which
- * the device follows bit for bit) */
+/* dense.cuh:79-214: out[t * out_stride + r] = (s0 + s1) + (s2 + s3), s_q the q-th quarter of the columns with its
+ * 32-column blocks folded in ascending order, acc = fmaf(d_w * d_x, (float) dot, acc) (the reference's term,
+ * dense.cuh:196-200, in this build's fixed order, which the device follows bit for bit) */
 void fnx_o_q8s_gemv(const int8_t* q, const uint16_t* d, int rows, int cols, const uint8_t* yq, float* out, int out_stride, int T);
 typedef struct {
     float base;

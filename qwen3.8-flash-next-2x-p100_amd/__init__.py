@@ -113,6 +113,7 @@ EXPORTS = {
     "fnx_add_rows": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "fnx_embed_rows": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]),
     "fnx_q8s_gemv": (C.c_int, [C.POINTER(Q8S), C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
+    "fnx_q8s_gemv_segs": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_void_p]),
     "fnx_attn_prep_append": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int,
                                        C.c_int, C.c_void_p, C.c_int, C.c_float, C.POINTER(Rope), C.c_void_p]),
     "fnx_attn_scratch_floats": (C.c_size_t, [C.c_int, C.c_int, C.c_int]),

@@ -972,27 +972,44 @@ int fnx_embed_rows(const uint16_t* emb, const int* tokens, int T, int vocab, int
     k_embed_rows<<<T, 256, 0, (hipStream_t) st>>>(emb, tokens, vocab, n, y);
     return launch_status("embed_rows");
 }
-int fnx_q8s_gemv(const fnx_q8s* W, const void* yq, float* out, int out_stride, int T, void* st) {
-    if (!W || !W->q || !W->d || !yq || !out) return fail("q8s_gemv: null argument");
-    if (W->n_out < 1 || W->n_in < 32 || W->n_in % 32) return fail("q8s_gemv: columns in whole 32-value blocks");
-    if (W->n_in % 256 || ((uintptr_t) W->q & 15) || ((uintptr_t) W->d & 15)) return fail("q8s_gemv: columns in 256s, 16-byte aligned rows");
-    if (T < 1 || T > FNX_MAXT) return fail("q8s_gemv: T out of range");
-    if (out_stride < W->n_out) return fail("q8s_gemv: out_stride smaller than the rows");
-    const size_t lds = (size_t) FNX_MAXT * (W->n_in + Q8S_XPAD) + (size_t) FNX_MAXT * (W->n_in / 32 + 2) * 4;
-    if (lds > 150 * 1024) return fail("q8s_gemv: the window's activations do not fit LDS");
+static int q8s_launch(const fnx_q8s* const* W, float* const* out, const int* out_stride, int n, const void* yq, int T, void* st, const char* who) {
+    if (!W || !out || !out_stride || !yq || n < 1 || n > 3) return fail(std::string(who) + ": null argument");
+    Q8sArgs a{};
+    long tiles = 0;
+    for (int s = 0; s < n; ++s) {
+        if (!W[s] || !W[s]->q || !W[s]->d || !out[s]) return fail(std::string(who) + ": null argument");
+        if (W[s]->n_out < 1 || W[s]->n_in < 256 || W[s]->n_in % 256) return fail(std::string(who) + ": columns in 256s");
+        if (W[s]->n_in != W[0]->n_in) return fail(std::string(who) + ": the matrices share the activations: the same columns");
+        if (((uintptr_t) W[s]->q & 15) || ((uintptr_t) W[s]->d & 3)) return fail(std::string(who) + ": 16-byte aligned rows");
+        if (s + 1 < n && W[s]->n_out % 16) return fail(std::string(who) + ": all but the last matrix in whole 16-row tiles");
+        if (out_stride[s] < W[s]->n_out) return fail(std::string(who) + ": out_stride smaller than the rows");
+        a.seg[s] = Q8sSeg{W[s]->q, W[s]->d, out[s], W[s]->n_out, out_stride[s]};
+        tiles += (W[s]->n_out + 15) / 16;
+    }
+    if (T < 1 || T > FNX_MAXT) return fail(std::string(who) + ": T out of range");
+    a.nseg = n;
+    a.cols = W[0]->n_in;
+    a.T = T;
+    a.yq = (const uint8_t*) yq;
+    const size_t lds = (size_t) FNX_MAXT * (a.cols + Q8S_XPAD) + (size_t) FNX_MAXT * (a.cols / 32 + 2) * 4 + Q8S_WAVES * 64 * 16;
+    if (lds > 150 * 1024) return fail(std::string(who) + ": the window's activations do not fit LDS");
     static bool attr_set[64] = {};
     int dev = 0;
     if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64 && !attr_set[dev]) {
         if (hipFuncSetAttribute((const void*) k_q8s_gemv, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024) != hipSuccess)
-            return fail("q8s_gemv: cannot raise the dynamic LDS limit");
+            return fail(std::string(who) + ": cannot raise the dynamic LDS limit");
         attr_set[dev] = true;
     }
-    const Q8sArgs a{W->q, W->d, W->n_out, W->n_in, (const uint8_t*) yq, out, out_stride, T};
-    const int tiles = (W->n_out + 15) / 16;
-    static const int per_cu = env_int("FNX_Q8S_BLOCKS_PER_CU", 2, 1, 8);
-    const int grid = std::max(1, std::min(per_cu * cu_count(), (tiles + Q8S_WAVES - 1) / Q8S_WAVES));
+    static const int per_cu = env_int("FNX_Q8S_BLOCKS_PER_CU", 4, 1, 16);
+    const int grid = (int) std::max(1l, std::min<long>((long) per_cu * cu_count(), tiles));
     k_q8s_gemv<<<grid, Q8S_WAVES * 64, lds, (hipStream_t) st>>>(a);
-    return launch_status("q8s_gemv");
+    return launch_status(who);
+}
+int fnx_q8s_gemv(const fnx_q8s* W, const void* yq, float* out, int out_stride, int T, void* st) {
+    return q8s_launch(&W, &out, &out_stride, 1, yq, T, st, "q8s_gemv");
+}
+int fnx_q8s_gemv_segs(const fnx_q8s* const* W, float* const* out, const int* out_stride, int n, const void* yq, int T, void* st) {
+    return q8s_launch(W, out, out_stride, n, yq, T, st, "q8s_gemv_segs");
 }
 int fnx_attn_prep_append(float* qg, float* k, const float* v, const float* q_norm, const float* k_norm, uint16_t* kc, uint16_t* vc, int nq,
                          int nkv, int T, const int* pos0, int max_ctx, float eps, const fnx_rope* rope, void* st) {
@@ -1024,7 +1041,8 @@ int fnx_attn(const float* qg, const uint16_t* kc, const uint16_t* vc, float* out
     const int nsplit = attn_splits(max_ctx), waves = (T * (nq / nkv) + 15) / 16;
     float* acc = scratch;
     AttPart* mz = reinterpret_cast<AttPart*>(scratch + (size_t) T * nq * nsplit * AT_HD);
-    k_attn_part<<<dim3(nsplit, nkv), 64 * waves, 0, (hipStream_t) st>>>(qg, kc, vc, acc, mz, nq, nkv, T, nsplit, pos0);
+    k_attn_part<<<dim3(nsplit, nkv, (waves + AT_WAVES - 1) / AT_WAVES), 64 * AT_WAVES, 0, (hipStream_t) st>>>(qg, kc, vc, acc, mz, nq, nkv, T,
+                                                                                                          nsplit, pos0);
     k_attn_combine<<<dim3(nq, T), AT_HD, 0, (hipStream_t) st>>>(qg, acc, mz, out, nq, nsplit);
     return launch_status("attn");
 }
@@ -1039,9 +1057,12 @@ static int dec_layer(const fnx_decoder* D, const fnx_dec_layer* L, int T, const 
     const int n = D->n, nq = D->nq, nkv = D->nkv;
     if (fnx_rms_norm_rows(ws->x, L->attn_norm, ws->xn, T, n, D->eps, st)) return 1;
     if (fnx_quantize_q8_1(ws->xn, ws->xq, n, T, st)) return 1;
-    if (fnx_q8s_gemv(&L->wq, ws->xq, ws->qg, nq * 2 * AT_HD, T, st)) return 1;
-    if (fnx_q8s_gemv(&L->wk, ws->xq, ws->k, nkv * AT_HD, T, st)) return 1;
-    if (fnx_q8s_gemv(&L->wv, ws->xq, ws->v, nkv * AT_HD, T, st)) return 1;
+    {   // q, k and v in one launch (engine.cu:1547-1552)
+        const fnx_q8s* w3[3] = {&L->wq, &L->wk, &L->wv};
+        float* const o3[3] = {ws->qg, ws->k, ws->v};
+        const int s3[3] = {nq * 2 * AT_HD, nkv * AT_HD, nkv * AT_HD};
+        if (fnx_q8s_gemv_segs(w3, o3, s3, 3, ws->xq, T, st)) return 1;
+    }
     if (fnx_attn_prep_append(ws->qg, ws->k, ws->v, L->q_norm, L->k_norm, L->kc, L->vc, nq, nkv, T, pos0, D->max_ctx, D->eps, &D->rope, st)) return 1;
     if (fnx_attn(ws->qg, L->kc, L->vc, ws->att, nq, nkv, pos0, T, D->max_ctx, ws->attn_scratch, st)) return 1;
     if (fnx_quantize_q8_1(ws->att, ws->xq, nq * AT_HD, T, st)) return 1;

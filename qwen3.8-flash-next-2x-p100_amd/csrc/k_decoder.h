@@ -34,30 +34,36 @@ __global__ void k_embed_rows(const uint16_t* __restrict__ emb, const int* __rest
 
 // ---------------------------------------------------------------- dense Q8_0, split layout (dense.cuh:79-214)
 // int8 values [rows][cols], f16 scales [rows][cols / 32]; activations q8_1 (up to 16 rows). The result is defined as
-//   out[t][r] = fold over the 32-column blocks b in ascending order of acc = fmaf(d_w[r][b] * d_x[t][b], (float) dot_b, acc)
+//   out[t][r] = (s0 + s1) + (s2 + s3),  s_q = fold over the 32-column blocks b of the q-th quarter of the columns, in
+//               ascending order, of acc = fmaf(d_w[r][b] * d_x[t][b], (float) dot_b, acc)
 // (dot_b the exact integer dot product of the block): the reference's term (dense.cuh:196-200) in one fixed order, which
 // the CPU oracle follows bit for bit.
-// On the matrix cores: a wave owns 16 weight rows; v_mfma_i32_16x16x32_i8 wants 8 bytes of k from each of 4 lane groups.
-// A lane loads 16 contiguous bytes of its row per 64 columns (group g: bytes 16 g ..), so groups 0-1 hold block 2 j and
-// groups 2-3 block 2 j + 1; each block's dot product is two MFMAs (the lanes' low and high 8 bytes) whose B operand is
-// zero in the other block's groups. The 16 x 16 integer sums then take their scales in 12 VALU ops, against 44 for
-// the same block on the vector ALU, and no cross-lane reduction is left.
-constexpr int Q8S_WAVES = 4, Q8S_XPAD = 16;
-struct Q8sArgs {
+// On the matrix cores: a block owns 16 weight rows, each of its four waves a quarter of the columns (so that a matrix
+// of a few hundred rows still fills the chip and a wave's chain of dependent loads is short). v_mfma_i32_16x16x32_i8
+// wants 8 bytes of k from each of 4 lane groups. A lane loads 16 contiguous bytes of its row per 64 columns (group g:
+// bytes 16 g ..), so groups 0-1 hold block 2 j and groups 2-3 block 2 j + 1; each block's dot product is two MFMAs (the
+// lanes' low and high 8 bytes) whose B operand is zero in the other block's groups. The 16 x 16 integer sums then take
+// their scales in 12 VALU ops, against 44 for the same block on the vector ALU, and no cross-lane reduction is left.
+constexpr int Q8S_WAVES = 4, Q8S_XPAD = 16, Q8S_BATCH = 4;   // double steps (64 columns) loaded at once
+struct Q8sSeg {
     const int8_t* q;
     const uint16_t* d;
-    int rows, cols;
-    const uint8_t* yq;   // q8_1 rows
     float* out;
-    int out_stride, T;
+    int rows, out_stride;
+};
+struct Q8sArgs {
+    Q8sSeg seg[3];       // up to three matrices over the same activations, their 16-row tiles one after another
+    int nseg, cols, T;
+    const uint8_t* yq;   // q8_1 rows
 };
 typedef int q8s_v4i __attribute__((ext_vector_type(4)));
 __global__ void __launch_bounds__(Q8S_WAVES * 64) k_q8s_gemv(const Q8sArgs a) {
     typedef __attribute__((address_space(1))) const at_v4u_t g128;
-    extern __shared__ __align__(16) uint8_t q8s_lds[];   // [16][cols + pad] int8, then [16][nb + 2] f32 scales
+    extern __shared__ __align__(16) uint8_t q8s_lds[];   // [16][cols + pad] int8, [16][nb + 2] f32 scales, [4][64][4] partial sums
     const int nb = a.cols >> 5, T = a.T, xld = a.cols + Q8S_XPAD, dld = nb + 2;
     int8_t* xs = reinterpret_cast<int8_t*>(q8s_lds);
     float* xd = reinterpret_cast<float*>(q8s_lds + (size_t) FNX_MAXT * xld);
+    float* part = xd + FNX_MAXT * dld;
     for (int i = threadIdx.x; i < FNX_MAXT * nb; i += blockDim.x) {
         const int t = i / nb, b = i - t * nb;
         uint32_t* dst = reinterpret_cast<uint32_t*>(xs + (size_t) t * xld + 32 * b);
@@ -74,57 +80,71 @@ __global__ void __launch_bounds__(Q8S_WAVES * 64) k_q8s_gemv(const Q8sArgs a) {
         }
     }
     __syncthreads();
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r16 = lane & 15, g = lane >> 4;
-    const int tiles = (a.rows + 15) / 16, nd = a.cols >> 6;   // double steps of 64 columns
+    const int lane = threadIdx.x & 63, wave = uniform(threadIdx.x >> 6), r16 = lane & 15, g = lane >> 4;
+    const int t0 = (a.seg[0].rows + 15) / 16, t1 = t0 + (a.nseg > 1 ? (a.seg[1].rows + 15) / 16 : 0),
+              tiles = t1 + (a.nseg > 2 ? (a.seg[2].rows + 15) / 16 : 0);
+    const int nq4 = a.cols >> 8;   // double steps per wave: a quarter of cols / 64
     const bool lo_groups = g < 2;
-    for (int tile = blockIdx.x * Q8S_WAVES + wave; tile < tiles; tile += gridDim.x * Q8S_WAVES) {
-        const int row0 = tile * 16;
-        const gbytes wrow = as_global(reinterpret_cast<const uint8_t*>(a.q) + (size_t) min(row0 + r16, a.rows - 1) * a.cols + 16 * g);
-        // the scales of the accumulator's rows 4 g .. 4 g + 3
-        const uint16_t* drow[4];
+    for (int tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+        const int si = tile < t0 ? 0 : tile < t1 ? 1 : 2;
+        const int8_t* sq = si == 0 ? a.seg[0].q : si == 1 ? a.seg[1].q : a.seg[2].q;
+        const uint16_t* sd = si == 0 ? a.seg[0].d : si == 1 ? a.seg[1].d : a.seg[2].d;
+        float* sout = si == 0 ? a.seg[0].out : si == 1 ? a.seg[1].out : a.seg[2].out;
+        const int srows = si == 0 ? a.seg[0].rows : si == 1 ? a.seg[1].rows : a.seg[2].rows;
+        const int sstride = si == 0 ? a.seg[0].out_stride : si == 1 ? a.seg[1].out_stride : a.seg[2].out_stride;
+        const int row0 = (tile - (si == 0 ? 0 : si == 1 ? t0 : t1)) * 16;
+        const int j0 = wave * nq4;   // this wave's first double step
+        const gbytes wrow = as_global(reinterpret_cast<const uint8_t*>(sq) + (size_t) min(row0 + r16, srows - 1) * a.cols + 16 * g + 64 * j0);
+        // the scales of the accumulator's rows 4 g .. 4 g + 3, from this wave's first block on
+        gbytes drow[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) drow[r] = a.d + (size_t) min(row0 + 4 * g + r, a.rows - 1) * nb;
+        for (int r = 0; r < 4; ++r)
+            drow[r] = as_global(reinterpret_cast<const uint8_t*>(sd + (size_t) min(row0 + 4 * g + r, srows - 1) * nb + 2 * j0));
         float acc[4] = {0.f, 0.f, 0.f, 0.f};
-        at_v4u_t wn = *(g128*) wrow;
-        // the rows' scales eight blocks (four double steps) at a time, fetched four double steps ahead
-        at_v4u_t dn[4];
+        for (int jb = 0; jb < nq4; jb += Q8S_BATCH) {   // nq4 is 1, 2 or a multiple of 4 (cols a multiple of 256)
+            const int nstep = min(Q8S_BATCH, nq4 - jb);
+            at_v4u_t w[Q8S_BATCH];
+            uint32_t dd[4][Q8S_BATCH];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) dn[r] = *(g128*) as_global(reinterpret_cast<const uint8_t*>(drow[r]));
-        for (int j4 = 0; j4 < nd; j4 += 4) {
-            at_v4u_t dc[4];
+            for (int u = 0; u < Q8S_BATCH; ++u) {
+                const int j = jb + min(u, nstep - 1);
+                w[u] = *(g128*) (wrow + 64 * j);
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                dc[r] = dn[r];
-                dn[r] = *(g128*) as_global(reinterpret_cast<const uint8_t*>(drow[r] + 2 * min(j4 + 4, nd - 4)));
+                for (int r = 0; r < 4; ++r) dd[r][u] = *(const __attribute__((address_space(1))) uint32_t*) (drow[r] + 4 * j);
             }
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const int j = j4 + u;
-                const at_v4u_t w = wn;
-                wn = *(g128*) (wrow + 64 * min(j + 1, nd - 1));   // past the end: the last piece again
-                const at_v4u_t x = *reinterpret_cast<const at_v4u_t*>(xs + (size_t) r16 * xld + 64 * j + 16 * g);
-                const float2 dx = *reinterpret_cast<const float2*>(xd + r16 * dld + 2 * j);
-                const long wl = (long) w.x | (long) w.y << 32, wh = (long) w.z | (long) w.w << 32;
-                const long xl = (long) x.x | (long) x.y << 32, xh = (long) x.z | (long) x.w << 32;
-                const long xl0 = lo_groups ? xl : 0, xh0 = lo_groups ? xh : 0, xl1 = lo_groups ? 0 : xl, xh1 = lo_groups ? 0 : xh;
-                q8s_v4i s0 = __builtin_amdgcn_mfma_i32_16x16x32_i8(wl, xl0, q8s_v4i{0, 0, 0, 0}, 0, 0, 0);
-                s0 = __builtin_amdgcn_mfma_i32_16x16x32_i8(wh, xh0, s0, 0, 0, 0);
-                q8s_v4i s1 = __builtin_amdgcn_mfma_i32_16x16x32_i8(wl, xl1, q8s_v4i{0, 0, 0, 0}, 0, 0, 0);
-                s1 = __builtin_amdgcn_mfma_i32_16x16x32_i8(wh, xh1, s1, 0, 0, 0);
+            for (int u = 0; u < Q8S_BATCH; ++u)
+                if (u < nstep) {
+                    const int j = j0 + jb + u;
+                    const at_v4u_t x = *reinterpret_cast<const at_v4u_t*>(xs + (size_t) r16 * xld + 64 * j + 16 * g);
+                    const float2 dx = *reinterpret_cast<const float2*>(xd + r16 * dld + 2 * j);
+                    const long wl = (long) w[u].x | (long) w[u].y << 32, wh = (long) w[u].z | (long) w[u].w << 32;
+                    const long xl = (long) x.x | (long) x.y << 32, xh = (long) x.z | (long) x.w << 32;
+                    const long xl0 = lo_groups ? xl : 0, xh0 = lo_groups ? xh : 0, xl1 = lo_groups ? 0 : xl, xh1 = lo_groups ? 0 : xh;
+                    q8s_v4i s0 = __builtin_amdgcn_mfma_i32_16x16x32_i8(wl, xl0, q8s_v4i{0, 0, 0, 0}, 0, 0, 0);
+                    s0 = __builtin_amdgcn_mfma_i32_16x16x32_i8(wh, xh0, s0, 0, 0, 0);
+                    q8s_v4i s1 = __builtin_amdgcn_mfma_i32_16x16x32_i8(wl, xl1, q8s_v4i{0, 0, 0, 0}, 0, 0, 0);
+                    s1 = __builtin_amdgcn_mfma_i32_16x16x32_i8(wh, xh1, s1, 0, 0, 0);
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const uint32_t dd = dc[r][u];   // blocks 2 j and 2 j + 1
-                    acc[r] = fmaf(half_bits_to_float(dd & 0xFFFFu) * dx.x, (float) s0[r], acc[r]);
-                    acc[r] = fmaf(half_bits_to_float(dd >> 16) * dx.y, (float) s1[r], acc[r]);
+                    for (int r = 0; r < 4; ++r) {
+                        acc[r] = fmaf(half_bits_to_float(dd[r][u] & 0xFFFFu) * dx.x, (float) s0[r], acc[r]);
+                        acc[r] = fmaf(half_bits_to_float(dd[r][u] >> 16) * dx.y, (float) s1[r], acc[r]);
+                    }
                 }
-            }
         }
-        // accumulator lane (g, token r16): rows row0 + 4 g + r
-        if (r16 < T) {
-            float* o = a.out + (size_t) r16 * a.out_stride + row0 + 4 * g;
+        // the four quarters through LDS: (s0 + s1) + (s2 + s3)
+        __syncthreads();   // the previous tile's sums have been read
+        *reinterpret_cast<float4*>(part + (wave * 64 + lane) * 4) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+        __syncthreads();
+        if (wave == 0 && r16 < T) {   // accumulator lane (g, token r16): rows row0 + 4 g + r
+            const float4 p0 = *reinterpret_cast<const float4*>(part + lane * 4), p1 = *reinterpret_cast<const float4*>(part + (64 + lane) * 4),
+                         p2 = *reinterpret_cast<const float4*>(part + (128 + lane) * 4), p3 = *reinterpret_cast<const float4*>(part + (192 + lane) * 4);
+            const float v[4] = {(p0.x + p1.x) + (p2.x + p3.x), (p0.y + p1.y) + (p2.y + p3.y), (p0.z + p1.z) + (p2.z + p3.z),
+                                (p0.w + p1.w) + (p2.w + p3.w)};
+            float* o = sout + (size_t) r16 * sstride + row0 + 4 * g;
 #pragma unroll
             for (int r = 0; r < 4; ++r)
-                if (row0 + 4 * g + r < a.rows) o[r] = acc[r];
+                if (row0 + 4 * g + r < srows) o[r] = v[r];
         }
     }
 }
@@ -185,8 +205,8 @@ __global__ void __launch_bounds__(AT_HD) k_attn_prep_append(float* __restrict__ 
 // splits, the splits merged by their maxima, the result times sigmoid(gate).)
 //
 // A window's rows times a kv head's q heads are up to 128 query vectors against the same K/V rows: a dense contraction,
-// so it runs on v_mfma_f32_16x16x32_f16. A block takes (split of AT_SPLIT positions, kv head); wave j of it takes the
-// 16 queries 16 j .. 16 j + 15 (query = row * heads-per-kv + head). Per chunk of 32 positions:
+// so it runs on v_mfma_f32_16x16x32_f16. A block takes (split of AT_SPLIT positions, kv head, half of the query tiles);
+// a wave takes 16 queries (query = row * heads-per-kv + head). Per chunk of 32 positions:
 //   S^T = K Q^T  : A = K rows (lane: position l % 16, the 64 dims of lane group l / 16, 16 bytes a step from the cache),
 //                  B = Q^T (held in registers for the whole split, scaled by 1/16, as two f16 terms hi + lo);
 //                  the accumulator leaves lane (group pg, query q) with positions 4 pg .. 4 pg + 3 of both 16-position
@@ -194,7 +214,7 @@ __global__ void __launch_bounds__(AT_HD) k_attn_prep_append(float* __restrict__ 
 //   O^T += V^T P^T: those eight positions are exactly lane group pg's contraction slots, so P goes from the accumulator
 //                  registers straight into the B operand, and V^T's A operand is two 8-byte loads because the V cache
 //                  keeps four positions of a dimension together ([position / 4][kv head][dim][position % 4]).
-// Nothing passes through LDS. Each (query, split) leaves its maximum, sum and 256 accumulators; k_attn_combine merges.
+// The probabilities never pass through LDS; K and V chunks do, once per block (a chunk ahead, double-buffered). Each (query, split) leaves its maximum, sum and 256 accumulators; k_attn_combine merges.
 constexpr int AT_SPLIT = 512, AT_CH = 32, AT_MAXQ = 8;
 struct AttPart {
     float m, z;
@@ -209,12 +229,14 @@ __device__ __forceinline__ size_t vcache_at(int pos, int nkv, int kvh, int d) { 
     return (((size_t) (pos >> 2) * nkv + kvh) * AT_HD + d) * 4 + (pos & 3);
 }
 
-__global__ void __launch_bounds__(512) k_attn_part(const float* __restrict__ qg, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
-                                                  float* __restrict__ acc_out, AttPart* __restrict__ mz_out, int nq, int nkv, int T,
-                                                  int nsplit, const int* __restrict__ pos0p) {
+constexpr int AT_WAVES = 4, AT_KLD = 2 * AT_HD + 16;   // q tiles (of 16 queries) per block, blockIdx.z picks which; LDS bytes per K row
+__global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) k_attn_part(const float* __restrict__ qg, const uint16_t* __restrict__ kc,
+                                                            const uint16_t* __restrict__ vc, float* __restrict__ acc_out,
+                                                            AttPart* __restrict__ mz_out, int nq, int nkv, int T, int nsplit,
+                                                            const int* __restrict__ pos0p) {
     typedef __attribute__((address_space(1))) const at_v4u g128;
     typedef __attribute__((address_space(1))) const at_v2u g64;
-    const int s = blockIdx.x, kvh = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int s = blockIdx.x, kvh = blockIdx.y, lane = threadIdx.x & 63, wave = blockIdx.z * AT_WAVES + (threadIdx.x >> 6);
     const int qpk = nq / nkv, nquery = T * qpk, pos0 = *pos0p;
     const int ql = lane & 15, pg = lane >> 4;
     const int qi = wave * 16 + ql;                      // this lane's query (as B column / accumulator column)
@@ -223,6 +245,11 @@ __global__ void __launch_bounds__(512) k_attn_part(const float* __restrict__ qg,
     const int ctx_q = qlive ? pos0 + qt + 1 : 0;        // positions [0, ctx_q) are this query's
     const int ctx_max = pos0 + T;                       // the window's last row sees this many
     const int p0 = s * AT_SPLIT, p1 = min(ctx_max, p0 + AT_SPLIT);
+    const size_t slot = ((size_t) qt * nq + qh) * nsplit + s;
+    if (p0 >= p1) {   // a split past the context: an empty part
+        if (qlive && pg == 0) mz_out[slot] = AttPart{-INFINITY, 0.f};
+        return;
+    }
     // Q^T operands: step ks holds dims 64 pg + 8 ks .. + 7 of query ql, times 1/16 (exact), as two f16 terms hi + lo:
     // the cache is f16 already, so with q (and below the probabilities) split this way the products carry fp32's
     // precision, as the reference's f32 arithmetic on the f16 cache does
@@ -246,30 +273,54 @@ __global__ void __launch_bounds__(512) k_attn_part(const float* __restrict__ qg,
 #pragma unroll
     for (int dt = 0; dt < 16; ++dt) O[dt] = at_v4f{0.f, 0.f, 0.f, 0.f};
     float m = -INFINITY, z = 0.f;
+    // A chunk's K rows (32 x 512 bytes) and V blocks (8 x 2048 bytes) are fetched once per block, 64 + 64 contiguous
+    // bytes per thread, a chunk ahead into registers and from there into one of two LDS buffers; the waves read their
+    // operands from LDS (K rows padded to 528 bytes: the 16 positions of a tile fall on different banks).
+    __shared__ __align__(16) uint8_t lk[2][AT_CH * AT_KLD];
+    __shared__ __align__(16) uint8_t lv[2][8 * AT_HD * 8];
+    const int tid = threadIdx.x;
     const gbytes kbase = as_global(reinterpret_cast<const uint8_t*>(kc));
     const gbytes vbase = as_global(reinterpret_cast<const uint8_t*>(vc));
-    for (int c0 = p0; c0 < p1; c0 += AT_CH) {
-        // K rows of the two position tiles (as A: position c0 + 16 tile + ql, dims 64 pg ..): clamped inside the window's rows
+    const int krow = tid >> 3, kpart = tid & 7, vblk = tid >> 5, vpart = tid & 31;
+    at_v4u kr[4], vr[4];
+    auto fetch = [&](int c0) {   // rows and blocks clamped inside the window's rows
+        const int pos = min(c0 + krow, ctx_max - 1), blk = min((c0 >> 2) + vblk, (ctx_max - 1) >> 2);
+        const gbytes kp = kbase + ((size_t) pos * nkv + kvh) * (AT_HD * 2) + 64 * kpart;
+        const gbytes vp = vbase + ((size_t) blk * nkv + kvh) * (AT_HD * 8) + 64 * vpart;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            kr[i] = *(g128*) (kp + 16 * i);
+            vr[i] = *(g128*) (vp + 16 * i);
+        }
+    };
+    auto stash = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            *reinterpret_cast<at_v4u*>(&lk[buf][krow * AT_KLD + 64 * kpart + 16 * i]) = kr[i];
+            *reinterpret_cast<at_v4u*>(&lv[buf][vblk * (AT_HD * 8) + 64 * vpart + 16 * i]) = vr[i];
+        }
+    };
+    fetch(p0);
+    stash(0);
+    fetch(min(p0 + AT_CH, p1 - 1));
+    __syncthreads();
+    int buf = 0;
+    for (int c0 = p0; c0 < p1; c0 += AT_CH, buf ^= 1) {
+        stash(buf ^ 1);                              // chunk c0 + 32, fetched during the last iteration
+        fetch(min(c0 + 2 * AT_CH, p1 - 1));          // past the split: some rows again, never used
         at_v4f S[2];
 #pragma unroll
         for (int tile = 0; tile < 2; ++tile) {
-            const int pos = min(c0 + 16 * tile + ql, ctx_max - 1);
-            const gbytes kr = kbase + (((size_t) pos * nkv + kvh) * AT_HD + 64 * pg) * 2;
-            at_v4u kreg[8];
-#pragma unroll
-            for (int ks = 0; ks < 8; ++ks) kreg[ks] = *(g128*) (kr + 16 * ks);
+            const uint8_t* krow_l = &lk[buf][(16 * tile + ql) * AT_KLD + 128 * pg];
             at_v4f acc = at_v4f{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int ks = 0; ks < 8; ++ks) {
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(at_v8h, kreg[ks]), Ql[ks], acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(at_v8h, kreg[ks]), Q[ks], acc, 0, 0, 0);
+                const at_v8h kk = __builtin_bit_cast(at_v8h, *reinterpret_cast<const at_v4u*>(krow_l + 16 * ks));
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(kk, Ql[ks], acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(kk, Q[ks], acc, 0, 0, 0);
             }
             S[tile] = acc;
         }
-        // V^T operands for the 16 dim tiles: positions c0 + 4 pg .. + 3 and c0 + 16 + 4 pg .. + 3, dim 16 dt + ql
-        // (clamped to the window's rows; the probabilities of positions past a query's own are zero)
-        const int vb0 = min(c0 + 4 * pg, (ctx_max - 1) & ~3) >> 2, vb1 = min(c0 + 16 + 4 * pg, (ctx_max - 1) & ~3) >> 2;
-        const gbytes v0 = vbase + (((size_t) vb0 * nkv + kvh) * AT_HD + ql) * 8, v1 = vbase + (((size_t) vb1 * nkv + kvh) * AT_HD + ql) * 8;
         // this lane: query ql, positions c0 + 4 pg + r (tile 0) and c0 + 16 + 4 pg + r (tile 1)
         float sv[8];
         float mx = -INFINITY;
@@ -300,7 +351,9 @@ __global__ void __launch_bounds__(512) k_attn_part(const float* __restrict__ qg,
             P[r] = hi;
             Pl[r] = (_Float16) (pw[r] - (float) hi);
         }
-        // positions past the window's rows were never written: whatever their cells hold must not reach the products
+        // V^T operands: positions c0 + 4 pg .. + 3 (block pg of the chunk) and c0 + 16 + 4 pg .. + 3 (block 4 + pg), dim
+        // 16 dt + ql. Positions past the window's rows were never written: whatever their cells hold must not reach the
+        // products (a block clamped to the window's last repeats that block: its probabilities are zero)
         const bool tail = c0 + AT_CH > ctx_max;
         unsigned keep0[2] = {~0u, ~0u}, keep1[2] = {~0u, ~0u};
         if (tail) {
@@ -310,9 +363,11 @@ __global__ void __launch_bounds__(512) k_attn_part(const float* __restrict__ qg,
                 if (c0 + 16 + 4 * pg + j >= ctx_max) keep1[j >> 1] &= (j & 1) ? 0x0000FFFFu : 0xFFFF0000u;
             }
         }
+        const uint8_t* v0 = &lv[buf][pg * (AT_HD * 8) + ql * 8];
+        const uint8_t* v1 = &lv[buf][(4 + pg) * (AT_HD * 8) + ql * 8];
 #pragma unroll
         for (int dt = 0; dt < 16; ++dt) {
-            const at_v2u a0 = *(g64*) (v0 + 128 * dt), a1 = *(g64*) (v1 + 128 * dt);
+            const at_v2u a0 = *reinterpret_cast<const at_v2u*>(v0 + 128 * dt), a1 = *reinterpret_cast<const at_v2u*>(v1 + 128 * dt);
             const at_v4u a = at_v4u{a0.x & keep0[0], a0.y & keep0[1], a1.x & keep1[0], a1.y & keep1[1]};
             at_v4f o = O[dt];
             o.x *= sc;
@@ -322,10 +377,10 @@ __global__ void __launch_bounds__(512) k_attn_part(const float* __restrict__ qg,
             o = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(at_v8h, a), Pl, o, 0, 0, 0);
             O[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(at_v8h, a), P, o, 0, 0, 0);
         }
+        __syncthreads();
     }
     if (!qlive) return;
     // accumulator lane (dim group pg, query ql): dims 16 dt + 4 pg + r
-    const size_t slot = ((size_t) qt * nq + qh) * nsplit + s;
 #pragma unroll
     for (int dt = 0; dt < 16; ++dt)
         *reinterpret_cast<float4*>(acc_out + slot * AT_HD + 16 * dt + 4 * pg) = make_float4(O[dt].x, O[dt].y, O[dt].z, O[dt].w);
