@@ -213,7 +213,11 @@ int fnx_moe_prefill_layer(const fnx_moe_layer* L, const float* x, int C, float* 
  * 64 dims rotated (model.hpp:41). */
 /* kernels.hpp:406  rms_norm_rows: y[r] = x[r] / sqrt(mean(x[r]^2) + eps) * w */
 int fnx_rms_norm_rows(const float* x, const float* w, float* y, int rows, int n, float eps, void* st);
-/* y = a + b over n floats (the residual adds between the halves of a layer) */
+/* x[r] += add[r] (add may be null); xn[r] = rms_norm(x[r]) * w; xq[r] = q8_1 of xn[r] (xn, xq may be null): the residual
+ * add, rms_norm_rows and quantize_q8_1 that follow one another between a layer's halves (engine.cu's hc_read takes
+ * the same place in the reference), one pass over each row; the values are the three operators' bit for bit. n <= 4096 */
+int fnx_add_norm_q8(float* x, const float* add, const float* w, float* xn, void* xq, int rows, int n, float eps, void* st);
+/* y = a + b over n floats */
 int fnx_add_rows(const float* a, const float* b, float* y, size_t n, void* st);
 /* rows tokens[t] of an f16 table [vocab][n] as f32 (the window's input rows) */
 int fnx_embed_rows(const uint16_t* emb, const int* tokens, int T, int vocab, int n, float* y, void* st);

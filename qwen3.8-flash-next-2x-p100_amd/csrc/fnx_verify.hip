@@ -960,6 +960,12 @@ int fnx_rms_norm_rows(const float* x, const float* w, float* y, int rows, int n,
     k_rms_norm_rows<<<rows, 256, 0, (hipStream_t) st>>>(x, w, y, n, eps);
     return launch_status("rms_norm_rows");
 }
+int fnx_add_norm_q8(float* x, const float* add, const float* w, float* xn, void* xq, int rows, int n, float eps, void* st) {
+    if (!x || !w) return fail("add_norm_q8: null argument");
+    if (rows < 1 || n < 32 || n % 32 || n > 256 * NQ_MAXJ) return fail("add_norm_q8: rows of 32 .. 4096 values in whole 32-value blocks");
+    k_add_norm_q8<<<rows, 256, 0, (hipStream_t) st>>>(x, add, w, xn, (uint8_t*) xq, n, eps);
+    return launch_status("add_norm_q8");
+}
 int fnx_add_rows(const float* a, const float* b, float* y, size_t n, void* st) {
     if (!a || !b || !y) return fail("add_rows: null argument");
     if (n == 0) return 0;
@@ -1037,13 +1043,14 @@ int fnx_attn(const float* qg, const uint16_t* kc, const uint16_t* vc, float* out
              float* scratch, void* st) {
     if (!qg || !kc || !vc || !out || !pos0 || !scratch) return fail("attn: null argument");
     if (nq < 1 || nkv < 1 || nq % nkv || nq / nkv > AT_MAXQ || T < 1 || T > FNX_MAXT || max_ctx < 1) return fail("attn: bad shape");
+    if (attn_splits(max_ctx) > AT_MAXSPLIT) return fail("attn: the cache is larger than the split table");
     // the grid covers the cache's capacity (the position is on the device): splits past the context write empty parts
     const int nsplit = attn_splits(max_ctx), waves = (T * (nq / nkv) + 15) / 16;
     float* acc = scratch;
     AttPart* mz = reinterpret_cast<AttPart*>(scratch + (size_t) T * nq * nsplit * AT_HD);
     k_attn_part<<<dim3(nsplit, nkv, (waves + AT_WAVES - 1) / AT_WAVES), 64 * AT_WAVES, 0, (hipStream_t) st>>>(qg, kc, vc, acc, mz, nq, nkv, T,
                                                                                                           nsplit, pos0);
-    k_attn_combine<<<dim3(nq, T), AT_HD, 0, (hipStream_t) st>>>(qg, acc, mz, out, nq, nsplit);
+    k_attn_combine<<<dim3(nq, T), AT_HD, 0, (hipStream_t) st>>>(qg, acc, mz, out, nq, nsplit, T, pos0);
     return launch_status("attn");
 }
 static int dec_ws_check(const fnx_dec_ws* ws, const char* who) {
@@ -1052,11 +1059,11 @@ static int dec_ws_check(const fnx_dec_ws* ws, const char* who) {
         return fail(std::string(who) + ": incomplete workspace");
     return 0;
 }
-// x (ws->x) through one layer, in place
-static int dec_layer(const fnx_decoder* D, const fnx_dec_layer* L, int T, const int* pos0, const fnx_dec_ws* ws, void* st) {
+// x (ws->x) through one layer, in place. pending (may be null): rows still to be added to x first (the layer before's
+// MoE output); the layer's own MoE output is left in ws->o, to be added by whatever comes next
+static int dec_layer(const fnx_decoder* D, const fnx_dec_layer* L, int T, const int* pos0, const fnx_dec_ws* ws, const float* pending, void* st) {
     const int n = D->n, nq = D->nq, nkv = D->nkv;
-    if (fnx_rms_norm_rows(ws->x, L->attn_norm, ws->xn, T, n, D->eps, st)) return 1;
-    if (fnx_quantize_q8_1(ws->xn, ws->xq, n, T, st)) return 1;
+    if (fnx_add_norm_q8(ws->x, pending, L->attn_norm, nullptr, ws->xq, T, n, D->eps, st)) return 1;
     {   // q, k and v in one launch (engine.cu:1547-1552)
         const fnx_q8s* w3[3] = {&L->wq, &L->wk, &L->wv};
         float* const o3[3] = {ws->qg, ws->k, ws->v};
@@ -1067,20 +1074,21 @@ static int dec_layer(const fnx_decoder* D, const fnx_dec_layer* L, int T, const 
     if (fnx_attn(ws->qg, L->kc, L->vc, ws->att, nq, nkv, pos0, T, D->max_ctx, ws->attn_scratch, st)) return 1;
     if (fnx_quantize_q8_1(ws->att, ws->xq, nq * AT_HD, T, st)) return 1;
     if (fnx_q8s_gemv(&L->wo, ws->xq, ws->o, n, T, st)) return 1;
-    if (fnx_add_rows(ws->x, ws->o, ws->x, (size_t) T * n, st)) return 1;
-    if (fnx_rms_norm_rows(ws->x, L->ffn_norm, ws->xn, T, n, D->eps, st)) return 1;
-    if (fnx_moe_verify_layer(&L->moe, ws->xn, T, ws->o, &ws->moe, st)) return 1;
-    return fnx_add_rows(ws->x, ws->o, ws->x, (size_t) T * n, st);
+    if (fnx_add_norm_q8(ws->x, ws->o, L->ffn_norm, ws->xn, nullptr, T, n, D->eps, st)) return 1;
+    return fnx_moe_verify_layer(&L->moe, ws->xn, T, ws->o, &ws->moe, st);
 }
 static int dec_shape_check(const fnx_decoder* D, int T, const char* who) {
-    if (D->n < 256 || D->n % 256 || D->nq < 1 || D->nkv < 1 || D->nq % D->nkv || D->nq / D->nkv > AT_MAXQ || D->vocab < 1 || D->max_ctx < 1)
+    if (D->n < 256 || D->n % 256 || D->n > 4096 || D->nq < 1 || D->nkv < 1 || D->nq % D->nkv || D->nq / D->nkv > AT_MAXQ || D->vocab < 1 ||
+        D->max_ctx < 4 || D->max_ctx % 4)
         return fail(std::string(who) + ": bad model shape");
     if (T < 1 || T > FNX_MAXT) return fail(std::string(who) + ": T out of range");
     return 0;
 }
-static int dec_head(const fnx_decoder* D, const float* norm, const fnx_q8s* head, int T, const fnx_dec_ws* ws, void* st) {
-    if (fnx_rms_norm_rows(ws->x, norm, ws->xn, T, D->n, D->eps, st)) return 1;
-    if (fnx_quantize_q8_1(ws->xn, ws->xq, D->n, T, st)) return 1;
+// x += pending; hidden = x; the output norm, the head, argmax
+static int dec_head(const fnx_decoder* D, const float* norm, const fnx_q8s* head, int T, const fnx_dec_ws* ws, const float* pending, void* st) {
+    if (fnx_add_norm_q8(ws->x, pending, norm, nullptr, ws->xq, T, D->n, D->eps, st)) return 1;
+    if (hipMemcpyAsync(ws->hidden, ws->x, (size_t) T * D->n * sizeof(float), hipMemcpyDeviceToDevice, (hipStream_t) st) != hipSuccess)
+        return fail("decoder: copy of the hidden rows failed");
     if (fnx_q8s_gemv(head, ws->xq, ws->logits, D->vocab, T, st)) return 1;
     return fnx_argmax(ws->logits, D->vocab, T, 0, ws->best_v, ws->best_i, ws->keys, ws->err, st);
 }
@@ -1089,29 +1097,22 @@ int fnx_decoder_verify(const fnx_decoder* D, const int* tokens, int T, const int
     if (dec_shape_check(D, T, "decoder_verify") || dec_ws_check(ws, "decoder_verify")) return 1;
     if (fnx_embed_rows(D->emb, tokens, T, D->vocab, D->n, ws->x, st)) return 1;
     for (int l = 0; l < D->nlayers; ++l)
-        if (dec_layer(D, &D->layers[l], T, pos0, ws, st)) return 1;
-    if (hipMemcpyAsync(ws->hidden, ws->x, (size_t) T * D->n * sizeof(float), hipMemcpyDeviceToDevice, (hipStream_t) st) != hipSuccess)
-        return fail("decoder_verify: copy of the hidden rows failed");
-    return dec_head(D, D->out_norm, &D->head, T, ws, st);
+        if (dec_layer(D, &D->layers[l], T, pos0, ws, l ? ws->o : nullptr, st)) return 1;
+    return dec_head(D, D->out_norm, &D->head, T, ws, D->nlayers ? ws->o : nullptr, st);
 }
 int fnx_mtp_draft(const fnx_decoder* D, const fnx_mtp* M, const float* src, const int* tokens, int T, const int* pos0, const fnx_dec_ws* ws,
                   void* st) {
     if (!D || !M || !src || !tokens || !pos0 || !ws || !M->norm_emb || !M->norm_hid || !M->out_norm || !D->emb) return fail("mtp_draft: null argument");
     if (dec_shape_check(D, T, "mtp_draft") || dec_ws_check(ws, "mtp_draft")) return 1;
     const int n = D->n;
-    // R = fc_hid(rms(src)) + fc_emb(rms(emb))
-    if (fnx_rms_norm_rows(src, M->norm_hid, ws->xn, T, n, D->eps, st)) return 1;
-    if (fnx_quantize_q8_1(ws->xn, ws->xq, n, T, st)) return 1;
+    // R = fc_hid(rms(src)) + fc_emb(rms(emb)): the sum is taken by the layer's first pass over the rows
+    if (fnx_add_norm_q8(const_cast<float*>(src), nullptr, M->norm_hid, nullptr, ws->xq, T, n, D->eps, st)) return 1;   // nothing to add: src is only read
     if (fnx_q8s_gemv(&M->fc_hid, ws->xq, ws->x, n, T, st)) return 1;
-    if (fnx_embed_rows(D->emb, tokens, T, D->vocab, n, ws->o, st)) return 1;
-    if (fnx_rms_norm_rows(ws->o, M->norm_emb, ws->xn, T, n, D->eps, st)) return 1;
-    if (fnx_quantize_q8_1(ws->xn, ws->xq, n, T, st)) return 1;
+    if (fnx_embed_rows(D->emb, tokens, T, D->vocab, n, ws->xn, st)) return 1;
+    if (fnx_add_norm_q8(ws->xn, nullptr, M->norm_emb, nullptr, ws->xq, T, n, D->eps, st)) return 1;
     if (fnx_q8s_gemv(&M->fc_emb, ws->xq, ws->o, n, T, st)) return 1;
-    if (fnx_add_rows(ws->x, ws->o, ws->x, (size_t) T * n, st)) return 1;
-    if (dec_layer(D, &M->layer, T, pos0, ws, st)) return 1;
-    if (hipMemcpyAsync(ws->hidden, ws->x, (size_t) T * n * sizeof(float), hipMemcpyDeviceToDevice, (hipStream_t) st) != hipSuccess)
-        return fail("mtp_draft: copy of the hidden rows failed");
-    return dec_head(D, M->out_norm, &M->head, T, ws, st);
+    if (dec_layer(D, &M->layer, T, pos0, ws, ws->o, st)) return 1;
+    return dec_head(D, M->out_norm, &M->head, T, ws, ws->o, st);
 }
 
 }  // extern "C"

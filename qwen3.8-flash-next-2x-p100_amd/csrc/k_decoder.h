@@ -23,6 +23,43 @@ __global__ void __launch_bounds__(256) k_rms_norm_rows(const float* __restrict__
     const float r = rsqrtf((sh[0] + sh[1] + sh[2] + sh[3]) / (float) n + eps);
     for (int i = threadIdx.x; i < n; i += 256) y[(size_t) blockIdx.x * n + i] = xr[i] * r * w[i];
 }
+// x[r] += add[r] (add may be null); xn[r] = rms_norm(x[r]) * w; xq[r] = q8_1(xn[r]) (either may be null): the residual add,
+// the norm and the quantisation that follow one another between a layer's halves, in one pass over the row. The sums
+// run in k_rms_norm_rows' and k_quantize_q8_1's orders, so the results are theirs bit for bit.
+constexpr int NQ_MAXJ = 16;   // rows of up to 4096 values
+__global__ void __launch_bounds__(256) k_add_norm_q8(float* __restrict__ x, const float* __restrict__ add, const float* __restrict__ w,
+                                                    float* __restrict__ xn, uint8_t* __restrict__ xq, int n, float eps) {
+    __shared__ float sh[4];
+    const size_t row = blockIdx.x;
+    float v[NQ_MAXJ];
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < NQ_MAXJ; ++j) {
+        const int i = threadIdx.x + 256 * j;
+        v[j] = 0.f;
+        if (i < n) {
+            v[j] = x[row * n + i];
+            if (add) {
+                v[j] += add[row * n + i];
+                x[row * n + i] = v[j];
+            }
+            s = fmaf(v[j], v[j], s);
+        }
+    }
+    s = group_sum<64>(s);
+    if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = s;
+    __syncthreads();
+    const float r = rsqrtf((sh[0] + sh[1] + sh[2] + sh[3]) / (float) n + eps);
+#pragma unroll
+    for (int j = 0; j < NQ_MAXJ; ++j) {
+        const int i = threadIdx.x + 256 * j;
+        if (i < n) {   // n is a multiple of 32: the 32 threads of a q8_1 block are live together
+            const float y = v[j] * r * w[i];
+            if (xn) xn[row * n + i] = y;
+            if (xq) q8_1_store(y, xq + (row * (n / 32) + i / 32) * FNX_Q8_1_BLOCK, threadIdx.x & 31);
+        }
+    }
+}
 __global__ void k_add_rows(const float* __restrict__ a, const float* __restrict__ b, float* __restrict__ y, size_t n) {
     for (size_t i = blockIdx.x * (size_t) blockDim.x + threadIdx.x; i < n; i += (size_t) gridDim.x * blockDim.x) y[i] = a[i] + b[i];
 }
@@ -386,20 +423,46 @@ __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per
         *reinterpret_cast<float4*>(acc_out + slot * AT_HD + 16 * dt + 4 * pg) = make_float4(O[dt].x, O[dt].y, O[dt].z, O[dt].w);
     if (pg == 0) mz_out[slot] = AttPart{m, z};
 }
+// a block per (head, row): the splits' weights exp(m_s - max) first (LDS), then every thread sums its dimension over the
+// splits that hold data, several loads in flight
+constexpr int AT_MAXSPLIT = 2048;
 __global__ void __launch_bounds__(AT_HD) k_attn_combine(const float* __restrict__ qg, const float* __restrict__ acc_in,
-                                                       const AttPart* __restrict__ mz_in, float* __restrict__ out, int nq, int nsplit) {
+                                                       const AttPart* __restrict__ mz_in, float* __restrict__ out, int nq, int nsplit, int T,
+                                                       const int* __restrict__ pos0p) {
+    __shared__ float wsp[AT_MAXSPLIT];
+    __shared__ float red[AT_HD / 64];
     const int h = blockIdx.x, t = blockIdx.y, i = threadIdx.x;
     const size_t base = ((size_t) t * nq + h) * nsplit;
+    const int nlive = min(nsplit, (*pos0p + T + AT_SPLIT - 1) / AT_SPLIT);   // splits the window's context reaches: their parts were written
     float mx = -INFINITY;
-    for (int s = 0; s < nsplit; ++s) mx = fmaxf(mx, mz_in[base + s].m);
-    float z = 0.f, acc = 0.f;
-    for (int s = 0; s < nsplit; ++s) {
+    for (int s = i; s < nlive; s += AT_HD) mx = fmaxf(mx, mz_in[base + s].m);
+    mx = group_max<64>(mx);
+    if ((i & 63) == 0) red[i >> 6] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    __syncthreads();
+    float zp = 0.f;
+    for (int s = i; s < nlive; s += AT_HD) {
         const AttPart p = mz_in[base + s];
-        if (p.m == -INFINITY) continue;
-        const float w = expf(p.m - mx);
-        z = fmaf(w, p.z, z);
-        acc = fmaf(w, acc_in[(base + s) * AT_HD + i], acc);
+        const float w = p.m == -INFINITY ? 0.f : expf(p.m - mx);
+        wsp[s] = w;
+        zp = fmaf(w, p.z, zp);
     }
+    zp = group_sum<64>(zp);
+    if ((i & 63) == 0) red[i >> 6] = zp;
+    __syncthreads();
+    const float z = (red[0] + red[1]) + (red[2] + red[3]);
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    const float* ap = acc_in + base * AT_HD + i;
+    int s = 0;
+    for (; s + 4 <= nlive; s += 4) {
+        a0 = fmaf(wsp[s], ap[(size_t) s * AT_HD], a0);
+        a1 = fmaf(wsp[s + 1], ap[(size_t) (s + 1) * AT_HD], a1);
+        a2 = fmaf(wsp[s + 2], ap[(size_t) (s + 2) * AT_HD], a2);
+        a3 = fmaf(wsp[s + 3], ap[(size_t) (s + 3) * AT_HD], a3);
+    }
+    for (; s < nlive; ++s) a0 = fmaf(wsp[s], ap[(size_t) s * AT_HD], a0);
+    const float acc = (a0 + a1) + (a2 + a3);
     out[((size_t) t * nq + h) * AT_HD + i] = acc / z * sigmoid_f(qg[((size_t) t * nq + h) * 2 * AT_HD + AT_HD + i]);
 }
 

@@ -273,6 +273,17 @@ class Dev:
         self.sync()
         return y.cpu().numpy()
 
+    def add_norm_q8(self, x, add, w, eps):
+        t = self.torch
+        rows, n = x.shape
+        dx, dw_ = self.up(x.astype(np.float32)), self.up(w.astype(np.float32))
+        da = self.up(add.astype(np.float32)) if add is not None else None
+        xn, xq = self.zeros((rows, n), t.float32), self.zeros(rows * (n // 32) * 36, t.uint8)
+        self.ok(self.lib.fnx_add_norm_q8(dx.data_ptr(), da.data_ptr() if da is not None else None, dw_.data_ptr(), xn.data_ptr(), xq.data_ptr(),
+                                         rows, n, eps, self.st()))
+        self.sync()
+        return dx.cpu().numpy(), xn.cpu().numpy(), xq.cpu().numpy()
+
     def q8s_gemv(self, q, d, yq, T):
         rows, cols = q.shape
         dq, dd, dy = self.up(q), self.up(d), self.up(yq)

@@ -43,6 +43,19 @@ def test_rms_norm_rows(dev, oracle):
     assert err <= 3e-6 * float(np.abs(want).max()), err
 
 
+@pytest.mark.parametrize("n,with_add", [(2048, True), (2048, False), (4096, True), (96, True)])
+def test_add_norm_q8_equals_the_three_operators(dev, n, with_add):
+    rng = np.random.default_rng(805 + n)
+    x, w = rng.standard_normal((5, n)).astype(np.float32) * 2, rng.standard_normal(n).astype(np.float32)
+    add = rng.standard_normal((5, n)).astype(np.float32) if with_add else None
+    x2, xn, xq = dev.add_norm_q8(x, add, w, 1e-6)
+    want_x = x + add if with_add else x
+    assert np.array_equal(x2, want_x)
+    want_n = dev.rms_norm_rows(want_x, w, 1e-6)
+    assert np.array_equal(xn.view(np.uint32), want_n.view(np.uint32))
+    assert np.array_equal(xq, dev.quantize_q8_1(want_n))
+
+
 @pytest.mark.parametrize("rows,cols,T", [(37, 1024, 3), (1000, 2048, 16), (2048, 4096, 16), (513, 256, 5), (8192, 2048, 1)])
 def test_q8s_gemv_bit_exact(dev, oracle, rows, cols, T):
     print(f"case q8s_gemv rows={rows} cols={cols} T={T}", flush=True)
