@@ -89,4 +89,36 @@ inline int accept_greedy(const std::vector<int>& rows, const std::vector<int>& o
 // load-time re-laying of an IQ3_S tensor (no counterpart in the reference's API; its own load-time layouts are model.hpp:78-82)
 inline void iq3s_repack(const void* src, void* dst, size_t n_weights, void* st) { ck(fnx_iq3s_repack(src, dst, n_weights, st)); }
 
+// ---- the prompt path (prefill.cu:288-377, kernels.hpp:328-330)
+using BigJob = fnx_bigjob;
+inline void pf_route(const float* logits, int C, int* topi, float* topw, int* cnt, int* jbase, BigJob* jobs_gu, BigJob* jobs_dn, int njobs_cap,
+                     int* njobs, void* st) {
+    ck(fnx_pf_route(logits, shape().NEXP + 1, C, shape().NEXP, shape().TOPK, topi, topw, cnt, jbase, jobs_gu, jobs_dn, njobs_cap, njobs, st));
+}
+inline void p100_f32_f16(const float* x, size_t n, uint16_t* out, void* st) { ck(fnx_f32_f16(x, n, out, st)); }
+inline void moe_gate_up_mma(const DW& A, size_t sa, const BigJob* jobs, const int* njobs, int njobs_cap, const uint16_t* xh, float* gu, void* st) {
+    ck(fnx_moe_gate_up_mma(&A, sa, jobs, njobs, njobs_cap, xh, gu, st));
+}
+inline void swiglu_h16(const float* gu, int ffs, int P, uint16_t* h16, void* st) { ck(fnx_swiglu_h16(gu, ffs, P, h16, st)); }
+inline void moe_down_mma(const DW& A, size_t sa, const BigJob* jobs, const int* njobs, int njobs_cap, const uint16_t* h16, float* part, void* st) {
+    ck(fnx_moe_down_mma(&A, sa, jobs, njobs, njobs_cap, h16, part, st));
+}
+// ---- around the MoE half (kernels.hpp:238, 259, 406, 414-418)
+using Q8S = fnx_q8s;
+using Rope = fnx_rope;
+inline void rms_norm_rows(const float* x, const float* w, float* y, int rows, int n, float eps, void* st) { ck(fnx_rms_norm_rows(x, w, y, rows, n, eps, st)); }
+inline void q8s_gemv(const Q8S& w, const void* y, float* out, int out_stride, int T, void* st) { ck(fnx_q8s_gemv(&w, y, out, out_stride, T, st)); }
+inline void q8s_gemv_segs(const Q8S* w, float* const* out, const int* out_stride, int n, const void* y, int T, void* st) {
+    const Q8S* p[3] = {&w[0], n > 1 ? &w[1] : nullptr, n > 2 ? &w[2] : nullptr};
+    ck(fnx_q8s_gemv_segs(p, out, out_stride, n, y, T, st));
+}
+inline void attn_prep_append(float* qg, float* k, const float* v, const float* q_norm, const float* k_norm, uint16_t* kc, uint16_t* vc, int nq,
+                             int nkv, int T, const int* pos0, int max_ctx, float eps, const Rope& base, void* st) {
+    ck(fnx_attn_prep_append(qg, k, v, q_norm, k_norm, kc, vc, nq, nkv, T, pos0, max_ctx, eps, &base, st));
+}
+inline void attn(const float* qg, const uint16_t* kc, const uint16_t* vc, float* out, int nq, int nkv, const int* pos0, int T, int max_ctx,
+                 float* scratch, void* st) {
+    ck(fnx_attn(qg, kc, vc, out, nq, nkv, pos0, T, max_ctx, scratch, st));
+}
+
 }  // namespace fnx
