@@ -487,27 +487,60 @@ __device__ __forceinline__ unsigned fkey(float v) {
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 __device__ __forceinline__ float fkey_inv(unsigned k) { return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k); }
-constexpr int AM_THREADS = 256, AM_PER_BLOCK = 4096;
-// keys[t] = max over the row of (fkey(value) << 32 | ~index): the greatest value, the lower index on a tie
+constexpr int AM_THREADS = 1024, AM_PER_BLOCK = 16384;
+// keys[t] = max over the row of (fkey(value) << 32 | ~index): the greatest value, the lower index on a tie. A block
+// folds its 16,384 values to one key (four independent 16-byte loads a thread, wave butterflies, LDS) and issues one
+// atomic: atomics on one address serialise, and a row's address would otherwise take one per wave.
 __global__ void __launch_bounds__(AM_THREADS) k_argmax(const float* __restrict__ logits, int rows, unsigned long long* __restrict__ keys,
                                                       unsigned* __restrict__ err) {
-    const int t = blockIdx.y, i0 = blockIdx.x * AM_PER_BLOCK, i1 = min(rows, i0 + AM_PER_BLOCK);
+    __shared__ unsigned long long wbest[AM_THREADS / 64];
+    __shared__ int wbad;
+    const int t = blockIdx.y, i0 = blockIdx.x * AM_PER_BLOCK, i1 = min(rows, i0 + AM_PER_BLOCK), tid = threadIdx.x;
     const float* r = logits + (size_t) t * rows;
+    if (tid == 0) wbad = 0;
     unsigned long long best = 0;
     bool bad = false;
-    for (int i = i0 + threadIdx.x; i < i1; i += AM_THREADS) {
-        const float v = r[i];
+    auto take = [&](float v, int i) {
         bad = bad || !isfinite(v);
         const unsigned long long k = (unsigned long long) fkey(v) << 32 | (unsigned) ~i;
         best = k > best ? k : best;
+    };
+    if ((((uintptr_t) r) & 15) == 0 && (i0 & 3) == 0) {
+        float4 v[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int i = i0 + 4 * (tid + AM_THREADS * j);
+            v[j] = i + 3 < i1 ? *reinterpret_cast<const float4*>(r + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int i = i0 + 4 * (tid + AM_THREADS * j);
+            if (i + 3 < i1) {
+                take(v[j].x, i);
+                take(v[j].y, i + 1);
+                take(v[j].z, i + 2);
+                take(v[j].w, i + 3);
+            } else {
+                for (int k = i; k < i1; ++k) take(r[k], k);
+            }
+        }
+    } else {
+        for (int i = i0 + tid; i < i1; i += AM_THREADS) take(r[i], i);
     }
-    if (bad) atomicOr(err, FNX_ERR_NONFINITE);
 #pragma unroll
     for (int o = 32; o; o >>= 1) {
         const unsigned long long ok = __shfl_xor(best, o, 64);
         best = ok > best ? ok : best;
     }
-    if ((threadIdx.x & 63) == 0) atomicMax(&keys[t], best);
+    __syncthreads();
+    if (bad) wbad = 1;
+    if ((tid & 63) == 0) wbest[tid >> 6] = best;
+    __syncthreads();
+    if (tid == 0) {
+        for (int w = 1; w < AM_THREADS / 64; ++w) best = wbest[w] > best ? wbest[w] : best;
+        atomicMax(&keys[t], best);
+        if (wbad) atomicOr(err, FNX_ERR_NONFINITE);
+    }
 }
 // decodes the keys into (value, index + v0) and leaves them at zero for the next argmax
 __global__ void k_argmax_fin(unsigned long long* keys, int T, int v0, float* bv, int* bi) {
@@ -533,10 +566,32 @@ __global__ void __launch_bounds__(LK_THREADS) k_lookup(const int* __restrict__ c
         int key[4];
         for (int j = 0; j < key_n; ++j) key[j] = ctx[n0 + j];
         int mine = -1;
-        for (int s = threadIdx.x; s < n0; s += LK_THREADS) {
-            bool eq = true;
-            for (int j = 0; j < key_n; ++j) eq = eq && ctx[s + j] == key[j];
-            if (eq) mine = s;   // ascending s: the last one kept is this thread's greatest
+        if ((((uintptr_t) ctx) & 15) == 0) {
+            // four start positions a step: the 4 + 3 tokens they need are two 16-byte loads; steps are independent
+            for (int s4 = 4 * threadIdx.x; s4 < n0; s4 += 4 * LK_THREADS) {
+                int4 a = make_int4(0, 0, 0, 0), b = make_int4(0, 0, 0, 0);
+                if (s4 + 3 < n_ctx) a = *reinterpret_cast<const int4*>(ctx + s4);
+                else
+                    for (int j = 0; j < 4 && s4 + j < n_ctx; ++j) (&a.x)[j] = ctx[s4 + j];
+                if (s4 + 7 < n_ctx) b = *reinterpret_cast<const int4*>(ctx + s4 + 4);
+                else
+                    for (int j = 0; j < 4 && s4 + 4 + j < n_ctx; ++j) (&b.x)[j] = ctx[s4 + 4 + j];
+                const int w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    bool eq = s4 + i < n0;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        if (j < key_n) eq = eq && w[i + j] == key[j];
+                    if (eq) mine = s4 + i;   // ascending: the last one kept is this thread's greatest
+                }
+            }
+        } else {
+            for (int s = threadIdx.x; s < n0; s += LK_THREADS) {
+                bool eq = true;
+                for (int j = 0; j < key_n; ++j) eq = eq && ctx[s + j] == key[j];
+                if (eq) mine = s;   // ascending s: the last one kept is this thread's greatest
+            }
         }
 #pragma unroll
         for (int o = 32; o; o >>= 1) mine = max(mine, __shfl_xor(mine, o, 64));
