@@ -961,6 +961,14 @@ static int mma_launch(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const 
     if (njobs_cap < 1) return fail(std::string(who) + ": no jobs");
     MmaArgs a{(const uint8_t*) A->p, sa, A->ep, A->n_out, A->n_in, jobs, njobs, njobs_cap, x, A->n_in, out};
     static const int per_cu = env_int("FNX_MMA_BLOCKS_PER_CU", 2, 1, 8), form = env_int("FNX_MMA_FORM", 1, 0, 1);
+    static const int tile = env_int("FNX_MMA_TILE", 1, 0, 2);   // 0: never, 1: rows of up to 512 columns, 2: always
+    if (tile && A->type == FNX_T_IQ3S_UNIT64 && A->n_out % 16 == 0 && (tile == 2 || A->n_in <= 512)) {
+        // tile form: a block per (job, 32 tokens, 256 rows) in stages of 256 columns, one block a CU (its LDS)
+        const long tasks = (long) njobs_cap * ((A->n_out + MB_ROWS - 1) / MB_ROWS) * (MM_TT / MM_TP);
+        const int grid = (int) std::max(1l, std::min<long>((long) cu_count(), tasks));
+        k_moe_mma_tile<<<grid, MM_THREADS, 0, (hipStream_t) st>>>(a);
+        return launch_status(who);
+    }
     if (form == 1 && A->type == FNX_T_IQ3S_UNIT64 && A->n_in % 512 == 0 && A->n_out % 16 == 0) {
         // block form: a block per (job, 32 tokens, 256 rows)
         const long tasks = (long) njobs_cap * ((A->n_out + MB_ROWS - 1) / MB_ROWS) * (MM_TT / MM_TP);

@@ -272,7 +272,6 @@ __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per
                                                             AttPart* __restrict__ mz_out, int nq, int nkv, int T, int nsplit,
                                                             const int* __restrict__ pos0p) {
     typedef __attribute__((address_space(1))) const at_v4u g128;
-    typedef __attribute__((address_space(1))) const at_v2u g64;
     const int s = blockIdx.x, kvh = blockIdx.y, lane = threadIdx.x & 63, wave = blockIdx.z * AT_WAVES + (threadIdx.x >> 6);
     const int qpk = nq / nkv, nquery = T * qpk, pos0 = *pos0p;
     const int ql = lane & 15, pg = lane >> 4;

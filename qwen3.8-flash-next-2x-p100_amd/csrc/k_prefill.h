@@ -466,4 +466,254 @@ __global__ void __launch_bounds__(MM_THREADS) k_moe_mma_block(const MmaArgs a) {
     }
 }
 
+// ---------------------------------------------------------------- the same products, tile form (unit64 weights, short rows)
+// With rows of 512 columns or fewer (the down projection) a task of the block form is one super-step: all prologue,
+// a chain of three dependent loads (job, token row number, activations) before any arithmetic. Here a block first puts
+// its tasks (the valid ones only), their expert pointers and their token / output row numbers in LDS; after that the
+// steady state has no dependent global loads and stages run across task boundaries. Nothing is loaded per lane either:
+// a stage (256 columns of 256 rows, 32 tokens) comes in as whole runs of the planes - consecutive lanes read consecutive
+// 16 bytes - through registers into LDS a stage ahead, next to the activation tile, and a lane reads its row's fields
+// from there. LDS reads run one unit (a sub-block of 16 rows: 8 gathers -> 4 A operands -> up to 8 MFMAs) ahead of the
+// arithmetic. Measured on MI355X for the down projection of 512 columns: 71 us against 94 us for the block form; with
+// rows of 2048 columns the block form's four barriers a task beat this form's eight (132 us against 140 us).
+constexpr int MT_K = 256;                  // columns per stage: 8 sub-blocks a row, two per lane
+constexpr int MT_WROW = 112;               // bytes per row record: A 64 | B 32 | C 8 | scales 4 | d 2 | pad (28 words: 16-byte reads of 16 rows hit 64 banks once)
+constexpr int MT_XROW = 2 * MT_K + 16;     // bytes per token of the activation tile (132 words: likewise)
+constexpr int MT_MAXTASK = 16;
+struct TileTask {
+    const uint8_t* we;
+    int t0, row0, ntile;
+};
+struct TileLds {
+    uint2 tab[SGRID_WORDS];
+    uint8_t wt[2][MB_ROWS * MT_WROW];
+    uint8_t xt[2][MB_TOK * MT_XROW];
+    int ytok[MT_MAXTASK][MB_TOK];      // activation row of each token of the task's tile (clamped to the job's last)
+    int otok[MT_MAXTASK][MB_TOK];      // its output row, or -1 past the job's end
+    TileTask task[MT_MAXTASK];
+    int ntask;
+};
+struct TileStaged {   // one thread's share of a stage, as loaded
+    v4u a[2], b, x[2];
+    v2u cs;
+};
+struct TileFields {   // a lane's two sub-blocks of one row
+    v4u A;
+    v2u B;
+    uint32_t C, sc, d;
+};
+__global__ void __launch_bounds__(MM_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) k_moe_mma_tile(const MmaArgs a) {
+    typedef __attribute__((address_space(1))) const v4u g128;
+    typedef __attribute__((address_space(1))) const v2u g64;
+    typedef __attribute__((address_space(1))) const uint32_t g32;
+    typedef __attribute__((address_space(1))) const unsigned short g16;
+    __shared__ TileLds L;
+    const int tid = threadIdx.x, lane = tid & 63, wave = uniform(tid >> 6), r = lane & 15, g = lane >> 4;
+    uint32_t treg[SGRID_WORDS / MM_THREADS];
+#pragma unroll
+    for (int i = 0; i < SGRID_WORDS / MM_THREADS; ++i) treg[i] = g_sgrid.v[tid + i * MM_THREADS];
+    const int nj = min(a.cap, uniform(*a.njobs));
+    const int ks = a.ncols >> 5, nsuper = a.ncols / MT_K, rblocks = (a.nrows + MB_ROWS - 1) / MB_ROWS;
+    constexpr int HALVES = MM_TT / MM_TP;
+    const int per_job = rblocks * HALVES, ntasks_all = nj * per_job;
+#pragma unroll
+    for (int i = 0; i < SGRID_WORDS / MM_THREADS; ++i) {
+        const uint32_t gg = treg[i];
+        v2h lo, hi;
+        lo.x = (_Float16) (int) (int8_t) (gg & 0xFFu);
+        lo.y = (_Float16) (int) (int8_t) ((gg >> 8) & 0xFFu);
+        hi.x = (_Float16) (int) (int8_t) ((gg >> 16) & 0xFFu);
+        hi.y = (_Float16) (int) (int8_t) (gg >> 24);
+        L.tab[tid + i * MM_THREADS] = make_uint2(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi));
+    }
+    for (int k0 = blockIdx.x; k0 < ntasks_all; k0 += gridDim.x * MT_MAXTASK) {
+        __syncthreads();   // the previous lists' last readers; the table on the first pass
+        if (wave == 0) {
+            const int task = k0 + lane * gridDim.x;
+            bool ok = lane < MT_MAXTASK && task < ntasks_all;
+            TileTask t{};
+            int ji = 0, n = 0;
+            if (ok) {
+                ji = task / per_job;
+                const int rem = task - ji * per_job;
+                t.t0 = (rem / rblocks) * MM_TP;
+                t.row0 = (rem % rblocks) * MB_ROWS;
+                const fnx_bigjob* jb = a.jobs + ji;
+                n = min(FNX_PF_JOB, jb->n);
+                const int e = jb->w;
+                ok = n >= 1 && t.t0 < ((n + 15) >> 4);
+                t.ntile = min(MM_TP, ((n + 15) >> 4) - t.t0);
+                if (ok) t.we = a.ep ? (const uint8_t*) a.ep[e] : a.w + (size_t) e * a.stride;
+            }
+            const unsigned long long m = __ballot(ok);
+            const int slot = __popcll(m & ((1ull << lane) - 1ull));
+            if (ok) {
+                L.task[slot] = t;
+                // the tile's token and output rows: 32 of each
+                const fnx_bigjob* jb = a.jobs + ji;
+                for (int j = 0; j < MB_TOK; ++j) {
+                    const int tok = t.t0 * 16 + j;
+                    L.ytok[slot][j] = jb->y[min(tok, n - 1)];
+                    L.otok[slot][j] = tok < n ? jb->out[tok] : -1;
+                }
+            }
+            if (lane == 0) L.ntask = __popcll(m);
+        }
+        __syncthreads();
+        const int ntask = L.ntask;
+        if (ntask == 0) continue;   // the same for every thread of the block
+        const int nst = ntask * nsuper;
+        auto issue = [&](int ti, int S) {
+            const TileTask t = L.task[ti];
+            auto unit_of = [&](int rowl, uint32_t& l0) {
+                const int row = min(t.row0 + rowl, a.nrows - 1);
+                const uint32_t Lq = (uint32_t) row * ks + 8 * S;
+                l0 = Lq & 63u;
+                return as_global(t.we + (size_t) (Lq >> 6) * UNIT_BYTES);
+            };
+            TileStaged o;
+            uint32_t l0;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const int c = tid + i * MM_THREADS;
+                const gbytes u = unit_of(c >> 2, l0);
+                o.a[i] = *(g128*) (u + 8 * l0 + 16 * (c & 3));
+            }
+            {
+                const gbytes u = unit_of(tid >> 1, l0);
+                o.b = *(g128*) (u + UNIT_B_AT + 4 * l0 + 16 * (tid & 1));
+            }
+            if (wave < MM_WAVES / 2) {
+                const gbytes u = unit_of(tid, l0);
+                o.cs = *(g64*) (u + UNIT_C_AT + l0);
+            } else {
+                const gbytes u = unit_of(tid - MM_THREADS / 2, l0);
+                o.cs.x = *(g32*) (u + UNIT_SCALES_AT + (l0 >> 1));
+                o.cs.y = *(g16*) (u + UNIT_D_AT + 2 * (l0 >> 3));
+            }
+            const g128* xp = (g128*) (uintptr_t) (a.x + (size_t) L.ytok[ti][tid >> 4] * a.ldx + S * MT_K + 8 * (tid & 15));
+            o.x[0] = xp[0];
+            o.x[1] = xp[16];   // + 256 bytes
+            return o;
+        };
+        auto stash = [&](const TileStaged& o, int buf) {
+            uint8_t* w = L.wt[buf];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const int c = tid + i * MM_THREADS;
+                *reinterpret_cast<v4u*>(w + (c >> 2) * MT_WROW + 16 * (c & 3)) = o.a[i];
+            }
+            *reinterpret_cast<v4u*>(w + (tid >> 1) * MT_WROW + 64 + 16 * (tid & 1)) = o.b;
+            if (wave < MM_WAVES / 2) *reinterpret_cast<v2u*>(w + tid * MT_WROW + 96) = o.cs;
+            else {
+                *reinterpret_cast<uint32_t*>(w + (tid - MM_THREADS / 2) * MT_WROW + 104) = o.cs.x;
+                *reinterpret_cast<uint16_t*>(w + (tid - MM_THREADS / 2) * MT_WROW + 108) = (uint16_t) o.cs.y;
+            }
+            uint8_t* x = L.xt[buf] + (tid >> 4) * MT_XROW + 16 * (tid & 15);
+            *reinterpret_cast<v4u*>(x) = o.x[0];
+            *reinterpret_cast<v4u*>(x + 256) = o.x[1];
+        };
+        v4f acc[MB_RG][MM_TP];
+#pragma unroll
+        for (int q = 0; q < MB_RG; ++q)
+#pragma unroll
+            for (int tt = 0; tt < MM_TP; ++tt) acc[q][tt] = v4f{0.f, 0.f, 0.f, 0.f};
+        struct Gath {
+            uint2 e[8];
+        };
+        auto gather = [&](const TileFields& f, int p, Gath& o) {
+            const v4u idx = {f.A[2 * p], f.A[2 * p + 1], f.B[p], (f.C >> (8 * p)) & 0xFFu};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) o.e[j] = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint8_t*>(L.tab) + 2 * packed_addr(idx, j));
+        };
+        auto bread = [&](int buf, int p, v4u (&B)[MM_TP][4], auto nt_tag) {
+#pragma unroll
+            for (int tt = 0; tt < decltype(nt_tag)::value; ++tt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) B[tt][i] = *reinterpret_cast<const v4u*>(&L.xt[buf][(tt * 16 + r) * MT_XROW + 128 * g + 64 * p + 16 * i]);
+        };
+        auto math = [&](const TileFields& f, int p, int q, const Gath& in, const v4u (&B)[MM_TP][4], auto nt_tag) {
+            const _Float16 sc = (_Float16) (int) (1 + 2 * ((f.sc >> (4 * p)) & 0xFu)), d = __builtin_bit_cast(_Float16, (unsigned short) f.d);
+            const v2h s2 = {sc, sc}, d2 = {d, d};
+            v8h A[4];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const v2h wl = (as_v2h(in.e[j].x) * s2) * d2, wh = (as_v2h(in.e[j].y) * s2) * d2;
+                A[j >> 1][4 * (j & 1) + 0] = wl.x;
+                A[j >> 1][4 * (j & 1) + 1] = wl.y;
+                A[j >> 1][4 * (j & 1) + 2] = wh.x;
+                A[j >> 1][4 * (j & 1) + 3] = wh.y;
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int tt = 0; tt < decltype(nt_tag)::value; ++tt)
+                    acc[q][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[i], __builtin_bit_cast(v8h, B[tt][i]), acc[q][tt], 0, 0, 0);
+        };
+        auto compute = [&](int buf, auto nt_tag) {
+            const uint8_t* w = L.wt[buf];
+            TileFields f[MB_RG];
+#pragma unroll
+            for (int q = 0; q < MB_RG; ++q) {
+                const uint8_t* rec = w + (wave * 16 * MB_RG + 16 * q + r) * MT_WROW;
+                f[q].A = *reinterpret_cast<const v4u*>(rec + 16 * g);
+                f[q].B = *reinterpret_cast<const v2u*>(rec + 64 + 8 * g);
+                f[q].C = *reinterpret_cast<const uint16_t*>(rec + 96 + 2 * g);
+                f[q].sc = rec[104 + g];
+                f[q].d = *reinterpret_cast<const uint16_t*>(rec + 108);
+            }
+            Gath G[2];
+            v4u Bb[2][MM_TP][4];
+            bread(buf, 0, Bb[0], nt_tag);
+            gather(f[0], 0, G[0]);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int p = u >> 1, q = u & 1;
+                if (u == 1) bread(buf, 1, Bb[1], nt_tag);
+                if (u < 3) gather(f[(u + 1) & 1], (u + 1) >> 1, G[(u + 1) & 1]);
+                __builtin_amdgcn_sched_barrier(0);
+                math(f[q], p, q, G[u & 1], Bb[p], nt_tag);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+        TileStaged st = issue(0, 0);
+        int ti = 0, S = 0;
+        for (int s = 0; s < nst; ++s) {
+            stash(st, s & 1);
+            __syncthreads();
+            int tn = ti, Sn = S + 1;
+            if (Sn == nsuper) {
+                Sn = 0;
+                ++tn;
+            }
+            if (s + 1 < nst) st = issue(tn, Sn);
+            const int row0 = L.task[ti].row0 + wave * 16 * MB_RG;
+            if (row0 < a.nrows) {   // per wave
+                if (L.task[ti].ntile > 1) compute(s & 1, std::integral_constant<int, 2>{});
+                else compute(s & 1, std::integral_constant<int, 1>{});
+                if (Sn == 0) {
+                    // lane: token r of each tile, weight rows 4 g .. 4 g + 3 of each group
+#pragma unroll
+                    for (int tt = 0; tt < MM_TP; ++tt) {
+                        const int orow = L.otok[ti][tt * 16 + r];
+                        if (orow >= 0) {
+                            float* o = a.out + (size_t) orow * a.nrows + row0 + 4 * g;
+#pragma unroll
+                            for (int q = 0; q < MB_RG; ++q)
+                                if (row0 + 16 * q < a.nrows) *reinterpret_cast<float4*>(o + 16 * q) = make_float4(acc[q][tt].x, acc[q][tt].y, acc[q][tt].z, acc[q][tt].w);
+                        }
+                    }
+#pragma unroll
+                    for (int q = 0; q < MB_RG; ++q)
+#pragma unroll
+                        for (int tt = 0; tt < MM_TP; ++tt) acc[q][tt] = v4f{0.f, 0.f, 0.f, 0.f};
+                }
+            }
+            ti = tn;
+            S = Sn;
+        }
+    }
+}
+
+
 }  // namespace fnx
