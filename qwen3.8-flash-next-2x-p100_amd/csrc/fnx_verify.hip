@@ -752,9 +752,16 @@ static int gemv_any(const void* W, bool bf, const float* x, float* y, int rows, 
     if (!W || !x || !y) return fail(std::string(who) + ": null argument");
     if (rows <= 0 || n <= 0 || n % 256) return fail(std::string(who) + ": n must be a positive multiple of 256");
     if (T < 1 || T > 65535 * FNX_MAXT) return fail(std::string(who) + ": T out of range");
+    hipStream_t s = (hipStream_t) st;
+    if (T > FNX_MAXT) {   // many rows of x: GR_ROWS weight rows a wave
+        const dim3 gm((rows + GM_WAVES * GR_ROWS - 1) / (GM_WAVES * GR_ROWS), (T + FNX_MAXT - 1) / FNX_MAXT);
+        if (bf) k_gemv_rows_many<true><<<gm, GM_WAVES * 64, 0, s>>>(W, x, y, rows, n, T);
+        else k_gemv_rows_many<false><<<gm, GM_WAVES * 64, 0, s>>>(W, x, y, rows, n, T);
+        return launch_status(who);
+    }
     const dim3 grid((rows + GV_WAVES - 1) / GV_WAVES, (T + FNX_MAXT - 1) / FNX_MAXT);
-    if (bf) k_gemv_rows<true><<<grid, GV_WAVES * 64, 0, (hipStream_t) st>>>(W, x, y, rows, n, T);
-    else k_gemv_rows<false><<<grid, GV_WAVES * 64, 0, (hipStream_t) st>>>(W, x, y, rows, n, T);
+    if (bf) k_gemv_rows<true><<<grid, GV_WAVES * 64, 0, s>>>(W, x, y, rows, n, T);
+    else k_gemv_rows<false><<<grid, GV_WAVES * 64, 0, s>>>(W, x, y, rows, n, T);
     return launch_status(who);
 }
 int fnx_gemv_f32(const float* W, const float* x, float* y, int rows, int n, int T, void* st) {

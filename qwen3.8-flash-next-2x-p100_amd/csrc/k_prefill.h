@@ -124,6 +124,86 @@ __global__ void k_swiglu_h16(const float* __restrict__ gu, int ffs, size_t total
     }
 }
 
+// ---------------------------------------------------------------- router logits of a chunk
+// The same sums for many activation rows (the prompt path's router logits): a wave takes GR_ROWS weight rows x a group
+// of FNX_MAXT activation rows, lane l the float4 chunks l, l + 64, ... of all of them, so every activation chunk it
+// loads (coalesced, straight from the caches: no LDS, no barriers) feeds GR_ROWS chains. Order per sum as above.
+constexpr int GM_WAVES = 8, GR_ROWS = 4, GM_BATCH = 8;
+static_assert(GR_ROWS * FNX_MAXT == 64, "64 sums a wave, one per lane in the end");
+template <bool BF>
+__global__ void __launch_bounds__(GM_WAVES * 64) k_gemv_rows_many(const void* __restrict__ Wv, const float* __restrict__ x, float* __restrict__ y,
+                                                                 int rows, int n, int T) {
+    x += (size_t) blockIdx.y * FNX_MAXT * n;
+    y += (size_t) blockIdx.y * FNX_MAXT * rows;
+    T = min(FNX_MAXT, T - (int) blockIdx.y * FNX_MAXT);
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int row0 = (blockIdx.x * GM_WAVES + wave) * GR_ROWS;
+    if (row0 >= rows) return;
+    float acc[GR_ROWS][FNX_MAXT];
+#pragma unroll
+    for (int r = 0; r < GR_ROWS; ++r)
+#pragma unroll
+        for (int t = 0; t < FNX_MAXT; ++t) acc[r][t] = 0.f;
+    const float4* xr[FNX_MAXT];
+#pragma unroll
+    for (int t = 0; t < FNX_MAXT; ++t) xr[t] = reinterpret_cast<const float4*>(x + (size_t) min(t, T - 1) * n) + lane;
+    for (int c0 = 0; c0 < n / 4; c0 += 64) {
+        float4 w[GR_ROWS];
+#pragma unroll
+        for (int r = 0; r < GR_ROWS; ++r) {
+            const size_t row = (size_t) min(row0 + r, rows - 1);
+            if constexpr (BF) {
+                const uint2 u = reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(Wv) + row * n)[c0 + lane];
+                w[r] = make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u), __uint_as_float(u.y << 16),
+                                   __uint_as_float(u.y & 0xffff0000u));
+            } else {
+                w[r] = reinterpret_cast<const float4*>(reinterpret_cast<const float*>(Wv) + row * n)[c0 + lane];
+            }
+        }
+        // GM_BATCH activation chunks in flight at a time (left to itself the compiler loads them one by one, each a cache
+        // round trip before its 16 fmaf)
+#pragma unroll
+        for (int t0 = 0; t0 < FNX_MAXT; t0 += GM_BATCH) {
+            float4 b[GM_BATCH];
+#pragma unroll
+            for (int t = 0; t < GM_BATCH; ++t) b[t] = xr[t0 + t][c0];
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int t = 0; t < GM_BATCH; ++t)
+#pragma unroll
+                for (int r = 0; r < GR_ROWS; ++r) {
+                    float a = acc[r][t0 + t];
+                    a = fmaf(w[r].x, b[t].x, a);
+                    a = fmaf(w[r].y, b[t].y, a);
+                    a = fmaf(w[r].z, b[t].z, a);
+                    a = fmaf(w[r].w, b[t].w, a);
+                    acc[r][t0 + t] = a;
+                }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    // The 64 sums (value j = 16 r + t) over the 64 lanes, all at once: at the butterfly's level for lane bit b a lane
+    // keeps the half of its values whose index has bit b equal to its own and adds its partner's copy of them - the
+    // same pairwise adds, level by level, as group_sum<64> makes for each value, in 63 exchanges instead of 384.
+    // Lane l ends with value l.
+    float v32[32], v16[16], v8[8];
+#pragma unroll
+    for (int i = 0; i < 32; ++i) v32[i] = swap32_add(acc[i >> 4][i & 15], acc[2 + (i >> 4)][i & 15]);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) v16[i] = swap16_add(v32[i], v32[i + 16]);
+    auto fold = [&](const float lo, const float hi, int o) {
+        const bool up = lane & o;
+        return (up ? hi : lo) + __shfl_xor(up ? lo : hi, o, WAVE);
+    };
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v8[i] = fold(v16[i], v16[i + 8], 8);
+    const float a0 = fold(v8[0], v8[4], 4), a1 = fold(v8[1], v8[5], 4), a2 = fold(v8[2], v8[6], 4), a3 = fold(v8[3], v8[7], 4);
+    const float b0 = fold(a0, a2, 2), b1 = fold(a1, a3, 2);
+    const float v = fold(b0, b1, 1);
+    const int r = lane >> 4, t = lane & 15;
+    if (t < T && row0 + r < rows) y[(size_t) t * rows + row0 + r] = v;
+}
+
 // ---------------------------------------------------------------- the routed experts on the matrix cores
 struct MmaArgs {
     const uint8_t* w;       // the experts' matrices: expert e at w + e * stride, or ep[e]

@@ -38,7 +38,7 @@ def test_quantize_q8_1_bit_exact(dev, oracle, rows, n):
 
 
 # ---------------------------------------------------------------- router mat-vec
-@pytest.mark.parametrize("rows,n,T", [(513, 2048, 16), (513, 2048, 1), (37, 256, 5), (8, 4096, 3)])
+@pytest.mark.parametrize("rows,n,T", [(513, 2048, 16), (513, 2048, 1), (37, 256, 5), (8, 4096, 3), (513, 2048, 100), (30, 512, 17), (3, 256, 64)])
 def test_gemv_f32_bit_exact(dev, oracle, rows, n, T):
     print(f"case gemv_f32 rows={rows} n={n} T={T}", flush=True)
     rng = np.random.default_rng(200 + rows + T)
@@ -47,10 +47,11 @@ def test_gemv_f32_bit_exact(dev, oracle, rows, n, T):
     assert np.array_equal(dev.gemv(W, x).view(np.uint32), oracle.gemv_f32(W, x).view(np.uint32))
 
 
-def test_gemv_bf16_bit_exact(dev, oracle):
+@pytest.mark.parametrize("T", [16, 45])   # 45 rows: the many-rows kernel, with a ragged last group
+def test_gemv_bf16_bit_exact(dev, oracle, T):
     rng = np.random.default_rng(210)
     W = ((rng.standard_normal((513, 2048)) * 0.02).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
-    x = rng.standard_normal((16, 2048)).astype(np.float32)
+    x = rng.standard_normal((T, 2048)).astype(np.float32)
     assert np.array_equal(dev.gemv(W, x, bf16=True).view(np.uint32), oracle.gemv_bf16(W, x).view(np.uint32))
 
 
