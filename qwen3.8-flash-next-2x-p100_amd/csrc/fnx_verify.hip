@@ -1076,7 +1076,7 @@ static int q8s_launch(const fnx_q8s* const* W, float* const* out, const int* out
             return fail(std::string(who) + ": cannot raise the dynamic LDS limit");
         attr_set[dev] = true;
     }
-    static const int per_cu = env_int("FNX_Q8S_BLOCKS_PER_CU", 4, 1, 16);
+    static const int per_cu = env_int("FNX_Q8S_BLOCKS_PER_CU", 3, 1, 16);   // what the LDS of a 2048-column matrix lets a CU hold
     const int grid = (int) std::max(1l, std::min<long>((long) per_cu * cu_count(), tiles));
     k_q8s_gemv<<<grid, Q8S_WAVES * 64, lds, (hipStream_t) st>>>(a);
     return launch_status(who);

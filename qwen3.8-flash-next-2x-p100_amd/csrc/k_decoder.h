@@ -101,6 +101,118 @@ __global__ void __launch_bounds__(Q8S_WAVES * 64) k_q8s_gemv(const Q8sArgs a) {
     int8_t* xs = reinterpret_cast<int8_t*>(q8s_lds);
     float* xd = reinterpret_cast<float*>(q8s_lds + (size_t) FNX_MAXT * xld);
     float* part = xd + FNX_MAXT * dld;
+    const int lane = threadIdx.x & 63, wave = uniform(threadIdx.x >> 6), r16 = lane & 15, g = lane >> 4;
+    const int t0 = (a.seg[0].rows + 15) / 16, t1 = t0 + (a.nseg > 1 ? (a.seg[1].rows + 15) / 16 : 0),
+              tiles = t1 + (a.nseg > 2 ? (a.seg[2].rows + 15) / 16 : 0);
+    const int nq4 = a.cols >> 8;   // double steps per wave: a quarter of cols / 64
+    const bool lo_groups = g < 2;
+    const int j0 = wave * nq4;     // this wave's first double step
+    struct Tile {
+        gbytes wrow, drow[4];
+        float* out;
+        int rows, row0;
+    };
+    auto tile_of = [&](int tile) {
+        const int si = tile < t0 ? 0 : tile < t1 ? 1 : 2;
+        const int8_t* sq = si == 0 ? a.seg[0].q : si == 1 ? a.seg[1].q : a.seg[2].q;
+        const uint16_t* sd = si == 0 ? a.seg[0].d : si == 1 ? a.seg[1].d : a.seg[2].d;
+        float* sout = si == 0 ? a.seg[0].out : si == 1 ? a.seg[1].out : a.seg[2].out;
+        const int sstride = si == 0 ? a.seg[0].out_stride : si == 1 ? a.seg[1].out_stride : a.seg[2].out_stride;
+        Tile c;
+        c.rows = si == 0 ? a.seg[0].rows : si == 1 ? a.seg[1].rows : a.seg[2].rows;
+        c.row0 = (tile - (si == 0 ? 0 : si == 1 ? t0 : t1)) * 16;
+        c.wrow = as_global(reinterpret_cast<const uint8_t*>(sq) + (size_t) min(c.row0 + r16, c.rows - 1) * a.cols + 16 * g + 64 * j0);
+        // the scales of the accumulator's rows 4 g .. 4 g + 3, from this wave's first block on
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            c.drow[r] = as_global(reinterpret_cast<const uint8_t*>(sd + (size_t) min(c.row0 + 4 * g + r, c.rows - 1) * nb + 2 * j0));
+        c.out = sout + (size_t) r16 * sstride + c.row0 + 4 * g;   // accumulator lane (g, token r16): rows row0 + 4 g + r
+        return c;
+    };
+    struct Batch {
+        at_v4u_t w[Q8S_BATCH];
+        at_v4u_t dd[4];   // per accumulator row: the scale pairs of the batch's double steps
+    };
+    static_assert(Q8S_BATCH == 4, "a row's scales of one batch are one 16-byte load");
+    auto load = [&](const Tile& c, int jb, Batch& o) {   // nq4 is 1, 2 or a multiple of 4 (cols a multiple of 256)
+        const int nstep = min(Q8S_BATCH, nq4 - jb);
+#pragma unroll
+        for (int u = 0; u < Q8S_BATCH; ++u) o.w[u] = *(g128*) (c.wrow + 64 * (jb + min(u, nstep - 1)));
+        if (nq4 >= Q8S_BATCH) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o.dd[r] = *(g128*) (c.drow[r] + 4 * jb);
+        } else {
+#pragma unroll
+            for (int u = 0; u < Q8S_BATCH; ++u)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) o.dd[r][u] = *(const __attribute__((address_space(1))) uint32_t*) (c.drow[r] + 4 * min(u, nstep - 1));
+        }
+    };
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    auto compute = [&](int jb, const Batch& in) {
+        const int nstep = min(Q8S_BATCH, nq4 - jb);
+#pragma unroll
+        for (int u = 0; u < Q8S_BATCH; ++u)
+            if (u < nstep) {
+                const int j = j0 + jb + u;
+                const at_v4u_t x = *reinterpret_cast<const at_v4u_t*>(xs + (size_t) r16 * xld + 64 * j + 16 * g);
+                const float2 dx = *reinterpret_cast<const float2*>(xd + r16 * dld + 2 * j);
+                const long wl = (long) in.w[u].x | (long) in.w[u].y << 32, wh = (long) in.w[u].z | (long) in.w[u].w << 32;
+                const long xl = (long) x.x | (long) x.y << 32, xh = (long) x.z | (long) x.w << 32;
+                const long xl0 = lo_groups ? xl : 0, xh0 = lo_groups ? xh : 0, xl1 = lo_groups ? 0 : xl, xh1 = lo_groups ? 0 : xh;
+                q8s_v4i s0 = __builtin_amdgcn_mfma_i32_16x16x32_i8(wl, xl0, q8s_v4i{0, 0, 0, 0}, 0, 0, 0);
+                s0 = __builtin_amdgcn_mfma_i32_16x16x32_i8(wh, xh0, s0, 0, 0, 0);
+                q8s_v4i s1 = __builtin_amdgcn_mfma_i32_16x16x32_i8(wl, xl1, q8s_v4i{0, 0, 0, 0}, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_i32_16x16x32_i8(wh, xh1, s1, 0, 0, 0);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    acc[r] = fmaf(half_bits_to_float(in.dd[r][u] & 0xFFFFu) * dx.x, (float) s0[r], acc[r]);
+                    acc[r] = fmaf(half_bits_to_float(in.dd[r][u] >> 16) * dx.y, (float) s1[r], acc[r]);
+                }
+            }
+    };
+    auto finish = [&](const Tile& c) {   // the four quarters through LDS: (s0 + s1) + (s2 + s3)
+        __syncthreads();   // the previous tile's sums have been read
+        *reinterpret_cast<float4*>(part + (wave * 64 + lane) * 4) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+        __syncthreads();
+        if (wave == 0 && r16 < T) {
+            const float4 p0 = *reinterpret_cast<const float4*>(part + lane * 4), p1 = *reinterpret_cast<const float4*>(part + (64 + lane) * 4),
+                         p2 = *reinterpret_cast<const float4*>(part + (128 + lane) * 4), p3 = *reinterpret_cast<const float4*>(part + (192 + lane) * 4);
+            const float v[4] = {(p0.x + p1.x) + (p2.x + p3.x), (p0.y + p1.y) + (p2.y + p3.y), (p0.z + p1.z) + (p2.z + p3.z),
+                                (p0.w + p1.w) + (p2.w + p3.w)};
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (c.row0 + 4 * g + r < c.rows) c.out[r] = v[r];
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[r] = 0.f;
+    };
+    // The (tile, batch) items of this block in one sequence: the next item's loads - the next tile's first ones too -
+    // are in flight while the current one is worked on and while a tile's quarters are summed.
+    int tile = blockIdx.x, jb = 0;
+    if (tile >= tiles) return;   // the same for every thread of the block
+    Tile cur = tile_of(tile);
+    bool more = true;
+    auto item = [&](const Batch& in, Batch& nxt) {
+        int ntile = tile, njb = jb + Q8S_BATCH;
+        if (njb >= nq4) {
+            njb = 0;
+            ntile += gridDim.x;
+        }
+        more = ntile < tiles;
+        const bool last = ntile != tile;
+        Tile tn = cur;
+        if (last && more) tn = tile_of(ntile);
+        if (more) load(tn, njb, nxt);
+        compute(jb, in);
+        if (last) finish(cur);
+        cur = tn;
+        tile = ntile;
+        jb = njb;
+    };
+    Batch b0, b1;
+    load(cur, 0, b0);
+    // the window's q8_1 rows into LDS (the first weights are on their way meanwhile)
     for (int i = threadIdx.x; i < FNX_MAXT * nb; i += blockDim.x) {
         const int t = i / nb, b = i - t * nb;
         uint32_t* dst = reinterpret_cast<uint32_t*>(xs + (size_t) t * xld + 32 * b);
@@ -117,72 +229,11 @@ __global__ void __launch_bounds__(Q8S_WAVES * 64) k_q8s_gemv(const Q8sArgs a) {
         }
     }
     __syncthreads();
-    const int lane = threadIdx.x & 63, wave = uniform(threadIdx.x >> 6), r16 = lane & 15, g = lane >> 4;
-    const int t0 = (a.seg[0].rows + 15) / 16, t1 = t0 + (a.nseg > 1 ? (a.seg[1].rows + 15) / 16 : 0),
-              tiles = t1 + (a.nseg > 2 ? (a.seg[2].rows + 15) / 16 : 0);
-    const int nq4 = a.cols >> 8;   // double steps per wave: a quarter of cols / 64
-    const bool lo_groups = g < 2;
-    for (int tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
-        const int si = tile < t0 ? 0 : tile < t1 ? 1 : 2;
-        const int8_t* sq = si == 0 ? a.seg[0].q : si == 1 ? a.seg[1].q : a.seg[2].q;
-        const uint16_t* sd = si == 0 ? a.seg[0].d : si == 1 ? a.seg[1].d : a.seg[2].d;
-        float* sout = si == 0 ? a.seg[0].out : si == 1 ? a.seg[1].out : a.seg[2].out;
-        const int srows = si == 0 ? a.seg[0].rows : si == 1 ? a.seg[1].rows : a.seg[2].rows;
-        const int sstride = si == 0 ? a.seg[0].out_stride : si == 1 ? a.seg[1].out_stride : a.seg[2].out_stride;
-        const int row0 = (tile - (si == 0 ? 0 : si == 1 ? t0 : t1)) * 16;
-        const int j0 = wave * nq4;   // this wave's first double step
-        const gbytes wrow = as_global(reinterpret_cast<const uint8_t*>(sq) + (size_t) min(row0 + r16, srows - 1) * a.cols + 16 * g + 64 * j0);
-        // the scales of the accumulator's rows 4 g .. 4 g + 3, from this wave's first block on
-        gbytes drow[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-            drow[r] = as_global(reinterpret_cast<const uint8_t*>(sd + (size_t) min(row0 + 4 * g + r, srows - 1) * nb + 2 * j0));
-        float acc[4] = {0.f, 0.f, 0.f, 0.f};
-        for (int jb = 0; jb < nq4; jb += Q8S_BATCH) {   // nq4 is 1, 2 or a multiple of 4 (cols a multiple of 256)
-            const int nstep = min(Q8S_BATCH, nq4 - jb);
-            at_v4u_t w[Q8S_BATCH];
-            uint32_t dd[4][Q8S_BATCH];
-#pragma unroll
-            for (int u = 0; u < Q8S_BATCH; ++u) {
-                const int j = jb + min(u, nstep - 1);
-                w[u] = *(g128*) (wrow + 64 * j);
-#pragma unroll
-                for (int r = 0; r < 4; ++r) dd[r][u] = *(const __attribute__((address_space(1))) uint32_t*) (drow[r] + 4 * j);
-            }
-#pragma unroll
-            for (int u = 0; u < Q8S_BATCH; ++u)
-                if (u < nstep) {
-                    const int j = j0 + jb + u;
-                    const at_v4u_t x = *reinterpret_cast<const at_v4u_t*>(xs + (size_t) r16 * xld + 64 * j + 16 * g);
-                    const float2 dx = *reinterpret_cast<const float2*>(xd + r16 * dld + 2 * j);
-                    const long wl = (long) w[u].x | (long) w[u].y << 32, wh = (long) w[u].z | (long) w[u].w << 32;
-                    const long xl = (long) x.x | (long) x.y << 32, xh = (long) x.z | (long) x.w << 32;
-                    const long xl0 = lo_groups ? xl : 0, xh0 = lo_groups ? xh : 0, xl1 = lo_groups ? 0 : xl, xh1 = lo_groups ? 0 : xh;
-                    q8s_v4i s0 = __builtin_amdgcn_mfma_i32_16x16x32_i8(wl, xl0, q8s_v4i{0, 0, 0, 0}, 0, 0, 0);
-                    s0 = __builtin_amdgcn_mfma_i32_16x16x32_i8(wh, xh0, s0, 0, 0, 0);
-                    q8s_v4i s1 = __builtin_amdgcn_mfma_i32_16x16x32_i8(wl, xl1, q8s_v4i{0, 0, 0, 0}, 0, 0, 0);
-                    s1 = __builtin_amdgcn_mfma_i32_16x16x32_i8(wh, xh1, s1, 0, 0, 0);
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        acc[r] = fmaf(half_bits_to_float(dd[r][u] & 0xFFFFu) * dx.x, (float) s0[r], acc[r]);
-                        acc[r] = fmaf(half_bits_to_float(dd[r][u] >> 16) * dx.y, (float) s1[r], acc[r]);
-                    }
-                }
-        }
-        // the four quarters through LDS: (s0 + s1) + (s2 + s3)
-        __syncthreads();   // the previous tile's sums have been read
-        *reinterpret_cast<float4*>(part + (wave * 64 + lane) * 4) = make_float4(acc[0], acc[1], acc[2], acc[3]);
-        __syncthreads();
-        if (wave == 0 && r16 < T) {   // accumulator lane (g, token r16): rows row0 + 4 g + r
-            const float4 p0 = *reinterpret_cast<const float4*>(part + lane * 4), p1 = *reinterpret_cast<const float4*>(part + (64 + lane) * 4),
-                         p2 = *reinterpret_cast<const float4*>(part + (128 + lane) * 4), p3 = *reinterpret_cast<const float4*>(part + (192 + lane) * 4);
-            const float v[4] = {(p0.x + p1.x) + (p2.x + p3.x), (p0.y + p1.y) + (p2.y + p3.y), (p0.z + p1.z) + (p2.z + p3.z),
-                                (p0.w + p1.w) + (p2.w + p3.w)};
-            float* o = sout + (size_t) r16 * sstride + row0 + 4 * g;
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-                if (row0 + 4 * g + r < srows) o[r] = v[r];
-        }
+    while (true) {
+        item(b0, b1);
+        if (!more) break;
+        item(b1, b0);
+        if (!more) break;
     }
 }
 
