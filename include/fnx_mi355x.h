@@ -217,6 +217,11 @@ int fnx_rms_norm_rows(const float* x, const float* w, float* y, int rows, int n,
  * add, rms_norm_rows and quantize_q8_1 that follow one another between a layer's halves (engine.cu's hc_read takes
  * the same place in the reference), one pass over each row; the values are the three operators' bit for bit. n <= 4096 */
 int fnx_add_norm_q8(float* x, const float* add, const float* w, float* xn, void* xq, int rows, int n, float eps, void* st);
+/* the same with the MoE half's combine (kernels.hpp's moe_combine, kernels.cu:412-419) as what is added: x[r] += sum_k
+ * topw[r][k] part[r topk + k] + sigmoid(sh_logit[r]) sh[r], then norm and q8_1 as above - fnx_moe_combine followed by
+ * fnx_add_norm_q8 in one launch, their values bit for bit (the decoder's layers hand over this way) */
+int fnx_combine_add_norm_q8(const float* part, const float* topw, const float* sh, const float* sh_logit, int sh_logit_stride, int topk, float* x,
+                            const float* w, float* xn, void* xq, int rows, int n, float eps, void* st);
 /* y = a + b over n floats */
 int fnx_add_rows(const float* a, const float* b, float* y, size_t n, void* st);
 /* rows tokens[t] of an f16 table [vocab][n] as f32 (the window's input rows) */

@@ -712,6 +712,7 @@ static int layer_fused(const fnx_moe_layer* L, const float* x, int T, float* out
     else k_moe_down_passes<32><<<grid, FL_THREADS, 0, s>>>(dn);
     prof_mark(4, s);
     if (launch_status("moe_verify_layer")) return 1;
+    if (!out) return 0;   // the caller combines (with what follows: fnx_combine_add_norm_q8)
     const int rc = fnx_moe_combine(ws->part, ws->topw, ws->part + (size_t) P * n, ws->logits + L->nexp, LS, out, T, n, L->topk, st);
     prof_mark(5, s);
     return rc;
@@ -904,8 +905,9 @@ int fnx_layer_profile_read(float* ms5) {
     return 0;
 }
 
-int fnx_moe_verify_layer(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st) {
-    if (!L || !x || !out || !ws) return fail("moe_verify_layer: null argument");
+// out null: the fused window without its combine (layer_fused_ok must hold)
+static int moe_layer_checked(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st) {
+    if (!L || !x || !ws) return fail("moe_verify_layer: null argument");
     if (!ws->xq || !ws->logits || !ws->topi || !ws->topw || !ws->jobs_gu || !ws->jobs_dn || !ws->njobs || !ws->gu || !ws->part)
         return fail("moe_verify_layer: incomplete workspace");
     if (topk_check(T, L->nexp, L->topk, "moe_verify_layer")) return 1;
@@ -915,6 +917,7 @@ int fnx_moe_verify_layer(const fnx_moe_layer* L, const float* x, int T, float* o
         L->sh_gu.n_out != 2 * ff || L->sh_down.n_in != ff || L->sh_down.n_out != n)
         return fail("moe_verify_layer: weight shapes do not match n / ff");
     if (layer_fused_ok(L, T)) return layer_fused(L, x, T, out, ws, st);
+    if (!out) return fail("moe_verify_layer: null argument");
     hipStream_t s = (hipStream_t) st;
     if (fnx_quantize_q8_1(x, ws->xq, n, T, st)) return 1;
     if (gemv_any(L->router, L->router_bf16 != 0, x, ws->logits, L->nexp + 1, n, T, st, "moe_verify_layer router")) return 1;
@@ -928,6 +931,10 @@ int fnx_moe_verify_layer(const fnx_moe_layer* L, const float* x, int T, float* o
     if (rows_launch(&L->down, L->down_stride, ws->jobs_dn, ws->njobs, P, nullptr, ws->part, n, st, "moe_verify_layer down")) return 1;
     if (rows_launch(&L->sh_down, 0, ws->jobs_dn + P, nullptr, 1, nullptr, ws->part, n, st, "moe_verify_layer shared down", true)) return 1;
     return fnx_moe_combine(ws->part, ws->topw, ws->part + (size_t) P * n, ws->logits + L->nexp, L->nexp + 1, out, T, n, L->topk, st);
+}
+int fnx_moe_verify_layer(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st) {
+    if (!out) return fail("moe_verify_layer: null argument");
+    return moe_layer_checked(L, x, T, out, ws, st);
 }
 
 // ---------------------------------------------------------------- the prompt path
@@ -1033,8 +1040,15 @@ int fnx_rms_norm_rows(const float* x, const float* w, float* y, int rows, int n,
 int fnx_add_norm_q8(float* x, const float* add, const float* w, float* xn, void* xq, int rows, int n, float eps, void* st) {
     if (!x || !w) return fail("add_norm_q8: null argument");
     if (rows < 1 || n < 32 || n % 32 || n > 256 * NQ_MAXJ) return fail("add_norm_q8: rows of 32 .. 4096 values in whole 32-value blocks");
-    k_add_norm_q8<<<rows, 256, 0, (hipStream_t) st>>>(x, add, w, xn, (uint8_t*) xq, n, eps);
+    k_add_norm_q8<<<rows, 256, 0, (hipStream_t) st>>>(x, add, CombineArgs{}, w, xn, (uint8_t*) xq, n, eps);
     return launch_status("add_norm_q8");
+}
+int fnx_combine_add_norm_q8(const float* part, const float* topw, const float* sh, const float* sh_logit, int sh_logit_stride, int topk, float* x,
+                            const float* w, float* xn, void* xq, int rows, int n, float eps, void* st) {
+    if (!part || !topw || !sh || !sh_logit || !x || !w) return fail("combine_add_norm_q8: null argument");
+    if (rows < 1 || n < 32 || n % 32 || n > 256 * NQ_MAXJ || topk < 1) return fail("combine_add_norm_q8: rows of 32 .. 4096 values in whole 32-value blocks");
+    k_add_norm_q8<<<rows, 256, 0, (hipStream_t) st>>>(x, nullptr, CombineArgs{part, topw, sh, sh_logit, sh_logit_stride, topk}, w, xn, (uint8_t*) xq, n, eps);
+    return launch_status("combine_add_norm_q8");
 }
 int fnx_add_rows(const float* a, const float* b, float* y, size_t n, void* st) {
     if (!a || !b || !y) return fail("add_rows: null argument");
@@ -1109,9 +1123,9 @@ int fnx_attn_prep_append(float* qg, float* k, const float* v, const float* q_nor
 // splits for a context of up to max_ctx positions
 static int attn_splits(int max_ctx) { return (max_ctx + AT_SPLIT - 1) / AT_SPLIT; }
 size_t fnx_attn_scratch_floats(int nq, int T, int max_ctx) { return (size_t) T * nq * attn_splits(max_ctx) * (AT_HD + 2); }
-int fnx_attn(const float* qg, const uint16_t* kc, const uint16_t* vc, float* out, int nq, int nkv, const int* pos0, int T, int max_ctx,
-             float* scratch, void* st) {
-    if (!qg || !kc || !vc || !out || !pos0 || !scratch) return fail("attn: null argument");
+static int attn_launch(const float* qg, const uint16_t* kc, const uint16_t* vc, float* out, uint8_t* outq, int nq, int nkv, const int* pos0, int T,
+                       int max_ctx, float* scratch, void* st) {
+    if (!qg || !kc || !vc || (!out && !outq) || !pos0 || !scratch) return fail("attn: null argument");
     if (nq < 1 || nkv < 1 || nq % nkv || nq / nkv > AT_MAXQ || T < 1 || T > FNX_MAXT || max_ctx < 1) return fail("attn: bad shape");
     if (attn_splits(max_ctx) > AT_MAXSPLIT) return fail("attn: the cache is larger than the split table");
     // the grid covers the cache's capacity (the position is on the device): splits past the context write empty parts
@@ -1120,8 +1134,13 @@ int fnx_attn(const float* qg, const uint16_t* kc, const uint16_t* vc, float* out
     AttPart* mz = reinterpret_cast<AttPart*>(scratch + (size_t) T * nq * nsplit * AT_HD);
     k_attn_part<<<dim3(nsplit, nkv, (waves + AT_WAVES - 1) / AT_WAVES), 64 * AT_WAVES, 0, (hipStream_t) st>>>(qg, kc, vc, acc, mz, nq, nkv, T,
                                                                                                           nsplit, pos0);
-    k_attn_combine<<<dim3(nq, T), AT_HD, 0, (hipStream_t) st>>>(qg, acc, mz, out, nq, nsplit, T, pos0);
+    k_attn_combine<<<dim3(nq, T), AT_HD, 0, (hipStream_t) st>>>(qg, acc, mz, out, outq, nq, nsplit, T, pos0);
     return launch_status("attn");
+}
+int fnx_attn(const float* qg, const uint16_t* kc, const uint16_t* vc, float* out, int nq, int nkv, const int* pos0, int T, int max_ctx,
+             float* scratch, void* st) {
+    if (!out) return fail("attn: null argument");
+    return attn_launch(qg, kc, vc, out, nullptr, nq, nkv, pos0, T, max_ctx, scratch, st);
 }
 static int dec_ws_check(const fnx_dec_ws* ws, const char* who) {
     if (!ws->x || !ws->xn || !ws->qg || !ws->k || !ws->v || !ws->att || !ws->o || !ws->attn_scratch || !ws->xq || !ws->hidden || !ws->logits ||
@@ -1129,11 +1148,23 @@ static int dec_ws_check(const fnx_dec_ws* ws, const char* who) {
         return fail(std::string(who) + ": incomplete workspace");
     return 0;
 }
-// x (ws->x) through one layer, in place. pending (may be null): rows still to be added to x first (the layer before's
-// MoE output); the layer's own MoE output is left in ws->o, to be added by whatever comes next
-static int dec_layer(const fnx_decoder* D, const fnx_dec_layer* L, int T, const int* pos0, const fnx_dec_ws* ws, const float* pending, void* st) {
+// What is still to be added to x when a layer (or the head) starts: rows (may be null), or the MoE half before it whose
+// partial sums (in ws->moe) have not been combined yet - the first pass over the rows then does that too.
+struct DecPending {
+    const float* rows;
+    const fnx_moe_layer* moe;
+};
+static int dec_add_norm_q8(const fnx_decoder* D, const DecPending& pend, const float* w, int T, const fnx_dec_ws* ws, void* st) {
+    if (!pend.moe) return fnx_add_norm_q8(ws->x, pend.rows, w, nullptr, ws->xq, T, D->n, D->eps, st);
+    const fnx_moe_layer* M = pend.moe;
+    const int P = T * M->topk;
+    return fnx_combine_add_norm_q8(ws->moe.part, ws->moe.topw, ws->moe.part + (size_t) P * D->n, ws->moe.logits + M->nexp, M->nexp + 1, M->topk, ws->x, w,
+                                   nullptr, ws->xq, T, D->n, D->eps, st);
+}
+// x (ws->x) through one layer, in place; the layer's own MoE output is left pending for whatever comes next
+static int dec_layer(const fnx_decoder* D, const fnx_dec_layer* L, int T, const int* pos0, const fnx_dec_ws* ws, DecPending& pend, void* st) {
     const int n = D->n, nq = D->nq, nkv = D->nkv;
-    if (fnx_add_norm_q8(ws->x, pending, L->attn_norm, nullptr, ws->xq, T, n, D->eps, st)) return 1;
+    if (dec_add_norm_q8(D, pend, L->attn_norm, T, ws, st)) return 1;
     {   // q, k and v in one launch (engine.cu:1547-1552)
         const fnx_q8s* w3[3] = {&L->wq, &L->wk, &L->wv};
         float* const o3[3] = {ws->qg, ws->k, ws->v};
@@ -1141,10 +1172,15 @@ static int dec_layer(const fnx_decoder* D, const fnx_dec_layer* L, int T, const 
         if (fnx_q8s_gemv_segs(w3, o3, s3, 3, ws->xq, T, st)) return 1;
     }
     if (fnx_attn_prep_append(ws->qg, ws->k, ws->v, L->q_norm, L->k_norm, L->kc, L->vc, nq, nkv, T, pos0, D->max_ctx, D->eps, &D->rope, st)) return 1;
-    if (fnx_attn(ws->qg, L->kc, L->vc, ws->att, nq, nkv, pos0, T, D->max_ctx, ws->attn_scratch, st)) return 1;
-    if (fnx_quantize_q8_1(ws->att, ws->xq, nq * AT_HD, T, st)) return 1;
+    // the attention's rows leave its last kernel in q8_1 form, ready for the output projection
+    if (attn_launch(ws->qg, L->kc, L->vc, nullptr, (uint8_t*) ws->xq, nq, nkv, pos0, T, D->max_ctx, ws->attn_scratch, st)) return 1;
     if (fnx_q8s_gemv(&L->wo, ws->xq, ws->o, n, T, st)) return 1;
     if (fnx_add_norm_q8(ws->x, ws->o, L->ffn_norm, ws->xn, nullptr, T, n, D->eps, st)) return 1;
+    if (layer_fused_ok(&L->moe, T)) {   // the window without its combine
+        pend = DecPending{nullptr, &L->moe};
+        return moe_layer_checked(&L->moe, ws->xn, T, nullptr, &ws->moe, st);
+    }
+    pend = DecPending{ws->o, nullptr};
     return fnx_moe_verify_layer(&L->moe, ws->xn, T, ws->o, &ws->moe, st);
 }
 static int dec_shape_check(const fnx_decoder* D, int T, const char* who) {
@@ -1155,8 +1191,8 @@ static int dec_shape_check(const fnx_decoder* D, int T, const char* who) {
     return 0;
 }
 // x += pending; hidden = x; the output norm, the head, argmax
-static int dec_head(const fnx_decoder* D, const float* norm, const fnx_q8s* head, int T, const fnx_dec_ws* ws, const float* pending, void* st) {
-    if (fnx_add_norm_q8(ws->x, pending, norm, nullptr, ws->xq, T, D->n, D->eps, st)) return 1;
+static int dec_head(const fnx_decoder* D, const float* norm, const fnx_q8s* head, int T, const fnx_dec_ws* ws, const DecPending& pend, void* st) {
+    if (dec_add_norm_q8(D, pend, norm, T, ws, st)) return 1;
     if (hipMemcpyAsync(ws->hidden, ws->x, (size_t) T * D->n * sizeof(float), hipMemcpyDeviceToDevice, (hipStream_t) st) != hipSuccess)
         return fail("decoder: copy of the hidden rows failed");
     if (fnx_q8s_gemv(head, ws->xq, ws->logits, D->vocab, T, st)) return 1;
@@ -1166,9 +1202,10 @@ int fnx_decoder_verify(const fnx_decoder* D, const int* tokens, int T, const int
     if (!D || !tokens || !pos0 || !ws || !D->layers || !D->out_norm || !D->emb) return fail("decoder_verify: null argument");
     if (dec_shape_check(D, T, "decoder_verify") || dec_ws_check(ws, "decoder_verify")) return 1;
     if (fnx_embed_rows(D->emb, tokens, T, D->vocab, D->n, ws->x, st)) return 1;
+    DecPending pend{nullptr, nullptr};
     for (int l = 0; l < D->nlayers; ++l)
-        if (dec_layer(D, &D->layers[l], T, pos0, ws, l ? ws->o : nullptr, st)) return 1;
-    return dec_head(D, D->out_norm, &D->head, T, ws, D->nlayers ? ws->o : nullptr, st);
+        if (dec_layer(D, &D->layers[l], T, pos0, ws, pend, st)) return 1;
+    return dec_head(D, D->out_norm, &D->head, T, ws, pend, st);
 }
 int fnx_mtp_draft(const fnx_decoder* D, const fnx_mtp* M, const float* src, const int* tokens, int T, const int* pos0, const fnx_dec_ws* ws,
                   void* st) {
@@ -1181,8 +1218,9 @@ int fnx_mtp_draft(const fnx_decoder* D, const fnx_mtp* M, const float* src, cons
     if (fnx_embed_rows(D->emb, tokens, T, D->vocab, n, ws->xn, st)) return 1;
     if (fnx_add_norm_q8(ws->xn, nullptr, M->norm_emb, nullptr, ws->xq, T, n, D->eps, st)) return 1;
     if (fnx_q8s_gemv(&M->fc_emb, ws->xq, ws->o, n, T, st)) return 1;
-    if (dec_layer(D, &M->layer, T, pos0, ws, ws->o, st)) return 1;
-    return dec_head(D, M->out_norm, &M->head, T, ws, ws->o, st);
+    DecPending pend{ws->o, nullptr};
+    if (dec_layer(D, &M->layer, T, pos0, ws, pend, st)) return 1;
+    return dec_head(D, M->out_norm, &M->head, T, ws, pend, st);
 }
 
 }  // extern "C"

@@ -26,26 +26,88 @@ __global__ void __launch_bounds__(256) k_rms_norm_rows(const float* __restrict__
 // x[r] += add[r] (add may be null); xn[r] = rms_norm(x[r]) * w; xq[r] = q8_1(xn[r]) (either may be null): the residual add,
 // the norm and the quantisation that follow one another between a layer's halves, in one pass over the row. The sums
 // run in k_rms_norm_rows' and k_quantize_q8_1's orders, so the results are theirs bit for bit.
+// With c.part set, what is added is the MoE half's combine (k_combine's chain, kernels.cu:412-419) of the partial sums,
+// made here instead of being written out and read back by a launch of its own.
 constexpr int NQ_MAXJ = 16;   // rows of up to 4096 values
-__global__ void __launch_bounds__(256) k_add_norm_q8(float* __restrict__ x, const float* __restrict__ add, const float* __restrict__ w,
-                                                    float* __restrict__ xn, uint8_t* __restrict__ xq, int n, float eps) {
+struct CombineArgs {
+    const float* part;   // null: no combine
+    const float* topw;
+    const float* sh;
+    const float* sh_logit;
+    int sh_logit_stride, topk;
+};
+__global__ void __launch_bounds__(256) k_add_norm_q8(float* __restrict__ x, const float* __restrict__ add, const CombineArgs c,
+                                                    const float* __restrict__ w, float* __restrict__ xn, uint8_t* __restrict__ xq, int n, float eps) {
     __shared__ float sh[4];
     const size_t row = blockIdx.x;
     float v[NQ_MAXJ];
     float s = 0.f;
+    if (c.part) {
+        // the combine's chains, NQ_KB experts' partial sums of all this thread's columns in flight at a time (one by one,
+        // each load would be a trip to the cache of its own)
+        constexpr int NQ_KB = 5;
+        float m[NQ_MAXJ];
+#pragma unroll
+        for (int j = 0; j < NQ_MAXJ; ++j) m[j] = 0.f;
+        for (int k0 = 0; k0 < c.topk; k0 += NQ_KB) {
+            float pv[NQ_KB][NQ_MAXJ], wk[NQ_KB];
+#pragma unroll
+            for (int kk = 0; kk < NQ_KB; ++kk) {
+                const int k = min(k0 + kk, c.topk - 1);
+                wk[kk] = c.topw[row * c.topk + k];
+#pragma unroll
+                for (int j = 0; j < NQ_MAXJ; ++j) {
+                    const int i = threadIdx.x + 256 * j;
+                    pv[kk][j] = i < n ? c.part[(row * c.topk + k) * n + i] : 0.f;
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int kk = 0; kk < NQ_KB; ++kk)
+                if (k0 + kk < c.topk) {
+#pragma unroll
+                    for (int j = 0; j < NQ_MAXJ; ++j) m[j] = fmaf(wk[kk], pv[kk][j], m[j]);
+                }
+        }
+        const float sg = sigmoid_f(c.sh_logit[row * c.sh_logit_stride]);
+        float shv[NQ_MAXJ];
+#pragma unroll
+        for (int j = 0; j < NQ_MAXJ; ++j) {
+            const int i = threadIdx.x + 256 * j;
+            v[j] = i < n ? x[row * n + i] : 0.f;
+            shv[j] = i < n ? c.sh[row * n + i] : 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < NQ_MAXJ; ++j) v[j] += m[j] + sg * shv[j];
+    } else {
+        // all loads first: a store to x between them would keep the next load waiting for it
+        float av[NQ_MAXJ];
+#pragma unroll
+        for (int j = 0; j < NQ_MAXJ; ++j) {
+            const int i = threadIdx.x + 256 * j;
+            v[j] = i < n ? x[row * n + i] : 0.f;
+            av[j] = add && i < n ? add[row * n + i] : 0.f;
+        }
+        if (add) {
+#pragma unroll
+            for (int j = 0; j < NQ_MAXJ; ++j) v[j] += av[j];
+        }
+    }
+    float wv[NQ_MAXJ];   // the norm's weights too, before any store
 #pragma unroll
     for (int j = 0; j < NQ_MAXJ; ++j) {
         const int i = threadIdx.x + 256 * j;
-        v[j] = 0.f;
-        if (i < n) {
-            v[j] = x[row * n + i];
-            if (add) {
-                v[j] += add[row * n + i];
-                x[row * n + i] = v[j];
-            }
-            s = fmaf(v[j], v[j], s);
+        wv[j] = i < n ? w[i] : 0.f;
+    }
+    if (add || c.part) {
+#pragma unroll
+        for (int j = 0; j < NQ_MAXJ; ++j) {
+            const int i = threadIdx.x + 256 * j;
+            if (i < n) x[row * n + i] = v[j];
         }
     }
+#pragma unroll
+    for (int j = 0; j < NQ_MAXJ; ++j) s = fmaf(v[j], v[j], s);   // columns past n hold zeros
     s = group_sum<64>(s);
     if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = s;
     __syncthreads();
@@ -54,7 +116,7 @@ __global__ void __launch_bounds__(256) k_add_norm_q8(float* __restrict__ x, cons
     for (int j = 0; j < NQ_MAXJ; ++j) {
         const int i = threadIdx.x + 256 * j;
         if (i < n) {   // n is a multiple of 32: the 32 threads of a q8_1 block are live together
-            const float y = v[j] * r * w[i];
+            const float y = v[j] * r * wv[j];
             if (xn) xn[row * n + i] = y;
             if (xq) q8_1_store(y, xq + (row * (n / 32) + i / 32) * FNX_Q8_1_BLOCK, threadIdx.x & 31);
         }
@@ -474,11 +536,11 @@ __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per
     if (pg == 0) mz_out[slot] = AttPart{m, z};
 }
 // a block per (head, row): the splits' weights exp(m_s - max) first (LDS), then every thread sums its dimension over the
-// splits that hold data, several loads in flight
+// splits that hold data, several loads in flight. out (f32) and outq (q8_1 rows) may each be null.
 constexpr int AT_MAXSPLIT = 2048;
 __global__ void __launch_bounds__(AT_HD) k_attn_combine(const float* __restrict__ qg, const float* __restrict__ acc_in,
-                                                       const AttPart* __restrict__ mz_in, float* __restrict__ out, int nq, int nsplit, int T,
-                                                       const int* __restrict__ pos0p) {
+                                                       const AttPart* __restrict__ mz_in, float* __restrict__ out, uint8_t* __restrict__ outq,
+                                                       int nq, int nsplit, int T, const int* __restrict__ pos0p) {
     __shared__ float wsp[AT_MAXSPLIT];
     __shared__ float red[AT_HD / 64];
     const int h = blockIdx.x, t = blockIdx.y, i = threadIdx.x;
@@ -513,7 +575,10 @@ __global__ void __launch_bounds__(AT_HD) k_attn_combine(const float* __restrict_
     }
     for (; s < nlive; ++s) a0 = fmaf(wsp[s], ap[(size_t) s * AT_HD], a0);
     const float acc = (a0 + a1) + (a2 + a3);
-    out[((size_t) t * nq + h) * AT_HD + i] = acc / z * sigmoid_f(qg[((size_t) t * nq + h) * 2 * AT_HD + AT_HD + i]);
+    const float v = acc / z * sigmoid_f(qg[((size_t) t * nq + h) * 2 * AT_HD + AT_HD + i]);
+    if (out) out[((size_t) t * nq + h) * AT_HD + i] = v;
+    // the row's q8_1 form (the input of the output projection): a head is eight blocks of 32 dims, a half-wave each
+    if (outq) q8_1_store(v, outq + (((size_t) t * nq + h) * (AT_HD / 32) + i / 32) * FNX_Q8_1_BLOCK, i & 31);
 }
 
 }  // namespace fnx

@@ -284,6 +284,27 @@ class Dev:
         self.sync()
         return dx.cpu().numpy(), xn.cpu().numpy(), xq.cpu().numpy()
 
+    def moe_combine(self, part, topw, sh, sh_logit):
+        T, topk = topw.shape
+        n = part.shape[1]
+        d = [self.up(a.astype(np.float32)) for a in (part, topw, sh, sh_logit)]
+        out = self.zeros((T, n), self.torch.float32)
+        self.ok(self.lib.fnx_moe_combine(d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), d[3].data_ptr(), 1, out.data_ptr(), T, n, topk, self.st()))
+        self.sync()
+        return out.cpu().numpy()
+
+    def combine_add_norm_q8(self, part, topw, sh, sh_logit, x, w, eps):
+        """part [T * topk][n], topw [T][topk], sh [T][n], sh_logit [T]: returns (x after the add, xn, xq)"""
+        t = self.torch
+        rows, n = x.shape
+        topk = topw.shape[1]
+        d = [self.up(a.astype(np.float32)) for a in (part, topw, sh, sh_logit, x, w)]
+        xn, xq = self.zeros((rows, n), t.float32), self.zeros(rows * (n // 32) * 36, t.uint8)
+        self.ok(self.lib.fnx_combine_add_norm_q8(d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), d[3].data_ptr(), 1, topk, d[4].data_ptr(),
+                                                 d[5].data_ptr(), xn.data_ptr(), xq.data_ptr(), rows, n, eps, self.st()))
+        self.sync()
+        return d[4].cpu().numpy(), xn.cpu().numpy(), xq.cpu().numpy()
+
     def q8s_gemv(self, q, d, yq, T):
         rows, cols = q.shape
         dq, dd, dy = self.up(q), self.up(d), self.up(yq)

@@ -56,6 +56,23 @@ def test_add_norm_q8_equals_the_three_operators(dev, n, with_add):
     assert np.array_equal(xq, dev.quantize_q8_1(want_n))
 
 
+@pytest.mark.parametrize("T,n,topk", [(16, 2048, 10), (3, 2048, 10), (5, 96, 2)])
+def test_combine_add_norm_q8_equals_combine_then_add_norm(dev, oracle, T, n, topk):
+    """the hand-over between two decoder layers in one launch: the values of fnx_moe_combine followed by fnx_add_norm_q8"""
+    rng = np.random.default_rng(806 + T)
+    part = rng.standard_normal((T * topk, n)).astype(np.float32)
+    topw = rng.random((T, topk)).astype(np.float32)
+    sh, shl = rng.standard_normal((T, n)).astype(np.float32), rng.standard_normal(T).astype(np.float32)
+    x, w = rng.standard_normal((T, n)).astype(np.float32) * 2, rng.standard_normal(n).astype(np.float32)
+    comb = dev.moe_combine(part, topw, sh, shl)
+    assert rel_l2(comb, oracle.moe_combine(part, topw, sh, shl)) <= 1e-6   # the sigmoid's expf is the device's
+    x2, xn, xq = dev.combine_add_norm_q8(part, topw, sh, shl, x, w, 1e-6)
+    want_x, want_n, want_q = dev.add_norm_q8(x, comb, w, 1e-6)
+    assert int(np.count_nonzero(x2.view(np.uint32) != want_x.view(np.uint32))) == 0
+    assert int(np.count_nonzero(xn.view(np.uint32) != want_n.view(np.uint32))) == 0
+    assert int(np.count_nonzero(xq != want_q)) == 0
+
+
 @pytest.mark.parametrize("rows,cols,T", [(37, 1024, 3), (1000, 2048, 16), (2048, 4096, 16), (513, 256, 5), (8192, 2048, 1)])
 def test_q8s_gemv_bit_exact(dev, oracle, rows, cols, T):
     print(f"case q8s_gemv rows={rows} cols={cols} T={T}", flush=True)
