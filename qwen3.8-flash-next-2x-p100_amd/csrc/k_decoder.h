@@ -379,6 +379,24 @@ __device__ __forceinline__ size_t vcache_at(int pos, int nkv, int kvh, int d) { 
     return (((size_t) (pos >> 2) * nkv + kvh) * AT_HD + d) * 4 + (pos & 3);
 }
 
+// maximum / sum over the four lanes l, l ^ 16, l ^ 32, l ^ 48 (a query's four lane groups), left in all four: two row
+// swaps each instead of two trips through the LDS crossbar. (Inline asm, with the wait states the swap needs after a
+// vector write, as for the other uses of these swaps.)
+__device__ __forceinline__ float groups4_max(float v) {
+    float x = v, y = v;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(x), "+v"(y));
+    x = y = fmaxf(x, y);
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(x), "+v"(y));
+    return fmaxf(x, y);
+}
+__device__ __forceinline__ float groups4_sum(float v) {
+    float x = v, y = v;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(x), "+v"(y));
+    x = y = x + y;
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(x), "+v"(y));
+    return x + y;
+}
+constexpr int AT_VLD = AT_HD * 8 + 128;   // LDS bytes per V block: the four lane groups' 128-byte reads of one instruction fall on different banks
 constexpr int AT_WAVES = 4, AT_KLD = 2 * AT_HD + 16;   // q tiles (of 16 queries) per block, blockIdx.z picks which; LDS bytes per K row
 __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) k_attn_part(const float* __restrict__ qg, const uint16_t* __restrict__ kc,
                                                             const uint16_t* __restrict__ vc, float* __restrict__ acc_out,
@@ -426,27 +444,27 @@ __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per
     // bytes per thread, a chunk ahead into registers and from there into one of two LDS buffers; the waves read their
     // operands from LDS (K rows padded to 528 bytes: the 16 positions of a tile fall on different banks).
     __shared__ __align__(16) uint8_t lk[2][AT_CH * AT_KLD];
-    __shared__ __align__(16) uint8_t lv[2][8 * AT_HD * 8];
+    __shared__ __align__(16) uint8_t lv[2][8 * AT_VLD];
     const int tid = threadIdx.x;
     const gbytes kbase = as_global(reinterpret_cast<const uint8_t*>(kc));
     const gbytes vbase = as_global(reinterpret_cast<const uint8_t*>(vc));
-    const int krow = tid >> 3, kpart = tid & 7, vblk = tid >> 5, vpart = tid & 31;
+    // piece tid + 256 i of the chunk's 1024 16-byte pieces of K (32 to a row) and of V (128 to a block): consecutive lanes
+    // load consecutive pieces, so a wave's load is whole runs of 512 or 1024 bytes
+    const int krow = tid >> 5, kcol = tid & 31, vblk = tid >> 7, vcol = tid & 127;
     at_v4u kr[4], vr[4];
     auto fetch = [&](int c0) {   // rows and blocks clamped inside the window's rows
-        const int pos = min(c0 + krow, ctx_max - 1), blk = min((c0 >> 2) + vblk, (ctx_max - 1) >> 2);
-        const gbytes kp = kbase + ((size_t) pos * nkv + kvh) * (AT_HD * 2) + 64 * kpart;
-        const gbytes vp = vbase + ((size_t) blk * nkv + kvh) * (AT_HD * 8) + 64 * vpart;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            kr[i] = *(g128*) (kp + 16 * i);
-            vr[i] = *(g128*) (vp + 16 * i);
+            const int pos = min(c0 + krow + 8 * i, ctx_max - 1), blk = min((c0 >> 2) + vblk + 2 * i, (ctx_max - 1) >> 2);
+            kr[i] = *(g128*) (kbase + ((size_t) pos * nkv + kvh) * (AT_HD * 2) + 16 * kcol);
+            vr[i] = *(g128*) (vbase + ((size_t) blk * nkv + kvh) * (AT_HD * 8) + 16 * vcol);
         }
     };
     auto stash = [&](int buf) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            *reinterpret_cast<at_v4u*>(&lk[buf][krow * AT_KLD + 64 * kpart + 16 * i]) = kr[i];
-            *reinterpret_cast<at_v4u*>(&lv[buf][vblk * (AT_HD * 8) + 64 * vpart + 16 * i]) = vr[i];
+            *reinterpret_cast<at_v4u*>(&lk[buf][(krow + 8 * i) * AT_KLD + 16 * kcol]) = kr[i];
+            *reinterpret_cast<at_v4u*>(&lv[buf][(vblk + 2 * i) * AT_VLD + 16 * vcol]) = vr[i];
         }
     };
     fetch(p0);
@@ -457,18 +475,24 @@ __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per
     for (int c0 = p0; c0 < p1; c0 += AT_CH, buf ^= 1) {
         stash(buf ^ 1);                              // chunk c0 + 32, fetched during the last iteration
         fetch(min(c0 + 2 * AT_CH, p1 - 1));          // past the split: some rows again, never used
+        // the two tiles' hi and lo terms in chains of their own, interleaved: a chain's next MFMA is four issues away, so
+        // none waits for the one before it
         at_v4f S[2];
-#pragma unroll
-        for (int tile = 0; tile < 2; ++tile) {
-            const uint8_t* krow_l = &lk[buf][(16 * tile + ql) * AT_KLD + 128 * pg];
-            at_v4f acc = at_v4f{0.f, 0.f, 0.f, 0.f};
+        {
+            const uint8_t* k0 = &lk[buf][ql * AT_KLD + 128 * pg];
+            const uint8_t* k1 = k0 + 16 * AT_KLD;
+            at_v4f a0 = at_v4f{0.f, 0.f, 0.f, 0.f}, a0l = a0, a1 = a0, a1l = a0;
 #pragma unroll
             for (int ks = 0; ks < 8; ++ks) {
-                const at_v8h kk = __builtin_bit_cast(at_v8h, *reinterpret_cast<const at_v4u*>(krow_l + 16 * ks));
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(kk, Ql[ks], acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(kk, Q[ks], acc, 0, 0, 0);
+                const at_v8h kk0 = __builtin_bit_cast(at_v8h, *reinterpret_cast<const at_v4u*>(k0 + 16 * ks));
+                const at_v8h kk1 = __builtin_bit_cast(at_v8h, *reinterpret_cast<const at_v4u*>(k1 + 16 * ks));
+                a0l = __builtin_amdgcn_mfma_f32_16x16x32_f16(kk0, Ql[ks], a0l, 0, 0, 0);
+                a1l = __builtin_amdgcn_mfma_f32_16x16x32_f16(kk1, Ql[ks], a1l, 0, 0, 0);
+                a0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kk0, Q[ks], a0, 0, 0, 0);
+                a1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kk1, Q[ks], a1, 0, 0, 0);
             }
-            S[tile] = acc;
+            S[0] = a0 + a0l;
+            S[1] = a1 + a1l;
         }
         // this lane: query ql, positions c0 + 4 pg + r (tile 0) and c0 + 16 + 4 pg + r (tile 1)
         float sv[8];
@@ -479,8 +503,7 @@ __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per
             sv[r] = pos < ctx_q && pos < p1 ? S[r >> 2][r & 3] : -INFINITY;
             mx = fmaxf(mx, sv[r]);
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        mx = groups4_max(mx);
         const float mn = fmaxf(m, mx);
         const float sc = m == -INFINITY ? 0.f : __expf(m - mn);
         float pw[8], ps = 0.f;
@@ -489,8 +512,7 @@ __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per
             pw[r] = sv[r] == -INFINITY ? 0.f : __expf(sv[r] - mn);
             ps += pw[r];
         }
-        ps += __shfl_xor(ps, 16, 64);
-        ps += __shfl_xor(ps, 32, 64);
+        ps = groups4_sum(ps);
         z = z * sc + ps;
         m = mn;
         at_v8h P, Pl;
@@ -512,19 +534,45 @@ __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per
                 if (c0 + 16 + 4 * pg + j >= ctx_max) keep1[j >> 1] &= (j & 1) ? 0x0000FFFFu : 0xFFFF0000u;
             }
         }
-        const uint8_t* v0 = &lv[buf][pg * (AT_HD * 8) + ql * 8];
-        const uint8_t* v1 = &lv[buf][(4 + pg) * (AT_HD * 8) + ql * 8];
+        if (__any(sc != 1.0f)) {   // the running maximum moved (rare once the first chunks are behind)
 #pragma unroll
-        for (int dt = 0; dt < 16; ++dt) {
-            const at_v2u a0 = *reinterpret_cast<const at_v2u*>(v0 + 128 * dt), a1 = *reinterpret_cast<const at_v2u*>(v1 + 128 * dt);
-            const at_v4u a = at_v4u{a0.x & keep0[0], a0.y & keep0[1], a1.x & keep1[0], a1.y & keep1[1]};
-            at_v4f o = O[dt];
-            o.x *= sc;
-            o.y *= sc;
-            o.z *= sc;
-            o.w *= sc;
-            o = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(at_v8h, a), Pl, o, 0, 0, 0);
-            O[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(at_v8h, a), P, o, 0, 0, 0);
+            for (int dt = 0; dt < 16; ++dt) {
+                O[dt].x *= sc;
+                O[dt].y *= sc;
+                O[dt].z *= sc;
+                O[dt].w *= sc;
+            }
+        }
+        const uint8_t* v0 = &lv[buf][pg * AT_VLD + ql * 8];
+        const uint8_t* v1 = &lv[buf][(4 + pg) * AT_VLD + ql * 8];
+        // (the masks on every chunk: a second copy of this loop without them for the chunks inside the window costs more in
+        // registers than the 64 ANDs it saves)
+        // four dim tiles at a time: the lo products of all four, then the hi ones (a chain's next MFMA four issues away);
+        // the next four tiles' V reads are issued before this group's arithmetic
+        at_v2u ra[2][4][2];
+        auto vread = [&](int d0, at_v2u (&o)[4][2]) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                o[u][0] = *reinterpret_cast<const at_v2u*>(v0 + 128 * (d0 + u));
+                o[u][1] = *reinterpret_cast<const at_v2u*>(v1 + 128 * (d0 + u));
+            }
+        };
+        vread(0, ra[0]);
+#pragma unroll
+        for (int gq = 0; gq < 4; ++gq) {
+            if (gq < 3) vread(4 * (gq + 1), ra[(gq + 1) & 1]);
+            __builtin_amdgcn_sched_barrier(0);
+            at_v8h a[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const at_v2u a0 = ra[gq & 1][u][0], a1 = ra[gq & 1][u][1];
+                a[u] = __builtin_bit_cast(at_v8h, at_v4u{a0.x & keep0[0], a0.y & keep0[1], a1.x & keep1[0], a1.y & keep1[1]});
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) O[4 * gq + u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[u], Pl, O[4 * gq + u], 0, 0, 0);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) O[4 * gq + u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[u], P, O[4 * gq + u], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
         }
         __syncthreads();
     }
