@@ -107,6 +107,11 @@ inline void moe_down_mma(const DW& A, size_t sa, const BigJob* jobs, const int* 
 using Q8S = fnx_q8s;
 using Rope = fnx_rope;
 inline void rms_norm_rows(const float* x, const float* w, float* y, int rows, int n, float eps, void* st) { ck(fnx_rms_norm_rows(x, w, y, rows, n, eps, st)); }
+// the hand-over between two layers: moe_combine of the partial sums, the residual add, rms_norm_rows and quantize_q8_1 in one pass
+inline void combine_add_norm_q8(const float* part, const float* topw, const float* sh, const float* sh_logit, float* x, const float* w, float* xn,
+                                void* xq, int T, float eps, void* st) {
+    ck(fnx_combine_add_norm_q8(part, topw, sh, sh_logit, 1, shape().TOPK, x, w, xn, xq, T, shape().N, eps, st));
+}
 inline void q8s_gemv(const Q8S& w, const void* y, float* out, int out_stride, int T, void* st) { ck(fnx_q8s_gemv(&w, y, out, out_stride, T, st)); }
 inline void q8s_gemv_segs(const Q8S* w, float* const* out, const int* out_stride, int n, const void* y, int T, void* st) {
     const Q8S* p[3] = {&w[0], n > 1 ? &w[1] : nullptr, n > 2 ? &w[2] : nullptr};
