@@ -476,9 +476,22 @@ __global__ void __launch_bounds__(256) k_combine(const float* __restrict__ part,
                                                 int topk) {
     const int t = blockIdx.y, i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
+    // the chain in pick order, eight partial sums in flight at a time (one load per trip of the loop otherwise)
+    const float shv = sh[(size_t) t * n + i], sg = sigmoid_f(sh_logit[(size_t) t * sh_logit_stride]);
     float s = 0.f;
-    for (int k = 0; k < topk; ++k) s = fmaf(topw[t * topk + k], part[((size_t) t * topk + k) * n + i], s);
-    out[(size_t) t * n + i] = s + sigmoid_f(sh_logit[(size_t) t * sh_logit_stride]) * sh[(size_t) t * n + i];
+    for (int k0 = 0; k0 < topk; k0 += 8) {
+        float pv[8], wk[8];
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) {
+            const int k = min(k0 + kk, topk - 1);
+            wk[kk] = topw[t * topk + k];
+            pv[kk] = part[((size_t) t * topk + k) * n + i];
+        }
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk)
+            if (k0 + kk < topk) s = fmaf(wk[kk], pv[kk], s);
+    }
+    out[(size_t) t * n + i] = s + sg * shv;
 }
 
 // ================================================================ argmax (kernels.cu:1045-1083)

@@ -302,12 +302,23 @@ __global__ void __launch_bounds__(FL_THREADS) k_router_quant(const RouterArgs a)
                 }
         __syncthreads();
     }
+    // The wave's eight sums over the 64 lanes at once: at the butterfly's levels 32, 16 and 8 a lane keeps the half of
+    // its values whose index bit equals its lane bit and adds its partner's copy of them (the pairwise adds group_sum<64>
+    // makes for each value, so the same bits), then levels 4, 2, 1 on the one value left: 10 exchanges instead of 48.
+    // Lanes 8 j .. 8 j + 7 end with token tb + j's sum.
+    static_assert(FNX_MAXT / 2 == 8, "eight sums a wave");
+    float v4[4], v2[2];
 #pragma unroll
-    for (int t = 0; t < FNX_MAXT / 2; ++t)
-        if (tb + t < T) {
-            const float v = group_sum<64>(acc[t]);
-            if (live && lane == 0) a.logits[(size_t) (tb + t) * LS + row] = v;
-        }
+    for (int i = 0; i < 4; ++i) v4[i] = swap32_add(acc[i], acc[i + 4]);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) v2[i] = swap16_add(v4[i], v4[i + 2]);
+    const bool up = lane & 8;
+    float v = (up ? v2[1] : v2[0]) + __shfl_xor(up ? v2[0] : v2[1], 8, WAVE);
+    v += __shfl_xor(v, 4, WAVE);
+    v += __shfl_xor(v, 2, WAVE);
+    v += __shfl_xor(v, 1, WAVE);
+    const int t = tb + (lane >> 3);
+    if (live && (lane & 7) == 0 && t < T) a.logits[(size_t) t * LS + row] = v;
 }
 
 // ---------------------------------------------------------------- launches 3 and 4: the passes of the plan
