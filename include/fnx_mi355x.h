@@ -124,7 +124,7 @@ int fnx_argmax(const float* logits, int rows, int T, int v0, float* best_v, int*
  * the reference's LOOKUP_N; 2 and 4 are this build's parameterisation. Returns the draft count (<= lk) or -1 on a
  * bad argument; *match (may be null) = the run's start or -1. */
 int fnx_lookup_drafts(const int* ctx, int n_ctx, int key_n, int lk, int d1, int* out, int* match);
-/* the same on device memory, asynchronous: ctx, d1, out (lk ints), n_out, match are device pointers */
+/* the same on device memory, asynchronous: ctx, d1, out (lk ints), n_out, match are device pointers; lk <= 64 */
 int fnx_lookup_drafts_dev(const int* ctx, int n_ctx, int key_n, int lk, const int* d1, int* out, int* n_out, int* match, void* st);
 
 /* session.cpp:573  greedy acceptance: n = 1; while (n < R && rows[n] == o[n-1]) ++n  (host memory) */

@@ -567,66 +567,84 @@ __global__ void k_argmax_fin(unsigned long long* keys, int T, int v0, float* bv,
 
 // ================================================================ prompt lookup and acceptance on the device
 // (session.cpp:428-447, 573). One block: every thread tests its share of start positions for the key, the block keeps
-// the greatest matching start, thread 0 walks the short backward match and copies the drafts.
-constexpr int LK_THREADS = 1024, LOOKUP_MIN = 3, IMAGE_TOK = 1 << 30;
+// the greatest matching start, the first wave measures the backward match and copies the drafts (a lane per token).
+// Nothing here waits for one load after another: a thread's loads of a round are issued together (four start positions
+// a step - the 4 + 3 tokens they need are two 16-byte loads - and LK_STEPS steps a round), and the match and the copy are
+// a ballot each.
+constexpr int LK_THREADS = 1024, LK_STEPS = 10, LOOKUP_MIN = 3, IMAGE_TOK = 1 << 30;   // 40,960 start positions a round
 __global__ void __launch_bounds__(LK_THREADS) k_lookup(const int* __restrict__ ctx, int n_ctx, int key_n, int lk, const int* __restrict__ d1p,
                                                       int* __restrict__ out, int* __restrict__ n_out, int* __restrict__ match) {
     __shared__ int best;
     if (threadIdx.x == 0) best = -1;
+    const int d1 = *d1p;   // asked for now, used at the end
     __syncthreads();
     const int n0 = n_ctx - key_n;
     if (lk > 0 && n0 > 0) {
         int key[4];
         for (int j = 0; j < key_n; ++j) key[j] = ctx[n0 + j];
         int mine = -1;
-        if ((((uintptr_t) ctx) & 15) == 0) {
-            // four start positions a step: the 4 + 3 tokens they need are two 16-byte loads; steps are independent
-            for (int s4 = 4 * threadIdx.x; s4 < n0; s4 += 4 * LK_THREADS) {
-                int4 a = make_int4(0, 0, 0, 0), b = make_int4(0, 0, 0, 0);
-                if (s4 + 3 < n_ctx) a = *reinterpret_cast<const int4*>(ctx + s4);
-                else
-                    for (int j = 0; j < 4 && s4 + j < n_ctx; ++j) (&a.x)[j] = ctx[s4 + j];
-                if (s4 + 7 < n_ctx) b = *reinterpret_cast<const int4*>(ctx + s4 + 4);
-                else
-                    for (int j = 0; j < 4 && s4 + 4 + j < n_ctx; ++j) (&b.x)[j] = ctx[s4 + 4 + j];
-                const int w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+        // start positions below vec_end are tested four at a time from whole 16-byte loads; the few after them one by one
+        const bool aligned = (((uintptr_t) ctx) & 15) == 0;
+        const int vec_end = aligned && n_ctx >= 8 ? ((n_ctx - 8) / 4) * 4 + 4 : 0;
+        for (int base = 0; base < vec_end; base += 4 * LK_THREADS * LK_STEPS) {
+            int4 a[LK_STEPS], b[LK_STEPS];
+#pragma unroll
+            for (int k = 0; k < LK_STEPS; ++k) {
+                const int s4 = min(base + 4 * ((int) threadIdx.x + LK_THREADS * k), vec_end - 4);   // past the end: the last step again
+                a[k] = *reinterpret_cast<const int4*>(ctx + s4);
+                b[k] = *reinterpret_cast<const int4*>(ctx + s4 + 4);
+            }
+#pragma unroll
+            for (int k = 0; k < LK_STEPS; ++k) {
+                const int s4 = base + 4 * ((int) threadIdx.x + LK_THREADS * k);
+                const int w[8] = {a[k].x, a[k].y, a[k].z, a[k].w, b[k].x, b[k].y, b[k].z, b[k].w};
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    bool eq = s4 + i < n0;
+                    bool eq = s4 < vec_end && s4 + i < n0;
 #pragma unroll
                     for (int j = 0; j < 4; ++j)
                         if (j < key_n) eq = eq && w[i + j] == key[j];
                     if (eq) mine = s4 + i;   // ascending: the last one kept is this thread's greatest
                 }
             }
-        } else {
-            for (int s = threadIdx.x; s < n0; s += LK_THREADS) {
-                bool eq = true;
-                for (int j = 0; j < key_n; ++j) eq = eq && ctx[s + j] == key[j];
-                if (eq) mine = s;   // ascending s: the last one kept is this thread's greatest
-            }
+        }
+        for (int s = vec_end + threadIdx.x; s < n0; s += LK_THREADS) {
+            bool eq = true;
+            for (int j = 0; j < key_n; ++j) eq = eq && ctx[s + j] == key[j];
+            if (eq) mine = s;   // ascending s: the last one kept is this thread's greatest
         }
 #pragma unroll
         for (int o = 32; o; o >>= 1) mine = max(mine, __shfl_xor(mine, o, 64));
         if ((threadIdx.x & 63) == 0 && mine >= 0) atomicMax(&best, mine);
     }
     __syncthreads();
-    if (threadIdx.x != 0) return;
+    if (threadIdx.x >= 64) return;
+    const int lane = threadIdx.x;
     int nr = 0, m_at = -1;
-    const int s = best, d1 = *d1p;
-    if (s >= 0 && s + key_n < n_ctx && (d1 < 0 || ctx[s + key_n] == d1)) {
-        int m = key_n;
-        while (m < lk && (m - key_n) < s && ctx[s - 1 - (m - key_n)] == ctx[n0 - 1 - (m - key_n)]) ++m;
-        const int k = min(lk, max(LOOKUP_MIN, m)), end = min(n_ctx, s + key_n + k);
-        for (int i = s + key_n; i < end; ++i) {
-            const int tok = ctx[i];
-            if (tok >= IMAGE_TOK) break;   // an image cell is never a draft, nor anything after it
-            out[nr++] = tok;
-        }
+    const int s = best;
+    if (s >= 0 && s + key_n < n_ctx) {
+        // one trip to memory for everything the rest needs: the tokens before the match and before the key (lane j: the
+        // j-th back), and the up to lk tokens after the match (lane i: the i-th)
+        const int back = min(lk - key_n, s);
+        const int before_s = lane < back ? ctx[s - 1 - lane] : 0, before_k = lane < back ? ctx[n0 - 1 - lane] : 1;
+        const int tok = lane < lk && s + key_n + lane < n_ctx ? ctx[s + key_n + lane] : 0;
+        const int first = __builtin_amdgcn_readfirstlane(tok);   // ctx[s + key_n]
+        if (d1 >= 0 && first != d1) goto done;
+        // m = key_n + the tokens before the match that also agree (at most lk - key_n of them, and not before the context's start)
+        const unsigned long long miss = ~__ballot(before_s == before_k);   // lanes >= back are misses: the count stops there at the latest
+        const int m = key_n + (int) __builtin_ctzll(miss | (1ull << 63));
+        const int k = min(lk, max(LOOKUP_MIN, m)), end = min(n_ctx, s + key_n + k), want = end - (s + key_n);
+        // the drafts: a lane per token; an image cell is never a draft, nor anything after it
+        const unsigned long long stop = __ballot(lane < want && tok >= IMAGE_TOK);
+        nr = stop ? min(want, (int) __builtin_ctzll(stop)) : want;
+        if (lane < nr) out[lane] = tok;
         m_at = s;
     }
-    *n_out = nr;
-    if (match) *match = m_at;
+done:
+    if (lane == 0) {
+        *n_out = nr;
+        if (match) *match = m_at;
+    }
 }
 __global__ void k_accept(const int* __restrict__ rows, const int* __restrict__ o, int R, int* __restrict__ n_accept) {
     const int i = threadIdx.x;   // one wave; lane i tests draft i + 1 against row i's pick
@@ -881,7 +899,7 @@ int fnx_lookup_drafts(const int* ctx, int n_ctx, int key_n, int lk, int d1, int*
 }
 int fnx_lookup_drafts_dev(const int* ctx, int n_ctx, int key_n, int lk, const int* d1, int* out, int* n_out, int* match, void* st) {
     if (!ctx || !d1 || !out || !n_out) return fail("lookup_drafts_dev: null argument");
-    if (n_ctx < 0 || lk < 0 || key_n < 1 || key_n > 4) return fail("lookup_drafts_dev: bad argument");
+    if (n_ctx < 0 || lk < 0 || lk > 64 || key_n < 1 || key_n > 4) return fail("lookup_drafts_dev: bad argument (keys of 1..4 tokens, up to 64 drafts)");
     k_lookup<<<1, LK_THREADS, 0, (hipStream_t) st>>>(ctx, n_ctx, key_n, lk, d1, out, n_out, match);
     return launch_status("lookup_drafts_dev");
 }
