@@ -996,8 +996,11 @@ int fnx_swiglu_h16(const float* gu, int ffs, int P, uint16_t* h16, void* st) {
     k_swiglu_h16<<<(unsigned) std::min<size_t>((total + 255) / 256, 8192), 256, 0, (hipStream_t) st>>>(gu, ffs, total, h16);
     return launch_status("swiglu_h16");
 }
+// A2 (may be null): one more matrix of the same shape and layout with a job list of its own (jobs2, njobs2, cap2), run in
+// the same launch where the kernel form can (block and tile forms), else right after
 static int mma_launch(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const int* njobs, int njobs_cap, const uint16_t* x, float* out,
-                      void* st, const char* who) {
+                      void* st, const char* who, const fnx_dw* A2 = nullptr, const fnx_bigjob* jobs2 = nullptr, const int* njobs2 = nullptr,
+                      int cap2 = 0) {
     if (!A || !jobs || !njobs || !x || !out) return fail(std::string(who) + ": null argument");
     if (!A->p && !A->ep) return fail(std::string(who) + ": no weights");
     if (A->type != FNX_T_IQ3_S && A->type != FNX_T_IQ3S_UNIT64) return fail(std::string(who) + ": IQ3_S weights only");
@@ -1007,16 +1010,31 @@ static int mma_launch(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const 
     MmaArgs a{(const uint8_t*) A->p, sa, A->ep, A->n_out, A->n_in, jobs, njobs, njobs_cap, x, A->n_in, out};
     static const int per_cu = env_int("FNX_MMA_BLOCKS_PER_CU", 2, 1, 8), form = env_int("FNX_MMA_FORM", 1, 0, 1);
     static const int tile = env_int("FNX_MMA_TILE", 1, 0, 2);   // 0: never, 1: rows of up to 512 columns, 2: always
-    if (tile && A->type == FNX_T_IQ3S_UNIT64 && A->n_out % 16 == 0 && (tile == 2 || A->n_in <= 512)) {
+    const bool use_tile = tile && A->type == FNX_T_IQ3S_UNIT64 && A->n_out % 16 == 0 && (tile == 2 || A->n_in <= 512);
+    const bool use_block = !use_tile && form == 1 && A->type == FNX_T_IQ3S_UNIT64 && A->n_in % 512 == 0 && A->n_out % 16 == 0;
+    const bool merged = A2 && (use_tile || use_block) && A2->p && A2->type == A->type && A2->n_in == A->n_in && A2->n_out == A->n_out;
+    if (A2 && !merged) {   // a form without the second list: two launches
+        if (mma_launch(A, sa, jobs, njobs, njobs_cap, x, out, st, who)) return 1;
+        return mma_launch(A2, 0, jobs2, njobs2, cap2, x, out, st, who);
+    }
+    if (merged) {
+        if (!jobs2 || !njobs2 || cap2 < 1) return fail(std::string(who) + ": null argument");
+        a.w2 = (const uint8_t*) A2->p;
+        a.jobs2 = jobs2;
+        a.njobs2 = njobs2;
+        a.cap2 = cap2;
+    }
+    const long caps = (long) njobs_cap + (merged ? cap2 : 0);
+    if (use_tile) {
         // tile form: a block per (job, 32 tokens, 256 rows) in stages of 256 columns, one block a CU (its LDS)
-        const long tasks = (long) njobs_cap * ((A->n_out + MB_ROWS - 1) / MB_ROWS) * (MM_TT / MM_TP);
+        const long tasks = caps * ((A->n_out + MB_ROWS - 1) / MB_ROWS) * (MM_TT / MM_TP);
         const int grid = (int) std::max(1l, std::min<long>((long) cu_count(), tasks));
         k_moe_mma_tile<<<grid, MM_THREADS, 0, (hipStream_t) st>>>(a);
         return launch_status(who);
     }
-    if (form == 1 && A->type == FNX_T_IQ3S_UNIT64 && A->n_in % 512 == 0 && A->n_out % 16 == 0) {
+    if (use_block) {
         // block form: a block per (job, 32 tokens, 256 rows)
-        const long tasks = (long) njobs_cap * ((A->n_out + MB_ROWS - 1) / MB_ROWS) * (MM_TT / MM_TP);
+        const long tasks = caps * ((A->n_out + MB_ROWS - 1) / MB_ROWS) * (MM_TT / MM_TP);
         const int grid = (int) std::max(1l, std::min<long>((long) per_cu * cu_count(), tasks));
         k_moe_mma_block<<<grid, MM_THREADS, 0, (hipStream_t) st>>>(a);
         return launch_status(who);
@@ -1053,11 +1071,14 @@ int fnx_moe_prefill_layer(const fnx_moe_layer* L, const float* x, int C, float* 
     k_pf_shared_jobs<<<(C + 255) / 256, 256, 0, s>>>(C, P, ws->jobs_gu + J, ws->jobs_dn + J, ws->njobs + 1);
     if (launch_status("moe_prefill_layer shared jobs")) return 1;
     if (fnx_f32_f16(x, (size_t) C * n, ws->xh, st)) return 1;
-    if (fnx_moe_gate_up_mma(&L->gu, L->gu_stride, ws->jobs_gu, ws->njobs, J, ws->xh, ws->gu, st)) return 1;
-    if (fnx_moe_gate_up_mma(&L->sh_gu, 0, ws->jobs_gu + J, ws->njobs + 1, S, ws->xh, ws->gu, st)) return 1;
+    // the routed experts' jobs and the shared expert's in one launch each way
+    if (mma_launch(&L->gu, L->gu_stride, ws->jobs_gu, ws->njobs, J, ws->xh, ws->gu, st, "moe_prefill_layer gate|up", &L->sh_gu, ws->jobs_gu + J,
+                   ws->njobs + 1, S))
+        return 1;
     if (fnx_swiglu_h16(ws->gu, ff, P + C, ws->h16, st)) return 1;
-    if (fnx_moe_down_mma(&L->down, L->down_stride, ws->jobs_dn, ws->njobs, J, ws->h16, ws->part, st)) return 1;
-    if (fnx_moe_down_mma(&L->sh_down, 0, ws->jobs_dn + J, ws->njobs + 1, S, ws->h16, ws->part, st)) return 1;
+    if (mma_launch(&L->down, L->down_stride, ws->jobs_dn, ws->njobs, J, ws->h16, ws->part, st, "moe_prefill_layer down", &L->sh_down, ws->jobs_dn + J,
+                   ws->njobs + 1, S))
+        return 1;
     return fnx_moe_combine(ws->part, ws->topw, ws->part + (size_t) P * n, ws->logits + nexp, nexp + 1, out, C, n, topk, st);
 }
 

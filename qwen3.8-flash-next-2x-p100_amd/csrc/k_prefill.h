@@ -216,6 +216,12 @@ struct MmaArgs {
     const uint16_t* x;      // f16 activation rows of ldx values
     int ldx;
     float* out;             // rows of nrows
+    // a second job list over one more matrix (the shared expert's, whatever its jobs' w says), in the same launch: alone
+    // its few jobs fill a quarter of the chip (block and tile forms)
+    const uint8_t* w2 = nullptr;
+    const fnx_bigjob* jobs2 = nullptr;
+    const int* njobs2 = nullptr;
+    int cap2 = 0;
 };
 constexpr int MM_THREADS = 512, MM_WAVES = MM_THREADS / 64, MM_TT = FNX_PF_JOB / 16;
 
@@ -429,7 +435,7 @@ __global__ void __launch_bounds__(MM_THREADS) k_moe_mma_block(const MmaArgs a) {
         L.tab[i] = make_uint2(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi));
     }
     const int tid = threadIdx.x, lane = tid & 63, wave = uniform(tid >> 6), r = lane & 15, g = lane >> 4;
-    const int nj = min(a.cap, uniform(*a.njobs));
+    const int nj = min(a.cap, uniform(*a.njobs)), nj2 = a.jobs2 ? min(a.cap2, uniform(*a.njobs2)) : 0;
     const int ks = a.ncols >> 5, nsuper = ks >> 4, rblocks = (a.nrows + MB_ROWS - 1) / MB_ROWS;
     constexpr int HALVES = MM_TT / MM_TP;
     const int per_job = rblocks * HALVES;
@@ -437,14 +443,14 @@ __global__ void __launch_bounds__(MM_THREADS) k_moe_mma_block(const MmaArgs a) {
     // (sub-block xsb of the 16); in LDS the sub-block 4 g + p goes to step p, lane group g
     const int xtok = tid >> 4, xsb = tid & 15;
     const int xdst = xtok * MB_XROW + (xsb & 3) * MB_XLD + (xsb >> 2) * 64;
-    for (int task = blockIdx.x; task < nj * per_job; task += gridDim.x) {
+    for (int task = blockIdx.x; task < (nj + nj2) * per_job; task += gridDim.x) {
         const int ji = task / per_job, rem = task - ji * per_job, t0 = (rem / rblocks) * MM_TP, row0 = (rem % rblocks) * MB_ROWS + wave * 16 * MB_RG;
-        const fnx_bigjob* jb = a.jobs + ji;
+        const fnx_bigjob* jb = ji < nj ? a.jobs + ji : a.jobs2 + (ji - nj);
         const int n = min(FNX_PF_JOB, uniform(jb->n)), e = uniform(jb->w), nt = (n + 15) >> 4;
         if (n < 1 || t0 >= nt) continue;   // the same for every thread of the block
         const int ntile = min(MM_TP, nt - t0);
         const bool rows_live = row0 < a.nrows;   // per wave
-        const uint8_t* we = a.ep ? (const uint8_t*) a.ep[e] : a.w + (size_t) e * a.stride;
+        const uint8_t* we = ji >= nj ? a.w2 : a.ep ? (const uint8_t*) a.ep[e] : a.w + (size_t) e * a.stride;
         const uint16_t* xrow = a.x + (size_t) jb->y[min(t0 * 16 + xtok, n - 1)] * a.ldx + 32 * xsb;
         struct XShare {
             v4u v[4];
@@ -592,10 +598,10 @@ __global__ void __launch_bounds__(MM_THREADS) __attribute__((amdgpu_waves_per_eu
     uint32_t treg[SGRID_WORDS / MM_THREADS];
 #pragma unroll
     for (int i = 0; i < SGRID_WORDS / MM_THREADS; ++i) treg[i] = g_sgrid.v[tid + i * MM_THREADS];
-    const int nj = min(a.cap, uniform(*a.njobs));
+    const int nj = min(a.cap, uniform(*a.njobs)), nj2 = a.jobs2 ? min(a.cap2, uniform(*a.njobs2)) : 0;
     const int ks = a.ncols >> 5, nsuper = a.ncols / MT_K, rblocks = (a.nrows + MB_ROWS - 1) / MB_ROWS;
     constexpr int HALVES = MM_TT / MM_TP;
-    const int per_job = rblocks * HALVES, ntasks_all = nj * per_job;
+    const int per_job = rblocks * HALVES, ntasks_all = (nj + nj2) * per_job;
 #pragma unroll
     for (int i = 0; i < SGRID_WORDS / MM_THREADS; ++i) {
         const uint32_t gg = treg[i];
@@ -618,19 +624,19 @@ __global__ void __launch_bounds__(MM_THREADS) __attribute__((amdgpu_waves_per_eu
                 const int rem = task - ji * per_job;
                 t.t0 = (rem / rblocks) * MM_TP;
                 t.row0 = (rem % rblocks) * MB_ROWS;
-                const fnx_bigjob* jb = a.jobs + ji;
+                const fnx_bigjob* jb = ji < nj ? a.jobs + ji : a.jobs2 + (ji - nj);
                 n = min(FNX_PF_JOB, jb->n);
                 const int e = jb->w;
                 ok = n >= 1 && t.t0 < ((n + 15) >> 4);
                 t.ntile = min(MM_TP, ((n + 15) >> 4) - t.t0);
-                if (ok) t.we = a.ep ? (const uint8_t*) a.ep[e] : a.w + (size_t) e * a.stride;
+                if (ok) t.we = ji >= nj ? a.w2 : a.ep ? (const uint8_t*) a.ep[e] : a.w + (size_t) e * a.stride;
             }
             const unsigned long long m = __ballot(ok);
             const int slot = __popcll(m & ((1ull << lane) - 1ull));
             if (ok) {
                 L.task[slot] = t;
                 // the tile's token and output rows: 32 of each
-                const fnx_bigjob* jb = a.jobs + ji;
+                const fnx_bigjob* jb = ji < nj ? a.jobs + ji : a.jobs2 + (ji - nj);
                 for (int j = 0; j < MB_TOK; ++j) {
                     const int tok = t.t0 * 16 + j;
                     L.ytok[slot][j] = jb->y[min(tok, n - 1)];
