@@ -1000,7 +1000,7 @@ int fnx_swiglu_h16(const float* gu, int ffs, int P, uint16_t* h16, void* st) {
 // the same launch where the kernel form can (block and tile forms), else right after
 static int mma_launch(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const int* njobs, int njobs_cap, const uint16_t* x, float* out,
                       void* st, const char* who, const fnx_dw* A2 = nullptr, const fnx_bigjob* jobs2 = nullptr, const int* njobs2 = nullptr,
-                      int cap2 = 0) {
+                      int cap2 = 0, uint16_t* h16 = nullptr, bool* h16_done = nullptr) {
     if (!A || !jobs || !njobs || !x || !out) return fail(std::string(who) + ": null argument");
     if (!A->p && !A->ep) return fail(std::string(who) + ": no weights");
     if (A->type != FNX_T_IQ3_S && A->type != FNX_T_IQ3S_UNIT64) return fail(std::string(who) + ": IQ3_S weights only");
@@ -1025,6 +1025,13 @@ static int mma_launch(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const 
         a.cap2 = cap2;
     }
     const long caps = (long) njobs_cap + (merged ? cap2 : 0);
+    // stacked gate|up matrices on the block form can leave h = silu(gate) * up themselves
+    if (h16_done) *h16_done = false;
+    if (h16 && use_block && merged == (A2 != nullptr) && A->n_out % 256 == 0) {
+        a.h16 = h16;
+        a.ffh = A->n_out / 2;
+        if (h16_done) *h16_done = true;
+    }
     if (use_tile) {
         // tile form: a block per (job, 32 tokens, 256 rows) in stages of 256 columns, one block a CU (its LDS)
         const long tasks = caps * ((A->n_out + MB_ROWS - 1) / MB_ROWS) * (MM_TT / MM_TP);
@@ -1072,10 +1079,11 @@ int fnx_moe_prefill_layer(const fnx_moe_layer* L, const float* x, int C, float* 
     if (launch_status("moe_prefill_layer shared jobs")) return 1;
     if (fnx_f32_f16(x, (size_t) C * n, ws->xh, st)) return 1;
     // the routed experts' jobs and the shared expert's in one launch each way
+    bool h16_done = false;
     if (mma_launch(&L->gu, L->gu_stride, ws->jobs_gu, ws->njobs, J, ws->xh, ws->gu, st, "moe_prefill_layer gate|up", &L->sh_gu, ws->jobs_gu + J,
-                   ws->njobs + 1, S))
+                   ws->njobs + 1, S, ws->h16, &h16_done))
         return 1;
-    if (fnx_swiglu_h16(ws->gu, ff, P + C, ws->h16, st)) return 1;
+    if (!h16_done && fnx_swiglu_h16(ws->gu, ff, P + C, ws->h16, st)) return 1;
     if (mma_launch(&L->down, L->down_stride, ws->jobs_dn, ws->njobs, J, ws->h16, ws->part, st, "moe_prefill_layer down", &L->sh_down, ws->jobs_dn + J,
                    ws->njobs + 1, S))
         return 1;

@@ -222,6 +222,11 @@ struct MmaArgs {
     const fnx_bigjob* jobs2 = nullptr;
     const int* njobs2 = nullptr;
     int cap2 = 0;
+    // block form, stacked gate|up matrices (nrows = 2 ffh, ffh in 128s): a wave's two row groups are 16 gate rows and the
+    // 16 up rows that go with them, and what is written is h = silu(gate) * up as f16 rows of ffh (k_swiglu_h16's values)
+    // instead of the products themselves
+    uint16_t* h16 = nullptr;
+    int ffh = 0;
 };
 constexpr int MM_THREADS = 512, MM_WAVES = MM_THREADS / 64, MM_TT = FNX_PF_JOB / 16;
 
@@ -444,12 +449,15 @@ __global__ void __launch_bounds__(MM_THREADS) k_moe_mma_block(const MmaArgs a) {
     const int xtok = tid >> 4, xsb = tid & 15;
     const int xdst = xtok * MB_XROW + (xsb & 3) * MB_XLD + (xsb >> 2) * 64;
     for (int task = blockIdx.x; task < (nj + nj2) * per_job; task += gridDim.x) {
-        const int ji = task / per_job, rem = task - ji * per_job, t0 = (rem / rblocks) * MM_TP, row0 = (rem % rblocks) * MB_ROWS + wave * 16 * MB_RG;
+        const int ji = task / per_job, rem = task - ji * per_job, t0 = (rem / rblocks) * MM_TP;
+        // the wave's first row: of its 32 consecutive rows, or (h16) of its 16 gate rows - the up rows lie ffh further
+        const int row0 = a.h16 ? (rem % rblocks) * (MB_ROWS / 2) + wave * 16 : (rem % rblocks) * MB_ROWS + wave * 16 * MB_RG;
+        const int rlimit = a.h16 ? a.ffh : a.nrows, qstep = a.h16 ? a.ffh : 16;
         const fnx_bigjob* jb = ji < nj ? a.jobs + ji : a.jobs2 + (ji - nj);
         const int n = min(FNX_PF_JOB, uniform(jb->n)), e = uniform(jb->w), nt = (n + 15) >> 4;
         if (n < 1 || t0 >= nt) continue;   // the same for every thread of the block
         const int ntile = min(MM_TP, nt - t0);
-        const bool rows_live = row0 < a.nrows;   // per wave
+        const bool rows_live = row0 < rlimit;   // per wave
         const uint8_t* we = ji >= nj ? a.w2 : a.ep ? (const uint8_t*) a.ep[e] : a.w + (size_t) e * a.stride;
         const uint16_t* xrow = a.x + (size_t) jb->y[min(t0 * 16 + xtok, n - 1)] * a.ldx + 32 * xsb;
         struct XShare {
@@ -473,7 +481,7 @@ __global__ void __launch_bounds__(MM_THREADS) k_moe_mma_block(const MmaArgs a) {
             for (int tt = 0; tt < MM_TP; ++tt) acc[q][tt] = v4f{0.f, 0.f, 0.f, 0.f};
         int rowq[MB_RG];
 #pragma unroll
-        for (int q = 0; q < MB_RG; ++q) rowq[q] = min(row0 + 16 * q + r, a.nrows - 1);
+        for (int q = 0; q < MB_RG; ++q) rowq[q] = min(row0 + qstep * q + r, a.nrows - 1);
         const XShare x0 = x_load(0);
         SuperFields w0[MB_RG], w1[MB_RG];
 #pragma unroll
@@ -542,10 +550,18 @@ __global__ void __launch_bounds__(MM_THREADS) k_moe_mma_block(const MmaArgs a) {
             for (int tt = 0; tt < MM_TP; ++tt) {
                 const int tok = (t0 + tt) * 16 + r;
                 if (tt < ntile && tok < n) {
-                    float* o = a.out + (size_t) jb->out[tok] * a.nrows + row0 + 4 * g;
+                    if (a.h16) {   // gate rows in acc[0], their up rows in acc[1]
+                        const v4f gt = acc[0][tt], up = acc[1][tt];
+                        uint2 hv;
+                        hv.x = (uint32_t) float_to_half_bits(silu_f(gt.x) * up.x) | (uint32_t) float_to_half_bits(silu_f(gt.y) * up.y) << 16;
+                        hv.y = (uint32_t) float_to_half_bits(silu_f(gt.z) * up.z) | (uint32_t) float_to_half_bits(silu_f(gt.w) * up.w) << 16;
+                        *reinterpret_cast<uint2*>(a.h16 + (size_t) jb->out[tok] * a.ffh + row0 + 4 * g) = hv;
+                    } else {
+                        float* o = a.out + (size_t) jb->out[tok] * a.nrows + row0 + 4 * g;
 #pragma unroll
-                    for (int q = 0; q < MB_RG; ++q)
-                        if (row0 + 16 * q < a.nrows) *reinterpret_cast<float4*>(o + 16 * q) = make_float4(acc[q][tt].x, acc[q][tt].y, acc[q][tt].z, acc[q][tt].w);
+                        for (int q = 0; q < MB_RG; ++q)
+                            if (row0 + 16 * q < a.nrows) *reinterpret_cast<float4*>(o + 16 * q) = make_float4(acc[q][tt].x, acc[q][tt].y, acc[q][tt].z, acc[q][tt].w);
+                    }
                 }
             }
         }
