@@ -479,14 +479,25 @@ __global__ void __launch_bounds__(256) k_combine(const float* __restrict__ part,
     // the chain in pick order, eight partial sums in flight at a time (one load per trip of the loop otherwise)
     const float shv = sh[(size_t) t * n + i], sg = sigmoid_f(sh_logit[(size_t) t * sh_logit_stride]);
     float s = 0.f;
-    for (int k0 = 0; k0 < topk; k0 += 8) {
+    int k0 = 0;
+    for (; k0 + 8 <= topk; k0 += 8) {
         float pv[8], wk[8];
 #pragma unroll
         for (int kk = 0; kk < 8; ++kk) {
-            const int k = min(k0 + kk, topk - 1);
-            wk[kk] = topw[t * topk + k];
-            pv[kk] = part[((size_t) t * topk + k) * n + i];
+            wk[kk] = topw[t * topk + k0 + kk];
+            pv[kk] = part[((size_t) t * topk + k0 + kk) * n + i];
         }
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) s = fmaf(wk[kk], pv[kk], s);
+    }
+    if (k0 < topk) {   // the last few together too
+        float pv[8], wk[8];
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk)
+            if (k0 + kk < topk) {
+                wk[kk] = topw[t * topk + k0 + kk];
+                pv[kk] = part[((size_t) t * topk + k0 + kk) * n + i];
+            }
 #pragma unroll
         for (int kk = 0; kk < 8; ++kk)
             if (k0 + kk < topk) s = fmaf(wk[kk], pv[kk], s);
@@ -969,8 +980,9 @@ int fnx_moe_verify_layer(const fnx_moe_layer* L, const float* x, int T, float* o
 }
 
 // ---------------------------------------------------------------- the prompt path
-int fnx_pf_route(const float* logits, int logits_stride, int C, int nexp, int topk, int* topi, float* topw, int* cnt, int* jbase,
-                 fnx_bigjob* jobs_gu, fnx_bigjob* jobs_dn, int njobs_cap, int* njobs, void* st) {
+// sh_gu, sh_dn, nsh (null or all set): the shared expert's jobs over every row and their count, from the same launch
+static int pf_route(const float* logits, int logits_stride, int C, int nexp, int topk, int* topi, float* topw, int* cnt, int* jbase,
+                    fnx_bigjob* jobs_gu, fnx_bigjob* jobs_dn, int njobs_cap, int* njobs, fnx_bigjob* sh_gu, fnx_bigjob* sh_dn, int* nsh, void* st) {
     if (!logits || !topi || !topw || !cnt || !jbase || !jobs_gu || !jobs_dn || !njobs) return fail("pf_route: null argument");
     if (C < 1 || nexp < 1 || nexp > TK_MAXE || topk < 1 || topk > 64 || topk > nexp) return fail("pf_route: bad shape");
     if (logits_stride < nexp) return fail("pf_route: logits_stride smaller than nexp");
@@ -980,8 +992,13 @@ int fnx_pf_route(const float* logits, int logits_stride, int C, int nexp, int to
     const int P = C * topk;
     k_pf_topk<<<(C + PF_TOPK_WAVES - 1) / PF_TOPK_WAVES, PF_TOPK_WAVES * 64, 0, s>>>(logits, logits_stride, C, nexp, topk, topi, topw);
     k_pf_jobbase<<<1, PF_BASE_THREADS, 0, s>>>(topi, P, nexp, cnt, jbase, njobs);
-    k_pf_fill<<<nexp, PF_FILL_THREADS, 0, s>>>(topi, P, topk, cnt, jbase, jobs_gu, jobs_dn, njobs_cap);
+    const int shb = sh_gu ? (C + PF_FILL_THREADS - 1) / PF_FILL_THREADS : 0;
+    k_pf_fill<<<nexp + shb, PF_FILL_THREADS, 0, s>>>(topi, P, topk, nexp, cnt, jbase, jobs_gu, jobs_dn, njobs_cap, C, sh_gu, sh_dn, nsh);
     return launch_status("pf_route");
+}
+int fnx_pf_route(const float* logits, int logits_stride, int C, int nexp, int topk, int* topi, float* topw, int* cnt, int* jbase,
+                 fnx_bigjob* jobs_gu, fnx_bigjob* jobs_dn, int njobs_cap, int* njobs, void* st) {
+    return pf_route(logits, logits_stride, C, nexp, topk, topi, topw, cnt, jbase, jobs_gu, jobs_dn, njobs_cap, njobs, nullptr, nullptr, nullptr, st);
 }
 int fnx_f32_f16(const float* x, size_t n, uint16_t* out, void* st) {
     if (!x || !out) return fail("f32_f16: null argument");
@@ -1071,12 +1088,11 @@ int fnx_moe_prefill_layer(const fnx_moe_layer* L, const float* x, int C, float* 
         L->sh_gu.n_out != 2 * ff || L->sh_down.n_in != ff || L->sh_down.n_out != n)
         return fail("moe_prefill_layer: weight shapes do not match n / ff");
     const int P = C * topk, J = P / FNX_PF_JOB + nexp, S = (C + FNX_PF_JOB - 1) / FNX_PF_JOB;
-    hipStream_t s = (hipStream_t) st;
+    // the router logits; the routed experts' jobs, and the shared expert's from the same launch; x as f16
     if (gemv_any(L->router, L->router_bf16 != 0, x, ws->logits, nexp + 1, n, C, st, "moe_prefill_layer router")) return 1;
-    if (fnx_pf_route(ws->logits, nexp + 1, C, nexp, topk, ws->topi, ws->topw, ws->cnt, ws->jbase, ws->jobs_gu, ws->jobs_dn, J, ws->njobs, st))
+    if (pf_route(ws->logits, nexp + 1, C, nexp, topk, ws->topi, ws->topw, ws->cnt, ws->jbase, ws->jobs_gu, ws->jobs_dn, J, ws->njobs, ws->jobs_gu + J,
+                 ws->jobs_dn + J, ws->njobs + 1, st))
         return 1;
-    k_pf_shared_jobs<<<(C + 255) / 256, 256, 0, s>>>(C, P, ws->jobs_gu + J, ws->jobs_dn + J, ws->njobs + 1);
-    if (launch_status("moe_prefill_layer shared jobs")) return 1;
     if (fnx_f32_f16(x, (size_t) C * n, ws->xh, st)) return 1;
     // the routed experts' jobs and the shared expert's in one launch each way
     bool h16_done = false;

@@ -56,58 +56,77 @@ __global__ void __launch_bounds__(PF_BASE_THREADS) k_pf_jobbase(const int* __res
     if (e == PF_BASE_THREADS - 1) njobs[0] = s[e];
 }
 // a block per expert: its pairs in ascending order into the slots of its jobs (a pair always lands in the same job and
-// slot, prefill.cu:340-343); ballot prefix sums over the pairs
-constexpr int PF_FILL_THREADS = 256;
-__global__ void __launch_bounds__(PF_FILL_THREADS) k_pf_fill(const int* __restrict__ topi, int P, int topk, const int* __restrict__ cnt,
+// slot, prefill.cu:340-343). A thread looks at PF_ROUNDS pairs a pass (p = p0 + 256 r + tid), all loaded together; the
+// slots come from the waves' ballot counts, one barrier a pass. Blocks past the experts write the shared expert's
+// jobs (every row: gate|up reads row t, writes row P + t; down reads and writes row P + t) and their count.
+constexpr int PF_FILL_THREADS = 256, PF_ROUNDS = 8;
+__global__ void __launch_bounds__(PF_FILL_THREADS) k_pf_fill(const int* __restrict__ topi, int P, int topk, int nexp, const int* __restrict__ cnt,
                                                             const int* __restrict__ jbase, fnx_bigjob* __restrict__ gu,
-                                                            fnx_bigjob* __restrict__ dn, int cap) {
-    const int e = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+                                                            fnx_bigjob* __restrict__ dn, int cap, int C, fnx_bigjob* __restrict__ sh_gu,
+                                                            fnx_bigjob* __restrict__ sh_dn, int* __restrict__ nsh) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if ((int) blockIdx.x >= nexp) {
+        if (!sh_gu) return;
+        const int t = ((int) blockIdx.x - nexp) * PF_FILL_THREADS + tid;
+        if (t == 0) *nsh = (C + FNX_PF_JOB - 1) / FNX_PF_JOB;
+        if (t >= C) return;
+        const int j = t / FNX_PF_JOB, k = t % FNX_PF_JOB;
+        sh_gu[j].y[k] = t;
+        sh_gu[j].out[k] = P + t;
+        sh_dn[j].y[k] = P + t;
+        sh_dn[j].out[k] = P + t;
+        if (k == 0) {
+            sh_gu[j].w = sh_dn[j].w = 0;
+            sh_gu[j].n = sh_dn[j].n = min(FNX_PF_JOB, C - j * FNX_PF_JOB);
+        }
+        return;
+    }
+    const int e = blockIdx.x;
     const int ce = cnt[e], jb = jbase[e];
     if (ce == 0) return;
-    __shared__ int wsum[PF_FILL_THREADS / 64];
+    constexpr int NW = PF_FILL_THREADS / 64;
+    __shared__ int wsum[PF_ROUNDS][NW];
     int base = 0;
-    for (int p0 = 0; p0 < P; p0 += PF_FILL_THREADS) {
-        const int p = p0 + tid;
-        const bool mine = p < P && topi[p] == e;
-        const unsigned long long m = __ballot(mine);
-        if (lane == 0) wsum[wave] = __popcll(m);
-        __syncthreads();
-        int before = 0, total = 0;
+    for (int p0 = 0; p0 < P; p0 += PF_FILL_THREADS * PF_ROUNDS) {
+        int pick[PF_ROUNDS];
 #pragma unroll
-        for (int w = 0; w < PF_FILL_THREADS / 64; ++w) {
-            before += w < wave ? wsum[w] : 0;
-            total += wsum[w];
+        for (int r = 0; r < PF_ROUNDS; ++r) {
+            const int p = p0 + r * PF_FILL_THREADS + tid;
+            pick[r] = p < P ? topi[p] : -1;
         }
-        if (mine) {
-            const int s = base + before + __popcll(m & ((1ull << lane) - 1ull)), j = jb + s / FNX_PF_JOB, k = s % FNX_PF_JOB;
-            if (j < cap) {
-                gu[j].y[k] = p / topk;
-                gu[j].out[k] = p;
-                dn[j].y[k] = p;
-                dn[j].out[k] = p;
-                if (k == 0) {
-                    gu[j].w = dn[j].w = e;
-                    gu[j].n = dn[j].n = min(FNX_PF_JOB, ce - (s / FNX_PF_JOB) * FNX_PF_JOB);
+        unsigned long long m[PF_ROUNDS];
+#pragma unroll
+        for (int r = 0; r < PF_ROUNDS; ++r) {
+            m[r] = __ballot(pick[r] == e);
+            if (lane == 0) wsum[r][wave] = __popcll(m[r]);
+        }
+        __syncthreads();
+        int before = base;   // pairs of this expert before round r's wave `wave`
+#pragma unroll
+        for (int r = 0; r < PF_ROUNDS; ++r) {
+            int mine_before = before;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) {
+                mine_before += w < wave ? wsum[r][w] : 0;
+                before += wsum[r][w];
+            }
+            if (pick[r] == e) {
+                const int p = p0 + r * PF_FILL_THREADS + tid;
+                const int s = mine_before + __popcll(m[r] & ((1ull << lane) - 1ull)), j = jb + s / FNX_PF_JOB, k = s % FNX_PF_JOB;
+                if (j < cap) {
+                    gu[j].y[k] = p / topk;
+                    gu[j].out[k] = p;
+                    dn[j].y[k] = p;
+                    dn[j].out[k] = p;
+                    if (k == 0) {
+                        gu[j].w = dn[j].w = e;
+                        gu[j].n = dn[j].n = min(FNX_PF_JOB, ce - (s / FNX_PF_JOB) * FNX_PF_JOB);
+                    }
                 }
             }
         }
-        base += total;
+        base = before;
         __syncthreads();
-    }
-}
-// the shared expert as jobs over every row: gate|up reads row t, writes row P + t; down reads and writes row P + t
-__global__ void k_pf_shared_jobs(int C, int P, fnx_bigjob* __restrict__ gu, fnx_bigjob* __restrict__ dn, int* __restrict__ nsh) {
-    const int t = blockIdx.x * blockDim.x + threadIdx.x;
-    if (t == 0) *nsh = (C + FNX_PF_JOB - 1) / FNX_PF_JOB;
-    if (t >= C) return;
-    const int j = t / FNX_PF_JOB, k = t % FNX_PF_JOB;
-    gu[j].y[k] = t;
-    gu[j].out[k] = P + t;
-    dn[j].y[k] = P + t;
-    dn[j].out[k] = P + t;
-    if (k == 0) {
-        gu[j].w = dn[j].w = 0;
-        gu[j].n = dn[j].n = min(FNX_PF_JOB, C - j * FNX_PF_JOB);
     }
 }
 
