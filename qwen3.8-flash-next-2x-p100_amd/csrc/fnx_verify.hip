@@ -980,9 +980,11 @@ int fnx_moe_verify_layer(const fnx_moe_layer* L, const float* x, int T, float* o
 }
 
 // ---------------------------------------------------------------- the prompt path
-// sh_gu, sh_dn, nsh (null or all set): the shared expert's jobs over every row and their count, from the same launch
+// sh_gu, sh_dn, nsh (null or all set): the shared expert's jobs over every row and their count, from the same launch;
+// cvt_x, cvt_n, cvt_y (cvt_n > 0): floats to turn into f16 on the way (the first launch carries them)
 static int pf_route(const float* logits, int logits_stride, int C, int nexp, int topk, int* topi, float* topw, int* cnt, int* jbase,
-                    fnx_bigjob* jobs_gu, fnx_bigjob* jobs_dn, int njobs_cap, int* njobs, fnx_bigjob* sh_gu, fnx_bigjob* sh_dn, int* nsh, void* st) {
+                    fnx_bigjob* jobs_gu, fnx_bigjob* jobs_dn, int njobs_cap, int* njobs, fnx_bigjob* sh_gu, fnx_bigjob* sh_dn, int* nsh, void* st,
+                    const float* cvt_x = nullptr, size_t cvt_n = 0, uint16_t* cvt_y = nullptr) {
     if (!logits || !topi || !topw || !cnt || !jbase || !jobs_gu || !jobs_dn || !njobs) return fail("pf_route: null argument");
     if (C < 1 || nexp < 1 || nexp > TK_MAXE || topk < 1 || topk > 64 || topk > nexp) return fail("pf_route: bad shape");
     if (logits_stride < nexp) return fail("pf_route: logits_stride smaller than nexp");
@@ -990,7 +992,9 @@ static int pf_route(const float* logits, int logits_stride, int C, int nexp, int
     if (njobs_cap < 1) return fail("pf_route: no room for jobs");
     hipStream_t s = (hipStream_t) st;
     const int P = C * topk;
-    k_pf_topk<<<(C + PF_TOPK_WAVES - 1) / PF_TOPK_WAVES, PF_TOPK_WAVES * 64, 0, s>>>(logits, logits_stride, C, nexp, topk, topi, topw);
+    const int cvt_blocks = cvt_n ? (int) std::min<size_t>((cvt_n + 4095) / 4096, 2048) : 0;   // 16 values a thread or more
+    k_pf_topk<<<(C + PF_TOPK_WAVES - 1) / PF_TOPK_WAVES + cvt_blocks, PF_TOPK_WAVES * 64, 0, s>>>(logits, logits_stride, C, nexp, topk, topi, topw,
+                                                                                                  cvt_x, cvt_n, cvt_y);
     k_pf_jobbase<<<1, PF_BASE_THREADS, 0, s>>>(topi, P, nexp, cnt, jbase, njobs);
     const int shb = sh_gu ? (C + PF_FILL_THREADS - 1) / PF_FILL_THREADS : 0;
     k_pf_fill<<<nexp + shb, PF_FILL_THREADS, 0, s>>>(topi, P, topk, nexp, cnt, jbase, jobs_gu, jobs_dn, njobs_cap, C, sh_gu, sh_dn, nsh);
@@ -1088,12 +1092,11 @@ int fnx_moe_prefill_layer(const fnx_moe_layer* L, const float* x, int C, float* 
         L->sh_gu.n_out != 2 * ff || L->sh_down.n_in != ff || L->sh_down.n_out != n)
         return fail("moe_prefill_layer: weight shapes do not match n / ff");
     const int P = C * topk, J = P / FNX_PF_JOB + nexp, S = (C + FNX_PF_JOB - 1) / FNX_PF_JOB;
-    // the router logits; the routed experts' jobs, and the shared expert's from the same launch; x as f16
+    // the router logits; the routed experts' jobs, the shared expert's and x as f16 from the same launches
     if (gemv_any(L->router, L->router_bf16 != 0, x, ws->logits, nexp + 1, n, C, st, "moe_prefill_layer router")) return 1;
     if (pf_route(ws->logits, nexp + 1, C, nexp, topk, ws->topi, ws->topw, ws->cnt, ws->jbase, ws->jobs_gu, ws->jobs_dn, J, ws->njobs, ws->jobs_gu + J,
-                 ws->jobs_dn + J, ws->njobs + 1, st))
+                 ws->jobs_dn + J, ws->njobs + 1, st, x, (size_t) C * n, ws->xh))
         return 1;
-    if (fnx_f32_f16(x, (size_t) C * n, ws->xh, st)) return 1;
     // the routed experts' jobs and the shared expert's in one launch each way
     bool h16_done = false;
     if (mma_launch(&L->gu, L->gu_stride, ws->jobs_gu, ws->njobs, J, ws->xh, ws->gu, st, "moe_prefill_layer gate|up", &L->sh_gu, ws->jobs_gu + J,

@@ -20,11 +20,29 @@ typedef _Float16 v2h __attribute__((ext_vector_type(2)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 
 // ---------------------------------------------------------------- routing (prefill.cu:288-377)
-// a wave per row: top-k of its logits, the weights
+// a wave per row: top-k of its logits, the weights. The blocks past the rows' (cvt_n > 0) turn cvt_n floats at cvt_x into
+// f16 at cvt_y: the activations' copy for the matrix cores, which waits for nothing, rides along instead of a launch.
 constexpr int PF_TOPK_WAVES = 4;
 __global__ void __launch_bounds__(PF_TOPK_WAVES * 64) k_pf_topk(const float* __restrict__ logits, int ls, int C, int nexp, int topk,
-                                                               int* __restrict__ topi, float* __restrict__ topw) {
+                                                               int* __restrict__ topi, float* __restrict__ topw, const float* __restrict__ cvt_x,
+                                                               size_t cvt_n, uint16_t* __restrict__ cvt_y) {
     __shared__ int ex[PF_TOPK_WAVES][64];
+    const int row_blocks = (C + PF_TOPK_WAVES - 1) / PF_TOPK_WAVES;
+    if ((int) blockIdx.x >= row_blocks) {   // four values a thread and step
+        const size_t nb = gridDim.x - row_blocks, stride = nb * blockDim.x * 4;
+        for (size_t i = ((size_t) (blockIdx.x - row_blocks) * blockDim.x + threadIdx.x) * 4; i < cvt_n; i += stride) {
+            if (i + 3 < cvt_n && ((uintptr_t) cvt_x & 15) == 0 && ((uintptr_t) cvt_y & 7) == 0) {
+                const float4 v = *reinterpret_cast<const float4*>(cvt_x + i);
+                uint2 h;
+                h.x = (uint32_t) float_to_half_bits(v.x) | (uint32_t) float_to_half_bits(v.y) << 16;
+                h.y = (uint32_t) float_to_half_bits(v.z) | (uint32_t) float_to_half_bits(v.w) << 16;
+                *reinterpret_cast<uint2*>(cvt_y + i) = h;
+            } else {
+                for (size_t j = i; j < i + 4 && j < cvt_n; ++j) cvt_y[j] = float_to_half_bits(cvt_x[j]);
+            }
+        }
+        return;
+    }
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, t = blockIdx.x * PF_TOPK_WAVES + wave;
     if (t >= C) return;
     if (nexp <= 512) wave_topk<8>(logits + (size_t) t * ls, nexp, topk, lane, ex[wave], topi + (size_t) t * topk, topw + (size_t) t * topk);
