@@ -1126,7 +1126,8 @@ int fnx_combine_add_norm_q8(const float* part, const float* topw, const float* s
                             const float* w, float* xn, void* xq, int rows, int n, float eps, void* st) {
     if (!part || !topw || !sh || !sh_logit || !x || !w) return fail("combine_add_norm_q8: null argument");
     if (rows < 1 || n < 32 || n % 32 || n > 256 * NQ_MAXJ || topk < 1) return fail("combine_add_norm_q8: rows of 32 .. 4096 values in whole 32-value blocks");
-    k_add_norm_q8<<<rows, 256, 0, (hipStream_t) st>>>(x, nullptr, CombineArgs{part, topw, sh, sh_logit, sh_logit_stride, topk}, w, xn, (uint8_t*) xq, n, eps);
+    k_add_norm_q8<<<rows, 256, 0, (hipStream_t) st>>>(x, nullptr, CombineArgs{part, topw, sh, sh_logit, sh_logit_stride, topk, nullptr}, w, xn,
+                                                      (uint8_t*) xq, n, eps);
     return launch_status("combine_add_norm_q8");
 }
 int fnx_add_rows(const float* a, const float* b, float* y, size_t n, void* st) {
@@ -1233,12 +1234,17 @@ struct DecPending {
     const float* rows;
     const fnx_moe_layer* moe;
 };
-static int dec_add_norm_q8(const fnx_decoder* D, const DecPending& pend, const float* w, int T, const fnx_dec_ws* ws, void* st) {
-    if (!pend.moe) return fnx_add_norm_q8(ws->x, pend.rows, w, nullptr, ws->xq, T, D->n, D->eps, st);
-    const fnx_moe_layer* M = pend.moe;
-    const int P = T * M->topk;
-    return fnx_combine_add_norm_q8(ws->moe.part, ws->moe.topw, ws->moe.part + (size_t) P * D->n, ws->moe.logits + M->nexp, M->nexp + 1, M->topk, ws->x, w,
-                                   nullptr, ws->xq, T, D->n, D->eps, st);
+// xcopy (may be null): the rows after the add go there too
+static int dec_add_norm_q8(const fnx_decoder* D, const DecPending& pend, const float* w, int T, const fnx_dec_ws* ws, void* st, float* xcopy = nullptr) {
+    CombineArgs c{};
+    if (pend.moe) {
+        const fnx_moe_layer* M = pend.moe;
+        c = CombineArgs{ws->moe.part, ws->moe.topw, ws->moe.part + (size_t) T * M->topk * D->n, ws->moe.logits + M->nexp, M->nexp + 1, M->topk, nullptr};
+    }
+    c.xcopy = xcopy;
+    if (D->n < 32 || D->n % 32 || D->n > 256 * NQ_MAXJ) return fail("decoder: rows of 32 .. 4096 values in whole 32-value blocks");
+    k_add_norm_q8<<<T, 256, 0, (hipStream_t) st>>>(ws->x, pend.moe ? nullptr : pend.rows, c, w, nullptr, (uint8_t*) ws->xq, D->n, D->eps);
+    return launch_status("decoder add_norm_q8");
 }
 // x (ws->x) through one layer, in place; the layer's own MoE output is left pending for whatever comes next
 static int dec_layer(const fnx_decoder* D, const fnx_dec_layer* L, int T, const int* pos0, const fnx_dec_ws* ws, DecPending& pend, void* st) {
@@ -1271,9 +1277,7 @@ static int dec_shape_check(const fnx_decoder* D, int T, const char* who) {
 }
 // x += pending; hidden = x; the output norm, the head, argmax
 static int dec_head(const fnx_decoder* D, const float* norm, const fnx_q8s* head, int T, const fnx_dec_ws* ws, const DecPending& pend, void* st) {
-    if (dec_add_norm_q8(D, pend, norm, T, ws, st)) return 1;
-    if (hipMemcpyAsync(ws->hidden, ws->x, (size_t) T * D->n * sizeof(float), hipMemcpyDeviceToDevice, (hipStream_t) st) != hipSuccess)
-        return fail("decoder: copy of the hidden rows failed");
+    if (dec_add_norm_q8(D, pend, norm, T, ws, st, ws->hidden)) return 1;   // hidden = x, written by the same pass
     if (fnx_q8s_gemv(head, ws->xq, ws->logits, D->vocab, T, st)) return 1;
     return fnx_argmax(ws->logits, D->vocab, T, 0, ws->best_v, ws->best_i, ws->keys, ws->err, st);
 }

@@ -35,6 +35,7 @@ struct CombineArgs {
     const float* sh;
     const float* sh_logit;
     int sh_logit_stride, topk;
+    float* xcopy;        // may be null: the rows after the add go there as well (the hidden rows the draft layer starts from)
 };
 __global__ void __launch_bounds__(256) k_add_norm_q8(float* __restrict__ x, const float* __restrict__ add, const CombineArgs c,
                                                     const float* __restrict__ w, float* __restrict__ xn, uint8_t* __restrict__ xq, int n, float eps) {
@@ -104,6 +105,13 @@ __global__ void __launch_bounds__(256) k_add_norm_q8(float* __restrict__ x, cons
         for (int j = 0; j < NQ_MAXJ; ++j) {
             const int i = threadIdx.x + 256 * j;
             if (i < n) x[row * n + i] = v[j];
+        }
+    }
+    if (c.xcopy) {
+#pragma unroll
+        for (int j = 0; j < NQ_MAXJ; ++j) {
+            const int i = threadIdx.x + 256 * j;
+            if (i < n) c.xcopy[row * n + i] = v[j];
         }
     }
 #pragma unroll
