@@ -1126,7 +1126,7 @@ int fnx_combine_add_norm_q8(const float* part, const float* topw, const float* s
                             const float* w, float* xn, void* xq, int rows, int n, float eps, void* st) {
     if (!part || !topw || !sh || !sh_logit || !x || !w) return fail("combine_add_norm_q8: null argument");
     if (rows < 1 || n < 32 || n % 32 || n > 256 * NQ_MAXJ || topk < 1) return fail("combine_add_norm_q8: rows of 32 .. 4096 values in whole 32-value blocks");
-    k_add_norm_q8<<<rows, 256, 0, (hipStream_t) st>>>(x, nullptr, CombineArgs{part, topw, sh, sh_logit, sh_logit_stride, topk, nullptr}, w, xn,
+    k_add_norm_q8<<<rows, 256, 0, (hipStream_t) st>>>(x, nullptr, CombineArgs{part, topw, sh, sh_logit, sh_logit_stride, topk, nullptr, nullptr, nullptr, 0}, w, xn,
                                                       (uint8_t*) xq, n, eps);
     return launch_status("combine_add_norm_q8");
 }
@@ -1233,15 +1233,22 @@ static int dec_ws_check(const fnx_dec_ws* ws, const char* who) {
 struct DecPending {
     const float* rows;
     const fnx_moe_layer* moe;
+    const int* tokens;   // not null: x itself is still to come - the embedding rows of these tokens (nothing else pending then)
 };
 // xcopy (may be null): the rows after the add go there too
 static int dec_add_norm_q8(const fnx_decoder* D, const DecPending& pend, const float* w, int T, const fnx_dec_ws* ws, void* st, float* xcopy = nullptr) {
     CombineArgs c{};
     if (pend.moe) {
         const fnx_moe_layer* M = pend.moe;
-        c = CombineArgs{ws->moe.part, ws->moe.topw, ws->moe.part + (size_t) T * M->topk * D->n, ws->moe.logits + M->nexp, M->nexp + 1, M->topk, nullptr};
+        c = CombineArgs{ws->moe.part, ws->moe.topw, ws->moe.part + (size_t) T * M->topk * D->n, ws->moe.logits + M->nexp, M->nexp + 1, M->topk, nullptr,
+                        nullptr, nullptr, 0};
     }
     c.xcopy = xcopy;
+    if (pend.tokens) {
+        c.emb = D->emb;
+        c.tokens = pend.tokens;
+        c.vocab = D->vocab;
+    }
     if (D->n < 32 || D->n % 32 || D->n > 256 * NQ_MAXJ) return fail("decoder: rows of 32 .. 4096 values in whole 32-value blocks");
     k_add_norm_q8<<<T, 256, 0, (hipStream_t) st>>>(ws->x, pend.moe ? nullptr : pend.rows, c, w, nullptr, (uint8_t*) ws->xq, D->n, D->eps);
     return launch_status("decoder add_norm_q8");
@@ -1262,10 +1269,10 @@ static int dec_layer(const fnx_decoder* D, const fnx_dec_layer* L, int T, const 
     if (fnx_q8s_gemv(&L->wo, ws->xq, ws->o, n, T, st)) return 1;
     if (fnx_add_norm_q8(ws->x, ws->o, L->ffn_norm, ws->xn, nullptr, T, n, D->eps, st)) return 1;
     if (layer_fused_ok(&L->moe, T)) {   // the window without its combine
-        pend = DecPending{nullptr, &L->moe};
+        pend = DecPending{nullptr, &L->moe, nullptr};
         return moe_layer_checked(&L->moe, ws->xn, T, nullptr, &ws->moe, st);
     }
-    pend = DecPending{ws->o, nullptr};
+    pend = DecPending{ws->o, nullptr, nullptr};
     return fnx_moe_verify_layer(&L->moe, ws->xn, T, ws->o, &ws->moe, st);
 }
 static int dec_shape_check(const fnx_decoder* D, int T, const char* who) {
@@ -1284,8 +1291,7 @@ static int dec_head(const fnx_decoder* D, const float* norm, const fnx_q8s* head
 int fnx_decoder_verify(const fnx_decoder* D, const int* tokens, int T, const int* pos0, const fnx_dec_ws* ws, void* st) {
     if (!D || !tokens || !pos0 || !ws || !D->layers || !D->out_norm || !D->emb) return fail("decoder_verify: null argument");
     if (dec_shape_check(D, T, "decoder_verify") || dec_ws_check(ws, "decoder_verify")) return 1;
-    if (fnx_embed_rows(D->emb, tokens, T, D->vocab, D->n, ws->x, st)) return 1;
-    DecPending pend{nullptr, nullptr};
+    DecPending pend{nullptr, nullptr, tokens};   // the window's input rows are read by the first pass over them
     for (int l = 0; l < D->nlayers; ++l)
         if (dec_layer(D, &D->layers[l], T, pos0, ws, pend, st)) return 1;
     return dec_head(D, D->out_norm, &D->head, T, ws, pend, st);
@@ -1301,7 +1307,7 @@ int fnx_mtp_draft(const fnx_decoder* D, const fnx_mtp* M, const float* src, cons
     if (fnx_embed_rows(D->emb, tokens, T, D->vocab, n, ws->xn, st)) return 1;
     if (fnx_add_norm_q8(ws->xn, nullptr, M->norm_emb, nullptr, ws->xq, T, n, D->eps, st)) return 1;
     if (fnx_q8s_gemv(&M->fc_emb, ws->xq, ws->o, n, T, st)) return 1;
-    DecPending pend{ws->o, nullptr};
+    DecPending pend{ws->o, nullptr, nullptr};
     if (dec_layer(D, &M->layer, T, pos0, ws, pend, st)) return 1;
     return dec_head(D, M->out_norm, &M->head, T, ws, pend, st);
 }

@@ -36,6 +36,9 @@ struct CombineArgs {
     const float* sh_logit;
     int sh_logit_stride, topk;
     float* xcopy;        // may be null: the rows after the add go there as well (the hidden rows the draft layer starts from)
+    const uint16_t* emb;  // may be null: the rows do not come from x but are rows tokens[r] of this f16 table (and go to x)
+    const int* tokens;
+    int vocab;
 };
 __global__ void __launch_bounds__(256) k_add_norm_q8(float* __restrict__ x, const float* __restrict__ add, const CombineArgs c,
                                                     const float* __restrict__ w, float* __restrict__ xn, uint8_t* __restrict__ xq, int n, float eps) {
@@ -83,10 +86,12 @@ __global__ void __launch_bounds__(256) k_add_norm_q8(float* __restrict__ x, cons
     } else {
         // all loads first: a store to x between them would keep the next load waiting for it
         float av[NQ_MAXJ];
+        const size_t erow = c.emb ? (size_t) min(max(c.tokens[row], 0), c.vocab - 1) : 0;   // k_embed_rows' clamp
 #pragma unroll
         for (int j = 0; j < NQ_MAXJ; ++j) {
             const int i = threadIdx.x + 256 * j;
-            v[j] = i < n ? x[row * n + i] : 0.f;
+            if (c.emb) v[j] = i < n ? half_bits_to_float(c.emb[erow * n + i]) : 0.f;
+            else v[j] = i < n ? x[row * n + i] : 0.f;
             av[j] = add && i < n ? add[row * n + i] : 0.f;
         }
         if (add) {
@@ -100,7 +105,7 @@ __global__ void __launch_bounds__(256) k_add_norm_q8(float* __restrict__ x, cons
         const int i = threadIdx.x + 256 * j;
         wv[j] = i < n ? w[i] : 0.f;
     }
-    if (add || c.part) {
+    if (add || c.part || c.emb) {
 #pragma unroll
         for (int j = 0; j < NQ_MAXJ; ++j) {
             const int i = threadIdx.x + 256 * j;
