@@ -1119,15 +1119,15 @@ int fnx_rms_norm_rows(const float* x, const float* w, float* y, int rows, int n,
 int fnx_add_norm_q8(float* x, const float* add, const float* w, float* xn, void* xq, int rows, int n, float eps, void* st) {
     if (!x || !w) return fail("add_norm_q8: null argument");
     if (rows < 1 || n < 32 || n % 32 || n > 256 * NQ_MAXJ) return fail("add_norm_q8: rows of 32 .. 4096 values in whole 32-value blocks");
-    k_add_norm_q8<<<rows, 256, 0, (hipStream_t) st>>>(x, add, CombineArgs{}, w, xn, (uint8_t*) xq, n, eps);
+    k_add_norm_q8<false><<<rows, 256, 0, (hipStream_t) st>>>(x, add, CombineArgs{}, w, xn, (uint8_t*) xq, n, eps);
     return launch_status("add_norm_q8");
 }
 int fnx_combine_add_norm_q8(const float* part, const float* topw, const float* sh, const float* sh_logit, int sh_logit_stride, int topk, float* x,
                             const float* w, float* xn, void* xq, int rows, int n, float eps, void* st) {
     if (!part || !topw || !sh || !sh_logit || !x || !w) return fail("combine_add_norm_q8: null argument");
     if (rows < 1 || n < 32 || n % 32 || n > 256 * NQ_MAXJ || topk < 1) return fail("combine_add_norm_q8: rows of 32 .. 4096 values in whole 32-value blocks");
-    k_add_norm_q8<<<rows, 256, 0, (hipStream_t) st>>>(x, nullptr, CombineArgs{part, topw, sh, sh_logit, sh_logit_stride, topk, nullptr, nullptr, nullptr, 0}, w, xn,
-                                                      (uint8_t*) xq, n, eps);
+    k_add_norm_q8<true><<<rows, 1024, 0, (hipStream_t) st>>>(x, nullptr, CombineArgs{part, topw, sh, sh_logit, sh_logit_stride, topk, nullptr, nullptr, nullptr, 0},
+                                                             w, xn, (uint8_t*) xq, n, eps);
     return launch_status("combine_add_norm_q8");
 }
 int fnx_add_rows(const float* a, const float* b, float* y, size_t n, void* st) {
@@ -1250,7 +1250,8 @@ static int dec_add_norm_q8(const fnx_decoder* D, const DecPending& pend, const f
         c.vocab = D->vocab;
     }
     if (D->n < 32 || D->n % 32 || D->n > 256 * NQ_MAXJ) return fail("decoder: rows of 32 .. 4096 values in whole 32-value blocks");
-    k_add_norm_q8<<<T, 256, 0, (hipStream_t) st>>>(ws->x, pend.moe ? nullptr : pend.rows, c, w, nullptr, (uint8_t*) ws->xq, D->n, D->eps);
+    if (pend.moe) k_add_norm_q8<true><<<T, 1024, 0, (hipStream_t) st>>>(ws->x, nullptr, c, w, nullptr, (uint8_t*) ws->xq, D->n, D->eps);
+    else k_add_norm_q8<false><<<T, 256, 0, (hipStream_t) st>>>(ws->x, pend.rows, c, w, nullptr, (uint8_t*) ws->xq, D->n, D->eps);
     return launch_status("decoder add_norm_q8");
 }
 // x (ws->x) through one layer, in place; the layer's own MoE output is left pending for whatever comes next

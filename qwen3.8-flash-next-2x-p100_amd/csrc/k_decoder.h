@@ -40,28 +40,34 @@ struct CombineArgs {
     const int* tokens;
     int vocab;
 };
-__global__ void __launch_bounds__(256) k_add_norm_q8(float* __restrict__ x, const float* __restrict__ add, const CombineArgs c,
-                                                    const float* __restrict__ w, float* __restrict__ xn, uint8_t* __restrict__ xq, int n, float eps) {
+// WIDE (the combine's form): 1024 threads make the row after the add - a thread the columns p, p + 1024, ..., with all
+// of an expert batch's partial sums in flight (256 threads with 8 columns each took 13 us a call, against 7 us without
+// the combine) - and hand it over in LDS to the first 256, which go on as in the narrow form: the same values and orders.
+template <bool WIDE>
+__global__ void __launch_bounds__(WIDE ? 1024 : 256) k_add_norm_q8(float* __restrict__ x, const float* __restrict__ add, const CombineArgs c,
+                                                                  const float* __restrict__ w, float* __restrict__ xn, uint8_t* __restrict__ xq, int n,
+                                                                  float eps) {
     __shared__ float sh[4];
+    __shared__ float vrow[WIDE ? 256 * NQ_MAXJ : 1];
     const size_t row = blockIdx.x;
     float v[NQ_MAXJ];
     float s = 0.f;
-    if (c.part) {
-        // the combine's chains, NQ_KB experts' partial sums of all this thread's columns in flight at a time (one by one,
-        // each load would be a trip to the cache of its own)
-        constexpr int NQ_KB = 5;
-        float m[NQ_MAXJ];
+    if constexpr (WIDE) {
+        // the combine's chains (k_combine's order: the picks ascending), NQ_KB experts' partial sums of this thread's
+        // columns in flight at a time (one by one, each load would be a trip to the cache of its own)
+        constexpr int NQ_KB = 5, NQ_WJ = NQ_MAXJ / 4;
+        float m[NQ_WJ];
 #pragma unroll
-        for (int j = 0; j < NQ_MAXJ; ++j) m[j] = 0.f;
+        for (int j = 0; j < NQ_WJ; ++j) m[j] = 0.f;
         for (int k0 = 0; k0 < c.topk; k0 += NQ_KB) {
-            float pv[NQ_KB][NQ_MAXJ], wk[NQ_KB];
+            float pv[NQ_KB][NQ_WJ], wk[NQ_KB];
 #pragma unroll
             for (int kk = 0; kk < NQ_KB; ++kk) {
                 const int k = min(k0 + kk, c.topk - 1);
                 wk[kk] = c.topw[row * c.topk + k];
 #pragma unroll
-                for (int j = 0; j < NQ_MAXJ; ++j) {
-                    const int i = threadIdx.x + 256 * j;
+                for (int j = 0; j < NQ_WJ; ++j) {
+                    const int i = threadIdx.x + 1024 * j;
                     pv[kk][j] = i < n ? c.part[(row * c.topk + k) * n + i] : 0.f;
                 }
             }
@@ -70,19 +76,31 @@ __global__ void __launch_bounds__(256) k_add_norm_q8(float* __restrict__ x, cons
             for (int kk = 0; kk < NQ_KB; ++kk)
                 if (k0 + kk < c.topk) {
 #pragma unroll
-                    for (int j = 0; j < NQ_MAXJ; ++j) m[j] = fmaf(wk[kk], pv[kk][j], m[j]);
+                    for (int j = 0; j < NQ_WJ; ++j) m[j] = fmaf(wk[kk], pv[kk][j], m[j]);
                 }
         }
         const float sg = sigmoid_f(c.sh_logit[row * c.sh_logit_stride]);
-        float shv[NQ_MAXJ];
+        float xv[NQ_WJ], shv[NQ_WJ];
 #pragma unroll
-        for (int j = 0; j < NQ_MAXJ; ++j) {
-            const int i = threadIdx.x + 256 * j;
-            v[j] = i < n ? x[row * n + i] : 0.f;
+        for (int j = 0; j < NQ_WJ; ++j) {
+            const int i = threadIdx.x + 1024 * j;
+            xv[j] = i < n ? x[row * n + i] : 0.f;
             shv[j] = i < n ? c.sh[row * n + i] : 0.f;
         }
 #pragma unroll
-        for (int j = 0; j < NQ_MAXJ; ++j) v[j] += m[j] + sg * shv[j];
+        for (int j = 0; j < NQ_WJ; ++j) {
+            const int i = threadIdx.x + 1024 * j;
+            const float r = xv[j] + (m[j] + sg * shv[j]);
+            vrow[i] = i < n ? r : 0.f;
+            if (i < n) {
+                x[row * n + i] = r;
+                if (c.xcopy) c.xcopy[row * n + i] = r;
+            }
+        }
+        __syncthreads();
+        if (threadIdx.x >= 256) return;
+#pragma unroll
+        for (int j = 0; j < NQ_MAXJ; ++j) v[j] = vrow[threadIdx.x + 256 * j];
     } else {
         // all loads first: a store to x between them would keep the next load waiting for it
         float av[NQ_MAXJ];
@@ -105,14 +123,14 @@ __global__ void __launch_bounds__(256) k_add_norm_q8(float* __restrict__ x, cons
         const int i = threadIdx.x + 256 * j;
         wv[j] = i < n ? w[i] : 0.f;
     }
-    if (add || c.part || c.emb) {
+    if (!WIDE && (add || c.emb)) {
 #pragma unroll
         for (int j = 0; j < NQ_MAXJ; ++j) {
             const int i = threadIdx.x + 256 * j;
             if (i < n) x[row * n + i] = v[j];
         }
     }
-    if (c.xcopy) {
+    if (!WIDE && c.xcopy) {
 #pragma unroll
         for (int j = 0; j < NQ_MAXJ; ++j) {
             const int i = threadIdx.x + 256 * j;
