@@ -209,12 +209,23 @@ __global__ void __launch_bounds__(RT_THREADS) k_route_plan(const RouteArgs a) {
         }
     }
     __syncthreads();
-    // passes: job j's rows two at a time; job j's first pass = the passes of the jobs before it
-    for (int j = tid; j <= nj; j += RT_THREADS) {
-        int at = 0;
-        for (int i = 0; i < j; ++i) at += (pl.job_n[i] + 1) >> 1;
-        L.pass0[j] = at;
-        if (j == nj) pl.npass = at + ((pl.job_n[j] + 1) >> 1);
+    // passes: job j's rows two at a time; job j's first pass = the passes of the jobs before it: a scan over the jobs
+    // (wave by wave with the waves' totals in LDS; a thread per job)
+    static_assert(FL_MAXJ <= RT_THREADS, "a thread per job");
+    {
+        const int cj = tid <= nj ? (pl.job_n[tid] + 1) >> 1 : 0;
+        int inc = cj;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const int up = __shfl_up(inc, o, 64);
+            if (lane >= o) inc += up;
+        }
+        if (lane == 63) L.wcnt[wave] = inc;
+        __syncthreads();
+        int before = 0;
+        for (int w = 0; w < wave; ++w) before += L.wcnt[w];
+        if (tid <= nj) L.pass0[tid] = before + inc - cj;
+        if (tid == nj) pl.npass = before + inc;
     }
     __syncthreads();
     for (int j = tid; j <= nj; j += RT_THREADS)
