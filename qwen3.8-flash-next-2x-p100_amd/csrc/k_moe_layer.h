@@ -70,20 +70,29 @@ __device__ __forceinline__ void wave_topk(const float* __restrict__ row, int nex
         const int e = lane + 64 * i;
         v[i] = e < nexp ? row[e] : -INFINITY;
     }
-    unsigned taken = 0;
     float top0 = 0.f, z = 0.f, wk = 0.f;
     for (int k = 0; k < topk; ++k) {
-        float bv = -INFINITY;
-        int bi = nexp;
+        // the lane's greatest value still to be picked (a picked one becomes -inf) and the lowest of its indexes that hold
+        // it, as a tree of maxima and a mask of equalities rather than a chain over the NE values. A NaN is never the
+        // maximum and never equal; a lane with nothing left (-inf) offers index nexp.
+        float bv = v[0];
+#pragma unroll
+        for (int i = 1; i + 1 < NE; i += 2) bv = fmaxf(bv, fmaxf(v[i], v[i + 1]));
+        bv = fmaxf(bv, v[NE - 1]);
+        unsigned eq = 0;
+#pragma unroll
+        for (int i = 0; i < NE; ++i) eq |= (v[i] == bv ? 1u : 0u) << i;
+        const int bi = bv > -INFINITY && eq ? lane + 64 * (int) __builtin_ctz(eq) : nexp;
+        const float m = wave_max(bv);
+        // the lowest index among the lanes that hold the maximum: nearly always one lane, found by a ballot
+        const unsigned long long holders = __ballot(bv == m);
+        int mi;
+        if (__popcll(holders) == 1) mi = __builtin_amdgcn_readlane(bi, (int) __builtin_ctzll(holders));
+        else mi = wave_min(bv == m ? bi : 0x7fffffff);
+        const bool mine = mi < nexp && (mi & 63) == lane;
 #pragma unroll
         for (int i = 0; i < NE; ++i)
-            if (!((taken >> i) & 1u) && v[i] > bv) {   // ascending i: a lane's lower index wins its own ties
-                bv = v[i];
-                bi = lane + 64 * i;
-            }
-        const float m = wave_max(bv);
-        const int mi = wave_min(bv == m ? bi : 0x7fffffff);   // the lowest index among the lanes that hold the maximum
-        if (mi < nexp && (mi & 63) == lane) taken |= 1u << (mi >> 6);
+            if (mine && (mi >> 6) == i) v[i] = -INFINITY;
         if (k == 0) top0 = m;
         const float ek = expf(m - top0);
         z += ek;
