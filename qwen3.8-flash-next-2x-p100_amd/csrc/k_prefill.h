@@ -526,10 +526,12 @@ __global__ void __launch_bounds__(MM_THREADS) k_moe_mma_block(const MmaArgs a) {
         __syncthreads();   // the previous task's last reads of the tile buffers; the table on the first pass
         x_store(x0, 0);
         __syncthreads();
-        auto step = [&](const SubFields (&cur)[MB_RG], int buf, int p) {
+        // nt_tag: the task's token tiles (1 or 2) as a constant: a lone tile's task reads and multiplies half as much
+        auto step = [&](const SubFields (&cur)[MB_RG], int buf, int p, auto nt_tag) {
+            constexpr int NT = decltype(nt_tag)::value;
             v4u B[MM_TP][4];
 #pragma unroll
-            for (int tt = 0; tt < MM_TP; ++tt)
+            for (int tt = 0; tt < NT; ++tt)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) B[tt][i] = *reinterpret_cast<const v4u*>(&L.xt[buf][(tt * 16 + r) * MB_XROW + p * MB_XLD + 64 * g + 16 * i]);
 #pragma unroll
@@ -547,15 +549,13 @@ __global__ void __launch_bounds__(MM_THREADS) k_moe_mma_block(const MmaArgs a) {
                     A[j >> 1][4 * (j & 1) + 3] = hi.y;
                 }
 #pragma unroll
-                for (int tt = 0; tt < MM_TP; ++tt)
-                    if (tt < ntile) {
+                for (int tt = 0; tt < NT; ++tt)
 #pragma unroll
-                        for (int i = 0; i < 4; ++i)
-                            acc[q][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[i], __builtin_bit_cast(v8h, B[tt][i]), acc[q][tt], 0, 0, 0);
-                    }
+                    for (int i = 0; i < 4; ++i)
+                        acc[q][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[i], __builtin_bit_cast(v8h, B[tt][i]), acc[q][tt], 0, 0, 0);
             }
         };
-        auto super = [&](SuperFields (&cur)[MB_RG], SuperFields (&nxt)[MB_RG], int S) {
+        auto super = [&](SuperFields (&cur)[MB_RG], SuperFields (&nxt)[MB_RG], int S, auto nt_tag) {
             const int buf = S & 1, Sn = min(S + 1, nsuper - 1);   // past the end: the last super-step's again
             const XShare xn = x_load(Sn);
 #pragma unroll
@@ -564,23 +564,30 @@ __global__ void __launch_bounds__(MM_THREADS) k_moe_mma_block(const MmaArgs a) {
                 SubFields c[MB_RG];
 #pragma unroll
                 for (int q = 0; q < MB_RG; ++q) c[q] = super_sub<0>(cur[q]);
-                step(c, buf, 0);
+                step(c, buf, 0, nt_tag);
 #pragma unroll
                 for (int q = 0; q < MB_RG; ++q) c[q] = super_sub<1>(cur[q]);
-                step(c, buf, 1);
+                step(c, buf, 1, nt_tag);
 #pragma unroll
                 for (int q = 0; q < MB_RG; ++q) c[q] = super_sub<2>(cur[q]);
-                step(c, buf, 2);
+                step(c, buf, 2, nt_tag);
 #pragma unroll
                 for (int q = 0; q < MB_RG; ++q) c[q] = super_sub<3>(cur[q]);
-                step(c, buf, 3);
+                step(c, buf, 3, nt_tag);
             }
             x_store(xn, buf ^ 1);
             __syncthreads();
         };
-        for (int S = 0; S < nsuper; S += 2) {
-            super(w0, w1, S);
-            if (S + 1 < nsuper) super(w1, w0, S + 1);
+        if (ntile > 1) {
+            for (int S = 0; S < nsuper; S += 2) {
+                super(w0, w1, S, std::integral_constant<int, 2>{});
+                if (S + 1 < nsuper) super(w1, w0, S + 1, std::integral_constant<int, 2>{});
+            }
+        } else {
+            for (int S = 0; S < nsuper; S += 2) {
+                super(w0, w1, S, std::integral_constant<int, 1>{});
+                if (S + 1 < nsuper) super(w1, w0, S + 1, std::integral_constant<int, 1>{});
+            }
         }
         if (rows_live) {
 #pragma unroll
