@@ -460,9 +460,21 @@ __device__ __forceinline__ SubFields super_sub(const SuperFields& f) {
     return s;
 }
 constexpr int MB_XROW = 4 * MB_XLD + 16;   // a token's four step pieces of a super-step (+16: the 16 tokens of a tile fall on different banks)
+constexpr int MB_MAXTASK = 16;
+struct BlockTask {
+    const uint8_t* we;
+    int t0, rb, ntile;   // first token tile, row block, token tiles (1 or 2)
+    int ji, n;           // the job (an index into both lists, the second list after the first) and its tokens
+};
 struct MmaLds {
     uint2 tab[SGRID_WORDS];
     uint8_t xt[2][MB_TOK * MB_XROW];   // [buffer][token][step p][lane group g][64 bytes], step rows padded to 272 bytes
+    // the block's tasks (the valid ones only), their tokens' activation rows (clamped to the job's last) and output rows
+    // (-1 past the job's end): read once when the kernel starts, so that a task begins without a chain of dependent loads
+    int ytok[MB_MAXTASK][MB_TOK];
+    int otok[MB_MAXTASK][MB_TOK];
+    BlockTask task[MB_MAXTASK];
+    int ntask;
 };
 __global__ void __launch_bounds__(MM_THREADS) k_moe_mma_block(const MmaArgs a) {
     typedef __attribute__((address_space(1))) const v4u gx4;
@@ -480,52 +492,79 @@ __global__ void __launch_bounds__(MM_THREADS) k_moe_mma_block(const MmaArgs a) {
     const int nj = min(a.cap, uniform(*a.njobs)), nj2 = a.jobs2 ? min(a.cap2, uniform(*a.njobs2)) : 0;
     const int ks = a.ncols >> 5, nsuper = ks >> 4, rblocks = (a.nrows + MB_ROWS - 1) / MB_ROWS;
     constexpr int HALVES = MM_TT / MM_TP;
-    const int per_job = rblocks * HALVES;
+    const int per_job = rblocks * HALVES, ntasks_all = (nj + nj2) * per_job;
     // this thread's share of a super-step's activation tile (32 tokens x 512 k): token xtok, 64 contiguous bytes
     // (sub-block xsb of the 16); in LDS the sub-block 4 g + p goes to step p, lane group g
     const int xtok = tid >> 4, xsb = tid & 15;
     const int xdst = xtok * MB_XROW + (xsb & 3) * MB_XLD + (xsb >> 2) * 64;
-    for (int task = blockIdx.x; task < (nj + nj2) * per_job; task += gridDim.x) {
-        const int ji = task / per_job, rem = task - ji * per_job, t0 = (rem / rblocks) * MM_TP;
-        // the wave's first row: of its 32 consecutive rows, or (h16) of its 16 gate rows - the up rows lie ffh further
-        const int row0 = a.h16 ? (rem % rblocks) * (MB_ROWS / 2) + wave * 16 : (rem % rblocks) * MB_ROWS + wave * 16 * MB_RG;
-        const int rlimit = a.h16 ? a.ffh : a.nrows, qstep = a.h16 ? a.ffh : 16;
-        const fnx_bigjob* jb = ji < nj ? a.jobs + ji : a.jobs2 + (ji - nj);
-        const int n = min(FNX_PF_JOB, uniform(jb->n)), e = uniform(jb->w), nt = (n + 15) >> 4;
-        if (n < 1 || t0 >= nt) continue;   // the same for every thread of the block
-        const int ntile = min(MM_TP, nt - t0);
-        const bool rows_live = row0 < rlimit;   // per wave
-        const uint8_t* we = ji >= nj ? a.w2 : a.ep ? (const uint8_t*) a.ep[e] : a.w + (size_t) e * a.stride;
-        const uint16_t* xrow = a.x + (size_t) jb->y[min(t0 * 16 + xtok, n - 1)] * a.ldx + 32 * xsb;
-        struct XShare {
-            v4u v[4];
-        };
-        auto x_load = [&](int S) {
+    const int rlimit = a.h16 ? a.ffh : a.nrows, qstep = a.h16 ? a.ffh : 16;
+    struct XShare {
+        v4u v[4];
+    };
+    auto x_store = [&](const XShare& t, int buf) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) *reinterpret_cast<v4u*>(&L.xt[buf][xdst + 16 * i]) = t.v[i];
+    };
+    for (int k0 = blockIdx.x; k0 < ntasks_all; k0 += gridDim.x * MB_MAXTASK) {
+        __syncthreads();   // the previous lists' and tiles' last readers; the table on the first pass
+        if (wave == 0) {
+            const int task = k0 + lane * gridDim.x;
+            bool ok = lane < MB_MAXTASK && task < ntasks_all;
+            BlockTask t{};
+            int ji = 0, n = 0;
+            if (ok) {
+                ji = task / per_job;
+                const int rem = task - ji * per_job;
+                t.t0 = (rem / rblocks) * MM_TP;
+                t.rb = rem % rblocks;
+                const fnx_bigjob* jb = ji < nj ? a.jobs + ji : a.jobs2 + (ji - nj);
+                n = min(FNX_PF_JOB, jb->n);
+                const int e = jb->w;
+                ok = n >= 1 && t.t0 < ((n + 15) >> 4);
+                t.ntile = min(MM_TP, ((n + 15) >> 4) - t.t0);
+                if (ok) t.we = ji >= nj ? a.w2 : a.ep ? (const uint8_t*) a.ep[e] : a.w + (size_t) e * a.stride;
+            }
+            const unsigned long long m = __ballot(ok);
+            const int slot = __popcll(m & ((1ull << lane) - 1ull));
+            if (ok) {
+                t.ji = ji;
+                t.n = n;
+                L.task[slot] = t;
+            }
+            if (lane == 0) L.ntask = __popcll(m);
+        }
+        __syncthreads();
+        const int ntask = L.ntask;
+        if (ntask == 0) continue;   // the same for every thread of the block
+        for (int i = tid; i < ntask * MB_TOK; i += MM_THREADS) {   // the tiles' token and output rows, all at once
+            const int slot = i / MB_TOK, j = i % MB_TOK, ji = L.task[slot].ji, n = L.task[slot].n, tok = L.task[slot].t0 * 16 + j;
+            const fnx_bigjob* jb = ji < nj ? a.jobs + ji : a.jobs2 + (ji - nj);
+            L.ytok[slot][j] = jb->y[min(tok, n - 1)];
+            L.otok[slot][j] = tok < n ? jb->out[tok] : -1;
+        }
+        __syncthreads();
+        const int nst = ntask * nsuper;
+        // the wave's first row in task ti: of its 32 consecutive rows, or (h16) of its 16 gate rows - the up rows lie ffh further
+        auto row0_of = [&](int ti) { return a.h16 ? L.task[ti].rb * (MB_ROWS / 2) + wave * 16 : L.task[ti].rb * MB_ROWS + wave * 16 * MB_RG; };
+        // a stage's loads: this thread's share of the activation tile and its lane's fields of both row groups
+        auto x_load = [&](int ti, int S) {
             XShare t;
-            const gx4* p = (gx4*) (uintptr_t) (xrow + 512 * S);
+            const gx4* p = (gx4*) (uintptr_t) (a.x + (size_t) L.ytok[ti][xtok] * a.ldx + 32 * xsb + 512 * S);
 #pragma unroll
             for (int i = 0; i < 4; ++i) t.v[i] = p[i];
             return t;
         };
-        auto x_store = [&](const XShare& t, int buf) {
+        auto w_load = [&](int ti, int S, SuperFields (&o)[MB_RG]) {
+            const int row0 = row0_of(ti);
+            const uint8_t* we = L.task[ti].we;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) *reinterpret_cast<v4u*>(&L.xt[buf][xdst + 16 * i]) = t.v[i];
+            for (int q = 0; q < MB_RG; ++q) o[q] = super_load(we, min(row0 + qstep * q + r, a.nrows - 1), 16 * S + 4 * g, ks);
         };
         v4f acc[MB_RG][MM_TP];
 #pragma unroll
         for (int q = 0; q < MB_RG; ++q)
 #pragma unroll
             for (int tt = 0; tt < MM_TP; ++tt) acc[q][tt] = v4f{0.f, 0.f, 0.f, 0.f};
-        int rowq[MB_RG];
-#pragma unroll
-        for (int q = 0; q < MB_RG; ++q) rowq[q] = min(row0 + qstep * q + r, a.nrows - 1);
-        const XShare x0 = x_load(0);
-        SuperFields w0[MB_RG], w1[MB_RG];
-#pragma unroll
-        for (int q = 0; q < MB_RG; ++q) w0[q] = super_load(we, rowq[q], 4 * g, ks);
-        __syncthreads();   // the previous task's last reads of the tile buffers; the table on the first pass
-        x_store(x0, 0);
-        __syncthreads();
         // nt_tag: the task's token tiles (1 or 2) as a constant: a lone tile's task reads and multiplies half as much
         auto step = [&](const SubFields (&cur)[MB_RG], int buf, int p, auto nt_tag) {
             constexpr int NT = decltype(nt_tag)::value;
@@ -555,59 +594,82 @@ __global__ void __launch_bounds__(MM_THREADS) k_moe_mma_block(const MmaArgs a) {
                         acc[q][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[i], __builtin_bit_cast(v8h, B[tt][i]), acc[q][tt], 0, 0, 0);
             }
         };
-        auto super = [&](SuperFields (&cur)[MB_RG], SuperFields (&nxt)[MB_RG], int S, auto nt_tag) {
-            const int buf = S & 1, Sn = min(S + 1, nsuper - 1);   // past the end: the last super-step's again
-            const XShare xn = x_load(Sn);
+        auto steps4 = [&](SuperFields (&cur)[MB_RG], int buf, auto nt_tag) {
+            SubFields c[MB_RG];
 #pragma unroll
-            for (int q = 0; q < MB_RG; ++q) nxt[q] = super_load(we, rowq[q], 16 * Sn + 4 * g, ks);
-            if (rows_live) {
-                SubFields c[MB_RG];
+            for (int q = 0; q < MB_RG; ++q) c[q] = super_sub<0>(cur[q]);
+            step(c, buf, 0, nt_tag);
 #pragma unroll
-                for (int q = 0; q < MB_RG; ++q) c[q] = super_sub<0>(cur[q]);
-                step(c, buf, 0, nt_tag);
+            for (int q = 0; q < MB_RG; ++q) c[q] = super_sub<1>(cur[q]);
+            step(c, buf, 1, nt_tag);
 #pragma unroll
-                for (int q = 0; q < MB_RG; ++q) c[q] = super_sub<1>(cur[q]);
-                step(c, buf, 1, nt_tag);
+            for (int q = 0; q < MB_RG; ++q) c[q] = super_sub<2>(cur[q]);
+            step(c, buf, 2, nt_tag);
 #pragma unroll
-                for (int q = 0; q < MB_RG; ++q) c[q] = super_sub<2>(cur[q]);
-                step(c, buf, 2, nt_tag);
-#pragma unroll
-                for (int q = 0; q < MB_RG; ++q) c[q] = super_sub<3>(cur[q]);
-                step(c, buf, 3, nt_tag);
-            }
-            x_store(xn, buf ^ 1);
-            __syncthreads();
+            for (int q = 0; q < MB_RG; ++q) c[q] = super_sub<3>(cur[q]);
+            step(c, buf, 3, nt_tag);
         };
-        if (ntile > 1) {
-            for (int S = 0; S < nsuper; S += 2) {
-                super(w0, w1, S, std::integral_constant<int, 2>{});
-                if (S + 1 < nsuper) super(w1, w0, S + 1, std::integral_constant<int, 2>{});
+        // Stage s = (task ti, super-step S) of the block's sequence: the next stage's loads - the next task's first ones
+        // too - are issued before this stage's arithmetic, its tile goes to the other LDS buffer after it: one barrier a stage
+        int ti = 0, S = 0;
+        auto stage = [&](SuperFields (&cur)[MB_RG], SuperFields (&nxt)[MB_RG], int s) {
+            const int buf = s & 1;
+            int tn = ti, Sn = S + 1;
+            if (Sn == nsuper) {
+                Sn = 0;
+                ++tn;
             }
-        } else {
-            for (int S = 0; S < nsuper; S += 2) {
-                super(w0, w1, S, std::integral_constant<int, 1>{});
-                if (S + 1 < nsuper) super(w1, w0, S + 1, std::integral_constant<int, 1>{});
+            const bool more = s + 1 < nst;
+            XShare xn;
+            if (more) {
+                xn = x_load(tn, Sn);
+                w_load(tn, Sn, nxt);
             }
-        }
-        if (rows_live) {
+            const int row0 = row0_of(ti);
+            if (row0 < rlimit) {   // per wave
+                if (L.task[ti].ntile > 1) steps4(cur, buf, std::integral_constant<int, 2>{});
+                else steps4(cur, buf, std::integral_constant<int, 1>{});
+                if (Sn == 0) {   // the task's last super-step: lane = token r of each tile, weight rows 4 g .. 4 g + 3 of each group
 #pragma unroll
-            for (int tt = 0; tt < MM_TP; ++tt) {
-                const int tok = (t0 + tt) * 16 + r;
-                if (tt < ntile && tok < n) {
-                    if (a.h16) {   // gate rows in acc[0], their up rows in acc[1]
-                        const v4f gt = acc[0][tt], up = acc[1][tt];
-                        uint2 hv;
-                        hv.x = (uint32_t) float_to_half_bits(silu_f(gt.x) * up.x) | (uint32_t) float_to_half_bits(silu_f(gt.y) * up.y) << 16;
-                        hv.y = (uint32_t) float_to_half_bits(silu_f(gt.z) * up.z) | (uint32_t) float_to_half_bits(silu_f(gt.w) * up.w) << 16;
-                        *reinterpret_cast<uint2*>(a.h16 + (size_t) jb->out[tok] * a.ffh + row0 + 4 * g) = hv;
-                    } else {
-                        float* o = a.out + (size_t) jb->out[tok] * a.nrows + row0 + 4 * g;
+                    for (int tt = 0; tt < MM_TP; ++tt) {
+                        const int orow = L.otok[ti][tt * 16 + r];
+                        if (orow >= 0) {
+                            if (a.h16) {   // gate rows in acc[0], their up rows in acc[1]
+                                const v4f gt = acc[0][tt], up = acc[1][tt];
+                                uint2 hv;
+                                hv.x = (uint32_t) float_to_half_bits(silu_f(gt.x) * up.x) | (uint32_t) float_to_half_bits(silu_f(gt.y) * up.y) << 16;
+                                hv.y = (uint32_t) float_to_half_bits(silu_f(gt.z) * up.z) | (uint32_t) float_to_half_bits(silu_f(gt.w) * up.w) << 16;
+                                *reinterpret_cast<uint2*>(a.h16 + (size_t) orow * a.ffh + row0 + 4 * g) = hv;
+                            } else {
+                                float* o = a.out + (size_t) orow * a.nrows + row0 + 4 * g;
 #pragma unroll
-                        for (int q = 0; q < MB_RG; ++q)
-                            if (row0 + 16 * q < a.nrows) *reinterpret_cast<float4*>(o + 16 * q) = make_float4(acc[q][tt].x, acc[q][tt].y, acc[q][tt].z, acc[q][tt].w);
+                                for (int q = 0; q < MB_RG; ++q)
+                                    if (row0 + 16 * q < a.nrows)
+                                        *reinterpret_cast<float4*>(o + 16 * q) = make_float4(acc[q][tt].x, acc[q][tt].y, acc[q][tt].z, acc[q][tt].w);
+                            }
+                        }
                     }
+#pragma unroll
+                    for (int q = 0; q < MB_RG; ++q)
+#pragma unroll
+                        for (int tt = 0; tt < MM_TP; ++tt) acc[q][tt] = v4f{0.f, 0.f, 0.f, 0.f};
                 }
             }
+            if (more) x_store(xn, buf ^ 1);
+            __syncthreads();
+            ti = tn;
+            S = Sn;
+        };
+        SuperFields w0[MB_RG], w1[MB_RG];
+        {
+            const XShare x0 = x_load(0, 0);
+            w_load(0, 0, w0);
+            x_store(x0, 0);
+        }
+        __syncthreads();
+        for (int s = 0; s < nst; s += 2) {
+            stage(w0, w1, s);
+            if (s + 1 < nst) stage(w1, w0, s + 1);
         }
     }
 }
@@ -629,6 +691,7 @@ constexpr int MT_MAXTASK = 16;
 struct TileTask {
     const uint8_t* we;
     int t0, row0, ntile;
+    int ji, n;   // the job (an index into both lists, the second list after the first) and its tokens
 };
 struct TileLds {
     uint2 tab[SGRID_WORDS];
@@ -694,20 +757,22 @@ __global__ void __launch_bounds__(MM_THREADS) __attribute__((amdgpu_waves_per_eu
             const unsigned long long m = __ballot(ok);
             const int slot = __popcll(m & ((1ull << lane) - 1ull));
             if (ok) {
+                t.ji = ji;
+                t.n = n;
                 L.task[slot] = t;
-                // the tile's token and output rows: 32 of each
-                const fnx_bigjob* jb = ji < nj ? a.jobs + ji : a.jobs2 + (ji - nj);
-                for (int j = 0; j < MB_TOK; ++j) {
-                    const int tok = t.t0 * 16 + j;
-                    L.ytok[slot][j] = jb->y[min(tok, n - 1)];
-                    L.otok[slot][j] = tok < n ? jb->out[tok] : -1;
-                }
             }
             if (lane == 0) L.ntask = __popcll(m);
         }
         __syncthreads();
         const int ntask = L.ntask;
         if (ntask == 0) continue;   // the same for every thread of the block
+        for (int i = tid; i < ntask * MB_TOK; i += MM_THREADS) {   // the tiles' token and output rows (32 of each), all at once
+            const int slot = i / MB_TOK, j = i % MB_TOK, ji = L.task[slot].ji, n = L.task[slot].n, tok = L.task[slot].t0 * 16 + j;
+            const fnx_bigjob* jb = ji < nj ? a.jobs + ji : a.jobs2 + (ji - nj);
+            L.ytok[slot][j] = jb->y[min(tok, n - 1)];
+            L.otok[slot][j] = tok < n ? jb->out[tok] : -1;
+        }
+        __syncthreads();
         const int nst = ntask * nsuper;
         auto issue = [&](int ti, int S) {
             const TileTask t = L.task[ti];
