@@ -1,5 +1,7 @@
 #!/usr/bin/env python3
-"""Benchmark of the MoE verify step (BASELINE config 2) on one MI355X.
+"""Benchmark of the MoE verify step on one MI355X. "benchmark config N" below: the N-th entry of BASELINE.json's "configs"
+(1: a lone IQ3_S mat-vec, 2: the MoE verify layer - the headline, 3: argmax + lookup + acceptance, 4: the reduced decoder's
+verify step, 5: the prompt path's MoE layer).
 
 A step = one MoE layer of a verify window: T = 16 rows, hidden 2048, 512 IQ3_S experts (gate|up 2048 -> 2 x 512, down
 512 -> 2048), top-10, one shared expert, f32 router of 513 rows. Inputs are resident in HBM before the timed region.
@@ -42,7 +44,7 @@ def main():
                     help="also run one plain device copy of 256 MiB, the known-size kernel that scales the FETCH_SIZE / WRITE_SIZE counters")
     ap.add_argument("--raw-layout", action="store_true", help="leave the weights as raw ggml blocks (skip the load-time re-laying)")
     ap.add_argument("--workload", choices=["verify", "prefill", "decoder", "head", "gemv"], default="verify",
-                    help="verify: BASELINE config 2 (the headline metric, the default); prefill: config 5, one MoE layer over prompt chunks of 512 "
+                    help="verify: benchmark config 2 (the headline metric, the default); prefill: config 5, one MoE layer over prompt chunks of 512 "
                          "rows; decoder: config 4, a verify step of the reduced decoder plus the draft layer; head: config 3, argmax + prompt "
                          "lookup + acceptance; gemv: config 1, one IQ3_S matrix over T = 1 and 16 rows")
     args = ap.parse_args()
@@ -220,7 +222,7 @@ def _rand_iq3s(torch, g, nblocks):
 
 
 def gemv_main(args):
-    """BASELINE config 1: one 4096 x 2048 IQ3_S matrix (3,604,480 bytes) over T = 1 and T = 16 q8_1 rows, cycling through
+    """benchmark config 1: one 4096 x 2048 IQ3_S matrix (3,604,480 bytes) over T = 1 and T = 16 q8_1 rows, cycling through
     1,024 distinct matrices (3.7 GB) so that every launch reads its weights from HBM."""
     import numpy as np
     import torch
@@ -270,7 +272,7 @@ def gemv_main(args):
 
 
 def head_main(args):
-    """BASELINE config 3: argmax over 16 x 151,936 f32 logits (forced to the draft on 70% of the rows), prompt lookup
+    """benchmark config 3: argmax over 16 x 151,936 f32 logits (forced to the draft on 70% of the rows), prompt lookup
     over a 38,862-token context with 200 copied spans, greedy acceptance; device forms, one stream."""
     import numpy as np
     import torch
@@ -359,7 +361,7 @@ def head_main(args):
 
 
 def decoder_main(args):
-    """BASELINE config 4: a verify step of the reduced decoder (4 layers of GQA attention, 16 q / 2 kv heads of 256, f16
+    """benchmark config 4: a verify step of the reduced decoder (4 layers of GQA attention, 16 q / 2 kv heads of 256, f16
     cache at 32,768 positions, and the config-2 MoE block) over 1 + 15 rows, the output head over 151,936 tokens, greedy
     acceptance, then the draft layer over the same rows. Random weights; a step's weights are cold (two model copies
     alternate is too large for the head, so the ~3.7 GB a step reads already exceeds the 256 MB cache many times)."""
@@ -475,7 +477,7 @@ def decoder_main(args):
 
 
 def prefill_main(args):
-    """BASELINE config 5: one MoE layer over prompt chunks of 512 rows (5,120 routed pairs), expert popularity Zipf(1.1)
+    """benchmark config 5: one MoE layer over prompt chunks of 512 rows (5,120 routed pairs), expert popularity Zipf(1.1)
     imposed through a constant input feature and a bias column of the router. A step = one chunk."""
     import numpy as np
     import torch

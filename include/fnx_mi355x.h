@@ -209,7 +209,7 @@ typedef struct fnx_pf_ws {
 int fnx_moe_prefill_layer(const fnx_moe_layer* L, const float* x, int C, float* out, const fnx_pf_ws* ws, void* st);
 
 /* ---- the rest of a verify step around the MoE half: norms, dense projections, attention, the draft layer
- * (BASELINE config 4: a reduced decoder of attention + MoE layers and the MTP draft layer). Head width 256, the first
+ * (benchmark config 4: a reduced decoder of attention + MoE layers and the MTP draft layer). Head width 256, the first
  * 64 dims rotated (model.hpp:41). */
 /* kernels.hpp:406  rms_norm_rows: y[r] = x[r] / sqrt(mean(x[r]^2) + eps) * w */
 int fnx_rms_norm_rows(const float* x, const float* w, float* y, int rows, int n, float eps, void* st);

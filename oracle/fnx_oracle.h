@@ -131,7 +131,7 @@ void fnx_o_swiglu_h16(const float* gu, int ffs, int P, uint16_t* h);
 void fnx_o_moe_prefill_layer(const fnx_o_moe_layer* L, const float* x, int C, int pf_job, float* out, float* logits, int* topi,
                              float* topw, int* njobs, int threads);
 
-/* ---- around the MoE half (BASELINE config 4): norms, dense Q8_0 projections, attention, the draft layer */
+/* ---- around the MoE half (benchmark config 4): norms, dense Q8_0 projections, attention, the draft layer */
 /* kernels.cu:2818-2826; the mean of squares summed in double */
 void fnx_o_rms_norm_rows(const float* x, const float* w, float* y, int rows, int n, float eps);
 /* ggml's Q8_0 in the reference's split layout (model.hpp:78-82): d = max|x| / 127 as f16, q = round(x / d) */

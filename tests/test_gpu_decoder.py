@@ -1,5 +1,5 @@
 """Parity of the norm / dense / attention operators, the reduced decoder's verify window, the draft layer and whole
-speculative rounds (BASELINE config 4 at test sizes) with the CPU oracle, through the C ABI.
+speculative rounds (benchmark config 4 at test sizes) with the CPU oracle, through the C ABI.
 
 Bar: bit-exact for the dense Q8_0 mat-vec (the summation order is shared with the oracle), for argmax picks, drafts,
 accepted lengths and emitted tokens; relative L2 <= 1e-3 for every operator's float output on identical inputs (norms

@@ -1,4 +1,4 @@
-"""Parity of the MoE verify layer (BASELINE config 2) with the CPU oracle: op by op and as one call."""
+"""Parity of the MoE verify layer (benchmark config 2) with the CPU oracle: op by op and as one call."""
 import ctypes as C
 
 import numpy as np

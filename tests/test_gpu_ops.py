@@ -125,7 +125,7 @@ def test_gemv_iq3s(dev, oracle, nrows, ncols, T, packed):
 
 @pytest.mark.parametrize("packed", [False, True])
 def test_gemv_iq3s_encoded_gaussian_weights(dev, oracle, packed):
-    # BASELINE config 1 in small: N(0, 0.02) weights through the encoder, N(0, 1) activations, against the q8_1 oracle
+    # benchmark config 1 in small: N(0, 0.02) weights through the encoder, N(0, 1) activations, against the q8_1 oracle
     # and within the int8 path's band of the exact f64 product
     rng = np.random.default_rng(410)
     nrows, ncols = 256, 2048
@@ -233,7 +233,7 @@ def test_accept_device_matches_oracle(dev, oracle):
 
 
 def test_config3_drafting_and_acceptance(dev, oracle):
-    # BASELINE config 3: context of 38,862 ids with 200 copied spans, key 3, up to 15 drafts; verify logits 16 x 151,936
+    # benchmark config 3: context of 38,862 ids with 200 copied spans, key 3, up to 15 drafts; verify logits 16 x 151,936
     # with the argmax forced to the draft on 70 % of the rows; outputs are the accepted lengths
     rng = np.random.default_rng(800)
     ctx = make_context(rng)

@@ -1,4 +1,4 @@
-"""A reduced decoder with random weights (BASELINE config 4's shape at test sizes), held as numpy arrays, and its two
+"""A reduced decoder with random weights (benchmark config 4's shape at test sizes), held as numpy arrays, and its two
 renderings: the oracle's C structs (host pointers) and the device library's C structs (device pointers)."""
 import ctypes as C
 
