@@ -144,3 +144,24 @@ def test_prefill_layer_matches_oracle(dev, oracle, n, ff, nexp, topk, Cn):
         assert int(r["njobs"][0]) == want["njobs"] and int(r["njobs"][1]) == (Cn + PF - 1) // PF
         assert np.all(np.isfinite(want["out"]))
         assert rel_l2(r["out"], want["out"]) <= REL_L2
+
+
+def test_prefill_layer_large_chunk_equals_small_chunks(dev):
+    """A size-independent property at a size the oracle does not reach: a row's result does not depend on what else is in
+    its chunk, so 8,192 rows in one call (more tasks than one pass of a block's task list holds, every kernel form's loop
+    over list passes) must equal the same rows in 16 calls of 512, bit for bit."""
+    n, ff, nexp, topk, Cn, small = 2048, 512, 64, 10, 8192, 512
+    print(f"case prefill_layer large n={n} ff={ff} nexp={nexp} topk={topk} C={Cn}", flush=True)
+    rng = np.random.default_rng(777)
+    nb = lambda rows, cols: rows * cols // 256
+    gu = random_iq3s(rng, nexp * nb(2 * ff, n), dmax=1e-3)
+    down = random_iq3s(rng, nexp * nb(n, ff), dmax=1e-3)
+    sh_gu, sh_down = random_iq3s(rng, nb(2 * ff, n), dmax=1e-3), random_iq3s(rng, nb(n, ff), dmax=1e-3)
+    router = (rng.standard_normal((nexp + 1, n)) * 0.05).astype(np.float32)
+    x = rng.standard_normal((Cn, n)).astype(np.float32)
+    big = fnx_gpu.PfLayerDev(dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, Cn, packed=True).run(x)["out"]
+    L = fnx_gpu.PfLayerDev(dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, small, packed=True)
+    assert np.all(np.isfinite(big))
+    for c0 in range(0, Cn, small):
+        part = L.run(x[c0:c0 + small])["out"]
+        assert int(np.count_nonzero(part.view(np.uint32) != big[c0:c0 + small].view(np.uint32))) == 0, f"rows {c0}.."
