@@ -1161,7 +1161,7 @@ static int q8s_launch(const fnx_q8s* const* W, float* const* out, const int* out
     a.cols = W[0]->n_in;
     a.T = T;
     a.yq = (const uint8_t*) yq;
-    const size_t lds = (size_t) FNX_MAXT * (a.cols + Q8S_XPAD) + (size_t) FNX_MAXT * (a.cols / 32 + 2) * 4 + Q8S_WAVES * 64 * 16;
+    const size_t lds = (size_t) FNX_MAXT * (a.cols + Q8S_XPAD) + (size_t) FNX_MAXT * (a.cols / 32 + 2) * 4 + (Q8S_WAVES - 1) * 64 * 16;
     if (lds > 150 * 1024) return fail(std::string(who) + ": the window's activations do not fit LDS");
     static bool attr_set[64] = {};
     int dev = 0;
@@ -1170,7 +1170,7 @@ static int q8s_launch(const fnx_q8s* const* W, float* const* out, const int* out
             return fail(std::string(who) + ": cannot raise the dynamic LDS limit");
         attr_set[dev] = true;
     }
-    static const int per_cu = env_int("FNX_Q8S_BLOCKS_PER_CU", 3, 1, 16);   // what the LDS of a 2048-column matrix lets a CU hold
+    static const int per_cu = env_int("FNX_Q8S_BLOCKS_PER_CU", 4, 1, 16);   // what the LDS of a 2048-column matrix lets a CU hold
     const int grid = (int) std::max(1l, std::min<long>((long) per_cu * cu_count(), tiles));
     k_q8s_gemv<<<grid, Q8S_WAVES * 64, lds, (hipStream_t) st>>>(a);
     return launch_status(who);

@@ -189,7 +189,7 @@ struct Q8sArgs {
 typedef int q8s_v4i __attribute__((ext_vector_type(4)));
 __global__ void __launch_bounds__(Q8S_WAVES * 64) k_q8s_gemv(const Q8sArgs a) {
     typedef __attribute__((address_space(1))) const at_v4u_t g128;
-    extern __shared__ __align__(16) uint8_t q8s_lds[];   // [16][cols + pad] int8, [16][nb + 2] f32 scales, [4][64][4] partial sums
+    extern __shared__ __align__(16) uint8_t q8s_lds[];   // [16][cols + pad] int8, [16][nb + 2] f32 scales, [3][64][4] partial sums
     const int nb = a.cols >> 5, T = a.T, xld = a.cols + Q8S_XPAD, dld = nb + 2;
     int8_t* xs = reinterpret_cast<int8_t*>(q8s_lds);
     float* xd = reinterpret_cast<float*>(q8s_lds + (size_t) FNX_MAXT * xld);
@@ -266,11 +266,11 @@ __global__ void __launch_bounds__(Q8S_WAVES * 64) k_q8s_gemv(const Q8sArgs a) {
     };
     auto finish = [&](const Tile& c) {   // the four quarters through LDS: (s0 + s1) + (s2 + s3)
         __syncthreads();   // the previous tile's sums have been read
-        *reinterpret_cast<float4*>(part + (wave * 64 + lane) * 4) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+        if (wave) *reinterpret_cast<float4*>(part + ((wave - 1) * 64 + lane) * 4) = make_float4(acc[0], acc[1], acc[2], acc[3]);
         __syncthreads();
-        if (wave == 0 && r16 < T) {
-            const float4 p0 = *reinterpret_cast<const float4*>(part + lane * 4), p1 = *reinterpret_cast<const float4*>(part + (64 + lane) * 4),
-                         p2 = *reinterpret_cast<const float4*>(part + (128 + lane) * 4), p3 = *reinterpret_cast<const float4*>(part + (192 + lane) * 4);
+        if (wave == 0 && r16 < T) {   // the first quarter's sums never leave its wave (and the block fits a CU four times)
+            const float4 p0 = make_float4(acc[0], acc[1], acc[2], acc[3]), p1 = *reinterpret_cast<const float4*>(part + lane * 4),
+                         p2 = *reinterpret_cast<const float4*>(part + (64 + lane) * 4), p3 = *reinterpret_cast<const float4*>(part + (128 + lane) * 4);
             const float v[4] = {(p0.x + p1.x) + (p2.x + p3.x), (p0.y + p1.y) + (p2.y + p3.y), (p0.z + p1.z) + (p2.z + p3.z),
                                 (p0.w + p1.w) + (p2.w + p3.w)};
 #pragma unroll
