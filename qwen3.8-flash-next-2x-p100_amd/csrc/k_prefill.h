@@ -554,11 +554,12 @@ __global__ void __launch_bounds__(MM_THREADS) k_moe_mma_block(const MmaArgs a) {
             for (int i = 0; i < 4; ++i) t.v[i] = p[i];
             return t;
         };
+        auto w_load_q = [&](int ti, int S, int q, SuperFields& o) {
+            o = super_load(L.task[ti].we, min(row0_of(ti) + qstep * q + r, a.nrows - 1), 16 * S + 4 * g, ks);
+        };
         auto w_load = [&](int ti, int S, SuperFields (&o)[MB_RG]) {
-            const int row0 = row0_of(ti);
-            const uint8_t* we = L.task[ti].we;
 #pragma unroll
-            for (int q = 0; q < MB_RG; ++q) o[q] = super_load(we, min(row0 + qstep * q + r, a.nrows - 1), 16 * S + 4 * g, ks);
+            for (int q = 0; q < MB_RG; ++q) w_load_q(ti, S, q, o[q]);
         };
         v4f acc[MB_RG][MM_TP];
 #pragma unroll
@@ -594,14 +595,19 @@ __global__ void __launch_bounds__(MM_THREADS) k_moe_mma_block(const MmaArgs a) {
                         acc[q][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[i], __builtin_bit_cast(v8h, B[tt][i]), acc[q][tt], 0, 0, 0);
             }
         };
-        auto steps4 = [&](SuperFields (&cur)[MB_RG], int buf, auto nt_tag) {
+        // pre(p): what the caller wants issued before step p (the next stage's loads, a part before each of the first steps,
+        // so that the waves' loads do not queue up behind one another at the stage's start)
+        auto steps4 = [&](SuperFields (&cur)[MB_RG], int buf, auto nt_tag, auto pre) {
             SubFields c[MB_RG];
+            pre(0);
 #pragma unroll
             for (int q = 0; q < MB_RG; ++q) c[q] = super_sub<0>(cur[q]);
             step(c, buf, 0, nt_tag);
+            pre(1);
 #pragma unroll
             for (int q = 0; q < MB_RG; ++q) c[q] = super_sub<1>(cur[q]);
             step(c, buf, 1, nt_tag);
+            pre(2);
 #pragma unroll
             for (int q = 0; q < MB_RG; ++q) c[q] = super_sub<2>(cur[q]);
             step(c, buf, 2, nt_tag);
@@ -621,14 +627,15 @@ __global__ void __launch_bounds__(MM_THREADS) k_moe_mma_block(const MmaArgs a) {
             }
             const bool more = s + 1 < nst;
             XShare xn;
-            if (more) {
-                xn = x_load(tn, Sn);
-                w_load(tn, Sn, nxt);
-            }
+            auto pre = [&](int p) {   // the weights (from HBM) first, the activations (cached) last
+                if (!more) return;
+                if (p < MB_RG) w_load_q(tn, Sn, p, nxt[p]);
+                else if (p == MB_RG) xn = x_load(tn, Sn);
+            };
             const int row0 = row0_of(ti);
             if (row0 < rlimit) {   // per wave
-                if (L.task[ti].ntile > 1) steps4(cur, buf, std::integral_constant<int, 2>{});
-                else steps4(cur, buf, std::integral_constant<int, 1>{});
+                if (L.task[ti].ntile > 1) steps4(cur, buf, std::integral_constant<int, 2>{}, pre);
+                else steps4(cur, buf, std::integral_constant<int, 1>{}, pre);
                 if (Sn == 0) {   // the task's last super-step: lane = token r of each tile, weight rows 4 g .. 4 g + 3 of each group
 #pragma unroll
                     for (int tt = 0; tt < MM_TP; ++tt) {
@@ -654,6 +661,9 @@ __global__ void __launch_bounds__(MM_THREADS) k_moe_mma_block(const MmaArgs a) {
 #pragma unroll
                         for (int tt = 0; tt < MM_TP; ++tt) acc[q][tt] = v4f{0.f, 0.f, 0.f, 0.f};
                 }
+            } else {
+#pragma unroll
+                for (int p = 0; p <= MB_RG; ++p) pre(p);
             }
             if (more) x_store(xn, buf ^ 1);
             __syncthreads();
