@@ -457,6 +457,45 @@ def decoder_main(args):
     torch.cuda.synchronize()
     attn_ms = float(np.mean([a.elapsed_time(c) for a, c in evs[3:]]))
     head_ms = float(np.mean([a.elapsed_time(c) for a, c in hv[3:]]))
+    # whole decode rounds that the host only enqueues (fnx_decode_round: verify, acceptance, commit, draft layer, prompt
+    # lookup and the next window, the state in device words): eagerly, and as replays of one captured round. With random
+    # weights no draft is ever right: a window is the last token and one draft, and a round keeps one token.
+    NR, P0 = 24, CTX - 4096
+    rctx = torch.randint(0, V, (CTX + 64,), dtype=torch.int32, device="cuda", generator=g)
+    rstate, rrows, rscratch = z(pkg.RS_WORDS, t.int32), z(16, t.int32), z(16, t.int32)
+    RD = pkg.Round(rstate.data_ptr(), rrows.data_ptr(), rctx.data_ptr(), CTX + 64, None, 0, 1, 3, 15, rscratch.data_ptr())
+
+    def reset_rounds():
+        rstate.zero_()
+        rstate[pkg.RS_NCTX], rstate[pkg.RS_POS], rstate[pkg.RS_ROWS] = P0 + 1, P0, 1
+        rrows.zero_()
+        rrows[0] = rctx[P0]
+
+    def a_round():
+        dev.ok(lib.fnx_decode_round(C.byref(D), C.byref(M), C.byref(RD), C.byref(ws), dev.st()))
+
+    def timed_rounds(run):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(NR):
+            run()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / NR * 1e3
+
+    reset_rounds()
+    for _ in range(3):
+        a_round()
+    round_eager_ms = timed_rounds(a_round)
+    kept_eager = int(rstate[pkg.RS_NCTX].item()) - (P0 + 1)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        a_round()
+    reset_rounds()
+    for _ in range(3):
+        graph.replay()
+    round_graph_ms = timed_rounds(graph.replay)
+    kept_graph = int(rstate[pkg.RS_NCTX].item()) - (P0 + 1)
+    assert int(rstate[pkg.RS_STOP].item()) == 0 and int(rstate[pkg.RS_ROUNDS].item()) == NR + 3 and kept_graph == kept_eager, "rounds went wrong"
     kv_bytes = 2 * CTX * NKV * HD * 2
     head_bytes = V * N + V * (N // 32) * 2
     dense_bytes = (NQ * 2 * HD * N + 2 * NKV * HD * N + N * NQ * HD) * 34 // 32
@@ -468,7 +507,10 @@ def decoder_main(args):
             "config": {"workload": "config 4: 4 layers (GQA 16q/2kv x 256 at 32,768 positions + MoE as config 2) + head 151,936 + acceptance + draft layer, 16 rows",
                        "step_algorithmic_bytes": step_bytes, "step_hbm_frac": step_bytes / (dt / steps) / HBM_PEAK,
                        "attention_ms_per_layer": attn_ms, "attention_GBps": kv_bytes / (attn_ms * 1e-3) / 1e9, "head_ms": head_ms,
-                       "head_GBps": head_bytes / (head_ms * 1e-3) / 1e9},
+                       "head_GBps": head_bytes / (head_ms * 1e-3) / 1e9,
+                       "decode_round": {"what": "verify 16 rows (2 count) + accept + commit + draft layer + lookup + next window at position 28,672, no host wait",
+                                        "rounds": NR, "ms_eager": round_eager_ms, "ms_graph_replay": round_graph_ms,
+                                        "tokens_kept_per_round": kept_graph / (NR + 3)}},
             "roofline": {"bound": "hbm", "kernel": "k_q8s_gemv (output head 151,936 x 2048)", "achieved": head_bytes / (head_ms * 1e-3) / 1e9,
                          "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": head_bytes / (head_ms * 1e-3) / HBM_PEAK, "traffic": None, "kernel_ms": head_ms,
                          "algorithmic_bytes": head_bytes},

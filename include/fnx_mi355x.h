@@ -297,6 +297,39 @@ typedef struct fnx_mtp {
 } fnx_mtp;
 int fnx_mtp_draft(const fnx_decoder* D, const fnx_mtp* M, const float* src, const int* tokens, int T, const int* pos0, const fnx_dec_ws* ws,
                   void* st);
+
+/* ---- a greedy decode round that the host only enqueues. session.cpp:530-679 (Session::generate) drives these steps
+ * from the host and waits for each; the reference's captured windows (engine_common.cu:993-1021) still hand the picks to
+ * the host for acceptance. Here the acceptance (session.cpp:565-573), the commit, the draft layer's pass over the rows
+ * kept (engine.cu:2095-2133) and the prompt lookup (session.cpp:428-447) read and leave their results in device words,
+ * so no argument of a round changes from one round to the next: rounds can be enqueued back to back, or captured once in
+ * a graph and replayed. The MTP chain is one draft long (the draft layer's pick for the last row kept) when the lookup
+ * finds nothing. */
+enum {
+    FNX_RS_NCTX = 0,     /* tokens in ctx: the prompt and everything emitted */
+    FNX_RS_POS = 1,      /* cache position of the window's first row (= FNX_RS_NCTX - 1) */
+    FNX_RS_ROWS = 2,     /* rows of the window that count: 1 + the drafts */
+    FNX_RS_ACCEPTED = 3, /* tokens the last round kept */
+    FNX_RS_POS_PREV = 4, /* the last window's position */
+    FNX_RS_ROUNDS = 5,   /* rounds done */
+    FNX_RS_STOP = 6,     /* set once the next window would not fit the caches or ctx: later rounds change nothing */
+    FNX_RS_WORDS = 8
+};
+typedef struct fnx_round {
+    int* state;    /* device, FNX_RS_WORDS ints (the caller sets NCTX, POS, ROWS and zeroes the others) */
+    int* rows;     /* device, FNX_MAXT ints: the window: the context's last token, then the drafts, then zeros */
+    int* ctx;      /* device, ctx_cap ints: the prompt, then every token emitted */
+    int ctx_cap;
+    int* log;      /* device, log_cap x 2 ints (drafts offered, tokens kept) a round, or null */
+    int log_cap;
+    int speculate; /* 0: plain greedy decoding, one row a round (no draft layer, no lookup) */
+    int key_n, lk; /* prompt lookup: tokens in the key (3 in the reference), most drafts (<= FNX_MAXT - 1) */
+    int* scratch;  /* device, FNX_MAXT ints */
+} fnx_round;
+/* one round: fnx_decoder_verify over the window -> acceptance and commit -> fnx_mtp_draft over the rows kept -> lookup
+ * -> the next window. Expert weights must be in the unit64 layout and hidden = 2048 (the five-launch window), since only
+ * that routes a row count held on the device. The draft layer uses the same workspace after the verify. */
+int fnx_decode_round(const fnx_decoder* D, const fnx_mtp* M, const fnx_round* R, const fnx_dec_ws* ws, void* st);
 #ifdef __cplusplus
 }
 #endif

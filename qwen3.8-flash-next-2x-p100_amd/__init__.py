@@ -75,6 +75,13 @@ class Mtp(C.Structure):
                 ("layer", DecLayer)]
 
 
+class Round(C.Structure):
+    _fields_ = [("state", C.c_void_p), ("rows", C.c_void_p), ("ctx", C.c_void_p), ("ctx_cap", C.c_int), ("log", C.c_void_p), ("log_cap", C.c_int),
+                ("speculate", C.c_int), ("key_n", C.c_int), ("lk", C.c_int), ("scratch", C.c_void_p)]
+
+
+RS_NCTX, RS_POS, RS_ROWS, RS_ACCEPTED, RS_POS_PREV, RS_ROUNDS, RS_STOP, RS_WORDS = 0, 1, 2, 3, 4, 5, 6, 8
+
 EXPORTS = {
     # name: (restype, argtypes)
     "fnx_last_error": (C.c_char_p, []),
@@ -124,6 +131,7 @@ EXPORTS = {
                            C.c_void_p]),
     "fnx_decoder_verify": (C.c_int, [C.POINTER(Decoder), C.c_void_p, C.c_int, C.c_void_p, C.POINTER(DecWs), C.c_void_p]),
     "fnx_mtp_draft": (C.c_int, [C.POINTER(Decoder), C.POINTER(Mtp), C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.POINTER(DecWs), C.c_void_p]),
+    "fnx_decode_round": (C.c_int, [C.POINTER(Decoder), C.POINTER(Mtp), C.POINTER(Round), C.POINTER(DecWs), C.c_void_p]),
     "fnx_moe_prefill_layer": (C.c_int, [C.POINTER(MoeLayer), C.c_void_p, C.c_int, C.c_void_p, C.POINTER(PfWs), C.c_void_p]),
 }
 

@@ -432,6 +432,7 @@ __global__ void __launch_bounds__(512) k_iq3s_jobs(const RowsArgs a) {
 #include "k_moe_layer.h"
 #include "k_prefill.h"
 #include "k_decoder.h"
+#include "k_round.h"
 namespace fnx {
 
 // any other row length (a multiple of 256): a wave per (row, job), sub-blocks dealt round-robin to the lanes, the
@@ -583,11 +584,15 @@ __global__ void k_argmax_fin(unsigned long long* keys, int T, int v0, float* bv,
 // a step - the 4 + 3 tokens they need are two 16-byte loads - and LK_STEPS steps a round), and the match and the copy are
 // a ballot each.
 constexpr int LK_THREADS = 1024, LK_STEPS = 10, LOOKUP_MIN = 3, IMAGE_TOK = 1 << 30;   // 40,960 start positions a round
+// n_ctx_p (may be null): the context's length is that device word instead of n_ctx; d1_at (may be null): d1 is
+// d1p[*d1_at - 1] instead of d1p[0] (the pick of the last row kept).
 __global__ void __launch_bounds__(LK_THREADS) k_lookup(const int* __restrict__ ctx, int n_ctx, int key_n, int lk, const int* __restrict__ d1p,
-                                                      int* __restrict__ out, int* __restrict__ n_out, int* __restrict__ match) {
+                                                      int* __restrict__ out, int* __restrict__ n_out, int* __restrict__ match,
+                                                      const int* __restrict__ n_ctx_p, const int* __restrict__ d1_at) {
     __shared__ int best;
     if (threadIdx.x == 0) best = -1;
-    const int d1 = *d1p;   // asked for now, used at the end
+    if (n_ctx_p) n_ctx = *n_ctx_p;
+    const int d1 = d1p[d1_at ? min(max(*d1_at, 1), FNX_MAXT) - 1 : 0];   // asked for now, used at the end
     __syncthreads();
     const int n0 = n_ctx - key_n;
     if (lk > 0 && n0 > 0) {
@@ -732,14 +737,15 @@ static void prof_mark(int i, hipStream_t s) {
     if (g_prof_on) (void) hipEventRecord(g_prof_ev[i], s);
 }
 // the window's MoE half in five launches (k_moe_layer.h)
-static int layer_fused(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st) {
+// live (may be null): a device word, the rows of the window that are routed (k_route_plan); the caller's combine skips the others
+static int layer_fused(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st, const int* live = nullptr) {
     hipStream_t s = (hipStream_t) st;
     const int n = L->n, ff = L->ff, P = T * L->topk, LS = L->nexp + 1;
     const int rblocks = (LS + RQ_ROWS - 1) / RQ_ROWS, qblocks = (T * 64 + 2 * FL_WAVES - 1) / (2 * FL_WAVES);
     prof_mark(0, s);
     k_router_quant<<<rblocks + qblocks, FL_THREADS, 0, s>>>(RouterArgs{L->nexp, T, x, L->router, L->router_bf16, ws->logits, (uint8_t*) ws->xq});
     prof_mark(1, s);
-    k_route_plan<<<T, RT_THREADS, 0, s>>>(RouteArgs{L->nexp, L->topk, T, ws->logits, ws->topi, ws->topw, ws->jobs_gu, ws->jobs_dn, ws->njobs});
+    k_route_plan<<<T, RT_THREADS, 0, s>>>(RouteArgs{L->nexp, L->topk, T, ws->logits, ws->topi, ws->topw, ws->jobs_gu, ws->jobs_dn, ws->njobs, live});
     prof_mark(2, s);
     static const int per_cu = env_int("FNX_LAYER_BLOCKS_PER_CU", 2, 1, 8);
     const int grid = per_cu * cu_count();
@@ -911,7 +917,7 @@ int fnx_lookup_drafts(const int* ctx, int n_ctx, int key_n, int lk, int d1, int*
 int fnx_lookup_drafts_dev(const int* ctx, int n_ctx, int key_n, int lk, const int* d1, int* out, int* n_out, int* match, void* st) {
     if (!ctx || !d1 || !out || !n_out) return fail("lookup_drafts_dev: null argument");
     if (n_ctx < 0 || lk < 0 || lk > 64 || key_n < 1 || key_n > 4) return fail("lookup_drafts_dev: bad argument (keys of 1..4 tokens, up to 64 drafts)");
-    k_lookup<<<1, LK_THREADS, 0, (hipStream_t) st>>>(ctx, n_ctx, key_n, lk, d1, out, n_out, match);
+    k_lookup<<<1, LK_THREADS, 0, (hipStream_t) st>>>(ctx, n_ctx, key_n, lk, d1, out, n_out, match, nullptr, nullptr);
     return launch_status("lookup_drafts_dev");
 }
 
@@ -948,7 +954,7 @@ int fnx_layer_profile_read(float* ms5) {
 }
 
 // out null: the fused window without its combine (layer_fused_ok must hold)
-static int moe_layer_checked(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st) {
+static int moe_layer_checked(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st, const int* live = nullptr) {
     if (!L || !x || !ws) return fail("moe_verify_layer: null argument");
     if (!ws->xq || !ws->logits || !ws->topi || !ws->topw || !ws->jobs_gu || !ws->jobs_dn || !ws->njobs || !ws->gu || !ws->part)
         return fail("moe_verify_layer: incomplete workspace");
@@ -958,7 +964,8 @@ static int moe_layer_checked(const fnx_moe_layer* L, const float* x, int T, floa
     if (L->gu.n_in != n || L->gu.n_out != 2 * ff || L->down.n_in != ff || L->down.n_out != n || L->sh_gu.n_in != n ||
         L->sh_gu.n_out != 2 * ff || L->sh_down.n_in != ff || L->sh_down.n_out != n)
         return fail("moe_verify_layer: weight shapes do not match n / ff");
-    if (layer_fused_ok(L, T)) return layer_fused(L, x, T, out, ws, st);
+    if (live && (out || !layer_fused_ok(L, T))) return fail("moe_verify_layer: a device-side row count needs the fused window without its combine");
+    if (layer_fused_ok(L, T)) return layer_fused(L, x, T, out, ws, st, live);
     if (!out) return fail("moe_verify_layer: null argument");
     hipStream_t s = (hipStream_t) st;
     if (fnx_quantize_q8_1(x, ws->xq, n, T, st)) return 1;
@@ -1234,6 +1241,7 @@ struct DecPending {
     const float* rows;
     const fnx_moe_layer* moe;
     const int* tokens;   // not null: x itself is still to come - the embedding rows of these tokens (nothing else pending then)
+    const int* live;     // with moe: the device word that said how many rows were routed, or null
 };
 // xcopy (may be null): the rows after the add go there too
 static int dec_add_norm_q8(const fnx_decoder* D, const DecPending& pend, const float* w, int T, const fnx_dec_ws* ws, void* st, float* xcopy = nullptr) {
@@ -1241,7 +1249,7 @@ static int dec_add_norm_q8(const fnx_decoder* D, const DecPending& pend, const f
     if (pend.moe) {
         const fnx_moe_layer* M = pend.moe;
         c = CombineArgs{ws->moe.part, ws->moe.topw, ws->moe.part + (size_t) T * M->topk * D->n, ws->moe.logits + M->nexp, M->nexp + 1, M->topk, nullptr,
-                        nullptr, nullptr, 0};
+                        nullptr, nullptr, 0, pend.live};
     }
     c.xcopy = xcopy;
     if (pend.tokens) {
@@ -1255,7 +1263,10 @@ static int dec_add_norm_q8(const fnx_decoder* D, const DecPending& pend, const f
     return launch_status("decoder add_norm_q8");
 }
 // x (ws->x) through one layer, in place; the layer's own MoE output is left pending for whatever comes next
-static int dec_layer(const fnx_decoder* D, const fnx_dec_layer* L, int T, const int* pos0, const fnx_dec_ws* ws, DecPending& pend, void* st) {
+// live (may be null): a device word, how many of the T rows count; the others still pass through the attention (their
+// cache cells are overwritten by the next window) but are not routed, so they pull no expert's weights
+static int dec_layer(const fnx_decoder* D, const fnx_dec_layer* L, int T, const int* pos0, const fnx_dec_ws* ws, DecPending& pend, void* st,
+                     const int* live = nullptr) {
     const int n = D->n, nq = D->nq, nkv = D->nkv;
     if (dec_add_norm_q8(D, pend, L->attn_norm, T, ws, st)) return 1;
     {   // q, k and v in one launch (engine.cu:1547-1552)
@@ -1270,10 +1281,11 @@ static int dec_layer(const fnx_decoder* D, const fnx_dec_layer* L, int T, const 
     if (fnx_q8s_gemv(&L->wo, ws->xq, ws->o, n, T, st)) return 1;
     if (fnx_add_norm_q8(ws->x, ws->o, L->ffn_norm, ws->xn, nullptr, T, n, D->eps, st)) return 1;
     if (layer_fused_ok(&L->moe, T)) {   // the window without its combine
-        pend = DecPending{nullptr, &L->moe, nullptr};
-        return moe_layer_checked(&L->moe, ws->xn, T, nullptr, &ws->moe, st);
+        pend = DecPending{nullptr, &L->moe, nullptr, live};
+        return moe_layer_checked(&L->moe, ws->xn, T, nullptr, &ws->moe, st, live);
     }
-    pend = DecPending{ws->o, nullptr, nullptr};
+    if (live) return fail("decoder: a device-side row count needs the fused window (unit64 experts, hidden 2048)");
+    pend = DecPending{ws->o, nullptr, nullptr, nullptr};
     return fnx_moe_verify_layer(&L->moe, ws->xn, T, ws->o, &ws->moe, st);
 }
 static int dec_shape_check(const fnx_decoder* D, int T, const char* who) {
@@ -1289,16 +1301,19 @@ static int dec_head(const fnx_decoder* D, const float* norm, const fnx_q8s* head
     if (fnx_q8s_gemv(head, ws->xq, ws->logits, D->vocab, T, st)) return 1;
     return fnx_argmax(ws->logits, D->vocab, T, 0, ws->best_v, ws->best_i, ws->keys, ws->err, st);
 }
-int fnx_decoder_verify(const fnx_decoder* D, const int* tokens, int T, const int* pos0, const fnx_dec_ws* ws, void* st) {
+static int decoder_verify(const fnx_decoder* D, const int* tokens, int T, const int* pos0, const fnx_dec_ws* ws, void* st, const int* live) {
     if (!D || !tokens || !pos0 || !ws || !D->layers || !D->out_norm || !D->emb) return fail("decoder_verify: null argument");
     if (dec_shape_check(D, T, "decoder_verify") || dec_ws_check(ws, "decoder_verify")) return 1;
-    DecPending pend{nullptr, nullptr, tokens};   // the window's input rows are read by the first pass over them
+    DecPending pend{nullptr, nullptr, tokens, nullptr};   // the window's input rows are read by the first pass over them
     for (int l = 0; l < D->nlayers; ++l)
-        if (dec_layer(D, &D->layers[l], T, pos0, ws, pend, st)) return 1;
+        if (dec_layer(D, &D->layers[l], T, pos0, ws, pend, st, live)) return 1;
     return dec_head(D, D->out_norm, &D->head, T, ws, pend, st);
 }
-int fnx_mtp_draft(const fnx_decoder* D, const fnx_mtp* M, const float* src, const int* tokens, int T, const int* pos0, const fnx_dec_ws* ws,
-                  void* st) {
+int fnx_decoder_verify(const fnx_decoder* D, const int* tokens, int T, const int* pos0, const fnx_dec_ws* ws, void* st) {
+    return decoder_verify(D, tokens, T, pos0, ws, st, nullptr);
+}
+static int mtp_draft(const fnx_decoder* D, const fnx_mtp* M, const float* src, const int* tokens, int T, const int* pos0, const fnx_dec_ws* ws,
+                     void* st, const int* live) {
     if (!D || !M || !src || !tokens || !pos0 || !ws || !M->norm_emb || !M->norm_hid || !M->out_norm || !D->emb) return fail("mtp_draft: null argument");
     if (dec_shape_check(D, T, "mtp_draft") || dec_ws_check(ws, "mtp_draft")) return 1;
     const int n = D->n;
@@ -1308,9 +1323,32 @@ int fnx_mtp_draft(const fnx_decoder* D, const fnx_mtp* M, const float* src, cons
     if (fnx_embed_rows(D->emb, tokens, T, D->vocab, n, ws->xn, st)) return 1;
     if (fnx_add_norm_q8(ws->xn, nullptr, M->norm_emb, nullptr, ws->xq, T, n, D->eps, st)) return 1;
     if (fnx_q8s_gemv(&M->fc_emb, ws->xq, ws->o, n, T, st)) return 1;
-    DecPending pend{ws->o, nullptr, nullptr};
-    if (dec_layer(D, &M->layer, T, pos0, ws, pend, st)) return 1;
+    DecPending pend{ws->o, nullptr, nullptr, nullptr};
+    if (dec_layer(D, &M->layer, T, pos0, ws, pend, st, live)) return 1;
     return dec_head(D, M->out_norm, &M->head, T, ws, pend, st);
+}
+int fnx_mtp_draft(const fnx_decoder* D, const fnx_mtp* M, const float* src, const int* tokens, int T, const int* pos0, const fnx_dec_ws* ws,
+                  void* st) {
+    return mtp_draft(D, M, src, tokens, T, pos0, ws, st, nullptr);
+}
+int fnx_decode_round(const fnx_decoder* D, const fnx_mtp* M, const fnx_round* R, const fnx_dec_ws* ws, void* st) {
+    if (!D || !R || !ws || !R->state || !R->rows || !R->ctx || !R->scratch) return fail("decode_round: null argument");
+    if (R->speculate && !M) return fail("decode_round: speculation needs the draft layer");
+    if (R->ctx_cap < 2 * FNX_MAXT || R->log_cap < 0 || (R->log_cap > 0 && !R->log)) return fail("decode_round: bad buffer sizes");
+    if (R->speculate && (R->key_n < 1 || R->key_n > 4 || R->lk < 0 || R->lk > FNX_MAXT - 1))
+        return fail("decode_round: keys of 1..4 tokens, up to 15 drafts");
+    hipStream_t s = (hipStream_t) st;
+    int* S = R->state;
+    if (decoder_verify(D, R->rows, FNX_MAXT, S + FNX_RS_POS, ws, st, S + FNX_RS_ROWS)) return 1;
+    k_round_commit<<<1, 64, 0, s>>>(R->rows, ws->best_i, S, R->ctx, R->ctx_cap, D->max_ctx, R->log_cap ? R->log : nullptr, R->log_cap);
+    if (R->speculate) {
+        // the rows kept and their picks are where the verify left them; the draft layer overwrites both only at its end
+        if (mtp_draft(D, M, ws->hidden, ws->best_i, FNX_MAXT, S + FNX_RS_POS_PREV, ws, st, S + FNX_RS_ACCEPTED)) return 1;
+        k_lookup<<<1, LK_THREADS, 0, s>>>(R->ctx, 0, R->key_n, R->lk, ws->best_i, R->scratch + 1, R->scratch, nullptr, S + FNX_RS_NCTX,
+                                          S + FNX_RS_ACCEPTED);
+    }
+    k_round_window<<<1, 64, 0, s>>>(R->ctx, S, R->scratch + 1, R->scratch, ws->best_i, R->speculate, R->rows);
+    return launch_status("decode_round");
 }
 
 }  // extern "C"

@@ -39,6 +39,7 @@ struct CombineArgs {
     const uint16_t* emb;  // may be null: the rows do not come from x but are rows tokens[r] of this f16 table (and go to x)
     const int* tokens;
     int vocab;
+    const int* live;      // may be null; else a device word: rows from *live on were not routed and get no combine added
 };
 // WIDE (the combine's form): 1024 threads make the row after the add - a thread the columns p, p + 1024, ..., with all
 // of an expert batch's partial sums in flight (256 threads with 8 columns each took 13 us a call, against 7 us without
@@ -59,11 +60,13 @@ __global__ void __launch_bounds__(WIDE ? 1024 : 256) k_add_norm_q8(float* __rest
         float m[NQ_WJ];
 #pragma unroll
         for (int j = 0; j < NQ_WJ; ++j) m[j] = 0.f;
-        for (int k0 = 0; k0 < c.topk; k0 += NQ_KB) {
+        const bool routed = !c.live || (int) row < *c.live;
+        const int topk = routed ? c.topk : 0;
+        for (int k0 = 0; k0 < topk; k0 += NQ_KB) {
             float pv[NQ_KB][NQ_WJ], wk[NQ_KB];
 #pragma unroll
             for (int kk = 0; kk < NQ_KB; ++kk) {
-                const int k = min(k0 + kk, c.topk - 1);
+                const int k = min(k0 + kk, topk - 1);
                 wk[kk] = c.topw[row * c.topk + k];
 #pragma unroll
                 for (int j = 0; j < NQ_WJ; ++j) {
@@ -74,7 +77,7 @@ __global__ void __launch_bounds__(WIDE ? 1024 : 256) k_add_norm_q8(float* __rest
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int kk = 0; kk < NQ_KB; ++kk)
-                if (k0 + kk < c.topk) {
+                if (k0 + kk < topk) {
 #pragma unroll
                     for (int j = 0; j < NQ_WJ; ++j) m[j] = fmaf(wk[kk], pv[kk][j], m[j]);
                 }
@@ -90,7 +93,7 @@ __global__ void __launch_bounds__(WIDE ? 1024 : 256) k_add_norm_q8(float* __rest
 #pragma unroll
         for (int j = 0; j < NQ_WJ; ++j) {
             const int i = threadIdx.x + 1024 * j;
-            const float r = xv[j] + (m[j] + sg * shv[j]);
+            const float r = routed ? xv[j] + (m[j] + sg * shv[j]) : xv[j];
             vrow[i] = i < n ? r : 0.f;
             if (i < n) {
                 x[row * n + i] = r;

@@ -119,6 +119,8 @@ struct RouteArgs {
     fnx_job* jobs_gu;
     fnx_job* jobs_dn;
     int* njobs;   // [0] the job count, [1] the block counter (left at zero)
+    const int* live;   // may be null; else a device word: only the window's first *live rows are routed (the others get no
+                       // pairs, and the shared expert's job stops before them), while the lists keep the indexes T gives them
 };
 constexpr int RT_THREADS = 256;
 struct RouteLds {
@@ -135,7 +137,8 @@ __global__ void __launch_bounds__(RT_THREADS) k_route_plan(const RouteArgs a) {
     __shared__ RouteLds L;
     const int tid = threadIdx.x, wave = uniform(tid >> 6), lane = tid & 63;
     const int T = a.T, topk = a.topk, P = T * topk, LS = a.nexp + 1, t = blockIdx.x;
-    if (wave == 0) {
+    const int Tl = a.live ? uniform(max(0, min(*a.live, T))) : T, Pl = Tl * topk;
+    if (wave == 0 && t < Tl) {
         if (a.nexp <= 512) wave_topk<8>(a.logits + (size_t) t * LS, a.nexp, topk, lane, L.ex, a.topi + t * topk, a.topw + t * topk);
         else wave_topk<16>(a.logits + (size_t) t * LS, a.nexp, topk, lane, L.ex, a.topi + t * topk, a.topw + t * topk);
     }
@@ -157,20 +160,20 @@ __global__ void __launch_bounds__(RT_THREADS) k_route_plan(const RouteArgs a) {
     }
     __syncthreads();
     // every row's picks (this block's own included) from memory
-    for (int p = tid; p < P; p += RT_THREADS) {
+    for (int p = tid; p < Pl; p += RT_THREADS) {
         const int e = __hip_atomic_load(&a.topi[p], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         L.ex[p] = e;
         atomicOr(&L.mask[e], 1u << (p / topk));
         atomicMin(&L.first[e], p);
         pl.pair_tok[p] = (uint8_t) (p / topk);
     }
-    if (tid < T) pl.pair_tok[P + tid] = (uint8_t) tid;
+    if (tid < Tl) pl.pair_tok[P + tid] = (uint8_t) tid;
     __syncthreads();
     // job numbers: the rank of an expert's first pair among all first pairs (ballots over the pairs in order)
     int base = 0;
-    for (int p0 = 0; p0 < P; p0 += RT_THREADS) {
+    for (int p0 = 0; p0 < Pl; p0 += RT_THREADS) {
         const int p = p0 + tid;
-        const bool isfirst = p < P && L.first[L.ex[p]] == p;
+        const bool isfirst = p < Pl && L.first[L.ex[p]] == p;
         const unsigned long long b = __ballot(isfirst);
         if (lane == 0) L.wcnt[wave] = __popcll(b);
         __syncthreads();
@@ -194,11 +197,11 @@ __global__ void __launch_bounds__(RT_THREADS) k_route_plan(const RouteArgs a) {
     if (tid == 0) {
         pl.nj = nj;
         pl.job_w[nj] = -1;   // the shared expert's job: every row of the window, pairs P + t
-        pl.job_n[nj] = (uint8_t) T;
+        pl.job_n[nj] = (uint8_t) Tl;
         a.njobs[0] = nj;
     }
     // a pair's slot in its job: the earlier rows in its expert's mask (pairs of a job ascend with the row)
-    for (int p = tid; p < P; p += RT_THREADS) {
+    for (int p = tid; p < Pl; p += RT_THREADS) {
         const int e = L.ex[p], j = L.jobof[e], row = p / topk, slot = __popc(L.mask[e] & ((1u << row) - 1u));
         pl.job_pairs[j][slot] = (uint8_t) p;
         a.jobs_gu[j].y[slot] = row;
@@ -206,7 +209,7 @@ __global__ void __launch_bounds__(RT_THREADS) k_route_plan(const RouteArgs a) {
         a.jobs_dn[j].y[slot] = p;
         a.jobs_dn[j].out[slot] = p;
     }
-    if (tid < T) {   // the shared expert's job, at index P of the lists the API returns (kernels.hpp:277-282)
+    if (tid < max(Tl, 1)) {   // the shared expert's job, at index P of the lists the API returns (kernels.hpp:277-282)
         pl.job_pairs[nj][tid] = (uint8_t) (P + tid);
         a.jobs_gu[P].y[tid] = tid;
         a.jobs_gu[P].out[tid] = P + tid;
@@ -214,7 +217,7 @@ __global__ void __launch_bounds__(RT_THREADS) k_route_plan(const RouteArgs a) {
         a.jobs_dn[P].out[tid] = P + tid;
         if (tid == 0) {
             a.jobs_gu[P].w = a.jobs_dn[P].w = 0;
-            a.jobs_gu[P].n = a.jobs_dn[P].n = T;
+            a.jobs_gu[P].n = a.jobs_dn[P].n = Tl;
         }
     }
     __syncthreads();

@@ -43,7 +43,11 @@ def _q8s(rng, oracle, rows, cols, scale):
 
 
 class TinyDecoder:
-    def __init__(self, oracle, seed=1, n=256, nq=4, nkv=2, nlayers=2, vocab=1000, max_ctx=128, nexp=8, topk=2, ff=256, rope_scaled=False):
+    def __init__(self, oracle, seed=1, n=256, nq=4, nkv=2, nlayers=2, vocab=1000, max_ctx=128, nexp=8, topk=2, ff=256, rope_scaled=False,
+                 cyclic=False):
+        """cyclic: a model whose pick depends on the row's token alone (the attention's output projections are zero) and
+        whose draft layer is the model's single layer behind an identity projection of the embedding, so greedy decoding
+        runs into a cycle, the draft layer mostly predicts the next token, prompt lookup fires and drafts are kept."""
         rng = np.random.default_rng(seed)
         self.oracle = oracle
         self.cfg = dict(n=n, nq=nq, nkv=nkv, nlayers=nlayers, vocab=vocab, max_ctx=max_ctx, nexp=nexp, topk=topk, ff=ff, eps=1e-6)
@@ -68,6 +72,16 @@ class TinyDecoder:
         self.mtp = dict(norm_emb=(1 + 0.1 * rng.standard_normal(n)).astype(np.float32), norm_hid=(1 + 0.1 * rng.standard_normal(n)).astype(np.float32),
                         out_norm=(1 + 0.1 * rng.standard_normal(n)).astype(np.float32), fc_emb=_q8s(rng, oracle, n, n, sw),
                         fc_hid=_q8s(rng, oracle, n, n, sw), head=_q8s(rng, oracle, vocab, n, sw), layer=layer())
+        if cyclic:
+            assert nlayers == 1
+            zero = lambda t: (np.zeros_like(t[0]), np.zeros_like(t[1]))
+            self.layers[0]["wo"] = zero(self.layers[0]["wo"])
+            e = self.emb.astype(np.float32)
+            self.emb = (e / np.sqrt((e * e).mean(axis=1, keepdims=True))).astype(np.float16)
+            eye_q, eye_d = np.zeros((n, n), dtype=np.int8), np.zeros((n, n // 32), dtype=np.uint16)
+            oracle.lib.fnx_o_quantize_q8_0_split(ol.ptr(np.eye(n, dtype=np.float32)), n, n, ol.ptr(eye_q), ol.ptr(eye_d))
+            self.mtp = dict(norm_emb=np.ones(n, dtype=np.float32), norm_hid=self.mtp["norm_hid"], out_norm=self.out_norm, fc_emb=(eye_q, eye_d),
+                            fc_hid=zero(self.mtp["fc_hid"]), head=self.head, layer=self.layers[0])
 
     # ---- the oracle's rendering: host arrays; the caches are numpy arrays kept here
     def oracle_structs(self):
