@@ -330,6 +330,52 @@ typedef struct fnx_round {
  * -> the next window. Expert weights must be in the unit64 layout and hidden = 2048 (the five-launch window), since only
  * that routes a row count held on the device. The draft layer uses the same workspace after the verify. */
 int fnx_decode_round(const fnx_decoder* D, const fnx_mtp* M, const fnx_round* R, const fnx_dec_ws* ws, void* st);
+
+/* ---- GGUF ingestion of a layer's experts (host code; the file format either side of the path).
+ * gguf.hpp:25-45 (Tensor, Gguf), gguf.cpp:219-320 (load_shard: the header walk and its checks, exercised by
+ * tools/gguf_test.cpp): a file, and the "-0000N-of-0000M" shards beside it, mapped read-only and indexed by tensor
+ * name; metadata of the first shard. A header that does not add up is refused with a message naming the tensor. */
+typedef struct fnx_gguf fnx_gguf;
+typedef struct fnx_gguf_tensor {
+    const char* name;   /* lives as long as the handle */
+    uint32_t type;      /* ggml type id (21 = IQ3_S, 0 = F32, 30 = BF16, 8 = Q8_0 ...) */
+    int n_dims;
+    int64_t ne[4];      /* ne[0] = values a row; unused dimensions are 1 */
+    const void* data;   /* in the mapping */
+    size_t nbytes;
+    int shard;          /* which file, and where in it */
+    uint64_t offset;
+} fnx_gguf_tensor;
+fnx_gguf* fnx_gguf_open(const char* first_shard);   /* null on failure: fnx_last_error() */
+void fnx_gguf_close(fnx_gguf* g);
+int fnx_gguf_shards(const fnx_gguf* g);
+int fnx_gguf_count(const fnx_gguf* g);                                        /* tensors over all shards */
+int fnx_gguf_at(const fnx_gguf* g, int i, fnx_gguf_tensor* t);                /* the i-th in name order */
+int fnx_gguf_find(const fnx_gguf* g, const char* name, fnx_gguf_tensor* t);   /* 0: found; 1: no such tensor */
+size_t fnx_gguf_row_bytes(const fnx_gguf_tensor* t);                          /* bytes of one ne[0] row; 0 for an unknown type */
+int fnx_gguf_key_type(const fnx_gguf* g, const char* key);                    /* the GGUF value type of a key of the first shard, or -1 */
+int fnx_gguf_int(const fnx_gguf* g, const char* key, int64_t* v);             /* 0: ok; 1: no such integer key */
+int fnx_gguf_num(const fnx_gguf* g, const char* key, double* v);              /* a number, integer or float as writers differ */
+const char* fnx_gguf_str(const fnx_gguf* g, const char* key);                 /* null: no such string key */
+/* model.cpp:722-741 expert_rows2: per expert, rows [r0, r1) of gate then of up, expert-major, into host memory dst
+ * (null: only *w's shape, *stride and the byte count are worked out). Returns 0 and fills w (w->p = dst) and stride. */
+int fnx_gguf_expert_rows2(const fnx_gguf_tensor* gate, const fnx_gguf_tensor* up, int r0, int r1, void* dst, size_t dst_bytes, fnx_dw* w,
+                          size_t* stride, size_t* bytes);
+/* model.cpp:768-790 expert_cols: per expert, every row's columns [c0, c1) (whole blocks of the tensor's type: multiples
+ * of 256 for IQ3_S; the reference counts 32-value blocks and so cannot slice an IQ3_S row at all) */
+int fnx_gguf_expert_cols(const fnx_gguf_tensor* down, int c0, int c1, void* dst, size_t dst_bytes, fnx_dw* w, size_t* stride, size_t* bytes);
+/* one layer's MoE block from "blk.<layer>.": ffn_gate_inp(.weight) + ffn_gate_inp_shexp -> router rows (F32 or BF16 in the
+ * file, f32 on the device); ffn_gate_exps / ffn_up_exps rows [ff0, ff1) -> gate|up; ffn_down_exps columns [ff0, ff1) ->
+ * down; the _shexp tensors likewise (model.cpp:988-989, 1063-1068 without the card split's other half). Experts must be
+ * IQ3_S; they are uploaded into the caller's device buffers and re-laid there (fnx_iq3s_repack), so *L is ready for
+ * fnx_moe_verify_layer / fnx_moe_prefill_layer. The upload is synchronous; the re-laying runs on st.
+ * topk <= 0: taken from "<general.architecture>.expert_used_count". */
+typedef struct fnx_moe_bufs {
+    void *router, *gu, *down, *sh_gu, *sh_down;   /* device */
+    size_t router_bytes, gu_bytes, down_bytes, sh_gu_bytes, sh_down_bytes;
+} fnx_moe_bufs;
+int fnx_gguf_moe_layer_bytes(const fnx_gguf* g, int layer, int ff0, int ff1, fnx_moe_bufs* sizes);
+int fnx_gguf_load_moe_layer(const fnx_gguf* g, int layer, int ff0, int ff1, int topk, const fnx_moe_bufs* dev, fnx_moe_layer* L, void* st);
 #ifdef __cplusplus
 }
 #endif

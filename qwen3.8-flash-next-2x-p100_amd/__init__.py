@@ -80,6 +80,16 @@ class Round(C.Structure):
                 ("speculate", C.c_int), ("key_n", C.c_int), ("lk", C.c_int), ("scratch", C.c_void_p)]
 
 
+class GgufTensor(C.Structure):
+    _fields_ = [("name", C.c_char_p), ("type", C.c_uint32), ("n_dims", C.c_int), ("ne", C.c_int64 * 4), ("data", C.c_void_p), ("nbytes", C.c_size_t),
+                ("shard", C.c_int), ("offset", C.c_uint64)]
+
+
+class MoeBufs(C.Structure):
+    _fields_ = [(k, C.c_void_p) for k in ("router", "gu", "down", "sh_gu", "sh_down")] + \
+               [(k, C.c_size_t) for k in ("router_bytes", "gu_bytes", "down_bytes", "sh_gu_bytes", "sh_down_bytes")]
+
+
 RS_NCTX, RS_POS, RS_ROWS, RS_ACCEPTED, RS_POS_PREV, RS_ROUNDS, RS_STOP, RS_WORDS = 0, 1, 2, 3, 4, 5, 6, 8
 
 EXPORTS = {
@@ -132,6 +142,23 @@ EXPORTS = {
     "fnx_decoder_verify": (C.c_int, [C.POINTER(Decoder), C.c_void_p, C.c_int, C.c_void_p, C.POINTER(DecWs), C.c_void_p]),
     "fnx_mtp_draft": (C.c_int, [C.POINTER(Decoder), C.POINTER(Mtp), C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.POINTER(DecWs), C.c_void_p]),
     "fnx_decode_round": (C.c_int, [C.POINTER(Decoder), C.POINTER(Mtp), C.POINTER(Round), C.POINTER(DecWs), C.c_void_p]),
+    "fnx_gguf_open": (C.c_void_p, [C.c_char_p]),
+    "fnx_gguf_close": (None, [C.c_void_p]),
+    "fnx_gguf_shards": (C.c_int, [C.c_void_p]),
+    "fnx_gguf_count": (C.c_int, [C.c_void_p]),
+    "fnx_gguf_at": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(GgufTensor)]),
+    "fnx_gguf_find": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(GgufTensor)]),
+    "fnx_gguf_row_bytes": (C.c_size_t, [C.POINTER(GgufTensor)]),
+    "fnx_gguf_key_type": (C.c_int, [C.c_void_p, C.c_char_p]),
+    "fnx_gguf_int": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(C.c_int64)]),
+    "fnx_gguf_num": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(C.c_double)]),
+    "fnx_gguf_str": (C.c_char_p, [C.c_void_p, C.c_char_p]),
+    "fnx_gguf_expert_rows2": (C.c_int, [C.POINTER(GgufTensor), C.POINTER(GgufTensor), C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.POINTER(DW),
+                                        C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
+    "fnx_gguf_expert_cols": (C.c_int, [C.POINTER(GgufTensor), C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.POINTER(DW), C.POINTER(C.c_size_t),
+                                       C.POINTER(C.c_size_t)]),
+    "fnx_gguf_moe_layer_bytes": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int, C.POINTER(MoeBufs)]),
+    "fnx_gguf_load_moe_layer": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(MoeBufs), C.POINTER(MoeLayer), C.c_void_p]),
     "fnx_moe_prefill_layer": (C.c_int, [C.POINTER(MoeLayer), C.c_void_p, C.c_int, C.c_void_p, C.POINTER(PfWs), C.c_void_p]),
 }
 

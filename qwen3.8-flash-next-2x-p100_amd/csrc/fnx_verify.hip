@@ -18,6 +18,7 @@
 
 #include "../../include/fnx_mi355x.h"
 #include "fnx_device.h"
+#include "host_gguf.h"
 
 namespace fnx {
 
@@ -1349,6 +1350,178 @@ int fnx_decode_round(const fnx_decoder* D, const fnx_mtp* M, const fnx_round* R,
     }
     k_round_window<<<1, 64, 0, s>>>(R->ctx, S, R->scratch + 1, R->scratch, ws->best_i, R->speculate, R->rows);
     return launch_status("decode_round");
+}
+
+// ---------------------------------------------------------------- GGUF ingestion (host_gguf.h)
+fnx_gguf* fnx_gguf_open(const char* first_shard) {
+    if (!first_shard) {
+        fail("gguf_open: null argument");
+        return nullptr;
+    }
+    try {
+        return new fnx_gguf(first_shard);
+    } catch (const std::exception& e) {
+        fail(e.what());
+        return nullptr;
+    }
+}
+void fnx_gguf_close(fnx_gguf* g) { delete g; }
+int fnx_gguf_shards(const fnx_gguf* g) { return g ? (int) g->maps.size() : 0; }
+int fnx_gguf_count(const fnx_gguf* g) { return g ? (int) g->order.size() : 0; }
+int fnx_gguf_at(const fnx_gguf* g, int i, fnx_gguf_tensor* t) {
+    if (!g || !t || i < 0 || i >= (int) g->order.size()) return fail("gguf_at: bad argument");
+    gguf::describe(*g->order[(size_t) i], t);
+    return 0;
+}
+int fnx_gguf_find(const fnx_gguf* g, const char* name, fnx_gguf_tensor* t) {
+    if (!g || !name || !t) return fail("gguf_find: null argument");
+    const auto it = g->tensors.find(name);
+    if (it == g->tensors.end()) return fail(std::string("gguf: no tensor ") + name);
+    gguf::describe(it->second, t);
+    return 0;
+}
+size_t fnx_gguf_row_bytes(const fnx_gguf_tensor* t) {
+    gguf::BlockShape bs;
+    if (!t || !gguf::block_shape(t->type, bs)) return 0;
+    return (size_t) (t->ne[0] / bs.values) * (size_t) bs.bytes;
+}
+int fnx_gguf_key_type(const fnx_gguf* g, const char* key) {
+    if (!g || !key) return -1;
+    const auto it = g->keys.find(key);
+    return it == g->keys.end() ? -1 : it->second;
+}
+int fnx_gguf_int(const fnx_gguf* g, const char* key, int64_t* v) {
+    if (!g || !key || !v) return fail("gguf_int: null argument");
+    const auto it = g->ints.find(key);
+    if (it == g->ints.end()) return fail(std::string("gguf: no integer key ") + key);
+    *v = it->second;
+    return 0;
+}
+int fnx_gguf_num(const fnx_gguf* g, const char* key, double* v) {
+    if (!g || !key || !v) return fail("gguf_num: null argument");
+    const auto ii = g->ints.find(key);
+    const auto fi = g->floats.find(key);
+    if (ii != g->ints.end()) *v = (double) ii->second;
+    else if (fi != g->floats.end()) *v = fi->second;
+    else return fail(std::string("gguf: no number key ") + key);
+    return 0;
+}
+const char* fnx_gguf_str(const fnx_gguf* g, const char* key) {
+    if (!g || !key) return nullptr;
+    const auto it = g->strings.find(key);
+    return it == g->strings.end() ? nullptr : it->second.c_str();
+}
+int fnx_gguf_expert_rows2(const fnx_gguf_tensor* gate, const fnx_gguf_tensor* up, int r0, int r1, void* dst, size_t dst_bytes, fnx_dw* w,
+                          size_t* stride, size_t* bytes) {
+    if (!gate || !up) return fail("gguf_expert_rows2: null argument");
+    try {
+        const size_t n = gguf::expert_rows2(*gate, *up, r0, r1, (uint8_t*) dst, dst_bytes, w, stride);
+        if (bytes) *bytes = n;
+        return 0;
+    } catch (const std::exception& e) {
+        return fail(e.what());
+    }
+}
+int fnx_gguf_expert_cols(const fnx_gguf_tensor* down, int c0, int c1, void* dst, size_t dst_bytes, fnx_dw* w, size_t* stride, size_t* bytes) {
+    if (!down) return fail("gguf_expert_cols: null argument");
+    try {
+        const size_t n = gguf::expert_cols(*down, c0, c1, (uint8_t*) dst, dst_bytes, w, stride);
+        if (bytes) *bytes = n;
+        return 0;
+    } catch (const std::exception& e) {
+        return fail(e.what());
+    }
+}
+namespace {
+struct MoeTensors {
+    fnx_gguf_tensor gi, gs, ge, ue, de, gsh, ush, dsh;
+};
+MoeTensors moe_tensors(const fnx_gguf* g, int layer) {
+    const std::string b = "blk." + std::to_string(layer) + ".";
+    const auto get = [&](const char* s) {
+        const auto it = g->tensors.find(b + s);
+        if (it == g->tensors.end()) throw std::runtime_error("gguf: no tensor " + b + s);
+        fnx_gguf_tensor t;
+        gguf::describe(it->second, &t);
+        return t;
+    };
+    MoeTensors m{get("ffn_gate_inp.weight"), get("ffn_gate_inp_shexp.weight"), get("ffn_gate_exps.weight"), get("ffn_up_exps.weight"),
+                 get("ffn_down_exps.weight"), get("ffn_gate_shexp.weight"), get("ffn_up_shexp.weight"), get("ffn_down_shexp.weight")};
+    for (const fnx_gguf_tensor* t : {&m.ge, &m.ue, &m.de, &m.gsh, &m.ush, &m.dsh})
+        if (t->type != gguf::T_IQ3_S) throw std::runtime_error(gguf::nm(*t) + ": ggml type " + std::to_string(t->type) + ", this path reads IQ3_S experts");
+    if (m.gi.ne[0] != m.ge.ne[0] || m.gi.ne[1] != m.ge.ne[2] || m.gs.ne[1] != 1 || m.de.ne[1] != m.ge.ne[0] || m.de.ne[0] != m.ge.ne[1] ||
+        m.de.ne[2] != m.ge.ne[2] || m.gsh.ne[0] != m.ge.ne[0] || m.dsh.ne[1] != m.ge.ne[0] || m.dsh.ne[0] != m.gsh.ne[1] || m.gsh.ne[2] != 1 ||
+        m.dsh.ne[2] != 1)
+        throw std::runtime_error("gguf: the MoE tensors of " + b + " do not fit one another");
+    return m;
+}
+void moe_sizes(const MoeTensors& m, int ff0, int ff1, fnx_moe_bufs* z) {
+    z->router_bytes = (size_t) (m.gi.ne[1] + 1) * (size_t) m.gi.ne[0] * 4;
+    z->gu_bytes = gguf::expert_rows2(m.ge, m.ue, ff0, ff1, nullptr, 0, nullptr, nullptr);
+    z->down_bytes = gguf::expert_cols(m.de, ff0, ff1, nullptr, 0, nullptr, nullptr);
+    z->sh_gu_bytes = gguf::expert_rows2(m.gsh, m.ush, ff0, ff1, nullptr, 0, nullptr, nullptr);
+    z->sh_down_bytes = gguf::expert_cols(m.dsh, ff0, ff1, nullptr, 0, nullptr, nullptr);
+}
+}  // namespace
+int fnx_gguf_moe_layer_bytes(const fnx_gguf* g, int layer, int ff0, int ff1, fnx_moe_bufs* sizes) {
+    if (!g || !sizes) return fail("gguf_moe_layer_bytes: null argument");
+    try {
+        moe_sizes(moe_tensors(g, layer), ff0, ff1, sizes);
+        return 0;
+    } catch (const std::exception& e) {
+        return fail(e.what());
+    }
+}
+int fnx_gguf_load_moe_layer(const fnx_gguf* g, int layer, int ff0, int ff1, int topk, const fnx_moe_bufs* dev, fnx_moe_layer* L, void* st) {
+    if (!g || !dev || !L || !dev->router || !dev->gu || !dev->down || !dev->sh_gu || !dev->sh_down) return fail("gguf_load_moe_layer: null argument");
+    try {
+        const MoeTensors m = moe_tensors(g, layer);
+        fnx_moe_bufs need{};
+        moe_sizes(m, ff0, ff1, &need);
+        if (dev->router_bytes < need.router_bytes || dev->gu_bytes < need.gu_bytes || dev->down_bytes < need.down_bytes ||
+            dev->sh_gu_bytes < need.sh_gu_bytes || dev->sh_down_bytes < need.sh_down_bytes)
+            return fail("gguf_load_moe_layer: a device buffer is smaller than fnx_gguf_moe_layer_bytes says");
+        if (topk <= 0) {
+            const char* arch = fnx_gguf_str(g, "general.architecture");
+            int64_t v = 0;
+            if (!arch || fnx_gguf_int(g, (std::string(arch) + ".expert_used_count").c_str(), &v)) return fail("gguf_load_moe_layer: no <architecture>.expert_used_count key and no topk given");
+            topk = (int) v;
+        }
+        std::memset(L, 0, sizeof *L);
+        L->n = (int) m.ge.ne[0];
+        L->ff = ff1 - ff0;
+        L->nexp = (int) m.ge.ne[2];
+        L->topk = topk;
+        std::vector<uint8_t> host(std::max({need.router_bytes, need.gu_bytes, need.down_bytes, need.sh_gu_bytes, need.sh_down_bytes}));
+        const auto upload = [&](void* d, size_t n, const char* what) {
+            if (hipMemcpy(d, host.data(), n, hipMemcpyHostToDevice) != hipSuccess) throw std::runtime_error(std::string("gguf_load_moe_layer: upload of ") + what + " failed");
+        };
+        const auto relay = [&](fnx_dw& w, void* d, size_t n) {   // raw ggml blocks -> the unit64 layout, in place
+            if (fnx_iq3s_repack(d, d, n / FNX_IQ3S_BLOCK * 256, st)) throw std::runtime_error(fnx_last_error());
+            w.p = d;
+            w.type = FNX_T_IQ3S_UNIT64;
+        };
+        gguf::router_rows(m.gi, m.gs, reinterpret_cast<float*>(host.data()));
+        upload(dev->router, need.router_bytes, "the router");
+        L->router = dev->router;
+        L->router_bf16 = 0;
+        gguf::expert_rows2(m.ge, m.ue, ff0, ff1, host.data(), host.size(), &L->gu, &L->gu_stride);
+        upload(dev->gu, need.gu_bytes, "gate|up");
+        relay(L->gu, dev->gu, need.gu_bytes);
+        gguf::expert_cols(m.de, ff0, ff1, host.data(), host.size(), &L->down, &L->down_stride);
+        upload(dev->down, need.down_bytes, "down");
+        relay(L->down, dev->down, need.down_bytes);
+        size_t unused;
+        gguf::expert_rows2(m.gsh, m.ush, ff0, ff1, host.data(), host.size(), &L->sh_gu, &unused);
+        upload(dev->sh_gu, need.sh_gu_bytes, "the shared gate|up");
+        relay(L->sh_gu, dev->sh_gu, need.sh_gu_bytes);
+        gguf::expert_cols(m.dsh, ff0, ff1, host.data(), host.size(), &L->sh_down, &unused);
+        upload(dev->sh_down, need.sh_down_bytes, "the shared down");
+        relay(L->sh_down, dev->sh_down, need.sh_down_bytes);
+        return 0;
+    } catch (const std::exception& e) {
+        return fail(e.what());
+    }
 }
 
 }  // extern "C"

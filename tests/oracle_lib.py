@@ -84,7 +84,7 @@ def load():
 
 
 def load_ref():
-    """The reference's own tensor_convert.hpp compiled as a shared library, or None when it was not built."""
+    """The reference's own tensor_convert.hpp and GGUF reader compiled as a shared library, or None when it was not built."""
     path = os.path.join(ORACLE_DIR, "_ref", "libfnx_ref.so")
     if not os.path.exists(path):
         return None
@@ -96,6 +96,24 @@ def load_ref():
     lib.fnx_ref_iq3s_grid.restype = C.POINTER(C.c_uint32)
     lib.fnx_ref_dequantize.restype = C.c_int
     lib.fnx_ref_dequantize.argtypes = [C.c_uint32, C.c_void_p, C.c_size_t, C.c_void_p]
+    if hasattr(lib, "fnx_ref_gguf_open"):   # the reference's GGUF reader (a library built before it was added lacks it)
+        lib.fnx_ref_gguf_open.restype = C.c_void_p
+        lib.fnx_ref_gguf_open.argtypes = [C.c_char_p, C.c_char_p, C.c_size_t]
+        lib.fnx_ref_gguf_close.restype = None
+        lib.fnx_ref_gguf_close.argtypes = [C.c_void_p]
+        for name in ("fnx_ref_gguf_count", "fnx_ref_gguf_shards"):
+            getattr(lib, name).restype = C.c_int
+            getattr(lib, name).argtypes = [C.c_void_p]
+        lib.fnx_ref_gguf_tensor.restype = C.c_int
+        lib.fnx_ref_gguf_tensor.argtypes = [C.c_void_p, C.c_int, C.c_char_p, C.c_size_t, C.POINTER(C.c_int64)]
+        lib.fnx_ref_gguf_data.restype = C.c_void_p
+        lib.fnx_ref_gguf_data.argtypes = [C.c_void_p, C.c_char_p]
+        lib.fnx_ref_gguf_has_key.restype = C.c_int
+        lib.fnx_ref_gguf_has_key.argtypes = [C.c_void_p, C.c_char_p]
+        lib.fnx_ref_gguf_num.restype = C.c_int
+        lib.fnx_ref_gguf_num.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_double)]
+        lib.fnx_ref_gguf_str.restype = C.c_int
+        lib.fnx_ref_gguf_str.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p, C.c_size_t]
     return lib
 
 

@@ -1,0 +1,70 @@
+"""A layer's experts from a GGUF file onto the device (fnx_gguf_load_moe_layer: model.cpp:988-989, 1063-1068 without the
+other card's half) and through the verify window, against the CPU oracle on the arrays the file was written from.
+Bar: router logits, picks and jobs bit-exact, the layer's output within 1e-3 relative L2 (as tests/test_gpu_moe.py)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import fnx_gpu
+import gguf_files as gf
+
+pytestmark = pytest.mark.gpu
+
+
+def rel_l2(a, b):
+    return float(np.linalg.norm(a.astype(np.float64) - b.astype(np.float64)) / max(np.linalg.norm(b.astype(np.float64)), 1e-30))
+
+
+@pytest.fixture(scope="module")
+def dev():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    return fnx_gpu.Dev()
+
+
+@pytest.mark.parametrize("router_type,ff0,ff1,topk_from_file", [(gf.F32, 0, 512, True), (gf.BF16, 0, 512, False), (gf.F32, 256, 512, False)])
+def test_layer_from_gguf_matches_oracle(dev, oracle, tmp_path, router_type, ff0, ff1, topk_from_file):
+    t, lib, pkg = dev.torch, dev.lib, dev.pkg
+    rng = np.random.default_rng(77)
+    n, ff_total, nexp, topk, T, layer = 2048, 512, 24, 10, 16, 7
+    ts, a = gf.moe_layer_tensors(rng, layer, n, ff_total, nexp, fnx_gpu.random_iq3s, router_type)
+    # the layer's tensors over two shards, other tensors between them
+    filler = ("blk.7.attn_norm.weight", gf.F32, [n], rng.standard_normal(n).astype(np.float32).tobytes())
+    keys = [gf.kv("general.architecture", gf.STR, "fnxtest"), gf.kv("fnxtest.expert_used_count", gf.U32, topk)]
+    first = gf.write(tmp_path / "layer-00001-of-00002.gguf", [filler] + ts[:4], keys=keys)
+    gf.write(tmp_path / "layer-00002-of-00002.gguf", ts[4:], keys=[])
+    print(f"case gguf layer router={router_type} ff=[{ff0},{ff1}) topk_from_file={topk_from_file}", flush=True)
+    g = lib.fnx_gguf_open(first.encode())
+    assert g, lib.fnx_last_error()
+    z = pkg.MoeBufs()
+    dev.ok(lib.fnx_gguf_moe_layer_bytes(g, layer, ff0, ff1, C.byref(z)))
+    bufs = [dev.zeros(getattr(z, k + "_bytes"), t.uint8) for k in ("router", "gu", "down", "sh_gu", "sh_down")]
+    for k, b in zip(("router", "gu", "down", "sh_gu", "sh_down"), bufs):
+        setattr(z, k, b.data_ptr())
+    L = pkg.MoeLayer()
+    dev.ok(lib.fnx_gguf_load_moe_layer(g, layer, ff0, ff1, 0 if topk_from_file else topk, C.byref(z), C.byref(L), dev.st()))
+    dev.sync()
+    lib.fnx_gguf_close(g)   # the device copies stand on their own
+    ff = ff1 - ff0
+    assert (L.n, L.ff, L.nexp, L.topk, L.gu.type, L.gu_stride, L.down_stride) == (n, ff, nexp, topk, pkg.T_IQ3S_UNIT64, 2 * ff * 880, n * ff // 256 * 110)
+    # the same slices for the oracle
+    gu = gf.slice_rows2(a["gate"], a["up"], n, ff_total, nexp, ff0, ff1)
+    down = gf.slice_cols(a["down"], n, ff_total, nexp, ff0, ff1)
+    sh_gu = gf.slice_rows2(a["sh_gate"], a["sh_up"], n, ff_total, 1, ff0, ff1)
+    sh_down = gf.slice_cols(a["sh_down"], n, ff_total, 1, ff0, ff1)
+    router = np.concatenate([a["router"], a["sh_router"]])
+    x = rng.standard_normal((T, n)).astype(np.float32)
+    want = oracle.moe_verify_layer(n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, x)
+    # a workspace as MoeLayerDev makes it
+    P = T * topk
+    w = dict(xq=dev.zeros(T * (n // 32) * 36, t.uint8), logits=dev.zeros((T, nexp + 1), t.float32), topi=dev.zeros((T, topk), t.int32),
+             topw=dev.zeros((T, topk), t.float32), jobs_gu=dev.zeros((P + 1) * 136, t.uint8), jobs_dn=dev.zeros((P + 1) * 136, t.uint8),
+             njobs=dev.zeros(2, t.int32), gu=dev.zeros((P + T, 2 * ff), t.float32), part=dev.zeros((P + T, n), t.float32))
+    ws = pkg.MoeWs(*(w[k].data_ptr() for k in ("xq", "logits", "topi", "topw", "jobs_gu", "jobs_dn", "njobs", "gu", "part")))
+    dx, out = dev.up(x), dev.zeros((T, n), t.float32)
+    dev.ok(lib.fnx_moe_verify_layer(C.byref(L), dx.data_ptr(), T, out.data_ptr(), C.byref(ws), dev.st()))
+    dev.sync()
+    assert np.array_equal(w["logits"].cpu().numpy().view(np.uint32), want["logits"].view(np.uint32)), "router logits bit-exact"
+    assert np.array_equal(w["topi"].cpu().numpy(), want["topi"]) and int(w["njobs"][0].item()) == want["njobs"]
+    assert rel_l2(out.cpu().numpy(), want["out"]) <= 1e-3
