@@ -330,6 +330,10 @@ def head_main(args):
         dev.ok(lib.fnx_accept_greedy_dev(drows.data_ptr(), bi.data_ptr(), len(rows), nacc.data_ptr(), st))
         dev.ok(lib.fnx_lookup_drafts_dev(dctx.data_ptr(), NCTX, 3, 15, dd1.data_ptr(), dout.data_ptr(), dn.data_ptr(), dm.data_ptr(), st))
     us_all = timed(all3, n)
+    # the sampler's candidates over the same rows (the non-greedy half of acceptance): 64 a row, no penalty or bias lists
+    tk_v, tk_i = dev.zeros((R, 64), t.float32), dev.zeros((R, 64), t.int32)
+    us_top = timed(lambda i: dev.ok(lib.fnx_top_tokens(logits[i % NL].data_ptr(), V, R, 0, None, None, None, 0, None, None, None, None, None,
+                                                       tk_v.data_ptr(), tk_i.data_ptr(), err.data_ptr(), st)), n)
     # parity on this exact input
     all3(0)
     t.cuda.synchronize()
@@ -350,7 +354,7 @@ def head_main(args):
             "steps": n, "warmup": 20, "ms_per_step": us_all / 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32 compare / int32",
             "data": "synthetic",
             "config": {"workload": "config 3: logits 16 x 151,936 f32, context 38,862 int32 with 200 copied spans, key 3, up to 15 drafts",
-                       "argmax_us": us_arg, "lookup_us": us_lk, "accept_us": us_acc, "drafts": int(len(drafts)), "accepted": int(nacc.item()),
+                       "argmax_us": us_arg, "lookup_us": us_lk, "accept_us": us_acc, "top_tokens_us": us_top, "drafts": int(len(drafts)), "accepted": int(nacc.item()),
                        "identical_to_oracle": same},
             "roofline": {"bound": "hbm", "kernel": "k_argmax", "achieved": arg_bytes / (us_arg * 1e-6) / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                          "frac": arg_bytes / (us_arg * 1e-6) / HBM_PEAK, "traffic": None, "algorithmic_bytes": arg_bytes,

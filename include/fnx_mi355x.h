@@ -331,6 +331,41 @@ typedef struct fnx_round {
  * that routes a row count held on the device. The draft layer uses the same workspace after the verify. */
 int fnx_decode_round(const fnx_decoder* D, const fnx_mtp* M, const fnx_round* R, const fnx_dec_ws* ws, void* st);
 
+/* ---- the sampler: the non-greedy half of acceptance.
+ * kernels.hpp:434-447 + topk.cuh (top_tokens): per row t < T of logits (n of the vocabulary from token v0) the row's
+ * logit_bias (bias_n[t] of them from bias_off[t] in bias_tok / bias_val, each token once) and penalties (pen_n[t] tokens
+ * and their counts at row t * pen_stride; pen_par: per row repeat, freq, present: a non-positive logit times repeat, a
+ * positive one divided by it, then minus count * freq and minus present) applied IN PLACE, then the row's FNX_TOPK_N
+ * highest into out_v / out_i (logit descending, token id ascending on ties, however many tie). err bit 16: a logit was NaN
+ * or inf before the penalties. pen_n and bias_n may be null (no such lists). n >= FNX_TOPK_N, n <= 327,680. The slices'
+ * candidates pass between the two launches in one library-owned device buffer: one top_tokens in flight per device. */
+#define FNX_TOPK_N 64
+int fnx_top_tokens(float* logits, int n, int T, int v0, const int* pen_tok, const int* pen_cnt, const int* pen_n, int pen_stride,
+                   const float* pen_par, const int* bias_tok, const float* bias_val, const int* bias_off, const int* bias_n, float* out_v,
+                   int* out_i, unsigned* err, void* st);
+/* kernels.hpp:434-436 penalize_row: pen = {k, k indexes into the row, their k counts}, par = {repeat, freq, present};
+ * k <= 4096 (engine.hpp:73 PEN_CAP; a greater count is cut there, as is a bias list's) */
+int fnx_penalize_row(float* row, int n, const int* pen, const float* par, void* st);
+/* session.hpp:17-26 Sampling, the values the distribution is made from (temperature > 0: greedy rows do not come here) */
+typedef struct fnx_sampling {
+    float temperature, top_p, min_p;
+    int top_k;   /* 0: no cut */
+} fnx_sampling;
+/* session.cpp:41-75 make_dist (host): a row's distribution from its candidates in top_tokens' order: top_k, then top_p
+ * over the untempered softmax of those (in double), then min_p as a logit threshold, then the temperature's softmax over
+ * the survivors. Returns how many survive (ids, p filled; both hold ncand), or -1. */
+int fnx_make_dist(const float* cand_v, const int* cand_i, int ncand, const fnx_sampling* s, int* ids, double* p);
+/* session.cpp:77-84 draw (host): the token at u in [0, 1) */
+int fnx_draw(const int* ids, const double* p, int n, double u);
+/* session.cpp:574-613 (host): speculative sampling over a window. cand_v / cand_i: T rows of ncand candidates; rows[0] the
+ * window's first token, rows[j + 1] draft j, drawn from q_j = (q_ids, q_p)[j * q_stride ..][q_n[j]] (q_n null or
+ * q_n[j] = 0: a fixed draft, all of q_j on it). Draft j stands with probability min(1, p_j / q_j); else row j's token is
+ * drawn from max(0, p_j - q_j) normalized and the window ends there; all standing: one more from the last row. The
+ * uniforms come from u in the order they are used (the reference draws them from its mt19937_64 as it goes); *used_u =
+ * how many were. Returns the tokens emitted n (o[0 .. n)), or -1. */
+int fnx_accept_sampled(const float* cand_v, const int* cand_i, int ncand, int T, const int* rows, const fnx_sampling* s, const int* q_ids,
+                       const double* q_p, const int* q_n, int q_stride, const double* u, int nu, int* o, int* used_u);
+
 /* ---- GGUF ingestion of a layer's experts (host code; the file format either side of the path).
  * gguf.hpp:25-45 (Tensor, Gguf), gguf.cpp:219-320 (load_shard: the header walk and its checks, exercised by
  * tools/gguf_test.cpp): a file, and the "-0000N-of-0000M" shards beside it, mapped read-only and indexed by tensor

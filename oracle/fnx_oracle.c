@@ -495,6 +495,141 @@ unsigned fnx_o_argmax(const float* logits, int rows, int T, int v0, float* best_
     return err;
 }
 
+/* ---------------------------------------------------------------- the sampler's candidates (topk.cuh, kernels.hpp:434-447) */
+static int cmp_desc_u64(const void* a, const void* b) {
+    const uint64_t x = *(const uint64_t*) a, y = *(const uint64_t*) b;
+    return x < y ? 1 : x > y ? -1 : 0;
+}
+/* kernels.cu:1771-1781 k_penalize_row; the same arithmetic as topk.cuh:40-46 */
+static float penalized(float l, int cnt, float repeat, float freq, float present) {
+    l = l <= 0.f ? l * repeat : l / repeat;
+    return l - (float) cnt * freq - present;
+}
+void fnx_o_penalize_row(float* row, int n, const int* pen, const float* par) {
+    const int k = pen[0];
+    for (int i = 0; i < k; ++i) {
+        const int j = pen[1 + i], cnt = pen[1 + k + i];
+        if (j < 0 || j >= n || cnt <= 0) continue;
+        row[j] = penalized(row[j], cnt, par[0], par[1], par[2]);
+    }
+}
+/* topk.cuh:18-156 k_topk_rows: the finite check on the head's logits, the row's logit_bias, then its penalties (in
+ * place), then the 64 greatest by (order-preserving key of the logit's bits descending, id ascending). The reference's
+ * radix select and its wide-tie pass are a way to that set; here every (key, id) pair is sorted. */
+unsigned fnx_o_top_tokens(float* logits, int n, int T, int v0, const int* pen_tok, const int* pen_cnt, const int* pen_n, int pen_stride,
+                          const float* pen_par, const int* bias_tok, const float* bias_val, const int* bias_off, const int* bias_n, float* out_v,
+                          int* out_i) {
+    unsigned err = 0;
+    uint64_t* keys = (uint64_t*) malloc((size_t) n * sizeof(uint64_t));
+    for (int t = 0; t < T; ++t) {
+        float* L = logits + (size_t) t * n;
+        for (int j = 0; j < n; ++j)
+            if (!isfinite(L[j])) err |= 16u;
+        for (int i = 0; bias_n && i < bias_n[t]; ++i) {
+            const int at = bias_off[t] + i, tok = bias_tok[at] - v0;
+            if (tok >= 0 && tok < n) L[tok] += bias_val[at];
+        }
+        for (int i = 0; pen_n && i < pen_n[t]; ++i) {
+            const int tok = pen_tok[t * pen_stride + i] - v0, cnt = pen_cnt[t * pen_stride + i];
+            if (tok < 0 || tok >= n || cnt <= 0) continue;
+            L[tok] = penalized(L[tok], cnt, pen_par[t * 3], pen_par[t * 3 + 1], pen_par[t * 3 + 2]);
+        }
+        for (int j = 0; j < n; ++j) keys[j] = (uint64_t) fkey(L[j]) << 32 | (uint32_t) (0xffffffffu - (uint32_t) j);
+        qsort(keys, (size_t) n, sizeof(uint64_t), cmp_desc_u64);
+        for (int r = 0; r < 64; ++r) {
+            const int j = (int) (0xffffffffu - (uint32_t) keys[r]);
+            out_i[t * 64 + r] = v0 + j;
+            out_v[t * 64 + r] = L[j];
+        }
+    }
+    free(keys);
+    return err;
+}
+
+/* ---------------------------------------------------------------- the sampler's draw (session.cpp:34-84, 574-613) */
+static double dist_prob(const int* ids, const double* p, int n, int id) { /* session.cpp:34-39 */
+    for (int i = 0; i < n; ++i)
+        if (ids[i] == id) return p[i];
+    return 0.0;
+}
+/* session.cpp:41-75 make_dist */
+int fnx_o_make_dist(const float* cv, const int* ci, int ncand, float temperature, float top_p, float min_p, int top_k, int* ids, double* p) {
+    const int k = (top_k <= 0 || top_k > ncand) ? ncand : top_k;
+    int keep = k;
+    const double mx = cv[0];
+    if (top_p < 1.f) {
+        double sum = 0.0, cum = 0.0;
+        for (int i = 0; i < k; ++i) sum += exp((double) cv[i] - mx);
+        for (int i = 0; i < k; ++i) {
+            cum += exp((double) cv[i] - mx) / sum;
+            if (cum >= (double) top_p) {
+                keep = i + 1;
+                break;
+            }
+        }
+    }
+    if (min_p > 0.f) {
+        const float thresh = cv[0] + logf(min_p);
+        for (int i = 1; i < keep; ++i)
+            if (cv[i] < thresh) {
+                keep = i;
+                break;
+            }
+    }
+    const double inv_t = 1.0 / temperature, smx = cv[0] * inv_t;
+    double sum = 0.0;
+    for (int i = 0; i < keep; ++i) {
+        ids[i] = ci[i];
+        p[i] = exp(cv[i] * inv_t - smx);
+        sum += p[i];
+    }
+    for (int i = 0; i < keep; ++i) p[i] /= sum;
+    return keep;
+}
+/* session.cpp:77-84 draw */
+int fnx_o_draw(const int* ids, const double* p, int n, double u) {
+    double cum = 0.0;
+    for (int i = 0; i < n; ++i) {
+        cum += p[i];
+        if (u < cum) return ids[i];
+    }
+    return ids[n - 1];
+}
+/* session.cpp:574-613: speculative sampling over a window of T rows; uniforms taken from u in the order of use */
+int fnx_o_accept_sampled(const float* cv, const int* ci, int ncand, int T, const int* rows, float temperature, float top_p, float min_p, int top_k,
+                         const int* q_ids, const double* q_p, const int* q_n, int q_stride, const double* u, int* o, int* used_u) {
+    int ids[64], n, at = 0;
+    double p[64], p0[64];
+    for (n = 0; n < T; ++n) {
+        int m = fnx_o_make_dist(cv + (size_t) n * ncand, ci + (size_t) n * ncand, ncand, temperature, top_p, min_p, top_k, ids, p);
+        if (n + 1 < T) {
+            const int dr = rows[n + 1], qn = q_n ? q_n[n] : 0, fixed = qn == 0;
+            const int* qi = q_ids ? q_ids + (size_t) n * q_stride : NULL;
+            const double* qp = q_p ? q_p + (size_t) n * q_stride : NULL;
+            if (u[at++] * (fixed ? 1.0 : dist_prob(qi, qp, qn, dr)) < dist_prob(ids, p, m, dr)) {
+                o[n] = dr;
+                continue;
+            }
+            double rest = 0.0;
+            memcpy(p0, p, sizeof(double) * (size_t) m);
+            for (int i = 0; i < m; ++i) {
+                const double q = fixed ? (ids[i] == dr ? 1.0 : 0.0) : dist_prob(qi, qp, qn, ids[i]);
+                p[i] = p[i] - q > 0.0 ? p[i] - q : 0.0;
+                rest += p[i];
+            }
+            if (rest > 1e-12)
+                for (int i = 0; i < m; ++i) p[i] /= rest;
+            else
+                memcpy(p, p0, sizeof(double) * (size_t) m);
+        }
+        o[n] = fnx_o_draw(ids, p, m, u[at++]);
+        ++n;
+        break;
+    }
+    if (used_u) *used_u = at;
+    return n;
+}
+
 /* ---------------------------------------------------------------- prompt lookup, acceptance */
 #define LOOKUP_MIN 3       /* session.cpp:18 */
 #define IMAGE_TOK (1 << 30) /* engine.hpp:84 */

@@ -12,7 +12,10 @@
  *             dp4a (selftest.cu's generator), vec_dot/mmvq (vs dequant in f64), q8_1 (closed forms, round trip),
  *             route/topk (two in-tree definitions agree; brute-force sort), jobs (two in-tree builders' invariants),
  *             argmax (brute force + tie/NaN cases), lookup (second in-tree implementation + brute force), accept
- *             (speculative == greedy invariant), swiglu/combine (f64 closed forms).
+ *             (speculative == greedy invariant), swiglu/combine (f64 closed forms), top_tokens (numpy lexsort on
+ *             (-key, id) incl. wide ties and signed zeros; penalties as a numpy f32 closed form), make_dist (numpy
+ *             vectorised softmax / cumulative cut, limiting cases), accept_sampled (the window's first token is
+ *             distributed as the target p whatever q is: exact measure over a grid of uniforms; fixed-draft closed form).
  *   parity unpinned: fnx_o_iq3s_quantize_row (the encoder). ggml's quantize_row_iq3_s is not in the reference tree
  *             (third_party/ggml holds only a commit hash) and nothing in the reference calls or tests it. The encoder
  *             here is this build's own; parity of the path is defined from the quantised bytes onward.
@@ -96,6 +99,16 @@ int fnx_o_lookup_drafts(const int* ctx, int n_ctx, int key_n, int lk, int d1, in
 int fnx_o_lookup_fixed(const int* ctx, int n_ctx, int key_n, int lk, int d1, int* out);
 /* session.cpp:573 */
 int fnx_o_accept_greedy(const int* rows, const int* o, int R);
+/* kernels.hpp:434-447, topk.cuh: the sampler's candidates (64 a row), logits changed in place; returns the err bits */
+unsigned fnx_o_top_tokens(float* logits, int n, int T, int v0, const int* pen_tok, const int* pen_cnt, const int* pen_n, int pen_stride,
+                          const float* pen_par, const int* bias_tok, const float* bias_val, const int* bias_off, const int* bias_n, float* out_v,
+                          int* out_i);
+void fnx_o_penalize_row(float* row, int n, const int* pen, const float* par);
+/* session.cpp:41-84, 574-613: a row's distribution, a draw, speculative sampling over a window (ncand <= 64) */
+int fnx_o_make_dist(const float* cv, const int* ci, int ncand, float temperature, float top_p, float min_p, int top_k, int* ids, double* p);
+int fnx_o_draw(const int* ids, const double* p, int n, double u);
+int fnx_o_accept_sampled(const float* cv, const int* ci, int ncand, int T, const int* rows, float temperature, float top_p, float min_p, int top_k,
+                         const int* q_ids, const double* q_p, const int* q_n, int q_stride, const double* u, int* o, int* used_u);
 
 /* prefill routing: top-k per row, histogram, jobs of <= pf_job rows per expert, pairs in ascending order.
  * prefill.cu:288-377. jobs: arrays of {w, n, y[pf_job], out[pf_job]} ints. returns the job count */

@@ -80,6 +80,10 @@ class Round(C.Structure):
                 ("speculate", C.c_int), ("key_n", C.c_int), ("lk", C.c_int), ("scratch", C.c_void_p)]
 
 
+class Sampling(C.Structure):
+    _fields_ = [("temperature", C.c_float), ("top_p", C.c_float), ("min_p", C.c_float), ("top_k", C.c_int)]
+
+
 class GgufTensor(C.Structure):
     _fields_ = [("name", C.c_char_p), ("type", C.c_uint32), ("n_dims", C.c_int), ("ne", C.c_int64 * 4), ("data", C.c_void_p), ("nbytes", C.c_size_t),
                 ("shard", C.c_int), ("offset", C.c_uint64)]
@@ -142,6 +146,13 @@ EXPORTS = {
     "fnx_decoder_verify": (C.c_int, [C.POINTER(Decoder), C.c_void_p, C.c_int, C.c_void_p, C.POINTER(DecWs), C.c_void_p]),
     "fnx_mtp_draft": (C.c_int, [C.POINTER(Decoder), C.POINTER(Mtp), C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.POINTER(DecWs), C.c_void_p]),
     "fnx_decode_round": (C.c_int, [C.POINTER(Decoder), C.POINTER(Mtp), C.POINTER(Round), C.POINTER(DecWs), C.c_void_p]),
+    "fnx_top_tokens": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p,
+                                 C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "fnx_penalize_row": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "fnx_make_dist": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.POINTER(Sampling), C.c_void_p, C.c_void_p]),
+    "fnx_draw": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_double]),
+    "fnx_accept_sampled": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.POINTER(Sampling), C.c_void_p, C.c_void_p, C.c_void_p,
+                                     C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.POINTER(C.c_int)]),
     "fnx_gguf_open": (C.c_void_p, [C.c_char_p]),
     "fnx_gguf_close": (None, [C.c_void_p]),
     "fnx_gguf_shards": (C.c_int, [C.c_void_p]),

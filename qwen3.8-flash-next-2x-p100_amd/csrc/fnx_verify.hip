@@ -15,6 +15,7 @@
 #include <cstring>
 #include <string>
 #include <type_traits>
+#include <vector>
 
 #include "../../include/fnx_mi355x.h"
 #include "fnx_device.h"
@@ -434,6 +435,7 @@ __global__ void __launch_bounds__(512) k_iq3s_jobs(const RowsArgs a) {
 #include "k_prefill.h"
 #include "k_decoder.h"
 #include "k_round.h"
+#include "k_sampler.h"
 namespace fnx {
 
 // any other row length (a multiple of 256): a wave per (row, job), sub-blocks dealt round-robin to the lanes, the
@@ -1350,6 +1352,155 @@ int fnx_decode_round(const fnx_decoder* D, const fnx_mtp* M, const fnx_round* R,
     }
     k_round_window<<<1, 64, 0, s>>>(R->ctx, S, R->scratch + 1, R->scratch, ws->best_i, R->speculate, R->rows);
     return launch_status("decode_round");
+}
+
+// ---------------------------------------------------------------- the sampler: candidates on the device, the draw on the host
+int fnx_top_tokens(float* logits, int n, int T, int v0, const int* pen_tok, const int* pen_cnt, const int* pen_n, int pen_stride,
+                   const float* pen_par, const int* bias_tok, const float* bias_val, const int* bias_off, const int* bias_n, float* out_v,
+                   int* out_i, unsigned* err, void* st) {
+    if (!logits || !out_v || !out_i || !err) return fail("top_tokens: null argument");
+    if (n < SM_N) return fail("top_tokens: a vocabulary slice smaller than the candidates");
+    if (T < 1 || T > FNX_MAXT) return fail("top_tokens: T out of range");
+    if (n > SM_MAXS * SM_SLICE) return fail("top_tokens: rows of up to 327,680 logits");
+    if ((pen_n && (!pen_tok || !pen_cnt || !pen_par || pen_stride < 0)) || (bias_n && (!bias_tok || !bias_val || !bias_off)))
+        return fail("top_tokens: a list's count without the list");
+    const int nslice = (n + SM_SLICE - 1) / SM_SLICE;
+    hipStream_t s = (hipStream_t) st;
+    k_top_slices<<<dim3(nslice, T), SM_THREADS, 0, s>>>(
+        TopArgs{logits, n, v0, nslice, pen_tok, pen_cnt, pen_n, pen_stride, pen_par, bias_tok, bias_val, bias_off, bias_n, err});
+    k_top_merge<<<T, SM_MERGE_THREADS, 0, s>>>(logits, n, v0, nslice, out_v, out_i);
+    return launch_status("top_tokens");
+}
+int fnx_penalize_row(float* row, int n, const int* pen, const float* par, void* st) {
+    if (!row || !pen || !par || n < 1) return fail("penalize_row: bad argument");
+    k_penalize_row<<<1, 256, 0, (hipStream_t) st>>>(row, n, pen, par);
+    return launch_status("penalize_row");
+}
+}  // extern "C"
+namespace {
+struct HostDist {
+    std::vector<int> ids;
+    std::vector<double> p;
+    double of(int id) const {
+        for (size_t i = 0; i < ids.size(); ++i)
+            if (ids[i] == id) return p[i];
+        return 0.0;
+    }
+};
+// session.cpp:41-75: top_k, then top_p over the untempered softmax of those, then min_p as a logit threshold, then the
+// temperature's softmax over what is left; all in double on the f32 candidates
+HostDist host_dist(const float* v, const int* id, int ncand, const fnx_sampling& s) {
+    const int k = (s.top_k <= 0 || s.top_k > ncand) ? ncand : s.top_k;
+    int keep = k;
+    const double top = v[0];
+    if (s.top_p < 1.f) {
+        double z = 0.0, run = 0.0;
+        for (int i = 0; i < k; ++i) z += std::exp((double) v[i] - top);
+        for (int i = 0; i < k; ++i) {
+            run += std::exp((double) v[i] - top) / z;
+            if (run >= (double) s.top_p) {
+                keep = i + 1;
+                break;
+            }
+        }
+    }
+    if (s.min_p > 0.f) {
+        const float floor_v = v[0] + std::log(s.min_p);
+        int i = 1;
+        while (i < keep && !(v[i] < floor_v)) ++i;
+        keep = std::min(keep, i);
+    }
+    HostDist d;
+    const double inv_t = 1.0 / s.temperature, shift = v[0] * inv_t;
+    double z = 0.0;
+    for (int i = 0; i < keep; ++i) {
+        d.ids.push_back(id[i]);
+        d.p.push_back(std::exp(v[i] * inv_t - shift));
+        z += d.p.back();
+    }
+    for (double& x : d.p) x /= z;
+    return d;
+}
+int host_draw(const HostDist& d, double u) {   // session.cpp:77-84
+    double run = 0.0;
+    for (size_t i = 0; i < d.ids.size(); ++i) {
+        run += d.p[i];
+        if (u < run) return d.ids[i];
+    }
+    return d.ids.back();
+}
+bool sampling_ok(const fnx_sampling* s, int ncand) {
+    return s && ncand >= 1 && std::isfinite(s->temperature) && s->temperature > 0.f && s->top_p > 0.f && s->top_p <= 1.f && s->min_p >= 0.f &&
+           s->min_p <= 1.f && s->top_k >= 0;
+}
+}  // namespace
+extern "C" {
+int fnx_make_dist(const float* cand_v, const int* cand_i, int ncand, const fnx_sampling* s, int* ids, double* p) {
+    if (!cand_v || !cand_i || !ids || !p || !sampling_ok(s, ncand)) {
+        fail("make_dist: bad argument (temperature > 0, top_p in (0, 1], min_p in [0, 1], top_k >= 0)");
+        return -1;
+    }
+    const HostDist d = host_dist(cand_v, cand_i, ncand, *s);
+    std::copy(d.ids.begin(), d.ids.end(), ids);
+    std::copy(d.p.begin(), d.p.end(), p);
+    return (int) d.ids.size();
+}
+int fnx_draw(const int* ids, const double* p, int n, double u) {
+    if (!ids || !p || n < 1) {
+        fail("draw: bad argument");
+        return -1;
+    }
+    HostDist d;
+    d.ids.assign(ids, ids + n);
+    d.p.assign(p, p + n);
+    return host_draw(d, u);
+}
+int fnx_accept_sampled(const float* cand_v, const int* cand_i, int ncand, int T, const int* rows, const fnx_sampling* s, const int* q_ids,
+                       const double* q_p, const int* q_n, int q_stride, const double* u, int nu, int* o, int* used_u) {
+    if (!cand_v || !cand_i || !rows || !u || !o || T < 1 || T > FNX_MAXT || !sampling_ok(s, ncand) || (q_n && (!q_ids || !q_p || q_stride < 1))) {
+        fail("accept_sampled: bad argument");
+        return -1;
+    }
+    int n = 0, at = 0;
+    const auto next_u = [&]() { return at < nu ? u[at++] : (++at, 0.0); };
+    for (; n < T; ++n) {
+        HostDist d = host_dist(cand_v + (size_t) n * ncand, cand_i + (size_t) n * ncand, ncand, *s);
+        if (n + 1 < T) {
+            const int draft = rows[n + 1];
+            HostDist q;   // empty: a fixed draft, all of q on it
+            if (q_n && q_n[n] > 0) {
+                q.ids.assign(q_ids + (size_t) n * q_stride, q_ids + (size_t) n * q_stride + q_n[n]);
+                q.p.assign(q_p + (size_t) n * q_stride, q_p + (size_t) n * q_stride + q_n[n]);
+            }
+            const bool fixed = q.ids.empty();
+            // the draft stands with probability min(1, p / q)
+            if (next_u() * (fixed ? 1.0 : q.of(draft)) < d.of(draft)) {
+                o[n] = draft;
+                continue;
+            }
+            // else the row's token comes from max(0, p - q), normalized; p <= q everywhere means p == q up to rounding: from p
+            const HostDist whole = d;
+            double rest = 0.0;
+            for (size_t i = 0; i < d.ids.size(); ++i) {
+                const double qi = fixed ? (d.ids[i] == draft ? 1.0 : 0.0) : q.of(d.ids[i]);
+                d.p[i] = std::max(0.0, d.p[i] - qi);
+                rest += d.p[i];
+            }
+            if (rest > 1e-12)
+                for (double& x : d.p) x /= rest;
+            else
+                d = whole;
+        }
+        o[n] = host_draw(d, next_u());
+        ++n;
+        break;
+    }
+    if (used_u) *used_u = at;
+    if (at > nu) {
+        fail("accept_sampled: more uniforms were needed than given");
+        return -1;
+    }
+    return n;
 }
 
 // ---------------------------------------------------------------- GGUF ingestion (host_gguf.h)

@@ -60,6 +60,11 @@ def load():
         "fnx_o_lookup_drafts": (i, [vp, i, i, i, i, vp, vp]),
         "fnx_o_lookup_fixed": (i, [vp, i, i, i, i, vp]),
         "fnx_o_accept_greedy": (i, [vp, vp, i]),
+        "fnx_o_top_tokens": (C.c_uint, [vp, i, i, i, vp, vp, vp, i, vp, vp, vp, vp, vp, vp, vp]),
+        "fnx_o_penalize_row": (None, [vp, i, vp, vp]),
+        "fnx_o_make_dist": (i, [vp, vp, i, f, f, f, i, vp, vp]),
+        "fnx_o_draw": (i, [vp, vp, i, C.c_double]),
+        "fnx_o_accept_sampled": (i, [vp, vp, i, i, vp, f, f, f, i, vp, vp, vp, i, vp, vp, vp]),
         "fnx_o_pf_jobs": (i, [vp, i, i, i, i, vp, vp, vp]),
         "fnx_o_moe_verify_layer": (None, [vp, vp, i, vp, vp, vp, vp, vp, i]),
         "fnx_o_iq3s_dequant_f16": (None, [vp, sz, vp]),
