@@ -73,7 +73,8 @@ def test_combine_add_norm_q8_equals_combine_then_add_norm(dev, oracle, T, n, top
     assert int(np.count_nonzero(xq != want_q)) == 0
 
 
-@pytest.mark.parametrize("rows,cols,T", [(37, 1024, 3), (1000, 2048, 16), (2048, 4096, 16), (513, 256, 5), (8192, 2048, 1)])
+@pytest.mark.parametrize("rows,cols,T", [(37, 1024, 3), (1000, 2048, 16), (2048, 4096, 16), (513, 256, 5), (8192, 2048, 1),
+                                         (151936, 2048, 16)])   # the last: benchmark config 4's output head
 def test_q8s_gemv_bit_exact(dev, oracle, rows, cols, T):
     print(f"case q8s_gemv rows={rows} cols={cols} T={T}", flush=True)
     rng = np.random.default_rng(810 + rows)
@@ -115,7 +116,8 @@ def test_attn_prep_append(dev, oracle, nq, nkv, T, pos0, rope):
     assert np.array_equal(gkc[:pos0], kc0[:pos0]) and np.array_equal(gkc[pos0 + T:], kc0[pos0 + T:]), "only the window's rows are written"
 
 
-@pytest.mark.parametrize("nq,nkv,T,pos0", [(4, 2, 3, 37), (16, 2, 16, 3000), (16, 2, 16, 0), (8, 1, 5, 511), (2, 2, 1, 64), (16, 2, 16, 1017), (16, 2, 7, 500)])
+@pytest.mark.parametrize("nq,nkv,T,pos0", [(4, 2, 3, 37), (16, 2, 16, 3000), (16, 2, 16, 0), (8, 1, 5, 511), (2, 2, 1, 64), (16, 2, 16, 1017), (16, 2, 7, 500),
+                                           (16, 2, 16, 32752)])   # the last: benchmark config 4's window at the end of a 32,768-position cache
 def test_attn_matches_oracle(dev, oracle, nq, nkv, T, pos0):
     print(f"case attn nq={nq} nkv={nkv} T={T} pos0={pos0}", flush=True)
     rng = np.random.default_rng(830 + nq + pos0)
