@@ -373,7 +373,8 @@ __device__ __forceinline__ void job_units(const uint32_t* __restrict__ tab, cons
     }
 }
 
-// WIDE: jobs of many rows go four tokens at a time (fewer units in flight to stay within the registers); the narrow
+// WIDE: jobs of many rows go up to sixteen tokens at a time in the unit64 layout (four with raw blocks, fewer units in
+// flight to stay within the registers); the narrow
 // variant takes one or two tokens a pass, which is what a verify window's routed jobs have (1.15 rows on average)
 template <int SBR, bool WIDE>
 __device__ __forceinline__ void job_range(const uint32_t* tab, const uint8_t* we, const RowsArgs& a, int ua, int ub, const fnx_job* jb,

@@ -183,7 +183,13 @@ __device__ __forceinline__ void packed_range(const uint32_t* tab, const uint8_t*
     for (int t0 = 0; t0 < n;) {
         const int nt = n - t0;
         packed_first(we, ua, ub, cur);
-        if (WIDE && nt >= 4) {
+        if (WIDE && nt >= 16) {
+            packed_units<SBR, 16>(tab, we, ua, ub, cur, JobPrep<SBR, 16>{jb, t0, y, out, out_stride});
+            t0 += 16;
+        } else if (WIDE && nt >= 8) {
+            packed_units<SBR, 8>(tab, we, ua, ub, cur, JobPrep<SBR, 8>{jb, t0, y, out, out_stride});
+            t0 += 8;
+        } else if (WIDE && nt >= 4) {
             packed_units<SBR, 4>(tab, we, ua, ub, cur, JobPrep<SBR, 4>{jb, t0, y, out, out_stride});
             t0 += 4;
         } else if (WIDE && nt == 3) {
