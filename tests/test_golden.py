@@ -1,5 +1,6 @@
-"""The committed vectors (tests/golden/verify_path.npz, made by tests/golden/make_fixtures.py) against the oracle
-(CPU) and against the device library (GPU)."""
+"""The committed vectors (tests/golden/verify_path.npz, made by tests/golden/make_fixtures.py; sampler_path.npz, made by
+tests/golden/make_sampler_fixtures.py) against the oracle (CPU), the library's host functions (CPU) and the device
+library (GPU)."""
 import os
 
 import numpy as np
@@ -58,3 +59,55 @@ def test_device_reproduces_the_fixtures():
         assert list(d) == list(G["lk_drafts"][G["lk_doff"][i]:G["lk_doff"][i + 1]]) and mm == m
     for i in range(12):
         assert dev.accept(G["acc_rows"][i], G["acc_o"][i]) == int(G["acc_n"][i])
+
+
+S = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "sampler_path.npz"))
+
+
+def sampler_lists():
+    """the fixture's penalty and bias lists as test_oracle_sampler's helpers take them"""
+    pen = [[(int(S["tk_pen_tok"][t, i]), int(S["tk_pen_cnt"][t, i])) for i in range(int(S["tk_pen_n"][t]))] for t in range(3)]
+    par = [tuple(float(v) for v in S["tk_par"][t]) for t in range(3)]
+    off = np.concatenate([[0], np.cumsum(S["tk_bias_n"])])
+    bias = [[(int(S["tk_bias_tok"][i]), float(S["tk_bias_val"][i])) for i in range(off[t], off[t + 1])] for t in range(3)]
+    return pen, par, bias
+
+
+def test_oracle_and_host_sampler_reproduce_the_fixtures(oracle):
+    import ctypes as C
+    from test_oracle_sampler import o_accept, o_dist, o_top_tokens
+    pen, par, bias = sampler_lists()
+    ov, oi, L, err = o_top_tokens(oracle, S["tk_logits"], v0=100, pen=pen, par=par, bias=bias)
+    assert np.array_equal(oi, S["tk_out_i"]) and np.array_equal(ov.view(np.uint32), S["tk_out_v"].view(np.uint32))
+    assert np.array_equal(L.view(np.uint32), S["tk_logits_after"].view(np.uint32)) and err == int(S["tk_err"][0]) == 16
+    t, top_p, min_p, top_k = (float(v) for v in S["sp_params"])
+    kw = dict(temperature=t, top_p=top_p, min_p=min_p, top_k=int(top_k))
+    ids, p = o_dist(oracle, S["tk_out_v"][0], S["tk_out_i"][0], **kw)
+    assert np.array_equal(ids, S["dist_ids"]) and np.array_equal(p, S["dist_p"])
+    pkg = fnx_gpu.package()
+    lib = pkg.lib()
+    s = pkg.Sampling(t, top_p, min_p, int(top_k))
+    hi, hp = np.zeros(64, np.int32), np.zeros(64, np.float64)
+    cv, ci = np.ascontiguousarray(S["tk_out_v"][:2]), np.ascontiguousarray(S["tk_out_i"][:2])
+    k = lib.fnx_make_dist(cv.ctypes.data, ci.ctypes.data, 64, C.byref(s), hi.ctypes.data, hp.ctypes.data)
+    assert k == len(S["dist_ids"]) and np.array_equal(hi[:k], S["dist_ids"]) and np.array_equal(hp[:k], S["dist_p"])
+    rows = np.ascontiguousarray(S["sp_rows"])
+    for i in range(8):
+        n, o, used = o_accept(oracle, cv, ci, rows, S["sp_u"][i], **kw)
+        want = (int(S["sp_n"][i]), [int(v) for v in S["sp_o"][i][:int(S["sp_n"][i])]], int(S["sp_used"][i]))
+        assert (n, o, used) == want
+        ho, hu = np.zeros(2, np.int32), C.c_int()
+        u = np.ascontiguousarray(S["sp_u"][i])
+        hn = lib.fnx_accept_sampled(cv.ctypes.data, ci.ctypes.data, 64, 2, rows.ctypes.data, C.byref(s), None, None, None, 1, u.ctypes.data, 3,
+                                    ho.ctypes.data, C.byref(hu))
+        assert (hn, [int(v) for v in ho[:hn]], hu.value) == want
+
+
+@pytest.mark.gpu
+def test_device_reproduces_the_sampler_fixtures():
+    from test_gpu_sampler import d_top_tokens
+    dev = fnx_gpu.Dev()
+    pen, par, bias = sampler_lists()
+    ov, oi, L, err = d_top_tokens(dev, S["tk_logits"], v0=100, pen=pen, par=par, bias=bias)
+    assert np.array_equal(oi, S["tk_out_i"]) and np.array_equal(ov.view(np.uint32), S["tk_out_v"].view(np.uint32))
+    assert np.array_equal(L.view(np.uint32), S["tk_logits_after"].view(np.uint32)) and err == 16
