@@ -52,9 +52,13 @@ typedef struct fnx_bigjob {
 /* model.hpp:84-94 (DW) without the split-Q8_0 twin, which this path does not use */
 typedef struct fnx_dw {
     const void* p;          /* raw ggml blocks, row-major over output rows */
-    uint32_t type;          /* FNX_T_IQ3_S (raw ggml blocks) or FNX_T_IQ3S_UNIT64 (after fnx_iq3s_repack) */
+    uint32_t type;          /* FNX_T_IQ3_S (raw ggml blocks) or FNX_T_IQ3S_UNIT64 (after fnx_iq3s_repack); the decode
+                             * operators (fnx_mmvq, fnx_moe_gate_up, fnx_moe_down, and fnx_moe_verify_layer operator by
+                             * operator) also take ggml's Q4_0 (2), Q8_0 (8), Q4_K (12), Q5_K (13) and IQ4_NL (20) rows, the
+                             * other types of kernels.cu:2454-2471 that the reference's host code can decode; the
+                             * prompt path's grouped GEMM and the five-launch window are IQ3_S only */
     int n_in, n_out;        /* columns, rows */
-    size_t row_bytes;       /* n_in / 256 * 110 */
+    size_t row_bytes;       /* n_in / 256 * 110 for IQ3_S; whole blocks of the type otherwise */
     const void* const* ep;  /* optional device table: expert e's matrix; null: expert e at p + e * stride */
 } fnx_dw;
 

@@ -495,6 +495,134 @@ unsigned fnx_o_argmax(const float* logits, int rows, int T, int v0, float* best_
     return err;
 }
 
+/* ---------------------------------------------------------------- other expert types at the boundary (kernels.cu:2454-2471)
+ * Decoders as tensor_convert.hpp:152-265 dequantises the types (the reference's own host code; pinned against it through
+ * oracle/_ref). The dot with q8_1 rows is ggml's vec_dot_<type>_q8_1 (ggml-cuda/vecdotq.cuh of llama.cpp @
+ * 3cf03257f219afbe7334045ff7c6a06ac68c627d, third_party/ggml/VERSION.txt - a fetched dependency, not in the tree):
+ * restated from its published form per 32 values; its per-thread split of a block and its warp order cannot be pinned, so
+ * the sums here run in this build's order (lane l of 64 takes sub-blocks l, l + 64, ...; then the xor butterfly). */
+#define T_Q4_0 2u
+#define T_Q8_0 8u
+#define T_Q4_K 12u
+#define T_Q5_K 13u
+#define T_IQ4_NL 20u
+static const int8_t KV_IQ4NL[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+int fnx_o_type_block(uint32_t type, int* values, int* bytes) {
+    switch (type) {
+        case T_Q4_0: *values = 32; *bytes = 18; return 0;
+        case T_Q8_0: *values = 32; *bytes = 34; return 0;
+        case T_IQ4_NL: *values = 32; *bytes = 18; return 0;
+        case T_Q4_K: *values = 256; *bytes = 144; return 0;
+        case T_Q5_K: *values = 256; *bytes = 176; return 0;
+    }
+    return 1;
+}
+/* get_scale_min_k4 (ggml; tensor_convert.hpp scale_min_k4): sub-block j's 6-bit scale and min out of the 12 bytes */
+static void k4_scale_min(int j, const uint8_t* q, int* sc, int* m) {
+    if (j < 4) {
+        *sc = q[j] & 63;
+        *m = q[j + 4] & 63;
+    } else {
+        *sc = (q[j + 4] & 0xF) | ((q[j - 4] >> 6) << 4);
+        *m = (q[j + 4] >> 4) | ((q[j] >> 6) << 4);
+    }
+}
+/* sub-block kb (32 values) of a row: its integers q[32] with value = scale * q - offset */
+typedef struct {
+    int q[32];
+    float d, dmin; /* the block's scales as floats (dmin: K-quants only) */
+    int sc, m;     /* K-quants: the sub-block's 6-bit scale and min */
+} sub_t;
+static void sub_decode(uint32_t type, const uint8_t* row, int kb, sub_t* o) {
+    uint16_t h;
+    o->dmin = 0.f;
+    o->sc = 1;
+    o->m = 0;
+    if (type == T_Q8_0) {
+        const uint8_t* p = row + (size_t) kb * 34;
+        memcpy(&h, p, 2);
+        o->d = fnx_o_h2f(h);
+        for (int j = 0; j < 32; ++j) o->q[j] = (int8_t) p[2 + j];
+    } else if (type == T_Q4_0 || type == T_IQ4_NL) {
+        const uint8_t* p = row + (size_t) kb * 18;
+        memcpy(&h, p, 2);
+        o->d = fnx_o_h2f(h);
+        for (int j = 0; j < 16; ++j) {
+            const int lo = p[2 + j] & 0xF, hi = p[2 + j] >> 4;
+            o->q[j] = type == T_Q4_0 ? lo : KV_IQ4NL[lo];      /* Q4_0: the - 8 is applied through the q8_1 sum */
+            o->q[j + 16] = type == T_Q4_0 ? hi : KV_IQ4NL[hi];
+        }
+    } else { /* Q4_K, Q5_K: super-block kb / 8, sub-block kb % 8 */
+        const int sb = kb & 7, five = type == T_Q5_K;
+        const uint8_t* p = row + (size_t) (kb >> 3) * (five ? 176 : 144);
+        memcpy(&h, p, 2);
+        o->d = fnx_o_h2f(h);
+        memcpy(&h, p + 2, 2);
+        o->dmin = fnx_o_h2f(h);
+        k4_scale_min(sb, p + 4, &o->sc, &o->m);
+        const uint8_t *qh = p + 16, *ql = p + (five ? 48 : 16) + 32 * (sb >> 1);
+        for (int l = 0; l < 32; ++l) {
+            int v = (sb & 1) ? ql[l] >> 4 : ql[l] & 0xF;
+            if (five && ((qh[l] >> sb) & 1)) v += 16;
+            o->q[l] = v;
+        }
+    }
+}
+void fnx_o_dequant(uint32_t type, const uint8_t* src, size_t n, float* y) {
+    for (size_t kb = 0; kb < n / 32; ++kb) {
+        sub_t s;
+        sub_decode(type, src, (int) kb, &s);
+        for (int j = 0; j < 32; ++j) {
+            if (type == T_Q4_0) y[kb * 32 + j] = s.d * (float) (s.q[j] - 8);
+            else if (type == T_Q4_K || type == T_Q5_K) y[kb * 32 + j] = (s.d * (float) s.sc) * (float) s.q[j] - s.dmin * (float) s.m;
+            else y[kb * 32 + j] = s.d * (float) s.q[j];
+        }
+    }
+}
+/* one sub-block's term of the dot with a q8_1 block {half d; half sum; int8 qs[32]} */
+float fnx_o_vec_dot_type(uint32_t type, const uint8_t* row, int kb, const uint8_t* q8) {
+    sub_t s;
+    uint16_t h;
+    sub_decode(type, row, kb, &s);
+    memcpy(&h, q8, 2);
+    const float dx = fnx_o_h2f(h);
+    memcpy(&h, q8 + 2, 2);
+    const float sx = fnx_o_h2f(h);
+    int dot = 0, qsum = 0;
+    for (int j = 0; j < 32; ++j) {
+        const int x = (int8_t) q8[4 + j];
+        dot += s.q[j] * x;
+        qsum += x;
+    }
+    if (type == T_Q4_0) return s.d * ((float) dot * dx - 8.0f * sx);                      /* vec_dot_q4_0_q8_1_impl */
+    if (type == T_Q4_K || type == T_Q5_K)                                               /* vec_dot_q4_K_q8_1_impl_vmmq */
+        return s.d * (dx * (float) (dot * s.sc)) - s.dmin * (dx * (float) (qsum * s.m));
+    return (s.d * dx) * (float) dot;                                                      /* vec_dot_q8_0_q8_1_impl, vec_dot_iq4_nl_q8_1 */
+}
+void fnx_o_mmvq_type(uint32_t type, const uint8_t* w, size_t w_stride, int nrows, int ncols, const fnx_o_job* jobs, int njobs, const uint8_t* y,
+                     float* out, int out_stride, int threads) {
+    int values, bytes;
+    if (fnx_o_type_block(type, &values, &bytes)) return;
+    const int sbr = ncols / 32;
+    const size_t row_bytes = (size_t) (ncols / values) * bytes;
+    (void) threads;
+#pragma omp parallel for collapse(2) num_threads(threads > 0 ? threads : 1)
+    for (int ji = 0; ji < njobs; ++ji)
+        for (int r = 0; r < nrows; ++r) {
+            const fnx_o_job* jb = jobs + ji;
+            const uint8_t* row = w + (size_t) jb->w * w_stride + (size_t) r * row_bytes;
+            for (int t = 0; t < jb->n; ++t) {
+                float lanes[64];
+                for (int l = 0; l < 64; ++l) {
+                    float acc = 0.f;
+                    for (int kb = l; kb < sbr; kb += 64) acc += fnx_o_vec_dot_type(type, row, kb, y + ((size_t) jb->y[t] * sbr + kb) * Q8_1_BLOCK);
+                    lanes[l] = acc;
+                }
+                out[(size_t) jb->out[t] * out_stride + r] = butterfly_sum(lanes, 64);
+            }
+        }
+}
+
 /* ---------------------------------------------------------------- the sampler's candidates (topk.cuh, kernels.hpp:434-447) */
 static int cmp_desc_u64(const void* a, const void* b) {
     const uint64_t x = *(const uint64_t*) a, y = *(const uint64_t*) b;

@@ -16,6 +16,13 @@
  *             (-key, id) incl. wide ties and signed zeros; penalties as a numpy f32 closed form), make_dist (numpy
  *             vectorised softmax / cumulative cut, limiting cases), accept_sampled (the window's first token is
  *             distributed as the target p whatever q is: exact measure over a grid of uniforms; fixed-draft closed form).
+ *   pinned:   the other expert types' decoders (fnx_o_dequant: Q4_0, Q8_0, Q4_K, Q5_K, IQ4_NL) against the reference's
+ *             own conv::dequantize through oracle/_ref and against numpy restatements; their dots (fnx_o_vec_dot_type)
+ *             against the decoded values times the q8_1 values in f64 (the Q4_0 form through the block's sum field to
+ *             within that field's f16 rounding).
+ *   parity unpinned: the float-operation order of ggml's vec_dot_<type>_q8_1 for those types (third-party, fetched at
+ *             build time, absent from the tree): the per-32-value terms follow its published form, the sums this build's
+ *             own fixed order.
  *   parity unpinned: fnx_o_iq3s_quantize_row (the encoder). ggml's quantize_row_iq3_s is not in the reference tree
  *             (third_party/ggml holds only a commit hash) and nothing in the reference calls or tests it. The encoder
  *             here is this build's own; parity of the path is defined from the quantised bytes onward.
@@ -99,6 +106,12 @@ int fnx_o_lookup_drafts(const int* ctx, int n_ctx, int key_n, int lk, int d1, in
 int fnx_o_lookup_fixed(const int* ctx, int n_ctx, int key_n, int lk, int d1, int* out);
 /* session.cpp:573 */
 int fnx_o_accept_greedy(const int* rows, const int* o, int R);
+/* other expert types at the boundary (kernels.cu:2454-2471): Q4_0 (2), Q8_0 (8), Q4_K (12), Q5_K (13), IQ4_NL (20) */
+int fnx_o_type_block(uint32_t type, int* values, int* bytes);
+void fnx_o_dequant(uint32_t type, const uint8_t* src, size_t n, float* y);
+float fnx_o_vec_dot_type(uint32_t type, const uint8_t* row, int kb, const uint8_t* q8);
+void fnx_o_mmvq_type(uint32_t type, const uint8_t* w, size_t w_stride, int nrows, int ncols, const fnx_o_job* jobs, int njobs, const uint8_t* y,
+                     float* out, int out_stride, int threads);
 /* kernels.hpp:434-447, topk.cuh: the sampler's candidates (64 a row), logits changed in place; returns the err bits */
 unsigned fnx_o_top_tokens(float* logits, int n, int T, int v0, const int* pen_tok, const int* pen_cnt, const int* pen_n, int pen_stride,
                           const float* pen_par, const int* bias_tok, const float* bias_val, const int* bias_off, const int* bias_n, float* out_v,

@@ -437,6 +437,7 @@ __global__ void __launch_bounds__(512) k_iq3s_jobs(const RowsArgs a) {
 #include "k_decoder.h"
 #include "k_round.h"
 #include "k_sampler.h"
+#include "k_qtypes.h"
 namespace fnx {
 
 // any other row length (a multiple of 256): a wave per (row, job), sub-blocks dealt round-robin to the lanes, the
@@ -688,8 +689,30 @@ static int cu_count() {
 static int rows_launch(const fnx_dw* W, size_t w_stride, const fnx_job* jobs, const int* njobs, int njobs_max, const void* y, float* out,
                        int out_stride, void* st, const char* who, bool wide = false, int y_rows = 0) {
     if (!W || !jobs || !out) return fail(std::string(who) + ": null argument");
+    if (W->type == QT_Q4_0 || W->type == QT_Q8_0 || W->type == QT_IQ4_NL || W->type == QT_Q4_K || W->type == QT_Q5_K) {
+        // the other types of kernels.cu:2454-2471 that the reference's own host code can decode (k_qtypes.h)
+        gguf::BlockShape bs{};
+        gguf::block_shape(W->type, bs);
+        if (W->n_in <= 0 || W->n_in % bs.values || W->n_out <= 0) return fail(std::string(who) + ": shape does not fit the type's blocks");
+        if (W->row_bytes != (size_t) (W->n_in / bs.values) * (size_t) bs.bytes) return fail(std::string(who) + ": row_bytes does not match n_in");
+        if (njobs_max <= 0) return fail(std::string(who) + ": njobs_max must be positive");
+        if (!W->p && !W->ep) return fail(std::string(who) + ": no weights");
+        const QtArgs q{(const uint8_t*) W->p, w_stride, (const uint8_t* const*) W->ep, W->row_bytes, W->n_out, W->n_in, jobs, njobs, njobs_max,
+                       (const uint8_t*) y, out, out_stride};
+        const dim3 grid((W->n_out + 3) / 4, njobs_max);
+        hipStream_t s = (hipStream_t) st;
+        switch (W->type) {
+            case QT_Q4_0: k_qt_jobs<QT_Q4_0><<<grid, 256, 0, s>>>(q); break;
+            case QT_Q8_0: k_qt_jobs<QT_Q8_0><<<grid, 256, 0, s>>>(q); break;
+            case QT_IQ4_NL: k_qt_jobs<QT_IQ4_NL><<<grid, 256, 0, s>>>(q); break;
+            case QT_Q4_K: k_qt_jobs<QT_Q4_K><<<grid, 256, 0, s>>>(q); break;
+            default: k_qt_jobs<QT_Q5_K><<<grid, 256, 0, s>>>(q); break;
+        }
+        return launch_status(who);
+    }
     if (W->type != FNX_T_IQ3_S && W->type != FNX_T_IQ3S_UNIT64)
-        return fail(std::string(who) + ": expert type " + std::to_string(W->type) + " not handled (IQ3_S only)");
+        return fail(std::string(who) + ": expert type " + std::to_string(W->type) +
+                    " not handled (IQ3_S, and Q4_0, Q8_0, IQ4_NL, Q4_K, Q5_K through the plain path)");
     if (W->n_in <= 0 || W->n_in % 256 || W->n_out <= 0) return fail(std::string(who) + ": shape does not fit IQ3_S super-blocks");
     if (W->row_bytes != (size_t) (W->n_in / 256) * FNX_IQ3S_BLOCK) return fail(std::string(who) + ": row_bytes does not match n_in");
     if (njobs_max <= 0) return fail(std::string(who) + ": njobs_max must be positive");

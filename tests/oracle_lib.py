@@ -60,6 +60,10 @@ def load():
         "fnx_o_lookup_drafts": (i, [vp, i, i, i, i, vp, vp]),
         "fnx_o_lookup_fixed": (i, [vp, i, i, i, i, vp]),
         "fnx_o_accept_greedy": (i, [vp, vp, i]),
+        "fnx_o_type_block": (i, [C.c_uint32, vp, vp]),
+        "fnx_o_dequant": (None, [C.c_uint32, vp, sz, vp]),
+        "fnx_o_vec_dot_type": (f, [C.c_uint32, vp, i, vp]),
+        "fnx_o_mmvq_type": (None, [C.c_uint32, vp, sz, i, i, vp, i, vp, vp, i, i]),
         "fnx_o_top_tokens": (C.c_uint, [vp, i, i, i, vp, vp, vp, i, vp, vp, vp, vp, vp, vp, vp]),
         "fnx_o_penalize_row": (None, [vp, i, vp, vp]),
         "fnx_o_make_dist": (i, [vp, vp, i, f, f, f, i, vp, vp]),

@@ -44,9 +44,11 @@ def test_bad_arguments_are_refused_with_a_message():
     assert lib.fnx_quantize_q8_1(None, buf, 32, 1, None) != 0
     assert lib.fnx_gemv_f32(buf, buf, buf, 4, 100, 1, None) != 0
     assert lib.fnx_gemv_f32(buf, buf, buf, 4, 256, 0, None) != 0 and b"T out of range" in lib.fnx_last_error()
-    bad = pkg.DW(buf, 8, 2048, 16, 880, None)               # Q8_0 experts are not handled
+    bad = pkg.DW(buf, 14, 2048, 16, 880, None)              # Q6_K experts are not handled
     assert lib.fnx_moe_gate_up(C.byref(bad), 0, buf, None, 10, buf, buf, 10, None) != 0
     assert b"IQ3_S" in lib.fnx_last_error()
+    bad = pkg.DW(buf, 8, 2048, 16, 880, None)               # Q8_0 rows of 2048 values take 2,176 bytes
+    assert lib.fnx_moe_gate_up(C.byref(bad), 0, buf, None, 10, buf, buf, 10, None) != 0 and b"row_bytes" in lib.fnx_last_error()
     bad = pkg.DW(buf, pkg.T_IQ3_S, 2048, 16, 881, None)     # row_bytes must be n_in / 256 * 110
     assert lib.fnx_mmvq(C.byref(bad), 0, buf, None, 1, buf, buf, 16, None) != 0
     assert lib.fnx_route(buf, 8, 1, 2000, 10, buf, buf, buf, buf, buf, None) != 0
