@@ -405,9 +405,10 @@ int fnx_gguf_expert_rows2(const fnx_gguf_tensor* gate, const fnx_gguf_tensor* up
 int fnx_gguf_expert_cols(const fnx_gguf_tensor* down, int c0, int c1, void* dst, size_t dst_bytes, fnx_dw* w, size_t* stride, size_t* bytes);
 /* one layer's MoE block from "blk.<layer>.": ffn_gate_inp(.weight) + ffn_gate_inp_shexp -> router rows (F32 or BF16 in the
  * file, f32 on the device); ffn_gate_exps / ffn_up_exps rows [ff0, ff1) -> gate|up; ffn_down_exps columns [ff0, ff1) ->
- * down; the _shexp tensors likewise (model.cpp:988-989, 1063-1068 without the card split's other half). Experts must be
- * IQ3_S; they are uploaded into the caller's device buffers and re-laid there (fnx_iq3s_repack), so *L is ready for
- * fnx_moe_verify_layer / fnx_moe_prefill_layer. The upload is synchronous; the re-laying runs on st.
+ * down; the _shexp tensors likewise (model.cpp:988-989, 1063-1068 without the card split's other half). Experts in
+ * IQ3_S are uploaded into the caller's device buffers and re-laid there (fnx_iq3s_repack), so *L is ready for
+ * fnx_moe_verify_layer / fnx_moe_prefill_layer; a layer with any tensor in Q4_0, Q8_0, IQ4_NL, Q4_K or Q5_K is left as the
+ * file has it (fnx_moe_verify_layer then runs operator by operator; the prompt path needs IQ3_S). The upload is synchronous; the re-laying runs on st.
  * topk <= 0: taken from "<general.architecture>.expert_used_count". */
 typedef struct fnx_moe_bufs {
     void *router, *gu, *down, *sh_gu, *sh_down;   /* device */

@@ -1623,7 +1623,9 @@ MoeTensors moe_tensors(const fnx_gguf* g, int layer) {
     MoeTensors m{get("ffn_gate_inp.weight"), get("ffn_gate_inp_shexp.weight"), get("ffn_gate_exps.weight"), get("ffn_up_exps.weight"),
                  get("ffn_down_exps.weight"), get("ffn_gate_shexp.weight"), get("ffn_up_shexp.weight"), get("ffn_down_shexp.weight")};
     for (const fnx_gguf_tensor* t : {&m.ge, &m.ue, &m.de, &m.gsh, &m.ush, &m.dsh})
-        if (t->type != gguf::T_IQ3_S) throw std::runtime_error(gguf::nm(*t) + ": ggml type " + std::to_string(t->type) + ", this path reads IQ3_S experts");
+        if (t->type != gguf::T_IQ3_S && t->type != QT_Q4_0 && t->type != QT_Q8_0 && t->type != QT_IQ4_NL && t->type != QT_Q4_K && t->type != QT_Q5_K)
+            throw std::runtime_error(gguf::nm(*t) + ": ggml type " + std::to_string(t->type) +
+                                     ", this path reads experts in IQ3_S (and Q4_0, Q8_0, IQ4_NL, Q4_K, Q5_K through its plain operators)");
     if (m.gi.ne[0] != m.ge.ne[0] || m.gi.ne[1] != m.ge.ne[2] || m.gs.ne[1] != 1 || m.de.ne[1] != m.ge.ne[0] || m.de.ne[0] != m.ge.ne[1] ||
         m.de.ne[2] != m.ge.ne[2] || m.gsh.ne[0] != m.ge.ne[0] || m.dsh.ne[1] != m.ge.ne[0] || m.dsh.ne[0] != m.gsh.ne[1] || m.gsh.ne[2] != 1 ||
         m.dsh.ne[2] != 1)
@@ -1671,9 +1673,12 @@ int fnx_gguf_load_moe_layer(const fnx_gguf* g, int layer, int ff0, int ff1, int 
         const auto upload = [&](void* d, size_t n, const char* what) {
             if (hipMemcpy(d, host.data(), n, hipMemcpyHostToDevice) != hipSuccess) throw std::runtime_error(std::string("gguf_load_moe_layer: upload of ") + what + " failed");
         };
-        const auto relay = [&](fnx_dw& w, void* d, size_t n) {   // raw ggml blocks -> the unit64 layout, in place
-            if (fnx_iq3s_repack(d, d, n / FNX_IQ3S_BLOCK * 256, st)) throw std::runtime_error(fnx_last_error());
+        // IQ3_S: raw ggml blocks -> the unit64 layout, in place; other types stay as the file has them
+        const bool all_iq3s = m.ge.type == gguf::T_IQ3_S && m.de.type == gguf::T_IQ3_S && m.gsh.type == gguf::T_IQ3_S && m.dsh.type == gguf::T_IQ3_S;
+        const auto relay = [&](fnx_dw& w, void* d, size_t n) {
             w.p = d;
+            if (!all_iq3s) return;   // the window's fast form needs all four; operator by operator raw blocks do as well
+            if (fnx_iq3s_repack(d, d, n / FNX_IQ3S_BLOCK * 256, st)) throw std::runtime_error(fnx_last_error());
             w.type = FNX_T_IQ3S_UNIT64;
         };
         gguf::router_rows(m.gi, m.gs, reinterpret_cast<float*>(host.data()));

@@ -68,3 +68,75 @@ def test_layer_from_gguf_matches_oracle(dev, oracle, tmp_path, router_type, ff0,
     assert np.array_equal(w["logits"].cpu().numpy().view(np.uint32), want["logits"].view(np.uint32)), "router logits bit-exact"
     assert np.array_equal(w["topi"].cpu().numpy(), want["topi"]) and int(w["njobs"][0].item()) == want["njobs"]
     assert rel_l2(out.cpu().numpy(), want["out"]) <= 1e-3
+
+
+def test_layer_with_other_expert_types_from_gguf(dev, oracle, tmp_path):
+    """Routed experts in Q4_K, the shared expert in Q8_0 (what a file with K-quant experts holds once its dense tensors
+    are Q8_0): loaded as the file has them, the window runs operator by operator; expected = the oracle's operators in
+    the reference's order (engine.cu:1569-1757)."""
+    import ctypes as C
+    import oracle_lib as ol
+    import qtype_blocks as qb
+    t, lib, pkg = dev.torch, dev.lib, dev.pkg
+    rng = np.random.default_rng(91)
+    n, ff, nexp, topk, T, layer = 512, 256, 6, 2, 5, 0
+    nbk = lambda rows, cols, qt: rows * cols // qb.SHAPE[qt][0]
+    gate, up = qb.random_blocks(rng, qb.Q4_K, nexp * nbk(ff, n, qb.Q4_K)), qb.random_blocks(rng, qb.Q4_K, nexp * nbk(ff, n, qb.Q4_K))
+    down = qb.random_blocks(rng, qb.Q4_K, nexp * nbk(n, ff, qb.Q4_K))
+    sgate, sup, sdown = (qb.random_blocks(rng, qb.Q8_0, nbk(r, c, qb.Q8_0)) for r, c in ((ff, n), (ff, n), (n, ff)))
+    router = (rng.standard_normal((nexp, n)) * 0.05).astype(np.float32)
+    srouter = (rng.standard_normal((1, n)) * 0.05).astype(np.float32)
+    b = "blk.0."
+    ts = [(b + "ffn_gate_inp.weight", gf.F32, [n, nexp], router.tobytes()), (b + "ffn_gate_inp_shexp.weight", gf.F32, [n, 1], srouter.tobytes()),
+          (b + "ffn_gate_exps.weight", qb.Q4_K, [n, ff, nexp], gate), (b + "ffn_up_exps.weight", qb.Q4_K, [n, ff, nexp], up),
+          (b + "ffn_down_exps.weight", qb.Q4_K, [ff, n, nexp], down), (b + "ffn_gate_shexp.weight", qb.Q8_0, [n, ff], sgate),
+          (b + "ffn_up_shexp.weight", qb.Q8_0, [n, ff], sup), (b + "ffn_down_shexp.weight", qb.Q8_0, [ff, n], sdown)]
+    path = gf.write(tmp_path / "mixed.gguf", ts)
+    print("case gguf layer with Q4_K experts and a Q8_0 shared expert", flush=True)
+    g = lib.fnx_gguf_open(path.encode())
+    assert g, lib.fnx_last_error()
+    z = pkg.MoeBufs()
+    dev.ok(lib.fnx_gguf_moe_layer_bytes(g, layer, 0, ff, C.byref(z)))
+    bufs = [dev.zeros(getattr(z, k + "_bytes"), t.uint8) for k in ("router", "gu", "down", "sh_gu", "sh_down")]
+    for k, bf in zip(("router", "gu", "down", "sh_gu", "sh_down"), bufs):
+        setattr(z, k, bf.data_ptr())
+    L = pkg.MoeLayer()
+    dev.ok(lib.fnx_gguf_load_moe_layer(g, layer, 0, ff, topk, C.byref(z), C.byref(L), dev.st()))
+    dev.sync()
+    lib.fnx_gguf_close(g)
+    assert (L.gu.type, L.down.type, L.sh_gu.type, L.sh_down.type) == (qb.Q4_K, qb.Q4_K, qb.Q8_0, qb.Q8_0)
+    gu_rb, dn_rb, sgu_rb, sdn_rb = n // 256 * 144, ff // 256 * 144, n // 32 * 34, ff // 32 * 34
+    gu_w = np.concatenate([gate.reshape(nexp, ff * gu_rb), up.reshape(nexp, ff * gu_rb)], axis=1).reshape(-1)
+    assert np.array_equal(bufs[1].cpu().numpy(), gu_w), "gate rows then up rows, expert by expert"
+    # the window
+    P = T * topk
+    w = dict(xq=dev.zeros(T * (n // 32) * 36, t.uint8), logits=dev.zeros((T, nexp + 1), t.float32), topi=dev.zeros((T, topk), t.int32),
+             topw=dev.zeros((T, topk), t.float32), jobs_gu=dev.zeros((P + 1) * 136, t.uint8), jobs_dn=dev.zeros((P + 1) * 136, t.uint8),
+             njobs=dev.zeros(2, t.int32), gu=dev.zeros((P + T, 2 * ff), t.float32), part=dev.zeros((P + T, n), t.float32))
+    ws = pkg.MoeWs(*(w[k].data_ptr() for k in ("xq", "logits", "topi", "topw", "jobs_gu", "jobs_dn", "njobs", "gu", "part")))
+    x = rng.standard_normal((T, n)).astype(np.float32)
+    dx, out = dev.up(x), dev.zeros((T, n), t.float32)
+    dev.ok(lib.fnx_moe_verify_layer(C.byref(L), dx.data_ptr(), T, out.data_ptr(), C.byref(ws), dev.st()))
+    dev.sync()
+    # the oracle's operators, in order
+    W = np.concatenate([router, srouter])
+    logits = oracle.gemv_f32(W, x)
+    topi, topw = oracle.topk_logits(logits, nexp, topk)
+    jg, jd = oracle.jobs(topi)
+    xq = oracle.quantize_q8_1(x)
+    gu = np.zeros((P + T, 2 * ff), np.float32)
+    mm = oracle.lib.fnx_o_mmvq_type
+    mm(qb.Q4_K, ol.ptr(gu_w), 2 * ff * gu_rb, 2 * ff, n, ol.ptr(np.ascontiguousarray(jg)), len(jg), ol.ptr(xq), ol.ptr(gu), 2 * ff, 8)
+    sh = np.zeros(1, dtype=fnx_gpu.JOB_DTYPE)
+    sh["n"][0] = T
+    sh["y"][0, :T], sh["out"][0, :T] = np.arange(T), P + np.arange(T)
+    sgu_w = np.concatenate([sgate, sup])
+    mm(qb.Q8_0, ol.ptr(sgu_w), 0, 2 * ff, n, ol.ptr(sh), 1, ol.ptr(xq), ol.ptr(gu), 2 * ff, 8)
+    hq = oracle.swiglu_stacked_q8_1(gu, ff)
+    part = np.zeros((P + T, n), np.float32)
+    mm(qb.Q4_K, ol.ptr(down), n * dn_rb, n, ff, ol.ptr(np.ascontiguousarray(jd)), len(jd), ol.ptr(hq), ol.ptr(part), n, 8)
+    sh["y"][0, :T] = P + np.arange(T)
+    mm(qb.Q8_0, ol.ptr(sdown), 0, n, ff, ol.ptr(sh), 1, ol.ptr(hq), ol.ptr(part), n, 8)
+    want = oracle.moe_combine(part[:P], topw, part[P:], logits[:, nexp])
+    assert np.array_equal(w["topi"].cpu().numpy(), topi)
+    assert rel_l2(out.cpu().numpy(), want) <= 1e-3
