@@ -10,6 +10,7 @@
 #include <cstdint>
 #include <stdexcept>
 #include <string>
+#include <utility>
 #include <vector>
 
 #include "../../include/fnx_mi355x.h"
@@ -125,5 +126,87 @@ inline void attn(const float* qg, const uint16_t* kc, const uint16_t* vc, float*
                  float* scratch, void* st) {
     ck(fnx_attn(qg, kc, vc, out, nq, nkv, pos0, T, max_ctx, scratch, st));
 }
+
+// ---- the sampler (kernels.hpp:434-447; session.hpp:17-26, 41-48)
+constexpr int TOPK_N = FNX_TOPK_N;
+inline void penalize_row(float* row, int n, const int* pen, const float* par, void* st) { ck(fnx_penalize_row(row, n, pen, par, st)); }
+inline void top_tokens(float* logits, int n, int T, int v0, const int* pen_tok, const int* pen_cnt, const int* pen_n, int pen_stride,
+                       const float* pen_par, const int* bias_tok, const float* bias_val, const int* bias_off, const int* bias_n, float* out_v,
+                       int* out_i, unsigned* err, void* st) {
+    ck(fnx_top_tokens(logits, n, T, v0, pen_tok, pen_cnt, pen_n, pen_stride, pen_par, bias_tok, bias_val, bias_off, bias_n, out_v, out_i, err, st));
+}
+struct Sampling {   // the values of session.hpp:17-26 a distribution is made from
+    float temperature = 1.f, top_p = 1.f, min_p = 0.f;
+    int top_k = 0;
+};
+struct Dist {
+    std::vector<int> ids;
+    std::vector<double> p;
+    double prob(int id) const {
+        for (size_t i = 0; i < ids.size(); ++i)
+            if (ids[i] == id) return p[i];
+        return 0.0;
+    }
+};
+inline Dist make_dist(const std::vector<std::pair<float, int>>& cand, const Sampling& s) {
+    std::vector<float> v(cand.size());
+    std::vector<int> id(cand.size());
+    for (size_t i = 0; i < cand.size(); ++i) {
+        v[i] = cand[i].first;
+        id[i] = cand[i].second;
+    }
+    const fnx_sampling fs{s.temperature, s.top_p, s.min_p, s.top_k};
+    Dist d;
+    d.ids.resize(cand.size());
+    d.p.resize(cand.size());
+    const int k = fnx_make_dist(v.data(), id.data(), (int) cand.size(), &fs, d.ids.data(), d.p.data());
+    if (k < 0) throw std::runtime_error(fnx_last_error());
+    d.ids.resize((size_t) k);
+    d.p.resize((size_t) k);
+    return d;
+}
+inline int draw(const Dist& d, double u) {
+    const int t = fnx_draw(d.ids.data(), d.p.data(), (int) d.ids.size(), u);
+    if (t < 0) throw std::runtime_error(fnx_last_error());
+    return t;
+}
+
+// ---- GGUF files (gguf.hpp:25-45): the handle closes with the object
+class Gguf {
+public:
+    explicit Gguf(const std::string& first_shard) : g_(fnx_gguf_open(first_shard.c_str())) {
+        if (!g_) throw std::runtime_error(fnx_last_error());
+    }
+    ~Gguf() { fnx_gguf_close(g_); }
+    Gguf(const Gguf&) = delete;
+    Gguf& operator=(const Gguf&) = delete;
+    fnx_gguf_tensor t(const std::string& name) const {   // throws when missing
+        fnx_gguf_tensor out;
+        ck(fnx_gguf_find(g_, name.c_str(), &out));
+        return out;
+    }
+    bool has_key(const std::string& key) const { return fnx_gguf_key_type(g_, key.c_str()) >= 0; }
+    int64_t i(const std::string& key) const {
+        int64_t v;
+        ck(fnx_gguf_int(g_, key.c_str(), &v));
+        return v;
+    }
+    double num(const std::string& key) const {
+        double v;
+        ck(fnx_gguf_num(g_, key.c_str(), &v));
+        return v;
+    }
+    std::string s(const std::string& key) const {
+        const char* v = fnx_gguf_str(g_, key.c_str());
+        if (!v) throw std::runtime_error("gguf: no string key " + key);
+        return v;
+    }
+    int shards() const { return fnx_gguf_shards(g_); }
+    int count() const { return fnx_gguf_count(g_); }
+    const fnx_gguf* handle() const { return g_; }
+
+private:
+    fnx_gguf* g_;
+};
 
 }  // namespace fnx
