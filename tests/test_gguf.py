@@ -205,3 +205,36 @@ def test_expert_slices_equal_numpy(lib, tmp_path):
                                                                                          per(2 * ff_total, n), per(n, ff_total))
     assert lib.fnx_gguf_moe_layer_bytes(g, 4, 0, ff_total, C.byref(z)) != 0 and b"no tensor blk.4." in lib.fnx_last_error()
     lib.fnx_gguf_close(g)
+
+
+def test_cut_and_corrupted_headers_never_read_out_of_bounds(lib, tmp_path):
+    # a valid layer file cut short at many lengths and with random bytes of its header changed: refused with a message, or,
+    # where the damage left a header that still adds up, every tensor's bytes can be read where the reader says they are
+    pkg = fnx_gpu.package()
+    rng = np.random.default_rng(17)
+    ts, _ = gf.moe_layer_tensors(rng, 0, 512, 256, 3, fnx_gpu.random_iq3s)
+    full = gf.build(ts, keys=[gf.kv("general.architecture", gf.STR, "q"), gf.kv("q.arr", gf.ARR, [1, 2, 3], gf.I32V),
+                              gf.kv("q.names", gf.ARR, ["a", "bc"], gf.STR)])
+    variants = [full[:cut] for cut in range(1, 900, 9)]
+    for _ in range(120):
+        b = bytearray(full)
+        for _ in range(3):
+            b[int(rng.integers(4, 800))] = int(rng.integers(0, 256))
+        variants.append(bytes(b))
+    p = tmp_path / "v.gguf"
+    refused = 0
+    for v in variants:
+        p.write_bytes(v)
+        g = lib.fnx_gguf_open(str(p).encode())
+        if not g:
+            assert lib.fnx_last_error().startswith(b"gguf:")
+            refused += 1
+            continue
+        for i in range(lib.fnx_gguf_count(g)):
+            t = pkg.GgufTensor()
+            assert lib.fnx_gguf_at(g, i, C.byref(t)) == 0
+            assert len(C.string_at(t.data, t.nbytes)) == t.nbytes and t.offset + t.nbytes <= len(v)
+        z = pkg.MoeBufs()
+        lib.fnx_gguf_moe_layer_bytes(g, 0, 0, 256, C.byref(z))   # either answer; never a fault
+        lib.fnx_gguf_close(g)
+    assert refused >= 150
