@@ -1347,8 +1347,14 @@ static int mtp_draft(const fnx_decoder* D, const fnx_mtp* M, const float* src, c
     // R = fc_hid(rms(src)) + fc_emb(rms(emb)): the sum is taken by the layer's first pass over the rows
     if (fnx_add_norm_q8(const_cast<float*>(src), nullptr, M->norm_hid, nullptr, ws->xq, T, n, D->eps, st)) return 1;   // nothing to add: src is only read
     if (fnx_q8s_gemv(&M->fc_hid, ws->xq, ws->x, n, T, st)) return 1;
-    if (fnx_embed_rows(D->emb, tokens, T, D->vocab, n, ws->xn, st)) return 1;
-    if (fnx_add_norm_q8(ws->xn, nullptr, M->norm_emb, nullptr, ws->xq, T, n, D->eps, st)) return 1;
+    {   // the tokens' embedding rows, normed and quantised by the pass that reads them from the table (rms(emb[tokens]))
+        CombineArgs c{};
+        c.emb = D->emb;
+        c.tokens = tokens;
+        c.vocab = D->vocab;
+        k_add_norm_q8<false><<<T, 256, 0, (hipStream_t) st>>>(ws->xn, nullptr, c, M->norm_emb, nullptr, (uint8_t*) ws->xq, n, D->eps);
+        if (launch_status("mtp_draft")) return 1;
+    }
     if (fnx_q8s_gemv(&M->fc_emb, ws->xq, ws->o, n, T, st)) return 1;
     DecPending pend{ws->o, nullptr, nullptr, nullptr};
     if (dec_layer(D, &M->layer, T, pos0, ws, pend, st, live)) return 1;
