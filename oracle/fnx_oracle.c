@@ -502,6 +502,7 @@ unsigned fnx_o_argmax(const float* logits, int rows, int T, int v0, float* best_
  * restated from its published form per 32 values; its per-thread split of a block and its warp order cannot be pinned, so
  * the sums here run in this build's order (lane l of 64 takes sub-blocks l, l + 64, ...; then the xor butterfly). */
 #define T_Q4_0 2u
+#define T_Q5_1 7u
 #define T_Q8_0 8u
 #define T_Q4_K 12u
 #define T_Q5_K 13u
@@ -510,6 +511,7 @@ static const int8_t KV_IQ4NL[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1,
 int fnx_o_type_block(uint32_t type, int* values, int* bytes) {
     switch (type) {
         case T_Q4_0: *values = 32; *bytes = 18; return 0;
+        case T_Q5_1: *values = 32; *bytes = 24; return 0;
         case T_Q8_0: *values = 32; *bytes = 34; return 0;
         case T_IQ4_NL: *values = 32; *bytes = 18; return 0;
         case T_Q4_K: *values = 256; *bytes = 144; return 0;
@@ -543,6 +545,19 @@ static void sub_decode(uint32_t type, const uint8_t* row, int kb, sub_t* o) {
         memcpy(&h, p, 2);
         o->d = fnx_o_h2f(h);
         for (int j = 0; j < 32; ++j) o->q[j] = (int8_t) p[2 + j];
+    } else if (type == T_Q5_1) { /* ggml block_q5_1 {half d; half m; u32 qh; u8 qs[16]}: value = d * q + m, q = nibble | bit << 4 (not
+                                    in tensor_convert.hpp: the layout is ggml's published one) */
+        const uint8_t* p = row + (size_t) kb * 24;
+        uint32_t qh;
+        memcpy(&h, p, 2);
+        o->d = fnx_o_h2f(h);
+        memcpy(&h, p + 2, 2);
+        o->dmin = fnx_o_h2f(h); /* the block's m (added, not subtracted) */
+        memcpy(&qh, p + 4, 4);
+        for (int j = 0; j < 16; ++j) {
+            o->q[j] = (p[8 + j] & 0xF) | (int) (((qh >> j) & 1u) << 4);
+            o->q[j + 16] = (p[8 + j] >> 4) | (int) (((qh >> (j + 16)) & 1u) << 4);
+        }
     } else if (type == T_Q4_0 || type == T_IQ4_NL) {
         const uint8_t* p = row + (size_t) kb * 18;
         memcpy(&h, p, 2);
@@ -574,6 +589,7 @@ void fnx_o_dequant(uint32_t type, const uint8_t* src, size_t n, float* y) {
         sub_decode(type, src, (int) kb, &s);
         for (int j = 0; j < 32; ++j) {
             if (type == T_Q4_0) y[kb * 32 + j] = s.d * (float) (s.q[j] - 8);
+            else if (type == T_Q5_1) y[kb * 32 + j] = s.d * (float) s.q[j] + s.dmin;
             else if (type == T_Q4_K || type == T_Q5_K) y[kb * 32 + j] = (s.d * (float) s.sc) * (float) s.q[j] - s.dmin * (float) s.m;
             else y[kb * 32 + j] = s.d * (float) s.q[j];
         }
@@ -595,6 +611,7 @@ float fnx_o_vec_dot_type(uint32_t type, const uint8_t* row, int kb, const uint8_
         qsum += x;
     }
     if (type == T_Q4_0) return s.d * ((float) dot * dx - 8.0f * sx);                      /* vec_dot_q4_0_q8_1_impl */
+    if (type == T_Q5_1) return (float) dot * (s.d * dx) + s.dmin * sx;                    /* vec_dot_q5_1_q8_1_impl */
     if (type == T_Q4_K || type == T_Q5_K)                                               /* vec_dot_q4_K_q8_1_impl_vmmq */
         return s.d * (dx * (float) (dot * s.sc)) - s.dmin * (dx * (float) (qsum * s.m));
     return (s.d * dx) * (float) dot;                                                      /* vec_dot_q8_0_q8_1_impl, vec_dot_iq4_nl_q8_1 */

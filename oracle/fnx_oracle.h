@@ -20,6 +20,8 @@
  *             own conv::dequantize through oracle/_ref and against numpy restatements; their dots (fnx_o_vec_dot_type)
  *             against the decoded values times the q8_1 values in f64 (the Q4_0 form through the block's sum field to
  *             within that field's f16 rounding).
+ *   parity unpinned: the Q5_1 decoder (type 7): the reference's host code has no dequantiser for it; the block layout is
+ *             ggml's published one, checked against a numpy restatement only.
  *   parity unpinned: the float-operation order of ggml's vec_dot_<type>_q8_1 for those types (third-party, fetched at
  *             build time, absent from the tree): the per-32-value terms follow its published form, the sums this build's
  *             own fixed order.
@@ -106,7 +108,7 @@ int fnx_o_lookup_drafts(const int* ctx, int n_ctx, int key_n, int lk, int d1, in
 int fnx_o_lookup_fixed(const int* ctx, int n_ctx, int key_n, int lk, int d1, int* out);
 /* session.cpp:573 */
 int fnx_o_accept_greedy(const int* rows, const int* o, int R);
-/* other expert types at the boundary (kernels.cu:2454-2471): Q4_0 (2), Q8_0 (8), Q4_K (12), Q5_K (13), IQ4_NL (20) */
+/* other expert types at the boundary (kernels.cu:2454-2471): Q4_0 (2), Q5_1 (7), Q8_0 (8), Q4_K (12), Q5_K (13), IQ4_NL (20) */
 int fnx_o_type_block(uint32_t type, int* values, int* bytes);
 void fnx_o_dequant(uint32_t type, const uint8_t* src, size_t n, float* y);
 float fnx_o_vec_dot_type(uint32_t type, const uint8_t* row, int kb, const uint8_t* q8);

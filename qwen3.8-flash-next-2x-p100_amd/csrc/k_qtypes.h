@@ -1,5 +1,5 @@
 // The other expert types the reference's operators take at the boundary (kernels.cu:2454-2471 moe_mm): rows of Q4_0, Q8_0,
-// IQ4_NL (32-value blocks) and Q4_K, Q5_K (256-value super-blocks of eight 32-value sub-blocks) against q8_1 activation
+// Q5_1, IQ4_NL (32-value blocks) and Q4_K, Q5_K (256-value super-blocks of eight 32-value sub-blocks) against q8_1 activation
 // rows, through the same job lists. Block layouts as tensor_convert.hpp:152-265 decodes them; a sub-block's term of the
 // dot is ggml's vec_dot_<type>_q8_1 per 32 values (the integers through sdot4, the q8_1 sum field for Q4_0's offset and
 // the activations' sum for the K-quants' minimum).
@@ -12,7 +12,7 @@
 
 namespace fnx {
 
-constexpr uint32_t QT_Q4_0 = 2, QT_Q8_0 = 8, QT_Q4_K = 12, QT_Q5_K = 13, QT_IQ4_NL = 20;
+constexpr uint32_t QT_Q4_0 = 2, QT_Q5_1 = 7, QT_Q8_0 = 8, QT_Q4_K = 12, QT_Q5_K = 13, QT_IQ4_NL = 20;
 __device__ const int8_t g_kvalues_iq4nl[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
 
 struct QtSub {
@@ -41,6 +41,23 @@ __device__ __forceinline__ QtSub qt_decode(const uint8_t* row, int kb) {
         o.d = half_bits_to_float((unsigned short) load_u16(p));
 #pragma unroll
         for (int j = 0; j < 8; ++j) o.w4[j] = (int) load_u32_a2(p + 2 + 4 * j);
+    } else if constexpr (TYPE == QT_Q5_1) {   // ggml block_q5_1 {half d; half m; u32 qh; u8 qs[16]}: value = d * q + m
+        const uint8_t* p = row + (size_t) kb * 24;
+        o.d = half_bits_to_float((unsigned short) load_u16(p));
+        o.dmin = half_bits_to_float((unsigned short) load_u16(p + 2));   // m: added
+        const uint32_t qh = load_u32_a2(p + 4);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {   // value j: nibble | bit j of qh << 4; value 16 + j: high nibble | bit 16 + j << 4
+            const uint32_t v = load_u32_a2(p + 8 + 4 * i);
+            uint32_t lo = v & 0x0F0F0F0Fu, hi = (v >> 4) & 0x0F0F0F0Fu;
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                lo |= ((qh >> (4 * i + b)) & 1u) << (8 * b + 4);
+                hi |= ((qh >> (16 + 4 * i + b)) & 1u) << (8 * b + 4);
+            }
+            o.w4[i] = (int) lo;
+            o.w4[4 + i] = (int) hi;
+        }
     } else if constexpr (TYPE == QT_Q4_0) {
         const uint8_t* p = row + (size_t) kb * 18;
         o.d = half_bits_to_float((unsigned short) load_u16(p));
@@ -96,6 +113,7 @@ __device__ __forceinline__ float qt_term(const QtSub& s, const uint8_t* yb) {
         if constexpr (TYPE == QT_Q4_K || TYPE == QT_Q5_K) qsum = __builtin_amdgcn_sdot4(0x01010101, x, qsum, false);
     }
     if constexpr (TYPE == QT_Q4_0) return s.d * ((float) dot * dx - 8.0f * half_bits_to_float((unsigned short) load_u16(yb + 2)));
+    else if constexpr (TYPE == QT_Q5_1) return (float) dot * (s.d * dx) + s.dmin * half_bits_to_float((unsigned short) load_u16(yb + 2));
     else if constexpr (TYPE == QT_Q4_K || TYPE == QT_Q5_K) return s.d * (dx * (float) (dot * s.sc)) - s.dmin * (dx * (float) (qsum * s.m));
     else return (s.d * dx) * (float) dot;
 }

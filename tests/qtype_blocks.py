@@ -2,8 +2,8 @@
 restatements of their decoders, written from the types' published layouts."""
 import numpy as np
 
-Q4_0, Q8_0, Q4_K, Q5_K, IQ4_NL = 2, 8, 12, 13, 20
-SHAPE = {Q4_0: (32, 18), Q8_0: (32, 34), IQ4_NL: (32, 18), Q4_K: (256, 144), Q5_K: (256, 176)}
+Q4_0, Q5_1, Q8_0, Q4_K, Q5_K, IQ4_NL = 2, 7, 8, 12, 13, 20
+SHAPE = {Q4_0: (32, 18), Q5_1: (32, 24), Q8_0: (32, 34), IQ4_NL: (32, 18), Q4_K: (256, 144), Q5_K: (256, 176)}
 KV = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], np.float32)
 
 
@@ -12,8 +12,8 @@ def random_blocks(rng, qtype, nblocks, dmax=0.02):
     b = rng.integers(0, 256, size=(nblocks, nbytes), dtype=np.uint8)
     d = (rng.random(nblocks) * dmax + 1e-4).astype(np.float16)
     b[:, 0:2] = d.view(np.uint8).reshape(nblocks, 2)
-    if qtype in (Q4_K, Q5_K):
-        m = (rng.random(nblocks) * dmax + 1e-4).astype(np.float16)
+    if qtype in (Q4_K, Q5_K, Q5_1):
+        m = ((rng.random(nblocks) - (0.5 if qtype == Q5_1 else 0.0)) * dmax + 1e-4).astype(np.float16)
         b[:, 2:4] = m.view(np.uint8).reshape(nblocks, 2)
     return b.reshape(-1)
 
@@ -38,6 +38,13 @@ def np_dequant(qtype, blocks):
     out = np.zeros((b.shape[0], values), f32)
     if qtype == Q8_0:
         out[:] = d[:, None] * b[:, 2:].view(np.int8).astype(f32)
+    elif qtype == Q5_1:
+        m = b[:, 2:4].copy().view(np.float16).astype(f32).reshape(-1)
+        qh = b[:, 4:8].copy().view(np.uint32).reshape(-1).astype(np.int64)
+        lo, hi = (b[:, 8:] & 0xF).astype(np.int64), (b[:, 8:] >> 4).astype(np.int64)
+        j = np.arange(16)
+        q = np.concatenate([lo | (((qh[:, None] >> j) & 1) << 4), hi | (((qh[:, None] >> (j + 16)) & 1) << 4)], axis=1)
+        out[:] = d[:, None] * q.astype(f32) + m[:, None]
     elif qtype in (Q4_0, IQ4_NL):
         lo, hi = (b[:, 2:] & 0xF).astype(np.int32), (b[:, 2:] >> 4).astype(np.int32)
         q = np.concatenate([lo, hi], axis=1)
