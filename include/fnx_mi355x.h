@@ -54,7 +54,7 @@ typedef struct fnx_dw {
     const void* p;          /* raw ggml blocks, row-major over output rows */
     uint32_t type;          /* FNX_T_IQ3_S (raw ggml blocks) or FNX_T_IQ3S_UNIT64 (after fnx_iq3s_repack); the decode
                              * operators (fnx_mmvq, fnx_moe_gate_up, fnx_moe_down, and fnx_moe_verify_layer operator by
-                             * operator) also take ggml's Q4_0 (2), Q5_1 (7), Q8_0 (8), Q4_K (12), Q5_K (13) and IQ4_NL (20) rows, the
+                             * operator) also take ggml's Q4_0 (2), Q5_1 (7), Q8_0 (8), Q4_K (12), Q5_K (13), IQ4_NL (20) and IQ4_XS (23) rows, the
                              * other types of kernels.cu:2454-2471 that the reference's host code can decode; the
                              * prompt path's grouped GEMM and the five-launch window are IQ3_S only */
     int n_in, n_out;        /* columns, rows */
@@ -407,7 +407,7 @@ int fnx_gguf_expert_cols(const fnx_gguf_tensor* down, int c0, int c1, void* dst,
  * file, f32 on the device); ffn_gate_exps / ffn_up_exps rows [ff0, ff1) -> gate|up; ffn_down_exps columns [ff0, ff1) ->
  * down; the _shexp tensors likewise (model.cpp:988-989, 1063-1068 without the card split's other half). Experts in
  * IQ3_S are uploaded into the caller's device buffers and re-laid there (fnx_iq3s_repack), so *L is ready for
- * fnx_moe_verify_layer / fnx_moe_prefill_layer; a layer with any tensor in Q4_0, Q5_1, Q8_0, IQ4_NL, Q4_K or Q5_K is left as the
+ * fnx_moe_verify_layer / fnx_moe_prefill_layer; a layer with any tensor in Q4_0, Q5_1, Q8_0, IQ4_NL, IQ4_XS, Q4_K or Q5_K is left as the
  * file has it (fnx_moe_verify_layer then runs operator by operator; the prompt path needs IQ3_S). The upload is synchronous; the re-laying runs on st.
  * topk <= 0: taken from "<general.architecture>.expert_used_count". */
 typedef struct fnx_moe_bufs {

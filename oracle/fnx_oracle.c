@@ -507,6 +507,7 @@ unsigned fnx_o_argmax(const float* logits, int rows, int T, int v0, float* best_
 #define T_Q4_K 12u
 #define T_Q5_K 13u
 #define T_IQ4_NL 20u
+#define T_IQ4_XS 23u
 static const int8_t KV_IQ4NL[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
 int fnx_o_type_block(uint32_t type, int* values, int* bytes) {
     switch (type) {
@@ -515,6 +516,7 @@ int fnx_o_type_block(uint32_t type, int* values, int* bytes) {
         case T_Q8_0: *values = 32; *bytes = 34; return 0;
         case T_IQ4_NL: *values = 32; *bytes = 18; return 0;
         case T_Q4_K: *values = 256; *bytes = 144; return 0;
+        case T_IQ4_XS: *values = 256; *bytes = 136; return 0;
         case T_Q5_K: *values = 256; *bytes = 176; return 0;
     }
     return 1;
@@ -567,6 +569,19 @@ static void sub_decode(uint32_t type, const uint8_t* row, int kb, sub_t* o) {
             o->q[j] = type == T_Q4_0 ? lo : KV_IQ4NL[lo];      /* Q4_0: the - 8 is applied through the q8_1 sum */
             o->q[j + 16] = type == T_Q4_0 ? hi : KV_IQ4NL[hi];
         }
+    } else if (type == T_IQ4_XS) { /* {half d; u16 scales_h; u8 scales_l[4]; u8 qs[128]}: sub-block ib has a 6-bit scale - 32 */
+        const int ib = kb & 7;
+        const uint8_t* p = row + (size_t) (kb >> 3) * 136;
+        uint16_t sh;
+        memcpy(&h, p, 2);
+        o->d = fnx_o_h2f(h);
+        memcpy(&sh, p + 2, 2);
+        o->sc = (((p[4 + ib / 2] >> (4 * (ib % 2))) & 0xF) | (((sh >> (2 * ib)) & 3) << 4)) - 32;
+        const uint8_t* qs = p + 8 + 16 * ib;
+        for (int j = 0; j < 16; ++j) {
+            o->q[j] = KV_IQ4NL[qs[j] & 0xF];
+            o->q[j + 16] = KV_IQ4NL[qs[j] >> 4];
+        }
     } else { /* Q4_K, Q5_K: super-block kb / 8, sub-block kb % 8 */
         const int sb = kb & 7, five = type == T_Q5_K;
         const uint8_t* p = row + (size_t) (kb >> 3) * (five ? 176 : 144);
@@ -590,6 +605,7 @@ void fnx_o_dequant(uint32_t type, const uint8_t* src, size_t n, float* y) {
         for (int j = 0; j < 32; ++j) {
             if (type == T_Q4_0) y[kb * 32 + j] = s.d * (float) (s.q[j] - 8);
             else if (type == T_Q5_1) y[kb * 32 + j] = s.d * (float) s.q[j] + s.dmin;
+            else if (type == T_IQ4_XS) y[kb * 32 + j] = (s.d * (float) s.sc) * (float) s.q[j];
             else if (type == T_Q4_K || type == T_Q5_K) y[kb * 32 + j] = (s.d * (float) s.sc) * (float) s.q[j] - s.dmin * (float) s.m;
             else y[kb * 32 + j] = s.d * (float) s.q[j];
         }
@@ -612,6 +628,7 @@ float fnx_o_vec_dot_type(uint32_t type, const uint8_t* row, int kb, const uint8_
     }
     if (type == T_Q4_0) return s.d * ((float) dot * dx - 8.0f * sx);                      /* vec_dot_q4_0_q8_1_impl */
     if (type == T_Q5_1) return (float) dot * (s.d * dx) + s.dmin * sx;                    /* vec_dot_q5_1_q8_1_impl */
+    if (type == T_IQ4_XS) return (s.d * dx) * (float) (dot * s.sc);                       /* vec_dot_iq4_xs_q8_1 */
     if (type == T_Q4_K || type == T_Q5_K)                                               /* vec_dot_q4_K_q8_1_impl_vmmq */
         return s.d * (dx * (float) (dot * s.sc)) - s.dmin * (dx * (float) (qsum * s.m));
     return (s.d * dx) * (float) dot;                                                      /* vec_dot_q8_0_q8_1_impl, vec_dot_iq4_nl_q8_1 */

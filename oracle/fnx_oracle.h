@@ -16,7 +16,7 @@
  *             (-key, id) incl. wide ties and signed zeros; penalties as a numpy f32 closed form), make_dist (numpy
  *             vectorised softmax / cumulative cut, limiting cases), accept_sampled (the window's first token is
  *             distributed as the target p whatever q is: exact measure over a grid of uniforms; fixed-draft closed form).
- *   pinned:   the other expert types' decoders (fnx_o_dequant: Q4_0, Q8_0, Q4_K, Q5_K, IQ4_NL) against the reference's
+ *   pinned:   the other expert types' decoders (fnx_o_dequant: Q4_0, Q8_0, Q4_K, Q5_K, IQ4_NL, IQ4_XS) against the reference's
  *             own conv::dequantize through oracle/_ref and against numpy restatements; their dots (fnx_o_vec_dot_type)
  *             against the decoded values times the q8_1 values in f64 (the Q4_0 form through the block's sum field to
  *             within that field's f16 rounding).
@@ -108,7 +108,7 @@ int fnx_o_lookup_drafts(const int* ctx, int n_ctx, int key_n, int lk, int d1, in
 int fnx_o_lookup_fixed(const int* ctx, int n_ctx, int key_n, int lk, int d1, int* out);
 /* session.cpp:573 */
 int fnx_o_accept_greedy(const int* rows, const int* o, int R);
-/* other expert types at the boundary (kernels.cu:2454-2471): Q4_0 (2), Q5_1 (7), Q8_0 (8), Q4_K (12), Q5_K (13), IQ4_NL (20) */
+/* other expert types at the boundary (kernels.cu:2454-2471): Q4_0 (2), Q5_1 (7), Q8_0 (8), Q4_K (12), Q5_K (13), IQ4_NL (20), IQ4_XS (23) */
 int fnx_o_type_block(uint32_t type, int* values, int* bytes);
 void fnx_o_dequant(uint32_t type, const uint8_t* src, size_t n, float* y);
 float fnx_o_vec_dot_type(uint32_t type, const uint8_t* row, int kb, const uint8_t* q8);

@@ -689,7 +689,7 @@ static int cu_count() {
 static int rows_launch(const fnx_dw* W, size_t w_stride, const fnx_job* jobs, const int* njobs, int njobs_max, const void* y, float* out,
                        int out_stride, void* st, const char* who, bool wide = false, int y_rows = 0) {
     if (!W || !jobs || !out) return fail(std::string(who) + ": null argument");
-    if (W->type == QT_Q4_0 || W->type == QT_Q5_1 || W->type == QT_Q8_0 || W->type == QT_IQ4_NL || W->type == QT_Q4_K || W->type == QT_Q5_K) {
+    if (W->type == QT_Q4_0 || W->type == QT_Q5_1 || W->type == QT_Q8_0 || W->type == QT_IQ4_NL || W->type == QT_IQ4_XS || W->type == QT_Q4_K || W->type == QT_Q5_K) {
         // the other types of kernels.cu:2454-2471 that the reference's own host code can decode (k_qtypes.h)
         gguf::BlockShape bs{};
         gguf::block_shape(W->type, bs);
@@ -706,6 +706,7 @@ static int rows_launch(const fnx_dw* W, size_t w_stride, const fnx_job* jobs, co
             case QT_Q5_1: k_qt_jobs<QT_Q5_1><<<grid, 256, 0, s>>>(q); break;
             case QT_Q8_0: k_qt_jobs<QT_Q8_0><<<grid, 256, 0, s>>>(q); break;
             case QT_IQ4_NL: k_qt_jobs<QT_IQ4_NL><<<grid, 256, 0, s>>>(q); break;
+            case QT_IQ4_XS: k_qt_jobs<QT_IQ4_XS><<<grid, 256, 0, s>>>(q); break;
             case QT_Q4_K: k_qt_jobs<QT_Q4_K><<<grid, 256, 0, s>>>(q); break;
             default: k_qt_jobs<QT_Q5_K><<<grid, 256, 0, s>>>(q); break;
         }
@@ -713,7 +714,7 @@ static int rows_launch(const fnx_dw* W, size_t w_stride, const fnx_job* jobs, co
     }
     if (W->type != FNX_T_IQ3_S && W->type != FNX_T_IQ3S_UNIT64)
         return fail(std::string(who) + ": expert type " + std::to_string(W->type) +
-                    " not handled (IQ3_S, and Q4_0, Q5_1, Q8_0, IQ4_NL, Q4_K, Q5_K through the plain path)");
+                    " not handled (IQ3_S, and Q4_0, Q5_1, Q8_0, IQ4_NL, IQ4_XS, Q4_K, Q5_K through the plain path)");
     if (W->n_in <= 0 || W->n_in % 256 || W->n_out <= 0) return fail(std::string(who) + ": shape does not fit IQ3_S super-blocks");
     if (W->row_bytes != (size_t) (W->n_in / 256) * FNX_IQ3S_BLOCK) return fail(std::string(who) + ": row_bytes does not match n_in");
     if (njobs_max <= 0) return fail(std::string(who) + ": njobs_max must be positive");
@@ -1630,9 +1631,9 @@ MoeTensors moe_tensors(const fnx_gguf* g, int layer) {
     MoeTensors m{get("ffn_gate_inp.weight"), get("ffn_gate_inp_shexp.weight"), get("ffn_gate_exps.weight"), get("ffn_up_exps.weight"),
                  get("ffn_down_exps.weight"), get("ffn_gate_shexp.weight"), get("ffn_up_shexp.weight"), get("ffn_down_shexp.weight")};
     for (const fnx_gguf_tensor* t : {&m.ge, &m.ue, &m.de, &m.gsh, &m.ush, &m.dsh})
-        if (t->type != gguf::T_IQ3_S && t->type != QT_Q4_0 && t->type != QT_Q5_1 && t->type != QT_Q8_0 && t->type != QT_IQ4_NL && t->type != QT_Q4_K && t->type != QT_Q5_K)
+        if (t->type != gguf::T_IQ3_S && t->type != QT_Q4_0 && t->type != QT_Q5_1 && t->type != QT_Q8_0 && t->type != QT_IQ4_NL && t->type != QT_IQ4_XS && t->type != QT_Q4_K && t->type != QT_Q5_K)
             throw std::runtime_error(gguf::nm(*t) + ": ggml type " + std::to_string(t->type) +
-                                     ", this path reads experts in IQ3_S (and Q4_0, Q5_1, Q8_0, IQ4_NL, Q4_K, Q5_K through its plain operators)");
+                                     ", this path reads experts in IQ3_S (and Q4_0, Q5_1, Q8_0, IQ4_NL, IQ4_XS, Q4_K, Q5_K through its plain operators)");
     if (m.gi.ne[0] != m.ge.ne[0] || m.gi.ne[1] != m.ge.ne[2] || m.gs.ne[1] != 1 || m.de.ne[1] != m.ge.ne[0] || m.de.ne[0] != m.ge.ne[1] ||
         m.de.ne[2] != m.ge.ne[2] || m.gsh.ne[0] != m.ge.ne[0] || m.dsh.ne[1] != m.ge.ne[0] || m.dsh.ne[0] != m.gsh.ne[1] || m.gsh.ne[2] != 1 ||
         m.dsh.ne[2] != 1)

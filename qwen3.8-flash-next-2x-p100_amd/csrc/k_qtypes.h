@@ -1,5 +1,5 @@
 // The other expert types the reference's operators take at the boundary (kernels.cu:2454-2471 moe_mm): rows of Q4_0, Q8_0,
-// Q5_1, IQ4_NL (32-value blocks) and Q4_K, Q5_K (256-value super-blocks of eight 32-value sub-blocks) against q8_1 activation
+// Q5_1, IQ4_NL (32-value blocks) and Q4_K, Q5_K, IQ4_XS (256-value super-blocks of eight 32-value sub-blocks) against q8_1 activation
 // rows, through the same job lists. Block layouts as tensor_convert.hpp:152-265 decodes them; a sub-block's term of the
 // dot is ggml's vec_dot_<type>_q8_1 per 32 values (the integers through sdot4, the q8_1 sum field for Q4_0's offset and
 // the activations' sum for the K-quants' minimum).
@@ -12,7 +12,7 @@
 
 namespace fnx {
 
-constexpr uint32_t QT_Q4_0 = 2, QT_Q5_1 = 7, QT_Q8_0 = 8, QT_Q4_K = 12, QT_Q5_K = 13, QT_IQ4_NL = 20;
+constexpr uint32_t QT_Q4_0 = 2, QT_Q5_1 = 7, QT_Q8_0 = 8, QT_Q4_K = 12, QT_Q5_K = 13, QT_IQ4_NL = 20, QT_IQ4_XS = 23;
 __device__ const int8_t g_kvalues_iq4nl[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
 
 struct QtSub {
@@ -67,12 +67,23 @@ __device__ __forceinline__ QtSub qt_decode(const uint8_t* row, int kb) {
             o.w4[i] = (int) (v & 0x0F0F0F0Fu);
             o.w4[4 + i] = (int) ((v >> 4) & 0x0F0F0F0Fu);
         }
-    } else if constexpr (TYPE == QT_IQ4_NL) {
-        const uint8_t* p = row + (size_t) kb * 18;
-        o.d = half_bits_to_float((unsigned short) load_u16(p));
+    } else if constexpr (TYPE == QT_IQ4_NL || TYPE == QT_IQ4_XS) {
+        const uint8_t* qs;
+        if constexpr (TYPE == QT_IQ4_NL) {
+            const uint8_t* p = row + (size_t) kb * 18;
+            o.d = half_bits_to_float((unsigned short) load_u16(p));
+            qs = p + 2;
+        } else {   // {half d; u16 scales_h; u8 scales_l[4]; u8 qs[128]}: sub-block ib's 6-bit scale - 32
+            const int ib = kb & 7;
+            const uint8_t* p = row + (size_t) (kb >> 3) * 136;
+            o.d = half_bits_to_float((unsigned short) load_u16(p));
+            const uint32_t sh = load_u16(p + 2);
+            o.sc = (int) (((p[4 + ib / 2] >> (4 * (ib % 2))) & 0xFu) | (((sh >> (2 * ib)) & 3u) << 4)) - 32;
+            qs = p + 8 + 16 * ib;
+        }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const uint32_t v = load_u32_a2(p + 2 + 4 * i);
+            const uint32_t v = load_u32_a2(qs + 4 * i);
             uint32_t lo = 0, hi = 0;
 #pragma unroll
             for (int b = 0; b < 4; ++b) {
@@ -115,6 +126,7 @@ __device__ __forceinline__ float qt_term(const QtSub& s, const uint8_t* yb) {
     if constexpr (TYPE == QT_Q4_0) return s.d * ((float) dot * dx - 8.0f * half_bits_to_float((unsigned short) load_u16(yb + 2)));
     else if constexpr (TYPE == QT_Q5_1) return (float) dot * (s.d * dx) + s.dmin * half_bits_to_float((unsigned short) load_u16(yb + 2));
     else if constexpr (TYPE == QT_Q4_K || TYPE == QT_Q5_K) return s.d * (dx * (float) (dot * s.sc)) - s.dmin * (dx * (float) (qsum * s.m));
+    else if constexpr (TYPE == QT_IQ4_XS) return (s.d * dx) * (float) (dot * s.sc);
     else return (s.d * dx) * (float) dot;
 }
 

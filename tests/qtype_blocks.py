@@ -2,8 +2,8 @@
 restatements of their decoders, written from the types' published layouts."""
 import numpy as np
 
-Q4_0, Q5_1, Q8_0, Q4_K, Q5_K, IQ4_NL = 2, 7, 8, 12, 13, 20
-SHAPE = {Q4_0: (32, 18), Q5_1: (32, 24), Q8_0: (32, 34), IQ4_NL: (32, 18), Q4_K: (256, 144), Q5_K: (256, 176)}
+Q4_0, Q5_1, Q8_0, Q4_K, Q5_K, IQ4_NL, IQ4_XS = 2, 7, 8, 12, 13, 20, 23
+SHAPE = {Q4_0: (32, 18), Q5_1: (32, 24), Q8_0: (32, 34), IQ4_NL: (32, 18), Q4_K: (256, 144), Q5_K: (256, 176), IQ4_XS: (256, 136)}
 KV = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], np.float32)
 
 
@@ -49,6 +49,15 @@ def np_dequant(qtype, blocks):
         lo, hi = (b[:, 2:] & 0xF).astype(np.int32), (b[:, 2:] >> 4).astype(np.int32)
         q = np.concatenate([lo, hi], axis=1)
         out[:] = d[:, None] * ((q - 8).astype(f32) if qtype == Q4_0 else KV[q])
+    elif qtype == IQ4_XS:
+        sh = b[:, 2:4].copy().view(np.uint16).reshape(-1).astype(np.int32)
+        for i in range(b.shape[0]):
+            for ib in range(8):
+                ls = ((int(b[i, 4 + ib // 2]) >> (4 * (ib % 2))) & 0xF) | (((sh[i] >> (2 * ib)) & 3) << 4)
+                qs = b[i, 8 + 16 * ib:8 + 16 * ib + 16].astype(np.int32)
+                dl = f32(d[i] * f32(ls - 32))
+                out[i, 32 * ib:32 * ib + 16] = dl * KV[qs & 0xF]
+                out[i, 32 * ib + 16:32 * ib + 32] = dl * KV[qs >> 4]
     else:
         mn = b[:, 2:4].copy().view(np.float16).astype(f32).reshape(-1)
         for i in range(b.shape[0]):

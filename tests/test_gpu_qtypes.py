@@ -12,7 +12,7 @@ import qtype_blocks as qb
 from fnx_gpu import JOB_DTYPE
 
 pytestmark = pytest.mark.gpu
-TYPES = [qb.Q4_0, qb.Q5_1, qb.Q8_0, qb.IQ4_NL, qb.Q4_K, qb.Q5_K]
+TYPES = [qb.Q4_0, qb.Q5_1, qb.Q8_0, qb.IQ4_NL, qb.IQ4_XS, qb.Q4_K, qb.Q5_K]
 
 
 def rel_l2(a, b):

@@ -9,7 +9,7 @@ import pytest
 import oracle_lib as ol
 import qtype_blocks as qb
 
-TYPES = [qb.Q4_0, qb.Q5_1, qb.Q8_0, qb.IQ4_NL, qb.Q4_K, qb.Q5_K]
+TYPES = [qb.Q4_0, qb.Q5_1, qb.Q8_0, qb.IQ4_NL, qb.IQ4_XS, qb.Q4_K, qb.Q5_K]
 
 
 def o_dequant(oracle, qtype, blocks):
