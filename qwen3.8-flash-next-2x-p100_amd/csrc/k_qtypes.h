@@ -13,7 +13,16 @@
 namespace fnx {
 
 constexpr uint32_t QT_Q4_0 = 2, QT_Q5_1 = 7, QT_Q8_0 = 8, QT_Q4_K = 12, QT_Q5_K = 13, QT_IQ4_NL = 20, QT_IQ4_XS = 23;
-__device__ const int8_t g_kvalues_iq4nl[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+// kvalues_iq4nl (tensor_convert.hpp): {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113}, four to a word.
+// Four 4-bit indexes (one a byte) -> their four table bytes: a byte permute over each half of the table (selector bytes
+// 0..3 take from the second operand, 4..7 from the first), the index's top bit choosing between the halves.
+__device__ __forceinline__ uint32_t iq4_values4(uint32_t idx4) {
+    constexpr uint32_t t0 = 0xBFAD9881u, t1 = 0xF6EADDCFu, t2 = 0x26190D01u, t3 = 0x71594535u;
+    const uint32_t sel = idx4 & 0x07070707u;
+    const uint32_t lo = __builtin_amdgcn_perm(t1, t0, sel), hi = __builtin_amdgcn_perm(t3, t2, sel);
+    const uint32_t upper = ((idx4 >> 3) & 0x01010101u) * 0xFFu;   // 0xFF in the bytes whose index is 8..15
+    return (hi & upper) | (lo & ~upper);
+}
 
 struct QtSub {
     int w4[8];       // the sub-block's 32 integers, four to a word
@@ -84,15 +93,8 @@ __device__ __forceinline__ QtSub qt_decode(const uint8_t* row, int kb) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const uint32_t v = load_u32_a2(qs + 4 * i);
-            uint32_t lo = 0, hi = 0;
-#pragma unroll
-            for (int b = 0; b < 4; ++b) {
-                const uint32_t byte = (v >> (8 * b)) & 0xFFu;
-                lo |= (uint32_t) (uint8_t) g_kvalues_iq4nl[byte & 0xF] << (8 * b);
-                hi |= (uint32_t) (uint8_t) g_kvalues_iq4nl[byte >> 4] << (8 * b);
-            }
-            o.w4[i] = (int) lo;
-            o.w4[4 + i] = (int) hi;
+            o.w4[i] = (int) iq4_values4(v & 0x0F0F0F0Fu);
+            o.w4[4 + i] = (int) iq4_values4((v >> 4) & 0x0F0F0F0Fu);
         }
     } else {
         constexpr bool FIVE = TYPE == QT_Q5_K;
