@@ -766,7 +766,7 @@ static void prof_mark(int i, hipStream_t s) {
     if (g_prof_on) (void) hipEventRecord(g_prof_ev[i], s);
 }
 // the window's MoE half in five launches (k_moe_layer.h)
-// live (may be null): a device word, the rows of the window that are routed (k_route_plan); the caller's combine skips the others
+// live (may be null): a device word, the rows of the window that are routed (k_route_topk, build_plan); the caller's combine skips the others
 static int layer_fused(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st, const int* live = nullptr) {
     hipStream_t s = (hipStream_t) st;
     const int n = L->n, ff = L->ff, P = T * L->topk, LS = L->nexp + 1;
@@ -774,16 +774,17 @@ static int layer_fused(const fnx_moe_layer* L, const float* x, int T, float* out
     prof_mark(0, s);
     k_router_quant<<<rblocks + qblocks, FL_THREADS, 0, s>>>(RouterArgs{L->nexp, T, x, L->router, L->router_bf16, ws->logits, (uint8_t*) ws->xq});
     prof_mark(1, s);
-    k_route_plan<<<T, RT_THREADS, 0, s>>>(RouteArgs{L->nexp, L->topk, T, ws->logits, ws->topi, ws->topw, ws->jobs_gu, ws->jobs_dn, ws->njobs, live});
+    const RouteArgs route{L->nexp, L->topk, T, ws->logits, ws->topi, ws->topw, ws->jobs_gu, ws->jobs_dn, ws->njobs, live};
+    k_route_topk<<<T, RT_THREADS, 0, s>>>(route);
     prof_mark(2, s);
     static const int per_cu = env_int("FNX_LAYER_BLOCKS_PER_CU", 2, 1, 8);
     const int grid = per_cu * cu_count();
     const PassArgs gu{2 * ff, (const uint8_t*) L->gu.p, L->gu_stride, (const uint8_t* const*) L->gu.ep, (const uint8_t*) L->sh_gu.p,
-                      (const uint8_t*) ws->xq, nullptr, ff, ws->gu};
+                      (const uint8_t*) ws->xq, nullptr, ff, ws->gu, route};
     k_moe_gate_up_passes<<<grid, FL_THREADS, 0, s>>>(gu);
     prof_mark(3, s);
     const PassArgs dn{n, (const uint8_t*) L->down.p, L->down_stride, (const uint8_t* const*) L->down.ep, (const uint8_t*) L->sh_down.p,
-                      nullptr, ws->gu, ff, ws->part};
+                      nullptr, ws->gu, ff, ws->part, RouteArgs{}};
     if (ff == 256) k_moe_down_passes<8><<<grid, FL_THREADS, 0, s>>>(dn);
     else if (ff == 512) k_moe_down_passes<16><<<grid, FL_THREADS, 0, s>>>(dn);
     else k_moe_down_passes<32><<<grid, FL_THREADS, 0, s>>>(dn);

@@ -106,11 +106,14 @@ __device__ __forceinline__ void wave_topk(const float* __restrict__ row, int nex
     if (lane < topk) topw[lane] = wk / z;
 }
 
-// ---------------------------------------------------------------- launch 2: top-k, jobs, plan
-// A block per row of the window: its first wave ranks the row's logits. The block that finishes last (a counter, as
-// k_router_route's last block, moe.cuh:324-330) builds the job lists and the plan from all rows' picks, without any
-// serial loop: a token picks an expert at most once, so a pair's slot in its job is the number of earlier tokens in the
-// expert's token mask, and a job's number is the rank of its first pair among the first pairs.
+// ---------------------------------------------------------------- launch 2: top-k; the plan, made by its readers
+// k_route_topk: a wave per row of the window ranks the row's logits. The job lists and the plan follow from all rows'
+// picks without any serial loop: a token picks an expert at most once, so a pair's slot in its job is the number of
+// earlier tokens in the expert's token mask, and a job's number is the rank of its first pair among the first pairs
+// (the order k_router_route's last block gives them, moe.cuh:324-330). Every block of the gate|up launch makes the plan
+// for itself in LDS from the 160 picks (build_plan), while its codebook loads are in flight; its block 0 also writes the
+// plan and the job lists to memory, for the down launch and for the caller. That is quicker than a last-block phase in
+// the top-k launch, which costs an atomic and two more memory round trips on the window's critical path.
 struct RouteArgs {
     int nexp, topk, T;
     const float* logits;
@@ -118,11 +121,21 @@ struct RouteArgs {
     float* topw;
     fnx_job* jobs_gu;
     fnx_job* jobs_dn;
-    int* njobs;   // [0] the job count, [1] the block counter (left at zero)
+    int* njobs;   // [0] the job count
     const int* live;   // may be null; else a device word: only the window's first *live rows are routed (the others get no
                        // pairs, and the shared expert's job stops before them), while the lists keep the indexes T gives them
 };
-constexpr int RT_THREADS = 256;
+constexpr int RT_THREADS = 64;
+__global__ void __launch_bounds__(RT_THREADS) k_route_topk(const RouteArgs a) {
+    __shared__ int ex[FL_MAXP];
+    const int lane = threadIdx.x, LS = a.nexp + 1, t = blockIdx.x, topk = a.topk;
+    const int Tl = a.live ? uniform(max(0, min(*a.live, a.T))) : a.T;
+    if (t >= Tl) return;
+    if (a.nexp <= 512) wave_topk<8>(a.logits + (size_t) t * LS, a.nexp, topk, lane, ex, a.topi + t * topk, a.topw + t * topk);
+    else wave_topk<16>(a.logits + (size_t) t * LS, a.nexp, topk, lane, ex, a.topi + t * topk, a.topw + t * topk);
+}
+
+template <int NT>
 struct RouteLds {
     LayerPlan plan;
     int ex[FL_MAXP];
@@ -130,100 +143,84 @@ struct RouteLds {
     int first[1024];          // per expert: its first pair
     int jobof[1024];
     int pass0[FL_MAXJ + 3];   // per job: its first pass
-    int wcnt[RT_THREADS / 64];
-    int last;
+    int wcnt[NT / 64];
 };
-__global__ void __launch_bounds__(RT_THREADS) k_route_plan(const RouteArgs a) {
-    __shared__ RouteLds L;
+// All NT threads of a block; ends with a barrier. publish: also write the lists and the plan to memory.
+template <int NT>
+__device__ __forceinline__ void build_plan(RouteLds<NT>& L, const RouteArgs& a, bool publish) {
+    static_assert(FL_MAXP <= NT && FL_MAXJ <= NT, "a thread per pair, a thread per job");
     const int tid = threadIdx.x, wave = uniform(tid >> 6), lane = tid & 63;
-    const int T = a.T, topk = a.topk, P = T * topk, LS = a.nexp + 1, t = blockIdx.x;
+    const int T = a.T, topk = a.topk, P = T * topk;
     const int Tl = a.live ? uniform(max(0, min(*a.live, T))) : T, Pl = Tl * topk;
-    if (wave == 0 && t < Tl) {
-        if (a.nexp <= 512) wave_topk<8>(a.logits + (size_t) t * LS, a.nexp, topk, lane, L.ex, a.topi + t * topk, a.topw + t * topk);
-        else wave_topk<16>(a.logits + (size_t) t * LS, a.nexp, topk, lane, L.ex, a.topi + t * topk, a.topw + t * topk);
-    }
-    __syncthreads();
-    if (tid == 0) {
-        __threadfence();
-        L.last = atomicAdd((unsigned*) &a.njobs[1], 1u) == (unsigned) T - 1;
-        if (L.last) {
-            __threadfence();
-            a.njobs[1] = 0;
-        }
-    }
-    __syncthreads();
-    if (!L.last) return;
     LayerPlan& pl = L.plan;
-    for (int e = tid; e < a.nexp; e += RT_THREADS) {
+    const int e_mine = tid < Pl ? a.topi[tid] : 0;   // asked for before the tables are cleared
+    for (int e = tid; e < a.nexp; e += NT) {
         L.mask[e] = 0u;
         L.first[e] = P;
     }
     __syncthreads();
-    // every row's picks (this block's own included) from memory
-    for (int p = tid; p < Pl; p += RT_THREADS) {
-        const int e = __hip_atomic_load(&a.topi[p], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        L.ex[p] = e;
-        atomicOr(&L.mask[e], 1u << (p / topk));
-        atomicMin(&L.first[e], p);
-        pl.pair_tok[p] = (uint8_t) (p / topk);
+    if (tid < Pl) {
+        L.ex[tid] = e_mine;
+        atomicOr(&L.mask[e_mine], 1u << (tid / topk));
+        atomicMin(&L.first[e_mine], tid);
+        pl.pair_tok[tid] = (uint8_t) (tid / topk);
     }
     if (tid < Tl) pl.pair_tok[P + tid] = (uint8_t) tid;
     __syncthreads();
     // job numbers: the rank of an expert's first pair among all first pairs (ballots over the pairs in order)
-    int base = 0;
-    for (int p0 = 0; p0 < Pl; p0 += RT_THREADS) {
-        const int p = p0 + tid;
-        const bool isfirst = p < Pl && L.first[L.ex[p]] == p;
-        const unsigned long long b = __ballot(isfirst);
-        if (lane == 0) L.wcnt[wave] = __popcll(b);
-        __syncthreads();
-        int before = base, total = 0;
-        for (int w = 0; w < RT_THREADS / 64; ++w) {
-            before += w < wave ? L.wcnt[w] : 0;
-            total += L.wcnt[w];
-        }
-        if (isfirst) {
-            const int e = L.ex[p], j = before + __popcll(b & ((1ull << lane) - 1ull)), cnt = __popc(L.mask[e]);
-            L.jobof[e] = j;
-            pl.job_w[j] = e;
-            pl.job_n[j] = (uint8_t) cnt;
-            a.jobs_gu[j].w = a.jobs_dn[j].w = e;
+    const bool isfirst = tid < Pl && L.first[e_mine] == tid;
+    const unsigned long long b = __ballot(isfirst);
+    if (lane == 0) L.wcnt[wave] = __popcll(b);
+    __syncthreads();
+    int before = 0, nj = 0;
+    for (int w = 0; w < NT / 64; ++w) {
+        before += w < wave ? L.wcnt[w] : 0;
+        nj += L.wcnt[w];
+    }
+    nj = uniform(nj);
+    if (isfirst) {
+        const int j = before + __popcll(b & ((1ull << lane) - 1ull)), cnt = __popc(L.mask[e_mine]);
+        L.jobof[e_mine] = j;
+        pl.job_w[j] = e_mine;
+        pl.job_n[j] = (uint8_t) cnt;
+        if (publish) {
+            a.jobs_gu[j].w = a.jobs_dn[j].w = e_mine;
             a.jobs_gu[j].n = a.jobs_dn[j].n = cnt;
         }
-        base += total;
-        __syncthreads();
     }
-    const int nj = base;
     if (tid == 0) {
         pl.nj = nj;
         pl.job_w[nj] = -1;   // the shared expert's job: every row of the window, pairs P + t
         pl.job_n[nj] = (uint8_t) Tl;
-        a.njobs[0] = nj;
+        if (publish) a.njobs[0] = nj;
     }
+    __syncthreads();
     // a pair's slot in its job: the earlier rows in its expert's mask (pairs of a job ascend with the row)
-    for (int p = tid; p < Pl; p += RT_THREADS) {
-        const int e = L.ex[p], j = L.jobof[e], row = p / topk, slot = __popc(L.mask[e] & ((1u << row) - 1u));
-        pl.job_pairs[j][slot] = (uint8_t) p;
-        a.jobs_gu[j].y[slot] = row;
-        a.jobs_gu[j].out[slot] = p;
-        a.jobs_dn[j].y[slot] = p;
-        a.jobs_dn[j].out[slot] = p;
+    if (tid < Pl) {
+        const int j = L.jobof[e_mine], row = tid / topk, slot = __popc(L.mask[e_mine] & ((1u << row) - 1u));
+        pl.job_pairs[j][slot] = (uint8_t) tid;
+        if (publish) {
+            a.jobs_gu[j].y[slot] = row;
+            a.jobs_gu[j].out[slot] = tid;
+            a.jobs_dn[j].y[slot] = tid;
+            a.jobs_dn[j].out[slot] = tid;
+        }
     }
     if (tid < max(Tl, 1)) {   // the shared expert's job, at index P of the lists the API returns (kernels.hpp:277-282)
         pl.job_pairs[nj][tid] = (uint8_t) (P + tid);
-        a.jobs_gu[P].y[tid] = tid;
-        a.jobs_gu[P].out[tid] = P + tid;
-        a.jobs_dn[P].y[tid] = P + tid;
-        a.jobs_dn[P].out[tid] = P + tid;
-        if (tid == 0) {
-            a.jobs_gu[P].w = a.jobs_dn[P].w = 0;
-            a.jobs_gu[P].n = a.jobs_dn[P].n = Tl;
+        if (publish) {
+            a.jobs_gu[P].y[tid] = tid;
+            a.jobs_gu[P].out[tid] = P + tid;
+            a.jobs_dn[P].y[tid] = P + tid;
+            a.jobs_dn[P].out[tid] = P + tid;
+            if (tid == 0) {
+                a.jobs_gu[P].w = a.jobs_dn[P].w = 0;
+                a.jobs_gu[P].n = a.jobs_dn[P].n = Tl;
+            }
         }
     }
-    __syncthreads();
     // passes: job j's rows two at a time; job j's first pass = the passes of the jobs before it: a scan over the jobs
     // (wave by wave with the waves' totals in LDS; a thread per job)
-    static_assert(FL_MAXJ <= RT_THREADS, "a thread per job");
     {
         const int cj = tid <= nj ? (pl.job_n[tid] + 1) >> 1 : 0;
         int inc = cj;
@@ -232,21 +229,22 @@ __global__ void __launch_bounds__(RT_THREADS) k_route_plan(const RouteArgs a) {
             const int up = __shfl_up(inc, o, 64);
             if (lane >= o) inc += up;
         }
-        if (lane == 63) L.wcnt[wave] = inc;
+        if (lane == 63) L.wcnt[wave] = inc;   // (the job count's readers of wcnt are behind a barrier)
         __syncthreads();
-        int before = 0;
-        for (int w = 0; w < wave; ++w) before += L.wcnt[w];
-        if (tid <= nj) L.pass0[tid] = before + inc - cj;
-        if (tid == nj) pl.npass = before + inc;
+        int bef = 0;
+        for (int w = 0; w < wave; ++w) bef += L.wcnt[w];
+        if (tid <= nj) {
+            const int p0 = bef + inc - cj, n = pl.job_n[tid];
+            for (int t0 = 0, k = 0; t0 < n; t0 += 2, ++k) {
+                pl.pass_job[p0 + k] = (uint8_t) tid;
+                pl.pass_t0[p0 + k] = (uint8_t) t0;
+            }
+        }
+        if (tid == nj) pl.npass = bef + inc;
     }
     __syncthreads();
-    for (int j = tid; j <= nj; j += RT_THREADS)
-        for (int t0 = 0, k = 0; t0 < pl.job_n[j]; t0 += 2, ++k) {
-            pl.pass_job[L.pass0[j] + k] = (uint8_t) j;
-            pl.pass_t0[L.pass0[j] + k] = (uint8_t) t0;
-        }
-    __syncthreads();
-    for (int i = tid; i < (int) (sizeof(LayerPlan) / 4); i += RT_THREADS) reinterpret_cast<int*>(&g_layer_plan)[i] = reinterpret_cast<const int*>(&pl)[i];
+    if (publish)
+        for (int i = tid; i < (int) (sizeof(LayerPlan) / 4); i += NT) reinterpret_cast<int*>(&g_layer_plan)[i] = reinterpret_cast<const int*>(&pl)[i];
 }
 
 // ---------------------------------------------------------------- launch 1: router logits | q8_1 rows of x
@@ -355,6 +353,7 @@ struct PassArgs {
     const float* gu;          // down: the gate|up outputs [pair][2 ff]
     int ff;
     float* out;               // [pair][rows]
+    RouteArgs route;          // gate|up: what the plan is made from
 };
 struct PassSeg {   // a stretch of one pass's units
     int ul, ue, ji, t0, nt;
@@ -378,15 +377,15 @@ __device__ __forceinline__ PassSeg pass_seg(const LayerPlan& pl, const PassArgs&
 __global__ void __launch_bounds__(FL_THREADS) k_moe_gate_up_passes(const PassArgs a) {
     constexpr int SBR = 64;
     __shared__ uint32_t tab[SGRID_WORDS];
-    __shared__ LayerPlan pl;
+    __shared__ RouteLds<FL_THREADS> L;
+    LayerPlan& pl = L.plan;
     const int tid = threadIdx.x, wave = uniform(tid >> 6), lane = tid & 63;
     // the codebook's loads go out first and land in registers; they are stored to LDS once the first weights have been
     // asked for, so that the latencies overlap
     uint32_t treg[SGRID_WORDS / FL_THREADS];
 #pragma unroll
     for (int i = 0; i < SGRID_WORDS / FL_THREADS; ++i) treg[i] = g_sgrid.v[tid + i * FL_THREADS];
-    for (int i = tid; i < (int) (sizeof(LayerPlan) / 4); i += FL_THREADS) reinterpret_cast<int*>(&pl)[i] = reinterpret_cast<const int*>(&g_layer_plan)[i];
-    __syncthreads();
+    build_plan<FL_THREADS>(L, a.route, blockIdx.x == 0);
     const int upj = a.rows;
     const long total = (long) pl.npass * upj;
     const long gw = (long) blockIdx.x * FL_WAVES + wave, nw = (long) gridDim.x * FL_WAVES;
