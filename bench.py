@@ -475,8 +475,12 @@ def decoder_main(args):
         rrows.zero_()
         rrows[0] = rctx[P0]
 
-    def a_round():
-        dev.ok(lib.fnx_decode_round(C.byref(D), C.byref(M), C.byref(RD), C.byref(ws), dev.st()))
+    # the same with an MTP chain of three drafts (random weights: the lookup never fires, so every round runs the chain)
+    chain_src = z(N, t.float32)
+    RD3 = pkg.Round(rstate.data_ptr(), rrows.data_ptr(), rctx.data_ptr(), CTX + 64, None, 0, 1, 3, 15, rscratch.data_ptr(), 3, chain_src.data_ptr())
+
+    def a_round(rd=None):
+        dev.ok(lib.fnx_decode_round(C.byref(D), C.byref(M), C.byref(rd if rd is not None else RD), C.byref(ws), dev.st()))
 
     def timed_rounds(run):
         torch.cuda.synchronize()
@@ -500,6 +504,15 @@ def decoder_main(args):
     round_graph_ms = timed_rounds(graph.replay)
     kept_graph = int(rstate[pkg.RS_NCTX].item()) - (P0 + 1)
     assert int(rstate[pkg.RS_STOP].item()) == 0 and int(rstate[pkg.RS_ROUNDS].item()) == NR + 3 and kept_graph == kept_eager, "rounds went wrong"
+    reset_rounds()
+    for _ in range(3):
+        a_round(RD3)
+    round_chain_ms = timed_rounds(lambda: a_round(RD3))
+    assert int(rstate[pkg.RS_STOP].item()) == 0 and int(rstate[pkg.RS_ROWS].item()) == 4, "the chain's rounds went wrong"
+    # what the chain's launches cost a round that does not run it: a stopped session repeats its round, chain switched off
+    rstate[pkg.RS_STOP] = 1
+    stopped_ms = timed_rounds(a_round)
+    stopped_chain_ms = timed_rounds(lambda: a_round(RD3))
     kv_bytes = 2 * CTX * NKV * HD * 2
     head_bytes = V * N + V * (N // 32) * 2
     dense_bytes = (NQ * 2 * HD * N + 2 * NKV * HD * N + N * NQ * HD) * 34 // 32
@@ -514,7 +527,9 @@ def decoder_main(args):
                        "head_GBps": head_bytes / (head_ms * 1e-3) / 1e9,
                        "decode_round": {"what": "verify 16 rows (2 count) + accept + commit + draft layer + lookup + next window at position 28,672, no host wait",
                                         "rounds": NR, "ms_eager": round_eager_ms, "ms_graph_replay": round_graph_ms,
-                                        "tokens_kept_per_round": kept_graph / (NR + 3)}},
+                                        "tokens_kept_per_round": kept_graph / (NR + 3),
+                                        "ms_eager_with_chain_of_3": round_chain_ms,
+                                        "ms_two_chain_steps_switched_off": stopped_chain_ms - stopped_ms}},
             "roofline": {"bound": "hbm", "kernel": "k_q8s_gemv (output head 151,936 x 2048)", "achieved": head_bytes / (head_ms * 1e-3) / 1e9,
                          "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": head_bytes / (head_ms * 1e-3) / HBM_PEAK, "traffic": None, "kernel_ms": head_ms,
                          "algorithmic_bytes": head_bytes},

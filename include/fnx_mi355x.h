@@ -307,8 +307,10 @@ int fnx_mtp_draft(const fnx_decoder* D, const fnx_mtp* M, const float* src, cons
  * the host for acceptance. Here the acceptance (session.cpp:565-573), the commit, the draft layer's pass over the rows
  * kept (engine.cu:2095-2133) and the prompt lookup (session.cpp:428-447) read and leave their results in device words,
  * so no argument of a round changes from one round to the next: rounds can be enqueued back to back, or captured once in
- * a graph and replayed. The MTP chain is one draft long (the draft layer's pick for the last row kept) when the lookup
- * finds nothing. */
+ * a graph and replayed. When the lookup finds nothing the MTP chain follows (session.cpp:666-678, at a fixed length
+ * fnx_round.chain; the reference's adaptive length and its min_p cut are the host's): each further draft is the draft
+ * layer's pick for the draft before, from its own hidden row. Its launches are always enqueued; in a round whose lookup
+ * found drafts their big kernels (the dense products, the attention's scan, the experts) leave at once on a device word. */
 enum {
     FNX_RS_NCTX = 0,     /* tokens in ctx: the prompt and everything emitted */
     FNX_RS_POS = 1,      /* cache position of the window's first row (= FNX_RS_NCTX - 1) */
@@ -317,7 +319,9 @@ enum {
     FNX_RS_POS_PREV = 4, /* the last window's position */
     FNX_RS_ROUNDS = 5,   /* rounds done */
     FNX_RS_STOP = 6,     /* set once the next window would not fit the caches or ctx: later rounds change nothing */
-    FNX_RS_WORDS = 8
+    FNX_RS_CHAIN = 7,    /* 1 while this round's MTP chain runs (the lookup found nothing), else 0 */
+    FNX_RS_CHAIN_POS = 8, /* FNX_MAXT words: the cache positions of the chain's steps */
+    FNX_RS_WORDS = 24
 };
 typedef struct fnx_round {
     int* state;    /* device, FNX_RS_WORDS ints (the caller sets NCTX, POS, ROWS and zeroes the others) */
@@ -329,6 +333,8 @@ typedef struct fnx_round {
     int speculate; /* 0: plain greedy decoding, one row a round (no draft layer, no lookup) */
     int key_n, lk; /* prompt lookup: tokens in the key (3 in the reference), most drafts (<= FNX_MAXT - 1) */
     int* scratch;  /* device, FNX_MAXT ints */
+    int chain;     /* drafts of an MTP chain (the reference's K), 1 .. FNX_MAXT - 1; 0 counts as 1 */
+    float* chain_src; /* device, n floats (the hidden row the chain starts from); may be null when chain <= 1 */
 } fnx_round;
 /* one round: fnx_decoder_verify over the window -> acceptance and commit -> fnx_mtp_draft over the rows kept -> lookup
  * -> the next window. Expert weights must be in the unit64 layout and hidden = 2048 (the five-launch window), since only

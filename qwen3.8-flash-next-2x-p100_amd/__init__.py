@@ -77,7 +77,7 @@ class Mtp(C.Structure):
 
 class Round(C.Structure):
     _fields_ = [("state", C.c_void_p), ("rows", C.c_void_p), ("ctx", C.c_void_p), ("ctx_cap", C.c_int), ("log", C.c_void_p), ("log_cap", C.c_int),
-                ("speculate", C.c_int), ("key_n", C.c_int), ("lk", C.c_int), ("scratch", C.c_void_p)]
+                ("speculate", C.c_int), ("key_n", C.c_int), ("lk", C.c_int), ("scratch", C.c_void_p), ("chain", C.c_int), ("chain_src", C.c_void_p)]
 
 
 class Sampling(C.Structure):
@@ -94,7 +94,7 @@ class MoeBufs(C.Structure):
                [(k, C.c_size_t) for k in ("router_bytes", "gu_bytes", "down_bytes", "sh_gu_bytes", "sh_down_bytes")]
 
 
-RS_NCTX, RS_POS, RS_ROWS, RS_ACCEPTED, RS_POS_PREV, RS_ROUNDS, RS_STOP, RS_WORDS = 0, 1, 2, 3, 4, 5, 6, 8
+RS_NCTX, RS_POS, RS_ROWS, RS_ACCEPTED, RS_POS_PREV, RS_ROUNDS, RS_STOP, RS_CHAIN, RS_CHAIN_POS, RS_WORDS = 0, 1, 2, 3, 4, 5, 6, 7, 8, 24
 
 EXPORTS = {
     # name: (restype, argtypes)

@@ -1179,7 +1179,8 @@ int fnx_embed_rows(const uint16_t* emb, const int* tokens, int T, int vocab, int
     k_embed_rows<<<T, 256, 0, (hipStream_t) st>>>(emb, tokens, vocab, n, y);
     return launch_status("embed_rows");
 }
-static int q8s_launch(const fnx_q8s* const* W, float* const* out, const int* out_stride, int n, const void* yq, int T, void* st, const char* who) {
+static int q8s_launch(const fnx_q8s* const* W, float* const* out, const int* out_stride, int n, const void* yq, int T, void* st, const char* who,
+                      const int* gate = nullptr) {
     if (!W || !out || !out_stride || !yq || n < 1 || n > 3) return fail(std::string(who) + ": null argument");
     Q8sArgs a{};
     long tiles = 0;
@@ -1209,6 +1210,7 @@ static int q8s_launch(const fnx_q8s* const* W, float* const* out, const int* out
     }
     static const int per_cu = env_int("FNX_Q8S_BLOCKS_PER_CU", 4, 1, 16);   // what the LDS of a 2048-column matrix lets a CU hold
     const int grid = (int) std::max(1l, std::min<long>((long) per_cu * cu_count(), tiles));
+    a.gate = gate;
     k_q8s_gemv<<<grid, Q8S_WAVES * 64, lds, (hipStream_t) st>>>(a);
     return launch_status(who);
 }
@@ -1240,8 +1242,11 @@ int fnx_attn_prep_append(float* qg, float* k, const float* v, const float* q_nor
 // splits for a context of up to max_ctx positions
 static int attn_splits(int max_ctx) { return (max_ctx + AT_SPLIT - 1) / AT_SPLIT; }
 size_t fnx_attn_scratch_floats(int nq, int T, int max_ctx) { return (size_t) T * nq * attn_splits(max_ctx) * (AT_HD + 2); }
+static int q8s_one(const fnx_q8s* W, const void* yq, float* out, int out_stride, int T, void* st, const int* gate) {
+    return q8s_launch(&W, &out, &out_stride, 1, yq, T, st, "q8s_gemv", gate);
+}
 static int attn_launch(const float* qg, const uint16_t* kc, const uint16_t* vc, float* out, uint8_t* outq, int nq, int nkv, const int* pos0, int T,
-                       int max_ctx, float* scratch, void* st) {
+                       int max_ctx, float* scratch, void* st, const int* gate = nullptr) {
     if (!qg || !kc || !vc || (!out && !outq) || !pos0 || !scratch) return fail("attn: null argument");
     if (nq < 1 || nkv < 1 || nq % nkv || nq / nkv > AT_MAXQ || T < 1 || T > FNX_MAXT || max_ctx < 1) return fail("attn: bad shape");
     if (attn_splits(max_ctx) > AT_MAXSPLIT) return fail("attn: the cache is larger than the split table");
@@ -1250,7 +1255,7 @@ static int attn_launch(const float* qg, const uint16_t* kc, const uint16_t* vc, 
     float* acc = scratch;
     AttPart* mz = reinterpret_cast<AttPart*>(scratch + (size_t) T * nq * nsplit * AT_HD);
     k_attn_part<<<dim3(nsplit, nkv, (waves + AT_WAVES - 1) / AT_WAVES), 64 * AT_WAVES, 0, (hipStream_t) st>>>(qg, kc, vc, acc, mz, nq, nkv, T,
-                                                                                                          nsplit, pos0);
+                                                                                                          nsplit, pos0, gate);
     k_attn_combine<<<dim3(nq, T), AT_HD, 0, (hipStream_t) st>>>(qg, acc, mz, out, outq, nq, nsplit, T, pos0);
     return launch_status("attn");
 }
@@ -1295,20 +1300,21 @@ static int dec_add_norm_q8(const fnx_decoder* D, const DecPending& pend, const f
 // x (ws->x) through one layer, in place; the layer's own MoE output is left pending for whatever comes next
 // live (may be null): a device word, how many of the T rows count; the others still pass through the attention (their
 // cache cells are overwritten by the next window) but are not routed, so they pull no expert's weights
+// gate (may be null): a device word; at zero the layer's dense products and its attention's scan leave at once
 static int dec_layer(const fnx_decoder* D, const fnx_dec_layer* L, int T, const int* pos0, const fnx_dec_ws* ws, DecPending& pend, void* st,
-                     const int* live = nullptr) {
+                     const int* live = nullptr, const int* gate = nullptr) {
     const int n = D->n, nq = D->nq, nkv = D->nkv;
     if (dec_add_norm_q8(D, pend, L->attn_norm, T, ws, st)) return 1;
     {   // q, k and v in one launch (engine.cu:1547-1552)
         const fnx_q8s* w3[3] = {&L->wq, &L->wk, &L->wv};
         float* const o3[3] = {ws->qg, ws->k, ws->v};
         const int s3[3] = {nq * 2 * AT_HD, nkv * AT_HD, nkv * AT_HD};
-        if (fnx_q8s_gemv_segs(w3, o3, s3, 3, ws->xq, T, st)) return 1;
+        if (q8s_launch(w3, o3, s3, 3, ws->xq, T, st, "q8s_gemv_segs", gate)) return 1;
     }
     if (fnx_attn_prep_append(ws->qg, ws->k, ws->v, L->q_norm, L->k_norm, L->kc, L->vc, nq, nkv, T, pos0, D->max_ctx, D->eps, &D->rope, st)) return 1;
     // the attention's rows leave its last kernel in q8_1 form, ready for the output projection
-    if (attn_launch(ws->qg, L->kc, L->vc, nullptr, (uint8_t*) ws->xq, nq, nkv, pos0, T, D->max_ctx, ws->attn_scratch, st)) return 1;
-    if (fnx_q8s_gemv(&L->wo, ws->xq, ws->o, n, T, st)) return 1;
+    if (attn_launch(ws->qg, L->kc, L->vc, nullptr, (uint8_t*) ws->xq, nq, nkv, pos0, T, D->max_ctx, ws->attn_scratch, st, gate)) return 1;
+    if (q8s_one(&L->wo, ws->xq, ws->o, n, T, st, gate)) return 1;
     if (fnx_add_norm_q8(ws->x, ws->o, L->ffn_norm, ws->xn, nullptr, T, n, D->eps, st)) return 1;
     if (layer_fused_ok(&L->moe, T)) {   // the window without its combine
         pend = DecPending{nullptr, &L->moe, nullptr, live};
@@ -1326,9 +1332,10 @@ static int dec_shape_check(const fnx_decoder* D, int T, const char* who) {
     return 0;
 }
 // x += pending; hidden = x; the output norm, the head, argmax
-static int dec_head(const fnx_decoder* D, const float* norm, const fnx_q8s* head, int T, const fnx_dec_ws* ws, const DecPending& pend, void* st) {
+static int dec_head(const fnx_decoder* D, const float* norm, const fnx_q8s* head, int T, const fnx_dec_ws* ws, const DecPending& pend, void* st,
+                    const int* gate = nullptr) {
     if (dec_add_norm_q8(D, pend, norm, T, ws, st, ws->hidden)) return 1;   // hidden = x, written by the same pass
-    if (fnx_q8s_gemv(head, ws->xq, ws->logits, D->vocab, T, st)) return 1;
+    if (q8s_one(head, ws->xq, ws->logits, D->vocab, T, st, gate)) return 1;
     return fnx_argmax(ws->logits, D->vocab, T, 0, ws->best_v, ws->best_i, ws->keys, ws->err, st);
 }
 static int decoder_verify(const fnx_decoder* D, const int* tokens, int T, const int* pos0, const fnx_dec_ws* ws, void* st, const int* live) {
@@ -1343,13 +1350,13 @@ int fnx_decoder_verify(const fnx_decoder* D, const int* tokens, int T, const int
     return decoder_verify(D, tokens, T, pos0, ws, st, nullptr);
 }
 static int mtp_draft(const fnx_decoder* D, const fnx_mtp* M, const float* src, const int* tokens, int T, const int* pos0, const fnx_dec_ws* ws,
-                     void* st, const int* live) {
+                     void* st, const int* live, const int* gate = nullptr) {
     if (!D || !M || !src || !tokens || !pos0 || !ws || !M->norm_emb || !M->norm_hid || !M->out_norm || !D->emb) return fail("mtp_draft: null argument");
     if (dec_shape_check(D, T, "mtp_draft") || dec_ws_check(ws, "mtp_draft")) return 1;
     const int n = D->n;
     // R = fc_hid(rms(src)) + fc_emb(rms(emb)): the sum is taken by the layer's first pass over the rows
     if (fnx_add_norm_q8(const_cast<float*>(src), nullptr, M->norm_hid, nullptr, ws->xq, T, n, D->eps, st)) return 1;   // nothing to add: src is only read
-    if (fnx_q8s_gemv(&M->fc_hid, ws->xq, ws->x, n, T, st)) return 1;
+    if (q8s_one(&M->fc_hid, ws->xq, ws->x, n, T, st, gate)) return 1;
     {   // the tokens' embedding rows, normed and quantised by the pass that reads them from the table (rms(emb[tokens]))
         CombineArgs c{};
         c.emb = D->emb;
@@ -1358,10 +1365,10 @@ static int mtp_draft(const fnx_decoder* D, const fnx_mtp* M, const float* src, c
         k_add_norm_q8<false><<<T, 256, 0, (hipStream_t) st>>>(ws->xn, nullptr, c, M->norm_emb, nullptr, (uint8_t*) ws->xq, n, D->eps);
         if (launch_status("mtp_draft")) return 1;
     }
-    if (fnx_q8s_gemv(&M->fc_emb, ws->xq, ws->o, n, T, st)) return 1;
+    if (q8s_one(&M->fc_emb, ws->xq, ws->o, n, T, st, gate)) return 1;
     DecPending pend{ws->o, nullptr, nullptr, nullptr};
-    if (dec_layer(D, &M->layer, T, pos0, ws, pend, st, live)) return 1;
-    return dec_head(D, M->out_norm, &M->head, T, ws, pend, st);
+    if (dec_layer(D, &M->layer, T, pos0, ws, pend, st, live, gate)) return 1;
+    return dec_head(D, M->out_norm, &M->head, T, ws, pend, st, gate);
 }
 int fnx_mtp_draft(const fnx_decoder* D, const fnx_mtp* M, const float* src, const int* tokens, int T, const int* pos0, const fnx_dec_ws* ws,
                   void* st) {
@@ -1373,6 +1380,9 @@ int fnx_decode_round(const fnx_decoder* D, const fnx_mtp* M, const fnx_round* R,
     if (R->ctx_cap < 2 * FNX_MAXT || R->log_cap < 0 || (R->log_cap > 0 && !R->log)) return fail("decode_round: bad buffer sizes");
     if (R->speculate && (R->key_n < 1 || R->key_n > 4 || R->lk < 0 || R->lk > FNX_MAXT - 1))
         return fail("decode_round: keys of 1..4 tokens, up to 15 drafts");
+    const int K = R->speculate ? std::max(R->chain, 1) : 1;
+    if (K > FNX_MAXT - 1) return fail("decode_round: a chain of up to 15 drafts");
+    if (K > 1 && !R->chain_src) return fail("decode_round: the chain needs its source row's buffer");
     hipStream_t s = (hipStream_t) st;
     int* S = R->state;
     if (decoder_verify(D, R->rows, FNX_MAXT, S + FNX_RS_POS, ws, st, S + FNX_RS_ROWS)) return 1;
@@ -1382,6 +1392,16 @@ int fnx_decode_round(const fnx_decoder* D, const fnx_mtp* M, const fnx_round* R,
         if (mtp_draft(D, M, ws->hidden, ws->best_i, FNX_MAXT, S + FNX_RS_POS_PREV, ws, st, S + FNX_RS_ACCEPTED)) return 1;
         k_lookup<<<1, LK_THREADS, 0, s>>>(R->ctx, 0, R->key_n, R->lk, ws->best_i, R->scratch + 1, R->scratch, nullptr, S + FNX_RS_NCTX,
                                           S + FNX_RS_ACCEPTED);
+        if (K > 1) {
+            // the chain (session.cpp:666-678): step j reads the draft before it at the position after it, from the draft
+            // layer's own row; one row, which counts (is routed, runs the big kernels) only while state[CHAIN] is set
+            const int* on = S + FNX_RS_CHAIN;
+            k_chain_begin<<<1, 256, 0, s>>>(S, R->scratch, ws->best_i, ws->hidden, D->n, R->chain_src, K);
+            for (int j = 1; j < K; ++j) {
+                if (mtp_draft(D, M, j == 1 ? R->chain_src : ws->hidden, R->scratch + j, 1, S + FNX_RS_CHAIN_POS + (j - 1), ws, st, on, on)) return 1;
+                k_chain_keep<<<1, 64, 0, s>>>(S, R->scratch, ws->best_i, j, K);
+            }
+        }
     }
     k_round_window<<<1, 64, 0, s>>>(R->ctx, S, R->scratch + 1, R->scratch, ws->best_i, R->speculate, R->rows);
     return launch_status("decode_round");

@@ -188,11 +188,13 @@ struct Q8sArgs {
     Q8sSeg seg[3];       // up to three matrices over the same activations, their 16-row tiles one after another
     int nseg, cols, T;
     const uint8_t* yq;   // q8_1 rows
+    const int* gate;     // may be null; else a device word: at zero the launch leaves at once (a chain step that does not count)
 };
 typedef int q8s_v4i __attribute__((ext_vector_type(4)));
 __global__ void __launch_bounds__(Q8S_WAVES * 64) k_q8s_gemv(const Q8sArgs a) {
     typedef __attribute__((address_space(1))) const at_v4u_t g128;
     extern __shared__ __align__(16) uint8_t q8s_lds[];   // [16][cols + pad] int8, [16][nb + 2] f32 scales, [3][64][4] partial sums
+    if (a.gate && uniform(*a.gate) == 0) return;
     const int nb = a.cols >> 5, T = a.T, xld = a.cols + Q8S_XPAD, dld = nb + 2;
     int8_t* xs = reinterpret_cast<int8_t*>(q8s_lds);
     float* xd = reinterpret_cast<float*>(q8s_lds + (size_t) FNX_MAXT * xld);
@@ -435,8 +437,9 @@ constexpr int AT_WAVES = 4, AT_KLD = 2 * AT_HD + 16;   // q tiles (of 16 queries
 __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) k_attn_part(const float* __restrict__ qg, const uint16_t* __restrict__ kc,
                                                             const uint16_t* __restrict__ vc, float* __restrict__ acc_out,
                                                             AttPart* __restrict__ mz_out, int nq, int nkv, int T, int nsplit,
-                                                            const int* __restrict__ pos0p) {
+                                                            const int* __restrict__ pos0p, const int* __restrict__ gate) {
     typedef __attribute__((address_space(1))) const at_v4u g128;
+    if (gate && uniform(*gate) == 0) return;   // a chain step that does not count: its parts stay what they were, nothing reads the result
     const int s = blockIdx.x, kvh = blockIdx.y, lane = threadIdx.x & 63, wave = blockIdx.z * AT_WAVES + (threadIdx.x >> 6);
     const int qpk = nq / nkv, nquery = T * qpk, pos0 = *pos0p;
     const int ql = lane & 15, pg = lane >> 4;

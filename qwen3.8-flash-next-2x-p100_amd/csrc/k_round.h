@@ -43,6 +43,30 @@ __global__ void k_round_commit(const int* __restrict__ rows, const int* __restri
     }
 }
 
+// the MTP chain (session.cpp:666-678) starts when the lookup found nothing: its first draft is the draft layer's pick for
+// the last row kept, its source that row of the draft layer's output. The steps' positions are written in any case (a
+// step that does not count still appends its row to the draft layer's cache, in cells that the next round's pass over the
+// rows kept writes again before anything reads them). One block.
+__global__ void k_chain_begin(int* __restrict__ state, int* __restrict__ scratch, const int* __restrict__ draft_best,
+                              const float* __restrict__ hidden, int n, float* __restrict__ chain_src, int K) {
+    const int kept = min(max(state[FNX_RS_ACCEPTED], 1), FNX_MAXT), pos = state[FNX_RS_POS];
+    const bool run = !state[FNX_RS_STOP] && scratch[0] <= 0;
+    __syncthreads();   // every thread has read the words that thread 0 is about to write
+    if (threadIdx.x < FNX_MAXT) state[FNX_RS_CHAIN_POS + threadIdx.x] = pos + threadIdx.x;
+    if (threadIdx.x == 0) {
+        state[FNX_RS_CHAIN] = run ? 1 : 0;
+        if (run) scratch[1] = draft_best[kept - 1];
+    }
+    if (run)
+        for (int i = threadIdx.x; i < n; i += blockDim.x) chain_src[i] = hidden[(size_t) (kept - 1) * n + i];
+}
+// after step j (1 .. K - 1) of the chain: its pick is draft j + 1; the last step hands the K drafts to the next window
+__global__ void k_chain_keep(const int* __restrict__ state, int* __restrict__ scratch, const int* __restrict__ best, int j, int K) {
+    if (threadIdx.x != 0 || !state[FNX_RS_CHAIN]) return;
+    scratch[1 + j] = best[0];
+    if (j == K - 1) scratch[0] = K;
+}
+
 // the next window (session.cpp:530-560): the last token of the context, then the lookup's drafts, or else the draft
 // layer's pick for the last row kept; without speculation the token alone. One wave.
 __global__ void k_round_window(const int* __restrict__ ctx, int* __restrict__ state, const int* __restrict__ drafts,

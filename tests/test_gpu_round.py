@@ -45,7 +45,7 @@ def repeating_prompt(seed):
 class RoundDev:
     """a DecoderDev whose prompt has been read, plus the device words of fnx_decode_round"""
 
-    def __init__(self, dev, model, prompt, speculate=True, lk=15, ctx_cap=512):
+    def __init__(self, dev, model, prompt, speculate=True, lk=15, ctx_cap=512, chain=0):
         t, pkg = dev.torch, dev.pkg
         self.dev, self.d, self.prompt, self.pkg = dev, fnx_gpu.DecoderDev(dev, model), list(prompt), pkg
         d = self.d
@@ -60,8 +60,9 @@ class RoundDev:
         self.ctx[:len(prompt)] = t.tensor(self.prompt, dtype=t.int32)
         self.state[pkg.RS_NCTX], self.state[pkg.RS_POS], self.state[pkg.RS_ROWS] = len(prompt), len(prompt) - 1, 1
         self.rows[0] = self.prompt[-1]
+        self.chain_src = dev.zeros(model.cfg["n"], t.float32)
         self.R = pkg.Round(self.state.data_ptr(), self.rows.data_ptr(), self.ctx.data_ptr(), ctx_cap, self.log.data_ptr(), 64, int(speculate), 3, lk,
-                           self.scratch.data_ptr())
+                           self.scratch.data_ptr(), chain, self.chain_src.data_ptr())
 
     def launch(self):
         d, dev = self.d, self.dev
@@ -76,11 +77,12 @@ class RoundDev:
         return out, [(int(a), int(b)) for a, b in log], st
 
 
-def host_loop(dev, model, prompt, max_new, speculate=True):
+def host_loop(dev, model, prompt, max_new, speculate=True, K=1, lk=15):
     def lookup_dev(ctx, lk, d1):
         return dev.lookup(np.asarray(ctx, dtype=np.int32), lk, d1)
 
-    return td.spec_generate(fnx_gpu.DecoderDev(dev, model), lookup_dev, lambda r, o: dev.accept(r, o), prompt, max_new, K=1, speculate=speculate)
+    return td.spec_generate(fnx_gpu.DecoderDev(dev, model), lookup_dev, lambda r, o: dev.accept(r, o), prompt, max_new, K=K, lk=lk,
+                            speculate=speculate)
 
 
 def test_verify_window_at_hidden_2048_matches_oracle(dev, oracle, model):
@@ -130,17 +132,46 @@ def test_rounds_without_the_host_equal_the_host_driven_rounds(dev, oracle, model
         assert all(entry == (0, 1) for entry in log)
 
 
-def test_rounds_replayed_from_one_graph(dev, oracle, cyclic_model):
+@pytest.mark.parametrize("which,K,lk", [("random", 3, 15), ("cyclic", 3, 15), ("cyclic", 4, 0)])
+def test_rounds_with_an_mtp_chain_equal_the_host_driven_rounds(dev, oracle, model, cyclic_model, which, K, lk):
+    # session.cpp:666-678: when the lookup finds nothing, K - 1 more drafts from the draft layer's own rows. Random
+    # weights: every round offers K drafts and keeps one token; the cyclic model with the lookup: most rounds take the
+    # lookup's drafts and the chain's launches leave on the device word; without the lookup (lk = 0): every round runs the
+    # chain, and its drafts are right
+    model = cyclic_model if which == "cyclic" else model
+    prompt = [t % model.cfg["vocab"] for t in repeating_prompt(12)]
+    r = RoundDev(dev, model, prompt, lk=lk, chain=K)
+    nrounds = 12
+    print(f"case decode_round chain model={which} K={K} lk={lk} rounds={nrounds}", flush=True)
+    for _ in range(nrounds):
+        r.launch()
+    out, log, st = r.result()
+    print("rounds", log, flush=True)
+    assert st[dev.pkg.RS_STOP] == 0 and st[dev.pkg.RS_ROUNDS] == nrounds and len(out) == sum(k for _, k in log)
+    assert int(r.d.b["err"].item()) == 0
+    out_h, rounds_h = host_loop(dev, model, prompt, len(out), K=K, lk=lk)
+    assert out == out_h, "the same tokens as the loop that waits for every step"
+    assert log == rounds_h, "and the same drafts offered and tokens kept, round by round"
+    if which == "random":
+        assert all(dr == K for dr, _ in log[1:]), "every round after the first offers the whole chain"
+    elif lk == 0:
+        assert all(dr == K for dr, _ in log[1:]) and max(k for _, k in log) > 2, "the chain's drafts were kept"
+    else:
+        assert max(dr for dr, _ in log) > K, "the lookup fired on some rounds"
+
+
+@pytest.mark.parametrize("chain,lk", [(0, 15), (3, 15), (3, 0)])
+def test_rounds_replayed_from_one_graph(dev, oracle, cyclic_model, chain, lk):
     torch = dev.torch
     model = cyclic_model
     prompt = [t % model.cfg["vocab"] for t in repeating_prompt(14)]
-    e = RoundDev(dev, model, prompt)
+    e = RoundDev(dev, model, prompt, lk=lk, chain=chain)
     nrounds = 16
     for _ in range(nrounds):
         e.launch()
     out_e, log_e, _ = e.result()
-    g = RoundDev(dev, model, prompt)
-    print("case decode_round graph", flush=True)
+    g = RoundDev(dev, model, prompt, lk=lk, chain=chain)
+    print(f"case decode_round graph chain={chain} lk={lk}", flush=True)
     g.launch()   # the first round eagerly; it is not part of the graph
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
