@@ -135,7 +135,7 @@ def main():
 
     # ---- the dominant kernel: the window's gate|up launch (routed experts + the shared expert), timed with events the
     # library records on the launch stream around each of the window's five launches (fnx_layer_profile)
-    names = ["router+q8_1", "topk/jobs/plan", "gate|up", "down", "combine"]
+    names = ["router+q8_1", "top-k", "plan+gate|up", "down", "combine"]
     per_launch = np.zeros(5)
     reps = max(50, min(args.steps, 200))
     ms5 = np.zeros(5, dtype=np.float32)

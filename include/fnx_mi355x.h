@@ -139,8 +139,8 @@ int fnx_accept_greedy_dev(const int* rows, const int* o, int R, int* n_accept, v
 /* ---- the whole MoE half of a verify window (engine.cu:1569-1757 Engine::ffn_half without cards and streaming):
  * quantize -> router_route -> gate|up (routed + shared) -> swiglu q8_1 -> down (routed + shared) -> combine.
  * Same results as the calls above made one by one (up to the order of a few float additions). With unit64 weights,
- * n = 2048 and ff of 256, 512 or 1024 the window runs in five launches: [router logits | q8_1 rows], [top-k, jobs],
- * [gate|up routed + shared], [SwiGLU + down routed + shared], [combine]; other shapes run operator by operator.
+ * n = 2048 and ff of 256, 512 or 1024 the window runs in five launches: [router logits | q8_1 rows], [top-k],
+ * [jobs + gate|up routed + shared], [SwiGLU + down routed + shared], [combine]; other shapes run operator by operator.
  * Like moe_down, one MoE may be in flight per device. */
 typedef struct fnx_moe_layer {
     int n, ff, nexp, topk;   /* hidden, expert width, experts, picks per token */
@@ -169,7 +169,7 @@ int fnx_moe_verify_layer(const fnx_moe_layer* L, const float* x, int T, float* o
 /* Profiling aid, the counterpart of the reference's FNX_PROF stamps in its window graph (engine.cu:1382-1530):
  * fnx_layer_profile(1) makes the five-launch window record events on its stream around each launch (not to be
  * used under graph capture), fnx_layer_profile(0) stops that; fnx_layer_profile_read waits for the last recorded
- * window and returns its five launches' durations in milliseconds: router + q8_1 rows, top-k/jobs/plan, gate|up,
+ * window and returns its five launches' durations in milliseconds: router + q8_1 rows, top-k, jobs + gate|up,
  * down, combine. One profiled window at a time per process. */
 int fnx_layer_profile(int on);
 int fnx_layer_profile_read(float* ms5);

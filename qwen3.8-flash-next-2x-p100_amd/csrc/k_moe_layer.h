@@ -1,5 +1,5 @@
 // The MoE half of a verify window (the work of Engine::ffn_half, engine.cu:1569-1757 of the reference, on one GPU) in
-// five launches: [router logits | q8_1 rows of x] -> [top-k, jobs, plan] -> [gate|up, routed and shared] ->
+// five launches: [router logits | q8_1 rows of x] -> [top-k] -> [jobs and plan, gate|up, routed and shared] ->
 // [SwiGLU to q8_1 on the fly + down, routed and shared] -> [combine].
 //
 // Arithmetic is the operators': the router sums in the fixed 64-lane order, top-k by (value, lower index), the q8_1
