@@ -158,6 +158,15 @@ def test_rounds_with_an_mtp_chain_equal_the_host_driven_rounds(dev, oracle, mode
         assert all(dr == K for dr, _ in log[1:]) and max(k for _, k in log) > 2, "the chain's drafts were kept"
     else:
         assert max(dr for dr, _ in log) > K, "the lookup fired on some rounds"
+    # fnx_run.cpp:1198-1238: whatever is drafted, the tokens are those of plain greedy decoding
+    plain = RoundDev(dev, model, prompt, speculate=False)
+    for _ in range(len(out)):
+        plain.launch()
+    out_p, _, _ = plain.result()
+    assert out_p[:len(out)] == out
+    out_o, _ = td.spec_generate(td.OracleSession(model), lambda c, lk_, d1: oracle.lookup_drafts(np.asarray(c, dtype=np.int32), lk_, d1),
+                                lambda rw, o: oracle.accept_greedy(rw, o), prompt, len(out), K=K, lk=lk)
+    assert same_until_near_tie(oracle, model, prompt, out, out_o) >= min(8, len(out))
 
 
 @pytest.mark.parametrize("chain,lk", [(0, 15), (3, 15), (3, 0)])
