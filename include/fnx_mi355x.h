@@ -310,7 +310,7 @@ int fnx_mtp_draft(const fnx_decoder* D, const fnx_mtp* M, const float* src, cons
  * a graph and replayed. When the lookup finds nothing the MTP chain follows (session.cpp:666-678, at a fixed length
  * fnx_round.chain; the reference's adaptive length and its min_p cut are the host's): each further draft is the draft
  * layer's pick for the draft before, from its own hidden row. Its launches are always enqueued; in a round whose lookup
- * found drafts their big kernels (the dense products, the attention's scan, the experts) leave at once on a device word. */
+ * found drafts their kernels leave at once on a device word. */
 enum {
     FNX_RS_NCTX = 0,     /* tokens in ctx: the prompt and everything emitted */
     FNX_RS_POS = 1,      /* cache position of the window's first row (= FNX_RS_NCTX - 1) */

@@ -772,7 +772,7 @@ static int layer_fused(const fnx_moe_layer* L, const float* x, int T, float* out
     const int n = L->n, ff = L->ff, P = T * L->topk, LS = L->nexp + 1;
     const int rblocks = (LS + RQ_ROWS - 1) / RQ_ROWS, qblocks = (T * 64 + 2 * FL_WAVES - 1) / (2 * FL_WAVES);
     prof_mark(0, s);
-    k_router_quant<<<rblocks + qblocks, FL_THREADS, 0, s>>>(RouterArgs{L->nexp, T, x, L->router, L->router_bf16, ws->logits, (uint8_t*) ws->xq});
+    k_router_quant<<<rblocks + qblocks, FL_THREADS, 0, s>>>(RouterArgs{L->nexp, T, x, L->router, L->router_bf16, ws->logits, (uint8_t*) ws->xq, live});
     prof_mark(1, s);
     const RouteArgs route{L->nexp, L->topk, T, ws->logits, ws->topi, ws->topw, ws->jobs_gu, ws->jobs_dn, ws->njobs, live};
     k_route_topk<<<T, RT_THREADS, 0, s>>>(route);
@@ -1220,8 +1220,9 @@ int fnx_q8s_gemv(const fnx_q8s* W, const void* yq, float* out, int out_stride, i
 int fnx_q8s_gemv_segs(const fnx_q8s* const* W, float* const* out, const int* out_stride, int n, const void* yq, int T, void* st) {
     return q8s_launch(W, out, out_stride, n, yq, T, st, "q8s_gemv_segs");
 }
-int fnx_attn_prep_append(float* qg, float* k, const float* v, const float* q_norm, const float* k_norm, uint16_t* kc, uint16_t* vc, int nq,
-                         int nkv, int T, const int* pos0, int max_ctx, float eps, const fnx_rope* rope, void* st) {
+}  // extern "C"
+static int attn_prep_append(float* qg, float* k, const float* v, const float* q_norm, const float* k_norm, uint16_t* kc, uint16_t* vc, int nq,
+                            int nkv, int T, const int* pos0, int max_ctx, float eps, const fnx_rope* rope, void* st, const int* gate) {
     if (!qg || !k || !v || !q_norm || !k_norm || !kc || !vc || !pos0 || !rope) return fail("attn_prep_append: null argument");
     if (nq < 1 || nkv < 1 || nq % nkv || T < 1 || T > FNX_MAXT || max_ctx < 4 || max_ctx % 4) return fail("attn_prep_append: bad shape (the cache holds a multiple of 4 positions)");
     RopeDev r;
@@ -1236,8 +1237,13 @@ int fnx_attn_prep_append(float* qg, float* k, const float* v, const float* q_nor
         r.freq[pair] = f;
     }
     r.mscale = rope->mscale;
-    k_attn_prep_append<<<dim3(nq + 2 * nkv, T), AT_HD, 0, (hipStream_t) st>>>(qg, k, v, q_norm, k_norm, kc, vc, nq, nkv, pos0, max_ctx, eps, r);
+    k_attn_prep_append<<<dim3(nq + 2 * nkv, T), AT_HD, 0, (hipStream_t) st>>>(qg, k, v, q_norm, k_norm, kc, vc, nq, nkv, pos0, max_ctx, eps, r, gate);
     return launch_status("attn_prep_append");
+}
+extern "C" {
+int fnx_attn_prep_append(float* qg, float* k, const float* v, const float* q_norm, const float* k_norm, uint16_t* kc, uint16_t* vc, int nq,
+                         int nkv, int T, const int* pos0, int max_ctx, float eps, const fnx_rope* rope, void* st) {
+    return attn_prep_append(qg, k, v, q_norm, k_norm, kc, vc, nq, nkv, T, pos0, max_ctx, eps, rope, st, nullptr);
 }
 // splits for a context of up to max_ctx positions
 static int attn_splits(int max_ctx) { return (max_ctx + AT_SPLIT - 1) / AT_SPLIT; }
@@ -1256,7 +1262,7 @@ static int attn_launch(const float* qg, const uint16_t* kc, const uint16_t* vc, 
     AttPart* mz = reinterpret_cast<AttPart*>(scratch + (size_t) T * nq * nsplit * AT_HD);
     k_attn_part<<<dim3(nsplit, nkv, (waves + AT_WAVES - 1) / AT_WAVES), 64 * AT_WAVES, 0, (hipStream_t) st>>>(qg, kc, vc, acc, mz, nq, nkv, T,
                                                                                                           nsplit, pos0, gate);
-    k_attn_combine<<<dim3(nq, T), AT_HD, 0, (hipStream_t) st>>>(qg, acc, mz, out, outq, nq, nsplit, T, pos0);
+    k_attn_combine<<<dim3(nq, T), AT_HD, 0, (hipStream_t) st>>>(qg, acc, mz, out, outq, nq, nsplit, T, pos0, gate);
     return launch_status("attn");
 }
 int fnx_attn(const float* qg, const uint16_t* kc, const uint16_t* vc, float* out, int nq, int nkv, const int* pos0, int T, int max_ctx,
@@ -1279,14 +1285,16 @@ struct DecPending {
     const int* live;     // with moe: the device word that said how many rows were routed, or null
 };
 // xcopy (may be null): the rows after the add go there too
-static int dec_add_norm_q8(const fnx_decoder* D, const DecPending& pend, const float* w, int T, const fnx_dec_ws* ws, void* st, float* xcopy = nullptr) {
+static int dec_add_norm_q8(const fnx_decoder* D, const DecPending& pend, const float* w, int T, const fnx_dec_ws* ws, void* st, float* xcopy = nullptr,
+                           const int* gate = nullptr) {
     CombineArgs c{};
     if (pend.moe) {
         const fnx_moe_layer* M = pend.moe;
         c = CombineArgs{ws->moe.part, ws->moe.topw, ws->moe.part + (size_t) T * M->topk * D->n, ws->moe.logits + M->nexp, M->nexp + 1, M->topk, nullptr,
-                        nullptr, nullptr, 0, pend.live};
+                        nullptr, nullptr, 0, pend.live, nullptr};
     }
     c.xcopy = xcopy;
+    c.gate = gate;
     if (pend.tokens) {
         c.emb = D->emb;
         c.tokens = pend.tokens;
@@ -1304,18 +1312,23 @@ static int dec_add_norm_q8(const fnx_decoder* D, const DecPending& pend, const f
 static int dec_layer(const fnx_decoder* D, const fnx_dec_layer* L, int T, const int* pos0, const fnx_dec_ws* ws, DecPending& pend, void* st,
                      const int* live = nullptr, const int* gate = nullptr) {
     const int n = D->n, nq = D->nq, nkv = D->nkv;
-    if (dec_add_norm_q8(D, pend, L->attn_norm, T, ws, st)) return 1;
+    if (dec_add_norm_q8(D, pend, L->attn_norm, T, ws, st, nullptr, gate)) return 1;
     {   // q, k and v in one launch (engine.cu:1547-1552)
         const fnx_q8s* w3[3] = {&L->wq, &L->wk, &L->wv};
         float* const o3[3] = {ws->qg, ws->k, ws->v};
         const int s3[3] = {nq * 2 * AT_HD, nkv * AT_HD, nkv * AT_HD};
         if (q8s_launch(w3, o3, s3, 3, ws->xq, T, st, "q8s_gemv_segs", gate)) return 1;
     }
-    if (fnx_attn_prep_append(ws->qg, ws->k, ws->v, L->q_norm, L->k_norm, L->kc, L->vc, nq, nkv, T, pos0, D->max_ctx, D->eps, &D->rope, st)) return 1;
+    if (attn_prep_append(ws->qg, ws->k, ws->v, L->q_norm, L->k_norm, L->kc, L->vc, nq, nkv, T, pos0, D->max_ctx, D->eps, &D->rope, st, gate)) return 1;
     // the attention's rows leave its last kernel in q8_1 form, ready for the output projection
     if (attn_launch(ws->qg, L->kc, L->vc, nullptr, (uint8_t*) ws->xq, nq, nkv, pos0, T, D->max_ctx, ws->attn_scratch, st, gate)) return 1;
     if (q8s_one(&L->wo, ws->xq, ws->o, n, T, st, gate)) return 1;
-    if (fnx_add_norm_q8(ws->x, ws->o, L->ffn_norm, ws->xn, nullptr, T, n, D->eps, st)) return 1;
+    {   // x += o; xn = norm(x) (fnx_add_norm_q8)
+        CombineArgs c{};
+        c.gate = gate;
+        k_add_norm_q8<false><<<T, 256, 0, (hipStream_t) st>>>(ws->x, ws->o, c, L->ffn_norm, ws->xn, nullptr, n, D->eps);
+        if (launch_status("decoder add_norm")) return 1;
+    }
     if (layer_fused_ok(&L->moe, T)) {   // the window without its combine
         pend = DecPending{nullptr, &L->moe, nullptr, live};
         return moe_layer_checked(&L->moe, ws->xn, T, nullptr, &ws->moe, st, live);
@@ -1334,7 +1347,7 @@ static int dec_shape_check(const fnx_decoder* D, int T, const char* who) {
 // x += pending; hidden = x; the output norm, the head, argmax
 static int dec_head(const fnx_decoder* D, const float* norm, const fnx_q8s* head, int T, const fnx_dec_ws* ws, const DecPending& pend, void* st,
                     const int* gate = nullptr) {
-    if (dec_add_norm_q8(D, pend, norm, T, ws, st, ws->hidden)) return 1;   // hidden = x, written by the same pass
+    if (dec_add_norm_q8(D, pend, norm, T, ws, st, ws->hidden, gate)) return 1;   // hidden = x, written by the same pass
     if (q8s_one(head, ws->xq, ws->logits, D->vocab, T, st, gate)) return 1;
     return fnx_argmax(ws->logits, D->vocab, T, 0, ws->best_v, ws->best_i, ws->keys, ws->err, st);
 }
@@ -1355,13 +1368,19 @@ static int mtp_draft(const fnx_decoder* D, const fnx_mtp* M, const float* src, c
     if (dec_shape_check(D, T, "mtp_draft") || dec_ws_check(ws, "mtp_draft")) return 1;
     const int n = D->n;
     // R = fc_hid(rms(src)) + fc_emb(rms(emb)): the sum is taken by the layer's first pass over the rows
-    if (fnx_add_norm_q8(const_cast<float*>(src), nullptr, M->norm_hid, nullptr, ws->xq, T, n, D->eps, st)) return 1;   // nothing to add: src is only read
+    {   // nothing to add: src is only read (fnx_add_norm_q8)
+        CombineArgs c{};
+        c.gate = gate;
+        k_add_norm_q8<false><<<T, 256, 0, (hipStream_t) st>>>(const_cast<float*>(src), nullptr, c, M->norm_hid, nullptr, (uint8_t*) ws->xq, n, D->eps);
+        if (launch_status("mtp_draft")) return 1;
+    }
     if (q8s_one(&M->fc_hid, ws->xq, ws->x, n, T, st, gate)) return 1;
     {   // the tokens' embedding rows, normed and quantised by the pass that reads them from the table (rms(emb[tokens]))
         CombineArgs c{};
         c.emb = D->emb;
         c.tokens = tokens;
         c.vocab = D->vocab;
+        c.gate = gate;
         k_add_norm_q8<false><<<T, 256, 0, (hipStream_t) st>>>(ws->xn, nullptr, c, M->norm_emb, nullptr, (uint8_t*) ws->xq, n, D->eps);
         if (launch_status("mtp_draft")) return 1;
     }

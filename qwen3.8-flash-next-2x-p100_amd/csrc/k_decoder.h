@@ -40,6 +40,7 @@ struct CombineArgs {
     const int* tokens;
     int vocab;
     const int* live;      // may be null; else a device word: rows from *live on were not routed and get no combine added
+    const int* gate;      // may be null; else a device word: at zero the launch leaves at once (a chain step that does not count)
 };
 // WIDE (the combine's form): 1024 threads make the row after the add - a thread the columns p, p + 1024, ..., with all
 // of an expert batch's partial sums in flight (256 threads with 8 columns each took 13 us a call, against 7 us without
@@ -50,6 +51,7 @@ __global__ void __launch_bounds__(WIDE ? 1024 : 256) k_add_norm_q8(float* __rest
                                                                   float eps) {
     __shared__ float sh[4];
     __shared__ float vrow[WIDE ? 256 * NQ_MAXJ : 1];
+    if (c.gate && uniform(*c.gate) == 0) return;
     const size_t row = blockIdx.x;
     float v[NQ_MAXJ];
     float s = 0.f;
@@ -348,9 +350,11 @@ struct RopeDev {
 __global__ void __launch_bounds__(AT_HD) k_attn_prep_append(float* __restrict__ qg, float* __restrict__ k, const float* __restrict__ v,
                                                            const float* __restrict__ qn, const float* __restrict__ kn,
                                                            uint16_t* __restrict__ kc, uint16_t* __restrict__ vc, int nq, int nkv,
-                                                           const int* __restrict__ pos0p, int max_ctx, float eps, RopeDev rope) {
+                                                           const int* __restrict__ pos0p, int max_ctx, float eps, RopeDev rope,
+                                                           const int* __restrict__ gate) {
     __shared__ float sh[AT_HD / 64];
     __shared__ float xs[AT_HD];
+    if (gate && uniform(*gate) == 0) return;   // a chain step that does not count appends nothing
     const int t = blockIdx.y, h = blockIdx.x, i = threadIdx.x, p = *pos0p + t;
     const bool is_q = h < nq, is_k = !is_q && h < nq + nkv;
     const int kh = h - nq - (is_k ? 0 : nkv);
@@ -625,9 +629,10 @@ __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per
 constexpr int AT_MAXSPLIT = 2048;
 __global__ void __launch_bounds__(AT_HD) k_attn_combine(const float* __restrict__ qg, const float* __restrict__ acc_in,
                                                        const AttPart* __restrict__ mz_in, float* __restrict__ out, uint8_t* __restrict__ outq,
-                                                       int nq, int nsplit, int T, const int* __restrict__ pos0p) {
+                                                       int nq, int nsplit, int T, const int* __restrict__ pos0p, const int* __restrict__ gate) {
     __shared__ float wsp[AT_MAXSPLIT];
     __shared__ float red[AT_HD / 64];
+    if (gate && uniform(*gate) == 0) return;
     const int h = blockIdx.x, t = blockIdx.y, i = threadIdx.x;
     const size_t base = ((size_t) t * nq + h) * nsplit;
     const int nlive = min(nsplit, (*pos0p + T + AT_SPLIT - 1) / AT_SPLIT);   // splits the window's context reaches: their parts were written

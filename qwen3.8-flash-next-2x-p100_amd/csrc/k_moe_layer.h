@@ -259,10 +259,12 @@ struct RouterArgs {
     int router_bf16;
     float* logits;
     uint8_t* xq;
+    const int* live;   // may be null; else a device word: with no row routed the launch leaves at once
 };
 constexpr int RQ_ROWS = 4;   // router rows per block: two waves per row, each with half of the window's rows
 __global__ void __launch_bounds__(FL_THREADS) k_router_quant(const RouterArgs a) {
     __shared__ float4 xt[FNX_MAXT][4][64];   // [token][chunk][lane]: half of x
+    if (a.live && uniform(*a.live) <= 0) return;
     const int tid = threadIdx.x, wave = uniform(tid >> 6), lane = tid & 63;
     const int T = a.T, n = FL_N, LS = a.nexp + 1;
     const int rblocks = (LS + RQ_ROWS - 1) / RQ_ROWS, b = blockIdx.x;
