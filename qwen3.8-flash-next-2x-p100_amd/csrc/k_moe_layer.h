@@ -435,9 +435,14 @@ __global__ void __launch_bounds__(FL_THREADS) k_moe_gate_up_passes(const PassArg
 // against 25 us, the block-wide barriers cost more than the repeated SwiGLU.)
 template <int SBR>
 __global__ void __launch_bounds__(FL_THREADS) k_moe_down_passes(const PassArgs a) {
-    constexpr int RW = 64 / SBR, VPL = 32 / RW;   // rows per unit; h values a lane makes
+    constexpr int RW = 64 / SBR;   // rows per unit
     __shared__ uint32_t tab[SGRID_WORDS];
     __shared__ LayerPlan pl;
+    // h = silu(gate) * up of the block's pairs in q8_1 form (k_moe_h, moe.cuh:597-608): per pair and 32-value block the
+    // 32 int8 values, then the block's scale as a float. A block's eight waves walk consecutive units, fewer than a pass
+    // has, so they are in two passes at most: four pairs, made once by the whole block ahead of the barrier that the
+    // codebook needs anyway (every wave making its own pairs' rows read the gate|up outputs 21 times over a pass).
+    __shared__ __align__(16) uint32_t hq[4][SBR][12];   // 8 words of values, the scale, 3 unused (16-byte rows)
     const int tid = threadIdx.x, wave = uniform(tid >> 6), lane = tid & 63;
     uint32_t treg[SGRID_WORDS / FL_THREADS];
 #pragma unroll
@@ -455,51 +460,61 @@ __global__ void __launch_bounds__(FL_THREADS) k_moe_down_passes(const PassArgs a
         s = pass_seg(pl, a, u, u1, upj);
         packed_first(s.we, s.ul, s.ue, cur);
     }
+    const int pass0 = (int) (total * ((long) blockIdx.x * FL_WAVES) / nw / upj);   // the block's first pass
+    {
+        constexpr int VPT = (SBR * 32 + FL_THREADS - 1) / FL_THREADS;   // values a thread and pair
+        float gv[4][VPT], uv[4][VPT];
+        bool on[4];
+#pragma unroll
+        for (int slot = 0; slot < 4; ++slot) {   // all the loads first: one trip to the cache for the four pairs
+            const int pi = pass0 + (slot >> 1), t = slot & 1;
+            const int pc = max(min(pi, pl.npass - 1), 0);
+            on[slot] = pi < pl.npass && pl.pass_t0[pc] + t < pl.job_n[pl.pass_job[pc]];
+            if (on[slot]) {   // the same for every thread of the block
+                const int ji = pl.pass_job[pi], pair = pl.job_pairs[ji][pl.pass_t0[pi] + t];
+                const float* gp = a.gu + (size_t) pair * 2 * ff;
+#pragma unroll
+                for (int k = 0; k < VPT; ++k) {
+                    const int i = tid + k * FL_THREADS;
+                    gv[slot][k] = i < ff ? gp[i] : 0.f;
+                    uv[slot][k] = i < ff ? gp[ff + i] : 0.f;
+                }
+            }
+        }
+#pragma unroll
+        for (int slot = 0; slot < 4; ++slot)
+            if (on[slot])
+#pragma unroll
+                for (int k = 0; k < VPT; ++k) {
+                    const int i = tid + k * FL_THREADS;
+                    if (i < ff) {   // whole 32-lane groups
+                        const float h = silu_f(gv[slot][k]) * uv[slot][k];
+                        const float amax = group_max<32>(fabsf(h));
+                        const float d = amax / 127.0f;
+                        const int q = amax == 0.0f ? 0 : (int) (int8_t) roundf(h / d);
+                        reinterpret_cast<int8_t*>(&hq[slot][i >> 5][0])[i & 31] = (int8_t) q;
+                        if ((i & 31) == 0) hq[slot][i >> 5][8] = __float_as_uint(half_bits_to_float(float_to_half_bits(d)));
+                    }
+                }
+    }
 #pragma unroll
     for (int i = 0; i < SGRID_WORDS / FL_THREADS; ++i) tab[tid + i * FL_THREADS] = treg[i];
     __syncthreads();
-    const int g = lane / SBR, kb = lane % SBR;
+    const int kb = lane % SBR;
     while (u < u1) {
-        const uint8_t* pairs = pl.job_pairs[s.ji] + s.t0;
+        const int slot0 = 2 * ((int) (u / upj) - pass0);   // 0 or 2
         auto prep_for = [&](auto nt_tag) {
             constexpr int NT = decltype(nt_tag)::value;
             return [=](int(&xs)[NT][8], float(&dx)[NT], float*(&orow)[NT]) {
+                const uint8_t* pairs = pl.job_pairs[s.ji] + s.t0;
 #pragma unroll
                 for (int t = 0; t < NT; ++t) {
-                    const int pair = uniform((int) pairs[t]);
-                    const float* gp = a.gu + (size_t) pair * 2 * ff + kb * 32 + g * VPL;
-                    float h[VPL];
-                    float amax = 0.f;
-#pragma unroll
-                    for (int j = 0; j < VPL; j += 4) {
-                        const float4 gv = *reinterpret_cast<const float4*>(gp + j), uv = *reinterpret_cast<const float4*>(gp + ff + j);
-                        h[j] = silu_f(gv.x) * uv.x;
-                        h[j + 1] = silu_f(gv.y) * uv.y;
-                        h[j + 2] = silu_f(gv.z) * uv.z;
-                        h[j + 3] = silu_f(gv.w) * uv.w;
-                    }
-#pragma unroll
-                    for (int j = 0; j < VPL; ++j) amax = fmaxf(amax, fabsf(h[j]));
-#pragma unroll
-                    for (int o = SBR; o < 64; o <<= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
-                    const float d = amax / 127.0f;
-                    int pk[VPL / 4];
-#pragma unroll
-                    for (int j = 0; j < VPL; j += 4) {
-                        uint32_t v = 0;
-#pragma unroll
-                        for (int k = 0; k < 4; ++k) {
-                            const int q = amax == 0.0f ? 0 : (int) (int8_t) roundf(h[j + k] / d);
-                            v |= ((uint32_t) q & 0xFFu) << (8 * k);
-                        }
-                        pk[j / 4] = (int) v;
-                    }
-#pragma unroll
-                    for (int gg = 0; gg < RW; ++gg)
-#pragma unroll
-                        for (int k = 0; k < VPL / 4; ++k) xs[t][gg * (VPL / 4) + k] = __shfl(pk[k], kb + SBR * gg, 64);
-                    dx[t] = half_bits_to_float(float_to_half_bits(d));
-                    orow[t] = a.out + (size_t) pair * a.rows;
+                    const uint32_t* hb = hq[slot0 + t][kb];
+                    const uint4 lo = *reinterpret_cast<const uint4*>(hb), hi = *reinterpret_cast<const uint4*>(hb + 4);
+                    xs[t][0] = (int) lo.x, xs[t][1] = (int) lo.y, xs[t][2] = (int) lo.z, xs[t][3] = (int) lo.w;
+                    xs[t][4] = (int) hi.x, xs[t][5] = (int) hi.y, xs[t][6] = (int) hi.z, xs[t][7] = (int) hi.w;
+                    dx[t] = __uint_as_float(hb[8]);
+                    orow[t] = a.out + (size_t) uniform((int) pairs[t]) * a.rows;
                 }
             };
         };
