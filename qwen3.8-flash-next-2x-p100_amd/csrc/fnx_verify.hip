@@ -1252,7 +1252,7 @@ static int q8s_one(const fnx_q8s* W, const void* yq, float* out, int out_stride,
     return q8s_launch(&W, &out, &out_stride, 1, yq, T, st, "q8s_gemv", gate);
 }
 static int attn_launch(const float* qg, const uint16_t* kc, const uint16_t* vc, float* out, uint8_t* outq, int nq, int nkv, const int* pos0, int T,
-                       int max_ctx, float* scratch, void* st, const int* gate = nullptr) {
+                       int max_ctx, float* scratch, void* st, const int* gate = nullptr, const int* live = nullptr) {
     if (!qg || !kc || !vc || (!out && !outq) || !pos0 || !scratch) return fail("attn: null argument");
     if (nq < 1 || nkv < 1 || nq % nkv || nq / nkv > AT_MAXQ || T < 1 || T > FNX_MAXT || max_ctx < 1) return fail("attn: bad shape");
     if (attn_splits(max_ctx) > AT_MAXSPLIT) return fail("attn: the cache is larger than the split table");
@@ -1261,8 +1261,8 @@ static int attn_launch(const float* qg, const uint16_t* kc, const uint16_t* vc, 
     float* acc = scratch;
     AttPart* mz = reinterpret_cast<AttPart*>(scratch + (size_t) T * nq * nsplit * AT_HD);
     k_attn_part<<<dim3(nsplit, nkv, (waves + AT_WAVES - 1) / AT_WAVES), 64 * AT_WAVES, 0, (hipStream_t) st>>>(qg, kc, vc, acc, mz, nq, nkv, T,
-                                                                                                          nsplit, pos0, gate);
-    k_attn_combine<<<dim3(nq, T), AT_HD, 0, (hipStream_t) st>>>(qg, acc, mz, out, outq, nq, nsplit, T, pos0, gate);
+                                                                                                          nsplit, pos0, gate, live);
+    k_attn_combine<<<dim3(nq, T), AT_HD, 0, (hipStream_t) st>>>(qg, acc, mz, out, outq, nq, nsplit, T, pos0, gate, live);
     return launch_status("attn");
 }
 int fnx_attn(const float* qg, const uint16_t* kc, const uint16_t* vc, float* out, int nq, int nkv, const int* pos0, int T, int max_ctx,
@@ -1306,8 +1306,8 @@ static int dec_add_norm_q8(const fnx_decoder* D, const DecPending& pend, const f
     return launch_status("decoder add_norm_q8");
 }
 // x (ws->x) through one layer, in place; the layer's own MoE output is left pending for whatever comes next
-// live (may be null): a device word, how many of the T rows count; the others still pass through the attention (their
-// cache cells are overwritten by the next window) but are not routed, so they pull no expert's weights
+// live (may be null): a device word, how many of the T rows count; the others still append their K and V (their cache
+// cells are overwritten by the next window) but ask no queries and are not routed, so they pull no expert's weights
 // gate (may be null): a device word; at zero the layer's dense products and its attention's scan leave at once
 static int dec_layer(const fnx_decoder* D, const fnx_dec_layer* L, int T, const int* pos0, const fnx_dec_ws* ws, DecPending& pend, void* st,
                      const int* live = nullptr, const int* gate = nullptr) {
@@ -1321,7 +1321,7 @@ static int dec_layer(const fnx_decoder* D, const fnx_dec_layer* L, int T, const 
     }
     if (attn_prep_append(ws->qg, ws->k, ws->v, L->q_norm, L->k_norm, L->kc, L->vc, nq, nkv, T, pos0, D->max_ctx, D->eps, &D->rope, st, gate)) return 1;
     // the attention's rows leave its last kernel in q8_1 form, ready for the output projection
-    if (attn_launch(ws->qg, L->kc, L->vc, nullptr, (uint8_t*) ws->xq, nq, nkv, pos0, T, D->max_ctx, ws->attn_scratch, st, gate)) return 1;
+    if (attn_launch(ws->qg, L->kc, L->vc, nullptr, (uint8_t*) ws->xq, nq, nkv, pos0, T, D->max_ctx, ws->attn_scratch, st, gate, live)) return 1;
     if (q8s_one(&L->wo, ws->xq, ws->o, n, T, st, gate)) return 1;
     {   // x += o; xn = norm(x) (fnx_add_norm_q8)
         CombineArgs c{};

@@ -441,11 +441,17 @@ constexpr int AT_WAVES = 4, AT_KLD = 2 * AT_HD + 16;   // q tiles (of 16 queries
 __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) k_attn_part(const float* __restrict__ qg, const uint16_t* __restrict__ kc,
                                                             const uint16_t* __restrict__ vc, float* __restrict__ acc_out,
                                                             AttPart* __restrict__ mz_out, int nq, int nkv, int T, int nsplit,
-                                                            const int* __restrict__ pos0p, const int* __restrict__ gate) {
+                                                            const int* __restrict__ pos0p, const int* __restrict__ gate,
+                                                            const int* __restrict__ live) {
     typedef __attribute__((address_space(1))) const at_v4u g128;
     if (gate && uniform(*gate) == 0) return;   // a chain step that does not count: its parts stay what they were, nothing reads the result
+    // live (may be null): a device word, the rows of the window that count; the others' queries are left out (nothing reads
+    // their results), the positions past the last row that counts with them
+    if (live) T = uniform(max(1, min(*live, T)));
     const int s = blockIdx.x, kvh = blockIdx.y, lane = threadIdx.x & 63, wave = blockIdx.z * AT_WAVES + (threadIdx.x >> 6);
     const int qpk = nq / nkv, nquery = T * qpk, pos0 = *pos0p;
+    if ((int) blockIdx.z * AT_WAVES * 16 >= nquery) return;   // none of the block's queries count
+    const bool wave_on = uniform(wave * 16 < nquery);         // a wave without queries still fetches its share of K and V
     const int ql = lane & 15, pg = lane >> 4;
     const int qi = wave * 16 + ql;                      // this lane's query (as B column / accumulator column)
     const bool qlive = qi < nquery;
@@ -516,6 +522,7 @@ __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per
     for (int c0 = p0; c0 < p1; c0 += AT_CH, buf ^= 1) {
         stash(buf ^ 1);                              // chunk c0 + 32, fetched during the last iteration
         fetch(min(c0 + 2 * AT_CH, p1 - 1));          // past the split: some rows again, never used
+        if (wave_on) {
         // the two tiles' hi and lo terms in chains of their own, interleaved: a chain's next MFMA is four issues away, so
         // none waits for the one before it
         at_v4f S[2];
@@ -615,6 +622,7 @@ __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per
             for (int u = 0; u < 4; ++u) O[4 * gq + u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[u], P, O[4 * gq + u], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
         }
+        }
         __syncthreads();
     }
     if (!qlive) return;
@@ -629,10 +637,13 @@ __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per
 constexpr int AT_MAXSPLIT = 2048;
 __global__ void __launch_bounds__(AT_HD) k_attn_combine(const float* __restrict__ qg, const float* __restrict__ acc_in,
                                                        const AttPart* __restrict__ mz_in, float* __restrict__ out, uint8_t* __restrict__ outq,
-                                                       int nq, int nsplit, int T, const int* __restrict__ pos0p, const int* __restrict__ gate) {
+                                                       int nq, int nsplit, int T, const int* __restrict__ pos0p, const int* __restrict__ gate,
+                                                       const int* __restrict__ live) {
     __shared__ float wsp[AT_MAXSPLIT];
     __shared__ float red[AT_HD / 64];
     if (gate && uniform(*gate) == 0) return;
+    if (live) T = uniform(max(1, min(*live, T)));
+    if ((int) blockIdx.y >= T) return;   // a row that does not count
     const int h = blockIdx.x, t = blockIdx.y, i = threadIdx.x;
     const size_t base = ((size_t) t * nq + h) * nsplit;
     const int nlive = min(nsplit, (*pos0p + T + AT_SPLIT - 1) / AT_SPLIT);   // splits the window's context reaches: their parts were written

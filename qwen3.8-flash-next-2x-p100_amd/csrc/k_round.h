@@ -4,9 +4,9 @@
 // What one step leaves for the next lives in device words (fnx_round.state), so a round's launches take no argument that
 // changes from round to round: rounds can be enqueued back to back, or captured once in a graph and replayed.
 //
-// A window always has FNX_MAXT rows; state[FNX_RS_ROWS] says how many of them count. The others hold token 0: they pass
-// through the attention like any row (their cache cells are overwritten by the next window, as a rejected draft's are)
-// but are not routed, so they pull no expert's weights, and acceptance never reaches them.
+// A window always has FNX_MAXT rows; state[FNX_RS_ROWS] says how many of them count. The others hold token 0: they
+// append their K and V like any row (their cache cells are overwritten by the next window, as a rejected draft's are)
+// but ask no queries and are not routed, so they pull no expert's weights, and acceptance never reaches them.
 #pragma once
 
 #include "../../include/fnx_mi355x.h"
