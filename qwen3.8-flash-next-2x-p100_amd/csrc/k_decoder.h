@@ -643,8 +643,12 @@ __global__ void __launch_bounds__(AT_HD) k_attn_combine(const float* __restrict_
     __shared__ float red[AT_HD / 64];
     if (gate && uniform(*gate) == 0) return;
     if (live) T = uniform(max(1, min(*live, T)));
-    if ((int) blockIdx.y >= T) return;   // a row that does not count
     const int h = blockIdx.x, t = blockIdx.y, i = threadIdx.x;
+    if (t >= T) {   // a row that does not count: zeros (its queries were left out; what follows it stays finite)
+        if (out) out[((size_t) t * nq + h) * AT_HD + i] = 0.f;
+        if (outq) q8_1_store(0.f, outq + (((size_t) t * nq + h) * (AT_HD / 32) + i / 32) * FNX_Q8_1_BLOCK, i & 31);
+        return;
+    }
     const size_t base = ((size_t) t * nq + h) * nsplit;
     const int nlive = min(nsplit, (*pos0p + T + AT_SPLIT - 1) / AT_SPLIT);   // splits the window's context reaches: their parts were written
     float mx = -INFINITY;
