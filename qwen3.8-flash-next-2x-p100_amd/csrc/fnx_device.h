@@ -29,6 +29,19 @@ struct SignedGrid {
     }
 };
 constexpr int SGRID_WORDS = 8192;
+// entry (s, g) from entry (0, g): the bytes whose bit of s is set, negated. No byte of the codebook is zero, so
+// (b ^ 0xFF) + 1 = 256 - b never carries into the next byte and the four bytes go in one xor and one add.
+constexpr bool grid_bytes_nonzero() {
+    for (int g = 0; g < 512; ++g)
+        for (int j = 0; j < 4; ++j)
+            if (((fnx_iq3s_grid_host[g] >> (8 * j)) & 255u) == 0) return false;
+    return true;
+}
+static_assert(grid_bytes_nonzero(), "signed_entry() counts on it");
+__device__ __forceinline__ uint32_t signed_entry(uint32_t g0, int s) {
+    const uint32_t m = ((s & 1) ? 0xFFu : 0u) | ((s & 2) ? 0xFF00u : 0u) | ((s & 4) ? 0xFF0000u : 0u) | ((s & 8) ? 0xFF000000u : 0u);
+    return (g0 ^ m) + (m & 0x01010101u);
+}
 
 __device__ __forceinline__ float half_bits_to_float(uint32_t h) {
     return __half2float(__ushort_as_half((unsigned short) h));

@@ -382,11 +382,11 @@ __global__ void __launch_bounds__(FL_THREADS) k_moe_gate_up_passes(const PassArg
     __shared__ RouteLds<FL_THREADS> L;
     LayerPlan& pl = L.plan;
     const int tid = threadIdx.x, wave = uniform(tid >> 6), lane = tid & 63;
-    // the codebook's loads go out first and land in registers; they are stored to LDS once the first weights have been
-    // asked for, so that the latencies overlap
-    uint32_t treg[SGRID_WORDS / FL_THREADS];
-#pragma unroll
-    for (int i = 0; i < SGRID_WORDS / FL_THREADS; ++i) treg[i] = g_sgrid.v[tid + i * FL_THREADS];
+    // the codebook's load goes out first (a thread's unsigned entry; its sixteen signed forms are made and stored to
+    // LDS once the first weights have been asked for, so that the latencies overlap: sixteen loads a thread and 16 MB
+    // from the caches over the grid if the whole table were read)
+    static_assert(FL_THREADS == 512, "a thread per 9-bit code: its sixteen signed entries are made from the first");
+    const uint32_t tab0 = g_sgrid.v[tid];
     build_plan<FL_THREADS>(L, a.route, blockIdx.x == 0);
     const int upj = a.rows;
     const long total = (long) pl.npass * upj;
@@ -400,7 +400,7 @@ __global__ void __launch_bounds__(FL_THREADS) k_moe_gate_up_passes(const PassArg
         packed_first(s.we, s.ul, s.ue, cur);
     }
 #pragma unroll
-    for (int i = 0; i < SGRID_WORDS / FL_THREADS; ++i) tab[tid + i * FL_THREADS] = treg[i];
+    for (int i = 0; i < SGRID_WORDS / FL_THREADS; ++i) tab[tid + i * FL_THREADS] = signed_entry(tab0, i);
     __syncthreads();
     while (u < u1) {
         const uint8_t* pairs = pl.job_pairs[s.ji] + s.t0;
@@ -444,9 +444,8 @@ __global__ void __launch_bounds__(FL_THREADS) k_moe_down_passes(const PassArgs a
     // codebook needs anyway (every wave making its own pairs' rows read the gate|up outputs 21 times over a pass).
     __shared__ __align__(16) uint32_t hq[4][SBR][12];   // 8 words of values, the scale, 3 unused (16-byte rows)
     const int tid = threadIdx.x, wave = uniform(tid >> 6), lane = tid & 63;
-    uint32_t treg[SGRID_WORDS / FL_THREADS];
-#pragma unroll
-    for (int i = 0; i < SGRID_WORDS / FL_THREADS; ++i) treg[i] = g_sgrid.v[tid + i * FL_THREADS];
+    static_assert(FL_THREADS == 512, "a thread per 9-bit code: its sixteen signed entries are made from the first");
+    const uint32_t tab0 = g_sgrid.v[tid];
     for (int i = tid; i < (int) (sizeof(LayerPlan) / 4); i += FL_THREADS) reinterpret_cast<int*>(&pl)[i] = reinterpret_cast<const int*>(&g_layer_plan)[i];
     __syncthreads();
     const int upj = a.rows / RW, ff = a.ff;
@@ -498,7 +497,7 @@ __global__ void __launch_bounds__(FL_THREADS) k_moe_down_passes(const PassArgs a
                 }
     }
 #pragma unroll
-    for (int i = 0; i < SGRID_WORDS / FL_THREADS; ++i) tab[tid + i * FL_THREADS] = treg[i];
+    for (int i = 0; i < SGRID_WORDS / FL_THREADS; ++i) tab[tid + i * FL_THREADS] = signed_entry(tab0, i);
     __syncthreads();
     const int kb = lane % SBR;
     while (u < u1) {
