@@ -780,7 +780,8 @@ static int layer_fused(const fnx_moe_layer* L, const float* x, int T, float* out
     static const int per_cu = env_int("FNX_LAYER_BLOCKS_PER_CU", 2, 1, 8);
     // at least as many blocks as a window can have passes: a block's share is then shorter than a pass, which the down
     // launch counts on (a block is in two passes at most)
-    const int grid = std::max(per_cu * cu_count(), FL_MAXP + FNX_MAXT);
+    // ... and few enough for the kernels' 32-bit unit arithmetic: (176 passes * 2048 units) * (8 waves * 1024 blocks) < 2^32
+    const int grid = std::min(std::max(per_cu * cu_count(), FL_MAXP + FNX_MAXT), 1024);
     const PassArgs gu{2 * ff, (const uint8_t*) L->gu.p, L->gu_stride, (const uint8_t* const*) L->gu.ep, (const uint8_t*) L->sh_gu.p,
                       (const uint8_t*) ws->xq, nullptr, ff, ws->gu, route};
     k_moe_gate_up_passes<<<grid, FL_THREADS, 0, s>>>(gu);

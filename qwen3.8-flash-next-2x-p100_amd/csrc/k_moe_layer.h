@@ -361,11 +361,19 @@ struct PassSeg {   // a stretch of one pass's units
     int ul, ue, ji, t0, nt;
     const uint8_t* we;
 };
-__device__ __forceinline__ PassSeg pass_seg(const LayerPlan& pl, const PassArgs& a, long uu, long u1, int upj) {
+// Unit numbers are 32-bit and a pass's units a power of two: 64-bit divisions (a few hundred instructions each, five of
+// them a wave) held the first weight loads up by one to two microseconds. The host keeps units * waves below 2^32.
+// (A division by the number of waves is forty instructions, twice a wave, on every wave of a SIMD at the same moment:
+// with a power of two - 2 x 256 CUs x 8 waves - it is a shift.)
+__device__ __forceinline__ uint32_t share_begin(uint32_t total, uint32_t gw, uint32_t nw) {
+    const uint32_t p = total * gw;
+    return (nw & (nw - 1)) == 0 ? p >> (31 - __clz(nw)) : p / nw;
+}
+__device__ __forceinline__ PassSeg pass_seg(const LayerPlan& pl, const PassArgs& a, uint32_t uu, uint32_t u1, int upj_log2) {
     PassSeg s;
-    const int pi = (int) (uu / upj);
-    s.ul = (int) (uu % upj);
-    s.ue = (int) min((long) upj, s.ul + (u1 - uu));
+    const int pi = (int) (uu >> upj_log2), upj = 1 << upj_log2;
+    s.ul = (int) (uu & (uint32_t) (upj - 1));
+    s.ue = (int) min((uint32_t) upj, s.ul + (u1 - uu));
     s.ji = uniform((int) pl.pass_job[pi]);
     s.t0 = uniform((int) pl.pass_t0[pi]);
     const int w = uniform(pl.job_w[s.ji]);
@@ -388,11 +396,11 @@ __global__ void __launch_bounds__(FL_THREADS) k_moe_gate_up_passes(const PassArg
     static_assert(FL_THREADS == 512, "a thread per 9-bit code: its sixteen signed entries are made from the first");
     const uint32_t tab0 = g_sgrid.v[tid];
     build_plan<FL_THREADS>(L, a.route, blockIdx.x == 0);
-    const int upj = a.rows;
-    const long total = (long) pl.npass * upj;
-    const long gw = (long) blockIdx.x * FL_WAVES + wave, nw = (long) gridDim.x * FL_WAVES;
-    long u = total * gw / nw;
-    const long u1 = total * (gw + 1) / nw;
+    const int upj = uniform(31 - __clz(a.rows));   // log2 of a pass's units
+    const uint32_t total = (uint32_t) pl.npass << upj;
+    const uint32_t gw = blockIdx.x * FL_WAVES + wave, nw = gridDim.x * FL_WAVES;
+    uint32_t u = share_begin(total, gw, nw);
+    const uint32_t u1 = share_begin(total, gw + 1, nw);
     PackedSub cur[4];
     PassSeg s{};
     if (u < u1) {
@@ -448,18 +456,18 @@ __global__ void __launch_bounds__(FL_THREADS) k_moe_down_passes(const PassArgs a
     const uint32_t tab0 = g_sgrid.v[tid];
     for (int i = tid; i < (int) (sizeof(LayerPlan) / 4); i += FL_THREADS) reinterpret_cast<int*>(&pl)[i] = reinterpret_cast<const int*>(&g_layer_plan)[i];
     __syncthreads();
-    const int upj = a.rows / RW, ff = a.ff;
-    const long total = (long) pl.npass * upj;
-    const long gw = (long) blockIdx.x * FL_WAVES + wave, nw = (long) gridDim.x * FL_WAVES;
-    long u = total * gw / nw;
-    const long u1 = total * (gw + 1) / nw;
+    const int upj = uniform(31 - __clz(a.rows / RW)), ff = a.ff;   // log2 of a pass's units
+    const uint32_t total = (uint32_t) pl.npass << upj;
+    const uint32_t gw = blockIdx.x * FL_WAVES + wave, nw = gridDim.x * FL_WAVES;
+    uint32_t u = share_begin(total, gw, nw);
+    const uint32_t u1 = share_begin(total, gw + 1, nw);
     PackedSub cur[4];
     PassSeg s{};
     if (u < u1) {
         s = pass_seg(pl, a, u, u1, upj);
         packed_first(s.we, s.ul, s.ue, cur);
     }
-    const int pass0 = (int) (total * ((long) blockIdx.x * FL_WAVES) / nw / upj);   // the block's first pass
+    const int pass0 = (int) (share_begin(total, blockIdx.x * FL_WAVES, nw) >> upj);   // the block's first pass
     {
         constexpr int VPT = (SBR * 32 + FL_THREADS - 1) / FL_THREADS;   // values a thread and pair
         float gv[4][VPT], uv[4][VPT];
@@ -501,7 +509,7 @@ __global__ void __launch_bounds__(FL_THREADS) k_moe_down_passes(const PassArgs a
     __syncthreads();
     const int kb = lane % SBR;
     while (u < u1) {
-        const int slot0 = 2 * ((int) (u / upj) - pass0);   // 0 or 2
+        const int slot0 = 2 * ((int) (u >> upj) - pass0);   // 0 or 2
         auto prep_for = [&](auto nt_tag) {
             constexpr int NT = decltype(nt_tag)::value;
             return [=](int(&xs)[NT][8], float(&dx)[NT], float*(&orow)[NT]) {
