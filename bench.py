@@ -24,8 +24,8 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 N, FF, NEXP, TOPK, T = 2048, 512, 512, 10, 16
 HBM_PEAK = 8.0e12
 # HBM bytes of one gate|up launch from the FETCH_SIZE / WRITE_SIZE counter runs (profiles/moe_gate_up_hbm_traffic.md),
-# as a ratio to the launch's algorithmic bytes at the profiled routing (139.2 distinct experts): 136.8 MB / 127.1 MB
-GATE_UP_TRAFFIC_RATIO = 1.076
+# as a ratio to the launch's algorithmic bytes at the profiled routing (139.75 distinct experts): 136.5 MB / 127.6 MB
+GATE_UP_TRAFFIC_RATIO = 1.070
 IQ3S_BLOCK = 110
 GU_BYTES = 2 * FF * (N // 256) * IQ3S_BLOCK      # 901,120 per expert
 DN_BYTES = N * (FF // 256) * IQ3S_BLOCK          # 450,560 per expert

@@ -412,16 +412,25 @@ __global__ void __launch_bounds__(512) k_iq3s_jobs(const RowsArgs a) {
     constexpr int RW = 64 / SBR;
     const int nj = a.njobs ? min(uniform(*a.njobs), a.njobs_max) : a.njobs_max;
     __syncthreads();
-    const int upj = a.nrows / RW;   // units per job
-    const long total = (long) nj * upj;
-    const int wpb = blockDim.x >> 6;
-    const long gw = (long) blockIdx.x * wpb + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), nw = (long) gridDim.x * wpb;
-    long u = total * gw / nw;
-    const long u1 = total * (gw + 1) / nw;
+    // unit numbers fit 32 bits (the launcher checks); the shares' products need 64 only for very large launches
+    // (a 64-bit division is a few hundred instructions, and every wave of the grid makes them as it starts)
+    const uint32_t upj = a.nrows / RW;   // units per job
+    const uint32_t total = (uint32_t) nj * upj;
+    const uint32_t wpb = blockDim.x >> 6;
+    const uint32_t gw = blockIdx.x * wpb + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), nw = gridDim.x * wpb;
+    uint32_t u, u1;
+    if ((unsigned long long) total * nw >> 32 == 0) {
+        u = total * gw / nw;
+        u1 = total * (gw + 1) / nw;
+    } else {
+        u = (uint32_t) ((unsigned long long) total * gw / nw);
+        u1 = (uint32_t) ((unsigned long long) total * (gw + 1) / nw);
+    }
     const uint8_t* y = a.y ? a.y : g_moe_hq;
     while (u < u1) {
-        const int ji = (int) (u / upj), ul = (int) (u % upj);
-        const int ue = (int) min((long) upj, ul + (u1 - u));
+        const uint32_t ji = u / upj;
+        const int ul = (int) (u - ji * upj);
+        const int ue = (int) min(upj, ul + (u1 - u));
         const fnx_job* jb = a.jobs + ji;
         const int w = uniform(jb->w);
         const uint8_t* we = a.ep ? uniform_ptr(a.ep[w]) : a.wbase + (size_t) w * a.w_stride;
@@ -726,6 +735,7 @@ static int rows_launch(const fnx_dw* W, size_t w_stride, const fnx_job* jobs, co
     static const int blocks = env_int("FNX_ROWS_BLOCKS", 0, 0, 65536), threads = env_int("FNX_ROWS_THREADS", 512, 64, 512) / 64 * 64;
     // no more waves than groups of four units: a wave with an empty range only fills the LDS
     const long units = (long) njobs_max * ((W->n_out * (long) (W->n_in / 32) + 63) / 64);
+    if (units >= (1L << 31)) return fail(std::string(who) + ": more than 2^31 units of 64 sub-blocks in one launch");
     const long want = (units / 4 + threads / 64 - 1) / (threads / 64);
     const int grid = (int) std::max(1L, std::min((long) (blocks ? blocks : 2 * cu_count()), want));
     const int sbr = W->n_in / 32;
