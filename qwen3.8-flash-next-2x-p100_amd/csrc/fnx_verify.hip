@@ -408,7 +408,11 @@ namespace fnx {
 template <int SBR, bool WIDE, bool PACKED>
 __global__ void __launch_bounds__(512) k_iq3s_jobs(const RowsArgs a) {
     __shared__ uint32_t tab[SGRID_WORDS];
-    for (int i = threadIdx.x; i < SGRID_WORDS; i += blockDim.x) tab[i] = g_sgrid.v[i];
+    for (int g = threadIdx.x; g < 512; g += blockDim.x) {   // a code's sixteen signed entries from its unsigned one
+        const uint32_t g0 = g_sgrid.v[g];
+#pragma unroll
+        for (int sg = 0; sg < 16; ++sg) tab[sg * 512 + g] = signed_entry(g0, sg);
+    }
     constexpr int RW = 64 / SBR;
     const int nj = a.njobs ? min(uniform(*a.njobs), a.njobs_max) : a.njobs_max;
     __syncthreads();

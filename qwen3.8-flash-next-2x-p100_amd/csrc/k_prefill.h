@@ -728,16 +728,15 @@ __global__ void __launch_bounds__(MM_THREADS) __attribute__((amdgpu_waves_per_eu
     typedef __attribute__((address_space(1))) const unsigned short g16;
     __shared__ TileLds L;
     const int tid = threadIdx.x, lane = tid & 63, wave = uniform(tid >> 6), r = lane & 15, g = lane >> 4;
-    uint32_t treg[SGRID_WORDS / MM_THREADS];
-#pragma unroll
-    for (int i = 0; i < SGRID_WORDS / MM_THREADS; ++i) treg[i] = g_sgrid.v[tid + i * MM_THREADS];
+    static_assert(MM_THREADS == 512, "a thread per 9-bit code: its sixteen signed entries are made from the first");
+    const uint32_t tab0 = g_sgrid.v[tid];
     const int nj = min(a.cap, uniform(*a.njobs)), nj2 = a.jobs2 ? min(a.cap2, uniform(*a.njobs2)) : 0;
     const int ks = a.ncols >> 5, nsuper = a.ncols / MT_K, rblocks = (a.nrows + MB_ROWS - 1) / MB_ROWS;
     constexpr int HALVES = MM_TT / MM_TP;
     const int per_job = rblocks * HALVES, ntasks_all = (nj + nj2) * per_job;
 #pragma unroll
     for (int i = 0; i < SGRID_WORDS / MM_THREADS; ++i) {
-        const uint32_t gg = treg[i];
+        const uint32_t gg = signed_entry(tab0, i);
         v2h lo, hi;
         lo.x = (_Float16) (int) (int8_t) (gg & 0xFFu);
         lo.y = (_Float16) (int) (int8_t) ((gg >> 8) & 0xFFu);
