@@ -329,8 +329,10 @@ template <bool PACKED, int RG>
 __global__ void __launch_bounds__(MM_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4))) k_moe_mma(const MmaArgs a) {
     typedef __attribute__((address_space(1))) const v4u gx4;
     __shared__ uint2 tab[SGRID_WORDS];
+    const uint32_t tab0 = g_sgrid.v[threadIdx.x];   // (512 threads: a thread's code, its sixteen signed entries made here)
+#pragma unroll
     for (int i = threadIdx.x; i < SGRID_WORDS; i += MM_THREADS) {
-        const uint32_t g = g_sgrid.v[i];
+        const uint32_t g = signed_entry(tab0, i >> 9);
         v2h lo, hi;
         lo.x = (_Float16) (int) (int8_t) (g & 0xFFu);
         lo.y = (_Float16) (int) (int8_t) ((g >> 8) & 0xFFu);
@@ -479,8 +481,10 @@ struct MmaLds {
 __global__ void __launch_bounds__(MM_THREADS) k_moe_mma_block(const MmaArgs a) {
     typedef __attribute__((address_space(1))) const v4u gx4;
     __shared__ MmaLds L;
+    const uint32_t tab0 = g_sgrid.v[threadIdx.x];   // (512 threads: a thread's code, its sixteen signed entries made here)
+#pragma unroll
     for (int i = threadIdx.x; i < SGRID_WORDS; i += MM_THREADS) {
-        const uint32_t g = g_sgrid.v[i];
+        const uint32_t g = signed_entry(tab0, i >> 9);
         v2h lo, hi;
         lo.x = (_Float16) (int) (int8_t) (g & 0xFFu);
         lo.y = (_Float16) (int) (int8_t) ((g >> 8) & 0xFFu);
