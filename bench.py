@@ -84,12 +84,8 @@ def main():
         sh_down = rand_iq3s(N * FF // 256)
         # the CPU leg reads raw ggml blocks: keep weight set 0's before the load-time re-laying (fnx_iq3s_repack, in place)
         raw = [a.cpu().numpy() for a in (gu, down, sh_gu, sh_down)] if not layers and args.cpu_seconds > 0 else None
-        if not args.raw_layout:
-            for w in (gu, down, sh_gu, sh_down):
-                dev.ok(lib.fnx_iq3s_repack(w.data_ptr(), w.data_ptr(), w.numel() // IQ3S_BLOCK * 256, dev.st()))
-        pk = not args.raw_layout
-        L = pkg.MoeLayer(N, FF, NEXP, TOPK, router.data_ptr(), 0, pkg.dw(gu, N, 2 * FF, packed=pk), GU_BYTES, pkg.dw(down, FF, N, packed=pk),
-                         DN_BYTES, pkg.dw(sh_gu, N, 2 * FF, packed=pk), pkg.dw(sh_down, FF, N, packed=pk))
+        (gu, down, sh_gu, sh_down), dws = fnx_gpu.pack_moe_weights(dev, [gu, down, sh_gu, sh_down], N, FF, not args.raw_layout)
+        L = pkg.MoeLayer(N, FF, NEXP, TOPK, router.data_ptr(), 0, dws[0], GU_BYTES, dws[1], DN_BYTES, dws[2], dws[3])
         layers.append((L, router, gu, down, sh_gu, sh_down, raw))
     NX = 64
     xs = torch.randn((NX, T, N), device="cuda", generator=g)
@@ -135,10 +131,10 @@ def main():
 
     # ---- the dominant kernel: the window's gate|up launch (routed experts + the shared expert), timed with events the
     # library records on the launch stream around each of the window's five launches (fnx_layer_profile)
-    names = ["router+q8_1", "top-k", "plan+gate|up", "down", "combine"]
-    per_launch = np.zeros(5)
+    names = ["router+q8_1", "top-k+plan+gate|up+swiglu", "down+combine"]
+    per_launch = np.zeros(3)
     reps = max(50, min(args.steps, 200))
-    ms5 = np.zeros(5, dtype=np.float32)
+    ms5 = np.zeros(3, dtype=np.float32)
     fused = not args.raw_layout
     if fused:
         dev.ok(lib.fnx_layer_profile(1))
@@ -149,11 +145,11 @@ def main():
                 per_launch += ms5
         dev.ok(lib.fnx_layer_profile(0))
         per_launch /= reps
-        k_ms = float(per_launch[2])
-        kernel_name = "k_moe_gate_up_passes (unit64)"
+        k_ms = float(per_launch[1])
+        kernel_name = "k_moe_gate_up_h (unit64)"
         # algorithmic bytes of one launch: the distinct experts' and the shared expert's gate|up blocks, the window's
-        # q8_1 rows, the f32 outputs
-        k_bytes = (u_mean + 1) * GU_BYTES + T * (N // 32) * 36 + (P + T) * 2 * FF * 4
+        # q8_1 rows and router logits, the q8_1 rows of h
+        k_bytes = (u_mean + 1) * GU_BYTES + T * (N // 32) * 36 + T * (NEXP + 1) * 4 + (P + T) * (FF // 32) * 36
     else:
         evs = []
         for i in range(reps + 10):

@@ -173,6 +173,15 @@ int fnx_moe_verify_layer(const fnx_moe_layer* L, const float* x, int T, float* o
  * down, combine. One profiled window at a time per process. */
 int fnx_layer_profile(int on);
 int fnx_layer_profile_read(float* ms5);
+/* Calibration aid (no counterpart in the reference): one read-only pass over `bytes` of device memory, nothing decoded,
+ * so that the expert mat-vec launches can be judged against what the memory system gives a plain read of the same shape.
+ * variant: 0 / 1 / 7 / 8: 16-byte loads a lane, 4 / 8 / 16 / 2 in flight, every wave one contiguous range; 2 / 3: the same 4 / 8
+ * with the 1 KiB chunks dealt round-robin to the waves; 4: 8-byte loads, 8 in flight; 5: as 1 with nontemporal loads;
+ * 6: the unit64 planes as the pass kernels load them (five loads a unit and lane, a group of four units in flight), every
+ * wave one contiguous range; 9: the groups dealt round-robin to the grid's waves; 10: every block one contiguous range,
+ * its waves taking the groups in turn; 11 / 12 / 13: as 6 / 9 / 10 with nontemporal loads. sink: one device word (never
+ * written in practice; it keeps the loads alive). */
+int fnx_stream_read(const void* p, size_t bytes, int variant, int blocks, int threads, void* sink, void* st);
 
 /* ---- the prompt path's MoE over a chunk of C rows (prefill.cu:1990-2083) */
 /* prefill.cu:288-377  k_pf_top10 / k_pf_count / k_pf_jobbase / k_pf_fill in one call: top-k and weights per row,

@@ -123,6 +123,7 @@ EXPORTS = {
     "fnx_accept_greedy_dev": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
     "fnx_layer_profile": (C.c_int, [C.c_int]),
     "fnx_layer_profile_read": (C.c_int, [C.c_void_p]),
+    "fnx_stream_read": (C.c_int, [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]),
     "fnx_moe_verify_layer": (C.c_int, [C.POINTER(MoeLayer), C.c_void_p, C.c_int, C.c_void_p, C.POINTER(MoeWs), C.c_void_p]),
     "fnx_pf_route": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),

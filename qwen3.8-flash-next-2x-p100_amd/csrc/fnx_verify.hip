@@ -260,7 +260,6 @@ struct RowsArgs {
     const uint8_t* y;   // q8_1 rows; null: the library's pair buffer
     float* out;
     int out_stride;
-    int y_rows;         // how many activation rows y holds when that is known to be at most a window's (else 0)
 };
 
 struct RawSub {   // one lane's share of a unit as read from memory; nothing is combined until it is used
@@ -451,6 +450,7 @@ __global__ void __launch_bounds__(512) k_iq3s_jobs(const RowsArgs a) {
 #include "k_round.h"
 #include "k_sampler.h"
 #include "k_qtypes.h"
+#include "k_stream.h"
 namespace fnx {
 
 // any other row length (a multiple of 256): a wave per (row, job), sub-blocks dealt round-robin to the lanes, the
@@ -700,7 +700,7 @@ static int cu_count() {
 }
 // wide: the jobs are expected to hold many rows each (a dense matrix over the whole window) rather than one or two
 static int rows_launch(const fnx_dw* W, size_t w_stride, const fnx_job* jobs, const int* njobs, int njobs_max, const void* y, float* out,
-                       int out_stride, void* st, const char* who, bool wide = false, int y_rows = 0) {
+                       int out_stride, void* st, const char* who, bool wide = false) {
     if (!W || !jobs || !out) return fail(std::string(who) + ": null argument");
     if (W->type == QT_Q4_0 || W->type == QT_Q5_1 || W->type == QT_Q8_0 || W->type == QT_IQ4_NL || W->type == QT_IQ4_XS || W->type == QT_Q4_K || W->type == QT_Q5_K) {
         // the other types of kernels.cu:2454-2471 that the reference's own host code can decode (k_qtypes.h)
@@ -733,7 +733,7 @@ static int rows_launch(const fnx_dw* W, size_t w_stride, const fnx_job* jobs, co
     if (njobs_max <= 0) return fail(std::string(who) + ": njobs_max must be positive");
     if (!W->p && !W->ep) return fail(std::string(who) + ": no weights");
     RowsArgs a{(const uint8_t*) W->p, w_stride, (const uint8_t* const*) W->ep, W->row_bytes, W->n_out, W->n_in,
-               jobs, njobs, njobs_max, (const uint8_t*) y, out, out_stride, y_rows};
+               jobs, njobs, njobs_max, (const uint8_t*) y, out, out_stride};
     hipStream_t s = (hipStream_t) st;
     // two blocks of 8 waves per CU by default: every block copies the 32 KiB codebook into LDS once
     static const int blocks = env_int("FNX_ROWS_BLOCKS", 0, 0, 65536), threads = env_int("FNX_ROWS_THREADS", 512, 64, 512) / 64 * 64;
@@ -765,52 +765,46 @@ static int rows_launch(const fnx_dw* W, size_t w_stride, const fnx_job* jobs, co
     return launch_status(who);
 }
 
+// the shapes and layouts the window's three launches take (k_moe_layer.h)
 static bool layer_fused_ok(const fnx_moe_layer* L, int T) {
     static const int on = env_int("FNX_LAYER_FUSED", 1, 0, 1);
     const auto packed = [](const fnx_dw& w) { return w.type == FNX_T_IQ3S_UNIT64; };
-    return on && L->n == FL_N && (L->ff == 256 || L->ff == 512 || L->ff == 1024) && L->nexp <= 1024 && T * L->topk <= FL_MAXP &&
-           packed(L->gu) && packed(L->down) && packed(L->sh_gu) && packed(L->sh_down) && L->gu_stride % UNIT_BYTES == 0 &&
-           L->down_stride % UNIT_BYTES == 0 && L->sh_gu.p && L->sh_down.p;
+    return on && L->n == FL_N && (L->ff == 256 || L->ff == 512 || L->ff == 1024) && L->nexp <= 1024 && L->topk <= FL_MAXK &&
+           T * L->topk <= FL_MAXP && packed(L->gu) && packed(L->sh_gu) && packed(L->down) && packed(L->sh_down) &&
+           L->gu_stride % UNIT_BYTES == 0 && L->down_stride % UNIT_BYTES == 0 && L->sh_gu.p && L->sh_down.p;
 }
-// per-launch timing of the window (fnx_layer_profile): events recorded on the launch stream around each of the five
+// per-launch timing of the window (fnx_layer_profile): events recorded on the launch stream around each of the three
 // launches; the counterpart of the reference's FNX_PROF stamps in its window graph (engine.cu:1382-1530)
 static bool g_prof_on = false;
-static hipEvent_t g_prof_ev[6] = {};
+static hipEvent_t g_prof_ev[4] = {};
 static void prof_mark(int i, hipStream_t s) {
     if (g_prof_on) (void) hipEventRecord(g_prof_ev[i], s);
 }
-// the window's MoE half in five launches (k_moe_layer.h)
-// live (may be null): a device word, the rows of the window that are routed (k_route_topk, build_plan); the caller's combine skips the others
+// the window's MoE half in three launches (k_moe_layer.h): [router logits | q8_1 rows], [top-k + plan + gate|up -> h as
+// q8_1 rows (in ws->gu)], [down + the combine's chains -> out]
+// live (may be null): a device word, the rows of the window that count; the others are not routed and their rows of out are left alone
 static int layer_fused(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st, const int* live = nullptr) {
     hipStream_t s = (hipStream_t) st;
-    const int n = L->n, ff = L->ff, P = T * L->topk, LS = L->nexp + 1;
+    const int n = L->n, ff = L->ff, LS = L->nexp + 1;
     const int rblocks = (LS + RQ_ROWS - 1) / RQ_ROWS, qblocks = (T * 64 + 2 * FL_WAVES - 1) / (2 * FL_WAVES);
     prof_mark(0, s);
     k_router_quant<<<rblocks + qblocks, FL_THREADS, 0, s>>>(RouterArgs{L->nexp, T, x, L->router, L->router_bf16, ws->logits, (uint8_t*) ws->xq, live});
     prof_mark(1, s);
     const RouteArgs route{L->nexp, L->topk, T, ws->logits, ws->topi, ws->topw, ws->jobs_gu, ws->jobs_dn, ws->njobs, live};
-    k_route_topk<<<T, RT_THREADS, 0, s>>>(route);
+    // at least as many blocks as the window has rows (a block's run of items then lies in two rows at most)
+    static const int gh_blocks = env_int("FNX_GH_BLOCKS", 0, 0, 4096);
+    const GateUpArgs ga{ff, (const uint8_t*) L->gu.p, L->gu_stride, (const uint8_t* const*) L->gu.ep, (const uint8_t*) L->sh_gu.p,
+                        (const uint8_t*) ws->xq, (uint32_t*) ws->gu, route};
+    k_moe_gate_up_h<<<std::max(gh_blocks ? gh_blocks : cu_count(), FNX_MAXT), GH_THREADS, 0, s>>>(ga);
     prof_mark(2, s);
-    static const int per_cu = env_int("FNX_LAYER_BLOCKS_PER_CU", 2, 1, 8);
-    // at least as many blocks as a window can have passes: a block's share is then shorter than a pass, which the down
-    // launch counts on (a block is in two passes at most)
-    // ... and few enough for the kernels' 32-bit unit arithmetic: (176 passes * 2048 units) * (8 waves * 1024 blocks) < 2^32
-    const int grid = std::min(std::max(per_cu * cu_count(), FL_MAXP + FNX_MAXT), 1024);
-    const PassArgs gu{2 * ff, (const uint8_t*) L->gu.p, L->gu_stride, (const uint8_t* const*) L->gu.ep, (const uint8_t*) L->sh_gu.p,
-                      (const uint8_t*) ws->xq, nullptr, ff, ws->gu, route};
-    k_moe_gate_up_passes<<<grid, FL_THREADS, 0, s>>>(gu);
+    const DownArgs da{n, ff, L->topk, T, L->nexp, (const uint8_t*) L->down.p, L->down_stride, (const uint8_t* const*) L->down.ep,
+                      (const uint8_t*) L->sh_down.p, (const uint32_t*) ws->gu, ws->topi, ws->topw, ws->logits, out, live, route};
+    // a block per row and 32 units of the output, and one more for the job lists
+    if (ff == 256) k_moe_down_combine<8><<<T * (n / (8 * 32)) + 1, FL_THREADS, 0, s>>>(da);
+    else if (ff == 512) k_moe_down_combine<16><<<T * (n / (4 * 32)) + 1, FL_THREADS, 0, s>>>(da);
+    else k_moe_down_combine<32><<<T * (n / (2 * 32)) + 1, FL_THREADS, 0, s>>>(da);
     prof_mark(3, s);
-    const PassArgs dn{n, (const uint8_t*) L->down.p, L->down_stride, (const uint8_t* const*) L->down.ep, (const uint8_t*) L->sh_down.p,
-                      nullptr, ws->gu, ff, ws->part, RouteArgs{}};
-    if (ff == 256) k_moe_down_passes<8><<<grid, FL_THREADS, 0, s>>>(dn);
-    else if (ff == 512) k_moe_down_passes<16><<<grid, FL_THREADS, 0, s>>>(dn);
-    else k_moe_down_passes<32><<<grid, FL_THREADS, 0, s>>>(dn);
-    prof_mark(4, s);
-    if (launch_status("moe_verify_layer")) return 1;
-    if (!out) return 0;   // the caller combines (with what follows: fnx_combine_add_norm_q8)
-    const int rc = fnx_moe_combine(ws->part, ws->topw, ws->part + (size_t) P * n, ws->logits + L->nexp, LS, out, T, n, L->topk, st);
-    prof_mark(5, s);
-    return rc;
+    return launch_status("moe_verify_layer");
 }
 
 }  // namespace fnx
@@ -830,7 +824,6 @@ int fnx_iq3s_repack(const void* src, void* dst, size_t n_weights, void* st) {
     k_iq3s_repack<<<(unsigned) ((units + 3) / 4), 256, 0, (hipStream_t) st>>>((const uint8_t*) src, (uint8_t*) dst, units);
     return launch_status("iq3s_repack");
 }
-
 int fnx_quantize_q8_1(const float* x, void* q, int n, int rows, void* st) {
     if (!x || !q) return fail("quantize_q8_1: null argument");
     if (n <= 0 || n % 32 || rows <= 0) return fail("quantize_q8_1: rows of whole 32-value blocks");
@@ -910,7 +903,7 @@ int fnx_moe_gate_up(const fnx_dw* A, size_t sa, const fnx_job* jobs, const int* 
     if (A && (A->n_out & 1)) return fail("moe_gate_up: rows are [gate | up], an even count");
     if (topk < 1 || njobs_max % topk) return fail("moe_gate_up: njobs_max is the window's pairs, a multiple of topk");
     // the window's rows: njobs_max / topk of them (kernels.cu:2449, T = njobs_max / TOPK); xq holds that many
-    return rows_launch(A, sa, jobs, njobs, njobs_max, xq, gu, A ? A->n_out : 0, st, "moe_gate_up", false, njobs_max / topk);
+    return rows_launch(A, sa, jobs, njobs, njobs_max, xq, gu, A ? A->n_out : 0, st, "moe_gate_up");
 }
 int fnx_moe_down(const fnx_dw* A, size_t sa, const fnx_job* jobs, const int* njobs, int njobs_max, const float* gu, float* part, void* st) {
     if (!A || !gu) return fail("moe_down: null argument");
@@ -991,16 +984,15 @@ int fnx_layer_profile(int on) {
     g_prof_on = on != 0;
     return 0;
 }
-int fnx_layer_profile_read(float* ms5) {
-    if (!ms5) return fail("layer_profile_read: null argument");
+int fnx_layer_profile_read(float* ms3) {
+    if (!ms3) return fail("layer_profile_read: null argument");
     if (!g_prof_ev[0]) return fail("layer_profile_read: profiling was never switched on");
-    if (hipEventSynchronize(g_prof_ev[5]) != hipSuccess) return fail("layer_profile_read: no window was recorded");
-    for (int i = 0; i < 5; ++i)
-        if (hipEventElapsedTime(&ms5[i], g_prof_ev[i], g_prof_ev[i + 1]) != hipSuccess) return fail("layer_profile_read: no window was recorded");
+    if (hipEventSynchronize(g_prof_ev[3]) != hipSuccess) return fail("layer_profile_read: no window was recorded");
+    for (int i = 0; i < 3; ++i)
+        if (hipEventElapsedTime(&ms3[i], g_prof_ev[i], g_prof_ev[i + 1]) != hipSuccess) return fail("layer_profile_read: no window was recorded");
     return 0;
 }
 
-// out null: the fused window without its combine (layer_fused_ok must hold)
 static int moe_layer_checked(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st, const int* live = nullptr) {
     if (!L || !x || !ws) return fail("moe_verify_layer: null argument");
     if (!ws->xq || !ws->logits || !ws->topi || !ws->topw || !ws->jobs_gu || !ws->jobs_dn || !ws->njobs || !ws->gu || !ws->part)
@@ -1011,17 +1003,17 @@ static int moe_layer_checked(const fnx_moe_layer* L, const float* x, int T, floa
     if (L->gu.n_in != n || L->gu.n_out != 2 * ff || L->down.n_in != ff || L->down.n_out != n || L->sh_gu.n_in != n ||
         L->sh_gu.n_out != 2 * ff || L->sh_down.n_in != ff || L->sh_down.n_out != n)
         return fail("moe_verify_layer: weight shapes do not match n / ff");
-    if (live && (out || !layer_fused_ok(L, T))) return fail("moe_verify_layer: a device-side row count needs the fused window without its combine");
-    if (layer_fused_ok(L, T)) return layer_fused(L, x, T, out, ws, st, live);
     if (!out) return fail("moe_verify_layer: null argument");
+    if (live && !layer_fused_ok(L, T)) return fail("moe_verify_layer: a device-side row count needs the three-launch window");
+    if (layer_fused_ok(L, T)) return layer_fused(L, x, T, out, ws, st, live);
     hipStream_t s = (hipStream_t) st;
     if (fnx_quantize_q8_1(x, ws->xq, n, T, st)) return 1;
     if (gemv_any(L->router, L->router_bf16 != 0, x, ws->logits, L->nexp + 1, n, T, st, "moe_verify_layer router")) return 1;
     k_topk_jobs<<<1, TK_THREADS, 0, s>>>(ws->logits, L->nexp + 1, T, L->nexp, L->topk, ws->topi, ws->topw, ws->jobs_gu, ws->jobs_dn, ws->njobs,
                                          0, 1);
     if (launch_status("moe_verify_layer topk")) return 1;
-    if (rows_launch(&L->gu, L->gu_stride, ws->jobs_gu, ws->njobs, P, ws->xq, ws->gu, 2 * ff, st, "moe_verify_layer gate|up", false, T)) return 1;
-    if (rows_launch(&L->sh_gu, 0, ws->jobs_gu + P, nullptr, 1, ws->xq, ws->gu, 2 * ff, st, "moe_verify_layer shared gate|up", true, T)) return 1;
+    if (rows_launch(&L->gu, L->gu_stride, ws->jobs_gu, ws->njobs, P, ws->xq, ws->gu, 2 * ff, st, "moe_verify_layer gate|up")) return 1;
+    if (rows_launch(&L->sh_gu, 0, ws->jobs_gu + P, nullptr, 1, ws->xq, ws->gu, 2 * ff, st, "moe_verify_layer shared gate|up", true)) return 1;
     k_swiglu_q8_1<<<dim3((ff / 32 + 7) / 8, P + T), 256, 0, s>>>(ws->gu, ws->gu + ff, (size_t) 2 * ff, nullptr, ff);
     if (launch_status("moe_verify_layer swiglu")) return 1;
     if (rows_launch(&L->down, L->down_stride, ws->jobs_dn, ws->njobs, P, nullptr, ws->part, n, st, "moe_verify_layer down")) return 1;
@@ -1031,6 +1023,42 @@ static int moe_layer_checked(const fnx_moe_layer* L, const float* x, int T, floa
 int fnx_moe_verify_layer(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st) {
     if (!out) return fail("moe_verify_layer: null argument");
     return moe_layer_checked(L, x, T, out, ws, st);
+}
+
+// ---------------------------------------------------------------- streaming calibration (k_stream.h)
+int fnx_stream_read(const void* p, size_t bytes, int variant, int blocks, int threads, void* sink, void* st) {
+    if (!p || !sink) return fail("stream_read: null argument");
+    if (threads < 64 || threads > 1024 || threads % 64) return fail("stream_read: 64..1024 threads in whole waves");
+    if (blocks < 1 || blocks > 65535) return fail("stream_read: 1..65535 blocks");
+    if (((uintptr_t) p & 15u) || bytes < 1024) return fail("stream_read: a 16-byte aligned buffer of at least 1 KiB");
+    hipStream_t s = (hipStream_t) st;
+    const uint8_t* b = (const uint8_t*) p;
+    uint32_t* k = (uint32_t*) sink;
+    const size_t c16 = bytes / 1024, c8 = bytes / 512;
+    switch (variant) {
+        case 0: k_stream_read<16, 4, false, true><<<blocks, threads, 0, s>>>(b, c16, k); break;
+        case 1: k_stream_read<16, 8, false, true><<<blocks, threads, 0, s>>>(b, c16, k); break;
+        case 2: k_stream_read<16, 4, false, false><<<blocks, threads, 0, s>>>(b, c16, k); break;
+        case 3: k_stream_read<16, 8, false, false><<<blocks, threads, 0, s>>>(b, c16, k); break;
+        case 4: k_stream_read<8, 8, false, true><<<blocks, threads, 0, s>>>(b, c8, k); break;
+        case 5: k_stream_read<16, 8, true, true><<<blocks, threads, 0, s>>>(b, c16, k); break;
+        case 6: k_stream_read_units<0, false><<<blocks, threads, 0, s>>>(b, bytes / UNIT_BYTES, k); break;
+        case 7: k_stream_read<16, 16, false, true><<<blocks, threads, 0, s>>>(b, c16, k); break;
+        case 8: k_stream_read<16, 2, false, true><<<blocks, threads, 0, s>>>(b, c16, k); break;
+        case 9: k_stream_read_units<1, false><<<blocks, threads, 0, s>>>(b, bytes / UNIT_BYTES, k); break;
+        case 10: k_stream_read_units<2, false><<<blocks, threads, 0, s>>>(b, bytes / UNIT_BYTES, k); break;
+        case 11: k_stream_read_units<0, true><<<blocks, threads, 0, s>>>(b, bytes / UNIT_BYTES, k); break;
+        case 12: k_stream_read_units<1, true><<<blocks, threads, 0, s>>>(b, bytes / UNIT_BYTES, k); break;
+        case 13: k_stream_read_units<2, true><<<blocks, threads, 0, s>>>(b, bytes / UNIT_BYTES, k); break;
+        default:
+            // 1000 s + K: segments of 256 s units (s = 4: a gate|up matrix, 2: a down matrix), K trips a wave and segment
+            if (variant >= 1000 && variant < 9000 && variant % 1000 >= 1 && variant % 1000 <= 64 && (256 * (variant / 1000) / 4) % (variant % 1000) == 0) {
+                k_stream_read_segments<<<blocks, threads, 0, s>>>(b, bytes / UNIT_BYTES, 256u * (variant / 1000), (uint32_t) (variant % 1000), k);
+                break;
+            }
+            return fail("stream_read: variants 0..13, or 1000 s + K");
+    }
+    return launch_status("stream_read");
 }
 
 // ---------------------------------------------------------------- the prompt path
@@ -1293,23 +1321,18 @@ static int dec_ws_check(const fnx_dec_ws* ws, const char* who) {
         return fail(std::string(who) + ": incomplete workspace");
     return 0;
 }
-// What is still to be added to x when a layer (or the head) starts: rows (may be null), or the MoE half before it whose
-// partial sums (in ws->moe) have not been combined yet - the first pass over the rows then does that too.
+// What is still to be added to x when a layer (or the head) starts: rows (may be null) - the attention half's or the MoE
+// half's output - of which only the first *live (live not null) were written.
 struct DecPending {
     const float* rows;
-    const fnx_moe_layer* moe;
     const int* tokens;   // not null: x itself is still to come - the embedding rows of these tokens (nothing else pending then)
-    const int* live;     // with moe: the device word that said how many rows were routed, or null
+    const int* live;
 };
 // xcopy (may be null): the rows after the add go there too
 static int dec_add_norm_q8(const fnx_decoder* D, const DecPending& pend, const float* w, int T, const fnx_dec_ws* ws, void* st, float* xcopy = nullptr,
                            const int* gate = nullptr) {
     CombineArgs c{};
-    if (pend.moe) {
-        const fnx_moe_layer* M = pend.moe;
-        c = CombineArgs{ws->moe.part, ws->moe.topw, ws->moe.part + (size_t) T * M->topk * D->n, ws->moe.logits + M->nexp, M->nexp + 1, M->topk, nullptr,
-                        nullptr, nullptr, 0, pend.live, nullptr};
-    }
+    c.live = pend.live;
     c.xcopy = xcopy;
     c.gate = gate;
     if (pend.tokens) {
@@ -1318,8 +1341,7 @@ static int dec_add_norm_q8(const fnx_decoder* D, const DecPending& pend, const f
         c.vocab = D->vocab;
     }
     if (D->n < 32 || D->n % 32 || D->n > 256 * NQ_MAXJ) return fail("decoder: rows of 32 .. 4096 values in whole 32-value blocks");
-    if (pend.moe) k_add_norm_q8<true><<<T, 1024, 0, (hipStream_t) st>>>(ws->x, nullptr, c, w, nullptr, (uint8_t*) ws->xq, D->n, D->eps);
-    else k_add_norm_q8<false><<<T, 256, 0, (hipStream_t) st>>>(ws->x, pend.rows, c, w, nullptr, (uint8_t*) ws->xq, D->n, D->eps);
+    k_add_norm_q8<false><<<T, 256, 0, (hipStream_t) st>>>(ws->x, pend.rows, c, w, nullptr, (uint8_t*) ws->xq, D->n, D->eps);
     return launch_status("decoder add_norm_q8");
 }
 // x (ws->x) through one layer, in place; the layer's own MoE output is left pending for whatever comes next
@@ -1346,13 +1368,10 @@ static int dec_layer(const fnx_decoder* D, const fnx_dec_layer* L, int T, const 
         k_add_norm_q8<false><<<T, 256, 0, (hipStream_t) st>>>(ws->x, ws->o, c, L->ffn_norm, ws->xn, nullptr, n, D->eps);
         if (launch_status("decoder add_norm")) return 1;
     }
-    if (layer_fused_ok(&L->moe, T)) {   // the window without its combine
-        pend = DecPending{nullptr, &L->moe, nullptr, live};
-        return moe_layer_checked(&L->moe, ws->xn, T, nullptr, &ws->moe, st, live);
-    }
-    if (live) return fail("decoder: a device-side row count needs the fused window (unit64 experts, hidden 2048)");
-    pend = DecPending{ws->o, nullptr, nullptr, nullptr};
-    return fnx_moe_verify_layer(&L->moe, ws->xn, T, ws->o, &ws->moe, st);
+    if (live && !layer_fused_ok(&L->moe, T)) return fail("decoder: a device-side row count needs the three-launch window (unit64 experts, hidden 2048)");
+    // the MoE half's rows (those that count) are added by the next pass over x
+    pend = DecPending{ws->o, nullptr, live};
+    return moe_layer_checked(&L->moe, ws->xn, T, ws->o, &ws->moe, st, live);
 }
 static int dec_shape_check(const fnx_decoder* D, int T, const char* who) {
     if (D->n < 256 || D->n % 256 || D->n > 4096 || D->nq < 1 || D->nkv < 1 || D->nq % D->nkv || D->nq / D->nkv > AT_MAXQ || D->vocab < 1 ||
@@ -1371,7 +1390,7 @@ static int dec_head(const fnx_decoder* D, const float* norm, const fnx_q8s* head
 static int decoder_verify(const fnx_decoder* D, const int* tokens, int T, const int* pos0, const fnx_dec_ws* ws, void* st, const int* live) {
     if (!D || !tokens || !pos0 || !ws || !D->layers || !D->out_norm || !D->emb) return fail("decoder_verify: null argument");
     if (dec_shape_check(D, T, "decoder_verify") || dec_ws_check(ws, "decoder_verify")) return 1;
-    DecPending pend{nullptr, nullptr, tokens, nullptr};   // the window's input rows are read by the first pass over them
+    DecPending pend{nullptr, tokens, nullptr};   // the window's input rows are read by the first pass over them
     for (int l = 0; l < D->nlayers; ++l)
         if (dec_layer(D, &D->layers[l], T, pos0, ws, pend, st, live)) return 1;
     return dec_head(D, D->out_norm, &D->head, T, ws, pend, st);
@@ -1402,7 +1421,7 @@ static int mtp_draft(const fnx_decoder* D, const fnx_mtp* M, const float* src, c
         if (launch_status("mtp_draft")) return 1;
     }
     if (q8s_one(&M->fc_emb, ws->xq, ws->o, n, T, st, gate)) return 1;
-    DecPending pend{ws->o, nullptr, nullptr, nullptr};
+    DecPending pend{ws->o, nullptr, nullptr};
     if (dec_layer(D, &M->layer, T, pos0, ws, pend, st, live, gate)) return 1;
     return dec_head(D, M->out_norm, &M->head, T, ws, pend, st, gate);
 }

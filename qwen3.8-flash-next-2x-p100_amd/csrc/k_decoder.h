@@ -117,7 +117,7 @@ __global__ void __launch_bounds__(WIDE ? 1024 : 256) k_add_norm_q8(float* __rest
             else v[j] = i < n ? x[row * n + i] : 0.f;
             av[j] = add && i < n ? add[row * n + i] : 0.f;
         }
-        if (add) {
+        if (add && (!c.live || (int) row < *c.live)) {
 #pragma unroll
             for (int j = 0; j < NQ_MAXJ; ++j) v[j] += av[j];
         }

@@ -1,6 +1,6 @@
 // The MoE half of a verify window (the work of Engine::ffn_half, engine.cu:1569-1757 of the reference, on one GPU) in
-// five launches: [router logits | q8_1 rows of x] -> [top-k] -> [jobs and plan, gate|up, routed and shared] ->
-// [SwiGLU to q8_1 on the fly + down, routed and shared] -> [combine].
+// three launches: [router logits | q8_1 rows of x] -> [top-k, jobs and plan, gate|up of the routed and the shared expert,
+// SwiGLU to q8_1] -> [down of the routed and the shared expert with the combine's chains].
 //
 // Arithmetic is the operators': the router sums in the fixed 64-lane order, top-k by (value, lower index), the q8_1
 // rounding, the IQ3_S sub-block terms, the combine's fmaf chain. Only the order in which a row's 64 (or 16) lane
@@ -19,21 +19,6 @@ constexpr int FL_THREADS = 512, FL_WAVES = FL_THREADS / 64;
 constexpr int FL_MAXP = FNX_MAXT * 10;    // routed pairs of a window (T * topk), at most
 constexpr int FL_MAXJ = FL_MAXP + 1;      // their jobs, and the shared expert's
 constexpr int FL_N = 2048;                // hidden size these kernels are built for (gate|up rows of 64 sub-blocks)
-
-// what the routing block hands to every other block: the jobs in compact form and the list of passes.
-// A pass = (job, first token, 1 or 2 tokens) over all the job's units; the passes' units are what the waves split
-// evenly, so a job of many rows (the shared expert's has the whole window) weighs as many times as it is walked.
-struct LayerPlan {
-    int nj, npass;
-    int job_w[FL_MAXJ];                       // expert, or -1 for the shared expert
-    uint8_t job_n[FL_MAXJ + 3];
-    uint8_t job_pairs[FL_MAXJ][FNX_MAXT];     // output rows (pairs t * topk + k, or P + t), ascending
-    uint8_t pair_tok[FL_MAXP + FNX_MAXT];     // the window row of a pair
-    uint8_t pass_job[FL_MAXP + FNX_MAXT];
-    uint8_t pass_t0[FL_MAXP + FNX_MAXT];
-};
-// one MoE in flight per device (as g_moe_hq)
-__device__ LayerPlan g_layer_plan;
 
 // wave-wide max / min with DPP moves; every lane gets the result
 __device__ __forceinline__ float wave_max(float v) {
@@ -61,9 +46,10 @@ __device__ __forceinline__ int wave_min(int v) {
 
 // one token's top-k: the lanes hold its logits (lane l: experts l, l + 64, ...). Picks into ex[0..topk), topi, topw.
 // moe.cuh:382-411: greater value first, the lower index on a tie; w_k = exp(l_k - l_0) / sum in pick order.
+// publish: also write topi and topw (else only ex)
 template <int NE>
 __device__ __forceinline__ void wave_topk(const float* __restrict__ row, int nexp, int topk, int lane, int* __restrict__ ex,
-                                          int* __restrict__ topi, float* __restrict__ topw) {
+                                          int* __restrict__ topi, float* __restrict__ topw, bool publish = true) {
     float v[NE];
 #pragma unroll
     for (int i = 0; i < NE; ++i) {
@@ -100,20 +86,18 @@ __device__ __forceinline__ void wave_topk(const float* __restrict__ row, int nex
             wk = ek;
             const int pick = mi < nexp ? mi : nexp - 1;   // fewer than topk finite logits: stay inside the tables
             ex[k] = pick;
-            topi[k] = pick;
+            if (publish) topi[k] = pick;
         }
     }
-    if (lane < topk) topw[lane] = wk / z;
+    if (publish && lane < topk) topw[lane] = wk / z;
 }
 
-// ---------------------------------------------------------------- launch 2: top-k; the plan, made by its readers
-// k_route_topk: a wave per row of the window ranks the row's logits. The job lists and the plan follow from all rows'
-// picks without any serial loop: a token picks an expert at most once, so a pair's slot in its job is the number of
-// earlier tokens in the expert's token mask, and a job's number is the rank of its first pair among the first pairs
-// (the order k_router_route's last block gives them, moe.cuh:324-330). Every block of the gate|up launch makes the plan
-// for itself in LDS from the 160 picks (build_plan), while its codebook loads are in flight; its block 0 also writes the
-// plan and the job lists to memory, for the down launch and for the caller. That is quicker than a last-block phase in
-// the top-k launch, which costs an atomic and two more memory round trips on the window's critical path.
+// ---------------------------------------------------------------- the job lists of a window's picks
+// The reference's window hands its caller the jobs as lists (kernels.hpp:18-23, 277-282); this window's own launches do
+// not read them (they walk a row's picks directly), so a spare block of the last launch writes them, off the critical
+// path. They follow from all rows' picks without any serial loop: a token picks an expert at most once, so a pair's
+// slot in its job is the number of earlier tokens in the expert's token mask, and a job's number is the rank of its first
+// pair among the first pairs (the order k_router_route's last block gives them, moe.cuh:324-330).
 struct RouteArgs {
     int nexp, topk, T;
     const float* logits;
@@ -125,47 +109,29 @@ struct RouteArgs {
     const int* live;   // may be null; else a device word: only the window's first *live rows are routed (the others get no
                        // pairs, and the shared expert's job stops before them), while the lists keep the indexes T gives them
 };
-constexpr int RT_THREADS = 64;
-__global__ void __launch_bounds__(RT_THREADS) k_route_topk(const RouteArgs a) {
-    __shared__ int ex[FL_MAXP];
-    const int lane = threadIdx.x, LS = a.nexp + 1, t = blockIdx.x, topk = a.topk;
-    const int Tl = a.live ? uniform(max(0, min(*a.live, a.T))) : a.T;
-    if (t >= Tl) return;
-    if (a.nexp <= 512) wave_topk<8>(a.logits + (size_t) t * LS, a.nexp, topk, lane, ex, a.topi + t * topk, a.topw + t * topk);
-    else wave_topk<16>(a.logits + (size_t) t * LS, a.nexp, topk, lane, ex, a.topi + t * topk, a.topw + t * topk);
-}
-
 template <int NT>
 struct RouteLds {
-    LayerPlan plan;
-    int ex[FL_MAXP];
     unsigned mask[1024];      // per expert: the window rows that picked it
     int first[1024];          // per expert: its first pair
     int jobof[1024];
-    int pass0[FL_MAXJ + 3];   // per job: its first pass
     int wcnt[NT / 64];
 };
-// All NT threads of a block; ends with a barrier. publish: also write the lists and the plan to memory.
+// All NT threads of a block. Tl: the rows that count.
 template <int NT>
-__device__ __forceinline__ void build_plan(RouteLds<NT>& L, const RouteArgs& a, bool publish) {
-    static_assert(FL_MAXP <= NT && FL_MAXJ <= NT, "a thread per pair, a thread per job");
+__device__ __forceinline__ void write_job_lists(RouteLds<NT>& L, const RouteArgs& a, int Tl) {
+    static_assert(FL_MAXP <= NT, "a thread per pair");
     const int tid = threadIdx.x, wave = uniform(tid >> 6), lane = tid & 63;
-    const int T = a.T, topk = a.topk, P = T * topk;
-    const int Tl = a.live ? uniform(max(0, min(*a.live, T))) : T, Pl = Tl * topk;
-    LayerPlan& pl = L.plan;
-    const int e_mine = tid < Pl ? a.topi[tid] : 0;   // asked for before the tables are cleared
+    const int T = a.T, topk = a.topk, P = T * topk, Pl = Tl * topk;
+    const int e_mine = tid < Pl ? a.topi[tid] : 0;
     for (int e = tid; e < a.nexp; e += NT) {
         L.mask[e] = 0u;
         L.first[e] = P;
     }
     __syncthreads();
     if (tid < Pl) {
-        L.ex[tid] = e_mine;
         atomicOr(&L.mask[e_mine], 1u << (tid / topk));
         atomicMin(&L.first[e_mine], tid);
-        pl.pair_tok[tid] = (uint8_t) (tid / topk);
     }
-    if (tid < Tl) pl.pair_tok[P + tid] = (uint8_t) tid;
     __syncthreads();
     // job numbers: the rank of an expert's first pair among all first pairs (ballots over the pairs in order)
     const bool isfirst = tid < Pl && L.first[e_mine] == tid;
@@ -177,74 +143,32 @@ __device__ __forceinline__ void build_plan(RouteLds<NT>& L, const RouteArgs& a, 
         before += w < wave ? L.wcnt[w] : 0;
         nj += L.wcnt[w];
     }
-    nj = uniform(nj);
     if (isfirst) {
         const int j = before + __popcll(b & ((1ull << lane) - 1ull)), cnt = __popc(L.mask[e_mine]);
         L.jobof[e_mine] = j;
-        pl.job_w[j] = e_mine;
-        pl.job_n[j] = (uint8_t) cnt;
-        if (publish) {
-            a.jobs_gu[j].w = a.jobs_dn[j].w = e_mine;
-            a.jobs_gu[j].n = a.jobs_dn[j].n = cnt;
-        }
+        a.jobs_gu[j].w = a.jobs_dn[j].w = e_mine;
+        a.jobs_gu[j].n = a.jobs_dn[j].n = cnt;
     }
-    if (tid == 0) {
-        pl.nj = nj;
-        pl.job_w[nj] = -1;   // the shared expert's job: every row of the window, pairs P + t
-        pl.job_n[nj] = (uint8_t) Tl;
-        if (publish) a.njobs[0] = nj;
-    }
+    if (tid == 0) a.njobs[0] = nj;
     __syncthreads();
     // a pair's slot in its job: the earlier rows in its expert's mask (pairs of a job ascend with the row)
     if (tid < Pl) {
         const int j = L.jobof[e_mine], row = tid / topk, slot = __popc(L.mask[e_mine] & ((1u << row) - 1u));
-        pl.job_pairs[j][slot] = (uint8_t) tid;
-        if (publish) {
-            a.jobs_gu[j].y[slot] = row;
-            a.jobs_gu[j].out[slot] = tid;
-            a.jobs_dn[j].y[slot] = tid;
-            a.jobs_dn[j].out[slot] = tid;
+        a.jobs_gu[j].y[slot] = row;
+        a.jobs_gu[j].out[slot] = tid;
+        a.jobs_dn[j].y[slot] = tid;
+        a.jobs_dn[j].out[slot] = tid;
+    }
+    if (tid < max(Tl, 1)) {   // the shared expert's job, at index P of the lists (kernels.hpp:277-282)
+        a.jobs_gu[P].y[tid] = tid;
+        a.jobs_gu[P].out[tid] = P + tid;
+        a.jobs_dn[P].y[tid] = P + tid;
+        a.jobs_dn[P].out[tid] = P + tid;
+        if (tid == 0) {
+            a.jobs_gu[P].w = a.jobs_dn[P].w = 0;
+            a.jobs_gu[P].n = a.jobs_dn[P].n = Tl;
         }
     }
-    if (tid < max(Tl, 1)) {   // the shared expert's job, at index P of the lists the API returns (kernels.hpp:277-282)
-        pl.job_pairs[nj][tid] = (uint8_t) (P + tid);
-        if (publish) {
-            a.jobs_gu[P].y[tid] = tid;
-            a.jobs_gu[P].out[tid] = P + tid;
-            a.jobs_dn[P].y[tid] = P + tid;
-            a.jobs_dn[P].out[tid] = P + tid;
-            if (tid == 0) {
-                a.jobs_gu[P].w = a.jobs_dn[P].w = 0;
-                a.jobs_gu[P].n = a.jobs_dn[P].n = Tl;
-            }
-        }
-    }
-    // passes: job j's rows two at a time; job j's first pass = the passes of the jobs before it: a scan over the jobs
-    // (wave by wave with the waves' totals in LDS; a thread per job)
-    {
-        const int cj = tid <= nj ? (pl.job_n[tid] + 1) >> 1 : 0;
-        int inc = cj;
-#pragma unroll
-        for (int o = 1; o < 64; o <<= 1) {
-            const int up = __shfl_up(inc, o, 64);
-            if (lane >= o) inc += up;
-        }
-        if (lane == 63) L.wcnt[wave] = inc;   // (the job count's readers of wcnt are behind a barrier)
-        __syncthreads();
-        int bef = 0;
-        for (int w = 0; w < wave; ++w) bef += L.wcnt[w];
-        if (tid <= nj) {
-            const int p0 = bef + inc - cj, n = pl.job_n[tid];
-            for (int t0 = 0, k = 0; t0 < n; t0 += 2, ++k) {
-                pl.pass_job[p0 + k] = (uint8_t) tid;
-                pl.pass_t0[p0 + k] = (uint8_t) t0;
-            }
-        }
-        if (tid == nj) pl.npass = bef + inc;
-    }
-    __syncthreads();
-    if (publish)
-        for (int i = tid; i < (int) (sizeof(LayerPlan) / 4); i += NT) reinterpret_cast<int*>(&g_layer_plan)[i] = reinterpret_cast<const int*>(&pl)[i];
 }
 
 // ---------------------------------------------------------------- launch 1: router logits | q8_1 rows of x
@@ -344,194 +268,305 @@ __global__ void __launch_bounds__(FL_THREADS) k_router_quant(const RouterArgs a)
     if (live && (lane & 7) == 0 && t < T) a.logits[(size_t) t * LS + row] = v;
 }
 
-// ---------------------------------------------------------------- launches 3 and 4: the passes of the plan
-struct PassArgs {
-    int rows;                 // rows of every matrix
+// ---------------------------------------------------------------- launch 2: top-k, gate|up, h in q8_1 form
+// An item = (pair, block of 32 h values): the 32 gate rows and the 32 up rows that one q8_1 block of
+// h = silu(gate) * up needs (k_moe_h, moe.cuh:597-608), 64 units of the pair's expert. A thread block of 16 waves takes
+// one item a sweep, four units a wave: gate rows 2 i, 2 i + 1 and up rows 2 i, 2 i + 1, whose four sums give two h values.
+// The items are numbered (row, block of 32, pick) and dealt to the blocks of the grid in runs: with a full window of 16
+// rows and 256 blocks a thread block has one row's one block of 32 for all the row's picks, the shared expert last. So
+// it needs the picks of one row only (two when a run crosses rows): it ranks that row itself, a wave a row, while its
+// codebook loads are in flight - no launch of its own for the top-k (a kernel boundary on the window's critical path),
+// no list of jobs, no plan - and its lanes keep their activations for the whole launch. An expert that several rows
+// picked is decoded once per row (the later reads come from the caches); in exchange every sweep of every block is the
+// same work, and at any time the grid reads one expert a row, each as one front moving through the matrix, which HBM
+// serves better than a range of its own per wave (25 against 29 us for a plain read of a window's gate|up bytes).
+// The sixteen waves' values of an item meet in LDS without a barrier: a wave writes its two values and its flag and goes
+// on; two sweeps later the wave whose turn it is makes the q8_1 block of that sweep and writes it out (by then the
+// others have long arrived; it waits if not).
+// hq rows as the down launch reads them: per pair and block of 32: 8 words of int8 values, the scale as a float, 3 unused.
+constexpr int GH_THREADS = 1024, GH_WAVES = GH_THREADS / 64, HQ_WORDS = 12, GH_SLOTS = 4, GH_LAG = 2;
+constexpr int FL_MAXK = 16;   // picks a row that the window's launches take
+struct GateUpArgs {
+    int ff;                   // expert width: the matrices have 2 ff rows (gate rows, then up rows) of FL_N columns
     const uint8_t* w;         // routed experts: expert e at w + e * stride, or ep[e]
     size_t stride;
     const uint8_t* const* ep;
     const uint8_t* w_shared;
-    const uint8_t* xq;        // gate|up: the window's q8_1 rows
-    const float* gu;          // down: the gate|up outputs [pair][2 ff]
-    int ff;
-    float* out;               // [pair][rows]
-    RouteArgs route;          // gate|up: what the plan is made from
+    const uint8_t* xq;        // the window's q8_1 rows
+    uint32_t* hq;             // [pair][ff / 32][HQ_WORDS]
+    RouteArgs route;          // logits in; picks and weights out (the block that has a row's first item writes them)
 };
-struct PassSeg {   // a stretch of one pass's units
-    int ul, ue, ji, t0, nt;
-    const uint8_t* we;
+struct GhLds {
+    uint32_t tab[SGRID_WORDS];
+    uint32_t wp[2][FL_MAXK + 1][2];   // the matrices of the block's (at most two) rows' picks, the shared expert's last
+    float hb[GH_SLOTS][32];           // [slot][h value of the block]
+    int flag[GH_SLOTS][GH_WAVES];     // sweep + 1 of the values a wave last wrote into the slot
+    int made[GH_SLOTS];               // sweeps whose block has been made from the slot: a writer of sweep s waits for made >= s - GH_SLOTS + 1
+    int ex[2][FL_MAXK];
 };
-// Unit numbers are 32-bit and a pass's units a power of two: 64-bit divisions (a few hundred instructions each, five of
-// them a wave) held the first weight loads up by one to two microseconds. The host keeps units * waves below 2^32.
-// (A division by the number of waves is forty instructions, twice a wave, on every wave of a SIMD at the same moment:
-// with a power of two - 2 x 256 CUs x 8 waves - it is a shift.)
-__device__ __forceinline__ uint32_t share_begin(uint32_t total, uint32_t gw, uint32_t nw) {
-    const uint32_t p = total * gw;
-    return (nw & (nw - 1)) == 0 ? p >> (31 - __clz(nw)) : p / nw;
-}
-__device__ __forceinline__ PassSeg pass_seg(const LayerPlan& pl, const PassArgs& a, uint32_t uu, uint32_t u1, int upj_log2) {
-    PassSeg s;
-    const int pi = (int) (uu >> upj_log2), upj = 1 << upj_log2;
-    s.ul = (int) (uu & (uint32_t) (upj - 1));
-    s.ue = (int) min((uint32_t) upj, s.ul + (u1 - uu));
-    s.ji = uniform((int) pl.pass_job[pi]);
-    s.t0 = uniform((int) pl.pass_t0[pi]);
-    const int w = uniform(pl.job_w[s.ji]);
-    s.nt = uniform((int) pl.job_n[s.ji]) - s.t0;
-    s.we = w < 0 ? a.w_shared : a.ep ? uniform_ptr(a.ep[w]) : a.w + (size_t) w * a.stride;
-    return s;
-}
-
-// gate|up: rows of 2048 columns; activations: the window's q8_1 rows. The waves of the grid split the passes' units
-// evenly and walk them in order.
-__global__ void __launch_bounds__(FL_THREADS) k_moe_gate_up_passes(const PassArgs a) {
-    constexpr int SBR = 64;
-    __shared__ uint32_t tab[SGRID_WORDS];
-    __shared__ RouteLds<FL_THREADS> L;
-    LayerPlan& pl = L.plan;
+struct GhItem {   // (row, block of 32, pick) of an item number, kept by stepping
+    int t, j, k;
+};
+__global__ void __launch_bounds__(GH_THREADS) k_moe_gate_up_h(const GateUpArgs a) {
+    __shared__ GhLds S;
     const int tid = threadIdx.x, wave = uniform(tid >> 6), lane = tid & 63;
-    // the codebook's load goes out first (a thread's unsigned entry; its sixteen signed forms are made and stored to
-    // LDS once the first weights have been asked for, so that the latencies overlap: sixteen loads a thread and 16 MB
-    // from the caches over the grid if the whole table were read)
-    static_assert(FL_THREADS == 512, "a thread per 9-bit code: its sixteen signed entries are made from the first");
-    const uint32_t tab0 = g_sgrid.v[tid];
-    build_plan<FL_THREADS>(L, a.route, blockIdx.x == 0);
-    const int upj = uniform(31 - __clz(a.rows));   // log2 of a pass's units
-    const uint32_t total = (uint32_t) pl.npass << upj;
-    const uint32_t gw = blockIdx.x * FL_WAVES + wave, nw = gridDim.x * FL_WAVES;
-    uint32_t u = share_begin(total, gw, nw);
-    const uint32_t u1 = share_begin(total, gw + 1, nw);
-    PackedSub cur[4];
-    PassSeg s{};
-    if (u < u1) {
-        s = pass_seg(pl, a, u, u1, upj);
-        packed_first(s.we, s.ul, s.ue, cur);
-    }
+    const int T = a.route.T, topk = a.route.topk, P = T * topk, qpp = a.ff >> 5, per_row = qpp * (topk + 1);
+    const int Tl = a.route.live ? uniform(max(0, min(*a.route.live, T))) : T;
+    // this block's run of items
+    const int total = Tl * per_row, nb = gridDim.x, ipb = (total + nb - 1) / nb;
+    const int I0 = (int) blockIdx.x * ipb, I1 = min(total, I0 + ipb), nsweep = I1 - I0;
+    if (nsweep <= 0) return;
+    const uint32_t tab0 = g_sgrid.v[tid & 511];
+    const int t0 = I0 / per_row, t1 = (I1 - 1) / per_row;   // ipb <= per_row (the launcher sees to it): two rows at most
+    auto load_x = [&](int t, int (&xs)[8], float& dx) {   // the lane's sub-block of row t's activations
+        const uint32_t* yb = reinterpret_cast<const uint32_t*>(a.xq + ((size_t) t * 64 + lane) * FNX_Q8_1_BLOCK);
+        dx = half_bits_to_float(yb[0] & 0xFFFFu);
 #pragma unroll
-    for (int i = 0; i < SGRID_WORDS / FL_THREADS; ++i) tab[tid + i * FL_THREADS] = signed_entry(tab0, i);
-    __syncthreads();
-    while (u < u1) {
-        const uint8_t* pairs = pl.job_pairs[s.ji] + s.t0;
-        auto prep_for = [&](auto nt_tag) {
-            constexpr int NT = decltype(nt_tag)::value;
-            const uint8_t* pair_tok = pl.pair_tok;
-            return [=](int(&xs)[NT][8], float(&dx)[NT], float*(&orow)[NT]) {
-#pragma unroll
-                for (int t = 0; t < NT; ++t) {
-                    const int pair = uniform((int) pairs[t]), tok = uniform((int) pair_tok[pair]);
-                    const uint8_t* yb = a.xq + ((size_t) tok * SBR + lane) * FNX_Q8_1_BLOCK;
-                    dx[t] = half_bits_to_float(*reinterpret_cast<const unsigned short*>(yb));
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) xs[t][j] = reinterpret_cast<const int*>(yb + 4)[j];
-                    orow[t] = a.out + (size_t) pair * a.rows;
-                }
-            };
-        };
-        if (s.nt >= 2) packed_units<SBR, 2>(tab, s.we, s.ul, s.ue, cur, prep_for(std::integral_constant<int, 2>{}));
-        else packed_units<SBR, 1>(tab, s.we, s.ul, s.ue, cur, prep_for(std::integral_constant<int, 1>{}));
-        u += s.ue - s.ul;
-        if (u < u1) {
-            s = pass_seg(pl, a, u, u1, upj);
-            packed_first(s.we, s.ul, s.ue, cur);
+        for (int j = 0; j < 8; ++j) xs[j] = (int) yb[j + 1];
+    };
+    int xs[8], tx = t0;
+    float dx;
+    load_x(t0, xs, dx);
+    if (wave < 2 && t0 + wave <= t1) {   // the rows' picks (moe.cuh:382-411), a wave a row; the row's first item's block writes them out
+        const int t = t0 + wave;
+        const bool publish = t * per_row >= I0;
+        const float* row = a.route.logits + (size_t) t * (a.route.nexp + 1);
+        if (a.route.nexp <= 512) wave_topk<8>(row, a.route.nexp, topk, lane, S.ex[wave], a.route.topi + t * topk, a.route.topw + t * topk, publish);
+        else wave_topk<16>(row, a.route.nexp, topk, lane, S.ex[wave], a.route.topi + t * topk, a.route.topw + t * topk, publish);
+        if (lane <= topk) {   // LDS writes of this wave, read back in order
+            const uint8_t* e = a.w_shared;
+            if (lane < topk) {
+                const int ei = S.ex[wave][lane];
+                e = a.ep ? a.ep[ei] : a.w + (size_t) ei * a.stride;
+            }
+            S.wp[wave][lane][0] = (uint32_t) (uintptr_t) e;
+            S.wp[wave][lane][1] = (uint32_t) ((uint64_t) (uintptr_t) e >> 32);
         }
     }
-}
-
-// down: rows of 32 SBR columns, split over the waves like gate|up. A wave makes the q8_1 form of h = silu(gate) * up
-// for its pass's pairs itself (k_moe_down without PRE, moe.cuh:630-641): the 64 / SBR lanes that share a sub-block
-// column split its 32 values. (Making h once per block in LDS for the block's 8 waves was measured slower: 30 us
-// against 25 us, the block-wide barriers cost more than the repeated SwiGLU.)
-template <int SBR>
-__global__ void __launch_bounds__(FL_THREADS) k_moe_down_passes(const PassArgs a) {
-    constexpr int RW = 64 / SBR;   // rows per unit
-    __shared__ uint32_t tab[SGRID_WORDS];
-    __shared__ LayerPlan pl;
-    // h = silu(gate) * up of the block's pairs in q8_1 form (k_moe_h, moe.cuh:597-608): per pair and 32-value block the
-    // 32 int8 values, then the block's scale as a float. A block's eight waves walk consecutive units, fewer than a pass
-    // has, so they are in two passes at most: four pairs, made once by the whole block ahead of the barrier that the
-    // codebook needs anyway (every wave making its own pairs' rows read the gate|up outputs 21 times over a pass).
-    __shared__ __align__(16) uint32_t hq[4][SBR][12];   // 8 words of values, the scale, 3 unused (16-byte rows)
-    const int tid = threadIdx.x, wave = uniform(tid >> 6), lane = tid & 63;
-    static_assert(FL_THREADS == 512, "a thread per 9-bit code: its sixteen signed entries are made from the first");
-    const uint32_t tab0 = g_sgrid.v[tid];
-    for (int i = tid; i < (int) (sizeof(LayerPlan) / 4); i += FL_THREADS) reinterpret_cast<int*>(&pl)[i] = reinterpret_cast<const int*>(&g_layer_plan)[i];
+    if (tid < GH_SLOTS * GH_WAVES) (&S.flag[0][0])[tid] = 0;
+    if (tid < GH_SLOTS) S.made[tid] = 0;
+    // the codebook: two threads a code, eight signed forms each
+#pragma unroll
+    for (int i = 0; i < 8; ++i) S.tab[tid + i * GH_THREADS] = signed_entry(tab0, (tid >> 9) + 2 * i);
     __syncthreads();
-    const int upj = uniform(31 - __clz(a.rows / RW)), ff = a.ff;   // log2 of a pass's units
-    const uint32_t total = (uint32_t) pl.npass << upj;
-    const uint32_t gw = blockIdx.x * FL_WAVES + wave, nw = gridDim.x * FL_WAVES;
-    uint32_t u = share_begin(total, gw, nw);
-    const uint32_t u1 = share_begin(total, gw + 1, nw);
-    PackedSub cur[4];
-    PassSeg s{};
-    if (u < u1) {
-        s = pass_seg(pl, a, u, u1, upj);
-        packed_first(s.we, s.ul, s.ue, cur);
-    }
-    const int pass0 = (int) (share_begin(total, blockIdx.x * FL_WAVES, nw) >> upj);   // the block's first pass
-    {
-        constexpr int VPT = (SBR * 32 + FL_THREADS - 1) / FL_THREADS;   // values a thread and pair
-        float gv[4][VPT], uv[4][VPT];
-        bool on[4];
-#pragma unroll
-        for (int slot = 0; slot < 4; ++slot) {   // all the loads first: one trip to the cache for the four pairs
-            const int pi = pass0 + (slot >> 1), t = slot & 1;
-            const int pc = max(min(pi, pl.npass - 1), 0);
-            on[slot] = pi < pl.npass && pl.pass_t0[pc] + t < pl.job_n[pl.pass_job[pc]];
-            if (on[slot]) {   // the same for every thread of the block
-                const int ji = pl.pass_job[pi], pair = pl.job_pairs[ji][pl.pass_t0[pi] + t];
-                const float* gp = a.gu + (size_t) pair * 2 * ff;
-#pragma unroll
-                for (int k = 0; k < VPT; ++k) {
-                    const int i = tid + k * FL_THREADS;
-                    gv[slot][k] = i < ff ? gp[i] : 0.f;
-                    uv[slot][k] = i < ff ? gp[ff + i] : 0.f;
-                }
+    const PackedOffs o = packed_offs(lane);
+    const int sc_shift = 4 * (lane & 1);
+    // byte offsets of the wave's gate units and up units from its item's first gate unit
+    const uint32_t uo_g = (uint32_t) (wave * 2) * UNIT_BYTES, uo_u = uo_g + (uint32_t) a.ff * UNIT_BYTES;
+    auto item_of = [&](int I) {
+        GhItem m;
+        m.t = I / per_row;
+        const int r = I - m.t * per_row;
+        m.j = r / (topk + 1);
+        m.k = r - m.j * (topk + 1);
+        return m;
+    };
+    auto step = [&](GhItem& m) {
+        if (++m.k > topk) {
+            m.k = 0;
+            if (++m.j == qpp) {
+                m.j = 0;
+                ++m.t;
             }
         }
+    };
+    auto issue = [&](PackedSub(&u)[4], const GhItem& m) {
+        const uint2 p = *reinterpret_cast<const uint2*>(S.wp[m.t - t0][m.k]);
+        const uint64_t e = (uint64_t) (uint32_t) uniform((int) p.x) | (uint64_t) (uint32_t) uniform((int) p.y) << 32;
+        const uint8_t* we = (const uint8_t*) (uintptr_t) e + (size_t) (m.j * 32) * UNIT_BYTES;
+        u[0] = load_packed(as_global(we + uo_g), o);
+        u[1] = load_packed(as_global(we + uo_g + UNIT_BYTES), o);
+        u[2] = load_packed(as_global(we + uo_u), o);
+        u[3] = load_packed(as_global(we + uo_u + UNIT_BYTES), o);
+    };
+    // the q8_1 block of sweep q, by the first half of the wave
+    auto make_block = [&](int q) {
+        const int slot = q & (GH_SLOTS - 1);
+        while (true) {   // all sixteen waves' values of sweep q must be there
+            const int f = lane < GH_WAVES ? __hip_atomic_load(&S.flag[slot][lane], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) : q + 1;
+            if (__ballot(f < q + 1) == 0ull) break;
+            __builtin_amdgcn_s_sleep(2);
+        }
+        const GhItem m = item_of(I0 + q);
+        const int pair = m.k < topk ? m.t * topk + m.k : P + m.t;
+        if (lane < 32) {
+            const float h = S.hb[slot][lane];
+            const float amax = group_max<32>(fabsf(h));
+            const float d = amax / 127.0f;
+            const uint32_t qv = amax == 0.0f ? 0u : (uint32_t) (uint8_t) (int8_t) roundf(h / d);
+            uint32_t word = qv | (uint32_t) __shfl_down((int) qv, 1, WAVE) << 8;
+            word |= (uint32_t) __shfl_down((int) word, 2, WAVE) << 16;
+            uint32_t* dst = a.hq + ((size_t) pair * qpp + m.j) * HQ_WORDS;
+            if ((lane & 3) == 0) dst[lane >> 2] = word;
+            if (lane == 0) dst[8] = __float_as_uint(half_bits_to_float(float_to_half_bits(d)));
+        }
+        if (lane == 0) __hip_atomic_store(&S.made[slot], q + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    };
+    auto decode = [&](const PackedSub(&u)[4], const GhItem& m, int sw) {
+        if (m.t != tx) {   // the run has crossed into its second row
+            tx = m.t;
+            load_x(tx, xs, dx);
+        }
+        float v[4];
 #pragma unroll
-        for (int slot = 0; slot < 4; ++slot)
-            if (on[slot])
+        for (int r = 0; r < 4; ++r) {
+            int w4[8];
 #pragma unroll
-                for (int k = 0; k < VPT; ++k) {
-                    const int i = tid + k * FL_THREADS;
-                    if (i < ff) {   // whole 32-lane groups
-                        const float h = silu_f(gv[slot][k]) * uv[slot][k];
-                        const float amax = group_max<32>(fabsf(h));
-                        const float d = amax / 127.0f;
-                        const int q = amax == 0.0f ? 0 : (int) (int8_t) roundf(h / d);
-                        reinterpret_cast<int8_t*>(&hq[slot][i >> 5][0])[i & 31] = (int8_t) q;
-                        if ((i & 31) == 0) hq[slot][i >> 5][8] = __float_as_uint(half_bits_to_float(float_to_half_bits(d)));
-                    }
-                }
+            for (int j = 0; j < 8; ++j) w4[j] = *reinterpret_cast<const int*>(reinterpret_cast<const uint8_t*>(S.tab) + packed_addr(u[r].idx, j));
+            const int sc = 1 + 2 * (int) ((u[r].sc >> sc_shift) & 0xFu);
+            const float dw = half_bits_to_float(u[r].d);
+            int sum = 0;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) sum = __builtin_amdgcn_sdot4(w4[j], xs[j], sum, false);
+            // one sub-block's term as the reference forms it: (d_w * d_x) * (float) (sumi * (1 + 2 s))
+            v[r] = (dw * dx) * (float) __mul24(sum, sc);
+        }
+        // units: gate 2 i, gate 2 i + 1, up 2 i, up 2 i + 1 -> the 16-lane rows hold gate 2 i, up 2 i, gate 2 i + 1, up 2 i + 1
+        const float z = reduce4_units(v[0], v[1], v[2], v[3]);
+        const int zi = __builtin_bit_cast(int, z);
+        const float g0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(zi, 0)), u0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(zi, 16));
+        const float g1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(zi, 32)), u1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(zi, 48));
+        const float h = silu_f(lane & 1 ? g1 : g0) * (lane & 1 ? u1 : u0);   // lane 0: h of row 2 i, lane 1: of row 2 i + 1
+        const int slot = sw & (GH_SLOTS - 1);
+        // the slot's last block (of sweep sw - GH_SLOTS) must have been made: nearly always long ago
+        if (sw >= GH_SLOTS)
+            while (uniform(__hip_atomic_load(&S.made[slot], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP)) < sw - GH_SLOTS + 1) __builtin_amdgcn_s_sleep(1);
+        if (lane < 2) S.hb[slot][2 * wave + lane] = h;
+        if (lane == 0) __hip_atomic_store(&S.flag[slot][wave], sw + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+        const int q = sw - GH_LAG;   // the sweep whose block is due; wave q mod 16 makes it
+        if (q >= 0 && (q & (GH_WAVES - 1)) == wave) make_block(q);
+    };
+    // every wave of the block makes the same sweeps: each slot sees all sixteen arrive
+    PackedSub cur[4], nxt[4];
+    GhItem mc = item_of(I0), mn = mc;
+    issue(cur, mc);
+    for (int sw = 0; sw < nsweep; ++sw) {
+        if (sw + 1 < nsweep) step(mn);
+        issue(nxt, mn);   // past the end: the last item again (a read of what the caches hold)
+        decode(cur, mc, sw);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) cur[r] = nxt[r];
+        mc = mn;
+    }
+    for (int q = max(nsweep - GH_LAG, 0); q < nsweep; ++q)   // the last sweeps' blocks
+        if ((q & (GH_WAVES - 1)) == wave) make_block(q);
+}
+
+// ---------------------------------------------------------------- launch 3: down and the combine
+// out[t][r] = sum_k topw[t][k] (down_{e(t,k)}[r] . h[t,k]) + sigmoid(gate logit) (down_shared[r] . h[shared, t]): the
+// work of k_moe_down (moe.cuh:613-658) and of the combine (kernels.cu:412-419) with one wave making a row's whole chain.
+// A block = one window row and 8 x 4 consecutive units of the output; its waves walk the row's picks in order, the shared
+// expert last, four units of that expert's matrix a trip, so at any time the grid reads a few experts' matrices front to
+// back. The chain is the combine's: s = fmaf(w_k, part_k, s) over the picks in order, then s + sigmoid * shared; part_k is
+// a unit row's sum over its lanes. An expert that several rows picked is read once per row (from the caches after the
+// first). The q8_1 rows of h of the row's pairs come from the gate|up launch; a block copies its row's into LDS.
+// (With the rows made here from f32 gate|up outputs - SwiGLU, the 32-value maxima, the rounding, for eleven pairs a
+// block - this launch took 24 us instead of 18: that work stood between the launch's start and its first decode.)
+struct DownArgs {
+    int rows, ff, topk, T, nexp;
+    const uint8_t* w;          // routed experts: expert e at w + e * stride, or ep[e]
+    size_t stride;
+    const uint8_t* const* ep;
+    const uint8_t* w_shared;
+    const uint32_t* hq;        // the pairs' h rows in q8_1 form, [pair][ff / 32][HQ_WORDS], as the gate|up launch leaves them
+    const int* topi;
+    const float* topw;
+    const float* logits;       // [T][nexp + 1]: the shared expert's gate logit is a row's last
+    float* out;                // [T][rows]
+    const int* live;           // may be null; else a device word: rows from *live on are left alone
+    RouteArgs route;           // the job lists that the grid's last block writes
+};
+template <int SBR>
+__global__ void __launch_bounds__(FL_THREADS) k_moe_down_combine(const DownArgs a) {
+    constexpr int RW = 64 / SBR, R = 4;   // rows a unit, units a trip
+    __shared__ uint32_t tab[SGRID_WORDS];
+    __shared__ __align__(16) uint32_t hq[FL_MAXK + 1][SBR][HQ_WORDS];
+    const int tid = threadIdx.x, wave = uniform(tid >> 6), lane = tid & 63, kb = lane % SBR, g = lane / SBR;
+    const int nug = a.rows / (RW * R * FL_WAVES);   // blocks a window row
+    const int t = blockIdx.x / nug, ug = blockIdx.x % nug;
+    const int Tl = a.live ? uniform(max(0, min(*a.live, a.T))) : a.T;
+    if (blockIdx.x == gridDim.x - 1) {   // the spare block: the job lists for the caller
+        write_job_lists<FL_THREADS>(*reinterpret_cast<RouteLds<FL_THREADS>*>(tab), a.route, Tl);
+        return;
+    }
+    if (t >= Tl) return;
+    const int topk = a.topk, P = a.T * topk;
+    const uint32_t tab0 = g_sgrid.v[tid];
+    // the row's h rows: asked for first (they depend on nothing the block computes), a pick's words side by side
+    constexpr int HQ_PER = SBR * HQ_WORDS, HQ_VPT = ((FL_MAXK + 1) * HQ_PER + FL_THREADS - 1) / FL_THREADS;
+    uint32_t hw[HQ_VPT];
+#pragma unroll
+    for (int j = 0; j < HQ_VPT; ++j) {
+        const int i = tid + j * FL_THREADS, k = i / HQ_PER;
+        hw[j] = k <= topk ? a.hq[(size_t) (k < topk ? t * topk + k : P + t) * HQ_PER + (i - k * HQ_PER)] : 0u;
+    }
+    // lane k: pick k's matrix and weight; lane topk: the shared expert's and its gate
+    const uint8_t* myw = a.w_shared;
+    float myg = 0.f;
+    if (lane < topk) {
+        const int e = a.topi[t * topk + lane];
+        myw = a.ep ? a.ep[e] : a.w + (size_t) e * a.stride;
+        myg = a.topw[t * topk + lane];
+    } else if (lane == topk) myg = sigmoid_f(a.logits[(size_t) t * (a.nexp + 1) + a.nexp]);
+    const uint32_t myw_lo = (uint32_t) (uintptr_t) myw, myw_hi = (uint32_t) ((uint64_t) (uintptr_t) myw >> 32);
+    const int u0 = (ug * FL_WAVES + wave) * R;   // this wave's units of every matrix
+    const PackedOffs o = packed_offs(lane);
+    auto issue = [&](PackedSub(&buf)[R], int k) {
+        const uint64_t p = (uint64_t) (uint32_t) __builtin_amdgcn_readlane((int) myw_lo, k) | (uint64_t) (uint32_t) __builtin_amdgcn_readlane((int) myw_hi, k) << 32;
+        const uint8_t* we = (const uint8_t*) (uintptr_t) p + (size_t) u0 * UNIT_BYTES;
+#pragma unroll
+        for (int r = 0; r < R; ++r) buf[r] = load_packed(as_global(we + r * UNIT_BYTES), o);
+    };
+    PackedSub A[R], B[R], C[R];
+    issue(A, 0);
+    issue(B, 1);   // topk >= 1: the shared expert is trip topk
+#pragma unroll
+    for (int j = 0; j < HQ_VPT; ++j) {
+        const int i = tid + j * FL_THREADS;
+        if (i < (topk + 1) * HQ_PER) (&hq[0][0][0])[i] = hw[j];
     }
 #pragma unroll
     for (int i = 0; i < SGRID_WORDS / FL_THREADS; ++i) tab[tid + i * FL_THREADS] = signed_entry(tab0, i);
     __syncthreads();
-    const int kb = lane % SBR;
-    while (u < u1) {
-        const int slot0 = 2 * ((int) (u >> upj) - pass0);   // 0 or 2
-        auto prep_for = [&](auto nt_tag) {
-            constexpr int NT = decltype(nt_tag)::value;
-            return [=](int(&xs)[NT][8], float(&dx)[NT], float*(&orow)[NT]) {
-                const uint8_t* pairs = pl.job_pairs[s.ji] + s.t0;
+    const int sc_shift = 4 * (lane & 1);
+    float acc[R], res[R];
 #pragma unroll
-                for (int t = 0; t < NT; ++t) {
-                    const uint32_t* hb = hq[slot0 + t][kb];
-                    const uint4 lo = *reinterpret_cast<const uint4*>(hb), hi = *reinterpret_cast<const uint4*>(hb + 4);
-                    xs[t][0] = (int) lo.x, xs[t][1] = (int) lo.y, xs[t][2] = (int) lo.z, xs[t][3] = (int) lo.w;
-                    xs[t][4] = (int) hi.x, xs[t][5] = (int) hi.y, xs[t][6] = (int) hi.z, xs[t][7] = (int) hi.w;
-                    dx[t] = __uint_as_float(hb[8]);
-                    orow[t] = a.out + (size_t) uniform((int) pairs[t]) * a.rows;
-                }
-            };
-        };
-        if (s.nt >= 2) packed_units<SBR, 2>(tab, s.we, s.ul, s.ue, cur, prep_for(std::integral_constant<int, 2>{}));
-        else packed_units<SBR, 1>(tab, s.we, s.ul, s.ue, cur, prep_for(std::integral_constant<int, 1>{}));
-        u += s.ue - s.ul;
-        if (u < u1) {
-            s = pass_seg(pl, a, u, u1, upj);
-            packed_first(s.we, s.ul, s.ue, cur);
+    for (int r = 0; r < R; ++r) acc[r] = res[r] = 0.f;
+    auto decode = [&](const PackedSub(&buf)[R], int k) {
+        const uint32_t* hb = hq[k][kb];
+        const uint4 lo = *reinterpret_cast<const uint4*>(hb), hi = *reinterpret_cast<const uint4*>(hb + 4);
+        const int xs[8] = {(int) lo.x, (int) lo.y, (int) lo.z, (int) lo.w, (int) hi.x, (int) hi.y, (int) hi.z, (int) hi.w};
+        const float dx = __uint_as_float(hb[8]);
+        const float gk = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, myg), k));
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            int w4[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) w4[j] = *reinterpret_cast<const int*>(reinterpret_cast<const uint8_t*>(tab) + packed_addr(buf[r].idx, j));
+            const int sc = 1 + 2 * (int) ((buf[r].sc >> sc_shift) & 0xFu);
+            const float dw = half_bits_to_float(buf[r].d);
+            int sum = 0;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) sum = __builtin_amdgcn_sdot4(w4[j], xs[j], sum, false);
+            const float z = dpp_group_sum<SBR>((dw * dx) * (float) __mul24(sum, sc));
+            if (k < topk) acc[r] = fmaf(gk, z, acc[r]);
+            else res[r] = acc[r] + gk * z;
         }
+    };
+    for (int k = 0; k <= topk; k += 3) {
+        if (k + 2 <= topk) issue(C, k + 2);
+        decode(A, k);
+        if (k + 1 > topk) break;
+        if (k + 3 <= topk) issue(A, k + 3);
+        decode(B, k + 1);
+        if (k + 2 > topk) break;
+        if (k + 4 <= topk) issue(B, k + 4);
+        decode(C, k + 2);
+    }
+    if (kb == SBR - 1) {
+        float* orow = a.out + (size_t) t * a.rows + (size_t) u0 * RW + g;
+#pragma unroll
+        for (int r = 0; r < R; ++r) orow[r * RW] = res[r];
     }
 }
 

@@ -343,6 +343,17 @@ class Dev:
         return out.cpu().numpy()
 
 
+def pack_moe_weights(dev, ws, n, ff, packed):
+    """ws: the device tensors [gate|up, down, shared gate|up, shared down] as raw ggml blocks. packed: the load-time
+    re-laying to unit64, in place (fnx_iq3s_repack). Returns the tensors and their fnx_dw."""
+    pkg = dev.pkg
+    if packed:
+        for w in ws:
+            dev.ok(dev.lib.fnx_iq3s_repack(w.data_ptr(), w.data_ptr(), w.numel() // 110 * 256, dev.st()))
+    p = bool(packed)
+    return ws, [pkg.dw(ws[0], n, 2 * ff, packed=p), pkg.dw(ws[1], ff, n, packed=p), pkg.dw(ws[2], n, 2 * ff, packed=p), pkg.dw(ws[3], ff, n, packed=p)]
+
+
 class DecoderDev:
     """tiny_decoder.TinyDecoder on the device: weights, caches, workspace; verify / draft through the C ABI"""
 
@@ -363,13 +374,10 @@ class DecoderDev:
             return pkg.Q8S(up(tq[0]).data_ptr(), up(tq[1]).data_ptr(), rows, cols)
 
         def lay(L):
-            ws = [up(L[k]) for k in ("gu", "down", "sh_gu", "sh_down")]
-            if packed:
-                for w in ws:
-                    dev.ok(dev.lib.fnx_iq3s_repack(w.data_ptr(), w.data_ptr(), w.numel() // 110 * 256, dev.st()))
-            moe = pkg.MoeLayer(n, ff, nexp, topk, up(L["router"]).data_ptr(), 0, pkg.dw(ws[0], n, 2 * ff, packed=packed),
-                               2 * ff * (n // 256) * 110, pkg.dw(ws[1], ff, n, packed=packed), n * (ff // 256) * 110,
-                               pkg.dw(ws[2], n, 2 * ff, packed=packed), pkg.dw(ws[3], ff, n, packed=packed))
+            ws, dws = pack_moe_weights(dev, [up(L[k]) for k in ("gu", "down", "sh_gu", "sh_down")], n, ff, packed)
+            self.keep.extend(ws)
+            moe = pkg.MoeLayer(n, ff, nexp, topk, up(L["router"]).data_ptr(), 0, dws[0], 2 * ff * (n // 256) * 110, dws[1], n * (ff // 256) * 110,
+                               dws[2], dws[3])
             kc, vc = dev.zeros((c["max_ctx"], nkv, 256), t.float16), dev.zeros((c["max_ctx"], nkv, 256), t.float16)
             self.keep.extend([kc, vc])
             return pkg.DecLayer(up(L["attn_norm"]).data_ptr(), up(L["q_norm"]).data_ptr(), up(L["k_norm"]).data_ptr(), up(L["ffn_norm"]).data_ptr(),
@@ -485,12 +493,9 @@ class MoeLayerDev:
         self.gu, self.down, self.sh_gu, self.sh_down = dev.up(gu), dev.up(down), dev.up(sh_gu), dev.up(sh_down)
         self.gu_stride = 2 * ff * (n // 256) * 110
         self.down_stride = n * (ff // 256) * 110
-        if packed:   # the load-time re-laying, in place
-            for w in (self.gu, self.down, self.sh_gu, self.sh_down):
-                dev.ok(dev.lib.fnx_iq3s_repack(w.data_ptr(), w.data_ptr(), w.numel() // 110 * 256, dev.st()))
-        self.L = pkg.MoeLayer(n, ff, nexp, topk, self.router.data_ptr(), 0, pkg.dw(self.gu, n, 2 * ff, packed=packed), self.gu_stride,
-                              pkg.dw(self.down, ff, n, packed=packed), self.down_stride, pkg.dw(self.sh_gu, n, 2 * ff, packed=packed),
-                              pkg.dw(self.sh_down, ff, n, packed=packed))
+        # the load-time re-laying, in place
+        (self.gu, self.down, self.sh_gu, self.sh_down), dws = pack_moe_weights(dev, [self.gu, self.down, self.sh_gu, self.sh_down], n, ff, packed)
+        self.L = pkg.MoeLayer(n, ff, nexp, topk, self.router.data_ptr(), 0, dws[0], self.gu_stride, dws[1], self.down_stride, dws[2], dws[3])
         P = T * topk
         self.P = P
         self.xq = dev.zeros(T * (n // 32) * 36, t.uint8)
