@@ -1025,6 +1025,9 @@ int fnx_moe_verify_layer(const fnx_moe_layer* L, const float* x, int T, float* o
     return moe_layer_checked(L, x, T, out, ws, st);
 }
 
+#ifdef FNX_TS
+int fnx_dbg_ts(void* out) { return hipMemcpyFromSymbol(out, HIP_SYMBOL(g_ts), sizeof(g_ts)) == hipSuccess ? 0 : 1; }
+#endif
 // ---------------------------------------------------------------- streaming calibration (k_stream.h)
 int fnx_stream_read(const void* p, size_t bytes, int variant, int blocks, int threads, void* sink, void* st) {
     if (!p || !sink) return fail("stream_read: null argument");

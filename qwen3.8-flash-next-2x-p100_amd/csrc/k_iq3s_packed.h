@@ -57,6 +57,28 @@ __device__ __forceinline__ PackedSub load_packed(gbytes unit, const PackedOffs& 
     r.d = *(gu16*) (unit + od);
     return r;
 }
+// The same loads through a buffer descriptor: base = a matrix (wave-uniform), a scalar byte offset for the unit, the
+// lane's five offsets as they are - no vector arithmetic per load, and the planes' positions ride in the instructions.
+struct PackedVOffs {
+    int a, b, c, sc, d;
+};
+__device__ __forceinline__ PackedVOffs packed_voffs(int lane) {
+    return PackedVOffs{8 * lane, 4 * lane, lane, lane >> 1, 2 * (lane >> 3)};
+}
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t matrix_rsrc(const uint8_t* base) {   // base: wave-uniform
+    return __builtin_amdgcn_make_buffer_rsrc((void*) base, 0, -1, 0x00020000);
+}
+__device__ __forceinline__ PackedSub load_packed_buf(__amdgpu_buffer_rsrc_t m, int unit_byte, const PackedVOffs& o) {   // unit_byte: wave-uniform
+    PackedSub r;
+    const v2u a = __builtin_amdgcn_raw_buffer_load_b64(m, o.a, unit_byte, 0);
+    r.idx.x = a.x;
+    r.idx.y = a.y;
+    r.idx.z = __builtin_amdgcn_raw_buffer_load_b32(m, o.b + UNIT_B_AT, unit_byte, 0);
+    r.idx.w = __builtin_amdgcn_raw_buffer_load_b8(m, o.c + UNIT_C_AT, unit_byte, 0);
+    r.sc = __builtin_amdgcn_raw_buffer_load_b8(m, o.sc + UNIT_SCALES_AT, unit_byte, 0);
+    r.d = __builtin_amdgcn_raw_buffer_load_b16(m, o.d + UNIT_D_AT, unit_byte, 0);
+    return r;
+}
 // LDS byte address of group j's entry in the signed codebook: field j << 2
 __device__ __forceinline__ uint32_t packed_addr(const v4u& q, int j) {
     const int bit = 13 * j, w = bit >> 5, s = bit & 31;

@@ -32,6 +32,32 @@ __device__ __forceinline__ float wave_max(float v) {
 #undef FNX_DPP_MAX
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
+// Ranking by unsigned keys: key(v) rises with v (kernels.cu:1045-1083 uses the same key for its argmax), -0 counts as +0 as
+// in a float comparison, a NaN gets key 0 and so is never taken; a value can be picked if its key is above -inf's.
+__device__ __forceinline__ unsigned rank_key(float v) {
+    const unsigned u = __float_as_uint(v + 0.0f);
+    return v != v ? 0u : (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float rank_key_inv(unsigned k) { return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k); }
+constexpr unsigned RANK_KEY_NEG_INF = 0x007FFFFFu;
+// every lane: the greatest key of its row of 16 lanes (one instruction a step; the s_nop cover the wait states between a
+// vector write and a DPP read of the same register, which the compiler cannot see inside the asm)
+__device__ __forceinline__ unsigned row_umax(unsigned v) {
+    asm volatile(
+        "s_nop 1\n\tv_max_u32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\tv_max_u32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\tv_max_u32_dpp %0, %0, %0 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\tv_max_u32_dpp %0, %0, %0 row_mirror row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1"
+        : "+v"(v));
+    return v;
+}
+__device__ __forceinline__ unsigned wave_umax(unsigned v) {   // the wave's greatest key, in a scalar register
+    const int r = (int) row_umax(v);
+    const unsigned a = (unsigned) __builtin_amdgcn_readlane(r, 0), b = (unsigned) __builtin_amdgcn_readlane(r, 16);
+    const unsigned c = (unsigned) __builtin_amdgcn_readlane(r, 32), d = (unsigned) __builtin_amdgcn_readlane(r, 48);
+    return max(max(a, b), max(c, d));
+}
 __device__ __forceinline__ int wave_min(int v) {
 #define FNX_DPP_MIN(ctrl, rmask) v = min(v, __builtin_amdgcn_update_dpp(v, v, ctrl, rmask, 0xF, false))
     FNX_DPP_MIN(0xB1, 0xF);
@@ -273,7 +299,8 @@ __global__ void __launch_bounds__(FL_THREADS) k_router_quant(const RouterArgs a)
 // h = silu(gate) * up needs (k_moe_h, moe.cuh:597-608), 64 units of the pair's expert. A thread block of 16 waves takes
 // one item a sweep, four units a wave: gate rows 2 i, 2 i + 1 and up rows 2 i, 2 i + 1, whose four sums give two h values.
 // The items are numbered (row, block of 32, pick) and dealt to the blocks of the grid in runs: with a full window of 16
-// rows and 256 blocks a thread block has one row's one block of 32 for all the row's picks, the shared expert last. So
+// rows and 256 blocks a thread block has one row's one block of 32 for the shared expert and then all the row's picks
+// (the shared expert's matrix is known before the picks are: its loads are in flight while the row is ranked). So
 // it needs the picks of one row only (two when a run crosses rows): it ranks that row itself, a wave a row, while its
 // codebook loads are in flight - no launch of its own for the top-k (a kernel boundary on the window's critical path),
 // no list of jobs, no plan - and its lanes keep their activations for the whole launch. An expert that several rows
@@ -298,66 +325,74 @@ struct GateUpArgs {
 };
 struct GhLds {
     uint32_t tab[SGRID_WORDS];
-    uint32_t wp[2][FL_MAXK + 1][2];   // the matrices of the block's (at most two) rows' picks, the shared expert's last
-    float hb[GH_SLOTS][32];           // [slot][h value of the block]
+    uint32_t wp[2][FL_MAXK + 1][2];   // the matrices of the block's (at most two) rows: the shared expert's, then the picks'
+    float hg[GH_SLOTS][32], hu[GH_SLOTS][32];   // [slot][row of the block of 32]: the gate sums, the up sums
     int flag[GH_SLOTS][GH_WAVES];     // sweep + 1 of the values a wave last wrote into the slot
     int made[GH_SLOTS];               // sweeps whose block has been made from the slot: a writer of sweep s waits for made >= s - GH_SLOTS + 1
-    int ex[2][FL_MAXK];
+    uint2 cand[2][16][FL_MAXK];       // the rows' candidates: per slice of 64 experts its greatest (value, expert) in order
+    int sliced[2 * 16];               // set once a slice's candidates are written
+    int ready[2];                     // how many of a row's picks' matrices are known
 };
-struct GhItem {   // (row, block of 32, pick) of an item number, kept by stepping
+struct GhItem {   // (row, block of 32, matrix: 0 the shared expert's, k pick k - 1's) of an item number, kept by stepping
     int t, j, k;
 };
+#ifdef FNX_TS
+__device__ unsigned long long g_ts[4096][8];
+#define TS_NOW() wall_clock64()
+#endif
 __global__ void __launch_bounds__(GH_THREADS) k_moe_gate_up_h(const GateUpArgs a) {
     __shared__ GhLds S;
+#ifdef FNX_TS
+    unsigned long long ts[8];
+    ts[0] = TS_NOW();
+#endif
     const int tid = threadIdx.x, wave = uniform(tid >> 6), lane = tid & 63;
-    const int T = a.route.T, topk = a.route.topk, P = T * topk, qpp = a.ff >> 5, per_row = qpp * (topk + 1);
+    // The codebook's 512 unsigned entries, the launch's first load (the barrier below waits for nothing else). Every thread
+    // of the grid wants them as the launch starts: read from one place, those 2 KiB - sixteen cache lines - kept the blocks
+    // waiting for 2 to 3 us. The table in memory holds all sixteen signed forms, 2 KiB apart, and a signed form negated
+    // again is the unsigned one: the half-blocks read different forms.
+    const int form = (2 * (int) blockIdx.x + (tid >> 9)) & 15;
+    const uint32_t tab0 = signed_entry(g_sgrid.v[(form << 9) + (tid & 511)], form);
+    const int T = a.route.T, topk = a.route.topk, nexp = a.route.nexp, P = T * topk, qpp = a.ff >> 5, per_row = qpp * (topk + 1);
     const int Tl = a.route.live ? uniform(max(0, min(*a.route.live, T))) : T;
+    // Quotients of small numbers (below 2^14, the divisor a few hundred at most) by a multiplication: with the divisor's
+    // reciprocal rounded once and the dividend moved half a step up, the product misses the exact quotient by less than
+    // the distance to the next integer. (Every wave of every block works these out: as integer divisions they were half
+    // of what a wave executes before the barrier.)
+    const float r_nb = 1.0f / (float) gridDim.x, r_row = 1.0f / (float) per_row, r_k1 = 1.0f / (float) (topk + 1);
+    auto quot = [](int x, float r) { return (int) (((float) x + 0.5f) * r); };
     // this block's run of items
-    const int total = Tl * per_row, nb = gridDim.x, ipb = (total + nb - 1) / nb;
+    const int total = Tl * per_row, nb = gridDim.x, ipb = quot(total + nb - 1, r_nb);
     const int I0 = (int) blockIdx.x * ipb, I1 = min(total, I0 + ipb), nsweep = I1 - I0;
     if (nsweep <= 0) return;
-    const uint32_t tab0 = g_sgrid.v[tid & 511];
-    const int t0 = I0 / per_row, t1 = (I1 - 1) / per_row;   // ipb <= per_row (the launcher sees to it): two rows at most
-    auto load_x = [&](int t, int (&xs)[8], float& dx) {   // the lane's sub-block of row t's activations
-        const uint32_t* yb = reinterpret_cast<const uint32_t*>(a.xq + ((size_t) t * 64 + lane) * FNX_Q8_1_BLOCK);
-        dx = half_bits_to_float(yb[0] & 0xFFFFu);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) xs[j] = (int) yb[j + 1];
+    const int t0 = quot(I0, r_row), t1 = quot(I1 - 1, r_row);   // ipb <= per_row (the launcher sees to it): two rows at most
+    const int nr = t1 - t0 + 1, ns = (nexp + 63) >> 6;           // rows of the run, slices of 64 experts a row
+    // this wave's first slice of logits: asked for now, ranked once the codebook is in LDS
+    float v0 = -INFINITY;
+    if (wave < nr * ns) {
+        const int r = wave / ns, e = 64 * (wave - r * ns) + lane;
+        if (e < nexp) v0 = a.route.logits[(size_t) (t0 + r) * (nexp + 1) + e];
+    }
+    auto load_x = [&](int t, int (&xs)[8], float& dx) {   // the lane's sub-block of row t's activations: 36 bytes in three loads
+        typedef unsigned u4a __attribute__((ext_vector_type(4), aligned(4)));
+        const uint8_t* yb = a.xq + ((size_t) t * 64 + lane) * FNX_Q8_1_BLOCK;
+        const uint32_t head = *reinterpret_cast<const uint32_t*>(yb);
+        const u4a lo = *reinterpret_cast<const u4a*>(yb + 4), hi = *reinterpret_cast<const u4a*>(yb + 20);
+        dx = half_bits_to_float(head & 0xFFFFu);
+        xs[0] = (int) lo.x, xs[1] = (int) lo.y, xs[2] = (int) lo.z, xs[3] = (int) lo.w;
+        xs[4] = (int) hi.x, xs[5] = (int) hi.y, xs[6] = (int) hi.z, xs[7] = (int) hi.w;
     };
     int xs[8], tx = t0;
     float dx;
     load_x(t0, xs, dx);
-    if (wave < 2 && t0 + wave <= t1) {   // the rows' picks (moe.cuh:382-411), a wave a row; the row's first item's block writes them out
-        const int t = t0 + wave;
-        const bool publish = t * per_row >= I0;
-        const float* row = a.route.logits + (size_t) t * (a.route.nexp + 1);
-        if (a.route.nexp <= 512) wave_topk<8>(row, a.route.nexp, topk, lane, S.ex[wave], a.route.topi + t * topk, a.route.topw + t * topk, publish);
-        else wave_topk<16>(row, a.route.nexp, topk, lane, S.ex[wave], a.route.topi + t * topk, a.route.topw + t * topk, publish);
-        if (lane <= topk) {   // LDS writes of this wave, read back in order
-            const uint8_t* e = a.w_shared;
-            if (lane < topk) {
-                const int ei = S.ex[wave][lane];
-                e = a.ep ? a.ep[ei] : a.w + (size_t) ei * a.stride;
-            }
-            S.wp[wave][lane][0] = (uint32_t) (uintptr_t) e;
-            S.wp[wave][lane][1] = (uint32_t) ((uint64_t) (uintptr_t) e >> 32);
-        }
-    }
-    if (tid < GH_SLOTS * GH_WAVES) (&S.flag[0][0])[tid] = 0;
-    if (tid < GH_SLOTS) S.made[tid] = 0;
-    // the codebook: two threads a code, eight signed forms each
-#pragma unroll
-    for (int i = 0; i < 8; ++i) S.tab[tid + i * GH_THREADS] = signed_entry(tab0, (tid >> 9) + 2 * i);
-    __syncthreads();
-    const PackedOffs o = packed_offs(lane);
-    const int sc_shift = 4 * (lane & 1);
+    const PackedVOffs o = packed_voffs(lane);
     // byte offsets of the wave's gate units and up units from its item's first gate unit
-    const uint32_t uo_g = (uint32_t) (wave * 2) * UNIT_BYTES, uo_u = uo_g + (uint32_t) a.ff * UNIT_BYTES;
+    const int uo_g = wave * 2 * UNIT_BYTES, uo_u = uo_g + a.ff * UNIT_BYTES;
     auto item_of = [&](int I) {
         GhItem m;
-        m.t = I / per_row;
+        m.t = quot(I, r_row);
         const int r = I - m.t * per_row;
-        m.j = r / (topk + 1);
+        m.j = quot(r, r_k1);
         m.k = r - m.j * (topk + 1);
         return m;
     };
@@ -370,16 +405,163 @@ __global__ void __launch_bounds__(GH_THREADS) k_moe_gate_up_h(const GateUpArgs a
             }
         }
     };
-    auto issue = [&](PackedSub(&u)[4], const GhItem& m) {
-        const uint2 p = *reinterpret_cast<const uint2*>(S.wp[m.t - t0][m.k]);
-        const uint64_t e = (uint64_t) (uint32_t) uniform((int) p.x) | (uint64_t) (uint32_t) uniform((int) p.y) << 32;
-        const uint8_t* we = (const uint8_t*) (uintptr_t) e + (size_t) (m.j * 32) * UNIT_BYTES;
-        u[0] = load_packed(as_global(we + uo_g), o);
-        u[1] = load_packed(as_global(we + uo_g + UNIT_BYTES), o);
-        u[2] = load_packed(as_global(we + uo_u), o);
-        u[3] = load_packed(as_global(we + uo_u + UNIT_BYTES), o);
+    PackedSub A[4];
+    auto issue_from = [&](const uint8_t* e, int j) {   // e: wave-uniform
+        const __amdgpu_buffer_rsrc_t mtx = matrix_rsrc(e);
+        const int ub = j * 32 * UNIT_BYTES;
+        A[0] = load_packed_buf(mtx, ub + uo_g, o);
+        A[1] = load_packed_buf(mtx, ub + uo_g + UNIT_BYTES, o);
+        A[2] = load_packed_buf(mtx, ub + uo_u, o);
+        A[3] = load_packed_buf(mtx, ub + uo_u + UNIT_BYTES, o);
     };
-    // the q8_1 block of sweep q, by the first half of the wave
+    GhItem ma = item_of(I0);
+    const bool early = ma.k == 0;   // the run starts with a shared expert's item: no pick needed to ask for it
+    if (tid < GH_SLOTS * GH_WAVES) (&S.flag[0][0])[tid] = 0;
+    if (tid < GH_SLOTS) S.made[tid] = 0;
+    if (tid < 32) S.sliced[tid] = 0;
+    if (tid < 2) S.ready[tid] = 0;
+#ifdef FNX_TS
+    ts[5] = TS_NOW();
+#endif
+    // the codebook: two threads a code, eight signed forms each
+#pragma unroll
+    for (int i = 0; i < 8; ++i) S.tab[tid + i * GH_THREADS] = signed_entry(tab0, (tid >> 9) + 2 * i);
+#ifdef FNX_TS
+    ts[4] = TS_NOW();
+#endif
+    __syncthreads();
+    if (early) issue_from(a.w_shared, ma.j);   // (asked for ahead of the barrier, these twenty loads a wave held the waves up on their way to it)
+#ifdef FNX_TS
+    ts[1] = TS_NOW();
+#endif
+    // The rows' picks (moe.cuh:382-411: greater value first, the lower index on a tie; w_k = exp(l_k - l_0) / sum in pick
+    // order), without another barrier. Every wave lists the topk greatest of a slice of 64 experts, in order (a wave-wide
+    // maximum a round); a wave a row then merges the slices' lists by their heads while the other waves decode the shared
+    // expert's item, and says when the row's matrices are known. (One wave ranking a whole row, eight values a lane, took
+    // 4.5 us, with every other wave of the block waiting for it.)
+    if (wave < nr * ns) __builtin_amdgcn_s_setprio(2);
+    for (int task = wave; task < nr * ns; task += GH_WAVES) {
+        const int r = task / ns, sl = task - r * ns;
+        float v = v0;
+        if (task != wave) {
+            const int e = 64 * sl + lane;
+            v = e < nexp ? a.route.logits[(size_t) (t0 + r) * (nexp + 1) + e] : -INFINITY;
+        }
+        unsigned key = rank_key(v);
+        for (int k = 0; k < topk; ++k) {
+            const unsigned m = wave_umax(key);
+            const unsigned long long hold = m > RANK_KEY_NEG_INF ? __ballot(key == m) : 0ull;
+            const int l = hold ? (int) __builtin_ctzll(hold) : 64;   // the lowest lane that holds the maximum is the lowest expert
+            key = lane == l ? 0u : key;
+            if (lane == 0) S.cand[r][sl][k] = make_uint2(hold ? m : 0u, (uint32_t) (hold ? 64 * sl + l : nexp));
+        }
+        if (lane == 0) __hip_atomic_store(&S.sliced[task], 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    __builtin_amdgcn_s_setprio(0);
+#ifdef FNX_TS
+    ts[2] = TS_NOW();
+    ts[3] = ts[2];
+#endif
+    if (wave < nr) {   // the merge; the row's first item's block writes the picks and their weights out
+        const int t = t0 + wave;
+        const bool publish = t * per_row >= I0;
+        __builtin_amdgcn_s_setprio(3);   // the other waves of the block will soon wait for this one
+        while (true) {
+            const int f = lane < ns ? __hip_atomic_load(&S.sliced[wave * ns + lane], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) : 1;
+            if (__ballot(f == 0) == 0ull) break;
+            __builtin_amdgcn_s_sleep(1);
+        }
+        // All of the row's candidates in registers, entry p of list j in lane (16 j + p) mod 64 of register (16 j + p) / 64
+        // (the LDS is busy with the other waves' codebook reads: a read a round of a list's next entry took longer than the
+        // rest of the round). Lane j < ns keeps list j's head and its position; the list whose head is picked gets its next
+        // entry by a read of that lane.
+        static_assert(FL_MAXK == 16, "sixteen entries a list, four lists a register");
+        int ck[4], ce[4];
+        {
+            const uint2* flat = &S.cand[wave][0][0];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint2 c = flat[q * 64 + lane];
+                ck[q] = (int) c.x;
+                ce[q] = (int) c.y;
+            }
+        }
+        unsigned hk = lane < ns ? S.cand[wave][min(lane, ns - 1)][0].x : 0u;
+        int he = S.cand[wave][min(lane, ns - 1)][0].y, hp = 0;
+        unsigned mk = 0u;
+        int ei = 0x7fffffff;
+        unsigned long long low_taken = 0ull;   // which of experts 0 .. 63 are picked: what a row with fewer than topk finite logits falls back on
+        for (int k = 0; k < topk; ++k) {
+            unsigned m = (unsigned) __builtin_amdgcn_readlane((int) row_umax(hk), 0);
+            const unsigned long long hold = m > RANK_KEY_NEG_INF ? __ballot(hk == m) & 0xFFFFull : 0ull;
+            const int l = hold ? (int) __builtin_ctzll(hold) : 64;   // the lowest lane that holds the maximum has the lowest expert
+            int idx;
+            unsigned nk = 0u;
+            int ne = nexp, np = 0;
+            if (hold) {
+                idx = __builtin_amdgcn_readlane(he, l);
+                np = __builtin_amdgcn_readlane(hp, l) + 1;
+                if (np < topk) {   // list l's next entry
+                    const int f = 16 * l + np, fl = f & 63, fq = f >> 6;
+                    const int k0 = __builtin_amdgcn_readlane(ck[0], fl), k1 = __builtin_amdgcn_readlane(ck[1], fl);
+                    const int k2 = __builtin_amdgcn_readlane(ck[2], fl), k3 = __builtin_amdgcn_readlane(ck[3], fl);
+                    const int e0 = __builtin_amdgcn_readlane(ce[0], fl), e1 = __builtin_amdgcn_readlane(ce[1], fl);
+                    const int e2 = __builtin_amdgcn_readlane(ce[2], fl), e3 = __builtin_amdgcn_readlane(ce[3], fl);
+                    nk = (unsigned) (fq == 0 ? k0 : fq == 1 ? k1 : fq == 2 ? k2 : k3);
+                    ne = fq == 0 ? e0 : fq == 1 ? e1 : fq == 2 ? e2 : e3;
+                }
+            } else {   // nothing finite is left: the lowest expert not picked yet, with weight exp(-inf) = 0
+                m = RANK_KEY_NEG_INF;
+                idx = (int) __builtin_ctzll(~low_taken);
+            }
+            if (idx < 64) low_taken |= 1ull << idx;
+            if (lane == l) {
+                hk = nk;
+                he = ne;
+                hp = np;
+            }
+            if (lane == k) {
+                mk = m;
+                ei = idx;
+            }
+            {   // the pick's matrix is handed out at once: the sweeps need not wait for the whole ranking
+                const uint8_t* e = a.ep ? a.ep[idx] : a.w + (size_t) idx * a.stride;
+                if (lane == 0) {
+                    S.wp[wave][1 + k][0] = (uint32_t) (uintptr_t) e;
+                    S.wp[wave][1 + k][1] = (uint32_t) ((uint64_t) (uintptr_t) e >> 32);
+                    __hip_atomic_store(&S.ready[wave], k + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+                }
+            }
+        }
+        const float top0 = rank_key_inv((unsigned) __builtin_amdgcn_readlane((int) mk, 0));
+        const float ek = expf(rank_key_inv(mk) - top0);
+        float z = 0.f;
+        for (int k = 0; k < topk; ++k) z += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, ek), k));
+        if (publish && lane < topk) {
+            a.route.topi[t * topk + lane] = ei;
+            a.route.topw[t * topk + lane] = ek / z;
+        }
+        __builtin_amdgcn_s_setprio(0);
+#ifdef FNX_TS
+        ts[3] = TS_NOW();
+#endif
+    }
+    // an item's loads, once its matrix is known: matrix 0 is the shared expert's, matrix k pick k - 1's, known as soon as
+    // the merge has found it. (Walking the picks by ascending expert instead, so that rows which share an expert reach it
+    // together and the later read hits the L2 of their common XCD, cut the fabric's traffic by 5% - 127 against 134 MB -
+    // and gained nothing: it needs the whole ranking before the first pick's sweep.)
+    auto issue = [&](const GhItem& m) {
+        const uint8_t* e = a.w_shared;
+        if (m.k > 0) {
+            const int r = m.t - t0;
+            while (uniform(__hip_atomic_load(&S.ready[r], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP)) < m.k) __builtin_amdgcn_s_sleep(1);
+            const uint2 p = *reinterpret_cast<const uint2*>(S.wp[r][m.k]);
+            e = (const uint8_t*) (uintptr_t) ((uint64_t) (uint32_t) uniform((int) p.x) | (uint64_t) (uint32_t) uniform((int) p.y) << 32);
+        }
+        issue_from(e, m.j);
+    };
+    const int sc_shift = 4 * (lane & 1);
+    // the q8_1 block of sweep q, by the first half of the wave (k_moe_h, moe.cuh:597-608)
     auto make_block = [&](int q) {
         const int slot = q & (GH_SLOTS - 1);
         while (true) {   // all sixteen waves' values of sweep q must be there
@@ -388,9 +570,9 @@ __global__ void __launch_bounds__(GH_THREADS) k_moe_gate_up_h(const GateUpArgs a
             __builtin_amdgcn_s_sleep(2);
         }
         const GhItem m = item_of(I0 + q);
-        const int pair = m.k < topk ? m.t * topk + m.k : P + m.t;
+        const int pair = m.k > 0 ? m.t * topk + m.k - 1 : P + m.t;
         if (lane < 32) {
-            const float h = S.hb[slot][lane];
+            const float h = silu_f(S.hg[slot][lane]) * S.hu[slot][lane];
             const float amax = group_max<32>(fabsf(h));
             const float d = amax / 127.0f;
             const uint32_t qv = amax == 0.0f ? 0u : (uint32_t) (uint8_t) (int8_t) roundf(h / d);
@@ -402,54 +584,63 @@ __global__ void __launch_bounds__(GH_THREADS) k_moe_gate_up_h(const GateUpArgs a
         }
         if (lane == 0) __hip_atomic_store(&S.made[slot], q + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     };
-    auto decode = [&](const PackedSub(&u)[4], const GhItem& m, int sw) {
+    // where a lane's sum goes after reduce4_units: the 16-lane rows hold gate 2 i, up 2 i, gate 2 i + 1, up 2 i + 1
+    float* const zdst0 = (lane & 16 ? &S.hu[0][0] : &S.hg[0][0]) + 2 * wave + (lane >> 5);
+    auto decode = [&](const GhItem& m, int sw) {
         if (m.t != tx) {   // the run has crossed into its second row
             tx = m.t;
             load_x(tx, xs, dx);
         }
+        const int slot = sw & (GH_SLOTS - 1);
+        // the slot's last block (of sweep sw - GH_SLOTS) must have been made: nearly always long ago (asked here, used below)
+        int made = sw >= GH_SLOTS ? __hip_atomic_load(&S.made[slot], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) : 0;
         float v[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             int w4[8];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) w4[j] = *reinterpret_cast<const int*>(reinterpret_cast<const uint8_t*>(S.tab) + packed_addr(u[r].idx, j));
-            const int sc = 1 + 2 * (int) ((u[r].sc >> sc_shift) & 0xFu);
-            const float dw = half_bits_to_float(u[r].d);
+            for (int j = 0; j < 8; ++j) w4[j] = *reinterpret_cast<const int*>(reinterpret_cast<const uint8_t*>(S.tab) + packed_addr(A[r].idx, j));
+            const int sc = 1 + 2 * (int) ((A[r].sc >> sc_shift) & 0xFu);
+            const float dw = half_bits_to_float(A[r].d);
             int sum = 0;
 #pragma unroll
             for (int j = 0; j < 8; ++j) sum = __builtin_amdgcn_sdot4(w4[j], xs[j], sum, false);
             // one sub-block's term as the reference forms it: (d_w * d_x) * (float) (sumi * (1 + 2 s))
             v[r] = (dw * dx) * (float) __mul24(sum, sc);
         }
-        // units: gate 2 i, gate 2 i + 1, up 2 i, up 2 i + 1 -> the 16-lane rows hold gate 2 i, up 2 i, gate 2 i + 1, up 2 i + 1
+        // units: gate 2 i, gate 2 i + 1, up 2 i, up 2 i + 1
         const float z = reduce4_units(v[0], v[1], v[2], v[3]);
-        const int zi = __builtin_bit_cast(int, z);
-        const float g0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(zi, 0)), u0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(zi, 16));
-        const float g1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(zi, 32)), u1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(zi, 48));
-        const float h = silu_f(lane & 1 ? g1 : g0) * (lane & 1 ? u1 : u0);   // lane 0: h of row 2 i, lane 1: of row 2 i + 1
-        const int slot = sw & (GH_SLOTS - 1);
-        // the slot's last block (of sweep sw - GH_SLOTS) must have been made: nearly always long ago
         if (sw >= GH_SLOTS)
-            while (uniform(__hip_atomic_load(&S.made[slot], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP)) < sw - GH_SLOTS + 1) __builtin_amdgcn_s_sleep(1);
-        if (lane < 2) S.hb[slot][2 * wave + lane] = h;
+            while (uniform(made) < sw - GH_SLOTS + 1) {
+                __builtin_amdgcn_s_sleep(1);
+                made = __hip_atomic_load(&S.made[slot], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
+        if ((lane & 15) == 0) zdst0[slot * 32] = z;
         if (lane == 0) __hip_atomic_store(&S.flag[slot][wave], sw + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    };
+    // Every wave of the block makes the same sweeps: each slot sees all sixteen arrive. An item's loads are asked for when
+    // the item before it has been decoded: with sixteen waves a CU that keeps about 56 KB a CU in flight, which is what HBM
+    // serves best (an item ahead - twice as much in flight - was measured slower, 35.1 against 33.8 us).
+    if (!early) issue(ma);
+    for (int sw = 0; sw < nsweep; ++sw) {
+#ifdef FNX_TS
+        if (sw == 1) ts[6] = TS_NOW();
+#endif
+        decode(ma, sw);
+        if (sw + 1 < nsweep) {
+            step(ma);
+            issue(ma);
+        }
         const int q = sw - GH_LAG;   // the sweep whose block is due; wave q mod 16 makes it
         if (q >= 0 && (q & (GH_WAVES - 1)) == wave) make_block(q);
-    };
-    // every wave of the block makes the same sweeps: each slot sees all sixteen arrive
-    PackedSub cur[4], nxt[4];
-    GhItem mc = item_of(I0), mn = mc;
-    issue(cur, mc);
-    for (int sw = 0; sw < nsweep; ++sw) {
-        if (sw + 1 < nsweep) step(mn);
-        issue(nxt, mn);   // past the end: the last item again (a read of what the caches hold)
-        decode(cur, mc, sw);
-#pragma unroll
-        for (int r = 0; r < 4; ++r) cur[r] = nxt[r];
-        mc = mn;
     }
     for (int q = max(nsweep - GH_LAG, 0); q < nsweep; ++q)   // the last sweeps' blocks
         if ((q & (GH_WAVES - 1)) == wave) make_block(q);
+#ifdef FNX_TS
+    ts[7] = TS_NOW();
+    if (lane == 0)
+        for (int i = 0; i < 8; ++i) g_ts[blockIdx.x * GH_WAVES + wave][i] = ts[i];
+#endif
 }
 
 // ---------------------------------------------------------------- launch 3: down and the combine
