@@ -336,16 +336,8 @@ struct GhLds {
 struct GhItem {   // (row, block of 32, matrix: 0 the shared expert's, k pick k - 1's) of an item number, kept by stepping
     int t, j, k;
 };
-#ifdef FNX_TS
-__device__ unsigned long long g_ts[4096][8];
-#define TS_NOW() wall_clock64()
-#endif
 __global__ void __launch_bounds__(GH_THREADS) k_moe_gate_up_h(const GateUpArgs a) {
     __shared__ GhLds S;
-#ifdef FNX_TS
-    unsigned long long ts[8];
-    ts[0] = TS_NOW();
-#endif
     const int tid = threadIdx.x, wave = uniform(tid >> 6), lane = tid & 63;
     // The codebook's 512 unsigned entries, the launch's first load (the barrier below waits for nothing else). Every thread
     // of the grid wants them as the launch starts: read from one place, those 2 KiB - sixteen cache lines - kept the blocks
@@ -420,20 +412,11 @@ __global__ void __launch_bounds__(GH_THREADS) k_moe_gate_up_h(const GateUpArgs a
     if (tid < GH_SLOTS) S.made[tid] = 0;
     if (tid < 32) S.sliced[tid] = 0;
     if (tid < 2) S.ready[tid] = 0;
-#ifdef FNX_TS
-    ts[5] = TS_NOW();
-#endif
     // the codebook: two threads a code, eight signed forms each
 #pragma unroll
     for (int i = 0; i < 8; ++i) S.tab[tid + i * GH_THREADS] = signed_entry(tab0, (tid >> 9) + 2 * i);
-#ifdef FNX_TS
-    ts[4] = TS_NOW();
-#endif
     __syncthreads();
     if (early) issue_from(a.w_shared, ma.j);   // (asked for ahead of the barrier, these twenty loads a wave held the waves up on their way to it)
-#ifdef FNX_TS
-    ts[1] = TS_NOW();
-#endif
     // The rows' picks (moe.cuh:382-411: greater value first, the lower index on a tie; w_k = exp(l_k - l_0) / sum in pick
     // order), without another barrier. Every wave lists the topk greatest of a slice of 64 experts, in order (a wave-wide
     // maximum a round); a wave a row then merges the slices' lists by their heads while the other waves decode the shared
@@ -458,10 +441,6 @@ __global__ void __launch_bounds__(GH_THREADS) k_moe_gate_up_h(const GateUpArgs a
         if (lane == 0) __hip_atomic_store(&S.sliced[task], 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
     __builtin_amdgcn_s_setprio(0);
-#ifdef FNX_TS
-    ts[2] = TS_NOW();
-    ts[3] = ts[2];
-#endif
     if (wave < nr) {   // the merge; the row's first item's block writes the picks and their weights out
         const int t = t0 + wave;
         const bool publish = t * per_row >= I0;
@@ -542,9 +521,6 @@ __global__ void __launch_bounds__(GH_THREADS) k_moe_gate_up_h(const GateUpArgs a
             a.route.topw[t * topk + lane] = ek / z;
         }
         __builtin_amdgcn_s_setprio(0);
-#ifdef FNX_TS
-        ts[3] = TS_NOW();
-#endif
     }
     // an item's loads, once its matrix is known: matrix 0 is the shared expert's, matrix k pick k - 1's, known as soon as
     // the merge has found it. (Walking the picks by ascending expert instead, so that rows which share an expert reach it
@@ -623,9 +599,6 @@ __global__ void __launch_bounds__(GH_THREADS) k_moe_gate_up_h(const GateUpArgs a
     // serves best (an item ahead - twice as much in flight - was measured slower, 35.1 against 33.8 us).
     if (!early) issue(ma);
     for (int sw = 0; sw < nsweep; ++sw) {
-#ifdef FNX_TS
-        if (sw == 1) ts[6] = TS_NOW();
-#endif
         decode(ma, sw);
         if (sw + 1 < nsweep) {
             step(ma);
@@ -636,11 +609,6 @@ __global__ void __launch_bounds__(GH_THREADS) k_moe_gate_up_h(const GateUpArgs a
     }
     for (int q = max(nsweep - GH_LAG, 0); q < nsweep; ++q)   // the last sweeps' blocks
         if ((q & (GH_WAVES - 1)) == wave) make_block(q);
-#ifdef FNX_TS
-    ts[7] = TS_NOW();
-    if (lane == 0)
-        for (int i = 0; i < 8; ++i) g_ts[blockIdx.x * GH_WAVES + wave][i] = ts[i];
-#endif
 }
 
 // ---------------------------------------------------------------- launch 3: down and the combine
@@ -681,9 +649,12 @@ __global__ void __launch_bounds__(FL_THREADS) k_moe_down_combine(const DownArgs 
         return;
     }
     if (t >= Tl) return;
+    // the codebook's unsigned entries, the launch's first load; the blocks read different signed forms of the table in
+    // memory and negate them back, so that not every wave of the grid asks the same sixteen cache lines at once
+    const int form = (int) blockIdx.x & 15;
+    const uint32_t tab0 = signed_entry(g_sgrid.v[(form << 9) + tid], form);
     const int topk = a.topk, P = a.T * topk;
-    const uint32_t tab0 = g_sgrid.v[tid];
-    // the row's h rows: asked for first (they depend on nothing the block computes), a pick's words side by side
+    // the row's h rows: asked for next (they depend on nothing the block computes), a pick's words side by side
     constexpr int HQ_PER = SBR * HQ_WORDS, HQ_VPT = ((FL_MAXK + 1) * HQ_PER + FL_THREADS - 1) / FL_THREADS;
     uint32_t hw[HQ_VPT];
 #pragma unroll
@@ -701,29 +672,37 @@ __global__ void __launch_bounds__(FL_THREADS) k_moe_down_combine(const DownArgs 
     } else if (lane == topk) myg = sigmoid_f(a.logits[(size_t) t * (a.nexp + 1) + a.nexp]);
     const uint32_t myw_lo = (uint32_t) (uintptr_t) myw, myw_hi = (uint32_t) ((uint64_t) (uintptr_t) myw >> 32);
     const int u0 = (ug * FL_WAVES + wave) * R;   // this wave's units of every matrix
-    const PackedOffs o = packed_offs(lane);
+    const PackedVOffs o = packed_voffs(lane);
     auto issue = [&](PackedSub(&buf)[R], int k) {
         const uint64_t p = (uint64_t) (uint32_t) __builtin_amdgcn_readlane((int) myw_lo, k) | (uint64_t) (uint32_t) __builtin_amdgcn_readlane((int) myw_hi, k) << 32;
-        const uint8_t* we = (const uint8_t*) (uintptr_t) p + (size_t) u0 * UNIT_BYTES;
+        const __amdgpu_buffer_rsrc_t mtx = matrix_rsrc((const uint8_t*) (uintptr_t) p);
 #pragma unroll
-        for (int r = 0; r < R; ++r) buf[r] = load_packed(as_global(we + r * UNIT_BYTES), o);
+        for (int r = 0; r < R; ++r) buf[r] = load_packed_buf(mtx, (u0 + r) * UNIT_BYTES, o);
     };
+    // Trip 0 is the shared expert's (its matrix is known without the picks: its loads go out with the launch's first),
+    // trips 1 .. topk the picks in order; the shared expert's sums wait in registers for the chain's last step.
+    auto pick_of = [&](int trip) { return trip == 0 ? topk : trip - 1; };   // the index of a trip's expert in hq and in the lanes
     PackedSub A[R], B[R], C[R];
-    issue(A, 0);
-    issue(B, 1);   // topk >= 1: the shared expert is trip topk
+    {
+        const __amdgpu_buffer_rsrc_t mtx = matrix_rsrc(a.w_shared);
+#pragma unroll
+        for (int r = 0; r < R; ++r) A[r] = load_packed_buf(mtx, (u0 + r) * UNIT_BYTES, o);
+    }
+#pragma unroll
+    for (int i = 0; i < SGRID_WORDS / FL_THREADS; ++i) tab[tid + i * FL_THREADS] = signed_entry(tab0, i);
 #pragma unroll
     for (int j = 0; j < HQ_VPT; ++j) {
         const int i = tid + j * FL_THREADS;
         if (i < (topk + 1) * HQ_PER) (&hq[0][0][0])[i] = hw[j];
     }
-#pragma unroll
-    for (int i = 0; i < SGRID_WORDS / FL_THREADS; ++i) tab[tid + i * FL_THREADS] = signed_entry(tab0, i);
+    issue(B, pick_of(1));   // topk >= 1
     __syncthreads();
     const int sc_shift = 4 * (lane & 1);
-    float acc[R], res[R];
+    float acc[R], zs[R];
 #pragma unroll
-    for (int r = 0; r < R; ++r) acc[r] = res[r] = 0.f;
-    auto decode = [&](const PackedSub(&buf)[R], int k) {
+    for (int r = 0; r < R; ++r) acc[r] = zs[r] = 0.f;
+    auto decode = [&](const PackedSub(&buf)[R], int trip) {
+        const int k = pick_of(trip);
         const uint32_t* hb = hq[k][kb];
         const uint4 lo = *reinterpret_cast<const uint4*>(hb), hi = *reinterpret_cast<const uint4*>(hb + 4);
         const int xs[8] = {(int) lo.x, (int) lo.y, (int) lo.z, (int) lo.w, (int) hi.x, (int) hi.y, (int) hi.z, (int) hi.w};
@@ -740,20 +719,24 @@ __global__ void __launch_bounds__(FL_THREADS) k_moe_down_combine(const DownArgs 
 #pragma unroll
             for (int j = 0; j < 8; ++j) sum = __builtin_amdgcn_sdot4(w4[j], xs[j], sum, false);
             const float z = dpp_group_sum<SBR>((dw * dx) * (float) __mul24(sum, sc));
-            if (k < topk) acc[r] = fmaf(gk, z, acc[r]);
-            else res[r] = acc[r] + gk * z;
+            if (trip == 0) zs[r] = gk * z;
+            else acc[r] = fmaf(gk, z, acc[r]);
         }
     };
-    for (int k = 0; k <= topk; k += 3) {
-        if (k + 2 <= topk) issue(C, k + 2);
-        decode(A, k);
-        if (k + 1 > topk) break;
-        if (k + 3 <= topk) issue(A, k + 3);
-        decode(B, k + 1);
-        if (k + 2 > topk) break;
-        if (k + 4 <= topk) issue(B, k + 4);
-        decode(C, k + 2);
+    // two trips' loads are in flight while a third is decoded: with eight waves a CU that is about 56 KB a CU
+    for (int trip = 0; trip <= topk; trip += 3) {
+        if (trip + 2 <= topk) issue(C, pick_of(trip + 2));
+        decode(A, trip);
+        if (trip + 1 > topk) break;
+        if (trip + 3 <= topk) issue(A, pick_of(trip + 3));
+        decode(B, trip + 1);
+        if (trip + 2 > topk) break;
+        if (trip + 4 <= topk) issue(B, pick_of(trip + 4));
+        decode(C, trip + 2);
     }
+    float res[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) res[r] = acc[r] + zs[r];   // the combine's last step: s + sigmoid * shared
     if (kb == SBR - 1) {
         float* orow = a.out + (size_t) t * a.rows + (size_t) u0 * RW + g;
 #pragma unroll
