@@ -166,6 +166,15 @@ typedef struct fnx_moe_ws {
     float* part;     /* [T * topk + T][n] */
 } fnx_moe_ws;
 int fnx_moe_verify_layer(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st);
+/* The same window without a workspace argument and without any allocation: no counterpart in the reference. For callers
+ * that cannot allocate device memory (code under graph capture, serving loops and harnesses that forbid it): the scratch
+ * of fnx_moe_ws lives in one array of FNX_MOE_STATIC_WS_BYTES in the library's device image, which each GPU the library
+ * runs on holds until the process ends. Only the three-launch window runs on it: unit64 experts, hidden 2048, ff 256,
+ * 512 or 1024, up to 1024 experts, up to 16 picks a row, T x topk <= 160; anything else is refused with a message. x and
+ * out are the caller's, as above; results are those of fnx_moe_verify_layer bit for bit. All calls on a GPU share that
+ * GPU's array: two of them in flight at once (two streams, two threads) race. */
+#define FNX_MOE_STATIC_WS_BYTES (448 * 1024)
+int fnx_moe_verify_layer_static(const fnx_moe_layer* L, const float* x, int T, float* out, void* st);
 /* Profiling aid, the counterpart of the reference's FNX_PROF stamps in its window graph (engine.cu:1382-1530):
  * fnx_layer_profile(1) makes the five-launch window record events on its stream around each launch (not to be
  * used under graph capture), fnx_layer_profile(0) stops that; fnx_layer_profile_read waits for the last recorded

@@ -1025,9 +1025,49 @@ int fnx_moe_verify_layer(const fnx_moe_layer* L, const float* x, int T, float* o
     return moe_layer_checked(L, x, T, out, ws, st);
 }
 
-#ifdef FNX_TS
-int fnx_dbg_ts(void* out) { return hipMemcpyFromSymbol(out, HIP_SYMBOL(g_ts), sizeof(g_ts)) == hipSuccess ? 0 : 1; }
-#endif
+// ---------------------------------------------------------------- the window on a workspace of the library's own
+// fnx_moe_verify_layer with its scratch (the q8_1 rows of x, the logits, the picks and weights, the job lists, the q8_1
+// rows of h) in a file-scope device array instead of a caller's fnx_moe_ws, for callers that cannot allocate. The array's
+// name is only a host-side handle: its device address is asked for once per device (hipGetSymbolAddress) and kept.
+constexpr size_t NA_XQ = (size_t) FNX_MAXT * (FL_N / 32) * FNX_Q8_1_BLOCK;            // 36,864
+constexpr size_t NA_LOGITS = (size_t) FNX_MAXT * (1024 + 1) * sizeof(float);           // 65,600
+constexpr size_t NA_TOP = (size_t) FL_MAXP * sizeof(int);                              // 640 (topi), 640 (topw)
+constexpr size_t NA_JOBS = (size_t) (FL_MAXP + 1) * sizeof(fnx_job);                   // 21,896 each
+constexpr size_t NA_HQ = (size_t) (FL_MAXP + FNX_MAXT) * (1024 / 32) * HQ_WORDS * 4;   // 270,336
+constexpr size_t na_up(size_t v) { return (v + 255) / 256 * 256; }
+constexpr size_t NA_OFF_LOGITS = na_up(NA_XQ), NA_OFF_TOPI = NA_OFF_LOGITS + na_up(NA_LOGITS), NA_OFF_TOPW = NA_OFF_TOPI + na_up(NA_TOP),
+                 NA_OFF_JGU = NA_OFF_TOPW + na_up(NA_TOP), NA_OFF_JDN = NA_OFF_JGU + na_up(NA_JOBS), NA_OFF_NJOBS = NA_OFF_JDN + na_up(NA_JOBS),
+                 NA_OFF_HQ = NA_OFF_NJOBS + 256, NA_BYTES = NA_OFF_HQ + na_up(NA_HQ);
+static_assert(NA_BYTES <= FNX_MOE_STATIC_WS_BYTES, "the header states the array's size");
+static __device__ __align__(256) unsigned char scratch[FNX_MOE_STATIC_WS_BYTES];
+static unsigned char* g_scratch_ptr[64] = {};   // per device: the array's address there
+int fnx_moe_verify_layer_static(const fnx_moe_layer* L, const float* x, int T, float* out, void* st) {
+    if (!L || !x || !out) return fail("moe_verify_layer_static: null argument");
+    if (T < 1 || T > FNX_MAXT) return fail("moe_verify_layer_static: T out of range");
+    if (!layer_fused_ok(L, T))
+        return fail("moe_verify_layer_static: only the three-launch window runs on the library's own workspace (unit64 experts, hidden 2048, "
+                    "ff 256 / 512 / 1024, up to 1024 experts, up to 16 picks a row, up to 160 pairs a window)");
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return fail("moe_verify_layer_static: no current device");
+    if (!g_scratch_ptr[dev]) {
+        unsigned char* p = nullptr;
+        const hipError_t e = hipGetSymbolAddress((void**) &p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) return fail(std::string("moe_verify_layer_static: hipGetSymbolAddress: ") + hipGetErrorString(e));
+        g_scratch_ptr[dev] = p;
+    }
+    unsigned char* w = g_scratch_ptr[dev];
+    // nothing in the workspace has to start at zero: every launch writes what it reads, and the job count is stored, not added to
+    const fnx_moe_ws ws{w, (float*) (w + NA_OFF_LOGITS), (int*) (w + NA_OFF_TOPI), (float*) (w + NA_OFF_TOPW), (fnx_job*) (w + NA_OFF_JGU),
+                        (fnx_job*) (w + NA_OFF_JDN), (int*) (w + NA_OFF_NJOBS), (float*) (w + NA_OFF_HQ), nullptr};
+    const int P = T * L->topk, n = L->n, ff = L->ff;
+    if (L->gu.n_in != n || L->gu.n_out != 2 * ff || L->down.n_in != ff || L->down.n_out != n || L->sh_gu.n_in != n ||
+        L->sh_gu.n_out != 2 * ff || L->sh_down.n_in != ff || L->sh_down.n_out != n)
+        return fail("moe_verify_layer_static: weight shapes do not match n / ff");
+    if (topk_check(T, L->nexp, L->topk, "moe_verify_layer_static")) return 1;
+    (void) P;
+    return layer_fused(L, x, T, out, &ws, st);
+}
+
 // ---------------------------------------------------------------- streaming calibration (k_stream.h)
 int fnx_stream_read(const void* p, size_t bytes, int variant, int blocks, int threads, void* sink, void* st) {
     if (!p || !sink) return fail("stream_read: null argument");
