@@ -1152,8 +1152,27 @@ static void dense_q8s(const fnx_o_q8s* W, const float* x, int T, float* out) { /
     fnx_o_q8s_gemv(W->q, W->d, W->n_out, W->n_in, xq, out, W->n_out, T);
     free(xq);
 }
+/* a test's view into the layers' routing: when set, the next `layers` calls of dec_layer copy their router logits
+ * ([T][nexp + 1]) and picks ([T][topk]) to consecutive slots of these arrays */
+static float* g_probe_logits;
+static int* g_probe_topi;
+static int g_probe_left, g_probe_at;
+void fnx_o_layer_probe(float* logits, int* topi, int layers) {
+    g_probe_logits = logits;
+    g_probe_topi = topi;
+    g_probe_left = logits && topi ? layers : 0;
+    g_probe_at = 0;
+}
 static void dec_layer(const fnx_o_decoder* D, const fnx_o_dec_layer* L, float* x, int T, int pos0, int threads) {
     const int n = D->n, nq = D->nq, nkv = D->nkv, hd = 256, nrot = 64;
+    float* probe_l = NULL;
+    int* probe_i = NULL;
+    if (g_probe_left > 0) {
+        probe_l = g_probe_logits + (size_t) g_probe_at * T * (L->moe.nexp + 1);
+        probe_i = g_probe_topi + (size_t) g_probe_at * T * L->moe.topk;
+        --g_probe_left;
+        ++g_probe_at;
+    }
     float* xn = (float*) malloc((size_t) T * n * sizeof(float));
     float* qg = (float*) malloc((size_t) T * nq * 2 * hd * sizeof(float));
     float* k = (float*) malloc((size_t) T * nkv * hd * sizeof(float));
@@ -1169,7 +1188,7 @@ static void dec_layer(const fnx_o_decoder* D, const fnx_o_dec_layer* L, float* x
     dense_q8s(&L->wo, att, T, o);
     for (size_t i = 0; i < (size_t) T * n; ++i) x[i] += o[i];
     fnx_o_rms_norm_rows(x, L->ffn_norm, xn, T, n, D->eps);
-    fnx_o_moe_verify_layer(&L->moe, xn, T, o, NULL, NULL, NULL, NULL, threads);
+    fnx_o_moe_verify_layer(&L->moe, xn, T, o, probe_l, probe_i, NULL, NULL, threads);
     for (size_t i = 0; i < (size_t) T * n; ++i) x[i] += o[i];
     free(xn); free(qg); free(k); free(v); free(att); free(o);
 }

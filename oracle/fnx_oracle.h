@@ -207,6 +207,9 @@ typedef struct {
 } fnx_o_mtp;
 /* the reduced decoder's window (engine.cu Engine::enqueue without streams, cards, GDN layers): hidden [T][n], logits
  * [T][vocab] (may be null), best [T] = argmax rows */
+/* test probe: the next `layers` decoder layers run (by either function below) copy their router logits [T][nexp + 1] and
+ * picks [T][topk] into consecutive slots of the two arrays; null pointers switch it off */
+void fnx_o_layer_probe(float* logits, int* topi, int layers);
 void fnx_o_decoder_verify(const fnx_o_decoder* D, const int* tokens, int T, int pos0, float* hidden, float* logits, int* best, int threads);
 /* engine.cu:2095-2133 without streams: R = fc_hid(rms(src)) + fc_emb(rms(emb[tokens])), one layer, norm, head, argmax */
 void fnx_o_mtp_draft(const fnx_o_decoder* D, const fnx_o_mtp* M, const float* src, const int* tokens, int T, int pos0, float* hidden,

@@ -22,9 +22,13 @@ def package():
     return mod
 
 
-def random_iq3s(rng, nblocks, dmax=3e-4):
-    """valid IQ3_S blocks with uniformly random codes, signs and scales (any byte pattern is a valid block)"""
-    b = rng.integers(0, 256, size=(nblocks, 110), dtype=np.uint8)
+def random_iq3s(rng, nblocks, dmax=3e-4, raw_bytes=False):
+    """valid IQ3_S blocks with uniformly random codes, signs and scales (any byte pattern is a valid block).
+    raw_bytes: the generator's byte stream as it comes (other values than the default draws; much faster for gigabytes)"""
+    if raw_bytes:
+        b = rng.integers(0, 1 << 64, size=(nblocks * 110 + 7) // 8, dtype=np.uint64).view(np.uint8)[:nblocks * 110].reshape(nblocks, 110)
+    else:
+        b = rng.integers(0, 256, size=(nblocks, 110), dtype=np.uint8)
     d = (rng.random(nblocks) * dmax + 1e-5).astype(np.float16)
     b[:, 0:2] = d.view(np.uint8).reshape(nblocks, 2)
     return b.reshape(-1)
@@ -419,6 +423,15 @@ class DecoderDev:
             out.append((k, v_rows(v)))
         return out
 
+    def set_caches(self, cells):
+        """cells: per layer (the draft layer last) a pair of [pos][nkv][256] float16 arrays, written from position 0"""
+        for (kc, vc), (k, v) in zip(self.caches + [self.mtp_cache], cells):
+            p = k.shape[0]
+            assert p % 4 == 0 and p <= self.c["max_ctx"]
+            kc[:p].copy_(self.dev.up(np.ascontiguousarray(k)))
+            vc.view(self.dev.torch.float16).reshape(-1)[:v.size].copy_(self.dev.up(v_blocked(v)).reshape(-1))
+        self.dev.sync()
+
     def _result(self, T):
         return dict(hidden=self.b["hidden"].cpu().numpy()[:T], logits=self.b["logits"].cpu().numpy()[:T], best=self.b["best_i"].cpu().numpy()[:T],
                     err=int(self.b["err"].item()))
@@ -430,6 +443,25 @@ class DecoderDev:
         dev.ok(dev.lib.fnx_decoder_verify(C.byref(self.D), tok.data_ptr(), len(tokens), self.pos.data_ptr(), C.byref(self.ws), dev.st()))
         dev.sync()
         return self._result(len(tokens))
+
+    def routing(self, T):
+        """the router logits and picks the last MoE layer run left in the workspace"""
+        return self.mb["logits"].cpu().numpy()[:T], self.mb["topi"].cpu().numpy()[:T]
+
+    def verify_routing(self, tokens, pos0):
+        """every layer's router logits and picks for this window: the window run at depths 1 .. nlayers (the workspace
+        keeps the last layer's; the cells a shallower run writes are the ones the full run writes)"""
+        lg, ti = [], []
+        for depth in range(1, self.c["nlayers"] + 1):
+            self.D.nlayers = depth
+            try:
+                self.verify(tokens, pos0)
+            finally:
+                self.D.nlayers = self.c["nlayers"]
+            a, b = self.routing(len(tokens))
+            lg.append(a)
+            ti.append(b)
+        return np.stack(lg), np.stack(ti)
 
     def draft(self, src, tokens, pos0):
         dev = self.dev

@@ -34,7 +34,15 @@ class MtpO(C.Structure):
                 ("layer", DecLayerO)]
 
 
-def _q8s(rng, oracle, rows, cols, scale):
+def _q8s_draw(rng, oracle, rows, cols, scale, cheap=False):
+    """a split-Q8_0 matrix (int8 values, f16 block scales) with entries of standard deviation `scale`: Gaussian weights
+    quantised by the oracle, or (cheap) uniformly random int8 values under block scales of scale / 74 with a random last
+    mantissa nibble (every (q, d) pair is a valid matrix; no float matrix is drawn)"""
+    if cheap:
+        q = rng.integers(0, 1 << 64, size=rows * cols // 8, dtype=np.uint64).view(np.int8).reshape(rows, cols)
+        d0 = np.array([scale / 74.0], dtype=np.float16).view(np.uint16)[0] & np.uint16(0xFFF0)
+        d = d0 | rng.integers(0, 16, (rows, cols // 32), dtype=np.uint16)
+        return q, d
     w = (rng.standard_normal((rows, cols)) * scale).astype(np.float32)
     q = np.zeros((rows, cols), dtype=np.int8)
     d = np.zeros((rows, cols // 32), dtype=np.uint16)
@@ -44,16 +52,20 @@ def _q8s(rng, oracle, rows, cols, scale):
 
 class TinyDecoder:
     def __init__(self, oracle, seed=1, n=256, nq=4, nkv=2, nlayers=2, vocab=1000, max_ctx=128, nexp=8, topk=2, ff=256, rope_scaled=False,
-                 cyclic=False):
-        """cyclic: a model whose pick depends on the row's token alone (the attention's output projections are zero) and
+                 cyclic=False, cheap_draws=False):
+        """cheap_draws: cheaper draws for full-size models (other values than the default draws): the dense matrices as random
+        int8 values, the embedding as f16 bit patterns, the IQ3_S blocks from the generator's 64-bit stream.
+        cyclic: a model whose pick depends on the row's token alone (the attention's output projections are zero) and
         whose draft layer is the model's single layer behind an identity projection of the embedding, so greedy decoding
         runs into a cycle, the draft layer mostly predicts the next token, prompt lookup fires and drafts are kept."""
         rng = np.random.default_rng(seed)
         self.oracle = oracle
+        _q8s = lambda rng, oracle, rows, cols, scale: _q8s_draw(rng, oracle, rows, cols, scale, cheap_draws)
         self.cfg = dict(n=n, nq=nq, nkv=nkv, nlayers=nlayers, vocab=vocab, max_ctx=max_ctx, nexp=nexp, topk=topk, ff=ff, eps=1e-6)
         self.rope = (1e7, 0, 0.0, 0.0, 1.0, 1.0) if not rope_scaled else (1e4, 1, 4.0, 20.0, 0.25, 1.0 + 0.1 * np.log(4.0))
         nb = lambda rows, cols: rows * cols // 256
         sw = 1.0 / np.sqrt(n)
+        iq3s = lambda nblocks: random_iq3s(rng, nblocks, dmax=4e-4, raw_bytes=cheap_draws)
 
         def layer():
             L = dict(attn_norm=(1 + 0.1 * rng.standard_normal(n)).astype(np.float32), q_norm=(1 + 0.1 * rng.standard_normal(HD)).astype(np.float32),
@@ -61,14 +73,17 @@ class TinyDecoder:
                      wq=_q8s(rng, oracle, nq * 2 * HD, n, sw), wk=_q8s(rng, oracle, nkv * HD, n, sw), wv=_q8s(rng, oracle, nkv * HD, n, sw),
                      wo=_q8s(rng, oracle, n, nq * HD, 1.0 / np.sqrt(nq * HD)),
                      router=(rng.standard_normal((nexp + 1, n)) * 0.05).astype(np.float32),
-                     gu=random_iq3s(rng, nexp * nb(2 * ff, n), dmax=4e-4), down=random_iq3s(rng, nexp * nb(n, ff), dmax=4e-4),
-                     sh_gu=random_iq3s(rng, nb(2 * ff, n), dmax=4e-4), sh_down=random_iq3s(rng, nb(n, ff), dmax=4e-4))
+                     gu=iq3s(nexp * nb(2 * ff, n)), down=iq3s(nexp * nb(n, ff)),
+                     sh_gu=iq3s(nb(2 * ff, n)), sh_down=iq3s(nb(n, ff)))
             return L
 
         self.layers = [layer() for _ in range(nlayers)]
         self.out_norm = (1 + 0.1 * rng.standard_normal(n)).astype(np.float32)
         self.head = _q8s(rng, oracle, vocab, n, sw)
-        self.emb = rng.standard_normal((vocab, n)).astype(np.float16)
+        if cheap_draws:   # f16 bit patterns drawn directly: a random sign, exponent field 12..15 (magnitudes 1/8 .. 2), random mantissa
+            self.emb = ((rng.integers(0, 1 << 16, (vocab, n), dtype=np.uint16) & np.uint16(0x8FFF)) | np.uint16(0x3000)).view(np.float16)
+        else:
+            self.emb = rng.standard_normal((vocab, n)).astype(np.float16)
         self.mtp = dict(norm_emb=(1 + 0.1 * rng.standard_normal(n)).astype(np.float32), norm_hid=(1 + 0.1 * rng.standard_normal(n)).astype(np.float32),
                         out_norm=(1 + 0.1 * rng.standard_normal(n)).astype(np.float32), fc_emb=_q8s(rng, oracle, n, n, sw),
                         fc_hid=_q8s(rng, oracle, n, n, sw), head=_q8s(rng, oracle, vocab, n, sw), layer=layer())
@@ -118,26 +133,40 @@ class TinyDecoder:
 class OracleSession:
     """verify / draft on the CPU oracle, with the caches kept between calls"""
 
-    def __init__(self, model):
-        self.m = model
+    def __init__(self, model, threads=8):
+        self.m, self.threads = model, threads
         self.D, self.M, self.caches, self.mtp_cache, self._keep = model.oracle_structs()
         lib = model.oracle.lib
         lib.fnx_o_decoder_verify.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]
         lib.fnx_o_decoder_verify.restype = None
         lib.fnx_o_mtp_draft.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]
         lib.fnx_o_mtp_draft.restype = None
+        lib.fnx_o_layer_probe.argtypes = [C.c_void_p, C.c_void_p, C.c_int]
+        lib.fnx_o_layer_probe.restype = None
 
-    def verify(self, tokens, pos0):
+    def _probe(self, T, layers):
+        c = self.m.cfg
+        lg, ti = np.zeros((layers, T, c["nexp"] + 1), dtype=np.float32), np.zeros((layers, T, c["topk"]), dtype=np.int32)
+        self.m.oracle.lib.fnx_o_layer_probe(ol.ptr(lg), ol.ptr(ti), layers)
+        return lg, ti
+
+    def verify(self, tokens, pos0, routing=False):
+        """routing: also every layer's router logits [layer][T][nexp + 1] and picks [layer][T][topk]"""
         c = self.m.cfg
         tok = np.ascontiguousarray(tokens, dtype=np.int32)
         T = len(tok)
         hidden = np.zeros((T, c["n"]), dtype=np.float32)
         logits = np.zeros((T, c["vocab"]), dtype=np.float32)
         best = np.zeros(T, dtype=np.int32)
-        self.m.oracle.lib.fnx_o_decoder_verify(C.byref(self.D), ol.ptr(tok), T, pos0, ol.ptr(hidden), ol.ptr(logits), ol.ptr(best), 8)
-        return dict(hidden=hidden, logits=logits, best=best)
+        probe = self._probe(T, c["nlayers"]) if routing else None
+        self.m.oracle.lib.fnx_o_decoder_verify(C.byref(self.D), ol.ptr(tok), T, pos0, ol.ptr(hidden), ol.ptr(logits), ol.ptr(best), self.threads)
+        self.m.oracle.lib.fnx_o_layer_probe(None, None, 0)
+        r = dict(hidden=hidden, logits=logits, best=best)
+        if routing:
+            r["route_logits"], r["route_topi"] = probe
+        return r
 
-    def draft(self, src, tokens, pos0):
+    def draft(self, src, tokens, pos0, routing=False):
         c = self.m.cfg
         tok = np.ascontiguousarray(tokens, dtype=np.int32)
         src = np.ascontiguousarray(src, dtype=np.float32)
@@ -145,9 +174,14 @@ class OracleSession:
         hidden = np.zeros((T, c["n"]), dtype=np.float32)
         logits = np.zeros((T, c["vocab"]), dtype=np.float32)
         best = np.zeros(T, dtype=np.int32)
+        probe = self._probe(T, 1) if routing else None
         self.m.oracle.lib.fnx_o_mtp_draft(C.byref(self.D), C.byref(self.M), ol.ptr(src), ol.ptr(tok), T, pos0, ol.ptr(hidden), ol.ptr(logits),
-                                          ol.ptr(best), 8)
-        return dict(hidden=hidden, logits=logits, best=best)
+                                          ol.ptr(best), self.threads)
+        self.m.oracle.lib.fnx_o_layer_probe(None, None, 0)
+        r = dict(hidden=hidden, logits=logits, best=best)
+        if routing:
+            r["route_logits"], r["route_topi"] = probe
+        return r
 
 
 def spec_generate(sess, lookup, accept, prompt, max_new, K=4, lk=15, speculate=True, forced=None):
