@@ -23,14 +23,101 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 N, FF, NEXP, TOPK, T = 2048, 512, 512, 10, 16
 HBM_PEAK = 8.0e12
-# HBM bytes of one gate|up launch from the FETCH_SIZE / WRITE_SIZE counter runs (profiles/moe_gate_up_hbm_traffic.md),
-# as a ratio to the launch's algorithmic bytes at the profiled routing (139.75 distinct experts): 136.5 MB / 127.6 MB
-GATE_UP_TRAFFIC_RATIO = 1.070
+# HBM bytes of one gate|up launch of the default run (gaussian weights, 16 sets, unit64), measured by two rocprofv3 --pmc
+# runs of this file (FETCH_SIZE, then WRITE_SIZE, each scaled by a 256 MiB copy: profiles/moe_gate_up_hbm_traffic.md), and
+# the distinct experts per step they were measured at. Not measured in the run: emitted only for that configuration.
+GATE_UP_TRAFFIC = {"bytes": None, "distinct_experts_per_step": None, "source": "profiles/moe_gate_up_hbm_traffic.md"}
 IQ3S_BLOCK = 110
 GU_BYTES = 2 * FF * (N // 256) * IQ3S_BLOCK      # 901,120 per expert
 DN_BYTES = N * (FF // 256) * IQ3S_BLOCK          # 450,560 per expert
 ROUTER_BYTES = (NEXP + 1) * N * 4                # 4,202,496
 XIO_BYTES = 2 * T * N * 4                        # x in + out
+
+
+def stream_calibration(dev, torch, np):
+    """What this GPU gives a kernel that only reads (fnx_stream_read: the library's calibration kernels, no decode): plain
+    and nontemporal 16-byte loads and the unit64 plane loads of the expert kernels over 1 GiB (the asymptote), and the
+    plane loads over one launch of the size of the window's gate|up and down launches (launch ramp included). Events on
+    the launch stream; every launch reads a region no launch of the last seven read."""
+    lib, st = dev.lib, dev.st()
+    UNIT = 880
+    buf = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").random_()
+    sink = torch.zeros(4, dtype=torch.int32, device="cuda")
+
+    def rate(variant, blocks, threads, nbytes):
+        regions = max(1, min(8, (1 << 30) // nbytes))
+        evs = []
+        for i in range(13):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            dev.ok(lib.fnx_stream_read(buf.data_ptr() + (i % regions) * nbytes, nbytes, variant, blocks, threads, sink.data_ptr(), st))
+            e1.record()
+            evs.append((e0, e1))
+        torch.cuda.synchronize()
+        return nbytes / (float(np.mean([a.elapsed_time(b) for a, b in evs[3:]])) * 1e-3) / 1e9
+
+    whole = (1 << 30) // (16 * UNIT) * (16 * UNIT)
+    gate_up, down = 152064 * UNIT, 75776 * UNIT   # about 148.5 matrices of 901,120 and of 450,560 bytes
+    return {"plain_16B_loads_1GiB": rate(1, 512, 512, whole), "nontemporal_16B_loads_1GiB": rate(5, 512, 512, whole),
+            "unit64_plane_loads_1GiB": rate(6, 512, 512, whole),
+            "unit64_plane_loads_one_launch_134MB": rate(9, 256, 1024, gate_up), "unit64_plane_loads_one_launch_67MB": rate(9, 256, 1024, down)}
+
+
+def gemv_measure(dev, torch, np, steps):
+    """benchmark config 1: a 4096 x 2048 IQ3_S matrix (3,604,480 bytes) over T = 1 and T = 16 q8_1 rows: (a) one matrix a
+    launch, cycling through 1,024 distinct matrices (3.7 GB) so that every launch reads its weights from HBM: a launch of
+    3.6 MB is bound by the launch, not by HBM; (b) one fnx_mmvq launch of 1,024 jobs over the 1,024 matrices through the
+    table of matrix pointers: the kernel's streaming rate."""
+    import fnx_gpu
+    pkg, lib, st = dev.pkg, dev.lib, dev.st()
+    g = torch.Generator(device="cuda")
+    g.manual_seed(11)
+    ROWS, COLS, NM = 4096, 2048, 1024
+    mbytes = ROWS * COLS // 256 * IQ3S_BLOCK
+    w = _rand_iq3s(torch, g, NM * ROWS * COLS // 256)
+    dev.ok(lib.fnx_iq3s_repack(w.data_ptr(), w.data_ptr(), w.numel() // IQ3S_BLOCK * 256, st))
+    ep = torch.tensor([w.data_ptr() + i * mbytes for i in torch.randperm(NM).tolist()], dtype=torch.int64, device="cuda")
+    lone, many = {}, {}
+    for T in (1, 16):
+        x = torch.randn((T, COLS), device="cuda", generator=g)
+        xq = torch.zeros(T * (COLS // 32) * 36, dtype=torch.uint8, device="cuda")
+        dev.ok(lib.fnx_quantize_q8_1(x.data_ptr(), xq.data_ptr(), COLS, T, st))
+        jobs = np.zeros(NM, dtype=fnx_gpu.JOB_DTYPE)
+        jobs["w"] = np.arange(NM)
+        jobs["n"] = T
+        jobs["y"][:, :T] = np.arange(T)[None, :]
+        jobs["out"][:, :T] = np.arange(NM)[:, None] * T + np.arange(T)[None, :]
+        dj = dev.up(jobs.view(np.uint8).reshape(-1))
+        out = torch.zeros((NM * T, ROWS), device="cuda")
+        Ws = [pkg.dw(w.data_ptr() + i * mbytes, COLS, ROWS, packed=True) for i in range(NM)]
+        n1 = max(steps, 512)
+        for i in range(64):
+            dev.ok(lib.fnx_mmvq(C.byref(Ws[i % NM]), 0, dj.data_ptr(), None, 1, xq.data_ptr(), out.data_ptr(), ROWS, st))
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for i in range(n1):
+            dev.ok(lib.fnx_mmvq(C.byref(Ws[(64 + i) % NM]), 0, dj.data_ptr(), None, 1, xq.data_ptr(), out.data_ptr(), ROWS, st))
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) / n1 * 1e3
+        nbytes = mbytes + T * (COLS // 32) * 36 + T * ROWS * 4
+        lone[f"T{T}"] = {"us_per_launch": us, "algorithmic_bytes": nbytes, "GBps": nbytes / (us * 1e-6) / 1e9, "hbm_frac": nbytes / (us * 1e-6) / HBM_PEAK}
+        Wall = pkg.dw(w.data_ptr(), COLS, ROWS, ep=ep.data_ptr(), packed=True)
+        evs = []
+        for i in range(8):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            dev.ok(lib.fnx_mmvq(C.byref(Wall), 0, dj.data_ptr(), None, NM, xq.data_ptr(), out.data_ptr(), ROWS, st))
+            b.record()
+            evs.append((a, b))
+        torch.cuda.synchronize()
+        us = float(np.mean([a.elapsed_time(b) for a, b in evs[2:]])) * 1e3
+        nbytes = NM * (mbytes + T * ROWS * 4) + T * (COLS // 32) * 36
+        many[f"T{T}"] = {"us_per_launch": us, "algorithmic_bytes": nbytes, "GBps": nbytes / (us * 1e-6) / 1e9, "hbm_frac": nbytes / (us * 1e-6) / HBM_PEAK}
+    del w, out
+    torch.cuda.empty_cache()
+    return {"lone_matrix_a_launch": lone, "launch_of_1024_matrices": many}
 
 
 def main():
@@ -42,6 +129,9 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0: skip)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain device copy of 256 MiB, the known-size kernel that scales the FETCH_SIZE / WRITE_SIZE counters")
+    ap.add_argument("--weights", choices=["gaussian", "bytes"], default="gaussian",
+                    help="gaussian: experts IQ3_S-encoded from N(0, 0.02) weights (benchmark config 2's recipe); bytes: uniformly random blocks")
+    ap.add_argument("--no-extras", action="store_true", help="skip the legs beside the headline (streaming calibration, config 1, the other weight kind)")
     ap.add_argument("--raw-layout", action="store_true", help="leave the weights as raw ggml blocks (skip the load-time re-laying)")
     ap.add_argument("--workload", choices=["verify", "prefill", "decoder", "head", "gemv"], default="verify",
                     help="verify: benchmark config 2 (the headline metric, the default); prefill: config 5, one MoE layer over prompt chunks of 512 "
@@ -75,18 +165,36 @@ def main():
         b[:, 0:2] = d.view(torch.uint8).reshape(nblocks, 2)
         return b.reshape(-1)
 
-    layers = []
-    for _ in range(args.layers):
-        router = (torch.randn((NEXP + 1, N), device="cuda", generator=g) * 0.02).contiguous()
-        gu = rand_iq3s(NEXP * 2 * FF * N // 256)
-        down = rand_iq3s(NEXP * N * FF // 256)
-        sh_gu = rand_iq3s(2 * FF * N // 256)
-        sh_down = rand_iq3s(N * FF // 256)
-        # the CPU leg reads raw ggml blocks: keep weight set 0's before the load-time re-laying (fnx_iq3s_repack, in place)
-        raw = [a.cpu().numpy() for a in (gu, down, sh_gu, sh_down)] if not layers and args.cpu_seconds > 0 else None
-        (gu, down, sh_gu, sh_down), dws = fnx_gpu.pack_moe_weights(dev, [gu, down, sh_gu, sh_down], N, FF, not args.raw_layout)
-        L = pkg.MoeLayer(N, FF, NEXP, TOPK, router.data_ptr(), 0, dws[0], GU_BYTES, dws[1], DN_BYTES, dws[2], dws[3])
-        layers.append((L, router, gu, down, sh_gu, sh_down, raw))
+    # the experts of benchmark config 2: IQ3_S blocks encoded from N(0, 0.02) weights. BANK distinct matrices of each kind
+    # are encoded (this build's encoder, on the GPU) and every expert of every weight set is a copy of one of them at an
+    # address of its own, so the bytes a step reads are as cold and as many as with 512 different experts
+    BANK = 32
+    bank = None
+    if args.weights == "gaussian":
+        import importlib
+        enc = importlib.import_module("fnx_mi355x_pkg.iq3s_encode")
+        bank = (enc.encode_iq3s(torch.randn((BANK, 2 * FF * N), device="cuda", generator=g) * 0.02).view(BANK, GU_BYTES),
+                enc.encode_iq3s(torch.randn((BANK, N * FF), device="cuda", generator=g) * 0.02).view(BANK, DN_BYTES))
+
+    def weight_set(kind, i):
+        if kind == "bytes":
+            return [rand_iq3s(NEXP * 2 * FF * N // 256), rand_iq3s(NEXP * N * FF // 256), rand_iq3s(2 * FF * N // 256), rand_iq3s(N * FF // 256)]
+        pick = torch.randint(0, BANK, (NEXP,), device="cuda", generator=g)
+        return [bank[0][pick].reshape(-1), bank[1][pick].reshape(-1), bank[0][i % BANK].clone(), bank[1][i % BANK].clone()]
+
+    def make_sets(kind, count, keep_raw):
+        sets = []
+        for i in range(count):
+            router = (torch.randn((NEXP + 1, N), device="cuda", generator=g) * 0.02).contiguous()
+            gu, down, sh_gu, sh_down = weight_set(kind, i)
+            # the CPU leg reads raw ggml blocks: keep weight set 0's before the load-time re-laying (fnx_iq3s_repack, in place)
+            raw = [a.cpu().numpy() for a in (gu, down, sh_gu, sh_down)] if not sets and keep_raw else None
+            (gu, down, sh_gu, sh_down), dws = fnx_gpu.pack_moe_weights(dev, [gu, down, sh_gu, sh_down], N, FF, not args.raw_layout)
+            L = pkg.MoeLayer(N, FF, NEXP, TOPK, router.data_ptr(), 0, dws[0], GU_BYTES, dws[1], DN_BYTES, dws[2], dws[3])
+            sets.append((L, router, gu, down, sh_gu, sh_down, raw))
+        return sets
+
+    layers = make_sets(args.weights, args.layers, args.cpu_seconds > 0)
     NX = 64
     xs = torch.randn((NX, T, N), device="cuda", generator=g)
     outs = torch.zeros((NX, T, N), device="cuda")
@@ -97,10 +205,20 @@ def main():
     ws = pkg.MoeWs(*(ws_t[k].data_ptr() for k in ("xq", "logits", "topi", "topw", "jobs_gu", "jobs_dn", "njobs", "gu", "part")))
     st = dev.st()
 
-    def step(i):
-        L = layers[i % args.layers][0]
+    def step(i, sets=None):
+        L = (sets or layers)[i % args.layers][0]
         x = xs[i % NX]
         dev.ok(lib.fnx_moe_verify_layer(C.byref(L), x.data_ptr(), T, outs[i % NX].data_ptr(), C.byref(ws), st))
+
+    def timed_steps(sets=None):
+        for i in range(args.warmup):
+            step(i, sets)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            step(args.warmup + i, sets)
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0
 
     if args.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").random_()
@@ -110,14 +228,7 @@ def main():
         torch.cuda.synchronize()
 
     # ---- whole steps
-    for i in range(args.warmup):
-        step(i)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        step(args.warmup + i)
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
+    dt = timed_steps()
     ms_per_step = dt / args.steps * 1e3
 
     # ---- distinct experts per step (for the algorithmic bytes), from the routing the steps produced
@@ -130,7 +241,7 @@ def main():
     step_bytes = u_mean * (GU_BYTES + DN_BYTES) + (GU_BYTES + DN_BYTES) + ROUTER_BYTES + XIO_BYTES
 
     # ---- the dominant kernel: the window's gate|up launch (routed experts + the shared expert), timed with events the
-    # library records on the launch stream around each of the window's five launches (fnx_layer_profile)
+    # library records on the launch stream around each of the window's three launches (fnx_layer_profile)
     names = ["router+q8_1", "top-k+plan+gate|up+swiglu", "down+combine"]
     per_launch = np.zeros(3)
     reps = max(50, min(args.steps, 200))
@@ -167,6 +278,22 @@ def main():
         k_bytes = u_mean * GU_BYTES + T * (N // 32) * 36 + P * 2 * FF * 4
     achieved = k_bytes / (k_ms * 1e-3)
 
+    # ---- beside the headline: what a read-only kernel reaches on this GPU, config 1, and the same steps over uniformly
+    # random blocks (the codebook lookups' bank conflicts depend on the codes)
+    stream = gemv = other_ms = None
+    if not args.no_extras and fused:
+        stream = stream_calibration(dev, torch, np)
+        other = "bytes" if args.weights == "gaussian" else "gaussian"
+        if other == "bytes" or bank is not None:
+            alt = make_sets(other, args.layers, False)
+            other_ms = timed_steps(alt) / args.steps * 1e3
+            del alt
+            torch.cuda.empty_cache()
+        gemv = gemv_measure(dev, torch, np, 512)
+    traffic = None
+    if fused and args.weights == "gaussian" and GATE_UP_TRAFFIC["bytes"] and abs(u_mean - GATE_UP_TRAFFIC["distinct_experts_per_step"]) < 0.5:
+        traffic = GATE_UP_TRAFFIC["bytes"]
+
     # ---- CPU baseline: the oracle on the host's cores, same workload (layer set 0), bounded sample
     cpu = None
     if args.cpu_seconds > 0:
@@ -198,13 +325,22 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "int8 x IQ3_S (i32 dot, f32 accumulate)", "data": "synthetic",
+        "dtype": "int8 x IQ3_S (i32 dot, f32 accumulate)",
+        "data": ("synthetic: experts IQ3_S-encoded from N(0, 0.02) weights by this build's encoder (32 distinct matrices of each kind, copied to "
+                 "512 experts x the weight sets at addresses of their own)" if args.weights == "gaussian" else
+                 "synthetic: uniformly random IQ3_S blocks") + ", f32 router N(0, 0.02), activations N(0, 1)",
         "config": {"workload": "config 2: one MoE verify layer, T=16, hidden 2048, 512 IQ3_S experts top-10, SwiGLU ff 512, shared expert, f32 router",
+                   "weights": args.weights,
                    "weight_layout": "raw ggml blocks" if args.raw_layout else "unit64 (re-laid once at load, same bytes)", "weight_sets": args.layers, "distinct_experts_per_step": u_mean, "step_algorithmic_bytes": step_bytes,
-                   "step_hbm_frac": step_bytes / (ms_per_step * 1e-3) / HBM_PEAK},
+                   "step_hbm_frac": step_bytes / (ms_per_step * 1e-3) / HBM_PEAK,
+                   "ms_per_step_other_weights": None if other_ms is None else {("bytes" if args.weights == "gaussian" else "gaussian"): other_ms},
+                   "gemv": gemv},
         "roofline": {"bound": "hbm", "kernel": kernel_name, "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK, "traffic": k_bytes * GATE_UP_TRAFFIC_RATIO if fused else None, "kernel_ms": k_ms, "algorithmic_bytes": k_bytes,
-                     "window_launch_us": {n_: round(float(v) * 1e3, 2) for n_, v in zip(names, per_launch)}},
+                     "frac": achieved / HBM_PEAK, "traffic": traffic, "traffic_source": GATE_UP_TRAFFIC["source"] if traffic else None,
+                     "kernel_ms": k_ms, "algorithmic_bytes": k_bytes,
+                     "window_launch_us": {n_: round(float(v) * 1e3, 2) for n_, v in zip(names, per_launch)},
+                     "stream_read_GBps": stream,
+                     "frac_of_stream_read": None if not stream else achieved / 1e9 / stream["unit64_plane_loads_one_launch_134MB"]},
         "cpu_baseline": cpu,
     }
     print(json.dumps(line))
@@ -218,51 +354,21 @@ def _rand_iq3s(torch, g, nblocks):
 
 
 def gemv_main(args):
-    """benchmark config 1: one 4096 x 2048 IQ3_S matrix (3,604,480 bytes) over T = 1 and T = 16 q8_1 rows, cycling through
-    1,024 distinct matrices (3.7 GB) so that every launch reads its weights from HBM."""
+    """benchmark config 1 on its own (gemv_measure)"""
     import numpy as np
     import torch
     import fnx_gpu
     dev = fnx_gpu.Dev()
-    pkg, lib = dev.pkg, dev.lib
-    g = torch.Generator(device="cuda")
-    g.manual_seed(11)
-    ROWS, COLS, NM = 4096, 2048, 1024
-    mbytes = ROWS * COLS // 256 * IQ3S_BLOCK
-    w = _rand_iq3s(torch, g, NM * ROWS * COLS // 256)
-    dev.ok(lib.fnx_iq3s_repack(w.data_ptr(), w.data_ptr(), w.numel() // IQ3S_BLOCK * 256, dev.st()))
-    st = dev.st()
-    res = {}
-    for T in (1, 16):
-        x = torch.randn((T, COLS), device="cuda", generator=g)
-        xq = torch.zeros(T * (COLS // 32) * 36, dtype=torch.uint8, device="cuda")
-        dev.ok(lib.fnx_quantize_q8_1(x.data_ptr(), xq.data_ptr(), COLS, T, st))
-        jobs = np.zeros(1, dtype=fnx_gpu.JOB_DTYPE)
-        jobs["n"][0] = T
-        jobs["y"][0, :T] = np.arange(T)
-        jobs["out"][0, :T] = np.arange(T)
-        dj = dev.up(jobs.view(np.uint8).reshape(-1))
-        out = torch.zeros((T, ROWS), device="cuda")
-        Ws = [pkg.dw(w.data_ptr() + i * mbytes, COLS, ROWS, packed=True) for i in range(NM)]
-        steps = max(args.steps, 512)
-        for i in range(64):
-            dev.ok(lib.fnx_mmvq(C.byref(Ws[i % NM]), 0, dj.data_ptr(), None, 1, xq.data_ptr(), out.data_ptr(), ROWS, st))
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        torch.cuda.synchronize()
-        e0.record()
-        for i in range(steps):
-            dev.ok(lib.fnx_mmvq(C.byref(Ws[(64 + i) % NM]), 0, dj.data_ptr(), None, 1, xq.data_ptr(), out.data_ptr(), ROWS, st))
-        e1.record()
-        torch.cuda.synchronize()
-        us = e0.elapsed_time(e1) / steps * 1e3
-        nbytes = mbytes + T * (COLS // 32) * 36 + T * ROWS * 4
-        res[T] = {"us_per_launch": us, "algorithmic_bytes": nbytes, "GBps": nbytes / (us * 1e-6) / 1e9, "hbm_frac": nbytes / (us * 1e-6) / HBM_PEAK}
-    line = {"metric": "IQ3_S GEMV achieved HBM GB/s (config 1: 4096 x 2048, T = 1 and 16)", "value": res[16]["GBps"], "unit": "GB/s", "n_gpus": 1,
-            "steps": max(args.steps, 512), "warmup": 64, "ms_per_step": res[16]["us_per_launch"] / 1e3, "higher_is_better": True, "scaling": "weak",
-            "vs_baseline": None, "dtype": "int8 x IQ3_S (i32 dot, f32 accumulate)", "data": "synthetic",
-            "config": {"workload": "config 1: one IQ3_S 4096 x 2048 mat-vec, 1,024 distinct matrices cycled", "T1": res[1], "T16": res[16]},
-            "roofline": {"bound": "hbm", "kernel": "k_iq3s_jobs (unit64, one job)", "achieved": res[16]["GBps"], "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                         "frac": res[16]["hbm_frac"], "traffic": None, "note": "back-to-back launches of 3.6 MB each: dominated by the launch, not by HBM"},
+    res = gemv_measure(dev, torch, np, args.steps)
+    many, lone = res["launch_of_1024_matrices"], res["lone_matrix_a_launch"]
+    line = {"metric": "IQ3_S GEMV achieved HBM GB/s (config 1: 4096 x 2048, T = 1 and 16)", "value": many["T16"]["GBps"], "unit": "GB/s", "n_gpus": 1,
+            "steps": max(args.steps, 512), "warmup": 64, "ms_per_step": many["T16"]["us_per_launch"] / 1e3, "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "int8 x IQ3_S (i32 dot, f32 accumulate)", "data": "synthetic: uniformly random IQ3_S blocks",
+            "config": {"workload": "config 1: IQ3_S 4096 x 2048 mat-vec over 1,024 distinct matrices, one launch for all (the value) and one launch each",
+                       "gemv": res},
+            "roofline": {"bound": "hbm", "kernel": "k_iq3s_jobs (unit64, 1,024 jobs of 16 rows)", "achieved": many["T16"]["GBps"], "peak": HBM_PEAK / 1e9,
+                         "unit": "GB/s", "frac": many["T16"]["hbm_frac"], "traffic": None,
+                         "note": "one matrix a launch (3.6 MB) is bound by the launch: " + f"{lone['T16']['us_per_launch']:.1f} us at T = 16"},
             "cpu_baseline": None}
     print(json.dumps(line))
 

@@ -240,3 +240,26 @@ def test_encoder_reconstruction(oracle):
     again = oracle.iq3s_dequant(oracle.iq3s_quantize(back))
     assert np.linalg.norm(again - back) <= 0.05 * np.linalg.norm(back)
     assert np.all(oracle.iq3s_dequant(oracle.iq3s_quantize(np.zeros(256, dtype=np.float32))) == 0)
+
+
+def test_torch_encoder_matches_the_oracles(oracle):
+    """the package's torch IQ3_S encoder (synthetic benchmark weights) against the oracle's C encoder: the same algorithm,
+    so nearly every byte agrees (distances are summed in another order: rare ties fall the other way), the decoded error
+    is the same, and the decoded weights are close to the source as 3.4 bits a weight allow"""
+    import importlib
+    import torch
+    import fnx_gpu
+    fnx_gpu.package()
+    enc = importlib.import_module("fnx_mi355x_pkg.iq3s_encode")
+    rng = np.random.default_rng(77)
+    w = (rng.standard_normal(64 * 256) * 0.02).astype(np.float32)
+    w[256:512] = 0   # an all-zero block
+    w[700] = 0.3     # an outlier
+    mine = enc.encode_iq3s(torch.from_numpy(w)).numpy()
+    theirs = oracle.iq3s_quantize(w)
+    assert mine.shape == theirs.shape
+    assert np.count_nonzero(mine != theirs) <= 0.01 * mine.size
+    dm, dt = oracle.iq3s_dequant(mine), oracle.iq3s_dequant(theirs)
+    em, et = float(np.linalg.norm(dm - w)), float(np.linalg.norm(dt - w))
+    assert em <= 1.01 * et and et / float(np.linalg.norm(w)) < 0.2
+    assert not dm[256:512].any()
