@@ -32,6 +32,9 @@ extern "C" {
 #define FNX_IQ3S_BLOCK 110 /* bytes per 256 weights */
 #define FNX_Q8_1_BLOCK 36  /* bytes per 32 activations: half d, half sum, int8 qs[32] */
 #define FNX_ERR_NONFINITE 16u /* error-word bit (engine_impl.hpp:211-218) */
+#define FNX_ERR_WINDOW 32u    /* error-word bit: a window at a position outside its cache (below 0, or its last row past max_ctx);
+                              * the attention then reads only cells that exist and the results mean nothing. No counterpart in the
+                              * reference, whose positions are host integers that it checks before launching */
 
 /* kernels.hpp:18-23 */
 typedef struct fnx_job {

@@ -1,0 +1,44 @@
+// The attention kernels' view of a window whose position lives in a device word: which cache positions a block may read.
+// The host cannot check a position it does not know, so the kernels bound every index by the cache's capacity here; a
+// window that does not fit is reported through an error bit and computed over the cells that exist. Plain functions of
+// integers, compiled for the device and (by the bounds test) for the host.
+#pragma once
+
+#if defined(__HIPCC__)
+#define FNX_HOST_DEVICE __host__ __device__
+#else
+#define FNX_HOST_DEVICE
+#endif
+
+namespace fnx {
+
+constexpr int AT_SPLIT = 512;   // positions a block of the first pass covers
+constexpr int AT_CH = 32;       // positions a chunk (one trip of a block's loop)
+
+FNX_HOST_DEVICE inline int att_min(int a, int b) { return a < b ? a : b; }
+FNX_HOST_DEVICE inline int att_max(int a, int b) { return a > b ? a : b; }
+FNX_HOST_DEVICE inline int attn_splits(int max_ctx) { return (max_ctx + AT_SPLIT - 1) / AT_SPLIT; }
+
+struct AttWindow {
+    int pos0;      // the first row's position, not below 0 and not past the cache's last cell
+    int ctx_max;   // the last row sees positions [0, ctx_max): 1 .. max_ctx
+};
+// T rows at positions pos0_raw .. pos0_raw + T - 1 of a cache of max_ctx >= 1 cells
+FNX_HOST_DEVICE inline AttWindow att_window(int pos0_raw, int T, int max_ctx) {
+    const int pos0 = att_min(att_max(pos0_raw, 0), max_ctx - 1);
+    return AttWindow{pos0, att_min(pos0 + att_max(T, 1), max_ctx)};
+}
+FNX_HOST_DEVICE inline bool att_window_fits(int pos0_raw, int T, int max_ctx) { return pos0_raw >= 0 && T >= 1 && pos0_raw <= max_ctx - T; }
+// row qt of the window sees positions [0, this)
+FNX_HOST_DEVICE inline int att_ctx_q(const AttWindow& w, int qt) { return att_min(w.pos0 + qt + 1, w.ctx_max); }
+// split s covers positions [p0, p1); empty when p0 >= p1
+FNX_HOST_DEVICE inline int att_split_begin(int s) { return s * AT_SPLIT; }
+FNX_HOST_DEVICE inline int att_split_end(const AttWindow& w, int s) { return att_min(w.ctx_max, s * AT_SPLIT + AT_SPLIT); }
+// the K row and the V block (of four positions) that a fetch of chunk c0 reads for its row r (0 .. AT_CH - 1) and block b
+// (0 .. AT_CH / 4 - 1): clamped inside the window's rows
+FNX_HOST_DEVICE inline int att_fetch_row(const AttWindow& w, int c0, int r) { return att_min(c0 + r, w.ctx_max - 1); }
+FNX_HOST_DEVICE inline int att_fetch_vblock(const AttWindow& w, int c0, int b) { return att_min((c0 >> 2) + b, (w.ctx_max - 1) >> 2); }
+// the splits whose parts the first pass wrote with data (the second pass reads these)
+FNX_HOST_DEVICE inline int att_live_splits(const AttWindow& w, int nsplit) { return att_min(nsplit, (w.ctx_max + AT_SPLIT - 1) / AT_SPLIT); }
+
+}  // namespace fnx

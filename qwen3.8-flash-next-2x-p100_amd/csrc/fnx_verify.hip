@@ -1334,13 +1334,12 @@ int fnx_attn_prep_append(float* qg, float* k, const float* v, const float* q_nor
     return attn_prep_append(qg, k, v, q_norm, k_norm, kc, vc, nq, nkv, T, pos0, max_ctx, eps, rope, st, nullptr);
 }
 // splits for a context of up to max_ctx positions
-static int attn_splits(int max_ctx) { return (max_ctx + AT_SPLIT - 1) / AT_SPLIT; }
 size_t fnx_attn_scratch_floats(int nq, int T, int max_ctx) { return (size_t) T * nq * attn_splits(max_ctx) * (AT_HD + 2); }
 static int q8s_one(const fnx_q8s* W, const void* yq, float* out, int out_stride, int T, void* st, const int* gate) {
     return q8s_launch(&W, &out, &out_stride, 1, yq, T, st, "q8s_gemv", gate);
 }
 static int attn_launch(const float* qg, const uint16_t* kc, const uint16_t* vc, float* out, uint8_t* outq, int nq, int nkv, const int* pos0, int T,
-                       int max_ctx, float* scratch, void* st, const int* gate = nullptr, const int* live = nullptr) {
+                       int max_ctx, float* scratch, void* st, const int* gate = nullptr, const int* live = nullptr, unsigned* err = nullptr) {
     if (!qg || !kc || !vc || (!out && !outq) || !pos0 || !scratch) return fail("attn: null argument");
     if (nq < 1 || nkv < 1 || nq % nkv || nq / nkv > AT_MAXQ || T < 1 || T > FNX_MAXT || max_ctx < 1) return fail("attn: bad shape");
     if (attn_splits(max_ctx) > AT_MAXSPLIT) return fail("attn: the cache is larger than the split table");
@@ -1349,8 +1348,8 @@ static int attn_launch(const float* qg, const uint16_t* kc, const uint16_t* vc, 
     float* acc = scratch;
     AttPart* mz = reinterpret_cast<AttPart*>(scratch + (size_t) T * nq * nsplit * AT_HD);
     k_attn_part<<<dim3(nsplit, nkv, (waves + AT_WAVES - 1) / AT_WAVES), 64 * AT_WAVES, 0, (hipStream_t) st>>>(qg, kc, vc, acc, mz, nq, nkv, T,
-                                                                                                          nsplit, pos0, gate, live);
-    k_attn_combine<<<dim3(nq, T), AT_HD, 0, (hipStream_t) st>>>(qg, acc, mz, out, outq, nq, nsplit, T, pos0, gate, live);
+                                                                                                          nsplit, pos0, max_ctx, gate, live);
+    k_attn_combine<<<dim3(nq, T), AT_HD, 0, (hipStream_t) st>>>(qg, acc, mz, out, outq, nq, nsplit, T, pos0, max_ctx, err, gate, live);
     return launch_status("attn");
 }
 int fnx_attn(const float* qg, const uint16_t* kc, const uint16_t* vc, float* out, int nq, int nkv, const int* pos0, int T, int max_ctx,
@@ -1403,7 +1402,8 @@ static int dec_layer(const fnx_decoder* D, const fnx_dec_layer* L, int T, const 
     }
     if (attn_prep_append(ws->qg, ws->k, ws->v, L->q_norm, L->k_norm, L->kc, L->vc, nq, nkv, T, pos0, D->max_ctx, D->eps, &D->rope, st, gate)) return 1;
     // the attention's rows leave its last kernel in q8_1 form, ready for the output projection
-    if (attn_launch(ws->qg, L->kc, L->vc, nullptr, (uint8_t*) ws->xq, nq, nkv, pos0, T, D->max_ctx, ws->attn_scratch, st, gate, live)) return 1;
+    if (attn_launch(ws->qg, L->kc, L->vc, nullptr, (uint8_t*) ws->xq, nq, nkv, pos0, T, D->max_ctx, ws->attn_scratch, st, gate, live, (unsigned*) ws->err))
+        return 1;
     if (q8s_one(&L->wo, ws->xq, ws->o, n, T, st, gate)) return 1;
     {   // x += o; xn = norm(x) (fnx_add_norm_q8)
         CombineArgs c{};
@@ -1483,6 +1483,7 @@ int fnx_decode_round(const fnx_decoder* D, const fnx_mtp* M, const fnx_round* R,
     if (K > 1 && !R->chain_src) return fail("decode_round: the chain needs its source row's buffer");
     hipStream_t s = (hipStream_t) st;
     int* S = R->state;
+    k_round_guard<<<1, 1, 0, s>>>(S, R->ctx_cap, D->max_ctx);
     if (decoder_verify(D, R->rows, FNX_MAXT, S + FNX_RS_POS, ws, st, S + FNX_RS_ROWS)) return 1;
     k_round_commit<<<1, 64, 0, s>>>(R->rows, ws->best_i, S, R->ctx, R->ctx_cap, D->max_ctx, R->log_cap ? R->log : nullptr, R->log_cap);
     if (R->speculate) {

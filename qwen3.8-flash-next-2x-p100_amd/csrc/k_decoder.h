@@ -2,6 +2,8 @@
 // projections and the output head, the attention's prepare/append and split-K decode kernels, embedding rows.
 #pragma once
 
+#include "attn_window.h"
+
 #include "fnx_device.h"
 
 namespace fnx {
@@ -405,7 +407,7 @@ __global__ void __launch_bounds__(AT_HD) k_attn_prep_append(float* __restrict__ 
 //                  registers straight into the B operand, and V^T's A operand is two 8-byte loads because the V cache
 //                  keeps four positions of a dimension together ([position / 4][kv head][dim][position % 4]).
 // The probabilities never pass through LDS; K and V chunks do, once per block (a chunk ahead, double-buffered). Each (query, split) leaves its maximum, sum and 256 accumulators; k_attn_combine merges.
-constexpr int AT_SPLIT = 512, AT_CH = 32, AT_MAXQ = 8;
+constexpr int AT_MAXQ = 8;   // AT_SPLIT, AT_CH: attn_window.h
 struct AttPart {
     float m, z;
 };
@@ -441,7 +443,7 @@ constexpr int AT_WAVES = 4, AT_KLD = 2 * AT_HD + 16;   // q tiles (of 16 queries
 __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) k_attn_part(const float* __restrict__ qg, const uint16_t* __restrict__ kc,
                                                             const uint16_t* __restrict__ vc, float* __restrict__ acc_out,
                                                             AttPart* __restrict__ mz_out, int nq, int nkv, int T, int nsplit,
-                                                            const int* __restrict__ pos0p, const int* __restrict__ gate,
+                                                            const int* __restrict__ pos0p, int max_ctx, const int* __restrict__ gate,
                                                             const int* __restrict__ live) {
     typedef __attribute__((address_space(1))) const at_v4u g128;
     if (gate && uniform(*gate) == 0) return;   // a chain step that does not count: its parts stay what they were, nothing reads the result
@@ -449,16 +451,17 @@ __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per
     // their results), the positions past the last row that counts with them
     if (live) T = uniform(max(1, min(*live, T)));
     const int s = blockIdx.x, kvh = blockIdx.y, lane = threadIdx.x & 63, wave = blockIdx.z * AT_WAVES + (threadIdx.x >> 6);
-    const int qpk = nq / nkv, nquery = T * qpk, pos0 = *pos0p;
+    const int qpk = nq / nkv, nquery = T * qpk;
+    const AttWindow win = att_window(*pos0p, T, max_ctx);   // no index below leaves the cache, whatever the device word holds
     if ((int) blockIdx.z * AT_WAVES * 16 >= nquery) return;   // none of the block's queries count
     const bool wave_on = uniform(wave * 16 < nquery);         // a wave without queries still fetches its share of K and V
     const int ql = lane & 15, pg = lane >> 4;
     const int qi = wave * 16 + ql;                      // this lane's query (as B column / accumulator column)
     const bool qlive = qi < nquery;
     const int qt = qlive ? qi / qpk : 0, qh = kvh * qpk + (qlive ? qi % qpk : 0);
-    const int ctx_q = qlive ? pos0 + qt + 1 : 0;        // positions [0, ctx_q) are this query's
-    const int ctx_max = pos0 + T;                       // the window's last row sees this many
-    const int p0 = s * AT_SPLIT, p1 = min(ctx_max, p0 + AT_SPLIT);
+    const int ctx_q = qlive ? att_ctx_q(win, qt) : 0;   // positions [0, ctx_q) are this query's
+    const int ctx_max = win.ctx_max;                    // the window's last row sees this many
+    const int p0 = att_split_begin(s), p1 = att_split_end(win, s);
     const size_t slot = ((size_t) qt * nq + qh) * nsplit + s;
     if (p0 >= p1) {   // a split past the context: an empty part
         if (qlive && pg == 0) mz_out[slot] = AttPart{-INFINITY, 0.f};
@@ -502,7 +505,7 @@ __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per
     auto fetch = [&](int c0) {   // rows and blocks clamped inside the window's rows
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int pos = min(c0 + krow + 8 * i, ctx_max - 1), blk = min((c0 >> 2) + vblk + 2 * i, (ctx_max - 1) >> 2);
+            const int pos = att_fetch_row(win, c0, krow + 8 * i), blk = att_fetch_vblock(win, c0, vblk + 2 * i);
             kr[i] = *(g128*) (kbase + ((size_t) pos * nkv + kvh) * (AT_HD * 2) + 16 * kcol);
             vr[i] = *(g128*) (vbase + ((size_t) blk * nkv + kvh) * (AT_HD * 8) + 16 * vcol);
         }
@@ -637,11 +640,13 @@ __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per
 constexpr int AT_MAXSPLIT = 2048;
 __global__ void __launch_bounds__(AT_HD) k_attn_combine(const float* __restrict__ qg, const float* __restrict__ acc_in,
                                                        const AttPart* __restrict__ mz_in, float* __restrict__ out, uint8_t* __restrict__ outq,
-                                                       int nq, int nsplit, int T, const int* __restrict__ pos0p, const int* __restrict__ gate,
-                                                       const int* __restrict__ live) {
+                                                       int nq, int nsplit, int T, const int* __restrict__ pos0p, int max_ctx, unsigned* __restrict__ err,
+                                                       const int* __restrict__ gate, const int* __restrict__ live) {
     __shared__ float wsp[AT_MAXSPLIT];
     __shared__ float red[AT_HD / 64];
     if (gate && uniform(*gate) == 0) return;
+    // a window that leaves the cache: reported (err may be null), and computed over the cells that exist
+    if (err && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0 && !att_window_fits(*pos0p, T, max_ctx)) atomicOr(err, FNX_ERR_WINDOW);
     if (live) T = uniform(max(1, min(*live, T)));
     const int h = blockIdx.x, t = blockIdx.y, i = threadIdx.x;
     if (t >= T) {   // a row that does not count: zeros (its queries were left out; what follows it stays finite)
@@ -650,7 +655,7 @@ __global__ void __launch_bounds__(AT_HD) k_attn_combine(const float* __restrict_
         return;
     }
     const size_t base = ((size_t) t * nq + h) * nsplit;
-    const int nlive = min(nsplit, (*pos0p + T + AT_SPLIT - 1) / AT_SPLIT);   // splits the window's context reaches: their parts were written
+    const int nlive = att_live_splits(att_window(*pos0p, T, max_ctx), nsplit);   // splits the window's context reaches: their parts were written
     float mx = -INFINITY;
     for (int s = i; s < nlive; s += AT_HD) mx = fmaxf(mx, mz_in[base + s].m);
     mx = group_max<64>(mx);

@@ -13,6 +13,13 @@
 
 namespace fnx {
 
+// before the verify: a session whose window does not fit the caches (or whose context buffer is full) stops here, so the
+// first round of a badly placed session changes nothing either (later rounds are kept inside by k_round_commit)
+__global__ void k_round_guard(int* __restrict__ state, int ctx_cap, int max_ctx) {
+    const int pos = state[FNX_RS_POS], n_ctx = state[FNX_RS_NCTX];
+    if (pos < 0 || pos + FNX_MAXT > max_ctx || n_ctx + FNX_MAXT > ctx_cap) state[FNX_RS_STOP] = 1;
+}
+
 // after the verify (session.cpp:565-573, 616-640): n = 1 + the drafts that equal the row before's pick; the picks of the
 // rows kept join the context; the positions move on by n. One wave.
 // A round whose next window would not fit the caches (max_ctx) or the context buffer raises FNX_RS_STOP and changes

@@ -1,0 +1,65 @@
+// Host-side bounds check of the attention kernels' index arithmetic (csrc/attn_window.h): for caches of 192, 520 and
+// 32,768 cells, every window position from well below 0 to well past the end, every row count and every block of the
+// first pass, walk the chunks as the kernel's loop does and check that each K row and V block it would fetch lies inside
+// the cache, that every query's context does, and that the fit predicate is exact. No GPU: an out-of-range position is
+// never run on one.
+#include <cstdio>
+#include <cstdlib>
+
+#include "attn_window.h"
+
+using namespace fnx;
+
+static long checked = 0;
+static void require(bool ok, const char* what, int max_ctx, int pos0, int T, int s, int c0) {
+    ++checked;
+    if (ok) return;
+    std::printf("FAILED %s: max_ctx %d pos0 %d T %d split %d chunk %d\n", what, max_ctx, pos0, T, s, c0);
+    std::exit(1);
+}
+
+int main() {
+    const int caps[] = {4, 192, 520, 32768};
+    for (int max_ctx : caps) {
+        const int nsplit = attn_splits(max_ctx), vblocks = (max_ctx + 3) / 4;
+        const int step = max_ctx > 1024 ? 97 : 1;
+        for (int pos0 = -40; pos0 <= max_ctx + 40; pos0 += (pos0 > 64 && pos0 < max_ctx - 64 ? step : 1))
+            for (int T = 1; T <= 16; ++T) {
+                const AttWindow w = att_window(pos0, T, max_ctx);
+                const bool fits = pos0 >= 0 && pos0 + T <= max_ctx;
+                require(att_window_fits(pos0, T, max_ctx) == fits, "fit predicate", max_ctx, pos0, T, -1, -1);
+                require(w.pos0 >= 0 && w.pos0 < max_ctx && w.ctx_max >= 1 && w.ctx_max <= max_ctx, "window", max_ctx, pos0, T, -1, -1);
+                if (fits) require(w.pos0 == pos0 && w.ctx_max == pos0 + T, "a window that fits is left alone", max_ctx, pos0, T, -1, -1);
+                for (int qt = 0; qt < T; ++qt) {
+                    const int c = att_ctx_q(w, qt);
+                    require(c >= 1 && c <= w.ctx_max, "query context", max_ctx, pos0, T, -1, qt);
+                    if (fits) require(c == pos0 + qt + 1, "query context of a window that fits", max_ctx, pos0, T, -1, qt);
+                }
+                require(att_live_splits(w, nsplit) >= 1 && att_live_splits(w, nsplit) <= nsplit, "live splits", max_ctx, pos0, T, -1, -1);
+                for (int s = 0; s < nsplit; ++s) {
+                    const int p0 = att_split_begin(s), p1 = att_split_end(w, s);
+                    if (p0 >= p1) {
+                        require(s >= att_live_splits(w, nsplit), "an empty split is not a live one", max_ctx, pos0, T, s, -1);
+                        continue;
+                    }
+                    require(s < att_live_splits(w, nsplit), "a split with data is a live one", max_ctx, pos0, T, s, -1);
+                    auto fetch = [&](int c0) {
+                        for (int r = 0; r < AT_CH; ++r) {
+                            const int row = att_fetch_row(w, c0, r);
+                            require(row >= 0 && row < max_ctx, "K row", max_ctx, pos0, T, s, c0);
+                        }
+                        for (int b = 0; b < AT_CH / 4; ++b) {
+                            const int blk = att_fetch_vblock(w, c0, b);
+                            require(blk >= 0 && blk < vblocks, "V block", max_ctx, pos0, T, s, c0);
+                        }
+                    };
+                    // the kernel's order: the first chunk, the second (or the split's last row), then two ahead each trip
+                    fetch(p0);
+                    fetch(att_min(p0 + AT_CH, p1 - 1));
+                    for (int c0 = p0; c0 < p1; c0 += AT_CH) fetch(att_min(c0 + 2 * AT_CH, p1 - 1));
+                }
+            }
+    }
+    std::printf("ok %ld\n", checked);
+    return 0;
+}

@@ -134,6 +134,22 @@ def test_attn_matches_oracle(dev, oracle, nq, nkv, T, pos0):
     assert np.all(np.isfinite(got))
 
 
+@pytest.mark.parametrize("max_ctx", [192, 520])
+def test_attn_window_ends_at_the_caches_last_cell(dev, oracle, max_ctx):
+    """a cache whose size is not a multiple of the split (512) or is smaller than one, the window's last row in the last
+    cell: the largest position that is in range (positions out of range are a matter of the host-side bounds test)"""
+    nq, nkv, T = 16, 2, 16
+    pos0 = max_ctx - T
+    print(f"case attn end of cache max_ctx={max_ctx} pos0={pos0}", flush=True)
+    rng = np.random.default_rng(840 + max_ctx)
+    qg = rng.standard_normal((T, nq, 512)).astype(np.float32)
+    kc, vc = rng.standard_normal((max_ctx, nkv, 256)).astype(np.float16), rng.standard_normal((max_ctx, nkv, 256)).astype(np.float16)
+    want = np.zeros((T, nq, 256), dtype=np.float32)
+    oracle.lib.fnx_o_attn(ol.ptr(qg), ol.ptr(kc), ol.ptr(vc), ol.ptr(want), nq, nkv, 256, T, pos0)
+    got = dev.attn(qg, kc, vc, nq, nkv, pos0)
+    assert rel_l2(got, want) <= 2e-5
+
+
 def chain_close(got, want, fresh):
     rows = [rel_l2(got[i], want[i]) for i in range(len(want))]
     assert max(rows) <= 1e-2, rows

@@ -28,3 +28,13 @@ def test_host_mirror_compiles_and_runs(oracle, tmp_path):
     assert lines[2] == f"dist 2 p0 {p0:.6f} draw 11 12"
     assert lines[3] == "gguf tensors 1 ne0 8 arch demo"
     assert lines[4] == "refused: gguf: no tensor missing"
+
+
+def test_attention_window_bounds(tmp_path):
+    """the attention kernels' index arithmetic for a position word the host cannot see, compiled for the host: caches of
+    192, 520 and 32,768 cells with windows from below 0 to past the end never index outside the cache"""
+    exe = str(tmp_path / "attn_window_check")
+    subprocess.run(["g++", "-std=c++17", "-O1", "-Wall", "-Wextra", "-Werror", "-I", os.path.join(fnx_gpu.PKG_DIR, "csrc"), "-o", exe,
+                    os.path.join(HERE, "attn_window_check.cpp")], check=True, capture_output=True, text=True)
+    r = subprocess.run([exe], check=True, capture_output=True, text=True, timeout=120)
+    assert r.stdout.startswith("ok "), r.stdout
