@@ -131,6 +131,8 @@ def main():
                     help="also run one plain device copy of 256 MiB, the known-size kernel that scales the FETCH_SIZE / WRITE_SIZE counters")
     ap.add_argument("--weights", choices=["gaussian", "bytes"], default="gaussian",
                     help="gaussian: experts IQ3_S-encoded from N(0, 0.02) weights (benchmark config 2's recipe); bytes: uniformly random blocks")
+    ap.add_argument("--shared-q8", action="store_true",
+                    help="the shared expert as dense split Q8_0 (the reference's own form, three more launches a window) instead of IQ3_S")
     ap.add_argument("--no-extras", action="store_true", help="skip the legs beside the headline (streaming calibration, config 1, the other weight kind)")
     ap.add_argument("--raw-layout", action="store_true", help="leave the weights as raw ggml blocks (skip the load-time re-laying)")
     ap.add_argument("--workload", choices=["verify", "prefill", "decoder", "head", "gemv"], default="verify",
@@ -191,6 +193,16 @@ def main():
             raw = [a.cpu().numpy() for a in (gu, down, sh_gu, sh_down)] if not sets and keep_raw else None
             (gu, down, sh_gu, sh_down), dws = fnx_gpu.pack_moe_weights(dev, [gu, down, sh_gu, sh_down], N, FF, not args.raw_layout)
             L = pkg.MoeLayer(N, FF, NEXP, TOPK, router.data_ptr(), 0, dws[0], GU_BYTES, dws[1], DN_BYTES, dws[2], dws[3])
+            if args.shared_q8:
+                q8 = [torch.randint(-127, 128, (2 * FF, N), dtype=torch.int8, device="cuda", generator=g),
+                      (torch.rand((2 * FF, N // 32), device="cuda", generator=g) * 3e-4 + 1e-5).to(torch.float16),
+                      torch.randint(-127, 128, (N, FF), dtype=torch.int8, device="cuda", generator=g),
+                      (torch.rand((N, FF // 32), device="cuda", generator=g) * 3e-4 + 1e-5).to(torch.float16)]
+                L.sh_gu_q8 = pkg.Q8S(q8[0].data_ptr(), q8[1].data_ptr(), 2 * FF, N)
+                L.sh_down_q8 = pkg.Q8S(q8[2].data_ptr(), q8[3].data_ptr(), N, FF)
+                if raw is not None:
+                    raw = raw[:2] + [None, None, ((q8[0].cpu().numpy(), q8[1].cpu().numpy().view(np.uint16)), (q8[2].cpu().numpy(), q8[3].cpu().numpy().view(np.uint16)))]
+                sh_gu = q8   # keeps the tensors alive
             sets.append((L, router, gu, down, sh_gu, sh_down, raw))
         return sets
 
@@ -301,9 +313,10 @@ def main():
         oracle = oracle_lib.Oracle()
         threads = min(os.cpu_count() or 1, 16)
         L, router = layers[0][0], layers[0][1]
-        h = [router.cpu().numpy()] + layers[0][6]
+        h = [router.cpu().numpy()] + layers[0][6][:4]
+        okw = dict(threads=threads, sh_q8=layers[0][6][4]) if args.shared_q8 else dict(threads=threads)
         xh = xs[0].cpu().numpy()
-        r = oracle.moe_verify_layer(N, FF, NEXP, TOPK, *h, xh, threads=threads)   # warm-up, and a last parity check
+        r = oracle.moe_verify_layer(N, FF, NEXP, TOPK, *h, xh, **okw)   # warm-up, and a last parity check
         dev.ok(lib.fnx_moe_verify_layer(C.byref(L), xs[0].data_ptr(), T, outs[0].data_ptr(), C.byref(ws), st))
         torch.cuda.synchronize()
         err = float(np.linalg.norm(outs[0].cpu().numpy() - r["out"]) / np.linalg.norm(r["out"]))
@@ -311,7 +324,7 @@ def main():
         c0 = time.perf_counter()
         n_cpu = 0
         while time.perf_counter() - c0 < args.cpu_seconds or n_cpu < 2:
-            oracle.moe_verify_layer(N, FF, NEXP, TOPK, *h, xh, threads=threads)
+            oracle.moe_verify_layer(N, FF, NEXP, TOPK, *h, xh, **okw)
             n_cpu += 1
         cdt = time.perf_counter() - c0
         cpu = {"value": n_cpu / cdt, "unit": "layer-steps/s", "cores": threads, "kind": "port",
@@ -330,7 +343,7 @@ def main():
                  "512 experts x the weight sets at addresses of their own)" if args.weights == "gaussian" else
                  "synthetic: uniformly random IQ3_S blocks") + ", f32 router N(0, 0.02), activations N(0, 1)",
         "config": {"workload": "config 2: one MoE verify layer, T=16, hidden 2048, 512 IQ3_S experts top-10, SwiGLU ff 512, shared expert, f32 router",
-                   "weights": args.weights,
+                   "weights": args.weights, "shared_expert": "split Q8_0 (dense launches)" if args.shared_q8 else "IQ3_S (inside the window's launches)",
                    "weight_layout": "raw ggml blocks" if args.raw_layout else "unit64 (re-laid once at load, same bytes)", "weight_sets": args.layers, "distinct_experts_per_step": u_mean, "step_algorithmic_bytes": step_bytes,
                    "step_hbm_frac": step_bytes / (ms_per_step * 1e-3) / HBM_PEAK,
                    "ms_per_step_other_weights": None if other_ms is None else {("bytes" if args.weights == "gaussian" else "gaussian"): other_ms},

@@ -145,6 +145,12 @@ int fnx_accept_greedy_dev(const int* rows, const int* o, int R, int* n_accept, v
  * n = 2048 and ff of 256, 512 or 1024 the window runs in five launches: [router logits | q8_1 rows], [top-k],
  * [jobs + gate|up routed + shared], [SwiGLU + down routed + shared], [combine]; other shapes run operator by operator.
  * Like moe_down, one MoE may be in flight per device. */
+/* model.hpp:78-82  Q8S: dense Q8_0 in the split layout: int8 values [n_out][n_in], f16 scale bits [n_out][n_in / 32] */
+typedef struct fnx_q8s {
+    const int8_t* q;
+    const uint16_t* d;
+    int n_out, n_in;
+} fnx_q8s;
 typedef struct fnx_moe_layer {
     int n, ff, nexp, topk;   /* hidden, expert width, experts, picks per token */
     const void* router;      /* [nexp + 1][n]: the router's rows, then the shared expert's gate */
@@ -155,6 +161,10 @@ typedef struct fnx_moe_layer {
     size_t down_stride;
     fnx_dw sh_gu;            /* shared expert gate|up */
     fnx_dw sh_down;          /* shared expert down */
+    /* the shared expert as dense split Q8_0 (model.hpp:84-94, DW::s; engine.cu:1600-1604 runs it as q8s_gemv ->
+     * swiglu_stacked_q8_1 -> q8s_gemv): when both q pointers are set these are used and sh_gu / sh_down are not read */
+    fnx_q8s sh_gu_q8;        /* n_out = 2 ff, n_in = n */
+    fnx_q8s sh_down_q8;      /* n_out = n, n_in = ff */
 } fnx_moe_layer;
 /* caller-owned scratch for one window; sizes from fnx_moe_ws_bytes */
 typedef struct fnx_moe_ws {
@@ -251,12 +261,6 @@ int fnx_combine_add_norm_q8(const float* part, const float* topw, const float* s
 int fnx_add_rows(const float* a, const float* b, float* y, size_t n, void* st);
 /* rows tokens[t] of an f16 table [vocab][n] as f32 (the window's input rows) */
 int fnx_embed_rows(const uint16_t* emb, const int* tokens, int T, int vocab, int n, float* y, void* st);
-/* model.hpp:78-82  Q8S: dense Q8_0 in the split layout: int8 values [n_out][n_in], f16 scale bits [n_out][n_in / 32] */
-typedef struct fnx_q8s {
-    const int8_t* q;
-    const uint16_t* d;
-    int n_out, n_in;
-} fnx_q8s;
 /* dense.cuh:79-214 (q8s_gemv): out[t * out_stride + r] = W[r] . y[t] for T <= 16 q8_1 rows; n_in a multiple of 256. The
  * result is (s0 + s1) + (s2 + s3), s_q the q-th quarter of the columns, its 32-column blocks folded in ascending order with
  * acc = fmaf(d_w * d_x, (float) dot, acc) */

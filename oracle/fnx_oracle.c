@@ -909,11 +909,14 @@ void fnx_o_moe_verify_layer(const fnx_o_moe_layer* L, const float* x, int T, flo
         sh.y[t] = t;
         sh.out[t] = P + t;
     }
-    fnx_o_mmvq_iq3s(L->sh_gu, 0, NULL, 2 * ff, n, &sh, 1, xq, gu, 2 * ff, threads);
+    if (L->sh_gu_q) fnx_o_q8s_gemv(L->sh_gu_q, L->sh_gu_d, 2 * ff, n, xq, gu + (size_t) P * 2 * ff, 2 * ff, T); /* engine.cu:1601 */
+    else fnx_o_mmvq_iq3s(L->sh_gu, 0, NULL, 2 * ff, n, &sh, 1, xq, gu, 2 * ff, threads);
     fnx_o_swiglu_stacked_q8_1(gu, hq, ff, P + T);
     fnx_o_mmvq_iq3s(L->down, dn_stride, NULL, n, ff, jdn, nj, hq, part, n, threads);
     for (int t = 0; t < T; ++t) sh.y[t] = P + t;
-    fnx_o_mmvq_iq3s(L->sh_down, 0, NULL, n, ff, &sh, 1, hq, part, n, threads);
+    if (L->sh_gu_q) /* engine.cu:1603: the rows P + t of hq and of part */
+        fnx_o_q8s_gemv(L->sh_down_q, L->sh_down_d, n, ff, hq + (size_t) P * (ff / 32) * Q8_1_BLOCK, part + (size_t) P * n, n, T);
+    else fnx_o_mmvq_iq3s(L->sh_down, 0, NULL, n, ff, &sh, 1, hq, part, n, threads);
     fnx_o_moe_combine(part, topw, part + (size_t) P * n, logits + nexp, nexp + 1, out, T, n, topk);
 
     if (logits_out) memcpy(logits_out, logits, (size_t) T * (nexp + 1) * sizeof(float));

@@ -138,6 +138,12 @@ typedef struct {
     const uint8_t* down;             /* [nexp][n][ff] IQ3_S */
     const uint8_t* sh_gu;            /* [2 ff][n] IQ3_S */
     const uint8_t* sh_down;          /* [n][ff] IQ3_S */
+    /* the shared expert as dense split Q8_0 instead (engine.cu:1600-1604: q8s_gemv -> swiglu_stacked_q8_1 -> q8s_gemv):
+     * when sh_gu_q is not null these four are used and sh_gu / sh_down are not read (the verify layer only) */
+    const int8_t* sh_gu_q;           /* [2 ff][n] */
+    const uint16_t* sh_gu_d;         /* [2 ff][n / 32] f16 bits */
+    const int8_t* sh_down_q;         /* [n][ff] */
+    const uint16_t* sh_down_d;       /* [n][ff / 32] */
 } fnx_o_moe_layer;
 /* out [T][n]; optional outputs (may be null): logits [T][nexp+1], topi/topw [T][topk], njobs */
 void fnx_o_moe_verify_layer(const fnx_o_moe_layer* L, const float* x, int T, float* out, float* logits, int* topi,

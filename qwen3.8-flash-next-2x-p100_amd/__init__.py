@@ -31,10 +31,14 @@ class DW(C.Structure):
                 ("ep", C.c_void_p)]
 
 
+class Q8S(C.Structure):
+    _fields_ = [("q", C.c_void_p), ("d", C.c_void_p), ("n_out", C.c_int), ("n_in", C.c_int)]
+
+
 class MoeLayer(C.Structure):
     _fields_ = [("n", C.c_int), ("ff", C.c_int), ("nexp", C.c_int), ("topk", C.c_int), ("router", C.c_void_p),
                 ("router_bf16", C.c_int), ("gu", DW), ("gu_stride", C.c_size_t), ("down", DW), ("down_stride", C.c_size_t),
-                ("sh_gu", DW), ("sh_down", DW)]
+                ("sh_gu", DW), ("sh_down", DW), ("sh_gu_q8", Q8S), ("sh_down_q8", Q8S)]
 
 
 class MoeWs(C.Structure):
@@ -44,10 +48,6 @@ class MoeWs(C.Structure):
 
 class PfWs(C.Structure):
     _fields_ = [(k, C.c_void_p) for k in ("logits", "topi", "topw", "cnt", "jbase", "jobs_gu", "jobs_dn", "njobs", "xh", "gu", "h16", "part")]
-
-
-class Q8S(C.Structure):
-    _fields_ = [("q", C.c_void_p), ("d", C.c_void_p), ("n_out", C.c_int), ("n_in", C.c_int)]
 
 
 class Rope(C.Structure):

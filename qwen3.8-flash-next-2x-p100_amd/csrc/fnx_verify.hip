@@ -766,12 +766,15 @@ static int rows_launch(const fnx_dw* W, size_t w_stride, const fnx_job* jobs, co
 }
 
 // the shapes and layouts the window's three launches take (k_moe_layer.h)
+// the shared expert as dense split Q8_0 (engine.cu:1600-1604) instead of sh_gu / sh_down
+static bool shared_is_q8(const fnx_moe_layer* L) { return L->sh_gu_q8.q && L->sh_down_q8.q; }
 static bool layer_fused_ok(const fnx_moe_layer* L, int T) {
     static const int on = env_int("FNX_LAYER_FUSED", 1, 0, 1);
     const auto packed = [](const fnx_dw& w) { return w.type == FNX_T_IQ3S_UNIT64; };
+    const bool shared_ok = shared_is_q8(L) || (packed(L->sh_gu) && packed(L->sh_down) && L->sh_gu.p && L->sh_down.p);
     return on && L->n == FL_N && (L->ff == 256 || L->ff == 512 || L->ff == 1024) && L->nexp <= 1024 && L->topk <= FL_MAXK &&
-           T * L->topk <= FL_MAXP && packed(L->gu) && packed(L->sh_gu) && packed(L->down) && packed(L->sh_down) &&
-           L->gu_stride % UNIT_BYTES == 0 && L->down_stride % UNIT_BYTES == 0 && L->sh_gu.p && L->sh_down.p;
+           T * L->topk <= FL_MAXP && packed(L->gu) && packed(L->down) && shared_ok && L->gu_stride % UNIT_BYTES == 0 &&
+           L->down_stride % UNIT_BYTES == 0;
 }
 // per-launch timing of the window (fnx_layer_profile): events recorded on the launch stream around each of the three
 // launches; the counterpart of the reference's FNX_PROF stamps in its window graph (engine.cu:1382-1530)
@@ -789,16 +792,30 @@ static int layer_fused(const fnx_moe_layer* L, const float* x, int T, float* out
     const int rblocks = (LS + RQ_ROWS - 1) / RQ_ROWS, qblocks = (T * 64 + 2 * FL_WAVES - 1) / (2 * FL_WAVES);
     prof_mark(0, s);
     k_router_quant<<<rblocks + qblocks, FL_THREADS, 0, s>>>(RouterArgs{L->nexp, T, x, L->router, L->router_bf16, ws->logits, (uint8_t*) ws->xq, live});
+    // a split-Q8_0 shared expert runs as the reference runs it, three dense launches on the q8_1 rows just made
+    // (q8s_gemv -> swiglu_stacked_q8_1 -> q8s_gemv); its f32 rows, q8_1 rows of h and down rows take the workspace's
+    // part buffer, which the three-launch window does not use otherwise; the down launch adds its gated rows
+    const bool q8sh = shared_is_q8(L);
+    float* sh_part = nullptr;
+    if (q8sh) {
+        float* sgu = ws->part;                                                              // [T][2 ff]
+        uint8_t* shq = reinterpret_cast<uint8_t*>(sgu + (size_t) T * 2 * ff);                // [T][ff / 32] q8_1 blocks
+        sh_part = sgu + (size_t) T * 2 * ff + ((size_t) T * (ff / 32) * FNX_Q8_1_BLOCK + 255) / 256 * 64;   // [T][n], 256-byte aligned after shq
+        if (fnx_q8s_gemv(&L->sh_gu_q8, ws->xq, sgu, 2 * ff, T, st)) return 1;
+        if (fnx_swiglu_stacked_q8_1(sgu, shq, ff, T, st)) return 1;
+        if (fnx_q8s_gemv(&L->sh_down_q8, shq, sh_part, n, T, st)) return 1;
+    }
     prof_mark(1, s);
     const RouteArgs route{L->nexp, L->topk, T, ws->logits, ws->topi, ws->topw, ws->jobs_gu, ws->jobs_dn, ws->njobs, live};
     // at least as many blocks as the window has rows (a block's run of items then lies in two rows at most)
     static const int gh_blocks = env_int("FNX_GH_BLOCKS", 0, 0, 4096);
-    const GateUpArgs ga{ff, (const uint8_t*) L->gu.p, L->gu_stride, (const uint8_t* const*) L->gu.ep, (const uint8_t*) L->sh_gu.p,
+    const GateUpArgs ga{ff, (const uint8_t*) L->gu.p, L->gu_stride, (const uint8_t* const*) L->gu.ep, q8sh ? nullptr : (const uint8_t*) L->sh_gu.p,
                         (const uint8_t*) ws->xq, (uint32_t*) ws->gu, route};
     k_moe_gate_up_h<<<std::max(gh_blocks ? gh_blocks : cu_count(), FNX_MAXT), GH_THREADS, 0, s>>>(ga);
     prof_mark(2, s);
     const DownArgs da{n, ff, L->topk, T, L->nexp, (const uint8_t*) L->down.p, L->down_stride, (const uint8_t* const*) L->down.ep,
-                      (const uint8_t*) L->sh_down.p, (const uint32_t*) ws->gu, ws->topi, ws->topw, ws->logits, out, live, route};
+                      q8sh ? nullptr : (const uint8_t*) L->sh_down.p, (const uint32_t*) ws->gu, ws->topi, ws->topw, ws->logits, out, live, route,
+                      sh_part};
     // a block per row and 32 units of the output, and one more for the job lists
     if (ff == 256) k_moe_down_combine<8><<<T * (n / (8 * 32)) + 1, FL_THREADS, 0, s>>>(da);
     else if (ff == 512) k_moe_down_combine<16><<<T * (n / (4 * 32)) + 1, FL_THREADS, 0, s>>>(da);
@@ -993,6 +1010,15 @@ int fnx_layer_profile_read(float* ms3) {
     return 0;
 }
 
+// the layer's matrices against n / ff; the shared expert in whichever form it comes
+static bool moe_shapes_ok(const fnx_moe_layer* L) {
+    const int n = L->n, ff = L->ff;
+    if (L->gu.n_in != n || L->gu.n_out != 2 * ff || L->down.n_in != ff || L->down.n_out != n) return false;
+    if (shared_is_q8(L))
+        return L->sh_gu_q8.d && L->sh_down_q8.d && L->sh_gu_q8.n_in == n && L->sh_gu_q8.n_out == 2 * ff && L->sh_down_q8.n_in == ff &&
+               L->sh_down_q8.n_out == n;
+    return L->sh_gu.n_in == n && L->sh_gu.n_out == 2 * ff && L->sh_down.n_in == ff && L->sh_down.n_out == n;
+}
 static int moe_layer_checked(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st, const int* live = nullptr) {
     if (!L || !x || !ws) return fail("moe_verify_layer: null argument");
     if (!ws->xq || !ws->logits || !ws->topi || !ws->topw || !ws->jobs_gu || !ws->jobs_dn || !ws->njobs || !ws->gu || !ws->part)
@@ -1000,9 +1026,7 @@ static int moe_layer_checked(const fnx_moe_layer* L, const float* x, int T, floa
     if (topk_check(T, L->nexp, L->topk, "moe_verify_layer")) return 1;
     const int P = T * L->topk, n = L->n, ff = L->ff;
     if (P + T > HQ_ROWS) return fail("moe_verify_layer: more pairs than the pair buffer holds");
-    if (L->gu.n_in != n || L->gu.n_out != 2 * ff || L->down.n_in != ff || L->down.n_out != n || L->sh_gu.n_in != n ||
-        L->sh_gu.n_out != 2 * ff || L->sh_down.n_in != ff || L->sh_down.n_out != n)
-        return fail("moe_verify_layer: weight shapes do not match n / ff");
+    if (!moe_shapes_ok(L)) return fail("moe_verify_layer: weight shapes do not match n / ff");
     if (!out) return fail("moe_verify_layer: null argument");
     if (live && !layer_fused_ok(L, T)) return fail("moe_verify_layer: a device-side row count needs the three-launch window");
     if (layer_fused_ok(L, T)) return layer_fused(L, x, T, out, ws, st, live);
@@ -1013,11 +1037,18 @@ static int moe_layer_checked(const fnx_moe_layer* L, const float* x, int T, floa
                                          0, 1);
     if (launch_status("moe_verify_layer topk")) return 1;
     if (rows_launch(&L->gu, L->gu_stride, ws->jobs_gu, ws->njobs, P, ws->xq, ws->gu, 2 * ff, st, "moe_verify_layer gate|up")) return 1;
-    if (rows_launch(&L->sh_gu, 0, ws->jobs_gu + P, nullptr, 1, ws->xq, ws->gu, 2 * ff, st, "moe_verify_layer shared gate|up", true)) return 1;
+    const bool q8sh = shared_is_q8(L);   // engine.cu:1600-1604: the rows P + t of gu, of the q8_1 rows of h and of part
+    if (q8sh) {
+        if (fnx_q8s_gemv(&L->sh_gu_q8, ws->xq, ws->gu + (size_t) P * 2 * ff, 2 * ff, T, st)) return 1;
+    } else if (rows_launch(&L->sh_gu, 0, ws->jobs_gu + P, nullptr, 1, ws->xq, ws->gu, 2 * ff, st, "moe_verify_layer shared gate|up", true)) return 1;
     k_swiglu_q8_1<<<dim3((ff / 32 + 7) / 8, P + T), 256, 0, s>>>(ws->gu, ws->gu + ff, (size_t) 2 * ff, nullptr, ff);
     if (launch_status("moe_verify_layer swiglu")) return 1;
     if (rows_launch(&L->down, L->down_stride, ws->jobs_dn, ws->njobs, P, nullptr, ws->part, n, st, "moe_verify_layer down")) return 1;
-    if (rows_launch(&L->sh_down, 0, ws->jobs_dn + P, nullptr, 1, nullptr, ws->part, n, st, "moe_verify_layer shared down", true)) return 1;
+    if (q8sh) {
+        const uint8_t* hq_dev = nullptr;   // the device's pair buffer of q8_1 rows (k_swiglu_q8_1 wrote it): the shared rows start at pair P
+        if (hipGetSymbolAddress((void**) &hq_dev, HIP_SYMBOL(g_moe_hq)) != hipSuccess) return fail("moe_verify_layer: no pair buffer");
+        if (fnx_q8s_gemv(&L->sh_down_q8, hq_dev + (size_t) P * (ff / 32) * FNX_Q8_1_BLOCK, ws->part + (size_t) P * n, n, T, st)) return 1;
+    } else if (rows_launch(&L->sh_down, 0, ws->jobs_dn + P, nullptr, 1, nullptr, ws->part, n, st, "moe_verify_layer shared down", true)) return 1;
     return fnx_moe_combine(ws->part, ws->topw, ws->part + (size_t) P * n, ws->logits + L->nexp, L->nexp + 1, out, T, n, L->topk, st);
 }
 int fnx_moe_verify_layer(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st) {
@@ -1060,9 +1091,8 @@ int fnx_moe_verify_layer_static(const fnx_moe_layer* L, const float* x, int T, f
     const fnx_moe_ws ws{w, (float*) (w + NA_OFF_LOGITS), (int*) (w + NA_OFF_TOPI), (float*) (w + NA_OFF_TOPW), (fnx_job*) (w + NA_OFF_JGU),
                         (fnx_job*) (w + NA_OFF_JDN), (int*) (w + NA_OFF_NJOBS), (float*) (w + NA_OFF_HQ), nullptr};
     const int P = T * L->topk, n = L->n, ff = L->ff;
-    if (L->gu.n_in != n || L->gu.n_out != 2 * ff || L->down.n_in != ff || L->down.n_out != n || L->sh_gu.n_in != n ||
-        L->sh_gu.n_out != 2 * ff || L->sh_down.n_in != ff || L->sh_down.n_out != n)
-        return fail("moe_verify_layer_static: weight shapes do not match n / ff");
+    if (shared_is_q8(L)) return fail("moe_verify_layer_static: a split-Q8_0 shared expert needs a caller's workspace (fnx_moe_verify_layer)");
+    if (!moe_shapes_ok(L)) return fail("moe_verify_layer_static: weight shapes do not match n / ff");
     if (topk_check(T, L->nexp, L->topk, "moe_verify_layer_static")) return 1;
     (void) P;
     return layer_fused(L, x, T, out, &ws, st);
@@ -1801,13 +1831,33 @@ int fnx_gguf_load_moe_layer(const fnx_gguf* g, int layer, int ff0, int ff1, int 
         const auto upload = [&](void* d, size_t n, const char* what) {
             if (hipMemcpy(d, host.data(), n, hipMemcpyHostToDevice) != hipSuccess) throw std::runtime_error(std::string("gguf_load_moe_layer: upload of ") + what + " failed");
         };
-        // IQ3_S: raw ggml blocks -> the unit64 layout, in place; other types stay as the file has them
-        const bool all_iq3s = m.ge.type == gguf::T_IQ3_S && m.de.type == gguf::T_IQ3_S && m.gsh.type == gguf::T_IQ3_S && m.dsh.type == gguf::T_IQ3_S;
+        // IQ3_S: raw ggml blocks -> the unit64 layout, in place; other types stay as the file has them. A Q8_0 shared
+        // expert (the reference's own form, engine.cu:1600-1604) becomes the split layout of fnx_q8s in its buffers, the
+        // same number of bytes: the int8 values of all rows, then the rows' f16 scales.
+        const bool routed_iq3s = m.ge.type == gguf::T_IQ3_S && m.de.type == gguf::T_IQ3_S;
+        const bool shared_iq3s = m.gsh.type == gguf::T_IQ3_S && m.dsh.type == gguf::T_IQ3_S;
+        const bool shared_q8 = m.gsh.type == QT_Q8_0 && m.dsh.type == QT_Q8_0;
+        const bool fast = routed_iq3s && (shared_iq3s || shared_q8);   // the three-launch window takes these
         const auto relay = [&](fnx_dw& w, void* d, size_t n) {
             w.p = d;
-            if (!all_iq3s) return;   // the window's fast form needs all four; operator by operator raw blocks do as well
+            if (!fast) return;   // operator by operator raw blocks do as well
             if (fnx_iq3s_repack(d, d, n / FNX_IQ3S_BLOCK * 256, st)) throw std::runtime_error(fnx_last_error());
             w.type = FNX_T_IQ3S_UNIT64;
+        };
+        std::vector<uint8_t> split;
+        const auto split_q8 = [&](fnx_dw& w, fnx_q8s& q, void* d, size_t n) {   // host holds the rows as raw Q8_0 blocks (34 bytes per 32 values)
+            const size_t nblk = n / 34, nval = nblk * 32;
+            split.resize(n);
+            for (size_t b = 0; b < nblk; ++b) {
+                std::memcpy(split.data() + 32 * b, host.data() + 34 * b + 2, 32);
+                std::memcpy(split.data() + nval + 2 * b, host.data() + 34 * b, 2);
+            }
+            if (hipMemcpy(d, split.data(), n, hipMemcpyHostToDevice) != hipSuccess) throw std::runtime_error("gguf_load_moe_layer: upload of the shared expert failed");
+            q.q = reinterpret_cast<const int8_t*>(d);
+            q.d = reinterpret_cast<const uint16_t*>(reinterpret_cast<const uint8_t*>(d) + nval);
+            q.n_out = w.n_out;
+            q.n_in = w.n_in;
+            w.p = nullptr;   // the raw form is not kept
         };
         gguf::router_rows(m.gi, m.gs, reinterpret_cast<float*>(host.data()));
         upload(dev->router, need.router_bytes, "the router");
@@ -1821,11 +1871,19 @@ int fnx_gguf_load_moe_layer(const fnx_gguf* g, int layer, int ff0, int ff1, int 
         relay(L->down, dev->down, need.down_bytes);
         size_t unused;
         gguf::expert_rows2(m.gsh, m.ush, ff0, ff1, host.data(), host.size(), &L->sh_gu, &unused);
-        upload(dev->sh_gu, need.sh_gu_bytes, "the shared gate|up");
-        relay(L->sh_gu, dev->sh_gu, need.sh_gu_bytes);
+        if (fast && shared_q8) split_q8(L->sh_gu, L->sh_gu_q8, dev->sh_gu, need.sh_gu_bytes);
+        else {
+            upload(dev->sh_gu, need.sh_gu_bytes, "the shared gate|up");
+            if (shared_iq3s) relay(L->sh_gu, dev->sh_gu, need.sh_gu_bytes);
+            else L->sh_gu.p = dev->sh_gu;
+        }
         gguf::expert_cols(m.dsh, ff0, ff1, host.data(), host.size(), &L->sh_down, &unused);
-        upload(dev->sh_down, need.sh_down_bytes, "the shared down");
-        relay(L->sh_down, dev->sh_down, need.sh_down_bytes);
+        if (fast && shared_q8) split_q8(L->sh_down, L->sh_down_q8, dev->sh_down, need.sh_down_bytes);
+        else {
+            upload(dev->sh_down, need.sh_down_bytes, "the shared down");
+            if (shared_iq3s) relay(L->sh_down, dev->sh_down, need.sh_down_bytes);
+            else L->sh_down.p = dev->sh_down;
+        }
         return 0;
     } catch (const std::exception& e) {
         return fail(e.what());

@@ -345,13 +345,15 @@ __global__ void __launch_bounds__(GH_THREADS) k_moe_gate_up_h(const GateUpArgs a
     // again is the unsigned one: the half-blocks read different forms.
     const int form = (2 * (int) blockIdx.x + (tid >> 9)) & 15;
     const uint32_t tab0 = signed_entry(g_sgrid.v[(form << 9) + (tid & 511)], form);
-    const int T = a.route.T, topk = a.route.topk, nexp = a.route.nexp, P = T * topk, qpp = a.ff >> 5, per_row = qpp * (topk + 1);
+    // k0: a row's first matrix - 0, the shared expert, or 1 when that one is not this launch's (w_shared null: run elsewhere)
+    const int T = a.route.T, topk = a.route.topk, nexp = a.route.nexp, P = T * topk, qpp = a.ff >> 5, k0 = a.w_shared ? 0 : 1;
+    const int nk = topk + 1 - k0, per_row = qpp * nk;
     const int Tl = a.route.live ? uniform(max(0, min(*a.route.live, T))) : T;
     // Quotients of small numbers (below 2^14, the divisor a few hundred at most) by a multiplication: with the divisor's
     // reciprocal rounded once and the dividend moved half a step up, the product misses the exact quotient by less than
     // the distance to the next integer. (Every wave of every block works these out: as integer divisions they were half
     // of what a wave executes before the barrier.)
-    const float r_nb = 1.0f / (float) gridDim.x, r_row = 1.0f / (float) per_row, r_k1 = 1.0f / (float) (topk + 1);
+    const float r_nb = 1.0f / (float) gridDim.x, r_row = 1.0f / (float) per_row, r_k1 = 1.0f / (float) nk;
     auto quot = [](int x, float r) { return (int) (((float) x + 0.5f) * r); };
     // this block's run of items
     const int total = Tl * per_row, nb = gridDim.x, ipb = quot(total + nb - 1, r_nb);
@@ -385,12 +387,12 @@ __global__ void __launch_bounds__(GH_THREADS) k_moe_gate_up_h(const GateUpArgs a
         m.t = quot(I, r_row);
         const int r = I - m.t * per_row;
         m.j = quot(r, r_k1);
-        m.k = r - m.j * (topk + 1);
+        m.k = k0 + r - m.j * nk;
         return m;
     };
     auto step = [&](GhItem& m) {
         if (++m.k > topk) {
-            m.k = 0;
+            m.k = k0;
             if (++m.j == qpp) {
                 m.j = 0;
                 ++m.t;
@@ -634,6 +636,7 @@ struct DownArgs {
     float* out;                // [T][rows]
     const int* live;           // may be null; else a device word: rows from *live on are left alone
     RouteArgs route;           // the job lists that the grid's last block writes
+    const float* sh_part;      // may be null; else [T][rows]: the shared expert's down rows, computed elsewhere (w_shared is then not read)
 };
 template <int SBR>
 __global__ void __launch_bounds__(FL_THREADS) k_moe_down_combine(const DownArgs a) {
@@ -663,6 +666,8 @@ __global__ void __launch_bounds__(FL_THREADS) k_moe_down_combine(const DownArgs 
         hw[j] = k <= topk ? a.hq[(size_t) (k < topk ? t * topk + k : P + t) * HQ_PER + (i - k * HQ_PER)] : 0u;
     }
     // lane k: pick k's matrix and weight; lane topk: the shared expert's and its gate
+    const bool ext = a.sh_part != nullptr;   // the shared expert's rows come from memory: the trips are the picks only
+    const int first = ext ? 1 : 0;
     const uint8_t* myw = a.w_shared;
     float myg = 0.f;
     if (lane < topk) {
@@ -683,10 +688,17 @@ __global__ void __launch_bounds__(FL_THREADS) k_moe_down_combine(const DownArgs 
     // trips 1 .. topk the picks in order; the shared expert's sums wait in registers for the chain's last step.
     auto pick_of = [&](int trip) { return trip == 0 ? topk : trip - 1; };   // the index of a trip's expert in hq and in the lanes
     PackedSub A[R], B[R], C[R];
-    {
+    float shp[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) shp[r] = 0.f;
+    if (!ext) {
         const __amdgpu_buffer_rsrc_t mtx = matrix_rsrc(a.w_shared);
 #pragma unroll
         for (int r = 0; r < R; ++r) A[r] = load_packed_buf(mtx, (u0 + r) * UNIT_BYTES, o);
+    } else if (kb == SBR - 1) {   // the lanes that store a row's result hold its shared part
+        const float* sp = a.sh_part + (size_t) t * a.rows + (size_t) u0 * RW + g;
+#pragma unroll
+        for (int r = 0; r < R; ++r) shp[r] = sp[r * RW];
     }
 #pragma unroll
     for (int i = 0; i < SGRID_WORDS / FL_THREADS; ++i) tab[tid + i * FL_THREADS] = signed_entry(tab0, i);
@@ -695,7 +707,8 @@ __global__ void __launch_bounds__(FL_THREADS) k_moe_down_combine(const DownArgs 
         const int i = tid + j * FL_THREADS;
         if (i < (topk + 1) * HQ_PER) (&hq[0][0][0])[i] = hw[j];
     }
-    issue(B, pick_of(1));   // topk >= 1
+    if (ext) issue(A, pick_of(1));   // topk >= 1
+    if (first + 1 <= topk) issue(B, pick_of(first + 1));
     __syncthreads();
     const int sc_shift = 4 * (lane & 1);
     float acc[R], zs[R];
@@ -724,7 +737,7 @@ __global__ void __launch_bounds__(FL_THREADS) k_moe_down_combine(const DownArgs 
         }
     };
     // two trips' loads are in flight while a third is decoded: with eight waves a CU that is about 56 KB a CU
-    for (int trip = 0; trip <= topk; trip += 3) {
+    for (int trip = first; trip <= topk; trip += 3) {
         if (trip + 2 <= topk) issue(C, pick_of(trip + 2));
         decode(A, trip);
         if (trip + 1 > topk) break;
@@ -733,6 +746,11 @@ __global__ void __launch_bounds__(FL_THREADS) k_moe_down_combine(const DownArgs 
         if (trip + 2 > topk) break;
         if (trip + 4 <= topk) issue(B, pick_of(trip + 4));
         decode(C, trip + 2);
+    }
+    if (ext) {
+        const float gs = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, myg), topk));
+#pragma unroll
+        for (int r = 0; r < R; ++r) zs[r] = gs * shp[r];
     }
     float res[R];
 #pragma unroll

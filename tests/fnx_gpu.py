@@ -517,7 +517,8 @@ class PfLayerDev:
 class MoeLayerDev:
     """One MoE layer's weights on the device plus a workspace, for fnx_moe_verify_layer and the per-op calls."""
 
-    def __init__(self, dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, T=16, packed=False):
+    def __init__(self, dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, T=16, packed=False, sh_q8=None):
+        """sh_q8: the shared expert as split Q8_0 instead of IQ3_S blocks: ((q, d) of gate|up, (q, d) of down)"""
         t = dev.torch
         self.dev, self.n, self.ff, self.nexp, self.topk = dev, n, ff, nexp, topk
         pkg = dev.pkg
@@ -528,6 +529,11 @@ class MoeLayerDev:
         # the load-time re-laying, in place
         (self.gu, self.down, self.sh_gu, self.sh_down), dws = pack_moe_weights(dev, [self.gu, self.down, self.sh_gu, self.sh_down], n, ff, packed)
         self.L = pkg.MoeLayer(n, ff, nexp, topk, self.router.data_ptr(), 0, dws[0], self.gu_stride, dws[1], self.down_stride, dws[2], dws[3])
+        if sh_q8 is not None:
+            self.q8 = [dev.up(a) for pair in sh_q8 for a in pair]
+            self.L.sh_gu_q8 = pkg.Q8S(self.q8[0].data_ptr(), self.q8[1].data_ptr(), 2 * ff, n)
+            self.L.sh_down_q8 = pkg.Q8S(self.q8[2].data_ptr(), self.q8[3].data_ptr(), n, ff)
+            self.L.sh_gu.p = self.L.sh_down.p = None   # not to be read
         P = T * topk
         self.P = P
         self.xq = dev.zeros(T * (n // 32) * 36, t.uint8)

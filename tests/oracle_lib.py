@@ -21,7 +21,8 @@ class Job(C.Structure):
 
 class MoeLayer(C.Structure):
     _fields_ = [("n", C.c_int), ("ff", C.c_int), ("nexp", C.c_int), ("topk", C.c_int), ("router", C.c_void_p),
-                ("gu", C.c_void_p), ("down", C.c_void_p), ("sh_gu", C.c_void_p), ("sh_down", C.c_void_p)]
+                ("gu", C.c_void_p), ("down", C.c_void_p), ("sh_gu", C.c_void_p), ("sh_down", C.c_void_p),
+                ("sh_gu_q", C.c_void_p), ("sh_gu_d", C.c_void_p), ("sh_down_q", C.c_void_p), ("sh_down_d", C.c_void_p)]
 
 
 JOB_DTYPE = np.dtype([("w", "<i4"), ("n", "<i4"), ("y", "<i4", (MAXT,)), ("out", "<i4", (MAXT,))])
@@ -336,11 +337,14 @@ class Oracle:
         return dict(out=out, logits=logits, topi=topi, topw=topw, njobs=nj.value)
 
     # ---- the layer
-    def moe_verify_layer(self, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, x, threads=8):
+    def moe_verify_layer(self, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, x, threads=8, sh_q8=None):
+        """sh_q8: the shared expert as split Q8_0 instead: ((q, d) of gate|up, (q, d) of down); sh_gu / sh_down may then be None"""
         router = np.ascontiguousarray(router, dtype=np.float32)
         x = np.ascontiguousarray(x, dtype=np.float32)
         T = x.shape[0]
         L = MoeLayer(n, ff, nexp, topk, ptr(router), ptr(gu), ptr(down), ptr(sh_gu), ptr(sh_down))
+        if sh_q8 is not None:
+            L.sh_gu_q, L.sh_gu_d, L.sh_down_q, L.sh_down_d = ptr(sh_q8[0][0]), ptr(sh_q8[0][1]), ptr(sh_q8[1][0]), ptr(sh_q8[1][1])
         out = np.zeros((T, n), dtype=np.float32)
         logits = np.zeros((T, nexp + 1), dtype=np.float32)
         topi = np.zeros((T, topk), dtype=np.int32)

@@ -140,3 +140,57 @@ def test_layer_with_other_expert_types_from_gguf(dev, oracle, tmp_path):
     want = oracle.moe_combine(part[:P], topw, part[P:], logits[:, nexp])
     assert np.array_equal(w["topi"].cpu().numpy(), topi)
     assert rel_l2(out.cpu().numpy(), want) <= 1e-3
+
+
+def test_layer_with_a_q8_0_shared_expert_from_gguf(dev, oracle, tmp_path):
+    """IQ3_S routed experts and a Q8_0 shared expert, the reference's own layer form (engine.cu:1600-1604): the loader
+    re-lays the experts to unit64 and the shared expert's raw Q8_0 blocks to the split layout, and the window runs in
+    its three launches plus the shared expert's dense ones."""
+    import qtype_blocks as qb
+    t, lib, pkg = dev.torch, dev.lib, dev.pkg
+    rng = np.random.default_rng(93)
+    n, ff, nexp, topk, T, layer = 2048, 512, 24, 10, 16, 3
+    ts, a = gf.moe_layer_tensors(rng, layer, n, ff, nexp, fnx_gpu.random_iq3s)
+    nbk = lambda rows, cols: rows * cols // 32
+    sgate, sup, sdown = (qb.random_blocks(rng, qb.Q8_0, nbk(r, c)) for r, c in ((ff, n), (ff, n), (n, ff)))
+    b = f"blk.{layer}."
+    ts = ts[:5] + [(b + "ffn_gate_shexp.weight", qb.Q8_0, [n, ff], sgate), (b + "ffn_up_shexp.weight", qb.Q8_0, [n, ff], sup),
+                   (b + "ffn_down_shexp.weight", qb.Q8_0, [ff, n], sdown)]
+    path = gf.write(tmp_path / "q8shared.gguf", ts)
+    print("case gguf layer with IQ3_S experts and a Q8_0 shared expert", flush=True)
+    g = lib.fnx_gguf_open(path.encode())
+    assert g, lib.fnx_last_error()
+    z = pkg.MoeBufs()
+    dev.ok(lib.fnx_gguf_moe_layer_bytes(g, layer, 0, ff, C.byref(z)))
+    bufs = [dev.zeros(getattr(z, k + "_bytes"), t.uint8) for k in ("router", "gu", "down", "sh_gu", "sh_down")]
+    for k, bf in zip(("router", "gu", "down", "sh_gu", "sh_down"), bufs):
+        setattr(z, k, bf.data_ptr())
+    L = pkg.MoeLayer()
+    dev.ok(lib.fnx_gguf_load_moe_layer(g, layer, 0, ff, topk, C.byref(z), C.byref(L), dev.st()))
+    dev.sync()
+    lib.fnx_gguf_close(g)
+    assert (L.gu.type, L.down.type) == (pkg.T_IQ3S_UNIT64, pkg.T_IQ3S_UNIT64)
+    assert L.sh_gu_q8.q == bufs[3].data_ptr() and (L.sh_gu_q8.n_out, L.sh_gu_q8.n_in, L.sh_down_q8.n_out, L.sh_down_q8.n_in) == (2 * ff, n, n, ff)
+
+    def split(raw, rows, cols):   # raw Q8_0 blocks (f16 d, 32 int8) -> the split arrays
+        blk = raw.reshape(rows, cols // 32, 34)
+        return np.ascontiguousarray(blk[:, :, 2:]).view(np.int8).reshape(rows, cols), np.ascontiguousarray(blk[:, :, :2]).view(np.uint16).reshape(rows, cols // 32)
+
+    sh_q8 = (split(np.concatenate([sgate, sup]), 2 * ff, n), split(sdown, n, ff))
+    got_q = bufs[3].cpu().numpy()
+    assert np.array_equal(got_q[:2 * ff * n].view(np.int8).reshape(2 * ff, n), sh_q8[0][0]), "the split layout on the device: the values"
+    assert np.array_equal(got_q[2 * ff * n:].view(np.uint16).reshape(2 * ff, n // 32), sh_q8[0][1]), "then the scales"
+    gu = gf.slice_rows2(a["gate"], a["up"], n, ff, nexp, 0, ff)
+    router = np.concatenate([a["router"], a["sh_router"]])
+    x = rng.standard_normal((T, n)).astype(np.float32)
+    want = oracle.moe_verify_layer(n, ff, nexp, topk, router, gu, a["down"], None, None, x, sh_q8=sh_q8)
+    P = T * topk
+    w = dict(xq=dev.zeros(T * (n // 32) * 36, t.uint8), logits=dev.zeros((T, nexp + 1), t.float32), topi=dev.zeros((T, topk), t.int32),
+             topw=dev.zeros((T, topk), t.float32), jobs_gu=dev.zeros((P + 1) * 136, t.uint8), jobs_dn=dev.zeros((P + 1) * 136, t.uint8),
+             njobs=dev.zeros(2, t.int32), gu=dev.zeros((P + T, 2 * ff), t.float32), part=dev.zeros((P + T, n), t.float32))
+    ws = pkg.MoeWs(*(w[k].data_ptr() for k in ("xq", "logits", "topi", "topw", "jobs_gu", "jobs_dn", "njobs", "gu", "part")))
+    dx, out = dev.up(x), dev.zeros((T, n), t.float32)
+    dev.ok(lib.fnx_moe_verify_layer(C.byref(L), dx.data_ptr(), T, out.data_ptr(), C.byref(ws), dev.st()))
+    dev.sync()
+    assert np.array_equal(w["topi"].cpu().numpy(), want["topi"]) and int(w["njobs"][0].item()) == want["njobs"]
+    assert rel_l2(out.cpu().numpy(), want["out"]) <= 1e-3

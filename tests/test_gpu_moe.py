@@ -82,6 +82,38 @@ def test_moe_verify_layer_shapes(dev, oracle, n, ff, nexp, topk, T, packed):
     check_layer(dev, oracle, n, ff, nexp, topk, T, 910 + T, packed)
 
 
+def q8_split(oracle, rng, rows, cols, scale):
+    import oracle_lib as ol
+    w = (rng.standard_normal((rows, cols)) * scale).astype(np.float32)
+    q, d = np.zeros((rows, cols), dtype=np.int8), np.zeros((rows, cols // 32), dtype=np.uint16)
+    oracle.lib.fnx_o_quantize_q8_0_split(ol.ptr(w), rows, cols, ol.ptr(q), ol.ptr(d))
+    return q, d
+
+
+@pytest.mark.parametrize("packed", [False, True])
+@pytest.mark.parametrize("n,ff,nexp,topk,T", [(2048, 512, 512, 10, 16), (2048, 512, 64, 1, 3), (2048, 256, 24, 4, 7)])
+def test_moe_verify_layer_with_a_q8_0_shared_expert(dev, oracle, n, ff, nexp, topk, T, packed):
+    """the reference's own form of the shared expert (engine.cu:1600-1604: split Q8_0 through q8s_gemv ->
+    swiglu_stacked_q8_1 -> q8s_gemv) beside IQ3_S routed experts: with unit64 experts inside the three-launch window,
+    with raw blocks operator by operator"""
+    print(f"case moe layer q8_0 shared n={n} ff={ff} nexp={nexp} topk={topk} T={T} packed={packed}", flush=True)
+    rng = np.random.default_rng(940 + T)
+    router, gu, down, sh_gu, sh_down = make_layer(rng, n, ff, nexp)
+    sh_q8 = (q8_split(oracle, rng, 2 * ff, n, 0.02), q8_split(oracle, rng, n, ff, 0.02))
+    layer = fnx_gpu.MoeLayerDev(dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, packed=packed, sh_q8=sh_q8)
+    for rows in (T, max(1, T // 2)):   # a second, shorter window on the same workspace
+        x = rng.standard_normal((rows, n)).astype(np.float32)
+        want = oracle.moe_verify_layer(n, ff, nexp, topk, router, gu, down, None, None, x, sh_q8=sh_q8)
+        with_iq3s = oracle.moe_verify_layer(n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, x)
+        assert rel_l2(want["out"], with_iq3s["out"]) > 1e-2, "the two shared experts differ, so the test tells them apart"
+        got = layer.run(x)
+        assert np.array_equal(got["logits"].view(np.uint32), want["logits"].view(np.uint32))
+        assert np.array_equal(got["topi"], want["topi"]) and got["njobs"] == want["njobs"]
+        err = rel_l2(got["out"], want["out"])
+        print("rel l2", err, flush=True)
+        assert err <= 1e-3
+
+
 def test_moe_verify_layer_repeated_windows(dev, oracle):
     # many windows back to back on one layer and workspace, varying T
     rng = np.random.default_rng(930)

@@ -52,7 +52,7 @@ def iq3s_matrix(oracle, blocks, rows, cols):
 
 
 # ---------------------------------------------------------------- the MoE verify layer
-def np_moe_layer(oracle, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, x, wrong=None):
+def np_moe_layer(oracle, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, x, wrong=None, sh_q8=None):
     T = x.shape[0]
     logits = oracle.gemv_f32(router, x)
     topi, topw = oracle.topk_logits(logits, nexp, topk)
@@ -73,7 +73,10 @@ def np_moe_layer(oracle, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, x,
                                               iq3s_matrix(oracle, down[e * ds:(e + 1) * ds], n, ff), xv[t])
         if wrong != "no_shared":
             gate = 1 / (1 + np.exp(-float(logits[t, nexp]))) if wrong != "shared_ungated" else 1.0
-            out[t] += gate * ffn(iq3s_matrix(oracle, sh_gu, 2 * ff, n), iq3s_matrix(oracle, sh_down, n, ff), xv[t])
+            if sh_q8 is not None:
+                out[t] += gate * ffn(q8s_values(sh_q8[0]), q8s_values(sh_q8[1]), xv[t])
+            else:
+                out[t] += gate * ffn(iq3s_matrix(oracle, sh_gu, 2 * ff, n), iq3s_matrix(oracle, sh_down, n, ff), xv[t])
     return out, logits, topi, topw
 
 
@@ -97,6 +100,30 @@ def test_moe_verify_layer_equals_its_parts(oracle):
     assert r["njobs"] == len(np.unique(topi))
     for wrong in ("gate_up", "no_shared", "shared_ungated"):
         bad = np_moe_layer(oracle, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, x, wrong=wrong)[0]
+        assert rel(r["out"], bad) >= MISS, wrong
+
+
+def test_moe_verify_layer_with_a_q8_0_shared_expert(oracle):
+    # engine.cu:1600-1604: the shared expert as dense split Q8_0 (q8s_gemv -> swiglu_stacked_q8_1 -> q8s_gemv)
+    rng = np.random.default_rng(22)
+    n, ff, nexp, topk, T = 256, 256, 8, 3, 5
+    nb = lambda rows, cols: rows * cols // 256
+    gu, down = random_iq3s(rng, nexp * nb(2 * ff, n), dmax=2e-2), random_iq3s(rng, nexp * nb(n, ff), dmax=2e-2)
+
+    def q8(rows, cols):
+        w = (rng.standard_normal((rows, cols)) * 2.0).astype(np.float32)
+        q, d = np.zeros((rows, cols), dtype=np.int8), np.zeros((rows, cols // 32), dtype=np.uint16)
+        oracle.lib.fnx_o_quantize_q8_0_split(ol.ptr(w), rows, cols, ol.ptr(q), ol.ptr(d))
+        return q, d
+
+    sh_q8 = (q8(2 * ff, n), q8(n, ff))
+    router = (rng.standard_normal((nexp + 1, n)) * 0.05).astype(np.float32)
+    x = rng.standard_normal((T, n)).astype(np.float32)
+    r = oracle.moe_verify_layer(n, ff, nexp, topk, router, gu, down, None, None, x, sh_q8=sh_q8)
+    want = np_moe_layer(oracle, n, ff, nexp, topk, router, gu, down, None, None, x, sh_q8=sh_q8)[0]
+    assert rel(r["out"], want) <= TOL
+    for wrong in ("gate_up", "no_shared", "shared_ungated"):
+        bad = np_moe_layer(oracle, n, ff, nexp, topk, router, gu, down, None, None, x, wrong=wrong, sh_q8=sh_q8)[0]
         assert rel(r["out"], bad) >= MISS, wrong
 
 
