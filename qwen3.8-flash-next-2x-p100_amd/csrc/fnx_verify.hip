@@ -13,6 +13,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <string>
 #include <type_traits>
 #include <vector>
@@ -698,6 +699,46 @@ static int cu_count() {
     }
     return cus[dev];
 }
+// The library's own device buffers that one call's kernels write and then read (the pair buffer of q8_1 rows behind
+// moe_down and the operator-by-operator window, the sampler's candidate lists): one per device, as the reference's
+// (moe.cuh:592-594), so calls that use one must not overlap. Calls on different streams are put in order here: a call
+// waits for the event the call before it recorded, and records its own when its launches are enqueued. A stream under
+// graph capture is left alone (waiting for an event from outside would end the capture): a captured graph that holds such
+// calls must not be replayed beside other users of the buffer.
+struct BufferOrder {
+    std::mutex m;
+    hipEvent_t ev[64] = {};
+    hipStream_t last[64] = {};
+    bool used[64] = {};
+    static bool capturing(hipStream_t s) {
+        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+        return hipStreamIsCapturing(s, &cs) == hipSuccess && cs != hipStreamCaptureStatusNone;
+    }
+    void enter(hipStream_t s) {
+        int dev = -1;
+        if (capturing(s) || hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return;
+        std::lock_guard<std::mutex> g(m);
+        if (used[dev] && last[dev] != s) (void) hipStreamWaitEvent(s, ev[dev], 0);
+    }
+    void leave(hipStream_t s) {
+        int dev = -1;
+        if (capturing(s) || hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return;
+        std::lock_guard<std::mutex> g(m);
+        if (!ev[dev] && hipEventCreateWithFlags(&ev[dev], hipEventDisableTiming) != hipSuccess) return;
+        if (hipEventRecord(ev[dev], s) == hipSuccess) {
+            used[dev] = true;
+            last[dev] = s;
+        }
+    }
+};
+static BufferOrder g_pair_order, g_cand_order;
+struct BufferScope {   // enter now, leave when the call returns
+    BufferOrder& o;
+    hipStream_t s;
+    BufferScope(BufferOrder& o_, void* st) : o(o_), s((hipStream_t) st) { o.enter(s); }
+    ~BufferScope() { o.leave(s); }
+};
+
 // wide: the jobs are expected to hold many rows each (a dense matrix over the whole window) rather than one or two
 static int rows_launch(const fnx_dw* W, size_t w_stride, const fnx_job* jobs, const int* njobs, int njobs_max, const void* y, float* out,
                        int out_stride, void* st, const char* who, bool wide = false) {
@@ -928,6 +969,7 @@ int fnx_moe_down(const fnx_dw* A, size_t sa, const fnx_job* jobs, const int* njo
     if (ffs <= 0 || ffs % 32 || ffs > HQ_MAX_FF) return fail("moe_down: expert width does not fit the pair buffer");
     if (njobs_max < 1 || njobs_max > HQ_ROWS) return fail("moe_down: more pairs than the pair buffer holds");
     // every pair's h once (moe.cuh:597-608), then the rows against it
+    BufferScope pair_buffer(g_pair_order, st);
     k_swiglu_q8_1<<<dim3((ffs / 32 + 7) / 8, njobs_max), 256, 0, (hipStream_t) st>>>(gu, gu + ffs, (size_t) 2 * ffs, nullptr, ffs);
     if (launch_status("moe_down")) return 1;
     return rows_launch(A, sa, jobs, njobs, njobs_max, nullptr, part, A->n_out, st, "moe_down");
@@ -1031,6 +1073,7 @@ static int moe_layer_checked(const fnx_moe_layer* L, const float* x, int T, floa
     if (live && !layer_fused_ok(L, T)) return fail("moe_verify_layer: a device-side row count needs the three-launch window");
     if (layer_fused_ok(L, T)) return layer_fused(L, x, T, out, ws, st, live);
     hipStream_t s = (hipStream_t) st;
+    BufferScope pair_buffer(g_pair_order, st);   // operator by operator the pairs' q8_1 rows go through the library's buffer
     if (fnx_quantize_q8_1(x, ws->xq, n, T, st)) return 1;
     if (gemv_any(L->router, L->router_bf16 != 0, x, ws->logits, L->nexp + 1, n, T, st, "moe_verify_layer router")) return 1;
     k_topk_jobs<<<1, TK_THREADS, 0, s>>>(ws->logits, L->nexp + 1, T, L->nexp, L->topk, ws->topi, ws->topw, ws->jobs_gu, ws->jobs_dn, ws->njobs,
@@ -1242,7 +1285,7 @@ int fnx_moe_prefill_layer(const fnx_moe_layer* L, const float* x, int C, float* 
         !ws->h16 || !ws->part)
         return fail("moe_prefill_layer: incomplete workspace");
     const int n = L->n, ff = L->ff, nexp = L->nexp, topk = L->topk;
-    if (C < 1 || C > 65536) return fail("moe_prefill_layer: 1..65536 rows a chunk");
+    if (C < 1 || C > 65535) return fail("moe_prefill_layer: 1..65535 rows a chunk (the combine takes a grid row per chunk row)");
     if (L->gu.n_in != n || L->gu.n_out != 2 * ff || L->down.n_in != ff || L->down.n_out != n || L->sh_gu.n_in != n ||
         L->sh_gu.n_out != 2 * ff || L->sh_down.n_in != ff || L->sh_down.n_out != n)
         return fail("moe_prefill_layer: weight shapes do not match n / ff");
@@ -1548,6 +1591,7 @@ int fnx_top_tokens(float* logits, int n, int T, int v0, const int* pen_tok, cons
         return fail("top_tokens: a list's count without the list");
     const int nslice = (n + SM_SLICE - 1) / SM_SLICE;
     hipStream_t s = (hipStream_t) st;
+    BufferScope candidates(g_cand_order, st);
     k_top_slices<<<dim3(nslice, T), SM_THREADS, 0, s>>>(
         TopArgs{logits, n, v0, nslice, pen_tok, pen_cnt, pen_n, pen_stride, pen_par, bias_tok, bias_val, bias_off, bias_n, err});
     k_top_merge<<<T, SM_MERGE_THREADS, 0, s>>>(logits, n, v0, nslice, out_v, out_i);

@@ -114,6 +114,37 @@ def test_moe_verify_layer_with_a_q8_0_shared_expert(dev, oracle, n, ff, nexp, to
         assert err <= 1e-3
 
 
+@pytest.mark.parametrize("packed", [False, True])
+def test_two_windows_on_two_streams(dev, oracle, packed):
+    """two layers, each with a workspace of its own, their windows enqueued on two streams with nothing between them: the
+    results are the single-stream ones. With unit64 weights a window touches only its workspace; operator by operator
+    the pairs' q8_1 rows go through the library's one buffer per device, and the library puts the calls in order."""
+    import ctypes as C
+    t = dev.torch
+    n, ff, nexp, topk, T = 2048, 512, 48, 10, 16
+    rng = np.random.default_rng(950)
+    layers, xs, want = [], [], []
+    for i in range(2):
+        router, gu, down, sh_gu, sh_down = make_layer(rng, n, ff, nexp)
+        layers.append(fnx_gpu.MoeLayerDev(dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, packed=packed))
+        xs.append([rng.standard_normal((T, n)).astype(np.float32) for _ in range(6)])
+        want.append([layers[i].run(x)["out"] for x in xs[i]])   # one at a time, each waited for
+    streams = [t.cuda.Stream(), t.cuda.Stream()]
+    dxs = [[dev.up(x) for x in xs[i]] for i in range(2)]
+    outs = [[dev.zeros((T, n), t.float32) for _ in xs[i]] for i in range(2)]
+    dev.sync()
+    print(f"case two streams packed={packed}", flush=True)
+    for j in range(6):
+        for i in range(2):
+            with t.cuda.stream(streams[i]):
+                dev.ok(dev.lib.fnx_moe_verify_layer(C.byref(layers[i].L), dxs[i][j].data_ptr(), T, outs[i][j].data_ptr(), C.byref(layers[i].ws), dev.st()))
+    for s_ in streams:
+        s_.synchronize()
+    for i in range(2):
+        for j in range(6):
+            assert np.array_equal(outs[i][j].cpu().numpy().view(np.uint32), want[i][j].view(np.uint32)), (i, j)
+
+
 def test_moe_verify_layer_repeated_windows(dev, oracle):
     # many windows back to back on one layer and workspace, varying T
     rng = np.random.default_rng(930)
