@@ -445,6 +445,7 @@ __global__ void __launch_bounds__(512) k_iq3s_jobs(const RowsArgs a) {
 }
 
 }  // namespace fnx
+#include "k_iq3s_mma.h"
 #include "k_moe_layer.h"
 #include "k_prefill.h"
 #include "k_decoder.h"
@@ -796,7 +797,12 @@ static int rows_launch(const fnx_dw* W, size_t w_stride, const fnx_job* jobs, co
         else if (sbr == 16) FNX_ROWS(16, WIDE_, PACKED_);                                                \
         else FNX_ROWS(8, WIDE_, PACKED_);                                                                \
     } while (0)
-    if (!whole_units) k_iq3s_jobs_any<<<dim3((W->n_out + 3) / 4, njobs_max), 256, 0, s>>>(a);
+    // rows of 2048 columns in whole groups of 16: jobs of five rows and more go to the matrix cores, decoded once (k_iq3s_mma.h)
+    static const int jobs_mma = env_int("FNX_JOBS_MMA", 1, 0, 1);
+    if (packed && jobs_mma && sbr == 64 && W->n_out % JM_ROWS == 0) {
+        const long items = (long) njobs_max * (W->n_out / JM_ROWS);
+        k_iq3s_jobs_mma<<<(int) std::max(1L, std::min((long) (blocks ? blocks : cu_count()), items)), JM_THREADS, 0, s>>>(a);
+    } else if (!whole_units) k_iq3s_jobs_any<<<dim3((W->n_out + 3) / 4, njobs_max), 256, 0, s>>>(a);
     else if (packed && wide) FNX_ROWS_SBR(true, true);
     else if (packed) FNX_ROWS_SBR(false, true);
     else if (wide) FNX_ROWS_SBR(true, false);
