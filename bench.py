@@ -26,7 +26,9 @@ HBM_PEAK = 8.0e12
 # HBM bytes of one gate|up launch of the default run (gaussian weights, 16 sets, unit64), measured by two rocprofv3 --pmc
 # runs of this file (FETCH_SIZE, then WRITE_SIZE, each scaled by a 256 MiB copy: profiles/moe_gate_up_hbm_traffic.md), and
 # the distinct experts per step they were measured at. Not measured in the run: emitted only for that configuration.
-GATE_UP_TRAFFIC = {"bytes": None, "distinct_experts_per_step": None, "source": "profiles/moe_gate_up_hbm_traffic.md"}
+GATE_UP_TRAFFIC = {"bytes": 137.08e6, "algorithmic_bytes": 125.83e6, "distinct_experts_per_step": 138.45,
+                   "source": "profiles/moe_gate_up_hbm_traffic.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this file's default workload; scaled to "
+                             "this run's algorithmic bytes; not measured in this run)"}
 IQ3S_BLOCK = 110
 GU_BYTES = 2 * FF * (N // 256) * IQ3S_BLOCK      # 901,120 per expert
 DN_BYTES = N * (FF // 256) * IQ3S_BLOCK          # 450,560 per expert
@@ -303,8 +305,8 @@ def main():
             torch.cuda.empty_cache()
         gemv = gemv_measure(dev, torch, np, 512)
     traffic = None
-    if fused and args.weights == "gaussian" and GATE_UP_TRAFFIC["bytes"] and abs(u_mean - GATE_UP_TRAFFIC["distinct_experts_per_step"]) < 0.5:
-        traffic = GATE_UP_TRAFFIC["bytes"]
+    if fused and not args.shared_q8 and GATE_UP_TRAFFIC["bytes"] and abs(u_mean - GATE_UP_TRAFFIC["distinct_experts_per_step"]) < 3:
+        traffic = GATE_UP_TRAFFIC["bytes"] * k_bytes / GATE_UP_TRAFFIC["algorithmic_bytes"]
 
     # ---- CPU baseline: the oracle on the host's cores, same workload (layer set 0), bounded sample
     cpu = None
