@@ -8,8 +8,10 @@ A step = one MoE layer of a verify window: T = 16 rows, hidden 2048, 512 IQ3_S e
 Steps cycle through LAYERS distinct weight sets (about 11 GB) and fresh activations so that a step's ~190 MB working set
 is cold with respect to the 256 MB Infinity Cache.
 
-Prints ONE JSON line: whole-step throughput, the roofline of the dominant kernel (the routed gate|up mat-vec, timed on
-its own with events on the launch stream) and the CPU baseline (the oracle on the host's cores, bounded sample).
+Prints ONE JSON line: whole-step throughput, the roofline of the dominant kernel (the window's gate|up launch, timed
+with events on the launch stream), what a read-only kernel reaches on the same GPU (roofline.stream_read_GBps), config 1
+(config.gemv), and the CPU baseline (the oracle on the host's cores, bounded sample). The experts are IQ3_S blocks encoded
+from N(0, 0.02) weights (--weights bytes: uniformly random blocks).
 """
 import argparse
 import ctypes as C

@@ -59,7 +59,7 @@ typedef struct fnx_dw {
                              * operators (fnx_mmvq, fnx_moe_gate_up, fnx_moe_down, and fnx_moe_verify_layer operator by
                              * operator) also take ggml's Q4_0 (2), Q5_1 (7), Q8_0 (8), Q4_K (12), Q5_K (13), IQ4_NL (20) and IQ4_XS (23) rows, the
                              * other types of kernels.cu:2454-2471 that the reference's host code can decode; the
-                             * prompt path's grouped GEMM and the five-launch window are IQ3_S only */
+                             * prompt path's grouped GEMM and the three-launch window are IQ3_S only */
     int n_in, n_out;        /* columns, rows */
     size_t row_bytes;       /* n_in / 256 * 110 for IQ3_S; whole blocks of the type otherwise */
     const void* const* ep;  /* optional device table: expert e's matrix; null: expert e at p + e * stride */
@@ -141,10 +141,13 @@ int fnx_accept_greedy_dev(const int* rows, const int* o, int R, int* n_accept, v
 
 /* ---- the whole MoE half of a verify window (engine.cu:1569-1757 Engine::ffn_half without cards and streaming):
  * quantize -> router_route -> gate|up (routed + shared) -> swiglu q8_1 -> down (routed + shared) -> combine.
- * Same results as the calls above made one by one (up to the order of a few float additions). With unit64 weights,
- * n = 2048 and ff of 256, 512 or 1024 the window runs in five launches: [router logits | q8_1 rows], [top-k],
- * [jobs + gate|up routed + shared], [SwiGLU + down routed + shared], [combine]; other shapes run operator by operator.
- * Like moe_down, one MoE may be in flight per device. */
+ * Same results as the calls above made one by one (up to the order of a few float additions). With unit64 experts,
+ * n = 2048 and ff of 256, 512 or 1024 the window runs in three launches: [router logits | q8_1 rows], [top-k + gate|up
+ * routed + shared + SwiGLU -> q8_1 rows of h], [down routed + shared + the combine's chains; the job lists for the
+ * caller]; these touch only the caller's workspace, so windows with workspaces of their own may run on different streams
+ * at once. Other shapes run operator by operator through the library's one pair buffer per device, like moe_down: the
+ * library puts such calls in order across streams (not under graph capture). A row with fewer than topk finite logits
+ * takes the lowest experts not yet taken for its remaining picks (the reference's result is undefined there). */
 /* model.hpp:78-82  Q8S: dense Q8_0 in the split layout: int8 values [n_out][n_in], f16 scale bits [n_out][n_in / 32] */
 typedef struct fnx_q8s {
     const int8_t* q;
@@ -175,8 +178,10 @@ typedef struct fnx_moe_ws {
     fnx_job* jobs_gu;/* [T * topk + 1] (the last one is the shared expert's) */
     fnx_job* jobs_dn;/* [T * topk + 1] */
     int* njobs;      /* [2], zeroed once */
-    float* gu;       /* [T * topk + T][2 ff] */
-    float* part;     /* [T * topk + T][n] */
+    float* gu;       /* [T * topk + T][2 ff] floats. Operator by operator: the gate|up outputs. The three-launch window keeps
+                      * the pairs' h there instead, as q8_1 rows of its own record size, and never writes f32 gate|up rows */
+    float* part;     /* [T * topk + T][n] floats. Operator by operator: the down outputs. The three-launch window uses it only
+                      * as scratch for a split-Q8_0 shared expert */
 } fnx_moe_ws;
 int fnx_moe_verify_layer(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st);
 /* The same window without a workspace argument and without any allocation: no counterpart in the reference. For callers
@@ -189,20 +194,23 @@ int fnx_moe_verify_layer(const fnx_moe_layer* L, const float* x, int T, float* o
 #define FNX_MOE_STATIC_WS_BYTES (448 * 1024)
 int fnx_moe_verify_layer_static(const fnx_moe_layer* L, const float* x, int T, float* out, void* st);
 /* Profiling aid, the counterpart of the reference's FNX_PROF stamps in its window graph (engine.cu:1382-1530):
- * fnx_layer_profile(1) makes the five-launch window record events on its stream around each launch (not to be
+ * fnx_layer_profile(1) makes the three-launch window record events on its stream around each launch (not to be
  * used under graph capture), fnx_layer_profile(0) stops that; fnx_layer_profile_read waits for the last recorded
- * window and returns its five launches' durations in milliseconds: router + q8_1 rows, top-k, jobs + gate|up,
- * down, combine. One profiled window at a time per process. */
+ * window and returns its three launches' durations in milliseconds: router + q8_1 rows (with a split-Q8_0 shared
+ * expert: and its three dense launches), top-k + gate|up + SwiGLU, down + combine. One profiled window at a time per
+ * process. */
 int fnx_layer_profile(int on);
-int fnx_layer_profile_read(float* ms5);
+int fnx_layer_profile_read(float* ms3);
 /* Calibration aid (no counterpart in the reference): one read-only pass over `bytes` of device memory, nothing decoded,
  * so that the expert mat-vec launches can be judged against what the memory system gives a plain read of the same shape.
  * variant: 0 / 1 / 7 / 8: 16-byte loads a lane, 4 / 8 / 16 / 2 in flight, every wave one contiguous range; 2 / 3: the same 4 / 8
  * with the 1 KiB chunks dealt round-robin to the waves; 4: 8-byte loads, 8 in flight; 5: as 1 with nontemporal loads;
- * 6: the unit64 planes as the pass kernels load them (five loads a unit and lane, a group of four units in flight), every
+ * 6: the unit64 planes as the expert kernels load them (five loads a unit and lane, a group of four units in flight), every
  * wave one contiguous range; 9: the groups dealt round-robin to the grid's waves; 10: every block one contiguous range,
- * its waves taking the groups in turn; 11 / 12 / 13: as 6 / 9 / 10 with nontemporal loads. sink: one device word (never
- * written in practice; it keeps the loads alive). */
+ * its waves taking the groups in turn; 11 / 12 / 13: as 6 / 9 / 10 with nontemporal loads; 1000 s + K (s = 1 .. 8, K = 1 .. 64
+ * dividing 64 s): the buffer as matrices of 256 s units (s = 4: a gate|up matrix of the benchmark's shape, 2: a down matrix)
+ * read in a shuffled order, a wave staying with a matrix for K trips of four units. sink: one device word (never written in
+ * practice; it keeps the loads alive). */
 int fnx_stream_read(const void* p, size_t bytes, int variant, int blocks, int threads, void* sink, void* st);
 
 /* ---- the prompt path's MoE over a chunk of C rows (prefill.cu:1990-2083) */
@@ -362,7 +370,7 @@ typedef struct fnx_round {
     float* chain_src; /* device, n floats (the hidden row the chain starts from); may be null when chain <= 1 */
 } fnx_round;
 /* one round: fnx_decoder_verify over the window -> acceptance and commit -> fnx_mtp_draft over the rows kept -> lookup
- * -> the next window. Expert weights must be in the unit64 layout and hidden = 2048 (the five-launch window), since only
+ * -> the next window. Expert weights must be in the unit64 layout and hidden = 2048 (the three-launch window), since only
  * that routes a row count held on the device. The draft layer uses the same workspace after the verify. */
 int fnx_decode_round(const fnx_decoder* D, const fnx_mtp* M, const fnx_round* R, const fnx_dec_ws* ws, void* st);
 

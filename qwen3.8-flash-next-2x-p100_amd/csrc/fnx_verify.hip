@@ -797,7 +797,7 @@ static int rows_launch(const fnx_dw* W, size_t w_stride, const fnx_job* jobs, co
         else if (sbr == 16) FNX_ROWS(16, WIDE_, PACKED_);                                                \
         else FNX_ROWS(8, WIDE_, PACKED_);                                                                \
     } while (0)
-    // rows of 2048 columns in whole groups of 16: jobs of five rows and more go to the matrix cores, decoded once (k_iq3s_mma.h)
+    // rows of 2048 columns in whole groups of 16: jobs of two rows and more go to the matrix cores, decoded once (k_iq3s_mma.h)
     static const int jobs_mma = env_int("FNX_JOBS_MMA", 1, 0, 1);
     if (packed && jobs_mma && sbr == 64 && W->n_out % JM_ROWS == 0) {
         const long items = (long) njobs_max * (W->n_out / JM_ROWS);

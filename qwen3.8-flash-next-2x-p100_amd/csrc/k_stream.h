@@ -14,7 +14,7 @@ typedef __attribute__((address_space(1))) const v2u g64v;
 __device__ __forceinline__ size_t stream_share(size_t total, uint32_t gw, uint32_t nw) { return (size_t) ((unsigned __int128) total * gw / nw); }
 
 // VB: bytes a lane and load (8 or 16). DEPTH: loads a lane has in flight. NT: nontemporal loads. RANGE: a wave reads one
-// contiguous range (as the pass kernels do); else chunk c goes to wave c mod the grid's waves.
+// contiguous range (as the job kernels do); else chunk c goes to wave c mod the grid's waves.
 template <int VB, int DEPTH, bool NT, bool RANGE>
 __global__ void __launch_bounds__(1024) k_stream_read(const uint8_t* __restrict__ p, size_t chunks, uint32_t* __restrict__ sink) {
     const uint32_t lane = threadIdx.x & 63, wpb = blockDim.x >> 6;
@@ -62,7 +62,7 @@ __global__ void __launch_bounds__(1024) k_stream_read(const uint8_t* __restrict_
     if (acc == 0x9E3779B9u) sink[0] = acc;   // keeps the loads alive; practically never taken
 }
 
-// the unit64 planes as the pass kernels ask for them: five loads a unit and lane, four units (a group) in flight.
+// the unit64 planes as the expert kernels ask for them: five loads a unit and lane, four units (a group) in flight.
 // SPLIT 0: every wave one contiguous range of units; 1: group g goes to wave g mod the grid's waves; 2: every block one
 // contiguous range, its waves taking the range's groups in turn. NT: nontemporal loads.
 template <bool NT>
@@ -122,7 +122,7 @@ __global__ void __launch_bounds__(1024) k_stream_read_units(const uint8_t* __res
     if (acc == 0x9E3779B9u) sink[0] = acc;
 }
 
-// the pass kernels' case: segments of `seg_units` units (an expert's matrix) scattered over the buffer, walked in a
+// the window kernels' case: segments of `seg_units` units (an expert's matrix) scattered over the buffer, walked in a
 // fixed shuffled order; wave gw keeps to a segment for K trips of one group, so the grid reads waves * K * 4 / seg_units
 // segments at a time, each as one front that moves through the segment
 __global__ void __launch_bounds__(1024) k_stream_read_segments(const uint8_t* __restrict__ p, size_t units, uint32_t seg_units, uint32_t K,

@@ -38,7 +38,7 @@ def check_jobs(got, want):
 
 
 def check_layer(dev, oracle, n, ff, nexp, topk, T, seed, packed=False):
-    """packed: the unit64 layout (eligible shapes then run as the five-launch window)"""
+    """packed: the unit64 layout (eligible shapes then run as the three-launch window)"""
     print(f"case moe layer n={n} ff={ff} nexp={nexp} topk={topk} T={T} seed={seed} packed={packed}", flush=True)
     rng = np.random.default_rng(seed)
     router, gu, down, sh_gu, sh_down = make_layer(rng, n, ff, nexp)
@@ -78,7 +78,7 @@ def test_moe_verify_layer_config2(dev, oracle, packed):
 @pytest.mark.parametrize("n,ff,nexp,topk,T", [(2048, 512, 64, 10, 1), (1024, 256, 32, 4, 16), (2048, 1024, 16, 2, 3), (512, 512, 16, 8, 7),
                                               (2048, 256, 40, 6, 9), (2048, 512, 1000, 10, 16), (2048, 512, 12, 10, 16)])
 def test_moe_verify_layer_shapes(dev, oracle, n, ff, nexp, topk, T, packed):
-    # with unit64 weights the shapes of hidden 2048 run as the five-launch window, the others operator by operator
+    # with unit64 weights the shapes of hidden 2048 run as the three-launch window, the others operator by operator
     check_layer(dev, oracle, n, ff, nexp, topk, T, 910 + T, packed)
 
 
