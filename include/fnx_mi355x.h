@@ -29,6 +29,7 @@ extern "C" {
 #define FNX_PF_JOB 64      /* rows per prefill job (kernels.hpp:27-30) */
 #define FNX_T_IQ3_S 21u    /* ggml type id (gguf.hpp:22-27) */
 #define FNX_T_IQ3S_UNIT64 1021u /* this library's load-time re-laying of IQ3_S (fnx_iq3s_repack); not a ggml type */
+#define FNX_T_IQ3S_TILE16 1022u /* the prompt path's own re-laying of IQ3_S (fnx_iq3s_tile16); not a ggml type */
 #define FNX_IQ3S_BLOCK 110 /* bytes per 256 weights */
 #define FNX_Q8_1_BLOCK 36  /* bytes per 32 activations: half d, half sum, int8 qs[32] */
 #define FNX_ERR_NONFINITE 16u /* error-word bit (engine_impl.hpp:211-218) */
@@ -77,6 +78,15 @@ const char* fnx_version(void);
  * fnx_dw.type = FNX_T_IQ3S_UNIT64: every operator below takes both types and gives the same results; the re-laid
  * type is the fast path. Rows must have 256, 512, 1024 or 2048 columns and expert strides must be multiples of 880. */
 int fnx_iq3s_repack(const void* src, void* dst, size_t n_weights, void* st);
+/* A second load-time layout, for the prompt path's matrix-core kernels only (fnx_moe_gate_up_mma, fnx_moe_prefill_layer's
+ * gate|up; no counterpart in the reference, whose prompt kernels read raw blocks): nmat matrices of nrows x ncols
+ * (rows in 16s, columns in 512s) from the unit64 layout into tiles of 16 rows x 512 columns in which the 64 lanes of a
+ * wave find their shares side by side (3,584 bytes a tile: 1.8 % more than the blocks). src: the matrices one after the
+ * other in unit64 form; dst: another buffer of fnx_iq3s_tile16_bytes(nrows, ncols, nmat) bytes, expert e at
+ * e * fnx_iq3s_tile16_bytes(nrows, ncols, 1). A fnx_dw over dst has type FNX_T_IQ3S_TILE16 (row_bytes as for IQ3_S). A
+ * model served with both paths keeps both copies (288 GB hold them). */
+int fnx_iq3s_tile16(const void* src, void* dst, int nrows, int ncols, int nmat, void* st);
+size_t fnx_iq3s_tile16_bytes(int nrows, int ncols, int nmat);
 
 /* kernels.hpp:41  quantize_q8_1: f32 rows of n -> q8_1 blocks, ggml's rounding (kernels.cu:131-145) */
 int fnx_quantize_q8_1(const float* x, void* q, int n, int rows, void* st);

@@ -14,6 +14,7 @@ MAXT = 16
 PF_JOB = 64
 T_IQ3_S = 21
 T_IQ3S_UNIT64 = 1021
+T_IQ3S_TILE16 = 1022
 IQ3S_BLOCK = 110
 Q8_1_BLOCK = 36
 
@@ -101,6 +102,8 @@ EXPORTS = {
     "fnx_last_error": (C.c_char_p, []),
     "fnx_version": (C.c_char_p, []),
     "fnx_iq3s_repack": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "fnx_iq3s_tile16": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]),
+    "fnx_iq3s_tile16_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int]),
     "fnx_quantize_q8_1": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
     "fnx_mmvq": (C.c_int, [C.POINTER(DW), C.c_size_t, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]),
     "fnx_gemv_f32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]),
@@ -202,9 +205,9 @@ def check(status):
         raise FnxError(lib().fnx_last_error().decode())
 
 
-def dw(tensor_or_ptr, n_in, n_out, ep=None, packed=False):
+def dw(tensor_or_ptr, n_in, n_out, ep=None, packed=False, tile16=False):
     p = tensor_or_ptr if isinstance(tensor_or_ptr, int) or tensor_or_ptr is None else tensor_or_ptr.data_ptr()
-    return DW(p, T_IQ3S_UNIT64 if packed else T_IQ3_S, n_in, n_out, n_in // 256 * IQ3S_BLOCK, ep)
+    return DW(p, T_IQ3S_TILE16 if tile16 else T_IQ3S_UNIT64 if packed else T_IQ3_S, n_in, n_out, n_in // 256 * IQ3S_BLOCK, ep)
 
 
 def stream_ptr():

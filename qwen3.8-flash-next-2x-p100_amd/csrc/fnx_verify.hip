@@ -888,6 +888,18 @@ int fnx_iq3s_repack(const void* src, void* dst, size_t n_weights, void* st) {
     k_iq3s_repack<<<(unsigned) ((units + 3) / 4), 256, 0, (hipStream_t) st>>>((const uint8_t*) src, (uint8_t*) dst, units);
     return launch_status("iq3s_repack");
 }
+int fnx_iq3s_tile16(const void* src, void* dst, int nrows, int ncols, int nmat, void* st) {
+    if (!src || !dst || src == dst) return fail("iq3s_tile16: two distinct buffers");
+    if (nrows < 16 || nrows % 16 || ncols < 512 || ncols % 512 || nmat < 1) return fail("iq3s_tile16: matrices of rows in 16s and columns in 512s");
+    const long tiles = (long) nmat * (nrows / 16) * (ncols / 512);
+    if ((tiles + 3) / 4 > 0x7fffffffL) return fail("iq3s_tile16: too many tiles for one launch");
+    k_iq3s_tile16<<<(unsigned) ((tiles + 3) / 4), 256, 0, (hipStream_t) st>>>((const uint8_t*) src, (uint8_t*) dst, nrows, ncols, tiles);
+    return launch_status("iq3s_tile16");
+}
+size_t fnx_iq3s_tile16_bytes(int nrows, int ncols, int nmat) {
+    if (nrows < 16 || nrows % 16 || ncols < 512 || ncols % 512 || nmat < 1) return 0;
+    return (size_t) nmat * (nrows / 16) * (ncols / 512) * TILE16_BYTES;
+}
 int fnx_quantize_q8_1(const float* x, void* q, int n, int rows, void* st) {
     if (!x || !q) return fail("quantize_q8_1: null argument");
     if (n <= 0 || n % 32 || rows <= 0) return fail("quantize_q8_1: rows of whole 32-value blocks");
@@ -1228,7 +1240,8 @@ static int mma_launch(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const 
                       int cap2 = 0, uint16_t* h16 = nullptr, bool* h16_done = nullptr) {
     if (!A || !jobs || !njobs || !x || !out) return fail(std::string(who) + ": null argument");
     if (!A->p && !A->ep) return fail(std::string(who) + ": no weights");
-    if (A->type != FNX_T_IQ3_S && A->type != FNX_T_IQ3S_UNIT64) return fail(std::string(who) + ": IQ3_S weights only");
+    if (A->type != FNX_T_IQ3_S && A->type != FNX_T_IQ3S_UNIT64 && A->type != FNX_T_IQ3S_TILE16) return fail(std::string(who) + ": IQ3_S weights only");
+    if (A->type == FNX_T_IQ3S_TILE16 && (A->n_in % 512 || A->n_out % 16)) return fail(std::string(who) + ": the tile16 layout takes rows in 16s and columns in 512s");
     if (A->n_in < 256 || A->n_in % 256 || A->n_out < 32 || A->n_out % 32) return fail(std::string(who) + ": columns in 256s, rows in 32s");
     if (A->type == FNX_T_IQ3S_UNIT64 && ((size_t) A->n_out * A->n_in) % 2048) return fail(std::string(who) + ": whole units of 2048 weights");
     if (njobs_cap < 1) return fail(std::string(who) + ": no jobs");
@@ -1236,7 +1249,8 @@ static int mma_launch(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const 
     static const int per_cu = env_int("FNX_MMA_BLOCKS_PER_CU", 2, 1, 8), form = env_int("FNX_MMA_FORM", 1, 0, 1);
     static const int tile = env_int("FNX_MMA_TILE", 1, 0, 2);   // 0: never, 1: rows of up to 512 columns, 2: always
     const bool use_tile = tile && A->type == FNX_T_IQ3S_UNIT64 && A->n_out % 16 == 0 && (tile == 2 || A->n_in <= 512);
-    const bool use_block = !use_tile && form == 1 && A->type == FNX_T_IQ3S_UNIT64 && A->n_in % 512 == 0 && A->n_out % 16 == 0;
+    const bool tile16 = A->type == FNX_T_IQ3S_TILE16;
+    const bool use_block = tile16 || (!use_tile && form == 1 && A->type == FNX_T_IQ3S_UNIT64 && A->n_in % 512 == 0 && A->n_out % 16 == 0);
     const bool merged = A2 && (use_tile || use_block) && A2->p && A2->type == A->type && A2->n_in == A->n_in && A2->n_out == A->n_out;
     if (A2 && !merged) {   // a form without the second list: two launches
         if (mma_launch(A, sa, jobs, njobs, njobs_cap, x, out, st, who)) return 1;
@@ -1264,11 +1278,21 @@ static int mma_launch(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const 
         k_moe_mma_tile<<<grid, MM_THREADS, 0, (hipStream_t) st>>>(a);
         return launch_status(who);
     }
+    static const int tok64 = env_int("FNX_MMA_TOK64", 1, 0, 1);
+    if (use_block && tok64) {
+        // block form, a block per (job, its up to 64 tokens, 256 rows): one block a CU (its LDS)
+        const long tasks = caps * ((A->n_out + MB_ROWS - 1) / MB_ROWS);
+        const int grid = (int) std::max(1l, std::min<long>((long) cu_count(), tasks));
+        if (tile16) k_moe_mma_block64<true><<<grid, MM_THREADS, 0, (hipStream_t) st>>>(a);
+        else k_moe_mma_block64<false><<<grid, MM_THREADS, 0, (hipStream_t) st>>>(a);
+        return launch_status(who);
+    }
     if (use_block) {
         // block form: a block per (job, 32 tokens, 256 rows)
         const long tasks = caps * ((A->n_out + MB_ROWS - 1) / MB_ROWS) * (MM_TT / MM_TP);
         const int grid = (int) std::max(1l, std::min<long>((long) per_cu * cu_count(), tasks));
-        k_moe_mma_block<<<grid, MM_THREADS, 0, (hipStream_t) st>>>(a);
+        if (tile16) k_moe_mma_block<true><<<grid, MM_THREADS, 0, (hipStream_t) st>>>(a);
+        else k_moe_mma_block<false><<<grid, MM_THREADS, 0, (hipStream_t) st>>>(a);
         return launch_status(who);
     }
     const long tasks = (long) njobs_cap * (A->n_out / 32) * (MM_TT / MM_TP);

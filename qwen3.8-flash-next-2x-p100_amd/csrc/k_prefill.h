@@ -461,6 +461,47 @@ __device__ __forceinline__ SubFields super_sub(const SuperFields& f) {
     s.d = f.d;
     return s;
 }
+// The same fields from the prompt path's own layout ("tile16", FNX_T_IQ3S_TILE16): a matrix as tiles of 16 rows x 512
+// columns, tile (row / 16, column / 512) at ((row / 16) * (ncols / 512) + column / 512) * TILE16_BYTES, and in a tile the
+// 64 lanes' shares side by side, plane by plane: lane (row % 16) + 16 g holds sub-blocks 4 g .. 4 g + 3 of the tile's 16 -
+// A 32 bytes a lane, B 16, C 4, the scale nibbles 2, d 2. Every load of a wave is then one contiguous run (2 KiB, 1 KiB,
+// 256, 128, 128 bytes) and a wave's super-steps follow each other in memory, where the unit64 planes give the matrix
+// cores' lanes - sixteen different rows - a cache line each. 3,584 bytes per 8,192 weights (unit64: 3,520; d is held by
+// both lanes of a super-block).
+constexpr int TILE16_BYTES = 3584, TILE16_B_AT = 2048, TILE16_C_AT = 3072, TILE16_SC_AT = 3328, TILE16_D_AT = 3456;
+__device__ __forceinline__ SuperFields tile16_load(const uint8_t* __restrict__ we, int row, int S, int nsuper) {   // row: the lane's row
+    typedef __attribute__((address_space(1))) const v4u g128;
+    typedef __attribute__((address_space(1))) const uint32_t g32;
+    typedef __attribute__((address_space(1))) const unsigned short g16;
+    const int lane = (row & 15) | (int) (threadIdx.x & 48u);
+    const gbytes u = as_global(we + ((size_t) (row >> 4) * nsuper + S) * TILE16_BYTES);
+    SuperFields r;
+    r.a0 = *(g128*) (u + 32 * lane);
+    r.a1 = *(g128*) (u + 32 * lane + 16);
+    r.b = *(g128*) (u + TILE16_B_AT + 16 * lane);
+    r.c = *(g32*) (u + TILE16_C_AT + 4 * lane);
+    r.sc = *(g16*) (u + TILE16_SC_AT + 2 * lane);
+    r.d = *(g16*) (u + TILE16_D_AT + 2 * lane);
+    return r;
+}
+// unit64 -> tile16 (once, at load; out of place): a wave a tile, every lane reads its share the way the block form does
+__global__ void __launch_bounds__(256) k_iq3s_tile16(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst, int nrows, int ncols, long tiles) {
+    const long t = (long) blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (t >= tiles) return;
+    const int lane = threadIdx.x & 63, nsuper = ncols >> 9, ks = ncols >> 5;
+    const long per = (long) (nrows >> 4) * nsuper;   // tiles a matrix
+    const long m = t / per, tl = t - m * per;
+    const int R = (int) (tl / nsuper), S = (int) (tl - (long) R * nsuper);
+    const uint8_t* we = src + (size_t) m * ((size_t) nrows * ks / 64 * UNIT_BYTES);
+    const SuperFields f = super_load(we, 16 * R + (lane & 15), 16 * S + 4 * (lane >> 4), ks);
+    uint8_t* u = dst + (size_t) t * TILE16_BYTES;
+    *reinterpret_cast<v4u*>(u + 32 * lane) = f.a0;
+    *reinterpret_cast<v4u*>(u + 32 * lane + 16) = f.a1;
+    *reinterpret_cast<v4u*>(u + TILE16_B_AT + 16 * lane) = f.b;
+    *reinterpret_cast<uint32_t*>(u + TILE16_C_AT + 4 * lane) = f.c;
+    *reinterpret_cast<unsigned short*>(u + TILE16_SC_AT + 2 * lane) = (unsigned short) f.sc;
+    *reinterpret_cast<unsigned short*>(u + TILE16_D_AT + 2 * lane) = (unsigned short) f.d;
+}
 constexpr int MB_XROW = 4 * MB_XLD + 16;   // a token's four step pieces of a super-step (+16: the 16 tokens of a tile fall on different banks)
 constexpr int MB_MAXTASK = 16;
 struct BlockTask {
@@ -478,6 +519,7 @@ struct MmaLds {
     BlockTask task[MB_MAXTASK];
     int ntask;
 };
+template <bool TILE16>
 __global__ void __launch_bounds__(MM_THREADS) k_moe_mma_block(const MmaArgs a) {
     typedef __attribute__((address_space(1))) const v4u gx4;
     __shared__ MmaLds L;
@@ -559,7 +601,9 @@ __global__ void __launch_bounds__(MM_THREADS) k_moe_mma_block(const MmaArgs a) {
             return t;
         };
         auto w_load_q = [&](int ti, int S, int q, SuperFields& o) {
-            o = super_load(L.task[ti].we, min(row0_of(ti) + qstep * q + r, a.nrows - 1), 16 * S + 4 * g, ks);
+            const int row = min(row0_of(ti) + qstep * q + r, a.nrows - 1);
+            if constexpr (TILE16) o = tile16_load(L.task[ti].we, row, S, nsuper);
+            else o = super_load(L.task[ti].we, row, 16 * S + 4 * g, ks);
         };
         auto w_load = [&](int ti, int S, SuperFields (&o)[MB_RG]) {
 #pragma unroll
@@ -679,6 +723,300 @@ __global__ void __launch_bounds__(MM_THREADS) k_moe_mma_block(const MmaArgs a) {
             const XShare x0 = x_load(0, 0);
             w_load(0, 0, w0);
             x_store(x0, 0);
+        }
+        __syncthreads();
+        for (int s = 0; s < nst; s += 2) {
+            stage(w0, w1, s);
+            if (s + 1 < nst) stage(w1, w0, s + 1);
+        }
+    }
+}
+
+// ---------------------------------------------------------------- block form, a task = (job, all of its up to 64 tokens, 256 weight rows)
+// kernels.hpp:27-30 (PF_JOB): "the expert's weight tile is then dequantized once for twice the tokens". The form above
+// decodes a sub-block once per 32 tokens, so a job of 33 to 64 tokens decodes every weight twice, and the codebook
+// lookups are what the launch waits for most. Here a lane's decoded operands of both row groups serve up to four token
+// tiles, two at a time (their B operands share registers). The 64-token activation tile takes the LDS of the two
+// 32-token buffers: it is replaced between two barriers at the end of a stage, its loads issued before the stage's last step.
+constexpr int MB_TP = 4, MB_TOK64 = 16 * MB_TP;
+constexpr int MB_SORTJ = 1024;   // jobs up to which the tasks are dealt by size
+struct MmaLds64 {
+    uint2 tab[SGRID_WORDS];
+    uint8_t xt[MB_TOK64 * MB_XROW];   // [token][step p][lane group g][64 bytes], step rows padded to 272 bytes
+    int ytok[MB_MAXTASK][MB_TOK64];
+    int otok[MB_MAXTASK][MB_TOK64];
+    BlockTask task[MB_MAXTASK];
+    int ntask;
+    uint8_t jkey[MB_SORTJ];            // a job's token tiles (0: no tokens)
+    unsigned short jorder[MB_SORTJ];   // the jobs, most token tiles first (the lower index first among equals)
+};
+template <bool TILE16>
+__global__ void __launch_bounds__(MM_THREADS) k_moe_mma_block64(const MmaArgs a) {
+    typedef __attribute__((address_space(1))) const v4u gx4;
+    __shared__ MmaLds64 L;
+    const uint32_t tab0 = g_sgrid.v[threadIdx.x];   // (512 threads: a thread's code, its sixteen signed entries made here)
+#pragma unroll
+    for (int i = threadIdx.x; i < SGRID_WORDS; i += MM_THREADS) {
+        const uint32_t g = signed_entry(tab0, i >> 9);
+        v2h lo, hi;
+        lo.x = (_Float16) (int) (int8_t) (g & 0xFFu);
+        lo.y = (_Float16) (int) (int8_t) ((g >> 8) & 0xFFu);
+        hi.x = (_Float16) (int) (int8_t) ((g >> 16) & 0xFFu);
+        hi.y = (_Float16) (int) (int8_t) (g >> 24);
+        L.tab[i] = make_uint2(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi));
+    }
+    const int tid = threadIdx.x, lane = tid & 63, wave = uniform(tid >> 6), r = lane & 15, g = lane >> 4;
+    const int nj = min(a.cap, uniform(*a.njobs)), nj2 = a.jobs2 ? min(a.cap2, uniform(*a.njobs2)) : 0;
+    const int ks = a.ncols >> 5, nsuper = ks >> 4, rblocks = (a.nrows + MB_ROWS - 1) / MB_ROWS;
+    constexpr int HALVES = 1;   // a task takes all of a job's token tiles
+    const int per_job = rblocks * HALVES, ntasks_all = (nj + nj2) * per_job;
+    // this thread's share of a super-step's activation tile (64 tokens x 512 k): tokens xtok and xtok + 32, 64 contiguous
+    // bytes each (sub-block xsb of the 16); in LDS the sub-block 4 g + p goes to step p, lane group g
+    const int xtok = tid >> 4, xsb = tid & 15;
+    const int xdst = xtok * MB_XROW + (xsb & 3) * MB_XLD + (xsb >> 2) * 64;
+    const int rlimit = a.h16 ? a.ffh : a.nrows, qstep = a.h16 ? a.ffh : 16;
+    struct XShare {
+        v4u v[8];
+    };
+    auto x_store = [&](const XShare& t) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            *reinterpret_cast<v4u*>(&L.xt[xdst + 16 * i]) = t.v[i];
+            *reinterpret_cast<v4u*>(&L.xt[xdst + 32 * MB_XROW + 16 * i]) = t.v[4 + i];
+        }
+    };
+    // A job's cost grows with its token tiles and a block gets two or three tasks of a chunk's few hundred: dealt in list
+    // order the slowest block took 84 us where the average took 58. So every block ranks the jobs by token tiles (the same
+    // order in every block: a job's rank is the count of jobs ahead of it) and the tasks are dealt in that order, to and
+    // fro over the blocks, the heaviest first.
+    const int njall = nj + nj2;
+    const bool sorted = njall <= MB_SORTJ;
+    if (sorted && wave == 0) {   // a counting sort by one wave, 64 jobs a trip: class totals, then every job's place
+        auto key_of = [&](int j) {
+            if (j >= njall) return -1;
+            const fnx_bigjob* jb = j < nj ? a.jobs + j : a.jobs2 + (j - nj);
+            return min(MB_TP, (max(0, min(FNX_PF_JOB, jb->n)) + 15) >> 4);
+        };
+        int total[MB_TP + 1];
+#pragma unroll
+        for (int c = 0; c <= MB_TP; ++c) total[c] = 0;
+        for (int j0 = 0; j0 < njall; j0 += 64) {
+            const int kj = key_of(j0 + lane);
+            if (j0 + lane < njall) L.jkey[j0 + lane] = (uint8_t) kj;
+#pragma unroll
+            for (int c = 0; c <= MB_TP; ++c) total[c] += __popcll(__ballot(kj == c));
+        }
+        int base[MB_TP + 1];   // where a class starts: the classes in descending order
+        base[MB_TP] = 0;
+#pragma unroll
+        for (int c = MB_TP - 1; c >= 0; --c) base[c] = base[c + 1] + total[c + 1];
+        for (int j0 = 0; j0 < njall; j0 += 64) {
+            const int kj = j0 + lane < njall ? (int) L.jkey[j0 + lane] : -1;
+#pragma unroll
+            for (int c = 0; c <= MB_TP; ++c) {
+                const unsigned long long m = __ballot(kj == c);
+                if (kj == c) L.jorder[base[c] + __popcll(m & ((1ull << lane) - 1ull))] = (unsigned short) (j0 + lane);
+                base[c] += __popcll(m);
+            }
+        }
+    }
+    for (int k0 = 0; k0 * (int) gridDim.x < ntasks_all; k0 += MB_MAXTASK) {   // MB_MAXTASK rounds a pass
+        __syncthreads();   // the previous lists' and tiles' last readers; the table and the jobs' order on the first pass
+        if (wave == 0) {
+            // this block's round k0 + lane: rounds go to and fro over the blocks
+            const int round = k0 + lane, pos = (round & 1) ? (int) gridDim.x - 1 - (int) blockIdx.x : (int) blockIdx.x;
+            const int task = round * (int) gridDim.x + pos;
+            bool ok = lane < MB_MAXTASK && task < ntasks_all;
+            BlockTask t{};
+            int ji = 0, n = 0;
+            if (ok) {
+                ji = task / per_job;
+                const int rem = task - ji * per_job;
+                if (sorted) ji = L.jorder[ji];
+                t.t0 = 0;
+                t.rb = rem % rblocks;
+                const fnx_bigjob* jb = ji < nj ? a.jobs + ji : a.jobs2 + (ji - nj);
+                n = min(FNX_PF_JOB, jb->n);
+                const int e = jb->w;
+                ok = n >= 1 && t.t0 < ((n + 15) >> 4);
+                t.ntile = min(MB_TP, (n + 15) >> 4);
+                if (ok) t.we = ji >= nj ? a.w2 : a.ep ? (const uint8_t*) a.ep[e] : a.w + (size_t) e * a.stride;
+            }
+            const unsigned long long m = __ballot(ok);
+            const int slot = __popcll(m & ((1ull << lane) - 1ull));
+            if (ok) {
+                t.ji = ji;
+                t.n = n;
+                L.task[slot] = t;
+            }
+            if (lane == 0) L.ntask = __popcll(m);
+        }
+        __syncthreads();
+        const int ntask = L.ntask;
+        if (ntask == 0) continue;   // the same for every thread of the block
+        for (int i = tid; i < ntask * MB_TOK64; i += MM_THREADS) {   // the tiles' token and output rows, all at once
+            const int slot = i / MB_TOK64, j = i % MB_TOK64, ji = L.task[slot].ji, n = L.task[slot].n, tok = L.task[slot].t0 * 16 + j;
+            const fnx_bigjob* jb = ji < nj ? a.jobs + ji : a.jobs2 + (ji - nj);
+            L.ytok[slot][j] = jb->y[min(tok, n - 1)];
+            L.otok[slot][j] = tok < n ? jb->out[tok] : -1;
+        }
+        __syncthreads();
+        const int nst = ntask * nsuper;
+        // the wave's first row in task ti: of its 32 consecutive rows, or (h16) of its 16 gate rows - the up rows lie ffh further
+        auto row0_of = [&](int ti) { return a.h16 ? L.task[ti].rb * (MB_ROWS / 2) + wave * 16 : L.task[ti].rb * MB_ROWS + wave * 16 * MB_RG; };
+        // a stage's loads: this thread's share of the activation tile and its lane's fields of both row groups
+        auto x_load = [&](int ti, int S) {
+            XShare t{};
+            // only the token tiles the task has: a job of up to 16 tokens asks for a quarter of the tile
+            const int ntok = 16 * L.task[ti].ntile;
+            const gx4* p = (gx4*) (uintptr_t) (a.x + (size_t) L.ytok[ti][xtok] * a.ldx + 32 * xsb + 512 * S);
+            const gx4* q = (gx4*) (uintptr_t) (a.x + (size_t) L.ytok[ti][xtok + 32] * a.ldx + 32 * xsb + 512 * S);
+            if (xtok < ntok) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) t.v[i] = p[i];
+            }
+            if (xtok + 32 < ntok) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) t.v[4 + i] = q[i];
+            }
+            return t;
+        };
+        auto w_load_q = [&](int ti, int S, int q, SuperFields& o) {
+            const int row = min(row0_of(ti) + qstep * q + r, a.nrows - 1);
+            if constexpr (TILE16) o = tile16_load(L.task[ti].we, row, S, nsuper);
+            else o = super_load(L.task[ti].we, row, 16 * S + 4 * g, ks);
+        };
+        auto w_load = [&](int ti, int S, SuperFields (&o)[MB_RG]) {
+#pragma unroll
+            for (int q = 0; q < MB_RG; ++q) w_load_q(ti, S, q, o[q]);
+        };
+        v4f acc[MB_RG][MB_TP];
+#pragma unroll
+        for (int q = 0; q < MB_RG; ++q)
+#pragma unroll
+            for (int tt = 0; tt < MB_TP; ++tt) acc[q][tt] = v4f{0.f, 0.f, 0.f, 0.f};
+        // nt_tag: the task's token tiles (1 or 2) as a constant: a lone tile's task reads and multiplies half as much
+        // the token tiles two at a time against both row groups' operands: a sub-block is decoded once for up to 64 tokens
+        auto pair = [&](const v8h (&A)[MB_RG][4], int p, auto t0_tag, auto cnt_tag) {
+            constexpr int T0 = decltype(t0_tag)::value, CNT = decltype(cnt_tag)::value;
+            v4u B[2][4];
+#pragma unroll
+            for (int tt = 0; tt < CNT; ++tt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) B[tt][i] = *reinterpret_cast<const v4u*>(&L.xt[((T0 + tt) * 16 + r) * MB_XROW + p * MB_XLD + 64 * g + 16 * i]);
+#pragma unroll
+            for (int q = 0; q < MB_RG; ++q)
+#pragma unroll
+                for (int tt = 0; tt < CNT; ++tt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        acc[q][T0 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[q][i], __builtin_bit_cast(v8h, B[tt][i]), acc[q][T0 + tt], 0, 0, 0);
+        };
+        auto step = [&](const SubFields (&cur)[MB_RG], int p, int nt) {
+            v8h A[MB_RG][4];
+#pragma unroll
+            for (int q = 0; q < MB_RG; ++q) {
+                const _Float16 sc = (_Float16) (int) (1 + 2 * cur[q].sc), d = __builtin_bit_cast(_Float16, (unsigned short) cur[q].d);
+                const v2h s2 = {sc, sc}, d2 = {d, d};
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const uint2 en = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint8_t*>(L.tab) + sub_entry<true>(cur[q], j));
+                    const v2h lo = (as_v2h(en.x) * s2) * d2, hi = (as_v2h(en.y) * s2) * d2;
+                    A[q][j >> 1][4 * (j & 1) + 0] = lo.x;
+                    A[q][j >> 1][4 * (j & 1) + 1] = lo.y;
+                    A[q][j >> 1][4 * (j & 1) + 2] = hi.x;
+                    A[q][j >> 1][4 * (j & 1) + 3] = hi.y;
+                }
+            }
+            using I0 = std::integral_constant<int, 0>;
+            using I1 = std::integral_constant<int, 1>;
+            using I2 = std::integral_constant<int, 2>;
+            if (nt >= 2) pair(A, p, I0{}, I2{});
+            else pair(A, p, I0{}, I1{});
+            if (nt == 3) pair(A, p, I2{}, I1{});
+            else if (nt == 4) pair(A, p, I2{}, I2{});
+        };
+        // pre(p): what the caller wants issued before step p (the next stage's loads, a part before each of the first steps,
+        // so that the waves' loads do not queue up behind one another at the stage's start)
+        auto steps4 = [&](SuperFields (&cur)[MB_RG], int nt, auto pre) {
+            SubFields c[MB_RG];
+            pre(0);
+#pragma unroll
+            for (int q = 0; q < MB_RG; ++q) c[q] = super_sub<0>(cur[q]);
+            step(c, 0, nt);
+            pre(1);
+#pragma unroll
+            for (int q = 0; q < MB_RG; ++q) c[q] = super_sub<1>(cur[q]);
+            step(c, 1, nt);
+            pre(2);
+#pragma unroll
+            for (int q = 0; q < MB_RG; ++q) c[q] = super_sub<2>(cur[q]);
+            step(c, 2, nt);
+            pre(3);
+#pragma unroll
+            for (int q = 0; q < MB_RG; ++q) c[q] = super_sub<3>(cur[q]);
+            step(c, 3, nt);
+        };
+        // Stage s = (task ti, super-step S) of the block's sequence: the next stage's loads - the next task's first ones
+        // too - are issued during this stage's arithmetic (the activations before its last step); its tile replaces this
+        // stage's in LDS between two barriers
+        int ti = 0, S = 0;
+        auto stage = [&](SuperFields (&cur)[MB_RG], SuperFields (&nxt)[MB_RG], int s) {
+            int tn = ti, Sn = S + 1;
+            if (Sn == nsuper) {
+                Sn = 0;
+                ++tn;
+            }
+            const bool more = s + 1 < nst;
+            XShare xn;
+            auto pre = [&](int p) {   // the weights (from HBM) first, the activations (cached) last
+                if (!more) return;
+                if (p < MB_RG) w_load_q(tn, Sn, p, nxt[p]);
+                else if (p == 3) xn = x_load(tn, Sn);
+            };
+            const int row0 = row0_of(ti);
+            if (row0 < rlimit) {   // per wave
+                steps4(cur, L.task[ti].ntile, pre);
+                if (Sn == 0) {   // the task's last super-step: lane = token r of each tile, weight rows 4 g .. 4 g + 3 of each group
+#pragma unroll
+                    for (int tt = 0; tt < MB_TP; ++tt) {
+                        const int orow = L.otok[ti][tt * 16 + r];
+                        if (orow >= 0) {
+                            if (a.h16) {   // gate rows in acc[0], their up rows in acc[1]
+                                const v4f gt = acc[0][tt], up = acc[1][tt];
+                                uint2 hv;
+                                hv.x = (uint32_t) float_to_half_bits(silu_f(gt.x) * up.x) | (uint32_t) float_to_half_bits(silu_f(gt.y) * up.y) << 16;
+                                hv.y = (uint32_t) float_to_half_bits(silu_f(gt.z) * up.z) | (uint32_t) float_to_half_bits(silu_f(gt.w) * up.w) << 16;
+                                *reinterpret_cast<uint2*>(a.h16 + (size_t) orow * a.ffh + row0 + 4 * g) = hv;
+                            } else {
+                                float* o = a.out + (size_t) orow * a.nrows + row0 + 4 * g;
+#pragma unroll
+                                for (int q = 0; q < MB_RG; ++q)
+                                    if (row0 + 16 * q < a.nrows)
+                                        *reinterpret_cast<float4*>(o + 16 * q) = make_float4(acc[q][tt].x, acc[q][tt].y, acc[q][tt].z, acc[q][tt].w);
+                            }
+                        }
+                    }
+#pragma unroll
+                    for (int q = 0; q < MB_RG; ++q)
+#pragma unroll
+                        for (int tt = 0; tt < MB_TP; ++tt) acc[q][tt] = v4f{0.f, 0.f, 0.f, 0.f};
+                }
+            } else {
+#pragma unroll
+                for (int p = 0; p <= 3; ++p) pre(p);
+            }
+            __syncthreads();   // this stage's tile has been read
+            if (more) x_store(xn);
+            __syncthreads();
+            ti = tn;
+            S = Sn;
+        };
+        SuperFields w0[MB_RG], w1[MB_RG];
+        {
+            const XShare x0 = x_load(0, 0);
+            w_load(0, 0, w0);
+            x_store(x0);
         }
         __syncthreads();
         for (int s = 0; s < nst; s += 2) {

@@ -477,7 +477,8 @@ class DecoderDev:
 class PfLayerDev:
     """One MoE layer's weights plus a chunk workspace, for fnx_moe_prefill_layer."""
 
-    def __init__(self, dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, C_rows, packed=True):
+    def __init__(self, dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, C_rows, packed=True, tile16=False):
+        """tile16 (with packed): the gate|up matrices also in the prompt path's own layout (fnx_iq3s_tile16), which the layer then uses"""
         t = dev.torch
         pkg = dev.pkg
         self.dev, self.n, self.ff, self.nexp, self.topk, self.C = dev, n, ff, nexp, topk, C_rows
@@ -491,6 +492,16 @@ class PfLayerDev:
         self.L = pkg.MoeLayer(n, ff, nexp, topk, self.router.data_ptr(), 0, pkg.dw(self.gu, n, 2 * ff, packed=packed), self.gu_stride,
                               pkg.dw(self.down, ff, n, packed=packed), self.down_stride, pkg.dw(self.sh_gu, n, 2 * ff, packed=packed),
                               pkg.dw(self.sh_down, ff, n, packed=packed))
+        if tile16:
+            assert packed
+            lib = dev.lib
+            self.gu16 = dev.zeros(lib.fnx_iq3s_tile16_bytes(2 * ff, n, nexp), t.uint8)
+            self.sh_gu16 = dev.zeros(lib.fnx_iq3s_tile16_bytes(2 * ff, n, 1), t.uint8)
+            dev.ok(lib.fnx_iq3s_tile16(self.gu.data_ptr(), self.gu16.data_ptr(), 2 * ff, n, nexp, dev.st()))
+            dev.ok(lib.fnx_iq3s_tile16(self.sh_gu.data_ptr(), self.sh_gu16.data_ptr(), 2 * ff, n, 1, dev.st()))
+            self.L.gu = pkg.dw(self.gu16, n, 2 * ff, tile16=True)
+            self.L.gu_stride = lib.fnx_iq3s_tile16_bytes(2 * ff, n, 1)
+            self.L.sh_gu = pkg.dw(self.sh_gu16, n, 2 * ff, tile16=True)
         P = C_rows * topk
         J, S = P // 64 + nexp, (C_rows + 63) // 64
         self.P, self.J = P, J

@@ -146,6 +146,26 @@ def test_prefill_layer_matches_oracle(dev, oracle, n, ff, nexp, topk, Cn):
         assert rel_l2(r["out"], want["out"]) <= REL_L2
 
 
+@pytest.mark.parametrize("n,ff,nexp,topk,Cn", [(2048, 512, 48, 10, 300), (1024, 256, 8, 2, 70)])
+def test_prefill_layer_tile16_equals_unit64(dev, oracle, n, ff, nexp, topk, Cn):
+    """the gate|up matrices in the prompt path's own layout: the same arithmetic on the same bytes found elsewhere, so the
+    chunk's result is that of the unit64 layout bit for bit (and the oracle's within the bar)"""
+    print(f"case prefill_layer tile16 n={n} ff={ff} nexp={nexp} topk={topk} C={Cn}", flush=True)
+    rng = np.random.default_rng(760 + nexp)
+    nb = lambda rows, cols: rows * cols // 256
+    gu = random_iq3s(rng, nexp * nb(2 * ff, n), dmax=1e-3)
+    down = random_iq3s(rng, nexp * nb(n, ff), dmax=1e-3)
+    sh_gu, sh_down = random_iq3s(rng, nb(2 * ff, n), dmax=1e-3), random_iq3s(rng, nb(n, ff), dmax=1e-3)
+    router = (rng.standard_normal((nexp + 1, n)) * 0.05).astype(np.float32)
+    x = rng.standard_normal((Cn, n)).astype(np.float32)
+    a = fnx_gpu.PfLayerDev(dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, Cn, packed=True).run(x)
+    b = fnx_gpu.PfLayerDev(dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, Cn, packed=True, tile16=True).run(x)
+    assert np.array_equal(a["topi"], b["topi"])
+    assert int(np.count_nonzero(a["out"].view(np.uint32) != b["out"].view(np.uint32))) == 0
+    want = oracle.moe_prefill_layer(n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, x)
+    assert rel_l2(b["out"], want["out"]) <= REL_L2
+
+
 def test_prefill_layer_large_chunk_equals_small_chunks(dev):
     """A size-independent property at a size the oracle does not reach: a row's result does not depend on what else is in
     its chunk, so 8,192 rows in one call (more tasks than one pass of a block's task list holds, every kernel form's loop
