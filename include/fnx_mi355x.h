@@ -156,8 +156,10 @@ int fnx_accept_greedy_dev(const int* rows, const int* o, int R, int* n_accept, v
  * routed + shared + SwiGLU -> q8_1 rows of h], [down routed + shared + the combine's chains; the job lists for the
  * caller]; these touch only the caller's workspace, so windows with workspaces of their own may run on different streams
  * at once. Other shapes run operator by operator through the library's one pair buffer per device, like moe_down: the
- * library puts such calls in order across streams (not under graph capture). A row with fewer than topk finite logits
- * takes the lowest experts not yet taken for its remaining picks (the reference's result is undefined there). */
+ * library puts such calls in order across streams (not under graph capture). A row with fewer than topk logits above
+ * -inf (masked or NaN entries) takes the lowest experts not yet taken for its remaining picks, at weight 0, so its picks
+ * stay distinct and no job exceeds 16 rows (the reference's result is undefined there); fnx_router_route and
+ * fnx_pf_route follow the same rule. */
 /* model.hpp:78-82  Q8S: dense Q8_0 in the split layout: int8 values [n_out][n_in], f16 scale bits [n_out][n_in / 32] */
 typedef struct fnx_q8s {
     const int8_t* q;

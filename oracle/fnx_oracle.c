@@ -368,13 +368,20 @@ void fnx_o_topk_logits(const float* logits, int stride, int T, int nexp, int top
                     bv = v[i];
                     bi = i;
                 }
+            const int found = bi < nexp;
+            if (!found) /* no logit above -inf is left (masked or NaN): the lowest index not yet picked, at weight 0 */
+                for (int i = 0; i < nexp; ++i)
+                    if (!taken[i]) {
+                        bi = i;
+                        break;
+                    }
             if (bi < nexp) taken[bi] = 1;
             if (k == 0) top0 = bv;
-            e[k] = expf(bv - top0);
+            e[k] = found ? expf(bv - top0) : 0.f;
             z += e[k];
-            topi[t * topk + k] = bi;
+            topi[t * topk + k] = bi < nexp ? bi : nexp - 1;
         }
-        for (int k = 0; k < topk; ++k) topw[t * topk + k] = e[k] / z;
+        for (int k = 0; k < topk; ++k) topw[t * topk + k] = z > 0.f ? e[k] / z : 0.f;
     }
     free(taken);
 }

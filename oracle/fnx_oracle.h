@@ -84,7 +84,10 @@ void fnx_o_gemv_exact(const uint8_t* w, int nrows, int ncols, const float* x, in
 void fnx_o_gemv_f32(const float* W, const float* x, float* y, int rows, int n, int T);
 void fnx_o_gemv_bf16(const uint16_t* W, const float* x, float* y, int rows, int n, int T);
 
-/* top-k by logit, ties to the lower index, w_k = exp(l_k - l_0) / sum (pick order). moe.cuh:382-411 */
+/* top-k by logit, ties to the lower index, w_k = exp(l_k - l_0) / sum (pick order). moe.cuh:382-411
+ * A row with fewer than topk logits above -inf (masked or NaN entries) is filled up with the lowest indexes not yet
+ * picked, at weight 0, so that a row's picks stay distinct (the reference emits the index NEXP there, which its callers
+ * do not define); a row with no such logit at all gets weights 0. This build's rule, shared with the device. */
 void fnx_o_topk_logits(const float* logits, int stride, int T, int nexp, int topk, int* topi, float* topw);
 /* softmax over all experts, top-k of the probabilities, renormalised. kernels.cu:338-378 */
 void fnx_o_topk_softmax(const float* logits, int stride, int T, int nexp, int topk, int* topi, float* topw);

@@ -181,18 +181,27 @@ __global__ void __launch_bounds__(TK_THREADS) k_topk_jobs(const float* __restric
                     bi = oi;
                 }
             }
+            const bool found = bi < nexp;
+            if (!found) {   // nothing above -inf is left (masked or NaN logits): the lowest index not yet picked, at weight 0
+                bi = 0x7fffffff;
+#pragma unroll
+                for (int i = TK_MAXE / 64 - 1; i >= 0; --i)
+                    if (lane + 64 * i < nexp && !((taken >> i) & 1u)) bi = lane + 64 * i;
+#pragma unroll
+                for (int o = 32; o; o >>= 1) bi = min(bi, __shfl_xor(bi, o, 64));
+            }
             if (bi < nexp && (bi & 63) == lane) taken |= 1u << (bi >> 6);
             if (k == 0) top0 = bv;
-            const float ek = expf(bv - top0);
+            const float ek = found ? expf(bv - top0) : 0.f;
             z += ek;
             if (lane == k) {
                 wk = ek;
-                const int pick = bi < nexp ? bi : nexp - 1;   // fewer than topk finite logits: stay inside the tables
+                const int pick = bi < nexp ? bi : nexp - 1;   // more picks than experts: refused by the host, kept inside the tables here
                 topi[t * topk + k] = pick;
                 ex[t * topk + k] = pick;
             }
         }
-        if (lane < topk) topw[t * topk + lane] = wk / z;
+        if (lane < topk) topw[t * topk + lane] = z > 0.f ? wk / z : 0.f;
     }
     __syncthreads();
     if (!gu) return;

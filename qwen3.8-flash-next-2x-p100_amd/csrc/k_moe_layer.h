@@ -83,6 +83,7 @@ __device__ __forceinline__ void wave_topk(const float* __restrict__ row, int nex
         v[i] = e < nexp ? row[e] : -INFINITY;
     }
     float top0 = 0.f, z = 0.f, wk = 0.f;
+    unsigned taken = 0;   // bit i: this lane's entry i has been picked
     for (int k = 0; k < topk; ++k) {
         // the lane's greatest value still to be picked (a picked one becomes -inf) and the lowest of its indexes that hold
         // it, as a tree of maxima and a mask of equalities rather than a chain over the NE values. A NaN is never the
@@ -101,21 +102,29 @@ __device__ __forceinline__ void wave_topk(const float* __restrict__ row, int nex
         int mi;
         if (__popcll(holders) == 1) mi = __builtin_amdgcn_readlane(bi, (int) __builtin_ctzll(holders));
         else mi = wave_min(bv == m ? bi : 0x7fffffff);
+        bool found = mi < nexp;
+        if (!found) {   // nothing above -inf is left (masked or NaN logits): the lowest index not yet picked, at weight 0
+            unsigned left = 0;
+#pragma unroll
+            for (int i = 0; i < NE; ++i) left |= (lane + 64 * i < nexp && !((taken >> i) & 1u) ? 1u : 0u) << i;
+            mi = wave_min(left ? lane + 64 * (int) __builtin_ctz(left) : 0x7fffffff);
+        }
         const bool mine = mi < nexp && (mi & 63) == lane;
 #pragma unroll
         for (int i = 0; i < NE; ++i)
             if (mine && (mi >> 6) == i) v[i] = -INFINITY;
+        if (mine) taken |= 1u << (mi >> 6);
         if (k == 0) top0 = m;
-        const float ek = expf(m - top0);
+        const float ek = found ? expf(m - top0) : 0.f;
         z += ek;
         if (lane == k) {
             wk = ek;
-            const int pick = mi < nexp ? mi : nexp - 1;   // fewer than topk finite logits: stay inside the tables
+            const int pick = mi < nexp ? mi : nexp - 1;   // more picks than experts: refused by the host, kept inside the tables here
             ex[k] = pick;
             if (publish) topi[k] = pick;
         }
     }
-    if (publish && lane < topk) topw[lane] = wk / z;
+    if (publish && lane < topk) topw[lane] = z > 0.f ? wk / z : 0.f;
 }
 
 // ---------------------------------------------------------------- the job lists of a window's picks

@@ -80,6 +80,26 @@ def test_route_bit_exact(dev, oracle, T, nexp, topk):
     assert r["njobs"][0] == len(gu) and r["njobs"][1] == len(gu)
 
 
+@pytest.mark.parametrize("T,nexp,topk", [(16, 512, 10), (5, 64, 6), (16, 1000, 16)])
+def test_route_with_fewer_finite_logits_than_picks(dev, oracle, T, nexp, topk):
+    # masked (-inf) and NaN logits: the picks stay distinct (the lowest indexes not yet picked, at weight 0) and no job
+    # takes a token twice
+    from test_oracle_routing import scarce_logits
+    print(f"case route scarce T={T} nexp={nexp} topk={topk}", flush=True)
+    logits = scarce_logits(np.random.default_rng(305 + T), T, nexp)
+    r = dev.route(logits, nexp, topk)
+    topi, topw = oracle.topk_logits(logits, nexp, topk)
+    assert np.array_equal(r["topi"], topi)
+    for t in range(T):
+        assert len(set(r["topi"][t].tolist())) == topk
+    assert np.array_equal(np.isfinite(r["topw"]), np.ones_like(topw, dtype=bool))
+    assert np.allclose(r["topw"], topw, rtol=2e-6, atol=0)
+    gu, dn = oracle.jobs(topi)
+    check_jobs(r["gu"], gu)
+    check_jobs(r["dn"], dn)
+    assert max(int(j["n"]) for j in r["gu"][:r["njobs"][0]]) <= T
+
+
 def test_router_route_fused_bit_exact(dev, oracle):
     rng = np.random.default_rng(310)
     T, n, nexp, topk = 16, 2048, 512, 10

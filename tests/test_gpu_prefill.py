@@ -60,6 +60,20 @@ def test_pf_route_bit_exact(dev, oracle, Cn, nexp, topk, zipf):
             assert np.array_equal(g[2:2 + n], w[2:2 + n]) and np.array_equal(g[2 + PF:2 + PF + n], w[2 + PF:2 + PF + n])
 
 
+def test_pf_route_with_fewer_finite_logits_than_picks(dev, oracle):
+    from test_oracle_routing import scarce_logits
+    Cn, nexp, topk = 70, 512, 10
+    print(f"case pf_route scarce C={Cn} nexp={nexp} topk={topk}", flush=True)
+    logits = scarce_logits(np.random.default_rng(705), Cn, nexp)
+    r = dev.pf_route(logits, nexp, topk)
+    topi, topw = oracle.topk_logits(logits, nexp, topk)
+    assert np.array_equal(r["topi"], topi)
+    assert all(len(set(row.tolist())) == topk for row in r["topi"])
+    assert np.all(np.isfinite(r["topw"])) and np.allclose(r["topw"], topw, rtol=2e-6, atol=0)
+    gu, dn, cnt = oracle.pf_jobs(topi, nexp, PF)
+    assert np.array_equal(r["cnt"], cnt) and r["njobs"] == len(gu)
+
+
 def test_f32_f16_bit_exact(dev, oracle):
     rng = np.random.default_rng(710)
     x = (rng.standard_normal((33, 257)) * 10.0 ** rng.integers(-8, 4, (33, 257))).astype(np.float32)

@@ -81,6 +81,43 @@ def test_topk_ignores_the_shared_gate_column(oracle):
     assert list(topi[0]) == [0, 1, 2]
 
 
+def scarce_logits(rng, T, nexp):
+    """rows with fewer selectable logits than picks: -inf masks and NaN entries; the last row has none at all"""
+    lg = rng.standard_normal((T, nexp + 1)).astype(np.float32)
+    lg[0, :nexp] = -np.inf
+    lg[0, [7, 3, nexp - 1]] = [0.5, 0.25, 1.5]          # three finite logits
+    if T > 1:
+        lg[1, :nexp] = np.nan
+        lg[1, [1, 4]] = [2.0, 2.0]                       # two finite logits, tied
+    if T > 2:
+        lg[2, 0:nexp:2] = -np.inf                        # half of the experts masked: enough left, nothing is filled in
+    if T > 3:
+        lg[T - 1, :nexp] = -np.inf                       # nothing to pick
+        lg[T - 1, 5] = np.nan
+    return lg
+
+
+def test_topk_with_fewer_finite_logits_than_picks(oracle):
+    rng = np.random.default_rng(16)
+    nexp, topk = 64, 6
+    lg = scarce_logits(rng, 5, nexp)
+    topi, topw = oracle.topk_logits(lg, nexp, topk)
+    for t in range(5):
+        assert len(set(topi[t].tolist())) == topk and topi[t].min() >= 0 and topi[t].max() < nexp
+    assert list(topi[0]) == [nexp - 1, 7, 3, 0, 1, 2]       # the finite ones by value, then the lowest indexes not yet picked
+    e = np.exp(np.array([0.0, -1.0, -1.25]))
+    assert np.allclose(topw[0, :3], e / e.sum(), rtol=1e-6) and np.all(topw[0, 3:] == 0)
+    assert list(topi[1]) == [1, 4, 0, 2, 3, 5]
+    assert np.allclose(topw[1, :2], 0.5) and np.all(topw[1, 2:] == 0)
+    assert list(topi[2]) == brute_topk(np.where(np.isinf(lg[2, :nexp]), -1e30, lg[2, :nexp]), topk)
+    assert abs(topw[2].sum() - 1) < 1e-6
+    assert list(topi[4]) == list(range(topk)) and np.all(topw[4] == 0)
+    # every job holds a token at most once
+    gu, dn = oracle.jobs(topi)
+    assert all(int(j["n"]) <= 5 for j in gu)
+    assert sum(int(j["n"]) for j in gu) == 5 * topk
+
+
 # ---------------------------------------------------------------- jobs
 def test_jobs_invariants(oracle):
     rng = np.random.default_rng(15)
