@@ -1455,6 +1455,7 @@ static int attn_launch(const float* qg, const uint16_t* kc, const uint16_t* vc, 
     if (!qg || !kc || !vc || (!out && !outq) || !pos0 || !scratch) return fail("attn: null argument");
     if (nq < 1 || nkv < 1 || nq % nkv || nq / nkv > AT_MAXQ || T < 1 || T > FNX_MAXT || max_ctx < 1) return fail("attn: bad shape");
     if (attn_splits(max_ctx) > AT_MAXSPLIT) return fail("attn: the cache is larger than the split table");
+    if (((unsigned long long) max_ctx + 3) * nkv * (AT_HD * 2) >= (1ull << 32)) return fail("attn: a cache of 4 GiB or more (the kernel's byte offsets are 32 bits)");
     // the grid covers the cache's capacity (the position is on the device): splits past the context write empty parts
     const int nsplit = attn_splits(max_ctx), waves = (T * (nq / nkv) + 15) / 16;
     float* acc = scratch;

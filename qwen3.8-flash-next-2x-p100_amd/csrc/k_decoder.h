@@ -438,7 +438,7 @@ __device__ __forceinline__ float groups4_sum(float v) {
     asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(x), "+v"(y));
     return x + y;
 }
-constexpr int AT_VLD = AT_HD * 8 + 128;   // LDS bytes per V block: the four lane groups' 128-byte reads of one instruction fall on different banks
+constexpr int AT_VPG = AT_HD * 16;   // LDS bytes of a lane group's V operands of a chunk: per dim the four positions of block pg, then those of block 4 + pg
 constexpr int AT_WAVES = 4, AT_KLD = 2 * AT_HD + 16;   // q tiles (of 16 queries) per block, blockIdx.z picks which; LDS bytes per K row
 __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) k_attn_part(const float* __restrict__ qg, const uint16_t* __restrict__ kc,
                                                             const uint16_t* __restrict__ vc, float* __restrict__ acc_out,
@@ -449,9 +449,22 @@ __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per
     if (gate && uniform(*gate) == 0) return;   // a chain step that does not count: its parts stay what they were, nothing reads the result
     // live (may be null): a device word, the rows of the window that count; the others' queries are left out (nothing reads
     // their results), the positions past the last row that counts with them
-    if (live) T = uniform(max(1, min(*live, T)));
     const int s = blockIdx.x, kvh = blockIdx.y, lane = threadIdx.x & 63, wave = blockIdx.z * AT_WAVES + (threadIdx.x >> 6);
-    const int qpk = nq / nkv, nquery = T * qpk;
+    const int qpk = nq / nkv;
+    // this lane's query row, 64 of its dims: loaded before anything that waits for a device word (a lane past the window's
+    // queries reads the last query's row; its operands become zeros below)
+    float4 qa[8], qb[8];
+    {
+        const int qc = min(wave * 16 + (lane & 15), T * qpk - 1);
+        const float* qr = qg + ((size_t) (qc / qpk) * nq + kvh * qpk + qc % qpk) * 2 * AT_HD + 64 * (lane >> 4);
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+            qa[ks] = *reinterpret_cast<const float4*>(qr + 8 * ks);
+            qb[ks] = *reinterpret_cast<const float4*>(qr + 8 * ks + 4);
+        }
+    }
+    if (live) T = uniform(max(1, min(*live, T)));
+    const int nquery = T * qpk;
     const AttWindow win = att_window(*pos0p, T, max_ctx);   // no index below leaves the cache, whatever the device word holds
     if ((int) blockIdx.z * AT_WAVES * 16 >= nquery) return;   // none of the block's queries count
     const bool wave_on = uniform(wave * 16 < nquery);         // a wave without queries still fetches its share of K and V
@@ -462,21 +475,79 @@ __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per
     const int ctx_q = qlive ? att_ctx_q(win, qt) : 0;   // positions [0, ctx_q) are this query's
     const int ctx_max = win.ctx_max;                    // the window's last row sees this many
     const int p0 = att_split_begin(s), p1 = att_split_end(win, s);
+    const int vis = uniform(wave_on ? min(att_ctx_q(win, (wave * 16) / qpk), p1) : 0);   // the wave's first query is its earliest row's
     const size_t slot = ((size_t) qt * nq + qh) * nsplit + s;
     if (p0 >= p1) {   // a split past the context: an empty part
         if (qlive && pg == 0) mz_out[slot] = AttPart{-INFINITY, 0.f};
         return;
     }
+    // A chunk's K rows (32 x 512 bytes) and V blocks (8 x 2048 bytes) are fetched once per block, 64 + 64 contiguous
+    // bytes per thread, a chunk ahead into registers and from there into one of two LDS buffers; the waves read their
+    // operands from LDS (K rows padded to 528 bytes: the 16 positions of a tile fall on different banks).
+    __shared__ __align__(16) uint8_t lk[2][AT_CH * AT_KLD];
+    __shared__ __align__(16) uint8_t lv[2][4 * AT_VPG];
+    const int tid = threadIdx.x;
+    const gbytes kbase = as_global(reinterpret_cast<const uint8_t*>(kc));
+    const gbytes vbase = as_global(reinterpret_cast<const uint8_t*>(vc));
+    // piece tid + 256 i of the chunk's 1024 16-byte pieces of K (32 to a row) and of V (128 to a block): consecutive lanes
+    // load consecutive pieces, so a wave's load is whole runs of 512 or 1024 bytes
+    // (byte offsets in 32 bits: the host refuses caches of 4 GiB and more)
+    const int krow = tid >> 5, kcol = tid & 31, vblk = tid >> 7, vcol = tid & 127;
+    const uint32_t krowb = (uint32_t) nkv * (AT_HD * 2), vblkb = (uint32_t) nkv * (AT_HD * 8);   // bytes between two rows of K, two blocks of V
+    const uint32_t koff0 = ((uint32_t) krow * nkv + kvh) * (AT_HD * 2) + 16 * kcol, voff0 = ((uint32_t) vblk * nkv + kvh) * (AT_HD * 8) + 16 * vcol;
+    at_v4u kr[4], vr[4];
+    int fc = 0;   // the chunk the registers hold
+    auto fetch = [&](int c0) {
+        fc = c0;
+        if (uniform(c0 + AT_CH <= ctx_max)) {   // a chunk inside the window's rows: a row or block is a constant further
+            const uint32_t ko = koff0 + (uint32_t) c0 * krowb, vo = voff0 + (uint32_t) (c0 >> 2) * vblkb;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                kr[i] = *(g128*) (kbase + (ko + 8 * i * krowb));
+                vr[i] = *(g128*) (vbase + (vo + 2 * i * vblkb));
+            }
+        } else {   // rows and blocks clamped inside the window's rows
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int pos = att_fetch_row(win, c0, krow + 8 * i), blk = att_fetch_vblock(win, c0, vblk + 2 * i);
+                kr[i] = *(g128*) (kbase + (((uint32_t) pos * nkv + kvh) * (AT_HD * 2) + 16 * kcol));
+                vr[i] = *(g128*) (vbase + (((uint32_t) blk * nkv + kvh) * (AT_HD * 8) + 16 * vcol));
+            }
+        }
+    };
+    // Positions past the window's rows were never written: whatever their cells hold must not reach the P V products (a
+    // zero probability does not stop a NaN). The slots of such positions are zeroed here, once per block and only in a
+    // chunk that reaches past the rows, instead of in every wave's operands; a block clamped to the window's last
+    // repeats that block, slots zeroed alike. A 16-byte piece is two dims x four positions of one block.
+    auto stash = [&](int buf) {
+        if (uniform(fc + AT_CH > ctx_max)) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int nv = ctx_max - 4 * att_fetch_vblock(win, fc, vblk + 2 * i);   // the block's written positions: 1 or more
+                const unsigned m01 = nv >= 2 ? ~0u : 0x0000FFFFu, m23 = nv >= 4 ? ~0u : nv == 3 ? 0x0000FFFFu : 0u;
+                vr[i] = at_v4u{vr[i].x & m01, vr[i].y & m23, vr[i].z & m01, vr[i].w & m23};
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            *reinterpret_cast<at_v4u*>(&lk[buf][(krow + 8 * i) * AT_KLD + 16 * kcol]) = kr[i];
+            // block b's dims 2 vcol and 2 vcol + 1 (8 bytes each: four positions) into half b / 4 of lane group b % 4's 16-byte operands
+            const int b = vblk + 2 * i;
+            uint8_t* dst = &lv[buf][(b & 3) * AT_VPG + 32 * vcol + 8 * (b >> 2)];
+            *reinterpret_cast<at_v2u*>(dst) = at_v2u{vr[i].x, vr[i].y};
+            *reinterpret_cast<at_v2u*>(dst + 16) = at_v2u{vr[i].z, vr[i].w};
+        }
+    };
+    fetch(p0);
     // Q^T operands: step ks holds dims 64 pg + 8 ks .. + 7 of query ql, times 1/16 (exact), as two f16 terms hi + lo:
     // the cache is f16 already, so with q (and below the probabilities) split this way the products carry fp32's
-    // precision, as the reference's f32 arithmetic on the f16 cache does
+    // precision, as the reference's f32 arithmetic on the f16 cache does. (Converted while the first chunk is on its way.)
     at_v8h Q[8], Ql[8];
     {
-        const float* qr = qg + ((size_t) qt * nq + qh) * 2 * AT_HD + 64 * pg;
         const float sc = qlive ? 0.0625f : 0.f;
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) {
-            const float4 a = *reinterpret_cast<const float4*>(qr + 8 * ks), b = *reinterpret_cast<const float4*>(qr + 8 * ks + 4);
+            const float4 a = qa[ks], b = qb[ks];
             const float v[8] = {a.x * sc, a.y * sc, a.z * sc, a.w * sc, b.x * sc, b.y * sc, b.z * sc, b.w * sc};
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
@@ -490,39 +561,25 @@ __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per
 #pragma unroll
     for (int dt = 0; dt < 16; ++dt) O[dt] = at_v4f{0.f, 0.f, 0.f, 0.f};
     float m = -INFINITY, z = 0.f;
-    // A chunk's K rows (32 x 512 bytes) and V blocks (8 x 2048 bytes) are fetched once per block, 64 + 64 contiguous
-    // bytes per thread, a chunk ahead into registers and from there into one of two LDS buffers; the waves read their
-    // operands from LDS (K rows padded to 528 bytes: the 16 positions of a tile fall on different banks).
-    __shared__ __align__(16) uint8_t lk[2][AT_CH * AT_KLD];
-    __shared__ __align__(16) uint8_t lv[2][8 * AT_VLD];
-    const int tid = threadIdx.x;
-    const gbytes kbase = as_global(reinterpret_cast<const uint8_t*>(kc));
-    const gbytes vbase = as_global(reinterpret_cast<const uint8_t*>(vc));
-    // piece tid + 256 i of the chunk's 1024 16-byte pieces of K (32 to a row) and of V (128 to a block): consecutive lanes
-    // load consecutive pieces, so a wave's load is whole runs of 512 or 1024 bytes
-    const int krow = tid >> 5, kcol = tid & 31, vblk = tid >> 7, vcol = tid & 127;
-    at_v4u kr[4], vr[4];
-    auto fetch = [&](int c0) {   // rows and blocks clamped inside the window's rows
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int pos = att_fetch_row(win, c0, krow + 8 * i), blk = att_fetch_vblock(win, c0, vblk + 2 * i);
-            kr[i] = *(g128*) (kbase + ((size_t) pos * nkv + kvh) * (AT_HD * 2) + 16 * kcol);
-            vr[i] = *(g128*) (vbase + ((size_t) blk * nkv + kvh) * (AT_HD * 8) + 16 * vcol);
-        }
-    };
-    auto stash = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            *reinterpret_cast<at_v4u*>(&lk[buf][(krow + 8 * i) * AT_KLD + 16 * kcol]) = kr[i];
-            *reinterpret_cast<at_v4u*>(&lv[buf][(vblk + 2 * i) * AT_VLD + 16 * vcol]) = vr[i];
-        }
-    };
-    fetch(p0);
     stash(0);
     fetch(min(p0 + AT_CH, p1 - 1));
     __syncthreads();
     int buf = 0;
     for (int c0 = p0; c0 < p1; c0 += AT_CH, buf ^= 1) {
+        // The K operands are read a group (two steps of both tiles: four 16-byte reads) ahead of the products that use them,
+        // the first group before the block's own stores and loads below: after the barrier the four waves ask the LDS for
+        // the same rows at the same time, and a read that is only issued when it is needed waits for all four.
+        const uint8_t* k0 = &lk[buf][ql * AT_KLD + 128 * pg];
+        const uint8_t* k1 = k0 + 16 * AT_KLD;
+        at_v4u kq[2][4];
+        auto kread = [&](int g, at_v4u (&o)[4]) {
+            o[0] = *reinterpret_cast<const at_v4u*>(k0 + 32 * g);
+            o[1] = *reinterpret_cast<const at_v4u*>(k1 + 32 * g);
+            o[2] = *reinterpret_cast<const at_v4u*>(k0 + 32 * g + 16);
+            o[3] = *reinterpret_cast<const at_v4u*>(k1 + 32 * g + 16);
+        };
+        if (wave_on) kread(0, kq[0]);
+        __builtin_amdgcn_sched_barrier(0);
         stash(buf ^ 1);                              // chunk c0 + 32, fetched during the last iteration
         fetch(min(c0 + 2 * AT_CH, p1 - 1));          // past the split: some rows again, never used
         if (wave_on) {
@@ -530,38 +587,54 @@ __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per
         // none waits for the one before it
         at_v4f S[2];
         {
-            const uint8_t* k0 = &lk[buf][ql * AT_KLD + 128 * pg];
-            const uint8_t* k1 = k0 + 16 * AT_KLD;
             at_v4f a0 = at_v4f{0.f, 0.f, 0.f, 0.f}, a0l = a0, a1 = a0, a1l = a0;
 #pragma unroll
-            for (int ks = 0; ks < 8; ++ks) {
-                const at_v8h kk0 = __builtin_bit_cast(at_v8h, *reinterpret_cast<const at_v4u*>(k0 + 16 * ks));
-                const at_v8h kk1 = __builtin_bit_cast(at_v8h, *reinterpret_cast<const at_v4u*>(k1 + 16 * ks));
-                a0l = __builtin_amdgcn_mfma_f32_16x16x32_f16(kk0, Ql[ks], a0l, 0, 0, 0);
-                a1l = __builtin_amdgcn_mfma_f32_16x16x32_f16(kk1, Ql[ks], a1l, 0, 0, 0);
-                a0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kk0, Q[ks], a0, 0, 0, 0);
-                a1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kk1, Q[ks], a1, 0, 0, 0);
+            for (int g = 0; g < 4; ++g) {
+                if (g < 3) kread(g + 1, kq[(g + 1) & 1]);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int ks = 2 * g + j;
+                    const at_v8h kk0 = __builtin_bit_cast(at_v8h, kq[g & 1][2 * j]), kk1 = __builtin_bit_cast(at_v8h, kq[g & 1][2 * j + 1]);
+                    a0l = __builtin_amdgcn_mfma_f32_16x16x32_f16(kk0, Ql[ks], a0l, 0, 0, 0);
+                    a1l = __builtin_amdgcn_mfma_f32_16x16x32_f16(kk1, Ql[ks], a1l, 0, 0, 0);
+                    a0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kk0, Q[ks], a0, 0, 0, 0);
+                    a1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kk1, Q[ks], a1, 0, 0, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
             S[0] = a0 + a0l;
             S[1] = a1 + a1l;
         }
-        // this lane: query ql, positions c0 + 4 pg + r (tile 0) and c0 + 16 + 4 pg + r (tile 1)
-        float sv[8];
-        float mx = -INFINITY;
+        // this lane: query ql, positions c0 + 4 pg + r (tile 0) and c0 + 16 + 4 pg + r (tile 1). A chunk that every query of
+        // the wave sees whole (all but the last ones of a context) needs no masks: its maximum is finite
+        float pw[8], ps = 0.f, mn, sc;
+        if (uniform(c0 + AT_CH <= vis)) {
+            const float mx = groups4_max(fmaxf(fmaxf(fmaxf(S[0][0], S[0][1]), fmaxf(S[0][2], S[0][3])), fmaxf(fmaxf(S[1][0], S[1][1]), fmaxf(S[1][2], S[1][3]))));
+            mn = fmaxf(m, mx);
+            sc = __expf(m - mn);   // m = -inf before the first chunk: 0
 #pragma unroll
-        for (int r = 0; r < 8; ++r) {
-            const int pos = c0 + 16 * (r >> 2) + 4 * pg + (r & 3);
-            sv[r] = pos < ctx_q && pos < p1 ? S[r >> 2][r & 3] : -INFINITY;
-            mx = fmaxf(mx, sv[r]);
-        }
-        mx = groups4_max(mx);
-        const float mn = fmaxf(m, mx);
-        const float sc = m == -INFINITY ? 0.f : __expf(m - mn);
-        float pw[8], ps = 0.f;
+            for (int r = 0; r < 8; ++r) {
+                pw[r] = __expf(S[r >> 2][r & 3] - mn);
+                ps += pw[r];
+            }
+        } else {
+            float sv[8];
+            float mx = -INFINITY;
 #pragma unroll
-        for (int r = 0; r < 8; ++r) {
-            pw[r] = sv[r] == -INFINITY ? 0.f : __expf(sv[r] - mn);
-            ps += pw[r];
+            for (int r = 0; r < 8; ++r) {
+                const int pos = c0 + 16 * (r >> 2) + 4 * pg + (r & 3);
+                sv[r] = pos < ctx_q && pos < p1 ? S[r >> 2][r & 3] : -INFINITY;
+                mx = fmaxf(mx, sv[r]);
+            }
+            mx = groups4_max(mx);
+            mn = fmaxf(m, mx);
+            sc = m == -INFINITY ? 0.f : __expf(m - mn);
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                pw[r] = sv[r] == -INFINITY ? 0.f : __expf(sv[r] - mn);
+                ps += pw[r];
+            }
         }
         ps = groups4_sum(ps);
         z = z * sc + ps;
@@ -574,17 +647,7 @@ __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per
             Pl[r] = (_Float16) (pw[r] - (float) hi);
         }
         // V^T operands: positions c0 + 4 pg .. + 3 (block pg of the chunk) and c0 + 16 + 4 pg .. + 3 (block 4 + pg), dim
-        // 16 dt + ql. Positions past the window's rows were never written: whatever their cells hold must not reach the
-        // products (a block clamped to the window's last repeats that block: its probabilities are zero)
-        const bool tail = c0 + AT_CH > ctx_max;
-        unsigned keep0[2] = {~0u, ~0u}, keep1[2] = {~0u, ~0u};
-        if (tail) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                if (c0 + 4 * pg + j >= ctx_max) keep0[j >> 1] &= (j & 1) ? 0x0000FFFFu : 0xFFFF0000u;
-                if (c0 + 16 + 4 * pg + j >= ctx_max) keep1[j >> 1] &= (j & 1) ? 0x0000FFFFu : 0xFFFF0000u;
-            }
-        }
+        // 16 dt + ql (slots past the window's rows hold zeros: stash)
         if (__any(sc != 1.0f)) {   // the running maximum moved (rare once the first chunks are behind)
 #pragma unroll
             for (int dt = 0; dt < 16; ++dt) {
@@ -594,19 +657,13 @@ __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per
                 O[dt].w *= sc;
             }
         }
-        const uint8_t* v0 = &lv[buf][pg * AT_VLD + ql * 8];
-        const uint8_t* v1 = &lv[buf][(4 + pg) * AT_VLD + ql * 8];
-        // (the masks on every chunk: a second copy of this loop without them for the chunks inside the window costs more in
-        // registers than the 64 ANDs it saves)
+        const uint8_t* vb = &lv[buf][pg * AT_VPG + ql * 16];   // dim 16 dt + ql: one 16-byte read, the operand's register order
         // four dim tiles at a time: the lo products of all four, then the hi ones (a chain's next MFMA four issues away);
         // the next four tiles' V reads are issued before this group's arithmetic
-        at_v2u ra[2][4][2];
-        auto vread = [&](int d0, at_v2u (&o)[4][2]) {
+        at_v4u ra[2][4];
+        auto vread = [&](int d0, at_v4u (&o)[4]) {
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                o[u][0] = *reinterpret_cast<const at_v2u*>(v0 + 128 * (d0 + u));
-                o[u][1] = *reinterpret_cast<const at_v2u*>(v1 + 128 * (d0 + u));
-            }
+            for (int u = 0; u < 4; ++u) o[u] = *reinterpret_cast<const at_v4u*>(vb + 256 * (d0 + u));
         };
         vread(0, ra[0]);
 #pragma unroll
@@ -615,10 +672,7 @@ __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per
             __builtin_amdgcn_sched_barrier(0);
             at_v8h a[4];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const at_v2u a0 = ra[gq & 1][u][0], a1 = ra[gq & 1][u][1];
-                a[u] = __builtin_bit_cast(at_v8h, at_v4u{a0.x & keep0[0], a0.y & keep0[1], a1.x & keep1[0], a1.y & keep1[1]});
-            }
+            for (int u = 0; u < 4; ++u) a[u] = __builtin_bit_cast(at_v8h, ra[gq & 1][u]);
 #pragma unroll
             for (int u = 0; u < 4; ++u) O[4 * gq + u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[u], Pl, O[4 * gq + u], 0, 0, 0);
 #pragma unroll
