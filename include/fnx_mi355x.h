@@ -296,8 +296,8 @@ typedef struct fnx_rope {
 } fnx_rope;
 /* kernels.hpp:259  attn_prep_append: q heads (qg [T][nq][q | gate], 2 x 256 each) and k heads RMS-normed with their
  * weights and rotated at positions *pos0 + t, in place; k and v appended to the f16 caches of max_ctx positions (a
- * multiple of 4): K is [position][nkv][256]; V is this library's own layout [position / 4][nkv][256][position % 4]
- * (four positions of a dimension together, the matrix-core attention's operand). */
+ * multiple of 8, under 4 GiB a cache): K is [position][nkv][256]; V is this library's own layout [position / 8][nkv][256][position % 8]
+ * (eight positions of a dimension together: 16 bytes, the matrix-core attention's operand of one lane). */
 int fnx_attn_prep_append(float* qg, float* k, const float* v, const float* q_norm, const float* k_norm, uint16_t* kc, uint16_t* vc, int nq,
                          int nkv, int T, const int* pos0, int max_ctx, float eps, const fnx_rope* rope, void* st);
 /* kernels.hpp:238  attn: row t attends positions [0, *pos0 + t]; out [T][nq][256] = softmax(q k / 16) v * sigmoid(gate).

@@ -11,6 +11,7 @@ FLAGS = [
     "-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-shared",
     "-ffp-contract=off",                       # fused multiply-adds only where the code says fmaf: part of the results' definition
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-mllvm", "-amdgpu-mfma-vgpr-form",       # matrix-core results in the ordinary registers: the kernels here take them up with vector instructions right away
     "-Wall", "-Wno-unused-function", "-Wno-unknown-attributes",
 ]
 

@@ -14,6 +14,7 @@ namespace fnx {
 
 constexpr int AT_SPLIT = 512;   // positions a block of the first pass covers
 constexpr int AT_CH = 32;       // positions a chunk (one trip of a block's loop)
+constexpr int AT_VB = 8;        // positions whose values of a dimension lie together in the V cache: [position / 8][kv head][dim][position % 8]
 
 FNX_HOST_DEVICE inline int att_min(int a, int b) { return a < b ? a : b; }
 FNX_HOST_DEVICE inline int att_max(int a, int b) { return a > b ? a : b; }
@@ -34,10 +35,10 @@ FNX_HOST_DEVICE inline int att_ctx_q(const AttWindow& w, int qt) { return att_mi
 // split s covers positions [p0, p1); empty when p0 >= p1
 FNX_HOST_DEVICE inline int att_split_begin(int s) { return s * AT_SPLIT; }
 FNX_HOST_DEVICE inline int att_split_end(const AttWindow& w, int s) { return att_min(w.ctx_max, s * AT_SPLIT + AT_SPLIT); }
-// the K row and the V block (of four positions) that a fetch of chunk c0 reads for its row r (0 .. AT_CH - 1) and block b
-// (0 .. AT_CH / 4 - 1): clamped inside the window's rows
+// the K row and the V block (of AT_VB positions) that a fetch of chunk c0 reads for its row r (0 .. AT_CH - 1) and block b
+// (0 .. AT_CH / AT_VB - 1): clamped inside the window's rows
 FNX_HOST_DEVICE inline int att_fetch_row(const AttWindow& w, int c0, int r) { return att_min(c0 + r, w.ctx_max - 1); }
-FNX_HOST_DEVICE inline int att_fetch_vblock(const AttWindow& w, int c0, int b) { return att_min((c0 >> 2) + b, (w.ctx_max - 1) >> 2); }
+FNX_HOST_DEVICE inline int att_fetch_vblock(const AttWindow& w, int c0, int b) { return att_min(c0 / AT_VB + b, (w.ctx_max - 1) / AT_VB); }
 // the splits whose parts the first pass wrote with data (the second pass reads these)
 FNX_HOST_DEVICE inline int att_live_splits(const AttWindow& w, int nsplit) { return att_min(nsplit, (w.ctx_max + AT_SPLIT - 1) / AT_SPLIT); }
 

@@ -1424,7 +1424,7 @@ int fnx_q8s_gemv_segs(const fnx_q8s* const* W, float* const* out, const int* out
 static int attn_prep_append(float* qg, float* k, const float* v, const float* q_norm, const float* k_norm, uint16_t* kc, uint16_t* vc, int nq,
                             int nkv, int T, const int* pos0, int max_ctx, float eps, const fnx_rope* rope, void* st, const int* gate) {
     if (!qg || !k || !v || !q_norm || !k_norm || !kc || !vc || !pos0 || !rope) return fail("attn_prep_append: null argument");
-    if (nq < 1 || nkv < 1 || nq % nkv || T < 1 || T > FNX_MAXT || max_ctx < 4 || max_ctx % 4) return fail("attn_prep_append: bad shape (the cache holds a multiple of 4 positions)");
+    if (nq < 1 || nkv < 1 || nq % nkv || T < 1 || T > FNX_MAXT || max_ctx < AT_VB || max_ctx % AT_VB) return fail("attn_prep_append: bad shape (the cache holds a multiple of 8 positions)");
     RopeDev r;
     for (int pair = 0; pair < AT_NROT / 2; ++pair) {   // rope.hpp:33-39
         const float fe = powf(rope->base, -2.0f * (float) pair / (float) AT_NROT);
@@ -1460,7 +1460,7 @@ static int attn_launch(const float* qg, const uint16_t* kc, const uint16_t* vc, 
     const int nsplit = attn_splits(max_ctx), waves = (T * (nq / nkv) + 15) / 16;
     float* acc = scratch;
     AttPart* mz = reinterpret_cast<AttPart*>(scratch + (size_t) T * nq * nsplit * AT_HD);
-    k_attn_part<<<dim3(nsplit, nkv, (waves + AT_WAVES - 1) / AT_WAVES), 64 * AT_WAVES, 0, (hipStream_t) st>>>(qg, kc, vc, acc, mz, nq, nkv, T,
+    k_attn_part<<<dim3(nsplit, nkv, (waves + AT_WAVES - 1) / AT_WAVES), AT_THREADS, 0, (hipStream_t) st>>>(qg, kc, vc, acc, mz, nq, nkv, T,
                                                                                                           nsplit, pos0, max_ctx, gate, live);
     k_attn_combine<<<dim3(nq, T), AT_HD, 0, (hipStream_t) st>>>(qg, acc, mz, out, outq, nq, nsplit, T, pos0, max_ctx, err, gate, live);
     return launch_status("attn");
@@ -1531,7 +1531,7 @@ static int dec_layer(const fnx_decoder* D, const fnx_dec_layer* L, int T, const 
 }
 static int dec_shape_check(const fnx_decoder* D, int T, const char* who) {
     if (D->n < 256 || D->n % 256 || D->n > 4096 || D->nq < 1 || D->nkv < 1 || D->nq % D->nkv || D->nq / D->nkv > AT_MAXQ || D->vocab < 1 ||
-        D->max_ctx < 4 || D->max_ctx % 4)
+        D->max_ctx < AT_VB || D->max_ctx % AT_VB)
         return fail(std::string(who) + ": bad model shape");
     if (T < 1 || T > FNX_MAXT) return fail(std::string(who) + ": T out of range");
     return 0;

@@ -346,9 +346,12 @@ struct RopeDev {
     float freq[AT_NROT / 2];
     float mscale;
 };
+__device__ __forceinline__ size_t vcache_at(int pos, int nkv, int kvh, int d) {   // the V cache's element index
+    return (((size_t) (pos / AT_VB) * nkv + kvh) * AT_HD + d) * AT_VB + (pos % AT_VB);
+}
 // block (head h, row t), AT_HD threads: q heads normed and rotated in place; k heads normed, rotated and appended; v heads
-// appended. The K cache is [position][kv head][AT_HD] f16; the V cache keeps four positions of a dimension together,
-// [position / 4][kv head][AT_HD][position % 4], which is what the matrix-core attention's V operand loads.
+// appended. The K cache is [position][kv head][AT_HD] f16; the V cache keeps eight positions of a dimension together,
+// [position / 8][kv head][AT_HD][position % 8]: 16 bytes, the matrix-core attention's V operand of one lane.
 __global__ void __launch_bounds__(AT_HD) k_attn_prep_append(float* __restrict__ qg, float* __restrict__ k, const float* __restrict__ v,
                                                            const float* __restrict__ qn, const float* __restrict__ kn,
                                                            uint16_t* __restrict__ kc, uint16_t* __restrict__ vc, int nq, int nkv,
@@ -389,7 +392,7 @@ __global__ void __launch_bounds__(AT_HD) k_attn_prep_append(float* __restrict__ 
     }
     if (p < 0 || p >= max_ctx) return;
     if (is_k) kc[((size_t) p * nkv + kh) * AT_HD + i] = float_to_half_bits(x);
-    else vc[(((size_t) (p >> 2) * nkv + kh) * AT_HD + i) * 4 + (p & 3)] = float_to_half_bits(x);   // vcache_at(p, nkv, kh, i)
+    else vc[vcache_at(p, nkv, kh, i)] = float_to_half_bits(x);
 }
 
 // ---------------------------------------------------------------- attention: split-K decode on the matrix cores
@@ -399,14 +402,17 @@ __global__ void __launch_bounds__(AT_HD) k_attn_prep_append(float* __restrict__ 
 // A window's rows times a kv head's q heads are up to 128 query vectors against the same K/V rows: a dense contraction,
 // so it runs on v_mfma_f32_16x16x32_f16. A block takes (split of AT_SPLIT positions, kv head, half of the query tiles);
 // a wave takes 16 queries (query = row * heads-per-kv + head). Per chunk of 32 positions:
-//   S^T = K Q^T  : A = K rows (lane: position l % 16, the 64 dims of lane group l / 16, 16 bytes a step from the cache),
-//                  B = Q^T (held in registers for the whole split, scaled by 1/16, as two f16 terms hi + lo);
-//                  the accumulator leaves lane (group pg, query q) with positions 4 pg .. 4 pg + 3 of both 16-position
-//                  tiles: the softmax of query q needs only in-lane work and two cross-group shuffles;
+//   S^T = K Q^T  : A = K rows (two tiles of 16 positions; row i of tile t is position 8 (i / 4) + 4 t + i % 4 of the chunk;
+//                  a lane holds the 64 dims of lane group l / 16, 16 bytes a step), B = Q^T (held in registers for the
+//                  whole split, scaled by 1/16, as two f16 terms hi + lo);
+//                  the accumulator leaves lane (group pg, query q) with rows 4 pg .. 4 pg + 3 of both tiles, which with
+//                  that order of the rows are positions 8 pg .. 8 pg + 7: the softmax of query q needs only in-lane work
+//                  and two cross-group shuffles;
 //   O^T += V^T P^T: those eight positions are exactly lane group pg's contraction slots, so P goes from the accumulator
-//                  registers straight into the B operand, and V^T's A operand is two 8-byte loads because the V cache
-//                  keeps four positions of a dimension together ([position / 4][kv head][dim][position % 4]).
-// The probabilities never pass through LDS; K and V chunks do, once per block (a chunk ahead, double-buffered). Each (query, split) leaves its maximum, sum and 256 accumulators; k_attn_combine merges.
+//                  registers straight into the B operand, and V^T's A operand is one 16-byte read because the V cache
+//                  keeps eight positions of a dimension together ([position / 8][kv head][dim][position % 8]).
+// The probabilities never pass through LDS; K and V chunks do, once per block, loaded straight into it two chunks ahead.
+// Each (query, split) leaves its maximum, sum and 256 accumulators; k_attn_combine merges.
 constexpr int AT_MAXQ = 8;   // AT_SPLIT, AT_CH: attn_window.h
 struct AttPart {
     float m, z;
@@ -417,9 +423,6 @@ typedef float at_v4f __attribute__((ext_vector_type(4)));
 typedef unsigned at_v4u __attribute__((ext_vector_type(4)));
 typedef unsigned at_v2u __attribute__((ext_vector_type(2)));
 
-__device__ __forceinline__ size_t vcache_at(int pos, int nkv, int kvh, int d) {   // the V cache's element index
-    return (((size_t) (pos >> 2) * nkv + kvh) * AT_HD + d) * 4 + (pos & 3);
-}
 
 // maximum / sum over the four lanes l, l ^ 16, l ^ 32, l ^ 48 (a query's four lane groups), left in all four: two row
 // swaps each instead of two trips through the LDS crossbar. (Inline asm, with the wait states the swap needs after a
@@ -438,9 +441,16 @@ __device__ __forceinline__ float groups4_sum(float v) {
     asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(x), "+v"(y));
     return x + y;
 }
-constexpr int AT_VPG = AT_HD * 16;   // LDS bytes of a lane group's V operands of a chunk: per dim the four positions of block pg, then those of block 4 + pg
-constexpr int AT_WAVES = 4, AT_KLD = 2 * AT_HD + 16;   // q tiles (of 16 queries) per block, blockIdx.z picks which; LDS bytes per K row
-__global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) k_attn_part(const float* __restrict__ qg, const uint16_t* __restrict__ kc,
+constexpr int AT_WAVES = 4;   // q tiles (of 16 queries) per block, blockIdx.z picks which
+constexpr int AT_THREADS = (AT_WAVES + 1) * 64;   // and one wave more that only brings the K and V chunks in
+// 64 lanes x 16 bytes from base + each lane's byte offset straight into LDS, laid down in lane order from lds_at on (a
+// wave-uniform LDS address, through M0). Written as an instruction so that the compiler, which cannot tell one LDS buffer
+// of such loads from another, does not wait for every one of them before each LDS read: the kernel counts them itself
+// (vmcnt) where it needs their data.
+__device__ __forceinline__ void lds_load16(const void* base, uint32_t lane_offset, uint32_t lds_at) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_at), "v"(lane_offset), "s"(base) : "memory");
+}
+__global__ void __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) k_attn_part(const float* __restrict__ qg, const uint16_t* __restrict__ kc,
                                                             const uint16_t* __restrict__ vc, float* __restrict__ acc_out,
                                                             AttPart* __restrict__ mz_out, int nq, int nkv, int T, int nsplit,
                                                             const int* __restrict__ pos0p, int max_ctx, const int* __restrict__ gate,
@@ -450,11 +460,12 @@ __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per
     // live (may be null): a device word, the rows of the window that count; the others' queries are left out (nothing reads
     // their results), the positions past the last row that counts with them
     const int s = blockIdx.x, kvh = blockIdx.y, lane = threadIdx.x & 63, wave = blockIdx.z * AT_WAVES + (threadIdx.x >> 6);
+    const bool loader = uniform((int) (threadIdx.x >> 6)) == AT_WAVES;   // the block's last wave: no queries, all the loads
     const int qpk = nq / nkv;
     // this lane's query row, 64 of its dims: loaded before anything that waits for a device word (a lane past the window's
     // queries reads the last query's row; its operands become zeros below)
     float4 qa[8], qb[8];
-    {
+    if (!loader) {
         const int qc = min(wave * 16 + (lane & 15), T * qpk - 1);
         const float* qr = qg + ((size_t) (qc / qpk) * nq + kvh * qpk + qc % qpk) * 2 * AT_HD + 64 * (lane >> 4);
 #pragma unroll
@@ -467,10 +478,10 @@ __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per
     const int nquery = T * qpk;
     const AttWindow win = att_window(*pos0p, T, max_ctx);   // no index below leaves the cache, whatever the device word holds
     if ((int) blockIdx.z * AT_WAVES * 16 >= nquery) return;   // none of the block's queries count
-    const bool wave_on = uniform(wave * 16 < nquery);         // a wave without queries still fetches its share of K and V
+    const bool wave_on = uniform(wave * 16 < nquery) && !loader;   // a wave without queries only meets the others
     const int ql = lane & 15, pg = lane >> 4;
     const int qi = wave * 16 + ql;                      // this lane's query (as B column / accumulator column)
-    const bool qlive = qi < nquery;
+    const bool qlive = qi < nquery && !loader;
     const int qt = qlive ? qi / qpk : 0, qh = kvh * qpk + (qlive ? qi % qpk : 0);
     const int ctx_q = qlive ? att_ctx_q(win, qt) : 0;   // positions [0, ctx_q) are this query's
     const int ctx_max = win.ctx_max;                    // the window's last row sees this many
@@ -481,64 +492,67 @@ __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per
         if (qlive && pg == 0) mz_out[slot] = AttPart{-INFINITY, 0.f};
         return;
     }
-    // A chunk's K rows (32 x 512 bytes) and V blocks (8 x 2048 bytes) are fetched once per block, 64 + 64 contiguous
-    // bytes per thread, a chunk ahead into registers and from there into one of two LDS buffers; the waves read their
-    // operands from LDS (K rows padded to 528 bytes: the 16 positions of a tile fall on different banks).
-    __shared__ __align__(16) uint8_t lk[2][AT_CH * AT_KLD];
-    __shared__ __align__(16) uint8_t lv[2][4 * AT_VPG];
-    const int tid = threadIdx.x;
-    const gbytes kbase = as_global(reinterpret_cast<const uint8_t*>(kc));
-    const gbytes vbase = as_global(reinterpret_cast<const uint8_t*>(vc));
-    // piece tid + 256 i of the chunk's 1024 16-byte pieces of K (32 to a row) and of V (128 to a block): consecutive lanes
-    // load consecutive pieces, so a wave's load is whole runs of 512 or 1024 bytes
+    // A chunk's K rows (32 x 512 bytes) and V blocks (8 x 2048 bytes) go from the caches straight into LDS
+    // (global_load_lds_dwordx4: a wave instruction lays its 64 lanes' 16-byte pieces down one after the other, 1 KiB from
+    // a wave-uniform address), two chunks ahead of the one being multiplied, into one of three stages; no registers and
+    // no stores of the block's own in between. 32 instructions a chunk, all issued by a wave of their own: the memory
+    // pipe takes an instruction every 16 cycles or so, and a wave that multiplies would stand still for a sixth of a
+    // chunk's time while its share is taken.
+    //   K: an instruction carries two rows. The LDS takes the rows' pieces in lane order, so the bank spread that padding
+    //      a row would give comes from which piece a lane loads: the second row of a pair holds piece c at place c ^ 2, and
+    //      a pair starts 1040 bytes after the one before (the 16 rows that an operand read touches then start at 16
+    //      different multiples of 16 bytes modulo 256).
+    //   V: an instruction carries a quarter of a block (64 dims x eight positions), the layout the operands are read in.
     // (byte offsets in 32 bits: the host refuses caches of 4 GiB and more)
-    const int krow = tid >> 5, kcol = tid & 31, vblk = tid >> 7, vcol = tid & 127;
-    const uint32_t krowb = (uint32_t) nkv * (AT_HD * 2), vblkb = (uint32_t) nkv * (AT_HD * 8);   // bytes between two rows of K, two blocks of V
-    const uint32_t koff0 = ((uint32_t) krow * nkv + kvh) * (AT_HD * 2) + 16 * kcol, voff0 = ((uint32_t) vblk * nkv + kvh) * (AT_HD * 8) + 16 * vcol;
-    at_v4u kr[4], vr[4];
-    int fc = 0;   // the chunk the registers hold
-    auto fetch = [&](int c0) {
-        fc = c0;
-        if (uniform(c0 + AT_CH <= ctx_max)) {   // a chunk inside the window's rows: a row or block is a constant further
-            const uint32_t ko = koff0 + (uint32_t) c0 * krowb, vo = voff0 + (uint32_t) (c0 >> 2) * vblkb;
+    constexpr int AT_STAGES = 3, AT_KPAIR = 2 * AT_HD * 2 + 16, AT_KSTAGE = (AT_CH / 2) * AT_KPAIR, AT_VBLK = AT_HD * AT_VB * 2, AT_VSTAGE = (AT_CH / AT_VB) * AT_VBLK;
+    __shared__ __align__(16) uint8_t lk[AT_STAGES * AT_KSTAGE];
+    __shared__ __align__(16) uint8_t lv[AT_STAGES * AT_VSTAGE];
+    const uint32_t lk_at = (uint32_t) (size_t) (__attribute__((address_space(3))) uint8_t*) lk, lv_at = (uint32_t) (size_t) (__attribute__((address_space(3))) uint8_t*) lv;
+    const uint32_t krowb = (uint32_t) nkv * (AT_HD * 2), vblkb = (uint32_t) nkv * AT_VBLK;   // bytes between two rows of K, two blocks of V
+    const int kh = lane >> 5;          // which row of a pair this lane loads, and
+    const uint32_t kpiece = 16u * ((uint32_t) (lane & 31) ^ (2u * kh));   // which piece of it
+    // chunk c0 into a stage: the loader wave's 32 instructions
+    auto fetch = [&](int c0, int stage) {
+        const bool inside = uniform(c0 + AT_CH <= ctx_max);   // a chunk inside the window's rows: no clamping
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                kr[i] = *(g128*) (kbase + (ko + 8 * i * krowb));
-                vr[i] = *(g128*) (vbase + (vo + 2 * i * vblkb));
-            }
-        } else {   // rows and blocks clamped inside the window's rows
+        for (int j = 0; j < AT_CH / 2; ++j) {   // K: rows c0 + 2 j, c0 + 2 j + 1
+            const int row = inside ? c0 + 2 * j + kh : att_fetch_row(win, c0, 2 * j + kh);
+            lds_load16(kc, (uint32_t) row * krowb + (uint32_t) kvh * (AT_HD * 2) + kpiece, lk_at + stage * AT_KSTAGE + j * AT_KPAIR);
+        }
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int pos = att_fetch_row(win, c0, krow + 8 * i), blk = att_fetch_vblock(win, c0, vblk + 2 * i);
-                kr[i] = *(g128*) (kbase + (((uint32_t) pos * nkv + kvh) * (AT_HD * 2) + 16 * kcol));
-                vr[i] = *(g128*) (vbase + (((uint32_t) blk * nkv + kvh) * (AT_HD * 8) + 16 * vcol));
-            }
+        for (int i = 0; i < 4 * (AT_CH / AT_VB); ++i) {   // V: quarter qq of block b of the chunk
+            const int b = i >> 2, qq = i & 3;
+            const int blk = inside ? c0 / AT_VB + b : att_fetch_vblock(win, c0, b);
+            lds_load16(vc, (uint32_t) blk * vblkb + (uint32_t) kvh * AT_VBLK + 1024u * qq + 16u * lane, lv_at + stage * AT_VSTAGE + b * AT_VBLK + qq * 1024);
         }
     };
-    // Positions past the window's rows were never written: whatever their cells hold must not reach the P V products (a
-    // zero probability does not stop a NaN). The slots of such positions are zeroed here, once per block and only in a
-    // chunk that reaches past the rows, instead of in every wave's operands; a block clamped to the window's last
-    // repeats that block, slots zeroed alike. A 16-byte piece is two dims x four positions of one block.
-    auto stash = [&](int buf) {
-        if (uniform(fc + AT_CH > ctx_max)) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int nv = ctx_max - 4 * att_fetch_vblock(win, fc, vblk + 2 * i);   // the block's written positions: 1 or more
-                const unsigned m01 = nv >= 2 ? ~0u : 0x0000FFFFu, m23 = nv >= 4 ? ~0u : nv == 3 ? 0x0000FFFFu : 0u;
-                vr[i] = at_v4u{vr[i].x & m01, vr[i].y & m23, vr[i].z & m01, vr[i].w & m23};
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            *reinterpret_cast<at_v4u*>(&lk[buf][(krow + 8 * i) * AT_KLD + 16 * kcol]) = kr[i];
-            // block b's dims 2 vcol and 2 vcol + 1 (8 bytes each: four positions) into half b / 4 of lane group b % 4's 16-byte operands
-            const int b = vblk + 2 * i;
-            uint8_t* dst = &lv[buf][(b & 3) * AT_VPG + 32 * vcol + 8 * (b >> 2)];
-            *reinterpret_cast<at_v2u*>(dst) = at_v2u{vr[i].x, vr[i].y};
-            *reinterpret_cast<at_v2u*>(dst + 16) = at_v2u{vr[i].z, vr[i].w};
-        }
+    // The block meets where a chunk's pieces must all have landed. The loader's loads complete in order, so it waits until
+    // only the newest chunk's 32 may be on their way (or none); the others wait for their LDS reads and writes; then all
+    // for one another. (A plain barrier instruction: __syncthreads() would also wait for the loads that are meant to stay
+    // in flight.)
+    auto meet = [&](bool newest_in_flight) {
+        __builtin_amdgcn_sched_barrier(0);
+        if (newest_in_flight) __builtin_amdgcn_s_waitcnt(0x8070);   // vmcnt(32) lgkmcnt(0)
+        else __builtin_amdgcn_s_waitcnt(0x0070);                    // vmcnt(0) lgkmcnt(0)
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
     };
-    fetch(p0);
+    // The loader: two chunks ahead of the others, meeting them at every barrier of theirs (one when the first chunk has
+    // landed, one at the end of every chunk, and one more in a chunk that reaches past the window's rows, whose V slots the
+    // others then zero).
+    if (loader) {
+        fetch(p0, 0);
+        if (p0 + AT_CH < p1) fetch(p0 + AT_CH, 1);
+        meet(p0 + AT_CH < p1);
+        int stage = 0;
+        for (int c0 = p0; c0 < p1; c0 += AT_CH, stage = stage == AT_STAGES - 1 ? 0 : stage + 1) {
+            if (uniform(c0 + AT_CH > ctx_max)) meet(false);
+            const bool more2 = uniform(c0 + 2 * AT_CH < p1);
+            if (more2) fetch(c0 + 2 * AT_CH, stage == 0 ? 2 : stage - 1);   // into the stage that the chunk before this one left
+            meet(more2);
+        }
+        return;
+    }
     // Q^T operands: step ks holds dims 64 pg + 8 ks .. + 7 of query ql, times 1/16 (exact), as two f16 terms hi + lo:
     // the cache is f16 already, so with q (and below the probabilities) split this way the products carry fp32's
     // precision, as the reference's f32 arithmetic on the f16 cache does. (Converted while the first chunk is on its way.)
@@ -561,27 +575,39 @@ __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per
 #pragma unroll
     for (int dt = 0; dt < 16; ++dt) O[dt] = at_v4f{0.f, 0.f, 0.f, 0.f};
     float m = -INFINITY, z = 0.f;
-    stash(0);
-    fetch(min(p0 + AT_CH, p1 - 1));
-    __syncthreads();
-    int buf = 0;
-    for (int c0 = p0; c0 < p1; c0 += AT_CH, buf ^= 1) {
+    meet(false);
+    // lane (ql, pg) as row ql of a tile of K: position 8 (ql / 4) + ql % 4 of the chunk (tile 1: four further, two pairs);
+    // an odd row is the second of its pair, where piece c lies at c ^ 2: steps 0, 1, 4, 5 and steps 2, 3, 6, 7 from two bases
+    const int krow = 8 * (ql >> 2) + (ql & 3), kswz = 32 * (krow & 1);
+    const uint8_t* kev = lk + (krow >> 1) * AT_KPAIR + (krow & 1) * (AT_HD * 2) + 128 * pg + kswz;
+    const uint8_t* kod = kev - 2 * kswz;
+    const uint8_t* vlane = lv + pg * AT_VBLK + 16 * ql;   // dim ql of block pg: the operand of dim tile dt lies 256 dt further
+    int stage = 0;
+    for (int c0 = p0; c0 < p1; c0 += AT_CH, stage = stage == AT_STAGES - 1 ? 0 : stage + 1) {
+        // Positions past the window's rows were never written: whatever their cells hold must not reach the P V products (a
+        // zero probability does not stop a NaN). In a chunk that reaches past the rows - the last one of a context, no
+        // other - their slots of the V stage are zeroed here, thread by dimension (a block clamped to the window's last
+        // repeats that block: all of its slots are past the rows).
+        if (uniform(c0 + AT_CH > ctx_max)) {
+            for (int p = max(ctx_max - c0, 0); p < AT_CH; ++p)   // (threads 0 .. 255: the loader is not here)
+                *reinterpret_cast<volatile uint16_t*>(lv + stage * AT_VSTAGE + (p / AT_VB) * AT_VBLK + threadIdx.x * (AT_VB * 2) + 2 * (p % AT_VB)) = 0;
+            meet(false);   // (nothing is in flight in a context's last chunk)
+        }
         // The K operands are read a group (two steps of both tiles: four 16-byte reads) ahead of the products that use them,
         // the first group before the block's own stores and loads below: after the barrier the four waves ask the LDS for
         // the same rows at the same time, and a read that is only issued when it is needed waits for all four.
-        const uint8_t* k0 = &lk[buf][ql * AT_KLD + 128 * pg];
-        const uint8_t* k1 = k0 + 16 * AT_KLD;
+        const uint8_t* k0a = kev + stage * AT_KSTAGE;   // tile 0, steps 0, 1, 4, 5; tile 1 lies two pairs further
+        const uint8_t* k0b = kod + stage * AT_KSTAGE;   // steps 2, 3, 6, 7
         at_v4u kq[2][4];
-        auto kread = [&](int g, at_v4u (&o)[4]) {
+        auto kread = [&](int g, at_v4u (&o)[4]) {   // steps 2 g and 2 g + 1 of both tiles
+            const uint8_t* k0 = (g & 1) ? k0b : k0a;
             o[0] = *reinterpret_cast<const at_v4u*>(k0 + 32 * g);
-            o[1] = *reinterpret_cast<const at_v4u*>(k1 + 32 * g);
+            o[1] = *reinterpret_cast<const at_v4u*>(k0 + 2 * AT_KPAIR + 32 * g);
             o[2] = *reinterpret_cast<const at_v4u*>(k0 + 32 * g + 16);
-            o[3] = *reinterpret_cast<const at_v4u*>(k1 + 32 * g + 16);
+            o[3] = *reinterpret_cast<const at_v4u*>(k0 + 2 * AT_KPAIR + 32 * g + 16);
         };
         if (wave_on) kread(0, kq[0]);
         __builtin_amdgcn_sched_barrier(0);
-        stash(buf ^ 1);                              // chunk c0 + 32, fetched during the last iteration
-        fetch(min(c0 + 2 * AT_CH, p1 - 1));          // past the split: some rows again, never used
         if (wave_on) {
         // the two tiles' hi and lo terms in chains of their own, interleaved: a chain's next MFMA is four issues away, so
         // none waits for the one before it
@@ -606,7 +632,7 @@ __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per
             S[0] = a0 + a0l;
             S[1] = a1 + a1l;
         }
-        // this lane: query ql, positions c0 + 4 pg + r (tile 0) and c0 + 16 + 4 pg + r (tile 1). A chunk that every query of
+        // this lane: query ql, positions c0 + 8 pg + r (tile 0) and c0 + 8 pg + 4 + r (tile 1). A chunk that every query of
         // the wave sees whole (all but the last ones of a context) needs no masks: its maximum is finite
         float pw[8], ps = 0.f, mn, sc;
         if (uniform(c0 + AT_CH <= vis)) {
@@ -623,7 +649,7 @@ __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per
             float mx = -INFINITY;
 #pragma unroll
             for (int r = 0; r < 8; ++r) {
-                const int pos = c0 + 16 * (r >> 2) + 4 * pg + (r & 3);
+                const int pos = c0 + 8 * pg + r;
                 sv[r] = pos < ctx_q && pos < p1 ? S[r >> 2][r & 3] : -INFINITY;
                 mx = fmaxf(mx, sv[r]);
             }
@@ -646,8 +672,8 @@ __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per
             P[r] = hi;
             Pl[r] = (_Float16) (pw[r] - (float) hi);
         }
-        // V^T operands: positions c0 + 4 pg .. + 3 (block pg of the chunk) and c0 + 16 + 4 pg .. + 3 (block 4 + pg), dim
-        // 16 dt + ql (slots past the window's rows hold zeros: stash)
+        // V^T operands: positions c0 + 8 pg .. + 7 (block pg of the chunk), dim 16 dt + ql (slots past the window's rows
+        // hold zeros: see the loop's top)
         if (__any(sc != 1.0f)) {   // the running maximum moved (rare once the first chunks are behind)
 #pragma unroll
             for (int dt = 0; dt < 16; ++dt) {
@@ -657,7 +683,7 @@ __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per
                 O[dt].w *= sc;
             }
         }
-        const uint8_t* vb = &lv[buf][pg * AT_VPG + ql * 16];   // dim 16 dt + ql: one 16-byte read, the operand's register order
+        const uint8_t* vb = vlane + stage * AT_VSTAGE;
         // four dim tiles at a time: the lo products of all four, then the hi ones (a chain's next MFMA four issues away);
         // the next four tiles' V reads are issued before this group's arithmetic
         at_v4u ra[2][4];
@@ -680,7 +706,7 @@ __global__ void __launch_bounds__(AT_WAVES * 64) __attribute__((amdgpu_waves_per
             __builtin_amdgcn_sched_barrier(0);
         }
         }
-        __syncthreads();
+        meet(false);   // the next chunk's pieces have landed, and this chunk's stage is free for the chunk after it
     }
     if (!qlive) return;
     // accumulator lane (dim group pg, query ql): dims 16 dt + 4 pg + r

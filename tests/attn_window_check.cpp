@@ -19,9 +19,9 @@ static void require(bool ok, const char* what, int max_ctx, int pos0, int T, int
 }
 
 int main() {
-    const int caps[] = {4, 192, 520, 32768};
+    const int caps[] = {8, 192, 520, 32768};
     for (int max_ctx : caps) {
-        const int nsplit = attn_splits(max_ctx), vblocks = (max_ctx + 3) / 4;
+        const int nsplit = attn_splits(max_ctx), vblocks = (max_ctx + AT_VB - 1) / AT_VB;
         const int step = max_ctx > 1024 ? 97 : 1;
         for (int pos0 = -40; pos0 <= max_ctx + 40; pos0 += (pos0 > 64 && pos0 < max_ctx - 64 ? step : 1))
             for (int T = 1; T <= 16; ++T) {
@@ -48,15 +48,16 @@ int main() {
                             const int row = att_fetch_row(w, c0, r);
                             require(row >= 0 && row < max_ctx, "K row", max_ctx, pos0, T, s, c0);
                         }
-                        for (int b = 0; b < AT_CH / 4; ++b) {
+                        for (int b = 0; b < AT_CH / AT_VB; ++b) {
                             const int blk = att_fetch_vblock(w, c0, b);
                             require(blk >= 0 && blk < vblocks, "V block", max_ctx, pos0, T, s, c0);
                         }
                     };
-                    // the kernel's order: the first chunk, the second (or the split's last row), then two ahead each trip
+                    // the kernel's order: the first chunk, the second if the split has one, then two ahead each trip
                     fetch(p0);
-                    fetch(att_min(p0 + AT_CH, p1 - 1));
-                    for (int c0 = p0; c0 < p1; c0 += AT_CH) fetch(att_min(c0 + 2 * AT_CH, p1 - 1));
+                    if (p0 + AT_CH < p1) fetch(p0 + AT_CH);
+                    for (int c0 = p0; c0 < p1; c0 += AT_CH)
+                        if (c0 + 2 * AT_CH < p1) fetch(c0 + 2 * AT_CH);
                 }
             }
     }

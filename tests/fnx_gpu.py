@@ -66,20 +66,24 @@ def pack_unit64(raw):
 JOB_DTYPE = np.dtype([("w", "<i4"), ("n", "<i4"), ("y", "<i4", (16,)), ("out", "<i4", (16,))])
 
 
+V_BLOCK = 8   # positions of a dimension that lie together in the library's V cache
+
+
 def v_blocked(vc):
-    """[pos][nkv][256] -> the library's V cache layout [pos / 4][nkv][256][pos % 4] (pos a multiple of 4)"""
+    """[pos][nkv][256] -> the library's V cache layout [pos / 8][nkv][256][pos % 8] (pos a multiple of 8)"""
     p, nkv, hd = vc.shape
-    return np.ascontiguousarray(vc.reshape(p // 4, 4, nkv, hd).transpose(0, 2, 3, 1))
+    return np.ascontiguousarray(vc.reshape(p // V_BLOCK, V_BLOCK, nkv, hd).transpose(0, 2, 3, 1))
 
 
 def v_rows(vb):
     """the inverse of v_blocked"""
     b, nkv, hd, _ = vb.shape
-    return np.ascontiguousarray(vb.transpose(0, 3, 1, 2)).reshape(b * 4, nkv, hd)
+    return np.ascontiguousarray(vb.transpose(0, 3, 1, 2)).reshape(b * V_BLOCK, nkv, hd)
 
 
 def pad4(a):
-    extra = (-a.shape[0]) % 4
+    """rows up to a whole block of the V cache"""
+    extra = (-a.shape[0]) % V_BLOCK
     return a if not extra else np.concatenate([a, np.zeros((extra,) + a.shape[1:], dtype=a.dtype)])
 
 
@@ -419,7 +423,7 @@ class DecoderDev:
         out = []
         for kc, vc in self.caches + [self.mtp_cache]:
             k = kc.cpu().numpy().view(np.uint16)
-            v = vc.cpu().numpy().view(np.uint16).reshape(self.c["max_ctx"] // 4, self.c["nkv"], 256, 4)
+            v = vc.cpu().numpy().view(np.uint16).reshape(self.c["max_ctx"] // V_BLOCK, self.c["nkv"], 256, V_BLOCK)
             out.append((k, v_rows(v)))
         return out
 
@@ -427,7 +431,7 @@ class DecoderDev:
         """cells: per layer (the draft layer last) a pair of [pos][nkv][256] float16 arrays, written from position 0"""
         for (kc, vc), (k, v) in zip(self.caches + [self.mtp_cache], cells):
             p = k.shape[0]
-            assert p % 4 == 0 and p <= self.c["max_ctx"]
+            assert p % V_BLOCK == 0 and p <= self.c["max_ctx"]
             kc[:p].copy_(self.dev.up(np.ascontiguousarray(k)))
             vc.view(self.dev.torch.float16).reshape(-1)[:v.size].copy_(self.dev.up(v_blocked(v)).reshape(-1))
         self.dev.sync()
