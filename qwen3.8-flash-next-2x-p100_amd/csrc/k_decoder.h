@@ -429,16 +429,16 @@ typedef unsigned at_v2u __attribute__((ext_vector_type(2)));
 // vector write, as for the other uses of these swaps.)
 __device__ __forceinline__ float groups4_max(float v) {
     float x = v, y = v;
-    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(x), "+v"(y));
+    asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(x), "+v"(y));
     x = y = fmaxf(x, y);
-    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(x), "+v"(y));
+    asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(x), "+v"(y));
     return fmaxf(x, y);
 }
 __device__ __forceinline__ float groups4_sum(float v) {
     float x = v, y = v;
-    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(x), "+v"(y));
+    asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(x), "+v"(y));
     x = y = x + y;
-    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(x), "+v"(y));
+    asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(x), "+v"(y));
     return x + y;
 }
 constexpr int AT_WAVES = 4;   // q tiles (of 16 queries) per block, blockIdx.z picks which
@@ -632,6 +632,16 @@ __global__ void __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu
             S[0] = a0 + a0l;
             S[1] = a1 + a1l;
         }
+        const uint8_t* vb = vlane + stage * AT_VSTAGE;
+        // four dim tiles at a time: the lo products of all four, then the hi ones (a chain's next MFMA four issues away);
+        // the next four tiles' V reads are issued before this group's arithmetic
+        at_v4u ra[2][4];
+        auto vread = [&](int d0, at_v4u (&o)[4]) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) o[u] = *reinterpret_cast<const at_v4u*>(vb + 256 * (d0 + u));
+        };
+        vread(0, ra[0]);   // (on its way during the softmax below)
+        __builtin_amdgcn_sched_barrier(0);
         // this lane: query ql, positions c0 + 8 pg + r (tile 0) and c0 + 8 pg + 4 + r (tile 1). A chunk that every query of
         // the wave sees whole (all but the last ones of a context) needs no masks: its maximum is finite
         float pw[8], ps = 0.f, mn, sc;
@@ -683,15 +693,6 @@ __global__ void __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu
                 O[dt].w *= sc;
             }
         }
-        const uint8_t* vb = vlane + stage * AT_VSTAGE;
-        // four dim tiles at a time: the lo products of all four, then the hi ones (a chain's next MFMA four issues away);
-        // the next four tiles' V reads are issued before this group's arithmetic
-        at_v4u ra[2][4];
-        auto vread = [&](int d0, at_v4u (&o)[4]) {
-#pragma unroll
-            for (int u = 0; u < 4; ++u) o[u] = *reinterpret_cast<const at_v4u*>(vb + 256 * (d0 + u));
-        };
-        vread(0, ra[0]);
 #pragma unroll
         for (int gq = 0; gq < 4; ++gq) {
             if (gq < 3) vread(4 * (gq + 1), ra[(gq + 1) & 1]);
