@@ -793,7 +793,12 @@ def prefill_main(args):
                      "unit": "GB/s", "frac": gu_bytes / (gu_ms * 1e-3) / HBM_PEAK, "traffic": None, "kernel_ms": gu_ms, "algorithmic_bytes": gu_bytes,
                      "mfma_tflops": gu_flops / (gu_ms * 1e-3) / 1e12, "mfma_frac": gu_flops / (gu_ms * 1e-3) / MFMA_F16,
                      "down": {"kernel_ms": dn_ms, "achieved": dn_bytes / (dn_ms * 1e-3) / 1e9, "mfma_tflops": dn_flops / (dn_ms * 1e-3) / 1e12},
-                     "swiglu_ms": sw_ms},
+                     "swiglu_ms": sw_ms,
+                     # the piecewise bound: a launch cannot be faster than its bytes at the HBM peak or its flops at the MFMA peak
+                     "piecewise_bound": {"gate_up_us": max(gu_bytes / HBM_PEAK, gu_flops / MFMA_F16) * 1e6,
+                                         "gate_up_frac": max(gu_bytes / HBM_PEAK, gu_flops / MFMA_F16) / (gu_ms * 1e-3),
+                                         "chunk_us": max(step_bytes / HBM_PEAK, step_flops / MFMA_F16) * 1e6,
+                                         "chunk_frac": max(step_bytes / HBM_PEAK, step_flops / MFMA_F16) / (dt / steps)}},
         "cpu_baseline": cpu,
     }
     print(json.dumps(line))
