@@ -1280,6 +1280,14 @@ static int mma_launch(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const 
         a.ffh = A->n_out / 2;
         if (h16_done) *h16_done = true;
     }
+    static const int tok64 = env_int("FNX_MMA_TOK64", 1, 0, 1);
+    if (use_tile && tok64) {
+        // tile form, a block per (job, its up to 64 tokens, 256 rows) in stages of 256 columns, one block a CU (its LDS)
+        const long tasks = caps * ((A->n_out + MB_ROWS - 1) / MB_ROWS);
+        const int grid = (int) std::max(1l, std::min<long>((long) cu_count(), tasks));
+        k_moe_mma_tile64<<<grid, MM_THREADS, 0, (hipStream_t) st>>>(a);
+        return launch_status(who);
+    }
     if (use_tile) {
         // tile form: a block per (job, 32 tokens, 256 rows) in stages of 256 columns, one block a CU (its LDS)
         const long tasks = caps * ((A->n_out + MB_ROWS - 1) / MB_ROWS) * (MM_TT / MM_TP);
@@ -1287,7 +1295,6 @@ static int mma_launch(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const 
         k_moe_mma_tile<<<grid, MM_THREADS, 0, (hipStream_t) st>>>(a);
         return launch_status(who);
     }
-    static const int tok64 = env_int("FNX_MMA_TOK64", 1, 0, 1);
     if (use_block && tok64) {
         // block form, a block per (job, its up to 64 tokens, 256 rows): one block a CU (its LDS)
         const long tasks = caps * ((A->n_out + MB_ROWS - 1) / MB_ROWS);

@@ -1278,4 +1278,291 @@ __global__ void __launch_bounds__(MM_THREADS) __attribute__((amdgpu_waves_per_eu
 }
 
 
+// ---------------------------------------------------------------- the tile form with a job's up to 64 tokens a task
+// As k_moe_mma_tile, but a task is (job, all of its token tiles, 256 rows): the weights of a stage are decoded once for
+// up to four token tiles instead of once for every two (a job of 33 to 64 tokens no longer decodes twice), the jobs are
+// ranked by token tiles and the tasks dealt to and fro over the blocks, and the activation tile of 64 tokens is single:
+// it is replaced between two barriers while the next stage's weights are already in the other weight buffer.
+constexpr int MT_TP64 = 4, MT_TOK64 = 16 * MT_TP64, MT_MAXTASK64 = 6;
+struct TileLds64 {
+    uint2 tab[SGRID_WORDS];
+    uint8_t wt[2][MB_ROWS * MT_WROW];
+    uint8_t xt[MT_TOK64 * MT_XROW];
+    int ytok[MT_MAXTASK64][MT_TOK64];
+    int otok[MT_MAXTASK64][MT_TOK64];
+    TileTask task[MT_MAXTASK64];
+    int ntask;
+    uint8_t jkey[MB_SORTJ];
+    unsigned short jorder[MB_SORTJ];
+};
+struct TileStaged64 {
+    v4u a[2], b, x[4];
+    v2u cs;
+};
+__global__ void __launch_bounds__(MM_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) k_moe_mma_tile64(const MmaArgs a) {
+    typedef __attribute__((address_space(1))) const v4u g128;
+    typedef __attribute__((address_space(1))) const v2u g64;
+    typedef __attribute__((address_space(1))) const uint32_t g32;
+    typedef __attribute__((address_space(1))) const unsigned short g16;
+    __shared__ TileLds64 L;
+    const int tid = threadIdx.x, lane = tid & 63, wave = uniform(tid >> 6), r = lane & 15, g = lane >> 4;
+    static_assert(MM_THREADS == 512, "a thread per 9-bit code: its sixteen signed entries are made from the first");
+    const uint32_t tab0 = g_sgrid.v[tid];
+    const int nj = min(a.cap, uniform(*a.njobs)), nj2 = a.jobs2 ? min(a.cap2, uniform(*a.njobs2)) : 0;
+    const int ks = a.ncols >> 5, nsuper = a.ncols / MT_K, rblocks = (a.nrows + MB_ROWS - 1) / MB_ROWS;
+    constexpr int HALVES = 1;   // a task takes all of a job's token tiles
+    const int per_job = rblocks * HALVES, ntasks_all = (nj + nj2) * per_job;
+#pragma unroll
+    for (int i = 0; i < SGRID_WORDS / MM_THREADS; ++i) {
+        const uint32_t gg = signed_entry(tab0, i);
+        v2h lo, hi;
+        lo.x = (_Float16) (int) (int8_t) (gg & 0xFFu);
+        lo.y = (_Float16) (int) (int8_t) ((gg >> 8) & 0xFFu);
+        hi.x = (_Float16) (int) (int8_t) ((gg >> 16) & 0xFFu);
+        hi.y = (_Float16) (int) (int8_t) (gg >> 24);
+        L.tab[tid + i * MM_THREADS] = make_uint2(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi));
+    }
+    // the jobs ranked by token tiles and the tasks dealt in that order, to and fro over the blocks (as k_moe_mma_block64 does)
+    const int njall = nj + nj2;
+    const bool sorted = njall <= MB_SORTJ;
+    if (sorted && wave == 0) {
+        auto key_of = [&](int j) {
+            if (j >= njall) return -1;
+            const fnx_bigjob* jb = j < nj ? a.jobs + j : a.jobs2 + (j - nj);
+            return min(MT_TP64, (max(0, min(FNX_PF_JOB, jb->n)) + 15) >> 4);
+        };
+        int total[MT_TP64 + 1];
+#pragma unroll
+        for (int c = 0; c <= MT_TP64; ++c) total[c] = 0;
+        for (int j0 = 0; j0 < njall; j0 += 64) {
+            const int kj = key_of(j0 + lane);
+            if (j0 + lane < njall) L.jkey[j0 + lane] = (uint8_t) kj;
+#pragma unroll
+            for (int c = 0; c <= MT_TP64; ++c) total[c] += __popcll(__ballot(kj == c));
+        }
+        int base[MT_TP64 + 1];   // where a class starts: the classes in descending order
+        base[MT_TP64] = 0;
+#pragma unroll
+        for (int c = MT_TP64 - 1; c >= 0; --c) base[c] = base[c + 1] + total[c + 1];
+        for (int j0 = 0; j0 < njall; j0 += 64) {
+            const int kj = j0 + lane < njall ? (int) L.jkey[j0 + lane] : -1;
+#pragma unroll
+            for (int c = 0; c <= MT_TP64; ++c) {
+                const unsigned long long m = __ballot(kj == c);
+                if (kj == c) L.jorder[base[c] + __popcll(m & ((1ull << lane) - 1ull))] = (unsigned short) (j0 + lane);
+                base[c] += __popcll(m);
+            }
+        }
+    }
+    for (int k0 = 0; k0 * (int) gridDim.x < ntasks_all; k0 += MT_MAXTASK64) {   // MT_MAXTASK64 rounds a pass
+        __syncthreads();   // the previous lists' and tiles' last readers; the table and the jobs' order on the first pass
+        if (wave == 0) {
+            const int round = k0 + lane, pos = (round & 1) ? (int) gridDim.x - 1 - (int) blockIdx.x : (int) blockIdx.x;
+            const int task = round * (int) gridDim.x + pos;
+            bool ok = lane < MT_MAXTASK64 && task < ntasks_all;
+            TileTask t{};
+            int ji = 0, n = 0;
+            if (ok) {
+                ji = task / per_job;
+                const int rem = task - ji * per_job;
+                if (sorted) ji = L.jorder[ji];
+                t.t0 = 0;
+                t.row0 = (rem % rblocks) * MB_ROWS;
+                const fnx_bigjob* jb = ji < nj ? a.jobs + ji : a.jobs2 + (ji - nj);
+                n = min(FNX_PF_JOB, jb->n);
+                const int e = jb->w;
+                ok = n >= 1 && t.t0 < ((n + 15) >> 4);
+                t.ntile = min(MT_TP64, (n + 15) >> 4);
+                if (ok) t.we = ji >= nj ? a.w2 : a.ep ? (const uint8_t*) a.ep[e] : a.w + (size_t) e * a.stride;
+            }
+            const unsigned long long m = __ballot(ok);
+            const int slot = __popcll(m & ((1ull << lane) - 1ull));
+            if (ok) {
+                t.ji = ji;
+                t.n = n;
+                L.task[slot] = t;
+            }
+            if (lane == 0) L.ntask = __popcll(m);
+        }
+        __syncthreads();
+        const int ntask = L.ntask;
+        if (ntask == 0) continue;   // the same for every thread of the block
+        for (int i = tid; i < ntask * MT_TOK64; i += MM_THREADS) {   // the tiles' token and output rows (64 of each), all at once
+            const int slot = i / MT_TOK64, j = i % MT_TOK64, ji = L.task[slot].ji, n = L.task[slot].n, tok = L.task[slot].t0 * 16 + j;
+            const fnx_bigjob* jb = ji < nj ? a.jobs + ji : a.jobs2 + (ji - nj);
+            L.ytok[slot][j] = jb->y[min(tok, n - 1)];
+            L.otok[slot][j] = tok < n ? jb->out[tok] : -1;
+        }
+        __syncthreads();
+        const int nst = ntask * nsuper;
+        auto issue = [&](int ti, int S) {
+            const TileTask t = L.task[ti];
+            auto unit_of = [&](int rowl, uint32_t& l0) {
+                const int row = min(t.row0 + rowl, a.nrows - 1);
+                const uint32_t Lq = (uint32_t) row * ks + 8 * S;
+                l0 = Lq & 63u;
+                return as_global(t.we + (size_t) (Lq >> 6) * UNIT_BYTES);
+            };
+            TileStaged64 o{};
+            uint32_t l0;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const int c = tid + i * MM_THREADS;
+                const gbytes u = unit_of(c >> 2, l0);
+                o.a[i] = *(g128*) (u + 8 * l0 + 16 * (c & 3));
+            }
+            {
+                const gbytes u = unit_of(tid >> 1, l0);
+                o.b = *(g128*) (u + UNIT_B_AT + 4 * l0 + 16 * (tid & 1));
+            }
+            if (wave < MM_WAVES / 2) {
+                const gbytes u = unit_of(tid, l0);
+                o.cs = *(g64*) (u + UNIT_C_AT + l0);
+            } else {
+                const gbytes u = unit_of(tid - MM_THREADS / 2, l0);
+                o.cs.x = *(g32*) (u + UNIT_SCALES_AT + (l0 >> 1));
+                o.cs.y = *(g16*) (u + UNIT_D_AT + 2 * (l0 >> 3));
+            }
+            // tokens tid / 16 and 32 further, 2 x 16 bytes of the stage's 512 each; only the token tiles the task has
+            const int ntok = 16 * t.ntile;
+            const g128* xp = (g128*) (uintptr_t) (a.x + (size_t) L.ytok[ti][tid >> 4] * a.ldx + S * MT_K + 8 * (tid & 15));
+            const g128* xq = (g128*) (uintptr_t) (a.x + (size_t) L.ytok[ti][(tid >> 4) + 32] * a.ldx + S * MT_K + 8 * (tid & 15));
+            if ((tid >> 4) < ntok) {
+                o.x[0] = xp[0];
+                o.x[1] = xp[16];   // + 256 bytes
+            }
+            if ((tid >> 4) + 32 < ntok) {
+                o.x[2] = xq[0];
+                o.x[3] = xq[16];
+            }
+            return o;
+        };
+        auto stash_w = [&](const TileStaged64& o, int buf) {
+            uint8_t* w = L.wt[buf];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const int c = tid + i * MM_THREADS;
+                *reinterpret_cast<v4u*>(w + (c >> 2) * MT_WROW + 16 * (c & 3)) = o.a[i];
+            }
+            *reinterpret_cast<v4u*>(w + (tid >> 1) * MT_WROW + 64 + 16 * (tid & 1)) = o.b;
+            if (wave < MM_WAVES / 2) *reinterpret_cast<v2u*>(w + tid * MT_WROW + 96) = o.cs;
+            else {
+                *reinterpret_cast<uint32_t*>(w + (tid - MM_THREADS / 2) * MT_WROW + 104) = o.cs.x;
+                *reinterpret_cast<uint16_t*>(w + (tid - MM_THREADS / 2) * MT_WROW + 108) = (uint16_t) o.cs.y;
+            }
+        };
+        auto stash_x = [&](const TileStaged64& o) {   // (zeros for a tile the task does not have: its products go nowhere)
+            uint8_t* x = L.xt + (tid >> 4) * MT_XROW + 16 * (tid & 15);
+            *reinterpret_cast<v4u*>(x) = o.x[0];
+            *reinterpret_cast<v4u*>(x + 256) = o.x[1];
+            *reinterpret_cast<v4u*>(x + 32 * MT_XROW) = o.x[2];
+            *reinterpret_cast<v4u*>(x + 32 * MT_XROW + 256) = o.x[3];
+        };
+        v4f acc[MB_RG][MT_TP64];
+#pragma unroll
+        for (int q = 0; q < MB_RG; ++q)
+#pragma unroll
+            for (int tt = 0; tt < MT_TP64; ++tt) acc[q][tt] = v4f{0.f, 0.f, 0.f, 0.f};
+        struct Gath {
+            uint2 e[8];
+        };
+        auto gather = [&](const TileFields& f, int p, Gath& o) {
+            const v4u idx = {f.A[2 * p], f.A[2 * p + 1], f.B[p], (f.C >> (8 * p)) & 0xFFu};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) o.e[j] = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint8_t*>(L.tab) + 2 * packed_addr(idx, j));
+        };
+        auto bread = [&](int p, v4u (&B)[MT_TP64][4], auto nt_tag) {
+#pragma unroll
+            for (int tt = 0; tt < decltype(nt_tag)::value; ++tt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) B[tt][i] = *reinterpret_cast<const v4u*>(&L.xt[(tt * 16 + r) * MT_XROW + 128 * g + 64 * p + 16 * i]);
+        };
+        auto math = [&](const TileFields& f, int p, int q, const Gath& in, const v4u (&B)[MT_TP64][4], auto nt_tag) {
+            const _Float16 sc = (_Float16) (int) (1 + 2 * ((f.sc >> (4 * p)) & 0xFu)), d = __builtin_bit_cast(_Float16, (unsigned short) f.d);
+            const v2h s2 = {sc, sc}, d2 = {d, d};
+            v8h A[4];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const v2h wl = (as_v2h(in.e[j].x) * s2) * d2, wh = (as_v2h(in.e[j].y) * s2) * d2;
+                A[j >> 1][4 * (j & 1) + 0] = wl.x;
+                A[j >> 1][4 * (j & 1) + 1] = wl.y;
+                A[j >> 1][4 * (j & 1) + 2] = wh.x;
+                A[j >> 1][4 * (j & 1) + 3] = wh.y;
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int tt = 0; tt < decltype(nt_tag)::value; ++tt)
+                    acc[q][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[i], __builtin_bit_cast(v8h, B[tt][i]), acc[q][tt], 0, 0, 0);
+        };
+        auto compute = [&](int buf, auto nt_tag) {
+            const uint8_t* w = L.wt[buf];
+            TileFields f[MB_RG];
+#pragma unroll
+            for (int q = 0; q < MB_RG; ++q) {
+                const uint8_t* rec = w + (wave * 16 * MB_RG + 16 * q + r) * MT_WROW;
+                f[q].A = *reinterpret_cast<const v4u*>(rec + 16 * g);
+                f[q].B = *reinterpret_cast<const v2u*>(rec + 64 + 8 * g);
+                f[q].C = *reinterpret_cast<const uint16_t*>(rec + 96 + 2 * g);
+                f[q].sc = rec[104 + g];
+                f[q].d = *reinterpret_cast<const uint16_t*>(rec + 108);
+            }
+            Gath G[2];
+            v4u Bb[MT_TP64][4];   // the tokens' operands of one half of the stage's columns: both row groups use them
+            bread(0, Bb, nt_tag);
+            gather(f[0], 0, G[0]);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int p = u >> 1, q = u & 1;
+                if (u == 2) bread(1, Bb, nt_tag);
+                if (u < 3) gather(f[(u + 1) & 1], (u + 1) >> 1, G[(u + 1) & 1]);
+                __builtin_amdgcn_sched_barrier(0);
+                math(f[q], p, q, G[u & 1], Bb, nt_tag);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+        TileStaged64 st = issue(0, 0);
+        int ti = 0, S = 0;
+        for (int s = 0; s < nst; ++s) {
+            stash_w(st, s & 1);   // (its buffer was last read two stages ago)
+            __syncthreads();      // the single activation tile's last readers
+            stash_x(st);
+            __syncthreads();
+            int tn = ti, Sn = S + 1;
+            if (Sn == nsuper) {
+                Sn = 0;
+                ++tn;
+            }
+            if (s + 1 < nst) st = issue(tn, Sn);
+            const int row0 = L.task[ti].row0 + wave * 16 * MB_RG;
+            if (row0 < a.nrows) {   // per wave
+                const int nt = L.task[ti].ntile;
+                if (nt > 2) compute(s & 1, std::integral_constant<int, 4>{});
+                else if (nt > 1) compute(s & 1, std::integral_constant<int, 2>{});
+                else compute(s & 1, std::integral_constant<int, 1>{});
+                if (Sn == 0) {
+                    // lane: token r of each tile, weight rows 4 g .. 4 g + 3 of each group
+#pragma unroll
+                    for (int tt = 0; tt < MT_TP64; ++tt) {
+                        const int orow = L.otok[ti][tt * 16 + r];
+                        if (orow >= 0) {
+                            float* o = a.out + (size_t) orow * a.nrows + row0 + 4 * g;
+#pragma unroll
+                            for (int q = 0; q < MB_RG; ++q)
+                                if (row0 + 16 * q < a.nrows) *reinterpret_cast<float4*>(o + 16 * q) = make_float4(acc[q][tt].x, acc[q][tt].y, acc[q][tt].z, acc[q][tt].w);
+                        }
+                    }
+#pragma unroll
+                    for (int q = 0; q < MB_RG; ++q)
+#pragma unroll
+                        for (int tt = 0; tt < MT_TP64; ++tt) acc[q][tt] = v4f{0.f, 0.f, 0.f, 0.f};
+                }
+            }
+            ti = tn;
+            S = Sn;
+        }
+    }
+}
+
+
 }  // namespace fnx
