@@ -1411,14 +1411,14 @@ static int q8s_launch(const fnx_q8s* const* W, float* const* out, const int* out
     static bool attr_set[64] = {};
     int dev = 0;
     if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64 && !attr_set[dev]) {
-        if (hipFuncSetAttribute((const void*) k_q8s_gemv, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024) != hipSuccess)
+        if (hipFuncSetAttribute((const void*) k_q8s_gemv<1>, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024) != hipSuccess)
             return fail(std::string(who) + ": cannot raise the dynamic LDS limit");
         attr_set[dev] = true;
     }
     static const int per_cu = env_int("FNX_Q8S_BLOCKS_PER_CU", 4, 1, 16);   // what the LDS of a 2048-column matrix lets a CU hold
     const int grid = (int) std::max(1l, std::min<long>((long) per_cu * cu_count(), tiles));
     a.gate = gate;
-    k_q8s_gemv<<<grid, Q8S_WAVES * 64, lds, (hipStream_t) st>>>(a);
+    k_q8s_gemv<1><<<grid, Q8S_WAVES * 64, lds, (hipStream_t) st>>>(a);
     return launch_status(who);
 }
 int fnx_q8s_gemv(const fnx_q8s* W, const void* yq, float* out, int out_stride, int T, void* st) {

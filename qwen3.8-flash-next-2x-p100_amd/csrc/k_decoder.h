@@ -195,6 +195,10 @@ struct Q8sArgs {
     const int* gate;     // may be null; else a device word: at zero the launch leaves at once (a chain step that does not count)
 };
 typedef int q8s_v4i __attribute__((ext_vector_type(4)));
+// DEPTH: the (tile, batch) items whose loads are in flight ahead of the one being worked on. (With 3 - all of a tile's
+// batches on their way before the activations are staged - a matrix of a few thousand rows was not faster: its launch is
+// the block's start, the staging of the activations and the first pass through the code, not the weights' round trips.)
+template <int DEPTH>
 __global__ void __launch_bounds__(Q8S_WAVES * 64) k_q8s_gemv(const Q8sArgs a) {
     typedef __attribute__((address_space(1))) const at_v4u_t g128;
     extern __shared__ __align__(16) uint8_t q8s_lds[];   // [16][cols + pad] int8, [16][nb + 2] f32 scales, [3][64][4] partial sums
@@ -289,32 +293,34 @@ __global__ void __launch_bounds__(Q8S_WAVES * 64) k_q8s_gemv(const Q8sArgs a) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) acc[r] = 0.f;
     };
-    // The (tile, batch) items of this block in one sequence: the next item's loads - the next tile's first ones too -
-    // are in flight while the current one is worked on and while a tile's quarters are summed.
-    int tile = blockIdx.x, jb = 0;
-    if (tile >= tiles) return;   // the same for every thread of the block
-    Tile cur = tile_of(tile);
-    bool more = true;
-    auto item = [&](const Batch& in, Batch& nxt) {
-        int ntile = tile, njb = jb + Q8S_BATCH;
-        if (njb >= nq4) {
-            njb = 0;
-            ntile += gridDim.x;
-        }
-        more = ntile < tiles;
-        const bool last = ntile != tile;
-        Tile tn = cur;
-        if (last && more) tn = tile_of(ntile);
-        if (more) load(tn, njb, nxt);
-        compute(jb, in);
-        if (last) finish(cur);
-        cur = tn;
-        tile = ntile;
-        jb = njb;
+    // The (tile, batch) items of this block in one sequence: the loads of the items ahead - the next tiles' first ones
+    // too - are in flight while the current one is worked on and while a tile's quarters are summed.
+    if ((int) blockIdx.x >= tiles) return;   // the same for every thread of the block
+    struct Cursor {
+        int tile, jb;
+        bool valid;
+        Tile t;
     };
-    Batch b0, b1;
-    load(cur, 0, b0);
-    // the window's q8_1 rows into LDS (the first weights are on their way meanwhile)
+    auto advance = [&](Cursor& c) {
+        c.jb += Q8S_BATCH;
+        if (c.jb >= nq4) {
+            c.jb = 0;
+            c.tile += gridDim.x;
+            c.valid = c.tile < tiles;
+            if (c.valid) c.t = tile_of(c.tile);
+        }
+    };
+    Cursor lc{(int) blockIdx.x, 0, true, tile_of(blockIdx.x)}, cc = lc;   // the loads' place and the arithmetic's
+    Batch ring[DEPTH + 1];
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d)
+        if (lc.valid) {
+            load(lc.t, lc.jb, ring[d]);
+            advance(lc);
+        }
+    // the window's q8_1 rows into LDS (the first weights are on their way meanwhile). The copy takes 3 us (6-7 us in a
+    // launch of 1,024 blocks, beside their weight loads) whatever the width of its loads - nine 16-byte loads for four
+    // blocks of a row were no faster than 4-byte ones - and wherever in the rows a block starts.
     for (int i = threadIdx.x; i < FNX_MAXT * nb; i += blockDim.x) {
         const int t = i / nb, b = i - t * nb;
         uint32_t* dst = reinterpret_cast<uint32_t*>(xs + (size_t) t * xld + 32 * b);
@@ -331,11 +337,18 @@ __global__ void __launch_bounds__(Q8S_WAVES * 64) k_q8s_gemv(const Q8sArgs a) {
         }
     }
     __syncthreads();
-    while (true) {
-        item(b0, b1);
-        if (!more) break;
-        item(b1, b0);
-        if (!more) break;
+    while (cc.valid) {
+#pragma unroll
+        for (int slot = 0; slot <= DEPTH; ++slot) {
+            if (!cc.valid) break;
+            if (lc.valid) {
+                load(lc.t, lc.jb, ring[(slot + DEPTH) % (DEPTH + 1)]);
+                advance(lc);
+            }
+            compute(cc.jb, ring[slot]);
+            if (cc.jb + Q8S_BATCH >= nq4) finish(cc.t);
+            advance(cc);
+        }
     }
 }
 
