@@ -1160,7 +1160,7 @@ int fnx_moe_verify_layer_static(const fnx_moe_layer* L, const float* x, int T, f
     // nothing in the workspace has to start at zero: every launch writes what it reads, and the job count is stored, not added to
     const fnx_moe_ws ws{w, (float*) (w + NA_OFF_LOGITS), (int*) (w + NA_OFF_TOPI), (float*) (w + NA_OFF_TOPW), (fnx_job*) (w + NA_OFF_JGU),
                         (fnx_job*) (w + NA_OFF_JDN), (int*) (w + NA_OFF_NJOBS), (float*) (w + NA_OFF_HQ), nullptr};
-    const int P = T * L->topk, n = L->n, ff = L->ff;
+    const int P = T * L->topk;
     if (shared_is_q8(L)) return fail("moe_verify_layer_static: a split-Q8_0 shared expert needs a caller's workspace (fnx_moe_verify_layer)");
     if (!moe_shapes_ok(L)) return fail("moe_verify_layer_static: weight shapes do not match n / ff");
     if (topk_check(T, L->nexp, L->topk, "moe_verify_layer_static")) return 1;

@@ -468,7 +468,6 @@ __global__ void __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu
                                                             AttPart* __restrict__ mz_out, int nq, int nkv, int T, int nsplit,
                                                             const int* __restrict__ pos0p, int max_ctx, const int* __restrict__ gate,
                                                             const int* __restrict__ live) {
-    typedef __attribute__((address_space(1))) const at_v4u g128;
     if (gate && uniform(*gate) == 0) return;   // a chain step that does not count: its parts stay what they were, nothing reads the result
     // live (may be null): a device word, the rows of the window that count; the others' queries are left out (nothing reads
     // their results), the positions past the last row that counts with them
