@@ -93,4 +93,12 @@ __device__ __forceinline__ uint32_t load_u16(const uint8_t* p) {
     return v;
 }
 
+// 64 lanes x 16 bytes from base + each lane's byte offset straight into LDS, laid down in lane order from lds_at on (a
+// wave-uniform LDS address, through M0). Written as an instruction so that the compiler, which cannot tell one LDS buffer
+// of such loads from another, does not wait for every one of them before each LDS read: the kernel counts them itself
+// (vmcnt) where it needs their data.
+__device__ __forceinline__ void lds_load16(const void* base, uint32_t lane_offset, uint32_t lds_at) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_at), "v"(lane_offset), "s"(base) : "memory");
+}
+
 }  // namespace fnx

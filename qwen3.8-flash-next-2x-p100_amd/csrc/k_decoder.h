@@ -456,13 +456,6 @@ __device__ __forceinline__ float groups4_sum(float v) {
 }
 constexpr int AT_WAVES = 4;   // q tiles (of 16 queries) per block, blockIdx.z picks which
 constexpr int AT_THREADS = (AT_WAVES + 1) * 64;   // and one wave more that only brings the K and V chunks in
-// 64 lanes x 16 bytes from base + each lane's byte offset straight into LDS, laid down in lane order from lds_at on (a
-// wave-uniform LDS address, through M0). Written as an instruction so that the compiler, which cannot tell one LDS buffer
-// of such loads from another, does not wait for every one of them before each LDS read: the kernel counts them itself
-// (vmcnt) where it needs their data.
-__device__ __forceinline__ void lds_load16(const void* base, uint32_t lane_offset, uint32_t lds_at) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_at), "v"(lane_offset), "s"(base) : "memory");
-}
 __global__ void __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) k_attn_part(const float* __restrict__ qg, const uint16_t* __restrict__ kc,
                                                             const uint16_t* __restrict__ vc, float* __restrict__ acc_out,
                                                             AttPart* __restrict__ mz_out, int nq, int nkv, int T, int nsplit,

@@ -167,15 +167,14 @@ __global__ void k_swiglu_h16(const float* __restrict__ gu, int ffs, size_t total
 // loads (coalesced, straight from the caches: no LDS, no barriers) feeds GR_ROWS chains. Order per sum as above.
 constexpr int GM_WAVES = 8, GR_ROWS = 4, GM_BATCH = 8;
 static_assert(GR_ROWS * FNX_MAXT == 64, "64 sums a wave, one per lane in the end");
+// one wave: weight rows row0 .. row0 + GR_ROWS - 1 against the activation rows FNX_MAXT tgroup ..
 template <bool BF>
-__global__ void __launch_bounds__(GM_WAVES * 64) k_gemv_rows_many(const void* __restrict__ Wv, const float* __restrict__ x, float* __restrict__ y,
-                                                                 int rows, int n, int T) {
-    x += (size_t) blockIdx.y * FNX_MAXT * n;
-    y += (size_t) blockIdx.y * FNX_MAXT * rows;
-    T = min(FNX_MAXT, T - (int) blockIdx.y * FNX_MAXT);
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int row0 = (blockIdx.x * GM_WAVES + wave) * GR_ROWS;
-    if (row0 >= rows) return;
+__device__ __forceinline__ void gemv_rows_many_wave(const void* __restrict__ Wv, const float* __restrict__ x, float* __restrict__ y, int rows, int n,
+                                                    int T, int row0, int tgroup, int lane) {
+    x += (size_t) tgroup * FNX_MAXT * n;
+    y += (size_t) tgroup * FNX_MAXT * rows;
+    T = min(FNX_MAXT, T - tgroup * FNX_MAXT);
+    if (row0 >= rows || T <= 0) return;
     float acc[GR_ROWS][FNX_MAXT];
 #pragma unroll
     for (int r = 0; r < GR_ROWS; ++r)
@@ -239,6 +238,260 @@ __global__ void __launch_bounds__(GM_WAVES * 64) k_gemv_rows_many(const void* __
     const float v = fold(b0, b1, 1);
     const int r = lane >> 4, t = lane & 15;
     if (t < T && row0 + r < rows) y[(size_t) t * rows + row0 + r] = v;
+}
+template <bool BF>
+__global__ void __launch_bounds__(GM_WAVES * 64) k_gemv_rows_many(const void* __restrict__ Wv, const float* __restrict__ x, float* __restrict__ y,
+                                                                 int rows, int n, int T, int row_begin) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    gemv_rows_many_wave<BF>(Wv, x, y, rows, n, T, row_begin + (blockIdx.x * GM_WAVES + wave) * GR_ROWS, blockIdx.y, lane);
+}
+
+// One weight row against four activation rows, every load of up to eight steps issued before the first fmaf: for the few
+// rows that the kernel below leaves over, where a wave's time is a chain of memory round trips. Order per sum as above.
+__device__ __forceinline__ void gemv_row_quad_wave(const float* __restrict__ W, const float* __restrict__ x, float* __restrict__ y, int rows, int n,
+                                                   int T, int row, int t0, int lane) {
+    if (row >= rows || t0 >= T) return;
+    const float4* wr = reinterpret_cast<const float4*>(W + (size_t) row * n) + lane;
+    const float4* xr[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) xr[t] = reinterpret_cast<const float4*>(x + (size_t) min(t0 + t, T - 1) * n) + lane;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    const int steps = n / 256;
+    for (int s0 = 0; s0 < steps; s0 += 8) {
+        float4 w[8], b[4][8];
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            const int c = min(s0 + s, steps - 1) * 64;
+            w[s] = wr[c];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) b[t][s] = xr[t][c];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < 8; ++s)
+            if (s0 + s < steps) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    float a = acc[t];
+                    a = fmaf(w[s].x, b[t][s].x, a);
+                    a = fmaf(w[s].y, b[t][s].y, a);
+                    a = fmaf(w[s].z, b[t][s].z, a);
+                    a = fmaf(w[s].w, b[t][s].w, a);
+                    acc[t] = a;
+                }
+            }
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        const float v = group_sum<64>(acc[t]);
+        if (lane == 0 && t0 + t < T) y[(size_t) (t0 + t) * rows + row] = v;
+    }
+}
+
+// ---------------------------------------------------------------- the same sums on the matrix cores
+// v_mfma_f32_32x32x1_2b_f32 is D = fma(a, b, D) element by element with one rounding - the fmaf of the chains above
+// (checked bit for bit on this GPU, products in the denormal range included). A chain of them over the chunks
+// l, l + 64, ... therefore leaves lane l's partial sum of 32 activation rows x 32 weight rows at once; the instruction's
+// two blocks take l and l + 32, the pair that the butterfly adds first. A block of four waves owns such a tile of
+// 32 x 32 sums. Wave w walks the lanes l = w mod 4 in eight phases - l = 8 a + 4 h + w and l + 32, (h; a) in the order
+// (0; 0, 2, 1, 3), (1; 0, 2, 1, 3) - so that the butterfly's levels 16, 8 and 4 are adds of whole accumulator tiles as
+// the phases end (done while the next phase multiplies into a second accumulator); levels 2 and 1 add the four waves'
+// tiles through LDS. The operands (f32 weights only) come through LDS: a stage is 64 rows (32 of x, 32 of W) x 256
+// bytes - two chunks of the four lanes l and of l + 32 - sent there by global_load_lds_dwordx4, three stages ahead,
+// into one of four buffers; an instruction carries four rows, a wave issues four of a stage's sixteen between its
+// MFMAs, and row r's piece p lies at place p ^ (r % 16), so that the 16 rows an operand read touches fall on 16
+// different bank groups. The waves read a stage's operands right after the meeting that says it has landed and
+// multiply the stage before it meanwhile.
+// The first blocks of the grid take the weight rows past the last full 32 (the router's 513th) with
+// gemv_row_quad_wave: 64 KB of LDS and 256 registers a lane let two blocks share a compute unit, so these run beside
+// the tiles' blocks, whose vector units are idle.
+typedef float v32f __attribute__((ext_vector_type(32)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+constexpr int RM_TILE = 32, RM_THREADS = 256, RM_ROWB = 256, RM_STAGE = 2 * RM_TILE * RM_ROWB, RM_BUFS = 4;
+__global__ void __launch_bounds__(RM_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
+k_gemv_rows_mfma(const float* __restrict__ W, const float* __restrict__ x, float* __restrict__ y, int rows, int n, int T, int ntt, int net,
+                 int tile_blocks, int left_blocks) {
+    __shared__ __align__(16) uint8_t lds[RM_BUFS * RM_STAGE];
+    const int wave = uniform((int) (threadIdx.x >> 6)), lane = threadIdx.x & 63;
+    if ((int) blockIdx.x < left_blocks) {   // the rows past the full tiles: a wave takes one of them against four rows of x
+        const int left = rows - net * RM_TILE, item = (int) blockIdx.x * (RM_THREADS / 64) + wave;
+        gemv_row_quad_wave(W, x, y, rows, n, T, net * RM_TILE + item % left, 4 * (item / left), lane);
+        return;
+    }
+    // Which tile: block ids go round the eight XCDs, each with an L2 of its own, so an XCD's blocks are given one patch of
+    // 4 x 8 tiles after another (1 MB of x and 2 MB of W for rows of 2048: its L2 holds them, every block re-reads both
+    // eight times over the phases). The grid covers whole patches; a block whose tile lies outside leaves.
+    const int id = (int) blockIdx.x - left_blocks;
+    const int lin = (id % 8) * (tile_blocks / 8) + id / 8, patches_e = (net + 7) / 8;
+    const int tt = 4 * ((lin / 32) / patches_e) + (lin % 32) / 8, et = 8 * ((lin / 32) % patches_e) + lin % 8;
+    if (tt >= ntt || et >= net) return;
+    const int t0 = tt * RM_TILE, e0 = et * RM_TILE;
+    const int nq = n / 512, S = 8 * nq;   // stages: phase-major, a row's stretches of 512 values within a phase
+    const uint32_t lds_at = (uint32_t) (size_t) (__attribute__((address_space(3))) uint8_t*) lds;
+    // The waves meet where a stage must have landed: a wave's loads complete in order, so it waits until only those of the
+    // two stages after it (eight instructions) may be on their way, and for its LDS reads; then for the others. (A plain
+    // barrier instruction: __syncthreads() would wait for every load.)
+    auto meet = [&](int in_flight) {
+        __builtin_amdgcn_sched_barrier(0);
+        if (in_flight == 8) __builtin_amdgcn_s_waitcnt(0x0078);        // vmcnt(8) lgkmcnt(0)
+        else if (in_flight == 4) __builtin_amdgcn_s_waitcnt(0x0074);   // vmcnt(4) lgkmcnt(0)
+        else __builtin_amdgcn_s_waitcnt(0x0070);                       // vmcnt(0) lgkmcnt(0)
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    // this wave's four load instructions of a stage: instruction j = 4 wave + jj carries rows 4 j .. 4 j + 3 (rows 0..31
+    // of x, 32..63 of W), this lane's piece of its row
+    uint32_t off[4];
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) {
+        const int row = 4 * (4 * wave + jj) + (lane >> 4), p = (lane & 15) ^ (row & 15);
+        const int r = wave < 2 ? min(t0 + row, T - 1) : e0 + row - RM_TILE;
+        off[jj] = (uint32_t) r * (uint32_t) n * 4u + 1024u * (p >> 3) + 512u * ((p >> 2) & 1) + 16u * (p & 3);
+    }
+    const uint8_t* src = reinterpret_cast<const uint8_t*>(wave < 2 ? x : W);
+    int fph = 0, fq = 0, fbuf = 0, fetched = 0;   // the next stage to fetch: phase, stretch, buffer, number
+    const uint8_t* fsrc = src;
+    uint32_t fat = 0;
+    auto fetch_begin = [&]() {   // the scalars of the next stage's loads
+        const int q = fph & 3, l0 = 8 * (((q & 1) << 1) | (q >> 1)) + 4 * (fph >> 2);
+        fsrc = src + 16 * l0 + 2048 * fq;
+        fat = lds_at + fbuf * RM_STAGE + wave * 4096;
+    };
+    auto fetch_one = [&](int jj) {
+        if (fetched < S) lds_load16(fsrc, off[jj], fat + jj * 1024);
+    };
+    auto fetch_end = [&]() {
+        if (++fq == nq) fq = 0, ++fph;
+        fbuf = fbuf == RM_BUFS - 1 ? 0 : fbuf + 1;
+        ++fetched;
+    };
+    const int i = lane & 31, b = lane >> 5;
+    // this lane's operands of a stage: row i of x and row i of W, chunks 0 and 1 of lane l (block b: l + 32)
+    const uint8_t* r0 = lds + i * RM_ROWB + 16 * ((4 * b + wave) ^ (i & 15));
+    const uint8_t* r1 = lds + i * RM_ROWB + 16 * ((8 + 4 * b + wave) ^ (i & 15));
+    float4 A[2][2], B[2][2];
+    int buf = 0, met = 0;   // the buffer whose operands are read next; meetings so far
+    auto next_stage = [&](float4 (&a)[2], float4 (&bb)[2]) {
+        meet(met + 2 < S ? 8 : met + 1 < S ? 4 : 0);   // stage `met` has landed
+        ++met;
+        const int o = buf * RM_STAGE;   // (past the last stage: a buffer's old contents, not used)
+        a[0] = *reinterpret_cast<const float4*>(r0 + o);
+        a[1] = *reinterpret_cast<const float4*>(r1 + o);
+        bb[0] = *reinterpret_cast<const float4*>(r0 + o + RM_TILE * RM_ROWB);
+        bb[1] = *reinterpret_cast<const float4*>(r1 + o + RM_TILE * RM_ROWB);
+        buf = buf == RM_BUFS - 1 ? 0 : buf + 1;
+        fetch_begin();
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    v32f acc[2];
+    v16f t, held, u0, sum;
+    // A stage's 8 steps into accumulator c (first: the phase's first stage, which starts from zero), this wave's loads of
+    // the stage three on after every other one. kind >= 0: the fold of the phase before, whose accumulator is cf - the
+    // butterfly's levels 32 (the instruction's two blocks), 16, 8 and 4 - goes in between on the vector unit. kind 0: the
+    // phase of a = 0 or a = 1: held; 1: a = 2, level 16 with a = 0; 3 and 4: a = 3, level 16 with a = 1, level 8, and for
+    // h = 1 (4) level 4.
+    auto fold_a = [&](const v32f& cf) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) t[v] = cf[v] + cf[16 + v];
+    };
+    auto fold_b = [&](auto kind_c) {
+        constexpr int kind = decltype(kind_c)::value;
+        if constexpr (kind == 0) held = t;
+        else if constexpr (kind == 1) u0 = held + t;
+        else t = held + t;
+    };
+    auto fold_c = [&](auto kind_c) {
+        constexpr int kind = decltype(kind_c)::value;
+        if constexpr (kind == 3) sum = u0 + t;
+        else if constexpr (kind == 4) sum = sum + (u0 + t);
+    };
+    auto multiply = [&](const float4 (&a)[2], const float4 (&bb)[2], v32f& c, auto first_c, auto kind_c, v32f& cf) {
+        constexpr bool first = decltype(first_c)::value;
+        constexpr int kind = decltype(kind_c)::value;
+        if constexpr (kind >= 0) asm volatile("" : "+v"(cf));   // (keeps the fold's adds on this side of the meeting)
+#pragma unroll
+        for (int cc = 0; cc < 2; ++cc) {
+            if (first && cc == 0) {
+                v32f z;
+#pragma unroll
+                for (int v = 0; v < 32; ++v) z[v] = 0.f;
+                c = __builtin_amdgcn_mfma_f32_32x32x1f32(a[cc].x, bb[cc].x, z, 0, 0, 0);
+            } else {
+                c = __builtin_amdgcn_mfma_f32_32x32x1f32(a[cc].x, bb[cc].x, c, 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            fetch_one(2 * cc);
+            if constexpr (kind >= 0) {
+                if (cc == 0) fold_a(cf);
+                else fold_c(kind_c);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            c = __builtin_amdgcn_mfma_f32_32x32x1f32(a[cc].y, bb[cc].y, c, 0, 0, 0);
+            c = __builtin_amdgcn_mfma_f32_32x32x1f32(a[cc].z, bb[cc].z, c, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            fetch_one(2 * cc + 1);
+            if constexpr (kind >= 0) {
+                if (cc == 0) fold_b(kind_c);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            c = __builtin_amdgcn_mfma_f32_32x32x1f32(a[cc].w, bb[cc].w, c, 0, 0, 0);
+        }
+        fetch_end();
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    using std::integral_constant;
+    constexpr integral_constant<bool, true> yes{};
+    constexpr integral_constant<bool, false> no{};
+    constexpr integral_constant<int, -1> none{};
+    // a phase into accumulator c, the phase before's fold along with its first stage (nq is even)
+    auto phase = [&](v32f& c, auto kind_c, v32f& cf) {
+        next_stage(A[1], B[1]);
+        multiply(A[0], B[0], c, yes, kind_c, cf);
+        next_stage(A[0], B[0]);
+        multiply(A[1], B[1], c, no, none, c);
+        for (int h2 = 2; h2 < nq; h2 += 2) {
+            next_stage(A[1], B[1]);
+            multiply(A[0], B[0], c, no, none, c);
+            next_stage(A[0], B[0]);
+            multiply(A[1], B[1], c, no, none, c);
+        }
+    };
+    // the first four stages on their way
+#pragma unroll 1
+    for (int k = 0; k < 4; ++k) {
+        fetch_begin();
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) fetch_one(jj);
+        fetch_end();
+    }
+#pragma unroll
+    for (int v = 0; v < 32; ++v) acc[1][v] = 0.f;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) held[v] = u0[v] = 0.f;
+    next_stage(A[0], B[0]);
+#pragma unroll 1
+    for (int h = 0; h < 2; ++h) {
+        phase(acc[0], integral_constant<int, 3>{}, acc[1]);   // (h = 0: of nothing, and what it leaves is overwritten)
+        phase(acc[1], integral_constant<int, 0>{}, acc[0]);
+        phase(acc[0], integral_constant<int, 1>{}, acc[1]);
+        phase(acc[1], integral_constant<int, 0>{}, acc[0]);
+    }
+    fold_a(acc[1]);
+    fold_b(integral_constant<int, 4>{});
+    fold_c(integral_constant<int, 4>{});
+    // levels 2 and 1 over the waves' tiles, in the buffer that the last stage left (all have read it; the one after it
+    // may still be being read, for nothing, by another wave)
+    float* red = reinterpret_cast<float*>(lds + ((S - 1) % RM_BUFS) * RM_STAGE);
+#pragma unroll
+    for (int v = 0; v < 16; ++v) red[(wave * 16 + v) * 64 + lane] = sum[v];
+    meet(0);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const int v = 4 * wave + q;
+        const float s = (red[v * 64 + lane] + red[(32 + v) * 64 + lane]) + (red[(16 + v) * 64 + lane] + red[(48 + v) * 64 + lane]);
+        const int tk = t0 + 8 * (v >> 2) + 4 * b + (v & 3);
+        if (tk < T) y[(size_t) tk * rows + e0 + i] = s;
+    }
 }
 
 // ---------------------------------------------------------------- the routed experts on the matrix cores

@@ -47,6 +47,19 @@ def test_gemv_f32_bit_exact(dev, oracle, rows, n, T):
     assert np.array_equal(dev.gemv(W, x).view(np.uint32), oracle.gemv_f32(W, x).view(np.uint32))
 
 
+# 64 rows of x and more against f32 weights with rows of a multiple of 2048: the tiles on the matrix cores (ragged last
+# tiles of both kinds, weight rows past the last full 32, more than one patch of tiles, rows of 4096), with values over
+# many binades so that a sum's bits depend on the order of its adds
+@pytest.mark.parametrize("rows,n,T", [(513, 2048, 512), (96, 2048, 70), (290, 2048, 200), (64, 4096, 64), (35, 2048, 129)])
+def test_gemv_f32_many_rows_bit_exact(dev, oracle, rows, n, T):
+    print(f"case gemv_f32 (tiles) rows={rows} n={n} T={T}", flush=True)
+    rng = np.random.default_rng(230 + rows + T)
+    W = (rng.standard_normal((rows, n)) * np.exp2(rng.integers(-12, 4, (rows, n)))).astype(np.float32)
+    x = (rng.standard_normal((T, n)) * np.exp2(rng.integers(-8, 8, (T, n)))).astype(np.float32)
+    x[rng.integers(0, T, 40), rng.integers(0, n, 40)] = 0.0
+    assert np.array_equal(dev.gemv(W, x).view(np.uint32), oracle.gemv_f32(W, x).view(np.uint32))
+
+
 @pytest.mark.parametrize("T", [16, 45])   # 45 rows: the many-rows kernel, with a ragged last group
 def test_gemv_bf16_bit_exact(dev, oracle, T):
     rng = np.random.default_rng(210)
