@@ -96,7 +96,9 @@ int fnx_quantize_q8_1(const float* x, void* q, int n, int rows, void* st);
 int fnx_mmvq(const fnx_dw* W, size_t w_stride, const fnx_job* jobs, const int* njobs, int njobs_max, const void* y,
              float* out, int out_stride, void* st);
 
-/* kernels.hpp:54-55  gemv_f32 / gemv_bf16: y[t][r] = W[r] . x[t], W [rows][n], T <= 16, n % 256 == 0 */
+/* kernels.hpp:54-55  gemv_f32 / gemv_bf16: y[t][r] = W[r] . x[t], W [rows][n], n % 256 == 0. The reference calls it
+ * with T <= 16; any T is taken here (the prompt path's router logits are one call over a chunk's rows), every sum in
+ * the same order of operations whatever T is. */
 int fnx_gemv_f32(const float* W, const float* x, float* y, int rows, int n, int T, void* st);
 int fnx_gemv_bf16(const uint16_t* W, const float* x, float* y, int rows, int n, int T, void* st);
 
