@@ -50,7 +50,7 @@ def test_gemv_f32_bit_exact(dev, oracle, rows, n, T):
 # 64 rows of x and more against f32 weights with rows of a multiple of 2048: the tiles on the matrix cores (ragged last
 # tiles of both kinds, weight rows past the last full 32, more than one patch of tiles, rows of 4096), with values over
 # many binades so that a sum's bits depend on the order of its adds
-@pytest.mark.parametrize("rows,n,T", [(513, 2048, 512), (96, 2048, 70), (290, 2048, 200), (64, 4096, 64), (35, 2048, 129)])
+@pytest.mark.parametrize("rows,n,T", [(513, 2048, 512), (96, 2048, 70), (290, 2048, 200), (64, 4096, 64), (35, 2048, 129), (33, 4096, 66), (65, 3072, 96)])
 def test_gemv_f32_many_rows_bit_exact(dev, oracle, rows, n, T):
     print(f"case gemv_f32 (tiles) rows={rows} n={n} T={T}", flush=True)
     rng = np.random.default_rng(230 + rows + T)
