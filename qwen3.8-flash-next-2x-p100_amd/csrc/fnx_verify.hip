@@ -927,14 +927,17 @@ static int gemv_any(const void* W, bool bf, const float* x, float* y, int rows, 
     if (rows <= 0 || n <= 0 || n % 256) return fail(std::string(who) + ": n must be a positive multiple of 256");
     if (T < 1 || T > 65535 * FNX_MAXT) return fail(std::string(who) + ": T out of range");
     hipStream_t s = (hipStream_t) st;
-    if (!bf && T >= 2 * RM_TILE && rows >= RM_TILE && n % 1024 == 0 && n >= 2048 && (uint64_t) T * n * 4 < (1ull << 32) &&
-        (uint64_t) rows * n * 4 < (1ull << 32)) {
-        // a chunk's worth of rows against f32 weights: tiles of 32 x 32 sums on the matrix cores, the weight rows past the
-        // last full 32 in blocks of their own beside them
+    if (!bf && T >= 2 * RM_TILE && rows >= RM_TILE && n % 2048 == 0 && (uint64_t) T * n * 4 < (1ull << 32) && (uint64_t) rows * n * 4 < (1ull << 32)) {
+        // a chunk's worth of rows against f32 weights: tiles of 32 x 32 sums on the matrix cores. The weight rows past the
+        // last full 32 ride with the tiles' blocks, an item a block (a row x four rows of x); if there are more items
+        // than blocks in a row of tiles, those rows go to the kernel below.
         const int ntt = (T + RM_TILE - 1) / RM_TILE, net = rows / RM_TILE, left = rows - net * RM_TILE;
         const int tile_blocks = ((ntt + 3) / 4) * ((net + 7) / 8) * 32;
-        const int items = left * ((T + 3) / 4), left_blocks = (items + RM_THREADS / 64 - 1) / (RM_THREADS / 64);
-        k_gemv_rows_mfma<<<left_blocks + tile_blocks, RM_THREADS, 0, s>>>((const float*) W, x, y, rows, n, T, ntt, net, tile_blocks, left_blocks);
+        const bool along = 8 * left <= net;   // a row and four rows of x a block, within the block's own rows of x
+        k_gemv_rows_mfma<<<tile_blocks, RM_THREADS, 0, s>>>((const float*) W, x, y, rows, n, T, ntt, net, tile_blocks, along ? 1 : 0);
+        if (left == 0 || along) return launch_status(who);
+        const dim3 gm((left + GM_WAVES * GR_ROWS - 1) / (GM_WAVES * GR_ROWS), (T + FNX_MAXT - 1) / FNX_MAXT);
+        k_gemv_rows_many<false><<<gm, GM_WAVES * 64, 0, s>>>(W, x, y, rows, n, T, net * RM_TILE);
         return launch_status(who);
     }
     if (T > FNX_MAXT) {   // many rows of x: GR_ROWS weight rows a wave

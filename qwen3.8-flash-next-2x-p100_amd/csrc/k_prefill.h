@@ -246,171 +246,186 @@ __global__ void __launch_bounds__(GM_WAVES * 64) k_gemv_rows_many(const void* __
     gemv_rows_many_wave<BF>(Wv, x, y, rows, n, T, row_begin + (blockIdx.x * GM_WAVES + wave) * GR_ROWS, blockIdx.y, lane);
 }
 
-// One weight row against four activation rows, every load of up to eight steps issued before the first fmaf: for the few
-// rows that the kernel below leaves over, where a wave's time is a chain of memory round trips. Order per sum as above.
-__device__ __forceinline__ void gemv_row_quad_wave(const float* __restrict__ W, const float* __restrict__ x, float* __restrict__ y, int rows, int n,
-                                                   int T, int row, int t0, int lane) {
-    if (row >= rows || t0 >= T) return;
-    const float4* wr = reinterpret_cast<const float4*>(W + (size_t) row * n) + lane;
-    const float4* xr[4];
-#pragma unroll
-    for (int t = 0; t < 4; ++t) xr[t] = reinterpret_cast<const float4*>(x + (size_t) min(t0 + t, T - 1) * n) + lane;
-    float acc[4] = {0.f, 0.f, 0.f, 0.f};
-    const int steps = n / 256;
-    for (int s0 = 0; s0 < steps; s0 += 8) {
-        float4 w[8], b[4][8];
-#pragma unroll
-        for (int s = 0; s < 8; ++s) {
-            const int c = min(s0 + s, steps - 1) * 64;
-            w[s] = wr[c];
-#pragma unroll
-            for (int t = 0; t < 4; ++t) b[t][s] = xr[t][c];
-        }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int s = 0; s < 8; ++s)
-            if (s0 + s < steps) {
-#pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    float a = acc[t];
-                    a = fmaf(w[s].x, b[t][s].x, a);
-                    a = fmaf(w[s].y, b[t][s].y, a);
-                    a = fmaf(w[s].z, b[t][s].z, a);
-                    a = fmaf(w[s].w, b[t][s].w, a);
-                    acc[t] = a;
-                }
-            }
-    }
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-        const float v = group_sum<64>(acc[t]);
-        if (lane == 0 && t0 + t < T) y[(size_t) (t0 + t) * rows + row] = v;
-    }
-}
-
 // ---------------------------------------------------------------- the same sums on the matrix cores
 // v_mfma_f32_32x32x1_2b_f32 is D = fma(a, b, D) element by element with one rounding - the fmaf of the chains above
 // (checked bit for bit on this GPU, products in the denormal range included). A chain of them over the chunks
 // l, l + 64, ... therefore leaves lane l's partial sum of 32 activation rows x 32 weight rows at once; the instruction's
-// two blocks take l and l + 32, the pair that the butterfly adds first. A block of four waves owns such a tile of
-// 32 x 32 sums. Wave w walks the lanes l = w mod 4 in eight phases - l = 8 a + 4 h + w and l + 32, (h; a) in the order
-// (0; 0, 2, 1, 3), (1; 0, 2, 1, 3) - so that the butterfly's levels 16, 8 and 4 are adds of whole accumulator tiles as
-// the phases end (done while the next phase multiplies into a second accumulator); levels 2 and 1 add the four waves'
-// tiles through LDS. The operands (f32 weights only) come through LDS: a stage is 64 rows (32 of x, 32 of W) x 256
-// bytes - two chunks of the four lanes l and of l + 32 - sent there by global_load_lds_dwordx4, three stages ahead,
-// into one of four buffers; an instruction carries four rows, a wave issues four of a stage's sixteen between its
-// MFMAs, and row r's piece p lies at place p ^ (r % 16), so that the 16 rows an operand read touches fall on 16
-// different bank groups. The waves read a stage's operands right after the meeting that says it has landed and
-// multiply the stage before it meanwhile.
-// The first blocks of the grid take the weight rows past the last full 32 (the router's 513th) with
-// gemv_row_quad_wave: 64 KB of LDS and 256 registers a lane let two blocks share a compute unit, so these run beside
-// the tiles' blocks, whose vector units are idle.
+// two blocks take l and l + 32, the pair that the butterfly adds first. A block owns such a tile of 32 x 32 sums. Wave
+// w of its RM_WAVES multiplying waves walks the lanes l = w mod 4 in eight phases - l = 8 a + 4 h + w and l + 32, (h; a)
+// in the order (0; 0, 2, 1, 3), (1; 0, 2, 1, 3) - so that the butterfly's levels 16, 8 and 4 are adds of whole
+// accumulator tiles as the phases end (done while the next phase multiplies into a second accumulator); levels 2 and 1
+// add the four waves' tiles through LDS. The operands (f32 weights only) come through LDS: a stage is 64 rows (32 of x,
+// 32 of W) x 512 bytes - four chunks of the four lanes l and of l + 32 - sent there by global_load_lds_dwordx4 from two
+// waves of their own (an instruction issued between MFMAs holds its wave up for about 40 cycles), two stages ahead, into
+// one of three buffers; an instruction carries two rows, and row r's piece p lies at place p ^ (r % 16) (within its
+// half of 16), so that the 16 rows an operand read touches fall on 16 different bank groups. The waves read a stage's
+// operands right after the meeting that says it has landed and multiply the stage before it meanwhile.
+// The weight rows past the last full 32 (the router's 513th) are left to the first loading wave, idle half of the
+// time: an item is one such row against four rows of x, its loads go out in pieces after the first stages' and are
+// back, the loads completing in order, where a stage asked for after them is waited for.
 typedef float v32f __attribute__((ext_vector_type(32)));
 typedef float v16f __attribute__((ext_vector_type(16)));
-constexpr int RM_TILE = 32, RM_THREADS = 256, RM_ROWB = 256, RM_STAGE = 2 * RM_TILE * RM_ROWB, RM_BUFS = 4;
-__global__ void __launch_bounds__(RM_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
-k_gemv_rows_mfma(const float* __restrict__ W, const float* __restrict__ x, float* __restrict__ y, int rows, int n, int T, int ntt, int net,
-                 int tile_blocks, int left_blocks) {
-    __shared__ __align__(16) uint8_t lds[RM_BUFS * RM_STAGE];
+constexpr int RM_TILE = 32, RM_WAVES = 4, RM_LOADERS = 2, RM_THREADS = (RM_WAVES + RM_LOADERS) * 64, RM_ROWB = 512, RM_STAGE = 2 * RM_TILE * RM_ROWB, RM_BUFS = 3;
+constexpr int RM_PIECE = 10 * 1024, RM_PIECES = 4;   // an item's loads of two steps (a weight row's and four x rows' chunks), pieces in LDS at a time
+constexpr int RM_ITEM_AT = 4;                        // the stage after whose loads an item's first piece goes out
+__global__ void __launch_bounds__(RM_THREADS) k_gemv_rows_mfma(const float* __restrict__ W, const float* __restrict__ x, float* __restrict__ y,
+                                                              int rows, int n, int T, int ntt, int net, int tile_blocks, int along) {
+    __shared__ __align__(16) uint8_t lds[RM_BUFS * RM_STAGE + RM_PIECES * RM_PIECE];
     const int wave = uniform((int) (threadIdx.x >> 6)), lane = threadIdx.x & 63;
-    if ((int) blockIdx.x < left_blocks) {   // the rows past the full tiles: a wave takes one of them against four rows of x
-        const int left = rows - net * RM_TILE, item = (int) blockIdx.x * (RM_THREADS / 64) + wave;
-        gemv_row_quad_wave(W, x, y, rows, n, T, net * RM_TILE + item % left, 4 * (item / left), lane);
-        return;
-    }
     // Which tile: block ids go round the eight XCDs, each with an L2 of its own, so an XCD's blocks are given one patch of
     // 4 x 8 tiles after another (1 MB of x and 2 MB of W for rows of 2048: its L2 holds them, every block re-reads both
     // eight times over the phases). The grid covers whole patches; a block whose tile lies outside leaves.
-    const int id = (int) blockIdx.x - left_blocks;
-    const int lin = (id % 8) * (tile_blocks / 8) + id / 8, patches_e = (net + 7) / 8;
+    const int lin = ((int) blockIdx.x % 8) * (tile_blocks / 8) + (int) blockIdx.x / 8, patches_e = (net + 7) / 8;
     const int tt = 4 * ((lin / 32) / patches_e) + (lin % 32) / 8, et = 8 * ((lin / 32) % patches_e) + lin % 8;
     if (tt >= ntt || et >= net) return;
     const int t0 = tt * RM_TILE, e0 = et * RM_TILE;
-    const int nq = n / 512, S = 8 * nq;   // stages: phase-major, a row's stretches of 512 values within a phase
+    const int nh = n / 1024, S = 8 * nh;   // stages: phase-major, a row's quarters of 1024 values within a phase (nh is even)
     const uint32_t lds_at = (uint32_t) (size_t) (__attribute__((address_space(3))) uint8_t*) lds;
-    // The waves meet where a stage must have landed: a wave's loads complete in order, so it waits until only those of the
-    // two stages after it (eight instructions) may be on their way, and for its LDS reads; then for the others. (A plain
-    // barrier instruction: __syncthreads() would wait for every load.)
+    // All waves meet where a stage must have landed. A loader's loads complete in order: it waits until only the newest
+    // stage's (and an item's pieces after them) may be on their way; the others wait for their own LDS reads. (A plain barrier instruction: __syncthreads() would wait for every load.)
     auto meet = [&](int in_flight) {
         __builtin_amdgcn_sched_barrier(0);
-        if (in_flight == 8) __builtin_amdgcn_s_waitcnt(0x0078);        // vmcnt(8) lgkmcnt(0)
-        else if (in_flight == 4) __builtin_amdgcn_s_waitcnt(0x0074);   // vmcnt(4) lgkmcnt(0)
-        else __builtin_amdgcn_s_waitcnt(0x0070);                       // vmcnt(0) lgkmcnt(0)
+        if (in_flight == 36) __builtin_amdgcn_s_waitcnt(0x8074);        // vmcnt(36) lgkmcnt(0)
+        else if (in_flight == 26) __builtin_amdgcn_s_waitcnt(0x407A);   // vmcnt(26) lgkmcnt(0)
+        else if (in_flight == 16) __builtin_amdgcn_s_waitcnt(0x4070);   // vmcnt(16) lgkmcnt(0)
+        else __builtin_amdgcn_s_waitcnt(0x0070);                        // vmcnt(0) lgkmcnt(0)
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
     };
-    // this wave's four load instructions of a stage: instruction j = 4 wave + jj carries rows 4 j .. 4 j + 3 (rows 0..31
-    // of x, 32..63 of W), this lane's piece of its row
-    uint32_t off[4];
+    if (wave >= RM_WAVES) {   // a loader: the first takes the stages' rows of x, the second those of W
+        const int lw = wave - RM_WAVES;
+        uint32_t off[16];   // instruction j: rows 2 j and 2 j + 1 of this loader's half of the stage, this lane's piece
 #pragma unroll
-    for (int jj = 0; jj < 4; ++jj) {
-        const int row = 4 * (4 * wave + jj) + (lane >> 4), p = (lane & 15) ^ (row & 15);
-        const int r = wave < 2 ? min(t0 + row, T - 1) : e0 + row - RM_TILE;
-        off[jj] = (uint32_t) r * (uint32_t) n * 4u + 1024u * (p >> 3) + 512u * ((p >> 2) & 1) + 16u * (p & 3);
+        for (int j = 0; j < 16; ++j) {
+            const int row = 2 * j + (lane >> 5), q = lane & 31, p = (q & 16) | ((q & 15) ^ (row & 15));
+            const int r = lw == 0 ? min(t0 + row, T - 1) : e0 + row;
+            off[j] = (uint32_t) r * (uint32_t) n * 4u + 1024u * (p >> 3) + 512u * ((p >> 2) & 1) + 16u * (p & 3);
+        }
+        const uint8_t* src = reinterpret_cast<const uint8_t*>(lw == 0 ? x : W);
+        int ph = 0, hf = 0;   // the next stage to fetch
+        auto fetch = [&](int buf) {
+            const int q = ph & 3, l0 = 8 * (((q & 1) << 1) | (q >> 1)) + 4 * (ph >> 2);
+            const uint8_t* from = src + 16 * l0 + 4096 * hf;
+#pragma unroll
+            for (int j = 0; j < 16; ++j) lds_load16(from, off[j], lds_at + buf * RM_STAGE + lw * (RM_TILE * RM_ROWB) + j * 1024);
+            if (++hf == nh) hf = 0, ++ph;
+        };
+        // This loader's item of the rows past the tiles: weight row irow against the rows it0 .. it0 + 3 of x, lane l the
+        // chunks l, l + 64, ... A piece - two steps' chunks, ten instructions - goes out after each of the first stages'
+        // loads, into LDS like them (so that every load in flight is one that the meetings count), and is added up three
+        // meetings later: the stage waited for there was asked for after it.
+        // (Block (tt, et) takes the row et / 8 past the tiles against the et % 8-th four of its own 32 rows of x: rows that its
+        // XCD's L2 holds anyway.)
+        const int steps = n / 256, pieces = steps / 2;
+        const bool has_item = lw == 0 && along && et < 8 * (rows - net * RM_TILE);
+        const int irow = has_item ? net * RM_TILE + et / 8 : 0, it0 = has_item ? t0 + 4 * (et % 8) : 0;
+        const uint8_t* irows[5] = {reinterpret_cast<const uint8_t*>(W + (size_t) irow * n), nullptr, nullptr, nullptr, nullptr};
+#pragma unroll
+        for (int t = 0; t < 4; ++t) irows[1 + t] = reinterpret_cast<const uint8_t*>(x + (size_t) min(it0 + t, T - 1) * n);
+        const uint8_t* ilds = lds + RM_BUFS * RM_STAGE;
+        float iacc[4] = {0.f, 0.f, 0.f, 0.f};
+        fetch(0);
+        fetch(1);   // (S >= 16)
+        int buf = 2;
+        for (int k = 0; k <= S; ++k) {   // (the others meet once more than there are stages: they read one ahead)
+            const int kp = k - RM_ITEM_AT;   // the piece that goes out in this round
+            const int younger = (has_item && kp >= 2 && kp - 2 < pieces ? 10 : 0) + (has_item && kp >= 1 && kp - 1 < pieces ? 10 : 0);
+            meet(k + 1 >= S ? 0 : 16 + younger);
+            if (k + 2 < S) fetch(buf);
+            buf = buf == RM_BUFS - 1 ? 0 : buf + 1;
+            if (has_item && kp >= 0 && kp < pieces) {
+                const uint32_t at = lds_at + RM_BUFS * RM_STAGE + (kp & (RM_PIECES - 1)) * RM_PIECE;
+#pragma unroll
+                for (int s = 0; s < 2; ++s)
+#pragma unroll
+                    for (int r = 0; r < 5; ++r) lds_load16(irows[r] + (2 * kp + s) * 1024, 16u * lane, at + (5 * s + r) * 1024);
+            }
+            if (has_item && kp >= 3 && kp - 3 < pieces) {
+                const uint8_t* p = ilds + ((kp - 3) & (RM_PIECES - 1)) * RM_PIECE + 16 * lane;
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    const float4 w = *reinterpret_cast<const float4*>(p + 5 * s * 1024);
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        const float4 bv = *reinterpret_cast<const float4*>(p + (5 * s + 1 + t) * 1024);
+                        float a = iacc[t];
+                        a = fmaf(w.x, bv.x, a);
+                        a = fmaf(w.y, bv.y, a);
+                        a = fmaf(w.z, bv.z, a);
+                        a = fmaf(w.w, bv.w, a);
+                        iacc[t] = a;
+                    }
+                }
+            }
+        }
+        meet(0);   // the tiles' meeting below
+        if (has_item) {   // the butterfly over the item's four sums (when nobody waits for this wave any more): levels 32 and 16
+                          // for all four at once, a 16-lane row then holds one sum's values for levels 8 .. 1
+            float v = swap16_add(swap32_add(iacc[0], iacc[1]), swap32_add(iacc[2], iacc[3]));   // rows: sums 0, 2, 1, 3
+#pragma unroll
+            for (int o = 8; o; o >>= 1) v += __shfl_xor(v, o, WAVE);
+            const int row = lane >> 4, ti = it0 + (((row & 1) << 1) | (row >> 1));
+            if ((lane & 15) == 0 && ti < T) y[(size_t) ti * rows + irow] = v;
+        }
+        return;
     }
-    const uint8_t* src = reinterpret_cast<const uint8_t*>(wave < 2 ? x : W);
-    int fph = 0, fq = 0, fbuf = 0, fetched = 0;   // the next stage to fetch: phase, stretch, buffer, number
-    const uint8_t* fsrc = src;
-    uint32_t fat = 0;
-    auto fetch_begin = [&]() {   // the scalars of the next stage's loads
-        const int q = fph & 3, l0 = 8 * (((q & 1) << 1) | (q >> 1)) + 4 * (fph >> 2);
-        fsrc = src + 16 * l0 + 2048 * fq;
-        fat = lds_at + fbuf * RM_STAGE + wave * 4096;
-    };
-    auto fetch_one = [&](int jj) {
-        if (fetched < S) lds_load16(fsrc, off[jj], fat + jj * 1024);
-    };
-    auto fetch_end = [&]() {
-        if (++fq == nq) fq = 0, ++fph;
-        fbuf = fbuf == RM_BUFS - 1 ? 0 : fbuf + 1;
-        ++fetched;
-    };
     const int i = lane & 31, b = lane >> 5;
-    // this lane's operands of a stage: row i of x and row i of W, chunks 0 and 1 of lane l (block b: l + 32)
-    const uint8_t* r0 = lds + i * RM_ROWB + 16 * ((4 * b + wave) ^ (i & 15));
-    const uint8_t* r1 = lds + i * RM_ROWB + 16 * ((8 + 4 * b + wave) ^ (i & 15));
-    float4 A[2][2], B[2][2];
-    int buf = 0, met = 0;   // the buffer whose operands are read next; meetings so far
-    auto next_stage = [&](float4 (&a)[2], float4 (&bb)[2]) {
-        meet(met + 2 < S ? 8 : met + 1 < S ? 4 : 0);   // stage `met` has landed
-        ++met;
+    // this lane's operands of a stage: row i of x and row i of W, chunks 0 .. 3 of lane l (block b: l + 32)
+    const uint8_t* r0 = lds + i * RM_ROWB + 16 * ((4 * b + wave) ^ (i & 15));       // chunks 0 and 2 (256 bytes on)
+    const uint8_t* r1 = lds + i * RM_ROWB + 16 * ((8 + 4 * b + wave) ^ (i & 15));   // chunks 1 and 3
+    float4 A[2][4], B[2][4];
+    int buf = 0;   // the buffer whose operands are read next
+    auto next_stage = [&](float4 (&a)[4], float4 (&bb)[4]) {
+        meet(0);
         const int o = buf * RM_STAGE;   // (past the last stage: a buffer's old contents, not used)
         a[0] = *reinterpret_cast<const float4*>(r0 + o);
         a[1] = *reinterpret_cast<const float4*>(r1 + o);
+        a[2] = *reinterpret_cast<const float4*>(r0 + o + 256);
+        a[3] = *reinterpret_cast<const float4*>(r1 + o + 256);
         bb[0] = *reinterpret_cast<const float4*>(r0 + o + RM_TILE * RM_ROWB);
         bb[1] = *reinterpret_cast<const float4*>(r1 + o + RM_TILE * RM_ROWB);
+        bb[2] = *reinterpret_cast<const float4*>(r0 + o + RM_TILE * RM_ROWB + 256);
+        bb[3] = *reinterpret_cast<const float4*>(r1 + o + RM_TILE * RM_ROWB + 256);
         buf = buf == RM_BUFS - 1 ? 0 : buf + 1;
-        fetch_begin();
         __builtin_amdgcn_sched_barrier(0);
     };
     v32f acc[2];
-    v16f t, held, u0, sum;
-    // A stage's 8 steps into accumulator c (first: the phase's first stage, which starts from zero), this wave's loads of
-    // the stage three on after every other one. kind >= 0: the fold of the phase before, whose accumulator is cf - the
-    // butterfly's levels 32 (the instruction's two blocks), 16, 8 and 4 - goes in between on the vector unit. kind 0: the
-    // phase of a = 0 or a = 1: held; 1: a = 2, level 16 with a = 0; 3 and 4: a = 3, level 16 with a = 1, level 8, and for
-    // h = 1 (4) level 4.
-    auto fold_a = [&](const v32f& cf) {
+    float held[16], u0[16], sum[16];   // (plain arrays: no need for runs of 16 registers)
+    // The fold of a phase, whose accumulator is cf: the butterfly's levels 32 (the instruction's two blocks; the sums
+    // take the place of the first block), 16, 8 and 4, in three pieces that go between the next phase's first MFMAs on
+    // the vector unit. The phases of a = 0 and a = 1 (kind 0) leave held; that of a = 2 (odd) adds level 16 with a = 0
+    // into u0; that of a = 3 adds level 16 with a = 1 and level 8 into sum, and at the very end (last) level 4. Which of
+    // the latter two it is, is a select on a scalar, not a branch: the stretch of MFMAs stays one block of code.
+    auto fold_a = [&](v32f& cf) {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) t[v] = cf[v] + cf[16 + v];
+        for (int v = 0; v < 16; ++v) cf[v] = cf[v] + cf[16 + v];
     };
-    auto fold_b = [&](auto kind_c) {
-        constexpr int kind = decltype(kind_c)::value;
-        if constexpr (kind == 0) held = t;
-        else if constexpr (kind == 1) u0 = held + t;
-        else t = held + t;
+    auto fold_b = [&](bool first_of_pair, bool odd, v32f& cf) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            if (first_of_pair) {
+                held[v] = cf[v];
+            } else {
+                cf[v] = held[v] + cf[v];
+                u0[v] = odd ? cf[v] : u0[v];
+            }
+        }
     };
-    auto fold_c = [&](auto kind_c) {
-        constexpr int kind = decltype(kind_c)::value;
-        if constexpr (kind == 3) sum = u0 + t;
-        else if constexpr (kind == 4) sum = sum + (u0 + t);
+    auto fold_c = [&](bool first_of_pair, bool odd, bool last, const v32f& cf) {
+        if (first_of_pair) return;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            if (last) sum[v] = sum[v] + (u0[v] + cf[v]);
+            else sum[v] = odd ? sum[v] : u0[v] + cf[v];
+        }
     };
-    auto multiply = [&](const float4 (&a)[2], const float4 (&bb)[2], v32f& c, auto first_c, auto kind_c, v32f& cf) {
+    // a stage's 16 steps into accumulator c (first: the phase's first stage, which starts from zero, with the fold of the
+    // phase before, unless it is a later stage)
+    auto multiply = [&](const float4 (&a)[4], const float4 (&bb)[4], v32f& c, auto first_c, bool first_of_pair, bool odd, v32f& cf) {
         constexpr bool first = decltype(first_c)::value;
-        constexpr int kind = decltype(kind_c)::value;
-        if constexpr (kind >= 0) asm volatile("" : "+v"(cf));   // (keeps the fold's adds on this side of the meeting)
+        if constexpr (first) asm volatile("" : "+v"(cf));   // (keeps the fold's adds on this side of the meeting)
 #pragma unroll
-        for (int cc = 0; cc < 2; ++cc) {
+        for (int cc = 0; cc < 4; ++cc) {
             if (first && cc == 0) {
                 v32f z;
 #pragma unroll
@@ -419,69 +434,55 @@ k_gemv_rows_mfma(const float* __restrict__ W, const float* __restrict__ x, float
             } else {
                 c = __builtin_amdgcn_mfma_f32_32x32x1f32(a[cc].x, bb[cc].x, c, 0, 0, 0);
             }
-            __builtin_amdgcn_sched_barrier(0);
-            fetch_one(2 * cc);
-            if constexpr (kind >= 0) {
-                if (cc == 0) fold_a(cf);
-                else fold_c(kind_c);
+            if constexpr (first) {
+                if (cc < 3) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (cc == 0) fold_a(cf);
+                    else if (cc == 1) fold_b(first_of_pair, odd, cf);
+                    else fold_c(first_of_pair, odd, false, cf);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
-            __builtin_amdgcn_sched_barrier(0);
             c = __builtin_amdgcn_mfma_f32_32x32x1f32(a[cc].y, bb[cc].y, c, 0, 0, 0);
             c = __builtin_amdgcn_mfma_f32_32x32x1f32(a[cc].z, bb[cc].z, c, 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
-            fetch_one(2 * cc + 1);
-            if constexpr (kind >= 0) {
-                if (cc == 0) fold_b(kind_c);
-            }
-            __builtin_amdgcn_sched_barrier(0);
             c = __builtin_amdgcn_mfma_f32_32x32x1f32(a[cc].w, bb[cc].w, c, 0, 0, 0);
         }
-        fetch_end();
         __builtin_amdgcn_sched_barrier(0);
     };
     using std::integral_constant;
     constexpr integral_constant<bool, true> yes{};
     constexpr integral_constant<bool, false> no{};
-    constexpr integral_constant<int, -1> none{};
-    // a phase into accumulator c, the phase before's fold along with its first stage (nq is even)
-    auto phase = [&](v32f& c, auto kind_c, v32f& cf) {
+    // a phase into accumulator c, the phase before's fold (accumulator cf) along with its first stage
+    auto phase = [&](v32f& c, bool first_of_pair, bool odd, v32f& cf) {
         next_stage(A[1], B[1]);
-        multiply(A[0], B[0], c, yes, kind_c, cf);
+        multiply(A[0], B[0], c, yes, first_of_pair, odd, cf);
         next_stage(A[0], B[0]);
-        multiply(A[1], B[1], c, no, none, c);
-        for (int h2 = 2; h2 < nq; h2 += 2) {
+        multiply(A[1], B[1], c, no, false, false, c);
+        for (int h2 = 2; h2 < nh; h2 += 2) {
             next_stage(A[1], B[1]);
-            multiply(A[0], B[0], c, no, none, c);
+            multiply(A[0], B[0], c, no, false, false, c);
             next_stage(A[0], B[0]);
-            multiply(A[1], B[1], c, no, none, c);
+            multiply(A[1], B[1], c, no, false, false, c);
         }
     };
-    // the first four stages on their way
-#pragma unroll 1
-    for (int k = 0; k < 4; ++k) {
-        fetch_begin();
-#pragma unroll
-        for (int jj = 0; jj < 4; ++jj) fetch_one(jj);
-        fetch_end();
-    }
 #pragma unroll
     for (int v = 0; v < 32; ++v) acc[1][v] = 0.f;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) held[v] = u0[v] = 0.f;
+    for (int v = 0; v < 16; ++v) held[v] = u0[v] = sum[v] = 0.f;
     next_stage(A[0], B[0]);
+    // pairs of phases: (a = 0, a = 2), (a = 1, a = 3), and again for h = 1. The first of a pair folds the second of the pair
+    // before (the very first: nothing, and what that leaves is overwritten), the second the first.
 #pragma unroll 1
-    for (int h = 0; h < 2; ++h) {
-        phase(acc[0], integral_constant<int, 3>{}, acc[1]);   // (h = 0: of nothing, and what it leaves is overwritten)
-        phase(acc[1], integral_constant<int, 0>{}, acc[0]);
-        phase(acc[0], integral_constant<int, 1>{}, acc[1]);
-        phase(acc[1], integral_constant<int, 0>{}, acc[0]);
+    for (int pp = 0; pp < 4; ++pp) {
+        phase(acc[0], false, (pp & 1) != 0, acc[1]);
+        phase(acc[1], true, false, acc[0]);
     }
     fold_a(acc[1]);
-    fold_b(integral_constant<int, 4>{});
-    fold_c(integral_constant<int, 4>{});
-    // levels 2 and 1 over the waves' tiles, in the buffer that the last stage left (all have read it; the one after it
-    // may still be being read, for nothing, by another wave)
-    float* red = reinterpret_cast<float*>(lds + ((S - 1) % RM_BUFS) * RM_STAGE);
+    fold_b(false, false, acc[1]);
+    fold_c(false, false, true, acc[1]);
+    // levels 2 and 1 over the waves' tiles, in the buffer that the stage before the last left (all have read it; the
+    // last one's successor may still be being read, for nothing, by another wave)
+    float* red = reinterpret_cast<float*>(lds + ((S - 2) % RM_BUFS) * RM_STAGE);
 #pragma unroll
     for (int v = 0; v < 16; ++v) red[(wave * 16 + v) * 64 + lane] = sum[v];
     meet(0);
