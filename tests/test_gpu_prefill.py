@@ -199,3 +199,36 @@ def test_prefill_layer_large_chunk_equals_small_chunks(dev):
     for c0 in range(0, Cn, small):
         part = L.run(x[c0:c0 + small])["out"]
         assert int(np.count_nonzero(part.view(np.uint32) != big[c0:c0 + small].view(np.uint32))) == 0, f"rows {c0}.."
+
+
+def test_prefill_layer_two_chunks_in_flight(dev):
+    """A layer's chunks are independent, and a call's state is all in its workspace: chunks dealt to two streams with a
+    workspace each must leave the bits that the same chunks leave one after the other on one stream."""
+    import ctypes as C
+    n, ff, nexp, topk, Cn, chunks = 2048, 512, 64, 10, 512, 6
+    print(f"case prefill_layer two streams n={n} ff={ff} nexp={nexp} topk={topk} C={Cn}", flush=True)
+    rng = np.random.default_rng(778)
+    nb = lambda rows, cols: rows * cols // 256
+    gu = random_iq3s(rng, nexp * nb(2 * ff, n), dmax=1e-3)
+    down = random_iq3s(rng, nexp * nb(n, ff), dmax=1e-3)
+    sh_gu, sh_down = random_iq3s(rng, nb(2 * ff, n), dmax=1e-3), random_iq3s(rng, nb(n, ff), dmax=1e-3)
+    router = (rng.standard_normal((nexp + 1, n)) * 0.05).astype(np.float32)
+    x = rng.standard_normal((chunks, Cn, n)).astype(np.float32)
+    A = fnx_gpu.PfLayerDev(dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, Cn, packed=True, tile16=True)
+    B = fnx_gpu.PfLayerDev(dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, Cn, packed=True, tile16=True)
+    want = [A.run(x[c])["out"] for c in range(chunks)]
+    t = dev.torch
+    dx = dev.up(x)
+    outs = dev.zeros((chunks, Cn, n), t.float32)
+    streams = [t.cuda.Stream(), t.cuda.Stream()]
+    t.cuda.synchronize()
+    for rep in range(3):
+        outs.zero_()
+        t.cuda.synchronize()
+        for c in range(chunks):
+            L, s = ((A, streams[0]), (B, streams[1]))[c & 1]
+            dev.ok(dev.lib.fnx_moe_prefill_layer(C.byref(L.L), dx[c].data_ptr(), Cn, outs[c].data_ptr(), C.byref(L.ws), s.cuda_stream))
+        t.cuda.synchronize()
+        got = outs.cpu().numpy()
+        for c in range(chunks):
+            assert int(np.count_nonzero(got[c].view(np.uint32) != want[c].view(np.uint32))) == 0, f"round {rep}, chunk {c}"
