@@ -137,7 +137,7 @@ def main():
                     help="gaussian: experts IQ3_S-encoded from N(0, 0.02) weights (benchmark config 2's recipe); bytes: uniformly random blocks")
     ap.add_argument("--shared-q8", action="store_true",
                     help="the shared expert as dense split Q8_0 (the reference's own form, three more launches a window) instead of IQ3_S")
-    ap.add_argument("--no-extras", action="store_true", help="skip the legs beside the headline (streaming calibration, config 1, the other weight kind)")
+    ap.add_argument("--no-extras", action="store_true", help="skip the legs beside the metric (verify: streaming calibration, config 1, the other weight kind; prefill: two chunks in flight)")
     ap.add_argument("--raw-layout", action="store_true", help="leave the weights as raw ggml blocks (skip the load-time re-laying)")
     ap.add_argument("--workload", choices=["verify", "prefill", "decoder", "head", "gemv"], default="verify",
                     help="verify: benchmark config 2 (the headline metric, the default); prefill: config 5, one MoE layer over prompt chunks of 512 "
@@ -737,22 +737,24 @@ def prefill_main(args):
     # Two chunks in flight: the chunks of a prompt are independent within a layer, so a caller may give every other chunk
     # a stream and a workspace of its own; one chunk's small routing launches then run beside the other's big ones.
     # (Reported beside the metric, which stays one chunk after the other on one stream.)
-    b2, ws2 = workspace()
-    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
-    both = [(ws, streams[0]), (ws2, streams[1])]
+    dt2 = None
+    if not args.no_extras:
+        b2, ws2 = workspace()
+        streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+        both = [(ws, streams[0]), (ws2, streams[1])]
 
-    def step2(i):
-        w, s_ = both[i & 1]
-        dev.ok(lib.fnx_moe_prefill_layer(C.byref(layers[i % nsets][0]), xs[i % NX].data_ptr(), CH, outs[i % NX].data_ptr(), C.byref(w), s_.cuda_stream))
+        def step2(i):
+            w, s_ = both[i & 1]
+            dev.ok(lib.fnx_moe_prefill_layer(C.byref(layers[i % nsets][0]), xs[i % NX].data_ptr(), CH, outs[i % NX].data_ptr(), C.byref(w), s_.cuda_stream))
 
-    for i in range(4):
-        step2(i)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(steps):
-        step2(4 + i)
-    torch.cuda.synchronize()
-    dt2 = time.perf_counter() - t0
+        for i in range(4):
+            step2(i)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            step2(4 + i)
+        torch.cuda.synchronize()
+        dt2 = time.perf_counter() - t0
     # routing statistics of the chunks
     active, jobs = [], []
     for i in range(min(steps, 16)):
@@ -824,7 +826,7 @@ def prefill_main(args):
                                          "chunk_frac": max(step_bytes / HBM_PEAK, step_flops / MFMA_F16) / (dt / steps)}},
         "cpu_baseline": cpu,
         # not the metric: two streams with a workspace each, chunks dealt to them in turn
-        "two_chunks_in_flight": {"ms_per_chunk": dt2 / steps * 1e3, "tokens_per_s": CH * steps / dt2},
+        "two_chunks_in_flight": {"ms_per_chunk": dt2 / steps * 1e3, "tokens_per_s": CH * steps / dt2} if dt2 else None,
     }
     print(json.dumps(line))
 
