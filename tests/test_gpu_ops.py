@@ -60,6 +60,41 @@ def test_gemv_f32_many_rows_bit_exact(dev, oracle, rows, n, T):
     assert np.array_equal(dev.gemv(W, x).view(np.uint32), oracle.gemv_f32(W, x).view(np.uint32))
 
 
+def test_gemv_f32_sum_does_not_depend_on_T(dev):
+    """A size-independent property at a size the oracle takes long for: a sum's bits do not depend on how many rows of x a
+    call brings, so 4,099 rows in one call (the matrix cores' tiles, several patches of them, a ragged last tile, the 513th
+    weight row with the loading waves) must equal the same rows in calls of 16 and fewer (the vector units' kernel)."""
+    rows, n, T = 513, 2048, 4099
+    print(f"case gemv_f32 T-independence rows={rows} n={n} T={T}", flush=True)
+    rng = np.random.default_rng(240)
+    W = (rng.standard_normal((rows, n)) * np.exp2(rng.integers(-10, 2, (rows, n)))).astype(np.float32)
+    x = (rng.standard_normal((T, n)) * np.exp2(rng.integers(-6, 6, (T, n)))).astype(np.float32)
+    big = dev.gemv(W, x).view(np.uint32)
+    for t0 in list(range(0, 256, 16)) + [1024, 2048, 4080, 4096]:
+        small = dev.gemv(W, x[t0:t0 + 16]).view(np.uint32)
+        assert np.array_equal(big[t0:t0 + len(small)], small), f"rows {t0}.."
+
+
+def test_gemv_f32_many_rows_non_finite(dev, oracle):
+    """Infinities and NaNs in x and W go through the matrix cores' chains as through fmaf: the same sums are NaN, the same
+    +-inf, the finite ones keep their bits (a NaN's payload is not compared)."""
+    rows, n, T = 65, 2048, 64
+    rng = np.random.default_rng(241)
+    W = (rng.standard_normal((rows, n)) * 0.02).astype(np.float32)
+    x = rng.standard_normal((T, n)).astype(np.float32)
+    x[3, 100] = np.inf
+    x[5, 7] = -np.inf
+    x[9, 2000] = np.nan
+    W[10, 100] = 0.0        # inf * 0 = NaN in row 3 x weight row 10
+    W[20, 50] = np.inf
+    W[64, 1] = np.nan       # the weight row past the tiles
+    got, want = dev.gemv(W, x), oracle.gemv_f32(W, x)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    ok = ~np.isnan(want)
+    assert np.array_equal(got[ok].view(np.uint32), want[ok].view(np.uint32))
+    assert np.isnan(want).any() and np.isinf(want).any()
+
+
 @pytest.mark.parametrize("T", [16, 45])   # 45 rows: the many-rows kernel, with a ragged last group
 def test_gemv_bf16_bit_exact(dev, oracle, T):
     rng = np.random.default_rng(210)
