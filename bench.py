@@ -31,6 +31,10 @@ HBM_PEAK = 8.0e12
 GATE_UP_TRAFFIC = {"bytes": 137.08e6, "algorithmic_bytes": 125.83e6, "distinct_experts_per_step": 138.45,
                    "source": "profiles/moe_gate_up_hbm_traffic.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this file's default workload; scaled to "
                              "this run's algorithmic bytes; not measured in this run)"}
+# the same for the prompt path's gate|up launch (profiles/prefill_chunk_counters.md: FETCH_SIZE x 2 + WRITE_SIZE)
+PF_GATE_UP_TRAFFIC = {"bytes": 160.9e6, "algorithmic_bytes": 113.4e6,
+                      "source": "profiles/prefill_chunk_counters.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this file's prefill workload; scaled "
+                                "to this run's algorithmic bytes; not measured in this run)"}
 IQ3S_BLOCK = 110
 GU_BYTES = 2 * FF * (N // 256) * IQ3S_BLOCK      # 901,120 per expert
 DN_BYTES = N * (FF // 256) * IQ3S_BLOCK          # 450,560 per expert
@@ -815,7 +819,9 @@ def prefill_main(args):
                    "weight_sets": nsets, "active_experts_per_chunk": u_mean, "jobs_per_chunk": j_mean, "step_algorithmic_bytes": step_bytes,
                    "step_flops": step_flops, "step_hbm_frac": step_bytes / (dt / steps) / HBM_PEAK, "step_mfma_frac": step_flops / (dt / steps) / MFMA_F16},
         "roofline": {"bound": "hbm", "kernel": "k_moe_mma_block64 (routed gate|up, tile16 layout, a job's up to 64 tokens a decode)", "achieved": gu_bytes / (gu_ms * 1e-3) / 1e9, "peak": HBM_PEAK / 1e9,
-                     "unit": "GB/s", "frac": gu_bytes / (gu_ms * 1e-3) / HBM_PEAK, "traffic": None, "kernel_ms": gu_ms, "algorithmic_bytes": gu_bytes,
+                     "unit": "GB/s", "frac": gu_bytes / (gu_ms * 1e-3) / HBM_PEAK,
+                     "traffic": PF_GATE_UP_TRAFFIC["bytes"] * gu_bytes / PF_GATE_UP_TRAFFIC["algorithmic_bytes"] if nsets == 4 else None,
+                     "traffic_source": PF_GATE_UP_TRAFFIC["source"] if nsets == 4 else None, "kernel_ms": gu_ms, "algorithmic_bytes": gu_bytes,
                      "mfma_tflops": gu_flops / (gu_ms * 1e-3) / 1e12, "mfma_frac": gu_flops / (gu_ms * 1e-3) / MFMA_F16,
                      "down": {"kernel_ms": dn_ms, "achieved": dn_bytes / (dn_ms * 1e-3) / 1e9, "mfma_tflops": dn_flops / (dn_ms * 1e-3) / 1e12},
                      "swiglu_ms": sw_ms,
