@@ -927,7 +927,8 @@ static int gemv_any(const void* W, bool bf, const float* x, float* y, int rows, 
     if (rows <= 0 || n <= 0 || n % 256) return fail(std::string(who) + ": n must be a positive multiple of 256");
     if (T < 1 || T > 65535 * FNX_MAXT) return fail(std::string(who) + ": T out of range");
     hipStream_t s = (hipStream_t) st;
-    if (!bf && T >= 2 * RM_TILE && rows >= RM_TILE && n % 2048 == 0 && (uint64_t) T * n * 4 < (1ull << 32) && (uint64_t) rows * n * 4 < (1ull << 32)) {
+    if (!bf && T >= 2 * RM_TILE && rows >= RM_TILE && n % 2048 == 0 && (uint64_t) T * n * 4 < (1ull << 32) && (uint64_t) rows * n * 4 < (1ull << 32) &&
+        (((uintptr_t) W | (uintptr_t) x) & 15) == 0) {
         // a chunk's worth of rows against f32 weights: tiles of 32 x 32 sums on the matrix cores. The weight rows past the
         // last full 32 ride with the tiles' blocks, an item a block (a row x four rows of x); if there are more items
         // than blocks in a row of tiles, those rows go to the kernel below.
