@@ -123,9 +123,39 @@ def gemv_measure(dev, torch, np, steps):
         us = float(np.mean([a.elapsed_time(b) for a, b in evs[2:]])) * 1e3
         nbytes = NM * (mbytes + T * ROWS * 4) + T * (COLS // 32) * 36
         many[f"T{T}"] = {"us_per_launch": us, "algorithmic_bytes": nbytes, "GBps": nbytes / (us * 1e-6) / 1e9, "hbm_frac": nbytes / (us * 1e-6) / HBM_PEAK}
-    del w, out
+    # (c) the same launch over copies in the prompt path's layout (tile16, fnx_iq3s_tile16): jobs of many rows decoded
+    # straight into the matrix cores' operands (k_iq3s_jobs_mma16); the layout to keep for experts that see many rows a job
+    many16 = {}
+    one16 = lib.fnx_iq3s_tile16_bytes(ROWS, COLS, 1)
+    w16 = torch.zeros(one16 * NM, dtype=torch.uint8, device="cuda")
+    dev.ok(lib.fnx_iq3s_tile16(w.data_ptr(), w16.data_ptr(), ROWS, COLS, NM, st))
+    ep16 = torch.tensor([w16.data_ptr() + i * one16 for i in torch.randperm(NM).tolist()], dtype=torch.int64, device="cuda")
+    for T in (1, 16):
+        x = torch.randn((T, COLS), device="cuda", generator=g)
+        xq = torch.zeros(T * (COLS // 32) * 36, dtype=torch.uint8, device="cuda")
+        dev.ok(lib.fnx_quantize_q8_1(x.data_ptr(), xq.data_ptr(), COLS, T, st))
+        jobs = np.zeros(NM, dtype=fnx_gpu.JOB_DTYPE)
+        jobs["w"] = np.arange(NM)
+        jobs["n"] = T
+        jobs["y"][:, :T] = np.arange(T)[None, :]
+        jobs["out"][:, :T] = np.arange(NM)[:, None] * T + np.arange(T)[None, :]
+        dj = dev.up(jobs.view(np.uint8).reshape(-1))
+        out = torch.zeros((NM * T, ROWS), device="cuda")
+        Wall = pkg.dw(w16.data_ptr(), COLS, ROWS, ep=ep16.data_ptr(), tile16=True)
+        evs = []
+        for i in range(8):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            dev.ok(lib.fnx_mmvq(C.byref(Wall), 0, dj.data_ptr(), None, NM, xq.data_ptr(), out.data_ptr(), ROWS, st))
+            b.record()
+            evs.append((a, b))
+        torch.cuda.synchronize()
+        us = float(np.mean([a.elapsed_time(b) for a, b in evs[2:]])) * 1e3
+        nbytes = NM * (one16 + T * ROWS * 4) + T * (COLS // 32) * 36
+        many16[f"T{T}"] = {"us_per_launch": us, "algorithmic_bytes": nbytes, "GBps": nbytes / (us * 1e-6) / 1e9, "hbm_frac": nbytes / (us * 1e-6) / HBM_PEAK}
+    del w, w16, out
     torch.cuda.empty_cache()
-    return {"lone_matrix_a_launch": lone, "launch_of_1024_matrices": many}
+    return {"lone_matrix_a_launch": lone, "launch_of_1024_matrices": many, "launch_of_1024_matrices_tile16": many16}
 
 
 def main():

@@ -92,7 +92,10 @@ size_t fnx_iq3s_tile16_bytes(int nrows, int ncols, int nmat);
 int fnx_quantize_q8_1(const float* x, void* q, int n, int rows, void* st);
 
 /* kernels.hpp:49  mmvq: out[job.out[j]][r] = W[job.w][r] . y[job.y[j]] for every job in jobs[0..*njobs)
- * (njobs null: njobs_max jobs). y: q8_1 rows of W->n_in. */
+ * (njobs null: njobs_max jobs). y: q8_1 rows of W->n_in. W (here and in fnx_moe_gate_up / fnx_moe_down): IQ3_S as ggml
+ * blocks, as unit64, or as tile16 (rows in 16s, 512 .. 2048 columns in 512s; w_stride then counts that layout's bytes):
+ * tile16 is the layout for jobs of many rows, whose weights go decoded straight into matrix-core operands, unit64 the
+ * one for jobs of one or two rows. */
 int fnx_mmvq(const fnx_dw* W, size_t w_stride, const fnx_job* jobs, const int* njobs, int njobs_max, const void* y,
              float* out, int out_stride, void* st);
 

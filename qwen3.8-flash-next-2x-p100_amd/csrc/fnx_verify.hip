@@ -457,6 +457,7 @@ __global__ void __launch_bounds__(512) k_iq3s_jobs(const RowsArgs a) {
 #include "k_iq3s_mma.h"
 #include "k_moe_layer.h"
 #include "k_prefill.h"
+#include "k_iq3s_mma16.h"
 #include "k_decoder.h"
 #include "k_round.h"
 #include "k_sampler.h"
@@ -774,6 +775,18 @@ static int rows_launch(const fnx_dw* W, size_t w_stride, const fnx_job* jobs, co
             case QT_Q4_K: k_qt_jobs<QT_Q4_K><<<grid, 256, 0, s>>>(q); break;
             default: k_qt_jobs<QT_Q5_K><<<grid, 256, 0, s>>>(q); break;
         }
+        return launch_status(who);
+    }
+    if (W->type == FNX_T_IQ3S_TILE16) {   // the prompt path's layout: jobs of many rows, decoded straight into matrix-core operands (k_iq3s_mma16.h)
+        if (W->n_in <= 0 || W->n_in % 512 || W->n_in > J16_MAXCOLS || W->n_out <= 0 || W->n_out % 16)
+            return fail(std::string(who) + ": the tile16 layout takes rows in 16s and 512, 1024, 1536 or 2048 columns here");
+        if (W->row_bytes != (size_t) (W->n_in / 256) * FNX_IQ3S_BLOCK) return fail(std::string(who) + ": row_bytes does not match n_in");
+        if (njobs_max <= 0) return fail(std::string(who) + ": njobs_max must be positive");
+        if (!W->p && !W->ep) return fail(std::string(who) + ": no weights");
+        const RowsArgs a{(const uint8_t*) W->p, w_stride, (const uint8_t* const*) W->ep, W->row_bytes, W->n_out, W->n_in,
+                         jobs, njobs, njobs_max, (const uint8_t*) y, out, out_stride};
+        const long items = (long) njobs_max * (W->n_out / 16);
+        k_iq3s_jobs_mma16<<<(int) std::max(1L, std::min((long) cu_count(), items)), J16_THREADS, 0, (hipStream_t) st>>>(a);
         return launch_status(who);
     }
     if (W->type != FNX_T_IQ3_S && W->type != FNX_T_IQ3S_UNIT64)

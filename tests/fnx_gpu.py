@@ -143,20 +143,30 @@ class Dev:
         self.sync()
         return dst.cpu().numpy()
 
-    def mmvq(self, w, w_stride, nrows, ncols, jobs, yq, out_rows, njobs_dev=True, packed=False):
+    def mmvq(self, w, w_stride, nrows, ncols, jobs, yq, out_rows, njobs_dev=True, packed=False, tile16=False):
+        """tile16: the matrices re-laid a second time into the prompt path's layout (w_stride then counts that layout's bytes)"""
         t = self.torch
         dw_, dj, dy = self.up(w), self.up(jobs.view(np.uint8).reshape(-1)), self.up(yq)
-        if packed:
+        if packed or tile16:
             self.ok(self.lib.fnx_iq3s_repack(dw_.data_ptr(), dw_.data_ptr(), w.size // 110 * 256, self.st()))
         out = self.zeros((out_rows, nrows), t.float32)
         W = self.pkg.dw(dw_, ncols, nrows, packed=packed)
+        if tile16:
+            nmat = w.size // (nrows * (ncols // 256) * 110)
+            one = self.lib.fnx_iq3s_tile16_bytes(nrows, ncols, 1)
+            assert one > 0
+            d16 = self.zeros(one * nmat, t.uint8)
+            self.ok(self.lib.fnx_iq3s_tile16(dw_.data_ptr(), d16.data_ptr(), nrows, ncols, nmat, self.st()))
+            W = self.pkg.dw(d16, ncols, nrows, tile16=True)
+            w_stride = one if w_stride else 0
+            self._keep = d16
         nj = self.up(np.array([len(jobs)], dtype=np.int32))
         self.ok(self.lib.fnx_mmvq(C.byref(W), w_stride, dj.data_ptr(), nj.data_ptr() if njobs_dev else None, len(jobs), dy.data_ptr(),
                                   out.data_ptr(), nrows, self.st()))
         self.sync()
         return out.cpu().numpy()
 
-    def gemv_iq3s(self, w, nrows, ncols, x, packed=False):
+    def gemv_iq3s(self, w, nrows, ncols, x, packed=False, tile16=False):
         T = x.shape[0]
         yq = self.quantize_q8_1(x)
         jobs = np.zeros((T + 15) // 16, dtype=JOB_DTYPE)
@@ -165,7 +175,7 @@ class Dev:
             jobs["n"][j] = nt
             jobs["y"][j, :nt] = np.arange(16 * j, 16 * j + nt)
             jobs["out"][j, :nt] = np.arange(16 * j, 16 * j + nt)
-        return self.mmvq(w, 0, nrows, ncols, jobs, yq, T, packed=packed)
+        return self.mmvq(w, 0, nrows, ncols, jobs, yq, T, packed=packed, tile16=tile16)
 
     def route(self, logits, nexp, topk, fused_W=None, x=None, bf16=False):
         t = self.torch

@@ -205,8 +205,32 @@ def test_gemv_iq3s_encoded_gaussian_weights(dev, oracle, packed):
         assert rel_l2(got, oracle.gemv_exact(w, nrows, ncols, x)) < 3e-2
 
 
-@pytest.mark.parametrize("packed", [False, True])
-def test_mmvq_jobs_pick_experts_and_rows(dev, oracle, packed):
+# the prompt path's layout under the mat-vec operators: jobs decoded straight into the matrix cores' operands
+@pytest.mark.parametrize("nrows,ncols,T", [(4096, 2048, 16), (4096, 2048, 1), (2048, 512, 16), (1024, 2048, 3), (32, 512, 2), (64, 1024, 7),
+                                           (48, 1536, 16), (16, 512, 35)])
+def test_gemv_iq3s_tile16(dev, oracle, nrows, ncols, T):
+    print(f"case gemv_iq3s tile16 nrows={nrows} ncols={ncols} T={T}", flush=True)
+    rng = np.random.default_rng(430 + nrows + ncols + T)
+    w = random_iq3s(rng, nrows * ncols // 256)
+    x = rng.standard_normal((T, ncols)).astype(np.float32)
+    got = dev.gemv_iq3s(w, nrows, ncols, x, tile16=True)
+    want = oracle.gemv_iq3s(w, nrows, ncols, x)
+    assert rel_l2(got, want) <= 1e-5, "only the order of a row's float adds differs"
+
+
+def test_gemv_iq3s_tile16_encoded_gaussian_weights(dev, oracle):
+    rng = np.random.default_rng(431)
+    nrows, ncols = 256, 2048
+    w = oracle.iq3s_quantize((rng.standard_normal(nrows * ncols) * 0.02).astype(np.float32))
+    for T in (1, 16):
+        x = rng.standard_normal((T, ncols)).astype(np.float32)
+        got = dev.gemv_iq3s(w, nrows, ncols, x, tile16=True)
+        assert rel_l2(got, oracle.gemv_iq3s(w, nrows, ncols, x)) <= 1e-5
+        assert rel_l2(got, oracle.gemv_exact(w, nrows, ncols, x)) < 3e-2
+
+
+@pytest.mark.parametrize("packed,tile16", [(False, False), (True, False), (False, True)])
+def test_mmvq_jobs_pick_experts_and_rows(dev, oracle, packed, tile16):
     # several experts, jobs with scattered activation and output rows, count read from device memory
     rng = np.random.default_rng(420)
     nexp, nrows, ncols, nrows_y = 6, 96, 2048, 9
@@ -222,11 +246,11 @@ def test_mmvq_jobs_pick_experts_and_rows(dev, oracle, packed):
         jobs["y"][j, :len(ys)] = ys
         jobs["out"][j, :len(ys)] = np.arange(at, at + len(ys))
         at += len(ys)
-    got = dev.mmvq(w, stride, nrows, ncols, jobs, yq, at, packed=packed)
+    got = dev.mmvq(w, stride, nrows, ncols, jobs, yq, at, packed=packed, tile16=tile16)
     want = oracle.mmvq(w, stride, nrows, ncols, jobs, yq, at)
     assert rel_l2(got, want) <= 1e-5
     # with the device count null the host count is used
-    assert np.array_equal(dev.mmvq(w, stride, nrows, ncols, jobs, yq, at, njobs_dev=False, packed=packed), got)
+    assert np.array_equal(dev.mmvq(w, stride, nrows, ncols, jobs, yq, at, njobs_dev=False, packed=packed, tile16=tile16), got)
 
 
 # ---------------------------------------------------------------- head, drafting, acceptance
