@@ -3,17 +3,17 @@
 // k_iq3s_jobs_mma (unit64: a lane = a sub-block of one row) has to turn its decoded rows by way of LDS before the matrix
 // cores can take 16 rows of a sub-block at once, and the 16 waves' partial sums meet there too: the LDS is its limit.
 // The prompt path's layout gives lane (r, g) of a wave four consecutive sub-blocks of row r of a tile of 16 rows - at
-// step p sub-block 4 g + p of the tile's 16 - which is the A operand of v_mfma_i32_16x16x64_i8 as it is decoded: row r,
-// lane group g, 16 bytes, two instructions a sub-block. The four lane groups then hold four different sub-blocks, whose
-// integer sums must not meet before they have taken their scales; so a step multiplies four times, each time with the
-// activations of three lane groups zeroed (the matrix core is idle most of the time anyway). What is left for the LDS:
-// the codebook lookups, the job's int8 activations (staged once a job, 32 bytes a lane and step), and the sixteen rows'
-// scales of a sub-block, which go from the decoding lanes (row r) to the accumulator's (rows 4 G .. 4 G + 3) through a
-// few words of the wave's own. A wave takes whole tiles of 16 rows and all the columns: no sums to add between waves,
-// no barrier but those around a job's staging.
+// step p sub-block 4 g + p of the tile's 16. v_mfma_i32_16x16x32_i8 wants a sub-block of 16 rows as lane (r, G): row r,
+// bytes 8 G .. 8 G + 7. What the four lane groups hold after a step's decode - four sub-blocks, 32 bytes a lane - is
+// that, for all four sub-blocks, up to a 4 x 4 transpose of 8-byte pairs between lane group and register pair: eight
+// permlane swaps. Then one MFMA a sub-block gives the 16 x 16 integer sums, which take their scales and are added; no
+// decoded weight ever reaches LDS. What is left for the LDS: the codebook lookups, the job's int8 activations (staged
+// once a job, four 8-byte reads a lane and step), and the sixteen rows' scales of a sub-block, which go from the
+// decoding lanes (row r) to the accumulator's (rows 4 G .. 4 G + 3) through a few words of the wave's own. A wave takes
+// whole tiles of 16 rows and all the columns: no sums to add between waves, no barrier but those around a job's staging.
 // out[job.out[j]][r] = W[job.w][r] . y[job.y[j]] as kernels.hpp:49 and moe.cuh:613-658 define it, a term as in
-// k_iq3s_jobs_mma: d_w (1 + 2 s) d_x sumi; a row's sub-blocks are added in the order the steps and lane groups give them
-// (16 S + p + 4 g for S, then p, then g ascending), whatever the job's rows are.
+// k_iq3s_jobs_mma: d_w (1 + 2 s) d_x sumi; a row's sub-blocks are added in the order the steps give them
+// (16 S + p + 4 j for S, then p, then j ascending), whatever the job's rows are.
 #pragma once
 
 #include "k_prefill.h"
@@ -21,8 +21,11 @@
 namespace fnx {
 
 constexpr int J16_THREADS = 1024, J16_WAVES = 16, J16_MAXCOLS = 2048;
-constexpr int J16_XLD = J16_MAXCOLS + 16;   // bytes of a token's int8 row in LDS: 16 lanes' 16-byte reads of one sub-block then fall on all 64 banks
+constexpr int J16_XLD = J16_MAXCOLS + 32;   // bytes of a token's int8 row in LDS: a wave's 8-byte reads of a sub-block then take the two passes their 512 bytes need
 typedef int j16_v4i __attribute__((ext_vector_type(4)));
+// x's lanes 32 .. 63 <-> y's lanes 0 .. 31; x's 16-lane rows 1, 3 <-> y's rows 0, 2 (as instructions: see swap32_add)
+__device__ __forceinline__ void swap32(uint32_t& x, uint32_t& y) { asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(x), "+v"(y)); }
+__device__ __forceinline__ void swap16(uint32_t& x, uint32_t& y) { asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(x), "+v"(y)); }
 struct J16Lds {
     uint32_t tab[SGRID_WORDS];
     __attribute__((aligned(16))) uint8_t xq[FNX_MAXT * J16_XLD];
@@ -36,9 +39,8 @@ __device__ __forceinline__ void j16_segment(J16Lds& L, const uint8_t* __restrict
     const int lane = threadIdx.x & 63, wave = uniform((int) (threadIdx.x >> 6));
     const int r = lane & 15, grp = lane >> 4;   // decoding: row r of the tile, lane group grp; accumulating: token r, rows 4 grp .. 4 grp + 3
     const int nsuper = ncols / 512;
-    const uint32_t keep[4] = {grp == 0 ? ~0u : 0u, grp == 1 ? ~0u : 0u, grp == 2 ? ~0u : 0u, grp == 3 ? ~0u : 0u};
     float* orow = out + (size_t) (r < n ? jb->out[r] : 0) * out_stride + 4 * grp;
-    const uint8_t* xrow = L.xq + r * J16_XLD + 128 * grp;   // sub-block 16 S + 4 grp + p of token r lies 512 S + 32 p further
+    const uint8_t* xrow = L.xq + r * J16_XLD + 8 * grp;   // bytes 8 grp .. of sub-block 16 S + 4 j + p of token r lie 512 S + 128 j + 32 p further
     float* myw = &L.sw[wave][grp][r];
     for (int g = g0 + wave; g < g1; g += J16_WAVES) {
         float acc[4] = {0.f, 0.f, 0.f, 0.f};
@@ -51,27 +53,33 @@ __device__ __forceinline__ void j16_segment(J16Lds& L, const uint8_t* __restrict
                 constexpr int p = decltype(p_c)::value;
                 const SubFields s = super_sub<p>(f);
                 const v4u idx = {s.q0, s.q1, s.q2, s.q3};
-                v4u lo, hi;
+                uint32_t w8[8];   // this lane's sub-block (row r, 16 S + 4 grp + p): 32 int8
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    lo[j] = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint8_t*>(L.tab) + packed_addr(idx, j));
-                    hi[j] = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint8_t*>(L.tab) + packed_addr(idx, 4 + j));
-                }
+                for (int j = 0; j < 8; ++j) w8[j] = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint8_t*>(L.tab) + packed_addr(idx, j));
                 *myw = half_bits_to_float(s.d) * (float) (int) (1u + 2u * s.sc);
-                const v4u b0 = *reinterpret_cast<const v4u*>(xrow + 512 * S + 32 * p), b1 = *reinterpret_cast<const v4u*>(xrow + 512 * S + 32 * p + 16);
+                long b[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) b[j] = *reinterpret_cast<const long*>(xrow + 512 * S + 128 * j + 32 * p);
                 const float4 dxv = *reinterpret_cast<const float4*>(&L.dx[((S * 4 + p) * FNX_MAXT + r) * 4]);
                 const float dxs[4] = {dxv.x, dxv.y, dxv.z, dxv.w};
+                // pair P_k = bytes 8 k .. 8 k + 7 of the lane's sub-block; afterwards pair j holds bytes 8 grp .. of lane group j's
+                swap32(w8[0], w8[4]);
+                swap32(w8[1], w8[5]);
+                swap32(w8[2], w8[6]);
+                swap32(w8[3], w8[7]);
+                swap16(w8[0], w8[2]);
+                swap16(w8[1], w8[3]);
+                swap16(w8[4], w8[6]);
+                swap16(w8[5], w8[7]);
 #pragma unroll
-                for (int gs = 0; gs < 4; ++gs) {   // lane group gs's sub-block: the other groups' activations zeroed
-                    const v4u m0 = {b0.x & keep[gs], b0.y & keep[gs], b0.z & keep[gs], b0.w & keep[gs]};
-                    const v4u m1 = {b1.x & keep[gs], b1.y & keep[gs], b1.z & keep[gs], b1.w & keep[gs]};
-                    j16_v4i d = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(j16_v4i, lo), __builtin_bit_cast(j16_v4i, m0), j16_v4i{0, 0, 0, 0}, 0, 0, 0);
-                    d = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(j16_v4i, hi), __builtin_bit_cast(j16_v4i, m1), d, 0, 0, 0);
-                    const float4 fw = *reinterpret_cast<const float4*>(&L.sw[wave][gs][4 * grp]);
-                    acc[0] = fmaf(fw.x * dxs[gs], (float) d[0], acc[0]);
-                    acc[1] = fmaf(fw.y * dxs[gs], (float) d[1], acc[1]);
-                    acc[2] = fmaf(fw.z * dxs[gs], (float) d[2], acc[2]);
-                    acc[3] = fmaf(fw.w * dxs[gs], (float) d[3], acc[3]);
+                for (int j = 0; j < 4; ++j) {   // lane group j's sub-block, 16 S + 4 j + p
+                    const long a = (long) ((unsigned long) w8[2 * j] | (unsigned long) w8[2 * j + 1] << 32);
+                    const j16_v4i d = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, b[j], j16_v4i{0, 0, 0, 0}, 0, 0, 0);
+                    const float4 fw = *reinterpret_cast<const float4*>(&L.sw[wave][j][4 * grp]);
+                    acc[0] = fmaf(fw.x * dxs[j], (float) d[0], acc[0]);
+                    acc[1] = fmaf(fw.y * dxs[j], (float) d[1], acc[1]);
+                    acc[2] = fmaf(fw.z * dxs[j], (float) d[2], acc[2]);
+                    acc[3] = fmaf(fw.w * dxs[j], (float) d[3], acc[3]);
                 }
             };
             step(std::integral_constant<int, 0>{});
