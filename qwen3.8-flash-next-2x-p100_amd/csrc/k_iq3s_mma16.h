@@ -26,8 +26,10 @@ typedef int j16_v4i __attribute__((ext_vector_type(4)));
 // x's lanes 32 .. 63 <-> y's lanes 0 .. 31; x's 16-lane rows 1, 3 <-> y's rows 0, 2 (as instructions: see swap32_add)
 __device__ __forceinline__ void swap32(uint32_t& x, uint32_t& y) { asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(x), "+v"(y)); }
 __device__ __forceinline__ void swap16(uint32_t& x, uint32_t& y) { asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(x), "+v"(y)); }
+// The signed codebook twice, entry i's two copies side by side (words 2 i and 2 i + 1): even lanes read the even words,
+// odd lanes the odd ones, so the 64 random lookups of a wave instruction are two sets of 32 over 32 banks each.
 struct J16Lds {
-    uint32_t tab[SGRID_WORDS];
+    uint32_t tab[2 * SGRID_WORDS];
     __attribute__((aligned(16))) uint8_t xq[FNX_MAXT * J16_XLD];
     __attribute__((aligned(16))) float dx[(J16_MAXCOLS / 128) * FNX_MAXT * 4];   // [super-step][step p][token][lane group g]: the activations' block scales
     __attribute__((aligned(16))) float sw[J16_WAVES][4][16];                     // [wave][lane group][row]: a step's weight scales d (1 + 2 s)
@@ -42,6 +44,7 @@ __device__ __forceinline__ void j16_segment(J16Lds& L, const uint8_t* __restrict
     float* orow = out + (size_t) (r < n ? jb->out[r] : 0) * out_stride + 4 * grp;
     const uint8_t* xrow = L.xq + r * J16_XLD + 8 * grp;   // bytes 8 grp .. of sub-block 16 S + 4 j + p of token r lie 512 S + 128 j + 32 p further
     float* myw = &L.sw[wave][grp][r];
+    const uint32_t copy_at = 4u * (lane & 1);
     for (int g = g0 + wave; g < g1; g += J16_WAVES) {
         float acc[4] = {0.f, 0.f, 0.f, 0.f};
         SuperFields f = tile16_load(we, 16 * g + r, 0, nsuper);
@@ -55,7 +58,7 @@ __device__ __forceinline__ void j16_segment(J16Lds& L, const uint8_t* __restrict
                 const v4u idx = {s.q0, s.q1, s.q2, s.q3};
                 uint32_t w8[8];   // this lane's sub-block (row r, 16 S + 4 grp + p): 32 int8
 #pragma unroll
-                for (int j = 0; j < 8; ++j) w8[j] = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint8_t*>(L.tab) + packed_addr(idx, j));
+                for (int j = 0; j < 8; ++j) w8[j] = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint8_t*>(L.tab) + 2 * packed_addr(idx, j) + copy_at);
                 *myw = half_bits_to_float(s.d) * (float) (int) (1u + 2u * s.sc);
                 long b[4];
 #pragma unroll
@@ -102,7 +105,7 @@ __global__ void __launch_bounds__(J16_THREADS) k_iq3s_jobs_mma16(const RowsArgs 
     for (int g = threadIdx.x; g < 512; g += J16_THREADS) {   // a code's sixteen signed entries from its unsigned one
         const uint32_t g0 = g_sgrid.v[g];
 #pragma unroll
-        for (int sg = 0; sg < 16; ++sg) L.tab[sg * 512 + g] = signed_entry(g0, sg);
+        for (int sg = 0; sg < 16; ++sg) L.tab[2 * (sg * 512 + g)] = L.tab[2 * (sg * 512 + g) + 1] = signed_entry(g0, sg);
     }
     const int nj = a.njobs ? min(uniform(*a.njobs), a.njobs_max) : a.njobs_max;
     const uint32_t gpj = (uint32_t) a.nrows / 16;   // items per job
