@@ -173,6 +173,7 @@ def main():
                     help="the shared expert as dense split Q8_0 (the reference's own form, three more launches a window) instead of IQ3_S")
     ap.add_argument("--no-extras", action="store_true", help="skip the legs beside the metric (verify: streaming calibration, config 1, the other weight kind; prefill: two chunks in flight)")
     ap.add_argument("--raw-layout", action="store_true", help="leave the weights as raw ggml blocks (skip the load-time re-laying)")
+    ap.add_argument("--down-unit64", action="store_true", help="prefill: leave the down matrices in the unit64 layout (k_moe_mma_tile64) instead of tile16 (k_moe_mma_wave16)")
     ap.add_argument("--workload", choices=["verify", "prefill", "decoder", "head", "gemv"], default="verify",
                     help="verify: benchmark config 2 (the headline metric, the default); prefill: config 5, one MoE layer over prompt chunks of 512 "
                          "rows; decoder: config 4, a verify step of the reduced decoder plus the draft layer; head: config 3, argmax + prompt "
@@ -738,6 +739,13 @@ def prefill_main(args):
             dev.ok(lib.fnx_iq3s_tile16(sh_gu.data_ptr(), sh16.data_ptr(), 2 * FF, N, 1, dev.st()))
             L.gu, L.gu_stride, L.sh_gu = pkg.dw(gu16, N, 2 * FF, tile16=True), lib.fnx_iq3s_tile16_bytes(2 * FF, N, 1), pkg.dw(sh16, N, 2 * FF, tile16=True)
             ws_ = ws_ + [gu16, sh16]
+            if not args.down_unit64:   # and the down matrices
+                dn16 = torch.zeros(lib.fnx_iq3s_tile16_bytes(N, FF, NEXP), dtype=torch.uint8, device="cuda")
+                shd16 = torch.zeros(lib.fnx_iq3s_tile16_bytes(N, FF, 1), dtype=torch.uint8, device="cuda")
+                dev.ok(lib.fnx_iq3s_tile16(down.data_ptr(), dn16.data_ptr(), N, FF, NEXP, dev.st()))
+                dev.ok(lib.fnx_iq3s_tile16(sh_down.data_ptr(), shd16.data_ptr(), N, FF, 1, dev.st()))
+                L.down, L.down_stride, L.sh_down = pkg.dw(dn16, FF, N, tile16=True), lib.fnx_iq3s_tile16_bytes(N, FF, 1), pkg.dw(shd16, FF, N, tile16=True)
+                ws_ = ws_ + [dn16, shd16]
         layers.append((L, router, ws_, raw))
     NX = 8
     xs = torch.randn((NX, CH, N), device="cuda", generator=g)

@@ -458,6 +458,7 @@ __global__ void __launch_bounds__(512) k_iq3s_jobs(const RowsArgs a) {
 #include "k_moe_layer.h"
 #include "k_prefill.h"
 #include "k_iq3s_mma16.h"
+#include "k_moe_mma_wave16.h"
 #include "k_decoder.h"
 #include "k_round.h"
 #include "k_sampler.h"
@@ -1307,7 +1308,13 @@ static int mma_launch(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const 
         a.ffh = A->n_out / 2;
         if (h16_done) *h16_done = true;
     }
-    static const int tok64 = env_int("FNX_MMA_TOK64", 1, 0, 1);
+    static const int tok64 = env_int("FNX_MMA_TOK64", 1, 0, 1), wave16 = env_int("FNX_MMA_WAVE16", 1, 0, 1);
+    if (tile16 && wave16 && !a.h16 && A->n_in == W16_COLS) {
+        // wave form: rows of 512 columns (the down projection), a job's whole activation tile in LDS, one block a CU
+        const int grid = (int) std::max(1l, std::min<long>((long) cu_count(), caps * (A->n_out / 16)));
+        k_moe_mma_wave16<<<grid, W16_THREADS, 0, (hipStream_t) st>>>(a);
+        return launch_status(who);
+    }
     if (use_tile && tok64) {
         // tile form, a block per (job, its up to 64 tokens, 256 rows) in stages of 256 columns, one block a CU (its LDS)
         const long tasks = caps * ((A->n_out + MB_ROWS - 1) / MB_ROWS);

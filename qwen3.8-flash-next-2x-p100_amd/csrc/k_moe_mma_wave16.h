@@ -1,0 +1,230 @@
+// The routed experts' down projection on the matrix cores over tile16 matrices of 512 columns, a wave a tile of 16 rows.
+//
+// The block and tile forms give a block one (job, 256 rows) task at a time and every stage of it two barriers: with rows
+// of 512 columns a task is a single stage, the eight waves of a block meet four times per 32 rows each, and at two waves
+// a SIMD little covers the codebook lookups' latency. Here the whole activation tile of a job - up to 64 tokens x 512
+// columns of f16, 64 KiB - is put in LDS once (by loads that write LDS directly, a token's row per wave instruction), and
+// after that a wave needs nothing from the others: it takes tiles of 16 rows, a lane decodes its four sub-blocks of its
+// row from one contiguous load of the tile16 layout, and the sixteen waves of a block (four a SIMD) meet only where the
+// block goes from one job to the next. The blocks split the (job, tile) items of all jobs by cost - a tile's decode and
+// its job's token tiles of multiplications - into contiguous runs.
+// part[job.out[t]][row] = W[job.w][row] . h16[job.y[t]] as kernels.hpp:330 (moe_down_mma) defines it, with the weights as
+// f16 (d (1 + 2 s) g, each product rounded as k_moe_mma_block64 rounds it) and a row's sub-blocks accumulated in the order
+// of that kernel's steps.
+#pragma once
+
+#include "k_prefill.h"
+
+namespace fnx {
+
+constexpr int W16_THREADS = 1024, W16_WAVES = 16, W16_COLS = 512;
+constexpr int W16_XROW = 2 * W16_COLS + 16;   // bytes of a token's f16 row in LDS (260 words: the 16 tokens of a 16-byte operand read fall on 64 different banks)
+#ifndef W16_DEC
+#define W16_DEC 3
+#endif
+constexpr int W16_MUL = 1;      // an item's cost: W16_DEC for its decode and W16_MUL a token tile of its job
+constexpr int W16_HELD = 2048;  // jobs of a list whose token counts and matrices are read into LDS at once, ahead of the split
+struct Wave16Lds {
+    uint2 tab[SGRID_WORDS];
+    __attribute__((aligned(16))) uint8_t xt[MB_TOK64 * W16_XROW];
+    int first_job, first_tile, last_job, last_tile;   // the block's run: from (first_job, first_tile) up to but not including (last_job, last_tile)
+    uint8_t jn[2][W16_HELD];                          // the token counts of the two lists' jobs, as far as they fit
+    int jw[W16_HELD];                                 // the first list's matrices
+};
+
+__global__ void __launch_bounds__(W16_THREADS) k_moe_mma_wave16(const MmaArgs a) {
+    __shared__ Wave16Lds L;
+    const int tid = threadIdx.x, lane = tid & 63, wave = uniform(tid >> 6), r = lane & 15, grp = lane >> 4;
+    // every job's token count and matrix, a thread a job, both lists at once (entries past a list's count are read too - the
+    // arrays hold cap jobs - and not used): one round of loads instead of dependent ones wherever a job's turn comes
+    // (asked for ahead of the codebook's entries, made meanwhile)
+    int hn[2] = {0, 0}, hn2 = 0, hw[2] = {0, 0};
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int j = tid + i * W16_THREADS;
+        if (j < min(a.cap, W16_HELD)) hn[i] = a.jobs[j].n, hw[i] = a.jobs[j].w;
+    }
+    if (a.jobs2 && tid < min(a.cap2, W16_HELD)) hn2 = a.jobs2[tid].n;
+    const int nj_raw = *a.njobs, nj2_raw = a.jobs2 ? *a.njobs2 : 0;
+    {
+        const uint32_t tab0 = g_sgrid.v[tid & 511];   // a thread's code: its sixteen signed entries are made here
+#pragma unroll
+        for (int i = tid; i < SGRID_WORDS; i += W16_THREADS) {
+            const uint32_t g = signed_entry(tab0, i >> 9);
+            v2h lo, hi;
+            lo.x = (_Float16) (int) (int8_t) (g & 0xFFu);
+            lo.y = (_Float16) (int) (int8_t) ((g >> 8) & 0xFFu);
+            hi.x = (_Float16) (int) (int8_t) ((g >> 16) & 0xFFu);
+            hi.y = (_Float16) (int) (int8_t) (g >> 24);
+            L.tab[i] = make_uint2(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi));
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int j = tid + i * W16_THREADS;
+        if (j < min(a.cap, W16_HELD)) L.jn[0][j] = (uint8_t) max(0, min(FNX_PF_JOB, hn[i])), L.jw[j] = hw[i];
+    }
+    if (a.jobs2) {
+        if (tid < min(a.cap2, W16_HELD)) L.jn[1][tid] = (uint8_t) max(0, min(FNX_PF_JOB, hn2));
+        for (int j = tid + W16_THREADS; j < min(a.cap2, W16_HELD); j += W16_THREADS) L.jn[1][j] = (uint8_t) max(0, min(FNX_PF_JOB, a.jobs2[j].n));
+    }
+    const int nj = min(a.cap, uniform(nj_raw)), nj2 = a.jobs2 ? min(a.cap2, uniform(nj2_raw)) : 0, njall = nj + nj2;
+    const int gpj = a.nrows >> 4;   // items a job
+    // a unit: a tile for every wave of the block - or, where that would leave blocks without work, a single tile
+    const int ut = (long) njall * ((gpj + W16_WAVES - 1) / W16_WAVES) >= 2l * gridDim.x ? W16_WAVES : 1, upj = (gpj + ut - 1) / ut;
+    auto job_at = [&](int j) { return j < nj ? a.jobs + j : a.jobs2 + (j - nj); };
+    auto n_of = [&](int j) {   // job j's tokens, 0 .. FNX_PF_JOB
+        const int l = j < nj ? 0 : 1, k = j < nj ? j : j - nj;
+        return k < W16_HELD ? (int) L.jn[l][k] : max(0, min(FNX_PF_JOB, job_at(j)->n));
+    };
+    __syncthreads();
+    // The block's run of items, in units (a run that ended inside a round of the block's waves would leave most of them
+    // waiting for the few). A unit of job j costs w_j = W16_DEC + W16_MUL * (token tiles of j), a job upj * w_j;
+    // unit (j, u) begins at (the cost of the jobs before j) + u * w_j, and block b takes the units that begin in
+    // [total * b / blocks, total * (b + 1) / blocks). One wave finds the run: a lane adds up a stretch of jobs, the
+    // stretches' sums are added up over the lanes, and the lanes whose stretch holds an end of the run walk it.
+    if (wave == 0) {
+        auto weight_of = [&](int j) {
+            const int n = n_of(j);
+            return n >= 1 ? (uint32_t) (W16_DEC + W16_MUL * ((n + 15) >> 4)) : 0u;
+        };
+        const int per = (njall + 63) >> 6, j0 = min(njall, lane * per), j1 = min(njall, j0 + per);
+        unsigned long long sum = 0;
+        for (int j = j0; j < j1; ++j) sum += (unsigned long long) weight_of(j) * (uint32_t) upj;
+        unsigned long long incl = sum;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const unsigned long long up = __shfl_up(incl, o);
+            if (lane >= o) incl += up;
+        }
+        const unsigned long long total = __shfl(incl, 63);
+        unsigned long long c0, c1;   // (64-bit quotients take a few hundred instructions)
+        if (total <= 0xFFFFFFFFull / gridDim.x) c0 = (uint32_t) total * blockIdx.x / gridDim.x, c1 = (uint32_t) total * (blockIdx.x + 1) / gridDim.x;
+        else c0 = total * blockIdx.x / gridDim.x, c1 = total * (blockIdx.x + 1) / gridDim.x;
+        if (lane == 0) {   // ends that lie past every job's items
+            L.first_job = L.last_job = njall;
+            L.first_tile = L.last_tile = 0;
+        }
+        // the first unit that begins at or after a point inside a job (past its last unit: the next job's first, as a tile past gpj)
+        auto find = [&](unsigned long long c, int& job, int& tile) {
+            unsigned long long at = incl - sum;   // where this lane's stretch begins
+            if (!(at <= c && c < at + sum)) return;
+            for (int j = j0; j < j1; ++j) {
+                const uint32_t w = weight_of(j);
+                const unsigned long long cj = (unsigned long long) w * (uint32_t) upj;
+                if (c < at + cj) {
+                    job = j;
+                    tile = ut * (int) ((uint32_t) (c - at + w - 1) / w);
+                    return;
+                }
+                at += cj;
+            }
+        };
+        find(c0, L.first_job, L.first_tile);
+        find(c1, L.last_job, L.last_tile);
+    }
+    __syncthreads();   // the codebook and the run
+    const int jA = uniform(L.first_job), tA = uniform(L.first_tile), jB = uniform(L.last_job), tB = uniform(L.last_tile);
+    const uint32_t xt_at = (uint32_t) (size_t) (__attribute__((address_space(3))) uint8_t*) L.xt;
+    const uint8_t* xlane = L.xt + r * W16_XROW + 256 * grp;   // token r of a tile, this lane group's four sub-blocks of a super-step
+    int yahead[MB_TP] = {0, 0, 0, 0}, ahead = -1;
+    for (int j = jA; j <= jB && j < njall; ++j) {
+        const int g0 = j == jA ? tA : 0, g1 = j == jB ? min(tB, gpj) : gpj;
+        const fnx_bigjob* jb = job_at(j);
+        const int n = uniform(n_of(j));
+        if (n < 1 || g0 >= g1) continue;   // the same for the whole block
+        const int nt = (n + 15) >> 4, e = j >= nj ? 0 : uniform(j < W16_HELD ? L.jw[j] : jb->w);
+        const uint8_t* we = j >= nj ? a.w2 : a.ep ? uniform_ptr((const uint8_t*) a.ep[e]) : a.w + (size_t) e * a.stride;
+        // the wave's tokens' rows, tokens wave, wave + 16, .. (past the job's last: that one again): asked for while the job
+        // before was multiplied, if that was the list's job before this one
+        int y[MB_TP];
+#pragma unroll
+        for (int i = 0; i < MB_TP; ++i) y[i] = ahead == j ? yahead[i] : uniform(jb->y[min(wave + 16 * i, n - 1)]);
+        __syncthreads();   // the job before has been read
+#pragma unroll
+        for (int i = 0; i < MB_TP; ++i)   // a token's row a wave instruction, 16 bytes a lane
+            if (i < nt) lds_load16(a.x + (size_t) y[i] * a.ldx, 16u * lane, xt_at + (wave + 16 * i) * W16_XROW);
+        if (j + 1 <= jB && j + 1 < njall) {
+            const int nn = uniform(n_of(j + 1));
+            const fnx_bigjob* jn = job_at(j + 1);
+#pragma unroll
+            for (int i = 0; i < MB_TP; ++i) yahead[i] = uniform(jn->y[max(0, min(wave + 16 * i, nn - 1))]);
+            ahead = j + 1;
+        }
+        int orow[MB_TP];
+#pragma unroll
+        for (int tt = 0; tt < MB_TP; ++tt) orow[tt] = tt * 16 + r < n ? jb->out[tt * 16 + r] : -1;
+        int g = g0 + wave;
+        SuperFields f = tile16_load(we, 16 * min(g, g1 - 1) + r, 0, 1);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        for (; g < g1; g += W16_WAVES) {
+            // The oldest wave of a SIMD goes first, so a block's waves drift apart and the first ones wait at the job's end
+            // for the last: every wave takes every priority in turn, a tile each
+#ifndef W16_NOPRIO
+            switch (((wave >> 2) + ((g - g0) >> 4)) & 3) {
+                case 0: __builtin_amdgcn_s_setprio(0); break;
+                case 1: __builtin_amdgcn_s_setprio(1); break;
+                case 2: __builtin_amdgcn_s_setprio(2); break;
+                default: __builtin_amdgcn_s_setprio(3); break;
+            }
+#endif
+            const SuperFields nf = tile16_load(we, 16 * (g + W16_WAVES < g1 ? g + W16_WAVES : g) + r, 0, 1);
+            v4f acc[MB_TP];
+#pragma unroll
+            for (int tt = 0; tt < MB_TP; ++tt) acc[tt] = v4f{0.f, 0.f, 0.f, 0.f};
+            // the token tiles two at a time against the sub-block's operands
+            auto pair = [&](const v8h (&A)[4], int p, auto t0_tag, auto cnt_tag) {
+                constexpr int T0 = decltype(t0_tag)::value, CNT = decltype(cnt_tag)::value;
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {   // two of the four operands at a time: the registers of a block of 1024 threads
+                    v4u B[2][2];
+#pragma unroll
+                    for (int tt = 0; tt < CNT; ++tt)
+#pragma unroll
+                        for (int i = 0; i < 2; ++i) B[tt][i] = *reinterpret_cast<const v4u*>(xlane + (T0 + tt) * 16 * W16_XROW + 64 * p + 32 * h + 16 * i);
+#pragma unroll
+                    for (int i = 0; i < 2; ++i)
+#pragma unroll
+                        for (int tt = 0; tt < CNT; ++tt)
+                            acc[T0 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[2 * h + i], __builtin_bit_cast(v8h, B[tt][i]), acc[T0 + tt], 0, 0, 0);
+                }
+            };
+            auto step = [&](auto p_c) {
+                constexpr int p = decltype(p_c)::value;
+                const SubFields s = super_sub<p>(f);
+                const _Float16 sc = (_Float16) (int) (1 + 2 * s.sc), d = __builtin_bit_cast(_Float16, (unsigned short) s.d);
+                const v2h s2 = {sc, sc}, d2 = {d, d};
+                v8h A[4];   // the lane's sub-block (row r, 4 grp + p) as 32 f16 weights
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    const uint2 en = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint8_t*>(L.tab) + sub_entry<true>(s, k));
+                    const v2h lo = (as_v2h(en.x) * s2) * d2, hi = (as_v2h(en.y) * s2) * d2;
+                    A[k >> 1][4 * (k & 1) + 0] = lo.x;
+                    A[k >> 1][4 * (k & 1) + 1] = lo.y;
+                    A[k >> 1][4 * (k & 1) + 2] = hi.x;
+                    A[k >> 1][4 * (k & 1) + 3] = hi.y;
+                }
+                using I0 = std::integral_constant<int, 0>;
+                using I1 = std::integral_constant<int, 1>;
+                using I2 = std::integral_constant<int, 2>;
+                if (nt >= 2) pair(A, p, I0{}, I2{});
+                else pair(A, p, I0{}, I1{});
+                if (nt == 3) pair(A, p, I2{}, I1{});
+                else if (nt == 4) pair(A, p, I2{}, I2{});
+            };
+            step(std::integral_constant<int, 0>{});
+            step(std::integral_constant<int, 1>{});
+            step(std::integral_constant<int, 2>{});
+            step(std::integral_constant<int, 3>{});
+            // lane: token r of each tile, rows 4 grp .. 4 grp + 3 of the tile
+#pragma unroll
+            for (int tt = 0; tt < MB_TP; ++tt)
+                if (orow[tt] >= 0)
+                    *reinterpret_cast<float4*>(a.out + (size_t) orow[tt] * a.nrows + 16 * g + 4 * grp) = make_float4(acc[tt].x, acc[tt].y, acc[tt].z, acc[tt].w);
+            f = nf;
+        }
+    }
+}
+
+}  // namespace fnx

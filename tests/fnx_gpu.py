@@ -265,7 +265,7 @@ class Dev:
         self.sync()
         return out.cpu().numpy()
 
-    def moe_mma(self, w, w_stride, nrows, ncols, jobs, x16, out_rows, packed=False, down=False, cap=None):
+    def moe_mma(self, w, w_stride, nrows, ncols, jobs, x16, out_rows, packed=False, down=False, cap=None, tile16=False):
         """jobs: int32 [njobs][130]; the job count is read from device memory, the arrays hold `cap` jobs"""
         t = self.torch
         cap = cap or len(jobs)
@@ -276,6 +276,13 @@ class Dev:
             self.ok(self.lib.fnx_iq3s_repack(dw_.data_ptr(), dw_.data_ptr(), w.size // 110 * 256, self.st()))
         out = self.zeros((out_rows, nrows), t.float32)
         W = self.pkg.dw(dw_, ncols, nrows, packed=packed)
+        if tile16:   # re-laid a second time into the prompt path's layout (w_stride then counts that layout's bytes)
+            assert packed
+            nmat = w.size // (nrows * ncols // 256 * 110)
+            d16 = self.zeros(self.lib.fnx_iq3s_tile16_bytes(nrows, ncols, nmat), t.uint8)
+            self.ok(self.lib.fnx_iq3s_tile16(dw_.data_ptr(), d16.data_ptr(), nrows, ncols, nmat, self.st()))
+            W = self.pkg.dw(d16, ncols, nrows, tile16=True)
+            w_stride = self.lib.fnx_iq3s_tile16_bytes(nrows, ncols, 1) if w_stride else 0
         nj = self.up(np.array([len(jobs)], dtype=np.int32))
         fn = self.lib.fnx_moe_down_mma if down else self.lib.fnx_moe_gate_up_mma
         self.ok(fn(C.byref(W), w_stride, dj.data_ptr(), nj.data_ptr(), cap, dx.data_ptr(), out.data_ptr(), self.st()))
@@ -492,7 +499,7 @@ class PfLayerDev:
     """One MoE layer's weights plus a chunk workspace, for fnx_moe_prefill_layer."""
 
     def __init__(self, dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, C_rows, packed=True, tile16=False):
-        """tile16 (with packed): the gate|up matrices also in the prompt path's own layout (fnx_iq3s_tile16), which the layer then uses"""
+        """tile16 (with packed): the gate|up matrices - and the down matrices, if ff comes in 512s - also in the prompt path's own layout (fnx_iq3s_tile16), which the layer then uses"""
         t = dev.torch
         pkg = dev.pkg
         self.dev, self.n, self.ff, self.nexp, self.topk, self.C = dev, n, ff, nexp, topk, C_rows
@@ -516,6 +523,14 @@ class PfLayerDev:
             self.L.gu = pkg.dw(self.gu16, n, 2 * ff, tile16=True)
             self.L.gu_stride = lib.fnx_iq3s_tile16_bytes(2 * ff, n, 1)
             self.L.sh_gu = pkg.dw(self.sh_gu16, n, 2 * ff, tile16=True)
+            if ff % 512 == 0:   # the down matrices too, where their columns come in 512s
+                self.down16 = dev.zeros(lib.fnx_iq3s_tile16_bytes(n, ff, nexp), t.uint8)
+                self.sh_down16 = dev.zeros(lib.fnx_iq3s_tile16_bytes(n, ff, 1), t.uint8)
+                dev.ok(lib.fnx_iq3s_tile16(self.down.data_ptr(), self.down16.data_ptr(), n, ff, nexp, dev.st()))
+                dev.ok(lib.fnx_iq3s_tile16(self.sh_down.data_ptr(), self.sh_down16.data_ptr(), n, ff, 1, dev.st()))
+                self.L.down = pkg.dw(self.down16, ff, n, tile16=True)
+                self.L.down_stride = lib.fnx_iq3s_tile16_bytes(n, ff, 1)
+                self.L.sh_down = pkg.dw(self.sh_down16, ff, n, tile16=True)
         P = C_rows * topk
         J, S = P // 64 + nexp, (C_rows + 63) // 64
         self.P, self.J = P, J

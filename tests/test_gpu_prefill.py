@@ -118,6 +118,28 @@ def test_moe_mma_matches_oracle(dev, oracle, nrows, ncols, down, packed):
     assert rel_l2(got, want) <= 1e-5, "f16 operands are the oracle's: only the summation order may differ"
 
 
+@pytest.mark.parametrize("nrows,nexp,sizes", [(2048, 40, [64, 1, 17, 0, 16, 33, 48, 5, 64, 64, 2, 0, 31, 64, 49, 15] * 6), (64, 3, [64, 1, 17, 16, 33, 48, 5]),
+                                              (32, 2, [3]), (2048, 2, [64])])
+def test_moe_mma_wave_form_tile16_rows_of_512(dev, oracle, nrows, nexp, sizes):
+    # the down projection over tile16 matrices of 512 columns (k_moe_mma_wave16): blocks that end inside a job and blocks
+    # that hold several, jobs without tokens, fewer items than blocks
+    print(f"case moe_mma wave form nrows={nrows} nexp={nexp} jobs={len(sizes)}", flush=True)
+    ncols = 512
+    rng = np.random.default_rng(733 + nrows + len(sizes))
+    stride = nrows * ncols // 256 * 110
+    w = random_iq3s(rng, nexp * nrows * ncols // 256, dmax=2e-2)
+    rows = max(200, sum(sizes))
+    x16 = rng.standard_normal((rows, ncols)).astype(np.float16)
+    jobs, total = make_jobs(rng, nexp, rows, sizes)
+    got = dev.moe_mma(w, stride, nrows, ncols, jobs, x16, total, packed=True, down=True, cap=len(jobs) + 5, tile16=True)
+    other = dev.moe_mma(w, stride, nrows, ncols, jobs, x16, total, packed=True, down=True, cap=len(jobs) + 5)   # the tile form over unit64
+    assert rel_l2(got, other) <= 1e-6, "the same f16 products: only the summation order differs"
+    assert np.array_equal(got == 0, other == 0)   # (rows no job writes stay as they were)
+    if len(sizes) <= 8:
+        want = oracle.moe_mma(w, stride, nrows, ncols, jobs, PF, x16, total)
+        assert rel_l2(got, want) <= 1e-5, "f16 operands are the oracle's: only the summation order may differ"
+
+
 def test_moe_mma_weights_equal_the_oracles_f16(dev, oracle):
     # x = unit vectors: the product returns single weights, so every dequantised f16 value is checked bit for bit,
     # subnormal ones included (tiny d)
@@ -162,8 +184,10 @@ def test_prefill_layer_matches_oracle(dev, oracle, n, ff, nexp, topk, Cn):
 
 @pytest.mark.parametrize("n,ff,nexp,topk,Cn", [(2048, 512, 48, 10, 300), (1024, 256, 8, 2, 70)])
 def test_prefill_layer_tile16_equals_unit64(dev, oracle, n, ff, nexp, topk, Cn):
-    """the gate|up matrices in the prompt path's own layout: the same arithmetic on the same bytes found elsewhere, so the
-    chunk's result is that of the unit64 layout bit for bit (and the oracle's within the bar)"""
+    """the gate|up matrices in the prompt path's own layout: the same arithmetic on the same bytes found elsewhere, so
+    h = silu(gate) * up is that of the unit64 layout bit for bit, and so is the chunk's result where the down matrices stay
+    unit64 (ff not in 512s); tile16 down matrices go through the wave form, which adds the same f16 products up in another
+    order than the unit64 tile form (and the oracle's within the bar either way)"""
     print(f"case prefill_layer tile16 n={n} ff={ff} nexp={nexp} topk={topk} C={Cn}", flush=True)
     rng = np.random.default_rng(760 + nexp)
     nb = lambda rows, cols: rows * cols // 256
@@ -175,17 +199,23 @@ def test_prefill_layer_tile16_equals_unit64(dev, oracle, n, ff, nexp, topk, Cn):
     a = fnx_gpu.PfLayerDev(dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, Cn, packed=True).run(x)
     b = fnx_gpu.PfLayerDev(dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, Cn, packed=True, tile16=True).run(x)
     assert np.array_equal(a["topi"], b["topi"])
-    assert int(np.count_nonzero(a["out"].view(np.uint32) != b["out"].view(np.uint32))) == 0
+    assert np.array_equal(a["h16"].view(np.uint16), b["h16"].view(np.uint16))
+    if ff % 512:
+        assert int(np.count_nonzero(a["out"].view(np.uint32) != b["out"].view(np.uint32))) == 0
+    else:
+        assert rel_l2(b["out"], a["out"]) <= 1e-6
     want = oracle.moe_prefill_layer(n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, x)
     assert rel_l2(b["out"], want["out"]) <= REL_L2
 
 
-def test_prefill_layer_large_chunk_equals_small_chunks(dev):
+@pytest.mark.parametrize("tile16", [False, True])
+def test_prefill_layer_large_chunk_equals_small_chunks(dev, tile16):
     """A size-independent property at a size the oracle does not reach: a row's result does not depend on what else is in
     its chunk, so 8,192 rows in one call (more tasks than one pass of a block's task list holds, every kernel form's loop
-    over list passes) must equal the same rows in 16 calls of 512, bit for bit."""
+    over list passes, a thousand jobs and more split over the wave form's blocks) must equal the same rows in 16 calls of
+    512, bit for bit, in either layout."""
     n, ff, nexp, topk, Cn, small = 2048, 512, 64, 10, 8192, 512
-    print(f"case prefill_layer large n={n} ff={ff} nexp={nexp} topk={topk} C={Cn}", flush=True)
+    print(f"case prefill_layer large n={n} ff={ff} nexp={nexp} topk={topk} C={Cn} tile16={tile16}", flush=True)
     rng = np.random.default_rng(777)
     nb = lambda rows, cols: rows * cols // 256
     gu = random_iq3s(rng, nexp * nb(2 * ff, n), dmax=1e-3)
@@ -193,8 +223,8 @@ def test_prefill_layer_large_chunk_equals_small_chunks(dev):
     sh_gu, sh_down = random_iq3s(rng, nb(2 * ff, n), dmax=1e-3), random_iq3s(rng, nb(n, ff), dmax=1e-3)
     router = (rng.standard_normal((nexp + 1, n)) * 0.05).astype(np.float32)
     x = rng.standard_normal((Cn, n)).astype(np.float32)
-    big = fnx_gpu.PfLayerDev(dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, Cn, packed=True).run(x)["out"]
-    L = fnx_gpu.PfLayerDev(dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, small, packed=True)
+    big = fnx_gpu.PfLayerDev(dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, Cn, packed=True, tile16=tile16).run(x)["out"]
+    L = fnx_gpu.PfLayerDev(dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, small, packed=True, tile16=tile16)
     assert np.all(np.isfinite(big))
     for c0 in range(0, Cn, small):
         part = L.run(x[c0:c0 + small])["out"]
