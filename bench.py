@@ -861,7 +861,7 @@ def prefill_main(args):
                      "traffic": PF_GATE_UP_TRAFFIC["bytes"] * gu_bytes / PF_GATE_UP_TRAFFIC["algorithmic_bytes"] if nsets == 4 else None,
                      "traffic_source": PF_GATE_UP_TRAFFIC["source"] if nsets == 4 else None, "kernel_ms": gu_ms, "algorithmic_bytes": gu_bytes,
                      "mfma_tflops": gu_flops / (gu_ms * 1e-3) / 1e12, "mfma_frac": gu_flops / (gu_ms * 1e-3) / MFMA_F16,
-                     "down": {"kernel_ms": dn_ms, "achieved": dn_bytes / (dn_ms * 1e-3) / 1e9, "mfma_tflops": dn_flops / (dn_ms * 1e-3) / 1e12},
+                     "down": {"kernel": "k_moe_mma_tile64 (unit64)" if args.down_unit64 or args.raw_layout else "k_moe_mma_wave16 (tile16)", "kernel_ms": dn_ms, "achieved": dn_bytes / (dn_ms * 1e-3) / 1e9, "mfma_tflops": dn_flops / (dn_ms * 1e-3) / 1e12},
                      "swiglu_ms": sw_ms,
                      # the piecewise bound: a launch cannot be faster than its bytes at the HBM peak or its flops at the MFMA peak
                      "piecewise_bound": {"gate_up_us": max(gu_bytes / HBM_PEAK, gu_flops / MFMA_F16) * 1e6,

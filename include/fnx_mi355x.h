@@ -78,8 +78,9 @@ const char* fnx_version(void);
  * fnx_dw.type = FNX_T_IQ3S_UNIT64: every operator below takes both types and gives the same results; the re-laid
  * type is the fast path. Rows must have 256, 512, 1024 or 2048 columns and expert strides must be multiples of 880. */
 int fnx_iq3s_repack(const void* src, void* dst, size_t n_weights, void* st);
-/* A second load-time layout, for the prompt path's matrix-core kernels only (fnx_moe_gate_up_mma, fnx_moe_prefill_layer's
- * gate|up; no counterpart in the reference, whose prompt kernels read raw blocks): nmat matrices of nrows x ncols
+/* A second load-time layout, for the prompt path's matrix-core kernels (fnx_moe_gate_up_mma, fnx_moe_down_mma - the
+ * latter's fast form where rows have 512 columns -, fnx_moe_prefill_layer's gate|up and down) and the mat-vec operators'
+ * jobs of many rows; no counterpart in the reference, whose prompt kernels read raw blocks: nmat matrices of nrows x ncols
  * (rows in 16s, columns in 512s) from the unit64 layout into tiles of 16 rows x 512 columns in which the 64 lanes of a
  * wave find their shares side by side (3,584 bytes a tile: 1.8 % more than the blocks). src: the matrices one after the
  * other in unit64 form; dst: another buffer of fnx_iq3s_tile16_bytes(nrows, ncols, nmat) bytes, expert e at
