@@ -32,9 +32,9 @@ GATE_UP_TRAFFIC = {"bytes": 137.08e6, "algorithmic_bytes": 125.83e6, "distinct_e
                    "source": "profiles/moe_gate_up_hbm_traffic.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this file's default workload; scaled to "
                              "this run's algorithmic bytes; not measured in this run)"}
 # the same for the prompt path's gate|up launch (profiles/prefill_chunk_counters.md: FETCH_SIZE x 2 + WRITE_SIZE)
-PF_GATE_UP_TRAFFIC = {"bytes": 160.9e6, "algorithmic_bytes": 113.4e6,
-                      "source": "profiles/prefill_chunk_counters.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this file's prefill workload; scaled "
-                                "to this run's algorithmic bytes; not measured in this run)"}
+PF_GATE_UP_TRAFFIC = {"bytes": 171.5e6, "algorithmic_bytes": 98.6e6,
+                      "source": "profiles/prefill_chunk_counters.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this file's prefill workload, k_moe_mma_wave16_gu; "
+                                "scaled to this run's algorithmic bytes; not measured in this run)"}
 IQ3S_BLOCK = 110
 GU_BYTES = 2 * FF * (N // 256) * IQ3S_BLOCK      # 901,120 per expert
 DN_BYTES = N * (FF // 256) * IQ3S_BLOCK          # 450,560 per expert
@@ -807,24 +807,30 @@ def prefill_main(args):
     u_mean, j_mean = float(np.mean(active)), float(np.mean(jobs))
     # the two matrix-core launches on their own, with events on the launch stream (torch's current stream)
     reps = 20
+    fused_h = not args.raw_layout   # unit64 and tile16 matrices leave h = silu(gate) * up from the gate|up launch itself
     evs = []
     for i in range(reps + 3):
         L = layers[i % nsets][0]
         step(i)   # routes chunk i: the jobs and xh in the workspace are this chunk's
-        e = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
+        e = [torch.cuda.Event(enable_timing=True) for _ in range(5)]
         e[0].record()
         dev.ok(lib.fnx_moe_gate_up_mma(C.byref(L.gu), L.gu_stride, ws.jobs_gu, ws.njobs, J, ws.xh, ws.gu, st))
         e[1].record()
         dev.ok(lib.fnx_swiglu_h16(ws.gu, FF, P + CH, ws.h16, st))
         e[2].record()
-        dev.ok(lib.fnx_moe_down_mma(C.byref(L.down), L.down_stride, ws.jobs_dn, ws.njobs, J, ws.h16, ws.part, st))
+        if fused_h:   # what the layer runs: the same h from one launch
+            dev.ok(lib.fnx_moe_gate_up_h16_mma(C.byref(L.gu), L.gu_stride, ws.jobs_gu, ws.njobs, J, ws.xh, ws.h16, st))
         e[3].record()
+        dev.ok(lib.fnx_moe_down_mma(C.byref(L.down), L.down_stride, ws.jobs_dn, ws.njobs, J, ws.h16, ws.part, st))
+        e[4].record()
         evs.append(e)
     torch.cuda.synchronize()
-    gu_ms = float(np.mean([e[0].elapsed_time(e[1]) for e in evs[3:]]))
+    gu2_ms = float(np.mean([e[0].elapsed_time(e[1]) for e in evs[3:]]))
     sw_ms = float(np.mean([e[1].elapsed_time(e[2]) for e in evs[3:]]))
-    dn_ms = float(np.mean([e[2].elapsed_time(e[3]) for e in evs[3:]]))
-    gu_bytes = u_mean * GU_BYTES + CH * N * 2 + P * 2 * FF * 4
+    gu_ms = float(np.mean([e[2].elapsed_time(e[3]) for e in evs[3:]])) if fused_h else gu2_ms
+    dn_ms = float(np.mean([e[3].elapsed_time(e[4]) for e in evs[3:]]))
+    # the routed gate|up launch: the experts' matrices, x as f16, and h as f16 (the products themselves, f32, where h is a launch of its own)
+    gu_bytes = u_mean * GU_BYTES + CH * N * 2 + (P * FF * 2 if fused_h else P * 2 * FF * 4)
     dn_bytes = u_mean * DN_BYTES + P * FF * 2 + P * N * 4
     gu_flops, dn_flops = 2.0 * P * 2 * FF * N, 2.0 * P * N * FF
     step_bytes = (u_mean + 1) * (GU_BYTES + DN_BYTES) + ROUTER_BYTES + 2 * CH * N * 4
@@ -848,6 +854,8 @@ def prefill_main(args):
         cpu = {"value": CS / cdt, "unit": "tokens/s per layer", "cores": threads, "kind": "port",
                "sample": f"one pass of the oracle's prefill layer over the first {CS} rows of chunk 0 (f16 operands, f64 accumulation)",
                "parity_rel_l2": err}
+    gu_kernel = ("k_moe_mma_wave16_gu (routed gate|up over tile16, leaves h = silu(gate) * up; a wave a pair of gate and up tiles, a job's up to 64 tokens a decode)"
+                 if fused_h else "k_moe_mma (routed gate|up over raw blocks)")
     line = {
         "metric": "prefill MoE tokens/sec per layer (chunks of 512 rows) + grouped IQ3_S expert GEMM achieved GB/s and MFMA utilisation",
         "value": CH * steps / dt, "unit": "tokens/s per layer", "n_gpus": 1, "steps": steps, "warmup": warmup,
@@ -856,13 +864,13 @@ def prefill_main(args):
         "config": {"workload": "config 5: one MoE layer over prompt chunks of 512 rows, 5,120 routed pairs, 512 IQ3_S experts top-10 with Zipf(1.1) popularity, shared expert",
                    "weight_sets": nsets, "active_experts_per_chunk": u_mean, "jobs_per_chunk": j_mean, "step_algorithmic_bytes": step_bytes,
                    "step_flops": step_flops, "step_hbm_frac": step_bytes / (dt / steps) / HBM_PEAK, "step_mfma_frac": step_flops / (dt / steps) / MFMA_F16},
-        "roofline": {"bound": "hbm", "kernel": "k_moe_mma_block64 (routed gate|up, tile16 layout, a job's up to 64 tokens a decode)", "achieved": gu_bytes / (gu_ms * 1e-3) / 1e9, "peak": HBM_PEAK / 1e9,
+        "roofline": {"bound": "hbm", "kernel": gu_kernel, "achieved": gu_bytes / (gu_ms * 1e-3) / 1e9, "peak": HBM_PEAK / 1e9,
                      "unit": "GB/s", "frac": gu_bytes / (gu_ms * 1e-3) / HBM_PEAK,
                      "traffic": PF_GATE_UP_TRAFFIC["bytes"] * gu_bytes / PF_GATE_UP_TRAFFIC["algorithmic_bytes"] if nsets == 4 else None,
                      "traffic_source": PF_GATE_UP_TRAFFIC["source"] if nsets == 4 else None, "kernel_ms": gu_ms, "algorithmic_bytes": gu_bytes,
                      "mfma_tflops": gu_flops / (gu_ms * 1e-3) / 1e12, "mfma_frac": gu_flops / (gu_ms * 1e-3) / MFMA_F16,
                      "down": {"kernel": "k_moe_mma_tile64 (unit64)" if args.down_unit64 or args.raw_layout else "k_moe_mma_wave16 (tile16)", "kernel_ms": dn_ms, "achieved": dn_bytes / (dn_ms * 1e-3) / 1e9, "mfma_tflops": dn_flops / (dn_ms * 1e-3) / 1e12},
-                     "swiglu_ms": sw_ms,
+                     "two_launches": {"gate_up_ms": gu2_ms, "swiglu_ms": sw_ms, "note": "fnx_moe_gate_up_mma (k_moe_mma_block64, f32 products written) and fnx_swiglu_h16"},
                      # the piecewise bound: a launch cannot be faster than its bytes at the HBM peak or its flops at the MFMA peak
                      "piecewise_bound": {"gate_up_us": max(gu_bytes / HBM_PEAK, gu_flops / MFMA_F16) * 1e6,
                                          "gate_up_frac": max(gu_bytes / HBM_PEAK, gu_flops / MFMA_F16) / (gu_ms * 1e-3),

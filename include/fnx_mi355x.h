@@ -246,6 +246,12 @@ int fnx_moe_gate_up_mma(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, cons
                         void* st);
 /* kernels.hpp:329  swiglu_h16: h16[p][ffs] = f16(silu(gate) * up) of the P stacked rows [gate | up] */
 int fnx_swiglu_h16(const float* gu, int ffs, int P, uint16_t* h16, void* st);
+/* kernels.hpp:328 + 329 in one launch: h16[jobs.out][ffs] = f16(silu(gate) * up) of the products of fnx_moe_gate_up_mma,
+ * which are not written (the same bits as the two calls one after the other; over unit64 rows of up to 512 columns the
+ * two calls add a row's products in another order). For unit64 and tile16 matrices with 2 ffs
+ * rows in 256s and columns in 512s (an error otherwise); fnx_moe_prefill_layer uses it where it can. */
+int fnx_moe_gate_up_h16_mma(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const int* njobs, int njobs_cap, const uint16_t* xh,
+                            uint16_t* h16, void* st);
 /* kernels.hpp:330  moe_down_mma: part[jobs.out][n] = W_e[n][ffs] . h16[jobs.y] */
 int fnx_moe_down_mma(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const int* njobs, int njobs_cap, const uint16_t* h16, float* part,
                      void* st);

@@ -1275,7 +1275,7 @@ int fnx_swiglu_h16(const float* gu, int ffs, int P, uint16_t* h16, void* st) {
 static int mma_launch(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const int* njobs, int njobs_cap, const uint16_t* x, float* out,
                       void* st, const char* who, const fnx_dw* A2 = nullptr, const fnx_bigjob* jobs2 = nullptr, const int* njobs2 = nullptr,
                       int cap2 = 0, uint16_t* h16 = nullptr, bool* h16_done = nullptr) {
-    if (!A || !jobs || !njobs || !x || !out) return fail(std::string(who) + ": null argument");
+    if (!A || !jobs || !njobs || !x || (!out && !h16)) return fail(std::string(who) + ": null argument");
     if (!A->p && !A->ep) return fail(std::string(who) + ": no weights");
     if (A->type != FNX_T_IQ3_S && A->type != FNX_T_IQ3S_UNIT64 && A->type != FNX_T_IQ3S_TILE16) return fail(std::string(who) + ": IQ3_S weights only");
     if (A->type == FNX_T_IQ3S_TILE16 && (A->n_in % 512 || A->n_out % 16)) return fail(std::string(who) + ": the tile16 layout takes rows in 16s and columns in 512s");
@@ -1285,7 +1285,8 @@ static int mma_launch(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const 
     MmaArgs a{(const uint8_t*) A->p, sa, A->ep, A->n_out, A->n_in, jobs, njobs, njobs_cap, x, A->n_in, out};
     static const int per_cu = env_int("FNX_MMA_BLOCKS_PER_CU", 2, 1, 8), form = env_int("FNX_MMA_FORM", 1, 0, 1);
     static const int tile = env_int("FNX_MMA_TILE", 1, 0, 2);   // 0: never, 1: rows of up to 512 columns, 2: always
-    const bool use_tile = tile && A->type == FNX_T_IQ3S_UNIT64 && A->n_out % 16 == 0 && (tile == 2 || A->n_in <= 512);
+    // (the tile form writes the products only: not where h alone is asked for)
+    const bool use_tile = tile && out && A->type == FNX_T_IQ3S_UNIT64 && A->n_out % 16 == 0 && (tile == 2 || A->n_in <= 512);
     const bool tile16 = A->type == FNX_T_IQ3S_TILE16;
     const bool use_block = tile16 || (!use_tile && form == 1 && A->type == FNX_T_IQ3S_UNIT64 && A->n_in % 512 == 0 && A->n_out % 16 == 0);
     const bool merged = A2 && (use_tile || use_block) && A2->p && A2->type == A->type && A2->n_in == A->n_in && A2->n_out == A->n_out;
@@ -1308,7 +1309,16 @@ static int mma_launch(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const 
         a.ffh = A->n_out / 2;
         if (h16_done) *h16_done = true;
     }
+    if (!out && !a.h16) return fail(std::string(who) + ": h alone is left by the block and wave forms only (unit64 or tile16, 2 ff rows in 256s, columns in 512s)");
     static const int tok64 = env_int("FNX_MMA_TOK64", 1, 0, 1), wave16 = env_int("FNX_MMA_WAVE16", 1, 0, 1);
+    static const int wave16_gu = env_int("FNX_MMA_WAVE16_GU", 1, 0, 1);
+    if (tile16 && wave16_gu && a.h16 && a.ffh % 16 == 0) {
+        // wave form for stacked gate|up matrices: a wave a (gate tile, up tile) pair over the row's super-steps, one block a CU
+        const long upj = (a.ffh / 16 + W16_WAVES - 1) / W16_WAVES;
+        const int grid = (int) std::max(1l, std::min<long>((long) cu_count(), caps * upj));
+        k_moe_mma_wave16_gu<<<grid, W16_THREADS, 0, (hipStream_t) st>>>(a);
+        return launch_status(who);
+    }
     if (tile16 && wave16 && !a.h16 && A->n_in == W16_COLS) {
         // wave form: rows of 512 columns (the down projection), a job's whole activation tile in LDS, one block a CU
         const int grid = (int) std::max(1l, std::min<long>((long) cu_count(), caps * (A->n_out / 16)));
@@ -1354,6 +1364,11 @@ static int mma_launch(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const 
 int fnx_moe_gate_up_mma(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const int* njobs, int njobs_cap, const uint16_t* xh, float* gu,
                         void* st) {
     return mma_launch(A, sa, jobs, njobs, njobs_cap, xh, gu, st, "moe_gate_up_mma");
+}
+int fnx_moe_gate_up_h16_mma(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const int* njobs, int njobs_cap, const uint16_t* xh,
+                            uint16_t* h16, void* st) {
+    if (!h16) return fail("moe_gate_up_h16_mma: null argument");
+    return mma_launch(A, sa, jobs, njobs, njobs_cap, xh, nullptr, st, "moe_gate_up_h16_mma", nullptr, nullptr, nullptr, 0, h16);
 }
 int fnx_moe_down_mma(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const int* njobs, int njobs_cap, const uint16_t* h16, float* part,
                      void* st) {

@@ -32,6 +32,55 @@ struct Wave16Lds {
     int jw[W16_HELD];                                 // the first list's matrices
 };
 
+// A tile's super-step: the lane's four sub-blocks of its row (fields f) as f16 operands, against the nt token tiles of
+// the activation tile in LDS (xlane: token r's row at this lane group's sub-blocks), added to acc
+__device__ __forceinline__ void w16_super_step(const uint2* tab, const uint8_t* xlane, const SuperFields& f, int nt, v4f (&acc)[MB_TP]) {
+    // the token tiles two at a time against the sub-block's operands
+    auto pair = [&](const v8h (&A)[4], int p, auto t0_tag, auto cnt_tag) {
+        constexpr int T0 = decltype(t0_tag)::value, CNT = decltype(cnt_tag)::value;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {   // two of the four operands at a time: the registers of a block of 1024 threads
+            v4u B[2][2];
+#pragma unroll
+            for (int tt = 0; tt < CNT; ++tt)
+#pragma unroll
+                for (int i = 0; i < 2; ++i) B[tt][i] = *reinterpret_cast<const v4u*>(xlane + (T0 + tt) * 16 * W16_XROW + 64 * p + 32 * h + 16 * i);
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int tt = 0; tt < CNT; ++tt)
+                    acc[T0 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[2 * h + i], __builtin_bit_cast(v8h, B[tt][i]), acc[T0 + tt], 0, 0, 0);
+        }
+    };
+    auto step = [&](auto p_c) {
+        constexpr int p = decltype(p_c)::value;
+        const SubFields s = super_sub<p>(f);
+        const _Float16 sc = (_Float16) (int) (1 + 2 * s.sc), d = __builtin_bit_cast(_Float16, (unsigned short) s.d);
+        const v2h s2 = {sc, sc}, d2 = {d, d};
+        v8h A[4];   // the lane's sub-block (row r, 4 grp + p) as 32 f16 weights
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const uint2 en = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint8_t*>(tab) + sub_entry<true>(s, k));
+            const v2h lo = (as_v2h(en.x) * s2) * d2, hi = (as_v2h(en.y) * s2) * d2;
+            A[k >> 1][4 * (k & 1) + 0] = lo.x;
+            A[k >> 1][4 * (k & 1) + 1] = lo.y;
+            A[k >> 1][4 * (k & 1) + 2] = hi.x;
+            A[k >> 1][4 * (k & 1) + 3] = hi.y;
+        }
+        using I0 = std::integral_constant<int, 0>;
+        using I1 = std::integral_constant<int, 1>;
+        using I2 = std::integral_constant<int, 2>;
+        if (nt >= 2) pair(A, p, I0{}, I2{});
+        else pair(A, p, I0{}, I1{});
+        if (nt == 3) pair(A, p, I2{}, I1{});
+        else if (nt == 4) pair(A, p, I2{}, I2{});
+    };
+    step(std::integral_constant<int, 0>{});
+    step(std::integral_constant<int, 1>{});
+    step(std::integral_constant<int, 2>{});
+    step(std::integral_constant<int, 3>{});
+}
+
 __global__ void __launch_bounds__(W16_THREADS) k_moe_mma_wave16(const MmaArgs a) {
     __shared__ Wave16Lds L;
     const int tid = threadIdx.x, lane = tid & 63, wave = uniform(tid >> 6), r = lane & 15, grp = lane >> 4;
@@ -173,50 +222,7 @@ __global__ void __launch_bounds__(W16_THREADS) k_moe_mma_wave16(const MmaArgs a)
             v4f acc[MB_TP];
 #pragma unroll
             for (int tt = 0; tt < MB_TP; ++tt) acc[tt] = v4f{0.f, 0.f, 0.f, 0.f};
-            // the token tiles two at a time against the sub-block's operands
-            auto pair = [&](const v8h (&A)[4], int p, auto t0_tag, auto cnt_tag) {
-                constexpr int T0 = decltype(t0_tag)::value, CNT = decltype(cnt_tag)::value;
-#pragma unroll
-                for (int h = 0; h < 2; ++h) {   // two of the four operands at a time: the registers of a block of 1024 threads
-                    v4u B[2][2];
-#pragma unroll
-                    for (int tt = 0; tt < CNT; ++tt)
-#pragma unroll
-                        for (int i = 0; i < 2; ++i) B[tt][i] = *reinterpret_cast<const v4u*>(xlane + (T0 + tt) * 16 * W16_XROW + 64 * p + 32 * h + 16 * i);
-#pragma unroll
-                    for (int i = 0; i < 2; ++i)
-#pragma unroll
-                        for (int tt = 0; tt < CNT; ++tt)
-                            acc[T0 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[2 * h + i], __builtin_bit_cast(v8h, B[tt][i]), acc[T0 + tt], 0, 0, 0);
-                }
-            };
-            auto step = [&](auto p_c) {
-                constexpr int p = decltype(p_c)::value;
-                const SubFields s = super_sub<p>(f);
-                const _Float16 sc = (_Float16) (int) (1 + 2 * s.sc), d = __builtin_bit_cast(_Float16, (unsigned short) s.d);
-                const v2h s2 = {sc, sc}, d2 = {d, d};
-                v8h A[4];   // the lane's sub-block (row r, 4 grp + p) as 32 f16 weights
-#pragma unroll
-                for (int k = 0; k < 8; ++k) {
-                    const uint2 en = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint8_t*>(L.tab) + sub_entry<true>(s, k));
-                    const v2h lo = (as_v2h(en.x) * s2) * d2, hi = (as_v2h(en.y) * s2) * d2;
-                    A[k >> 1][4 * (k & 1) + 0] = lo.x;
-                    A[k >> 1][4 * (k & 1) + 1] = lo.y;
-                    A[k >> 1][4 * (k & 1) + 2] = hi.x;
-                    A[k >> 1][4 * (k & 1) + 3] = hi.y;
-                }
-                using I0 = std::integral_constant<int, 0>;
-                using I1 = std::integral_constant<int, 1>;
-                using I2 = std::integral_constant<int, 2>;
-                if (nt >= 2) pair(A, p, I0{}, I2{});
-                else pair(A, p, I0{}, I1{});
-                if (nt == 3) pair(A, p, I2{}, I1{});
-                else if (nt == 4) pair(A, p, I2{}, I2{});
-            };
-            step(std::integral_constant<int, 0>{});
-            step(std::integral_constant<int, 1>{});
-            step(std::integral_constant<int, 2>{});
-            step(std::integral_constant<int, 3>{});
+            w16_super_step(L.tab, xlane, f, nt, acc);
             // lane: token r of each tile, rows 4 grp .. 4 grp + 3 of the tile
 #pragma unroll
             for (int tt = 0; tt < MB_TP; ++tt)
@@ -224,6 +230,184 @@ __global__ void __launch_bounds__(W16_THREADS) k_moe_mma_wave16(const MmaArgs a)
                     *reinterpret_cast<float4*>(a.out + (size_t) orow[tt] * a.nrows + 16 * g + 4 * grp) = make_float4(acc[tt].x, acc[tt].y, acc[tt].z, acc[tt].w);
             f = nf;
         }
+    }
+}
+
+// ---------------------------------------------------------------- the same form for stacked gate|up matrices (rows of 512 S columns)
+// A job's activations are S tiles of 64 tokens x 512 columns here, and LDS holds one: a block takes units of (job, sixteen
+// gate tiles and the sixteen up tiles that go with them), a wave one such pair, and walks the S super-steps with the
+// pair's accumulators in registers - activation tile S in (two barriers), the gate tile's super-step, the up tile's -
+// and leaves h = silu(gate) * up as f16 (k_swiglu_h16's values). A unit is eight rounds of the down kernel's kind, so the
+// units are dealt like the block form's tasks: the jobs ranked by token tiles, the heaviest first, to and fro over the
+// blocks. The weights of the next tile's super-step are asked for a tile ahead.
+constexpr int W16_SORTJ = 1024, W16_GU_HELD = 1024;
+struct Wave16GuLds {
+    uint2 tab[SGRID_WORDS];
+    __attribute__((aligned(16))) uint8_t xt[MB_TOK64 * W16_XROW];
+    __attribute__((aligned(16))) uint8_t xs[16 * W16_XROW];   // a second tile for jobs of up to 16 tokens: super-step S + 1 comes in while S is multiplied
+    uint8_t jn[2][W16_GU_HELD];
+    int jw[W16_GU_HELD];
+    unsigned short jorder[W16_SORTJ];   // the jobs, most token tiles first (the lower index first among equals)
+};
+__global__ void __launch_bounds__(W16_THREADS) k_moe_mma_wave16_gu(const MmaArgs a) {
+    __shared__ Wave16GuLds L;
+    const int tid = threadIdx.x, lane = tid & 63, wave = uniform(tid >> 6), r = lane & 15, grp = lane >> 4;
+    int hn[2] = {0, 0}, hn2 = 0, hw[2] = {0, 0};
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int j = tid + i * W16_THREADS;
+        if (j < min(a.cap, W16_GU_HELD)) hn[i] = a.jobs[j].n, hw[i] = a.jobs[j].w;
+    }
+    if (a.jobs2 && tid < min(a.cap2, W16_GU_HELD)) hn2 = a.jobs2[tid].n;
+    const int nj_raw = *a.njobs, nj2_raw = a.jobs2 ? *a.njobs2 : 0;
+    {
+        const uint32_t tab0 = g_sgrid.v[tid & 511];
+#pragma unroll
+        for (int i = tid; i < SGRID_WORDS; i += W16_THREADS) {
+            const uint32_t g = signed_entry(tab0, i >> 9);
+            v2h lo, hi;
+            lo.x = (_Float16) (int) (int8_t) (g & 0xFFu);
+            lo.y = (_Float16) (int) (int8_t) ((g >> 8) & 0xFFu);
+            hi.x = (_Float16) (int) (int8_t) ((g >> 16) & 0xFFu);
+            hi.y = (_Float16) (int) (int8_t) (g >> 24);
+            L.tab[i] = make_uint2(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi));
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int j = tid + i * W16_THREADS;
+        if (j < min(a.cap, W16_GU_HELD)) L.jn[0][j] = (uint8_t) max(0, min(FNX_PF_JOB, hn[i])), L.jw[j] = hw[i];
+    }
+    if (a.jobs2) {
+        if (tid < min(a.cap2, W16_GU_HELD)) L.jn[1][tid] = (uint8_t) max(0, min(FNX_PF_JOB, hn2));
+        for (int j = tid + W16_THREADS; j < min(a.cap2, W16_GU_HELD); j += W16_THREADS) L.jn[1][j] = (uint8_t) max(0, min(FNX_PF_JOB, a.jobs2[j].n));
+    }
+    const int nj = min(a.cap, uniform(nj_raw)), nj2 = a.jobs2 ? min(a.cap2, uniform(nj2_raw)) : 0, njall = nj + nj2;
+    const int ffh = a.ffh, nsuper = a.ncols >> 9, ppj = ffh >> 4, upj = (ppj + W16_WAVES - 1) / W16_WAVES;   // pairs of tiles, units a job
+    auto job_at = [&](int j) { return j < nj ? a.jobs + j : a.jobs2 + (j - nj); };
+    auto n_of = [&](int j) {
+        const int l = j < nj ? 0 : 1, k = j < nj ? j : j - nj;
+        return k < W16_GU_HELD ? (int) L.jn[l][k] : max(0, min(FNX_PF_JOB, job_at(j)->n));
+    };
+    __syncthreads();
+    const bool sorted = njall <= W16_SORTJ;
+    if (sorted && wave == 0) {   // a counting sort by one wave, 64 jobs a trip: class totals, then every job's place
+        int total[MB_TP + 1];
+#pragma unroll
+        for (int c = 0; c <= MB_TP; ++c) total[c] = 0;
+        for (int j0 = 0; j0 < njall; j0 += 64) {
+            const int kj = j0 + lane < njall ? (n_of(j0 + lane) + 15) >> 4 : -1;
+#pragma unroll
+            for (int c = 0; c <= MB_TP; ++c) total[c] += __popcll(__ballot(kj == c));
+        }
+        int base[MB_TP + 1];   // where a class starts: the classes in descending order
+        base[MB_TP] = 0;
+#pragma unroll
+        for (int c = MB_TP - 1; c >= 0; --c) base[c] = base[c + 1] + total[c + 1];
+        for (int j0 = 0; j0 < njall; j0 += 64) {
+            const int kj = j0 + lane < njall ? (n_of(j0 + lane) + 15) >> 4 : -1;
+#pragma unroll
+            for (int c = 0; c <= MB_TP; ++c) {
+                const unsigned long long m = __ballot(kj == c);
+                if (kj == c) L.jorder[base[c] + __popcll(m & ((1ull << lane) - 1ull))] = (unsigned short) (j0 + lane);
+                base[c] += __popcll(m);
+            }
+        }
+    }
+    __syncthreads();   // the codebook and the order
+    const uint32_t xt_at = (uint32_t) (size_t) (__attribute__((address_space(3))) uint8_t*) L.xt;
+    const uint32_t xs_at = (uint32_t) (size_t) (__attribute__((address_space(3))) uint8_t*) L.xs;
+    const uint8_t* xlane = L.xt + r * W16_XROW + 256 * grp;
+    const uint8_t* xlane_s = L.xs + r * W16_XROW + 256 * grp;
+    const int units = njall * upj;
+    int yahead[MB_TP] = {0, 0, 0, 0}, ahead = -1;
+    for (int round = 0; round * (int) gridDim.x < units; ++round) {
+        const int pos = (round & 1) ? (int) gridDim.x - 1 - (int) blockIdx.x : (int) blockIdx.x, u = round * (int) gridDim.x + pos;
+        if (u >= units) continue;   // the same for the whole block
+        const int jo = u / upj, q = u - jo * upj, j = sorted ? (int) uniform(L.jorder[jo]) : jo;
+        const fnx_bigjob* jb = job_at(j);
+        const int n = uniform(n_of(j));
+        if (n < 1) continue;
+        const int nt = (n + 15) >> 4, e = j >= nj ? 0 : uniform(j < W16_GU_HELD ? L.jw[j] : jb->w);
+        const uint8_t* we = j >= nj ? a.w2 : a.ep ? uniform_ptr((const uint8_t*) a.ep[e]) : a.w + (size_t) e * a.stride;
+        const int pr = q * W16_WAVES + wave;   // the wave's pair: gate rows 16 pr .., up rows ffh + 16 pr ..
+        const bool mine = pr < ppj;
+        const int grow = 16 * min(pr, ppj - 1) + r;
+        // the wave's tokens' rows (tokens wave, wave + 16, ..; past the job's last: that one again): asked for during the unit
+        // before, if this block knew then what its next unit would be
+        int y[MB_TP];
+#pragma unroll
+        for (int i = 0; i < MB_TP; ++i) y[i] = ahead == u ? yahead[i] : uniform(jb->y[min(wave + 16 * i, n - 1)]);
+        int orow[MB_TP];
+#pragma unroll
+        for (int tt = 0; tt < MB_TP; ++tt) orow[tt] = mine && tt * 16 + r < n ? jb->out[tt * 16 + r] : -1;
+        v4f accg[MB_TP], accu[MB_TP];
+#pragma unroll
+        for (int tt = 0; tt < MB_TP; ++tt) accg[tt] = accu[tt] = v4f{0.f, 0.f, 0.f, 0.f};
+        SuperFields f = tile16_load(we, grow, 0, nsuper);
+        auto next_unit = [&]() {   // the row numbers of the unit after this one
+            const int rn = round + 1, pn = (rn & 1) ? (int) gridDim.x - 1 - (int) blockIdx.x : (int) blockIdx.x, un = rn * (int) gridDim.x + pn;
+            if (un >= units) return;
+            const int jon = un / upj, jn = sorted ? (int) uniform(L.jorder[jon]) : jon, nn = uniform(n_of(jn));
+            const fnx_bigjob* jbn = job_at(jn);
+#pragma unroll
+            for (int i = 0; i < MB_TP; ++i) yahead[i] = uniform(jbn->y[max(0, min(wave + 16 * i, nn - 1))]);
+            ahead = un;
+        };
+        // The oldest wave of a SIMD goes first and the block's waves drift apart between two barriers: every wave takes each
+        // priority in turn, a super-step each
+        auto turn = [&](int S) {
+            switch (((wave >> 2) + S) & 3) {
+                case 0: __builtin_amdgcn_s_setprio(0); break;
+                case 1: __builtin_amdgcn_s_setprio(1); break;
+                case 2: __builtin_amdgcn_s_setprio(2); break;
+                default: __builtin_amdgcn_s_setprio(3); break;
+            }
+        };
+        if (nt == 1) {
+            // up to 16 tokens: two tiles in turn, the next super-step's asked for before this one is multiplied
+            __syncthreads();   // the unit before has been read
+            lds_load16(a.x + (size_t) y[0] * a.ldx, 16u * lane, xt_at + wave * W16_XROW);
+            next_unit();
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            for (int S = 0; S < nsuper; ++S) {
+                turn(S);
+                if (S + 1 < nsuper) lds_load16(a.x + (size_t) y[0] * a.ldx + 512 * (S + 1), 16u * lane, ((S & 1) ? xt_at : xs_at) + wave * W16_XROW);
+                const uint8_t* xl = (S & 1) ? xlane_s : xlane;
+                const SuperFields fu = tile16_load(we, ffh + grow, S, nsuper);
+                if (mine) w16_super_step(L.tab, xl, f, 1, accg);
+                f = tile16_load(we, grow, min(S + 1, nsuper - 1), nsuper);
+                if (mine) w16_super_step(L.tab, xl, fu, 1, accu);
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __syncthreads();   // the other tile has landed, this one has been read
+            }
+        } else {
+            for (int S = 0; S < nsuper; ++S) {
+                __syncthreads();   // the tile before has been read
+#pragma unroll
+                for (int i = 0; i < MB_TP; ++i)   // a token's 512 columns a wave instruction, 16 bytes a lane
+                    if (i < nt) lds_load16(a.x + (size_t) y[i] * a.ldx + 512 * S, 16u * lane, xt_at + (wave + 16 * i) * W16_XROW);
+                if (S == 0) next_unit();
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __syncthreads();
+                turn(S);
+                const SuperFields fu = tile16_load(we, ffh + grow, S, nsuper);
+                if (mine) w16_super_step(L.tab, xlane, f, nt, accg);
+                f = tile16_load(we, grow, min(S + 1, nsuper - 1), nsuper);
+                if (mine) w16_super_step(L.tab, xlane, fu, nt, accu);
+            }
+        }
+        // lane: token r of each tile, rows 4 grp .. 4 grp + 3 of the pair's tiles
+#pragma unroll
+        for (int tt = 0; tt < MB_TP; ++tt)
+            if (orow[tt] >= 0) {
+                const v4f gt = accg[tt], up = accu[tt];
+                uint2 hv;
+                hv.x = (uint32_t) float_to_half_bits(silu_f(gt.x) * up.x) | (uint32_t) float_to_half_bits(silu_f(gt.y) * up.y) << 16;
+                hv.y = (uint32_t) float_to_half_bits(silu_f(gt.z) * up.z) | (uint32_t) float_to_half_bits(silu_f(gt.w) * up.w) << 16;
+                *reinterpret_cast<uint2*>(a.h16 + (size_t) orow[tt] * ffh + 16 * pr + 4 * grp) = hv;
+            }
     }
 }
 

@@ -265,7 +265,7 @@ class Dev:
         self.sync()
         return out.cpu().numpy()
 
-    def moe_mma(self, w, w_stride, nrows, ncols, jobs, x16, out_rows, packed=False, down=False, cap=None, tile16=False):
+    def moe_mma(self, w, w_stride, nrows, ncols, jobs, x16, out_rows, packed=False, down=False, cap=None, tile16=False, h16=False):
         """jobs: int32 [njobs][130]; the job count is read from device memory, the arrays hold `cap` jobs"""
         t = self.torch
         cap = cap or len(jobs)
@@ -284,6 +284,14 @@ class Dev:
             W = self.pkg.dw(d16, ncols, nrows, tile16=True)
             w_stride = self.lib.fnx_iq3s_tile16_bytes(nrows, ncols, 1) if w_stride else 0
         nj = self.up(np.array([len(jobs)], dtype=np.int32))
+        if h16:   # nrows = 2 ffs stacked: h = silu(gate) * up as f16 from one launch, and from the two operators one after the other
+            ffs = nrows // 2
+            one, two = self.zeros((out_rows, ffs), t.float16), self.zeros((out_rows, ffs), t.float16)
+            self.ok(self.lib.fnx_moe_gate_up_h16_mma(C.byref(W), w_stride, dj.data_ptr(), nj.data_ptr(), cap, dx.data_ptr(), one.data_ptr(), self.st()))
+            self.ok(self.lib.fnx_moe_gate_up_mma(C.byref(W), w_stride, dj.data_ptr(), nj.data_ptr(), cap, dx.data_ptr(), out.data_ptr(), self.st()))
+            self.ok(self.lib.fnx_swiglu_h16(out.data_ptr(), ffs, out_rows, two.data_ptr(), self.st()))
+            self.sync()
+            return one.cpu().numpy(), two.cpu().numpy()
         fn = self.lib.fnx_moe_down_mma if down else self.lib.fnx_moe_gate_up_mma
         self.ok(fn(C.byref(W), w_stride, dj.data_ptr(), nj.data_ptr(), cap, dx.data_ptr(), out.data_ptr(), self.st()))
         self.sync()

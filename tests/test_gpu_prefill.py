@@ -140,6 +140,29 @@ def test_moe_mma_wave_form_tile16_rows_of_512(dev, oracle, nrows, nexp, sizes):
         assert rel_l2(got, want) <= 1e-5, "f16 operands are the oracle's: only the summation order may differ"
 
 
+@pytest.mark.parametrize("tile16", [False, True])
+@pytest.mark.parametrize("ffs,ncols,nexp,sizes", [(512, 2048, 24, [64, 1, 17, 0, 16, 33, 48, 5, 64, 64, 2, 0, 31, 64, 49, 15] * 3), (128, 512, 3, [64, 1, 17, 16, 33, 48, 5]),
+                                                  (256, 1024, 2, [3]), (640, 2048, 2, [64, 9])])
+def test_moe_gate_up_h16_one_launch_equals_two(dev, ffs, ncols, nexp, sizes, tile16):
+    # h = silu(gate) * up straight from the matrix-core launch (block form over unit64, wave form over tile16): the bits of
+    # fnx_moe_gate_up_mma followed by fnx_swiglu_h16, whatever the mix of job sizes, with rows no job writes left alone
+    print(f"case moe_gate_up_h16 ffs={ffs} ncols={ncols} nexp={nexp} jobs={len(sizes)} tile16={tile16}", flush=True)
+    nrows = 2 * ffs
+    rng = np.random.default_rng(741 + ffs + len(sizes))
+    stride = nrows * ncols // 256 * 110
+    w = random_iq3s(rng, nexp * nrows * ncols // 256, dmax=2e-2)
+    rows = max(200, sum(sizes))
+    x16 = rng.standard_normal((rows, ncols)).astype(np.float16)
+    jobs, total = make_jobs(rng, nexp, rows, sizes)
+    one, two = dev.moe_mma(w, stride, nrows, ncols, jobs, x16, total + 3, packed=True, cap=len(jobs) + 5, tile16=tile16, h16=True)
+    assert np.all(np.isfinite(two.astype(np.float32)))
+    if tile16 or ncols > 512:
+        assert np.array_equal(one.view(np.uint16), two.view(np.uint16))
+    else:   # unit64 rows of up to 512 columns: the products alone come from the tile form, which adds in another order
+        assert rel_l2(one.astype(np.float32), two.astype(np.float32)) <= 1e-3
+    assert np.any(one[:total] != 0) and not np.any(one[total:])
+
+
 def test_moe_mma_weights_equal_the_oracles_f16(dev, oracle):
     # x = unit vectors: the product returns single weights, so every dequantised f16 value is checked bit for bit,
     # subnormal ones included (tiny d)
