@@ -1314,8 +1314,8 @@ static int mma_launch(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const 
     static const int wave16_gu = env_int("FNX_MMA_WAVE16_GU", 1, 0, 1);
     if (tile16 && wave16_gu && a.h16 && a.ffh % 16 == 0) {
         // wave form for stacked gate|up matrices: a wave a (gate tile, up tile) pair over the row's super-steps, one block a CU
-        const long upj = (a.ffh / 16 + W16_WAVES - 1) / W16_WAVES;
-        const int grid = (int) std::max(1l, std::min<long>((long) cu_count(), caps * upj));
+        const long upj = (a.ffh / 16 + 7) / 8;   // the finer of its two kinds of units
+        const int grid = (int) std::max(1l, std::min<long>(std::min(cu_count(), 64 * W16_PLAN), caps * upj));
         k_moe_mma_wave16_gu<<<grid, W16_THREADS, 0, (hipStream_t) st>>>(a);
         return launch_status(who);
     }

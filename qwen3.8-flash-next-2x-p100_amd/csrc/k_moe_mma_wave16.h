@@ -237,17 +237,23 @@ __global__ void __launch_bounds__(W16_THREADS) k_moe_mma_wave16(const MmaArgs a)
 // A job's activations are S tiles of 64 tokens x 512 columns here, and LDS holds one: a block takes units of (job, sixteen
 // gate tiles and the sixteen up tiles that go with them), a wave one such pair, and walks the S super-steps with the
 // pair's accumulators in registers - activation tile S in (two barriers), the gate tile's super-step, the up tile's -
-// and leaves h = silu(gate) * up as f16 (k_swiglu_h16's values). A unit is eight rounds of the down kernel's kind, so the
-// units are dealt like the block form's tasks: the jobs ranked by token tiles, the heaviest first, to and fro over the
-// blocks. The weights of the next tile's super-step are asked for a tile ahead.
-constexpr int W16_SORTJ = 1024, W16_GU_HELD = 1024;
+// and leaves h = silu(gate) * up as f16 (k_swiglu_h16's values). Such a unit is eight rounds of the down kernel's kind:
+// too coarse for runs by cost, and two of even the lightest on one block made the launch half as long again as its mean
+// block. So the jobs are ranked by token tiles, the units of those with two token tiles and more dealt heaviest first,
+// to and fro over the blocks, and the jobs of up to 16 tokens cut finer - eight pairs a unit, a wave a single tile, all S
+// tiles of the 16 tokens in LDS at once, the up tiles' sums handed to the gate tiles' waves through LDS - and spread so
+// that every block comes near the mean load. The weights of the next tile's super-step are asked for a tile ahead. Every
+// tile is accumulated in the block form's order (S, then the four steps, then a step's four operands): h has the bits
+// of k_moe_mma_block64's whatever a job's size.
+constexpr int W16_SORTJ = 1024, W16_GU_HELD = 1024, W16_PLAN = 4;   // (W16_PLAN: blocks a lane of the planning wave looks after)
 struct Wave16GuLds {
     uint2 tab[SGRID_WORDS];
     __attribute__((aligned(16))) uint8_t xt[MB_TOK64 * W16_XROW];
-    __attribute__((aligned(16))) uint8_t xs[16 * W16_XROW];   // a second tile for jobs of up to 16 tokens: super-step S + 1 comes in while S is multiplied
+    __attribute__((aligned(16))) uint8_t xs[8 * 64 * 16];      // the up tiles' sums of a light unit on their way to the gate tiles' waves
     uint8_t jn[2][W16_GU_HELD];
     int jw[W16_GU_HELD];
     unsigned short jorder[W16_SORTJ];   // the jobs, most token tiles first (the lower index first among equals)
+    int p_total[MB_TP + 1], p_sumk, p_s0, p_k;   // the jobs by token tiles; the plan where one wave made it: this block's share of the light units
 };
 __global__ void __launch_bounds__(W16_THREADS) k_moe_mma_wave16_gu(const MmaArgs a) {
     __shared__ Wave16GuLds L;
@@ -283,7 +289,8 @@ __global__ void __launch_bounds__(W16_THREADS) k_moe_mma_wave16_gu(const MmaArgs
         for (int j = tid + W16_THREADS; j < min(a.cap2, W16_GU_HELD); j += W16_THREADS) L.jn[1][j] = (uint8_t) max(0, min(FNX_PF_JOB, a.jobs2[j].n));
     }
     const int nj = min(a.cap, uniform(nj_raw)), nj2 = a.jobs2 ? min(a.cap2, uniform(nj2_raw)) : 0, njall = nj + nj2;
-    const int ffh = a.ffh, nsuper = a.ncols >> 9, ppj = ffh >> 4, upj = (ppj + W16_WAVES - 1) / W16_WAVES;   // pairs of tiles, units a job
+    const int ffh = a.ffh, nsuper = a.ncols >> 9, ppj = ffh >> 4;                      // pairs of tiles a job
+    const int upj = (ppj + W16_WAVES - 1) / W16_WAVES, upj_s = (ppj + 7) / 8;   // units a job: of sixteen pairs, of eight
     auto job_at = [&](int j) { return j < nj ? a.jobs + j : a.jobs2 + (j - nj); };
     auto n_of = [&](int j) {
         const int l = j < nj ? 0 : 1, k = j < nj ? j : j - nj;
@@ -313,31 +320,127 @@ __global__ void __launch_bounds__(W16_THREADS) k_moe_mma_wave16_gu(const MmaArgs
                 base[c] += __popcll(m);
             }
         }
+        // The plan. Jobs of two token tiles and more go as units of sixteen pairs (a wave a pair), dealt heaviest first, to
+        // and fro over the blocks. Jobs of up to 16 tokens (where a row's S <= 4 activation tiles of 16 tokens fit LDS
+        // together) go as units of eight pairs, a wave a single tile, and fill the blocks up to the mean load: block b
+        // takes k_b = (mean - its heavy units' cost) / (a light unit's cost) of them, rounded, in the order of the blocks
+        // from the last one down (the lightest first); what the rounding leaves over goes one a block in that order.
+        const int G = gridDim.x, ome = G - 1 - (int) blockIdx.x;
+        const bool split = nsuper <= 4;
+        const int nbj = total[4] + total[3] + total[2] + (split ? 0 : total[1]), nb = nbj * upj, ns = split ? total[1] * upj_s : 0;
+        // costs as measured for S = 4 (us: 20 + 5.5 a token tile the heavy unit, 13.5 the light one), in halves of a us
+        if (lane == 0) {
+#pragma unroll
+            for (int c = 0; c <= MB_TP; ++c) L.p_total[c] = total[c];
+        }
+        const int cs = 27 * nsuper;
+        if (nb > G) {   // (heavy units on one block or none: the same plan in closed form, below, by every wave)
+        auto big_cost = [&](int u) {
+            const int jo = u / upj, nt_ = jo < total[4] ? 4 : jo < total[4] + total[3] ? 3 : jo < total[4] + total[3] + total[2] ? 2 : 1;
+            return (40 + 11 * nt_) * nsuper;
+        };
+        auto load_of = [&](int bb) {   // block bb's heavy units
+            int l = 0;
+            for (int k = 0; k * G < nb; ++k) {
+                const int u = k * G + ((k & 1) ? G - 1 - bb : bb);
+                if (u < nb) l += big_cost(u);
+            }
+            return l;
+        };
+        // a lane looks after W16_PLAN blocks (a grid of up to 64 W16_PLAN), in the order from the last block down
+        const int o0 = lane * W16_PLAN;
+        int ld[W16_PLAN], mine_sum = 0;
+#pragma unroll
+        for (int i = 0; i < W16_PLAN; ++i) {
+            ld[i] = o0 + i < G ? load_of(G - 1 - (o0 + i)) : 0;
+            mine_sum += ld[i];
+        }
+#pragma unroll
+        for (int sh = 32; sh >= 1; sh >>= 1) mine_sum += __shfl_xor(mine_sum, sh);
+        const int mean = (int) (((long) mine_sum + (long) ns * cs + G - 1) / G);
+        int kk[W16_PLAN], kl = 0;
+#pragma unroll
+        for (int i = 0; i < W16_PLAN; ++i) {
+            kk[i] = o0 + i < G ? max(0, (mean - ld[i] + cs / 2) / cs) : 0;
+            kl += kk[i];
+        }
+        int incl = kl;
+#pragma unroll
+        for (int sh = 1; sh < 64; sh <<= 1) {
+            const int up = __shfl_up(incl, sh);
+            if (lane >= sh) incl += up;
+        }
+        const int sumk = __shfl(incl, 63);
+        if (o0 <= ome && ome < o0 + W16_PLAN) {
+            int s0 = incl - kl;
+#pragma unroll
+            for (int i = 0; i < W16_PLAN; ++i) {
+                if (o0 + i < ome) s0 += kk[i];
+                if (o0 + i == ome) L.p_k = kk[i];
+            }
+            L.p_s0 = s0;
+        }
+        if (lane == 0) L.p_sumk = sumk;
+        }
     }
-    __syncthreads();   // the codebook and the order
+    __syncthreads();   // the codebook, the order and the plan
     const uint32_t xt_at = (uint32_t) (size_t) (__attribute__((address_space(3))) uint8_t*) L.xt;
-    const uint32_t xs_at = (uint32_t) (size_t) (__attribute__((address_space(3))) uint8_t*) L.xs;
     const uint8_t* xlane = L.xt + r * W16_XROW + 256 * grp;
-    const uint8_t* xlane_s = L.xs + r * W16_XROW + 256 * grp;
-    const int units = njall * upj;
-    int yahead[MB_TP] = {0, 0, 0, 0}, ahead = -1;
-    for (int round = 0; round * (int) gridDim.x < units; ++round) {
-        const int pos = (round & 1) ? (int) gridDim.x - 1 - (int) blockIdx.x : (int) blockIdx.x, u = round * (int) gridDim.x + pos;
-        if (u >= units) continue;   // the same for the whole block
+    const int G = gridDim.x;
+    int tot[MB_TP + 1] = {0, 0, 0, 0, 0};
+    if (sorted) {
+#pragma unroll
+        for (int c = 0; c <= MB_TP; ++c) tot[c] = uniform(L.p_total[c]);
+    }
+    const bool split = nsuper <= 4;
+    const int nbj = sorted ? tot[4] + tot[3] + tot[2] + (split ? 0 : tot[1]) : njall, nb = nbj * upj, ns = sorted && split ? tot[1] * upj_s : 0;
+    int sumk, s0, kme;
+    if (nb <= G) {
+        // every heavy unit on a block of its own, block b's of the class its place in the order says: the blocks of a class
+        // take the same number of light units, and the blocks after b (they come first) are counted class by class
+        const int cs = 27 * nsuper, b1 = (int) blockIdx.x + 1;
+        const int hi4 = tot[4] * upj, hi3 = hi4 + tot[3] * upj, hi2 = hi3 + tot[2] * upj;   // where the classes end (class 1: nb)
+        const int c4 = 84 * nsuper, c3 = 73 * nsuper, c2 = 62 * nsuper, c1 = 51 * nsuper;      // (40 + 11 token tiles) S
+        const int mean = (hi4 * c4 + (hi3 - hi4) * c3 + (hi2 - hi3) * c2 + (nb - hi2) * c1 + ns * cs + G - 1) / G;
+        auto k_for = [&](int load) { return max(0, (mean - load + cs / 2) / cs); };
+        const int k4 = k_for(c4), k3 = k_for(c3), k2 = k_for(c2), k1 = k_for(c1), k0 = k_for(0);
+        auto after = [&](int lo, int hi) { return max(0, hi - max(lo, b1)); };   // blocks of [lo, hi) past this one
+        s0 = after(nb, G) * k0 + after(hi2, nb) * k1 + after(hi3, hi2) * k2 + after(hi4, hi3) * k3 + after(0, hi4) * k4;
+        kme = b1 > nb ? k0 : b1 > hi2 ? k1 : b1 > hi3 ? k2 : b1 > hi4 ? k3 : k4;
+        sumk = (G - nb) * k0 + (nb - hi2) * k1 + (hi2 - hi3) * k2 + (hi3 - hi4) * k3 + hi4 * k4;
+    } else {
+        sumk = sorted ? uniform(L.p_sumk) : 0, s0 = sorted ? uniform(L.p_s0) : 0, kme = sorted ? uniform(L.p_k) : 0;
+    }
+    // The oldest wave of a SIMD goes first and the block's waves drift apart between two barriers: every wave takes each
+    // priority in turn, a super-step each
+    auto turn = [&](int S) {
+        switch (((wave >> 2) + S) & 3) {
+            case 0: __builtin_amdgcn_s_setprio(0); break;
+            case 1: __builtin_amdgcn_s_setprio(1); break;
+            case 2: __builtin_amdgcn_s_setprio(2); break;
+            default: __builtin_amdgcn_s_setprio(3); break;
+        }
+    };
+    auto matrix_of = [&](int j, const fnx_bigjob* jb) {
+        const int e = j >= nj ? 0 : uniform(j < W16_GU_HELD ? L.jw[j] : jb->w);
+        return j >= nj ? a.w2 : a.ep ? uniform_ptr((const uint8_t*) a.ep[e]) : a.w + (size_t) e * a.stride;
+    };
+    // ---- the heavy units: sixteen pairs of tiles, a pair a wave
+    for (int round = 0; round * G < nb; ++round) {
+        const int u = round * G + ((round & 1) ? G - 1 - (int) blockIdx.x : (int) blockIdx.x);
+        if (u >= nb) continue;   // the same for the whole block
         const int jo = u / upj, q = u - jo * upj, j = sorted ? (int) uniform(L.jorder[jo]) : jo;
         const fnx_bigjob* jb = job_at(j);
         const int n = uniform(n_of(j));
         if (n < 1) continue;
-        const int nt = (n + 15) >> 4, e = j >= nj ? 0 : uniform(j < W16_GU_HELD ? L.jw[j] : jb->w);
-        const uint8_t* we = j >= nj ? a.w2 : a.ep ? uniform_ptr((const uint8_t*) a.ep[e]) : a.w + (size_t) e * a.stride;
+        const int nt = (n + 15) >> 4;
+        const uint8_t* we = matrix_of(j, jb);
         const int pr = q * W16_WAVES + wave;   // the wave's pair: gate rows 16 pr .., up rows ffh + 16 pr ..
         const bool mine = pr < ppj;
         const int grow = 16 * min(pr, ppj - 1) + r;
-        // the wave's tokens' rows (tokens wave, wave + 16, ..; past the job's last: that one again): asked for during the unit
-        // before, if this block knew then what its next unit would be
-        int y[MB_TP];
+        int y[MB_TP];   // the wave's tokens' rows: tokens wave, wave + 16, .. (past the job's last: that one again)
 #pragma unroll
-        for (int i = 0; i < MB_TP; ++i) y[i] = ahead == u ? yahead[i] : uniform(jb->y[min(wave + 16 * i, n - 1)]);
+        for (int i = 0; i < MB_TP; ++i) y[i] = uniform(jb->y[min(wave + 16 * i, n - 1)]);
         int orow[MB_TP];
 #pragma unroll
         for (int tt = 0; tt < MB_TP; ++tt) orow[tt] = mine && tt * 16 + r < n ? jb->out[tt * 16 + r] : -1;
@@ -345,58 +448,18 @@ __global__ void __launch_bounds__(W16_THREADS) k_moe_mma_wave16_gu(const MmaArgs
 #pragma unroll
         for (int tt = 0; tt < MB_TP; ++tt) accg[tt] = accu[tt] = v4f{0.f, 0.f, 0.f, 0.f};
         SuperFields f = tile16_load(we, grow, 0, nsuper);
-        auto next_unit = [&]() {   // the row numbers of the unit after this one
-            const int rn = round + 1, pn = (rn & 1) ? (int) gridDim.x - 1 - (int) blockIdx.x : (int) blockIdx.x, un = rn * (int) gridDim.x + pn;
-            if (un >= units) return;
-            const int jon = un / upj, jn = sorted ? (int) uniform(L.jorder[jon]) : jon, nn = uniform(n_of(jn));
-            const fnx_bigjob* jbn = job_at(jn);
+        for (int S = 0; S < nsuper; ++S) {
+            __syncthreads();   // the tile before has been read
 #pragma unroll
-            for (int i = 0; i < MB_TP; ++i) yahead[i] = uniform(jbn->y[max(0, min(wave + 16 * i, nn - 1))]);
-            ahead = un;
-        };
-        // The oldest wave of a SIMD goes first and the block's waves drift apart between two barriers: every wave takes each
-        // priority in turn, a super-step each
-        auto turn = [&](int S) {
-            switch (((wave >> 2) + S) & 3) {
-                case 0: __builtin_amdgcn_s_setprio(0); break;
-                case 1: __builtin_amdgcn_s_setprio(1); break;
-                case 2: __builtin_amdgcn_s_setprio(2); break;
-                default: __builtin_amdgcn_s_setprio(3); break;
-            }
-        };
-        if (nt == 1) {
-            // up to 16 tokens: two tiles in turn, the next super-step's asked for before this one is multiplied
-            __syncthreads();   // the unit before has been read
-            lds_load16(a.x + (size_t) y[0] * a.ldx, 16u * lane, xt_at + wave * W16_XROW);
-            next_unit();
+            for (int i = 0; i < MB_TP; ++i)   // a token's 512 columns a wave instruction, 16 bytes a lane
+                if (i < nt) lds_load16(a.x + (size_t) y[i] * a.ldx + 512 * S, 16u * lane, xt_at + (wave + 16 * i) * W16_XROW);
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             __syncthreads();
-            for (int S = 0; S < nsuper; ++S) {
-                turn(S);
-                if (S + 1 < nsuper) lds_load16(a.x + (size_t) y[0] * a.ldx + 512 * (S + 1), 16u * lane, ((S & 1) ? xt_at : xs_at) + wave * W16_XROW);
-                const uint8_t* xl = (S & 1) ? xlane_s : xlane;
-                const SuperFields fu = tile16_load(we, ffh + grow, S, nsuper);
-                if (mine) w16_super_step(L.tab, xl, f, 1, accg);
-                f = tile16_load(we, grow, min(S + 1, nsuper - 1), nsuper);
-                if (mine) w16_super_step(L.tab, xl, fu, 1, accu);
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-                __syncthreads();   // the other tile has landed, this one has been read
-            }
-        } else {
-            for (int S = 0; S < nsuper; ++S) {
-                __syncthreads();   // the tile before has been read
-#pragma unroll
-                for (int i = 0; i < MB_TP; ++i)   // a token's 512 columns a wave instruction, 16 bytes a lane
-                    if (i < nt) lds_load16(a.x + (size_t) y[i] * a.ldx + 512 * S, 16u * lane, xt_at + (wave + 16 * i) * W16_XROW);
-                if (S == 0) next_unit();
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-                __syncthreads();
-                turn(S);
-                const SuperFields fu = tile16_load(we, ffh + grow, S, nsuper);
-                if (mine) w16_super_step(L.tab, xlane, f, nt, accg);
-                f = tile16_load(we, grow, min(S + 1, nsuper - 1), nsuper);
-                if (mine) w16_super_step(L.tab, xlane, fu, nt, accu);
-            }
+            turn(S);
+            const SuperFields fu = tile16_load(we, ffh + grow, S, nsuper);
+            if (mine) w16_super_step(L.tab, xlane, f, nt, accg);
+            f = tile16_load(we, grow, min(S + 1, nsuper - 1), nsuper);
+            if (mine) w16_super_step(L.tab, xlane, fu, nt, accu);
         }
         // lane: token r of each tile, rows 4 grp .. 4 grp + 3 of the pair's tiles
 #pragma unroll
@@ -408,6 +471,54 @@ __global__ void __launch_bounds__(W16_THREADS) k_moe_mma_wave16_gu(const MmaArgs
                 hv.y = (uint32_t) float_to_half_bits(silu_f(gt.z) * up.z) | (uint32_t) float_to_half_bits(silu_f(gt.w) * up.w) << 16;
                 *reinterpret_cast<uint2*>(a.h16 + (size_t) orow[tt] * ffh + 16 * pr + 4 * grp) = hv;
             }
+    }
+    if (!sorted) return;
+    // ---- the light units: eight pairs of tiles, waves 0 .. 7 the gate tiles, 8 .. 15 the up tiles; the job's up to 16 tokens'
+    // S tiles all in LDS ([S][token]), so the waves do not meet until the up tiles' sums go over to the gate tiles' waves
+    const int ome = G - 1 - (int) blockIdx.x;
+    float4* ex = reinterpret_cast<float4*>(L.xs);
+    for (int t = 0;; ++t) {
+        const int idx = t < kme ? s0 + t : sumk + (t - kme) * G + ome;
+        if (t < kme ? idx >= min(ns, sumk) : idx >= ns) {
+            if (t < kme) {   // (this block's share was cut short: on to what is left over, if anything)
+                t = kme - 1;
+                continue;
+            }
+            break;
+        }
+        const int jo = idx / upj_s, q = idx - jo * upj_s, j = (int) uniform(L.jorder[nbj + jo]);
+        const fnx_bigjob* jb = job_at(j);
+        const int n = uniform(n_of(j));   // 1 .. 16
+        const uint8_t* we = matrix_of(j, jb);
+        const int pr = q * 8 + (wave & 7), up_wave = wave >> 3;
+        const bool mine = pr < ppj;
+        const int row = up_wave * ffh + 16 * min(pr, ppj - 1) + r;
+        const int y = uniform(jb->y[min(wave, n - 1)]);
+        const int orow = mine && !up_wave && r < n ? jb->out[r] : -1;
+        SuperFields f = tile16_load(we, row, 0, nsuper);
+        __syncthreads();   // the unit before has been read, its sums handed over
+        for (int S = 0; S < nsuper; ++S) lds_load16(a.x + (size_t) y * a.ldx + 512 * S, 16u * lane, xt_at + (16 * S + wave) * W16_XROW);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        v4f acc[MB_TP];
+#pragma unroll
+        for (int tt = 0; tt < MB_TP; ++tt) acc[tt] = v4f{0.f, 0.f, 0.f, 0.f};
+        for (int S = 0; S < nsuper; ++S) {
+            turn(S);
+            const SuperFields nf = tile16_load(we, row, min(S + 1, nsuper - 1), nsuper);
+            if (mine) w16_super_step(L.tab, xlane + S * 16 * W16_XROW, f, 1, acc);
+            f = nf;
+        }
+        if (up_wave) ex[(wave & 7) * 64 + lane] = make_float4(acc[0].x, acc[0].y, acc[0].z, acc[0].w);
+        __syncthreads();
+        if (orow >= 0) {
+            const float4 up = ex[wave * 64 + lane];
+            const v4f gt = acc[0];
+            uint2 hv;
+            hv.x = (uint32_t) float_to_half_bits(silu_f(gt.x) * up.x) | (uint32_t) float_to_half_bits(silu_f(gt.y) * up.y) << 16;
+            hv.y = (uint32_t) float_to_half_bits(silu_f(gt.z) * up.z) | (uint32_t) float_to_half_bits(silu_f(gt.w) * up.w) << 16;
+            *reinterpret_cast<uint2*>(a.h16 + (size_t) orow * ffh + 16 * pr + 4 * grp) = hv;
+        }
     }
 }
 

@@ -231,13 +231,13 @@ def test_prefill_layer_tile16_equals_unit64(dev, oracle, n, ff, nexp, topk, Cn):
     assert rel_l2(b["out"], want["out"]) <= REL_L2
 
 
-@pytest.mark.parametrize("tile16", [False, True])
-def test_prefill_layer_large_chunk_equals_small_chunks(dev, tile16):
+@pytest.mark.parametrize("tile16,Cn", [(False, 8192), (True, 8192), (True, 2048)])
+def test_prefill_layer_large_chunk_equals_small_chunks(dev, tile16, Cn):
     """A size-independent property at a size the oracle does not reach: a row's result does not depend on what else is in
     its chunk, so 8,192 rows in one call (more tasks than one pass of a block's task list holds, every kernel form's loop
     over list passes, a thousand jobs and more split over the wave form's blocks) must equal the same rows in 16 calls of
-    512, bit for bit, in either layout."""
-    n, ff, nexp, topk, Cn, small = 2048, 512, 64, 10, 8192, 512
+    512, bit for bit, in either layout. (2,048 rows: a few hundred jobs, ranked, their heavy units several to a block.)"""
+    n, ff, nexp, topk, small = 2048, 512, 64, 10, 512
     print(f"case prefill_layer large n={n} ff={ff} nexp={nexp} topk={topk} C={Cn} tile16={tile16}", flush=True)
     rng = np.random.default_rng(777)
     nb = lambda rows, cols: rows * cols // 256
