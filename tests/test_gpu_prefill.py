@@ -142,10 +142,11 @@ def test_moe_mma_wave_form_tile16_rows_of_512(dev, oracle, nrows, nexp, sizes):
 
 @pytest.mark.parametrize("tile16", [False, True])
 @pytest.mark.parametrize("ffs,ncols,nexp,sizes", [(512, 2048, 24, [64, 1, 17, 0, 16, 33, 48, 5, 64, 64, 2, 0, 31, 64, 49, 15] * 3), (128, 512, 3, [64, 1, 17, 16, 33, 48, 5]),
-                                                  (256, 1024, 2, [3]), (640, 2048, 2, [64, 9])])
+                                                  (256, 1024, 2, [3]), (640, 2048, 2, [64, 9]), (128, 2560, 2, [5, 64, 20, 16])])
 def test_moe_gate_up_h16_one_launch_equals_two(dev, ffs, ncols, nexp, sizes, tile16):
     # h = silu(gate) * up straight from the matrix-core launch (block form over unit64, wave form over tile16): the bits of
     # fnx_moe_gate_up_mma followed by fnx_swiglu_h16, whatever the mix of job sizes, with rows no job writes left alone
+    # (640: a job's last unit is short of pairs; 2560 columns: five activation tiles a row, so small jobs go as heavy units)
     print(f"case moe_gate_up_h16 ffs={ffs} ncols={ncols} nexp={nexp} jobs={len(sizes)} tile16={tile16}", flush=True)
     nrows = 2 * ffs
     rng = np.random.default_rng(741 + ffs + len(sizes))
