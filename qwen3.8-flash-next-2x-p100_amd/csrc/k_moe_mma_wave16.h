@@ -6,8 +6,8 @@
 // columns of f16, 64 KiB - is put in LDS once (by loads that write LDS directly, a token's row per wave instruction), and
 // after that a wave needs nothing from the others: it takes tiles of 16 rows, a lane decodes its four sub-blocks of its
 // row from one contiguous load of the tile16 layout, and the sixteen waves of a block (four a SIMD) meet only where the
-// block goes from one job to the next. The blocks split the (job, tile) items of all jobs by cost - a tile's decode and
-// its job's token tiles of multiplications - into contiguous runs.
+// block goes from one job to the next. The blocks split the (job, sixteen tiles) units of all jobs by cost - a tile's
+// decode and its job's token tiles of multiplications - into contiguous runs.
 // part[job.out[t]][row] = W[job.w][row] . h16[job.y[t]] as kernels.hpp:330 (moe_down_mma) defines it, with the weights as
 // f16 (d (1 + 2 s) g, each product rounded as k_moe_mma_block64 rounds it) and a row's sub-blocks accumulated in the order
 // of that kernel's steps.
@@ -19,10 +19,8 @@ namespace fnx {
 
 constexpr int W16_THREADS = 1024, W16_WAVES = 16, W16_COLS = 512;
 constexpr int W16_XROW = 2 * W16_COLS + 16;   // bytes of a token's f16 row in LDS (260 words: the 16 tokens of a 16-byte operand read fall on 64 different banks)
-#ifndef W16_DEC
-#define W16_DEC 3
-#endif
-constexpr int W16_MUL = 1;      // an item's cost: W16_DEC for its decode and W16_MUL a token tile of its job
+constexpr int W16_DEC = 3, W16_MUL = 1;   // an item's cost: W16_DEC for its decode and W16_MUL a token tile of its job (measured: 2.7 us a round of
+                                          // sixteen tiles with one token tile, 4.7 us with four)
 constexpr int W16_HELD = 2048;  // jobs of a list whose token counts and matrices are read into LDS at once, ahead of the split
 struct Wave16Lds {
     uint2 tab[SGRID_WORDS];
@@ -210,14 +208,12 @@ __global__ void __launch_bounds__(W16_THREADS) k_moe_mma_wave16(const MmaArgs a)
         for (; g < g1; g += W16_WAVES) {
             // The oldest wave of a SIMD goes first, so a block's waves drift apart and the first ones wait at the job's end
             // for the last: every wave takes every priority in turn, a tile each
-#ifndef W16_NOPRIO
             switch (((wave >> 2) + ((g - g0) >> 4)) & 3) {
                 case 0: __builtin_amdgcn_s_setprio(0); break;
                 case 1: __builtin_amdgcn_s_setprio(1); break;
                 case 2: __builtin_amdgcn_s_setprio(2); break;
                 default: __builtin_amdgcn_s_setprio(3); break;
             }
-#endif
             const SuperFields nf = tile16_load(we, 16 * (g + W16_WAVES < g1 ? g + W16_WAVES : g) + r, 0, 1);
             v4f acc[MB_TP];
 #pragma unroll
