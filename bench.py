@@ -172,7 +172,7 @@ def main():
     ap.add_argument("--shared-q8", action="store_true",
                     help="the shared expert as dense split Q8_0 (the reference's own form, three more launches a window) instead of IQ3_S")
     ap.add_argument("--no-extras", action="store_true", help="skip the legs beside the metric (verify: streaming calibration, config 1, the other weight kind; prefill: two chunks in flight)")
-    ap.add_argument("--raw-layout", action="store_true", help="leave the weights as raw ggml blocks (skip the load-time re-laying)")
+    ap.add_argument("--raw-layout", action="store_true", help="verify: leave the weights as raw ggml blocks (skip the load-time re-laying); prefill: unit64 only, no tile16 copies")
     ap.add_argument("--down-unit64", action="store_true", help="prefill: leave the down matrices in the unit64 layout (k_moe_mma_tile64) instead of tile16 (k_moe_mma_wave16)")
     ap.add_argument("--workload", choices=["verify", "prefill", "decoder", "head", "gemv"], default="verify",
                     help="verify: benchmark config 2 (the headline metric, the default); prefill: config 5, one MoE layer over prompt chunks of 512 "
@@ -807,7 +807,7 @@ def prefill_main(args):
     u_mean, j_mean = float(np.mean(active)), float(np.mean(jobs))
     # the two matrix-core launches on their own, with events on the launch stream (torch's current stream)
     reps = 20
-    fused_h = not args.raw_layout   # unit64 and tile16 matrices leave h = silu(gate) * up from the gate|up launch itself
+    fused_h = True   # unit64 and tile16 matrices (this workload has no other) leave h = silu(gate) * up from the gate|up launch itself
     evs = []
     for i in range(reps + 3):
         L = layers[i % nsets][0]
@@ -854,8 +854,8 @@ def prefill_main(args):
         cpu = {"value": CS / cdt, "unit": "tokens/s per layer", "cores": threads, "kind": "port",
                "sample": f"one pass of the oracle's prefill layer over the first {CS} rows of chunk 0 (f16 operands, f64 accumulation)",
                "parity_rel_l2": err}
-    gu_kernel = ("k_moe_mma_wave16_gu (routed gate|up over tile16, leaves h = silu(gate) * up; a wave a pair of gate and up tiles, a job's up to 64 tokens a decode)"
-                 if fused_h else "k_moe_mma (routed gate|up over raw blocks)")
+    gu_kernel = ("k_moe_mma_block64 (routed gate|up over unit64, leaves h = silu(gate) * up; a job's up to 64 tokens a decode)" if args.raw_layout else
+                 "k_moe_mma_wave16_gu (routed gate|up over tile16, leaves h = silu(gate) * up; a wave a pair of gate and up tiles, a job's up to 64 tokens a decode)")
     line = {
         "metric": "prefill MoE tokens/sec per layer (chunks of 512 rows) + grouped IQ3_S expert GEMM achieved GB/s and MFMA utilisation",
         "value": CH * steps / dt, "unit": "tokens/s per layer", "n_gpus": 1, "steps": steps, "warmup": warmup,
@@ -866,8 +866,8 @@ def prefill_main(args):
                    "step_flops": step_flops, "step_hbm_frac": step_bytes / (dt / steps) / HBM_PEAK, "step_mfma_frac": step_flops / (dt / steps) / MFMA_F16},
         "roofline": {"bound": "hbm", "kernel": gu_kernel, "achieved": gu_bytes / (gu_ms * 1e-3) / 1e9, "peak": HBM_PEAK / 1e9,
                      "unit": "GB/s", "frac": gu_bytes / (gu_ms * 1e-3) / HBM_PEAK,
-                     "traffic": PF_GATE_UP_TRAFFIC["bytes"] * gu_bytes / PF_GATE_UP_TRAFFIC["algorithmic_bytes"] if nsets == 4 else None,
-                     "traffic_source": PF_GATE_UP_TRAFFIC["source"] if nsets == 4 else None, "kernel_ms": gu_ms, "algorithmic_bytes": gu_bytes,
+                     "traffic": PF_GATE_UP_TRAFFIC["bytes"] * gu_bytes / PF_GATE_UP_TRAFFIC["algorithmic_bytes"] if nsets == 4 and not args.raw_layout else None,
+                     "traffic_source": PF_GATE_UP_TRAFFIC["source"] if nsets == 4 and not args.raw_layout else None, "kernel_ms": gu_ms, "algorithmic_bytes": gu_bytes,
                      "mfma_tflops": gu_flops / (gu_ms * 1e-3) / 1e12, "mfma_frac": gu_flops / (gu_ms * 1e-3) / MFMA_F16,
                      "down": {"kernel": "k_moe_mma_tile64 (unit64)" if args.down_unit64 or args.raw_layout else "k_moe_mma_wave16 (tile16)", "kernel_ms": dn_ms, "achieved": dn_bytes / (dn_ms * 1e-3) / 1e9, "mfma_tflops": dn_flops / (dn_ms * 1e-3) / 1e12},
                      "two_launches": {"gate_up_ms": gu2_ms, "swiglu_ms": sw_ms, "note": "fnx_moe_gate_up_mma (k_moe_mma_block64, f32 products written) and fnx_swiglu_h16"},
