@@ -101,6 +101,10 @@ inline void moe_gate_up_mma(const DW& A, size_t sa, const BigJob* jobs, const in
     ck(fnx_moe_gate_up_mma(&A, sa, jobs, njobs, njobs_cap, xh, gu, st));
 }
 inline void swiglu_h16(const float* gu, int ffs, int P, uint16_t* h16, void* st) { ck(fnx_swiglu_h16(gu, ffs, P, h16, st)); }
+// moe_gate_up_mma and swiglu_h16 as one launch that writes h only (no counterpart of its own in kernels.hpp: lines 328 + 329)
+inline void moe_gate_up_h16_mma(const DW& A, size_t sa, const BigJob* jobs, const int* njobs, int njobs_cap, const uint16_t* xh, uint16_t* h16, void* st) {
+    ck(fnx_moe_gate_up_h16_mma(&A, sa, jobs, njobs, njobs_cap, xh, h16, st));
+}
 inline void moe_down_mma(const DW& A, size_t sa, const BigJob* jobs, const int* njobs, int njobs_cap, const uint16_t* h16, float* part, void* st) {
     ck(fnx_moe_down_mma(&A, sa, jobs, njobs, njobs_cap, h16, part, st));
 }
