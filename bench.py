@@ -68,7 +68,12 @@ def stream_calibration(dev, torch, np):
     gate_up, down = 152064 * UNIT, 75776 * UNIT   # about 148.5 matrices of 901,120 and of 450,560 bytes
     return {"plain_16B_loads_1GiB": rate(1, 512, 512, whole), "nontemporal_16B_loads_1GiB": rate(5, 512, 512, whole),
             "unit64_plane_loads_1GiB": rate(6, 512, 512, whole),
-            "unit64_plane_loads_one_launch_134MB": rate(9, 256, 1024, gate_up), "unit64_plane_loads_one_launch_67MB": rate(9, 256, 1024, down)}
+            "unit64_plane_loads_one_launch_134MB": rate(9, 256, 1024, gate_up), "unit64_plane_loads_one_launch_67MB": rate(9, 256, 1024, down),
+            # four units as one lane-interleaved record (six loads a lane of 16, 16, 16, 4, 4, 8 bytes), plain and nontemporal
+            "quad_records_1GiB": rate(14, 512, 512, whole), "quad_records_nontemporal_1GiB": rate(15, 512, 512, whole),
+            "quad_records_one_launch_134MB": rate(14, 256, 1024, gate_up), "quad_records_nontemporal_one_launch_134MB": rate(15, 256, 1024, gate_up),
+            "quad_records_nontemporal_one_launch_67MB": rate(15, 256, 1024, down),
+            "nontemporal_16B_loads_one_launch_134MB": rate(5, 256, 1024, gate_up)}
 
 
 def gemv_measure(dev, torch, np, steps):
@@ -182,14 +187,10 @@ def main():
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
         sys.exit(2)
-    if args.workload == "prefill":
-        return prefill_main(args)
-    if args.workload == "decoder":
-        return decoder_main(args)
-    if args.workload == "head":
-        return head_main(args)
-    if args.workload == "gemv":
-        return gemv_main(args)
+    other = {"prefill": prefill_main, "decoder": decoder_main, "head": head_main, "gemv": gemv_main}.get(args.workload)
+    if other:
+        print(json.dumps(other(args)))
+        return
 
     import numpy as np
     import torch
@@ -261,13 +262,25 @@ def main():
         x = xs[i % NX]
         dev.ok(lib.fnx_moe_verify_layer(C.byref(L), x.data_ptr(), T, outs[i % NX].data_ptr(), C.byref(ws), st))
 
+    PREROLL_MS = 50.0
+    preroll = {"ms": 0.0, "steps": 0}
+
     def timed_steps(sets=None):
+        """W warm-up steps, then untimed steps until PREROLL_MS have passed whatever W is (so that a short timed region is
+        not measured on clocks that have just come up from idle), then exactly K timed steps between two synchronisations"""
         for i in range(args.warmup):
             step(i, sets)
         torch.cuda.synchronize()
+        p0, n_pre = time.perf_counter(), 0
+        while (time.perf_counter() - p0) * 1e3 < PREROLL_MS:
+            for i in range(64):
+                step(args.warmup + n_pre + i, sets)
+            n_pre += 64
+            torch.cuda.synchronize()
+        preroll["ms"], preroll["steps"] = (time.perf_counter() - p0) * 1e3, n_pre
         t0 = time.perf_counter()
         for i in range(args.steps):
-            step(args.warmup + i, sets)
+            step(args.warmup + n_pre + i, sets)
         torch.cuda.synchronize()
         return time.perf_counter() - t0
 
@@ -281,6 +294,7 @@ def main():
     # ---- whole steps
     dt = timed_steps()
     ms_per_step = dt / args.steps * 1e3
+    headline_preroll = dict(preroll)
 
     # ---- distinct experts per step (for the algorithmic bytes), from the routing the steps produced
     njobs = []
@@ -370,11 +384,39 @@ def main():
                "sample": f"{n_cpu} layer-steps of the same workload (weight set 0, T=16) on the oracle (q8_1 x IQ3_S restated from the reference, not ggml's Q8_K kernel)",
                "parity_rel_l2": err, "routing_identical": same}
 
+    # ---- the other workloads in short (their own lines: --workload head / decoder / prefill): a few steps each, CPU legs off
+    others = None
+    if not args.no_extras and fused:
+        import copy
+        del layers, xs, outs
+        torch.cuda.empty_cache()
+        short = copy.copy(args)
+        short.cpu_seconds, short.no_extras = 0.0, True
+        short.steps, short.warmup = 200, 20
+        hd = head_main(short)
+        short.steps, short.warmup = 30, 5
+        dc = decoder_main(short)
+        torch.cuda.empty_cache()
+        short.steps, short.warmup, short.layers = 76, 8, 4
+        pf = prefill_main(short)
+        others = {
+            "head": {"workload": hd["config"]["workload"], "us_per_round": hd["ms_per_step"] * 1e3, "argmax_us": hd["config"]["argmax_us"],
+                     "lookup_us": hd["config"]["lookup_us"], "accept_us": hd["config"]["accept_us"], "identical_to_oracle": hd["config"]["identical_to_oracle"]},
+            "decoder": {"workload": dc["config"]["workload"], "ms_per_step": dc["ms_per_step"], "steps": dc["steps"], "step_hbm_frac": dc["config"]["step_hbm_frac"],
+                        "attention_TBps": dc["config"]["attention_GBps"] / 1e3, "head_TBps": dc["config"]["head_GBps"] / 1e3,
+                        "decode_round_ms_graph_replay": dc["config"]["decode_round"]["ms_graph_replay"]},
+            "prefill": {"workload": pf["config"]["workload"], "chunk_us": pf["ms_per_step"] * 1e3, "steps": pf["steps"], "tokens_per_s": pf["value"],
+                        "piecewise_bound_frac": pf["roofline"]["piecewise_bound"]["chunk_frac"], "gate_up_us": pf["roofline"]["kernel_ms"] * 1e3,
+                        "gate_up_mfma_frac": pf["roofline"]["mfma_frac"], "gate_up_hbm_frac": pf["roofline"]["frac"],
+                        "down_us": pf["roofline"]["down"]["kernel_ms"] * 1e3,
+                        "gate_up_traffic_ratio": (pf["roofline"]["traffic"] / pf["roofline"]["algorithmic_bytes"]) if pf["roofline"]["traffic"] else None},
+        }
+
     line = {
         "metric": "MoE verify steps/sec at T=16 + IQ3_S expert GEMV achieved HBM GB/s (% peak)",
         "value": args.steps / dt,
         "unit": "layer-steps/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "preroll_ms": headline_preroll["ms"], "preroll_steps": headline_preroll["steps"],
         "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int8 x IQ3_S (i32 dot, f32 accumulate)",
@@ -386,7 +428,7 @@ def main():
                    "weight_layout": "raw ggml blocks" if args.raw_layout else "unit64 (re-laid once at load, same bytes)", "weight_sets": args.layers, "distinct_experts_per_step": u_mean, "step_algorithmic_bytes": step_bytes,
                    "step_hbm_frac": step_bytes / (ms_per_step * 1e-3) / HBM_PEAK,
                    "ms_per_step_other_weights": None if other_ms is None else {("bytes" if args.weights == "gaussian" else "gaussian"): other_ms},
-                   "gemv": gemv},
+                   "gemv": gemv, "others": others},
         "roofline": {"bound": "hbm", "kernel": kernel_name, "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK, "traffic": traffic, "traffic_source": GATE_UP_TRAFFIC["source"] if traffic else None,
                      "kernel_ms": k_ms, "algorithmic_bytes": k_bytes,
@@ -422,7 +464,7 @@ def gemv_main(args):
                          "unit": "GB/s", "frac": many["T16"]["hbm_frac"], "traffic": None,
                          "note": "one matrix a launch (3.6 MB) is bound by the launch: " + f"{lone['T16']['us_per_launch']:.1f} us at T = 16"},
             "cpu_baseline": None}
-    print(json.dumps(line))
+    return line
 
 
 def head_main(args):
@@ -497,12 +539,12 @@ def head_main(args):
         list(dout.cpu().numpy()[:int(dn.item())]) == list(drafts) and int(dm.item()) == match
     c0 = time.perf_counter()
     reps = 0
-    while time.perf_counter() - c0 < min(args.cpu_seconds, 5.0) or reps < 2:
+    while args.cpu_seconds > 0 and (time.perf_counter() - c0 < min(args.cpu_seconds, 5.0) or reps < 2):
         oracle.argmax(logits[0].cpu().numpy()) if reps == 0 else None
         oracle.lookup_drafts(ctx, 15, d1)
         oracle.accept_greedy(rows, o[:len(rows)])
         reps += 1
-    cpu_us = (time.perf_counter() - c0) / reps * 1e6
+    cpu_us = (time.perf_counter() - c0) / max(reps, 1) * 1e6
     arg_bytes = R * V * 4
     line = {"metric": "verify head: argmax + acceptance + prompt lookup per round (config 3)", "value": 1e6 / us_all, "unit": "rounds/s", "n_gpus": 1,
             "steps": n, "warmup": 20, "ms_per_step": us_all / 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32 compare / int32",
@@ -513,9 +555,9 @@ def head_main(args):
             "roofline": {"bound": "hbm", "kernel": "k_argmax", "achieved": arg_bytes / (us_arg * 1e-6) / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                          "frac": arg_bytes / (us_arg * 1e-6) / HBM_PEAK, "traffic": None, "algorithmic_bytes": arg_bytes,
                          "note": "two launches of about 4 us fixed cost each; the scan itself is 1.2 us at peak"},
-            "cpu_baseline": {"value": 1e6 / cpu_us, "unit": "rounds/s", "cores": 1, "kind": "port",
-                             "sample": f"{reps} rounds of lookup + acceptance on the oracle (the argmax scan once)"}}
-    print(json.dumps(line))
+            "cpu_baseline": None if not reps else {"value": 1e6 / cpu_us, "unit": "rounds/s", "cores": 1, "kind": "port",
+                                                   "sample": f"{reps} rounds of lookup + acceptance on the oracle (the argmax scan once)"}}
+    return line
 
 
 def decoder_main(args):
@@ -693,7 +735,7 @@ def decoder_main(args):
                          "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": head_bytes / (head_ms * 1e-3) / HBM_PEAK, "traffic": None, "kernel_ms": head_ms,
                          "algorithmic_bytes": head_bytes},
             "cpu_baseline": cpu}
-    print(json.dumps(line))
+    return line
 
 
 def prefill_main(args):
@@ -880,7 +922,7 @@ def prefill_main(args):
         # not the metric: two streams with a workspace each, chunks dealt to them in turn
         "two_chunks_in_flight": {"ms_per_chunk": dt2 / steps * 1e3, "tokens_per_s": CH * steps / dt2} if dt2 else None,
     }
-    print(json.dumps(line))
+    return line
 
 
 if __name__ == "__main__":

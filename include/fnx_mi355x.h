@@ -225,7 +225,8 @@ int fnx_layer_profile_read(float* ms3);
  * with the 1 KiB chunks dealt round-robin to the waves; 4: 8-byte loads, 8 in flight; 5: as 1 with nontemporal loads;
  * 6: the unit64 planes as the expert kernels load them (five loads a unit and lane, a group of four units in flight), every
  * wave one contiguous range; 9: the groups dealt round-robin to the grid's waves; 10: every block one contiguous range,
- * its waves taking the groups in turn; 11 / 12 / 13: as 6 / 9 / 10 with nontemporal loads; 1000 s + K (s = 1 .. 8, K = 1 .. 64
+ * its waves taking the groups in turn; 11 / 12 / 13: as 6 / 9 / 10 with nontemporal loads; 14 / 15: four units as one lane-interleaved
+ * record of 3,520 bytes (six loads a lane of 16, 16, 16, 4, 4 and 8 bytes), the records dealt round-robin to the grid's waves, plain / nontemporal; 1000 s + K (s = 1 .. 8, K = 1 .. 64
  * dividing 64 s): the buffer as matrices of 256 s units (s = 4: a gate|up matrix of the benchmark's shape, 2: a down matrix)
  * read in a shuffled order, a wave staying with a matrix for K trips of four units. sink: one device word (never written in
  * practice; it keeps the loads alive). */

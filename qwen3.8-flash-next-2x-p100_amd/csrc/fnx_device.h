@@ -98,7 +98,13 @@ __device__ __forceinline__ uint32_t load_u16(const uint8_t* p) {
 // of such loads from another, does not wait for every one of them before each LDS read: the kernel counts them itself
 // (vmcnt) where it needs their data.
 __device__ __forceinline__ void lds_load16(const void* base, uint32_t lane_offset, uint32_t lds_at) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_at), "v"(lane_offset), "s"(base) : "memory");
+    // M0 is put back before the statement ends: the compiler keeps values of its own there (it does not accept M0 in a
+    // clobber list); the load has taken its LDS address by then
+    uint32_t m0_kept;
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3\n\ts_mov_b32 m0, %0"
+                 : "=&s"(m0_kept)
+                 : "s"(lds_at), "v"(lane_offset), "s"(base)
+                 : "memory");
 }
 
 }  // namespace fnx

@@ -1127,6 +1127,8 @@ static int moe_layer_checked(const fnx_moe_layer* L, const float* x, int T, floa
     if (!out) return fail("moe_verify_layer: null argument");
     if (live && !layer_fused_ok(L, T)) return fail("moe_verify_layer: a device-side row count needs the three-launch window");
     if (layer_fused_ok(L, T)) return layer_fused(L, x, T, out, ws, st, live);
+    // operator by operator the pairs' q8_1 rows of h go through the library's pair buffer, rows of ff / 32 blocks
+    if (ff <= 0 || ff % 32 || ff > HQ_MAX_FF) return fail("moe_verify_layer: expert width does not fit the pair buffer");
     hipStream_t s = (hipStream_t) st;
     BufferScope pair_buffer(g_pair_order, st);   // operator by operator the pairs' q8_1 rows go through the library's buffer
     if (fnx_quantize_q8_1(x, ws->xq, n, T, st)) return 1;
@@ -1170,6 +1172,7 @@ constexpr size_t NA_OFF_LOGITS = na_up(NA_XQ), NA_OFF_TOPI = NA_OFF_LOGITS + na_
 static_assert(NA_BYTES <= FNX_MOE_STATIC_WS_BYTES, "the header states the array's size");
 static __device__ __align__(256) unsigned char scratch[FNX_MOE_STATIC_WS_BYTES];
 static unsigned char* g_scratch_ptr[64] = {};   // per device: the array's address there
+static std::mutex g_scratch_mutex;
 int fnx_moe_verify_layer_static(const fnx_moe_layer* L, const float* x, int T, float* out, void* st) {
     if (!L || !x || !out) return fail("moe_verify_layer_static: null argument");
     if (T < 1 || T > FNX_MAXT) return fail("moe_verify_layer_static: T out of range");
@@ -1178,11 +1181,14 @@ int fnx_moe_verify_layer_static(const fnx_moe_layer* L, const float* x, int T, f
                     "ff 256 / 512 / 1024, up to 1024 experts, up to 16 picks a row, up to 160 pairs a window)");
     int dev = -1;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return fail("moe_verify_layer_static: no current device");
-    if (!g_scratch_ptr[dev]) {
-        unsigned char* p = nullptr;
-        const hipError_t e = hipGetSymbolAddress((void**) &p, HIP_SYMBOL(scratch));
-        if (e != hipSuccess || !p) return fail(std::string("moe_verify_layer_static: hipGetSymbolAddress: ") + hipGetErrorString(e));
-        g_scratch_ptr[dev] = p;
+    {   // once per device, with that device current; threads that arrive together take turns (a failed query is asked again)
+        std::lock_guard<std::mutex> g(g_scratch_mutex);
+        if (!g_scratch_ptr[dev]) {
+            unsigned char* p = nullptr;
+            const hipError_t e = hipGetSymbolAddress((void**) &p, HIP_SYMBOL(scratch));
+            if (e != hipSuccess || !p) return fail(std::string("moe_verify_layer_static: hipGetSymbolAddress: ") + hipGetErrorString(e));
+            g_scratch_ptr[dev] = p;
+        }
     }
     unsigned char* w = g_scratch_ptr[dev];
     // nothing in the workspace has to start at zero: every launch writes what it reads, and the job count is stored, not added to
@@ -1221,13 +1227,15 @@ int fnx_stream_read(const void* p, size_t bytes, int variant, int blocks, int th
         case 11: k_stream_read_units<0, true><<<blocks, threads, 0, s>>>(b, bytes / UNIT_BYTES, k); break;
         case 12: k_stream_read_units<1, true><<<blocks, threads, 0, s>>>(b, bytes / UNIT_BYTES, k); break;
         case 13: k_stream_read_units<2, true><<<blocks, threads, 0, s>>>(b, bytes / UNIT_BYTES, k); break;
+        case 14: k_stream_read_quads<false><<<blocks, threads, 0, s>>>(b, bytes / QUAD_BYTES, k); break;
+        case 15: k_stream_read_quads<true><<<blocks, threads, 0, s>>>(b, bytes / QUAD_BYTES, k); break;
         default:
             // 1000 s + K: segments of 256 s units (s = 4: a gate|up matrix, 2: a down matrix), K trips a wave and segment
             if (variant >= 1000 && variant < 9000 && variant % 1000 >= 1 && variant % 1000 <= 64 && (256 * (variant / 1000) / 4) % (variant % 1000) == 0) {
                 k_stream_read_segments<<<blocks, threads, 0, s>>>(b, bytes / UNIT_BYTES, 256u * (variant / 1000), (uint32_t) (variant % 1000), k);
                 break;
             }
-            return fail("stream_read: variants 0..13, or 1000 s + K");
+            return fail("stream_read: variants 0..15, or 1000 s + K");
     }
     return launch_status("stream_read");
 }
@@ -1509,7 +1517,9 @@ static int q8s_one(const fnx_q8s* W, const void* yq, float* out, int out_stride,
 static int attn_launch(const float* qg, const uint16_t* kc, const uint16_t* vc, float* out, uint8_t* outq, int nq, int nkv, const int* pos0, int T,
                        int max_ctx, float* scratch, void* st, const int* gate = nullptr, const int* live = nullptr, unsigned* err = nullptr) {
     if (!qg || !kc || !vc || (!out && !outq) || !pos0 || !scratch) return fail("attn: null argument");
-    if (nq < 1 || nkv < 1 || nq % nkv || nq / nkv > AT_MAXQ || T < 1 || T > FNX_MAXT || max_ctx < 1) return fail("attn: bad shape");
+    if (nq < 1 || nkv < 1 || nq % nkv || nq / nkv > AT_MAXQ || T < 1 || T > FNX_MAXT) return fail("attn: bad shape");
+    // the V cache lies in blocks of AT_VB positions and the kernel fetches whole blocks: a capacity that ends inside a block would be read past its end
+    if (max_ctx < AT_VB || max_ctx % AT_VB) return fail("attn: the cache holds a multiple of 8 positions");
     if (attn_splits(max_ctx) > AT_MAXSPLIT) return fail("attn: the cache is larger than the split table");
     if (((unsigned long long) max_ctx + 3) * nkv * (AT_HD * 2) >= (1ull << 32)) return fail("attn: a cache of 4 GiB or more (the kernel's byte offsets are 32 bits)");
     // the grid covers the cache's capacity (the position is on the device): splits past the context write empty parts

@@ -122,6 +122,55 @@ __global__ void __launch_bounds__(1024) k_stream_read_units(const uint8_t* __res
     if (acc == 0x9E3779B9u) sink[0] = acc;
 }
 
+// Four units a lane-interleaved record of 3,520 bytes (the planes of four units side by side a lane): six loads a lane of
+// 16, 16, 16, 4, 4 and 8 bytes instead of the twenty of four unit64 units. Record q goes to wave q mod the grid's waves,
+// one record in flight while one is summed. NT: nontemporal loads.
+constexpr int QUAD_BYTES = 4 * UNIT_BYTES, QUAD_B_AT = 2048, QUAD_C_AT = 3072, QUAD_SC_AT = 3328, QUAD_D_AT = 3456;
+struct QuadRaw {
+    v4u a0, a1, b;
+    uint32_t c, sc;
+    v2u d;
+};
+template <bool NT>
+__device__ __forceinline__ QuadRaw stream_load_quad(gbytes q, uint32_t lane) {
+    uint32_t oa = 32 * lane, ob = QUAD_B_AT + 16 * lane, oc = QUAD_C_AT + 4 * lane, os = QUAD_SC_AT + 4 * (lane >> 1), od = QUAD_D_AT + 8 * (lane >> 3);
+    asm volatile("" : "+v"(oa), "+v"(ob), "+v"(oc), "+v"(os), "+v"(od));
+    typedef __attribute__((address_space(1))) const uint32_t g32;
+    QuadRaw r;
+    if constexpr (NT) {
+        r.a0 = __builtin_nontemporal_load((g128*) (q + oa));
+        r.a1 = __builtin_nontemporal_load((g128*) (q + oa + 16));
+        r.b = __builtin_nontemporal_load((g128*) (q + ob));
+        r.c = __builtin_nontemporal_load((g32*) (q + oc));
+        r.sc = __builtin_nontemporal_load((g32*) (q + os));
+        r.d = __builtin_nontemporal_load((g64v*) (q + od));
+    } else {
+        r.a0 = *(g128*) (q + oa);
+        r.a1 = *(g128*) (q + oa + 16);
+        r.b = *(g128*) (q + ob);
+        r.c = *(g32*) (q + oc);
+        r.sc = *(g32*) (q + os);
+        r.d = *(g64v*) (q + od);
+    }
+    return r;
+}
+template <bool NT>
+__global__ void __launch_bounds__(1024) k_stream_read_quads(const uint8_t* __restrict__ p, size_t quads, uint32_t* __restrict__ sink) {
+    const uint32_t wpb = blockDim.x >> 6, wave = (uint32_t) uniform((int) (threadIdx.x >> 6)), lane = threadIdx.x & 63;
+    const uint32_t gw = blockIdx.x * wpb + wave, nw = gridDim.x * wpb;
+    if (gw >= quads) return;
+    auto quad_at = [&](size_t qi) { return as_global(uniform_ptr(p + (qi < quads ? qi : quads - 1) * QUAD_BYTES)); };
+    uint32_t acc = 0;
+    QuadRaw cur = stream_load_quad<NT>(quad_at(gw), lane);
+    for (size_t q = gw; q < quads; q += nw) {
+        const QuadRaw nxt = stream_load_quad<NT>(quad_at(q + nw < quads ? q + nw : q), lane);
+        acc ^= cur.a0.x ^ cur.a0.y ^ cur.a0.z ^ cur.a0.w ^ cur.a1.x ^ cur.a1.y ^ cur.a1.z ^ cur.a1.w ^ cur.b.x ^ cur.b.y ^ cur.b.z ^ cur.b.w ^ cur.c ^ cur.sc ^
+               cur.d.x ^ cur.d.y;
+        cur = nxt;
+    }
+    if (acc == 0x9E3779B9u) sink[0] = acc;
+}
+
 // the window kernels' case: segments of `seg_units` units (an expert's matrix) scattered over the buffer, walked in a
 // fixed shuffled order; wave gw keeps to a segment for K trips of one group, so the grid reads waves * K * 4 / seg_units
 // segments at a time, each as one front that moves through the segment

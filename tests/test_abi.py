@@ -53,6 +53,23 @@ def test_bad_arguments_are_refused_with_a_message():
     assert lib.fnx_mmvq(C.byref(bad), 0, buf, None, 1, buf, buf, 16, None) != 0
     assert lib.fnx_route(buf, 8, 1, 2000, 10, buf, buf, buf, buf, buf, None) != 0
     assert lib.fnx_argmax(buf, 0, 1, 0, buf, buf, buf, buf, None) != 0
+    # a cache whose capacity ends inside a block of eight positions would be read past its end by the attention's V fetches
+    assert lib.fnx_attn(buf, buf, buf, buf, 16, 2, buf, 1, 100, buf, None) != 0 and b"multiple of 8" in lib.fnx_last_error()
+    assert lib.fnx_attn(buf, buf, buf, buf, 16, 2, buf, 1, 4, buf, None) != 0 and b"multiple of 8" in lib.fnx_last_error()
+
+
+def test_a_layer_wider_than_the_pair_buffer_is_refused():
+    """operator by operator (raw ggml blocks) the pairs' q8_1 rows of h go through the library's pair buffer of rows of at most
+    1024 values: a wider expert is refused before anything is launched"""
+    pkg = fnx_gpu.package()
+    lib = pkg.lib()
+    buf = np.zeros(64, dtype=np.float32).ctypes.data
+    n, ff, nexp, topk = 2048, 2048, 32, 10
+    gu, down = pkg.dw(buf, n, 2 * ff), pkg.dw(buf, ff, n)
+    L = pkg.MoeLayer(n, ff, nexp, topk, buf, 0, gu, 0, down, 0, gu, down)
+    ws = pkg.MoeWs(*([buf] * len(pkg.MoeWs._fields_)))
+    assert lib.fnx_moe_verify_layer(C.byref(L), buf, 16, buf, C.byref(ws), None) != 0
+    assert b"pair buffer" in lib.fnx_last_error()
 
 
 def test_host_lookup_and_accept_match_the_oracle(oracle):

@@ -130,29 +130,59 @@ def test_config4_window_at_the_end_of_the_cache(dev, oracle):
     rows_close(db["logits"], da["logits"], "draft logits", parted)
 
 
-def test_config5_chunk_of_512_rows(dev, oracle):
-    n, ff, nexp, topk, Cn = 2048, 512, 512, 10, 512
-    print(f"case config 5 full shape n={n} ff={ff} nexp={nexp} topk={topk} C={Cn}", flush=True)
-    rng = np.random.default_rng(505)
+def config5_inputs(rng, n, ff, nexp, Cn, zipf):
     nb = lambda rows, cols: rows * cols // 256
     gu = random_iq3s(rng, nexp * nb(2 * ff, n), dmax=1e-3)   # d small enough that h = silu(g) u stays inside f16's range
     down = random_iq3s(rng, nexp * nb(n, ff), dmax=1e-3)
     sh_gu, sh_down = random_iq3s(rng, nb(2 * ff, n), dmax=1e-3), random_iq3s(rng, nb(n, ff), dmax=1e-3)
-    pop = 1.0 / np.arange(1, nexp + 1) ** 1.1
     router = (rng.standard_normal((nexp + 1, n)) * 0.02).astype(np.float32)
-    router[:nexp, 0] = np.log(pop / pop.sum())[rng.permutation(nexp)]
-    router[nexp, 0] = 0
     x = rng.standard_normal((Cn, n)).astype(np.float32)
-    x[:, 0] = 1.0
+    if zipf:
+        pop = 1.0 / np.arange(1, nexp + 1) ** 1.1
+        router[:nexp, 0] = np.log(pop / pop.sum())[rng.permutation(nexp)]
+        router[nexp, 0] = 0
+        x[:, 0] = 1.0
+    return router, gu, down, sh_gu, sh_down, x
+
+
+# unit64: every matrix in the verify path's layout (k_moe_mma_block64 / k_moe_mma_tile64); tile16: the prompt path's own
+# copies of gate|up and down, the layout the benchmark's prefill workload times (k_moe_mma_wave16_gu, k_moe_mma_wave16)
+@pytest.mark.parametrize("layout", ["unit64", "tile16"])
+def test_config5_chunk_of_512_rows(dev, oracle, layout):
+    n, ff, nexp, topk, Cn = 2048, 512, 512, 10, 512
+    print(f"case config 5 full shape n={n} ff={ff} nexp={nexp} topk={topk} C={Cn} layout={layout}", flush=True)
+    router, gu, down, sh_gu, sh_down, x = config5_inputs(np.random.default_rng(505), n, ff, nexp, Cn, zipf=True)
     want = oracle.moe_prefill_layer(n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, x, threads=16)
     cnt = np.bincount(want["topi"].reshape(-1), minlength=nexp)
     print(f"experts in use {np.count_nonzero(cnt)}, the busiest takes {cnt.max()} of {Cn} rows, jobs {want['njobs']}", flush=True)
     assert cnt.max() >= Cn // 2 and np.count_nonzero(cnt) >= 64, "the popularity is skewed and still wide"
-    r = fnx_gpu.PfLayerDev(dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, Cn, packed=True).run(x)
+    r = fnx_gpu.PfLayerDev(dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, Cn, packed=True, tile16=layout == "tile16").run(x)
     assert np.array_equal(r["logits"].view(np.uint32), want["logits"].view(np.uint32))
     assert np.array_equal(r["topi"], want["topi"])
     assert int(r["njobs"][0]) == want["njobs"]
     assert np.all(np.isfinite(want["out"]))
     err = rel_l2(r["out"], want["out"])
     print("config 5 chunk rel l2", err, flush=True)
+    assert err <= REL_L2
+    if layout == "tile16":   # h as the wave kernels leave it = h of the unit64 block form, bit for bit (one accumulation order per tile)
+        r64 = fnx_gpu.PfLayerDev(dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, Cn, packed=True).run(x)
+        assert np.array_equal(r["h16"].view(np.uint16), r64["h16"].view(np.uint16))
+
+
+def test_config5_uniform_routing_tile16(dev, oracle):
+    """the same chunk without the popularity skew: every expert takes about ten rows, so no job has two token tiles and the
+    wave kernels' plan spreads light units only (the Zipf chunk above has blocks with heavy units)"""
+    n, ff, nexp, topk, Cn = 2048, 512, 512, 10, 512
+    print(f"case config 5 uniform routing n={n} ff={ff} nexp={nexp} topk={topk} C={Cn} layout=tile16", flush=True)
+    router, gu, down, sh_gu, sh_down, x = config5_inputs(np.random.default_rng(506), n, ff, nexp, Cn, zipf=False)
+    want = oracle.moe_prefill_layer(n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, x, threads=16)
+    cnt = np.bincount(want["topi"].reshape(-1), minlength=nexp)
+    print(f"experts in use {np.count_nonzero(cnt)}, the busiest takes {cnt.max()} of {Cn} rows, jobs {want['njobs']}", flush=True)
+    assert cnt.max() <= 32 and np.count_nonzero(cnt) >= 500
+    r = fnx_gpu.PfLayerDev(dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, Cn, packed=True, tile16=True).run(x)
+    assert np.array_equal(r["logits"].view(np.uint32), want["logits"].view(np.uint32))
+    assert np.array_equal(r["topi"], want["topi"])
+    assert int(r["njobs"][0]) == want["njobs"]
+    err = rel_l2(r["out"], want["out"])
+    print("config 5 uniform chunk rel l2", err, flush=True)
     assert err <= REL_L2
