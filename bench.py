@@ -253,8 +253,9 @@ def main():
     P = T * TOPK
     ws_t = dict(xq=dev.zeros(T * (N // 32) * 36, t.uint8), logits=dev.zeros((T, NEXP + 1), t.float32), topi=dev.zeros((T, TOPK), t.int32),
                 topw=dev.zeros((T, TOPK), t.float32), jobs_gu=dev.zeros((P + 1) * 136, t.uint8), jobs_dn=dev.zeros((P + 1) * 136, t.uint8),
-                njobs=dev.zeros(2, t.int32), gu=dev.zeros((P + T, 2 * FF), t.float32), part=dev.zeros((P + T, N), t.float32))
-    ws = pkg.MoeWs(*(ws_t[k].data_ptr() for k in ("xq", "logits", "topi", "topw", "jobs_gu", "jobs_dn", "njobs", "gu", "part")))
+                njobs=dev.zeros(2, t.int32), gu=dev.zeros((P + T, 2 * FF), t.float32), part=dev.zeros((P + T, N), t.float32),
+                sync=dev.zeros(pkg.MOE_SYNC_WORDS, t.int32))
+    ws = pkg.MoeWs(*(ws_t[k].data_ptr() for k in ("xq", "logits", "topi", "topw", "jobs_gu", "jobs_dn", "njobs", "gu", "part", "sync")))
     st = dev.st()
 
     def step(i, sets=None):

@@ -32,6 +32,8 @@ extern "C" {
 #define FNX_T_IQ3S_TILE16 1022u /* the prompt path's own re-laying of IQ3_S (fnx_iq3s_tile16); not a ggml type */
 #define FNX_IQ3S_BLOCK 110 /* bytes per 256 weights */
 #define FNX_Q8_1_BLOCK 36  /* bytes per 32 activations: half d, half sum, int8 qs[32] */
+#define FNX_ERR_BARRIER 4u    /* error-word bit (engine_impl.hpp:211-218: "a grid barrier timed out"): a block of the verify window gave up
+                              * waiting for the blocks of its row (fnx_moe_ws.sync word 0) */
 #define FNX_ERR_NONFINITE 16u /* error-word bit (engine_impl.hpp:211-218) */
 #define FNX_ERR_WINDOW 32u    /* error-word bit: a window at a position outside its cache (below 0, or its last row past max_ctx);
                               * the attention then reads only cells that exist and the results mean nothing. No counterpart in the
@@ -196,11 +198,16 @@ typedef struct fnx_moe_ws {
     fnx_job* jobs_gu;/* [T * topk + 1] (the last one is the shared expert's) */
     fnx_job* jobs_dn;/* [T * topk + 1] */
     int* njobs;      /* [2], zeroed once */
-    float* gu;       /* [T * topk + T][2 ff] floats. Operator by operator: the gate|up outputs. The three-launch window keeps
+    float* gu;       /* [T * topk + T][2 ff] floats. Operator by operator: the gate|up outputs. The one-launch window keeps
                       * the pairs' h there instead, as q8_1 rows of its own record size, and never writes f32 gate|up rows */
-    float* part;     /* [T * topk + T][n] floats. Operator by operator: the down outputs. The three-launch window uses it only
+    float* part;     /* [T * topk + T][n] floats. Operator by operator: the down outputs. The one-launch window uses it only
                       * as scratch for a split-Q8_0 shared expert */
+    unsigned* sync;  /* [FNX_MOE_SYNC_WORDS], zeroed once: the arrival counters through which the blocks of the one-launch window
+                      * hand over within a window row (every window leaves them zero), and in word 0 the window's error bits:
+                      * FNX_ERR_BARRIER if a block gave up waiting for its row (kernels.cu:884, 899 bound the reference's device waits
+                      * the same way). After that error the results mean nothing and the words must be zeroed again */
 } fnx_moe_ws;
+#define FNX_MOE_SYNC_WORDS 544
 int fnx_moe_verify_layer(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st);
 /* The same window without a workspace argument and without any allocation: no counterpart in the reference. For callers
  * that cannot allocate device memory (code under graph capture, serving loops and harnesses that forbid it): the scratch

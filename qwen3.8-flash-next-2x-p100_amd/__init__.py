@@ -17,6 +17,8 @@ T_IQ3S_UNIT64 = 1021
 T_IQ3S_TILE16 = 1022
 IQ3S_BLOCK = 110
 Q8_1_BLOCK = 36
+MOE_SYNC_WORDS = 544   # fnx_moe_ws.sync: uint32 words, zeroed once
+ERR_BARRIER = 4
 
 
 class Job(C.Structure):
@@ -44,7 +46,7 @@ class MoeLayer(C.Structure):
 
 class MoeWs(C.Structure):
     _fields_ = [("xq", C.c_void_p), ("logits", C.c_void_p), ("topi", C.c_void_p), ("topw", C.c_void_p), ("jobs_gu", C.c_void_p),
-                ("jobs_dn", C.c_void_p), ("njobs", C.c_void_p), ("gu", C.c_void_p), ("part", C.c_void_p)]
+                ("jobs_dn", C.c_void_p), ("njobs", C.c_void_p), ("gu", C.c_void_p), ("part", C.c_void_p), ("sync", C.c_void_p)]
 
 
 class PfWs(C.Structure):

@@ -456,6 +456,7 @@ __global__ void __launch_bounds__(512) k_iq3s_jobs(const RowsArgs a) {
 }  // namespace fnx
 #include "k_iq3s_mma.h"
 #include "k_moe_layer.h"
+#include "k_moe_window.h"
 #include "k_prefill.h"
 #include "k_iq3s_mma16.h"
 #include "k_moe_mma_wave16.h"
@@ -844,7 +845,7 @@ static bool layer_fused_ok(const fnx_moe_layer* L, int T) {
     const bool shared_ok = shared_is_q8(L) || (packed(L->sh_gu) && packed(L->sh_down) && L->sh_gu.p && L->sh_down.p);
     return on && L->n == FL_N && (L->ff == 256 || L->ff == 512 || L->ff == 1024) && L->nexp <= 1024 && L->topk <= FL_MAXK &&
            T * L->topk <= FL_MAXP && packed(L->gu) && packed(L->down) && shared_ok && L->gu_stride % UNIT_BYTES == 0 &&
-           L->down_stride % UNIT_BYTES == 0;
+           L->down_stride % UNIT_BYTES == 0 && cu_count() >= WN_WAVES * T;   // sixteen blocks a row at least (moe_window_plan.h)
 }
 // per-launch timing of the window (fnx_layer_profile): events recorded on the launch stream around each of the three
 // launches; the counterpart of the reference's FNX_PROF stamps in its window graph (engine.cu:1382-1530)
@@ -858,38 +859,36 @@ static void prof_mark(int i, hipStream_t s) {
 // live (may be null): a device word, the rows of the window that count; the others are not routed and their rows of out are left alone
 static int layer_fused(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st, const int* live = nullptr) {
     hipStream_t s = (hipStream_t) st;
-    const int n = L->n, ff = L->ff, LS = L->nexp + 1;
-    const int rblocks = (LS + RQ_ROWS - 1) / RQ_ROWS, qblocks = (T * 64 + 2 * FL_WAVES - 1) / (2 * FL_WAVES);
+    const int n = L->n, ff = L->ff;
     prof_mark(0, s);
-    k_router_quant<<<rblocks + qblocks, FL_THREADS, 0, s>>>(RouterArgs{L->nexp, T, x, L->router, L->router_bf16, ws->logits, (uint8_t*) ws->xq, live});
-    // a split-Q8_0 shared expert runs as the reference runs it, three dense launches on the q8_1 rows just made
+    // a split-Q8_0 shared expert runs as the reference runs it, three dense launches on the q8_1 rows of x
     // (q8s_gemv -> swiglu_stacked_q8_1 -> q8s_gemv); its f32 rows, q8_1 rows of h and down rows take the workspace's
-    // part buffer, which the three-launch window does not use otherwise; the down launch adds its gated rows
+    // part buffer, which the window does not use otherwise; the window's down phase adds its gated rows
     const bool q8sh = shared_is_q8(L);
     float* sh_part = nullptr;
     if (q8sh) {
         float* sgu = ws->part;                                                              // [T][2 ff]
         uint8_t* shq = reinterpret_cast<uint8_t*>(sgu + (size_t) T * 2 * ff);                // [T][ff / 32] q8_1 blocks
         sh_part = sgu + (size_t) T * 2 * ff + ((size_t) T * (ff / 32) * FNX_Q8_1_BLOCK + 255) / 256 * 64;   // [T][n], 256-byte aligned after shq
+        if (fnx_quantize_q8_1(x, ws->xq, n, T, st)) return 1;
         if (fnx_q8s_gemv(&L->sh_gu_q8, ws->xq, sgu, 2 * ff, T, st)) return 1;
         if (fnx_swiglu_stacked_q8_1(sgu, shq, ff, T, st)) return 1;
         if (fnx_q8s_gemv(&L->sh_down_q8, shq, sh_part, n, T, st)) return 1;
     }
     prof_mark(1, s);
-    const RouteArgs route{L->nexp, L->topk, T, ws->logits, ws->topi, ws->topw, ws->jobs_gu, ws->jobs_dn, ws->njobs, live};
-    // at least as many blocks as the window has rows (a block's run of items then lies in two rows at most)
-    static const int gh_blocks = env_int("FNX_GH_BLOCKS", 0, 0, 4096);
-    const GateUpArgs ga{ff, (const uint8_t*) L->gu.p, L->gu_stride, (const uint8_t* const*) L->gu.ep, q8sh ? nullptr : (const uint8_t*) L->sh_gu.p,
-                        (const uint8_t*) ws->xq, (uint32_t*) ws->gu, route};
-    k_moe_gate_up_h<<<std::max(gh_blocks ? gh_blocks : cu_count(), FNX_MAXT), GH_THREADS, 0, s>>>(ga);
+    // a wait for another block gives up after this many ticks of the 100 MHz wall clock (FNX_WINDOW_WAIT_TICKS: for tests of the error path)
+    static const long long wait_ticks = env_int("FNX_WINDOW_WAIT_TICKS", 20000000, 0, 2000000000);
+    const WindowArgs wa{ff, L->nexp, L->topk, T, n, x, L->router, L->router_bf16,
+                        (const uint8_t*) L->gu.p, L->gu_stride, (const uint8_t* const*) L->gu.ep, q8sh ? nullptr : (const uint8_t*) L->sh_gu.p,
+                        (const uint8_t*) L->down.p, L->down_stride, (const uint8_t* const*) L->down.ep, q8sh ? nullptr : (const uint8_t*) L->sh_down.p,
+                        sh_part, ws->logits, ws->topi, ws->topw, (uint8_t*) ws->xq, (uint32_t*) ws->gu, out, ws->sync, live,
+                        ws->jobs_gu, ws->jobs_dn, ws->njobs, wait_ticks};
+    // one block a CU; a row's blocks are a power of two of at least sixteen (moe_window_plan.h)
+    const int nb = cu_count();
+    if (ff == 256) k_moe_window<8><<<nb, WN_THREADS, 0, s>>>(wa);
+    else if (ff == 512) k_moe_window<16><<<nb, WN_THREADS, 0, s>>>(wa);
+    else k_moe_window<32><<<nb, WN_THREADS, 0, s>>>(wa);
     prof_mark(2, s);
-    const DownArgs da{n, ff, L->topk, T, L->nexp, (const uint8_t*) L->down.p, L->down_stride, (const uint8_t* const*) L->down.ep,
-                      q8sh ? nullptr : (const uint8_t*) L->sh_down.p, (const uint32_t*) ws->gu, ws->topi, ws->topw, ws->logits, out, live, route,
-                      sh_part};
-    // a block per row and 32 units of the output, and one more for the job lists
-    if (ff == 256) k_moe_down_combine<8><<<T * (n / (8 * 32)) + 1, FL_THREADS, 0, s>>>(da);
-    else if (ff == 512) k_moe_down_combine<16><<<T * (n / (4 * 32)) + 1, FL_THREADS, 0, s>>>(da);
-    else k_moe_down_combine<32><<<T * (n / (2 * 32)) + 1, FL_THREADS, 0, s>>>(da);
     prof_mark(3, s);
     return launch_status("moe_verify_layer");
 }
@@ -1118,7 +1117,7 @@ static bool moe_shapes_ok(const fnx_moe_layer* L) {
 }
 static int moe_layer_checked(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st, const int* live = nullptr) {
     if (!L || !x || !ws) return fail("moe_verify_layer: null argument");
-    if (!ws->xq || !ws->logits || !ws->topi || !ws->topw || !ws->jobs_gu || !ws->jobs_dn || !ws->njobs || !ws->gu || !ws->part)
+    if (!ws->xq || !ws->logits || !ws->topi || !ws->topw || !ws->jobs_gu || !ws->jobs_dn || !ws->njobs || !ws->gu || !ws->part || !ws->sync)
         return fail("moe_verify_layer: incomplete workspace");
     if (topk_check(T, L->nexp, L->topk, "moe_verify_layer")) return 1;
     const int P = T * L->topk, n = L->n, ff = L->ff;
@@ -1168,7 +1167,7 @@ constexpr size_t NA_HQ = (size_t) (FL_MAXP + FNX_MAXT) * (1024 / 32) * HQ_WORDS 
 constexpr size_t na_up(size_t v) { return (v + 255) / 256 * 256; }
 constexpr size_t NA_OFF_LOGITS = na_up(NA_XQ), NA_OFF_TOPI = NA_OFF_LOGITS + na_up(NA_LOGITS), NA_OFF_TOPW = NA_OFF_TOPI + na_up(NA_TOP),
                  NA_OFF_JGU = NA_OFF_TOPW + na_up(NA_TOP), NA_OFF_JDN = NA_OFF_JGU + na_up(NA_JOBS), NA_OFF_NJOBS = NA_OFF_JDN + na_up(NA_JOBS),
-                 NA_OFF_HQ = NA_OFF_NJOBS + 256, NA_BYTES = NA_OFF_HQ + na_up(NA_HQ);
+                 NA_OFF_SYNC = NA_OFF_NJOBS + 256, NA_OFF_HQ = NA_OFF_SYNC + na_up(FNX_MOE_SYNC_WORDS * 4), NA_BYTES = NA_OFF_HQ + na_up(NA_HQ);
 static_assert(NA_BYTES <= FNX_MOE_STATIC_WS_BYTES, "the header states the array's size");
 static __device__ __align__(256) unsigned char scratch[FNX_MOE_STATIC_WS_BYTES];
 static unsigned char* g_scratch_ptr[64] = {};   // per device: the array's address there
@@ -1191,9 +1190,10 @@ int fnx_moe_verify_layer_static(const fnx_moe_layer* L, const float* x, int T, f
         }
     }
     unsigned char* w = g_scratch_ptr[dev];
-    // nothing in the workspace has to start at zero: every launch writes what it reads, and the job count is stored, not added to
+    // the sync words start at zero with the device image and every window leaves them zero; nothing else has to: every
+    // launch writes what it reads, and the job count is stored, not added to
     const fnx_moe_ws ws{w, (float*) (w + NA_OFF_LOGITS), (int*) (w + NA_OFF_TOPI), (float*) (w + NA_OFF_TOPW), (fnx_job*) (w + NA_OFF_JGU),
-                        (fnx_job*) (w + NA_OFF_JDN), (int*) (w + NA_OFF_NJOBS), (float*) (w + NA_OFF_HQ), nullptr};
+                        (fnx_job*) (w + NA_OFF_JDN), (int*) (w + NA_OFF_NJOBS), (float*) (w + NA_OFF_HQ), nullptr, (unsigned*) (w + NA_OFF_SYNC)};
     const int P = T * L->topk;
     if (shared_is_q8(L)) return fail("moe_verify_layer_static: a split-Q8_0 shared expert needs a caller's workspace (fnx_moe_verify_layer)");
     if (!moe_shapes_ok(L)) return fail("moe_verify_layer_static: weight shapes do not match n / ff");
@@ -1202,6 +1202,11 @@ int fnx_moe_verify_layer_static(const fnx_moe_layer* L, const float* x, int T, f
     return layer_fused(L, x, T, out, &ws, st);
 }
 
+#ifdef FNX_WIN_TS
+int fnx_debug_win_ts(unsigned long long* host, size_t words) {   // timing build only
+    return hipMemcpyFromSymbol(host, HIP_SYMBOL(g_win_ts), words * 8) == hipSuccess ? 0 : fail("debug_win_ts");
+}
+#endif
 // ---------------------------------------------------------------- streaming calibration (k_stream.h)
 int fnx_stream_read(const void* p, size_t bytes, int variant, int blocks, int threads, void* sink, void* st) {
     if (!p || !sink) return fail("stream_read: null argument");

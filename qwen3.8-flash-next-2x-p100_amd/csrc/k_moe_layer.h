@@ -157,7 +157,8 @@ __device__ __forceinline__ void write_job_lists(RouteLds<NT>& L, const RouteArgs
     static_assert(FL_MAXP <= NT, "a thread per pair");
     const int tid = threadIdx.x, wave = uniform(tid >> 6), lane = tid & 63;
     const int T = a.T, topk = a.topk, P = T * topk, Pl = Tl * topk;
-    const int e_mine = tid < Pl ? a.topi[tid] : 0;
+    // the picks were written by other blocks of this launch: read at the device's level, past this XCD's L2
+    const int e_mine = tid < Pl ? __hip_atomic_load(&a.topi[tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0;
     for (int e = tid; e < a.nexp; e += NT) {
         L.mask[e] = 0u;
         L.first[e] = P;

@@ -1,0 +1,676 @@
+// The MoE half of a verify window (the work of Engine::ffn_half, engine.cu:1569-1757 of the reference, on one GPU) as ONE
+// launch: router logits -> top-k -> gate|up of the shared and the routed experts -> SwiGLU to q8_1 -> down with the
+// combine's chains. The reference runs these as operators of their own inside a captured graph; on this GPU every
+// kernel boundary costs the start and the drain of a launch that streams ~100 MB (a fifth of its time), and the
+// dependencies between the phases are local to a window row: a row's router logits are needed by that row's blocks only,
+// and a row's h (8 KB) is made and used by the same sixteen blocks. So a block belongs to one row for the whole launch
+// and the row's blocks hand over through two arrival counters in the workspace - never the whole grid.
+//
+//   phase R   block (t, g) computes row t's logits of its slice of the router (slice g is read by the blocks g of all
+//             rows, which share an XCD and its L2: the router leaves HBM once) and the q8_1 blocks of x[t] (kept in LDS),
+//             then arrives on the row's first counter; the shared expert's gate|up item, which needs no pick, runs
+//             while the row's logits gather.
+//   phase G   every block ranks its row itself (slices of 64 experts a wave, one wave merges) and sweeps its gate|up
+//             items - (32 values of h) x (matrix) - as k_moe_gate_up_h does; a sweep's h leaves as a q8_1 block; the
+//             block arrives on the row's second counter.
+//   phase D   the block's units of the down matrices: the first trips' weights are asked for before the wait for the row's
+//             h; then the trips with the combine's fmaf chain in pick order (kernels.cu:412-419).
+//
+// What crosses blocks (logits, picks, h) is written and read with agent-scope accesses that go past the XCDs' own L2s;
+// no fence that writes back or invalidates a cache is needed. Every wait is bounded: a wait on another block by a
+// wall-clock budget, a wait inside the block by a trip count; a wait that gives up sets FNX_ERR_BARRIER in the
+// workspace's sync word 0 and the block leaves (the reference bounds its device waits the same way, kernels.cu:884, 899,
+// bit 4 of engine_impl.hpp:211-218). A block waits only for blocks of its own row, which lie next to it in the grid: with
+// blocks dispatched in order a row's blocks are resident together, or become so as earlier rows finish.
+//
+// Arithmetic is the operators': the router sums in the fixed 64-lane order, top-k by (value, lower index), the q8_1
+// rounding, the IQ3_S sub-block terms, the combine's fmaf chain.
+#pragma once
+
+#include "k_moe_layer.h"
+#include "moe_window_plan.h"
+
+namespace fnx {
+
+constexpr int WN_THREADS = WN_WAVES * 64;
+constexpr int WN_SLOTS = 4, WN_LAG = 2;
+constexpr unsigned WN_LDS_SPINS = 1u << 22;   // trips of a wait inside the block before it gives up (tenths of a second)
+// the workspace's sync words (zero before the first window; every window leaves them zero)
+constexpr int WS_ERR = 0, WS_ROUTED = 1, WS_FIN = 2, WS_ROW0 = 32, WS_ROW_STRIDE = 32;   // a row's words: 0 logits arrivals, 1 h arrivals, 2 blocks done
+static_assert(WS_ROW0 + FNX_MAXT * WS_ROW_STRIDE <= FNX_MOE_SYNC_WORDS, "the header states the sync area's size");
+
+struct WindowArgs {
+    int ff, nexp, topk, T, rows;
+    const float* x;           // [T][FL_N]
+    const void* router;       // [nexp + 1][FL_N]
+    int router_bf16;
+    const uint8_t* gu;        // routed gate|up: expert e at gu + e * gu_stride, or gu_ep[e]
+    size_t gu_stride;
+    const uint8_t* const* gu_ep;
+    const uint8_t* gu_shared; // null: the shared expert runs elsewhere (its down rows come in sh_part)
+    const uint8_t* dn;
+    size_t dn_stride;
+    const uint8_t* const* dn_ep;
+    const uint8_t* dn_shared;
+    const float* sh_part;     // [T][rows] when gu_shared is null
+    float* logits;            // [T][nexp + 1]
+    int* topi;                // [T][topk]
+    float* topw;
+    uint8_t* xq;              // [T][FL_N / 32] q8_1 blocks (an output for the caller; the blocks keep their own copy in LDS)
+    uint32_t* hq;             // [pair][ff / 32][HQ_WORDS]
+    float* out;               // [T][rows]
+    unsigned* sync;           // FNX_MOE_SYNC_WORDS words
+    const int* live;          // may be null; else a device word: rows from *live on are left alone
+    fnx_job* jobs_gu;
+    fnx_job* jobs_dn;
+    int* njobs;
+    long long wait_ticks;     // budget of a wait for another block, in ticks of the 100 MHz wall clock
+};
+
+template <int SBR>
+struct WinLds {
+    uint32_t tab[SGRID_WORDS];
+    uint32_t wp[FL_MAXK + 1][2];       // gate|up matrices: the shared expert's, then the picks'
+    float hgu[WN_SLOTS][64];           // a sweep's sums: the 32 gate rows', then the 32 up rows'
+    int flag[WN_SLOTS][WN_WAVES];
+    int made[WN_SLOTS];
+    uint2 cand[16][FL_MAXK];
+    int sliced[16];
+    int ready;                         // picks whose matrices are known
+    int pe[FL_MAXK];                   // the picks
+    float pw[FL_MAXK];                 // their weights
+    float gate;                        // sigmoid of the shared expert's gate logit
+    int rarrive, harrive;              // waves of the block that have stored their logits / finished their sweeps
+    int lready, hready;                // 1: the row's logits / h rows are complete; -1: the wait gave up
+    int abort;                         // a wait inside the block gave up
+    int last;                          // this block is the last of its row to finish
+    int fin;                           // the row's ticket among the rows that have finished
+    int lists;                         // 1: every row has been ranked, the job lists can be written; -1: the wait gave up
+    uint32_t xq[FL_N / 32][FNX_Q8_1_BLOCK / 4];          // the row's q8_1 blocks
+    __attribute__((aligned(16))) uint32_t hq[FL_MAXK + 1][SBR][HQ_WORDS];   // the row's pairs' h rows (phase D)
+};
+
+// A wait of one wave for a word of another block's. False: the budget ran out (the error bit is set).
+__device__ __forceinline__ bool win_wait_word(const unsigned* p, unsigned want, long long ticks, unsigned* err) {
+    const long long t0 = (long long) wall_clock64();
+    while (true) {
+        const unsigned v = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (uniform((int) v) >= (int) want) return true;
+        if ((long long) wall_clock64() - t0 > ticks) {
+            if ((threadIdx.x & 63) == 0) atomicOr(err, FNX_ERR_BARRIER);
+            return false;
+        }
+        __builtin_amdgcn_s_sleep(4);
+    }
+}
+#ifdef FNX_WIN_TS
+// timing build only: wall-clock stamps of every wave at the phases' ends
+constexpr int WIN_NTS = 32;
+__device__ unsigned long long g_win_ts[1024 * WN_WAVES * WIN_NTS];
+#define WIN_TS(i)                                                                                                 \
+    do {                                                                                                          \
+        if ((threadIdx.x & 63) == 0) g_win_ts[((size_t) blockIdx.x * WN_WAVES + (threadIdx.x >> 6)) * WIN_NTS + (i)] = wall_clock64(); \
+    } while (0)
+#else
+#define WIN_TS(i)
+#endif
+// all of this wave's memory writes have been taken at the device's level before anything after this line
+__device__ __forceinline__ void win_stores_done() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+template <int SBR>
+__global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
+    __shared__ WinLds<SBR> S;
+    constexpr int RW = 64 / SBR, RMAX = SBR / 8, NB = RMAX == 4 ? 2 : 3;   // rows a unit; units a wave and trip at most; trips' buffers
+    const int tid = threadIdx.x, wave = uniform(tid >> 6), lane = tid & 63;
+    // the codebook's 512 unsigned entries: the launch's first load; the blocks read different signed forms of the table in
+    // memory (2 KiB apart) and negate them back, so that not every wave of the grid asks the same sixteen cache lines at once
+    const int form = (2 * (int) blockIdx.x + (tid >> 9)) & 15;
+    const uint32_t tab0 = signed_entry(g_sgrid.v[(form << 9) + (tid & 511)], form);
+    const int T = a.T, topk = a.topk, nexp = a.nexp, LS = nexp + 1, P = T * topk;
+    const int Tl = a.live ? uniform(max(0, min(*a.live, T))) : T;
+    if (Tl <= 0) return;
+    const WinPlan pl = win_plan((int) gridDim.x, Tl, nexp, topk, a.gu_shared != nullptr, a.ff);
+    const int t = (int) blockIdx.x / pl.G, g = (int) blockIdx.x - t * pl.G;
+    if (t >= Tl) return;
+    WIN_TS(0);
+    const int k0 = pl.k0, nk = pl.nk, qpp = pl.qpp;
+    unsigned* const srow = a.sync + WS_ROW0 + t * WS_ROW_STRIDE;
+    unsigned* const serr = a.sync + WS_ERR;
+    const float* xrow = a.x + (size_t) t * FL_N;
+
+    // ---------------------------------------------------------------- phase R: loads
+    // the row of x as the router's sums take it (lane l: float4 chunks l, l + 64, ...), and the values this wave quantises
+    // (blocks 4 wave .. 4 wave + 3 of the row's 64, a half-wave a block)
+    float4 xr[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) xr[c] = reinterpret_cast<const float4*>(xrow)[c * 64 + lane];
+    float xv[2];
+#pragma unroll
+    for (int r = 0; r < 2; ++r) xv[r] = xrow[(4 * wave + 2 * r + (lane >> 5)) * 32 + (lane & 31)];
+    // this wave's router rows: rows r0 + wave, r0 + wave + 16, ... of the block's slice, two at a time
+    const int r0 = g * pl.rpb, r1 = min(nexp, r0 + pl.rpb);
+    auto load_router_row = [&](int row, float4(&w)[8]) {
+        if (row >= r1) {
+#pragma unroll
+            for (int c = 0; c < 8; ++c) w[c] = make_float4(0.f, 0.f, 0.f, 0.f);
+        } else if (a.router_bf16) {
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                const uint2 u = reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(a.router) + (size_t) row * FL_N)[c * 64 + lane];
+                w[c] = make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u), __uint_as_float(u.y << 16),
+                                   __uint_as_float(u.y & 0xffff0000u));
+            }
+        } else {
+#pragma unroll
+            for (int c = 0; c < 8; ++c) w[c] = reinterpret_cast<const float4*>(reinterpret_cast<const float*>(a.router) + (size_t) row * FL_N)[c * 64 + lane];
+        }
+    };
+    // the fixed order of k_gemv_rows (and of the CPU oracle): chunks in order, fmaf over x, y, z, w, then the xor butterfly
+    auto router_dot = [&](const float4(&w)[8]) {
+        float s = 0.f;
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            s = fmaf(w[c].x, xr[c].x, s);
+            s = fmaf(w[c].y, xr[c].y, s);
+            s = fmaf(w[c].z, xr[c].z, s);
+            s = fmaf(w[c].w, xr[c].w, s);
+        }
+        return group_sum<64>(s);
+    };
+    float4 wa[8], wb[8];
+    load_router_row(r0 + wave, wa);
+    load_router_row(r0 + wave + WN_WAVES, wb);
+
+    // ---------------------------------------------------------------- LDS: flags, the codebook, the row's q8_1 blocks
+    if (tid < WN_SLOTS * WN_WAVES) (&S.flag[0][0])[tid] = 0;
+    if (tid < WN_SLOTS) S.made[tid] = 0;
+    if (tid < 16) S.sliced[tid] = 0;
+    if (tid == 0) {
+        S.ready = 0;
+        S.rarrive = S.harrive = 0;
+        S.lready = S.hready = 0;
+        S.abort = 0;
+        S.last = 0;
+        S.fin = -1;
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) S.tab[tid + i * WN_THREADS] = signed_entry(tab0, (tid >> 9) + 2 * i);
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {   // kernels.cu:131-145 (quantize_q8_1), a half-wave a block
+        const int b = 4 * wave + 2 * r + (lane >> 5), l32 = lane & 31;
+        const float xi = xv[r];
+        const float amax = group_max<32>(fabsf(xi)), sum = group_sum<32>(xi);
+        const float d = amax / 127.0f;
+        const int8_t qv = amax == 0.0f ? (int8_t) 0 : (int8_t) roundf(xi / d);
+        reinterpret_cast<int8_t*>(&S.xq[b][1])[l32] = qv;
+        if (l32 == 0) S.xq[b][0] = (uint32_t) float_to_half_bits(d) | (uint32_t) float_to_half_bits(sum) << 16;
+    }
+    __syncthreads();
+    WIN_TS(1);
+    if (g == 0 && tid < (FL_N / 32) * (FNX_Q8_1_BLOCK / 4))   // the caller's copy of the row's q8_1 blocks
+        reinterpret_cast<uint32_t*>(a.xq + (size_t) t * (FL_N / 32) * FNX_Q8_1_BLOCK)[tid] = (&S.xq[0][0])[tid];
+
+    // ---------------------------------------------------------------- phase R: the sums, the arrival
+    {
+        int row = r0 + wave;
+        while (true) {
+            const float va = router_dot(wa), vb = router_dot(wb);
+            if (lane == 0) {
+                if (row < r1) __hip_atomic_store(&a.logits[(size_t) t * LS + row], va, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (row + WN_WAVES < r1) __hip_atomic_store(&a.logits[(size_t) t * LS + row + WN_WAVES], vb, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            row += 2 * WN_WAVES;
+            if (row >= r1) break;
+            load_router_row(row, wa);
+            load_router_row(row + WN_WAVES, wb);
+        }
+        win_stores_done();
+        WIN_TS(2);
+        int old = 0;
+        if (lane == 0) old = atomicAdd(&S.rarrive, 1);
+        if (uniform(old) == WN_WAVES - 1)   // the block's last wave to get here: the block's logits are out
+            if (lane == 0) __hip_atomic_fetch_add(&srow[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+
+    // ---------------------------------------------------------------- phase G
+    // the lane's sub-block of the row's activations
+    int xs[8];
+    float dx;
+    {
+        const uint32_t* xb = S.xq[lane];
+        dx = half_bits_to_float(xb[0] & 0xFFFFu);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) xs[j] = (int) xb[1 + j];
+    }
+    const int I0 = g * pl.ipb, I1 = min(pl.per_row, I0 + pl.ipb), nsweep = max(I1 - I0, 0);   // this block's items of its row
+    const PackedVOffs o = packed_voffs(lane);
+    const int uo_g = wave * 2 * UNIT_BYTES, uo_u = uo_g + a.ff * UNIT_BYTES;   // the wave's gate units and up units from an item's first gate unit
+    struct Item {
+        int j, k;   // block of 32 h values, matrix (0: the shared expert's, k: pick k - 1's)
+    };
+    auto item_of = [&](int I) {
+        Item m;
+        m.j = uniform(I / nk);
+        m.k = k0 + I - m.j * nk;
+        return m;
+    };
+    auto step = [&](Item& m) {
+        if (++m.k > topk) {
+            m.k = k0;
+            ++m.j;
+        }
+    };
+    PackedSub A[4];
+    auto issue_from = [&](const uint8_t* e, int j) {   // e: wave-uniform
+        const __amdgpu_buffer_rsrc_t mtx = matrix_rsrc(e);
+        const int ub = uniform(j) * 32 * UNIT_BYTES;
+        A[0] = load_packed_buf(mtx, ub + uo_g, o);
+        A[1] = load_packed_buf(mtx, ub + uo_g + UNIT_BYTES, o);
+        A[2] = load_packed_buf(mtx, ub + uo_u, o);
+        A[3] = load_packed_buf(mtx, ub + uo_u + UNIT_BYTES, o);
+    };
+    // a wait on a word of this block's LDS; false: gave up (or another wave did)
+    auto lds_wait = [&](auto cond) {
+        for (unsigned n = 0; !cond(); ++n) {
+            // (every condition here is wave-uniform and says so: a loop left on a per-lane condition would make the compiler treat
+            // the item counters that live across it as per-lane values, and every load that takes one as a loop over the lanes)
+            if (n >= WN_LDS_SPINS || uniform(__hip_atomic_load(&S.abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP))) {
+                if (lane == 0) {
+                    __hip_atomic_store(&S.abort, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    atomicOr(serr, FNX_ERR_BARRIER);
+                }
+                return false;
+            }
+            __builtin_amdgcn_s_sleep(1);
+        }
+        return true;
+    };
+    Item ma = item_of(I0);
+    const bool early = nsweep > 0 && ma.k == 0;   // the run starts with a shared expert's item: no pick needed to ask for it
+    if (early) issue_from(a.gu_shared, ma.j);
+    // the row's logits: one wave waits for the row's blocks, the others for its word
+    if (wave == WN_WAVES - 1) {
+        const bool ok = win_wait_word(&srow[0], (unsigned) pl.G, a.wait_ticks, serr);
+        if (lane == 0) __hip_atomic_store(&S.lready, ok ? 1 : -1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    const int sc_shift = 4 * (lane & 1);
+    // where a lane's sum goes after reduce4_units: the 16-lane rows hold gate 2 i, up 2 i, gate 2 i + 1, up 2 i + 1
+    const int zidx = (lane & 16 ? 32 : 0) + 2 * wave + (lane >> 5);
+    auto decode = [&](int sw) {
+        const int slot = sw & (WN_SLOTS - 1);
+        float v[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            int w4[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) w4[j] = *reinterpret_cast<const int*>(reinterpret_cast<const uint8_t*>(S.tab) + packed_addr(A[r].idx, j));
+            const int sc = 1 + 2 * (int) ((A[r].sc >> sc_shift) & 0xFu);
+            const float dw = half_bits_to_float(A[r].d);
+            int sum = 0;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) sum = __builtin_amdgcn_sdot4(w4[j], xs[j], sum, false);
+            // one sub-block's term as the reference forms it: (d_w * d_x) * (float) (sumi * (1 + 2 s))
+            v[r] = (dw * dx) * (float) __mul24(sum, sc);
+        }
+        const float z = reduce4_units(v[0], v[1], v[2], v[3]);   // units: gate 2 i, gate 2 i + 1, up 2 i, up 2 i + 1
+        // the slot's last block (of sweep sw - WN_SLOTS) must have been made: nearly always long ago
+        if (sw >= WN_SLOTS &&
+            !lds_wait([&] { return uniform(__hip_atomic_load(&S.made[slot], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP)) >= sw - WN_SLOTS + 1; }))
+            return false;
+        if ((lane & 15) == 0) S.hgu[slot][zidx] = z;
+        if (lane == 0) __hip_atomic_store(&S.flag[slot][wave], sw + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+        return true;
+    };
+    // the q8_1 block of sweep q, by the first half of the wave whose turn it is (k_moe_h, moe.cuh:597-608)
+    auto make_block = [&](int q) {
+        const int slot = q & (WN_SLOTS - 1);
+        if (!lds_wait([&] {   // all sixteen waves' values of sweep q must be there
+                const int f = lane < WN_WAVES ? __hip_atomic_load(&S.flag[slot][lane], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) : q + 1;
+                return __ballot(f < q + 1) == 0ull;
+            }))
+            return false;
+        const Item m = item_of(I0 + q);
+        const int pair = m.k > 0 ? t * topk + m.k - 1 : P + t;
+        if (lane < 32) {
+            const float h = silu_f(S.hgu[slot][lane]) * S.hgu[slot][32 + lane];
+            const float amax = group_max<32>(fabsf(h));
+            const float d = amax / 127.0f;
+            const uint32_t qv = amax == 0.0f ? 0u : (uint32_t) (uint8_t) (int8_t) roundf(h / d);
+            uint32_t word = qv | (uint32_t) __shfl_down((int) qv, 1, WAVE) << 8;
+            word |= (uint32_t) __shfl_down((int) word, 2, WAVE) << 16;
+            uint32_t* dst = a.hq + ((size_t) pair * qpp + m.j) * HQ_WORDS;
+            if ((lane & 3) == 0) __hip_atomic_store(&dst[lane >> 2], word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (lane == 0) __hip_atomic_store(&dst[8], __float_as_uint(half_bits_to_float(float_to_half_bits(d))), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (lane == 0) __hip_atomic_store(&S.made[slot], q + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+        return true;
+    };
+    int sw = 0;
+    if (early) {   // the shared expert's item while the row's logits gather
+        if (!decode(0)) return;
+        sw = 1;
+    }
+    WIN_TS(13);
+    // The row's picks (moe.cuh:382-411: greater value first, the lower index on a tie; w_k = exp(l_k - l_0) / sum in pick
+    // order). Every wave with a slice lists the topk greatest of its 64 experts in order; wave 0 merges the slices' lists by
+    // their heads and hands each pick's matrix out as soon as it is known.
+    if (!lds_wait([&] { return uniform(__hip_atomic_load(&S.lready, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP)) != 0; })) return;
+    if (uniform(__hip_atomic_load(&S.lready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) < 0) return;
+    WIN_TS(3);
+    const int ns = (nexp + 63) >> 6;   // slices of 64 experts
+    for (int sl = wave; sl < ns; sl += WN_WAVES) {
+        const int e = 64 * sl + lane;
+        const float v = e < nexp ? __hip_atomic_load(&a.logits[(size_t) t * LS + e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : -INFINITY;
+        unsigned key = rank_key(v);
+        for (int k = 0; k < topk; ++k) {
+            const unsigned m = wave_umax(key);
+            const unsigned long long hold = m > RANK_KEY_NEG_INF ? __ballot(key == m) : 0ull;
+            const int l = hold ? (int) __builtin_ctzll(hold) : 64;   // the lowest lane that holds the maximum is the lowest expert
+            key = lane == l ? 0u : key;
+            if (lane == 0) S.cand[sl][k] = make_uint2(hold ? m : 0u, (uint32_t) (hold ? 64 * sl + l : nexp));
+        }
+        if (lane == 0) __hip_atomic_store(&S.sliced[sl], 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    WIN_TS(4);
+    if (wave == 0) {   // the merge; the row's first block writes the picks and their weights out
+        const bool publish = g == 0;
+        if (!lds_wait([&] {
+                const int f = lane < ns ? __hip_atomic_load(&S.sliced[lane], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) : 1;
+                return __ballot(f == 0) == 0ull;
+            }))
+            return;
+        // All of the row's candidates in registers, entry p of list j in lane (16 j + p) mod 64 of register (16 j + p) / 64;
+        // lane j < ns keeps list j's head and its position; the list whose head is picked gets its next entry by a read of
+        // that lane.
+        static_assert(FL_MAXK == 16, "sixteen entries a list, four lists a register");
+        int ck[4], ce[4];
+        {
+            const uint2* flat = &S.cand[0][0];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint2 c = flat[q * 64 + lane];
+                ck[q] = (int) c.x;
+                ce[q] = (int) c.y;
+            }
+        }
+        unsigned hk = lane < ns ? S.cand[min(lane, ns - 1)][0].x : 0u;
+        int he = S.cand[min(lane, ns - 1)][0].y, hp = 0;
+        unsigned mk = 0u;
+        int ei = 0x7fffffff;
+        unsigned long long low_taken = 0ull;   // which of experts 0 .. 63 are picked: what a row with fewer than topk finite logits falls back on
+        for (int k = 0; k < topk; ++k) {
+            unsigned m = (unsigned) __builtin_amdgcn_readlane((int) row_umax(hk), 0);
+            const unsigned long long hold = m > RANK_KEY_NEG_INF ? __ballot(hk == m) & 0xFFFFull : 0ull;
+            const int l = hold ? (int) __builtin_ctzll(hold) : 64;   // the lowest lane that holds the maximum has the lowest expert
+            int idx;
+            unsigned nkey = 0u;
+            int ne = nexp, np = 0;
+            if (hold) {
+                idx = __builtin_amdgcn_readlane(he, l);
+                np = __builtin_amdgcn_readlane(hp, l) + 1;
+                if (np < topk) {   // list l's next entry
+                    const int f = 16 * l + np, fl = f & 63, fq = f >> 6;
+                    const int k0_ = __builtin_amdgcn_readlane(ck[0], fl), k1_ = __builtin_amdgcn_readlane(ck[1], fl);
+                    const int k2_ = __builtin_amdgcn_readlane(ck[2], fl), k3_ = __builtin_amdgcn_readlane(ck[3], fl);
+                    const int e0_ = __builtin_amdgcn_readlane(ce[0], fl), e1_ = __builtin_amdgcn_readlane(ce[1], fl);
+                    const int e2_ = __builtin_amdgcn_readlane(ce[2], fl), e3_ = __builtin_amdgcn_readlane(ce[3], fl);
+                    nkey = (unsigned) (fq == 0 ? k0_ : fq == 1 ? k1_ : fq == 2 ? k2_ : k3_);
+                    ne = fq == 0 ? e0_ : fq == 1 ? e1_ : fq == 2 ? e2_ : e3_;
+                }
+            } else {   // nothing finite is left: the lowest expert not picked yet, with weight exp(-inf) = 0
+                m = RANK_KEY_NEG_INF;
+                idx = (int) __builtin_ctzll(~low_taken);
+            }
+            if (idx < 64) low_taken |= 1ull << idx;
+            if (lane == l) {
+                hk = nkey;
+                he = ne;
+                hp = np;
+            }
+            if (lane == k) {
+                mk = m;
+                ei = idx;
+            }
+            {   // the pick's matrix is handed out at once: the sweeps need not wait for the whole ranking
+                const uint8_t* e = a.gu_ep ? a.gu_ep[idx] : a.gu + (size_t) idx * a.gu_stride;
+                if (lane == 0) {
+                    S.wp[1 + k][0] = (uint32_t) (uintptr_t) e;
+                    S.wp[1 + k][1] = (uint32_t) ((uint64_t) (uintptr_t) e >> 32);
+                    S.pe[k] = idx;
+                    __hip_atomic_store(&S.ready, k + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+                }
+            }
+        }
+        const float top0 = rank_key_inv((unsigned) __builtin_amdgcn_readlane((int) mk, 0));
+        const float ek = expf(rank_key_inv(mk) - top0);
+        float z = 0.f;
+        for (int k = 0; k < topk; ++k) z += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, ek), k));
+        if (lane < topk) S.pw[lane] = ek / z;
+        if (publish) {
+            if (lane < topk) {
+                __hip_atomic_store(&a.topi[t * topk + lane], ei, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(&a.topw[t * topk + lane], ek / z, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            win_stores_done();
+            if (lane == 0) __hip_atomic_fetch_add(&a.sync[WS_ROUTED], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        WIN_TS(5);
+    }
+    // an item's loads, once its matrix is known: matrix 0 is the shared expert's, matrix k pick k - 1's
+    auto issue = [&](const Item& m) {
+        const uint8_t* e = a.gu_shared;
+        const int mk_ = uniform(m.k);
+        if (mk_ > 0) {
+            if (!lds_wait([&] { return uniform(__hip_atomic_load(&S.ready, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP)) >= mk_; })) return false;
+            const uint2 p = *reinterpret_cast<const uint2*>(S.wp[mk_]);
+            e = (const uint8_t*) (uintptr_t) ((uint64_t) (uint32_t) uniform((int) p.x) | (uint64_t) (uint32_t) uniform((int) p.y) << 32);
+        }
+        issue_from(e, m.j);
+        return true;
+    };
+    // Every wave of the block makes the same sweeps: each slot sees all sixteen arrive. An item's loads are asked for when
+    // the item before it has been decoded; two sweeps later the wave whose turn it is makes the sweep's q8_1 block.
+    if (nsweep > 0) {
+        if (early) {
+            if (nsweep > 1) {
+                step(ma);
+                if (!issue(ma)) return;
+            }
+        } else if (!issue(ma)) return;
+        for (; sw < nsweep; ++sw) {
+            if (!decode(sw)) return;
+            WIN_TS(16 + (sw & 15));
+            if (sw + 1 < nsweep) {
+                step(ma);
+                if (!issue(ma)) return;
+            }
+            const int q = sw - WN_LAG;   // the sweep whose block is due; wave q mod 16 makes it
+            if (q >= 0 && (q & (WN_WAVES - 1)) == wave)
+                if (!make_block(q)) return;
+        }
+        for (int q = max(nsweep - WN_LAG, 0); q < nsweep; ++q)   // the last sweeps' blocks
+            if ((q & (WN_WAVES - 1)) == wave)
+                if (!make_block(q)) return;
+    }
+
+    WIN_TS(6);
+    // ---------------------------------------------------------------- phase D
+    const bool ext = a.sh_part != nullptr;   // the shared expert's rows come from memory: the trips are the picks only
+    const int first = ext ? 1 : 0;
+    const bool dwave = wave < pl.dwaves;
+    const int R = pl.R, u0 = g * pl.upb + wave * R;   // this wave's units of every matrix
+    const int kb = lane % SBR, gl = lane / SBR;
+    // trip 0 is the shared expert's, trips 1 .. topk the picks in order
+    auto down_matrix = [&](int trip) -> const uint8_t* {
+        if (trip == 0) return a.dn_shared;
+        const int e = uniform(S.pe[trip - 1]);
+        return a.dn_ep ? a.dn_ep[e] : a.dn + (size_t) e * a.dn_stride;
+    };
+    PackedSub B[NB][RMAX];
+    auto issue_trip = [&](PackedSub(&buf)[RMAX], int trip) {
+        const __amdgpu_buffer_rsrc_t mtx = matrix_rsrc(uniform_ptr(down_matrix(trip)));
+#pragma unroll
+        for (int r = 0; r < RMAX; ++r)
+            if (r < R) buf[r] = load_packed_buf(mtx, (u0 + r) * UNIT_BYTES, o);
+    };
+    // The picks are known (this block ranked its row), so the first trips' weights are asked for before the wait for h.
+    // (The hand-over of the last pick's matrix has been seen by every wave that swept; a block without items waits here.)
+    if (!lds_wait([&] { return uniform(__hip_atomic_load(&S.ready, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP)) >= topk; })) return;
+    if (nsweep > 0) {   // this wave's h blocks are out: arrive
+        win_stores_done();
+        int old = 0;
+        if (lane == 0) old = atomicAdd(&S.harrive, 1);
+        if (uniform(old) == WN_WAVES - 1)
+            if (lane == 0) __hip_atomic_fetch_add(&srow[1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    WIN_TS(7);
+    if (dwave) {
+        issue_trip(B[0], first);
+        if (first + 1 <= topk) issue_trip(B[1], first + 1);
+    }
+    if (wave == 1) {   // the shared expert's gate: the router's last row against the row of x, in the router's order
+        float4 wg[8];
+        int l2 = lane;
+        asm volatile("" : "+v"(l2));   // the addresses are worked out here, not kept in registers since phase R
+#pragma unroll
+        for (int c = 0; c < 8; ++c) xr[c] = reinterpret_cast<const float4*>(xrow)[c * 64 + l2];
+        if (a.router_bf16) {
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                const uint2 u = reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(a.router) + (size_t) nexp * FL_N)[c * 64 + l2];
+                wg[c] = make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u), __uint_as_float(u.y << 16),
+                                    __uint_as_float(u.y & 0xffff0000u));
+            }
+        } else {
+#pragma unroll
+            for (int c = 0; c < 8; ++c) wg[c] = reinterpret_cast<const float4*>(reinterpret_cast<const float*>(a.router) + (size_t) nexp * FL_N)[c * 64 + l2];
+        }
+        const float v = router_dot(wg);
+        if (lane == 0) {
+            S.gate = sigmoid_f(v);
+            if (g == 0) a.logits[(size_t) t * LS + nexp] = v;
+        }
+    }
+    if (wave == 0) {   // the row's h rows: wait for the row's blocks that make them
+        const bool ok = win_wait_word(&srow[1], (unsigned) pl.nbi, a.wait_ticks, serr);
+        if (lane == 0) __hip_atomic_store(&S.hready, ok ? 1 : -1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    if (!lds_wait([&] { return uniform(__hip_atomic_load(&S.hready, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP)) != 0; })) return;
+    if (uniform(__hip_atomic_load(&S.hready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) < 0) return;
+    WIN_TS(8);
+    {   // the row's pairs' h rows into LDS, a pick's words side by side; the shared expert's are index topk
+        constexpr int HQ_PER = SBR * HQ_WORDS, HQ_VPT = ((FL_MAXK + 1) * HQ_PER + WN_THREADS - 1) / WN_THREADS;
+        uint32_t hw[HQ_VPT];
+#pragma unroll
+        for (int j = 0; j < HQ_VPT; ++j) {
+            const int i = tid + j * WN_THREADS, k = i / HQ_PER;
+            const bool has = k < topk || (k == topk && !ext);
+            hw[j] = has ? __hip_atomic_load(&a.hq[(size_t) (k < topk ? t * topk + k : P + t) * HQ_PER + (i - k * HQ_PER)], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+        }
+#pragma unroll
+        for (int j = 0; j < HQ_VPT; ++j) {
+            const int i = tid + j * WN_THREADS;
+            if (i < (topk + 1) * HQ_PER) (&S.hq[0][0][0])[i] = hw[j];
+        }
+    }
+    __syncthreads();
+    WIN_TS(9);
+    if (dwave) {
+        auto pick_of = [&](int trip) { return trip == 0 ? topk : trip - 1; };   // the index of a trip's expert in S.hq
+        float acc[RMAX], zs[RMAX];
+#pragma unroll
+        for (int r = 0; r < RMAX; ++r) acc[r] = zs[r] = 0.f;
+        const float gate = S.gate;
+        auto decode_trip = [&](const PackedSub(&buf)[RMAX], int trip) {
+            const int k = pick_of(trip);
+            const uint32_t* hb = S.hq[k][kb];
+            const uint4 lo = *reinterpret_cast<const uint4*>(hb), hi = *reinterpret_cast<const uint4*>(hb + 4);
+            const int hx[8] = {(int) lo.x, (int) lo.y, (int) lo.z, (int) lo.w, (int) hi.x, (int) hi.y, (int) hi.z, (int) hi.w};
+            const float dh = __uint_as_float(hb[8]);
+            const float gk = trip == 0 ? gate : S.pw[trip - 1];
+#pragma unroll
+            for (int r = 0; r < RMAX; ++r)
+                if (r < R) {
+                    int w4[8];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) w4[j] = *reinterpret_cast<const int*>(reinterpret_cast<const uint8_t*>(S.tab) + packed_addr(buf[r].idx, j));
+                    const int sc = 1 + 2 * (int) ((buf[r].sc >> sc_shift) & 0xFu);
+                    const float dw = half_bits_to_float(buf[r].d);
+                    int sum = 0;
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) sum = __builtin_amdgcn_sdot4(w4[j], hx[j], sum, false);
+                    const float z = dpp_group_sum<SBR>((dw * dh) * (float) __mul24(sum, sc));
+                    if (trip == 0) zs[r] = gk * z;
+                    else acc[r] = fmaf(gk, z, acc[r]);
+                }
+        };
+        if constexpr (NB == 3) {   // two trips' loads in flight while a third is decoded
+            for (int trip = first; trip <= topk; trip += 3) {
+                if (trip + 2 <= topk) issue_trip(B[2], trip + 2);
+                decode_trip(B[0], trip);
+                if (trip + 1 > topk) break;
+                if (trip + 3 <= topk) issue_trip(B[0], trip + 3);
+                decode_trip(B[1], trip + 1);
+                if (trip + 2 > topk) break;
+                if (trip + 4 <= topk) issue_trip(B[1], trip + 4);
+                decode_trip(B[2], trip + 2);
+            }
+        } else {   // four units a trip: one trip's loads in flight while another is decoded
+            for (int trip = first; trip <= topk; trip += 2) {
+                decode_trip(B[0], trip);
+                if (trip + 1 > topk) break;
+                if (trip + 2 <= topk) issue_trip(B[0], trip + 2);
+                decode_trip(B[1], trip + 1);
+                if (trip + 3 <= topk) issue_trip(B[1], trip + 3);
+            }
+        }
+        if (kb == SBR - 1) {   // the combine's last step: s + sigmoid * shared
+            float* orow = a.out + (size_t) t * a.rows + (size_t) u0 * RW + gl;
+#pragma unroll
+            for (int r = 0; r < RMAX; ++r)
+                if (r < R) {
+                    const float shared = ext ? gate * a.sh_part[(size_t) t * a.rows + (size_t) (u0 + r) * RW + gl] : zs[r];
+                    orow[r * RW] = acc[r] + shared;
+                }
+        }
+    }
+
+    WIN_TS(10);
+    // ---------------------------------------------------------------- the end of the block, of the row, of the window
+    // The last block of a row to get here puts the row's counters back; it takes the row's ticket among the finished
+    // rows: the first row to finish writes the job lists the operator API promises the caller (kernels.hpp:18-23, 277-282;
+    // nothing in this launch reads them), the last one puts the window's counters back.
+    __syncthreads();
+    if (tid == 0) {
+        const unsigned done = __hip_atomic_fetch_add(&srow[2], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (done == (unsigned) pl.G - 1) {
+            __hip_atomic_store(&srow[0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&srow[1], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&srow[2], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            S.fin = (int) __hip_atomic_fetch_add(&a.sync[WS_FIN], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            S.last = 1;
+        }
+    }
+    __syncthreads();
+    WIN_TS(11);
+    if (!S.last) return;
+    const int fin = S.fin;
+    if (fin == 0) {   // every row has been ranked long ago; the count says so
+        if (wave == 0) {
+            const bool ok = win_wait_word(&a.sync[WS_ROUTED], (unsigned) Tl, a.wait_ticks, serr);
+            if (lane == 0) {
+                S.lists = ok ? 1 : -1;
+                if (ok) __hip_atomic_store(&a.sync[WS_ROUTED], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        __syncthreads();
+        if (S.lists == 1) {
+            const RouteArgs route{nexp, topk, T, a.logits, a.topi, a.topw, a.jobs_gu, a.jobs_dn, a.njobs, a.live};
+            write_job_lists<WN_THREADS>(*reinterpret_cast<RouteLds<WN_THREADS>*>(S.tab), route, Tl);
+        }
+    }
+    if (fin == Tl - 1 && tid == 0) __hip_atomic_store(&a.sync[WS_FIN], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    WIN_TS(12);
+}
+
+}  // namespace fnx

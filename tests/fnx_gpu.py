@@ -436,9 +436,9 @@ class DecoderDev:
                       hidden=z((T, n), t.float32), logits=z((T, c["vocab"]), t.float32), best_v=z(T, t.float32), best_i=z(T, t.int32),
                       keys=z(16, t.int64), err=z(1, t.int32))
         self.mb = dict(xq=z(T * (n // 32) * 36, t.uint8), logits=z((T, nexp + 1), t.float32), topi=z((T, topk), t.int32),
-                       topw=z((T, topk), t.float32), jobs_gu=z((P + 1) * 136, t.uint8), jobs_dn=z((P + 1) * 136, t.uint8), njobs=z(2, t.int32),
+                       topw=z((T, topk), t.float32), jobs_gu=z((P + 1) * 136, t.uint8), jobs_dn=z((P + 1) * 136, t.uint8), njobs=z(2, t.int32), sync=z(pkg.MOE_SYNC_WORDS, t.int32),
                        gu=z((P + T, 2 * ff), t.float32), part=z((P + T, n), t.float32))
-        moe_ws = pkg.MoeWs(*(self.mb[k].data_ptr() for k in ("xq", "logits", "topi", "topw", "jobs_gu", "jobs_dn", "njobs", "gu", "part")))
+        moe_ws = pkg.MoeWs(*(self.mb[k].data_ptr() for k in ("xq", "logits", "topi", "topw", "jobs_gu", "jobs_dn", "njobs", "gu", "part", "sync")))
         self.ws = pkg.DecWs(*[self.b[k].data_ptr() for k in ("x", "xn", "qg", "k", "v", "att", "o", "attn_scratch", "xq", "hidden", "logits",
                                                              "best_v", "best_i", "keys", "err")], moe_ws)
         self.pos = dev.zeros(1, t.int32)
@@ -591,10 +591,11 @@ class MoeLayerDev:
         self.jobs_gu = dev.zeros((P + 1) * 136, t.uint8)
         self.jobs_dn = dev.zeros((P + 1) * 136, t.uint8)
         self.njobs = dev.zeros(2, t.int32)
+        self.sync = dev.zeros(pkg.MOE_SYNC_WORDS, t.int32)
         self.gu_out = dev.zeros((P + T, 2 * ff), t.float32)
         self.part = dev.zeros((P + T, n), t.float32)
         self.ws = pkg.MoeWs(self.xq.data_ptr(), self.logits.data_ptr(), self.topi.data_ptr(), self.topw.data_ptr(), self.jobs_gu.data_ptr(),
-                            self.jobs_dn.data_ptr(), self.njobs.data_ptr(), self.gu_out.data_ptr(), self.part.data_ptr())
+                            self.jobs_dn.data_ptr(), self.njobs.data_ptr(), self.gu_out.data_ptr(), self.part.data_ptr(), self.sync.data_ptr())
 
     def run(self, x):
         dev = self.dev
@@ -606,4 +607,5 @@ class MoeLayerDev:
         return dict(out=out.cpu().numpy(), logits=self.logits.cpu().numpy()[:T], topi=self.topi.cpu().numpy()[:T],
                     topw=self.topw.cpu().numpy()[:T], njobs=int(self.njobs.cpu().numpy()[0]),
                     gu=self.gu_out.cpu().numpy(), part=self.part.cpu().numpy(),
-                    jobs_gu=self.jobs_gu.cpu().numpy().view(JOB_DTYPE), jobs_dn=self.jobs_dn.cpu().numpy().view(JOB_DTYPE))
+                    jobs_gu=self.jobs_gu.cpu().numpy().view(JOB_DTYPE), jobs_dn=self.jobs_dn.cpu().numpy().view(JOB_DTYPE),
+                    sync=self.sync.cpu().numpy().view(np.uint32))

@@ -60,8 +60,9 @@ def test_layer_from_gguf_matches_oracle(dev, oracle, tmp_path, router_type, ff0,
     P = T * topk
     w = dict(xq=dev.zeros(T * (n // 32) * 36, t.uint8), logits=dev.zeros((T, nexp + 1), t.float32), topi=dev.zeros((T, topk), t.int32),
              topw=dev.zeros((T, topk), t.float32), jobs_gu=dev.zeros((P + 1) * 136, t.uint8), jobs_dn=dev.zeros((P + 1) * 136, t.uint8),
-             njobs=dev.zeros(2, t.int32), gu=dev.zeros((P + T, 2 * ff), t.float32), part=dev.zeros((P + T, n), t.float32))
-    ws = pkg.MoeWs(*(w[k].data_ptr() for k in ("xq", "logits", "topi", "topw", "jobs_gu", "jobs_dn", "njobs", "gu", "part")))
+             njobs=dev.zeros(2, t.int32), gu=dev.zeros((P + T, 2 * ff), t.float32), part=dev.zeros((P + T, n), t.float32),
+             sync=dev.zeros(pkg.MOE_SYNC_WORDS, t.int32))
+    ws = pkg.MoeWs(*(w[k].data_ptr() for k in ("xq", "logits", "topi", "topw", "jobs_gu", "jobs_dn", "njobs", "gu", "part", "sync")))
     dx, out = dev.up(x), dev.zeros((T, n), t.float32)
     dev.ok(lib.fnx_moe_verify_layer(C.byref(L), dx.data_ptr(), T, out.data_ptr(), C.byref(ws), dev.st()))
     dev.sync()
@@ -112,8 +113,9 @@ def test_layer_with_other_expert_types_from_gguf(dev, oracle, tmp_path):
     P = T * topk
     w = dict(xq=dev.zeros(T * (n // 32) * 36, t.uint8), logits=dev.zeros((T, nexp + 1), t.float32), topi=dev.zeros((T, topk), t.int32),
              topw=dev.zeros((T, topk), t.float32), jobs_gu=dev.zeros((P + 1) * 136, t.uint8), jobs_dn=dev.zeros((P + 1) * 136, t.uint8),
-             njobs=dev.zeros(2, t.int32), gu=dev.zeros((P + T, 2 * ff), t.float32), part=dev.zeros((P + T, n), t.float32))
-    ws = pkg.MoeWs(*(w[k].data_ptr() for k in ("xq", "logits", "topi", "topw", "jobs_gu", "jobs_dn", "njobs", "gu", "part")))
+             njobs=dev.zeros(2, t.int32), gu=dev.zeros((P + T, 2 * ff), t.float32), part=dev.zeros((P + T, n), t.float32),
+             sync=dev.zeros(pkg.MOE_SYNC_WORDS, t.int32))
+    ws = pkg.MoeWs(*(w[k].data_ptr() for k in ("xq", "logits", "topi", "topw", "jobs_gu", "jobs_dn", "njobs", "gu", "part", "sync")))
     x = rng.standard_normal((T, n)).astype(np.float32)
     dx, out = dev.up(x), dev.zeros((T, n), t.float32)
     dev.ok(lib.fnx_moe_verify_layer(C.byref(L), dx.data_ptr(), T, out.data_ptr(), C.byref(ws), dev.st()))
@@ -187,8 +189,9 @@ def test_layer_with_a_q8_0_shared_expert_from_gguf(dev, oracle, tmp_path):
     P = T * topk
     w = dict(xq=dev.zeros(T * (n // 32) * 36, t.uint8), logits=dev.zeros((T, nexp + 1), t.float32), topi=dev.zeros((T, topk), t.int32),
              topw=dev.zeros((T, topk), t.float32), jobs_gu=dev.zeros((P + 1) * 136, t.uint8), jobs_dn=dev.zeros((P + 1) * 136, t.uint8),
-             njobs=dev.zeros(2, t.int32), gu=dev.zeros((P + T, 2 * ff), t.float32), part=dev.zeros((P + T, n), t.float32))
-    ws = pkg.MoeWs(*(w[k].data_ptr() for k in ("xq", "logits", "topi", "topw", "jobs_gu", "jobs_dn", "njobs", "gu", "part")))
+             njobs=dev.zeros(2, t.int32), gu=dev.zeros((P + T, 2 * ff), t.float32), part=dev.zeros((P + T, n), t.float32),
+             sync=dev.zeros(pkg.MOE_SYNC_WORDS, t.int32))
+    ws = pkg.MoeWs(*(w[k].data_ptr() for k in ("xq", "logits", "topi", "topw", "jobs_gu", "jobs_dn", "njobs", "gu", "part", "sync")))
     dx, out = dev.up(x), dev.zeros((T, n), t.float32)
     dev.ok(lib.fnx_moe_verify_layer(C.byref(L), dx.data_ptr(), T, out.data_ptr(), C.byref(ws), dev.st()))
     dev.sync()

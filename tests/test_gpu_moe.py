@@ -38,7 +38,7 @@ def check_jobs(got, want):
 
 
 def check_layer(dev, oracle, n, ff, nexp, topk, T, seed, packed=False):
-    """packed: the unit64 layout (eligible shapes then run as the three-launch window)"""
+    """packed: the unit64 layout (eligible shapes then run as the one-launch window)"""
     print(f"case moe layer n={n} ff={ff} nexp={nexp} topk={topk} T={T} seed={seed} packed={packed}", flush=True)
     rng = np.random.default_rng(seed)
     router, gu, down, sh_gu, sh_down = make_layer(rng, n, ff, nexp)
@@ -47,6 +47,7 @@ def check_layer(dev, oracle, n, ff, nexp, topk, T, seed, packed=False):
     layer = fnx_gpu.MoeLayerDev(dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, packed=packed)
     layer.raw = (gu, down, sh_gu, sh_down)
     got = layer.run(x)
+    assert not got["sync"].any(), "no block gave up a wait, and the window put its arrival counters back to zero"
     assert np.array_equal(got["logits"].view(np.uint32), want["logits"].view(np.uint32)), "router logits bit-exact"
     assert np.array_equal(got["topi"], want["topi"]), "routing picks bit-exact"
     assert got["njobs"] == want["njobs"]
@@ -78,7 +79,7 @@ def test_moe_verify_layer_config2(dev, oracle, packed):
 @pytest.mark.parametrize("n,ff,nexp,topk,T", [(2048, 512, 64, 10, 1), (1024, 256, 32, 4, 16), (2048, 1024, 16, 2, 3), (512, 512, 16, 8, 7),
                                               (2048, 256, 40, 6, 9), (2048, 512, 1000, 10, 16), (2048, 512, 12, 10, 16)])
 def test_moe_verify_layer_shapes(dev, oracle, n, ff, nexp, topk, T, packed):
-    # with unit64 weights the shapes of hidden 2048 run as the three-launch window, the others operator by operator
+    # with unit64 weights the shapes of hidden 2048 run as the one-launch window, the others operator by operator
     check_layer(dev, oracle, n, ff, nexp, topk, T, 910 + T, packed)
 
 
@@ -94,7 +95,7 @@ def q8_split(oracle, rng, rows, cols, scale):
 @pytest.mark.parametrize("n,ff,nexp,topk,T", [(2048, 512, 512, 10, 16), (2048, 512, 64, 1, 3), (2048, 256, 24, 4, 7)])
 def test_moe_verify_layer_with_a_q8_0_shared_expert(dev, oracle, n, ff, nexp, topk, T, packed):
     """the reference's own form of the shared expert (engine.cu:1600-1604: split Q8_0 through q8s_gemv ->
-    swiglu_stacked_q8_1 -> q8s_gemv) beside IQ3_S routed experts: with unit64 experts inside the three-launch window,
+    swiglu_stacked_q8_1 -> q8s_gemv) beside IQ3_S routed experts: with unit64 experts inside the one-launch window,
     with raw blocks operator by operator"""
     print(f"case moe layer q8_0 shared n={n} ff={ff} nexp={nexp} topk={topk} T={T} packed={packed}", flush=True)
     rng = np.random.default_rng(940 + T)

@@ -38,3 +38,13 @@ def test_attention_window_bounds(tmp_path):
                     os.path.join(HERE, "attn_window_check.cpp")], check=True, capture_output=True, text=True)
     r = subprocess.run([exe], check=True, capture_output=True, text=True, timeout=120)
     assert r.stdout.startswith("ok "), r.stdout
+
+
+def test_window_plan(tmp_path):
+    """the one-launch verify window's split of a window over the grid, compiled for the host: every router row, gate|up item
+    and unit of the down matrices is taken exactly once and every hand-over waits for exactly the blocks that arrive"""
+    exe = str(tmp_path / "moe_window_plan_check")
+    subprocess.run(["g++", "-std=c++17", "-O1", "-Wall", "-Wextra", "-Werror", "-I", os.path.join(fnx_gpu.PKG_DIR, "csrc"), "-o", exe,
+                    os.path.join(HERE, "moe_window_plan_check.cpp")], check=True, capture_output=True, text=True)
+    r = subprocess.run([exe], check=True, capture_output=True, text=True, timeout=120)
+    assert r.stdout.startswith("ok "), r.stdout
