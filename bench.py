@@ -8,7 +8,7 @@ A step = one MoE layer of a verify window: T = 16 rows, hidden 2048, 512 IQ3_S e
 Steps cycle through LAYERS distinct weight sets (about 11 GB) and fresh activations so that a step's ~190 MB working set
 is cold with respect to the 256 MB Infinity Cache.
 
-Prints ONE JSON line: whole-step throughput, the roofline of the dominant kernel (the window's gate|up launch, timed
+Prints ONE JSON line: whole-step throughput, the roofline of the dominant kernel (the window's one launch, timed
 with events on the launch stream), what a read-only kernel reaches on the same GPU (roofline.stream_read_GBps), config 1
 (config.gemv), and the CPU baseline (the oracle on the host's cores, bounded sample). The experts are IQ3_S blocks encoded
 from N(0, 0.02) weights (--weights bytes: uniformly random blocks).
@@ -25,14 +25,14 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 N, FF, NEXP, TOPK, T = 2048, 512, 512, 10, 16
 HBM_PEAK = 8.0e12
-# HBM bytes of one gate|up launch of the default run (gaussian weights, 16 sets, unit64), measured by two rocprofv3 --pmc
+# HBM bytes of one window launch of the default run (gaussian weights, 16 sets, unit64), measured by two rocprofv3 --pmc
 # runs of this file (FETCH_SIZE, then WRITE_SIZE, each scaled by a 256 MiB copy: profiles/moe_gate_up_hbm_traffic.md), and
 # the distinct experts per step they were measured at. Not measured in the run: emitted only for that configuration.
-GATE_UP_TRAFFIC = {"bytes": 137.08e6, "algorithmic_bytes": 125.83e6, "distinct_experts_per_step": 138.45,
-                   "source": "profiles/moe_gate_up_hbm_traffic.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this file's default workload; scaled to "
+WINDOW_TRAFFIC = {"bytes": None, "algorithmic_bytes": 192.3e6, "distinct_experts_per_step": 138.45,
+                   "source": "profiles/moe_window_hbm_traffic.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this file's default workload; scaled to "
                              "this run's algorithmic bytes; not measured in this run)"}
 # the same for the prompt path's gate|up launch (profiles/prefill_chunk_counters.md: FETCH_SIZE x 2 + WRITE_SIZE)
-PF_GATE_UP_TRAFFIC = {"bytes": 162.6e6, "algorithmic_bytes": 98.6e6,
+PF_WINDOW_TRAFFIC = {"bytes": 162.6e6, "algorithmic_bytes": 98.6e6,
                       "source": "profiles/prefill_chunk_counters.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this file's prefill workload, k_moe_mma_wave16_gu; "
                                 "scaled to this run's algorithmic bytes; not measured in this run)"}
 IQ3S_BLOCK = 110
@@ -306,27 +306,26 @@ def main():
     u_mean = float(np.mean(njobs))
     step_bytes = u_mean * (GU_BYTES + DN_BYTES) + (GU_BYTES + DN_BYTES) + ROUTER_BYTES + XIO_BYTES
 
-    # ---- the dominant kernel: the window's gate|up launch (routed experts + the shared expert), timed with events the
-    # library records on the launch stream around each of the window's three launches (fnx_layer_profile)
-    names = ["router+q8_1", "top-k+plan+gate|up+swiglu", "down+combine"]
-    per_launch = np.zeros(3)
+    # ---- the dominant kernel: the window's one launch (router, top-k, gate|up, SwiGLU, down, combine), timed with events the
+    # library records on the launch stream around it (fnx_layer_profile)
+    names = ["before the window (a split-Q8_0 shared expert's dense launches)", "k_moe_window"]
+    per_launch = np.zeros(2)
     reps = max(50, min(args.steps, 200))
-    ms5 = np.zeros(3, dtype=np.float32)
+    ms2 = np.zeros(2, dtype=np.float32)
     fused = not args.raw_layout
     if fused:
         dev.ok(lib.fnx_layer_profile(1))
         for i in range(reps + 10):
             step(args.warmup + i)
-            dev.ok(lib.fnx_layer_profile_read(ms5.ctypes.data))
+            dev.ok(lib.fnx_layer_profile_read(ms2.ctypes.data))
             if i >= 10:
-                per_launch += ms5
+                per_launch += ms2
         dev.ok(lib.fnx_layer_profile(0))
         per_launch /= reps
         k_ms = float(per_launch[1])
-        kernel_name = "k_moe_gate_up_h (unit64)"
-        # algorithmic bytes of one launch: the distinct experts' and the shared expert's gate|up blocks, the window's
-        # q8_1 rows and router logits, the q8_1 rows of h
-        k_bytes = (u_mean + 1) * GU_BYTES + T * (N // 32) * 36 + T * (NEXP + 1) * 4 + (P + T) * (FF // 32) * 36
+        kernel_name = "k_moe_window (unit64; the whole window is this one launch)"
+        # algorithmic bytes of the launch: the step's (the distinct experts' and the shared expert's blocks, the router, x in, out)
+        k_bytes = step_bytes
     else:
         evs = []
         for i in range(reps + 10):
@@ -357,8 +356,8 @@ def main():
             torch.cuda.empty_cache()
         gemv = gemv_measure(dev, torch, np, 512)
     traffic = None
-    if fused and not args.shared_q8 and GATE_UP_TRAFFIC["bytes"] and abs(u_mean - GATE_UP_TRAFFIC["distinct_experts_per_step"]) < 3:
-        traffic = GATE_UP_TRAFFIC["bytes"] * k_bytes / GATE_UP_TRAFFIC["algorithmic_bytes"]
+    if fused and not args.shared_q8 and WINDOW_TRAFFIC["bytes"] and abs(u_mean - WINDOW_TRAFFIC["distinct_experts_per_step"]) < 3:
+        traffic = WINDOW_TRAFFIC["bytes"] * k_bytes / WINDOW_TRAFFIC["algorithmic_bytes"]
 
     # ---- CPU baseline: the oracle on the host's cores, same workload (layer set 0), bounded sample
     cpu = None
@@ -431,11 +430,11 @@ def main():
                    "ms_per_step_other_weights": None if other_ms is None else {("bytes" if args.weights == "gaussian" else "gaussian"): other_ms},
                    "gemv": gemv, "others": others},
         "roofline": {"bound": "hbm", "kernel": kernel_name, "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK, "traffic": traffic, "traffic_source": GATE_UP_TRAFFIC["source"] if traffic else None,
+                     "frac": achieved / HBM_PEAK, "traffic": traffic, "traffic_source": WINDOW_TRAFFIC["source"] if traffic else None,
                      "kernel_ms": k_ms, "algorithmic_bytes": k_bytes,
                      "window_launch_us": {n_: round(float(v) * 1e3, 2) for n_, v in zip(names, per_launch)},
                      "stream_read_GBps": stream,
-                     "frac_of_stream_read": None if not stream else achieved / 1e9 / stream["unit64_plane_loads_one_launch_134MB"]},
+                     "frac_of_stream_read_1GiB": None if not stream else achieved / 1e9 / stream["unit64_plane_loads_1GiB"]},
         "cpu_baseline": cpu,
     }
     print(json.dumps(line))
@@ -909,8 +908,8 @@ def prefill_main(args):
                    "step_flops": step_flops, "step_hbm_frac": step_bytes / (dt / steps) / HBM_PEAK, "step_mfma_frac": step_flops / (dt / steps) / MFMA_F16},
         "roofline": {"bound": "hbm", "kernel": gu_kernel, "achieved": gu_bytes / (gu_ms * 1e-3) / 1e9, "peak": HBM_PEAK / 1e9,
                      "unit": "GB/s", "frac": gu_bytes / (gu_ms * 1e-3) / HBM_PEAK,
-                     "traffic": PF_GATE_UP_TRAFFIC["bytes"] * gu_bytes / PF_GATE_UP_TRAFFIC["algorithmic_bytes"] if nsets == 4 and not args.raw_layout else None,
-                     "traffic_source": PF_GATE_UP_TRAFFIC["source"] if nsets == 4 and not args.raw_layout else None, "kernel_ms": gu_ms, "algorithmic_bytes": gu_bytes,
+                     "traffic": PF_WINDOW_TRAFFIC["bytes"] * gu_bytes / PF_WINDOW_TRAFFIC["algorithmic_bytes"] if nsets == 4 and not args.raw_layout else None,
+                     "traffic_source": PF_WINDOW_TRAFFIC["source"] if nsets == 4 and not args.raw_layout else None, "kernel_ms": gu_ms, "algorithmic_bytes": gu_bytes,
                      "mfma_tflops": gu_flops / (gu_ms * 1e-3) / 1e12, "mfma_frac": gu_flops / (gu_ms * 1e-3) / MFMA_F16,
                      "down": {"kernel": "k_moe_mma_tile64 (unit64)" if args.down_unit64 or args.raw_layout else "k_moe_mma_wave16 (tile16)", "kernel_ms": dn_ms, "achieved": dn_bytes / (dn_ms * 1e-3) / 1e9, "mfma_tflops": dn_flops / (dn_ms * 1e-3) / 1e12},
                      "two_launches": {"gate_up_ms": gu2_ms, "swiglu_ms": sw_ms, "note": "fnx_moe_gate_up_mma (k_moe_mma_block64, f32 products written) and fnx_swiglu_h16"},

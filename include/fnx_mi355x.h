@@ -62,7 +62,7 @@ typedef struct fnx_dw {
                              * operators (fnx_mmvq, fnx_moe_gate_up, fnx_moe_down, and fnx_moe_verify_layer operator by
                              * operator) also take ggml's Q4_0 (2), Q5_1 (7), Q8_0 (8), Q4_K (12), Q5_K (13), IQ4_NL (20) and IQ4_XS (23) rows, the
                              * other types of kernels.cu:2454-2471 that the reference's host code can decode; the
-                             * prompt path's grouped GEMM and the three-launch window are IQ3_S only */
+                             * prompt path's grouped GEMM and the one-launch window are IQ3_S only */
     int n_in, n_out;        /* columns, rows */
     size_t row_bytes;       /* n_in / 256 * 110 for IQ3_S; whole blocks of the type otherwise */
     const void* const* ep;  /* optional device table: expert e's matrix; null: expert e at p + e * stride */
@@ -160,10 +160,11 @@ int fnx_accept_greedy_dev(const int* rows, const int* o, int R, int* n_accept, v
 /* ---- the whole MoE half of a verify window (engine.cu:1569-1757 Engine::ffn_half without cards and streaming):
  * quantize -> router_route -> gate|up (routed + shared) -> swiglu q8_1 -> down (routed + shared) -> combine.
  * Same results as the calls above made one by one (up to the order of a few float additions). With unit64 experts,
- * n = 2048 and ff of 256, 512 or 1024 the window runs in three launches: [router logits | q8_1 rows], [top-k + gate|up
- * routed + shared + SwiGLU -> q8_1 rows of h], [down routed + shared + the combine's chains; the job lists for the
- * caller]; these touch only the caller's workspace, so windows with workspaces of their own may run on different streams
- * at once. Other shapes run operator by operator through the library's one pair buffer per device, like moe_down: the
+ * n = 2048 and ff of 256, 512 or 1024 (and a GPU of at least 16 CUs a window row) the window is one launch: a window
+ * row's blocks compute its router logits, rank it, run its gate|up sweeps (SwiGLU -> q8_1 rows of h) and its down trips
+ * with the combine's chains, handing over within the row through the workspace's sync words (fnx_moe_ws.sync, zeroed
+ * once); a block of the launch also writes the job lists for the caller. It touches only the caller's workspace, so
+ * windows with workspaces of their own may run on different streams at once. Other shapes run operator by operator through the library's one pair buffer per device, like moe_down: the
  * library puts such calls in order across streams (not under graph capture). A row with fewer than topk logits above
  * -inf (masked or NaN entries) takes the lowest experts not yet taken for its remaining picks, at weight 0, so its picks
  * stay distinct and no job exceeds 16 rows (the reference's result is undefined there); fnx_router_route and
@@ -212,20 +213,20 @@ int fnx_moe_verify_layer(const fnx_moe_layer* L, const float* x, int T, float* o
 /* The same window without a workspace argument and without any allocation: no counterpart in the reference. For callers
  * that cannot allocate device memory (code under graph capture, serving loops and harnesses that forbid it): the scratch
  * of fnx_moe_ws lives in one array of FNX_MOE_STATIC_WS_BYTES in the library's device image, which each GPU the library
- * runs on holds until the process ends. Only the three-launch window runs on it: unit64 experts, hidden 2048, ff 256,
+ * runs on holds until the process ends. Only the one-launch window runs on it: unit64 experts, hidden 2048, ff 256,
  * 512 or 1024, up to 1024 experts, up to 16 picks a row, T x topk <= 160; anything else is refused with a message. x and
  * out are the caller's, as above; results are those of fnx_moe_verify_layer bit for bit. All calls on a GPU share that
  * GPU's array: two of them in flight at once (two streams, two threads) race. */
 #define FNX_MOE_STATIC_WS_BYTES (448 * 1024)
 int fnx_moe_verify_layer_static(const fnx_moe_layer* L, const float* x, int T, float* out, void* st);
 /* Profiling aid, the counterpart of the reference's FNX_PROF stamps in its window graph (engine.cu:1382-1530):
- * fnx_layer_profile(1) makes the three-launch window record events on its stream around each launch (not to be
- * used under graph capture), fnx_layer_profile(0) stops that; fnx_layer_profile_read waits for the last recorded
- * window and returns its three launches' durations in milliseconds: router + q8_1 rows (with a split-Q8_0 shared
- * expert: and its three dense launches), top-k + gate|up + SwiGLU, down + combine. One profiled window at a time per
- * process. */
+ * fnx_layer_profile(1) makes the one-launch window record events on its stream around its launch (not to be used under
+ * graph capture), fnx_layer_profile(0) stops that; fnx_layer_profile_read waits for the last recorded window and returns two
+ * durations in milliseconds: [0] what runs before the window's launch (the three dense launches of a split-Q8_0 shared
+ * expert; next to nothing otherwise), [1] the window's launch (router, top-k, gate|up, SwiGLU, down, combine). One profiled
+ * window at a time per process. */
 int fnx_layer_profile(int on);
-int fnx_layer_profile_read(float* ms3);
+int fnx_layer_profile_read(float* ms2);
 /* Calibration aid (no counterpart in the reference): one read-only pass over `bytes` of device memory, nothing decoded,
  * so that the expert mat-vec launches can be judged against what the memory system gives a plain read of the same shape.
  * variant: 0 / 1 / 7 / 8: 16-byte loads a lane, 4 / 8 / 16 / 2 in flight, every wave one contiguous range; 2 / 3: the same 4 / 8
@@ -402,7 +403,7 @@ typedef struct fnx_round {
     float* chain_src; /* device, n floats (the hidden row the chain starts from); may be null when chain <= 1 */
 } fnx_round;
 /* one round: fnx_decoder_verify over the window -> acceptance and commit -> fnx_mtp_draft over the rows kept -> lookup
- * -> the next window. Expert weights must be in the unit64 layout and hidden = 2048 (the three-launch window), since only
+ * -> the next window. Expert weights must be in the unit64 layout and hidden = 2048 (the one-launch window), since only
  * that routes a row count held on the device. The draft layer uses the same workspace after the verify. */
 int fnx_decode_round(const fnx_decoder* D, const fnx_mtp* M, const fnx_round* R, const fnx_dec_ws* ws, void* st);
 

@@ -836,7 +836,7 @@ static int rows_launch(const fnx_dw* W, size_t w_stride, const fnx_job* jobs, co
     return launch_status(who);
 }
 
-// the shapes and layouts the window's three launches take (k_moe_layer.h)
+// the shapes and layouts the one-launch window takes (k_moe_window.h)
 // the shared expert as dense split Q8_0 (engine.cu:1600-1604) instead of sh_gu / sh_down
 static bool shared_is_q8(const fnx_moe_layer* L) { return L->sh_gu_q8.q && L->sh_down_q8.q; }
 static bool layer_fused_ok(const fnx_moe_layer* L, int T) {
@@ -847,15 +847,16 @@ static bool layer_fused_ok(const fnx_moe_layer* L, int T) {
            T * L->topk <= FL_MAXP && packed(L->gu) && packed(L->down) && shared_ok && L->gu_stride % UNIT_BYTES == 0 &&
            L->down_stride % UNIT_BYTES == 0 && cu_count() >= WN_WAVES * T;   // sixteen blocks a row at least (moe_window_plan.h)
 }
-// per-launch timing of the window (fnx_layer_profile): events recorded on the launch stream around each of the three
-// launches; the counterpart of the reference's FNX_PROF stamps in its window graph (engine.cu:1382-1530)
+// timing of the window (fnx_layer_profile): events recorded on the launch stream around the window's launch (and around the
+// dense launches of a split-Q8_0 shared expert before it); the counterpart of the reference's FNX_PROF stamps in its window
+// graph (engine.cu:1382-1530)
 static bool g_prof_on = false;
-static hipEvent_t g_prof_ev[4] = {};
+static hipEvent_t g_prof_ev[3] = {};
 static void prof_mark(int i, hipStream_t s) {
     if (g_prof_on) (void) hipEventRecord(g_prof_ev[i], s);
 }
-// the window's MoE half in three launches (k_moe_layer.h): [router logits | q8_1 rows], [top-k + plan + gate|up -> h as
-// q8_1 rows (in ws->gu)], [down + the combine's chains -> out]
+// the window's MoE half as one launch (k_moe_window.h): router logits, top-k, gate|up -> h as q8_1 rows (in ws->gu), down with
+// the combine's chains -> out
 // live (may be null): a device word, the rows of the window that count; the others are not routed and their rows of out are left alone
 static int layer_fused(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st, const int* live = nullptr) {
     hipStream_t s = (hipStream_t) st;
@@ -889,7 +890,6 @@ static int layer_fused(const fnx_moe_layer* L, const float* x, int T, float* out
     else if (ff == 512) k_moe_window<16><<<nb, WN_THREADS, 0, s>>>(wa);
     else k_moe_window<32><<<nb, WN_THREADS, 0, s>>>(wa);
     prof_mark(2, s);
-    prof_mark(3, s);
     return launch_status("moe_verify_layer");
 }
 
@@ -1097,12 +1097,12 @@ int fnx_layer_profile(int on) {
     g_prof_on = on != 0;
     return 0;
 }
-int fnx_layer_profile_read(float* ms3) {
-    if (!ms3) return fail("layer_profile_read: null argument");
+int fnx_layer_profile_read(float* ms2) {
+    if (!ms2) return fail("layer_profile_read: null argument");
     if (!g_prof_ev[0]) return fail("layer_profile_read: profiling was never switched on");
-    if (hipEventSynchronize(g_prof_ev[3]) != hipSuccess) return fail("layer_profile_read: no window was recorded");
-    for (int i = 0; i < 3; ++i)
-        if (hipEventElapsedTime(&ms3[i], g_prof_ev[i], g_prof_ev[i + 1]) != hipSuccess) return fail("layer_profile_read: no window was recorded");
+    if (hipEventSynchronize(g_prof_ev[2]) != hipSuccess) return fail("layer_profile_read: no window was recorded");
+    for (int i = 0; i < 2; ++i)
+        if (hipEventElapsedTime(&ms2[i], g_prof_ev[i], g_prof_ev[i + 1]) != hipSuccess) return fail("layer_profile_read: no window was recorded");
     return 0;
 }
 
@@ -1124,7 +1124,7 @@ static int moe_layer_checked(const fnx_moe_layer* L, const float* x, int T, floa
     if (P + T > HQ_ROWS) return fail("moe_verify_layer: more pairs than the pair buffer holds");
     if (!moe_shapes_ok(L)) return fail("moe_verify_layer: weight shapes do not match n / ff");
     if (!out) return fail("moe_verify_layer: null argument");
-    if (live && !layer_fused_ok(L, T)) return fail("moe_verify_layer: a device-side row count needs the three-launch window");
+    if (live && !layer_fused_ok(L, T)) return fail("moe_verify_layer: a device-side row count needs the one-launch window");
     if (layer_fused_ok(L, T)) return layer_fused(L, x, T, out, ws, st, live);
     // operator by operator the pairs' q8_1 rows of h go through the library's pair buffer, rows of ff / 32 blocks
     if (ff <= 0 || ff % 32 || ff > HQ_MAX_FF) return fail("moe_verify_layer: expert width does not fit the pair buffer");
@@ -1176,7 +1176,7 @@ int fnx_moe_verify_layer_static(const fnx_moe_layer* L, const float* x, int T, f
     if (!L || !x || !out) return fail("moe_verify_layer_static: null argument");
     if (T < 1 || T > FNX_MAXT) return fail("moe_verify_layer_static: T out of range");
     if (!layer_fused_ok(L, T))
-        return fail("moe_verify_layer_static: only the three-launch window runs on the library's own workspace (unit64 experts, hidden 2048, "
+        return fail("moe_verify_layer_static: only the one-launch window runs on the library's own workspace (unit64 experts, hidden 2048, "
                     "ff 256 / 512 / 1024, up to 1024 experts, up to 16 picks a row, up to 160 pairs a window)");
     int dev = -1;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return fail("moe_verify_layer_static: no current device");
@@ -1595,7 +1595,7 @@ static int dec_layer(const fnx_decoder* D, const fnx_dec_layer* L, int T, const 
         k_add_norm_q8<false><<<T, 256, 0, (hipStream_t) st>>>(ws->x, ws->o, c, L->ffn_norm, ws->xn, nullptr, n, D->eps);
         if (launch_status("decoder add_norm")) return 1;
     }
-    if (live && !layer_fused_ok(&L->moe, T)) return fail("decoder: a device-side row count needs the three-launch window (unit64 experts, hidden 2048)");
+    if (live && !layer_fused_ok(&L->moe, T)) return fail("decoder: a device-side row count needs the one-launch window (unit64 experts, hidden 2048)");
     // the MoE half's rows (those that count) are added by the next pass over x
     pend = DecPending{ws->o, nullptr, live};
     return moe_layer_checked(&L->moe, ws->xn, T, ws->o, &ws->moe, st, live);
@@ -1992,7 +1992,7 @@ int fnx_gguf_load_moe_layer(const fnx_gguf* g, int layer, int ff0, int ff1, int 
         const bool routed_iq3s = m.ge.type == gguf::T_IQ3_S && m.de.type == gguf::T_IQ3_S;
         const bool shared_iq3s = m.gsh.type == gguf::T_IQ3_S && m.dsh.type == gguf::T_IQ3_S;
         const bool shared_q8 = m.gsh.type == QT_Q8_0 && m.dsh.type == QT_Q8_0;
-        const bool fast = routed_iq3s && (shared_iq3s || shared_q8);   // the three-launch window takes these
+        const bool fast = routed_iq3s && (shared_iq3s || shared_q8);   // the one-launch window takes these
         const auto relay = [&](fnx_dw& w, void* d, size_t n) {
             w.p = d;
             if (!fast) return;   // operator by operator raw blocks do as well

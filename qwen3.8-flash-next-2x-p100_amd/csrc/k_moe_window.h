@@ -11,8 +11,9 @@
 //             then arrives on the row's first counter; the shared expert's gate|up item, which needs no pick, runs
 //             while the row's logits gather.
 //   phase G   every block ranks its row itself (slices of 64 experts a wave, one wave merges) and sweeps its gate|up
-//             items - (32 values of h) x (matrix) - as k_moe_gate_up_h does; a sweep's h leaves as a q8_1 block; the
-//             block arrives on the row's second counter.
+//             items - (32 values of h) x (matrix), sixteen waves x four units (gate rows 2 i, 2 i + 1 and their up rows) a
+//             sweep, the next item's loads asked for before the current one is decoded; a sweep's sums meet in LDS behind
+//             flags and leave as a q8_1 block two sweeps later; the block arrives on the row's second counter.
 //   phase D   the block's units of the down matrices: the first trips' weights are asked for before the wait for the row's
 //             h; then the trips with the combine's fmaf chain in pick order (kernels.cu:412-419).
 //
@@ -87,6 +88,7 @@ struct WinLds {
     int fin;                           // the row's ticket among the rows that have finished
     int lists;                         // 1: every row has been ranked, the job lists can be written; -1: the wait gave up
     uint32_t xq[FL_N / 32][FNX_Q8_1_BLOCK / 4];          // the row's q8_1 blocks
+    float4 xf[FL_N / 4];                                 // the row of x
     __attribute__((aligned(16))) uint32_t hq[FL_MAXK + 1][SBR][HQ_WORDS];   // the row's pairs' h rows (phase D)
 };
 
@@ -114,13 +116,20 @@ __device__ unsigned long long g_win_ts[1024 * WN_WAVES * WIN_NTS];
 #else
 #define WIN_TS(i)
 #endif
+// The block's barrier as the plain instruction, with the wait for this wave's LDS accesses written out: __syncthreads()
+// also waits for every global load in flight, and the down phase meets with its first trips' weights on their way.
+__device__ __forceinline__ void win_meet() {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
 // all of this wave's memory writes have been taken at the device's level before anything after this line
 __device__ __forceinline__ void win_stores_done() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 template <int SBR>
 __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
     __shared__ WinLds<SBR> S;
-    constexpr int RW = 64 / SBR, RMAX = SBR / 8, NB = RMAX == 4 ? 2 : 3;   // rows a unit; units a wave and trip at most; trips' buffers
+    constexpr int RW = 64 / SBR, RMAX = SBR / 8, NB = RMAX == 4 ? 2 : 3, DEPTH = RMAX == 4 ? 1 : 2;   // rows a unit; units a wave and trip at most; trips' buffers
     const int tid = threadIdx.x, wave = uniform(tid >> 6), lane = tid & 63;
     // the codebook's 512 unsigned entries: the launch's first load; the blocks read different signed forms of the table in
     // memory (2 KiB apart) and negate them back, so that not every wave of the grid asks the same sixteen cache lines at once
@@ -141,9 +150,10 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
     // ---------------------------------------------------------------- phase R: loads
     // the row of x as the router's sums take it (lane l: float4 chunks l, l + 64, ...), and the values this wave quantises
     // (blocks 4 wave .. 4 wave + 3 of the row's 64, a half-wave a block)
-    float4 xr[8];
-#pragma unroll
-    for (int c = 0; c < 8; ++c) xr[c] = reinterpret_cast<const float4*>(xrow)[c * 64 + lane];
+    // (a row of x is 512 float4: half the block's threads bring one each into LDS for all sixteen waves; every wave loading
+    // the row itself was 128 KB through the CU's vector cache on top of the router's rows)
+    float4 xmine = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (tid < FL_N / 4) xmine = reinterpret_cast<const float4*>(xrow)[tid];
     float xv[2];
 #pragma unroll
     for (int r = 0; r < 2; ++r) xv[r] = xrow[(4 * wave + 2 * r + (lane >> 5)) * 32 + (lane & 31)];
@@ -166,14 +176,14 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
         }
     };
     // the fixed order of k_gemv_rows (and of the CPU oracle): chunks in order, fmaf over x, y, z, w, then the xor butterfly
-    auto router_dot = [&](const float4(&w)[8]) {
+    auto router_dot = [&](const float4(&w)[8], const float4(&x)[8]) {
         float s = 0.f;
 #pragma unroll
         for (int c = 0; c < 8; ++c) {
-            s = fmaf(w[c].x, xr[c].x, s);
-            s = fmaf(w[c].y, xr[c].y, s);
-            s = fmaf(w[c].z, xr[c].z, s);
-            s = fmaf(w[c].w, xr[c].w, s);
+            s = fmaf(w[c].x, x[c].x, s);
+            s = fmaf(w[c].y, x[c].y, s);
+            s = fmaf(w[c].z, x[c].z, s);
+            s = fmaf(w[c].w, x[c].w, s);
         }
         return group_sum<64>(s);
     };
@@ -195,6 +205,7 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
     }
 #pragma unroll
     for (int i = 0; i < 8; ++i) S.tab[tid + i * WN_THREADS] = signed_entry(tab0, (tid >> 9) + 2 * i);
+    if (tid < FL_N / 4) S.xf[tid] = xmine;
 #pragma unroll
     for (int r = 0; r < 2; ++r) {   // kernels.cu:131-145 (quantize_q8_1), a half-wave a block
         const int b = 4 * wave + 2 * r + (lane >> 5), l32 = lane & 31;
@@ -205,16 +216,20 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
         reinterpret_cast<int8_t*>(&S.xq[b][1])[l32] = qv;
         if (l32 == 0) S.xq[b][0] = (uint32_t) float_to_half_bits(d) | (uint32_t) float_to_half_bits(sum) << 16;
     }
-    __syncthreads();
+    // the block meets with the router's rows still on their way: they were asked for last, after what the lines above wait for
+    win_meet();
     WIN_TS(1);
     if (g == 0 && tid < (FL_N / 32) * (FNX_Q8_1_BLOCK / 4))   // the caller's copy of the row's q8_1 blocks
         reinterpret_cast<uint32_t*>(a.xq + (size_t) t * (FL_N / 32) * FNX_Q8_1_BLOCK)[tid] = (&S.xq[0][0])[tid];
 
     // ---------------------------------------------------------------- phase R: the sums, the arrival
+    float4 xr[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) xr[c] = S.xf[c * 64 + lane];
     {
         int row = r0 + wave;
         while (true) {
-            const float va = router_dot(wa), vb = router_dot(wb);
+            const float va = router_dot(wa, xr), vb = router_dot(wb, xr);
             if (lane == 0) {
                 if (row < r1) __hip_atomic_store(&a.logits[(size_t) t * LS + row], va, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 if (row + WN_WAVES < r1) __hip_atomic_store(&a.logits[(size_t) t * LS + row + WN_WAVES], vb, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -478,6 +493,14 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
             }
         } else if (!issue(ma)) return;
         for (; sw < nsweep; ++sw) {
+            // the oldest wave of a SIMD issues first, so a block's waves drift apart sweep by sweep: every wave takes each of
+            // the four priorities in turn
+            switch ((wave >> 2) + sw & 3) {
+                case 0: __builtin_amdgcn_s_setprio(0); break;
+                case 1: __builtin_amdgcn_s_setprio(1); break;
+                case 2: __builtin_amdgcn_s_setprio(2); break;
+                default: __builtin_amdgcn_s_setprio(3); break;
+            }
             if (!decode(sw)) return;
             WIN_TS(16 + (sw & 15));
             if (sw + 1 < nsweep) {
@@ -493,6 +516,7 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
                 if (!make_block(q)) return;
     }
 
+    __builtin_amdgcn_s_setprio(0);
     WIN_TS(6);
     // ---------------------------------------------------------------- phase D
     const bool ext = a.sh_part != nullptr;   // the shared expert's rows come from memory: the trips are the picks only
@@ -524,16 +548,12 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
             if (lane == 0) __hip_atomic_fetch_add(&srow[1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     WIN_TS(7);
-    if (dwave) {
-        issue_trip(B[0], first);
-        if (first + 1 <= topk) issue_trip(B[1], first + 1);
-    }
     if (wave == 1) {   // the shared expert's gate: the router's last row against the row of x, in the router's order
         float4 wg[8];
         int l2 = lane;
         asm volatile("" : "+v"(l2));   // the addresses are worked out here, not kept in registers since phase R
 #pragma unroll
-        for (int c = 0; c < 8; ++c) xr[c] = reinterpret_cast<const float4*>(xrow)[c * 64 + l2];
+        for (int c = 0; c < 8; ++c) xr[c] = S.xf[c * 64 + l2];
         if (a.router_bf16) {
 #pragma unroll
             for (int c = 0; c < 8; ++c) {
@@ -545,15 +565,25 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
 #pragma unroll
             for (int c = 0; c < 8; ++c) wg[c] = reinterpret_cast<const float4*>(reinterpret_cast<const float*>(a.router) + (size_t) nexp * FL_N)[c * 64 + l2];
         }
-        const float v = router_dot(wg);
+        const float v = router_dot(wg, xr);
         if (lane == 0) {
             S.gate = sigmoid_f(v);
             if (g == 0) a.logits[(size_t) t * LS + nexp] = v;
         }
     }
-    if (wave == 0) {   // the row's h rows: wait for the row's blocks that make them
+    // The row's h rows: wave 0 waits for the row's blocks that make them. A wave's loads return in order, so it asks for its
+    // own first trips' weights only afterwards: the count it waits for is then not queued behind them. The other waves'
+    // first trips are on their way while the row's last blocks finish their sweeps.
+    auto first_trips = [&] {
+#pragma unroll
+        for (int i = 0; i < NB; ++i)
+            if (first + i <= topk) issue_trip(B[i], first + i);
+    };
+    if (dwave && wave != 0) first_trips();
+    if (wave == 0) {
         const bool ok = win_wait_word(&srow[1], (unsigned) pl.nbi, a.wait_ticks, serr);
         if (lane == 0) __hip_atomic_store(&S.hready, ok ? 1 : -1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+        if (dwave) first_trips();
     }
     if (!lds_wait([&] { return uniform(__hip_atomic_load(&S.hready, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP)) != 0; })) return;
     if (uniform(__hip_atomic_load(&S.hready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) < 0) return;
@@ -562,18 +592,18 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
         constexpr int HQ_PER = SBR * HQ_WORDS, HQ_VPT = ((FL_MAXK + 1) * HQ_PER + WN_THREADS - 1) / WN_THREADS;
         uint32_t hw[HQ_VPT];
 #pragma unroll
-        for (int j = 0; j < HQ_VPT; ++j) {
-            const int i = tid + j * WN_THREADS, k = i / HQ_PER;
+        for (int q = 0; q < HQ_VPT; ++q) {
+            const int i = tid + q * WN_THREADS, k = i / HQ_PER;
             const bool has = k < topk || (k == topk && !ext);
-            hw[j] = has ? __hip_atomic_load(&a.hq[(size_t) (k < topk ? t * topk + k : P + t) * HQ_PER + (i - k * HQ_PER)], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+            hw[q] = has ? __hip_atomic_load(&a.hq[(size_t) (k < topk ? t * topk + k : P + t) * HQ_PER + (i - k * HQ_PER)], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
         }
 #pragma unroll
-        for (int j = 0; j < HQ_VPT; ++j) {
-            const int i = tid + j * WN_THREADS;
-            if (i < (topk + 1) * HQ_PER) (&S.hq[0][0][0])[i] = hw[j];
+        for (int q = 0; q < HQ_VPT; ++q) {
+            const int i = tid + q * WN_THREADS;
+            if (i < (topk + 1) * HQ_PER) (&S.hq[0][0][0])[i] = hw[q];
         }
     }
-    __syncthreads();
+    win_meet();
     WIN_TS(9);
     if (dwave) {
         auto pick_of = [&](int trip) { return trip == 0 ? topk : trip - 1; };   // the index of a trip's expert in S.hq
@@ -582,6 +612,12 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
         for (int r = 0; r < RMAX; ++r) acc[r] = zs[r] = 0.f;
         const float gate = S.gate;
         auto decode_trip = [&](const PackedSub(&buf)[RMAX], int trip) {
+            switch ((wave >> 2) + trip & 3) {   // every wave takes each of the four priorities in turn (see the sweeps)
+                case 0: __builtin_amdgcn_s_setprio(0); break;
+                case 1: __builtin_amdgcn_s_setprio(1); break;
+                case 2: __builtin_amdgcn_s_setprio(2); break;
+                default: __builtin_amdgcn_s_setprio(3); break;
+            }
             const int k = pick_of(trip);
             const uint32_t* hb = S.hq[k][kb];
             const uint4 lo = *reinterpret_cast<const uint4*>(hb), hi = *reinterpret_cast<const uint4*>(hb + 4);
@@ -604,26 +640,17 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
                     else acc[r] = fmaf(gk, z, acc[r]);
                 }
         };
-        if constexpr (NB == 3) {   // two trips' loads in flight while a third is decoded
-            for (int trip = first; trip <= topk; trip += 3) {
-                if (trip + 2 <= topk) issue_trip(B[2], trip + 2);
-                decode_trip(B[0], trip);
-                if (trip + 1 > topk) break;
-                if (trip + 3 <= topk) issue_trip(B[0], trip + 3);
-                decode_trip(B[1], trip + 1);
-                if (trip + 2 > topk) break;
-                if (trip + 4 <= topk) issue_trip(B[1], trip + 4);
-                decode_trip(B[2], trip + 2);
-            }
-        } else {   // four units a trip: one trip's loads in flight while another is decoded
-            for (int trip = first; trip <= topk; trip += 2) {
-                decode_trip(B[0], trip);
-                if (trip + 1 > topk) break;
-                if (trip + 2 <= topk) issue_trip(B[0], trip + 2);
-                decode_trip(B[1], trip + 1);
-                if (trip + 3 <= topk) issue_trip(B[1], trip + 3);
+        for (int trip = first; trip <= topk; trip += NB) {
+#pragma unroll
+            for (int i = 0; i < NB; ++i) {
+                const int tr = trip + i;
+                if (tr > topk) break;
+                decode_trip(B[i], tr);
+                const int nx = tr + DEPTH;   // the buffer it goes to held trip nx - NB, decoded before this one
+                if (nx >= first + NB && nx <= topk) issue_trip(B[(i + DEPTH) % NB], nx);
             }
         }
+        __builtin_amdgcn_s_setprio(0);
         if (kb == SBR - 1) {   // the combine's last step: s + sigmoid * shared
             float* orow = a.out + (size_t) t * a.rows + (size_t) u0 * RW + gl;
 #pragma unroll

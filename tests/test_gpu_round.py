@@ -1,7 +1,7 @@
 """Whole greedy decode rounds enqueued without the host in between (fnx_decode_round: verify -> accept -> commit -> draft
 -> prompt lookup -> next window, the state in device words) against the host-driven round of tests/tiny_decoder.py
 (session.cpp:530-679: the host waits for every step) on the device and on the CPU oracle, at hidden 2048 with unit64
-experts (the three-launch window).
+experts (the one-launch window).
 
 Bar: emitted tokens, drafts offered and tokens kept per round identical to the host-driven device loop (the same kernels
 on the same rows: rows past the window's count are neither routed nor accepted); against the oracle: identical up to a
@@ -86,7 +86,7 @@ def host_loop(dev, model, prompt, max_new, speculate=True, K=1, lk=15):
 
 
 def test_verify_window_at_hidden_2048_matches_oracle(dev, oracle, model):
-    # the decoder over the three-launch window, which the rounds below use
+    # the decoder over the one-launch window, which the rounds below use
     o, d = td.OracleSession(model), fnx_gpu.DecoderDev(dev, model)
     pos = 0
     for toks in ([3, 1, 4, 1, 5, 9, 2, 6, 5, 3, 5, 8, 9, 7, 9, 3], [2, 7, 18], [281]):

@@ -37,5 +37,5 @@ def test_static_workspace_window_equals_the_workspace_one():
     x = dev.up(rng.standard_normal((4, n)).astype(np.float32))
     out = dev.zeros((4, n), dev.torch.float32)
     assert dev.lib.fnx_moe_verify_layer_static(C.byref(raw.L), x.data_ptr(), 4, out.data_ptr(), dev.st()) != 0
-    assert b"three-launch window" in dev.lib.fnx_last_error()
+    assert b"one-launch window" in dev.lib.fnx_last_error()
     assert dev.lib.fnx_moe_verify_layer_static(C.byref(layer.L), x.data_ptr(), 17, out.data_ptr(), dev.st()) != 0
