@@ -357,6 +357,12 @@ typedef struct fnx_dec_ws {
 /* engine.cu (Engine::enqueue, reduced): the window's rows through every layer, the output norm, the head and argmax:
  * ws->hidden, ws->logits, ws->best_i. tokens: device, T ids; their K/V go to positions *pos0 + t. */
 int fnx_decoder_verify(const fnx_decoder* D, const int* tokens, int T, const int* pos0, const fnx_dec_ws* ws, void* st);
+/* engine.cu (Engine::enqueue): the body of its layer loop, one layer on rows the caller gives (x: device, [T][n]; L: one of D's
+ * layers or the draft layer's). Leaves in the workspace what the layer loop hands on: ws->x = x + the attention half's
+ * rows, ws->xq = the attention's rows in q8_1 form (what the output projection read), ws->xn = the normed rows the MoE
+ * half read, ws->o = the MoE half's rows (the next layer's first pass adds them); the layer's K and V rows go into its
+ * caches at *pos0 + t. For callers that drive the layers themselves, and for layer-by-layer comparisons. */
+int fnx_decoder_layer(const fnx_decoder* D, const fnx_dec_layer* L, const float* x, int T, const int* pos0, const fnx_dec_ws* ws, void* st);
 /* engine.cu:2095-2133 (mtp_enqueue, without hyper-connection streams): R = fc_hid(rms(src)) + fc_emb(rms(emb[tokens])),
  * one decoder layer (its own cache), the output norm, the head, argmax. src: [T][n] hidden rows (the verify's, or the
  * draft layer's own for a chain). ws->hidden receives the layer's output rows. */

@@ -10,6 +10,7 @@
 #include <omp.h>
 #endif
 
+#include "../include/fnx_expf.h" /* the one exp both sides use, fixed operation by operation */
 #include "iq3s_grid.h"
 
 #define IQ3S_BLOCK 110
@@ -353,6 +354,10 @@ void fnx_o_gemv_bf16(const uint16_t* W, const float* x, float* y, int rows, int 
         for (int t = 0; t < T; ++t) y[(size_t) t * rows + r] = dot64(NULL, W + (size_t) r * n, x + (size_t) t * n, n);
 }
 
+void fnx_o_expf(const float* x, size_t n, float* y) {
+    for (size_t i = 0; i < n; ++i) y[i] = fnx_expf(x[i]);
+}
+
 /* ---------------------------------------------------------------- routing */
 void fnx_o_topk_logits(const float* logits, int stride, int T, int nexp, int topk, int* topi, float* topw) {
     unsigned char* taken = (unsigned char*) malloc((size_t) nexp);
@@ -377,7 +382,7 @@ void fnx_o_topk_logits(const float* logits, int stride, int T, int nexp, int top
                     }
             if (bi < nexp) taken[bi] = 1;
             if (k == 0) top0 = bv;
-            e[k] = found ? expf(bv - top0) : 0.f;
+            e[k] = found ? fnx_expf(bv - top0) : 0.f;
             z += e[k];
             topi[t * topk + k] = bi < nexp ? bi : nexp - 1;
         }
@@ -392,7 +397,7 @@ void fnx_o_topk_softmax(const float* logits, int stride, int T, int nexp, int to
         float m = -INFINITY, z = 0.f;
         for (int i = 0; i < nexp; ++i) m = fmaxf(m, l[i]);
         for (int i = 0; i < nexp; ++i) {
-            p[i] = expf(l[i] - m);
+            p[i] = fnx_expf(l[i] - m);
             z += p[i];
         }
         for (int i = 0; i < nexp; ++i) p[i] = p[i] / z;
@@ -439,8 +444,10 @@ int fnx_o_jobs(const int* topi, int T, int topk, fnx_o_job* gu, fnx_o_job* dn) {
 }
 
 /* ---------------------------------------------------------------- swiglu, combine (kernels.cu:67-68, 400-419) */
-static float sigm(float x) { return 1.0f / (1.0f + expf(-x)); }
-static float silu(float x) { return x / (1.0f + expf(-x)); }
+/* kernels.cu:67-68, with exp as include/fnx_expf.h fixes it (the reference's __expf is the CUDA toolkit's: its bits cannot be
+ * restated; any exp within a few units in the last place is "the reference's" to the tolerance its own tests use) */
+static float sigm(float x) { return 1.0f / (1.0f + fnx_expf(-x)); }
+static float silu(float x) { return x / (1.0f + fnx_expf(-x)); }
 void fnx_o_swiglu_q8_1(const float* g, const float* u, uint8_t* q, int n, int rows) {
     float h[32];
     for (int r = 0; r < rows; ++r)
@@ -1173,6 +1180,22 @@ void fnx_o_layer_probe(float* logits, int* topi, int layers) {
     g_probe_left = logits && topi ? layers : 0;
     g_probe_at = 0;
 }
+/* what a test may ask a layer for besides x: the rows as they go into the layer (x_in), the attention's rows before the output
+ * projection (att: [T][nq * 256], the rows whose q8_1 form feeds wo), x after the attention half (x_mid), the MoE half's
+ * rows (moe); any of them may be null. The probe below sets the same for the layers of a whole window. */
+typedef struct layer_taps {
+    float *x_in, *att, *x_mid, *moe;
+} layer_taps;
+static layer_taps g_taps; /* per layer: slot g_taps_at of each array */
+static int g_taps_left, g_taps_at;
+void fnx_o_layer_taps(float* x_in, float* att, float* x_mid, float* moe, int layers) {
+    g_taps.x_in = x_in;
+    g_taps.att = att;
+    g_taps.x_mid = x_mid;
+    g_taps.moe = moe;
+    g_taps_left = layers;
+    g_taps_at = 0;
+}
 static void dec_layer(const fnx_o_decoder* D, const fnx_o_dec_layer* L, float* x, int T, int pos0, int threads) {
     const int n = D->n, nq = D->nq, nkv = D->nkv, hd = 256, nrot = 64;
     float* probe_l = NULL;
@@ -1183,24 +1206,42 @@ static void dec_layer(const fnx_o_decoder* D, const fnx_o_dec_layer* L, float* x
         --g_probe_left;
         ++g_probe_at;
     }
+    layer_taps tap = {NULL, NULL, NULL, NULL};
+    if (g_taps_left > 0) {
+        const size_t at = (size_t) g_taps_at * T;
+        if (g_taps.x_in) tap.x_in = g_taps.x_in + at * n;
+        if (g_taps.att) tap.att = g_taps.att + at * nq * hd;
+        if (g_taps.x_mid) tap.x_mid = g_taps.x_mid + at * n;
+        if (g_taps.moe) tap.moe = g_taps.moe + at * n;
+        --g_taps_left;
+        ++g_taps_at;
+    }
     float* xn = (float*) malloc((size_t) T * n * sizeof(float));
     float* qg = (float*) malloc((size_t) T * nq * 2 * hd * sizeof(float));
     float* k = (float*) malloc((size_t) T * nkv * hd * sizeof(float));
     float* v = (float*) malloc((size_t) T * nkv * hd * sizeof(float));
     float* att = (float*) malloc((size_t) T * nq * hd * sizeof(float));
     float* o = (float*) malloc((size_t) T * n * sizeof(float));
+    if (tap.x_in) memcpy(tap.x_in, x, (size_t) T * n * sizeof(float));
     fnx_o_rms_norm_rows(x, L->attn_norm, xn, T, n, D->eps);
     dense_q8s(&L->wq, xn, T, qg);
     dense_q8s(&L->wk, xn, T, k);
     dense_q8s(&L->wv, xn, T, v);
     fnx_o_attn_prep_append(qg, k, v, L->q_norm, L->k_norm, L->kc, L->vc, nq, nkv, hd, nrot, T, pos0, D->eps, &D->rope);
     fnx_o_attn(qg, L->kc, L->vc, att, nq, nkv, hd, T, pos0);
+    if (tap.att) memcpy(tap.att, att, (size_t) T * nq * hd * sizeof(float));
     dense_q8s(&L->wo, att, T, o);
     for (size_t i = 0; i < (size_t) T * n; ++i) x[i] += o[i];
+    if (tap.x_mid) memcpy(tap.x_mid, x, (size_t) T * n * sizeof(float));
     fnx_o_rms_norm_rows(x, L->ffn_norm, xn, T, n, D->eps);
     fnx_o_moe_verify_layer(&L->moe, xn, T, o, probe_l, probe_i, NULL, NULL, threads);
+    if (tap.moe) memcpy(tap.moe, o, (size_t) T * n * sizeof(float));
     for (size_t i = 0; i < (size_t) T * n; ++i) x[i] += o[i];
     free(xn); free(qg); free(k); free(v); free(att); free(o);
+}
+/* one layer on rows given by the caller (engine.cu's layer loop body): x in place; the layer's K and V go into its cache */
+void fnx_o_decoder_layer(const fnx_o_decoder* D, const fnx_o_dec_layer* L, float* x, int T, int pos0, int threads) {
+    dec_layer(D, L, x, T, pos0, threads);
 }
 static void dec_head(const fnx_o_decoder* D, const float* norm, const fnx_o_q8s* head, const float* x, int T, float* logits_out, int* best) {
     float* xn = (float*) malloc((size_t) T * D->n * sizeof(float));

@@ -59,6 +59,9 @@ uint16_t fnx_o_f2h_rn(float x);
 
 /* p100_compat.h:18-22 (the scalar definition of the 4-way signed byte dot) */
 int fnx_o_dp4a(int a, int b, int c);
+/* exp as include/fnx_expf.h fixes it (the one exp behind sigm, silu_ and the routing weights on both sides) over n values;
+ * pinned against numpy's float64 exp in tests/test_oracle_routing.py */
+void fnx_o_expf(const float* x, size_t n, float* y);
 
 /* IQ3_S: 110-byte blocks of 256 weights. tensor_convert.hpp:295-322 */
 void fnx_o_iq3s_dequant(const uint8_t* src, size_t n, float* y);
@@ -219,6 +222,13 @@ typedef struct {
 /* test probe: the next `layers` decoder layers run (by either function below) copy their router logits [T][nexp + 1] and
  * picks [T][topk] into consecutive slots of the two arrays; null pointers switch it off */
 void fnx_o_layer_probe(float* logits, int* topi, int layers);
+/* the next `layers` layers copy, to slot 0, 1, ... of the arrays given (any may be null): the rows going into the layer
+ * [T][n], the attention's rows before the output projection [T][nq * 256], the rows after the attention half [T][n], the
+ * MoE half's rows [T][n]. layers = 0 switches it off */
+void fnx_o_layer_taps(float* x_in, float* att, float* x_mid, float* moe, int layers);
+/* one layer (engine.cu: the body of the layer loop, attention half then MoE half) on the caller's rows, in place; L may be
+ * one of D's layers or the draft layer's */
+void fnx_o_decoder_layer(const fnx_o_decoder* D, const fnx_o_dec_layer* L, float* x, int T, int pos0, int threads);
 void fnx_o_decoder_verify(const fnx_o_decoder* D, const int* tokens, int T, int pos0, float* hidden, float* logits, int* best, int threads);
 /* engine.cu:2095-2133 without streams: R = fc_hid(rms(src)) + fc_emb(rms(emb[tokens])), one layer, norm, head, argmax */
 void fnx_o_mtp_draft(const fnx_o_decoder* D, const fnx_o_mtp* M, const float* src, const int* tokens, int T, int pos0, float* hidden,

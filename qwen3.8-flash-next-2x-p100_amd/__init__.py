@@ -152,6 +152,7 @@ EXPORTS = {
     "fnx_attn": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p,
                            C.c_void_p]),
     "fnx_decoder_verify": (C.c_int, [C.POINTER(Decoder), C.c_void_p, C.c_int, C.c_void_p, C.POINTER(DecWs), C.c_void_p]),
+    "fnx_decoder_layer": (C.c_int, [C.POINTER(Decoder), C.POINTER(DecLayer), C.c_void_p, C.c_int, C.c_void_p, C.POINTER(DecWs), C.c_void_p]),
     "fnx_mtp_draft": (C.c_int, [C.POINTER(Decoder), C.POINTER(Mtp), C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.POINTER(DecWs), C.c_void_p]),
     "fnx_decode_round": (C.c_int, [C.POINTER(Decoder), C.POINTER(Mtp), C.POINTER(Round), C.POINTER(DecWs), C.c_void_p]),
     "fnx_top_tokens": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p,

@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "../../include/fnx_expf.h"
 #include "iq3s_grid.h"
 
 namespace fnx {
@@ -63,8 +64,43 @@ __device__ __forceinline__ float group_max(float v) {
     return v;
 }
 
-__device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
-__device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x)); }
+// kernels.cu:67-68 (sigm, silu_) over this library's exp (include/fnx_expf.h: fixed operation by operation, the CPU oracle
+// includes the same lines), so that the q8_1 codes of h and the combine's gate come out bit for bit on both sides
+__device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + fnx_expf(-x)); }
+__device__ __forceinline__ float silu_f(float x) { return x / (1.0f + fnx_expf(-x)); }
+
+// Sums over a weight row's lanes in the reference's order: lane l holds the terms of sub-block l of the row (for rows of 64
+// sub-blocks: l and l + 32 are the two super-blocks a lane of the reference's 32 takes, kernels.cu:209-228, moe.cuh:664-670),
+// and the lanes' sums meet in an xor butterfly width / 2, ..., 2, 1. Every add is of two partners' values, so it commutes:
+// every lane of a group ends with the same bits, and they are the CPU oracle's.
+// (The swaps are written as inline asm: with this toolchain the two results of the __builtin_amdgcn_permlane*_swap builtins
+// were folded into one register when both fed the same add. The s_nop covers the VALU-write -> swap-read wait states.)
+__device__ __forceinline__ float swap32_add(float x, float y) {   // lanes 0..31: x[l] + x[l + 32]; lanes 32..63: y[l - 32] + y[l]
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(x), "+v"(y));
+    return x + y;
+}
+__device__ __forceinline__ float swap16_add(float x, float y) {   // 16-lane rows 0, 2: x's rows 0 + 1, 2 + 3; rows 1, 3: y's
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(x), "+v"(y));
+    return x + y;
+}
+template <int width>
+__device__ __forceinline__ float butterfly_sum(float v) {
+#define FNX_DPP_ADD(ctrl) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, 0xF, 0xF, false))
+    if constexpr (width >= 64) v = swap32_add(v, v);   // l ^ 32
+    if constexpr (width >= 32) v = swap16_add(v, v);   // l ^ 16
+    if constexpr (width >= 16) FNX_DPP_ADD(0x128);     // row_ror:8 = l ^ 8
+    if constexpr (width >= 16) {
+        FNX_DPP_ADD(0x124);   // row_ror:4: after the step before lanes l and l ^ 8 hold the same value, so lane (l + 4) mod 16 holds lane l ^ 4's
+    } else if constexpr (width >= 8) {   // l ^ 4 without that symmetry: lanes 0-3 and 8-11 of a row look four up, the others four down
+        int t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x104, 0xF, 0x5, false);    // row_shl:4 into banks 0 and 2
+        t = __builtin_amdgcn_update_dpp(t, __builtin_bit_cast(int, v), 0x114, 0xF, 0xA, false);        // row_shr:4 into banks 1 and 3
+        v += __builtin_bit_cast(float, t);
+    }
+    if constexpr (width >= 4) FNX_DPP_ADD(0x4E);   // quad_perm [2,3,0,1] = l ^ 2
+    if constexpr (width >= 2) FNX_DPP_ADD(0xB1);   // quad_perm [1,0,3,2] = l ^ 1
+#undef FNX_DPP_ADD
+    return v;
+}
 
 // A value every lane of the wave holds alike, moved to a scalar register: what is computed from it (addresses, loop
 // bounds) then runs on the scalar unit. Loads from memory the kernel may also write are vector loads even at a uniform

@@ -192,7 +192,7 @@ __global__ void __launch_bounds__(TK_THREADS) k_topk_jobs(const float* __restric
             }
             if (bi < nexp && (bi & 63) == lane) taken |= 1u << (bi >> 6);
             if (k == 0) top0 = bv;
-            const float ek = found ? expf(bv - top0) : 0.f;
+            const float ek = found ? fnx_expf(bv - top0) : 0.f;
             z += ek;
             if (lane == k) {
                 wk = ek;
@@ -373,7 +373,7 @@ __device__ __forceinline__ void job_units(const uint32_t* __restrict__ tab, cons
 #pragma unroll
                 for (int j = 0; j < 8; ++j) sum = __builtin_amdgcn_sdot4(w4[j], xs[t][j], sum, false);
                 // one sub-block's term exactly as the reference forms it: (d_w * d_x) * (float) (sumi * (1 + 2 s))
-                const float v = dpp_group_sum<SBR>((dw * dx[t]) * (float) __mul24(sum, sc));
+                const float v = butterfly_sum<SBR>((dw * dx[t]) * (float) __mul24(sum, sc));
                 if (store) orow[t][(size_t) (u + r) * RW] = v;
             }
         }
@@ -1624,6 +1624,14 @@ static int decoder_verify(const fnx_decoder* D, const int* tokens, int T, const 
 }
 int fnx_decoder_verify(const fnx_decoder* D, const int* tokens, int T, const int* pos0, const fnx_dec_ws* ws, void* st) {
     return decoder_verify(D, tokens, T, pos0, ws, st, nullptr);
+}
+int fnx_decoder_layer(const fnx_decoder* D, const fnx_dec_layer* L, const float* x, int T, const int* pos0, const fnx_dec_ws* ws, void* st) {
+    if (!D || !L || !x || !pos0 || !ws) return fail("decoder_layer: null argument");
+    if (dec_shape_check(D, T, "decoder_layer") || dec_ws_check(ws, "decoder_layer")) return 1;
+    if (hipMemcpyAsync(ws->x, x, (size_t) T * D->n * sizeof(float), hipMemcpyDeviceToDevice, (hipStream_t) st) != hipSuccess)
+        return fail("decoder_layer: copy of the rows failed");
+    DecPending pend{nullptr, nullptr, nullptr};   // nothing is still to be added to the rows
+    return dec_layer(D, L, T, pos0, ws, pend, st);
 }
 static int mtp_draft(const fnx_decoder* D, const fnx_mtp* M, const float* src, const int* tokens, int T, const int* pos0, const fnx_dec_ws* ws,
                      void* st, const int* live, const int* gate = nullptr) {

@@ -88,22 +88,12 @@ __device__ __forceinline__ uint32_t packed_addr(const v4u& q, int j) {
     return v & 0x7FFCu;
 }
 
-// four per-lane partial sums (one per unit) -> each unit's total over the 64 lanes. On return every lane of 16-lane
-// row 0 holds a's total, row 1 c's, row 2 b's, row 3 d's. Ten VALU ops instead of four six-step reductions.
-// (The swaps are written as inline asm: with this toolchain the two results of the __builtin_amdgcn_permlane*_swap
-// builtins were folded into one register when both fed the same add. The s_nop covers the VALU-write -> swap-read
-// wait states the compiler would otherwise insert itself.)
-__device__ __forceinline__ float swap32_add(float x, float y) {   // lanes 0..31: x over both halves; 32..63: y
-    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(x), "+v"(y));
-    return x + y;
-}
-__device__ __forceinline__ float swap16_add(float x, float y) {   // rows 0, 2: x's row pairs; rows 1, 3: y's
-    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(x), "+v"(y));
-    return x + y;
-}
+// four per-lane partial sums (one per unit, a unit a row of 64 sub-blocks) -> each unit's total over the 64 lanes, in
+// butterfly_sum<64>'s order (l ^ 32, l ^ 16, then 8, 4, 2, 1) with the first two steps of the four units done together. On
+// return every lane of 16-lane row 0 holds a's total, row 1 c's, row 2 b's, row 3 d's.
 __device__ __forceinline__ float reduce4_units(float a, float b, float c, float d) {
     const float p = swap32_add(a, b), q = swap32_add(c, d);
-    return dpp_group_sum<16>(swap16_add(p, q));   // rows: a, c, b, d
+    return butterfly_sum<16>(swap16_add(p, q));   // rows: a, c, b, d
 }
 // which of the four units a lane's 16-lane row holds after reduce4_units
 __device__ __forceinline__ int reduce4_unit_of_row(int row) { return ((row & 1) << 1) | (row >> 1); }
@@ -167,7 +157,7 @@ __device__ __forceinline__ void packed_units(const uint32_t* __restrict__ tab, c
             for (int r = 0; r < R; ++r)
 #pragma unroll
                 for (int t = 0; t < NT; ++t) {
-                    const float z = dpp_group_sum<SBR>(v[r][t]);
+                    const float z = butterfly_sum<SBR>(v[r][t]);
                     if (kb == SBR - 1 && u + r < ub) orow[t][(size_t) (u + r) * RW + g] = z;
                 }
         }

@@ -106,7 +106,7 @@ __device__ __forceinline__ void wave_topk(const float* __restrict__ row, int nex
             if (mine && (mi >> 6) == i) v[i] = -INFINITY;
         if (mine) taken |= 1u << (mi >> 6);
         if (k == 0) top0 = m;
-        const float ek = found ? expf(m - top0) : 0.f;
+        const float ek = found ? fnx_expf(m - top0) : 0.f;
         z += ek;
         if (lane == k) {
             wk = ek;

@@ -457,14 +457,15 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
             }
         }
         const float top0 = rank_key_inv((unsigned) __builtin_amdgcn_readlane((int) mk, 0));
-        const float ek = expf(rank_key_inv(mk) - top0);
+        const float ek = mk > RANK_KEY_NEG_INF ? fnx_expf(rank_key_inv(mk) - top0) : 0.f;   // a pick without a finite logit weighs nothing
         float z = 0.f;
         for (int k = 0; k < topk; ++k) z += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, ek), k));
-        if (lane < topk) S.pw[lane] = ek / z;
+        const float wk = z > 0.f ? ek / z : 0.f;
+        if (lane < topk) S.pw[lane] = wk;
         if (publish) {
             if (lane < topk) {
                 __hip_atomic_store(&a.topi[t * topk + lane], ei, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                __hip_atomic_store(&a.topw[t * topk + lane], ek / z, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(&a.topw[t * topk + lane], wk, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
             win_stores_done();
             if (lane == 0) __hip_atomic_fetch_add(&a.sync[WS_ROUTED], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -635,7 +636,7 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
                     int sum = 0;
 #pragma unroll
                     for (int j = 0; j < 8; ++j) sum = __builtin_amdgcn_sdot4(w4[j], hx[j], sum, false);
-                    const float z = dpp_group_sum<SBR>((dw * dh) * (float) __mul24(sum, sc));
+                    const float z = butterfly_sum<SBR>((dw * dh) * (float) __mul24(sum, sc));
                     if (trip == 0) zs[r] = gk * z;
                     else acc[r] = fmaf(gk, z, acc[r]);
                 }

@@ -473,6 +473,39 @@ class DecoderDev:
         dev.sync()
         return self._result(len(tokens))
 
+    def layer(self, x, l, pos0):
+        """one layer (l: its number, or -1 for the draft layer's) on the rows x [T][n]: what fnx_decoder_layer leaves in the
+        workspace - the rows after the attention half, the attention's rows in q8_1 form (what the output projection read),
+        the MoE half's rows - and the router's picks"""
+        dev = self.dev
+        T = x.shape[0]
+        dx = dev.up(np.ascontiguousarray(x, dtype=np.float32))
+        self.pos.fill_(pos0)
+        L = self.M.layer if l < 0 else self.layer_arr[l]
+        dev.ok(dev.lib.fnx_decoder_layer(C.byref(self.D), C.byref(L), dx.data_ptr(), T, self.pos.data_ptr(), C.byref(self.ws), dev.st()))
+        dev.sync()
+        nb = self.c["nq"] * 256 // 32
+        return dict(x_mid=self.b["x"].cpu().numpy()[:T], moe=self.b["o"].cpu().numpy()[:T],
+                    att_q8=self.b["xq"].cpu().numpy().reshape(-1)[:T * nb * 36].reshape(T, nb, 36).copy(),
+                    topi=self.mb["topi"].cpu().numpy()[:T], err=int(self.b["err"].item()))
+
+    def moe_half(self, x_mid, l, normed=None):
+        """the MoE half of layer l (-1: the draft layer's) on the rows x_mid: the norm, then the window. With normed
+        rows given the window runs on those instead of the device's own norm of x_mid. Returns (normed rows, output)."""
+        dev = self.dev
+        T, n = x_mid.shape
+        L = self.M.layer if l < 0 else self.layer_arr[l]
+        out = dev.zeros((T, n), dev.torch.float32)
+        if normed is None:
+            dx = dev.up(np.ascontiguousarray(x_mid, dtype=np.float32))
+            xn = dev.zeros((T, n), dev.torch.float32)
+            dev.ok(dev.lib.fnx_rms_norm_rows(dx.data_ptr(), L.ffn_norm, xn.data_ptr(), T, n, self.c["eps"], dev.st()))
+        else:
+            xn = dev.up(np.ascontiguousarray(normed, dtype=np.float32))
+        dev.ok(dev.lib.fnx_moe_verify_layer(C.byref(L.moe), xn.data_ptr(), T, out.data_ptr(), C.byref(self.ws.moe), dev.st()))
+        dev.sync()
+        return xn.cpu().numpy(), out.cpu().numpy()
+
     def routing(self, T):
         """the router logits and picks the last MoE layer run left in the workspace"""
         return self.mb["logits"].cpu().numpy()[:T], self.mb["topi"].cpu().numpy()[:T]

@@ -43,6 +43,7 @@ def load():
         "fnx_o_f2h": (C.c_uint16, [f]),
         "fnx_o_f2h_rn": (C.c_uint16, [f]),
         "fnx_o_dp4a": (i, [i, i, i]),
+        "fnx_o_expf": (None, [vp, C.c_size_t, vp]),
         "fnx_o_iq3s_dequant": (None, [vp, sz, vp]),
         "fnx_o_iq3s_quantize": (None, [vp, sz, vp]),
         "fnx_o_quantize_q8_1": (None, [vp, vp, i, i]),
@@ -143,6 +144,12 @@ class Oracle:
         assert w.size % 256 == 0
         out = np.zeros(w.size // 256 * IQ3S_BLOCK, dtype=np.uint8)
         self.lib.fnx_o_iq3s_quantize(ptr(w), w.size, ptr(out))
+        return out
+
+    def expf(self, x):
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        out = np.empty_like(x)
+        self.lib.fnx_o_expf(ptr(x), x.size, ptr(out))
         return out
 
     def iq3s_dequant(self, blocks):

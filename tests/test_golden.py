@@ -42,7 +42,7 @@ def test_device_reproduces_the_fixtures():
         y = dev.gemv_iq3s(G["w64x512"], 64, 512, G["x3"], packed=packed)
         assert np.linalg.norm(y - G["y3"]) <= 1e-5 * np.linalg.norm(G["y3"])
     r = dev.route(G["logits"], 512, 10)
-    assert np.array_equal(r["topi"], G["topi"]) and np.allclose(r["topw"], G["topw"], rtol=2e-6, atol=0)
+    assert np.array_equal(r["topi"], G["topi"]) and np.array_equal(r["topw"].view(np.uint32), G["topw"].view(np.uint32))
     want = np.ascontiguousarray(G["jobs_gu"]).reshape(-1).view(JOB_DTYPE)
     assert len(r["gu"]) == len(want)
     for g, w in zip(r["gu"], want):

@@ -121,7 +121,7 @@ def test_route_bit_exact(dev, oracle, T, nexp, topk):
     r = dev.route(logits, nexp, topk)
     topi, topw = oracle.topk_logits(logits, nexp, topk)
     assert np.array_equal(r["topi"], topi)
-    assert np.allclose(r["topw"], topw, rtol=2e-6, atol=0)
+    assert np.array_equal(r["topw"].view(np.uint32), topw.view(np.uint32))
     gu, dn = oracle.jobs(topi)
     check_jobs(r["gu"], gu)
     check_jobs(r["dn"], dn)
@@ -141,7 +141,7 @@ def test_route_with_fewer_finite_logits_than_picks(dev, oracle, T, nexp, topk):
     for t in range(T):
         assert len(set(r["topi"][t].tolist())) == topk
     assert np.array_equal(np.isfinite(r["topw"]), np.ones_like(topw, dtype=bool))
-    assert np.allclose(r["topw"], topw, rtol=2e-6, atol=0)
+    assert np.array_equal(r["topw"].view(np.uint32), topw.view(np.uint32))
     gu, dn = oracle.jobs(topi)
     check_jobs(r["gu"], gu)
     check_jobs(r["dn"], dn)
@@ -158,7 +158,7 @@ def test_router_route_fused_bit_exact(dev, oracle):
     assert np.array_equal(r["logits"].view(np.uint32), logits.view(np.uint32))
     topi, topw = oracle.topk_logits(logits, nexp, topk)
     assert np.array_equal(r["topi"], topi)
-    assert np.allclose(r["topw"], topw, rtol=2e-6, atol=0)
+    assert np.array_equal(r["topw"].view(np.uint32), topw.view(np.uint32))
     gu, dn = oracle.jobs(topi)
     check_jobs(r["gu"], gu)
     check_jobs(r["dn"], dn)

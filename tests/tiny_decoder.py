@@ -143,6 +143,10 @@ class OracleSession:
         lib.fnx_o_mtp_draft.restype = None
         lib.fnx_o_layer_probe.argtypes = [C.c_void_p, C.c_void_p, C.c_int]
         lib.fnx_o_layer_probe.restype = None
+        lib.fnx_o_layer_taps.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]
+        lib.fnx_o_layer_taps.restype = None
+        lib.fnx_o_decoder_layer.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int]
+        lib.fnx_o_decoder_layer.restype = None
 
     def _probe(self, T, layers):
         c = self.m.cfg
@@ -150,8 +154,18 @@ class OracleSession:
         self.m.oracle.lib.fnx_o_layer_probe(ol.ptr(lg), ol.ptr(ti), layers)
         return lg, ti
 
-    def verify(self, tokens, pos0, routing=False):
-        """routing: also every layer's router logits [layer][T][nexp + 1] and picks [layer][T][topk]"""
+    def _taps(self, T, layers):
+        """arrays the next `layers` layers fill: the rows going in, the attention's rows before the output projection, the rows
+        after the attention half, the MoE half's rows"""
+        c = self.m.cfg
+        t = dict(x_in=np.zeros((layers, T, c["n"]), dtype=np.float32), att=np.zeros((layers, T, c["nq"] * HD), dtype=np.float32),
+                 x_mid=np.zeros((layers, T, c["n"]), dtype=np.float32), moe=np.zeros((layers, T, c["n"]), dtype=np.float32))
+        self.m.oracle.lib.fnx_o_layer_taps(ol.ptr(t["x_in"]), ol.ptr(t["att"]), ol.ptr(t["x_mid"]), ol.ptr(t["moe"]), layers)
+        return t
+
+    def verify(self, tokens, pos0, routing=False, taps=False):
+        """routing: also every layer's router logits [layer][T][nexp + 1] and picks [layer][T][topk]; taps: also every layer's
+        rows on their way through it (see _taps)"""
         c = self.m.cfg
         tok = np.ascontiguousarray(tokens, dtype=np.int32)
         T = len(tok)
@@ -159,12 +173,29 @@ class OracleSession:
         logits = np.zeros((T, c["vocab"]), dtype=np.float32)
         best = np.zeros(T, dtype=np.int32)
         probe = self._probe(T, c["nlayers"]) if routing else None
+        tp = self._taps(T, c["nlayers"]) if taps else None
         self.m.oracle.lib.fnx_o_decoder_verify(C.byref(self.D), ol.ptr(tok), T, pos0, ol.ptr(hidden), ol.ptr(logits), ol.ptr(best), self.threads)
         self.m.oracle.lib.fnx_o_layer_probe(None, None, 0)
+        self.m.oracle.lib.fnx_o_layer_taps(None, None, None, None, 0)
         r = dict(hidden=hidden, logits=logits, best=best)
         if routing:
             r["route_logits"], r["route_topi"] = probe
+        if taps:
+            r["taps"] = tp
         return r
+
+    def layer(self, x, l, pos0):
+        """one layer (l: its number, or -1 for the draft layer's) on the rows x, with its rows on their way through it"""
+        x = np.array(x, dtype=np.float32, order="C")
+        T = x.shape[0]
+        tp = self._taps(T, 1)
+        lp = C.byref(self.M.layer) if l < 0 else C.cast(C.addressof(self._layer_arr()[l]), C.c_void_p)
+        self.m.oracle.lib.fnx_o_decoder_layer(C.byref(self.D), lp, ol.ptr(x), T, pos0, self.threads)
+        self.m.oracle.lib.fnx_o_layer_taps(None, None, None, None, 0)
+        return dict(x_out=x, att=tp["att"][0], x_mid=tp["x_mid"][0], moe=tp["moe"][0])
+
+    def _layer_arr(self):
+        return self._keep[-3]   # the DecLayerO array oracle_structs built
 
     def draft(self, src, tokens, pos0, routing=False):
         c = self.m.cfg
