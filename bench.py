@@ -21,14 +21,37 @@ import sys
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
-sys.path.insert(0, os.path.join(ROOT, "tests"))
+PKG_DIR = os.path.join(ROOT, "qwen3.8-flash-next-2x-p100_amd")
+
+
+def harness():
+    """the package's host-side harness over the C ABI (the package's directory name is not a Python identifier)"""
+    import importlib
+    import importlib.util
+    name = "fnx_mi355x_pkg"
+    if name not in sys.modules:
+        spec = importlib.util.spec_from_file_location(name, os.path.join(PKG_DIR, "__init__.py"), submodule_search_locations=[PKG_DIR])
+        mod = importlib.util.module_from_spec(spec)
+        sys.modules[name] = mod
+        spec.loader.exec_module(mod)
+    return importlib.import_module(name + ".harness")
+
+
+def oracle_side():
+    """the CPU oracle's bindings (test infrastructure, under tests/): for the cpu_baseline legs only"""
+    tests = os.path.join(ROOT, "tests")
+    if tests not in sys.path:
+        sys.path.insert(0, tests)
+    import oracle_lib
+    return oracle_lib
+
 
 N, FF, NEXP, TOPK, T = 2048, 512, 512, 10, 16
 HBM_PEAK = 8.0e12
 # HBM bytes of one window launch of the default run (gaussian weights, 16 sets, unit64), measured by two rocprofv3 --pmc
-# runs of this file (FETCH_SIZE, then WRITE_SIZE, each scaled by a 256 MiB copy: profiles/moe_gate_up_hbm_traffic.md), and
+# runs of this file (FETCH_SIZE, then WRITE_SIZE, each scaled by a 256 MiB copy: profiles/moe_window_hbm_traffic.md), and
 # the distinct experts per step they were measured at. Not measured in the run: emitted only for that configuration.
-WINDOW_TRAFFIC = {"bytes": None, "algorithmic_bytes": 192.3e6, "distinct_experts_per_step": 138.45,
+WINDOW_TRAFFIC = {"bytes": 208.94e6, "algorithmic_bytes": 192.96e6, "distinct_experts_per_step": 138.45,
                    "source": "profiles/moe_window_hbm_traffic.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this file's default workload; scaled to "
                              "this run's algorithmic bytes; not measured in this run)"}
 # the same for the prompt path's gate|up launch (profiles/prefill_chunk_counters.md: FETCH_SIZE x 2 + WRITE_SIZE)
@@ -81,7 +104,7 @@ def gemv_measure(dev, torch, np, steps):
     launch, cycling through 1,024 distinct matrices (3.7 GB) so that every launch reads its weights from HBM: a launch of
     3.6 MB is bound by the launch, not by HBM; (b) one fnx_mmvq launch of 1,024 jobs over the 1,024 matrices through the
     table of matrix pointers: the kernel's streaming rate."""
-    import fnx_gpu
+    fnx_gpu = harness()
     pkg, lib, st = dev.pkg, dev.lib, dev.st()
     g = torch.Generator(device="cuda")
     g.manual_seed(11)
@@ -194,7 +217,7 @@ def main():
 
     import numpy as np
     import torch
-    import fnx_gpu
+    fnx_gpu = harness()
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = fnx_gpu.Dev()
     pkg, lib, t = dev.pkg, dev.lib, torch
@@ -279,11 +302,16 @@ def main():
             n_pre += 64
             torch.cuda.synchronize()
         preroll["ms"], preroll["steps"] = (time.perf_counter() - p0) * 1e3, n_pre
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)   # on the launch stream (torch's current one)
         t0 = time.perf_counter()
+        e0.record()
         for i in range(args.steps):
             step(args.warmup + n_pre + i, sets)
+        e1.record()
         torch.cuda.synchronize()
-        return time.perf_counter() - t0
+        dt = time.perf_counter() - t0
+        preroll["event_ms"] = e0.elapsed_time(e1)
+        return dt
 
     if args.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").random_()
@@ -322,7 +350,9 @@ def main():
                 per_launch += ms2
         dev.ok(lib.fnx_layer_profile(0))
         per_launch /= reps
-        k_ms = float(per_launch[1])
+        # the kernel's average duration: events on the launch stream around the timed region's K launches, which follow one
+        # another with nothing between them (per_launch: one launch at a time from an idle GPU, with an event either side)
+        k_ms = headline_preroll["event_ms"] / args.steps if not args.shared_q8 else float(per_launch[1])
         kernel_name = "k_moe_window (unit64; the whole window is this one launch)"
         # algorithmic bytes of the launch: the step's (the distinct experts' and the shared expert's blocks, the router, x in, out)
         k_bytes = step_bytes
@@ -362,7 +392,7 @@ def main():
     # ---- CPU baseline: the oracle on the host's cores, same workload (layer set 0), bounded sample
     cpu = None
     if args.cpu_seconds > 0:
-        import oracle_lib
+        oracle_lib = oracle_side()
         oracle = oracle_lib.Oracle()
         threads = min(os.cpu_count() or 1, 16)
         L, router = layers[0][0], layers[0][1]
@@ -451,7 +481,7 @@ def gemv_main(args):
     """benchmark config 1 on its own (gemv_measure)"""
     import numpy as np
     import torch
-    import fnx_gpu
+    fnx_gpu = harness()
     dev = fnx_gpu.Dev()
     res = gemv_measure(dev, torch, np, args.steps)
     many, lone = res["launch_of_1024_matrices"], res["lone_matrix_a_launch"]
@@ -472,8 +502,8 @@ def head_main(args):
     over a 38,862-token context with 200 copied spans, greedy acceptance; device forms, one stream."""
     import numpy as np
     import torch
-    import fnx_gpu
-    import oracle_lib
+    fnx_gpu = harness()
+    oracle_lib = oracle_side()
     dev = fnx_gpu.Dev()
     lib = dev.lib
     oracle = oracle_lib.Oracle()
@@ -568,8 +598,7 @@ def decoder_main(args):
     once on the oracle and compares the two."""
     import numpy as np
     import torch
-    import fnx_gpu
-    import tiny_decoder as td
+    fnx_gpu = harness()
     dev = fnx_gpu.Dev()
     pkg, lib, t = dev.pkg, dev.lib, torch
     g = torch.Generator(device="cuda")
@@ -577,9 +606,9 @@ def decoder_main(args):
     NQ, NKV, HD, NL, V, CTX, R = 16, 2, 256, 4, 151936, 32768, 16
     oracle = None
     if args.cpu_seconds > 0:
-        import oracle_lib
+        oracle_lib = oracle_side()
         oracle = oracle_lib.Oracle()
-    model = td.TinyDecoder(oracle, seed=44, n=N, nq=NQ, nkv=NKV, nlayers=NL, vocab=V, max_ctx=CTX, nexp=NEXP, topk=TOPK, ff=FF, cheap_draws=True)
+    model = fnx_gpu.SyntheticDecoder(seed=44, n=N, nq=NQ, nkv=NKV, nlayers=NL, vocab=V, max_ctx=CTX, nexp=NEXP, topk=TOPK, ff=FF, cheap_draws=True)
     dd = fnx_gpu.DecoderDev(dev, model)
     rng = np.random.default_rng(45)
     cells = [(rng.standard_normal((CTX - R, NKV, HD), dtype=np.float32).astype(np.float16),
@@ -682,7 +711,8 @@ def decoder_main(args):
     cpu = None
     if oracle is not None:
         threads = min(os.cpu_count() or 1, 16)
-        sess = td.OracleSession(model, threads=threads)
+        import tiny_decoder as td   # under tests/, on the path since oracle_side()
+        sess = td.OracleSession(td.TinyDecoder.of(model, oracle), threads=threads)
         for (kc, vc), (k, v) in zip(sess.caches + [sess.mtp_cache], cells):
             kc[:CTX - R], vc[:CTX - R] = k.view(np.uint16), v.view(np.uint16)
         rows = [int(x) for x in toks[0].cpu().numpy()]
@@ -743,7 +773,7 @@ def prefill_main(args):
     imposed through a constant input feature and a bias column of the router. A step = one chunk."""
     import numpy as np
     import torch
-    import fnx_gpu
+    fnx_gpu = harness()
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = fnx_gpu.Dev()
     pkg, lib, t = dev.pkg, dev.lib, torch
@@ -880,7 +910,7 @@ def prefill_main(args):
     MFMA_F16 = 2.5e15
     cpu = None
     if args.cpu_seconds > 0:
-        import oracle_lib
+        oracle_lib = oracle_side()
         oracle = oracle_lib.Oracle()
         threads = min(os.cpu_count() or 1, 16)
         CS = 64   # rows of the CPU sample

@@ -1,5 +1,8 @@
 """Parity of the MoE verify layer (benchmark config 2) with the CPU oracle: op by op and as one call."""
 import ctypes as C
+import os
+import subprocess
+import sys
 
 import numpy as np
 import pytest
@@ -199,3 +202,18 @@ def test_moe_ops_one_by_one_equal_the_fused_call(dev, oracle):
     assert np.array_equal(sh_hq.cpu().numpy().reshape(-1, 36), hq_want.reshape(-1, 36))
     comb = oracle.moe_combine(part.cpu().numpy()[:P], topw.cpu().numpy(), sh_part.cpu().numpy(), logits.cpu().numpy()[:, nexp])
     assert np.array_equal(out.cpu().numpy().view(np.uint32), comb.view(np.uint32))
+
+
+def test_a_window_whose_waits_run_out_leaves_and_says_so(dev):
+    """the error path of the window's cross-block waits, forced from the host: with no wait budget (a child process, since the
+    library reads the budget once) every block still leaves, the launch ends, and the workspace's error word carries
+    FNX_ERR_BARRIER - the caller's sign to discard the window's results and zero the sync words before the next one"""
+    env = dict(os.environ, FNX_WINDOW_WAIT_TICKS="0")
+    child = os.path.join(os.path.dirname(os.path.abspath(__file__)), "window_timeout_child.py")
+    print("case window with no wait budget (child process)", flush=True)
+    r = subprocess.run([sys.executable, "-u", child], env=env, capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0, r.stdout + r.stderr
+    line = [l for l in r.stdout.splitlines() if l.startswith("window left err=")]
+    assert line, r.stdout + r.stderr
+    err = int(line[0].split("=")[1])
+    assert err & dev.pkg.ERR_BARRIER, "a wait that gives up sets the error bit"

@@ -5,7 +5,7 @@ import ctypes as C
 import numpy as np
 
 import oracle_lib as ol
-from fnx_gpu import random_iq3s
+from fnx_gpu import SyntheticDecoder
 
 HD = 256
 
@@ -34,69 +34,32 @@ class MtpO(C.Structure):
                 ("layer", DecLayerO)]
 
 
-def _q8s_draw(rng, oracle, rows, cols, scale, cheap=False):
-    """a split-Q8_0 matrix (int8 values, f16 block scales) with entries of standard deviation `scale`: Gaussian weights
-    quantised by the oracle, or (cheap) uniformly random int8 values under block scales of scale / 74 with a random last
-    mantissa nibble (every (q, d) pair is a valid matrix; no float matrix is drawn)"""
-    if cheap:
-        q = rng.integers(0, 1 << 64, size=rows * cols // 8, dtype=np.uint64).view(np.int8).reshape(rows, cols)
-        d0 = np.array([scale / 74.0], dtype=np.float16).view(np.uint16)[0] & np.uint16(0xFFF0)
-        d = d0 | rng.integers(0, 16, (rows, cols // 32), dtype=np.uint16)
+def _oracle_q8s(oracle):
+    def quantize(w):
+        rows, cols = w.shape
+        q = np.zeros((rows, cols), dtype=np.int8)
+        d = np.zeros((rows, cols // 32), dtype=np.uint16)
+        oracle.lib.fnx_o_quantize_q8_0_split(ol.ptr(w), rows, cols, ol.ptr(q), ol.ptr(d))
         return q, d
-    w = (rng.standard_normal((rows, cols)) * scale).astype(np.float32)
-    q = np.zeros((rows, cols), dtype=np.int8)
-    d = np.zeros((rows, cols // 32), dtype=np.uint16)
-    oracle.lib.fnx_o_quantize_q8_0_split(ol.ptr(w), rows, cols, ol.ptr(q), ol.ptr(d))
-    return q, d
+    return quantize
 
 
-class TinyDecoder:
-    def __init__(self, oracle, seed=1, n=256, nq=4, nkv=2, nlayers=2, vocab=1000, max_ctx=128, nexp=8, topk=2, ff=256, rope_scaled=False,
-                 cyclic=False, cheap_draws=False):
-        """cheap_draws: cheaper draws for full-size models (other values than the default draws): the dense matrices as random
-        int8 values, the embedding as f16 bit patterns, the IQ3_S blocks from the generator's 64-bit stream.
-        cyclic: a model whose pick depends on the row's token alone (the attention's output projections are zero) and
-        whose draft layer is the model's single layer behind an identity projection of the embedding, so greedy decoding
-        runs into a cycle, the draft layer mostly predicts the next token, prompt lookup fires and drafts are kept."""
-        rng = np.random.default_rng(seed)
+class TinyDecoder(SyntheticDecoder):
+    """the package's synthetic model (Gaussian dense matrices quantised by the oracle unless cheap_draws), with the oracle's
+    rendering of it beside the device's"""
+
+    def __init__(self, oracle, **kw):
+        super().__init__(quantize=_oracle_q8s(oracle) if oracle is not None else None, **kw)
         self.oracle = oracle
-        _q8s = lambda rng, oracle, rows, cols, scale: _q8s_draw(rng, oracle, rows, cols, scale, cheap_draws)
-        self.cfg = dict(n=n, nq=nq, nkv=nkv, nlayers=nlayers, vocab=vocab, max_ctx=max_ctx, nexp=nexp, topk=topk, ff=ff, eps=1e-6)
-        self.rope = (1e7, 0, 0.0, 0.0, 1.0, 1.0) if not rope_scaled else (1e4, 1, 4.0, 20.0, 0.25, 1.0 + 0.1 * np.log(4.0))
-        nb = lambda rows, cols: rows * cols // 256
-        sw = 1.0 / np.sqrt(n)
-        iq3s = lambda nblocks: random_iq3s(rng, nblocks, dmax=4e-4, raw_bytes=cheap_draws)
 
-        def layer():
-            L = dict(attn_norm=(1 + 0.1 * rng.standard_normal(n)).astype(np.float32), q_norm=(1 + 0.1 * rng.standard_normal(HD)).astype(np.float32),
-                     k_norm=(1 + 0.1 * rng.standard_normal(HD)).astype(np.float32), ffn_norm=(1 + 0.1 * rng.standard_normal(n)).astype(np.float32),
-                     wq=_q8s(rng, oracle, nq * 2 * HD, n, sw), wk=_q8s(rng, oracle, nkv * HD, n, sw), wv=_q8s(rng, oracle, nkv * HD, n, sw),
-                     wo=_q8s(rng, oracle, n, nq * HD, 1.0 / np.sqrt(nq * HD)),
-                     router=(rng.standard_normal((nexp + 1, n)) * 0.05).astype(np.float32),
-                     gu=iq3s(nexp * nb(2 * ff, n)), down=iq3s(nexp * nb(n, ff)),
-                     sh_gu=iq3s(nb(2 * ff, n)), sh_down=iq3s(nb(n, ff)))
-            return L
+    @classmethod
+    def of(cls, model, oracle):
+        """a SyntheticDecoder built elsewhere, with the oracle's rendering added"""
+        m = cls.__new__(cls)
+        m.__dict__.update(model.__dict__)
+        m.oracle = oracle
+        return m
 
-        self.layers = [layer() for _ in range(nlayers)]
-        self.out_norm = (1 + 0.1 * rng.standard_normal(n)).astype(np.float32)
-        self.head = _q8s(rng, oracle, vocab, n, sw)
-        if cheap_draws:   # f16 bit patterns drawn directly: a random sign, exponent field 12..15 (magnitudes 1/8 .. 2), random mantissa
-            self.emb = ((rng.integers(0, 1 << 16, (vocab, n), dtype=np.uint16) & np.uint16(0x8FFF)) | np.uint16(0x3000)).view(np.float16)
-        else:
-            self.emb = rng.standard_normal((vocab, n)).astype(np.float16)
-        self.mtp = dict(norm_emb=(1 + 0.1 * rng.standard_normal(n)).astype(np.float32), norm_hid=(1 + 0.1 * rng.standard_normal(n)).astype(np.float32),
-                        out_norm=(1 + 0.1 * rng.standard_normal(n)).astype(np.float32), fc_emb=_q8s(rng, oracle, n, n, sw),
-                        fc_hid=_q8s(rng, oracle, n, n, sw), head=_q8s(rng, oracle, vocab, n, sw), layer=layer())
-        if cyclic:
-            assert nlayers == 1
-            zero = lambda t: (np.zeros_like(t[0]), np.zeros_like(t[1]))
-            self.layers[0]["wo"] = zero(self.layers[0]["wo"])
-            e = self.emb.astype(np.float32)
-            self.emb = (e / np.sqrt((e * e).mean(axis=1, keepdims=True))).astype(np.float16)
-            eye_q, eye_d = np.zeros((n, n), dtype=np.int8), np.zeros((n, n // 32), dtype=np.uint16)
-            oracle.lib.fnx_o_quantize_q8_0_split(ol.ptr(np.eye(n, dtype=np.float32)), n, n, ol.ptr(eye_q), ol.ptr(eye_d))
-            self.mtp = dict(norm_emb=np.ones(n, dtype=np.float32), norm_hid=self.mtp["norm_hid"], out_norm=self.out_norm, fc_emb=(eye_q, eye_d),
-                            fc_hid=zero(self.mtp["fc_hid"]), head=self.head, layer=self.layers[0])
 
     # ---- the oracle's rendering: host arrays; the caches are numpy arrays kept here
     def oracle_structs(self):
