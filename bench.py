@@ -201,7 +201,7 @@ def main():
                     help="the shared expert as dense split Q8_0 (the reference's own form, three more launches a window) instead of IQ3_S")
     ap.add_argument("--no-extras", action="store_true", help="skip the legs beside the metric (verify: streaming calibration, config 1, the other weight kind; prefill: two chunks in flight)")
     ap.add_argument("--raw-layout", action="store_true", help="verify: leave the weights as raw ggml blocks (skip the load-time re-laying); prefill: unit64 only, no tile16 copies")
-    ap.add_argument("--down-unit64", action="store_true", help="prefill: leave the down matrices in the unit64 layout (k_moe_mma_tile64) instead of tile16 (k_moe_mma_wave16)")
+    ap.add_argument("--down-unit64", action="store_true", help="prefill: leave the down matrices in the unit64 layout (k_moe_mma) instead of tile16 (k_moe_mma_wave16)")
     ap.add_argument("--workload", choices=["verify", "prefill", "decoder", "head", "gemv"], default="verify",
                     help="verify: benchmark config 2 (the headline metric, the default); prefill: config 5, one MoE layer over prompt chunks of 512 "
                          "rows; decoder: config 4, a verify step of the reduced decoder plus the draft layer; head: config 3, argmax + prompt "
@@ -531,7 +531,7 @@ def head_main(args):
     dctx, dd1 = dev.up(ctx), dev.up(np.array([d1], dtype=np.int32))
     dout, dn, dm = dev.zeros(15, t.int32), dev.zeros(1, t.int32), dev.zeros(1, t.int32)
     drows = dev.up(np.pad(rows, (0, R - len(rows))))
-    bv, bi, keys, err, nacc = dev.zeros(R, t.float32), dev.zeros(R, t.int32), dev.zeros(16, t.int64), dev.zeros(1, t.int32), dev.zeros(1, t.int32)
+    bv, bi, keys, err, nacc = dev.zeros(R, t.float32), dev.zeros(R, t.int32), dev.zeros(32, t.int64), dev.zeros(1, t.int32), dev.zeros(1, t.int32)
     st = dev.st()
 
     def timed(fn, n):
@@ -802,7 +802,8 @@ def prefill_main(args):
         for w in ws_:
             dev.ok(lib.fnx_iq3s_repack(w.data_ptr(), w.data_ptr(), w.numel() // IQ3S_BLOCK * 256, dev.st()))
         gu, down, sh_gu, sh_down = ws_
-        L = pkg.MoeLayer(N, FF, NEXP, TOPK, router.data_ptr(), 0, pkg.dw(gu, N, 2 * FF, packed=True), GU_BYTES, pkg.dw(down, FF, N, packed=True),
+        gu64 = pkg.dw(gu, N, 2 * FF, packed=True)   # the unit64 copy's descriptor, kept for the two-launch leg
+        L = pkg.MoeLayer(N, FF, NEXP, TOPK, router.data_ptr(), 0, gu64, GU_BYTES, pkg.dw(down, FF, N, packed=True),
                          DN_BYTES, pkg.dw(sh_gu, N, 2 * FF, packed=True), pkg.dw(sh_down, FF, N, packed=True))
         if not args.raw_layout:   # the gate|up matrices in the prompt path's own layout beside the unit64 copy
             gu16 = torch.zeros(lib.fnx_iq3s_tile16_bytes(2 * FF, N, NEXP), dtype=torch.uint8, device="cuda")
@@ -818,7 +819,7 @@ def prefill_main(args):
                 dev.ok(lib.fnx_iq3s_tile16(sh_down.data_ptr(), shd16.data_ptr(), N, FF, 1, dev.st()))
                 L.down, L.down_stride, L.sh_down = pkg.dw(dn16, FF, N, tile16=True), lib.fnx_iq3s_tile16_bytes(N, FF, 1), pkg.dw(shd16, FF, N, tile16=True)
                 ws_ = ws_ + [dn16, shd16]
-        layers.append((L, router, ws_, raw))
+        layers.append((L, router, ws_, raw, gu64))
     NX = 8
     xs = torch.randn((NX, CH, N), device="cuda", generator=g)
     xs[:, :, 0] = 1.0   # the constant feature the router's bias column multiplies
@@ -879,18 +880,19 @@ def prefill_main(args):
     u_mean, j_mean = float(np.mean(active)), float(np.mean(jobs))
     # the two matrix-core launches on their own, with events on the launch stream (torch's current stream)
     reps = 20
-    fused_h = True   # unit64 and tile16 matrices (this workload has no other) leave h = silu(gate) * up from the gate|up launch itself
+    fused_h = not args.raw_layout   # tile16 gate|up matrices leave h = silu(gate) * up from the gate|up launch itself
     evs = []
     for i in range(reps + 3):
         L = layers[i % nsets][0]
         step(i)   # routes chunk i: the jobs and xh in the workspace are this chunk's
         e = [torch.cuda.Event(enable_timing=True) for _ in range(5)]
         e[0].record()
-        dev.ok(lib.fnx_moe_gate_up_mma(C.byref(L.gu), L.gu_stride, ws.jobs_gu, ws.njobs, J, ws.xh, ws.gu, st))
+        # the products as a launch of their own (fnx_moe_gate_up_mma takes raw blocks and unit64: the unit64 copy), then SwiGLU
+        dev.ok(lib.fnx_moe_gate_up_mma(C.byref(layers[i % nsets][4]), GU_BYTES, ws.jobs_gu, ws.njobs, J, ws.xh, ws.gu, st))
         e[1].record()
         dev.ok(lib.fnx_swiglu_h16(ws.gu, FF, P + CH, ws.h16, st))
         e[2].record()
-        if fused_h:   # what the layer runs: the same h from one launch
+        if fused_h:   # what the layer runs: h from one launch
             dev.ok(lib.fnx_moe_gate_up_h16_mma(C.byref(L.gu), L.gu_stride, ws.jobs_gu, ws.njobs, J, ws.xh, ws.h16, st))
         e[3].record()
         dev.ok(lib.fnx_moe_down_mma(C.byref(L.down), L.down_stride, ws.jobs_dn, ws.njobs, J, ws.h16, ws.part, st))
@@ -926,7 +928,7 @@ def prefill_main(args):
         cpu = {"value": CS / cdt, "unit": "tokens/s per layer", "cores": threads, "kind": "port",
                "sample": f"one pass of the oracle's prefill layer over the first {CS} rows of chunk 0 (f16 operands, f64 accumulation)",
                "parity_rel_l2": err}
-    gu_kernel = ("k_moe_mma_block64 (routed gate|up over unit64, leaves h = silu(gate) * up; a job's up to 64 tokens a decode)" if args.raw_layout else
+    gu_kernel = ("k_moe_mma (routed gate|up over unit64, a wave a task of 32 rows x 32 tokens; h by fnx_swiglu_h16)" if args.raw_layout else
                  "k_moe_mma_wave16_gu (routed gate|up over tile16, leaves h = silu(gate) * up; a wave a pair of gate and up tiles, a job's up to 64 tokens a decode)")
     line = {
         "metric": "prefill MoE tokens/sec per layer (chunks of 512 rows) + grouped IQ3_S expert GEMM achieved GB/s and MFMA utilisation",
@@ -941,8 +943,8 @@ def prefill_main(args):
                      "traffic": PF_WINDOW_TRAFFIC["bytes"] * gu_bytes / PF_WINDOW_TRAFFIC["algorithmic_bytes"] if nsets == 4 and not args.raw_layout else None,
                      "traffic_source": PF_WINDOW_TRAFFIC["source"] if nsets == 4 and not args.raw_layout else None, "kernel_ms": gu_ms, "algorithmic_bytes": gu_bytes,
                      "mfma_tflops": gu_flops / (gu_ms * 1e-3) / 1e12, "mfma_frac": gu_flops / (gu_ms * 1e-3) / MFMA_F16,
-                     "down": {"kernel": "k_moe_mma_tile64 (unit64)" if args.down_unit64 or args.raw_layout else "k_moe_mma_wave16 (tile16)", "kernel_ms": dn_ms, "achieved": dn_bytes / (dn_ms * 1e-3) / 1e9, "mfma_tflops": dn_flops / (dn_ms * 1e-3) / 1e12},
-                     "two_launches": {"gate_up_ms": gu2_ms, "swiglu_ms": sw_ms, "note": "fnx_moe_gate_up_mma (k_moe_mma_block64, f32 products written) and fnx_swiglu_h16"},
+                     "down": {"kernel": "k_moe_mma (unit64)" if args.down_unit64 or args.raw_layout else "k_moe_mma_wave16 (tile16)", "kernel_ms": dn_ms, "achieved": dn_bytes / (dn_ms * 1e-3) / 1e9, "mfma_tflops": dn_flops / (dn_ms * 1e-3) / 1e12},
+                     "two_launches": {"gate_up_ms": gu2_ms, "swiglu_ms": sw_ms, "note": "fnx_moe_gate_up_mma (k_moe_mma over the unit64 copy, f32 products written) and fnx_swiglu_h16"},
                      # the piecewise bound: a launch cannot be faster than its bytes at the HBM peak or its flops at the MFMA peak
                      "piecewise_bound": {"gate_up_us": max(gu_bytes / HBM_PEAK, gu_flops / MFMA_F16) * 1e6,
                                          "gate_up_frac": max(gu_bytes / HBM_PEAK, gu_flops / MFMA_F16) / (gu_ms * 1e-3),

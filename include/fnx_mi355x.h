@@ -80,8 +80,8 @@ const char* fnx_version(void);
  * fnx_dw.type = FNX_T_IQ3S_UNIT64: every operator below takes both types and gives the same results; the re-laid
  * type is the fast path. Rows must have 256, 512, 1024 or 2048 columns and expert strides must be multiples of 880. */
 int fnx_iq3s_repack(const void* src, void* dst, size_t n_weights, void* st);
-/* A second load-time layout, for the prompt path's matrix-core kernels (fnx_moe_gate_up_mma, fnx_moe_down_mma - the
- * latter's fast form where rows have 512 columns -, fnx_moe_prefill_layer's gate|up and down) and the mat-vec operators'
+/* A second load-time layout, for the prompt path's matrix-core kernels (fnx_moe_gate_up_h16_mma over stacked gate|up
+ * matrices, fnx_moe_down_mma over rows of 512 columns, fnx_moe_prefill_layer's gate|up and down) and the mat-vec operators'
  * jobs of many rows; no counterpart in the reference, whose prompt kernels read raw blocks: nmat matrices of nrows x ncols
  * (rows in 16s, columns in 512s) from the unit64 layout into tiles of 16 rows x 512 columns in which the 64 lanes of a
  * wave find their shares side by side (3,584 bytes a tile: 1.8 % more than the blocks). src: the matrices one after the
@@ -139,8 +139,10 @@ int fnx_moe_down(const fnx_dw* A, size_t sa, const fnx_job* jobs, const int* njo
 int fnx_moe_combine(const float* part, const float* topw, const float* sh, const float* sh_logit, int sh_logit_stride, float* out,
                     int T, int n, int topk, void* st);
 
-/* kernels.hpp:433  argmax: best[t] = (value, index + v0), the lowest index on ties. keys: 16 words, zeroed once (left
- * at zero). err bit 16: a logit was NaN or inf */
+/* kernels.hpp:433  argmax: best[t] = (value, index + v0), the lowest index on ties. One launch: a row's last block to
+ * arrive decodes the row's key. keys: FNX_ARGMAX_WORDS words, zeroed once (left at zero): a key a row, then a count of
+ * arrived blocks a row - twice the reference's MAXT words (engine.cu:314). err bit 16: a logit was NaN or inf */
+#define FNX_ARGMAX_WORDS (2 * FNX_MAXT)
 int fnx_argmax(const float* logits, int rows, int T, int v0, float* best_v, int* best_i, unsigned long long* keys, unsigned* err,
                void* st);
 
@@ -250,18 +252,19 @@ int fnx_pf_route(const float* logits, int logits_stride, int C, int nexp, int to
 /* kernels.hpp (p100_f32_f16): f32 -> f16, round to nearest even */
 int fnx_f32_f16(const float* x, size_t n, uint16_t* out, void* st);
 /* kernels.hpp:328  moe_gate_up_mma: gu[jobs.out][2 ffs] = W_e[2 ffs][n] . xh[jobs.y] with f16 weights (each the f32
- * value rounded once), f16 activations, fp32 accumulation, on the matrix cores. xh rows of A->n_in halves. */
+ * value rounded once), f16 activations, fp32 accumulation, on the matrix cores. xh rows of A->n_in halves. Raw blocks and
+ * unit64 (tile16 gate|up matrices go through fnx_moe_gate_up_h16_mma, which leaves h). */
 int fnx_moe_gate_up_mma(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const int* njobs, int njobs_cap, const uint16_t* xh, float* gu,
                         void* st);
 /* kernels.hpp:329  swiglu_h16: h16[p][ffs] = f16(silu(gate) * up) of the P stacked rows [gate | up] */
 int fnx_swiglu_h16(const float* gu, int ffs, int P, uint16_t* h16, void* st);
-/* kernels.hpp:328 + 329 in one launch: h16[jobs.out][ffs] = f16(silu(gate) * up) of the products of fnx_moe_gate_up_mma,
- * which are not written (the same bits as the two calls one after the other; over unit64 rows of up to 512 columns the
- * two calls add a row's products in another order). For unit64 and tile16 matrices with 2 ffs
- * rows in 256s and columns in 512s (an error otherwise); fnx_moe_prefill_layer uses it where it can. */
+/* kernels.hpp:328 + 329 in one launch: h16[jobs.out][ffs] = f16(silu(gate) * up) of the products, which are not written.
+ * For tile16 matrices (2 ffs rows in 32s, columns in 512s; an error otherwise); fnx_moe_prefill_layer uses it where it
+ * can. The products are fnx_moe_gate_up_mma's up to the order in which a row's f16 products are added. */
 int fnx_moe_gate_up_h16_mma(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const int* njobs, int njobs_cap, const uint16_t* xh,
                             uint16_t* h16, void* st);
-/* kernels.hpp:330  moe_down_mma: part[jobs.out][n] = W_e[n][ffs] . h16[jobs.y] */
+/* kernels.hpp:330  moe_down_mma: part[jobs.out][n] = W_e[n][ffs] . h16[jobs.y]. Raw blocks, unit64, or tile16 with
+ * ffs = 512 */
 int fnx_moe_down_mma(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const int* njobs, int njobs_cap, const uint16_t* h16, float* part,
                      void* st);
 /* caller-owned scratch for one chunk; P = C * topk, J = P / FNX_PF_JOB + nexp, S = ceil(C / FNX_PF_JOB) */
@@ -350,7 +353,7 @@ typedef struct fnx_dec_ws {
     void* xq;                               /* q8_1 rows of max(n, nq * 256) values */
     float *hidden, *logits, *best_v;        /* [T][n] (the rows before the output norm), [T][vocab], [T] */
     int* best_i;                            /* [T] */
-    unsigned long long* keys;               /* [16], zero */
+    unsigned long long* keys;               /* [FNX_ARGMAX_WORDS], zero */
     unsigned* err;                          /* [1] */
     fnx_moe_ws moe;
 } fnx_dec_ws;
@@ -368,8 +371,15 @@ int fnx_decoder_layer(const fnx_decoder* D, const fnx_dec_layer* L, const float*
  * draft layer's own for a chain). ws->hidden receives the layer's output rows. */
 typedef struct fnx_mtp {
     const float *norm_emb, *norm_hid, *out_norm;   /* [n] each */
-    fnx_q8s fc_emb, fc_hid, head;                  /* [n][n], [n][n], [vocab][n] */
+    fnx_q8s fc_emb, fc_hid, head;                  /* [n][n], [n][n], [dv1 - dv0][n] */
     fnx_dec_layer layer;
+    /* model.hpp:233-243, engine.cu:2130-2131: the head's rows are the tokens [dv0, dv1) of the vocabulary (a card's share of
+     * the draft head); dv0 == dv1 == 0: all of it. Rows of ws->logits then have dv1 - dv0 values, and the picks are token ids
+     * (dv0 added, as argmax's v0). pen / pen_par (null: none): the LAST row's penalty list in fnx_penalize_row's format, its
+     * indexes relative to dv0 (engine_common.cu:1602), applied to that row's logits in place before the picks. */
+    int dv0, dv1;
+    const int* pen;
+    const float* pen_par;
 } fnx_mtp;
 int fnx_mtp_draft(const fnx_decoder* D, const fnx_mtp* M, const float* src, const int* tokens, int T, const int* pos0, const fnx_dec_ws* ws,
                   void* st);

@@ -1243,13 +1243,16 @@ static void dec_layer(const fnx_o_decoder* D, const fnx_o_dec_layer* L, float* x
 void fnx_o_decoder_layer(const fnx_o_decoder* D, const fnx_o_dec_layer* L, float* x, int T, int pos0, int threads) {
     dec_layer(D, L, x, T, pos0, threads);
 }
-static void dec_head(const fnx_o_decoder* D, const float* norm, const fnx_o_q8s* head, const float* x, int T, float* logits_out, int* best) {
+/* nv head rows for the tokens from v0; pen (may be null): the last row's penalties before the picks (engine.cu:2130-2131) */
+static void dec_head(const fnx_o_decoder* D, const float* norm, const fnx_o_q8s* head, const float* x, int T, float* logits_out, int* best,
+                     int nv, int v0, const int* pen, const float* pen_par) {
     float* xn = (float*) malloc((size_t) T * D->n * sizeof(float));
-    float* logits = logits_out ? logits_out : (float*) malloc((size_t) T * D->vocab * sizeof(float));
+    float* logits = logits_out ? logits_out : (float*) malloc((size_t) T * nv * sizeof(float));
     float* bv = (float*) malloc((size_t) T * sizeof(float));
     fnx_o_rms_norm_rows(x, norm, xn, T, D->n, D->eps);
     dense_q8s(head, xn, T, logits);
-    fnx_o_argmax(logits, D->vocab, T, 0, bv, best);
+    if (pen) fnx_o_penalize_row(logits + (size_t) (T - 1) * nv, nv, pen, pen_par);
+    fnx_o_argmax(logits, nv, T, v0, bv, best);
     free(xn);
     free(bv);
     if (!logits_out) free(logits);
@@ -1257,7 +1260,7 @@ static void dec_head(const fnx_o_decoder* D, const float* norm, const fnx_o_q8s*
 void fnx_o_decoder_verify(const fnx_o_decoder* D, const int* tokens, int T, int pos0, float* hidden, float* logits, int* best, int threads) {
     embed_rows(D->emb, tokens, T, D->n, hidden);
     for (int l = 0; l < D->nlayers; ++l) dec_layer(D, &D->layers[l], hidden, T, pos0, threads);
-    dec_head(D, D->out_norm, &D->head, hidden, T, logits, best);
+    dec_head(D, D->out_norm, &D->head, hidden, T, logits, best, D->vocab, 0, NULL, NULL);
 }
 void fnx_o_mtp_draft(const fnx_o_decoder* D, const fnx_o_mtp* M, const float* src, const int* tokens, int T, int pos0, float* hidden,
                      float* logits, int* best, int threads) {
@@ -1274,7 +1277,7 @@ void fnx_o_mtp_draft(const fnx_o_decoder* D, const fnx_o_mtp* M, const float* sr
     for (size_t i = 0; i < (size_t) T * n; ++i) x[i] += e2[i];
     dec_layer(D, &M->layer, x, T, pos0, threads);
     memcpy(hidden, x, (size_t) T * n * sizeof(float));
-    dec_head(D, M->out_norm, &M->head, x, T, logits, best);
+    dec_head(D, M->out_norm, &M->head, x, T, logits, best, M->dv1 > M->dv0 ? M->dv1 - M->dv0 : D->vocab, M->dv0, M->pen, M->pen_par);
     free(xn); free(e); free(e2); free(x);
 }
 

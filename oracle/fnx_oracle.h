@@ -216,6 +216,11 @@ typedef struct {
     const float *norm_emb, *norm_hid, *out_norm;
     fnx_o_q8s fc_emb, fc_hid, head;
     fnx_o_dec_layer layer;
+    /* engine.cu:2130-2131: the head's rows are the tokens [dv0, dv1) (both 0: the whole vocabulary); pen / pen_par (null: none):
+     * the last row's penalty list (fnx_o_penalize_row's format, indexes relative to dv0), applied before the picks */
+    int dv0, dv1;
+    const int* pen;
+    const float* pen_par;
 } fnx_o_mtp;
 /* the reduced decoder's window (engine.cu Engine::enqueue without streams, cards, GDN layers): hidden [T][n], logits
  * [T][vocab] (may be null), best [T] = argmax rows */

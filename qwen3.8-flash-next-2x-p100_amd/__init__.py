@@ -17,7 +17,8 @@ T_IQ3S_UNIT64 = 1021
 T_IQ3S_TILE16 = 1022
 IQ3S_BLOCK = 110
 Q8_1_BLOCK = 36
-MOE_SYNC_WORDS = 544   # fnx_moe_ws.sync: uint32 words, zeroed once
+MOE_SYNC_WORDS = 544
+ARGMAX_WORDS = 32   # FNX_ARGMAX_WORDS: a key and an arrival count a row   # fnx_moe_ws.sync: uint32 words, zeroed once
 ERR_BARRIER = 4
 
 
@@ -75,7 +76,7 @@ class DecWs(C.Structure):
 
 class Mtp(C.Structure):
     _fields_ = [("norm_emb", C.c_void_p), ("norm_hid", C.c_void_p), ("out_norm", C.c_void_p), ("fc_emb", Q8S), ("fc_hid", Q8S), ("head", Q8S),
-                ("layer", DecLayer)]
+                ("layer", DecLayer), ("dv0", C.c_int), ("dv1", C.c_int), ("pen", C.c_void_p), ("pen_par", C.c_void_p)]
 
 
 class Round(C.Structure):

@@ -547,9 +547,11 @@ __device__ __forceinline__ float fkey_inv(unsigned k) { return __uint_as_float((
 constexpr int AM_THREADS = 1024, AM_PER_BLOCK = 16384;
 // keys[t] = max over the row of (fkey(value) << 32 | ~index): the greatest value, the lower index on a tie. A block
 // folds its 16,384 values to one key (four independent 16-byte loads a thread, wave butterflies, LDS) and issues one
-// atomic: atomics on one address serialise, and a row's address would otherwise take one per wave.
+// atomic: atomics on one address serialise, and a row's address would otherwise take one per wave. The row's last block
+// to arrive (a count beside the keys, keys[FNX_MAXT + t]) decodes the key into (value, index + v0) and leaves both words
+// at zero for the next argmax.
 __global__ void __launch_bounds__(AM_THREADS) k_argmax(const float* __restrict__ logits, int rows, unsigned long long* __restrict__ keys,
-                                                      unsigned* __restrict__ err) {
+                                                      unsigned* __restrict__ err, int v0, float* __restrict__ bv, int* __restrict__ bi) {
     __shared__ unsigned long long wbest[AM_THREADS / 64];
     __shared__ int wbad;
     const int t = blockIdx.y, i0 = blockIdx.x * AM_PER_BLOCK, i1 = min(rows, i0 + AM_PER_BLOCK), tid = threadIdx.x;
@@ -595,18 +597,20 @@ __global__ void __launch_bounds__(AM_THREADS) k_argmax(const float* __restrict__
     __syncthreads();
     if (tid == 0) {
         for (int w = 1; w < AM_THREADS / 64; ++w) best = wbest[w] > best ? wbest[w] : best;
-        atomicMax(&keys[t], best);
         if (wbad) atomicOr(err, FNX_ERR_NONFINITE);
+        // the maximum has been taken at the device's level (its old value is back) before this block counts as arrived
+        const unsigned long long old = __hip_atomic_fetch_max(&keys[t], best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned long long mine = old > best ? old : best;
+        asm volatile("" ::"v"(mine));
+        const unsigned long long arrived = __hip_atomic_fetch_add(&keys[FNX_MAXT + t], 1ull, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        if (arrived == gridDim.x - 1) {
+            const unsigned long long k = __hip_atomic_load(&keys[t], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            bv[t] = fkey_inv((unsigned) (k >> 32));
+            bi[t] = (int) ~(unsigned) k + v0;
+            __hip_atomic_store(&keys[t], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&keys[FNX_MAXT + t], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
     }
-}
-// decodes the keys into (value, index + v0) and leaves them at zero for the next argmax
-__global__ void k_argmax_fin(unsigned long long* keys, int T, int v0, float* bv, int* bi) {
-    const int t = threadIdx.x;
-    if (t >= T) return;
-    const unsigned long long k = keys[t];
-    bv[t] = fkey_inv((unsigned) (k >> 32));
-    bi[t] = (int) ~(unsigned) k + v0;
-    keys[t] = 0ull;
 }
 
 // ================================================================ prompt lookup and acceptance on the device
@@ -1039,8 +1043,7 @@ int fnx_moe_combine(const float* part, const float* topw, const float* sh, const
 int fnx_argmax(const float* logits, int rows, int T, int v0, float* best_v, int* best_i, unsigned long long* keys, unsigned* err, void* st) {
     if (!logits || !best_v || !best_i || !keys || !err) return fail("argmax: null argument");
     if (rows < 1 || T < 1 || T > FNX_MAXT) return fail("argmax: bad shape");
-    k_argmax<<<dim3((rows + AM_PER_BLOCK - 1) / AM_PER_BLOCK, T), AM_THREADS, 0, (hipStream_t) st>>>(logits, rows, keys, err);
-    k_argmax_fin<<<1, 64, 0, (hipStream_t) st>>>(keys, T, v0, best_v, best_i);
+    k_argmax<<<dim3((rows + AM_PER_BLOCK - 1) / AM_PER_BLOCK, T), AM_THREADS, 0, (hipStream_t) st>>>(logits, rows, keys, err, v0, best_v, best_i);
     return launch_status("argmax");
 }
 
@@ -1284,7 +1287,7 @@ int fnx_swiglu_h16(const float* gu, int ffs, int P, uint16_t* h16, void* st) {
     return launch_status("swiglu_h16");
 }
 // A2 (may be null): one more matrix of the same shape and layout with a job list of its own (jobs2, njobs2, cap2), run in
-// the same launch where the kernel form can (block and tile forms), else right after
+// the same launch by the wave forms (tile16), else right after
 static int mma_launch(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const int* njobs, int njobs_cap, const uint16_t* x, float* out,
                       void* st, const char* who, const fnx_dw* A2 = nullptr, const fnx_bigjob* jobs2 = nullptr, const int* njobs2 = nullptr,
                       int cap2 = 0, uint16_t* h16 = nullptr, bool* h16_done = nullptr) {
@@ -1296,14 +1299,12 @@ static int mma_launch(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const 
     if (A->type == FNX_T_IQ3S_UNIT64 && ((size_t) A->n_out * A->n_in) % 2048) return fail(std::string(who) + ": whole units of 2048 weights");
     if (njobs_cap < 1) return fail(std::string(who) + ": no jobs");
     MmaArgs a{(const uint8_t*) A->p, sa, A->ep, A->n_out, A->n_in, jobs, njobs, njobs_cap, x, A->n_in, out};
-    static const int per_cu = env_int("FNX_MMA_BLOCKS_PER_CU", 2, 1, 8), form = env_int("FNX_MMA_FORM", 1, 0, 1);
-    static const int tile = env_int("FNX_MMA_TILE", 1, 0, 2);   // 0: never, 1: rows of up to 512 columns, 2: always
-    // (the tile form writes the products only: not where h alone is asked for)
-    const bool use_tile = tile && out && A->type == FNX_T_IQ3S_UNIT64 && A->n_out % 16 == 0 && (tile == 2 || A->n_in <= 512);
     const bool tile16 = A->type == FNX_T_IQ3S_TILE16;
-    const bool use_block = tile16 || (!use_tile && form == 1 && A->type == FNX_T_IQ3S_UNIT64 && A->n_in % 512 == 0 && A->n_out % 16 == 0);
-    const bool merged = A2 && (use_tile || use_block) && A2->p && A2->type == A->type && A2->n_in == A->n_in && A2->n_out == A->n_out;
-    if (A2 && !merged) {   // a form without the second list: two launches
+    // the wave forms (tile16) take the second list - the shared expert's matrix - in the same launch
+    const bool merged = A2 && tile16 && A2->p && A2->type == A->type && A2->n_in == A->n_in && A2->n_out == A->n_out;
+    if (A2 && !merged) {   // two launches
+        if (h16_done) *h16_done = false;
+        if (!out) return fail(std::string(who) + ": h alone is left by the wave form only (both matrices tile16)");
         if (mma_launch(A, sa, jobs, njobs, njobs_cap, x, out, st, who)) return 1;
         return mma_launch(A2, 0, jobs2, njobs2, cap2, x, out, st, who);
     }
@@ -1315,59 +1316,28 @@ static int mma_launch(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const 
         a.cap2 = cap2;
     }
     const long caps = (long) njobs_cap + (merged ? cap2 : 0);
-    // stacked gate|up matrices on the block form can leave h = silu(gate) * up themselves
     if (h16_done) *h16_done = false;
-    if (h16 && use_block && merged == (A2 != nullptr) && A->n_out % 256 == 0) {
+    if (tile16 && h16 && A->n_out % 32 == 0) {
+        // wave form for stacked gate|up matrices, which leaves h = silu(gate) * up itself: a wave a (gate tile, up tile) pair over
+        // the row's super-steps, one block a CU
         a.h16 = h16;
         a.ffh = A->n_out / 2;
         if (h16_done) *h16_done = true;
-    }
-    if (!out && !a.h16) return fail(std::string(who) + ": h alone is left by the block and wave forms only (unit64 or tile16, 2 ff rows in 256s, columns in 512s)");
-    static const int tok64 = env_int("FNX_MMA_TOK64", 1, 0, 1), wave16 = env_int("FNX_MMA_WAVE16", 1, 0, 1);
-    static const int wave16_gu = env_int("FNX_MMA_WAVE16_GU", 1, 0, 1);
-    if (tile16 && wave16_gu && a.h16 && a.ffh % 16 == 0) {
-        // wave form for stacked gate|up matrices: a wave a (gate tile, up tile) pair over the row's super-steps, one block a CU
         const long upj = (a.ffh / 16 + 7) / 8;   // the finer of its two kinds of units
         const int grid = (int) std::max(1l, std::min<long>(std::min(cu_count(), 64 * W16_PLAN), caps * upj));
         k_moe_mma_wave16_gu<<<grid, W16_THREADS, 0, (hipStream_t) st>>>(a);
         return launch_status(who);
     }
-    if (tile16 && wave16 && !a.h16 && A->n_in == W16_COLS) {
+    if (!out) return fail(std::string(who) + ": h alone is left by the wave form only (tile16 gate|up, 2 ff rows in 32s)");
+    if (tile16 && A->n_in == W16_COLS) {
         // wave form: rows of 512 columns (the down projection), a job's whole activation tile in LDS, one block a CU
         const int grid = (int) std::max(1l, std::min<long>((long) cu_count(), caps * (A->n_out / 16)));
         k_moe_mma_wave16<<<grid, W16_THREADS, 0, (hipStream_t) st>>>(a);
         return launch_status(who);
     }
-    if (use_tile && tok64) {
-        // tile form, a block per (job, its up to 64 tokens, 256 rows) in stages of 256 columns, one block a CU (its LDS)
-        const long tasks = caps * ((A->n_out + MB_ROWS - 1) / MB_ROWS);
-        const int grid = (int) std::max(1l, std::min<long>((long) cu_count(), tasks));
-        k_moe_mma_tile64<<<grid, MM_THREADS, 0, (hipStream_t) st>>>(a);
-        return launch_status(who);
-    }
-    if (use_tile) {
-        // tile form: a block per (job, 32 tokens, 256 rows) in stages of 256 columns, one block a CU (its LDS)
-        const long tasks = caps * ((A->n_out + MB_ROWS - 1) / MB_ROWS) * (MM_TT / MM_TP);
-        const int grid = (int) std::max(1l, std::min<long>((long) cu_count(), tasks));
-        k_moe_mma_tile<<<grid, MM_THREADS, 0, (hipStream_t) st>>>(a);
-        return launch_status(who);
-    }
-    if (use_block && tok64) {
-        // block form, a block per (job, its up to 64 tokens, 256 rows): one block a CU (its LDS)
-        const long tasks = caps * ((A->n_out + MB_ROWS - 1) / MB_ROWS);
-        const int grid = (int) std::max(1l, std::min<long>((long) cu_count(), tasks));
-        if (tile16) k_moe_mma_block64<true><<<grid, MM_THREADS, 0, (hipStream_t) st>>>(a);
-        else k_moe_mma_block64<false><<<grid, MM_THREADS, 0, (hipStream_t) st>>>(a);
-        return launch_status(who);
-    }
-    if (use_block) {
-        // block form: a block per (job, 32 tokens, 256 rows)
-        const long tasks = caps * ((A->n_out + MB_ROWS - 1) / MB_ROWS) * (MM_TT / MM_TP);
-        const int grid = (int) std::max(1l, std::min<long>((long) per_cu * cu_count(), tasks));
-        if (tile16) k_moe_mma_block<true><<<grid, MM_THREADS, 0, (hipStream_t) st>>>(a);
-        else k_moe_mma_block<false><<<grid, MM_THREADS, 0, (hipStream_t) st>>>(a);
-        return launch_status(who);
-    }
+    if (tile16) return fail(std::string(who) + ": tile16 matrices are the prompt path's two: stacked gate|up leaving h, and rows of 512 columns");
+    // raw blocks and unit64: a wave a task of 32 rows x 32 tokens
+    static const int per_cu = env_int("FNX_MMA_BLOCKS_PER_CU", 2, 1, 8);
     const long tasks = (long) njobs_cap * (A->n_out / 32) * (MM_TT / MM_TP);
     const int grid = (int) std::max(1l, std::min<long>((long) per_cu * cu_count(), (tasks + MM_WAVES - 1) / MM_WAVES));
     if (A->type == FNX_T_IQ3S_UNIT64) k_moe_mma<true, 2><<<grid, MM_THREADS, 0, (hipStream_t) st>>>(a);
@@ -1608,11 +1578,14 @@ static int dec_shape_check(const fnx_decoder* D, int T, const char* who) {
     return 0;
 }
 // x += pending; hidden = x; the output norm, the head, argmax
+// nv head rows for the tokens from v0; pen (may be null): the last row's penalty list, applied before the picks (engine.cu:2130-2131)
 static int dec_head(const fnx_decoder* D, const float* norm, const fnx_q8s* head, int T, const fnx_dec_ws* ws, const DecPending& pend, void* st,
-                    const int* gate = nullptr) {
+                    const int* gate = nullptr, int nv = 0, int v0 = 0, const int* pen = nullptr, const float* pen_par = nullptr) {
+    if (nv == 0) nv = D->vocab;
     if (dec_add_norm_q8(D, pend, norm, T, ws, st, ws->hidden, gate)) return 1;   // hidden = x, written by the same pass
-    if (q8s_one(head, ws->xq, ws->logits, D->vocab, T, st, gate)) return 1;
-    return fnx_argmax(ws->logits, D->vocab, T, 0, ws->best_v, ws->best_i, ws->keys, ws->err, st);
+    if (q8s_one(head, ws->xq, ws->logits, nv, T, st, gate)) return 1;
+    if (pen && fnx_penalize_row(ws->logits + (size_t) (T - 1) * nv, nv, pen, pen_par, st)) return 1;
+    return fnx_argmax(ws->logits, nv, T, v0, ws->best_v, ws->best_i, ws->keys, ws->err, st);
 }
 static int decoder_verify(const fnx_decoder* D, const int* tokens, int T, const int* pos0, const fnx_dec_ws* ws, void* st, const int* live) {
     if (!D || !tokens || !pos0 || !ws || !D->layers || !D->out_norm || !D->emb) return fail("decoder_verify: null argument");
@@ -1637,6 +1610,11 @@ static int mtp_draft(const fnx_decoder* D, const fnx_mtp* M, const float* src, c
                      void* st, const int* live, const int* gate = nullptr) {
     if (!D || !M || !src || !tokens || !pos0 || !ws || !M->norm_emb || !M->norm_hid || !M->out_norm || !D->emb) return fail("mtp_draft: null argument");
     if (dec_shape_check(D, T, "mtp_draft") || dec_ws_check(ws, "mtp_draft")) return 1;
+    const bool whole = M->dv0 == 0 && M->dv1 == 0;
+    if (!whole && (M->dv0 < 0 || M->dv1 <= M->dv0 || M->dv1 > D->vocab)) return fail("mtp_draft: the head's tokens [dv0, dv1) must lie in the vocabulary");
+    const int nv = whole ? D->vocab : M->dv1 - M->dv0;
+    if (M->head.n_out != nv) return fail("mtp_draft: the head has one row a token of [dv0, dv1)");
+    if (M->pen && !M->pen_par) return fail("mtp_draft: a penalty list without its parameters");
     const int n = D->n;
     // R = fc_hid(rms(src)) + fc_emb(rms(emb)): the sum is taken by the layer's first pass over the rows
     {   // nothing to add: src is only read (fnx_add_norm_q8)
@@ -1658,7 +1636,7 @@ static int mtp_draft(const fnx_decoder* D, const fnx_mtp* M, const float* src, c
     if (q8s_one(&M->fc_emb, ws->xq, ws->o, n, T, st, gate)) return 1;
     DecPending pend{ws->o, nullptr, nullptr};
     if (dec_layer(D, &M->layer, T, pos0, ws, pend, st, live, gate)) return 1;
-    return dec_head(D, M->out_norm, &M->head, T, ws, pend, st, gate);
+    return dec_head(D, M->out_norm, &M->head, T, ws, pend, st, gate, nv, M->dv0, M->pen, M->pen_par);
 }
 int fnx_mtp_draft(const fnx_decoder* D, const fnx_mtp* M, const float* src, const int* tokens, int T, const int* pos0, const fnx_dec_ws* ws,
                   void* st) {

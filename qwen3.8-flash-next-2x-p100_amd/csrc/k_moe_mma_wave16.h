@@ -1,16 +1,16 @@
 // The routed experts' down projection on the matrix cores over tile16 matrices of 512 columns, a wave a tile of 16 rows.
 //
-// The block and tile forms give a block one (job, 256 rows) task at a time and every stage of it two barriers: with rows
-// of 512 columns a task is a single stage, the eight waves of a block meet four times per 32 rows each, and at two waves
-// a SIMD little covers the codebook lookups' latency. Here the whole activation tile of a job - up to 64 tokens x 512
+// A block that takes one (job, 256 rows) task at a time, its activations staged per step, meets at two barriers a stage:
+// with rows of 512 columns a task is a single stage, the eight waves of such a block meet four times per 32 rows each, and
+// at two waves a SIMD little covers the codebook lookups' latency. Here the whole activation tile of a job - up to 64 tokens x 512
 // columns of f16, 64 KiB - is put in LDS once (by loads that write LDS directly, a token's row per wave instruction), and
 // after that a wave needs nothing from the others: it takes tiles of 16 rows, a lane decodes its four sub-blocks of its
 // row from one contiguous load of the tile16 layout, and the sixteen waves of a block (four a SIMD) meet only where the
 // block goes from one job to the next. The blocks split the (job, sixteen tiles) units of all jobs by cost - a tile's
 // decode and its job's token tiles of multiplications - into contiguous runs.
 // part[job.out[t]][row] = W[job.w][row] . h16[job.y[t]] as kernels.hpp:330 (moe_down_mma) defines it, with the weights as
-// f16 (d (1 + 2 s) g, each product rounded as k_moe_mma_block64 rounds it) and a row's sub-blocks accumulated in the order
-// of that kernel's steps.
+// f16 (d (1 + 2 s) g, the f32 value rounded once, as k_moe_mma rounds it) and a row's sub-blocks accumulated super-step by
+// super-step (S, then the four steps, then a step's four operands).
 #pragma once
 
 #include "k_prefill.h"
@@ -239,8 +239,8 @@ __global__ void __launch_bounds__(W16_THREADS) k_moe_mma_wave16(const MmaArgs a)
 // to and fro over the blocks, and the jobs of up to 16 tokens cut finer - eight pairs a unit, a wave a single tile, all S
 // tiles of the 16 tokens in LDS at once, the up tiles' sums handed to the gate tiles' waves through LDS - and spread so
 // that every block comes near the mean load. The weights of the next tile's super-step are asked for a tile ahead. Every
-// tile is accumulated in the block form's order (S, then the four steps, then a step's four operands): h has the bits
-// of k_moe_mma_block64's whatever a job's size.
+// tile is accumulated in one order (S, then the four steps, then a step's four operands) whatever a job's size or the
+// unit it falls in: a row's h does not depend on what else is in the chunk.
 constexpr int W16_SORTJ = 1024, W16_GU_HELD = 1024, W16_PLAN = 4;   // (W16_PLAN: blocks a lane of the planning wave looks after)
 struct Wave16GuLds {
     uint2 tab[SGRID_WORDS];

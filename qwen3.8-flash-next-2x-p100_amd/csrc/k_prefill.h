@@ -508,12 +508,12 @@ struct MmaArgs {
     int ldx;
     float* out;             // rows of nrows
     // a second job list over one more matrix (the shared expert's, whatever its jobs' w says), in the same launch: alone
-    // its few jobs fill a quarter of the chip (block and tile forms)
+    // its few jobs fill a quarter of the chip (the wave forms)
     const uint8_t* w2 = nullptr;
     const fnx_bigjob* jobs2 = nullptr;
     const int* njobs2 = nullptr;
     int cap2 = 0;
-    // block form, stacked gate|up matrices (nrows = 2 ffh, ffh in 128s): a wave's two row groups are 16 gate rows and the
+    // wave form, stacked gate|up matrices (nrows = 2 ffh, ffh in 16s): a wave's two tiles are 16 gate rows and the
     // 16 up rows that go with them, and what is written is h = silu(gate) * up as f16 rows of ffh (k_swiglu_h16's values)
     // instead of the products themselves
     uint16_t* h16 = nullptr;
@@ -675,16 +675,12 @@ __global__ void __launch_bounds__(MM_THREADS) __attribute__((amdgpu_waves_per_eu
     }
 }
 
-// ---------------------------------------------------------------- the same products, block form (unit64 weights, ncols % 512 == 0)
-// What limits the wave form above on MI355X is the vector-memory front end: every wave gathers its own activation
-// operands from 16 rows and its weights 32 bytes per row at a time, so each cache line is fetched four times and the
-// L1 sees a thousand lane accesses per k-step. Here a block of 8 waves takes one (job, 32 tokens, 256 weight rows):
-//   * the step's activation tile (32 tokens x 128 k, 8 KiB) is loaded once per block, one 16-byte load per thread,
-//     into LDS (rows padded to 272 bytes: conflict-free 16-byte operand reads), double-buffered: one barrier a step;
-//   * a lane owns four consecutive sub-blocks of its row per super-step of 512 k (sub-block 16 S + 4 g + p at step p),
-//     so its weight loads are whole 32/16/4/2-byte runs of the planes: 6 loads per row group and super-step, each
-//     line of a plane touched once; the next super-step's loads are issued a super-step ahead.
-constexpr int MB_RG = 2, MB_ROWS = MM_WAVES * 16 * MB_RG, MB_TOK = 16 * MM_TP, MB_XLD = 272;   // bytes per LDS activation row
+// ---------------------------------------------------------------- a lane's four consecutive sub-blocks of a row
+// What limits the wave-a-task kernel above on MI355X is the vector-memory front end: every wave gathers its weights 32
+// bytes per row at a time, so each cache line is fetched four times. A lane that owns four consecutive sub-blocks of its
+// row per super-step of 512 columns (sub-block 16 S + 4 g + p at step p) loads whole 32/16/4/2-byte runs of the planes,
+// 6 loads per row and super-step, each line of a plane touched once: the loads of the tile16 re-laying below and of the
+// wave forms (k_moe_mma_wave16.h), which read the same fields from the tile16 layout.
 struct SuperFields {   // a lane's four sub-blocks of one row as loaded
     v4u a0, a1, b;
     uint32_t c, sc, d;
@@ -738,7 +734,7 @@ __device__ __forceinline__ SuperFields tile16_load(const uint8_t* __restrict__ w
     r.d = *(g16*) (u + TILE16_D_AT + 2 * lane);
     return r;
 }
-// unit64 -> tile16 (once, at load; out of place): a wave a tile, every lane reads its share the way the block form does
+// unit64 -> tile16 (once, at load; out of place): a wave a tile, every lane reads its four sub-blocks of its row
 __global__ void __launch_bounds__(256) k_iq3s_tile16(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst, int nrows, int ncols, long tiles) {
     const long t = (long) blockIdx.x * 4 + (threadIdx.x >> 6);
     if (t >= tiles) return;
@@ -756,1067 +752,7 @@ __global__ void __launch_bounds__(256) k_iq3s_tile16(const uint8_t* __restrict__
     *reinterpret_cast<unsigned short*>(u + TILE16_SC_AT + 2 * lane) = (unsigned short) f.sc;
     *reinterpret_cast<unsigned short*>(u + TILE16_D_AT + 2 * lane) = (unsigned short) f.d;
 }
-constexpr int MB_XROW = 4 * MB_XLD + 16;   // a token's four step pieces of a super-step (+16: the 16 tokens of a tile fall on different banks)
-constexpr int MB_MAXTASK = 16;
-struct BlockTask {
-    const uint8_t* we;
-    int t0, rb, ntile;   // first token tile, row block, token tiles (1 or 2)
-    int ji, n;           // the job (an index into both lists, the second list after the first) and its tokens
-};
-struct MmaLds {
-    uint2 tab[SGRID_WORDS];
-    uint8_t xt[2][MB_TOK * MB_XROW];   // [buffer][token][step p][lane group g][64 bytes], step rows padded to 272 bytes
-    // the block's tasks (the valid ones only), their tokens' activation rows (clamped to the job's last) and output rows
-    // (-1 past the job's end): read once when the kernel starts, so that a task begins without a chain of dependent loads
-    int ytok[MB_MAXTASK][MB_TOK];
-    int otok[MB_MAXTASK][MB_TOK];
-    BlockTask task[MB_MAXTASK];
-    int ntask;
-};
-template <bool TILE16>
-__global__ void __launch_bounds__(MM_THREADS) k_moe_mma_block(const MmaArgs a) {
-    typedef __attribute__((address_space(1))) const v4u gx4;
-    __shared__ MmaLds L;
-    const uint32_t tab0 = g_sgrid.v[threadIdx.x];   // (512 threads: a thread's code, its sixteen signed entries made here)
-#pragma unroll
-    for (int i = threadIdx.x; i < SGRID_WORDS; i += MM_THREADS) {
-        const uint32_t g = signed_entry(tab0, i >> 9);
-        v2h lo, hi;
-        lo.x = (_Float16) (int) (int8_t) (g & 0xFFu);
-        lo.y = (_Float16) (int) (int8_t) ((g >> 8) & 0xFFu);
-        hi.x = (_Float16) (int) (int8_t) ((g >> 16) & 0xFFu);
-        hi.y = (_Float16) (int) (int8_t) (g >> 24);
-        L.tab[i] = make_uint2(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi));
-    }
-    const int tid = threadIdx.x, lane = tid & 63, wave = uniform(tid >> 6), r = lane & 15, g = lane >> 4;
-    const int nj = min(a.cap, uniform(*a.njobs)), nj2 = a.jobs2 ? min(a.cap2, uniform(*a.njobs2)) : 0;
-    const int ks = a.ncols >> 5, nsuper = ks >> 4, rblocks = (a.nrows + MB_ROWS - 1) / MB_ROWS;
-    constexpr int HALVES = MM_TT / MM_TP;
-    const int per_job = rblocks * HALVES, ntasks_all = (nj + nj2) * per_job;
-    // this thread's share of a super-step's activation tile (32 tokens x 512 k): token xtok, 64 contiguous bytes
-    // (sub-block xsb of the 16); in LDS the sub-block 4 g + p goes to step p, lane group g
-    const int xtok = tid >> 4, xsb = tid & 15;
-    const int xdst = xtok * MB_XROW + (xsb & 3) * MB_XLD + (xsb >> 2) * 64;
-    const int rlimit = a.h16 ? a.ffh : a.nrows, qstep = a.h16 ? a.ffh : 16;
-    struct XShare {
-        v4u v[4];
-    };
-    auto x_store = [&](const XShare& t, int buf) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) *reinterpret_cast<v4u*>(&L.xt[buf][xdst + 16 * i]) = t.v[i];
-    };
-    for (int k0 = blockIdx.x; k0 < ntasks_all; k0 += gridDim.x * MB_MAXTASK) {
-        __syncthreads();   // the previous lists' and tiles' last readers; the table on the first pass
-        if (wave == 0) {
-            const int task = k0 + lane * gridDim.x;
-            bool ok = lane < MB_MAXTASK && task < ntasks_all;
-            BlockTask t{};
-            int ji = 0, n = 0;
-            if (ok) {
-                ji = task / per_job;
-                const int rem = task - ji * per_job;
-                t.t0 = (rem / rblocks) * MM_TP;
-                t.rb = rem % rblocks;
-                const fnx_bigjob* jb = ji < nj ? a.jobs + ji : a.jobs2 + (ji - nj);
-                n = min(FNX_PF_JOB, jb->n);
-                const int e = jb->w;
-                ok = n >= 1 && t.t0 < ((n + 15) >> 4);
-                t.ntile = min(MM_TP, ((n + 15) >> 4) - t.t0);
-                if (ok) t.we = ji >= nj ? a.w2 : a.ep ? (const uint8_t*) a.ep[e] : a.w + (size_t) e * a.stride;
-            }
-            const unsigned long long m = __ballot(ok);
-            const int slot = __popcll(m & ((1ull << lane) - 1ull));
-            if (ok) {
-                t.ji = ji;
-                t.n = n;
-                L.task[slot] = t;
-            }
-            if (lane == 0) L.ntask = __popcll(m);
-        }
-        __syncthreads();
-        const int ntask = L.ntask;
-        if (ntask == 0) continue;   // the same for every thread of the block
-        for (int i = tid; i < ntask * MB_TOK; i += MM_THREADS) {   // the tiles' token and output rows, all at once
-            const int slot = i / MB_TOK, j = i % MB_TOK, ji = L.task[slot].ji, n = L.task[slot].n, tok = L.task[slot].t0 * 16 + j;
-            const fnx_bigjob* jb = ji < nj ? a.jobs + ji : a.jobs2 + (ji - nj);
-            L.ytok[slot][j] = jb->y[min(tok, n - 1)];
-            L.otok[slot][j] = tok < n ? jb->out[tok] : -1;
-        }
-        __syncthreads();
-        const int nst = ntask * nsuper;
-        // the wave's first row in task ti: of its 32 consecutive rows, or (h16) of its 16 gate rows - the up rows lie ffh further
-        auto row0_of = [&](int ti) { return a.h16 ? L.task[ti].rb * (MB_ROWS / 2) + wave * 16 : L.task[ti].rb * MB_ROWS + wave * 16 * MB_RG; };
-        // a stage's loads: this thread's share of the activation tile and its lane's fields of both row groups
-        auto x_load = [&](int ti, int S) {
-            XShare t;
-            const gx4* p = (gx4*) (uintptr_t) (a.x + (size_t) L.ytok[ti][xtok] * a.ldx + 32 * xsb + 512 * S);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) t.v[i] = p[i];
-            return t;
-        };
-        auto w_load_q = [&](int ti, int S, int q, SuperFields& o) {
-            const int row = min(row0_of(ti) + qstep * q + r, a.nrows - 1);
-            if constexpr (TILE16) o = tile16_load(L.task[ti].we, row, S, nsuper);
-            else o = super_load(L.task[ti].we, row, 16 * S + 4 * g, ks);
-        };
-        auto w_load = [&](int ti, int S, SuperFields (&o)[MB_RG]) {
-#pragma unroll
-            for (int q = 0; q < MB_RG; ++q) w_load_q(ti, S, q, o[q]);
-        };
-        v4f acc[MB_RG][MM_TP];
-#pragma unroll
-        for (int q = 0; q < MB_RG; ++q)
-#pragma unroll
-            for (int tt = 0; tt < MM_TP; ++tt) acc[q][tt] = v4f{0.f, 0.f, 0.f, 0.f};
-        // nt_tag: the task's token tiles (1 or 2) as a constant: a lone tile's task reads and multiplies half as much
-        auto step = [&](const SubFields (&cur)[MB_RG], int buf, int p, auto nt_tag) {
-            constexpr int NT = decltype(nt_tag)::value;
-            v4u B[MM_TP][4];
-#pragma unroll
-            for (int tt = 0; tt < NT; ++tt)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) B[tt][i] = *reinterpret_cast<const v4u*>(&L.xt[buf][(tt * 16 + r) * MB_XROW + p * MB_XLD + 64 * g + 16 * i]);
-#pragma unroll
-            for (int q = 0; q < MB_RG; ++q) {
-                v8h A[4];
-                const _Float16 sc = (_Float16) (int) (1 + 2 * cur[q].sc), d = __builtin_bit_cast(_Float16, (unsigned short) cur[q].d);
-                const v2h s2 = {sc, sc}, d2 = {d, d};
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const uint2 en = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint8_t*>(L.tab) + sub_entry<true>(cur[q], j));
-                    const v2h lo = (as_v2h(en.x) * s2) * d2, hi = (as_v2h(en.y) * s2) * d2;
-                    A[j >> 1][4 * (j & 1) + 0] = lo.x;
-                    A[j >> 1][4 * (j & 1) + 1] = lo.y;
-                    A[j >> 1][4 * (j & 1) + 2] = hi.x;
-                    A[j >> 1][4 * (j & 1) + 3] = hi.y;
-                }
-#pragma unroll
-                for (int tt = 0; tt < NT; ++tt)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i)
-                        acc[q][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[i], __builtin_bit_cast(v8h, B[tt][i]), acc[q][tt], 0, 0, 0);
-            }
-        };
-        // pre(p): what the caller wants issued before step p (the next stage's loads, a part before each of the first steps,
-        // so that the waves' loads do not queue up behind one another at the stage's start)
-        auto steps4 = [&](SuperFields (&cur)[MB_RG], int buf, auto nt_tag, auto pre) {
-            SubFields c[MB_RG];
-            pre(0);
-#pragma unroll
-            for (int q = 0; q < MB_RG; ++q) c[q] = super_sub<0>(cur[q]);
-            step(c, buf, 0, nt_tag);
-            pre(1);
-#pragma unroll
-            for (int q = 0; q < MB_RG; ++q) c[q] = super_sub<1>(cur[q]);
-            step(c, buf, 1, nt_tag);
-            pre(2);
-#pragma unroll
-            for (int q = 0; q < MB_RG; ++q) c[q] = super_sub<2>(cur[q]);
-            step(c, buf, 2, nt_tag);
-#pragma unroll
-            for (int q = 0; q < MB_RG; ++q) c[q] = super_sub<3>(cur[q]);
-            step(c, buf, 3, nt_tag);
-        };
-        // Stage s = (task ti, super-step S) of the block's sequence: the next stage's loads - the next task's first ones
-        // too - are issued before this stage's arithmetic, its tile goes to the other LDS buffer after it: one barrier a stage
-        int ti = 0, S = 0;
-        auto stage = [&](SuperFields (&cur)[MB_RG], SuperFields (&nxt)[MB_RG], int s) {
-            const int buf = s & 1;
-            int tn = ti, Sn = S + 1;
-            if (Sn == nsuper) {
-                Sn = 0;
-                ++tn;
-            }
-            const bool more = s + 1 < nst;
-            XShare xn;
-            auto pre = [&](int p) {   // the weights (from HBM) first, the activations (cached) last
-                if (!more) return;
-                if (p < MB_RG) w_load_q(tn, Sn, p, nxt[p]);
-                else if (p == MB_RG) xn = x_load(tn, Sn);
-            };
-            const int row0 = row0_of(ti);
-            if (row0 < rlimit) {   // per wave
-                if (L.task[ti].ntile > 1) steps4(cur, buf, std::integral_constant<int, 2>{}, pre);
-                else steps4(cur, buf, std::integral_constant<int, 1>{}, pre);
-                if (Sn == 0) {   // the task's last super-step: lane = token r of each tile, weight rows 4 g .. 4 g + 3 of each group
-#pragma unroll
-                    for (int tt = 0; tt < MM_TP; ++tt) {
-                        const int orow = L.otok[ti][tt * 16 + r];
-                        if (orow >= 0) {
-                            if (a.h16) {   // gate rows in acc[0], their up rows in acc[1]
-                                const v4f gt = acc[0][tt], up = acc[1][tt];
-                                uint2 hv;
-                                hv.x = (uint32_t) float_to_half_bits(silu_f(gt.x) * up.x) | (uint32_t) float_to_half_bits(silu_f(gt.y) * up.y) << 16;
-                                hv.y = (uint32_t) float_to_half_bits(silu_f(gt.z) * up.z) | (uint32_t) float_to_half_bits(silu_f(gt.w) * up.w) << 16;
-                                *reinterpret_cast<uint2*>(a.h16 + (size_t) orow * a.ffh + row0 + 4 * g) = hv;
-                            } else {
-                                float* o = a.out + (size_t) orow * a.nrows + row0 + 4 * g;
-#pragma unroll
-                                for (int q = 0; q < MB_RG; ++q)
-                                    if (row0 + 16 * q < a.nrows)
-                                        *reinterpret_cast<float4*>(o + 16 * q) = make_float4(acc[q][tt].x, acc[q][tt].y, acc[q][tt].z, acc[q][tt].w);
-                            }
-                        }
-                    }
-#pragma unroll
-                    for (int q = 0; q < MB_RG; ++q)
-#pragma unroll
-                        for (int tt = 0; tt < MM_TP; ++tt) acc[q][tt] = v4f{0.f, 0.f, 0.f, 0.f};
-                }
-            } else {
-#pragma unroll
-                for (int p = 0; p <= MB_RG; ++p) pre(p);
-            }
-            if (more) x_store(xn, buf ^ 1);
-            __syncthreads();
-            ti = tn;
-            S = Sn;
-        };
-        SuperFields w0[MB_RG], w1[MB_RG];
-        {
-            const XShare x0 = x_load(0, 0);
-            w_load(0, 0, w0);
-            x_store(x0, 0);
-        }
-        __syncthreads();
-        for (int s = 0; s < nst; s += 2) {
-            stage(w0, w1, s);
-            if (s + 1 < nst) stage(w1, w0, s + 1);
-        }
-    }
-}
-
-// ---------------------------------------------------------------- block form, a task = (job, all of its up to 64 tokens, 256 weight rows)
-// kernels.hpp:27-30 (PF_JOB): "the expert's weight tile is then dequantized once for twice the tokens". The form above
-// decodes a sub-block once per 32 tokens, so a job of 33 to 64 tokens decodes every weight twice, and the codebook
-// lookups are what the launch waits for most. Here a lane's decoded operands of both row groups serve up to four token
-// tiles, two at a time (their B operands share registers). The 64-token activation tile takes the LDS of the two
-// 32-token buffers: it is replaced between two barriers at the end of a stage, its loads issued before the stage's last step.
+// tokens of a job's tile that the wave forms (k_moe_mma_wave16.h) multiply at a time: four tiles of 16
 constexpr int MB_TP = 4, MB_TOK64 = 16 * MB_TP;
-constexpr int MB_SORTJ = 1024;   // jobs up to which the tasks are dealt by size
-struct MmaLds64 {
-    uint2 tab[SGRID_WORDS];
-    uint8_t xt[MB_TOK64 * MB_XROW];   // [token][step p][lane group g][64 bytes], step rows padded to 272 bytes
-    int ytok[MB_MAXTASK][MB_TOK64];
-    int otok[MB_MAXTASK][MB_TOK64];
-    BlockTask task[MB_MAXTASK];
-    int ntask;
-    uint8_t jkey[MB_SORTJ];            // a job's token tiles (0: no tokens)
-    unsigned short jorder[MB_SORTJ];   // the jobs, most token tiles first (the lower index first among equals)
-};
-template <bool TILE16>
-__global__ void __launch_bounds__(MM_THREADS) k_moe_mma_block64(const MmaArgs a) {
-    typedef __attribute__((address_space(1))) const v4u gx4;
-    __shared__ MmaLds64 L;
-    const uint32_t tab0 = g_sgrid.v[threadIdx.x];   // (512 threads: a thread's code, its sixteen signed entries made here)
-#pragma unroll
-    for (int i = threadIdx.x; i < SGRID_WORDS; i += MM_THREADS) {
-        const uint32_t g = signed_entry(tab0, i >> 9);
-        v2h lo, hi;
-        lo.x = (_Float16) (int) (int8_t) (g & 0xFFu);
-        lo.y = (_Float16) (int) (int8_t) ((g >> 8) & 0xFFu);
-        hi.x = (_Float16) (int) (int8_t) ((g >> 16) & 0xFFu);
-        hi.y = (_Float16) (int) (int8_t) (g >> 24);
-        L.tab[i] = make_uint2(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi));
-    }
-    const int tid = threadIdx.x, lane = tid & 63, wave = uniform(tid >> 6), r = lane & 15, g = lane >> 4;
-    const int nj = min(a.cap, uniform(*a.njobs)), nj2 = a.jobs2 ? min(a.cap2, uniform(*a.njobs2)) : 0;
-    const int ks = a.ncols >> 5, nsuper = ks >> 4, rblocks = (a.nrows + MB_ROWS - 1) / MB_ROWS;
-    constexpr int HALVES = 1;   // a task takes all of a job's token tiles
-    const int per_job = rblocks * HALVES, ntasks_all = (nj + nj2) * per_job;
-    // this thread's share of a super-step's activation tile (64 tokens x 512 k): tokens xtok and xtok + 32, 64 contiguous
-    // bytes each (sub-block xsb of the 16); in LDS the sub-block 4 g + p goes to step p, lane group g
-    const int xtok = tid >> 4, xsb = tid & 15;
-    const int xdst = xtok * MB_XROW + (xsb & 3) * MB_XLD + (xsb >> 2) * 64;
-    const int rlimit = a.h16 ? a.ffh : a.nrows, qstep = a.h16 ? a.ffh : 16;
-    struct XShare {
-        v4u v[8];
-    };
-    auto x_store = [&](const XShare& t) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            *reinterpret_cast<v4u*>(&L.xt[xdst + 16 * i]) = t.v[i];
-            *reinterpret_cast<v4u*>(&L.xt[xdst + 32 * MB_XROW + 16 * i]) = t.v[4 + i];
-        }
-    };
-    // A job's cost grows with its token tiles and a block gets two or three tasks of a chunk's few hundred: dealt in list
-    // order the slowest block took 84 us where the average took 58. So every block ranks the jobs by token tiles (the same
-    // order in every block: a job's rank is the count of jobs ahead of it) and the tasks are dealt in that order, to and
-    // fro over the blocks, the heaviest first.
-    const int njall = nj + nj2;
-    const bool sorted = njall <= MB_SORTJ;
-    if (sorted && wave == 0) {   // a counting sort by one wave, 64 jobs a trip: class totals, then every job's place
-        auto key_of = [&](int j) {
-            if (j >= njall) return -1;
-            const fnx_bigjob* jb = j < nj ? a.jobs + j : a.jobs2 + (j - nj);
-            return min(MB_TP, (max(0, min(FNX_PF_JOB, jb->n)) + 15) >> 4);
-        };
-        int total[MB_TP + 1];
-#pragma unroll
-        for (int c = 0; c <= MB_TP; ++c) total[c] = 0;
-        for (int j0 = 0; j0 < njall; j0 += 64) {
-            const int kj = key_of(j0 + lane);
-            if (j0 + lane < njall) L.jkey[j0 + lane] = (uint8_t) kj;
-#pragma unroll
-            for (int c = 0; c <= MB_TP; ++c) total[c] += __popcll(__ballot(kj == c));
-        }
-        int base[MB_TP + 1];   // where a class starts: the classes in descending order
-        base[MB_TP] = 0;
-#pragma unroll
-        for (int c = MB_TP - 1; c >= 0; --c) base[c] = base[c + 1] + total[c + 1];
-        for (int j0 = 0; j0 < njall; j0 += 64) {
-            const int kj = j0 + lane < njall ? (int) L.jkey[j0 + lane] : -1;
-#pragma unroll
-            for (int c = 0; c <= MB_TP; ++c) {
-                const unsigned long long m = __ballot(kj == c);
-                if (kj == c) L.jorder[base[c] + __popcll(m & ((1ull << lane) - 1ull))] = (unsigned short) (j0 + lane);
-                base[c] += __popcll(m);
-            }
-        }
-    }
-    for (int k0 = 0; k0 * (int) gridDim.x < ntasks_all; k0 += MB_MAXTASK) {   // MB_MAXTASK rounds a pass
-        __syncthreads();   // the previous lists' and tiles' last readers; the table and the jobs' order on the first pass
-        if (wave == 0) {
-            // this block's round k0 + lane: rounds go to and fro over the blocks
-            const int round = k0 + lane, pos = (round & 1) ? (int) gridDim.x - 1 - (int) blockIdx.x : (int) blockIdx.x;
-            const int task = round * (int) gridDim.x + pos;
-            bool ok = lane < MB_MAXTASK && task < ntasks_all;
-            BlockTask t{};
-            int ji = 0, n = 0;
-            if (ok) {
-                ji = task / per_job;
-                const int rem = task - ji * per_job;
-                if (sorted) ji = L.jorder[ji];
-                t.t0 = 0;
-                t.rb = rem % rblocks;
-                const fnx_bigjob* jb = ji < nj ? a.jobs + ji : a.jobs2 + (ji - nj);
-                n = min(FNX_PF_JOB, jb->n);
-                const int e = jb->w;
-                ok = n >= 1 && t.t0 < ((n + 15) >> 4);
-                t.ntile = min(MB_TP, (n + 15) >> 4);
-                if (ok) t.we = ji >= nj ? a.w2 : a.ep ? (const uint8_t*) a.ep[e] : a.w + (size_t) e * a.stride;
-            }
-            const unsigned long long m = __ballot(ok);
-            const int slot = __popcll(m & ((1ull << lane) - 1ull));
-            if (ok) {
-                t.ji = ji;
-                t.n = n;
-                L.task[slot] = t;
-            }
-            if (lane == 0) L.ntask = __popcll(m);
-        }
-        __syncthreads();
-        const int ntask = L.ntask;
-        if (ntask == 0) continue;   // the same for every thread of the block
-        for (int i = tid; i < ntask * MB_TOK64; i += MM_THREADS) {   // the tiles' token and output rows, all at once
-            const int slot = i / MB_TOK64, j = i % MB_TOK64, ji = L.task[slot].ji, n = L.task[slot].n, tok = L.task[slot].t0 * 16 + j;
-            const fnx_bigjob* jb = ji < nj ? a.jobs + ji : a.jobs2 + (ji - nj);
-            L.ytok[slot][j] = jb->y[min(tok, n - 1)];
-            L.otok[slot][j] = tok < n ? jb->out[tok] : -1;
-        }
-        __syncthreads();
-        const int nst = ntask * nsuper;
-        // the wave's first row in task ti: of its 32 consecutive rows, or (h16) of its 16 gate rows - the up rows lie ffh further
-        auto row0_of = [&](int ti) { return a.h16 ? L.task[ti].rb * (MB_ROWS / 2) + wave * 16 : L.task[ti].rb * MB_ROWS + wave * 16 * MB_RG; };
-        // a stage's loads: this thread's share of the activation tile and its lane's fields of both row groups
-        auto x_load = [&](int ti, int S) {
-            XShare t{};
-            // only the token tiles the task has: a job of up to 16 tokens asks for a quarter of the tile
-            const int ntok = 16 * L.task[ti].ntile;
-            const gx4* p = (gx4*) (uintptr_t) (a.x + (size_t) L.ytok[ti][xtok] * a.ldx + 32 * xsb + 512 * S);
-            const gx4* q = (gx4*) (uintptr_t) (a.x + (size_t) L.ytok[ti][xtok + 32] * a.ldx + 32 * xsb + 512 * S);
-            if (xtok < ntok) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i) t.v[i] = p[i];
-            }
-            if (xtok + 32 < ntok) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i) t.v[4 + i] = q[i];
-            }
-            return t;
-        };
-        auto w_load_q = [&](int ti, int S, int q, SuperFields& o) {
-            const int row = min(row0_of(ti) + qstep * q + r, a.nrows - 1);
-            if constexpr (TILE16) o = tile16_load(L.task[ti].we, row, S, nsuper);
-            else o = super_load(L.task[ti].we, row, 16 * S + 4 * g, ks);
-        };
-        auto w_load = [&](int ti, int S, SuperFields (&o)[MB_RG]) {
-#pragma unroll
-            for (int q = 0; q < MB_RG; ++q) w_load_q(ti, S, q, o[q]);
-        };
-        v4f acc[MB_RG][MB_TP];
-#pragma unroll
-        for (int q = 0; q < MB_RG; ++q)
-#pragma unroll
-            for (int tt = 0; tt < MB_TP; ++tt) acc[q][tt] = v4f{0.f, 0.f, 0.f, 0.f};
-        // nt_tag: the task's token tiles (1 or 2) as a constant: a lone tile's task reads and multiplies half as much
-        // the token tiles two at a time against both row groups' operands: a sub-block is decoded once for up to 64 tokens
-        auto pair = [&](const v8h (&A)[MB_RG][4], int p, auto t0_tag, auto cnt_tag) {
-            constexpr int T0 = decltype(t0_tag)::value, CNT = decltype(cnt_tag)::value;
-            v4u B[2][4];
-#pragma unroll
-            for (int tt = 0; tt < CNT; ++tt)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) B[tt][i] = *reinterpret_cast<const v4u*>(&L.xt[((T0 + tt) * 16 + r) * MB_XROW + p * MB_XLD + 64 * g + 16 * i]);
-#pragma unroll
-            for (int q = 0; q < MB_RG; ++q)
-#pragma unroll
-                for (int tt = 0; tt < CNT; ++tt)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i)
-                        acc[q][T0 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[q][i], __builtin_bit_cast(v8h, B[tt][i]), acc[q][T0 + tt], 0, 0, 0);
-        };
-        auto step = [&](const SubFields (&cur)[MB_RG], int p, int nt) {
-            v8h A[MB_RG][4];
-#pragma unroll
-            for (int q = 0; q < MB_RG; ++q) {
-                const _Float16 sc = (_Float16) (int) (1 + 2 * cur[q].sc), d = __builtin_bit_cast(_Float16, (unsigned short) cur[q].d);
-                const v2h s2 = {sc, sc}, d2 = {d, d};
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const uint2 en = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint8_t*>(L.tab) + sub_entry<true>(cur[q], j));
-                    const v2h lo = (as_v2h(en.x) * s2) * d2, hi = (as_v2h(en.y) * s2) * d2;
-                    A[q][j >> 1][4 * (j & 1) + 0] = lo.x;
-                    A[q][j >> 1][4 * (j & 1) + 1] = lo.y;
-                    A[q][j >> 1][4 * (j & 1) + 2] = hi.x;
-                    A[q][j >> 1][4 * (j & 1) + 3] = hi.y;
-                }
-            }
-            using I0 = std::integral_constant<int, 0>;
-            using I1 = std::integral_constant<int, 1>;
-            using I2 = std::integral_constant<int, 2>;
-            if (nt >= 2) pair(A, p, I0{}, I2{});
-            else pair(A, p, I0{}, I1{});
-            if (nt == 3) pair(A, p, I2{}, I1{});
-            else if (nt == 4) pair(A, p, I2{}, I2{});
-        };
-        // pre(p): what the caller wants issued before step p (the next stage's loads, a part before each of the first steps,
-        // so that the waves' loads do not queue up behind one another at the stage's start)
-        auto steps4 = [&](SuperFields (&cur)[MB_RG], int nt, auto pre) {
-            SubFields c[MB_RG];
-            pre(0);
-#pragma unroll
-            for (int q = 0; q < MB_RG; ++q) c[q] = super_sub<0>(cur[q]);
-            step(c, 0, nt);
-            pre(1);
-#pragma unroll
-            for (int q = 0; q < MB_RG; ++q) c[q] = super_sub<1>(cur[q]);
-            step(c, 1, nt);
-            pre(2);
-#pragma unroll
-            for (int q = 0; q < MB_RG; ++q) c[q] = super_sub<2>(cur[q]);
-            step(c, 2, nt);
-            pre(3);
-#pragma unroll
-            for (int q = 0; q < MB_RG; ++q) c[q] = super_sub<3>(cur[q]);
-            step(c, 3, nt);
-        };
-        // Stage s = (task ti, super-step S) of the block's sequence: the next stage's loads - the next task's first ones
-        // too - are issued during this stage's arithmetic (the activations before its last step); its tile replaces this
-        // stage's in LDS between two barriers
-        int ti = 0, S = 0;
-        auto stage = [&](SuperFields (&cur)[MB_RG], SuperFields (&nxt)[MB_RG], int s) {
-            int tn = ti, Sn = S + 1;
-            if (Sn == nsuper) {
-                Sn = 0;
-                ++tn;
-            }
-            const bool more = s + 1 < nst;
-            XShare xn;
-            auto pre = [&](int p) {   // the weights (from HBM) first, the activations (cached) last
-                if (!more) return;
-                if (p < MB_RG) w_load_q(tn, Sn, p, nxt[p]);
-                else if (p == 3) xn = x_load(tn, Sn);
-            };
-            const int row0 = row0_of(ti);
-            if (row0 < rlimit) {   // per wave
-                steps4(cur, L.task[ti].ntile, pre);
-                if (Sn == 0) {   // the task's last super-step: lane = token r of each tile, weight rows 4 g .. 4 g + 3 of each group
-#pragma unroll
-                    for (int tt = 0; tt < MB_TP; ++tt) {
-                        const int orow = L.otok[ti][tt * 16 + r];
-                        if (orow >= 0) {
-                            if (a.h16) {   // gate rows in acc[0], their up rows in acc[1]
-                                const v4f gt = acc[0][tt], up = acc[1][tt];
-                                uint2 hv;
-                                hv.x = (uint32_t) float_to_half_bits(silu_f(gt.x) * up.x) | (uint32_t) float_to_half_bits(silu_f(gt.y) * up.y) << 16;
-                                hv.y = (uint32_t) float_to_half_bits(silu_f(gt.z) * up.z) | (uint32_t) float_to_half_bits(silu_f(gt.w) * up.w) << 16;
-                                *reinterpret_cast<uint2*>(a.h16 + (size_t) orow * a.ffh + row0 + 4 * g) = hv;
-                            } else {
-                                float* o = a.out + (size_t) orow * a.nrows + row0 + 4 * g;
-#pragma unroll
-                                for (int q = 0; q < MB_RG; ++q)
-                                    if (row0 + 16 * q < a.nrows)
-                                        *reinterpret_cast<float4*>(o + 16 * q) = make_float4(acc[q][tt].x, acc[q][tt].y, acc[q][tt].z, acc[q][tt].w);
-                            }
-                        }
-                    }
-#pragma unroll
-                    for (int q = 0; q < MB_RG; ++q)
-#pragma unroll
-                        for (int tt = 0; tt < MB_TP; ++tt) acc[q][tt] = v4f{0.f, 0.f, 0.f, 0.f};
-                }
-            } else {
-#pragma unroll
-                for (int p = 0; p <= 3; ++p) pre(p);
-            }
-            __syncthreads();   // this stage's tile has been read
-            if (more) x_store(xn);
-            __syncthreads();
-            ti = tn;
-            S = Sn;
-        };
-        SuperFields w0[MB_RG], w1[MB_RG];
-        {
-            const XShare x0 = x_load(0, 0);
-            w_load(0, 0, w0);
-            x_store(x0);
-        }
-        __syncthreads();
-        for (int s = 0; s < nst; s += 2) {
-            stage(w0, w1, s);
-            if (s + 1 < nst) stage(w1, w0, s + 1);
-        }
-    }
-}
-
-// ---------------------------------------------------------------- the same products, tile form (unit64 weights, short rows)
-// With rows of 512 columns or fewer (the down projection) a task of the block form is one super-step: all prologue,
-// a chain of three dependent loads (job, token row number, activations) before any arithmetic. Here a block first puts
-// its tasks (the valid ones only), their expert pointers and their token / output row numbers in LDS; after that the
-// steady state has no dependent global loads and stages run across task boundaries. Nothing is loaded per lane either:
-// a stage (256 columns of 256 rows, 32 tokens) comes in as whole runs of the planes - consecutive lanes read consecutive
-// 16 bytes - through registers into LDS a stage ahead, next to the activation tile, and a lane reads its row's fields
-// from there. LDS reads run one unit (a sub-block of 16 rows: 8 gathers -> 4 A operands -> up to 8 MFMAs) ahead of the
-// arithmetic. Measured on MI355X for the down projection of 512 columns: 71 us against 94 us for the block form; with
-// rows of 2048 columns the block form's four barriers a task beat this form's eight (132 us against 140 us).
-constexpr int MT_K = 256;                  // columns per stage: 8 sub-blocks a row, two per lane
-constexpr int MT_WROW = 112;               // bytes per row record: A 64 | B 32 | C 8 | scales 4 | d 2 | pad (28 words: 16-byte reads of 16 rows hit 64 banks once)
-constexpr int MT_XROW = 2 * MT_K + 16;     // bytes per token of the activation tile (132 words: likewise)
-constexpr int MT_MAXTASK = 16;
-struct TileTask {
-    const uint8_t* we;
-    int t0, row0, ntile;
-    int ji, n;   // the job (an index into both lists, the second list after the first) and its tokens
-};
-struct TileLds {
-    uint2 tab[SGRID_WORDS];
-    uint8_t wt[2][MB_ROWS * MT_WROW];
-    uint8_t xt[2][MB_TOK * MT_XROW];
-    int ytok[MT_MAXTASK][MB_TOK];      // activation row of each token of the task's tile (clamped to the job's last)
-    int otok[MT_MAXTASK][MB_TOK];      // its output row, or -1 past the job's end
-    TileTask task[MT_MAXTASK];
-    int ntask;
-};
-struct TileStaged {   // one thread's share of a stage, as loaded
-    v4u a[2], b, x[2];
-    v2u cs;
-};
-struct TileFields {   // a lane's two sub-blocks of one row
-    v4u A;
-    v2u B;
-    uint32_t C, sc, d;
-};
-__global__ void __launch_bounds__(MM_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) k_moe_mma_tile(const MmaArgs a) {
-    typedef __attribute__((address_space(1))) const v4u g128;
-    typedef __attribute__((address_space(1))) const v2u g64;
-    typedef __attribute__((address_space(1))) const uint32_t g32;
-    typedef __attribute__((address_space(1))) const unsigned short g16;
-    __shared__ TileLds L;
-    const int tid = threadIdx.x, lane = tid & 63, wave = uniform(tid >> 6), r = lane & 15, g = lane >> 4;
-    static_assert(MM_THREADS == 512, "a thread per 9-bit code: its sixteen signed entries are made from the first");
-    const uint32_t tab0 = g_sgrid.v[tid];
-    const int nj = min(a.cap, uniform(*a.njobs)), nj2 = a.jobs2 ? min(a.cap2, uniform(*a.njobs2)) : 0;
-    const int ks = a.ncols >> 5, nsuper = a.ncols / MT_K, rblocks = (a.nrows + MB_ROWS - 1) / MB_ROWS;
-    constexpr int HALVES = MM_TT / MM_TP;
-    const int per_job = rblocks * HALVES, ntasks_all = (nj + nj2) * per_job;
-#pragma unroll
-    for (int i = 0; i < SGRID_WORDS / MM_THREADS; ++i) {
-        const uint32_t gg = signed_entry(tab0, i);
-        v2h lo, hi;
-        lo.x = (_Float16) (int) (int8_t) (gg & 0xFFu);
-        lo.y = (_Float16) (int) (int8_t) ((gg >> 8) & 0xFFu);
-        hi.x = (_Float16) (int) (int8_t) ((gg >> 16) & 0xFFu);
-        hi.y = (_Float16) (int) (int8_t) (gg >> 24);
-        L.tab[tid + i * MM_THREADS] = make_uint2(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi));
-    }
-    for (int k0 = blockIdx.x; k0 < ntasks_all; k0 += gridDim.x * MT_MAXTASK) {
-        __syncthreads();   // the previous lists' last readers; the table on the first pass
-        if (wave == 0) {
-            const int task = k0 + lane * gridDim.x;
-            bool ok = lane < MT_MAXTASK && task < ntasks_all;
-            TileTask t{};
-            int ji = 0, n = 0;
-            if (ok) {
-                ji = task / per_job;
-                const int rem = task - ji * per_job;
-                t.t0 = (rem / rblocks) * MM_TP;
-                t.row0 = (rem % rblocks) * MB_ROWS;
-                const fnx_bigjob* jb = ji < nj ? a.jobs + ji : a.jobs2 + (ji - nj);
-                n = min(FNX_PF_JOB, jb->n);
-                const int e = jb->w;
-                ok = n >= 1 && t.t0 < ((n + 15) >> 4);
-                t.ntile = min(MM_TP, ((n + 15) >> 4) - t.t0);
-                if (ok) t.we = ji >= nj ? a.w2 : a.ep ? (const uint8_t*) a.ep[e] : a.w + (size_t) e * a.stride;
-            }
-            const unsigned long long m = __ballot(ok);
-            const int slot = __popcll(m & ((1ull << lane) - 1ull));
-            if (ok) {
-                t.ji = ji;
-                t.n = n;
-                L.task[slot] = t;
-            }
-            if (lane == 0) L.ntask = __popcll(m);
-        }
-        __syncthreads();
-        const int ntask = L.ntask;
-        if (ntask == 0) continue;   // the same for every thread of the block
-        for (int i = tid; i < ntask * MB_TOK; i += MM_THREADS) {   // the tiles' token and output rows (32 of each), all at once
-            const int slot = i / MB_TOK, j = i % MB_TOK, ji = L.task[slot].ji, n = L.task[slot].n, tok = L.task[slot].t0 * 16 + j;
-            const fnx_bigjob* jb = ji < nj ? a.jobs + ji : a.jobs2 + (ji - nj);
-            L.ytok[slot][j] = jb->y[min(tok, n - 1)];
-            L.otok[slot][j] = tok < n ? jb->out[tok] : -1;
-        }
-        __syncthreads();
-        const int nst = ntask * nsuper;
-        auto issue = [&](int ti, int S) {
-            const TileTask t = L.task[ti];
-            auto unit_of = [&](int rowl, uint32_t& l0) {
-                const int row = min(t.row0 + rowl, a.nrows - 1);
-                const uint32_t Lq = (uint32_t) row * ks + 8 * S;
-                l0 = Lq & 63u;
-                return as_global(t.we + (size_t) (Lq >> 6) * UNIT_BYTES);
-            };
-            TileStaged o;
-            uint32_t l0;
-#pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                const int c = tid + i * MM_THREADS;
-                const gbytes u = unit_of(c >> 2, l0);
-                o.a[i] = *(g128*) (u + 8 * l0 + 16 * (c & 3));
-            }
-            {
-                const gbytes u = unit_of(tid >> 1, l0);
-                o.b = *(g128*) (u + UNIT_B_AT + 4 * l0 + 16 * (tid & 1));
-            }
-            if (wave < MM_WAVES / 2) {
-                const gbytes u = unit_of(tid, l0);
-                o.cs = *(g64*) (u + UNIT_C_AT + l0);
-            } else {
-                const gbytes u = unit_of(tid - MM_THREADS / 2, l0);
-                o.cs.x = *(g32*) (u + UNIT_SCALES_AT + (l0 >> 1));
-                o.cs.y = *(g16*) (u + UNIT_D_AT + 2 * (l0 >> 3));
-            }
-            const g128* xp = (g128*) (uintptr_t) (a.x + (size_t) L.ytok[ti][tid >> 4] * a.ldx + S * MT_K + 8 * (tid & 15));
-            o.x[0] = xp[0];
-            o.x[1] = xp[16];   // + 256 bytes
-            return o;
-        };
-        auto stash = [&](const TileStaged& o, int buf) {
-            uint8_t* w = L.wt[buf];
-#pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                const int c = tid + i * MM_THREADS;
-                *reinterpret_cast<v4u*>(w + (c >> 2) * MT_WROW + 16 * (c & 3)) = o.a[i];
-            }
-            *reinterpret_cast<v4u*>(w + (tid >> 1) * MT_WROW + 64 + 16 * (tid & 1)) = o.b;
-            if (wave < MM_WAVES / 2) *reinterpret_cast<v2u*>(w + tid * MT_WROW + 96) = o.cs;
-            else {
-                *reinterpret_cast<uint32_t*>(w + (tid - MM_THREADS / 2) * MT_WROW + 104) = o.cs.x;
-                *reinterpret_cast<uint16_t*>(w + (tid - MM_THREADS / 2) * MT_WROW + 108) = (uint16_t) o.cs.y;
-            }
-            uint8_t* x = L.xt[buf] + (tid >> 4) * MT_XROW + 16 * (tid & 15);
-            *reinterpret_cast<v4u*>(x) = o.x[0];
-            *reinterpret_cast<v4u*>(x + 256) = o.x[1];
-        };
-        v4f acc[MB_RG][MM_TP];
-#pragma unroll
-        for (int q = 0; q < MB_RG; ++q)
-#pragma unroll
-            for (int tt = 0; tt < MM_TP; ++tt) acc[q][tt] = v4f{0.f, 0.f, 0.f, 0.f};
-        struct Gath {
-            uint2 e[8];
-        };
-        auto gather = [&](const TileFields& f, int p, Gath& o) {
-            const v4u idx = {f.A[2 * p], f.A[2 * p + 1], f.B[p], (f.C >> (8 * p)) & 0xFFu};
-#pragma unroll
-            for (int j = 0; j < 8; ++j) o.e[j] = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint8_t*>(L.tab) + 2 * packed_addr(idx, j));
-        };
-        auto bread = [&](int buf, int p, v4u (&B)[MM_TP][4], auto nt_tag) {
-#pragma unroll
-            for (int tt = 0; tt < decltype(nt_tag)::value; ++tt)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) B[tt][i] = *reinterpret_cast<const v4u*>(&L.xt[buf][(tt * 16 + r) * MT_XROW + 128 * g + 64 * p + 16 * i]);
-        };
-        auto math = [&](const TileFields& f, int p, int q, const Gath& in, const v4u (&B)[MM_TP][4], auto nt_tag) {
-            const _Float16 sc = (_Float16) (int) (1 + 2 * ((f.sc >> (4 * p)) & 0xFu)), d = __builtin_bit_cast(_Float16, (unsigned short) f.d);
-            const v2h s2 = {sc, sc}, d2 = {d, d};
-            v8h A[4];
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const v2h wl = (as_v2h(in.e[j].x) * s2) * d2, wh = (as_v2h(in.e[j].y) * s2) * d2;
-                A[j >> 1][4 * (j & 1) + 0] = wl.x;
-                A[j >> 1][4 * (j & 1) + 1] = wl.y;
-                A[j >> 1][4 * (j & 1) + 2] = wh.x;
-                A[j >> 1][4 * (j & 1) + 3] = wh.y;
-            }
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int tt = 0; tt < decltype(nt_tag)::value; ++tt)
-                    acc[q][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[i], __builtin_bit_cast(v8h, B[tt][i]), acc[q][tt], 0, 0, 0);
-        };
-        auto compute = [&](int buf, auto nt_tag) {
-            const uint8_t* w = L.wt[buf];
-            TileFields f[MB_RG];
-#pragma unroll
-            for (int q = 0; q < MB_RG; ++q) {
-                const uint8_t* rec = w + (wave * 16 * MB_RG + 16 * q + r) * MT_WROW;
-                f[q].A = *reinterpret_cast<const v4u*>(rec + 16 * g);
-                f[q].B = *reinterpret_cast<const v2u*>(rec + 64 + 8 * g);
-                f[q].C = *reinterpret_cast<const uint16_t*>(rec + 96 + 2 * g);
-                f[q].sc = rec[104 + g];
-                f[q].d = *reinterpret_cast<const uint16_t*>(rec + 108);
-            }
-            Gath G[2];
-            v4u Bb[2][MM_TP][4];
-            bread(buf, 0, Bb[0], nt_tag);
-            gather(f[0], 0, G[0]);
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const int p = u >> 1, q = u & 1;
-                if (u == 1) bread(buf, 1, Bb[1], nt_tag);
-                if (u < 3) gather(f[(u + 1) & 1], (u + 1) >> 1, G[(u + 1) & 1]);
-                __builtin_amdgcn_sched_barrier(0);
-                math(f[q], p, q, G[u & 1], Bb[p], nt_tag);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        };
-        TileStaged st = issue(0, 0);
-        int ti = 0, S = 0;
-        for (int s = 0; s < nst; ++s) {
-            stash(st, s & 1);
-            __syncthreads();
-            int tn = ti, Sn = S + 1;
-            if (Sn == nsuper) {
-                Sn = 0;
-                ++tn;
-            }
-            if (s + 1 < nst) st = issue(tn, Sn);
-            const int row0 = L.task[ti].row0 + wave * 16 * MB_RG;
-            if (row0 < a.nrows) {   // per wave
-                if (L.task[ti].ntile > 1) compute(s & 1, std::integral_constant<int, 2>{});
-                else compute(s & 1, std::integral_constant<int, 1>{});
-                if (Sn == 0) {
-                    // lane: token r of each tile, weight rows 4 g .. 4 g + 3 of each group
-#pragma unroll
-                    for (int tt = 0; tt < MM_TP; ++tt) {
-                        const int orow = L.otok[ti][tt * 16 + r];
-                        if (orow >= 0) {
-                            float* o = a.out + (size_t) orow * a.nrows + row0 + 4 * g;
-#pragma unroll
-                            for (int q = 0; q < MB_RG; ++q)
-                                if (row0 + 16 * q < a.nrows) *reinterpret_cast<float4*>(o + 16 * q) = make_float4(acc[q][tt].x, acc[q][tt].y, acc[q][tt].z, acc[q][tt].w);
-                        }
-                    }
-#pragma unroll
-                    for (int q = 0; q < MB_RG; ++q)
-#pragma unroll
-                        for (int tt = 0; tt < MM_TP; ++tt) acc[q][tt] = v4f{0.f, 0.f, 0.f, 0.f};
-                }
-            }
-            ti = tn;
-            S = Sn;
-        }
-    }
-}
-
-
-// ---------------------------------------------------------------- the tile form with a job's up to 64 tokens a task
-// As k_moe_mma_tile, but a task is (job, all of its token tiles, 256 rows): the weights of a stage are decoded once for
-// up to four token tiles instead of once for every two (a job of 33 to 64 tokens no longer decodes twice), the jobs are
-// ranked by token tiles and the tasks dealt to and fro over the blocks, and the activation tile of 64 tokens is single:
-// it is replaced between two barriers while the next stage's weights are already in the other weight buffer.
-constexpr int MT_TP64 = 4, MT_TOK64 = 16 * MT_TP64, MT_MAXTASK64 = 6;
-struct TileLds64 {
-    uint2 tab[SGRID_WORDS];
-    uint8_t wt[2][MB_ROWS * MT_WROW];
-    uint8_t xt[MT_TOK64 * MT_XROW];
-    int ytok[MT_MAXTASK64][MT_TOK64];
-    int otok[MT_MAXTASK64][MT_TOK64];
-    TileTask task[MT_MAXTASK64];
-    int ntask;
-    uint8_t jkey[MB_SORTJ];
-    unsigned short jorder[MB_SORTJ];
-};
-struct TileStaged64 {
-    v4u a[2], b, x[4];
-    v2u cs;
-};
-__global__ void __launch_bounds__(MM_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) k_moe_mma_tile64(const MmaArgs a) {
-    typedef __attribute__((address_space(1))) const v4u g128;
-    typedef __attribute__((address_space(1))) const v2u g64;
-    typedef __attribute__((address_space(1))) const uint32_t g32;
-    typedef __attribute__((address_space(1))) const unsigned short g16;
-    __shared__ TileLds64 L;
-    const int tid = threadIdx.x, lane = tid & 63, wave = uniform(tid >> 6), r = lane & 15, g = lane >> 4;
-    static_assert(MM_THREADS == 512, "a thread per 9-bit code: its sixteen signed entries are made from the first");
-    const uint32_t tab0 = g_sgrid.v[tid];
-    const int nj = min(a.cap, uniform(*a.njobs)), nj2 = a.jobs2 ? min(a.cap2, uniform(*a.njobs2)) : 0;
-    const int ks = a.ncols >> 5, nsuper = a.ncols / MT_K, rblocks = (a.nrows + MB_ROWS - 1) / MB_ROWS;
-    constexpr int HALVES = 1;   // a task takes all of a job's token tiles
-    const int per_job = rblocks * HALVES, ntasks_all = (nj + nj2) * per_job;
-#pragma unroll
-    for (int i = 0; i < SGRID_WORDS / MM_THREADS; ++i) {
-        const uint32_t gg = signed_entry(tab0, i);
-        v2h lo, hi;
-        lo.x = (_Float16) (int) (int8_t) (gg & 0xFFu);
-        lo.y = (_Float16) (int) (int8_t) ((gg >> 8) & 0xFFu);
-        hi.x = (_Float16) (int) (int8_t) ((gg >> 16) & 0xFFu);
-        hi.y = (_Float16) (int) (int8_t) (gg >> 24);
-        L.tab[tid + i * MM_THREADS] = make_uint2(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi));
-    }
-    // the jobs ranked by token tiles and the tasks dealt in that order, to and fro over the blocks (as k_moe_mma_block64 does)
-    const int njall = nj + nj2;
-    const bool sorted = njall <= MB_SORTJ;
-    if (sorted && wave == 0) {
-        auto key_of = [&](int j) {
-            if (j >= njall) return -1;
-            const fnx_bigjob* jb = j < nj ? a.jobs + j : a.jobs2 + (j - nj);
-            return min(MT_TP64, (max(0, min(FNX_PF_JOB, jb->n)) + 15) >> 4);
-        };
-        int total[MT_TP64 + 1];
-#pragma unroll
-        for (int c = 0; c <= MT_TP64; ++c) total[c] = 0;
-        for (int j0 = 0; j0 < njall; j0 += 64) {
-            const int kj = key_of(j0 + lane);
-            if (j0 + lane < njall) L.jkey[j0 + lane] = (uint8_t) kj;
-#pragma unroll
-            for (int c = 0; c <= MT_TP64; ++c) total[c] += __popcll(__ballot(kj == c));
-        }
-        int base[MT_TP64 + 1];   // where a class starts: the classes in descending order
-        base[MT_TP64] = 0;
-#pragma unroll
-        for (int c = MT_TP64 - 1; c >= 0; --c) base[c] = base[c + 1] + total[c + 1];
-        for (int j0 = 0; j0 < njall; j0 += 64) {
-            const int kj = j0 + lane < njall ? (int) L.jkey[j0 + lane] : -1;
-#pragma unroll
-            for (int c = 0; c <= MT_TP64; ++c) {
-                const unsigned long long m = __ballot(kj == c);
-                if (kj == c) L.jorder[base[c] + __popcll(m & ((1ull << lane) - 1ull))] = (unsigned short) (j0 + lane);
-                base[c] += __popcll(m);
-            }
-        }
-    }
-    for (int k0 = 0; k0 * (int) gridDim.x < ntasks_all; k0 += MT_MAXTASK64) {   // MT_MAXTASK64 rounds a pass
-        __syncthreads();   // the previous lists' and tiles' last readers; the table and the jobs' order on the first pass
-        if (wave == 0) {
-            const int round = k0 + lane, pos = (round & 1) ? (int) gridDim.x - 1 - (int) blockIdx.x : (int) blockIdx.x;
-            const int task = round * (int) gridDim.x + pos;
-            bool ok = lane < MT_MAXTASK64 && task < ntasks_all;
-            TileTask t{};
-            int ji = 0, n = 0;
-            if (ok) {
-                ji = task / per_job;
-                const int rem = task - ji * per_job;
-                if (sorted) ji = L.jorder[ji];
-                t.t0 = 0;
-                t.row0 = (rem % rblocks) * MB_ROWS;
-                const fnx_bigjob* jb = ji < nj ? a.jobs + ji : a.jobs2 + (ji - nj);
-                n = min(FNX_PF_JOB, jb->n);
-                const int e = jb->w;
-                ok = n >= 1 && t.t0 < ((n + 15) >> 4);
-                t.ntile = min(MT_TP64, (n + 15) >> 4);
-                if (ok) t.we = ji >= nj ? a.w2 : a.ep ? (const uint8_t*) a.ep[e] : a.w + (size_t) e * a.stride;
-            }
-            const unsigned long long m = __ballot(ok);
-            const int slot = __popcll(m & ((1ull << lane) - 1ull));
-            if (ok) {
-                t.ji = ji;
-                t.n = n;
-                L.task[slot] = t;
-            }
-            if (lane == 0) L.ntask = __popcll(m);
-        }
-        __syncthreads();
-        const int ntask = L.ntask;
-        if (ntask == 0) continue;   // the same for every thread of the block
-        for (int i = tid; i < ntask * MT_TOK64; i += MM_THREADS) {   // the tiles' token and output rows (64 of each), all at once
-            const int slot = i / MT_TOK64, j = i % MT_TOK64, ji = L.task[slot].ji, n = L.task[slot].n, tok = L.task[slot].t0 * 16 + j;
-            const fnx_bigjob* jb = ji < nj ? a.jobs + ji : a.jobs2 + (ji - nj);
-            L.ytok[slot][j] = jb->y[min(tok, n - 1)];
-            L.otok[slot][j] = tok < n ? jb->out[tok] : -1;
-        }
-        __syncthreads();
-        const int nst = ntask * nsuper;
-        auto issue = [&](int ti, int S) {
-            const TileTask t = L.task[ti];
-            auto unit_of = [&](int rowl, uint32_t& l0) {
-                const int row = min(t.row0 + rowl, a.nrows - 1);
-                const uint32_t Lq = (uint32_t) row * ks + 8 * S;
-                l0 = Lq & 63u;
-                return as_global(t.we + (size_t) (Lq >> 6) * UNIT_BYTES);
-            };
-            TileStaged64 o{};
-            uint32_t l0;
-#pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                const int c = tid + i * MM_THREADS;
-                const gbytes u = unit_of(c >> 2, l0);
-                o.a[i] = *(g128*) (u + 8 * l0 + 16 * (c & 3));
-            }
-            {
-                const gbytes u = unit_of(tid >> 1, l0);
-                o.b = *(g128*) (u + UNIT_B_AT + 4 * l0 + 16 * (tid & 1));
-            }
-            if (wave < MM_WAVES / 2) {
-                const gbytes u = unit_of(tid, l0);
-                o.cs = *(g64*) (u + UNIT_C_AT + l0);
-            } else {
-                const gbytes u = unit_of(tid - MM_THREADS / 2, l0);
-                o.cs.x = *(g32*) (u + UNIT_SCALES_AT + (l0 >> 1));
-                o.cs.y = *(g16*) (u + UNIT_D_AT + 2 * (l0 >> 3));
-            }
-            // tokens tid / 16 and 32 further, 2 x 16 bytes of the stage's 512 each; only the token tiles the task has
-            const int ntok = 16 * t.ntile;
-            const g128* xp = (g128*) (uintptr_t) (a.x + (size_t) L.ytok[ti][tid >> 4] * a.ldx + S * MT_K + 8 * (tid & 15));
-            const g128* xq = (g128*) (uintptr_t) (a.x + (size_t) L.ytok[ti][(tid >> 4) + 32] * a.ldx + S * MT_K + 8 * (tid & 15));
-            if ((tid >> 4) < ntok) {
-                o.x[0] = xp[0];
-                o.x[1] = xp[16];   // + 256 bytes
-            }
-            if ((tid >> 4) + 32 < ntok) {
-                o.x[2] = xq[0];
-                o.x[3] = xq[16];
-            }
-            return o;
-        };
-        auto stash_w = [&](const TileStaged64& o, int buf) {
-            uint8_t* w = L.wt[buf];
-#pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                const int c = tid + i * MM_THREADS;
-                *reinterpret_cast<v4u*>(w + (c >> 2) * MT_WROW + 16 * (c & 3)) = o.a[i];
-            }
-            *reinterpret_cast<v4u*>(w + (tid >> 1) * MT_WROW + 64 + 16 * (tid & 1)) = o.b;
-            if (wave < MM_WAVES / 2) *reinterpret_cast<v2u*>(w + tid * MT_WROW + 96) = o.cs;
-            else {
-                *reinterpret_cast<uint32_t*>(w + (tid - MM_THREADS / 2) * MT_WROW + 104) = o.cs.x;
-                *reinterpret_cast<uint16_t*>(w + (tid - MM_THREADS / 2) * MT_WROW + 108) = (uint16_t) o.cs.y;
-            }
-        };
-        auto stash_x = [&](const TileStaged64& o) {   // (zeros for a tile the task does not have: its products go nowhere)
-            uint8_t* x = L.xt + (tid >> 4) * MT_XROW + 16 * (tid & 15);
-            *reinterpret_cast<v4u*>(x) = o.x[0];
-            *reinterpret_cast<v4u*>(x + 256) = o.x[1];
-            *reinterpret_cast<v4u*>(x + 32 * MT_XROW) = o.x[2];
-            *reinterpret_cast<v4u*>(x + 32 * MT_XROW + 256) = o.x[3];
-        };
-        v4f acc[MB_RG][MT_TP64];
-#pragma unroll
-        for (int q = 0; q < MB_RG; ++q)
-#pragma unroll
-            for (int tt = 0; tt < MT_TP64; ++tt) acc[q][tt] = v4f{0.f, 0.f, 0.f, 0.f};
-        struct Gath {
-            uint2 e[8];
-        };
-        auto gather = [&](const TileFields& f, int p, Gath& o) {
-            const v4u idx = {f.A[2 * p], f.A[2 * p + 1], f.B[p], (f.C >> (8 * p)) & 0xFFu};
-#pragma unroll
-            for (int j = 0; j < 8; ++j) o.e[j] = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint8_t*>(L.tab) + 2 * packed_addr(idx, j));
-        };
-        auto bread = [&](int p, v4u (&B)[MT_TP64][4], auto nt_tag) {
-#pragma unroll
-            for (int tt = 0; tt < decltype(nt_tag)::value; ++tt)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) B[tt][i] = *reinterpret_cast<const v4u*>(&L.xt[(tt * 16 + r) * MT_XROW + 128 * g + 64 * p + 16 * i]);
-        };
-        auto math = [&](const TileFields& f, int p, int q, const Gath& in, const v4u (&B)[MT_TP64][4], auto nt_tag) {
-            const _Float16 sc = (_Float16) (int) (1 + 2 * ((f.sc >> (4 * p)) & 0xFu)), d = __builtin_bit_cast(_Float16, (unsigned short) f.d);
-            const v2h s2 = {sc, sc}, d2 = {d, d};
-            v8h A[4];
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const v2h wl = (as_v2h(in.e[j].x) * s2) * d2, wh = (as_v2h(in.e[j].y) * s2) * d2;
-                A[j >> 1][4 * (j & 1) + 0] = wl.x;
-                A[j >> 1][4 * (j & 1) + 1] = wl.y;
-                A[j >> 1][4 * (j & 1) + 2] = wh.x;
-                A[j >> 1][4 * (j & 1) + 3] = wh.y;
-            }
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int tt = 0; tt < decltype(nt_tag)::value; ++tt)
-                    acc[q][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[i], __builtin_bit_cast(v8h, B[tt][i]), acc[q][tt], 0, 0, 0);
-        };
-        auto compute = [&](int buf, auto nt_tag) {
-            const uint8_t* w = L.wt[buf];
-            TileFields f[MB_RG];
-#pragma unroll
-            for (int q = 0; q < MB_RG; ++q) {
-                const uint8_t* rec = w + (wave * 16 * MB_RG + 16 * q + r) * MT_WROW;
-                f[q].A = *reinterpret_cast<const v4u*>(rec + 16 * g);
-                f[q].B = *reinterpret_cast<const v2u*>(rec + 64 + 8 * g);
-                f[q].C = *reinterpret_cast<const uint16_t*>(rec + 96 + 2 * g);
-                f[q].sc = rec[104 + g];
-                f[q].d = *reinterpret_cast<const uint16_t*>(rec + 108);
-            }
-            Gath G[2];
-            v4u Bb[MT_TP64][4];   // the tokens' operands of one half of the stage's columns: both row groups use them
-            bread(0, Bb, nt_tag);
-            gather(f[0], 0, G[0]);
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const int p = u >> 1, q = u & 1;
-                if (u == 2) bread(1, Bb, nt_tag);
-                if (u < 3) gather(f[(u + 1) & 1], (u + 1) >> 1, G[(u + 1) & 1]);
-                __builtin_amdgcn_sched_barrier(0);
-                math(f[q], p, q, G[u & 1], Bb, nt_tag);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        };
-        TileStaged64 st = issue(0, 0);
-        int ti = 0, S = 0;
-        for (int s = 0; s < nst; ++s) {
-            stash_w(st, s & 1);   // (its buffer was last read two stages ago)
-            __syncthreads();      // the single activation tile's last readers
-            stash_x(st);
-            __syncthreads();
-            int tn = ti, Sn = S + 1;
-            if (Sn == nsuper) {
-                Sn = 0;
-                ++tn;
-            }
-            if (s + 1 < nst) st = issue(tn, Sn);
-            const int row0 = L.task[ti].row0 + wave * 16 * MB_RG;
-            if (row0 < a.nrows) {   // per wave
-                const int nt = L.task[ti].ntile;
-                if (nt > 2) compute(s & 1, std::integral_constant<int, 4>{});
-                else if (nt > 1) compute(s & 1, std::integral_constant<int, 2>{});
-                else compute(s & 1, std::integral_constant<int, 1>{});
-                if (Sn == 0) {
-                    // lane: token r of each tile, weight rows 4 g .. 4 g + 3 of each group
-#pragma unroll
-                    for (int tt = 0; tt < MT_TP64; ++tt) {
-                        const int orow = L.otok[ti][tt * 16 + r];
-                        if (orow >= 0) {
-                            float* o = a.out + (size_t) orow * a.nrows + row0 + 4 * g;
-#pragma unroll
-                            for (int q = 0; q < MB_RG; ++q)
-                                if (row0 + 16 * q < a.nrows) *reinterpret_cast<float4*>(o + 16 * q) = make_float4(acc[q][tt].x, acc[q][tt].y, acc[q][tt].z, acc[q][tt].w);
-                        }
-                    }
-#pragma unroll
-                    for (int q = 0; q < MB_RG; ++q)
-#pragma unroll
-                        for (int tt = 0; tt < MT_TP64; ++tt) acc[q][tt] = v4f{0.f, 0.f, 0.f, 0.f};
-                }
-            }
-            ti = tn;
-            S = Sn;
-        }
-    }
-}
-
 
 }  // namespace fnx

@@ -172,7 +172,8 @@ class Dev:
         if packed or tile16:
             self.ok(self.lib.fnx_iq3s_repack(dw_.data_ptr(), dw_.data_ptr(), w.size // 110 * 256, self.st()))
         out = self.zeros((out_rows, nrows), t.float32)
-        W = self.pkg.dw(dw_, ncols, nrows, packed=packed)
+        W = W0 = self.pkg.dw(dw_, ncols, nrows, packed=packed)
+        w_stride0 = w_stride
         if tile16:
             nmat = w.size // (nrows * (ncols // 256) * 110)
             one = self.lib.fnx_iq3s_tile16_bytes(nrows, ncols, 1)
@@ -231,7 +232,7 @@ class Dev:
         T, rows = logits.shape
         dl = self.up(logits.astype(np.float32))
         bv, bi = self.zeros(T, t.float32), self.zeros(T, t.int32)
-        keys, err = self.zeros(16, t.int64), self.zeros(1, t.int32)
+        keys, err = self.zeros(self.pkg.ARGMAX_WORDS, t.int64), self.zeros(1, t.int32)
         self.ok(self.lib.fnx_argmax(dl.data_ptr(), rows, T, v0, bv.data_ptr(), bi.data_ptr(), keys.data_ptr(), err.data_ptr(), self.st()))
         self.sync()
         assert int(keys.abs().sum().item()) == 0, "argmax leaves its keys at zero"
@@ -297,7 +298,8 @@ class Dev:
         if packed:
             self.ok(self.lib.fnx_iq3s_repack(dw_.data_ptr(), dw_.data_ptr(), w.size // 110 * 256, self.st()))
         out = self.zeros((out_rows, nrows), t.float32)
-        W = self.pkg.dw(dw_, ncols, nrows, packed=packed)
+        W = W0 = self.pkg.dw(dw_, ncols, nrows, packed=packed)
+        w_stride0 = w_stride
         if tile16:   # re-laid a second time into the prompt path's layout (w_stride then counts that layout's bytes)
             assert packed
             nmat = w.size // (nrows * ncols // 256 * 110)
@@ -306,11 +308,11 @@ class Dev:
             W = self.pkg.dw(d16, ncols, nrows, tile16=True)
             w_stride = self.lib.fnx_iq3s_tile16_bytes(nrows, ncols, 1) if w_stride else 0
         nj = self.up(np.array([len(jobs)], dtype=np.int32))
-        if h16:   # nrows = 2 ffs stacked: h = silu(gate) * up as f16 from one launch, and from the two operators one after the other
+        if h16:   # nrows = 2 ffs stacked: h = silu(gate) * up as f16 from one launch (tile16), and from the two operators one after the other (unit64)
             ffs = nrows // 2
             one, two = self.zeros((out_rows, ffs), t.float16), self.zeros((out_rows, ffs), t.float16)
             self.ok(self.lib.fnx_moe_gate_up_h16_mma(C.byref(W), w_stride, dj.data_ptr(), nj.data_ptr(), cap, dx.data_ptr(), one.data_ptr(), self.st()))
-            self.ok(self.lib.fnx_moe_gate_up_mma(C.byref(W), w_stride, dj.data_ptr(), nj.data_ptr(), cap, dx.data_ptr(), out.data_ptr(), self.st()))
+            self.ok(self.lib.fnx_moe_gate_up_mma(C.byref(W0), w_stride0, dj.data_ptr(), nj.data_ptr(), cap, dx.data_ptr(), out.data_ptr(), self.st()))
             self.ok(self.lib.fnx_swiglu_h16(out.data_ptr(), ffs, out_rows, two.data_ptr(), self.st()))
             self.sync()
             return one.cpu().numpy(), two.cpu().numpy()
@@ -456,7 +458,7 @@ class DecoderDev:
                       v=z((T, nkv * 256), t.float32), att=z((T, nq * 256), t.float32), o=z((T, n), t.float32),
                       attn_scratch=z(dev.lib.fnx_attn_scratch_floats(nq, T, c["max_ctx"]), t.float32), xq=z(T * (max(n, nq * 256) // 32) * 36, t.uint8),
                       hidden=z((T, n), t.float32), logits=z((T, c["vocab"]), t.float32), best_v=z(T, t.float32), best_i=z(T, t.int32),
-                      keys=z(16, t.int64), err=z(1, t.int32))
+                      keys=z(pkg.ARGMAX_WORDS, t.int64), err=z(1, t.int32))
         self.mb = dict(xq=z(T * (n // 32) * 36, t.uint8), logits=z((T, nexp + 1), t.float32), topi=z((T, topk), t.int32),
                        topw=z((T, topk), t.float32), jobs_gu=z((P + 1) * 136, t.uint8), jobs_dn=z((P + 1) * 136, t.uint8), njobs=z(2, t.int32), sync=z(pkg.MOE_SYNC_WORDS, t.int32),
                        gu=z((P + T, 2 * ff), t.float32), part=z((P + T, n), t.float32))
@@ -547,15 +549,29 @@ class DecoderDev:
             ti.append(b)
         return np.stack(lg), np.stack(ti)
 
-    def draft(self, src, tokens, pos0):
+    def draft(self, src, tokens, pos0, dv=None, pen=None, par=None):
+        """dv = (dv0, dv1): the head's rows for those tokens only; pen = (indexes relative to dv0, counts), par = (repeat, freq,
+        present): the last row's penalties"""
         dev = self.dev
         tok = dev.up(np.asarray(tokens, dtype=np.int32))
         dsrc = dev.up(np.ascontiguousarray(src, dtype=np.float32))
         self.pos.fill_(pos0)
-        dev.ok(dev.lib.fnx_mtp_draft(C.byref(self.D), C.byref(self.M), dsrc.data_ptr(), tok.data_ptr(), len(tokens), self.pos.data_ptr(),
-                                     C.byref(self.ws), dev.st()))
+        M, keep, T, n = self.M, [], len(tokens), self.c["n"]
+        if dv is not None or pen is not None:
+            M = type(self.M).from_buffer_copy(self.M)
+            if dv is not None:
+                M.dv0, M.dv1 = dv
+                M.head = dev.pkg.Q8S(self.M.head.q + dv[0] * n, self.M.head.d + dv[0] * (n // 32) * 2, dv[1] - dv[0], n)
+            if pen is not None:
+                keep = [dev.up(np.concatenate([[len(pen[0])], pen[0], pen[1]]).astype(np.int32)), dev.up(np.asarray(par, dtype=np.float32))]
+                M.pen, M.pen_par = keep[0].data_ptr(), keep[1].data_ptr()
+        dev.ok(dev.lib.fnx_mtp_draft(C.byref(self.D), C.byref(M), dsrc.data_ptr(), tok.data_ptr(), T, self.pos.data_ptr(), C.byref(self.ws), dev.st()))
         dev.sync()
-        return self._result(len(tokens))
+        r = self._result(T)
+        if dv is not None:   # the workspace's logits rows are dv1 - dv0 values long in this call
+            nv = dv[1] - dv[0]
+            r["logits"] = self.b["logits"].cpu().numpy().reshape(-1)[:T * nv].reshape(T, nv)
+        return r
 
 
 class PfLayerDev:

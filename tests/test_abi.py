@@ -58,6 +58,20 @@ def test_bad_arguments_are_refused_with_a_message():
     assert lib.fnx_attn(buf, buf, buf, buf, 16, 2, buf, 1, 4, buf, None) != 0 and b"multiple of 8" in lib.fnx_last_error()
 
 
+def test_the_grouped_gemm_takes_tile16_in_its_two_forms_only():
+    """tile16 matrices are the prompt path's stacked gate|up (which leaves h) and rows of 512 columns; h alone comes from
+    tile16 only: everything else is refused before a launch"""
+    pkg = fnx_gpu.package()
+    lib = pkg.lib()
+    buf = np.zeros(64, dtype=np.float32).ctypes.data
+    gu16, dn16_1024 = pkg.dw(buf, 2048, 1024, tile16=True), pkg.dw(buf, 1024, 2048, tile16=True)
+    assert lib.fnx_moe_gate_up_mma(C.byref(gu16), 0, buf, buf, 4, buf, buf, None) != 0 and b"tile16" in lib.fnx_last_error()
+    assert lib.fnx_moe_down_mma(C.byref(dn16_1024), 0, buf, buf, 4, buf, buf, None) != 0 and b"tile16" in lib.fnx_last_error()
+    for packed in (False, True):
+        w = pkg.dw(buf, 2048, 1024, packed=packed)
+        assert lib.fnx_moe_gate_up_h16_mma(C.byref(w), 0, buf, buf, 4, buf, buf, None) != 0 and b"h alone" in lib.fnx_last_error()
+
+
 def test_a_layer_wider_than_the_pair_buffer_is_refused():
     """operator by operator (raw ggml blocks) the pairs' q8_1 rows of h go through the library's pair buffer of rows of at most
     1024 values: a wider expert is refused before anything is launched"""

@@ -10,6 +10,8 @@ difference upstream now and then moves one int8 code by one step (1/127 of its b
 that row's logits while every other row agrees to 1e-7; cache cells written from such rows (f16) carry the step on to
 later rows and windows through the attention. For chains the tests therefore ask: picks identical, every row within
 1e-2, and on a fresh cache at least one row within 1e-5 (the arithmetic is the same; the rest is such steps)."""
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -180,6 +182,36 @@ def test_decoder_verify_and_draft(dev, oracle, model):
     for (ka, va), (kb, vb) in zip(o.caches + [o.mtp_cache], d.caches_numpy()):
         assert rel_l2(kb.view(np.float16)[:pos], ka.view(np.float16)[:pos]) <= REL_L2
         assert rel_l2(vb.view(np.float16)[:pos], va.view(np.float16)[:pos]) <= REL_L2
+
+
+def test_draft_head_options(dev, oracle, model):
+    """engine.cu:2130-2131: the draft head over the tokens [dv0, dv1) alone and the last row's penalty list, against the oracle's
+    same call; the control without the list keeps the last row's own pick"""
+    o, d = td.OracleSession(model), fnx_gpu.DecoderDev(dev, model)
+    toks = [3, 1, 4, 1, 5, 9, 2, 6]
+    a = o.verify(toks, 0)
+    nxt = toks[1:] + [int(a["best"][-1])]
+    dv = (96, 608)
+    plain_o, plain_d = o.draft(a["hidden"], nxt, 0, dv=dv), d.draft(a["hidden"], nxt, 0, dv=dv)
+    assert plain_d["err"] == 0 and plain_d["logits"].shape == (len(toks), dv[1] - dv[0])
+    assert np.array_equal(plain_o["best"], plain_d["best"]) and all(dv[0] <= int(b) < dv[1] for b in plain_d["best"])
+    chain_close(plain_d["logits"], plain_o["logits"], True)
+    top = int(plain_o["best"][-1]) - dv[0]
+    pen, par = (np.array([top, 7, -3, dv[1] - dv[0]]), np.array([3, 0, 1, 1])), (1.2, 0.5, 40.0)
+    print("case mtp_draft with dv0, dv1 and a penalty list", flush=True)
+    po, pd = o.draft(a["hidden"], nxt, 0, dv=dv, pen=pen, par=par), d.draft(a["hidden"], nxt, 0, dv=dv, pen=pen, par=par)
+    assert pd["err"] == 0
+    assert np.array_equal(po["best"], pd["best"]) and int(pd["best"][-1]) != dv[0] + top
+    chain_close(pd["logits"], po["logits"], True)
+    # the list changed one value of the last row and nothing else
+    changed = np.argwhere(pd["logits"] != plain_d["logits"])
+    assert changed.tolist() == [[len(toks) - 1, top]]
+    # a head whose row count is not dv1 - dv0 is refused before any launch
+    M = type(d.M).from_buffer_copy(d.M)
+    M.dv0, M.dv1 = 0, 10
+    tok = dev.up(np.asarray(nxt, dtype=np.int32))
+    src = dev.up(a["hidden"])
+    assert dev.lib.fnx_mtp_draft(C.byref(d.D), C.byref(M), src.data_ptr(), tok.data_ptr(), len(nxt), d.pos.data_ptr(), C.byref(d.ws), dev.st()) != 0
 
 
 def same_until_near_tie(oracle, model, prompt, a, b):

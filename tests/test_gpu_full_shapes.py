@@ -237,7 +237,7 @@ def config5_inputs(rng, n, ff, nexp, Cn, zipf):
     return router, gu, down, sh_gu, sh_down, x
 
 
-# unit64: every matrix in the verify path's layout (k_moe_mma_block64 / k_moe_mma_tile64); tile16: the prompt path's own
+# unit64: every matrix in the verify path's layout (k_moe_mma, a wave a task); tile16: the prompt path's own
 # copies of gate|up and down, the layout the benchmark's prefill workload times (k_moe_mma_wave16_gu, k_moe_mma_wave16)
 @pytest.mark.parametrize("layout", ["unit64", "tile16"])
 def test_config5_chunk_of_512_rows(dev, oracle, layout):
@@ -256,9 +256,11 @@ def test_config5_chunk_of_512_rows(dev, oracle, layout):
     err = rel_l2(r["out"], want["out"])
     print("config 5 chunk rel l2", err, flush=True)
     assert err <= REL_L2
-    if layout == "tile16":   # h as the wave kernels leave it = h of the unit64 block form, bit for bit (one accumulation order per tile)
+    if layout == "tile16":   # h as the wave kernels leave it against h of the unit64 kernel: the same f16 operands, another order of sums
         r64 = fnx_gpu.PfLayerDev(dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, Cn, packed=True).run(x)
-        assert np.array_equal(r["h16"].view(np.uint16), r64["h16"].view(np.uint16))
+        differ = int((r["h16"].view(np.uint16) != r64["h16"].view(np.uint16)).sum())
+        print(f"{differ} of {r['h16'].size} f16 values of h differ between the layouts", flush=True)
+        assert differ <= r["h16"].size // 100 and rel_l2(r["h16"].astype(np.float32), r64["h16"].astype(np.float32)) <= 1e-4
 
 
 def test_config5_uniform_routing_tile16(dev, oracle):

@@ -88,6 +88,14 @@ def test_swiglu_h16(dev, oracle):
     assert diff.max() <= 1 and np.count_nonzero(diff) <= 1e-3 * diff.size
 
 
+def h16_close(a, b):
+    """two kernels' h = f16(silu(gate) * up) from the same f16 operands added up in different orders: nearly every value the
+    same f16, the rest a rounding step apart"""
+    differ = int((a.view(np.uint16) != b.view(np.uint16)).sum())
+    print(f"{differ} of {a.size} f16 values of h differ", flush=True)
+    assert differ <= a.size // 100 and rel_l2(a.astype(np.float32), b.astype(np.float32)) <= 1e-4
+
+
 def make_jobs(rng, nexp, rows_avail, sizes):
     jobs = np.zeros((len(sizes), 2 + 2 * PF), dtype=np.int32)
     at = 0
@@ -132,7 +140,7 @@ def test_moe_mma_wave_form_tile16_rows_of_512(dev, oracle, nrows, nexp, sizes):
     x16 = rng.standard_normal((rows, ncols)).astype(np.float16)
     jobs, total = make_jobs(rng, nexp, rows, sizes)
     got = dev.moe_mma(w, stride, nrows, ncols, jobs, x16, total, packed=True, down=True, cap=len(jobs) + 5, tile16=True)
-    other = dev.moe_mma(w, stride, nrows, ncols, jobs, x16, total, packed=True, down=True, cap=len(jobs) + 5)   # the tile form over unit64
+    other = dev.moe_mma(w, stride, nrows, ncols, jobs, x16, total, packed=True, down=True, cap=len(jobs) + 5)   # the wave-a-task kernel over unit64
     assert rel_l2(got, other) <= 1e-6, "the same f16 products: only the summation order differs"
     assert np.array_equal(got == 0, other == 0)   # (rows no job writes stay as they were)
     if len(sizes) <= 8:
@@ -140,14 +148,14 @@ def test_moe_mma_wave_form_tile16_rows_of_512(dev, oracle, nrows, nexp, sizes):
         assert rel_l2(got, want) <= 1e-5, "f16 operands are the oracle's: only the summation order may differ"
 
 
-@pytest.mark.parametrize("tile16", [False, True])
 @pytest.mark.parametrize("ffs,ncols,nexp,sizes", [(512, 2048, 24, [64, 1, 17, 0, 16, 33, 48, 5, 64, 64, 2, 0, 31, 64, 49, 15] * 3), (128, 512, 3, [64, 1, 17, 16, 33, 48, 5]),
                                                   (256, 1024, 2, [3]), (640, 2048, 2, [64, 9]), (128, 2560, 2, [5, 64, 20, 16])])
-def test_moe_gate_up_h16_one_launch_equals_two(dev, ffs, ncols, nexp, sizes, tile16):
-    # h = silu(gate) * up straight from the matrix-core launch (block form over unit64, wave form over tile16): the bits of
-    # fnx_moe_gate_up_mma followed by fnx_swiglu_h16, whatever the mix of job sizes, with rows no job writes left alone
+def test_moe_gate_up_h16_one_launch_equals_two(dev, oracle, ffs, ncols, nexp, sizes):
+    # h = silu(gate) * up straight from the matrix-core launch (the wave form over tile16) against fnx_moe_gate_up_mma over
+    # the unit64 copy followed by fnx_swiglu_h16, whatever the mix of job sizes, with rows no job writes left alone
     # (640: a job's last unit is short of pairs; 2560 columns: five activation tiles a row, so small jobs go as heavy units)
-    print(f"case moe_gate_up_h16 ffs={ffs} ncols={ncols} nexp={nexp} jobs={len(sizes)} tile16={tile16}", flush=True)
+    tile16 = True
+    print(f"case moe_gate_up_h16 ffs={ffs} ncols={ncols} nexp={nexp} jobs={len(sizes)}", flush=True)
     nrows = 2 * ffs
     rng = np.random.default_rng(741 + ffs + len(sizes))
     stride = nrows * ncols // 256 * 110
@@ -157,11 +165,14 @@ def test_moe_gate_up_h16_one_launch_equals_two(dev, ffs, ncols, nexp, sizes, til
     jobs, total = make_jobs(rng, nexp, rows, sizes)
     one, two = dev.moe_mma(w, stride, nrows, ncols, jobs, x16, total + 3, packed=True, cap=len(jobs) + 5, tile16=tile16, h16=True)
     assert np.all(np.isfinite(two.astype(np.float32)))
-    if tile16 or ncols > 512:
-        assert np.array_equal(one.view(np.uint16), two.view(np.uint16))
-    else:   # unit64 rows of up to 512 columns: the products alone come from the tile form, which adds in another order
-        assert rel_l2(one.astype(np.float32), two.astype(np.float32)) <= 1e-3
+    # the same f16 operands on both sides; the two kernels add a row's products in different orders, which now and then moves
+    # an f16 value of h by one step
+    h16_close(one, two)
     assert np.any(one[:total] != 0) and not np.any(one[total:])
+    if len(sizes) <= 8:   # against the oracle: its products, its SwiGLU
+        gu = oracle.moe_mma(w, stride, nrows, ncols, jobs, PF, x16, total + 3)
+        want = oracle.swiglu_h16(gu, ffs)
+        assert rel_l2(one.astype(np.float32), want.astype(np.float32)) <= 1e-3
 
 
 def test_moe_mma_weights_equal_the_oracles_f16(dev, oracle):
@@ -208,10 +219,9 @@ def test_prefill_layer_matches_oracle(dev, oracle, n, ff, nexp, topk, Cn):
 
 @pytest.mark.parametrize("n,ff,nexp,topk,Cn", [(2048, 512, 48, 10, 300), (1024, 256, 8, 2, 70)])
 def test_prefill_layer_tile16_equals_unit64(dev, oracle, n, ff, nexp, topk, Cn):
-    """the gate|up matrices in the prompt path's own layout: the same arithmetic on the same bytes found elsewhere, so
-    h = silu(gate) * up is that of the unit64 layout bit for bit, and so is the chunk's result where the down matrices stay
-    unit64 (ff not in 512s); tile16 down matrices go through the wave form, which adds the same f16 products up in another
-    order than the unit64 tile form (and the oracle's within the bar either way)"""
+    """the gate|up matrices (and the down matrices, where ff comes in 512s) in the prompt path's own layout: the same f16
+    weights and activations as the unit64 layout's kernel, whose tasks add a row's products up in another order, so h and the
+    chunk's result agree to float rounding (and with the oracle's within the bar either way)"""
     print(f"case prefill_layer tile16 n={n} ff={ff} nexp={nexp} topk={topk} C={Cn}", flush=True)
     rng = np.random.default_rng(760 + nexp)
     nb = lambda rows, cols: rows * cols // 256
@@ -223,11 +233,8 @@ def test_prefill_layer_tile16_equals_unit64(dev, oracle, n, ff, nexp, topk, Cn):
     a = fnx_gpu.PfLayerDev(dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, Cn, packed=True).run(x)
     b = fnx_gpu.PfLayerDev(dev, n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, Cn, packed=True, tile16=True).run(x)
     assert np.array_equal(a["topi"], b["topi"])
-    assert np.array_equal(a["h16"].view(np.uint16), b["h16"].view(np.uint16))
-    if ff % 512:
-        assert int(np.count_nonzero(a["out"].view(np.uint32) != b["out"].view(np.uint32))) == 0
-    else:
-        assert rel_l2(b["out"], a["out"]) <= 1e-6
+    h16_close(a["h16"], b["h16"])
+    assert rel_l2(b["out"], a["out"]) <= 1e-5
     want = oracle.moe_prefill_layer(n, ff, nexp, topk, router, gu, down, sh_gu, sh_down, x)
     assert rel_l2(b["out"], want["out"]) <= REL_L2
 

@@ -253,3 +253,34 @@ def test_mtp_draft_equals_its_wiring(oracle):
         got, miss = s2.draft(src[:4], nxt[:4], 0), bad.draft(src[:4], nxt[:4], 0)
         which = "logits" if wrong == "mtp_head_norm" else "hidden"
         assert rel(got[which], miss[which]) >= MISS, wrong
+
+
+def test_mtp_draft_head_options_equal_their_wiring(oracle):
+    """engine.cu:2130-2131: a head of the tokens [dv0, dv1) alone gives those logits and token ids from dv0; the penalty list
+    touches the last row only, before its pick. Control: the same call without the list keeps the row's unpenalised pick."""
+    m = td.TinyDecoder(oracle, seed=33)
+    src = td.OracleSession(m).verify(TOKS[:6], 0)["hidden"]
+    nxt = TOKS[1:7]
+    full = NpDecoder(m).draft(src[:4], nxt[:4], 0)["logits"]
+    dv0, dv1 = 200, 700
+    part = full[:, dv0:dv1]
+    top = int(np.argmax(part[3]))
+    # the row's top token (counted twice), a token whose count is zero (skipped), and indexes outside the head (skipped)
+    idx, cnt = np.array([top, 5, -1, dv1 - dv0]), np.array([2, 0, 1, 1])
+    par = (1.3, 0.25, 50.0)
+    want = part.copy()
+    l = want[3, top]
+    want[3, top] = (l * par[0] if l <= 0 else l / par[0]) - 2 * par[1] - par[2]
+    got = td.OracleSession(m).draft(src[:4], nxt[:4], 0, dv=(dv0, dv1), pen=(idx, cnt), par=par)
+    assert got["logits"].shape == (4, dv1 - dv0)
+    assert rel(got["logits"], want) <= TOL
+    assert rel(got["logits"][3, top], want[3, top]) <= TOL and got["logits"][3, 5] == td.OracleSession(m).draft(src[:4], nxt[:4], 0, dv=(dv0, dv1))["logits"][3, 5]
+    assert all(dv0 <= int(b) < dv1 for b in got["best"])
+    check_best(got["best"] - dv0, want)
+    assert int(got["best"][3]) != dv0 + top, "the penalised token lost the row"
+    ctl = td.OracleSession(m).draft(src[:4], nxt[:4], 0, dv=(dv0, dv1))
+    assert rel(ctl["logits"], part) <= TOL and int(ctl["best"][3]) == dv0 + top
+    assert np.array_equal(ctl["best"][:3], got["best"][:3]), "rows before the last are not penalised"
+    # the whole vocabulary (dv0 = dv1 = 0) with a list: the same row rule
+    whole = td.OracleSession(m).draft(src[:4], nxt[:4], 0, pen=(np.array([int(np.argmax(full[3]))]), np.array([1])), par=par)
+    assert int(whole["best"][3]) != int(np.argmax(full[3])) and np.array_equal(whole["logits"][:3], td.OracleSession(m).draft(src[:4], nxt[:4], 0)["logits"][:3])

@@ -31,7 +31,7 @@ class DecoderO(C.Structure):
 
 class MtpO(C.Structure):
     _fields_ = [("norm_emb", C.c_void_p), ("norm_hid", C.c_void_p), ("out_norm", C.c_void_p), ("fc_emb", Q8sO), ("fc_hid", Q8sO), ("head", Q8sO),
-                ("layer", DecLayerO)]
+                ("layer", DecLayerO), ("dv0", C.c_int), ("dv1", C.c_int), ("pen", C.c_void_p), ("pen_par", C.c_void_p)]
 
 
 def _oracle_q8s(oracle):
@@ -160,16 +160,29 @@ class OracleSession:
     def _layer_arr(self):
         return self._keep[-3]   # the DecLayerO array oracle_structs built
 
-    def draft(self, src, tokens, pos0, routing=False):
+    def draft(self, src, tokens, pos0, routing=False, dv=None, pen=None, par=None):
+        """dv = (dv0, dv1): the head's rows for those tokens only; pen = (indexes relative to dv0, counts), par = (repeat, freq,
+        present): the last row's penalties (engine.cu:2130-2131)"""
         c = self.m.cfg
         tok = np.ascontiguousarray(tokens, dtype=np.int32)
         src = np.ascontiguousarray(src, dtype=np.float32)
         T = len(tok)
         hidden = np.zeros((T, c["n"]), dtype=np.float32)
-        logits = np.zeros((T, c["vocab"]), dtype=np.float32)
+        M, keep = self.M, []
+        if dv is not None or pen is not None:
+            M = MtpO.from_buffer_copy(self.M)
+            if dv is not None:
+                q, d = self.m.mtp["head"]
+                keep = [np.ascontiguousarray(q[dv[0]:dv[1]]), np.ascontiguousarray(d[dv[0]:dv[1]])]
+                M.dv0, M.dv1 = dv
+                M.head = Q8sO(ol.ptr(keep[0]), ol.ptr(keep[1]), dv[1] - dv[0], c["n"])
+            if pen is not None:
+                keep += [np.concatenate([[len(pen[0])], pen[0], pen[1]]).astype(np.int32), np.asarray(par, dtype=np.float32)]
+                M.pen, M.pen_par = ol.ptr(keep[-2]), ol.ptr(keep[-1])
+        logits = np.zeros((T, dv[1] - dv[0] if dv is not None else c["vocab"]), dtype=np.float32)
         best = np.zeros(T, dtype=np.int32)
         probe = self._probe(T, 1) if routing else None
-        self.m.oracle.lib.fnx_o_mtp_draft(C.byref(self.D), C.byref(self.M), ol.ptr(src), ol.ptr(tok), T, pos0, ol.ptr(hidden), ol.ptr(logits),
+        self.m.oracle.lib.fnx_o_mtp_draft(C.byref(self.D), C.byref(M), ol.ptr(src), ol.ptr(tok), T, pos0, ol.ptr(hidden), ol.ptr(logits),
                                           ol.ptr(best), self.threads)
         self.m.oracle.lib.fnx_o_layer_probe(None, None, 0)
         r = dict(hidden=hidden, logits=logits, best=best)
