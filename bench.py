@@ -903,6 +903,30 @@ def prefill_main(args):
     sw_ms = float(np.mean([e[1].elapsed_time(e[2]) for e in evs[3:]]))
     gu_ms = float(np.mean([e[2].elapsed_time(e[3]) for e in evs[3:]])) if fused_h else gu2_ms
     dn_ms = float(np.mean([e[3].elapsed_time(e[4]) for e in evs[3:]]))
+    # the reference's other prompt family (kernels.hpp:324-325, its moe_q8 mode): the same jobs over q8_1 activations on the int8
+    # matrix cores - a stated option beside the metric's f16 family, whose results differ from it by the q8_1 rounding
+    q8 = None
+    if not args.raw_layout and not args.down_unit64 and not args.no_extras:
+        xq = torch.zeros(CH * (N // 32) * 36, dtype=torch.uint8, device="cuda")
+        evq = []
+        for i in range(reps + 3):
+            L = layers[i % nsets][0]
+            step(i)
+            e = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
+            e[0].record()
+            dev.ok(lib.fnx_quantize_q8_1(xs[i % NX].data_ptr(), xq.data_ptr(), N, CH, st))
+            e[1].record()
+            dev.ok(lib.fnx_moe_gate_up_big(C.byref(L.gu), L.gu_stride, ws.jobs_gu, ws.njobs, J, xq.data_ptr(), ws.gu, st))
+            e[2].record()
+            dev.ok(lib.fnx_moe_down_big(C.byref(L.down), L.down_stride, ws.jobs_dn, ws.njobs, J, ws.gu, ws.part, st))
+            e[3].record()
+            evq.append(e)
+        torch.cuda.synchronize()
+        q8 = {"quantize_us": float(np.mean([e[0].elapsed_time(e[1]) for e in evq[3:]])) * 1e3,
+              "gate_up_big_us": float(np.mean([e[1].elapsed_time(e[2]) for e in evq[3:]])) * 1e3,
+              "down_big_us": float(np.mean([e[2].elapsed_time(e[3]) for e in evq[3:]])) * 1e3,
+              "note": "routed jobs only, k_iq3s_jobs_mma16<1 | 2> over the tile16 copies; the f16 family's routed launches beside them: "
+                      f"{gu_ms * 1e3:.1f} + {dn_ms * 1e3:.1f} us"}
     # the routed gate|up launch: the experts' matrices, x as f16, and h as f16 (the products themselves, f32, where h is a launch of its own)
     gu_bytes = u_mean * GU_BYTES + CH * N * 2 + (P * FF * 2 if fused_h else P * 2 * FF * 4)
     dn_bytes = u_mean * DN_BYTES + P * FF * 2 + P * N * 4
@@ -953,6 +977,7 @@ def prefill_main(args):
         "cpu_baseline": cpu,
         # not the metric: two streams with a workspace each, chunks dealt to them in turn
         "two_chunks_in_flight": {"ms_per_chunk": dt2 / steps * 1e3, "tokens_per_s": CH * steps / dt2} if dt2 else None,
+        "q8_1_family": q8,
     }
     return line
 

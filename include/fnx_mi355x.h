@@ -251,6 +251,18 @@ int fnx_pf_route(const float* logits, int logits_stride, int C, int nexp, int to
                  fnx_bigjob* jobs_gu, fnx_bigjob* jobs_dn, int njobs_cap, int* njobs, void* st);
 /* kernels.hpp (p100_f32_f16): f32 -> f16, round to nearest even */
 int fnx_f32_f16(const float* x, size_t n, uint16_t* out, void* st);
+/* kernels.hpp:324-325  moe_gate_up_big, moe_down_big: the prompt path's jobs over q8_1 activations (the reference's moe_q8
+ * mode of the prompt pass, prefill.cu:1842-1844) - fnx_moe_gate_up's and fnx_moe_down's terms (mmvq semantics: integer dot
+ * products of a sub-block, then d_w (1 + 2 s) d_x) for jobs of up to FNX_PF_JOB rows. gate_up: gu[jobs.out][2 ffs] from the
+ * q8_1 rows xq[jobs.y] of A->n_in values; down: part[jobs.out][n] from h = silu(gate) * up of the rows gu[jobs.y] ([gate |
+ * up] of 2 * A->n_in floats), quantised to q8_1 on the way (moe.cuh:597-608). tile16 matrices (rows in 16s, 512 .. 2048
+ * columns in 512s), 1 .. 4096 jobs a launch; a job's rows go sixteen at a time through the int8 matrix cores. The two
+ * families of prompt kernels - these and the f16 ones below - differ by the activations' q8_1 rounding: a caller's choice,
+ * as the reference's. */
+int fnx_moe_gate_up_big(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const int* njobs, int njobs_cap, const void* xq, float* gu,
+                        void* st);
+int fnx_moe_down_big(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const int* njobs, int njobs_cap, const float* gu, float* part,
+                     void* st);
 /* kernels.hpp:328  moe_gate_up_mma: gu[jobs.out][2 ffs] = W_e[2 ffs][n] . xh[jobs.y] with f16 weights (each the f32
  * value rounded once), f16 activations, fp32 accumulation, on the matrix cores. xh rows of A->n_in halves. Raw blocks and
  * unit64 (tile16 gate|up matrices go through fnx_moe_gate_up_h16_mma, which leaves h). */

@@ -270,6 +270,10 @@ struct RowsArgs {
     const uint8_t* y;   // q8_1 rows; null: the library's pair buffer
     float* out;
     int out_stride;
+    // the prompt path's jobs of up to FNX_PF_JOB rows (k_iq3s_jobs_mma16<1 | 2>), instead of `jobs`; gu: their activations are
+    // made on the way from rows [gate | up] of 2 ncols floats (h = silu(gate) * up as q8_1), instead of read from y
+    const fnx_bigjob* big = nullptr;
+    const float* gu = nullptr;
 };
 
 struct RawSub {   // one lane's share of a unit as read from memory; nothing is combined until it is used
@@ -792,7 +796,7 @@ static int rows_launch(const fnx_dw* W, size_t w_stride, const fnx_job* jobs, co
         const RowsArgs a{(const uint8_t*) W->p, w_stride, (const uint8_t* const*) W->ep, W->row_bytes, W->n_out, W->n_in,
                          jobs, njobs, njobs_max, (const uint8_t*) y, out, out_stride};
         const long items = (long) njobs_max * (W->n_out / 16);
-        k_iq3s_jobs_mma16<<<(int) std::max(1L, std::min((long) cu_count(), items)), J16_THREADS, 0, (hipStream_t) st>>>(a);
+        k_iq3s_jobs_mma16<0><<<(int) std::max(1L, std::min((long) cu_count(), items)), J16_THREADS, 0, (hipStream_t) st>>>(a);
         return launch_status(who);
     }
     if (W->type != FNX_T_IQ3_S && W->type != FNX_T_IQ3S_UNIT64)
@@ -1031,6 +1035,39 @@ int fnx_moe_down(const fnx_dw* A, size_t sa, const fnx_job* jobs, const int* njo
     k_swiglu_q8_1<<<dim3((ffs / 32 + 7) / 8, njobs_max), 256, 0, (hipStream_t) st>>>(gu, gu + ffs, (size_t) 2 * ffs, nullptr, ffs);
     if (launch_status("moe_down")) return 1;
     return rows_launch(A, sa, jobs, njobs, njobs_max, nullptr, part, A->n_out, st, "moe_down");
+}
+// the prompt path's jobs over q8_1 activations (kernels.hpp:324-325): tile16 matrices, a job's rows sixteen at a time on the
+// int8 matrix cores (k_iq3s_mma16.h)
+static int big_launch(const fnx_dw* W, size_t w_stride, const fnx_bigjob* jobs, const int* njobs, int njobs_cap, const void* xq, const float* gu,
+                      float* out, const char* who) {
+    if (!W || !jobs || !njobs || !out || (!xq && !gu)) return fail(std::string(who) + ": null argument");
+    if (W->type != FNX_T_IQ3S_TILE16) return fail(std::string(who) + ": jobs of up to FNX_PF_JOB rows take tile16 matrices (fnx_iq3s_tile16)");
+    if (W->n_in <= 0 || W->n_in % 512 || W->n_in > J16_MAXCOLS || W->n_out <= 0 || W->n_out % 16)
+        return fail(std::string(who) + ": the tile16 layout takes rows in 16s and 512, 1024, 1536 or 2048 columns here");
+    if (W->row_bytes != (size_t) (W->n_in / 256) * FNX_IQ3S_BLOCK) return fail(std::string(who) + ": row_bytes does not match n_in");
+    if (njobs_cap < 1 || njobs_cap > J16_MAXJOBS) return fail(std::string(who) + ": 1 .. 4096 jobs a launch");
+    if (!W->p && !W->ep) return fail(std::string(who) + ": no weights");
+    if (gu && ((uintptr_t) gu & 15)) return fail(std::string(who) + ": 16-byte aligned rows");
+    return 0;
+}
+int fnx_moe_gate_up_big(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const int* njobs, int njobs_cap, const void* xq, float* gu, void* st) {
+    if (big_launch(A, sa, jobs, njobs, njobs_cap, xq, nullptr, gu, "moe_gate_up_big")) return 1;
+    RowsArgs a{(const uint8_t*) A->p, sa, (const uint8_t* const*) A->ep, A->row_bytes, A->n_out, A->n_in, nullptr, njobs, njobs_cap,
+               (const uint8_t*) xq, gu, A->n_out};
+    a.big = jobs;
+    const long items = (long) njobs_cap * (FNX_PF_JOB / FNX_MAXT) * (A->n_out / 16);
+    k_iq3s_jobs_mma16<1><<<(int) std::max(1L, std::min((long) cu_count(), items)), J16_THREADS, 0, (hipStream_t) st>>>(a);
+    return launch_status("moe_gate_up_big");
+}
+int fnx_moe_down_big(const fnx_dw* A, size_t sa, const fnx_bigjob* jobs, const int* njobs, int njobs_cap, const float* gu, float* part, void* st) {
+    if (big_launch(A, sa, jobs, njobs, njobs_cap, nullptr, gu, part, "moe_down_big")) return 1;
+    RowsArgs a{(const uint8_t*) A->p, sa, (const uint8_t* const*) A->ep, A->row_bytes, A->n_out, A->n_in, nullptr, njobs, njobs_cap,
+               nullptr, part, A->n_out};
+    a.big = jobs;
+    a.gu = gu;
+    const long items = (long) njobs_cap * (FNX_PF_JOB / FNX_MAXT) * (A->n_out / 16);
+    k_iq3s_jobs_mma16<2><<<(int) std::max(1L, std::min((long) cu_count(), items)), J16_THREADS, 0, (hipStream_t) st>>>(a);
+    return launch_status("moe_down_big");
 }
 int fnx_moe_combine(const float* part, const float* topw, const float* sh, const float* sh_logit, int sh_logit_stride, float* out, int T, int n,
                     int topk, void* st) {

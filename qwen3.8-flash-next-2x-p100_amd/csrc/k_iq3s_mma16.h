@@ -36,12 +36,12 @@ struct J16Lds {
 };
 
 // tiles [g0, g1) of 16 rows of matrix `we` (ncols columns) against the job's tokens, staged in L: the whole block
-__device__ __forceinline__ void j16_segment(J16Lds& L, const uint8_t* __restrict__ we, int g0, int g1, int ncols, const fnx_job* __restrict__ jb, int n,
+__device__ __forceinline__ void j16_segment(J16Lds& L, const uint8_t* __restrict__ we, int g0, int g1, int ncols, const int* __restrict__ outs, int n,
                                             float* __restrict__ out, int out_stride) {
     const int lane = threadIdx.x & 63, wave = uniform((int) (threadIdx.x >> 6));
     const int r = lane & 15, grp = lane >> 4;   // decoding: row r of the tile, lane group grp; accumulating: token r, rows 4 grp .. 4 grp + 3
     const int nsuper = ncols / 512;
-    float* orow = out + (size_t) (r < n ? jb->out[r] : 0) * out_stride + 4 * grp;
+    float* orow = out + (size_t) (r < n ? outs[r] : 0) * out_stride + 4 * grp;
     const uint8_t* xrow = L.xq + r * J16_XLD + 8 * grp;   // bytes 8 grp .. of sub-block 16 S + 4 j + p of token r lie 512 S + 128 j + 32 p further
     float* myw = &L.sw[wave][grp][r];
     const uint32_t copy_at = 4u * (lane & 1);
@@ -100,36 +100,112 @@ __device__ __forceinline__ void j16_segment(J16Lds& L, const uint8_t* __restrict
 
 // tile16 matrices of up to 2048 columns (a multiple of 512), rows in 16s. The blocks split the (job, tile of 16 rows) items
 // of all jobs evenly and walk them in order; a job's activations are staged when the block comes to it.
+// MODE 0: jobs of up to FNX_MAXT rows (kernels.hpp:18-23) over q8_1 rows. MODE 1: the prompt path's jobs of up to
+// FNX_PF_JOB rows (kernels.hpp:324, moe_gate_up_big): a job's rows in tiles of sixteen, each (job, token tile) a unit that
+// is staged and walked like a job of MODE 0; the units are counted first (a prefix sum over the jobs' tile counts in LDS)
+// so that the blocks split live units only. MODE 2 (kernels.hpp:325, moe_down_big): the same with the unit's activations
+// made on the way from the rows [gate | up] of 2 ncols floats: h = silu(gate) * up quantised as k_swiglu_q8_1 does it.
+constexpr int J16_MAXJOBS = 4096;   // big jobs a launch (their tile counts' prefix sums live in LDS)
+template <int MODE>
 __global__ void __launch_bounds__(J16_THREADS) k_iq3s_jobs_mma16(const RowsArgs a) {
     __shared__ J16Lds L;
+    __shared__ uint32_t before[MODE ? J16_MAXJOBS + 1 : 1];   // units of the jobs before job j
     for (int g = threadIdx.x; g < 512; g += J16_THREADS) {   // a code's sixteen signed entries from its unsigned one
         const uint32_t g0 = g_sgrid.v[g];
 #pragma unroll
         for (int sg = 0; sg < 16; ++sg) L.tab[2 * (sg * 512 + g)] = L.tab[2 * (sg * 512 + g) + 1] = signed_entry(g0, sg);
     }
-    const int nj = a.njobs ? min(uniform(*a.njobs), a.njobs_max) : a.njobs_max;
-    const uint32_t gpj = (uint32_t) a.nrows / 16;   // items per job
-    const unsigned long long total = (unsigned long long) nj * gpj;
+    const int nj = min(a.njobs ? min(uniform(*a.njobs), a.njobs_max) : a.njobs_max, MODE ? J16_MAXJOBS : a.njobs_max);
+    const uint32_t gpj = (uint32_t) a.nrows / 16;   // items per unit
+    uint32_t units = (uint32_t) nj;
+    if constexpr (MODE != 0) {
+        // token tiles a job, then their running sum: a wave's lanes take consecutive runs of jobs
+        for (int j = threadIdx.x; j < nj; j += J16_THREADS) before[j + 1] = (uint32_t) (min(max(a.big[j].n, 0), FNX_PF_JOB) + 15) / 16;
+        if (threadIdx.x == 0) before[0] = 0;
+        __syncthreads();
+        if (threadIdx.x < 64) {
+            const int per = (nj + 63) / 64, j0 = min(nj, (int) threadIdx.x * per), j1 = min(nj, j0 + per);
+            uint32_t mine = 0;
+            for (int j = j0; j < j1; ++j) mine += before[j + 1];
+            uint32_t incl = mine;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {
+                const uint32_t v = __shfl_up(incl, o, 64);
+                if ((int) threadIdx.x >= o) incl += v;
+            }
+            uint32_t run = incl - mine;
+            for (int j = j0; j < j1; ++j) {
+                run += before[j + 1];
+                before[j + 1] = run;
+            }
+        }
+        __syncthreads();
+        units = before[nj];
+    }
+    const unsigned long long total = (unsigned long long) units * gpj;
     uint32_t i = (uint32_t) (total * blockIdx.x / gridDim.x);
     const uint32_t i1 = (uint32_t) (total * (blockIdx.x + 1) / gridDim.x);
     const uint8_t* y = a.y ? a.y : g_moe_hq;
     const int nsb = a.ncols / 32;
     while (i < i1) {
-        const uint32_t ji = i / gpj;
-        const int g0 = (int) (i - ji * gpj), g1 = (int) min(gpj, g0 + (i1 - i));
-        const fnx_job* jb = a.jobs + ji;
-        const int n = uniform(min(jb->n, FNX_MAXT)), w = uniform(jb->w);
+        const uint32_t ui = i / gpj;
+        const int g0 = (int) (i - ui * gpj), g1 = (int) min(gpj, g0 + (i1 - i));
+        int n, w;
+        const int *ys, *outs;
+        if constexpr (MODE == 0) {
+            const fnx_job* jb = a.jobs + ui;
+            n = uniform(min(jb->n, FNX_MAXT)), w = uniform(jb->w);
+            ys = jb->y, outs = jb->out;
+        } else {
+            int lo = 0, hi = nj - 1;   // the job whose units hold ui: before[j] <= ui < before[j + 1]
+            while (lo < hi) {
+                const int mid = (lo + hi) >> 1;
+                if (before[mid + 1] <= ui) lo = mid + 1;
+                else hi = mid;
+            }
+            const fnx_bigjob* jb = a.big + uniform(lo);
+            const int q = (int) (ui - before[lo]);
+            n = uniform(min(min(max(jb->n, 0), FNX_PF_JOB) - 16 * q, FNX_MAXT)), w = uniform(jb->w);
+            ys = jb->y + 16 * q, outs = jb->out + 16 * q;
+        }
         const uint8_t* we = a.ep ? uniform_ptr(a.ep[w]) : a.wbase + (size_t) w * a.w_stride;
-        __syncthreads();   // the job before has been read (and the codebook written)
+        __syncthreads();   // the unit before has been read (and the codebook written)
         for (int q = threadIdx.x; q < FNX_MAXT * nsb; q += J16_THREADS) {   // (token, sub-block): its 32 int8 and its scale
             const int t = q / nsb, sb = q - t * nsb;
             uint32_t v[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};
             float d = 0.f;
             if (t < n) {
-                const uint8_t* yb = y + ((size_t) jb->y[t] * nsb + sb) * FNX_Q8_1_BLOCK;
-                d = half_bits_to_float(*reinterpret_cast<const unsigned short*>(yb));
+                if constexpr (MODE == 2) {
+                    const float* gp = a.gu + (size_t) ys[t] * (2 * a.ncols) + 32 * sb;
+                    float4 gv[8], uv[8];
 #pragma unroll
-                for (int k = 0; k < 8; ++k) v[k] = *reinterpret_cast<const uint32_t*>(yb + 4 + 4 * k);
+                    for (int k = 0; k < 8; ++k) gv[k] = reinterpret_cast<const float4*>(gp)[k], uv[k] = reinterpret_cast<const float4*>(gp + a.ncols)[k];
+                    float h[32], amax = 0.f;
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) {
+                        h[4 * k] = silu_f(gv[k].x) * uv[k].x, h[4 * k + 1] = silu_f(gv[k].y) * uv[k].y;
+                        h[4 * k + 2] = silu_f(gv[k].z) * uv[k].z, h[4 * k + 3] = silu_f(gv[k].w) * uv[k].w;
+                    }
+#pragma unroll
+                    for (int k = 0; k < 32; ++k) amax = fmaxf(amax, fabsf(h[k]));
+                    const float dq = amax / 127.0f;   // q8_1_store's arithmetic (kernels.cu:131-145)
+                    d = half_bits_to_float(float_to_half_bits(dq));
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) {
+                        uint32_t word = 0;
+#pragma unroll
+                        for (int b = 0; b < 4; ++b) {
+                            const int8_t qv = amax == 0.0f ? (int8_t) 0 : (int8_t) roundf(h[4 * k + b] / dq);
+                            word |= (uint32_t) (uint8_t) qv << (8 * b);
+                        }
+                        v[k] = word;
+                    }
+                } else {
+                    const uint8_t* yb = y + ((size_t) ys[t] * nsb + sb) * FNX_Q8_1_BLOCK;
+                    d = half_bits_to_float(*reinterpret_cast<const unsigned short*>(yb));
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) v[k] = *reinterpret_cast<const uint32_t*>(yb + 4 + 4 * k);
+                }
             }
             uint32_t* dst = reinterpret_cast<uint32_t*>(L.xq + t * J16_XLD + 32 * sb);
 #pragma unroll
@@ -137,7 +213,7 @@ __global__ void __launch_bounds__(J16_THREADS) k_iq3s_jobs_mma16(const RowsArgs 
             L.dx[(((sb >> 4) * 4 + (sb & 3)) * FNX_MAXT + t) * 4 + ((sb >> 2) & 3)] = d;
         }
         __syncthreads();
-        if (n >= 1) j16_segment(L, we, g0, g1, a.ncols, jb, n, a.out, a.out_stride);
+        if (n >= 1) j16_segment(L, we, g0, g1, a.ncols, outs, n, a.out, a.out_stride);
         i += (uint32_t) (g1 - g0);
     }
 }

@@ -322,6 +322,27 @@ class Dev:
         return out.cpu().numpy()
 
 
+    def moe_big(self, w, w_stride, nrows, ncols, jobs, acts, out_rows, down=False, cap=None):
+        """the prompt path's jobs over q8_1 activations (fnx_moe_gate_up_big / fnx_moe_down_big), tile16 matrices.
+        jobs: int32 [njobs][130]; acts: q8_1 rows as bytes (gate|up), or f32 rows [gate | up] of 2 ncols (down)"""
+        t = self.torch
+        cap = cap or len(jobs)
+        jpad = np.zeros((cap, 130), dtype=np.int32)
+        jpad[:len(jobs)] = jobs
+        dw_, dj, da = self.up(w), self.up(jpad), self.up(np.ascontiguousarray(acts))
+        self.ok(self.lib.fnx_iq3s_repack(dw_.data_ptr(), dw_.data_ptr(), w.size // 110 * 256, self.st()))
+        nmat = w.size // (nrows * ncols // 256 * 110)
+        d16 = self.zeros(self.lib.fnx_iq3s_tile16_bytes(nrows, ncols, nmat), t.uint8)
+        self.ok(self.lib.fnx_iq3s_tile16(dw_.data_ptr(), d16.data_ptr(), nrows, ncols, nmat, self.st()))
+        W = self.pkg.dw(d16, ncols, nrows, tile16=True)
+        w_stride = self.lib.fnx_iq3s_tile16_bytes(nrows, ncols, 1) if w_stride else 0
+        nj = self.up(np.array([len(jobs)], dtype=np.int32))
+        out = self.zeros((out_rows, nrows), t.float32)
+        fn = self.lib.fnx_moe_down_big if down else self.lib.fnx_moe_gate_up_big
+        self.ok(fn(C.byref(W), w_stride, dj.data_ptr(), nj.data_ptr(), cap, da.data_ptr(), out.data_ptr(), self.st()))
+        self.sync()
+        return out.cpu().numpy()
+
     # ---- around the MoE half
     def rms_norm_rows(self, x, w, eps):
         dx, dw_ = self.up(x.astype(np.float32)), self.up(w.astype(np.float32))

@@ -97,6 +97,13 @@ inline void pf_route(const float* logits, int C, int* topi, float* topw, int* cn
     ck(fnx_pf_route(logits, shape().NEXP + 1, C, shape().NEXP, shape().TOPK, topi, topw, cnt, jbase, jobs_gu, jobs_dn, njobs_cap, njobs, st));
 }
 inline void p100_f32_f16(const float* x, size_t n, uint16_t* out, void* st) { ck(fnx_f32_f16(x, n, out, st)); }
+// kernels.hpp:324-325
+inline void moe_gate_up_big(const DW& A, size_t sa, const BigJob* jobs, const int* njobs, int njobs_cap, const void* xq, float* gu, void* st) {
+    ck(fnx_moe_gate_up_big(&A, sa, jobs, njobs, njobs_cap, xq, gu, st));
+}
+inline void moe_down_big(const DW& A, size_t sa, const BigJob* jobs, const int* njobs, int njobs_cap, const float* gu, float* part, void* st) {
+    ck(fnx_moe_down_big(&A, sa, jobs, njobs, njobs_cap, gu, part, st));
+}
 inline void moe_gate_up_mma(const DW& A, size_t sa, const BigJob* jobs, const int* njobs, int njobs_cap, const uint16_t* xh, float* gu, void* st) {
     ck(fnx_moe_gate_up_mma(&A, sa, jobs, njobs, njobs_cap, xh, gu, st));
 }

@@ -70,6 +70,10 @@ def test_the_grouped_gemm_takes_tile16_in_its_two_forms_only():
     for packed in (False, True):
         w = pkg.dw(buf, 2048, 1024, packed=packed)
         assert lib.fnx_moe_gate_up_h16_mma(C.byref(w), 0, buf, buf, 4, buf, buf, None) != 0 and b"h alone" in lib.fnx_last_error()
+        # the q8_1 family's jobs of up to 64 rows: tile16 only
+        assert lib.fnx_moe_gate_up_big(C.byref(w), 0, buf, buf, 4, buf, buf, None) != 0 and b"tile16" in lib.fnx_last_error()
+        assert lib.fnx_moe_down_big(C.byref(w), 0, buf, buf, 4, buf, buf, None) != 0 and b"tile16" in lib.fnx_last_error()
+    assert lib.fnx_moe_gate_up_big(C.byref(gu16), 0, buf, buf, 5000, buf, buf, None) != 0 and b"4096" in lib.fnx_last_error()
 
 
 def test_a_layer_wider_than_the_pair_buffer_is_refused():

@@ -175,6 +175,49 @@ def test_moe_gate_up_h16_one_launch_equals_two(dev, oracle, ffs, ncols, nexp, si
         assert rel_l2(one.astype(np.float32), want.astype(np.float32)) <= 1e-3
 
 
+def split_in_16s(jobs):
+    """jobs of up to 64 rows as the jobs of up to 16 rows they consist of (the oracle's mmvq takes those)"""
+    out = []
+    for jb in jobs:
+        n = int(jb[1])
+        for t0 in range(0, n, 16):
+            k = min(16, n - t0)
+            j = np.zeros(1, dtype=fnx_gpu.JOB_DTYPE)
+            j["w"], j["n"] = jb[0], k
+            j["y"][0, :k], j["out"][0, :k] = jb[2 + t0:2 + t0 + k], jb[2 + PF + t0:2 + PF + t0 + k]
+            out.append(j)
+    return np.concatenate(out) if out else np.zeros(0, dtype=fnx_gpu.JOB_DTYPE)
+
+
+@pytest.mark.parametrize("nrows,ncols,nexp,sizes", [(1024, 2048, 24, [64, 1, 17, 0, 16, 33, 48, 5, 64, 64, 2, 0, 31, 64, 49, 15] * 3), (64, 512, 3, [64, 1, 17, 16, 33, 48, 5]),
+                                                  (32, 1024, 2, [3]), (2048, 512, 2, [64, 9, 0, 0, 40])])
+def test_moe_big_jobs_over_q8_1_match_the_oracle(dev, oracle, nrows, ncols, nexp, sizes):
+    """kernels.hpp:324-325: the prompt path's jobs with mmvq's terms. gate|up form: q8_1 rows in, the oracle's mmvq over the same
+    jobs cut into sixteens; down form (where the matrix's columns allow rows [gate | up]): h = silu(gate) * up quantised on
+    the way, against the oracle's SwiGLU -> q8_1 -> mmvq. The integer sums are exact; a row's sub-block terms are added in
+    another order than the oracle's."""
+    print(f"case moe_big nrows={nrows} ncols={ncols} nexp={nexp} jobs={len(sizes)}", flush=True)
+    rng = np.random.default_rng(771 + nrows + len(sizes))
+    stride = nrows * ncols // 256 * 110
+    w = random_iq3s(rng, nexp * nrows * ncols // 256, dmax=2e-2)
+    rows = max(200, sum(sizes))
+    jobs, total = make_jobs(rng, nexp, rows, sizes)
+    small = split_in_16s(jobs)
+    x = rng.standard_normal((rows, ncols)).astype(np.float32)
+    xq = oracle.quantize_q8_1(x)
+    want = oracle.mmvq(w, stride, nrows, ncols, small, xq, total + 3)
+    got = dev.moe_big(w, stride, nrows, ncols, jobs, xq, total + 3, cap=len(jobs) + 5)
+    assert rel_l2(got, want) <= 1e-5
+    assert np.any(got[:total] != 0) and not np.any(got[total:])
+    # the down form: the same matrix read as rows of ncols = ffs, fed rows [gate | up]
+    gu = (rng.standard_normal((rows, 2 * ncols)) * 2).astype(np.float32)
+    hq = oracle.swiglu_stacked_q8_1(gu, ncols)
+    want = oracle.mmvq(w, stride, nrows, ncols, small, hq, total + 3)
+    got = dev.moe_big(w, stride, nrows, ncols, jobs, gu, total + 3, down=True, cap=len(jobs) + 5)
+    assert rel_l2(got, want) <= 1e-5
+    assert not np.any(got[total:])
+
+
 def test_moe_mma_weights_equal_the_oracles_f16(dev, oracle):
     # x = unit vectors: the product returns single weights, so every dequantised f16 value is checked bit for bit,
     # subnormal ones included (tiny d)
