@@ -584,7 +584,7 @@ def head_main(args):
                        "identical_to_oracle": same},
             "roofline": {"bound": "hbm", "kernel": "k_argmax", "achieved": arg_bytes / (us_arg * 1e-6) / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                          "frac": arg_bytes / (us_arg * 1e-6) / HBM_PEAK, "traffic": None, "algorithmic_bytes": arg_bytes,
-                         "note": "two launches of about 4 us fixed cost each; the scan itself is 1.2 us at peak"},
+                         "note": "one launch whose rows' last blocks decode the keys: about 4 us of fixed cost and 3 us for the chain of atomics at its end; the scan itself is 1.2 us at peak"},
             "cpu_baseline": None if not reps else {"value": 1e6 / cpu_us, "unit": "rounds/s", "cores": 1, "kind": "port",
                                                    "sample": f"{reps} rounds of lookup + acceptance on the oracle (the argmax scan once)"}}
     return line
@@ -717,7 +717,7 @@ def decoder_main(args):
             kc[:CTX - R], vc[:CTX - R] = k.view(np.uint16), v.view(np.uint16)
         rows = [int(x) for x in toks[0].cpu().numpy()]
         c0 = time.perf_counter()
-        a = sess.verify(rows, CTX - R, routing=True)
+        a = sess.verify(rows, CTX - R, routing=True, taps=True)
         na = oracle.accept_greedy(np.asarray(rows, dtype=np.int32), a["best"])
         da = sess.draft(a["hidden"], rows, CTX - R)
         cdt = time.perf_counter() - c0
@@ -730,6 +730,22 @@ def decoder_main(args):
         rows_h = [rel(got["hidden"][r_], a["hidden"][r_]) for r_ in range(R) if same_route[r_]]
         rows_l = [rel(got["logits"][r_], a["logits"][r_]) for r_ in range(R) if same_route[r_]]
         gd = dd.draft(a["hidden"], rows, CTX - R)
+        # where the chain's rows can part from the oracle's: the q8_1 codes of each layer's output-projection input (the
+        # attention's rows), the device's chain walked layer by layer (fnx_decoder_layer: the window's own launches)
+        def differ(l, r):
+            want_q = oracle.quantize_q8_1(a["taps"]["att"][l]).reshape(r["att_q8"].shape)
+            return (int(np.count_nonzero(r["att_q8"][..., 4:] != want_q[..., 4:])) +
+                    int(np.count_nonzero(r["att_q8"][..., :2].view(np.uint16) != want_q[..., :2].view(np.uint16))))
+
+        code_steps, own_steps, layer_rel, x = [], [], [], a["taps"]["x_in"][0]
+        for l in range(NL):
+            r = dd.layer(x, l, CTX - R)
+            code_steps.append(differ(l, r))
+            x = r["x_mid"] + r["moe"]
+            # the same layer on the oracle's own input rows: the steps that start in this layer, and the layer's rows against the oracle's
+            r = dd.layer(a["taps"]["x_in"][l], l, CTX - R)
+            own_steps.append(differ(l, r))
+            layer_rel.append(rel(r["x_mid"] + r["moe"], a["taps"]["x_mid"][l] + a["taps"]["moe"][l]))
         cpu = {"value": 1.0 / cdt, "unit": "steps/s", "cores": threads, "kind": "port",
                "sample": "1 step of the same workload (window of 16 rows at position 32,752, acceptance, draft layer) on the oracle",
                "parity": {"rows_routed_as_the_oracle": int(sum(same_route)), "rows": R,
@@ -740,10 +756,16 @@ def decoder_main(args):
                           "logits_rel_l2_rows_max": max(rows_l), "logits_rel_l2_rows_median": float(np.median(rows_l)),
                           "draft_picks_identical": int(np.count_nonzero(gd["best"] == da["best"])),
                           "draft_hidden_rel_l2": rel(gd["hidden"], da["hidden"]),
+                          "q8_1_codes_and_scales_that_differ_at_each_layers_output_projection_input": code_steps,
+                          "codes_there_per_layer": int(R * NQ * HD),
+                          "the_same_with_each_layer_fed_the_oracles_rows": own_steps,
+                          "layer_output_rel_l2_with_each_layer_fed_the_oracles_rows": layer_rel,
                           "note": "float figures over the rows whose ten experts are the oracle's in every layer (a row that parts does so at a near-tie of "
-                                  "two router logits: tests/test_gpu_full_shapes.py proves it per row). Rows differ from the oracle's by steps of one "
-                                  "q8_1 code of an activation between operators (~1e-3 of a row each, set off by last-bit differences); rows without "
-                                  "one agree to 1e-6"}}
+                                  "two router logits: tests/test_gpu_full_shapes.py proves it per row). The MoE half is the oracle's bit for bit on equal "
+                                  "inputs; the attention's rows differ in the last bits (MFMA sums, sin/cos), which now and then moves one q8_1 code of the "
+                                  "output projection's input by one step (counted above, per layer): ~1e-3 of that row, carried on by the layers after it; "
+                                  "rows without a step upstream are the oracle's bit for bit. A layer fed the oracle's own rows meets 1e-3 over the whole tensor and starts a handful of "
+                                  "steps at most; the counts of the chain's later layers are those first steps' consequences (rows already 1e-3 apart flip codes by the percent)"}}
     kv_bytes = 2 * CTX * NKV * HD * 2
     head_bytes = V * N + V * (N // 32) * 2
     dense_bytes = (NQ * 2 * HD * N + 2 * NKV * HD * N + N * NQ * HD) * 34 // 32

@@ -221,6 +221,10 @@ int fnx_moe_verify_layer(const fnx_moe_layer* L, const float* x, int T, float* o
  * GPU's array: two of them in flight at once (two streams, two threads) race. */
 #define FNX_MOE_STATIC_WS_BYTES (448 * 1024)
 int fnx_moe_verify_layer_static(const fnx_moe_layer* L, const float* x, int T, float* out, void* st);
+/* The error word of that array's windows (fnx_moe_ws.sync word 0 of the library's own workspace on the current device),
+ * for the caller who cannot see it otherwise: waits for the stream, copies the word to *err and, if FNX_ERR_BARRIER is set
+ * there, zeroes the array's sync words so that the next window starts clean. Not for the hot path (it synchronises). */
+int fnx_moe_static_status(unsigned* err, void* st);
 /* Profiling aid, the counterpart of the reference's FNX_PROF stamps in its window graph (engine.cu:1382-1530):
  * fnx_layer_profile(1) makes the one-launch window record events on its stream around its launch (not to be used under
  * graph capture), fnx_layer_profile(0) stops that; fnx_layer_profile_read waits for the last recorded window and returns two

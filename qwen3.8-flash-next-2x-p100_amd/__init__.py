@@ -132,6 +132,7 @@ EXPORTS = {
     "fnx_stream_read": (C.c_int, [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]),
     "fnx_moe_verify_layer": (C.c_int, [C.POINTER(MoeLayer), C.c_void_p, C.c_int, C.c_void_p, C.POINTER(MoeWs), C.c_void_p]),
     "fnx_moe_verify_layer_static": (C.c_int, [C.POINTER(MoeLayer), C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
+    "fnx_moe_static_status": (C.c_int, [C.c_void_p, C.c_void_p]),
     "fnx_pf_route": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
     "fnx_f32_f16": (C.c_int, [C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p]),

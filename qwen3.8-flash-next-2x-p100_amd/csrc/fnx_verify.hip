@@ -753,6 +753,30 @@ struct BufferOrder {
     }
 };
 static BufferOrder g_pair_order, g_cand_order;
+// The one-launch window's blocks wait for each other, which needs all of them resident: a grid of one block a CU, alone
+// on the chip. Two windows enqueued on two streams could be dispatched block by block beside each other, each holding
+// CUs the other waits for, until both give up their waits. So a window on another stream than the window before it first
+// waits for everything enqueued on that stream so far (an event recorded there now); windows on one stream, the usual
+// case, pay nothing. A stream under graph capture is left alone, as in BufferOrder.
+struct WindowOrder {
+    std::mutex m;
+    hipEvent_t ev[64] = {};
+    hipStream_t last[64] = {};
+    bool used[64] = {};
+    void enter(hipStream_t s) {
+        int dev = -1;
+        if (BufferOrder::capturing(s) || hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return;
+        std::lock_guard<std::mutex> g(m);
+        if (used[dev] && last[dev] != s) {
+            if (!ev[dev] && hipEventCreateWithFlags(&ev[dev], hipEventDisableTiming) != hipSuccess) ev[dev] = nullptr;
+            if (ev[dev] && hipEventRecord(ev[dev], last[dev]) == hipSuccess) (void) hipStreamWaitEvent(s, ev[dev], 0);
+            else (void) hipGetLastError();   // (the stream before may be gone: then nothing of it is left to wait for)
+        }
+        used[dev] = true;
+        last[dev] = s;
+    }
+};
+static WindowOrder g_window_order;
 struct BufferScope {   // enter now, leave when the call returns
     BufferOrder& o;
     hipStream_t s;
@@ -869,6 +893,7 @@ static void prof_mark(int i, hipStream_t s) {
 static int layer_fused(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st, const int* live = nullptr) {
     hipStream_t s = (hipStream_t) st;
     const int n = L->n, ff = L->ff;
+    g_window_order.enter(s);
     prof_mark(0, s);
     // a split-Q8_0 shared expert runs as the reference runs it, three dense launches on the q8_1 rows of x
     // (q8s_gemv -> swiglu_stacked_q8_1 -> q8s_gemv); its f32 rows, q8_1 rows of h and down rows take the workspace's
@@ -1212,24 +1237,43 @@ static_assert(NA_BYTES <= FNX_MOE_STATIC_WS_BYTES, "the header states the array'
 static __device__ __align__(256) unsigned char scratch[FNX_MOE_STATIC_WS_BYTES];
 static unsigned char* g_scratch_ptr[64] = {};   // per device: the array's address there
 static std::mutex g_scratch_mutex;
+// the array's address on the current device: asked once per device, with that device current; threads that arrive together
+// take turns (a failed query is asked again)
+static unsigned char* static_ws(const char* who) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+        fail(std::string(who) + ": no current device");
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> g(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        unsigned char* p = nullptr;
+        const hipError_t e = hipGetSymbolAddress((void**) &p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            fail(std::string(who) + ": hipGetSymbolAddress: " + hipGetErrorString(e));
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = p;
+    }
+    return g_scratch_ptr[dev];
+}
+int fnx_moe_static_status(unsigned* err, void* st) {
+    if (!err) return fail("moe_static_status: null argument");
+    unsigned char* w = static_ws("moe_static_status");
+    if (!w) return 1;
+    if (hipStreamSynchronize((hipStream_t) st) != hipSuccess) return fail("moe_static_status: the stream failed");
+    if (hipMemcpy(err, w + NA_OFF_SYNC, sizeof(unsigned), hipMemcpyDeviceToHost) != hipSuccess) return fail("moe_static_status: copy failed");
+    if (*err && hipMemset(w + NA_OFF_SYNC, 0, FNX_MOE_SYNC_WORDS * sizeof(unsigned)) != hipSuccess) return fail("moe_static_status: reset failed");
+    return 0;
+}
 int fnx_moe_verify_layer_static(const fnx_moe_layer* L, const float* x, int T, float* out, void* st) {
     if (!L || !x || !out) return fail("moe_verify_layer_static: null argument");
     if (T < 1 || T > FNX_MAXT) return fail("moe_verify_layer_static: T out of range");
     if (!layer_fused_ok(L, T))
         return fail("moe_verify_layer_static: only the one-launch window runs on the library's own workspace (unit64 experts, hidden 2048, "
                     "ff 256 / 512 / 1024, up to 1024 experts, up to 16 picks a row, up to 160 pairs a window)");
-    int dev = -1;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return fail("moe_verify_layer_static: no current device");
-    {   // once per device, with that device current; threads that arrive together take turns (a failed query is asked again)
-        std::lock_guard<std::mutex> g(g_scratch_mutex);
-        if (!g_scratch_ptr[dev]) {
-            unsigned char* p = nullptr;
-            const hipError_t e = hipGetSymbolAddress((void**) &p, HIP_SYMBOL(scratch));
-            if (e != hipSuccess || !p) return fail(std::string("moe_verify_layer_static: hipGetSymbolAddress: ") + hipGetErrorString(e));
-            g_scratch_ptr[dev] = p;
-        }
-    }
-    unsigned char* w = g_scratch_ptr[dev];
+    unsigned char* w = static_ws("moe_verify_layer_static");
+    if (!w) return 1;
     // the sync words start at zero with the device image and every window leaves them zero; nothing else has to: every
     // launch writes what it reads, and the job count is stored, not added to
     const fnx_moe_ws ws{w, (float*) (w + NA_OFF_LOGITS), (int*) (w + NA_OFF_TOPI), (float*) (w + NA_OFF_TOPW), (fnx_job*) (w + NA_OFF_JGU),

@@ -31,6 +31,9 @@ def test_static_workspace_window_equals_the_workspace_one():
         dev.sync()
         got = out.cpu().numpy()
         assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), f"T={T}: the two windows differ"
+        err = C.c_uint(99)
+        dev.ok(dev.lib.fnx_moe_static_status(C.byref(err), dev.st()))
+        assert err.value == 0, "no block of the window gave up a wait"
     # shapes beyond the array are refused with a message, before any launch
     raw = fnx_gpu.MoeLayerDev(dev, n, ff, nexp, topk, router, random_iq3s(rng, nexp * nb(2 * ff, n)), random_iq3s(rng, nexp * nb(n, ff)),
                               random_iq3s(rng, nb(2 * ff, n)), random_iq3s(rng, nb(n, ff)), packed=False)
