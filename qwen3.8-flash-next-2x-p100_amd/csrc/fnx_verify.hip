@@ -890,7 +890,20 @@ static void prof_mark(int i, hipStream_t s) {
 // the window's MoE half as one launch (k_moe_window.h): router logits, top-k, gate|up -> h as q8_1 rows (in ws->gu), down with
 // the combine's chains -> out
 // live (may be null): a device word, the rows of the window that count; the others are not routed and their rows of out are left alone
-static int layer_fused(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st, const int* live = nullptr) {
+// What a decoder does with the window's rows next, handed to the window's launch (k_moe_window.h: the row's last block):
+// x[t] += out[t], then the q8_1 rows of rms_norm(x[t]) * w, the rows after the add copied to xcopy if wanted
+// pre_w: the pass before the window too (x[t] += pre_o[t], the norm with pre_w): the window's input is then x itself
+struct WinNext {
+    float* x = nullptr;
+    const float* w = nullptr;
+    void* xq = nullptr;
+    float* xcopy = nullptr;
+    float eps = 0.f;
+    const float* pre_o = nullptr;
+    const float* pre_w = nullptr;
+};
+static int layer_fused(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st, const int* live = nullptr,
+                       const WinNext* next = nullptr) {
     hipStream_t s = (hipStream_t) st;
     const int n = L->n, ff = L->ff;
     g_window_order.enter(s);
@@ -912,14 +925,27 @@ static int layer_fused(const fnx_moe_layer* L, const float* x, int T, float* out
     prof_mark(1, s);
     // a wait for another block gives up after this many ticks of the 100 MHz wall clock (FNX_WINDOW_WAIT_TICKS: for tests of the error path)
     static const long long wait_ticks = env_int("FNX_WINDOW_WAIT_TICKS", 20000000, 0, 2000000000);
-    const WindowArgs wa{ff, L->nexp, L->topk, T, n, x, L->router, L->router_bf16,
+    WindowArgs wa{ff, L->nexp, L->topk, T, n, x, L->router, L->router_bf16,
                         (const uint8_t*) L->gu.p, L->gu_stride, (const uint8_t* const*) L->gu.ep, q8sh ? nullptr : (const uint8_t*) L->sh_gu.p,
                         (const uint8_t*) L->down.p, L->down_stride, (const uint8_t* const*) L->down.ep, q8sh ? nullptr : (const uint8_t*) L->sh_down.p,
                         sh_part, ws->logits, ws->topi, ws->topw, (uint8_t*) ws->xq, (uint32_t*) ws->gu, out, ws->sync, live,
                         ws->jobs_gu, ws->jobs_dn, ws->njobs, wait_ticks};
+    if (next && next->x) {
+        wa.next_x = next->x;
+        wa.next_w = next->w;
+        wa.next_xq = (uint8_t*) next->xq;
+        wa.next_xcopy = next->xcopy;
+        wa.next_eps = next->eps;
+        wa.pre_o = next->pre_o;
+        wa.pre_w = next->pre_w;
+    }
     // one block a CU; a row's blocks are a power of two of at least sixteen (moe_window_plan.h)
     const int nb = cu_count();
-    if (ff == 256) k_moe_window<8><<<nb, WN_THREADS, 0, s>>>(wa);
+    if (wa.next_x) {
+        if (ff == 256) k_moe_window<8, true><<<nb, WN_THREADS, 0, s>>>(wa);
+        else if (ff == 512) k_moe_window<16, true><<<nb, WN_THREADS, 0, s>>>(wa);
+        else k_moe_window<32, true><<<nb, WN_THREADS, 0, s>>>(wa);
+    } else if (ff == 256) k_moe_window<8><<<nb, WN_THREADS, 0, s>>>(wa);
     else if (ff == 512) k_moe_window<16><<<nb, WN_THREADS, 0, s>>>(wa);
     else k_moe_window<32><<<nb, WN_THREADS, 0, s>>>(wa);
     prof_mark(2, s);
@@ -1180,7 +1206,10 @@ static bool moe_shapes_ok(const fnx_moe_layer* L) {
                L->sh_down_q8.n_out == n;
     return L->sh_gu.n_in == n && L->sh_gu.n_out == 2 * ff && L->sh_down.n_in == ff && L->sh_down.n_out == n;
 }
-static int moe_layer_checked(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st, const int* live = nullptr) {
+// next (may be null): see WinNext; *next_done says whether the window's launch took it over (the one-launch window does)
+static int moe_layer_checked(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st, const int* live = nullptr,
+                             const WinNext* next = nullptr, bool* next_done = nullptr) {
+    if (next_done) *next_done = false;
     if (!L || !x || !ws) return fail("moe_verify_layer: null argument");
     if (!ws->xq || !ws->logits || !ws->topi || !ws->topw || !ws->jobs_gu || !ws->jobs_dn || !ws->njobs || !ws->gu || !ws->part || !ws->sync)
         return fail("moe_verify_layer: incomplete workspace");
@@ -1190,7 +1219,10 @@ static int moe_layer_checked(const fnx_moe_layer* L, const float* x, int T, floa
     if (!moe_shapes_ok(L)) return fail("moe_verify_layer: weight shapes do not match n / ff");
     if (!out) return fail("moe_verify_layer: null argument");
     if (live && !layer_fused_ok(L, T)) return fail("moe_verify_layer: a device-side row count needs the one-launch window");
-    if (layer_fused_ok(L, T)) return layer_fused(L, x, T, out, ws, st, live);
+    if (layer_fused_ok(L, T)) {
+        if (next_done) *next_done = next && next->x;
+        return layer_fused(L, x, T, out, ws, st, live, next);
+    }
     // operator by operator the pairs' q8_1 rows of h go through the library's pair buffer, rows of ff / 32 blocks
     if (ff <= 0 || ff % 32 || ff > HQ_MAX_FF) return fail("moe_verify_layer: expert width does not fit the pair buffer");
     hipStream_t s = (hipStream_t) st;
@@ -1604,10 +1636,15 @@ struct DecPending {
     const float* rows;
     const int* tokens;   // not null: x itself is still to come - the embedding rows of these tokens (nothing else pending then)
     const int* live;
+    // set by a layer whose window already made the pass that would come next: the add, the norm with these weights, the
+    // q8_1 rows in ws->xq and the copy (if any) - the pass is then skipped by whoever asks for exactly that
+    const float* done_w = nullptr;
+    const float* done_xcopy = nullptr;
 };
 // xcopy (may be null): the rows after the add go there too
 static int dec_add_norm_q8(const fnx_decoder* D, const DecPending& pend, const float* w, int T, const fnx_dec_ws* ws, void* st, float* xcopy = nullptr,
                            const int* gate = nullptr) {
+    if (pend.done_w && pend.done_w == w && (!xcopy || pend.done_xcopy == xcopy)) return 0;   // the window before made this pass
     CombineArgs c{};
     c.live = pend.live;
     c.xcopy = xcopy;
@@ -1618,15 +1655,18 @@ static int dec_add_norm_q8(const fnx_decoder* D, const DecPending& pend, const f
         c.vocab = D->vocab;
     }
     if (D->n < 32 || D->n % 32 || D->n > 256 * NQ_MAXJ) return fail("decoder: rows of 32 .. 4096 values in whole 32-value blocks");
-    k_add_norm_q8<false><<<T, 256, 0, (hipStream_t) st>>>(ws->x, pend.rows, c, w, nullptr, (uint8_t*) ws->xq, D->n, D->eps);
+    // (after a window that made another pass than this one, x already holds the add)
+    k_add_norm_q8<false><<<T, 256, 0, (hipStream_t) st>>>(ws->x, pend.done_w ? nullptr : pend.rows, c, w, nullptr, (uint8_t*) ws->xq, D->n, D->eps);
     return launch_status("decoder add_norm_q8");
 }
 // x (ws->x) through one layer, in place; the layer's own MoE output is left pending for whatever comes next
 // live (may be null): a device word, how many of the T rows count; the others still append their K and V (their cache
 // cells are overwritten by the next window) but ask no queries and are not routed, so they pull no expert's weights
 // gate (may be null): a device word; at zero the layer's dense products and its attention's scan leave at once
+// next_w (may be null): the weights of the norm that follows this layer (the next layer's, or the head's), next_xcopy where
+// the rows after the add are wanted as well: the window's launch then makes that pass itself
 static int dec_layer(const fnx_decoder* D, const fnx_dec_layer* L, int T, const int* pos0, const fnx_dec_ws* ws, DecPending& pend, void* st,
-                     const int* live = nullptr, const int* gate = nullptr) {
+                     const int* live = nullptr, const int* gate = nullptr, const float* next_w = nullptr, float* next_xcopy = nullptr) {
     const int n = D->n, nq = D->nq, nkv = D->nkv;
     if (dec_add_norm_q8(D, pend, L->attn_norm, T, ws, st, nullptr, gate)) return 1;
     {   // q, k and v in one launch (engine.cu:1547-1552)
@@ -1640,13 +1680,26 @@ static int dec_layer(const fnx_decoder* D, const fnx_dec_layer* L, int T, const 
     if (attn_launch(ws->qg, L->kc, L->vc, nullptr, (uint8_t*) ws->xq, nq, nkv, pos0, T, D->max_ctx, ws->attn_scratch, st, gate, live, (unsigned*) ws->err))
         return 1;
     if (q8s_one(&L->wo, ws->xq, ws->o, n, T, st, gate)) return 1;
+    if (live && !layer_fused_ok(&L->moe, T)) return fail("decoder: a device-side row count needs the one-launch window (unit64 experts, hidden 2048)");
+    if (next_w && layer_fused_ok(&L->moe, T) && !shared_is_q8(&L->moe)) {
+        // The one-launch window takes the passes either side of it: every block makes its row's x + o and the norm for itself,
+        // the row's last block adds the window's rows and makes the next norm's q8_1 rows (k_moe_window.h). Its rows go to
+        // ws->xn, which nothing else needs then (ws->o holds the attention half's rows until the last block has read them)
+        const WinNext next{ws->x, next_w, ws->xq, next_xcopy, D->eps, ws->o, L->ffn_norm};
+        bool done = false;
+        if (moe_layer_checked(&L->moe, ws->x, T, ws->xn, &ws->moe, st, live, &next, &done)) return 1;
+        if (!done) return fail("decoder: the window did not take the passes around it");
+        pend = DecPending{nullptr, nullptr, live};
+        pend.done_w = next_w;
+        pend.done_xcopy = next_xcopy;
+        return 0;
+    }
     {   // x += o; xn = norm(x) (fnx_add_norm_q8)
         CombineArgs c{};
         c.gate = gate;
         k_add_norm_q8<false><<<T, 256, 0, (hipStream_t) st>>>(ws->x, ws->o, c, L->ffn_norm, ws->xn, nullptr, n, D->eps);
         if (launch_status("decoder add_norm")) return 1;
     }
-    if (live && !layer_fused_ok(&L->moe, T)) return fail("decoder: a device-side row count needs the one-launch window (unit64 experts, hidden 2048)");
     // the MoE half's rows (those that count) are added by the next pass over x
     pend = DecPending{ws->o, nullptr, live};
     return moe_layer_checked(&L->moe, ws->xn, T, ws->o, &ws->moe, st, live);
@@ -1672,8 +1725,11 @@ static int decoder_verify(const fnx_decoder* D, const int* tokens, int T, const 
     if (!D || !tokens || !pos0 || !ws || !D->layers || !D->out_norm || !D->emb) return fail("decoder_verify: null argument");
     if (dec_shape_check(D, T, "decoder_verify") || dec_ws_check(ws, "decoder_verify")) return 1;
     DecPending pend{nullptr, tokens, nullptr};   // the window's input rows are read by the first pass over them
-    for (int l = 0; l < D->nlayers; ++l)
-        if (dec_layer(D, &D->layers[l], T, pos0, ws, pend, st, live)) return 1;
+    for (int l = 0; l < D->nlayers; ++l) {
+        const bool last = l + 1 == D->nlayers;
+        if (dec_layer(D, &D->layers[l], T, pos0, ws, pend, st, live, nullptr, last ? D->out_norm : D->layers[l + 1].attn_norm, last ? ws->hidden : nullptr))
+            return 1;
+    }
     return dec_head(D, D->out_norm, &D->head, T, ws, pend, st);
 }
 int fnx_decoder_verify(const fnx_decoder* D, const int* tokens, int T, const int* pos0, const fnx_dec_ws* ws, void* st) {
@@ -1716,7 +1772,7 @@ static int mtp_draft(const fnx_decoder* D, const fnx_mtp* M, const float* src, c
     }
     if (q8s_one(&M->fc_emb, ws->xq, ws->o, n, T, st, gate)) return 1;
     DecPending pend{ws->o, nullptr, nullptr};
-    if (dec_layer(D, &M->layer, T, pos0, ws, pend, st, live, gate)) return 1;
+    if (dec_layer(D, &M->layer, T, pos0, ws, pend, st, live, gate, M->out_norm, ws->hidden)) return 1;
     return dec_head(D, M->out_norm, &M->head, T, ws, pend, st, gate, nv, M->dv0, M->pen, M->pen_par);
 }
 int fnx_mtp_draft(const fnx_decoder* D, const fnx_mtp* M, const float* src, const int* tokens, int T, const int* pos0, const fnx_dec_ws* ws,

@@ -66,6 +66,19 @@ struct WindowArgs {
     fnx_job* jobs_dn;
     int* njobs;
     long long wait_ticks;     // budget of a wait for another block, in ticks of the 100 MHz wall clock
+    // What follows the window in a decoder, done here by the row's last block instead of by a launch of its own
+    // (fnx_add_norm_q8's pass: the residual add, the next RMS norm, its q8_1 rows). next_x null: not wanted.
+    float* next_x = nullptr;            // [T][rows]: x[t] += out[t] for the rows that count
+    const float* next_w = nullptr;      // [rows]: the next norm's weights
+    uint8_t* next_xq = nullptr;         // [T][rows / 32] q8_1 blocks of rms_norm(x[t]) * next_w
+    float* next_xcopy = nullptr;        // may be null: the rows after the add go there as well
+    float next_eps = 0.f;
+    // What comes before the window in a decoder, done by every block for its own row instead of by a launch (fnx_add_norm_q8's
+    // pass without the q8_1 rows): with pre_w set, x is not the normed row but the row before the attention's rows are
+    // added: the window's input is rms_norm(x[t] + pre_o[t]) * pre_w (eps = next_eps), and what the row's last block adds
+    // the window's rows to is x[t] + pre_o[t]. Only together with next_x = x.
+    const float* pre_o = nullptr;       // [T][rows]
+    const float* pre_w = nullptr;       // [rows]
 };
 
 template <int SBR>
@@ -126,7 +139,66 @@ __device__ __forceinline__ void win_meet() {
 // all of this wave's memory writes have been taken at the device's level before anything after this line
 __device__ __forceinline__ void win_stores_done() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
-template <int SBR>
+// Row t of the pass that follows a window in a decoder - k_add_norm_q8<false>'s values in its orders: v = x (+ out, read at
+// the device's level: other blocks wrote it), the sum of squares as 256 threads' fmaf chains over columns tid, tid + 256, ...,
+// a 64-lane sum a wave, (s0 + s1 + s2 + s3), the row times rsqrtf and the weights, q8_1 blocks a half-wave each. Called by
+// all threads of the block (the first 256 work); sh: four floats of LDS.
+__device__ __forceinline__ void win_next_row(const WindowArgs& a, int t, bool add, float* sh) {
+    constexpr int MAXJ = FL_N / 256;
+    const int tid = threadIdx.x, n = a.rows;
+    float v[MAXJ], wv[MAXJ];
+    float s = 0.f;
+    if (tid < 256) {
+#pragma unroll
+        for (int j = 0; j < MAXJ; ++j) {
+            const int i = tid + 256 * j;
+            v[j] = a.next_x[(size_t) t * n + i];
+            wv[j] = a.next_w[i];
+        }
+        if (a.pre_o) {   // (the pass before the window, which its blocks made for themselves only: the same add)
+            float pv[MAXJ];
+#pragma unroll
+            for (int j = 0; j < MAXJ; ++j) pv[j] = a.pre_o[(size_t) t * n + tid + 256 * j];
+#pragma unroll
+            for (int j = 0; j < MAXJ; ++j) v[j] += pv[j];
+        }
+        if (add) {
+            float av[MAXJ];
+#pragma unroll
+            for (int j = 0; j < MAXJ; ++j)
+                av[j] = __uint_as_float(__hip_atomic_load(reinterpret_cast<const unsigned*>(a.out) + (size_t) t * n + tid + 256 * j, __ATOMIC_RELAXED,
+                                                          __HIP_MEMORY_SCOPE_AGENT));
+#pragma unroll
+            for (int j = 0; j < MAXJ; ++j) v[j] += av[j];
+        }
+        if (add || a.pre_o) {
+#pragma unroll
+            for (int j = 0; j < MAXJ; ++j) a.next_x[(size_t) t * n + tid + 256 * j] = v[j];
+        }
+        if (a.next_xcopy) {
+#pragma unroll
+            for (int j = 0; j < MAXJ; ++j) a.next_xcopy[(size_t) t * n + tid + 256 * j] = v[j];
+        }
+#pragma unroll
+        for (int j = 0; j < MAXJ; ++j) s = fmaf(v[j], v[j], s);
+        s = group_sum<64>(s);
+        if ((tid & 63) == 0) sh[tid >> 6] = s;
+    }
+    __syncthreads();
+    if (tid < 256) {
+        const float r = rsqrtf((sh[0] + sh[1] + sh[2] + sh[3]) / (float) n + a.next_eps);
+#pragma unroll
+        for (int j = 0; j < MAXJ; ++j) {
+            const int i = tid + 256 * j;
+            q8_1_store(v[j] * r * wv[j], a.next_xq + ((size_t) t * (n / 32) + i / 32) * FNX_Q8_1_BLOCK, tid & 31);
+        }
+    }
+    __syncthreads();   // sh may be written again
+}
+
+// DEC: the launch of a decoder's layer, which may also take the passes either side of the window (next_x, pre_w); without it
+// those arguments are not looked at and their code is not there
+template <int SBR, bool DEC = false>
 __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
     __shared__ WinLds<SBR> S;
     constexpr int RW = 64 / SBR, RMAX = SBR / 8, NB = RMAX == 4 ? 2 : 3, DEPTH = RMAX == 4 ? 1 : 2;   // rows a unit; units a wave and trip at most; trips' buffers
@@ -157,6 +229,27 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
     float xv[2];
 #pragma unroll
     for (int r = 0; r < 2; ++r) xv[r] = xrow[(4 * wave + 2 * r + (lane >> 5)) * 32 + (lane & 31)];
+    // With pre_w the row is still to be made: (x + o) * rsqrt(mean square + eps) * w, k_add_norm_q8's values in its orders - the
+    // sum of squares as 256 threads' fmaf chains over columns tid, tid + 256, ..., a 64-lane sum a wave, (s0 + s1 + s2 + s3).
+    // Every block of the row makes it for itself; its loads go out here, before the router's rows, which stay in flight
+    // while the sum is made
+    const bool pre = DEC && a.pre_w != nullptr;
+    const float* orow = pre ? a.pre_o + (size_t) t * FL_N : xrow;
+    const float* wrow = pre ? a.pre_w : xrow;
+    float4 om = make_float4(0.f, 0.f, 0.f, 0.f), wm = om;
+    float ov[2] = {0.f, 0.f}, wv2[2] = {0.f, 0.f}, sq[FL_N / 256], so[FL_N / 256];
+    if (pre) {
+        if (tid < FL_N / 4) om = reinterpret_cast<const float4*>(orow)[tid], wm = reinterpret_cast<const float4*>(wrow)[tid];
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            const int i = (4 * wave + 2 * r + (lane >> 5)) * 32 + (lane & 31);
+            ov[r] = orow[i], wv2[r] = wrow[i];
+        }
+        if (tid < 256) {
+#pragma unroll
+            for (int j = 0; j < FL_N / 256; ++j) sq[j] = xrow[tid + 256 * j], so[j] = orow[tid + 256 * j];
+        }
+    }
     // this wave's router rows: rows r0 + wave, r0 + wave + 16, ... of the block's slice, two at a time
     const int r0 = g * pl.rpb, r1 = min(nexp, r0 + pl.rpb);
     auto load_router_row = [&](int row, float4(&w)[8]) {
@@ -190,6 +283,24 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
     float4 wa[8], wb[8];
     load_router_row(r0 + wave, wa);
     load_router_row(r0 + wave + WN_WAVES, wb);
+    if (pre) {
+        if (tid < 256) {
+            float s = 0.f;
+#pragma unroll
+            for (int j = 0; j < FL_N / 256; ++j) {
+                const float v = sq[j] + so[j];
+                s = fmaf(v, v, s);
+            }
+            s = group_sum<64>(s);
+            if (lane == 0) S.hgu[0][wave] = s;
+        }
+        win_meet();
+        const float rn = rsqrtf((S.hgu[0][0] + S.hgu[0][1] + S.hgu[0][2] + S.hgu[0][3]) / (float) FL_N + a.next_eps);
+        xmine = make_float4((xmine.x + om.x) * rn * wm.x, (xmine.y + om.y) * rn * wm.y, (xmine.z + om.z) * rn * wm.z, (xmine.w + om.w) * rn * wm.w);
+#pragma unroll
+        for (int r = 0; r < 2; ++r) xv[r] = (xv[r] + ov[r]) * rn * wv2[r];
+        win_meet();   // S.hgu is free again
+    }
 
     // ---------------------------------------------------------------- LDS: flags, the codebook, the row's q8_1 blocks
     if (tid < WN_SLOTS * WN_WAVES) (&S.flag[0][0])[tid] = 0;
@@ -658,10 +769,15 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
             for (int r = 0; r < RMAX; ++r)
                 if (r < R) {
                     const float shared = ext ? gate * a.sh_part[(size_t) t * a.rows + (size_t) (u0 + r) * RW + gl] : zs[r];
-                    orow[r * RW] = acc[r] + shared;
+                    // (at the device's level: the row's last block may read the row back below, from another XCD)
+                    __hip_atomic_store(reinterpret_cast<unsigned*>(orow + r * RW), __float_as_uint(acc[r] + shared), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
         }
     }
+    win_stores_done();
+    // rows past the ones that count get no window's rows added, but whatever follows still reads their normed rows: block g of
+    // row 0 makes row Tl + g's (nothing else in this launch touches those rows; G >= 16 >= T - Tl)
+    if (DEC && a.next_x && t == 0 && Tl + g < T) win_next_row(a, Tl + g, false, reinterpret_cast<float*>(&S.hgu[0][0]));
 
     WIN_TS(10);
     // ---------------------------------------------------------------- the end of the block, of the row, of the window
@@ -682,6 +798,8 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
     __syncthreads();
     WIN_TS(11);
     if (!S.last) return;
+    // the row is complete (every block of it waited for its stores before it counted itself done)
+    if (DEC && a.next_x) win_next_row(a, t, true, reinterpret_cast<float*>(&S.hgu[0][0]));
     const int fin = S.fin;
     if (fin == 0) {   // every row has been ranked long ago; the count says so
         if (wave == 0) {
