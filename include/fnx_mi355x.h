@@ -176,6 +176,7 @@ typedef struct fnx_q8s {
     const int8_t* q;
     const uint16_t* d;
     int n_out, n_in;
+    int tiled;   /* 0: q is [n_out][n_in] as the reference's split layout (model.hpp:78-82); 1: q was re-laid by fnx_q8s_tile */
 } fnx_q8s;
 typedef struct fnx_moe_layer {
     int n, ff, nexp, topk;   /* hidden, expert width, experts, picks per token */
@@ -321,6 +322,13 @@ int fnx_combine_add_norm_q8(const float* part, const float* topw, const float* s
 int fnx_add_rows(const float* a, const float* b, float* y, size_t n, void* st);
 /* rows tokens[t] of an f16 table [vocab][n] as f32 (the window's input rows) */
 int fnx_embed_rows(const uint16_t* emb, const int* tokens, int T, int vocab, int n, float* y, void* st);
+/* A load-time layout of a dense matrix's int8 values, the counterpart of the reference's own load-time split (model.hpp:
+ * 78-82): tiles of 16 rows, a tile its 64-column steps one after another (1 KiB each, a wave's lanes' 16-byte shares side
+ * by side), so that the mat-vec below streams whole cache lines (the output head: 4.7 against 4.1 TB/s). src [rows][cols]
+ * int8 -> dst, another buffer of fnx_q8s_tile_bytes(rows, cols) bytes (rows padded to 16); the scales stay as they are; a
+ * fnx_q8s over dst has tiled = 1. Both layouts give the same bits. cols a multiple of 256. */
+int fnx_q8s_tile(const int8_t* src, int8_t* dst, int rows, int cols, void* st);
+size_t fnx_q8s_tile_bytes(int rows, int cols);
 /* dense.cuh:79-214 (q8s_gemv): out[t * out_stride + r] = W[r] . y[t] for T <= 16 q8_1 rows; n_in a multiple of 256. The
  * result is (s0 + s1) + (s2 + s3), s_q the q-th quarter of the columns, its 32-column blocks folded in ascending order with
  * acc = fmaf(d_w * d_x, (float) dot, acc) */

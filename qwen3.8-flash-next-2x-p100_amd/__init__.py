@@ -36,7 +36,7 @@ class DW(C.Structure):
 
 
 class Q8S(C.Structure):
-    _fields_ = [("q", C.c_void_p), ("d", C.c_void_p), ("n_out", C.c_int), ("n_in", C.c_int)]
+    _fields_ = [("q", C.c_void_p), ("d", C.c_void_p), ("n_out", C.c_int), ("n_in", C.c_int), ("tiled", C.c_int)]
 
 
 class MoeLayer(C.Structure):
@@ -148,6 +148,8 @@ EXPORTS = {
                                           C.c_int, C.c_int, C.c_float, C.c_void_p]),
     "fnx_add_rows": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "fnx_embed_rows": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]),
+    "fnx_q8s_tile": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
+    "fnx_q8s_tile_bytes": (C.c_size_t, [C.c_int, C.c_int]),
     "fnx_q8s_gemv": (C.c_int, [C.POINTER(Q8S), C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
     "fnx_q8s_gemv_segs": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_void_p]),
     "fnx_attn_prep_append": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int,

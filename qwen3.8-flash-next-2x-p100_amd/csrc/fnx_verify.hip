@@ -1542,6 +1542,7 @@ static int q8s_launch(const fnx_q8s* const* W, float* const* out, const int* out
         if (W[s]->n_in != W[0]->n_in) return fail(std::string(who) + ": the matrices share the activations: the same columns");
         if (((uintptr_t) W[s]->q & 15) || ((uintptr_t) W[s]->d & 3)) return fail(std::string(who) + ": 16-byte aligned rows");
         if (s + 1 < n && W[s]->n_out % 16) return fail(std::string(who) + ": all but the last matrix in whole 16-row tiles");
+        if ((W[s]->tiled != 0) != (W[0]->tiled != 0)) return fail(std::string(who) + ": the matrices of one launch share a layout");
         if (out_stride[s] < W[s]->n_out) return fail(std::string(who) + ": out_stride smaller than the rows");
         a.seg[s] = Q8sSeg{W[s]->q, W[s]->d, out[s], W[s]->n_out, out_stride[s]};
         tiles += (W[s]->n_out + 15) / 16;
@@ -1556,15 +1557,26 @@ static int q8s_launch(const fnx_q8s* const* W, float* const* out, const int* out
     static bool attr_set[64] = {};
     int dev = 0;
     if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64 && !attr_set[dev]) {
-        if (hipFuncSetAttribute((const void*) k_q8s_gemv<1>, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024) != hipSuccess)
+        if (hipFuncSetAttribute((const void*) k_q8s_gemv<1>, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024) != hipSuccess ||
+            hipFuncSetAttribute((const void*) k_q8s_gemv<1, true>, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024) != hipSuccess)
             return fail(std::string(who) + ": cannot raise the dynamic LDS limit");
         attr_set[dev] = true;
     }
     static const int per_cu = env_int("FNX_Q8S_BLOCKS_PER_CU", 4, 1, 16);   // what the LDS of a 2048-column matrix lets a CU hold
     const int grid = (int) std::max(1l, std::min<long>((long) per_cu * cu_count(), tiles));
     a.gate = gate;
-    k_q8s_gemv<1><<<grid, Q8S_WAVES * 64, lds, (hipStream_t) st>>>(a);
+    if (W[0]->tiled) k_q8s_gemv<1, true><<<grid, Q8S_WAVES * 64, lds, (hipStream_t) st>>>(a);
+    else k_q8s_gemv<1><<<grid, Q8S_WAVES * 64, lds, (hipStream_t) st>>>(a);
     return launch_status(who);
+}
+size_t fnx_q8s_tile_bytes(int rows, int cols) { return rows < 1 || cols < 64 || cols % 64 ? 0 : (size_t) ((rows + 15) / 16) * 16 * (size_t) cols; }
+int fnx_q8s_tile(const int8_t* src, int8_t* dst, int rows, int cols, void* st) {
+    if (!src || !dst || src == dst) return fail("q8s_tile: two buffers");
+    if (rows < 1 || cols < 256 || cols % 256) return fail("q8s_tile: columns in 256s");
+    if (((uintptr_t) src & 15) || ((uintptr_t) dst & 15)) return fail("q8s_tile: 16-byte aligned buffers");
+    const size_t pieces = fnx_q8s_tile_bytes(rows, cols) / 16;
+    k_q8s_tile<<<(unsigned) std::min<size_t>((pieces + 255) / 256, 65536), 256, 0, (hipStream_t) st>>>(src, dst, rows, cols);
+    return launch_status("q8s_tile");
 }
 int fnx_q8s_gemv(const fnx_q8s* W, const void* yq, float* out, int out_stride, int T, void* st) {
     return q8s_launch(&W, &out, &out_stride, 1, yq, T, st, "q8s_gemv");
@@ -2135,6 +2147,7 @@ int fnx_gguf_load_moe_layer(const fnx_gguf* g, int layer, int ff0, int ff1, int 
             q.d = reinterpret_cast<const uint16_t*>(reinterpret_cast<const uint8_t*>(d) + nval);
             q.n_out = w.n_out;
             q.n_in = w.n_in;
+            q.tiled = 0;
             w.p = nullptr;   // the raw form is not kept
         };
         gguf::router_rows(m.gi, m.gs, reinterpret_cast<float*>(host.data()));

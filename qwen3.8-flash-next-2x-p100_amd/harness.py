@@ -383,11 +383,20 @@ class Dev:
         self.sync()
         return d[4].cpu().numpy(), xn.cpu().numpy(), xq.cpu().numpy()
 
-    def q8s_gemv(self, q, d, yq, T):
+    def q8s_tiled(self, dq, rows, cols):
+        """the int8 values of a dense matrix (a device tensor [rows][cols]) re-laid tile-major (fnx_q8s_tile): a new tensor"""
+        dst = self.zeros(self.lib.fnx_q8s_tile_bytes(rows, cols), self.torch.int8)
+        self.ok(self.lib.fnx_q8s_tile(dq.data_ptr(), dst.data_ptr(), rows, cols, self.st()))
+        self.sync()
+        return dst
+
+    def q8s_gemv(self, q, d, yq, T, tiled=False):
         rows, cols = q.shape
         dq, dd, dy = self.up(q), self.up(d), self.up(yq)
         out = self.zeros((T, rows), self.torch.float32)
-        W = self.pkg.Q8S(dq.data_ptr(), dd.data_ptr(), rows, cols)
+        if tiled:
+            dq = self.q8s_tiled(dq, rows, cols)
+        W = self.pkg.Q8S(dq.data_ptr(), dd.data_ptr(), rows, cols, 1 if tiled else 0)
         self.ok(self.lib.fnx_q8s_gemv(C.byref(W), dy.data_ptr(), out.data_ptr(), rows, T, self.st()))
         self.sync()
         return out.cpu().numpy()
@@ -435,7 +444,8 @@ def pack_moe_weights(dev, ws, n, ff, packed):
 class DecoderDev:
     """a SyntheticDecoder on the device: weights, caches, workspace; verify / draft through the C ABI"""
 
-    def __init__(self, dev, model, packed=True):
+    def __init__(self, dev, model, packed=True, tiled=True):
+        """tiled: the dense matrices' int8 values in the tile-major layout (fnx_q8s_tile), as a caller would re-lay them at load"""
         t = dev.torch
         pkg = dev.pkg
         c = model.cfg
@@ -449,7 +459,11 @@ class DecoderDev:
             return d
 
         def q8s(tq, rows, cols):
-            return pkg.Q8S(up(tq[0]).data_ptr(), up(tq[1]).data_ptr(), rows, cols)
+            if tiled:
+                dq = dev.q8s_tiled(dev.up(tq[0]), rows, cols)
+                self.keep.append(dq)
+                return pkg.Q8S(dq.data_ptr(), up(tq[1]).data_ptr(), rows, cols, 1)
+            return pkg.Q8S(up(tq[0]).data_ptr(), up(tq[1]).data_ptr(), rows, cols, 0)
 
         def lay(L):
             ws, dws = pack_moe_weights(dev, [up(L[k]) for k in ("gu", "down", "sh_gu", "sh_down")], n, ff, packed)
@@ -582,7 +596,8 @@ class DecoderDev:
             M = type(self.M).from_buffer_copy(self.M)
             if dv is not None:
                 M.dv0, M.dv1 = dv
-                M.head = dev.pkg.Q8S(self.M.head.q + dv[0] * n, self.M.head.d + dv[0] * (n // 32) * 2, dv[1] - dv[0], n)
+                assert dv[0] % 16 == 0, "a tile-major head is cut at whole tiles of 16 rows"
+                M.head = dev.pkg.Q8S(self.M.head.q + dv[0] * n, self.M.head.d + dv[0] * (n // 32) * 2, dv[1] - dv[0], n, self.M.head.tiled)
             if pen is not None:
                 keep = [dev.up(np.concatenate([[len(pen[0])], pen[0], pen[1]]).astype(np.int32)), dev.up(np.asarray(par, dtype=np.float32))]
                 M.pen, M.pen_par = keep[0].data_ptr(), keep[1].data_ptr()

@@ -124,6 +124,8 @@ inline void combine_add_norm_q8(const float* part, const float* topw, const floa
                                 void* xq, int T, float eps, void* st) {
     ck(fnx_combine_add_norm_q8(part, topw, sh, sh_logit, 1, shape().TOPK, x, w, xn, xq, T, shape().N, eps, st));
 }
+// the load-time tile-major layout of a dense matrix's int8 values (no counterpart in kernels.hpp: model.hpp:78-82 is the reference's load-time split)
+inline void q8s_tile(const int8_t* src, int8_t* dst, int rows, int cols, void* st) { ck(fnx_q8s_tile(src, dst, rows, cols, st)); }
 inline void q8s_gemv(const Q8S& w, const void* y, float* out, int out_stride, int T, void* st) { ck(fnx_q8s_gemv(&w, y, out, out_stride, T, st)); }
 inline void q8s_gemv_segs(const Q8S* w, float* const* out, const int* out_stride, int n, const void* y, int T, void* st) {
     const Q8S* p[3] = {&w[0], n > 1 ? &w[1] : nullptr, n > 2 ? &w[2] : nullptr};

@@ -53,6 +53,8 @@ def test_bad_arguments_are_refused_with_a_message():
     assert lib.fnx_mmvq(C.byref(bad), 0, buf, None, 1, buf, buf, 16, None) != 0
     assert lib.fnx_route(buf, 8, 1, 2000, 10, buf, buf, buf, buf, buf, None) != 0
     assert lib.fnx_argmax(buf, 0, 1, 0, buf, buf, buf, buf, None) != 0
+    assert lib.fnx_q8s_tile(buf, buf, 16, 256, None) != 0 and b"two buffers" in lib.fnx_last_error()
+    assert lib.fnx_q8s_tile_bytes(17, 256) == 32 * 256 and lib.fnx_q8s_tile_bytes(16, 100) == 0
     # a cache whose capacity ends inside a block of eight positions would be read past its end by the attention's V fetches
     assert lib.fnx_attn(buf, buf, buf, buf, 16, 2, buf, 1, 100, buf, None) != 0 and b"multiple of 8" in lib.fnx_last_error()
     assert lib.fnx_attn(buf, buf, buf, buf, 16, 2, buf, 1, 4, buf, None) != 0 and b"multiple of 8" in lib.fnx_last_error()

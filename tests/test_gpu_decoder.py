@@ -90,6 +90,9 @@ def test_q8s_gemv_bit_exact(dev, oracle, rows, cols, T):
     got = dev.q8s_gemv(q, d, yq, T)
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
     assert rel_l2(got, x.astype(np.float64) @ w.astype(np.float64).T) < 2e-2   # and it is the product it claims to be
+    # the same values found elsewhere: the tile-major layout (fnx_q8s_tile), rows that do not fill the last tile included
+    tiled = dev.q8s_gemv(q, d, yq, T, tiled=True)
+    assert np.array_equal(tiled.view(np.uint32), want.view(np.uint32))
 
 
 @pytest.mark.parametrize("rope", [ROPE, YARN])
@@ -163,8 +166,10 @@ def model(oracle):
     return td.TinyDecoder(oracle, seed=11)
 
 
-def test_decoder_verify_and_draft(dev, oracle, model):
-    o, d = td.OracleSession(model), fnx_gpu.DecoderDev(dev, model)
+@pytest.mark.parametrize("tiled", [True, False])
+def test_decoder_verify_and_draft(dev, oracle, model, tiled):
+    """tiled: the dense matrices tile-major (fnx_q8s_tile) or as the reference's split layout"""
+    o, d = td.OracleSession(model), fnx_gpu.DecoderDev(dev, model, tiled=tiled)
     pos = 0
     for toks in ([3, 1, 4, 1, 5, 9, 2, 6, 5, 3, 5, 8, 9, 7, 9, 3], [2, 7, 18], [281]):
         print(f"case decoder_verify T={len(toks)} pos={pos}", flush=True)
