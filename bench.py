@@ -55,7 +55,7 @@ WINDOW_TRAFFIC = {"bytes": 208.94e6, "algorithmic_bytes": 192.96e6, "distinct_ex
                    "source": "profiles/moe_window_hbm_traffic.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this file's default workload; scaled to "
                              "this run's algorithmic bytes; not measured in this run)"}
 # the same for the prompt path's gate|up launch (profiles/prefill_chunk_counters.md: FETCH_SIZE x 2 + WRITE_SIZE)
-PF_WINDOW_TRAFFIC = {"bytes": 162.6e6, "algorithmic_bytes": 98.6e6,
+PF_WINDOW_TRAFFIC = {"bytes": 132.0e6, "algorithmic_bytes": 98.6e6,
                       "source": "profiles/prefill_chunk_counters.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this file's prefill workload, k_moe_mma_wave16_gu; "
                                 "scaled to this run's algorithmic bytes; not measured in this run)"}
 IQ3S_BLOCK = 110

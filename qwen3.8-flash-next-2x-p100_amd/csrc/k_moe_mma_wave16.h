@@ -80,6 +80,9 @@ __device__ __forceinline__ void w16_super_step(const uint2* tab, const uint8_t* 
 }
 
 __global__ void __launch_bounds__(W16_THREADS) k_moe_mma_wave16(const MmaArgs a) {
+    // the block's place in the plan: blocks with neighbouring places run on one XCD (workgroups go to the eight XCDs in turn), so
+    // the units of one expert, which the plan deals to neighbouring places, find the expert's weights in that XCD's L2
+    const unsigned vb = gridDim.x % 8 == 0 ? (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8 : blockIdx.x;
     __shared__ Wave16Lds L;
     const int tid = threadIdx.x, lane = tid & 63, wave = uniform(tid >> 6), r = lane & 15, grp = lane >> 4;
     // every job's token count and matrix, a thread a job, both lists at once (entries past a list's count are read too - the
@@ -146,8 +149,8 @@ __global__ void __launch_bounds__(W16_THREADS) k_moe_mma_wave16(const MmaArgs a)
         }
         const unsigned long long total = __shfl(incl, 63);
         unsigned long long c0, c1;   // (64-bit quotients take a few hundred instructions)
-        if (total <= 0xFFFFFFFFull / gridDim.x) c0 = (uint32_t) total * blockIdx.x / gridDim.x, c1 = (uint32_t) total * (blockIdx.x + 1) / gridDim.x;
-        else c0 = total * blockIdx.x / gridDim.x, c1 = total * (blockIdx.x + 1) / gridDim.x;
+        if (total <= 0xFFFFFFFFull / gridDim.x) c0 = (uint32_t) total * vb / gridDim.x, c1 = (uint32_t) total * (vb + 1) / gridDim.x;
+        else c0 = total * vb / gridDim.x, c1 = total * (vb + 1) / gridDim.x;
         if (lane == 0) {   // ends that lie past every job's items
             L.first_job = L.last_job = njall;
             L.first_tile = L.last_tile = 0;
@@ -252,6 +255,9 @@ struct Wave16GuLds {
     int p_total[MB_TP + 1], p_sumk, p_s0, p_k;   // the jobs by token tiles; the plan where one wave made it: this block's share of the light units
 };
 __global__ void __launch_bounds__(W16_THREADS) k_moe_mma_wave16_gu(const MmaArgs a) {
+    // the block's place in the plan: blocks with neighbouring places run on one XCD (workgroups go to the eight XCDs in turn), so
+    // the units of one expert, which the plan deals to neighbouring places, find the expert's weights in that XCD's L2
+    const unsigned vb = gridDim.x % 8 == 0 ? (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8 : blockIdx.x;
     __shared__ Wave16GuLds L;
     const int tid = threadIdx.x, lane = tid & 63, wave = uniform(tid >> 6), r = lane & 15, grp = lane >> 4;
     int hn[2] = {0, 0}, hn2 = 0, hw[2] = {0, 0};
@@ -321,7 +327,7 @@ __global__ void __launch_bounds__(W16_THREADS) k_moe_mma_wave16_gu(const MmaArgs
         // together) go as units of eight pairs, a wave a single tile, and fill the blocks up to the mean load: block b
         // takes k_b = (mean - its heavy units' cost) / (a light unit's cost) of them, rounded, in the order of the blocks
         // from the last one down (the lightest first); what the rounding leaves over goes one a block in that order.
-        const int G = gridDim.x, ome = G - 1 - (int) blockIdx.x;
+        const int G = gridDim.x, ome = G - 1 - (int) vb;
         const bool split = nsuper <= 4;
         const int nbj = total[4] + total[3] + total[2] + (split ? 0 : total[1]), nb = nbj * upj, ns = split ? total[1] * upj_s : 0;
         // costs as measured for S = 4 (us: 20 + 5.5 a token tile the heavy unit, 13.5 the light one), in halves of a us
@@ -394,7 +400,7 @@ __global__ void __launch_bounds__(W16_THREADS) k_moe_mma_wave16_gu(const MmaArgs
     if (nb <= G) {
         // every heavy unit on a block of its own, block b's of the class its place in the order says: the blocks of a class
         // take the same number of light units, and the blocks after b (they come first) are counted class by class
-        const int cs = 27 * nsuper, b1 = (int) blockIdx.x + 1;
+        const int cs = 27 * nsuper, b1 = (int) vb + 1;
         const int hi4 = tot[4] * upj, hi3 = hi4 + tot[3] * upj, hi2 = hi3 + tot[2] * upj;   // where the classes end (class 1: nb)
         const int c4 = 84 * nsuper, c3 = 73 * nsuper, c2 = 62 * nsuper, c1 = 51 * nsuper;      // (40 + 11 token tiles) S
         const int mean = (hi4 * c4 + (hi3 - hi4) * c3 + (hi2 - hi3) * c2 + (nb - hi2) * c1 + ns * cs + G - 1) / G;
@@ -423,7 +429,7 @@ __global__ void __launch_bounds__(W16_THREADS) k_moe_mma_wave16_gu(const MmaArgs
     };
     // ---- the heavy units: sixteen pairs of tiles, a pair a wave
     for (int round = 0; round * G < nb; ++round) {
-        const int u = round * G + ((round & 1) ? G - 1 - (int) blockIdx.x : (int) blockIdx.x);
+        const int u = round * G + ((round & 1) ? G - 1 - (int) vb : (int) vb);
         if (u >= nb) continue;   // the same for the whole block
         const int jo = u / upj, q = u - jo * upj, j = sorted ? (int) uniform(L.jorder[jo]) : jo;
         const fnx_bigjob* jb = job_at(j);
@@ -471,7 +477,7 @@ __global__ void __launch_bounds__(W16_THREADS) k_moe_mma_wave16_gu(const MmaArgs
     if (!sorted) return;
     // ---- the light units: eight pairs of tiles, waves 0 .. 7 the gate tiles, 8 .. 15 the up tiles; the job's up to 16 tokens'
     // S tiles all in LDS ([S][token]), so the waves do not meet until the up tiles' sums go over to the gate tiles' waves
-    const int ome = G - 1 - (int) blockIdx.x;
+    const int ome = G - 1 - (int) vb;
     float4* ex = reinterpret_cast<float4*>(L.xs);
     for (int t = 0;; ++t) {
         const int idx = t < kme ? s0 + t : sumk + (t - kme) * G + ome;
