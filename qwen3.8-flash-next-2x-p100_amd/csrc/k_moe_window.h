@@ -28,6 +28,8 @@
 // rounding, the IQ3_S sub-block terms, the combine's fmaf chain.
 #pragma once
 
+#include <type_traits>
+
 #include "k_moe_layer.h"
 #include "moe_window_plan.h"
 
@@ -84,7 +86,8 @@ struct WindowArgs {
 template <int SBR>
 struct WinLds {
     uint32_t tab[SGRID_WORDS];
-    uint32_t wp[FL_MAXK + 1][2];       // gate|up matrices: the shared expert's, then the picks'
+    uint32_t wp[FL_MAXK + 1][2];       // the picks' gate|up matrices at 1 + k, when they come from a table of pointers
+    uint32_t dp[FL_MAXK + 1][2];       // down matrices, the same way
     float hgu[WN_SLOTS][64];           // a sweep's sums: the 32 gate rows', then the 32 up rows'
     int flag[WN_SLOTS][WN_WAVES];
     int made[WN_SLOTS];
@@ -92,6 +95,7 @@ struct WinLds {
     int sliced[16];
     int ready;                         // picks whose matrices are known
     int pe[FL_MAXK];                   // the picks
+    unsigned pk[FL_MAXK];              // their keys
     float pw[FL_MAXK];                 // their weights
     float gate;                        // sigmoid of the shared expert's gate logit
     int rarrive, harrive;              // waves of the block that have stored their logits / finished their sweeps
@@ -498,89 +502,93 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
         if (lane == 0) __hip_atomic_store(&S.sliced[sl], 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
     WIN_TS(4);
-    if (wave == 0) {   // the merge; the row's first block writes the picks and their weights out
-        const bool publish = g == 0;
+    if (wave == 0) {   // the merge
         if (!lds_wait([&] {
                 const int f = lane < ns ? __hip_atomic_load(&S.sliced[lane], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) : 1;
                 return __ballot(f == 0) == 0ull;
             }))
             return;
-        // All of the row's candidates in registers, entry p of list j in lane (16 j + p) mod 64 of register (16 j + p) / 64;
-        // lane j < ns keeps list j's head and its position; the list whose head is picked gets its next entry by a read of
-        // that lane.
+        // All of the row's candidates in registers, entry p of list j in lane (16 j + p) mod 64 of register (16 j + p) / 64: a
+        // pick is the greatest key of them all, and among equal keys the first in that order - the lists follow the experts'
+        // order and each list its own, so that is the lowest expert. (Entries past a list's topk, and lists past the last
+        // slice, count as nothing.) The merging wave goes first on its SIMD: the block's sweeps wait for its picks.
         static_assert(FL_MAXK == 16, "sixteen entries a list, four lists a register");
-        int ck[4], ce[4];
-        {
-            const uint2* flat = &S.cand[0][0];
+        WIN_TS(14);
+        __builtin_amdgcn_s_setprio(3);
+        // (once for rows of up to 512 experts - two registers of candidates - and once for more: the merging wave's instructions
+        // are the block's critical path here)
+        auto merge = [&](auto NRC) {
+            constexpr int NR = decltype(NRC)::value;
+            unsigned ck[NR];
+            int ce[NR];
+            {
+                const uint2* flat = &S.cand[0][0];
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const uint2 c = flat[q * 64 + lane];
-                ck[q] = (int) c.x;
-                ce[q] = (int) c.y;
-            }
-        }
-        unsigned hk = lane < ns ? S.cand[min(lane, ns - 1)][0].x : 0u;
-        int he = S.cand[min(lane, ns - 1)][0].y, hp = 0;
-        unsigned mk = 0u;
-        int ei = 0x7fffffff;
-        unsigned long long low_taken = 0ull;   // which of experts 0 .. 63 are picked: what a row with fewer than topk finite logits falls back on
-        for (int k = 0; k < topk; ++k) {
-            unsigned m = (unsigned) __builtin_amdgcn_readlane((int) row_umax(hk), 0);
-            const unsigned long long hold = m > RANK_KEY_NEG_INF ? __ballot(hk == m) & 0xFFFFull : 0ull;
-            const int l = hold ? (int) __builtin_ctzll(hold) : 64;   // the lowest lane that holds the maximum has the lowest expert
-            int idx;
-            unsigned nkey = 0u;
-            int ne = nexp, np = 0;
-            if (hold) {
-                idx = __builtin_amdgcn_readlane(he, l);
-                np = __builtin_amdgcn_readlane(hp, l) + 1;
-                if (np < topk) {   // list l's next entry
-                    const int f = 16 * l + np, fl = f & 63, fq = f >> 6;
-                    const int k0_ = __builtin_amdgcn_readlane(ck[0], fl), k1_ = __builtin_amdgcn_readlane(ck[1], fl);
-                    const int k2_ = __builtin_amdgcn_readlane(ck[2], fl), k3_ = __builtin_amdgcn_readlane(ck[3], fl);
-                    const int e0_ = __builtin_amdgcn_readlane(ce[0], fl), e1_ = __builtin_amdgcn_readlane(ce[1], fl);
-                    const int e2_ = __builtin_amdgcn_readlane(ce[2], fl), e3_ = __builtin_amdgcn_readlane(ce[3], fl);
-                    nkey = (unsigned) (fq == 0 ? k0_ : fq == 1 ? k1_ : fq == 2 ? k2_ : k3_);
-                    ne = fq == 0 ? e0_ : fq == 1 ? e1_ : fq == 2 ? e2_ : e3_;
+                for (int q = 0; q < NR; ++q) {
+                    const uint2 c = flat[q * 64 + lane];
+                    const bool there = 4 * q + (lane >> 4) < ns && (lane & 15) < topk;
+                    ck[q] = there ? c.x : 0u;
+                    ce[q] = (int) c.y;
                 }
-            } else {   // nothing finite is left: the lowest expert not picked yet, with weight exp(-inf) = 0
-                m = RANK_KEY_NEG_INF;
-                idx = (int) __builtin_ctzll(~low_taken);
             }
-            if (idx < 64) low_taken |= 1ull << idx;
-            if (lane == l) {
-                hk = nkey;
-                he = ne;
-                hp = np;
-            }
-            if (lane == k) {
-                mk = m;
-                ei = idx;
-            }
-            {   // the pick's matrix is handed out at once: the sweeps need not wait for the whole ranking
-                const uint8_t* e = a.gu_ep ? a.gu_ep[idx] : a.gu + (size_t) idx * a.gu_stride;
+            unsigned long long low_taken = 0ull;   // which of experts 0 .. 63 are picked: what a row with fewer than topk finite logits falls back on
+            for (int k = 0; k < topk; ++k) {
+                unsigned mx = ck[0];
+#pragma unroll
+                for (int q = 1; q < NR; ++q) mx = max(mx, ck[q]);
+                unsigned m = wave_umax(mx);
+                int idx;
+                if (m > RANK_KEY_NEG_INF) {
+                    unsigned long long b[NR];
+#pragma unroll
+                    for (int q = 0; q < NR; ++q) b[q] = __ballot(ck[q] == m);
+                    int q0 = NR - 1;
+                    unsigned long long bb = b[NR - 1];
+#pragma unroll
+                    for (int q = NR - 2; q >= 0; --q)
+                        if (b[q]) q0 = q, bb = b[q];
+                    const int l = (int) __builtin_ctzll(bb);
+                    idx = __builtin_amdgcn_readlane(ce[NR - 1], l);
+#pragma unroll
+                    for (int q = NR - 2; q >= 0; --q) {
+                        const int e = __builtin_amdgcn_readlane(ce[q], l);
+                        if (q0 == q) idx = e;
+                    }
+#pragma unroll
+                    for (int r = 0; r < NR; ++r) ck[r] = r == q0 && lane == l ? 0u : ck[r];
+                } else {   // nothing finite is left: the lowest expert not picked yet, with weight exp(-inf) = 0
+                    m = RANK_KEY_NEG_INF;
+                    idx = (int) __builtin_ctzll(~low_taken);
+                }
+                if (idx < 64) low_taken |= 1ull << idx;
+                // The pick is handed out at once: the sweeps need not wait for the whole ranking. Matrices that lie a stride apart
+                // are found by the waves that want them; a table of pointers is looked up here, for both matrices (a sweep or trip
+                // that looked its pointer up in memory would wait for the lookup, and with it for every load of weights in flight).
+                if (a.gu_ep) {
+                    const uint8_t* e = a.gu_ep[idx];
+                    if (lane == 0) {
+                        S.wp[1 + k][0] = (uint32_t) (uintptr_t) e;
+                        S.wp[1 + k][1] = (uint32_t) ((uint64_t) (uintptr_t) e >> 32);
+                    }
+                }
+                if (a.dn_ep) {
+                    const uint8_t* ed = a.dn_ep[idx];
+                    if (lane == 0) {
+                        S.dp[1 + k][0] = (uint32_t) (uintptr_t) ed;
+                        S.dp[1 + k][1] = (uint32_t) ((uint64_t) (uintptr_t) ed >> 32);
+                    }
+                }
                 if (lane == 0) {
-                    S.wp[1 + k][0] = (uint32_t) (uintptr_t) e;
-                    S.wp[1 + k][1] = (uint32_t) ((uint64_t) (uintptr_t) e >> 32);
                     S.pe[k] = idx;
+                    S.pk[k] = m;
                     __hip_atomic_store(&S.ready, k + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
                 }
             }
-        }
-        const float top0 = rank_key_inv((unsigned) __builtin_amdgcn_readlane((int) mk, 0));
-        const float ek = mk > RANK_KEY_NEG_INF ? fnx_expf(rank_key_inv(mk) - top0) : 0.f;   // a pick without a finite logit weighs nothing
-        float z = 0.f;
-        for (int k = 0; k < topk; ++k) z += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, ek), k));
-        const float wk = z > 0.f ? ek / z : 0.f;
-        if (lane < topk) S.pw[lane] = wk;
-        if (publish) {
-            if (lane < topk) {
-                __hip_atomic_store(&a.topi[t * topk + lane], ei, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                __hip_atomic_store(&a.topw[t * topk + lane], wk, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-            win_stores_done();
-            if (lane == 0) __hip_atomic_fetch_add(&a.sync[WS_ROUTED], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
+        };
+        if (ns <= 8) merge(std::integral_constant<int, 2>{});
+        else merge(std::integral_constant<int, 4>{});
+        __builtin_amdgcn_s_setprio(0);
+        WIN_TS(15);
         WIN_TS(5);
     }
     // an item's loads, once its matrix is known: matrix 0 is the shared expert's, matrix k pick k - 1's
@@ -589,8 +597,12 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
         const int mk_ = uniform(m.k);
         if (mk_ > 0) {
             if (!lds_wait([&] { return uniform(__hip_atomic_load(&S.ready, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP)) >= mk_; })) return false;
-            const uint2 p = *reinterpret_cast<const uint2*>(S.wp[mk_]);
-            e = (const uint8_t*) (uintptr_t) ((uint64_t) (uint32_t) uniform((int) p.x) | (uint64_t) (uint32_t) uniform((int) p.y) << 32);
+            if (a.gu_ep) {
+                const uint2 p = *reinterpret_cast<const uint2*>(S.wp[mk_]);
+                e = (const uint8_t*) (uintptr_t) ((uint64_t) (uint32_t) uniform((int) p.x) | (uint64_t) (uint32_t) uniform((int) p.y) << 32);
+            } else {
+                e = a.gu + (size_t) uniform(S.pe[mk_ - 1]) * a.gu_stride;
+            }
         }
         issue_from(e, m.j);
         return true;
@@ -639,19 +651,24 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
     // trip 0 is the shared expert's, trips 1 .. topk the picks in order
     auto down_matrix = [&](int trip) -> const uint8_t* {
         if (trip == 0) return a.dn_shared;
-        const int e = uniform(S.pe[trip - 1]);
-        return a.dn_ep ? a.dn_ep[e] : a.dn + (size_t) e * a.dn_stride;
+        if (!a.dn_ep) return a.dn + (size_t) uniform(S.pe[trip - 1]) * a.dn_stride;
+        const uint2 p = *reinterpret_cast<const uint2*>(S.dp[trip]);
+        return (const uint8_t*) (uintptr_t) ((uint64_t) (uint32_t) uniform((int) p.x) | (uint64_t) (uint32_t) uniform((int) p.y) << 32);
     };
-    PackedSub B[NB][RMAX];
-    auto issue_trip = [&](PackedSub(&buf)[RMAX], int trip) {
-        const __amdgpu_buffer_rsrc_t mtx = matrix_rsrc(uniform_ptr(down_matrix(trip)));
+    // The rest of the phase once for every number of units a wave can have (RC::value == R): with the count a constant, every
+    // load of a trip is issued on every path, the compiler knows how many loads lie behind the one it waits for, and a decode
+    // waits for its own trip's weights only - not, as with loads under "if (r < R)", for everything in flight.
+    auto down_phase = [&](auto RC) -> bool {
+    constexpr int RR = decltype(RC)::value;
+    PackedSub B[NB][RR];
+    auto issue_trip = [&](PackedSub(&buf)[RR], int trip) {
+        const __amdgpu_buffer_rsrc_t mtx = matrix_rsrc(down_matrix(trip));
 #pragma unroll
-        for (int r = 0; r < RMAX; ++r)
-            if (r < R) buf[r] = load_packed_buf(mtx, (u0 + r) * UNIT_BYTES, o);
+        for (int r = 0; r < RR; ++r) buf[r] = load_packed_buf(mtx, (u0 + r) * UNIT_BYTES, o);
     };
     // The picks are known (this block ranked its row), so the first trips' weights are asked for before the wait for h.
     // (The hand-over of the last pick's matrix has been seen by every wave that swept; a block without items waits here.)
-    if (!lds_wait([&] { return uniform(__hip_atomic_load(&S.ready, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP)) >= topk; })) return;
+    if (!lds_wait([&] { return uniform(__hip_atomic_load(&S.ready, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP)) >= topk; })) return false;
     if (nsweep > 0) {   // this wave's h blocks are out: arrive
         win_stores_done();
         int old = 0;
@@ -660,6 +677,25 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
             if (lane == 0) __hip_atomic_fetch_add(&srow[1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     WIN_TS(7);
+    if (wave == 2) {   // the picks' weights from their keys (the merging wave has the block waiting for it: it leaves this to a
+                       // wave that waits for the row's h here); the row's first block writes the picks and their weights out
+        const unsigned mk = lane < topk ? S.pk[lane] : 0u;
+        const int ei = lane < topk ? S.pe[lane] : 0x7fffffff;
+        const float top0 = rank_key_inv((unsigned) __builtin_amdgcn_readlane((int) mk, 0));
+        const float ek = mk > RANK_KEY_NEG_INF ? fnx_expf(rank_key_inv(mk) - top0) : 0.f;   // a pick without a finite logit weighs nothing
+        float z = 0.f;
+        for (int k = 0; k < topk; ++k) z += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, ek), k));
+        const float wk = z > 0.f ? ek / z : 0.f;
+        if (lane < topk) S.pw[lane] = wk;
+        if (g == 0) {
+            if (lane < topk) {
+                __hip_atomic_store(&a.topi[t * topk + lane], ei, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(&a.topw[t * topk + lane], wk, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            win_stores_done();
+            if (lane == 0) __hip_atomic_fetch_add(&a.sync[WS_ROUTED], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
     if (wave == 1) {   // the shared expert's gate: the router's last row against the row of x, in the router's order
         float4 wg[8];
         int l2 = lane;
@@ -697,8 +733,8 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
         if (lane == 0) __hip_atomic_store(&S.hready, ok ? 1 : -1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
         if (dwave) first_trips();
     }
-    if (!lds_wait([&] { return uniform(__hip_atomic_load(&S.hready, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP)) != 0; })) return;
-    if (uniform(__hip_atomic_load(&S.hready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) < 0) return;
+    if (!lds_wait([&] { return uniform(__hip_atomic_load(&S.hready, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP)) != 0; })) return false;
+    if (uniform(__hip_atomic_load(&S.hready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) < 0) return false;
     WIN_TS(8);
     {   // the row's pairs' h rows into LDS, a pick's words side by side; the shared expert's are index topk
         constexpr int HQ_PER = SBR * HQ_WORDS, HQ_VPT = ((FL_MAXK + 1) * HQ_PER + WN_THREADS - 1) / WN_THREADS;
@@ -719,11 +755,11 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
     WIN_TS(9);
     if (dwave) {
         auto pick_of = [&](int trip) { return trip == 0 ? topk : trip - 1; };   // the index of a trip's expert in S.hq
-        float acc[RMAX], zs[RMAX];
+        float acc[RR], zs[RR];
 #pragma unroll
-        for (int r = 0; r < RMAX; ++r) acc[r] = zs[r] = 0.f;
+        for (int r = 0; r < RR; ++r) acc[r] = zs[r] = 0.f;
         const float gate = S.gate;
-        auto decode_trip = [&](const PackedSub(&buf)[RMAX], int trip) {
+        auto decode_trip = [&](const PackedSub(&buf)[RR], int trip) {
             switch ((wave >> 2) + trip & 3) {   // every wave takes each of the four priorities in turn (see the sweeps)
                 case 0: __builtin_amdgcn_s_setprio(0); break;
                 case 1: __builtin_amdgcn_s_setprio(1); break;
@@ -737,8 +773,7 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
             const float dh = __uint_as_float(hb[8]);
             const float gk = trip == 0 ? gate : S.pw[trip - 1];
 #pragma unroll
-            for (int r = 0; r < RMAX; ++r)
-                if (r < R) {
+            for (int r = 0; r < RR; ++r) {
                     int w4[8];
 #pragma unroll
                     for (int j = 0; j < 8; ++j) w4[j] = *reinterpret_cast<const int*>(reinterpret_cast<const uint8_t*>(S.tab) + packed_addr(buf[r].idx, j));
@@ -752,13 +787,30 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
                     else acc[r] = fmaf(gk, z, acc[r]);
                 }
         };
-        for (int trip = first; trip <= topk; trip += NB) {
+        // A trip's loads go to the buffer that held trip nx - NB, decoded before this one. The rounds in which every trip exists
+        // and so does the one it asks for come first, without a condition on a load (see above); the last trips follow with them.
+        int trip = first;
+        if (topk + 1 - first >= NB + DEPTH) {
+#pragma unroll
+            for (int i = 0; i < NB; ++i) {   // the first round: its own buffers came before the wait for h
+                decode_trip(B[i], first + i);
+                if (i + DEPTH >= NB) issue_trip(B[(i + DEPTH) % NB], first + i + DEPTH);
+            }
+            for (trip = first + NB; trip + NB - 1 + DEPTH <= topk; trip += NB) {
+#pragma unroll
+                for (int i = 0; i < NB; ++i) {
+                    decode_trip(B[i], trip + i);
+                    issue_trip(B[(i + DEPTH) % NB], trip + i + DEPTH);
+                }
+            }
+        }
+        for (; trip <= topk; trip += NB) {
 #pragma unroll
             for (int i = 0; i < NB; ++i) {
                 const int tr = trip + i;
                 if (tr > topk) break;
                 decode_trip(B[i], tr);
-                const int nx = tr + DEPTH;   // the buffer it goes to held trip nx - NB, decoded before this one
+                const int nx = tr + DEPTH;
                 if (nx >= first + NB && nx <= topk) issue_trip(B[(i + DEPTH) % NB], nx);
             }
         }
@@ -766,13 +818,21 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
         if (kb == SBR - 1) {   // the combine's last step: s + sigmoid * shared
             float* orow = a.out + (size_t) t * a.rows + (size_t) u0 * RW + gl;
 #pragma unroll
-            for (int r = 0; r < RMAX; ++r)
-                if (r < R) {
+            for (int r = 0; r < RR; ++r) {
                     const float shared = ext ? gate * a.sh_part[(size_t) t * a.rows + (size_t) (u0 + r) * RW + gl] : zs[r];
                     // (at the device's level: the row's last block may read the row back below, from another XCD)
                     __hip_atomic_store(reinterpret_cast<unsigned*>(orow + r * RW), __float_as_uint(acc[r] + shared), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
         }
+    }
+    return true;
+    };
+    {
+        bool ok;
+        if (R == RMAX) ok = down_phase(std::integral_constant<int, RMAX>{});
+        else if (RMAX > 2 && R == 2) ok = down_phase(std::integral_constant<int, (RMAX > 2 ? 2 : 1)>{});
+        else ok = down_phase(std::integral_constant<int, 1>{});
+        if (!ok) return;
     }
     win_stores_done();
     // rows past the ones that count get no window's rows added, but whatever follows still reads their normed rows: block g of
