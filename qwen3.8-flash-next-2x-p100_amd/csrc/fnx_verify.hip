@@ -1368,6 +1368,7 @@ static int pf_route(const float* logits, int logits_stride, int C, int nexp, int
                     fnx_bigjob* jobs_gu, fnx_bigjob* jobs_dn, int njobs_cap, int* njobs, fnx_bigjob* sh_gu, fnx_bigjob* sh_dn, int* nsh, void* st,
                     const float* cvt_x = nullptr, size_t cvt_n = 0, uint16_t* cvt_y = nullptr) {
     if (!logits || !topi || !topw || !cnt || !jbase || !jobs_gu || !jobs_dn || !njobs) return fail("pf_route: null argument");
+    static_assert(TK_MAXE <= PF_MAXE, "k_pf_fill counts every expert's pairs in LDS");
     if (C < 1 || nexp < 1 || nexp > TK_MAXE || topk < 1 || topk > 64 || topk > nexp) return fail("pf_route: bad shape");
     if (logits_stride < nexp) return fail("pf_route: logits_stride smaller than nexp");
     if ((long) C * topk > (1l << 30)) return fail("pf_route: too many pairs");
@@ -1377,9 +1378,8 @@ static int pf_route(const float* logits, int logits_stride, int C, int nexp, int
     const int cvt_blocks = cvt_n ? (int) std::min<size_t>((cvt_n + 4095) / 4096, 2048) : 0;   // 16 values a thread or more
     k_pf_topk<<<(C + PF_TOPK_WAVES - 1) / PF_TOPK_WAVES + cvt_blocks, PF_TOPK_WAVES * 64, 0, s>>>(logits, logits_stride, C, nexp, topk, topi, topw,
                                                                                                   cvt_x, cvt_n, cvt_y);
-    k_pf_jobbase<<<1, PF_BASE_THREADS, 0, s>>>(topi, P, nexp, cnt, jbase, njobs);
     const int shb = sh_gu ? (C + PF_FILL_THREADS - 1) / PF_FILL_THREADS : 0;
-    k_pf_fill<<<nexp + shb, PF_FILL_THREADS, 0, s>>>(topi, P, topk, nexp, cnt, jbase, jobs_gu, jobs_dn, njobs_cap, C, sh_gu, sh_dn, nsh);
+    k_pf_fill<<<nexp + shb, PF_FILL_THREADS, 0, s>>>(topi, P, topk, nexp, cnt, jbase, njobs, jobs_gu, jobs_dn, njobs_cap, C, sh_gu, sh_dn, nsh);
     return launch_status("pf_route");
 }
 int fnx_pf_route(const float* logits, int logits_stride, int C, int nexp, int topk, int* topi, float* topw, int* cnt, int* jbase,

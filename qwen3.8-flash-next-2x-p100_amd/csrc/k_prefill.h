@@ -48,38 +48,17 @@ __global__ void __launch_bounds__(PF_TOPK_WAVES * 64) k_pf_topk(const float* __r
     if (nexp <= 512) wave_topk<8>(logits + (size_t) t * ls, nexp, topk, lane, ex[wave], topi + (size_t) t * topk, topw + (size_t) t * topk);
     else wave_topk<16>(logits + (size_t) t * ls, nexp, topk, lane, ex[wave], topi + (size_t) t * topk, topw + (size_t) t * topk);
 }
-// one block: the experts' pair counts, each expert's first job (ceil(count / FNX_PF_JOB) jobs each), the job count
-constexpr int PF_BASE_THREADS = 1024;
-__global__ void __launch_bounds__(PF_BASE_THREADS) k_pf_jobbase(const int* __restrict__ topi, int P, int nexp, int* __restrict__ cnt,
-                                                               int* __restrict__ jbase, int* __restrict__ njobs) {
-    __shared__ int c[PF_BASE_THREADS], s[PF_BASE_THREADS];
-    const int e = threadIdx.x;
-    c[e] = 0;
-    __syncthreads();
-    for (int p = e; p < P; p += PF_BASE_THREADS) atomicAdd(&c[topi[p]], 1);
-    __syncthreads();
-    const int nj = e < nexp ? (c[e] + FNX_PF_JOB - 1) / FNX_PF_JOB : 0;
-    s[e] = nj;
-    __syncthreads();
-    for (int o = 1; o < PF_BASE_THREADS; o <<= 1) {
-        const int a = e >= o ? s[e - o] : 0;
-        __syncthreads();
-        s[e] += a;
-        __syncthreads();
-    }
-    if (e < nexp) {
-        cnt[e] = c[e];
-        jbase[e] = s[e] - nj;
-    }
-    if (e == PF_BASE_THREADS - 1) njobs[0] = s[e];
-}
 // a block per expert: its pairs in ascending order into the slots of its jobs (a pair always lands in the same job and
 // slot, prefill.cu:340-343). A thread looks at PF_ROUNDS pairs a pass (p = p0 + 256 r + tid), all loaded together; the
 // slots come from the waves' ballot counts, one barrier a pass. Blocks past the experts write the shared expert's
 // jobs (every row: gate|up reads row t, writes row P + t; down reads and writes row P + t) and their count.
-constexpr int PF_FILL_THREADS = 256, PF_ROUNDS = 8;
-__global__ void __launch_bounds__(PF_FILL_THREADS) k_pf_fill(const int* __restrict__ topi, int P, int topk, int nexp, const int* __restrict__ cnt,
-                                                            const int* __restrict__ jbase, fnx_bigjob* __restrict__ gu,
+// Where its jobs start an expert's block works out for itself - every expert's pair count (the picks are a few KB, which each
+// block reads anyway), ceil(count / FNX_PF_JOB) jobs each, the jobs of the experts before it - instead of waiting for a
+// launch of one block that does it for all; it leaves its expert's count and first job (cnt, jbase), the last expert's
+// block the job count.
+constexpr int PF_FILL_THREADS = 256, PF_ROUNDS = 8, PF_MAXE = 1024;   // (PF_MAXE: the most experts)
+__global__ void __launch_bounds__(PF_FILL_THREADS) k_pf_fill(const int* __restrict__ topi, int P, int topk, int nexp, int* __restrict__ cnt,
+                                                            int* __restrict__ jbase, int* __restrict__ njobs, fnx_bigjob* __restrict__ gu,
                                                             fnx_bigjob* __restrict__ dn, int cap, int C, fnx_bigjob* __restrict__ sh_gu,
                                                             fnx_bigjob* __restrict__ sh_dn, int* __restrict__ nsh) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -100,10 +79,29 @@ __global__ void __launch_bounds__(PF_FILL_THREADS) k_pf_fill(const int* __restri
         return;
     }
     const int e = blockIdx.x;
-    const int ce = cnt[e], jb = jbase[e];
-    if (ce == 0) return;
     constexpr int NW = PF_FILL_THREADS / 64;
+    __shared__ int hist[PF_MAXE], wjobs[NW];
     __shared__ int wsum[PF_ROUNDS][NW];
+    for (int i = tid; i < nexp; i += PF_FILL_THREADS) hist[i] = 0;
+    __syncthreads();
+    for (int p = tid; p < P; p += PF_FILL_THREADS) atomicAdd(&hist[topi[p]], 1);
+    __syncthreads();
+    int before_me = 0;   // jobs of the experts before this one
+    for (int i = tid; i < e; i += PF_FILL_THREADS) before_me += (hist[i] + FNX_PF_JOB - 1) / FNX_PF_JOB;
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) before_me += __shfl_xor(before_me, o, 64);
+    if (lane == 0) wjobs[wave] = before_me;
+    __syncthreads();
+    int jb = 0;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) jb += wjobs[w];
+    const int ce = hist[e];
+    if (tid == 0) {
+        cnt[e] = ce;
+        jbase[e] = jb;
+        if (e == nexp - 1) njobs[0] = jb + (ce + FNX_PF_JOB - 1) / FNX_PF_JOB;
+    }
+    if (ce == 0) return;
     int base = 0;
     for (int p0 = 0; p0 < P; p0 += PF_FILL_THREADS * PF_ROUNDS) {
         int pick[PF_ROUNDS];
