@@ -86,6 +86,31 @@ def test_moe_verify_layer_shapes(dev, oracle, n, ff, nexp, topk, T, packed):
     check_layer(dev, oracle, n, ff, nexp, topk, T, 910 + T, packed)
 
 
+@pytest.mark.parametrize("packed", [False, True])
+def test_moe_verify_layer_with_experts_from_pointer_tables(dev, oracle, packed):
+    """fnx_dw.ep: an expert's matrix by a table of device pointers instead of base + e * stride (an engine whose experts
+    sit in allocations of their own). The tables here list the experts in a shuffled memory order and the bases are null,
+    so only a launch that goes by the tables can give the oracle's bits."""
+    import torch
+    n, ff, nexp, topk, T = 2048, 512, 48, 10, 16
+    got, want, layer, x = check_layer(dev, oracle, n, ff, nexp, topk, T, 930, packed)
+    rng = np.random.default_rng(931)
+    perm = rng.permutation(nexp)   # expert e's matrices lie at place perm[e]
+    tables = []
+    for w, stride in ((layer.gu, layer.gu_stride), (layer.down, layer.down_stride)):
+        moved = torch.empty_like(w)
+        src = w.view(nexp, stride)
+        moved.view(nexp, stride)[torch.as_tensor(perm, device=w.device)] = src
+        table = torch.as_tensor(moved.data_ptr() + perm.astype(np.int64) * stride, dtype=torch.int64, device=w.device)
+        tables.append((moved, table))
+    layer.L.gu.p = layer.L.down.p = None
+    layer.L.gu.ep, layer.L.down.ep = tables[0][1].data_ptr(), tables[1][1].data_ptr()
+    got2 = layer.run(x)
+    assert not got2["sync"].any()
+    assert np.array_equal(got2["topi"], want["topi"])
+    assert np.array_equal(got2["out"].view(np.uint32), want["out"].view(np.uint32)), rel_l2(got2["out"], want["out"])
+
+
 def q8_split(oracle, rng, rows, cols, scale):
     import oracle_lib as ol
     w = (rng.standard_normal((rows, cols)) * scale).astype(np.float32)
