@@ -40,6 +40,11 @@ constexpr int WN_SLOTS = 4, WN_LAG = 2;
 constexpr unsigned WN_LDS_SPINS = 1u << 22;   // trips of a wait inside the block before it gives up (tenths of a second)
 // the workspace's sync words (zero before the first window; every window leaves them zero)
 constexpr int WS_ERR = 0, WS_ROUTED = 1, WS_FIN = 2, WS_ROW0 = 32, WS_ROW_STRIDE = 32;   // a row's words: 0 logits arrivals, 1 h arrivals, 2 blocks done
+// A window of few rows has many blocks a row, and their arrivals on one word are taken one after another (some 40 ns
+// each: 128 of them were most of such a window's hand-overs). The sixteen rows' cache lines are dealt to the rows that
+// count - win_lines(Tl) lines a row, row t's first at line t * win_lines(Tl) - and block g arrives on line g mod lines;
+// a wait adds the lines' words up. (The blocks-done word stays on the row's first line: nothing waits for it.)
+__host__ __device__ constexpr int win_lines(int Tl) { return Tl <= 1 ? 16 : Tl <= 2 ? 8 : Tl <= 4 ? 4 : Tl <= 8 ? 2 : 1; }
 static_assert(WS_ROW0 + FNX_MAXT * WS_ROW_STRIDE <= FNX_MOE_SYNC_WORDS, "the header states the sync area's size");
 
 struct WindowArgs {
@@ -109,6 +114,22 @@ struct WinLds {
     __attribute__((aligned(16))) uint32_t hq[FL_MAXK + 1][SBR][HQ_WORDS];   // the row's pairs' h rows (phase D)
 };
 
+// A wait of one wave for the sum of a word over `lines` consecutive rows' lines. False: the budget ran out (the error bit is set).
+__device__ __forceinline__ bool win_wait_lines(const unsigned* p, int lines, unsigned want, long long ticks, unsigned* err) {
+    const long long t0 = (long long) wall_clock64();
+    const int lane = threadIdx.x & 63;
+    while (true) {
+        unsigned v = lane < lines ? __hip_atomic_load(p + lane * WS_ROW_STRIDE, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+#pragma unroll
+        for (int o = 8; o >= 1; o >>= 1) v += (unsigned) __shfl_xor((int) v, o, 64);   // (lines <= 16)
+        if (uniform((int) v) >= (int) want) return true;
+        if ((long long) wall_clock64() - t0 > ticks) {
+            if (lane == 0) atomicOr(err, FNX_ERR_BARRIER);
+            return false;
+        }
+        __builtin_amdgcn_s_sleep(4);
+    }
+}
 // A wait of one wave for a word of another block's. False: the budget ran out (the error bit is set).
 __device__ __forceinline__ bool win_wait_word(const unsigned* p, unsigned want, long long ticks, unsigned* err) {
     const long long t0 = (long long) wall_clock64();
@@ -219,7 +240,9 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
     if (t >= Tl) return;
     WIN_TS(0);
     const int k0 = pl.k0, nk = pl.nk, qpp = pl.qpp;
-    unsigned* const srow = a.sync + WS_ROW0 + t * WS_ROW_STRIDE;
+    unsigned* const srow = a.sync + WS_ROW0 + t * win_lines(Tl) * WS_ROW_STRIDE;   // the row's first line
+    // the line this block arrives on (worked out where it is wanted: one value fewer to keep through the launch)
+    auto arrival_line = [&] { return srow + (g & (win_lines(Tl) - 1)) * WS_ROW_STRIDE; };
     unsigned* const serr = a.sync + WS_ERR;
     const float* xrow = a.x + (size_t) t * FL_N;
 
@@ -359,7 +382,7 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
         int old = 0;
         if (lane == 0) old = atomicAdd(&S.rarrive, 1);
         if (uniform(old) == WN_WAVES - 1)   // the block's last wave to get here: the block's logits are out
-            if (lane == 0) __hip_atomic_fetch_add(&srow[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (lane == 0) __hip_atomic_fetch_add(&arrival_line()[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 
     // ---------------------------------------------------------------- phase G
@@ -420,7 +443,7 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
     if (early) issue_from(a.gu_shared, ma.j);
     // the row's logits: one wave waits for the row's blocks, the others for its word
     if (wave == WN_WAVES - 1) {
-        const bool ok = win_wait_word(&srow[0], (unsigned) pl.G, a.wait_ticks, serr);
+        const bool ok = win_wait_lines(&srow[0], win_lines(Tl), (unsigned) pl.G, a.wait_ticks, serr);
         if (lane == 0) __hip_atomic_store(&S.lready, ok ? 1 : -1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
     const int sc_shift = 4 * (lane & 1);
@@ -674,7 +697,7 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
         int old = 0;
         if (lane == 0) old = atomicAdd(&S.harrive, 1);
         if (uniform(old) == WN_WAVES - 1)
-            if (lane == 0) __hip_atomic_fetch_add(&srow[1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (lane == 0) __hip_atomic_fetch_add(&arrival_line()[1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     WIN_TS(7);
     if (wave == 2) {   // the picks' weights from their keys (the merging wave has the block waiting for it: it leaves this to a
@@ -729,7 +752,7 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
     };
     if (dwave && wave != 0) first_trips();
     if (wave == 0) {
-        const bool ok = win_wait_word(&srow[1], (unsigned) pl.nbi, a.wait_ticks, serr);
+        const bool ok = win_wait_lines(&srow[1], win_lines(Tl), (unsigned) pl.nbi, a.wait_ticks, serr);
         if (lane == 0) __hip_atomic_store(&S.hready, ok ? 1 : -1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
         if (dwave) first_trips();
     }
@@ -848,8 +871,10 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
     if (tid == 0) {
         const unsigned done = __hip_atomic_fetch_add(&srow[2], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (done == (unsigned) pl.G - 1) {
-            __hip_atomic_store(&srow[0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(&srow[1], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (int l = 0; l < win_lines(Tl); ++l) {
+                __hip_atomic_store(&srow[l * WS_ROW_STRIDE + 0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(&srow[l * WS_ROW_STRIDE + 1], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
             __hip_atomic_store(&srow[2], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             S.fin = (int) __hip_atomic_fetch_add(&a.sync[WS_FIN], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             S.last = 1;
