@@ -45,9 +45,11 @@ __device__ __forceinline__ void j16_segment(J16Lds& L, const uint8_t* __restrict
     const uint8_t* xrow = L.xq + r * J16_XLD + 8 * grp;   // bytes 8 grp .. of sub-block 16 S + 4 j + p of token r lie 512 S + 128 j + 32 p further
     float* myw = &L.sw[wave][grp][r];
     const uint32_t copy_at = 4u * (lane & 1);
+    if (g0 + wave >= g1) return;
+    // the fields of the super-step at hand; a tile's last super-step leaves the next tile's first ones here
+    SuperFields f = tile16_load(we, 16 * (g0 + wave) + r, 0, nsuper);
     for (int g = g0 + wave; g < g1; g += J16_WAVES) {
         float acc[4] = {0.f, 0.f, 0.f, 0.f};
-        SuperFields f = tile16_load(we, 16 * g + r, 0, nsuper);
         for (int S = 0; S < nsuper; ++S) {
             // the next super-step's fields (past the tile's last: the next tile of this wave, or this one again)
             const int gn = S + 1 < nsuper ? g : (g + J16_WAVES < g1 ? g + J16_WAVES : g);
