@@ -1766,23 +1766,40 @@ static int mtp_draft(const fnx_decoder* D, const fnx_mtp* M, const float* src, c
     if (M->pen && !M->pen_par) return fail("mtp_draft: a penalty list without its parameters");
     const int n = D->n;
     // R = fc_hid(rms(src)) + fc_emb(rms(emb)): the sum is taken by the layer's first pass over the rows
-    {   // nothing to add: src is only read (fnx_add_norm_q8)
+    if (D->nq * AT_HD >= 2 * n) {
+        // both inputs' passes in one launch (fnx_add_norm_q8's, twice): src is only read, nothing is added; the tokens' embedding
+        // rows are normed and quantised by the pass that reads them from the table (rms(emb[tokens])). Their q8_1 rows go to
+        // the second half of the workspace's q8_1 rows, which hold max(n, nq * 256) values a row.
+        uint8_t* xq2 = (uint8_t*) ws->xq + (size_t) FNX_MAXT * (n / 32) * FNX_Q8_1_BLOCK;
         CombineArgs c{};
         c.gate = gate;
-        k_add_norm_q8<false><<<T, 256, 0, (hipStream_t) st>>>(const_cast<float*>(src), nullptr, c, M->norm_hid, nullptr, (uint8_t*) ws->xq, n, D->eps);
-        if (launch_status("mtp_draft")) return 1;
-    }
-    if (q8s_one(&M->fc_hid, ws->xq, ws->x, n, T, st, gate)) return 1;
-    {   // the tokens' embedding rows, normed and quantised by the pass that reads them from the table (rms(emb[tokens]))
-        CombineArgs c{};
-        c.emb = D->emb;
         c.tokens = tokens;
         c.vocab = D->vocab;
-        c.gate = gate;
-        k_add_norm_q8<false><<<T, 256, 0, (hipStream_t) st>>>(ws->xn, nullptr, c, M->norm_emb, nullptr, (uint8_t*) ws->xq, n, D->eps);
+        c.rows1 = T, c.rows2 = T;
+        c.x2 = ws->xn, c.w2 = M->norm_emb, c.xq2 = xq2, c.emb2 = D->emb;
+        k_add_norm_q8<false><<<2 * T, 256, 0, (hipStream_t) st>>>(const_cast<float*>(src), nullptr, c, M->norm_hid, nullptr, (uint8_t*) ws->xq, n, D->eps);
         if (launch_status("mtp_draft")) return 1;
+        if (q8s_one(&M->fc_hid, ws->xq, ws->x, n, T, st, gate)) return 1;
+        if (q8s_one(&M->fc_emb, xq2, ws->o, n, T, st, gate)) return 1;
+    } else {
+        {   // nothing to add: src is only read (fnx_add_norm_q8)
+            CombineArgs c{};
+            c.gate = gate;
+            k_add_norm_q8<false><<<T, 256, 0, (hipStream_t) st>>>(const_cast<float*>(src), nullptr, c, M->norm_hid, nullptr, (uint8_t*) ws->xq, n, D->eps);
+            if (launch_status("mtp_draft")) return 1;
+        }
+        if (q8s_one(&M->fc_hid, ws->xq, ws->x, n, T, st, gate)) return 1;
+        {   // the tokens' embedding rows (rms(emb[tokens]))
+            CombineArgs c{};
+            c.emb = D->emb;
+            c.tokens = tokens;
+            c.vocab = D->vocab;
+            c.gate = gate;
+            k_add_norm_q8<false><<<T, 256, 0, (hipStream_t) st>>>(ws->xn, nullptr, c, M->norm_emb, nullptr, (uint8_t*) ws->xq, n, D->eps);
+            if (launch_status("mtp_draft")) return 1;
+        }
+        if (q8s_one(&M->fc_emb, ws->xq, ws->o, n, T, st, gate)) return 1;
     }
-    if (q8s_one(&M->fc_emb, ws->xq, ws->o, n, T, st, gate)) return 1;
     DecPending pend{ws->o, nullptr, nullptr};
     if (dec_layer(D, &M->layer, T, pos0, ws, pend, st, live, gate, M->out_norm, ws->hidden)) return 1;
     return dec_head(D, M->out_norm, &M->head, T, ws, pend, st, gate, nv, M->dv0, M->pen, M->pen_par);

@@ -43,6 +43,14 @@ struct CombineArgs {
     int vocab;
     const int* live;      // may be null; else a device word: rows from *live on were not routed and get no combine added
     const int* gate;      // may be null; else a device word: at zero the launch leaves at once (a chain step that does not count)
+    // A second pass in the same launch (the narrow form; rows2 > 0): blocks from rows1 on are rows 0 .. rows2 - 1 of a pass over
+    // x2 with the weights w2, into xq2, their rows from the table if emb2 is set (the draft layer's two inputs, each with a
+    // norm of its own, are one launch this way)
+    int rows1, rows2;
+    float* x2;
+    const float* w2;
+    uint8_t* xq2;
+    const uint16_t* emb2;
 };
 // WIDE (the combine's form): 1024 threads make the row after the add - a thread the columns p, p + 1024, ..., with all
 // of an expert batch's partial sums in flight (256 threads with 8 columns each took 13 us a call, against 7 us without
@@ -54,7 +62,13 @@ __global__ void __launch_bounds__(WIDE ? 1024 : 256) k_add_norm_q8(float* __rest
     __shared__ float sh[4];
     __shared__ float vrow[WIDE ? 256 * NQ_MAXJ : 1];
     if (c.gate && uniform(*c.gate) == 0) return;
-    const size_t row = blockIdx.x;
+    size_t row = blockIdx.x;
+    const uint16_t* emb = c.emb;
+    if (!WIDE && c.rows2 > 0 && (int) blockIdx.x >= c.rows1) {   // the launch's second pass
+        row = blockIdx.x - c.rows1;
+        x = c.x2, w = c.w2, xq = c.xq2, emb = c.emb2;
+        xn = nullptr, add = nullptr;
+    }
     float v[NQ_MAXJ];
     float s = 0.f;
     if constexpr (WIDE) {
@@ -111,11 +125,11 @@ __global__ void __launch_bounds__(WIDE ? 1024 : 256) k_add_norm_q8(float* __rest
     } else {
         // all loads first: a store to x between them would keep the next load waiting for it
         float av[NQ_MAXJ];
-        const size_t erow = c.emb ? (size_t) min(max(c.tokens[row], 0), c.vocab - 1) : 0;   // k_embed_rows' clamp
+        const size_t erow = emb ? (size_t) min(max(c.tokens[row], 0), c.vocab - 1) : 0;   // k_embed_rows' clamp
 #pragma unroll
         for (int j = 0; j < NQ_MAXJ; ++j) {
             const int i = threadIdx.x + 256 * j;
-            if (c.emb) v[j] = i < n ? half_bits_to_float(c.emb[erow * n + i]) : 0.f;
+            if (emb) v[j] = i < n ? half_bits_to_float(emb[erow * n + i]) : 0.f;
             else v[j] = i < n ? x[row * n + i] : 0.f;
             av[j] = add && i < n ? add[row * n + i] : 0.f;
         }
@@ -130,7 +144,7 @@ __global__ void __launch_bounds__(WIDE ? 1024 : 256) k_add_norm_q8(float* __rest
         const int i = threadIdx.x + 256 * j;
         wv[j] = i < n ? w[i] : 0.f;
     }
-    if (!WIDE && (add || c.emb)) {
+    if (!WIDE && (add || emb)) {
 #pragma unroll
         for (int j = 0; j < NQ_MAXJ; ++j) {
             const int i = threadIdx.x + 256 * j;
