@@ -1531,8 +1531,10 @@ int fnx_embed_rows(const uint16_t* emb, const int* tokens, int T, int vocab, int
     k_embed_rows<<<T, 256, 0, (hipStream_t) st>>>(emb, tokens, vocab, n, y);
     return launch_status("embed_rows");
 }
+// yq2 (may be null): two matrices, the second one over rows of its own - as long as every block has one tile, which is then of
+// one matrix (else refused: the caller launches twice)
 static int q8s_launch(const fnx_q8s* const* W, float* const* out, const int* out_stride, int n, const void* yq, int T, void* st, const char* who,
-                      const int* gate = nullptr) {
+                      const int* gate = nullptr, const void* yq2 = nullptr) {
     if (!W || !out || !out_stride || !yq || n < 1 || n > 3) return fail(std::string(who) + ": null argument");
     Q8sArgs a{};
     long tiles = 0;
@@ -1565,6 +1567,10 @@ static int q8s_launch(const fnx_q8s* const* W, float* const* out, const int* out
     static const int per_cu = env_int("FNX_Q8S_BLOCKS_PER_CU", 4, 1, 16);   // what the LDS of a 2048-column matrix lets a CU hold
     const int grid = (int) std::max(1l, std::min<long>((long) per_cu * cu_count(), tiles));
     a.gate = gate;
+    if (yq2) {
+        if (n != 2 || grid < tiles) return fail(std::string(who) + ": two sets of rows want two matrices and a block a tile");
+        a.yq2 = (const uint8_t*) yq2;
+    }
     if (W[0]->tiled) k_q8s_gemv<1, true><<<grid, Q8S_WAVES * 64, lds, (hipStream_t) st>>>(a);
     else k_q8s_gemv<1><<<grid, Q8S_WAVES * 64, lds, (hipStream_t) st>>>(a);
     return launch_status(who);
@@ -1779,8 +1785,19 @@ static int mtp_draft(const fnx_decoder* D, const fnx_mtp* M, const float* src, c
         c.x2 = ws->xn, c.w2 = M->norm_emb, c.xq2 = xq2, c.emb2 = D->emb;
         k_add_norm_q8<false><<<2 * T, 256, 0, (hipStream_t) st>>>(const_cast<float*>(src), nullptr, c, M->norm_hid, nullptr, (uint8_t*) ws->xq, n, D->eps);
         if (launch_status("mtp_draft")) return 1;
-        if (q8s_one(&M->fc_hid, ws->xq, ws->x, n, T, st, gate)) return 1;
-        if (q8s_one(&M->fc_emb, xq2, ws->o, n, T, st, gate)) return 1;
+        // and the two projections one: a block a tile of one of the two matrices, over that matrix's rows
+        const long fc_tiles = (M->fc_hid.n_out + 15) / 16 + (M->fc_emb.n_out + 15) / 16;
+        static const int per_cu = env_int("FNX_Q8S_BLOCKS_PER_CU", 4, 1, 16);
+        if (fc_tiles <= (long) per_cu * cu_count() && M->fc_hid.n_out % 16 == 0 && M->fc_hid.n_in == M->fc_emb.n_in &&
+            (M->fc_hid.tiled != 0) == (M->fc_emb.tiled != 0)) {
+            const fnx_q8s* W2[2] = {&M->fc_hid, &M->fc_emb};
+            float* out2[2] = {ws->x, ws->o};
+            const int stride2[2] = {n, n};
+            if (q8s_launch(W2, out2, stride2, 2, ws->xq, T, st, "q8s_gemv", gate, xq2)) return 1;
+        } else {
+            if (q8s_one(&M->fc_hid, ws->xq, ws->x, n, T, st, gate)) return 1;
+            if (q8s_one(&M->fc_emb, xq2, ws->o, n, T, st, gate)) return 1;
+        }
     } else {
         {   // nothing to add: src is only read (fnx_add_norm_q8)
             CombineArgs c{};

@@ -225,6 +225,7 @@ struct Q8sArgs {
     int nseg, cols, T;
     const uint8_t* yq;   // q8_1 rows
     const int* gate;     // may be null; else a device word: at zero the launch leaves at once (a chain step that does not count)
+    const uint8_t* yq2;  // may be null; else the second matrix's rows are these (two matrices, a block a tile: the host sees to that)
 };
 typedef int q8s_v4i __attribute__((ext_vector_type(4)));
 // DEPTH: the (tile, batch) items whose loads are in flight ahead of the one being worked on. (With 3 - all of a tile's
@@ -364,7 +365,7 @@ __global__ void __launch_bounds__(Q8S_WAVES * 64) k_q8s_gemv(const Q8sArgs a) {
         const int t = i / nb, b = i - t * nb;
         uint32_t* dst = reinterpret_cast<uint32_t*>(xs + (size_t) t * xld + 32 * b);
         if (t < T) {
-            const uint8_t* blk = a.yq + (size_t) i * 36;
+            const uint8_t* blk = (a.yq2 && (int) blockIdx.x >= t0 ? a.yq2 : a.yq) + (size_t) i * 36;
             xd[t * dld + b] = half_bits_to_float(load_u16(blk));
             const uint32_t* src = reinterpret_cast<const uint32_t*>(blk + 4);
 #pragma unroll
