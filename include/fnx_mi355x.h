@@ -206,12 +206,13 @@ typedef struct fnx_moe_ws {
                       * the pairs' h there instead, as q8_1 rows of its own record size, and never writes f32 gate|up rows */
     float* part;     /* [T * topk + T][n] floats. Operator by operator: the down outputs. The one-launch window uses it only
                       * as scratch for a split-Q8_0 shared expert */
-    unsigned* sync;  /* [FNX_MOE_SYNC_WORDS], zeroed once: the arrival counters through which the blocks of the one-launch window
-                      * hand over within a window row (every window leaves them zero), and in word 0 the window's error bits:
+    unsigned* sync;  /* [FNX_MOE_SYNC_WORDS], 8-byte aligned, zeroed once: the arrival counters and the marked words through which
+                      * the blocks of the one-launch window hand over within a window row (every window leaves them zero), and
+                      * in word 0 the window's error bits:
                       * FNX_ERR_BARRIER if a block gave up waiting for its row (kernels.cu:884, 899 bound the reference's device waits
                       * the same way). After that error the results mean nothing and the words must be zeroed again */
 } fnx_moe_ws;
-#define FNX_MOE_SYNC_WORDS 544
+#define FNX_MOE_SYNC_WORDS 33568
 int fnx_moe_verify_layer(const fnx_moe_layer* L, const float* x, int T, float* out, const fnx_moe_ws* ws, void* st);
 /* The same window without a workspace argument and without any allocation: no counterpart in the reference. For callers
  * that cannot allocate device memory (code under graph capture, serving loops and harnesses that forbid it): the scratch
@@ -220,7 +221,7 @@ int fnx_moe_verify_layer(const fnx_moe_layer* L, const float* x, int T, float* o
  * 512 or 1024, up to 1024 experts, up to 16 picks a row, T x topk <= 160; anything else is refused with a message. x and
  * out are the caller's, as above; results are those of fnx_moe_verify_layer bit for bit. All calls on a GPU share that
  * GPU's array: two of them in flight at once (two streams, two threads) race. */
-#define FNX_MOE_STATIC_WS_BYTES (448 * 1024)
+#define FNX_MOE_STATIC_WS_BYTES (576 * 1024)
 int fnx_moe_verify_layer_static(const fnx_moe_layer* L, const float* x, int T, float* out, void* st);
 /* The error word of that array's windows (fnx_moe_ws.sync word 0 of the library's own workspace on the current device),
  * for the caller who cannot see it otherwise: waits for the stream, copies the word to *err and, if FNX_ERR_BARRIER is set

@@ -17,7 +17,7 @@ T_IQ3S_UNIT64 = 1021
 T_IQ3S_TILE16 = 1022
 IQ3S_BLOCK = 110
 Q8_1_BLOCK = 36
-MOE_SYNC_WORDS = 544
+MOE_SYNC_WORDS = 33568
 ARGMAX_WORDS = 32   # FNX_ARGMAX_WORDS: a key and an arrival count a row   # fnx_moe_ws.sync: uint32 words, zeroed once
 ERR_BARRIER = 4
 

@@ -1213,6 +1213,7 @@ static int moe_layer_checked(const fnx_moe_layer* L, const float* x, int T, floa
     if (!L || !x || !ws) return fail("moe_verify_layer: null argument");
     if (!ws->xq || !ws->logits || !ws->topi || !ws->topw || !ws->jobs_gu || !ws->jobs_dn || !ws->njobs || !ws->gu || !ws->part || !ws->sync)
         return fail("moe_verify_layer: incomplete workspace");
+    if ((uintptr_t) ws->sync & 7) return fail("moe_verify_layer: the sync words are 8-byte aligned");
     if (topk_check(T, L->nexp, L->topk, "moe_verify_layer")) return 1;
     const int P = T * L->topk, n = L->n, ff = L->ff;
     if (P + T > HQ_ROWS) return fail("moe_verify_layer: more pairs than the pair buffer holds");

@@ -45,7 +45,13 @@ constexpr int WS_ERR = 0, WS_ROUTED = 1, WS_FIN = 2, WS_ROW0 = 32, WS_ROW_STRIDE
 // count - win_lines(Tl) lines a row, row t's first at line t * win_lines(Tl) - and block g arrives on line g mod lines;
 // a wait adds the lines' words up. (The blocks-done word stays on the row's first line: nothing waits for it.)
 __host__ __device__ constexpr int win_lines(int Tl) { return Tl <= 1 ? 16 : Tl <= 2 ? 8 : Tl <= 4 ? 4 : Tl <= 8 ? 2 : 1; }
-static_assert(WS_ROW0 + FNX_MAXT * WS_ROW_STRIDE <= FNX_MOE_SYNC_WORDS, "the header states the sync area's size");
+// After the rows' lines: the rows' router logits as the blocks hand them to one another, a 64-bit word an expert - the logit's
+// bits and a mark above them - so that a word that has been written says so itself: a block takes its row's logits as soon
+// as their words are there, without an arrival count in between (a count costs its own trip to memory, and the wait for the
+// stores before it). Zero (not written) before a window and again after it: the row's last block clears them.
+constexpr int WS_LX0 = WS_ROW0 + FNX_MAXT * WS_ROW_STRIDE, WS_LX_STRIDE = 1032;   // (64-bit words a row: up to 1,024 experts)
+constexpr unsigned long long WS_LX_MARK = 1ull << 32;
+static_assert(WS_LX0 % 2 == 0 && WS_LX0 + 2 * FNX_MAXT * WS_LX_STRIDE <= FNX_MOE_SYNC_WORDS, "the header states the sync area's size");
 
 struct WindowArgs {
     int ff, nexp, topk, T, rows;
@@ -103,8 +109,8 @@ struct WinLds {
     unsigned pk[FL_MAXK];              // their keys
     float pw[FL_MAXK];                 // their weights
     float gate;                        // sigmoid of the shared expert's gate logit
-    int rarrive, harrive;              // waves of the block that have stored their logits / finished their sweeps
-    int lready, hready;                // 1: the row's logits / h rows are complete; -1: the wait gave up
+    int harrive;                       // waves of the block that have finished their sweeps
+    int hready;                        // 1: the row's h rows are complete; -1: the wait gave up
     int abort;                         // a wait inside the block gave up
     int last;                          // this block is the last of its row to finish
     int fin;                           // the row's ticket among the rows that have finished
@@ -244,6 +250,7 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
     // the line this block arrives on (worked out where it is wanted: one value fewer to keep through the launch)
     auto arrival_line = [&] { return srow + (g & (win_lines(Tl) - 1)) * WS_ROW_STRIDE; };
     unsigned* const serr = a.sync + WS_ERR;
+    unsigned long long* const lx = reinterpret_cast<unsigned long long*>(a.sync + WS_LX0) + (size_t) t * WS_LX_STRIDE;   // the row's logits on their way
     const float* xrow = a.x + (size_t) t * FL_N;
 
     // ---------------------------------------------------------------- phase R: loads
@@ -335,8 +342,8 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
     if (tid < 16) S.sliced[tid] = 0;
     if (tid == 0) {
         S.ready = 0;
-        S.rarrive = S.harrive = 0;
-        S.lready = S.hready = 0;
+        S.harrive = 0;
+        S.hready = 0;
         S.abort = 0;
         S.last = 0;
         S.fin = -1;
@@ -368,21 +375,22 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
         int row = r0 + wave;
         while (true) {
             const float va = router_dot(wa, xr), vb = router_dot(wb, xr);
-            if (lane == 0) {
-                if (row < r1) __hip_atomic_store(&a.logits[(size_t) t * LS + row], va, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                if (row + WN_WAVES < r1) __hip_atomic_store(&a.logits[(size_t) t * LS + row + WN_WAVES], vb, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (lane == 0) {   // to the caller's array, and marked to the row's other blocks
+                if (row < r1) {
+                    a.logits[(size_t) t * LS + row] = va;
+                    __hip_atomic_store(&lx[row], WS_LX_MARK | __float_as_uint(va), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+                if (row + WN_WAVES < r1) {
+                    a.logits[(size_t) t * LS + row + WN_WAVES] = vb;
+                    __hip_atomic_store(&lx[row + WN_WAVES], WS_LX_MARK | __float_as_uint(vb), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
             }
             row += 2 * WN_WAVES;
             if (row >= r1) break;
             load_router_row(row, wa);
             load_router_row(row + WN_WAVES, wb);
         }
-        win_stores_done();
         WIN_TS(2);
-        int old = 0;
-        if (lane == 0) old = atomicAdd(&S.rarrive, 1);
-        if (uniform(old) == WN_WAVES - 1)   // the block's last wave to get here: the block's logits are out
-            if (lane == 0) __hip_atomic_fetch_add(&arrival_line()[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 
     // ---------------------------------------------------------------- phase G
@@ -441,11 +449,6 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
     Item ma = item_of(I0);
     const bool early = nsweep > 0 && ma.k == 0;   // the run starts with a shared expert's item: no pick needed to ask for it
     if (early) issue_from(a.gu_shared, ma.j);
-    // the row's logits: one wave waits for the row's blocks, the others for its word
-    if (wave == WN_WAVES - 1) {
-        const bool ok = win_wait_lines(&srow[0], win_lines(Tl), (unsigned) pl.G, a.wait_ticks, serr);
-        if (lane == 0) __hip_atomic_store(&S.lready, ok ? 1 : -1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
-    }
     const int sc_shift = 4 * (lane & 1);
     // where a lane's sum goes after reduce4_units: the 16-lane rows hold gate 2 i, up 2 i, gate 2 i + 1, up 2 i + 1
     const int zidx = (lane & 16 ? 32 : 0) + 2 * wave + (lane >> 5);
@@ -507,13 +510,28 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
     // The row's picks (moe.cuh:382-411: greater value first, the lower index on a tie; w_k = exp(l_k - l_0) / sum in pick
     // order). Every wave with a slice lists the topk greatest of its 64 experts in order; wave 0 merges the slices' lists by
     // their heads and hands each pick's matrix out as soon as it is known.
-    if (!lds_wait([&] { return uniform(__hip_atomic_load(&S.lready, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP)) != 0; })) return;
-    if (uniform(__hip_atomic_load(&S.lready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) < 0) return;
-    WIN_TS(3);
     const int ns = (nexp + 63) >> 6;   // slices of 64 experts
     for (int sl = wave; sl < ns; sl += WN_WAVES) {
         const int e = 64 * sl + lane;
-        const float v = e < nexp ? __hip_atomic_load(&a.logits[(size_t) t * LS + e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : -INFINITY;
+        // the slice's logits, as soon as the row's blocks have written them all: every word says so itself
+        unsigned long long lw;
+        {
+            const long long t0 = (long long) wall_clock64();
+            while (true) {
+                lw = e < nexp ? __hip_atomic_load(&lx[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : WS_LX_MARK | __float_as_uint(-INFINITY);
+                if (__ballot(lw == 0ull) == 0ull) break;
+                if ((long long) wall_clock64() - t0 > a.wait_ticks || uniform(__hip_atomic_load(&S.abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP))) {
+                    if (lane == 0) {
+                        __hip_atomic_store(&S.abort, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                        atomicOr(serr, FNX_ERR_BARRIER);
+                    }
+                    return;
+                }
+                __builtin_amdgcn_s_sleep(2);
+            }
+        }
+        WIN_TS(3);
+        const float v = __uint_as_float((unsigned) lw);
         unsigned key = rank_key(v);
         for (int k = 0; k < topk; ++k) {
             const unsigned m = wave_umax(key);
@@ -871,10 +889,7 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
     if (tid == 0) {
         const unsigned done = __hip_atomic_fetch_add(&srow[2], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (done == (unsigned) pl.G - 1) {
-            for (int l = 0; l < win_lines(Tl); ++l) {
-                __hip_atomic_store(&srow[l * WS_ROW_STRIDE + 0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                __hip_atomic_store(&srow[l * WS_ROW_STRIDE + 1], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
+            for (int l = 0; l < win_lines(Tl); ++l) __hip_atomic_store(&srow[l * WS_ROW_STRIDE + 1], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __hip_atomic_store(&srow[2], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             S.fin = (int) __hip_atomic_fetch_add(&a.sync[WS_FIN], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             S.last = 1;
@@ -883,7 +898,9 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
     __syncthreads();
     WIN_TS(11);
     if (!S.last) return;
-    // the row is complete (every block of it waited for its stores before it counted itself done)
+    // the row is complete (every block of it waited for its stores before it counted itself done); its logits' words, which
+    // every block of the row has long read, go back to "not written"
+    for (int i = tid; i < nexp; i += WN_THREADS) __hip_atomic_store(&lx[i], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (DEC && a.next_x) win_next_row(a, t, true, reinterpret_cast<float*>(&S.hgu[0][0]));
     const int fin = S.fin;
     if (fin == 0) {   // every row has been ranked long ago; the count says so
