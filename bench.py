@@ -51,7 +51,7 @@ HBM_PEAK = 8.0e12
 # HBM bytes of one window launch of the default run (gaussian weights, 16 sets, unit64), measured by two rocprofv3 --pmc
 # runs of this file (FETCH_SIZE, then WRITE_SIZE, each scaled by a 256 MiB copy: profiles/moe_window_hbm_traffic.md), and
 # the distinct experts per step they were measured at. Not measured in the run: emitted only for that configuration.
-WINDOW_TRAFFIC = {"bytes": 209.14e6, "algorithmic_bytes": 192.96e6, "distinct_experts_per_step": 138.45,
+WINDOW_TRAFFIC = {"bytes": 209.47e6, "algorithmic_bytes": 192.96e6, "distinct_experts_per_step": 138.45,
                    "source": "profiles/moe_window_hbm_traffic.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this file's default workload; scaled to "
                              "this run's algorithmic bytes; not measured in this run)"}
 # the same for the prompt path's gate|up launch (profiles/prefill_chunk_counters.md: FETCH_SIZE x 2 + WRITE_SIZE)
