@@ -941,13 +941,19 @@ static int layer_fused(const fnx_moe_layer* L, const float* x, int T, float* out
     }
     // one block a CU; a row's blocks are a power of two of at least sixteen (moe_window_plan.h)
     const int nb = cu_count();
-    if (wa.next_x) {
-        if (ff == 256) k_moe_window<8, true><<<nb, WN_THREADS, 0, s>>>(wa);
-        else if (ff == 512) k_moe_window<16, true><<<nb, WN_THREADS, 0, s>>>(wa);
-        else k_moe_window<32, true><<<nb, WN_THREADS, 0, s>>>(wa);
-    } else if (ff == 256) k_moe_window<8><<<nb, WN_THREADS, 0, s>>>(wa);
-    else if (ff == 512) k_moe_window<16><<<nb, WN_THREADS, 0, s>>>(wa);
-    else k_moe_window<32><<<nb, WN_THREADS, 0, s>>>(wa);
+    const auto launch = [&](auto sbr, auto dec) {
+        constexpr int SBR = decltype(sbr)::value;
+        constexpr bool DEC = decltype(dec)::value;
+        if (wa.router_bf16) k_moe_window<SBR, DEC, true><<<nb, WN_THREADS, 0, s>>>(wa);
+        else k_moe_window<SBR, DEC, false><<<nb, WN_THREADS, 0, s>>>(wa);
+    };
+    const auto launch_dec = [&](auto sbr) {
+        if (wa.next_x) launch(sbr, std::true_type{});
+        else launch(sbr, std::false_type{});
+    };
+    if (ff == 256) launch_dec(std::integral_constant<int, 8>{});
+    else if (ff == 512) launch_dec(std::integral_constant<int, 16>{});
+    else launch_dec(std::integral_constant<int, 32>{});
     prof_mark(2, s);
     return launch_status("moe_verify_layer");
 }

@@ -229,7 +229,10 @@ __device__ __forceinline__ void win_next_row(const WindowArgs& a, int t, bool ad
 
 // DEC: the launch of a decoder's layer, which may also take the passes either side of the window (next_x, pre_w); without it
 // those arguments are not looked at and their code is not there
-template <int SBR, bool DEC = false>
+// RBF: the router's rows are bf16 (a.router_bf16). A template argument, and a row past the block's slice is loaded all the same
+// (the slice's last, its sum thrown away): the number of loads behind the block's row of x is then the same on every path,
+// the compiler knows it, and the block's first meeting does not wait for the router's rows as well.
+template <int SBR, bool DEC = false, bool RBF = false>
 __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
     __shared__ WinLds<SBR> S;
     constexpr int RW = 64 / SBR, RMAX = SBR / 8, NB = RMAX == 4 ? 2 : 3, DEPTH = RMAX == 4 ? 1 : 2;   // rows a unit; units a wave and trip at most; trips' buffers
@@ -287,10 +290,8 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
     // this wave's router rows: rows r0 + wave, r0 + wave + 16, ... of the block's slice, two at a time
     const int r0 = g * pl.rpb, r1 = min(nexp, r0 + pl.rpb);
     auto load_router_row = [&](int row, float4(&w)[8]) {
-        if (row >= r1) {
-#pragma unroll
-            for (int c = 0; c < 8; ++c) w[c] = make_float4(0.f, 0.f, 0.f, 0.f);
-        } else if (a.router_bf16) {
+        row = min(row, max(r1, 1) - 1);
+        if constexpr (RBF) {
 #pragma unroll
             for (int c = 0; c < 8; ++c) {
                 const uint2 u = reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(a.router) + (size_t) row * FL_N)[c * 64 + lane];
@@ -743,7 +744,7 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
         asm volatile("" : "+v"(l2));   // the addresses are worked out here, not kept in registers since phase R
 #pragma unroll
         for (int c = 0; c < 8; ++c) xr[c] = S.xf[c * 64 + l2];
-        if (a.router_bf16) {
+        if constexpr (RBF) {
 #pragma unroll
             for (int c = 0; c < 8; ++c) {
                 const uint2 u = reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(a.router) + (size_t) nexp * FL_N)[c * 64 + l2];

@@ -111,6 +111,28 @@ def test_moe_verify_layer_with_experts_from_pointer_tables(dev, oracle, packed):
     assert np.array_equal(got2["out"].view(np.uint32), want["out"].view(np.uint32)), rel_l2(got2["out"], want["out"])
 
 
+@pytest.mark.parametrize("packed", [False, True])
+@pytest.mark.parametrize("n,ff,nexp,topk,T", [(2048, 512, 512, 10, 16), (2048, 256, 40, 6, 3)])
+def test_moe_verify_layer_with_a_bf16_router(dev, oracle, n, ff, nexp, topk, T, packed):
+    """fnx_moe_layer.router_bf16: the router's rows as bf16 (the upper halves of f32 values), multiplied as the f32 values
+    they stand for - so the oracle over those f32 values gives the bits."""
+    import torch
+    rng = np.random.default_rng(940 + T)
+    router, gu, down, sh_gu, sh_down = make_layer(rng, n, ff, nexp)
+    bits = (router.view(np.uint32) >> 16).astype(np.uint16)             # truncated to bf16
+    router_as_f32 = (bits.astype(np.uint32) << 16).view(np.float32)
+    x = rng.standard_normal((T, n)).astype(np.float32)
+    want = oracle.moe_verify_layer(n, ff, nexp, topk, router_as_f32, gu, down, sh_gu, sh_down, x)
+    layer = fnx_gpu.MoeLayerDev(dev, n, ff, nexp, topk, router_as_f32, gu, down, sh_gu, sh_down, packed=packed)
+    rb = torch.from_numpy(bits.view(np.int16).copy()).to("cuda")
+    layer.L.router, layer.L.router_bf16 = rb.data_ptr(), 1
+    got = layer.run(x)
+    assert not got["sync"].any()
+    assert np.array_equal(got["logits"].view(np.uint32), want["logits"].view(np.uint32)), "router logits bit-exact"
+    assert np.array_equal(got["topi"], want["topi"])
+    assert np.array_equal(got["out"].view(np.uint32), want["out"].view(np.uint32)), rel_l2(got["out"], want["out"])
+
+
 def q8_split(oracle, rng, rows, cols, scale):
     import oracle_lib as ol
     w = (rng.standard_normal((rows, cols)) * scale).astype(np.float32)
