@@ -32,14 +32,27 @@ FNX_HOST_DEVICE inline AttWindow att_window(int pos0_raw, int T, int max_ctx) {
 FNX_HOST_DEVICE inline bool att_window_fits(int pos0_raw, int T, int max_ctx) { return pos0_raw >= 0 && T >= 1 && pos0_raw <= max_ctx - T; }
 // row qt of the window sees positions [0, this)
 FNX_HOST_DEVICE inline int att_ctx_q(const AttWindow& w, int qt) { return att_min(w.pos0 + qt + 1, w.ctx_max); }
-// split s covers positions [p0, p1); empty when p0 >= p1
-FNX_HOST_DEVICE inline int att_split_begin(int s) { return s * AT_SPLIT; }
-FNX_HOST_DEVICE inline int att_split_end(const AttWindow& w, int s) { return att_min(w.ctx_max, s * AT_SPLIT + AT_SPLIT); }
+// A window of few queries (those of a kv head fit one block of the first pass: AT_HALF_QUERIES) leaves the blocks of the
+// grid's second layer without queries; they take the second half of their split instead, so that such a window - a decode
+// round's, most of the time - is spread over as many blocks as a full one. Part (s, z) of the first pass covers positions
+// [begin, end) (empty when begin >= end) and is part number att_part_index of its query; halves: the window is such a one.
+constexpr int AT_HALF_QUERIES = 64;
+FNX_HOST_DEVICE inline bool att_halves(int nquery) { return nquery <= AT_HALF_QUERIES; }
+FNX_HOST_DEVICE inline int att_part_begin(int s, int z, bool halves) { return s * AT_SPLIT + (halves ? z * (AT_SPLIT / 2) : 0); }
+FNX_HOST_DEVICE inline int att_part_end(const AttWindow& w, int s, int z, bool halves) {
+    return att_min(w.ctx_max, att_part_begin(s, z, halves) + (halves ? AT_SPLIT / 2 : AT_SPLIT));
+}
+FNX_HOST_DEVICE inline int att_part_index(int s, int z, bool halves) { return halves ? 2 * s + z : s; }
+// the parts a query's row of the scratch area has room for, and the parts that the first pass wrote with data (the second
+// pass reads these)
+FNX_HOST_DEVICE inline int att_part_slots(int nsplit) { return 2 * nsplit; }
+FNX_HOST_DEVICE inline int att_live_parts(const AttWindow& w, int nsplit, bool halves) {
+    const int len = halves ? AT_SPLIT / 2 : AT_SPLIT;
+    return att_min(halves ? 2 * nsplit : nsplit, (w.ctx_max + len - 1) / len);
+}
 // the K row and the V block (of AT_VB positions) that a fetch of chunk c0 reads for its row r (0 .. AT_CH - 1) and block b
 // (0 .. AT_CH / AT_VB - 1): clamped inside the window's rows
 FNX_HOST_DEVICE inline int att_fetch_row(const AttWindow& w, int c0, int r) { return att_min(c0 + r, w.ctx_max - 1); }
 FNX_HOST_DEVICE inline int att_fetch_vblock(const AttWindow& w, int c0, int b) { return att_min(c0 / AT_VB + b, (w.ctx_max - 1) / AT_VB); }
-// the splits whose parts the first pass wrote with data (the second pass reads these)
-FNX_HOST_DEVICE inline int att_live_splits(const AttWindow& w, int nsplit) { return att_min(nsplit, (w.ctx_max + AT_SPLIT - 1) / AT_SPLIT); }
 
 }  // namespace fnx

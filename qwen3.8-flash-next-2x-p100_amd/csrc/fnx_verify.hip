@@ -1623,7 +1623,7 @@ int fnx_attn_prep_append(float* qg, float* k, const float* v, const float* q_nor
     return attn_prep_append(qg, k, v, q_norm, k_norm, kc, vc, nq, nkv, T, pos0, max_ctx, eps, rope, st, nullptr);
 }
 // splits for a context of up to max_ctx positions
-size_t fnx_attn_scratch_floats(int nq, int T, int max_ctx) { return (size_t) T * nq * attn_splits(max_ctx) * (AT_HD + 2); }
+size_t fnx_attn_scratch_floats(int nq, int T, int max_ctx) { return (size_t) T * nq * att_part_slots(attn_splits(max_ctx)) * (AT_HD + 2); }
 static int q8s_one(const fnx_q8s* W, const void* yq, float* out, int out_stride, int T, void* st, const int* gate) {
     return q8s_launch(&W, &out, &out_stride, 1, yq, T, st, "q8s_gemv", gate);
 }
@@ -1636,12 +1636,13 @@ static int attn_launch(const float* qg, const uint16_t* kc, const uint16_t* vc, 
     if (attn_splits(max_ctx) > AT_MAXSPLIT) return fail("attn: the cache is larger than the split table");
     if (((unsigned long long) max_ctx + 3) * nkv * (AT_HD * 2) >= (1ull << 32)) return fail("attn: a cache of 4 GiB or more (the kernel's byte offsets are 32 bits)");
     // the grid covers the cache's capacity (the position is on the device): splits past the context write empty parts
+    // (two layers of blocks always: for a window whose queries fit one, the second takes the splits' second halves)
     const int nsplit = attn_splits(max_ctx), waves = (T * (nq / nkv) + 15) / 16;
     float* acc = scratch;
-    AttPart* mz = reinterpret_cast<AttPart*>(scratch + (size_t) T * nq * nsplit * AT_HD);
-    k_attn_part<<<dim3(nsplit, nkv, (waves + AT_WAVES - 1) / AT_WAVES), AT_THREADS, 0, (hipStream_t) st>>>(qg, kc, vc, acc, mz, nq, nkv, T,
-                                                                                                          nsplit, pos0, max_ctx, gate, live);
-    k_attn_combine<<<dim3(nq, T), AT_HD, 0, (hipStream_t) st>>>(qg, acc, mz, out, outq, nq, nsplit, T, pos0, max_ctx, err, gate, live);
+    AttPart* mz = reinterpret_cast<AttPart*>(scratch + (size_t) T * nq * att_part_slots(nsplit) * AT_HD);
+    k_attn_part<<<dim3(nsplit, nkv, std::max(2, (waves + AT_WAVES - 1) / AT_WAVES)), AT_THREADS, 0, (hipStream_t) st>>>(qg, kc, vc, acc, mz, nq, nkv, T,
+                                                                                                                       nsplit, pos0, max_ctx, gate, live);
+    k_attn_combine<<<dim3(nq, T), AT_HD, 0, (hipStream_t) st>>>(qg, acc, mz, out, outq, nq, nkv, nsplit, T, pos0, max_ctx, err, gate, live);
     return launch_status("attn");
 }
 int fnx_attn(const float* qg, const uint16_t* kc, const uint16_t* vc, float* out, int nq, int nkv, const int* pos0, int T, int max_ctx,

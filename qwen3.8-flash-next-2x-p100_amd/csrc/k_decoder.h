@@ -504,11 +504,16 @@ __global__ void __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu
     if (gate && uniform(*gate) == 0) return;   // a chain step that does not count: its parts stay what they were, nothing reads the result
     // live (may be null): a device word, the rows of the window that count; the others' queries are left out (nothing reads
     // their results), the positions past the last row that counts with them
-    const int s = blockIdx.x, kvh = blockIdx.y, lane = threadIdx.x & 63, wave = blockIdx.z * AT_WAVES + (threadIdx.x >> 6);
+    const int s = blockIdx.x, kvh = blockIdx.y, lane = threadIdx.x & 63;
     const bool loader = uniform((int) (threadIdx.x >> 6)) == AT_WAVES;   // the block's last wave: no queries, all the loads
     const int qpk = nq / nkv;
-    // this lane's query row, 64 of its dims: loaded before anything that waits for a device word (a lane past the window's
-    // queries reads the last query's row; its operands become zeros below)
+    if (live) T = uniform(max(1, min(*live, T)));
+    const int nquery = T * qpk;
+    // a window of few queries: the grid's second layer of blocks takes the second halves of the splits (attn_window.h)
+    const bool halves = att_halves(nquery);
+    const int wave = (halves ? 0 : blockIdx.z * AT_WAVES) + (threadIdx.x >> 6);
+    // this lane's query row, 64 of its dims: loaded before anything that waits for the window's position (a lane past the
+    // window's queries reads the last query's row; its operands become zeros below)
     float4 qa[8], qb[8];
     if (!loader) {
         const int qc = min(wave * 16 + (lane & 15), T * qpk - 1);
@@ -519,10 +524,8 @@ __global__ void __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu
             qb[ks] = *reinterpret_cast<const float4*>(qr + 8 * ks + 4);
         }
     }
-    if (live) T = uniform(max(1, min(*live, T)));
-    const int nquery = T * qpk;
     const AttWindow win = att_window(*pos0p, T, max_ctx);   // no index below leaves the cache, whatever the device word holds
-    if ((int) blockIdx.z * AT_WAVES * 16 >= nquery) return;   // none of the block's queries count
+    if (!halves && (int) blockIdx.z * AT_WAVES * 16 >= nquery) return;   // none of the block's queries count
     const bool wave_on = uniform(wave * 16 < nquery) && !loader;   // a wave without queries only meets the others
     const int ql = lane & 15, pg = lane >> 4;
     const int qi = wave * 16 + ql;                      // this lane's query (as B column / accumulator column)
@@ -530,10 +533,10 @@ __global__ void __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu
     const int qt = qlive ? qi / qpk : 0, qh = kvh * qpk + (qlive ? qi % qpk : 0);
     const int ctx_q = qlive ? att_ctx_q(win, qt) : 0;   // positions [0, ctx_q) are this query's
     const int ctx_max = win.ctx_max;                    // the window's last row sees this many
-    const int p0 = att_split_begin(s), p1 = att_split_end(win, s);
+    const int p0 = att_part_begin(s, blockIdx.z, halves), p1 = att_part_end(win, s, blockIdx.z, halves);
     const int vis = uniform(wave_on ? min(att_ctx_q(win, (wave * 16) / qpk), p1) : 0);   // the wave's first query is its earliest row's
-    const size_t slot = ((size_t) qt * nq + qh) * nsplit + s;
-    if (p0 >= p1) {   // a split past the context: an empty part
+    const size_t slot = ((size_t) qt * nq + qh) * att_part_slots(nsplit) + att_part_index(s, blockIdx.z, halves);
+    if (p0 >= p1) {   // a part past the context: empty
         if (qlive && pg == 0) mz_out[slot] = AttPart{-INFINITY, 0.f};
         return;
     }
@@ -763,12 +766,12 @@ __global__ void __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu
 }
 // a block per (head, row): the splits' weights exp(m_s - max) first (LDS), then every thread sums its dimension over the
 // splits that hold data, several loads in flight. out (f32) and outq (q8_1 rows) may each be null.
-constexpr int AT_MAXSPLIT = 2048;
+constexpr int AT_MAXSPLIT = 2048;   // splits of the largest cache; a query has twice as many parts at most
 __global__ void __launch_bounds__(AT_HD) k_attn_combine(const float* __restrict__ qg, const float* __restrict__ acc_in,
                                                        const AttPart* __restrict__ mz_in, float* __restrict__ out, uint8_t* __restrict__ outq,
-                                                       int nq, int nsplit, int T, const int* __restrict__ pos0p, int max_ctx, unsigned* __restrict__ err,
-                                                       const int* __restrict__ gate, const int* __restrict__ live) {
-    __shared__ float wsp[AT_MAXSPLIT];
+                                                       int nq, int nkv, int nsplit, int T, const int* __restrict__ pos0p, int max_ctx,
+                                                       unsigned* __restrict__ err, const int* __restrict__ gate, const int* __restrict__ live) {
+    __shared__ float wsp[2 * AT_MAXSPLIT];
     __shared__ float red[AT_HD / 64];
     if (gate && uniform(*gate) == 0) return;
     // a window that leaves the cache: reported (err may be null), and computed over the cells that exist
@@ -780,8 +783,9 @@ __global__ void __launch_bounds__(AT_HD) k_attn_combine(const float* __restrict_
         if (outq) q8_1_store(0.f, outq + (((size_t) t * nq + h) * (AT_HD / 32) + i / 32) * FNX_Q8_1_BLOCK, i & 31);
         return;
     }
-    const size_t base = ((size_t) t * nq + h) * nsplit;
-    const int nlive = att_live_splits(att_window(*pos0p, T, max_ctx), nsplit);   // splits the window's context reaches: their parts were written
+    const size_t base = ((size_t) t * nq + h) * att_part_slots(nsplit);
+    // the parts the window's context reaches: they were written (whole splits, or their halves for a window of few queries)
+    const int nlive = att_live_parts(att_window(*pos0p, T, max_ctx), nsplit, att_halves(T * (nq / nkv)));
     float mx = -INFINITY;
     for (int s = i; s < nlive; s += AT_HD) mx = fmaxf(mx, mz_in[base + s].m);
     mx = group_max<64>(mx);
