@@ -118,6 +118,7 @@ struct WinLds {
     uint32_t xq[FL_N / 32][FNX_Q8_1_BLOCK / 4];          // the row's q8_1 blocks
     float4 xf[FL_N / 4];                                 // the row of x
     __attribute__((aligned(16))) uint32_t hq[FL_MAXK + 1][SBR][HQ_WORDS];   // the row's pairs' h rows (phase D)
+    float zx[FL_MAXK + 1][WN_WAVES / 2][64 / SBR];   // a block of few units: a trip's sums of a unit's rows, from the wave that made them
 };
 
 // A wait of one wave for the sum of a word over `lines` consecutive rows' lines. False: the budget ran out (the error bit is set).
@@ -687,8 +688,12 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
     // ---------------------------------------------------------------- phase D
     const bool ext = a.sh_part != nullptr;   // the shared expert's rows come from memory: the trips are the picks only
     const int first = ext ? 1 : 0;
-    const bool dwave = wave < pl.dwaves;
-    const int R = pl.R, u0 = g * pl.upb + wave * R;   // this wave's units of every matrix
+    // A block of few units (a window of few rows, whose rows have many blocks) would leave most waves standing by while one
+    // wave a unit makes the row's trips one after the other: there the trips are dealt out as well - wave w takes unit
+    // w % dwaves and, of the row's trips, every TG-th from trip w / dwaves on; the sums meet in LDS and the units' first
+    // waves run the combine's chain over them in the picks' order (the same operations on the same values).
+    // (Only where a wave has one unit: the other forms of the phase are compiled without it.)
+    const int R = pl.R;
     const int kb = lane % SBR, gl = lane / SBR;
     // trip 0 is the shared expert's, trips 1 .. topk the picks in order
     auto down_matrix = [&](int trip) -> const uint8_t* {
@@ -702,6 +707,12 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
     // waits for its own trip's weights only - not, as with loads under "if (r < R)", for everything in flight.
     auto down_phase = [&](auto RC) -> bool {
     constexpr int RR = decltype(RC)::value;
+    int TG = 1;
+    if constexpr (RR == 1) TG = pl.dwaves <= WN_WAVES / 2 && WN_WAVES % pl.dwaves == 0 ? WN_WAVES / pl.dwaves : 1;
+    const bool dwave = TG > 1 || wave < pl.dwaves;
+    const int tgrp = TG > 1 ? wave / pl.dwaves : 0, uw = TG > 1 ? wave - tgrp * pl.dwaves : wave;
+    const int u0 = g * pl.upb + uw * RR;   // this wave's units of every matrix
+    auto trip_of = [&](int i) { return first + tgrp + i * TG; };   // the wave's i-th trip
     PackedSub B[NB][RR];
     auto issue_trip = [&](PackedSub(&buf)[RR], int trip) {
         const __amdgpu_buffer_rsrc_t mtx = matrix_rsrc(down_matrix(trip));
@@ -767,7 +778,7 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
     auto first_trips = [&] {
 #pragma unroll
         for (int i = 0; i < NB; ++i)
-            if (first + i <= topk) issue_trip(B[i], first + i);
+            if (trip_of(i) <= topk) issue_trip(B[i], trip_of(i));
     };
     if (dwave && wave != 0) first_trips();
     if (wave == 0) {
@@ -801,6 +812,27 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
 #pragma unroll
         for (int r = 0; r < RR; ++r) acc[r] = zs[r] = 0.f;
         const float gate = S.gate;
+        // a trip's sums of this wave's units' rows (every lane of a row's group holds the row's)
+        auto trip_rows = [&](const PackedSub(&buf)[RR], int trip, auto after_h, auto sink) {
+            const int k = pick_of(trip);
+            const uint32_t* hb = S.hq[k][kb];
+            const uint4 lo = *reinterpret_cast<const uint4*>(hb), hi = *reinterpret_cast<const uint4*>(hb + 4);
+            const int hx[8] = {(int) lo.x, (int) lo.y, (int) lo.z, (int) lo.w, (int) hi.x, (int) hi.y, (int) hi.z, (int) hi.w};
+            const float dh = __uint_as_float(hb[8]);
+            after_h();
+#pragma unroll
+            for (int r = 0; r < RR; ++r) {
+                int w4[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) w4[j] = *reinterpret_cast<const int*>(reinterpret_cast<const uint8_t*>(S.tab) + packed_addr(buf[r].idx, j));
+                const int sc = 1 + 2 * (int) ((buf[r].sc >> sc_shift) & 0xFu);
+                const float dw = half_bits_to_float(buf[r].d);
+                int sum = 0;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) sum = __builtin_amdgcn_sdot4(w4[j], hx[j], sum, false);
+                sink(r, butterfly_sum<SBR>((dw * dh) * (float) __mul24(sum, sc)));
+            }
+        };
         auto decode_trip = [&](const PackedSub(&buf)[RR], int trip) {
             switch ((wave >> 2) + trip & 3) {   // every wave takes each of the four priorities in turn (see the sweeps)
                 case 0: __builtin_amdgcn_s_setprio(0); break;
@@ -808,27 +840,44 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
                 case 2: __builtin_amdgcn_s_setprio(2); break;
                 default: __builtin_amdgcn_s_setprio(3); break;
             }
-            const int k = pick_of(trip);
-            const uint32_t* hb = S.hq[k][kb];
-            const uint4 lo = *reinterpret_cast<const uint4*>(hb), hi = *reinterpret_cast<const uint4*>(hb + 4);
-            const int hx[8] = {(int) lo.x, (int) lo.y, (int) lo.z, (int) lo.w, (int) hi.x, (int) hi.y, (int) hi.z, (int) hi.w};
-            const float dh = __uint_as_float(hb[8]);
-            const float gk = trip == 0 ? gate : S.pw[trip - 1];
-#pragma unroll
-            for (int r = 0; r < RR; ++r) {
-                    int w4[8];
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) w4[j] = *reinterpret_cast<const int*>(reinterpret_cast<const uint8_t*>(S.tab) + packed_addr(buf[r].idx, j));
-                    const int sc = 1 + 2 * (int) ((buf[r].sc >> sc_shift) & 0xFu);
-                    const float dw = half_bits_to_float(buf[r].d);
-                    int sum = 0;
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) sum = __builtin_amdgcn_sdot4(w4[j], hx[j], sum, false);
-                    const float z = butterfly_sum<SBR>((dw * dh) * (float) __mul24(sum, sc));
+            float gk;
+            trip_rows(
+                buf, trip, [&] { gk = trip == 0 ? gate : S.pw[trip - 1]; },
+                [&](int r, float z) {
                     if (trip == 0) zs[r] = gk * z;
                     else acc[r] = fmaf(gk, z, acc[r]);
-                }
+                });
         };
+        if constexpr (RR == 1) {
+            if (TG > 1) {   // (the same for the whole block)
+                constexpr int MAXI = (FL_MAXK + 2) / 2;   // trips a wave at most (TG >= 2)
+#pragma unroll
+                for (int i = 0; i < MAXI; ++i) {
+                    const int trip = trip_of(i);
+                    if (trip <= topk) {
+                        trip_rows(
+                            B[i % NB], trip, [] {},
+                            [&](int, float z) {
+                                if (kb == SBR - 1) S.zx[trip][uw][gl] = z;
+                            });
+                        if (trip_of(i + NB) <= topk) issue_trip(B[i % NB], trip_of(i + NB));
+                    }
+                }
+                win_meet();
+                if (tgrp == 0 && kb == SBR - 1) {
+                    float s = 0.f, shared = 0.f;
+                    for (int trip = first; trip <= topk; ++trip) {
+                        const float zt = S.zx[trip][uw][gl], gk = trip == 0 ? gate : S.pw[trip - 1];
+                        if (trip == 0) shared = gk * zt;
+                        else s = fmaf(gk, zt, s);
+                    }
+                    if (ext) shared = gate * a.sh_part[(size_t) t * a.rows + (size_t) u0 * RW + gl];
+                    __hip_atomic_store(reinterpret_cast<unsigned*>(a.out + (size_t) t * a.rows + (size_t) u0 * RW + gl), __float_as_uint(s + shared), __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+                }
+                return true;
+            }
+        }
         // A trip's loads go to the buffer that held trip nx - NB, decoded before this one. The rounds in which every trip exists
         // and so does the one it asks for come first, without a condition on a load (see above); the last trips follow with them.
         int trip = first;
