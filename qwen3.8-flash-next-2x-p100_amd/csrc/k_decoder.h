@@ -501,13 +501,15 @@ __global__ void __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu
                                                             AttPart* __restrict__ mz_out, int nq, int nkv, int T, int nsplit,
                                                             const int* __restrict__ pos0p, int max_ctx, const int* __restrict__ gate,
                                                             const int* __restrict__ live) {
-    if (gate && uniform(*gate) == 0) return;   // a chain step that does not count: its parts stay what they were, nothing reads the result
+    // the launch's device words, asked for together (one after the other, each would be a trip to memory of its own)
+    const int gate_v = gate ? *gate : 1, live_v = live ? *live : T, pos0_v = *pos0p;
+    if (uniform(gate_v) == 0) return;   // a chain step that does not count: its parts stay what they were, nothing reads the result
     // live (may be null): a device word, the rows of the window that count; the others' queries are left out (nothing reads
     // their results), the positions past the last row that counts with them
     const int s = blockIdx.x, kvh = blockIdx.y, lane = threadIdx.x & 63;
     const bool loader = uniform((int) (threadIdx.x >> 6)) == AT_WAVES;   // the block's last wave: no queries, all the loads
     const int qpk = nq / nkv;
-    if (live) T = uniform(max(1, min(*live, T)));
+    T = uniform(max(1, min(live_v, T)));
     const int nquery = T * qpk;
     // a window of few queries: the grid's second layer of blocks takes the second halves of the splits (attn_window.h)
     const bool halves = att_halves(nquery);
@@ -524,7 +526,7 @@ __global__ void __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu
             qb[ks] = *reinterpret_cast<const float4*>(qr + 8 * ks + 4);
         }
     }
-    const AttWindow win = att_window(*pos0p, T, max_ctx);   // no index below leaves the cache, whatever the device word holds
+    const AttWindow win = att_window(uniform(pos0_v), T, max_ctx);   // no index below leaves the cache, whatever the device word holds
     if (!halves && (int) blockIdx.z * AT_WAVES * 16 >= nquery) return;   // none of the block's queries count
     const bool wave_on = uniform(wave * 16 < nquery) && !loader;   // a wave without queries only meets the others
     const int ql = lane & 15, pg = lane >> 4;
@@ -773,10 +775,11 @@ __global__ void __launch_bounds__(AT_HD) k_attn_combine(const float* __restrict_
                                                        unsigned* __restrict__ err, const int* __restrict__ gate, const int* __restrict__ live) {
     __shared__ float wsp[2 * AT_MAXSPLIT];
     __shared__ float red[AT_HD / 64];
-    if (gate && uniform(*gate) == 0) return;
+    const int gate_v = gate ? *gate : 1, live_v = live ? *live : T, pos0_v = uniform(*pos0p);   // (asked for together)
+    if (uniform(gate_v) == 0) return;
     // a window that leaves the cache: reported (err may be null), and computed over the cells that exist
-    if (err && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0 && !att_window_fits(*pos0p, T, max_ctx)) atomicOr(err, FNX_ERR_WINDOW);
-    if (live) T = uniform(max(1, min(*live, T)));
+    if (err && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0 && !att_window_fits(pos0_v, T, max_ctx)) atomicOr(err, FNX_ERR_WINDOW);
+    T = uniform(max(1, min(live_v, T)));
     const int h = blockIdx.x, t = blockIdx.y, i = threadIdx.x;
     if (t >= T) {   // a row that does not count: zeros (its queries were left out; what follows it stays finite)
         if (out) out[((size_t) t * nq + h) * AT_HD + i] = 0.f;
@@ -785,7 +788,7 @@ __global__ void __launch_bounds__(AT_HD) k_attn_combine(const float* __restrict_
     }
     const size_t base = ((size_t) t * nq + h) * att_part_slots(nsplit);
     // the parts the window's context reaches: they were written (whole splits, or their halves for a window of few queries)
-    const int nlive = att_live_parts(att_window(*pos0p, T, max_ctx), nsplit, att_halves(T * (nq / nkv)));
+    const int nlive = att_live_parts(att_window(pos0_v, T, max_ctx), nsplit, att_halves(T * (nq / nkv)));
     float mx = -INFINITY;
     for (int s = i; s < nlive; s += AT_HD) mx = fmaxf(mx, mz_in[base + s].m);
     mx = group_max<64>(mx);
@@ -807,6 +810,23 @@ __global__ void __launch_bounds__(AT_HD) k_attn_combine(const float* __restrict_
     float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
     const float* ap = acc_in + base * AT_HD + i;
     int s = 0;
+    // A window of few rows has few blocks here, each with twice the parts: its time is the round trips of a thread's loads one
+    // batch after the other, so thirty-two are asked for at once (the chains take them in the same order; with a block a
+    // (head, row) of a full window, whose parts' 17 MB are the time, that was slower than four).
+    if (T * nq <= 128) {
+        for (; s + 32 <= nlive; s += 32) {
+            float v[32];
+#pragma unroll
+            for (int j = 0; j < 32; ++j) v[j] = ap[(size_t) (s + j) * AT_HD];
+#pragma unroll
+            for (int j = 0; j < 32; j += 4) {
+                a0 = fmaf(wsp[s + j], v[j], a0);
+                a1 = fmaf(wsp[s + j + 1], v[j + 1], a1);
+                a2 = fmaf(wsp[s + j + 2], v[j + 2], a2);
+                a3 = fmaf(wsp[s + j + 3], v[j + 3], a3);
+            }
+        }
+    }
     for (; s + 4 <= nlive; s += 4) {
         a0 = fmaf(wsp[s], ap[(size_t) s * AT_HD], a0);
         a1 = fmaf(wsp[s + 1], ap[(size_t) (s + 1) * AT_HD], a1);
