@@ -1538,10 +1538,14 @@ int fnx_embed_rows(const uint16_t* emb, const int* tokens, int T, int vocab, int
     k_embed_rows<<<T, 256, 0, (hipStream_t) st>>>(emb, tokens, vocab, n, y);
     return launch_status("embed_rows");
 }
+// (the forms of the kernel for a launch with a device-side row count: defined at the end of this file)
+static bool q8s_live_lds(int bytes);
+static void q8s_live_launch(bool tiled, int grid, size_t lds, hipStream_t st, const Q8sArgs& a);
 // yq2 (may be null): two matrices, the second one over rows of its own - as long as every block has one tile, which is then of
 // one matrix (else refused: the caller launches twice)
+// live (may be null): a device word, the rows that count; the others are not read and their products are zeros
 static int q8s_launch(const fnx_q8s* const* W, float* const* out, const int* out_stride, int n, const void* yq, int T, void* st, const char* who,
-                      const int* gate = nullptr, const void* yq2 = nullptr) {
+                      const int* gate = nullptr, const void* yq2 = nullptr, const int* live = nullptr) {
     if (!W || !out || !out_stride || !yq || n < 1 || n > 3) return fail(std::string(who) + ": null argument");
     Q8sArgs a{};
     long tiles = 0;
@@ -1567,18 +1571,21 @@ static int q8s_launch(const fnx_q8s* const* W, float* const* out, const int* out
     int dev = 0;
     if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64 && !attr_set[dev]) {
         if (hipFuncSetAttribute((const void*) k_q8s_gemv<1>, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024) != hipSuccess ||
-            hipFuncSetAttribute((const void*) k_q8s_gemv<1, true>, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024) != hipSuccess)
+            hipFuncSetAttribute((const void*) k_q8s_gemv<1, true>, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024) != hipSuccess ||
+            !q8s_live_lds(150 * 1024))
             return fail(std::string(who) + ": cannot raise the dynamic LDS limit");
         attr_set[dev] = true;
     }
     static const int per_cu = env_int("FNX_Q8S_BLOCKS_PER_CU", 4, 1, 16);   // what the LDS of a 2048-column matrix lets a CU hold
     const int grid = (int) std::max(1l, std::min<long>((long) per_cu * cu_count(), tiles));
     a.gate = gate;
+    a.live = live;
     if (yq2) {
         if (n != 2 || grid < tiles) return fail(std::string(who) + ": two sets of rows want two matrices and a block a tile");
         a.yq2 = (const uint8_t*) yq2;
     }
-    if (W[0]->tiled) k_q8s_gemv<1, true><<<grid, Q8S_WAVES * 64, lds, (hipStream_t) st>>>(a);
+    if (live) q8s_live_launch(W[0]->tiled != 0, grid, lds, (hipStream_t) st, a);
+    else if (W[0]->tiled) k_q8s_gemv<1, true><<<grid, Q8S_WAVES * 64, lds, (hipStream_t) st>>>(a);
     else k_q8s_gemv<1><<<grid, Q8S_WAVES * 64, lds, (hipStream_t) st>>>(a);
     return launch_status(who);
 }
@@ -1624,8 +1631,8 @@ int fnx_attn_prep_append(float* qg, float* k, const float* v, const float* q_nor
 }
 // splits for a context of up to max_ctx positions
 size_t fnx_attn_scratch_floats(int nq, int T, int max_ctx) { return (size_t) T * nq * att_part_slots(attn_splits(max_ctx)) * (AT_HD + 2); }
-static int q8s_one(const fnx_q8s* W, const void* yq, float* out, int out_stride, int T, void* st, const int* gate) {
-    return q8s_launch(&W, &out, &out_stride, 1, yq, T, st, "q8s_gemv", gate);
+static int q8s_one(const fnx_q8s* W, const void* yq, float* out, int out_stride, int T, void* st, const int* gate, const int* live = nullptr) {
+    return q8s_launch(&W, &out, &out_stride, 1, yq, T, st, "q8s_gemv", gate, nullptr, live);
 }
 static int attn_launch(const float* qg, const uint16_t* kc, const uint16_t* vc, float* out, uint8_t* outq, int nq, int nkv, const int* pos0, int T,
                        int max_ctx, float* scratch, void* st, const int* gate = nullptr, const int* live = nullptr, unsigned* err = nullptr) {
@@ -1699,13 +1706,13 @@ static int dec_layer(const fnx_decoder* D, const fnx_dec_layer* L, int T, const 
         const fnx_q8s* w3[3] = {&L->wq, &L->wk, &L->wv};
         float* const o3[3] = {ws->qg, ws->k, ws->v};
         const int s3[3] = {nq * 2 * AT_HD, nkv * AT_HD, nkv * AT_HD};
-        if (q8s_launch(w3, o3, s3, 3, ws->xq, T, st, "q8s_gemv_segs", gate)) return 1;
+        if (q8s_launch(w3, o3, s3, 3, ws->xq, T, st, "q8s_gemv_segs", gate, nullptr, live)) return 1;
     }
     if (attn_prep_append(ws->qg, ws->k, ws->v, L->q_norm, L->k_norm, L->kc, L->vc, nq, nkv, T, pos0, D->max_ctx, D->eps, &D->rope, st, gate)) return 1;
     // the attention's rows leave its last kernel in q8_1 form, ready for the output projection
     if (attn_launch(ws->qg, L->kc, L->vc, nullptr, (uint8_t*) ws->xq, nq, nkv, pos0, T, D->max_ctx, ws->attn_scratch, st, gate, live, (unsigned*) ws->err))
         return 1;
-    if (q8s_one(&L->wo, ws->xq, ws->o, n, T, st, gate)) return 1;
+    if (q8s_one(&L->wo, ws->xq, ws->o, n, T, st, gate, live)) return 1;
     if (live && !layer_fused_ok(&L->moe, T)) return fail("decoder: a device-side row count needs the one-launch window (unit64 experts, hidden 2048)");
     if (next_w && layer_fused_ok(&L->moe, T) && !shared_is_q8(&L->moe)) {
         // The one-launch window takes the passes either side of it: every block makes its row's x + o and the norm for itself,
@@ -1740,10 +1747,11 @@ static int dec_shape_check(const fnx_decoder* D, int T, const char* who) {
 // x += pending; hidden = x; the output norm, the head, argmax
 // nv head rows for the tokens from v0; pen (may be null): the last row's penalty list, applied before the picks (engine.cu:2130-2131)
 static int dec_head(const fnx_decoder* D, const float* norm, const fnx_q8s* head, int T, const fnx_dec_ws* ws, const DecPending& pend, void* st,
-                    const int* gate = nullptr, int nv = 0, int v0 = 0, const int* pen = nullptr, const float* pen_par = nullptr) {
+                    const int* gate = nullptr, int nv = 0, int v0 = 0, const int* pen = nullptr, const float* pen_par = nullptr,
+                    const int* live = nullptr) {
     if (nv == 0) nv = D->vocab;
     if (dec_add_norm_q8(D, pend, norm, T, ws, st, ws->hidden, gate)) return 1;   // hidden = x, written by the same pass
-    if (q8s_one(head, ws->xq, ws->logits, nv, T, st, gate)) return 1;
+    if (q8s_one(head, ws->xq, ws->logits, nv, T, st, gate, live)) return 1;
     if (pen && fnx_penalize_row(ws->logits + (size_t) (T - 1) * nv, nv, pen, pen_par, st)) return 1;
     return fnx_argmax(ws->logits, nv, T, v0, ws->best_v, ws->best_i, ws->keys, ws->err, st);
 }
@@ -1756,7 +1764,7 @@ static int decoder_verify(const fnx_decoder* D, const int* tokens, int T, const 
         if (dec_layer(D, &D->layers[l], T, pos0, ws, pend, st, live, nullptr, last ? D->out_norm : D->layers[l + 1].attn_norm, last ? ws->hidden : nullptr))
             return 1;
     }
-    return dec_head(D, D->out_norm, &D->head, T, ws, pend, st);
+    return dec_head(D, D->out_norm, &D->head, T, ws, pend, st, nullptr, 0, 0, nullptr, nullptr, live);
 }
 int fnx_decoder_verify(const fnx_decoder* D, const int* tokens, int T, const int* pos0, const fnx_dec_ws* ws, void* st) {
     return decoder_verify(D, tokens, T, pos0, ws, st, nullptr);
@@ -1801,10 +1809,10 @@ static int mtp_draft(const fnx_decoder* D, const fnx_mtp* M, const float* src, c
             const fnx_q8s* W2[2] = {&M->fc_hid, &M->fc_emb};
             float* out2[2] = {ws->x, ws->o};
             const int stride2[2] = {n, n};
-            if (q8s_launch(W2, out2, stride2, 2, ws->xq, T, st, "q8s_gemv", gate, xq2)) return 1;
+            if (q8s_launch(W2, out2, stride2, 2, ws->xq, T, st, "q8s_gemv", gate, xq2, live)) return 1;
         } else {
-            if (q8s_one(&M->fc_hid, ws->xq, ws->x, n, T, st, gate)) return 1;
-            if (q8s_one(&M->fc_emb, xq2, ws->o, n, T, st, gate)) return 1;
+            if (q8s_one(&M->fc_hid, ws->xq, ws->x, n, T, st, gate, live)) return 1;
+            if (q8s_one(&M->fc_emb, xq2, ws->o, n, T, st, gate, live)) return 1;
         }
     } else {
         {   // nothing to add: src is only read (fnx_add_norm_q8)
@@ -1813,7 +1821,7 @@ static int mtp_draft(const fnx_decoder* D, const fnx_mtp* M, const float* src, c
             k_add_norm_q8<false><<<T, 256, 0, (hipStream_t) st>>>(const_cast<float*>(src), nullptr, c, M->norm_hid, nullptr, (uint8_t*) ws->xq, n, D->eps);
             if (launch_status("mtp_draft")) return 1;
         }
-        if (q8s_one(&M->fc_hid, ws->xq, ws->x, n, T, st, gate)) return 1;
+        if (q8s_one(&M->fc_hid, ws->xq, ws->x, n, T, st, gate, live)) return 1;
         {   // the tokens' embedding rows (rms(emb[tokens]))
             CombineArgs c{};
             c.emb = D->emb;
@@ -1823,11 +1831,11 @@ static int mtp_draft(const fnx_decoder* D, const fnx_mtp* M, const float* src, c
             k_add_norm_q8<false><<<T, 256, 0, (hipStream_t) st>>>(ws->xn, nullptr, c, M->norm_emb, nullptr, (uint8_t*) ws->xq, n, D->eps);
             if (launch_status("mtp_draft")) return 1;
         }
-        if (q8s_one(&M->fc_emb, ws->xq, ws->o, n, T, st, gate)) return 1;
+        if (q8s_one(&M->fc_emb, ws->xq, ws->o, n, T, st, gate, live)) return 1;
     }
     DecPending pend{ws->o, nullptr, nullptr};
     if (dec_layer(D, &M->layer, T, pos0, ws, pend, st, live, gate, M->out_norm, ws->hidden)) return 1;
-    return dec_head(D, M->out_norm, &M->head, T, ws, pend, st, gate, nv, M->dv0, M->pen, M->pen_par);
+    return dec_head(D, M->out_norm, &M->head, T, ws, pend, st, gate, nv, M->dv0, M->pen, M->pen_par, live);
 }
 int fnx_mtp_draft(const fnx_decoder* D, const fnx_mtp* M, const float* src, const int* tokens, int T, const int* pos0, const fnx_dec_ws* ws,
                   void* st) {
@@ -2224,3 +2232,14 @@ int fnx_gguf_load_moe_layer(const fnx_gguf* g, int layer, int ff0, int ff1, int 
 }
 
 }  // extern "C"
+
+// The dense mat-vec's forms for a launch with a device-side row count (k_q8s_gemv<.., LIVE = true>), asked for here, after
+// everything else, so that the kernels before them lie in the code object where they lay without them.
+static bool q8s_live_lds(int bytes) {
+    return hipFuncSetAttribute((const void*) fnx::k_q8s_gemv<1, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) == hipSuccess &&
+           hipFuncSetAttribute((const void*) fnx::k_q8s_gemv<1, true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) == hipSuccess;
+}
+static void q8s_live_launch(bool tiled, int grid, size_t lds, hipStream_t st, const fnx::Q8sArgs& a) {
+    if (tiled) fnx::k_q8s_gemv<1, true, true><<<grid, fnx::Q8S_WAVES * 64, lds, st>>>(a);
+    else fnx::k_q8s_gemv<1, false, true><<<grid, fnx::Q8S_WAVES * 64, lds, st>>>(a);
+}

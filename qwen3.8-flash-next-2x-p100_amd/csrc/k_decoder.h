@@ -226,6 +226,7 @@ struct Q8sArgs {
     const uint8_t* yq;   // q8_1 rows
     const int* gate;     // may be null; else a device word: at zero the launch leaves at once (a chain step that does not count)
     const uint8_t* yq2;  // may be null; else the second matrix's rows are these (two matrices, a block a tile: the host sees to that)
+    const int* live;     // may be null; else a device word: rows from *live on do not count - they are not read and their products are zeros
 };
 typedef int q8s_v4i __attribute__((ext_vector_type(4)));
 // DEPTH: the (tile, batch) items whose loads are in flight ahead of the one being worked on. (With 3 - all of a tile's
@@ -234,7 +235,9 @@ typedef int q8s_v4i __attribute__((ext_vector_type(4)));
 // TILED: the int8 values in the tile-major layout of k_q8s_tile below (every matrix of the launch): a wave's load is then
 // 1 KiB in a row - eight whole cache lines instead of half a line of each of sixteen rows - and takes the streaming policy
 // (read once). 4.7 against 4.1 TB/s for the output head; with the policy alone, over rows, 3.9.
-template <int DEPTH, bool TILED = false>
+// LIVE: a.live is set (a launch of its own: the word is then read on every path, through the scalar unit, and waiting for it
+// does not wait for the weights on their way).
+template <int DEPTH, bool TILED = false, bool LIVE = false>
 __global__ void __launch_bounds__(Q8S_WAVES * 64) k_q8s_gemv(const Q8sArgs a) {
     typedef __attribute__((address_space(1))) const at_v4u_t g128;
     extern __shared__ __align__(16) uint8_t q8s_lds[];   // [16][cols + pad] int8, [16][nb + 2] f32 scales, [3][64][4] partial sums
@@ -361,10 +364,12 @@ __global__ void __launch_bounds__(Q8S_WAVES * 64) k_q8s_gemv(const Q8sArgs a) {
     // the window's q8_1 rows into LDS (the first weights are on their way meanwhile). The copy takes 3 us (6-7 us in a
     // launch of 1,024 blocks, beside their weight loads) whatever the width of its loads - nine 16-byte loads for four
     // blocks of a row were no faster than 4-byte ones - and wherever in the rows a block starts.
+    int Tl = T;   // (a window of a decode round: most of its sixteen rows do not count)
+    if constexpr (LIVE) Tl = max(1, min(*a.live, T));
     for (int i = threadIdx.x; i < FNX_MAXT * nb; i += blockDim.x) {
         const int t = i / nb, b = i - t * nb;
         uint32_t* dst = reinterpret_cast<uint32_t*>(xs + (size_t) t * xld + 32 * b);
-        if (t < T) {
+        if (t < Tl) {
             const uint8_t* blk = (a.yq2 && (int) blockIdx.x >= t0 ? a.yq2 : a.yq) + (size_t) i * 36;
             xd[t * dld + b] = half_bits_to_float(load_u16(blk));
             const uint32_t* src = reinterpret_cast<const uint32_t*>(blk + 4);
