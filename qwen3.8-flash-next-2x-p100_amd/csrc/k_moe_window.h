@@ -953,6 +953,16 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
     for (int i = tid; i < nexp; i += WN_THREADS) __hip_atomic_store(&lx[i], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (DEC && a.next_x) win_next_row(a, t, true, reinterpret_cast<float*>(&S.hgu[0][0]));
     const int fin = S.fin;
+    // (A decoder's layer has no caller for the job lists - nothing reads them - and a window of few rows would end with them:
+    // there the count of ranked rows is put back by the last row to finish, by when every row has counted itself.)
+    if (DEC && a.next_x) {
+        if (fin == Tl - 1 && tid == 0) {
+            __hip_atomic_store(&a.sync[WS_ROUTED], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&a.sync[WS_FIN], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        WIN_TS(12);
+        return;
+    }
     if (fin == 0) {   // every row has been ranked long ago; the count says so
         if (wave == 0) {
             const bool ok = win_wait_word(&a.sync[WS_ROUTED], (unsigned) Tl, a.wait_ticks, serr);
