@@ -555,9 +555,12 @@ constexpr int AM_THREADS = 1024, AM_PER_BLOCK = 16384;
 // to arrive (a count beside the keys, keys[FNX_MAXT + t]) decodes the key into (value, index + v0) and leaves both words
 // at zero for the next argmax.
 __global__ void __launch_bounds__(AM_THREADS) k_argmax(const float* __restrict__ logits, int rows, unsigned long long* __restrict__ keys,
-                                                      unsigned* __restrict__ err, int v0, float* __restrict__ bv, int* __restrict__ bi) {
+                                                      unsigned* __restrict__ err, int v0, float* __restrict__ bv, int* __restrict__ bi,
+                                                      const int* __restrict__ live) {
     __shared__ unsigned long long wbest[AM_THREADS / 64];
     __shared__ int wbad;
+    // live (may be null): a device word; rows from *live on do not count: they are not scanned and their picks stay what they were
+    if (live && (int) blockIdx.y >= max(1, *live)) return;
     const int t = blockIdx.y, i0 = blockIdx.x * AM_PER_BLOCK, i1 = min(rows, i0 + AM_PER_BLOCK), tid = threadIdx.x;
     const float* r = logits + (size_t) t * rows;
     if (tid == 0) wbad = 0;
@@ -1134,11 +1137,15 @@ int fnx_moe_combine(const float* part, const float* topw, const float* sh, const
     return launch_status("moe_combine");
 }
 
-int fnx_argmax(const float* logits, int rows, int T, int v0, float* best_v, int* best_i, unsigned long long* keys, unsigned* err, void* st) {
+static int argmax_launch(const float* logits, int rows, int T, int v0, float* best_v, int* best_i, unsigned long long* keys, unsigned* err, void* st,
+                         const int* live) {
     if (!logits || !best_v || !best_i || !keys || !err) return fail("argmax: null argument");
     if (rows < 1 || T < 1 || T > FNX_MAXT) return fail("argmax: bad shape");
-    k_argmax<<<dim3((rows + AM_PER_BLOCK - 1) / AM_PER_BLOCK, T), AM_THREADS, 0, (hipStream_t) st>>>(logits, rows, keys, err, v0, best_v, best_i);
+    k_argmax<<<dim3((rows + AM_PER_BLOCK - 1) / AM_PER_BLOCK, T), AM_THREADS, 0, (hipStream_t) st>>>(logits, rows, keys, err, v0, best_v, best_i, live);
     return launch_status("argmax");
+}
+int fnx_argmax(const float* logits, int rows, int T, int v0, float* best_v, int* best_i, unsigned long long* keys, unsigned* err, void* st) {
+    return argmax_launch(logits, rows, T, v0, best_v, best_i, keys, err, st, nullptr);
 }
 
 int fnx_lookup_drafts(const int* ctx, int n_ctx, int key_n, int lk, int d1, int* out, int* match) {
@@ -1753,7 +1760,7 @@ static int dec_head(const fnx_decoder* D, const float* norm, const fnx_q8s* head
     if (dec_add_norm_q8(D, pend, norm, T, ws, st, ws->hidden, gate)) return 1;   // hidden = x, written by the same pass
     if (q8s_one(head, ws->xq, ws->logits, nv, T, st, gate, live)) return 1;
     if (pen && fnx_penalize_row(ws->logits + (size_t) (T - 1) * nv, nv, pen, pen_par, st)) return 1;
-    return fnx_argmax(ws->logits, nv, T, v0, ws->best_v, ws->best_i, ws->keys, ws->err, st);
+    return argmax_launch(ws->logits, nv, T, v0, ws->best_v, ws->best_i, ws->keys, ws->err, st, live);
 }
 static int decoder_verify(const fnx_decoder* D, const int* tokens, int T, const int* pos0, const fnx_dec_ws* ws, void* st, const int* live) {
     if (!D || !tokens || !pos0 || !ws || !D->layers || !D->out_norm || !D->emb) return fail("decoder_verify: null argument");
