@@ -950,7 +950,8 @@ __global__ void __launch_bounds__(WN_THREADS) k_moe_window(const WindowArgs a) {
     if (!S.last) return;
     // the row is complete (every block of it waited for its stores before it counted itself done); its logits' words, which
     // every block of the row has long read, go back to "not written"
-    for (int i = tid; i < nexp; i += WN_THREADS) __hip_atomic_store(&lx[i], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // (by the block's upper half: the lower one's first waves make the row's pass below, whose loads would wait behind these stores)
+    for (int i = tid - WN_THREADS / 2; i >= 0 && i < nexp; i += WN_THREADS / 2) __hip_atomic_store(&lx[i], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (DEC && a.next_x) win_next_row(a, t, true, reinterpret_cast<float*>(&S.hgu[0][0]));
     const int fin = S.fin;
     // (A decoder's layer has no caller for the job lists - nothing reads them - and a window of few rows would end with them:
