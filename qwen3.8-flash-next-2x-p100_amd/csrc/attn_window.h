@@ -46,6 +46,9 @@ FNX_HOST_DEVICE inline int att_part_index(int s, int z, bool halves) { return ha
 // the parts a query's row of the scratch area has room for, and the parts that the first pass wrote with data (the second
 // pass reads these)
 FNX_HOST_DEVICE inline int att_part_slots(int nsplit) { return 2 * nsplit; }
+// the parts between one query's first and the next one's in the scratch area: a full window's lie as closely as they did
+// without the halves (the window's mode is the same for both passes: they read the same device words)
+FNX_HOST_DEVICE inline int att_part_stride(int nsplit, bool halves) { return halves ? 2 * nsplit : nsplit; }
 FNX_HOST_DEVICE inline int att_live_parts(const AttWindow& w, int nsplit, bool halves) {
     const int len = halves ? AT_SPLIT / 2 : AT_SPLIT;
     return att_min(halves ? 2 * nsplit : nsplit, (w.ctx_max + len - 1) / len);

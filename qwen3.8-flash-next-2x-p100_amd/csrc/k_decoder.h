@@ -542,7 +542,7 @@ __global__ void __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu
     const int ctx_max = win.ctx_max;                    // the window's last row sees this many
     const int p0 = att_part_begin(s, blockIdx.z, halves), p1 = att_part_end(win, s, blockIdx.z, halves);
     const int vis = uniform(wave_on ? min(att_ctx_q(win, (wave * 16) / qpk), p1) : 0);   // the wave's first query is its earliest row's
-    const size_t slot = ((size_t) qt * nq + qh) * att_part_slots(nsplit) + att_part_index(s, blockIdx.z, halves);
+    const size_t slot = ((size_t) qt * nq + qh) * att_part_stride(nsplit, halves) + att_part_index(s, blockIdx.z, halves);
     if (p0 >= p1) {   // a part past the context: empty
         if (qlive && pg == 0) mz_out[slot] = AttPart{-INFINITY, 0.f};
         return;
@@ -791,9 +791,10 @@ __global__ void __launch_bounds__(AT_HD) k_attn_combine(const float* __restrict_
         if (outq) q8_1_store(0.f, outq + (((size_t) t * nq + h) * (AT_HD / 32) + i / 32) * FNX_Q8_1_BLOCK, i & 31);
         return;
     }
-    const size_t base = ((size_t) t * nq + h) * att_part_slots(nsplit);
+    const bool halves = att_halves(T * (nq / nkv));
+    const size_t base = ((size_t) t * nq + h) * att_part_stride(nsplit, halves);
     // the parts the window's context reaches: they were written (whole splits, or their halves for a window of few queries)
-    const int nlive = att_live_parts(att_window(pos0_v, T, max_ctx), nsplit, att_halves(T * (nq / nkv)));
+    const int nlive = att_live_parts(att_window(pos0_v, T, max_ctx), nsplit, halves);
     float mx = -INFINITY;
     for (int s = i; s < nlive; s += AT_HD) mx = fmaxf(mx, mz_in[base + s].m);
     mx = group_max<64>(mx);
@@ -832,6 +833,7 @@ __global__ void __launch_bounds__(AT_HD) k_attn_combine(const float* __restrict_
             }
         }
     }
+#pragma unroll 4
     for (; s + 4 <= nlive; s += 4) {
         a0 = fmaf(wsp[s], ap[(size_t) s * AT_HD], a0);
         a1 = fmaf(wsp[s + 1], ap[(size_t) (s + 1) * AT_HD], a1);

@@ -43,7 +43,8 @@ int main() {
                         for (int z = 0; z < (halves ? 2 : 1); ++z) {
                             const int p0 = att_part_begin(s, z, halves != 0), p1 = att_part_end(w, s, z, halves != 0);
                             const int idx = att_part_index(s, z, halves != 0);
-                            require(idx == seen && idx < att_part_slots(nsplit), "parts are numbered in position order", max_ctx, pos0, T, s, z);
+                            require(idx == seen && idx < att_part_stride(nsplit, halves != 0) && att_part_stride(nsplit, halves != 0) <= att_part_slots(nsplit),
+                                    "parts are numbered in position order, inside a query's stride", max_ctx, pos0, T, s, z);
                             ++seen;
                             if (p0 >= p1) {
                                 require(idx >= live, "an empty part is not a live one", max_ctx, pos0, T, s, z);
