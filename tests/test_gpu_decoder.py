@@ -122,7 +122,10 @@ def test_attn_prep_append(dev, oracle, nq, nkv, T, pos0, rope):
 
 
 @pytest.mark.parametrize("nq,nkv,T,pos0", [(4, 2, 3, 37), (16, 2, 16, 3000), (16, 2, 16, 0), (8, 1, 5, 511), (2, 2, 1, 64), (16, 2, 16, 1017), (16, 2, 7, 500),
-                                           (16, 2, 16, 32752)])   # the last: benchmark config 4's window at the end of a 32,768-position cache
+                                           (16, 2, 16, 32752),   # benchmark config 4's window at the end of a 32,768-position cache
+                                           # windows of few queries (up to 64 a kv head) run half a split a block: the last such row count,
+                                           # the first that does not, a decode round's window at a long context, a context that ends in a second half
+                                           (16, 2, 8, 700), (16, 2, 9, 700), (16, 2, 2, 32752), (16, 2, 4, 300)])
 def test_attn_matches_oracle(dev, oracle, nq, nkv, T, pos0):
     print(f"case attn nq={nq} nkv={nkv} T={T} pos0={pos0}", flush=True)
     rng = np.random.default_rng(830 + nq + pos0)
