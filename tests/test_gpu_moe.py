@@ -80,7 +80,9 @@ def test_moe_verify_layer_config2(dev, oracle, packed):
 
 @pytest.mark.parametrize("packed", [False, True])
 @pytest.mark.parametrize("n,ff,nexp,topk,T", [(2048, 512, 64, 10, 1), (1024, 256, 32, 4, 16), (2048, 1024, 16, 2, 3), (512, 512, 16, 8, 7),
-                                              (2048, 256, 40, 6, 9), (2048, 512, 1000, 10, 16), (2048, 512, 12, 10, 16)])
+                                              (2048, 256, 40, 6, 9), (2048, 512, 1000, 10, 16), (2048, 512, 12, 10, 16),
+                                              # windows of few rows: a block has four or eight units and deals the row's trips over its waves
+                                              (2048, 512, 64, 10, 2), (2048, 512, 128, 10, 4), (2048, 512, 512, 10, 3)])
 def test_moe_verify_layer_shapes(dev, oracle, n, ff, nexp, topk, T, packed):
     # with unit64 weights the shapes of hidden 2048 run as the one-launch window, the others operator by operator
     check_layer(dev, oracle, n, ff, nexp, topk, T, 910 + T, packed)
