@@ -1859,7 +1859,6 @@ int fnx_decode_round(const fnx_decoder* D, const fnx_mtp* M, const fnx_round* R,
     if (K > 1 && !R->chain_src) return fail("decode_round: the chain needs its source row's buffer");
     hipStream_t s = (hipStream_t) st;
     int* S = R->state;
-    k_round_guard<<<1, 1, 0, s>>>(S, R->ctx_cap, D->max_ctx);
     if (decoder_verify(D, R->rows, FNX_MAXT, S + FNX_RS_POS, ws, st, S + FNX_RS_ROWS)) return 1;
     k_round_commit<<<1, 64, 0, s>>>(R->rows, ws->best_i, S, R->ctx, R->ctx_cap, D->max_ctx, R->log_cap ? R->log : nullptr, R->log_cap);
     if (R->speculate) {

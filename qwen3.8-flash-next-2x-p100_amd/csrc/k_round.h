@@ -13,17 +13,12 @@
 
 namespace fnx {
 
-// before the verify: a session whose window does not fit the caches (or whose context buffer is full) stops here, so the
-// first round of a badly placed session changes nothing either (later rounds are kept inside by k_round_commit)
-__global__ void k_round_guard(int* __restrict__ state, int ctx_cap, int max_ctx) {
-    const int pos = state[FNX_RS_POS], n_ctx = state[FNX_RS_NCTX];
-    if (pos < 0 || pos + FNX_MAXT > max_ctx || n_ctx + FNX_MAXT > ctx_cap) state[FNX_RS_STOP] = 1;
-}
-
 // after the verify (session.cpp:565-573, 616-640): n = 1 + the drafts that equal the row before's pick; the picks of the
 // rows kept join the context; the positions move on by n. One wave.
 // A round whose next window would not fit the caches (max_ctx) or the context buffer raises FNX_RS_STOP and changes
-// nothing; every later round then finds the same state and repeats the same work.
+// nothing; every later round then finds the same state and repeats the same work. So does the first round of a badly
+// placed session (a position below zero, or a window that does not fit to begin with: the verify before this computed
+// over the cells that exist and is not kept).
 __global__ void k_round_commit(const int* __restrict__ rows, const int* __restrict__ best, int* __restrict__ state, int* __restrict__ ctx,
                                int ctx_cap, int max_ctx, int* __restrict__ log, int log_cap) {
     const int i = threadIdx.x;
@@ -32,7 +27,7 @@ __global__ void k_round_commit(const int* __restrict__ rows, const int* __restri
     const bool ok = i + 1 < R && rows[i + 1] == best[i];
     const int n = 1 + (int) __builtin_ctzll(~__ballot(ok));
     const int pick = i < n ? best[i] : 0;
-    if (stop || pos + n + FNX_MAXT > max_ctx || n_ctx + n + FNX_MAXT > ctx_cap) {
+    if (stop || pos < 0 || pos + n + FNX_MAXT > max_ctx || n_ctx + n + FNX_MAXT > ctx_cap) {
         if (i == 0) state[FNX_RS_STOP] = 1;
         return;
     }
