@@ -628,14 +628,19 @@ __global__ void __launch_bounds__(AM_THREADS) k_argmax(const float* __restrict__
 // a ballot each.
 constexpr int LK_THREADS = 1024, LK_STEPS = 10, LOOKUP_MIN = 3, IMAGE_TOK = 1 << 30;   // 40,960 start positions a round
 // n_ctx_p (may be null): the context's length is that device word instead of n_ctx; d1_at (may be null): d1 is
-// d1p[*d1_at - 1] instead of d1p[0] (the pick of the last row kept).
+// d1p[*d1_at - 1] instead of d1p[0] (the pick of the last row kept). rs, rs_rows (may be null; only with n_ctx_p and d1_at
+// the round's own words): a decode round's state and window - the round's next window (k_round_window's rows and count,
+// k_round.h) is made here as well, from the drafts this launch finds: a launch less a round.
 __global__ void __launch_bounds__(LK_THREADS) k_lookup(const int* __restrict__ ctx, int n_ctx, int key_n, int lk, const int* __restrict__ d1p,
                                                       int* __restrict__ out, int* __restrict__ n_out, int* __restrict__ match,
-                                                      const int* __restrict__ n_ctx_p, const int* __restrict__ d1_at) {
+                                                      const int* __restrict__ n_ctx_p, const int* __restrict__ d1_at,
+                                                      int* __restrict__ rs = nullptr, int* __restrict__ rs_rows = nullptr) {
     __shared__ int best;
     if (threadIdx.x == 0) best = -1;
     if (n_ctx_p) n_ctx = *n_ctx_p;
     const int d1 = d1p[d1_at ? min(max(*d1_at, 1), FNX_MAXT) - 1 : 0];   // asked for now, used at the end
+    // (what the next window needs beside the drafts, asked for now as well)
+    const int rs_stop = rs ? rs[FNX_RS_STOP] : 1, last_tok = rs && n_ctx > 0 ? ctx[n_ctx - 1] : 0;
     __syncthreads();
     const int n0 = n_ctx - key_n;
     if (lk > 0 && n0 > 0) {
@@ -679,7 +684,7 @@ __global__ void __launch_bounds__(LK_THREADS) k_lookup(const int* __restrict__ c
     __syncthreads();
     if (threadIdx.x >= 64) return;
     const int lane = threadIdx.x;
-    int nr = 0, m_at = -1;
+    int nr = 0, m_at = -1, dtok = 0;   // (dtok: this lane's draft)
     const int s = best;
     if (s >= 0 && s + key_n < n_ctx) {
         // one trip to memory for everything the rest needs: the tokens before the match and before the key (lane j: the
@@ -696,13 +701,22 @@ __global__ void __launch_bounds__(LK_THREADS) k_lookup(const int* __restrict__ c
         // the drafts: a lane per token; an image cell is never a draft, nor anything after it
         const unsigned long long stop = __ballot(lane < want && tok >= IMAGE_TOK);
         nr = stop ? min(want, (int) __builtin_ctzll(stop)) : want;
-        if (lane < nr) out[lane] = tok;
+        if (lane < nr) out[lane] = dtok = tok;
         m_at = s;
     }
 done:
     if (lane == 0) {
         *n_out = nr;
         if (match) *match = m_at;
+    }
+    if (rs && !rs_stop) {   // session.cpp:530-560: the context's last token, then the drafts, or else the draft layer's pick
+        const int nd = min(nr, FNX_MAXT - 1), before = __shfl_up(dtok, 1, 64);   // lane i: draft i - 1
+        int tok = 0;
+        if (lane == 0) tok = last_tok;
+        else if (nd > 0) tok = lane <= nd ? before : 0;
+        else if (lane == 1) tok = d1;
+        if (lane < FNX_MAXT) rs_rows[lane] = tok;
+        if (lane == 0) rs[FNX_RS_ROWS] = nd > 0 ? 1 + nd : 2;
     }
 }
 __global__ void k_accept(const int* __restrict__ rows, const int* __restrict__ o, int R, int* __restrict__ n_accept) {
@@ -1864,8 +1878,9 @@ int fnx_decode_round(const fnx_decoder* D, const fnx_mtp* M, const fnx_round* R,
     if (R->speculate) {
         // the rows kept and their picks are where the verify left them; the draft layer overwrites both only at its end
         if (mtp_draft(D, M, ws->hidden, ws->best_i, FNX_MAXT, S + FNX_RS_POS_PREV, ws, st, S + FNX_RS_ACCEPTED)) return 1;
+        // (with a single draft a round the lookup's launch makes the next window too)
         k_lookup<<<1, LK_THREADS, 0, s>>>(R->ctx, 0, R->key_n, R->lk, ws->best_i, R->scratch + 1, R->scratch, nullptr, S + FNX_RS_NCTX,
-                                          S + FNX_RS_ACCEPTED);
+                                          S + FNX_RS_ACCEPTED, K == 1 ? S : nullptr, K == 1 ? R->rows : nullptr);
         if (K > 1) {
             // the chain (session.cpp:666-678): step j reads the draft before it at the position after it, from the draft
             // layer's own row; one row, which counts (is routed, runs the big kernels) only while state[CHAIN] is set
@@ -1877,7 +1892,7 @@ int fnx_decode_round(const fnx_decoder* D, const fnx_mtp* M, const fnx_round* R,
             }
         }
     }
-    k_round_window<<<1, 64, 0, s>>>(R->ctx, S, R->scratch + 1, R->scratch, ws->best_i, R->speculate, R->rows);
+    if (!R->speculate || K > 1) k_round_window<<<1, 64, 0, s>>>(R->ctx, S, R->scratch + 1, R->scratch, ws->best_i, R->speculate, R->rows);
     return launch_status("decode_round");
 }
 
